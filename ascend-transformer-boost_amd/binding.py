@@ -1,0 +1,332 @@
+"""ctypes binding of the two in-tree libraries.
+
+`kernels()` loads lib/libatbmi_kernels.so (the C ABI of the HIP kernels) and
+`atb()` loads lib/libatb.so (the atb::Operation layer through its flat C view).
+Both raise if the library has not been built: there is no fallback path.
+
+The classes below are a thin driver in the order the reference's own test
+harness uses (reference tests/framework/c++/atb_torch/operation/operation_torch.cpp:313-415):
+create the operation from its param, InferShape, allocate outputs, build the
+VariantPack, bind host tensors (contextLens), Setup, allocate the workspace,
+Execute. PyTorch is used only to hold device memory and the HIP stream.
+"""
+import ctypes
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_PKG, "lib")
+
+# aclDataType / aclFormat values (include/acl/acl.h)
+ACL_FLOAT, ACL_FLOAT16, ACL_INT8, ACL_INT32, ACL_INT64, ACL_BF16 = 0, 1, 2, 3, 9, 27
+ACL_FORMAT_ND, ACL_FORMAT_FRACTAL_NZ = 2, 29
+ACL_DTYPE_BY_NAME = {
+    "float": 0, "float16": 1, "int8": 2, "int32": 3, "uint8": 4, "int16": 6, "uint16": 7, "uint32": 8,
+    "int64": 9, "uint64": 10, "double": 11, "bool": 12, "bf16": 27,
+}
+ACL_FORMAT_BY_NAME = {"nchw": 0, "nhwc": 1, "nd": 2, "fractal_nz": 29}
+
+# atb::ErrorType (include/atb/types.h)
+ERROR_NAMES = [
+    "NO_ERROR", "ERROR_INVALID_PARAM", "ERROR_INVALID_GRAPH", "ERROR_INTERNAL_ERROR", "ERROR_RT_FAIL",
+    "ERROR_INVALID_IN_TENSOR_NUM", "ERROR_INVALID_TENSOR_DTYPE", "ERROR_INVALID_TENSOR_FORMAT",
+    "ERROR_INVALID_TENSOR_DIM", "ERROR_INVALID_TENSOR_SIZE", "ERROR_OPERATION_NULL_RUNNER",
+    "ERROR_GRAPH_INFERSHAPE_FUNC_FAIL", "ERROR_CANN_ERROR", "ERROR_INVALID_TENSOR_INI_MATCH",
+    "ERROR_INVALID_TENSOR_ADDR", "ERROR_INVALID_TENSOR_NUM", "ERROR_INVALID_TENSOR_DIM_NUM",
+    "ERROR_INVALID_SINGLE_OPERATION_PARAM", "ERROR_GRAPH_NODE_RESHAPE_FUNC_FAIL", "ERROR_INVALID_GRAPH_NODE_CHUNK",
+    "ERROR_INVALID_CONTEXT_ADDR", "ERROR_INVALID_STREAM", "ERROR_INVALID_WORKSPACE_SIZE",
+    "ERROR_INVALID_WORKSPACE_ADDR", "ERROR_INVALID_OPERATION_ADDR", "ERROR_HCCL_FAIL",
+    "ERROR_OUT_OF_DEVICE_MEMORY", "ERROR_OUT_OF_HOST_MEMORY", "ERROR_COMM_EMPTY", "ERROR_COPY_HOST_MEMORY_FAIL",
+]
+ERROR_CODE = {n: i for i, n in enumerate(ERROR_NAMES)}
+
+ATBMI_F16, ATBMI_BF16, ATBMI_INT8 = 0, 1, 2
+ATBMI_PA_KERNEL_AUTO, ATBMI_PA_KERNEL_SCALAR, ATBMI_PA_KERNEL_MFMA = 0, 1, 2
+
+
+class AtbCTensor(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ctypes.c_int32), ("format", ctypes.c_int32), ("dims", ctypes.c_int64 * 8),
+        ("dimNum", ctypes.c_uint64), ("deviceData", ctypes.c_void_p), ("hostData", ctypes.c_void_p),
+        ("dataSize", ctypes.c_uint64),
+    ]
+
+
+class PagedAttentionParam(ctypes.Structure):
+    """Byte image of atb::infer::PagedAttentionParam (120 bytes)."""
+    _fields_ = [
+        ("headNum", ctypes.c_int32), ("qkScale", ctypes.c_float), ("kvHeadNum", ctypes.c_int32),
+        ("maskType", ctypes.c_int32), ("batchRunStatusEnable", ctypes.c_bool), ("quantType", ctypes.c_int32),
+        ("outDataType", ctypes.c_int32), ("hasQuantOffset", ctypes.c_bool), ("compressType", ctypes.c_int32),
+        ("calcType", ctypes.c_int32), ("scaleType", ctypes.c_int32), ("inputLayout", ctypes.c_int32),
+        ("mlaVHeadSize", ctypes.c_uint32), ("qScale", ctypes.c_float), ("rsv", ctypes.c_uint8 * 64),
+    ]
+
+    def __init__(self, **kw):
+        super().__init__()
+        self.qkScale = 1.0
+        self.outDataType = -1
+        for k, v in kw.items():
+            if not hasattr(self, k):
+                raise AttributeError("PagedAttentionParam has no field " + k)
+            setattr(self, k, v)
+
+
+class ReshapeAndCacheParam(ctypes.Structure):
+    """Byte image of atb::infer::ReshapeAndCacheParam (24 bytes)."""
+    _fields_ = [("compressType", ctypes.c_int32), ("kvCacheCfg", ctypes.c_int32), ("rsv", ctypes.c_uint8 * 16)]
+
+    def __init__(self, **kw):
+        super().__init__()
+        for k, v in kw.items():
+            if not hasattr(self, k):
+                raise AttributeError("ReshapeAndCacheParam has no field " + k)
+            setattr(self, k, v)
+
+
+class AtbmiPaShape(ctypes.Structure):
+    _fields_ = [
+        ("qDtype", ctypes.c_int32), ("kvDtype", ctypes.c_int32), ("numHeads", ctypes.c_int32),
+        ("numKvHeads", ctypes.c_int32), ("headDimK", ctypes.c_int32), ("headDimV", ctypes.c_int32),
+        ("blockSize", ctypes.c_int32), ("numBlocks", ctypes.c_int32), ("maxBlocksPerSeq", ctypes.c_int32),
+        ("numQueryRows", ctypes.c_int32), ("mlaCombined", ctypes.c_int32), ("hasOffset", ctypes.c_int32),
+        ("kernel", ctypes.c_int32), ("reserved", ctypes.c_int32), ("qkScale", ctypes.c_float),
+        ("qScale", ctypes.c_float),
+    ]
+
+
+class AtbmiPaTensors(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_void_p) for n in
+                ("query", "keyCache", "valueCache", "blockTables", "kScale", "kOffset", "vScale", "vOffset", "out")]
+
+
+_kernels = None
+_atb = None
+
+
+def _load(name):
+    path = os.path.join(_LIB, name)
+    if not os.path.exists(path):
+        raise RuntimeError("%s is not built; run `python3 %s`" % (path, os.path.join(_PKG, "build.py")))
+    return ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
+
+
+def kernels():
+    """libatbmi_kernels.so with argument types set."""
+    global _kernels
+    if _kernels is None:
+        lib = _load("libatbmi_kernels.so")
+        vp, i32, i64, u64 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_uint64
+        lib.atbmi_last_error.restype = ctypes.c_char_p
+        lib.atbmi_last_error.argtypes = []
+        lib.atbmi_device_count.restype = ctypes.c_int
+        lib.atbmi_reshape_and_cache.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]
+        lib.atbmi_quant_per_channel.argtypes = [vp, i32, vp, vp, vp, i64, i64, vp]
+        lib.atbmi_reshape_and_cache_quant.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]
+        lib.atbmi_pa_plan_create.argtypes = [ctypes.POINTER(AtbmiPaShape), ctypes.POINTER(vp)]
+        lib.atbmi_pa_plan_update.argtypes = [vp, vp, i32]
+        lib.atbmi_pa_plan_workspace_size.argtypes = [vp]
+        lib.atbmi_pa_plan_workspace_size.restype = u64
+        lib.atbmi_pa_plan_num_chunks.argtypes = [vp]
+        lib.atbmi_pa_plan_num_chunks.restype = i64
+        lib.atbmi_pa_plan_algorithmic_bytes.argtypes = [vp]
+        lib.atbmi_pa_plan_algorithmic_bytes.restype = u64
+        lib.atbmi_pa_decode.argtypes = [vp, ctypes.POINTER(AtbmiPaTensors), vp, u64, vp]
+        lib.atbmi_pa_plan_destroy.argtypes = [vp]
+        lib.atbmi_pa_plan_destroy.restype = None
+        lib.atbmi_timing_enable.argtypes = [i32]
+        lib.atbmi_timing_read.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(i64)]
+        _kernels = lib
+    return _kernels
+
+
+def atb():
+    """libatb.so (flat C view of atb::Operation) with argument types set."""
+    global _atb
+    if _atb is None:
+        kernels()  # libatb.so depends on it
+        lib = _load("libatb.so")
+        vp, i32, u32, u64 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_uint32, ctypes.c_uint64
+        tp = ctypes.POINTER(AtbCTensor)
+        lib.atb_c_create_context.argtypes = [vp, ctypes.POINTER(vp)]
+        lib.atb_c_context_set_stream.argtypes = [vp, vp]
+        lib.atb_c_context_set_execute_type.argtypes = [vp, i32]
+        lib.atb_c_destroy_context.argtypes = [vp]
+        lib.atb_c_create_operation.argtypes = [ctypes.c_char_p, vp, u64, ctypes.POINTER(vp)]
+        lib.atb_c_destroy_operation.argtypes = [vp]
+        lib.atb_c_op_input_num.argtypes = [vp]
+        lib.atb_c_op_input_num.restype = u32
+        lib.atb_c_op_output_num.argtypes = [vp]
+        lib.atb_c_op_output_num.restype = u32
+        lib.atb_c_op_name.argtypes = [vp, ctypes.c_char_p, u64]
+        lib.atb_c_op_infer_shape.argtypes = [vp, tp, u32, tp, u32, ctypes.POINTER(u32)]
+        lib.atb_c_op_setup.argtypes = [vp, tp, u32, tp, u32, ctypes.POINTER(u64), vp]
+        lib.atb_c_op_execute.argtypes = [vp, tp, u32, tp, u32, vp, u64, vp]
+        lib.atb_c_tensor_size.argtypes = [tp]
+        lib.atb_c_tensor_size.restype = u64
+        lib.atb_c_sizeof_paged_attention_param.restype = u64
+        lib.atb_c_sizeof_reshape_and_cache_param.restype = u64
+        _atb = lib
+    return _atb
+
+
+def last_kernel_error():
+    return kernels().atbmi_last_error().decode()
+
+
+def make_tensor(dtype, shape, device_ptr=None, host_ptr=None, fmt=ACL_FORMAT_ND, data_size=None):
+    """AtbCTensor from raw pieces; dataSize defaults to Utils::GetTensorSize."""
+    t = AtbCTensor()
+    t.dtype = ACL_DTYPE_BY_NAME[dtype] if isinstance(dtype, str) else int(dtype)
+    t.format = ACL_FORMAT_BY_NAME[fmt] if isinstance(fmt, str) else int(fmt)
+    t.dimNum = len(shape)
+    for i, d in enumerate(shape[:8]):
+        t.dims[i] = int(d)
+    t.deviceData = device_ptr
+    t.hostData = host_ptr
+    t.dataSize = atb().atb_c_tensor_size(ctypes.byref(t)) if data_size is None else int(data_size)
+    return t
+
+
+def _torch_acl_dtype(t):
+    import torch
+    return {torch.float16: ACL_FLOAT16, torch.bfloat16: ACL_BF16, torch.int8: ACL_INT8, torch.int32: ACL_INT32,
+            torch.float32: ACL_FLOAT, torch.int64: ACL_INT64}[t.dtype]
+
+
+def tensor_of(t, host=None):
+    """AtbCTensor describing a contiguous torch tensor on the GPU; `host` is an
+    optional contiguous CPU tensor bound as hostData (contextLens)."""
+    if not t.is_contiguous():
+        raise ValueError("tensor must be contiguous")
+    c = make_tensor(_torch_acl_dtype(t), list(t.shape), device_ptr=t.data_ptr() if t.is_cuda else None,
+                    host_ptr=(host.data_ptr() if host is not None else (None if t.is_cuda else t.data_ptr())))
+    return c
+
+
+class Context:
+    """atb::Context bound to a HIP stream (a torch.cuda.Stream or a raw handle)."""
+
+    def __init__(self, stream):
+        self.stream = stream
+        handle = stream.cuda_stream if hasattr(stream, "cuda_stream") else stream
+        self.ptr = ctypes.c_void_p()
+        st = atb().atb_c_create_context(ctypes.c_void_p(handle), ctypes.byref(self.ptr))
+        if st != 0:
+            raise RuntimeError("CreateContext failed: %s" % ERROR_NAMES[st])
+
+    def set_execute_type(self, t):
+        return atb().atb_c_context_set_execute_type(self.ptr, int(t))
+
+    def close(self):
+        if self.ptr:
+            atb().atb_c_destroy_context(self.ptr)
+            self.ptr = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Operation:
+    """An atb::Operation created from a param struct. create() returns the status
+    instead of raising, so error-path tests can read it."""
+
+    def __init__(self, name, param):
+        self.name = name
+        self.param = param
+        self.ptr = ctypes.c_void_p()
+        self.status = atb().atb_c_create_operation(name.encode(), ctypes.byref(param), ctypes.sizeof(param),
+                                                   ctypes.byref(self.ptr))
+        self._keep = None
+
+    @property
+    def ok(self):
+        return self.status == 0 and bool(self.ptr)
+
+    def input_num(self):
+        return atb().atb_c_op_input_num(self.ptr)
+
+    def output_num(self):
+        return atb().atb_c_op_output_num(self.ptr)
+
+    def get_name(self):
+        buf = ctypes.create_string_buffer(128)
+        atb().atb_c_op_name(self.ptr, buf, 128)
+        return buf.value.decode()
+
+    def infer_shape(self, in_descs):
+        arr = (AtbCTensor * max(1, len(in_descs)))(*in_descs)
+        out = (AtbCTensor * 8)()
+        n = ctypes.c_uint32(0)
+        st = atb().atb_c_op_infer_shape(self.ptr, arr, len(in_descs), out, 8, ctypes.byref(n))
+        return st, [out[i] for i in range(n.value)] if st == 0 else []
+
+    def setup(self, in_tensors, out_tensors, context):
+        ia = (AtbCTensor * max(1, len(in_tensors)))(*in_tensors)
+        oa = (AtbCTensor * max(1, len(out_tensors)))(*out_tensors)
+        ws = ctypes.c_uint64(0)
+        ctx = context.ptr if isinstance(context, Context) else context
+        st = atb().atb_c_op_setup(self.ptr, ia, len(in_tensors), oa, len(out_tensors), ctypes.byref(ws), ctx)
+        return st, ws.value
+
+    def execute(self, in_tensors, out_tensors, workspace_ptr, workspace_size, context):
+        ia = (AtbCTensor * max(1, len(in_tensors)))(*in_tensors)
+        oa = (AtbCTensor * max(1, len(out_tensors)))(*out_tensors)
+        ctx = context.ptr if isinstance(context, Context) else context
+        return atb().atb_c_op_execute(self.ptr, ia, len(in_tensors), oa, len(out_tensors),
+                                      ctypes.c_void_p(workspace_ptr), workspace_size, ctx)
+
+    def close(self):
+        if self.ptr:
+            atb().atb_c_destroy_operation(self.ptr)
+            self.ptr = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class OperationRunner:
+    """Runs one operation on torch GPU tensors the way the reference harness does:
+    InferShape -> allocate outputs (or take caller-owned ones) -> Setup ->
+    workspace -> Execute. The workspace tensor is kept and grown on demand."""
+
+    def __init__(self, name, param, context):
+        self.op = Operation(name, param)
+        if not self.op.ok:
+            raise RuntimeError("CreateOperation(%s) failed: %s" % (name, ERROR_NAMES[self.op.status]))
+        self.context = context
+        self.workspace = None
+
+    def run(self, inputs, outputs=None, host_inputs=None):
+        """inputs: torch GPU tensors; host_inputs: {index: CPU tensor} bound as
+        hostData; outputs: caller-owned output tensors (in-place cache update)
+        or None to allocate from InferShape. Returns the output tensors."""
+        import torch
+        host_inputs = host_inputs or {}
+        ins = [tensor_of(t, host_inputs.get(i)) for i, t in enumerate(inputs)]
+        if outputs is None:
+            st, descs = self.op.infer_shape(ins)
+            if st != 0:
+                raise RuntimeError("InferShape failed: %s" % ERROR_NAMES[st])
+            rev = {ACL_FLOAT16: torch.float16, ACL_BF16: torch.bfloat16, ACL_INT8: torch.int8}
+            outputs = [torch.empty([d.dims[i] for i in range(d.dimNum)], dtype=rev[d.dtype], device=inputs[0].device)
+                       for d in descs]
+        outs = [tensor_of(t) for t in outputs]
+        st, ws = self.op.setup(ins, outs, self.context)
+        if st != 0:
+            raise RuntimeError("Setup failed: %s" % ERROR_NAMES[st])
+        if ws > 0 and (self.workspace is None or self.workspace.numel() < ws):
+            self.workspace = torch.empty(int(ws), dtype=torch.uint8, device=inputs[0].device)
+        wptr = self.workspace.data_ptr() if ws > 0 else None
+        st = self.op.execute(ins, outs, wptr, ws, self.context)
+        if st != 0:
+            raise RuntimeError("Execute failed: %s (%s)" % (ERROR_NAMES[st], last_kernel_error()))
+        return outputs
+
+    def close(self):
+        self.op.close()

@@ -1,0 +1,486 @@
+// Host side of paged decode attention: shape validation, the split-KV
+// planner, plan upload and kernel dispatch.
+//
+// The planner plays the part of the reference's PagedAttentionTiling
+// (reference src/kernels/mixkernels/pagedattention/tiling/paged_attention_tiling.cpp:419-470
+// and tiling/paged_attention_tiling_dependency.cpp:186-259,406-521): it decides how the
+// KV range of every sequence is cut into chunks. Unlike the reference, which
+// cuts by the longest sequence, chunks here are cut per sequence from its own
+// length so a skewed batch still spreads evenly over the 256 CUs.
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <vector>
+#include "pa_internal.h"
+
+namespace atbmi {
+
+namespace {
+thread_local char g_lastError[512] = "";
+}
+
+int Fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_lastError, sizeof(g_lastError), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+namespace {
+
+constexpr uint64_t WS_ALIGN = 256;
+constexpr int RING = 4;
+constexpr int NUM_CUS = 256;
+
+uint64_t AlignUp(uint64_t v, uint64_t a)
+{
+    return (v + a - 1) / a * a;
+}
+
+int64_t EnvInt(const char *name, int64_t fallback)
+{
+    const char *v = getenv(name);
+    if (!v || !*v) {
+        return fallback;
+    }
+    char *end = nullptr;
+    long long parsed = strtoll(v, &end, 10);
+    return (end && *end == '\0') ? parsed : fallback;
+}
+
+struct TimingRecord {
+    hipEvent_t begin;
+    hipEvent_t end;
+};
+std::mutex g_timingMutex;
+bool g_timingEnabled = false;
+std::vector<TimingRecord> g_timingRecords;
+
+} // namespace
+} // namespace atbmi
+
+using namespace atbmi;
+
+struct AtbmiPaPlan {
+    AtbmiPaShape shape;
+    bool useMfma = false;
+    int headTile = 1;        // query heads per workgroup
+    int partialsPerItem = 1; // partial slots one work item writes
+    int tokenUnit = 1;       // chunk lengths are multiples of this
+    int64_t chunkOverride = 0;
+
+    std::vector<PaWorkItem> items;
+    std::vector<PaSeqInfo> reduceSeqs;
+    int64_t numPartials = 0;
+    int32_t batch = 0;
+    int64_t totalCtx = 0;
+    int64_t tableEntries = 0;
+    int32_t nonEmpty = 0;
+
+    uint64_t offItems = 0, offSeqs = 0, offPartO = 0, offPartLse = 0, blobBytes = 0, wsBytes = 0;
+    std::vector<uint8_t> blob; // items then reduceSeqs, as uploaded
+
+    // Pinned staging ring for the asynchronous plan upload. A slot is reused
+    // only after the copy that last read it has finished.
+    void *pinned[RING] = {nullptr, nullptr, nullptr, nullptr};
+    size_t pinnedCap[RING] = {0, 0, 0, 0};
+    hipEvent_t copied[RING] = {nullptr, nullptr, nullptr, nullptr};
+    bool inFlight[RING] = {false, false, false, false};
+    int ringPos = 0;
+};
+
+extern "C" const char *atbmi_last_error(void)
+{
+    return g_lastError;
+}
+
+extern "C" int atbmi_device_count(void)
+{
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    return n;
+}
+
+extern "C" int atbmi_pa_plan_create(const AtbmiPaShape *shape, AtbmiPaPlan **plan)
+{
+    if (!shape || !plan) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: null argument");
+    }
+    const AtbmiPaShape &s = *shape;
+    if (s.qDtype != ATBMI_F16 && s.qDtype != ATBMI_BF16) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: query must be fp16 or bf16");
+    }
+    if (s.kvDtype != ATBMI_INT8 && s.kvDtype != s.qDtype) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: cache dtype must equal the query dtype or be int8");
+    }
+    if (s.numHeads <= 0 || s.numKvHeads <= 0 || s.numHeads % s.numKvHeads != 0) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: heads %d / kv heads %d", s.numHeads, s.numKvHeads);
+    }
+    if (s.headDimK <= 0 || s.headDimK > 576 || s.headDimV <= 0 || s.headDimV > 576) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: head sizes %d/%d outside (0,576]", s.headDimK, s.headDimV);
+    }
+    if (s.mlaCombined && (s.headDimV > s.headDimK || s.kvDtype == ATBMI_INT8)) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: combined cache needs Dv <= D and a 16-bit cache");
+    }
+    if (s.blockSize <= 0 || s.numBlocks <= 0 || s.maxBlocksPerSeq <= 0 || s.numQueryRows <= 0) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: bad block/batch extents");
+    }
+    if (s.hasOffset && s.kvDtype != ATBMI_INT8) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: offsets only apply to an int8 cache");
+    }
+    AtbmiPaPlan *p = new (std::nothrow) AtbmiPaPlan();
+    if (!p) {
+        return Fail(ERR_OUT_OF_HOST_MEMORY, "pa_plan_create: out of host memory");
+    }
+    p->shape = s;
+    int kernel = s.kernel;
+    const char *forced = getenv("ATBMI_PA_KERNEL");
+    if (kernel == ATBMI_PA_KERNEL_AUTO && forced) {
+        if (!strcmp(forced, "scalar")) {
+            kernel = ATBMI_PA_KERNEL_SCALAR;
+        } else if (!strcmp(forced, "mfma")) {
+            kernel = ATBMI_PA_KERNEL_MFMA;
+        }
+    }
+    const bool mfmaOk = PaMfmaSupports(s);
+    if (kernel == ATBMI_PA_KERNEL_MFMA && !mfmaOk) {
+        delete p;
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: the MFMA kernel does not cover this shape");
+    }
+    p->useMfma = (kernel == ATBMI_PA_KERNEL_MFMA) || (kernel == ATBMI_PA_KERNEL_AUTO && mfmaOk);
+    if (p->useMfma) {
+        p->headTile = PA_MFMA_HEAD_TILE;
+        p->partialsPerItem = 1;
+        p->tokenUnit = PA_MFMA_STEP * PA_MFMA_WAVES;
+    } else {
+        p->headTile = PA_SCALAR_HEAD_TILE;
+        p->partialsPerItem = PA_SCALAR_WAVES;
+        p->tokenUnit = PA_SCALAR_WAVES;
+    }
+    p->chunkOverride = EnvInt("ATBMI_PA_CHUNK_TOKENS", 0);
+    *plan = p;
+    return OK;
+}
+
+extern "C" int atbmi_pa_plan_update(AtbmiPaPlan *plan, const int32_t *ctx, int32_t batch)
+{
+    if (!plan || !ctx) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_update: null argument");
+    }
+    const AtbmiPaShape &s = plan->shape;
+    if (batch <= 0) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_update: batch %d", batch);
+    }
+    int64_t total = 0, tableEntries = 0;
+    int32_t nonEmpty = 0;
+    const int64_t maxCtx = static_cast<int64_t>(s.maxBlocksPerSeq) * s.blockSize;
+    for (int32_t b = 0; b < batch; ++b) {
+        if (ctx[b] < 0 || ctx[b] > maxCtx) {
+            return Fail(ERR_INVALID_PARAM, "pa_plan_update: contextLens[%d]=%d outside [0,%lld]", b, ctx[b],
+                        (long long)maxCtx);
+        }
+        if (ctx[b] > 0) {
+            ++nonEmpty;
+            total += ctx[b];
+            tableEntries += (ctx[b] + s.blockSize - 1) / s.blockSize;
+        }
+    }
+    if (nonEmpty > s.numQueryRows) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_update: %d non-empty sequences but only %d query rows", nonEmpty,
+                    s.numQueryRows);
+    }
+    plan->batch = batch;
+    plan->totalCtx = total;
+    plan->tableEntries = tableEntries;
+    plan->nonEmpty = nonEmpty;
+    plan->items.clear();
+    plan->reduceSeqs.clear();
+
+    // Chunk length: enough workgroups to load every CU several times over,
+    // but chunks long enough that the per-chunk prologue/epilogue stays small.
+    const int groupSize = s.numHeads / s.numKvHeads;
+    const int headTiles = (groupSize + plan->headTile - 1) / plan->headTile;
+    const int64_t wgPerItem = static_cast<int64_t>(s.numKvHeads) * headTiles;
+    const int64_t unit = plan->tokenUnit;
+    int64_t chunk = plan->chunkOverride;
+    if (chunk <= 0) {
+        const int64_t targetWgs = static_cast<int64_t>(NUM_CUS) * 8;
+        const int64_t targetItems = std::max<int64_t>(1, targetWgs / wgPerItem);
+        chunk = (total + targetItems - 1) / std::max<int64_t>(1, targetItems);
+        const int64_t minChunk = plan->useMfma ? 2 * unit : 64;
+        chunk = std::min<int64_t>(std::max<int64_t>(chunk, minChunk), 4096);
+    }
+    chunk = std::max<int64_t>(unit, (chunk + unit - 1) / unit * unit);
+
+    int64_t partials = 0;
+    int32_t qRow = 0;
+    try {
+        for (int32_t b = 0; b < batch; ++b) {
+            const int64_t len = ctx[b];
+            if (len == 0) {
+                continue;
+            }
+            const int64_t n = (len + chunk - 1) / chunk;
+            int64_t each = (len + n - 1) / n;
+            each = (each + unit - 1) / unit * unit;
+            const bool direct = plan->useMfma && n == 1;
+            const int64_t first = partials;
+            for (int64_t i = 0; i * each < len; ++i) {
+                PaWorkItem it{};
+                it.qRow = qRow;
+                it.seq = b;
+                it.tokBegin = static_cast<int32_t>(i * each);
+                it.tokEnd = static_cast<int32_t>(std::min<int64_t>(len, (i + 1) * each));
+                it.direct = direct ? 1 : 0;
+                it.partialBase = direct ? -1 : static_cast<int32_t>(partials);
+                if (!direct) {
+                    partials += plan->partialsPerItem;
+                }
+                plan->items.push_back(it);
+            }
+            if (!direct) {
+                PaSeqInfo si{};
+                si.qRow = qRow;
+                si.firstPartial = static_cast<int32_t>(first);
+                si.numPartials = static_cast<int32_t>(partials - first);
+                si.ctxLen = static_cast<int32_t>(len);
+                plan->reduceSeqs.push_back(si);
+            }
+            ++qRow;
+        }
+        // Longest chunks first, so the stragglers at the end of the launch are short.
+        std::stable_sort(plan->items.begin(), plan->items.end(), [](const PaWorkItem &x, const PaWorkItem &y) {
+            return (x.tokEnd - x.tokBegin) > (y.tokEnd - y.tokBegin);
+        });
+        plan->numPartials = partials;
+        const uint64_t itemBytes = plan->items.size() * sizeof(PaWorkItem);
+        const uint64_t seqBytes = plan->reduceSeqs.size() * sizeof(PaSeqInfo);
+        plan->offItems = 0;
+        plan->offSeqs = AlignUp(itemBytes, 16);
+        plan->blobBytes = plan->offSeqs + seqBytes;
+        plan->blob.assign(plan->blobBytes, 0);
+        if (itemBytes) {
+            memcpy(plan->blob.data() + plan->offItems, plan->items.data(), itemBytes);
+        }
+        if (seqBytes) {
+            memcpy(plan->blob.data() + plan->offSeqs, plan->reduceSeqs.data(), seqBytes);
+        }
+    } catch (const std::bad_alloc &) {
+        return Fail(ERR_OUT_OF_HOST_MEMORY, "pa_plan_update: out of host memory");
+    }
+    plan->offPartO = AlignUp(plan->blobBytes, WS_ALIGN);
+    const uint64_t partOBytes = static_cast<uint64_t>(partials) * s.numHeads * s.headDimV * sizeof(float);
+    plan->offPartLse = AlignUp(plan->offPartO + partOBytes, WS_ALIGN);
+    plan->wsBytes = AlignUp(plan->offPartLse + static_cast<uint64_t>(partials) * s.numHeads * sizeof(float), WS_ALIGN);
+    return OK;
+}
+
+extern "C" uint64_t atbmi_pa_plan_workspace_size(const AtbmiPaPlan *plan)
+{
+    return plan ? plan->wsBytes : 0;
+}
+
+extern "C" int64_t atbmi_pa_plan_num_chunks(const AtbmiPaPlan *plan)
+{
+    return plan ? static_cast<int64_t>(plan->items.size()) : 0;
+}
+
+extern "C" uint64_t atbmi_pa_plan_algorithmic_bytes(const AtbmiPaPlan *plan)
+{
+    if (!plan) {
+        return 0;
+    }
+    const AtbmiPaShape &s = plan->shape;
+    const uint64_t kvSize = s.kvDtype == ATBMI_INT8 ? 1 : 2;
+    const uint64_t perToken =
+        static_cast<uint64_t>(s.numKvHeads) * (s.mlaCombined ? s.headDimK : s.headDimK + s.headDimV) * kvSize;
+    uint64_t bytes = static_cast<uint64_t>(plan->totalCtx) * perToken;
+    bytes += static_cast<uint64_t>(plan->nonEmpty) * s.numHeads * (s.headDimK + s.headDimV) * 2;
+    bytes += static_cast<uint64_t>(plan->tableEntries) * 4 + static_cast<uint64_t>(plan->batch) * 4;
+    if (s.kvDtype == ATBMI_INT8) {
+        const uint64_t vec = static_cast<uint64_t>(s.numKvHeads) * (s.headDimK + s.headDimV) * 4;
+        bytes += vec * (s.hasOffset ? 2 : 1);
+    }
+    return bytes;
+}
+
+extern "C" void atbmi_pa_plan_destroy(AtbmiPaPlan *plan)
+{
+    if (!plan) {
+        return;
+    }
+    for (int i = 0; i < RING; ++i) {
+        if (plan->copied[i]) {
+            if (plan->inFlight[i]) {
+                (void)hipEventSynchronize(plan->copied[i]);
+            }
+            (void)hipEventDestroy(plan->copied[i]);
+        }
+        if (plan->pinned[i]) {
+            (void)hipHostFree(plan->pinned[i]);
+        }
+    }
+    delete plan;
+}
+
+namespace {
+
+// Copies the plan blob into the next pinned slot and enqueues its upload.
+int UploadPlan(AtbmiPaPlan *plan, void *workspace, hipStream_t stream)
+{
+    if (plan->blobBytes == 0) {
+        return OK;
+    }
+    const int slot = plan->ringPos;
+    plan->ringPos = (plan->ringPos + 1) % RING;
+    if (plan->inFlight[slot]) {
+        ATBMI_HIP_CHECK(hipEventSynchronize(plan->copied[slot]));
+        plan->inFlight[slot] = false;
+    }
+    if (plan->pinnedCap[slot] < plan->blobBytes) {
+        if (plan->pinned[slot]) {
+            ATBMI_HIP_CHECK(hipHostFree(plan->pinned[slot]));
+            plan->pinned[slot] = nullptr;
+            plan->pinnedCap[slot] = 0;
+        }
+        const size_t cap = static_cast<size_t>(AlignUp(plan->blobBytes * 2, 4096));
+        ATBMI_HIP_CHECK(hipHostMalloc(&plan->pinned[slot], cap, hipHostMallocDefault));
+        plan->pinnedCap[slot] = cap;
+    }
+    if (!plan->copied[slot]) {
+        ATBMI_HIP_CHECK(hipEventCreateWithFlags(&plan->copied[slot], hipEventDisableTiming));
+    }
+    memcpy(plan->pinned[slot], plan->blob.data(), plan->blobBytes);
+    ATBMI_HIP_CHECK(hipMemcpyAsync(workspace, plan->pinned[slot], plan->blobBytes, hipMemcpyHostToDevice, stream));
+    ATBMI_HIP_CHECK(hipEventRecord(plan->copied[slot], stream));
+    plan->inFlight[slot] = true;
+    return OK;
+}
+
+} // namespace
+
+extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void *workspace, uint64_t workspaceBytes,
+                               void *streamHandle)
+{
+    if (!plan || !t) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: null argument");
+    }
+    const AtbmiPaShape &s = plan->shape;
+    if (plan->items.empty()) {
+        return OK; // every sequence is empty: nothing is written
+    }
+    if (!t->query || !t->keyCache || !t->blockTables || !t->out || (!s.mlaCombined && !t->valueCache)) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: a required tensor is null");
+    }
+    if (s.kvDtype == ATBMI_INT8 && (!t->kScale || !t->vScale)) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: int8 cache needs kScale and vScale");
+    }
+    if (s.hasOffset && (!t->kOffset || !t->vOffset)) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: hasOffset needs kOffset and vOffset");
+    }
+    if (plan->wsBytes > 0 && (!workspace || workspaceBytes < plan->wsBytes)) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: workspace of %llu bytes, %llu needed",
+                    (unsigned long long)workspaceBytes, (unsigned long long)plan->wsBytes);
+    }
+    if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: workspace must be 16-byte aligned");
+    }
+    hipStream_t stream = static_cast<hipStream_t>(streamHandle);
+    int rc = UploadPlan(plan, workspace, stream);
+    if (rc != OK) {
+        return rc;
+    }
+
+    uint8_t *ws = static_cast<uint8_t *>(workspace);
+    PaArgs a{};
+    a.q = t->query;
+    a.kc = t->keyCache;
+    a.vc = s.mlaCombined ? t->keyCache : t->valueCache;
+    a.tables = t->blockTables;
+    a.kScale = t->kScale;
+    a.kOff = s.hasOffset ? t->kOffset : nullptr;
+    a.vScale = t->vScale;
+    a.vOff = s.hasOffset ? t->vOffset : nullptr;
+    a.out = t->out;
+    a.items = reinterpret_cast<const PaWorkItem *>(ws + plan->offItems);
+    a.seqs = reinterpret_cast<const PaSeqInfo *>(ws + plan->offSeqs);
+    a.partO = reinterpret_cast<float *>(ws + plan->offPartO);
+    a.partLse = reinterpret_cast<float *>(ws + plan->offPartLse);
+    a.H = s.numHeads;
+    a.G = s.numKvHeads;
+    a.D = s.headDimK;
+    a.Dv = s.headDimV;
+    a.blockSize = s.blockSize;
+    a.maxBlocksPerSeq = s.maxBlocksPerSeq;
+    a.qIsBf16 = s.qDtype == ATBMI_BF16;
+    a.groupSize = s.numHeads / s.numKvHeads;
+    a.qkScale = s.qkScale;
+    a.qScale = (s.qScale == 0.0f || s.qScale == 1.0f) ? 0.0f : s.qScale;
+    a.kRowStride = static_cast<int64_t>(s.numKvHeads) * s.headDimK;
+    a.vRowStride = s.mlaCombined ? a.kRowStride : static_cast<int64_t>(s.numKvHeads) * s.headDimV;
+    a.vHeadStride = s.mlaCombined ? s.headDimK : s.headDimV;
+    a.finishV = (plan->useMfma && s.kvDtype == ATBMI_INT8) ? 1 : 0;
+
+    TimingRecord rec{nullptr, nullptr};
+    bool timed = false;
+    {
+        std::lock_guard<std::mutex> lock(g_timingMutex);
+        timed = g_timingEnabled;
+    }
+    if (timed) {
+        ATBMI_HIP_CHECK(hipEventCreate(&rec.begin));
+        ATBMI_HIP_CHECK(hipEventCreate(&rec.end));
+        ATBMI_HIP_CHECK(hipEventRecord(rec.begin, stream));
+    }
+    const int numItems = static_cast<int>(plan->items.size());
+    rc = plan->useMfma ? LaunchPaMfma(s, a, numItems, stream) : LaunchPaScalar(s, a, numItems, stream);
+    if (timed) {
+        ATBMI_HIP_CHECK(hipEventRecord(rec.end, stream));
+        std::lock_guard<std::mutex> lock(g_timingMutex);
+        g_timingRecords.push_back(rec);
+    }
+    if (rc != OK) {
+        return rc;
+    }
+    return LaunchPaReduce(s, a, static_cast<int>(plan->reduceSeqs.size()), stream);
+}
+
+extern "C" int atbmi_timing_enable(int32_t enable)
+{
+    std::lock_guard<std::mutex> lock(g_timingMutex);
+    g_timingEnabled = enable != 0;
+    return OK;
+}
+
+extern "C" int atbmi_timing_read(double *totalMs, int64_t *launches)
+{
+    std::vector<TimingRecord> records;
+    {
+        std::lock_guard<std::mutex> lock(g_timingMutex);
+        records.swap(g_timingRecords);
+    }
+    double sum = 0.0;
+    for (const TimingRecord &r : records) {
+        ATBMI_HIP_CHECK(hipEventSynchronize(r.end));
+        float ms = 0.0f;
+        ATBMI_HIP_CHECK(hipEventElapsedTime(&ms, r.begin, r.end));
+        sum += ms;
+        (void)hipEventDestroy(r.begin);
+        (void)hipEventDestroy(r.end);
+    }
+    if (totalMs) {
+        *totalMs = sum;
+    }
+    if (launches) {
+        *launches = static_cast<int64_t>(records.size());
+    }
+    return OK;
+}

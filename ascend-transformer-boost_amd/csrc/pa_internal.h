@@ -1,0 +1,32 @@
+// Internal interfaces between the decode-attention planner/launcher and the
+// kernels. Not part of the C ABI.
+#ifndef ATBMI_PA_INTERNAL_H
+#define ATBMI_PA_INTERNAL_H
+#include "atbmi_common.h"
+
+namespace atbmi {
+
+// Waves per workgroup of the scalar kernel; each wave writes its own partial.
+constexpr int PA_SCALAR_WAVES = 4;
+// Query heads one scalar-kernel workgroup handles.
+constexpr int PA_SCALAR_HEAD_TILE = 8;
+
+// Tokens one MFMA-kernel wave consumes per step, waves per workgroup, and
+// query heads per workgroup (the N extent of a 16x16 MFMA tile).
+constexpr int PA_MFMA_STEP = 32;
+constexpr int PA_MFMA_WAVES = 4;
+constexpr int PA_MFMA_HEAD_TILE = 16;
+
+// Scalar (VALU) kernel: any head size up to 576, any block size, any group.
+// Always writes PA_SCALAR_WAVES partials per work item.
+int LaunchPaScalar(const AtbmiPaShape &shape, const PaArgs &args, int numItems, hipStream_t stream);
+
+// MFMA kernel: head sizes and block sizes listed by PaMfmaSupports.
+bool PaMfmaSupports(const AtbmiPaShape &shape);
+int LaunchPaMfma(const AtbmiPaShape &shape, const PaArgs &args, int numItems, hipStream_t stream);
+
+// Merges the partials of every sequence that has more than one.
+int LaunchPaReduce(const AtbmiPaShape &shape, const PaArgs &args, int numSeqs, hipStream_t stream);
+
+} // namespace atbmi
+#endif

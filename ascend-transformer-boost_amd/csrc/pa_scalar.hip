@@ -1,0 +1,200 @@
+// Scalar (VALU) paged decode-attention kernel for gfx950.
+//
+// The fallback for shapes the MFMA kernel is not built for: any head size up
+// to 576, any block size, any GQA group. fp32 arithmetic throughout, in the
+// same order of operations as the reference golden (int8 rows are dequantised
+// as (q + offset) * scale in fp32; reference
+// tests/apitest/kernelstest/mix/test_paged_attention_common.py:85-108,229-276).
+//
+// One workgroup = one (work item, KV head, tile of up to 8 query heads).
+// Its four waves take tokens round-robin; a wave spreads the channels of one
+// K/V row over its 64 lanes (lane L owns channels L, L+64, ...), so a row is
+// read as consecutive 2- or 1-byte elements by consecutive lanes. Each wave
+// keeps its own online-softmax state and writes its own partial; the merge
+// kernel combines them.
+#include "pa_internal.h"
+
+namespace atbmi {
+namespace {
+
+constexpr int HT = PA_SCALAR_HEAD_TILE;
+
+__device__ __forceinline__ float WaveSum(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        v += __shfl_xor(v, off, WAVE);
+    }
+    return v;
+}
+
+// KV8 = true: int8 cache rows; false: 16-bit rows of the query's type.
+template <bool KV8, int EPL>
+__global__ __launch_bounds__(PA_SCALAR_WAVES * WAVE) void PaScalarKernel(const PaArgs a)
+{
+    const int g = blockIdx.x % a.G;
+    const int headTiles = (a.groupSize + HT - 1) / HT;
+    const int rest = blockIdx.x / a.G;
+    const int ht = rest % headTiles;
+    const PaWorkItem it = a.items[rest / headTiles];
+    const int wave = threadIdx.x / WAVE;
+    const int lane = threadIdx.x % WAVE;
+    const bool bf16 = a.qIsBf16 != 0;
+    const int h0 = g * a.groupSize + ht * HT;
+    const int nh = min(HT, a.groupSize - ht * HT);
+    constexpr float LOG2E = 1.4426950408889634f;
+    const float scale2 = a.qkScale * LOG2E;
+
+    float q[HT][EPL];
+#pragma unroll
+    for (int hh = 0; hh < HT; ++hh) {
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            const int d = lane + WAVE * e;
+            float v = 0.0f;
+            if (hh < nh && d < a.D) {
+                const int64_t idx = (static_cast<int64_t>(it.qRow) * a.H + h0 + hh) * a.D + d;
+                v = Load16(a.q, idx, bf16);
+                if (a.qScale != 0.0f) {
+                    // the reference pre-multiplies Q in its own dtype
+                    v *= a.qScale;
+                    v = bf16 ? Bf16ToFloat(FloatToBf16(v)) : HalfBitsToFloat(FloatToHalfBits(v));
+                }
+            }
+            q[hh][e] = v;
+        }
+    }
+
+    float kS[EPL], kO[EPL], vS[EPL], vO[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+        const int d = lane + WAVE * e;
+        kS[e] = 1.0f; kO[e] = 0.0f; vS[e] = 1.0f; vO[e] = 0.0f;
+        if (KV8) {
+            if (d < a.D) {
+                kS[e] = a.kScale[g * a.D + d];
+                kO[e] = a.kOff ? static_cast<float>(a.kOff[g * a.D + d]) : 0.0f;
+            }
+            if (d < a.Dv) {
+                vS[e] = a.vScale[g * a.Dv + d];
+                vO[e] = a.vOff ? static_cast<float>(a.vOff[g * a.Dv + d]) : 0.0f;
+            }
+        }
+    }
+
+    float m[HT], l[HT], acc[HT][EPL];
+#pragma unroll
+    for (int hh = 0; hh < HT; ++hh) {
+        m[hh] = -INFINITY;
+        l[hh] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            acc[hh][e] = 0.0f;
+        }
+    }
+
+    const int32_t *table = a.tables + static_cast<int64_t>(it.seq) * a.maxBlocksPerSeq;
+    for (int t = it.tokBegin + wave; t < it.tokEnd; t += PA_SCALAR_WAVES) {
+        const int64_t row = static_cast<int64_t>(table[t / a.blockSize]) * a.blockSize + (t % a.blockSize);
+        const int64_t kBase = row * a.kRowStride + static_cast<int64_t>(g) * a.D;
+        const int64_t vBase = row * a.vRowStride + static_cast<int64_t>(g) * a.vHeadStride;
+        float k[EPL], v[EPL];
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            const int d = lane + WAVE * e;
+            k[e] = 0.0f;
+            v[e] = 0.0f;
+            if (KV8) {
+                if (d < a.D) {
+                    k[e] = (static_cast<float>(reinterpret_cast<const int8_t *>(a.kc)[kBase + d]) + kO[e]) * kS[e];
+                }
+                if (d < a.Dv) {
+                    v[e] = (static_cast<float>(reinterpret_cast<const int8_t *>(a.vc)[vBase + d]) + vO[e]) * vS[e];
+                }
+            } else {
+                if (d < a.D) {
+                    k[e] = Load16(a.kc, kBase + d, bf16);
+                }
+                if (d < a.Dv) {
+                    v[e] = Load16(a.vc, vBase + d, bf16);
+                }
+            }
+        }
+#pragma unroll
+        for (int hh = 0; hh < HT; ++hh) {
+            if (hh < nh) {
+                float s = 0.0f;
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) {
+                    s += q[hh][e] * k[e];
+                }
+                s = WaveSum(s) * scale2;
+                const float mNew = fmaxf(m[hh], s);
+                const float corr = exp2f(m[hh] - mNew);
+                const float p = exp2f(s - mNew);
+                m[hh] = mNew;
+                l[hh] = l[hh] * corr + p;
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) {
+                    acc[hh][e] = acc[hh][e] * corr + p * v[e];
+                }
+            }
+        }
+    }
+
+    const int64_t part = static_cast<int64_t>(it.partialBase) + wave;
+#pragma unroll
+    for (int hh = 0; hh < HT; ++hh) {
+        if (hh < nh) {
+            const int64_t ph = part * a.H + h0 + hh;
+            const float inv = l[hh] > 0.0f ? 1.0f / l[hh] : 0.0f;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                const int d = lane + WAVE * e;
+                if (d < a.Dv) {
+                    a.partO[ph * a.Dv + d] = acc[hh][e] * inv;
+                }
+            }
+            if (lane == 0) {
+                a.partLse[ph] = l[hh] > 0.0f ? m[hh] + log2f(l[hh]) : -INFINITY;
+            }
+        }
+    }
+}
+
+template <bool KV8>
+int LaunchScalarByWidth(const AtbmiPaShape &shape, const PaArgs &args, unsigned grid, hipStream_t stream)
+{
+    const int width = shape.headDimK > shape.headDimV ? shape.headDimK : shape.headDimV;
+    constexpr int threads = PA_SCALAR_WAVES * WAVE;
+    if (width <= 64) {
+        PaScalarKernel<KV8, 1><<<grid, threads, 0, stream>>>(args);
+    } else if (width <= 128) {
+        PaScalarKernel<KV8, 2><<<grid, threads, 0, stream>>>(args);
+    } else if (width <= 256) {
+        PaScalarKernel<KV8, 4><<<grid, threads, 0, stream>>>(args);
+    } else if (width <= 576) {
+        PaScalarKernel<KV8, 9><<<grid, threads, 0, stream>>>(args);
+    } else {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: head size %d exceeds 576", width);
+    }
+    ATBMI_HIP_CHECK(hipGetLastError());
+    return OK;
+}
+
+} // namespace
+
+int LaunchPaScalar(const AtbmiPaShape &shape, const PaArgs &args, int numItems, hipStream_t stream)
+{
+    const int headTiles = (args.groupSize + HT - 1) / HT;
+    const int64_t grid = static_cast<int64_t>(numItems) * headTiles * args.G;
+    if (grid <= 0 || grid > 0x7fffffffLL) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: grid of %lld workgroups is out of range", (long long)grid);
+    }
+    if (shape.kvDtype == ATBMI_INT8) {
+        return LaunchScalarByWidth<true>(shape, args, static_cast<unsigned>(grid), stream);
+    }
+    return LaunchScalarByWidth<false>(shape, args, static_cast<unsigned>(grid), stream);
+}
+
+} // namespace atbmi

@@ -1,0 +1,502 @@
+// PagedAttentionOperation on MI355X: the decode-attention operator of ATB.
+//
+// Creation-time parameter checks, tensor counts, InferShape and the dim
+// checks follow the reference operator for its Atlas 800I A2 (910B) feature
+// set (reference src/ops/ops_infer/paged_attention/paged_attention_operation.cpp:
+// 53-70 common, 92-143 create, 145-365 per-feature checks, 408-472 counts and
+// InferShape, 561-632 cache dim rules, 663-695 and 926-963 setup dim checks);
+// the second validation layer of the reference kernel library is restated in
+// PlanImpl (src/kernels/mixkernels/pagedattention/paged_attention_operation.cpp:159-210,
+// 284-340, 446-495 and tiling/paged_attention_tiling.cpp:156-192,357-358).
+// Context lengths are read from contextLens.hostData during Setup, as the
+// reference runner does (src/ops/ops_infer/paged_attention/param.cpp:16-62).
+//
+// Implemented feature set: fp16/bf16 caches, int8 caches with fp32 per-channel
+// descale (+ int32 offset), and the MLA combined cache (mlaVHeadSize > 0).
+// Masks, dynamic batch status, LogN scale, speculative (multi-token) queries,
+// head compression, BNSD layout, int8 queries and int64-packed descales are
+// legal in the reference but not implemented here; such params are rejected
+// at creation with ERROR_INVALID_PARAM.
+#include <cmath>
+#include <new>
+#include "atb/infer_op_params.h"
+#include "atb/utils.h"
+#include "atbmi_kernels.h"
+#include "log.h"
+#include "operation_base.h"
+
+namespace atb {
+namespace {
+using Param = infer::PagedAttentionParam;
+
+constexpr int64_t MAX_HEAD_SIZE = 576;
+constexpr int64_t MLA_THRESHOLD = 256;
+constexpr int64_t BLOCK_LIMIT = 128 * 128;
+constexpr int64_t MAX_MLA_BATCH = 8192;
+
+// Reference paged_attention_operation.cpp:53-70.
+bool CommonParamCheck(const Param &p)
+{
+    if (p.headNum <= 0) {
+        ATB_LOG(ERROR) << "headNum should be greater than zero";
+        return false;
+    }
+    if (p.kvHeadNum < 0) {
+        ATB_LOG(ERROR) << "kvHeadNum should be no less than zero";
+        return false;
+    }
+    if (p.kvHeadNum != 0 && p.headNum % p.kvHeadNum != 0) {
+        ATB_LOG(ERROR) << "headNum mod kvHeadNum should be zero";
+        return false;
+    }
+    return true;
+}
+
+// The cross-feature rules of the reference (:145-365), in its order.
+bool FeatureParamCheck(const Param &p)
+{
+    if (p.maskType == Param::MASK_TYPE_NORM_COMPRESS) {
+        ATB_LOG(ERROR) << "MASK_TYPE_NORM_COMPRESS is an Atlas 300I Duo feature";
+        return false;
+    }
+    if (p.compressType >= Param::COMPRESS_TYPE_MAX || p.compressType < Param::COMPRESS_TYPE_UNDEFINED) {
+        ATB_LOG(ERROR) << "compressType out of range";
+        return false;
+    }
+    if (p.compressType == Param::COMPRESS_TYPE_KVHEAD_ROPE &&
+        (p.maskType != Param::UNDEFINED || p.batchRunStatusEnable)) {
+        ATB_LOG(ERROR) << "COMPRESS_TYPE_KVHEAD_ROPE needs maskType UNDEFINED and no dynamic batch";
+        return false;
+    }
+    if (p.calcType != Param::CALC_TYPE_UNDEFINED) {
+        if (p.batchRunStatusEnable || p.compressType != Param::COMPRESS_TYPE_UNDEFINED) {
+            ATB_LOG(ERROR) << "SPEC does not support dynamic batch or head compression";
+            return false;
+        }
+        if (p.mlaVHeadSize == 0 && p.maskType != Param::MASK_TYPE_NORM && p.maskType != Param::MASK_TYPE_SPEC) {
+            ATB_LOG(ERROR) << "SPEC only supports norm mask and spec mask";
+            return false;
+        }
+    }
+    if (p.quantType == Param::TYPE_DEQUANT_FUSION && p.calcType != Param::CALC_TYPE_UNDEFINED) {
+        ATB_LOG(ERROR) << "dequant fusion needs calcType CALC_TYPE_UNDEFINED";
+        return false;
+    }
+    if (p.quantType == Param::TYPE_QUANT_QKV_OFFLINE || p.quantType == Param::TYPE_QUANT_QKV_ONLINE) {
+        if ((p.outDataType != ACL_FLOAT16 && p.outDataType != ACL_BF16) || p.hasQuantOffset ||
+            p.compressType != Param::COMPRESS_TYPE_UNDEFINED || p.calcType != Param::CALC_TYPE_UNDEFINED) {
+            ATB_LOG(ERROR) << "QKV quant: outDataType fp16/bf16, no offset, no compress, no SPEC";
+            return false;
+        }
+    }
+    if (p.scaleType >= Param::SCALE_TYPE_MAX || p.scaleType < Param::SCALE_TYPE_TOR) {
+        ATB_LOG(ERROR) << "scaleType out of range";
+        return false;
+    }
+    if (p.scaleType == Param::SCALE_TYPE_LOGN &&
+        (p.quantType != Param::TYPE_QUANT_UNQUANT || p.calcType != Param::CALC_TYPE_UNDEFINED ||
+         p.compressType != Param::COMPRESS_TYPE_UNDEFINED)) {
+        ATB_LOG(ERROR) << "logN does not combine with quant, SPEC or head compression";
+        return false;
+    }
+    if (p.inputLayout == infer::TYPE_BNSD &&
+        (p.calcType == Param::CALC_TYPE_SPEC || p.compressType != Param::COMPRESS_TYPE_UNDEFINED ||
+         p.quantType != Param::TYPE_QUANT_UNQUANT || p.scaleType != Param::SCALE_TYPE_TOR)) {
+        ATB_LOG(ERROR) << "BNSD does not combine with SPEC, compress, quant or logN";
+        return false;
+    }
+    if (p.mlaVHeadSize > 0) {
+        if (p.maskType == Param::MASK_TYPE_ALIBI) {
+            ATB_LOG(ERROR) << "mla mode does not support alibi mask";
+            return false;
+        }
+        if (p.calcType == Param::CALC_TYPE_SPEC &&
+            (p.maskType == Param::MASK_TYPE_NORM || p.quantType != Param::TYPE_QUANT_UNQUANT ||
+             p.batchRunStatusEnable)) {
+            ATB_LOG(ERROR) << "mla SPEC does not support norm mask, quant or dynamic batch";
+            return false;
+        }
+        if (p.compressType != Param::COMPRESS_TYPE_UNDEFINED || p.quantType == Param::TYPE_DEQUANT_FUSION ||
+            p.scaleType != Param::SCALE_TYPE_TOR || p.inputLayout != infer::TYPE_BSND) {
+            ATB_LOG(ERROR) << "mla mode does not support compress, dequant fusion, logN or BNSD";
+            return false;
+        }
+        if (p.kvHeadNum != 1) {
+            ATB_LOG(ERROR) << "kvHeadNum should be 1, mla mode only supports MQA";
+            return false;
+        }
+        if (p.mlaVHeadSize > MAX_HEAD_SIZE) {
+            ATB_LOG(ERROR) << "mlaVHeadSize should be no greater than 576";
+            return false;
+        }
+    }
+    return true;
+}
+
+// Features that are legal in the reference but have no MI355X kernel yet.
+bool ImplementedCheck(const Param &p)
+{
+    const char *what = nullptr;
+    if (p.maskType != Param::UNDEFINED) {
+        what = "attention masks";
+    } else if (p.batchRunStatusEnable) {
+        what = "batchRunStatus";
+    } else if (p.compressType != Param::COMPRESS_TYPE_UNDEFINED) {
+        what = "head compression";
+    } else if (p.calcType != Param::CALC_TYPE_UNDEFINED) {
+        what = "speculative (multi-token) queries";
+    } else if (p.scaleType != Param::SCALE_TYPE_TOR) {
+        what = "LogN scaling";
+    } else if (p.inputLayout != infer::TYPE_BSND) {
+        what = "BNSD layout";
+    } else if (p.quantType == Param::TYPE_QUANT_QKV_OFFLINE || p.quantType == Param::TYPE_QUANT_QKV_ONLINE) {
+        what = "int8 query quantisation";
+    } else if (p.quantType != Param::TYPE_QUANT_UNQUANT && p.quantType != Param::TYPE_DEQUANT_FUSION) {
+        what = "this quantType";
+    }
+    if (what) {
+        ATB_LOG(ERROR) << "PagedAttention: " << what << " not implemented on MI355X";
+        return false;
+    }
+    return true;
+}
+
+OpIr MakeIr(const Param &p)
+{
+    OpIr ir;
+    const aclFormat nd = ACL_FORMAT_ND;
+    for (aclDataType q : {ACL_FLOAT16, ACL_BF16}) {
+        IrCombo c;
+        if (p.mlaVHeadSize > 0) {
+            c.inDtypes = {q, q, ACL_INT32, ACL_INT32};
+        } else if (p.quantType == Param::TYPE_DEQUANT_FUSION) {
+            c.inDtypes = {q, ACL_INT8, ACL_INT8, ACL_INT32, ACL_INT32, ACL_FLOAT};
+            if (p.hasQuantOffset) {
+                c.inDtypes.push_back(ACL_INT32);
+            }
+            c.inDtypes.push_back(ACL_FLOAT);
+            if (p.hasQuantOffset) {
+                c.inDtypes.push_back(ACL_INT32);
+            }
+        } else {
+            c.inDtypes = {q, q, q, ACL_INT32, ACL_INT32};
+        }
+        c.inFormats.assign(c.inDtypes.size(), nd);
+        c.outDtypes = {q};
+        c.outFormats = {nd};
+        ir.push_back(c);
+    }
+    return ir;
+}
+
+class PagedAttentionOperation : public OperationBase {
+public:
+    explicit PagedAttentionOperation(const Param &param)
+        : OperationBase("PagedAttentionOperation"), param_(param), mla_(param.mlaVHeadSize > 0),
+          dequant_(param.quantType == Param::TYPE_DEQUANT_FUSION), irTable_(MakeIr(param))
+    {
+        ir_ = &irTable_;
+        tablesIdx_ = mla_ ? 2 : 3;
+        lensIdx_ = mla_ ? 3 : 4;
+    }
+
+    ~PagedAttentionOperation() override
+    {
+        if (plan_) {
+            atbmi_pa_plan_destroy(plan_);
+        }
+    }
+
+    uint32_t GetInputNum() const override
+    {
+        uint32_t n = 5;
+        if (dequant_) {
+            n += param_.hasQuantOffset ? 4 : 2;
+        }
+        if (mla_) {
+            n -= 1;
+        }
+        return n;
+    }
+    uint32_t GetOutputNum() const override { return 1; }
+
+protected:
+    Status InferShapeImpl(const SVector<TensorDesc> &in, SVector<TensorDesc> &out) const override
+    {
+        out.at(0) = in.at(0);
+        const int64_t dv = mla_ ? static_cast<int64_t>(param_.mlaVHeadSize)
+                                : in.at(2).shape.dims[in.at(2).shape.dimNum - 1];
+        out.at(0).shape.dims[out.at(0).shape.dimNum - 1] = dv;
+        return NO_ERROR;
+    }
+
+    // Reference :697-726 (InferShapeDimCheck) + :634-661 (KVCacheDimCheck).
+    Status InferShapeCheckImpl(const SVector<TensorDesc> &in) const override
+    {
+        if (!mla_ && in.at(2).shape.dimNum != 4) {
+            ATB_LOG(ERROR) << "valueCache should have 4 dims";
+            return ERROR_INVALID_TENSOR_DIM_NUM;
+        }
+        if (in.at(0).shape.dimNum != 3 || in.at(1).shape.dimNum != 4 || in.at(tablesIdx_).shape.dimNum != 2 ||
+            in.at(lensIdx_).shape.dimNum != 1) {
+            ATB_LOG(ERROR) << "expected dims: query 3, keyCache 4, blockTables 2, contextLens 1";
+            return ERROR_INVALID_TENSOR_DIM_NUM;
+        }
+        const Dims &kc = in.at(1).shape;
+        if (!mla_) {
+            const Dims &vc = in.at(2).shape;
+            if (kc.dims[0] != vc.dims[0] || kc.dims[1] != vc.dims[1] || kc.dims[2] != vc.dims[2]) {
+                ATB_LOG(ERROR) << "keyCache and valueCache must agree on numBlocks, blockSize and heads";
+                return ERROR_INVALID_TENSOR_DIM;
+            }
+        }
+        return CacheDimCheck(in);
+    }
+
+    // Reference :492-525 (SetupCheckImpl) + :926-963 (SetupDimCheck) + :856-877 (BlockDimCheck).
+    Status SetupCheckImpl(const SVector<Tensor> &inTensors, const SVector<Tensor> &outTensors) const override
+    {
+        if (inTensors.at(1).desc.shape.dimNum != 4) {
+            ATB_LOG(ERROR) << "keyCache should have 4 dims";
+            return ERROR_INVALID_TENSOR_DIM_NUM;
+        }
+        SVector<TensorDesc> in;
+        for (size_t i = 0; i < inTensors.size(); ++i) {
+            in.push_back(inTensors.at(i).desc);
+        }
+        Status st = InferShapeCheckImpl(in);
+        if (st != NO_ERROR) {
+            return st;
+        }
+        const Dims &out = outTensors.at(0).desc.shape;
+        const int64_t dv = mla_ ? static_cast<int64_t>(param_.mlaVHeadSize) : in.at(2).shape.dims[3];
+        if (out.dimNum < 3 || out.dims[2] != dv) {
+            ATB_LOG(ERROR) << "head size of the output should be " << dv;
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (in.at(0).shape.dims[1] != out.dims[1]) {
+            ATB_LOG(ERROR) << "query and output must have the same head count";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        return NO_ERROR;
+    }
+
+    Status PlanImpl(const VariantPack &pack, uint64_t &workspaceSize) override
+    {
+        const Tensor &q = pack.inTensors.at(0);
+        const Tensor &kc = pack.inTensors.at(1);
+        const Tensor &tables = pack.inTensors.at(tablesIdx_);
+        const Tensor &lens = pack.inTensors.at(lensIdx_);
+        const Tensor &out = pack.outTensors.at(0);
+        if (!lens.hostData) {
+            ATB_LOG(ERROR) << "contextLens.hostData is null; the lengths are read on the host during Setup";
+            return ERROR_INVALID_PARAM;
+        }
+        const int64_t kvHeads = param_.kvHeadNum > 0 ? param_.kvHeadNum : param_.headNum;
+        const int64_t d = kc.desc.shape.dims[3];
+        const int64_t dv = mla_ ? static_cast<int64_t>(param_.mlaVHeadSize) : pack.inTensors.at(2).desc.shape.dims[3];
+        const int64_t blockSize = kc.desc.shape.dims[1];
+        // Kernel-library level checks of the reference.
+        if (q.desc.shape.dims[1] != param_.headNum) {
+            ATB_LOG(ERROR) << "query head count " << q.desc.shape.dims[1] << " != headNum " << param_.headNum;
+            return ERROR_INVALID_PARAM;
+        }
+        if (kc.desc.shape.dims[2] != kvHeads) {
+            ATB_LOG(ERROR) << "cache head count " << kc.desc.shape.dims[2] << " != kvHeadNum " << kvHeads;
+            return ERROR_INVALID_PARAM;
+        }
+        if (blockSize % 16 != 0) {
+            ATB_LOG(ERROR) << "blockSize must be a multiple of 16";
+            return ERROR_INVALID_PARAM;
+        }
+        if (d > MLA_THRESHOLD || dv > MLA_THRESHOLD) {
+            if (blockSize > 128) {
+                ATB_LOG(ERROR) << "blockSize should not exceed 128 when a head size exceeds 256";
+                return ERROR_INVALID_PARAM;
+            }
+        } else if (d == MLA_THRESHOLD && dv == MLA_THRESHOLD && blockSize >= 128) {
+            if (blockSize % 128 != 0) {
+                ATB_LOG(ERROR) << "head size 256 needs a 128-aligned blockSize";
+                return ERROR_INVALID_PARAM;
+            }
+        } else if (d == dv && d * blockSize > BLOCK_LIMIT) {
+            ATB_LOG(ERROR) << "headSize * blockSize should not exceed 128 * 128";
+            return ERROR_INVALID_PARAM;
+        }
+        if (tables.desc.shape.dims[0] < lens.desc.shape.dims[0]) {
+            ATB_LOG(ERROR) << "blockTables has fewer rows than contextLens";
+            return ERROR_INVALID_PARAM;
+        }
+        if (out.desc.shape.dims[0] != q.desc.shape.dims[0]) {
+            ATB_LOG(ERROR) << "output and query must have the same token count";
+            return ERROR_INVALID_PARAM;
+        }
+        if (dequant_) {
+            const size_t kScaleIdx = 5;
+            const size_t vScaleIdx = param_.hasQuantOffset ? 7 : 6;
+            const int64_t kLen = kvHeads * d;
+            const int64_t vLen = kvHeads * dv;
+            if (pack.inTensors.at(kScaleIdx).desc.shape.dims[0] != kLen ||
+                pack.inTensors.at(vScaleIdx).desc.shape.dims[0] != vLen) {
+                ATB_LOG(ERROR) << "descale vectors must have kvHeadNum * headSize elements";
+                return ERROR_INVALID_PARAM;
+            }
+            if (param_.hasQuantOffset && (pack.inTensors.at(6).desc.shape.dims[0] != kLen ||
+                                          pack.inTensors.at(8).desc.shape.dims[0] != vLen)) {
+                ATB_LOG(ERROR) << "offset vectors must have kvHeadNum * headSize elements";
+                return ERROR_INVALID_PARAM;
+            }
+        }
+
+        AtbmiPaShape shape{};
+        shape.qDtype = q.desc.dtype == ACL_BF16 ? ATBMI_BF16 : ATBMI_F16;
+        shape.kvDtype = kc.desc.dtype == ACL_INT8 ? ATBMI_INT8 : shape.qDtype;
+        shape.numHeads = param_.headNum;
+        shape.numKvHeads = static_cast<int32_t>(kvHeads);
+        shape.headDimK = static_cast<int32_t>(d);
+        shape.headDimV = static_cast<int32_t>(dv);
+        shape.blockSize = static_cast<int32_t>(blockSize);
+        shape.numBlocks = static_cast<int32_t>(kc.desc.shape.dims[0]);
+        shape.maxBlocksPerSeq = static_cast<int32_t>(tables.desc.shape.dims[1]);
+        shape.numQueryRows = static_cast<int32_t>(q.desc.shape.dims[0]);
+        shape.mlaCombined = mla_ ? 1 : 0;
+        shape.hasOffset = (dequant_ && param_.hasQuantOffset) ? 1 : 0;
+        shape.kernel = ATBMI_PA_KERNEL_AUTO;
+        shape.qkScale = param_.qkScale;
+        shape.qScale = param_.qScale;
+        if (!plan_ || !SameShape(shape, planShape_)) {
+            if (plan_) {
+                atbmi_pa_plan_destroy(plan_);
+                plan_ = nullptr;
+            }
+            int rc = atbmi_pa_plan_create(&shape, &plan_);
+            if (rc != 0) {
+                ATB_LOG(ERROR) << "PagedAttention plan: " << atbmi_last_error();
+                return rc;
+            }
+            planShape_ = shape;
+        }
+        // Lengths are re-read on every Setup, like the reference runner does.
+        int rc = atbmi_pa_plan_update(plan_, static_cast<const int32_t *>(lens.hostData),
+                                      static_cast<int32_t>(lens.desc.shape.dims[0]));
+        if (rc != 0) {
+            ATB_LOG(ERROR) << "PagedAttention plan: " << atbmi_last_error();
+            return rc;
+        }
+        workspaceSize = atbmi_pa_plan_workspace_size(plan_);
+        return NO_ERROR;
+    }
+
+    Status LaunchImpl(const VariantPack &pack, uint8_t *workspace, uint64_t workspaceSize,
+                      aclrtStream stream) override
+    {
+        AtbmiPaTensors t{};
+        t.query = pack.inTensors.at(0).deviceData;
+        t.keyCache = pack.inTensors.at(1).deviceData;
+        t.valueCache = mla_ ? nullptr : pack.inTensors.at(2).deviceData;
+        t.blockTables = static_cast<const int32_t *>(pack.inTensors.at(tablesIdx_).deviceData);
+        if (dequant_) {
+            size_t i = 5;
+            t.kScale = static_cast<const float *>(pack.inTensors.at(i++).deviceData);
+            if (param_.hasQuantOffset) {
+                t.kOffset = static_cast<const int32_t *>(pack.inTensors.at(i++).deviceData);
+            }
+            t.vScale = static_cast<const float *>(pack.inTensors.at(i++).deviceData);
+            if (param_.hasQuantOffset) {
+                t.vOffset = static_cast<const int32_t *>(pack.inTensors.at(i++).deviceData);
+            }
+        }
+        t.out = pack.outTensors.at(0).deviceData;
+        int rc = atbmi_pa_decode(plan_, &t, workspace, workspaceSize, stream);
+        if (rc != 0) {
+            ATB_LOG(ERROR) << "PagedAttention launch failed: " << atbmi_last_error();
+        }
+        return rc;
+    }
+
+private:
+    static bool SameShape(const AtbmiPaShape &a, const AtbmiPaShape &b)
+    {
+        return a.qDtype == b.qDtype && a.kvDtype == b.kvDtype && a.numHeads == b.numHeads &&
+               a.numKvHeads == b.numKvHeads && a.headDimK == b.headDimK && a.headDimV == b.headDimV &&
+               a.blockSize == b.blockSize && a.numBlocks == b.numBlocks && a.maxBlocksPerSeq == b.maxBlocksPerSeq &&
+               a.numQueryRows == b.numQueryRows && a.mlaCombined == b.mlaCombined && a.hasOffset == b.hasOffset &&
+               a.qkScale == b.qkScale && a.qScale == b.qScale;
+    }
+
+    // Reference :585-632 (KVCacheDimCheck910B) with :561-572 (IsInMLAIncompatible).
+    Status CacheDimCheck(const SVector<TensorDesc> &in) const
+    {
+        const int64_t d = in.at(1).shape.dims[3];
+        if (d != in.at(0).shape.dims[2]) {
+            ATB_LOG(ERROR) << "headSize of keyCache and query should be same";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        const int64_t blockSize = in.at(1).shape.dims[1];
+        if (dequant_) {
+            // strict regime: features that predate the split K/V head sizes
+            if (d != in.at(2).shape.dims[3]) {
+                ATB_LOG(ERROR) << "headSize of keyCache and valueCache should be same";
+                return ERROR_INVALID_TENSOR_DIM;
+            }
+            if (d > 256 || d * blockSize > BLOCK_LIMIT) {
+                ATB_LOG(ERROR) << "headSize should be <= 256 and blockSize * headSize <= 128 * 128";
+                return ERROR_INVALID_TENSOR_DIM;
+            }
+            return NO_ERROR;
+        }
+        if (static_cast<int64_t>(param_.mlaVHeadSize) > d) {
+            ATB_LOG(ERROR) << "mlaVHeadSize should be no greater than headSizeK";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        const int64_t dv = mla_ ? static_cast<int64_t>(param_.mlaVHeadSize) : in.at(2).shape.dims[3];
+        if (d > MAX_HEAD_SIZE || dv > MAX_HEAD_SIZE) {
+            ATB_LOG(ERROR) << "head sizes should be no greater than 576";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (mla_ && in.at(lensIdx_).shape.dims[0] > MAX_MLA_BATCH) {
+            ATB_LOG(ERROR) << "batch should be <= 8192 in mla mode";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        const bool blockSize256 = mla_ && blockSize == 256 && param_.kvHeadNum == 1 &&
+                                  (param_.headNum == 16 || param_.headNum == 32) && d == 576 && dv == 512;
+        if (blockSize256) {
+            return NO_ERROR;
+        }
+        if ((d > 256 || dv > 256) && blockSize > 128) {
+            ATB_LOG(ERROR) << "blockSize should be no greater than 128 if a head size exceeds 256";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        return NO_ERROR;
+    }
+
+    Param param_;
+    bool mla_;
+    bool dequant_;
+    OpIr irTable_;
+    size_t tablesIdx_ = 3;
+    size_t lensIdx_ = 4;
+    AtbmiPaPlan *plan_ = nullptr;
+    AtbmiPaShape planShape_{};
+};
+} // namespace
+
+template <> Status CreateOperation(const infer::PagedAttentionParam &opParam, Operation **operation)
+{
+    if (operation == nullptr) {
+        return ERROR_INVALID_PARAM;
+    }
+    if (!ReservedIsZero(opParam)) {
+        ATB_LOG(ERROR) << "PagedAttentionParam rsv has a non-zero byte";
+        return ERROR_INVALID_PARAM;
+    }
+    if (!CommonParamCheck(opParam) || !FeatureParamCheck(opParam) || !ImplementedCheck(opParam)) {
+        return ERROR_INVALID_PARAM;
+    }
+    *operation = new (std::nothrow) PagedAttentionOperation(opParam);
+    if (*operation == nullptr) {
+        return ERROR_OUT_OF_HOST_MEMORY;
+    }
+    return NO_ERROR;
+}
+} // namespace atb

@@ -1,0 +1,146 @@
+"""Seeded synthetic decode-step workloads (the five benchmark configurations).
+
+Each workload is one decode step: new K/V rows for every sequence, the paged
+caches, block tables, context lengths (the new token is the last position),
+slot mapping and the query. Lengths, tables and slots come from a numpy
+PCG64 generator (seed 1000 + config number) so they are identical everywhere;
+tensor contents come from a torch generator on the target device with the
+same seed.
+"""
+import math
+
+import numpy as np
+
+CONFIGS = {
+    # name: batch, heads, kv_heads, d, dv, block, ctx range, dtype, kv dtype, distribution, value scale
+    "c1": dict(batch=4, heads=8, kv_heads=8, d=128, dv=128, block=128, ctx=(64, 512), dtype="float16",
+               kv="float16", dist="uniform", std=1.0, pool=64),
+    "c2": dict(batch=64, heads=32, kv_heads=8, d=128, dv=128, block=128, ctx=(1024, 4096), dtype="bf16",
+               kv="bf16", dist="uniform", std=0.5, pool=None),
+    "c2_fp16": dict(batch=64, heads=32, kv_heads=8, d=128, dv=128, block=128, ctx=(1024, 4096), dtype="float16",
+                    kv="float16", dist="uniform", std=0.5, pool=None),
+    "c3": dict(batch=128, heads=64, kv_heads=8, d=128, dv=128, block=128, ctx=(2048, 8192), dtype="float16",
+               kv="int8", dist="uniform", std=1.0, pool=None),
+    "c4": dict(batch=16, heads=32, kv_heads=8, d=128, dv=128, block=128, ctx=(256, 32768), dtype="float16",
+               kv="float16", dist="lognormal", std=1.0, pool=None),
+    "c5": dict(batch=64, heads=128, kv_heads=1, d=576, dv=512, block=128, ctx=(2048, 4096), dtype="bf16",
+               kv="bf16", dist="uniform", std=0.3, pool=None, mla=True),
+}
+SEEDS = {"c1": 1001, "c2": 1002, "c2_fp16": 1002, "c3": 1003, "c4": 1004, "c5": 1005}
+
+
+def config(name, **overrides):
+    cfg = dict(CONFIGS[name])
+    cfg["name"] = name
+    cfg.setdefault("mla", False)
+    cfg.update(overrides)
+    return cfg
+
+
+def qk_scale(cfg):
+    # DeepSeek-V3 MLA scales by the un-absorbed head size (128 nope + 64 rope).
+    return 1.0 / math.sqrt(192.0) if cfg.get("mla") else 1.0 / math.sqrt(cfg["d"])
+
+
+def draw_lengths(cfg, rng):
+    lo, hi = cfg["ctx"]
+    b = cfg["batch"]
+    if cfg["dist"] == "lognormal":
+        # median 8192, sigma 1.0, clipped to the configured range
+        x = np.exp(rng.normal(math.log(8192.0), 1.0, size=b))
+        return np.clip(np.rint(x), lo, hi).astype(np.int32)
+    return rng.integers(lo, hi + 1, size=b, dtype=np.int64).astype(np.int32)
+
+
+def layout(cfg, seed=None):
+    """Host-side structure of a step: lengths, block tables, slot mapping."""
+    rng = np.random.Generator(np.random.PCG64(SEEDS.get(cfg["name"], 1) if seed is None else seed))
+    ctx = draw_lengths(cfg, rng)
+    bs = cfg["block"]
+    blocks_per_seq = (ctx.astype(np.int64) + bs - 1) // bs
+    total = int(blocks_per_seq.sum())
+    pool = cfg["pool"] if cfg.get("pool") else int(math.ceil(total * 1.1))
+    max_blocks = int(blocks_per_seq.max())
+    perm = rng.permutation(pool)[:total]  # drawn without replacement: every block has one owner
+    tables = np.zeros((cfg["batch"], max_blocks), dtype=np.int32)
+    pos = 0
+    for b in range(cfg["batch"]):
+        n = int(blocks_per_seq[b])
+        tables[b, :n] = perm[pos:pos + n]
+        tables[b, n:] = perm[pos]  # unused entries stay valid block ids
+        pos += n
+    last = ctx.astype(np.int64) - 1
+    slots = (tables[np.arange(cfg["batch"]), last // bs].astype(np.int64) * bs + last % bs).astype(np.int32)
+    return dict(ctx=ctx, tables=tables, slots=slots, pool=pool, max_blocks=max_blocks)
+
+
+def torch_dtype(name):
+    import torch
+    return {"float16": torch.float16, "bf16": torch.bfloat16, "int8": torch.int8}[name]
+
+
+def make_step(cfg, device, seed=None):
+    """Tensors of one decode step on `device` (torch). Returns a dict:
+    q, k_new, v_new (query dtype), key_cache, value_cache (kv dtype; value_cache
+    is None for MLA), k_scale/v_scale (fp32, int8 caches only), block_tables,
+    slot_mapping (int32, device), context_lens (int32, CPU) and cfg/layout."""
+    import torch
+    lay = layout(cfg, seed)
+    gen = torch.Generator(device=device)
+    gen.manual_seed(SEEDS.get(cfg["name"], 1) if seed is None else seed)
+    qdt = torch_dtype(cfg["dtype"])
+    b, h, g, d, dv, bs = cfg["batch"], cfg["heads"], cfg["kv_heads"], cfg["d"], cfg["dv"], cfg["block"]
+    pool = lay["pool"]
+    std = cfg["std"]
+
+    def normal(shape, s):
+        return torch.randn(shape, generator=gen, device=device, dtype=torch.float32) * s
+
+    out = dict(cfg=cfg, layout=lay)
+    out["q"] = normal((b, h, d), 1.0 if cfg["kv"] == "int8" else std).to(qdt)
+    if cfg["kv"] == "int8":
+        out["k_scale"] = torch.rand((g * d,), generator=gen, device=device) * 0.015 + 0.005
+        out["v_scale"] = torch.rand((g * dv,), generator=gen, device=device) * 0.015 + 0.005
+        out["key_cache"] = torch.randint(-127, 128, (pool, bs, g, d), generator=gen, device=device,
+                                         dtype=torch.int8)
+        out["value_cache"] = torch.randint(-127, 128, (pool, bs, g, dv), generator=gen, device=device,
+                                           dtype=torch.int8)
+        out["k_new"] = normal((b, g, d), 0.5).to(qdt)
+        out["v_new"] = normal((b, g, dv), 0.5).to(qdt)
+    else:
+        # generated block-wise so the fp32 staging buffer stays small
+        kc = torch.empty((pool, bs, g, d), device=device, dtype=qdt)
+        step = max(1, (1 << 26) // (bs * g * d))
+        for i in range(0, pool, step):
+            n = min(step, pool - i)
+            kc[i:i + n] = normal((n, bs, g, d), std).to(qdt)
+        out["key_cache"] = kc
+        if cfg.get("mla"):
+            out["value_cache"] = None
+        else:
+            vc = torch.empty((pool, bs, g, dv), device=device, dtype=qdt)
+            for i in range(0, pool, step):
+                n = min(step, pool - i)
+                vc[i:i + n] = normal((n, bs, g, dv), std).to(qdt)
+            out["value_cache"] = vc
+        out["k_new"] = normal((b, g, d), std).to(qdt)
+        out["v_new"] = None if cfg.get("mla") else normal((b, g, dv), std).to(qdt)
+    out["block_tables"] = torch.from_numpy(lay["tables"]).to(device)
+    out["slot_mapping"] = torch.from_numpy(lay["slots"]).to(device)
+    out["context_lens"] = torch.from_numpy(lay["ctx"].copy())
+    return out
+
+
+def algorithmic_bytes(cfg, ctx):
+    """HBM bytes a decode-attention call must move: valid K/V rows + q + out +
+    block-table entries + context lengths (+ scale vectors for an int8 cache)."""
+    kv = 1 if cfg["kv"] == "int8" else 2
+    g, d, dv, h, bs = cfg["kv_heads"], cfg["d"], cfg["dv"], cfg["heads"], cfg["block"]
+    ctx = np.asarray(ctx, dtype=np.int64)
+    per_tok = g * (d if cfg.get("mla") else d + dv) * kv
+    rows = int((ctx > 0).sum())
+    total = int(ctx.sum()) * per_tok + rows * h * (d + dv) * 2
+    total += int(((ctx + bs - 1) // bs).sum()) * 4 + len(ctx) * 4
+    if cfg["kv"] == "int8":
+        total += g * (d + dv) * 4
+    return total

@@ -1,0 +1,109 @@
+// Parameter structs of the two inference operators this library implements:
+// ReshapeAndCache (KV-cache write) and PagedAttention (decode attention over
+// a block-table-addressed KV cache). Field order, enumerator values and sizes
+// follow the reference so that a param filled by existing code is read the
+// same way (reference include/atb/infer_op_params.h:39-42, :488-526,
+// :1859-1963; sizes pinned by tests/unittest/ops/test_op_param_size.cpp:47,51).
+#ifndef ATB_INFER_OP_PARAMS_H
+#define ATB_INFER_OP_PARAMS_H
+#include <cstdint>
+#include <acl/acl.h>
+#include "atb/svector.h"
+
+namespace atb {
+namespace infer {
+
+enum InputLayout : int {
+    TYPE_BSND = 0, // [tokens, heads, head_dim] queries, [blocks, block, heads, dim] caches
+    TYPE_BNSD      // head-major caches; not implemented on MI355X
+};
+
+// Writes one K row and one V row per token into the paged caches at the
+// slot the slot mapping names; negative slots are skipped.
+struct ReshapeAndCacheParam {
+    enum CompressType : int {
+        COMPRESS_TYPE_UNDEFINED = 0,
+        COMPRESS_TYPE_KVHEAD,     // head compression (alibi); not implemented on MI355X
+        COMPRESS_TYPE_KVHEAD_ROPE // head compression (rope); not implemented on MI355X
+    };
+    enum KvCacheCfg : int {
+        K_CACHE_V_CACHE = 0, // inputs: key, value, keyCache, valueCache, slotMapping
+        K_CACHE_V_BYPASS,    // inputs: key, keyCache, slotMapping (single cache, e.g. MLA latent)
+        K_CACHE_V_CACHE_NZ   // fractal-NZ caches; not implemented on MI355X
+    };
+
+    CompressType compressType = COMPRESS_TYPE_UNDEFINED;
+    KvCacheCfg kvCacheCfg = K_CACHE_V_CACHE;
+    uint8_t rsv[16] = {0}; // must stay zero
+};
+
+// Decode attention: one query token per sequence against that sequence's
+// cached keys/values, found through blockTables and bounded by contextLens.
+struct PagedAttentionParam {
+    int32_t headNum = 0;   // query heads, > 0
+    float qkScale = 1.0;   // multiplies Q.K^T before the softmax
+    int32_t kvHeadNum = 0; // KV heads; 0 means "same as headNum"
+
+    enum MaskType : int {
+        UNDEFINED = 0, // no mask input
+        MASK_TYPE_NORM,
+        MASK_TYPE_ALIBI,
+        MASK_TYPE_SPEC,
+        MASK_TYPE_MASK_FREE,
+        MASK_TYPE_NORM_COMPRESS
+    };
+    MaskType maskType = UNDEFINED;
+
+    bool batchRunStatusEnable = false;
+
+    enum QuantType : int {
+        TYPE_QUANT_UNDEFINED = 0,
+        TYPE_QUANT_UNQUANT = 0,     // fp16/bf16 query and caches
+        TYPE_DEQUANT_FUSION = 1,    // fp16/bf16 query, int8 caches + per-channel descale (and offset)
+        TYPE_QUANT_QKV_OFFLINE = 2, // int8 query and caches
+        TYPE_QUANT_QKV_ONLINE = 3
+    };
+    QuantType quantType = TYPE_QUANT_UNQUANT;
+
+    aclDataType outDataType = ACL_DT_UNDEFINED; // only read by the QKV-quant modes
+
+    bool hasQuantOffset = false; // dequant fusion: kOffset / vOffset inputs present
+
+    enum CompressType : int {
+        COMPRESS_TYPE_UNDEFINED = 0,
+        COMPRESS_TYPE_KVHEAD,
+        COMPRESS_TYPE_KVHEAD_ROPE,
+        COMPRESS_TYPE_MAX
+    };
+    CompressType compressType = COMPRESS_TYPE_UNDEFINED;
+
+    enum CalcType : int {
+        CALC_TYPE_UNDEFINED = 0,
+        CALC_TYPE_SPEC // several query tokens per sequence (speculative decode)
+    };
+    CalcType calcType = CALC_TYPE_UNDEFINED;
+
+    enum ScaleType : int {
+        SCALE_TYPE_TOR = 0,
+        SCALE_TYPE_LOGN,
+        SCALE_TYPE_MAX
+    };
+    ScaleType scaleType = SCALE_TYPE_TOR;
+
+    InputLayout inputLayout = TYPE_BSND;
+
+    // > 0: the key cache is a combined MLA latent cache and V is its first
+    // mlaVHeadSize channels; no valueCache input. Range [0, 576].
+    uint32_t mlaVHeadSize = 0;
+
+    float qScale = 0; // pre-multiplies Q; ignored when 0 or 1
+
+    uint8_t rsv[64] = {0}; // must stay zero
+};
+
+static_assert(sizeof(ReshapeAndCacheParam) == 24, "ReshapeAndCacheParam ABI size");
+static_assert(sizeof(PagedAttentionParam) == 120, "PagedAttentionParam ABI size");
+
+} // namespace infer
+} // namespace atb
+#endif

@@ -1,0 +1,74 @@
+/*
+ * atb_capi.h - flat C view of the atb::Operation API, for callers that cannot
+ * include C++ headers (ctypes / cffi / JNI test drivers and benchmarks).
+ *
+ * Each function forwards to the C++ call named in its comment and returns its
+ * atb::Status unchanged. It plays the part of the reference's own test
+ * driver, which builds an operation from a param, binds host tensors, then
+ * runs InferShape -> Setup -> Execute
+ * (reference tests/framework/c++/atb_torch/operation/operation_torch.cpp:313-415).
+ * The reference ships C wrappers only for other operators
+ * (include/atb/atb_acl.h:99-116); PagedAttention and ReshapeAndCache have none.
+ */
+#ifndef ATB_CAPI_H
+#define ATB_CAPI_H
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* atb::Tensor flattened: desc {dtype, format, shape}, deviceData, hostData, dataSize. */
+typedef struct AtbCTensor {
+    int32_t dtype;  /* aclDataType */
+    int32_t format; /* aclFormat */
+    int64_t dims[8];
+    uint64_t dimNum;
+    void *deviceData;
+    void *hostData;
+    uint64_t dataSize;
+} AtbCTensor;
+
+/* atb::CreateContext + Context::SetExecuteStream(stream). */
+int32_t atb_c_create_context(void *stream, void **context);
+/* Context::SetExecuteStream. */
+int32_t atb_c_context_set_stream(void *context, void *stream);
+/* Context::SetExecuteType (0 normal, 1 pre-launch, 2 launch). */
+int32_t atb_c_context_set_execute_type(void *context, int32_t type);
+/* atb::DestroyContext. */
+int32_t atb_c_destroy_context(void *context);
+
+/* atb::CreateOperation<infer::PagedAttentionParam> / <infer::ReshapeAndCacheParam>.
+ * opName is "PagedAttentionOperation" or "ReshapeAndCacheOperation"; param
+ * points at the bytes of the matching C++ param struct (120 / 24 bytes). */
+int32_t atb_c_create_operation(const char *opName, const void *param, uint64_t paramSize, void **operation);
+/* atb::DestroyOperation. */
+int32_t atb_c_destroy_operation(void *operation);
+
+/* Operation::GetInputNum / GetOutputNum / GetName (name copied into buf). */
+uint32_t atb_c_op_input_num(void *operation);
+uint32_t atb_c_op_output_num(void *operation);
+int32_t atb_c_op_name(void *operation, char *buf, uint64_t bufSize);
+
+/* Operation::InferShape; only desc fields of the tensors are read/written. */
+int32_t atb_c_op_infer_shape(void *operation, const AtbCTensor *inDescs, uint32_t numIn, AtbCTensor *outDescs,
+                             uint32_t outCapacity, uint32_t *numOut);
+/* Operation::Setup. context may be NULL to exercise the error path. */
+int32_t atb_c_op_setup(void *operation, const AtbCTensor *inTensors, uint32_t numIn, const AtbCTensor *outTensors,
+                       uint32_t numOut, uint64_t *workspaceSize, void *context);
+/* Operation::Execute. */
+int32_t atb_c_op_execute(void *operation, const AtbCTensor *inTensors, uint32_t numIn,
+                         const AtbCTensor *outTensors, uint32_t numOut, void *workspace, uint64_t workspaceSize,
+                         void *context);
+
+/* atb::Utils::GetTensorSize on the desc fields. */
+uint64_t atb_c_tensor_size(const AtbCTensor *tensor);
+
+/* sizeof(infer::PagedAttentionParam), sizeof(infer::ReshapeAndCacheParam). */
+uint64_t atb_c_sizeof_paged_attention_param(void);
+uint64_t atb_c_sizeof_reshape_and_cache_param(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,170 @@
+/*
+ * atbmi_kernels.h - C ABI of the MI355X (gfx950) kernel layer under the ATB
+ * PagedAttention / ReshapeAndCache operators.
+ *
+ * This is the boundary the C++ operator layer (atb::Operation) calls, and the
+ * one a foreign-language binding would bind: plain pointers, sizes and POD
+ * structs, no C++ types, no exceptions. Every pointer named "device" is an HBM
+ * address; "host" pointers are ordinary CPU memory. `stream` is a hipStream_t
+ * passed as void* (NULL = the default stream). All launches are asynchronous.
+ *
+ * Return value: 0 on success, otherwise an atb::ErrorType value
+ * (1 = invalid parameter, 4 = HIP runtime failure, 26 = out of device memory,
+ * 27 = out of host memory). atbmi_last_error() gives a readable reason.
+ *
+ * In the reference these entry points correspond to the device side of the
+ * MKI kernels that the ATB runners launch:
+ *   reshape_and_cache  -> src/kernels/mixkernels/reshape_and_cache/op_kernel/reshape_and_cache_nd.cpp:146-192
+ *   quant_per_channel  -> ElewiseOperation ELEWISE_QUANT_PER_CHANNEL (include/atb/infer_op_params.h:378)
+ *   pa_plan_*          -> PagedAttentionTiling (src/kernels/mixkernels/pagedattention/tiling/paged_attention_tiling.cpp:419-470)
+ *   pa_decode          -> paged_attention_mask (src/kernels/mixkernels/pagedattention/op_kernel/paged_attention_mask_mix.cce:24-163)
+ *                         and the MLA combined-cache kernel (op_kernel/paged_MLAttention_combine_cache_mask_mix.cce)
+ */
+#ifndef ATBMI_KERNELS_H
+#define ATBMI_KERNELS_H
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element types of tensors crossing this boundary. */
+typedef enum AtbmiDtype {
+    ATBMI_F16 = 0,
+    ATBMI_BF16 = 1,
+    ATBMI_INT8 = 2
+} AtbmiDtype;
+
+/* Which attention kernel a plan uses. AUTO picks the MFMA kernel when the
+ * shape is one it is built for and the scalar kernel otherwise. */
+typedef enum AtbmiPaKernel {
+    ATBMI_PA_KERNEL_AUTO = 0,
+    ATBMI_PA_KERNEL_SCALAR = 1,
+    ATBMI_PA_KERNEL_MFMA = 2
+} AtbmiPaKernel;
+
+/* Readable reason for the last non-zero return on the calling thread. */
+const char *atbmi_last_error(void);
+
+/* Number of HIP devices visible, or a negative value when the HIP runtime
+ * cannot be initialised. Makes no allocation. */
+int atbmi_device_count(void);
+
+/*
+ * KV-cache write. For each token i in [0, numTokens): s = slotMapping[i];
+ * s < 0 (or s >= numSlots) skips the token, otherwise the numKvHeads*headDimK
+ * elements of key[i] are copied to keyCache viewed as [numSlots, numKvHeads*headDimK]
+ * at row s, and the same for value/valueCache with headDimV. A byte copy:
+ * elemBytes (1 or 2) is all that matters about the dtype. value and valueCache
+ * may both be NULL (single-cache form).
+ * Replaces: reshape_and_cache_nd.cpp:90-124 (ProcessKVUnequal et al.).
+ */
+int atbmi_reshape_and_cache(const void *keyDevice, const void *valueDevice, void *keyCacheDevice,
+                            void *valueCacheDevice, const int32_t *slotMappingDevice, int64_t numTokens,
+                            int64_t numKvHeads, int64_t headDimK, int64_t headDimV, int64_t numSlots,
+                            int32_t elemBytes, void *stream);
+
+/*
+ * Per-channel int8 quantiser: out[r][c] = clamp(rint(float(x[r][c]) / scale[c]) + offset[c], -128, 127),
+ * IEEE fp32 divide, round-half-even, NaN -> 0. offset may be NULL.
+ * Replaces: the ELEWISE_QUANT_PER_CHANNEL kernel (golden
+ * tests/apitest/opstest/python/operations/elewise/test_elewise_quant.py:24-32).
+ */
+int atbmi_quant_per_channel(const void *xDevice, int32_t xDtype, const float *scaleDevice,
+                            const int32_t *offsetDevice, int8_t *outDevice, int64_t rows, int64_t channels,
+                            void *stream);
+
+/*
+ * Fused quantise + KV-cache write (extension; the reference runs the
+ * quantiser and ReshapeAndCache as two operators): key/value are fp16/bf16
+ * [numTokens, numKvHeads, headDim*], kScale/vScale are fp32 [numKvHeads*headDim*],
+ * caches are int8. Same slot rules as atbmi_reshape_and_cache, same
+ * arithmetic as atbmi_quant_per_channel with no offset.
+ */
+int atbmi_reshape_and_cache_quant(const void *keyDevice, const void *valueDevice, int32_t kvDtype,
+                                  const float *kScaleDevice, const float *vScaleDevice, int8_t *keyCacheDevice,
+                                  int8_t *valueCacheDevice, const int32_t *slotMappingDevice, int64_t numTokens,
+                                  int64_t numKvHeads, int64_t headDimK, int64_t headDimV, int64_t numSlots,
+                                  void *stream);
+
+/* Static description of a paged decode-attention problem. */
+typedef struct AtbmiPaShape {
+    int32_t qDtype;          /* ATBMI_F16 or ATBMI_BF16; the output has the same type */
+    int32_t kvDtype;         /* ATBMI_F16 / ATBMI_BF16 (== qDtype) or ATBMI_INT8 */
+    int32_t numHeads;        /* query heads H */
+    int32_t numKvHeads;      /* KV heads G, H % G == 0 */
+    int32_t headDimK;        /* D: channels of q and of a key row */
+    int32_t headDimV;        /* Dv: channels of a value row and of the output */
+    int32_t blockSize;       /* tokens per cache block */
+    int32_t numBlocks;       /* blocks in the cache pool */
+    int32_t maxBlocksPerSeq; /* row length of blockTables */
+    int32_t numQueryRows;    /* rows of q / out */
+    int32_t mlaCombined;     /* 1: no value cache; V = first Dv channels of the key cache row */
+    int32_t hasOffset;       /* int8 KV: kOffset / vOffset are given */
+    int32_t kernel;          /* AtbmiPaKernel */
+    int32_t reserved;
+    float qkScale;           /* multiplies q.k before the softmax */
+    float qScale;            /* pre-multiplies q (rounded to qDtype) unless 0 or 1 */
+} AtbmiPaShape;
+
+/* Device tensors of one decode call.
+ *   query       [numQueryRows, H, D]                qDtype
+ *   keyCache    [numBlocks, blockSize, G, D]        kvDtype
+ *   valueCache  [numBlocks, blockSize, G, Dv]       kvDtype (NULL when mlaCombined)
+ *   blockTables [batch, maxBlocksPerSeq]            int32
+ *   kScale/vScale [G*D] / [G*Dv] fp32, kOffset/vOffset same length int32 (int8 KV only)
+ *   out         [numQueryRows, H, Dv]               qDtype
+ */
+typedef struct AtbmiPaTensors {
+    const void *query;
+    const void *keyCache;
+    const void *valueCache;
+    const int32_t *blockTables;
+    const float *kScale;
+    const int32_t *kOffset;
+    const float *vScale;
+    const int32_t *vOffset;
+    void *out;
+} AtbmiPaTensors;
+
+typedef struct AtbmiPaPlan AtbmiPaPlan; /* opaque; owned by the caller, not thread-safe */
+
+/* Validates the shape and creates an empty plan. Host only. */
+int atbmi_pa_plan_create(const AtbmiPaShape *shape, AtbmiPaPlan **plan);
+
+/* Splits the batch into KV chunks for the given host context lengths
+ * (sequence b attends to tokens [0, hostContextLens[b])). A sequence of length
+ * 0 is skipped and takes no query row: query/out row index = number of
+ * non-empty sequences before it. Host only, O(batch + chunks). */
+int atbmi_pa_plan_update(AtbmiPaPlan *plan, const int32_t *hostContextLens, int32_t batch);
+
+/* Device workspace bytes atbmi_pa_decode needs for the current plan. */
+uint64_t atbmi_pa_plan_workspace_size(const AtbmiPaPlan *plan);
+
+/* Number of KV chunks (workgroup launches per KV head) in the current plan. */
+int64_t atbmi_pa_plan_num_chunks(const AtbmiPaPlan *plan);
+
+/* Algorithmic HBM bytes of one decode call with the current plan: valid K/V
+ * rows + q + out + block-table entries + context lengths + scale vectors. */
+uint64_t atbmi_pa_plan_algorithmic_bytes(const AtbmiPaPlan *plan);
+
+/* Uploads the plan into the workspace and launches the attention kernel (and
+ * the split merge kernel when any sequence has more than one chunk). */
+int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *tensors, void *workspaceDevice,
+                    uint64_t workspaceBytes, void *stream);
+
+void atbmi_pa_plan_destroy(AtbmiPaPlan *plan);
+
+/*
+ * Kernel timing for benchmarks. When enabled, every atbmi_pa_decode brackets
+ * its attention kernel with HIP events on the launch stream.
+ * atbmi_timing_read waits for the recorded events, adds them up, returns the
+ * sum in milliseconds and the number of launches, and clears the record.
+ */
+int atbmi_timing_enable(int32_t enable);
+int atbmi_timing_read(double *totalMs, int64_t *launches);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

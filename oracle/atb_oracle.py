@@ -1,0 +1,241 @@
+"""CPU oracle for the PagedAttention-decode / ReshapeAndCache path.
+
+TEST INFRASTRUCTURE ONLY. This is the checker the GPU kernels are compared
+against; nothing in the product may import it (only tests/, the smoke entry
+and the benchmark's cpu_baseline leg do).
+
+It restates, in numpy, the reference's own CPU goldens for these operators.
+The reference itself cannot be built here (its host code needs the CANN
+toolkit and the MKI library, its device code the AscendC compiler), and its
+Python test files import torch_npu at module level, so nothing of it is
+executed; every function below follows the cited reference lines and is
+pinned by tests/test_oracle.py against closed forms, fp64 brute force and
+the invariants of the mathematics (no function is left "parity unpinned"):
+
+  reshape_and_cache   tests/apitest/kernelstest/mix/test_reshape_and_cache.py:45-65
+  quant_per_channel   tests/apitest/opstest/python/operations/elewise/test_elewise_quant.py:24-32,
+                      tests/apitest/kernelstest/elewise/test_quant_per_channel.py:22-40
+  paged_attention     tests/apitest/kernelstest/mix/test_paged_attention_common.py:85-118 (grouped
+                      matmul, int8 dequant (q + offset) * scale per channel g*D + d), :132-139
+                      (softmax), :229-276 (the fp32 "out_high" branch), :278-365 (paged gather,
+                      zero-length sequences are skipped and take no query row);
+                      MLA: tests/apitest/opstest/python/operations/paged_attention/
+                      test_paged_attention_operation_mla.py:229-262 (V = K[..., :head_size_vo])
+  merge_partials      src/kernels/mixkernels/pagedattention/op_kernel/
+                      paged_attention_decoder_nd_common.cce:6568-6760,7959-7975 (split-KV combine)
+
+Arithmetic is fp32 throughout ("fp32-accumulated golden"); inputs arrive as
+float32 arrays holding fp16/bf16-representable values, or int8 caches.
+"""
+import numpy as np
+
+
+def bf16_round(x):
+    """Rounds float32 values to the nearest bfloat16 (ties to even), returned as float32."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32).astype(np.uint64)
+    rounded = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    out = rounded.astype(np.uint32).view(np.float32).reshape(x.shape)
+    return np.where(np.isnan(x), x, out)
+
+
+def round_to(x, dtype):
+    """Rounds float32 values to `dtype` ("float16" | "bf16" | "float32"), returned as float32."""
+    if dtype == "float16":
+        return np.asarray(x, dtype=np.float32).astype(np.float16).astype(np.float32)
+    if dtype == "bf16":
+        return bf16_round(x)
+    return np.asarray(x, dtype=np.float32)
+
+
+def reshape_and_cache(key, value, key_cache, value_cache, slot_mapping):
+    """Returns updated copies of the caches: for token i with slot s >= 0 the row
+    key[i] ([heads, head_size_k]) lands in key_cache[s // block, s % block] and
+    value[i] in value_cache likewise; negative slots are skipped. value /
+    value_cache may be None (single-cache form). Pure data movement."""
+    kc = np.array(key_cache, copy=True)
+    vc = None if value_cache is None else np.array(value_cache, copy=True)
+    block_size = kc.shape[1]
+    for i, slot in enumerate(np.asarray(slot_mapping).tolist()):
+        if slot < 0:
+            continue
+        kc[slot // block_size, slot % block_size] = key[i]
+        if vc is not None:
+            vc[slot // block_size, slot % block_size] = value[i]
+    return kc, vc
+
+
+def quant_per_channel(x, scale, offset=None):
+    """int8 = clip(round_half_even(x / scale) (+ offset), -128, 127) with the
+    division in IEEE fp32; scale/offset broadcast over the trailing (channel)
+    axis. NaN quantises to 0. The reference golden divides in the tensor's own
+    dtype (fp16) and is compared with atol=1; this is its fp32 form, which is
+    the one a bit-exact quantised cache is defined by."""
+    x = np.asarray(x, dtype=np.float32)
+    s = np.asarray(scale, dtype=np.float32)
+    with np.errstate(divide="ignore", invalid="ignore", over="ignore"):
+        r = np.rint(x / s)
+    if offset is not None:
+        r = r + np.asarray(offset, dtype=np.float32)
+    r = np.where(np.isnan(r), np.float32(0), r)
+    return np.clip(r, -128, 127).astype(np.int8)
+
+
+def quant_per_channel_golden_dtype(x_fp16, scale_fp16, offset=None):
+    """The golden exactly as the reference test writes it: fp16 / fp16 division."""
+    with np.errstate(divide="ignore", invalid="ignore", over="ignore"):
+        r = np.round(np.asarray(x_fp16, dtype=np.float16) / np.asarray(scale_fp16, dtype=np.float16))
+    if offset is not None:
+        r = r + offset
+    r = np.where(np.isnan(r), 0, r)
+    return np.clip(r, -128, 127).astype(np.int8)
+
+
+def softmax_rows(sim):
+    """Row softmax in fp32, max-subtracted (reference softmax_numpy)."""
+    row_max = np.max(sim, axis=-1, keepdims=True)
+    e = np.exp(sim - row_max)
+    return e / np.sum(e, axis=-1, keepdims=True)
+
+
+def _dequant(rows_i8, scale, offset, g, dim):
+    """(int8 + offset) * scale with the per-(kv head, channel) vectors sliced at g*dim."""
+    f = rows_i8.astype(np.float32)
+    if offset is not None:
+        f = f + np.asarray(offset[g * dim:(g + 1) * dim], dtype=np.float32)
+    return f * np.asarray(scale[g * dim:(g + 1) * dim], dtype=np.float32)
+
+
+def gather_rows(cache, block_table, context_len):
+    """Rows 0..context_len-1 of one sequence: token j lives in block
+    block_table[j // block_size] at offset j % block_size. -> [ctx, kv_heads, dim]"""
+    block_size = cache.shape[1]
+    j = np.arange(context_len)
+    return cache[np.asarray(block_table)[j // block_size], j % block_size]
+
+
+def attention_one(q, keys, values, scale, k_descale=None, k_offset=None, v_descale=None, v_offset=None):
+    """One query token against gathered rows. q [heads, D] float32; keys
+    [ctx, kv_heads, D]; values [ctx, kv_heads, Dv] (float32 or int8).
+    Returns float32 [heads, Dv]: softmax(scale * q k^T) v per GQA group."""
+    heads = q.shape[0]
+    kv_heads = keys.shape[1]
+    group = heads // kv_heads
+    out = np.empty((heads, values.shape[2]), dtype=np.float32)
+    for g in range(kv_heads):
+        k = keys[:, g, :]
+        v = values[:, g, :]
+        if k.dtype == np.int8:
+            k = _dequant(k, k_descale, k_offset, g, keys.shape[2])
+            v = _dequant(v, v_descale, v_offset, g, values.shape[2])
+        k = k.astype(np.float32)
+        v = v.astype(np.float32)
+        qg = q[g * group:(g + 1) * group].astype(np.float32)
+        sim = (qg @ k.T) * np.float32(scale)
+        p = softmax_rows(sim)
+        out[g * group:(g + 1) * group] = p @ v
+    return out
+
+
+def paged_attention(query, key_cache, value_cache, block_tables, context_lens, scale, k_descale=None,
+                    k_offset=None, v_descale=None, v_offset=None, mla_v_head_size=0, q_scale=0.0,
+                    q_dtype="float32", out_init=0.0):
+    """Decode attention over paged caches.
+
+    query [rows, heads, D] float32; key_cache [blocks, block, kv_heads, D];
+    value_cache [blocks, block, kv_heads, Dv], or None with mla_v_head_size > 0
+    (V is then the first mla_v_head_size channels of the key rows).
+    Sequence i with context_lens[i] == 0 is skipped and consumes no query row:
+    the n-th non-empty sequence uses query row n and writes output row n.
+    Rows never written keep `out_init`. q_scale not in {0, 1} pre-multiplies the
+    query and rounds it to q_dtype, as the reference's separate multiply node does.
+    Returns float32 [rows, heads, Dv]."""
+    query = np.asarray(query, dtype=np.float32)
+    if mla_v_head_size > 0:
+        dv = mla_v_head_size
+    else:
+        dv = value_cache.shape[3]
+    out = np.full((query.shape[0], query.shape[1], dv), out_init, dtype=np.float32)
+    if q_scale not in (0.0, 1.0):
+        query = round_to(query * np.float32(q_scale), q_dtype)
+    row = 0
+    for i, ctx in enumerate(np.asarray(context_lens).tolist()):
+        if ctx == 0:
+            continue
+        keys = gather_rows(key_cache, block_tables[i], ctx)
+        values = keys[..., :dv] if mla_v_head_size > 0 else gather_rows(value_cache, block_tables[i], ctx)
+        out[row] = attention_one(query[row], keys, values, scale, k_descale, k_offset, v_descale, v_offset)
+        row += 1
+    return out
+
+
+def paged_attention_loops(query, key_cache, value_cache, block_tables, context_lens, scale):
+    """The same computation written as plain Python loops in float64, for tiny
+    inputs only: an independent check of the vectorised version (no numpy
+    matmul, no broadcasting, no shared helper)."""
+    import math
+    rows, heads, d = query.shape
+    _, block_size, kv_heads, _ = key_cache.shape
+    dv = value_cache.shape[3]
+    group = heads // kv_heads
+    out = [[[0.0] * dv for _ in range(heads)] for _ in range(rows)]
+    row = 0
+    for i in range(len(context_lens)):
+        ctx = int(context_lens[i])
+        if ctx == 0:
+            continue
+        for h in range(heads):
+            g = h // group
+            scores = []
+            for j in range(ctx):
+                blk = int(block_tables[i][j // block_size])
+                off = j % block_size
+                s = 0.0
+                for c in range(d):
+                    s += float(query[row][h][c]) * float(key_cache[blk][off][g][c])
+                scores.append(s * float(scale))
+            m = max(scores)
+            w = [math.exp(s - m) for s in scores]
+            z = sum(w)
+            for c in range(dv):
+                acc = 0.0
+                for j in range(ctx):
+                    blk = int(block_tables[i][j // block_size])
+                    off = j % block_size
+                    acc += w[j] * float(value_cache[blk][off][g][c])
+                out[row][h][c] = acc / z
+        row += 1
+    return np.array(out, dtype=np.float64)
+
+
+def partial_attention(q, keys, values, scale):
+    """Attention over a KV sub-range, in the form a split produces: the
+    normalised output [heads, Dv] and the natural-log log-sum-exp [heads]."""
+    heads = q.shape[0]
+    kv_heads = keys.shape[1]
+    group = heads // kv_heads
+    out = np.empty((heads, values.shape[2]), dtype=np.float32)
+    lse = np.empty((heads,), dtype=np.float32)
+    for g in range(kv_heads):
+        qg = q[g * group:(g + 1) * group].astype(np.float32)
+        sim = (qg @ keys[:, g, :].astype(np.float32).T) * np.float32(scale)
+        m = sim.max(axis=-1, keepdims=True)
+        e = np.exp(sim - m)
+        l = e.sum(axis=-1, keepdims=True)
+        out[g * group:(g + 1) * group] = (e @ values[:, g, :].astype(np.float32)) / l
+        lse[g * group:(g + 1) * group] = (np.log(l) + m)[:, 0]
+    return out, lse
+
+
+def merge_partials(outs, lses):
+    """Split-KV combine: M = max lse; L = log(sum exp(lse - M)) + M;
+    O = sum exp(lse_s - L) O_s. outs [splits, heads, Dv], lses [splits, heads];
+    an empty split carries lse = -inf and weighs nothing."""
+    outs = np.asarray(outs, dtype=np.float32)
+    lses = np.asarray(lses, dtype=np.float32)
+    m = lses.max(axis=0)
+    with np.errstate(invalid="ignore"):
+        big_l = np.log(np.exp(lses - m).sum(axis=0)) + m
+        w = np.exp(lses - big_l)
+    w = np.where(np.isneginf(lses), np.float32(0), w)
+    return (w[:, :, None] * outs).sum(axis=0)

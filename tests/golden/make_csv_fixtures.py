@@ -1,0 +1,74 @@
+#!/usr/bin/env python3
+"""Extracts the host-validation test tables of the reference into JSON fixtures.
+
+The reference keeps its operator API tests as CSV rows (one row = operator
+param JSON + input dtypes/formats/shapes + output dtype/shape + the expected
+status, tagged C: for CreateOperation, I: for InferShape, S: for Setup):
+    tests/apitest/opstest/csv/paged_attention.csv
+    tests/apitest/opstest/csv/reshape_and_cache.csv
+Those rows are data, not code. This script copies the rows written for the
+Ascend910B feature set (the one this library mirrors) into
+    tests/golden/paged_attention_cases.json
+    tests/golden/reshape_and_cache_cases.json
+so the parity tests can run where the reference tree is absent.
+
+Run from the repository root in a container that has /root/reference:
+    python3 tests/golden/make_csv_fixtures.py
+"""
+import csv
+import json
+import os
+import sys
+
+REF = os.environ.get("ATB_REFERENCE", "/root/reference")
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def split(field):
+    return [x.strip() for x in field.split(";") if x.strip() != ""]
+
+
+def shapes(field):
+    out = []
+    for s in split(field):
+        out.append([int(x) for x in s.split(",") if x.strip() != ""])
+    return out
+
+
+def convert(name):
+    path = os.path.join(REF, "tests/apitest/opstest/csv", name + ".csv")
+    rows = list(csv.reader(open(path, newline=""), delimiter="|"))
+    header = [h.strip() for h in rows[0]]
+    cases = []
+    for line_no, row in enumerate(rows[1:], start=2):
+        if not any(c.strip() for c in row):
+            continue
+        d = {h: v.strip() for h, v in zip(header, row)}
+        if d.get("SocVersion") != "Ascend910B":
+            continue
+        cases.append({
+            "csv_line": line_no,
+            "case": int(d["CaseNum"]),
+            "name": d["CaseName"],
+            "op": d["OpName"],
+            "param": json.loads(d["OpParam"]),
+            "in_dtypes": split(d["InDType"]),
+            "in_formats": split(d["InFormat"]),
+            "in_shapes": shapes(d["InShape"]),
+            "out_dtypes": split(d["OutDType"]),
+            "out_formats": split(d["OutFormat"]),
+            "out_shapes": shapes(d["OutShape"]),
+            "expected": d["ExpectedError"],
+        })
+    out = os.path.join(HERE, name + "_cases.json")
+    with open(out, "w") as f:
+        json.dump({"source": "tests/apitest/opstest/csv/%s.csv (rows with SocVersion Ascend910B)" % name,
+                   "cases": cases}, f, indent=1)
+    print(out, len(cases), "cases")
+
+
+if __name__ == "__main__":
+    if not os.path.isdir(REF):
+        sys.exit("reference tree not found at " + REF)
+    convert("paged_attention")
+    convert("reshape_and_cache")

@@ -1,0 +1,114 @@
+"""Helpers shared by the GPU tests: run the kernels through the C ABI or the
+atb::Operation layer on torch tensors, and turn tensors into oracle inputs."""
+import ctypes
+import os
+
+import numpy as np
+import torch
+
+
+def to_oracle(t):
+    """float32 numpy copy of a float tensor; int8 tensors stay int8."""
+    if t is None:
+        return None
+    if t.dtype == torch.int8 or t.dtype == torch.int32:
+        return t.cpu().numpy()
+    return t.float().cpu().numpy()
+
+
+def dtype_code(binding, t):
+    return {torch.float16: binding.ATBMI_F16, torch.bfloat16: binding.ATBMI_BF16, torch.int8: binding.ATBMI_INT8}[t.dtype]
+
+
+def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=None, v_scale=None,
+                   v_off=None, mla_dv=0, q_scale=0.0, kernel=0, chunk_tokens=None, out=None, return_plan_info=False):
+    """atbmi_pa_plan_* + atbmi_pa_decode on `stream`; returns the output tensor."""
+    k = binding.kernels()
+    rows, heads, d = q.shape
+    dv = mla_dv if mla_dv else vc.shape[3]
+    shape = binding.AtbmiPaShape(
+        qDtype=dtype_code(binding, q), kvDtype=dtype_code(binding, kc), numHeads=heads, numKvHeads=kc.shape[2],
+        headDimK=d, headDimV=dv, blockSize=kc.shape[1], numBlocks=kc.shape[0], maxBlocksPerSeq=tables.shape[1],
+        numQueryRows=rows, mlaCombined=1 if mla_dv else 0, hasOffset=1 if k_off is not None else 0, kernel=kernel,
+        qkScale=scale, qScale=q_scale)
+    old = os.environ.get("ATBMI_PA_CHUNK_TOKENS")
+    if chunk_tokens is not None:
+        os.environ["ATBMI_PA_CHUNK_TOKENS"] = str(chunk_tokens)
+    plan = ctypes.c_void_p()
+    try:
+        rc = k.atbmi_pa_plan_create(ctypes.byref(shape), ctypes.byref(plan))
+    finally:
+        if chunk_tokens is not None:
+            if old is None:
+                del os.environ["ATBMI_PA_CHUNK_TOKENS"]
+            else:
+                os.environ["ATBMI_PA_CHUNK_TOKENS"] = old
+    if rc != 0:
+        raise RuntimeError("plan_create: " + binding.last_kernel_error())
+    try:
+        lens = np.ascontiguousarray(np.asarray(ctx_host, dtype=np.int32))
+        rc = k.atbmi_pa_plan_update(plan, lens.ctypes.data, len(lens))
+        if rc != 0:
+            raise RuntimeError("plan_update: " + binding.last_kernel_error())
+        ws_bytes = k.atbmi_pa_plan_workspace_size(plan)
+        with torch.cuda.stream(stream):
+            ws = torch.empty(max(int(ws_bytes), 16), dtype=torch.uint8, device=q.device)
+            if out is None:
+                out = torch.zeros((rows, heads, dv), dtype=q.dtype, device=q.device)
+            t = binding.AtbmiPaTensors()
+            t.query = q.data_ptr()
+            t.keyCache = kc.data_ptr()
+            t.valueCache = vc.data_ptr() if vc is not None else None
+            t.blockTables = tables.data_ptr()
+            t.kScale = k_scale.data_ptr() if k_scale is not None else None
+            t.kOffset = k_off.data_ptr() if k_off is not None else None
+            t.vScale = v_scale.data_ptr() if v_scale is not None else None
+            t.vOffset = v_off.data_ptr() if v_off is not None else None
+            t.out = out.data_ptr()
+            rc = k.atbmi_pa_decode(plan, ctypes.byref(t), ws.data_ptr(), ws_bytes, stream.cuda_stream)
+            if rc != 0:
+                raise RuntimeError("pa_decode: " + binding.last_kernel_error())
+        stream.synchronize()
+        info = dict(chunks=k.atbmi_pa_plan_num_chunks(plan), bytes=k.atbmi_pa_plan_algorithmic_bytes(plan),
+                    workspace=ws_bytes)
+    finally:
+        k.atbmi_pa_plan_destroy(plan)
+    return (out, info) if return_plan_info else out
+
+
+def oracle_pa(oracle, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=None, v_scale=None, v_off=None,
+              mla_dv=0, q_scale=0.0, out_init=0.0):
+    qd = "bf16" if q.dtype == torch.bfloat16 else "float16"
+    return oracle.paged_attention(
+        to_oracle(q), to_oracle(kc), to_oracle(vc), tables.cpu().numpy(), np.asarray(ctx_host), scale,
+        to_oracle(k_scale), to_oracle(k_off), to_oracle(v_scale), to_oracle(v_off), mla_v_head_size=mla_dv,
+        q_scale=q_scale, q_dtype=qd, out_init=out_init)
+
+
+def assert_close(got, want, tol, what=""):
+    """|got - want| <= tol + tol * |want| elementwise (rtol = atol = tol)."""
+    got = got.float().cpu().numpy() if isinstance(got, torch.Tensor) else np.asarray(got, dtype=np.float32)
+    want = np.asarray(want, dtype=np.float32)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    err = np.abs(got - want)
+    lim = tol + tol * np.abs(want)
+    bad = err > lim
+    assert not bad.any() and np.isfinite(got).all(), "%s: %d of %d outside tol %g, max err %g at %s" % (
+        what, int(bad.sum()), bad.size, tol, float(err.max()), np.unravel_index(int(err.argmax()), err.shape))
+
+
+def random_tables(rng, ctx, block, pool, unique=True):
+    """Block tables for the given lengths; unused entries hold valid ids."""
+    ctx = np.asarray(ctx, dtype=np.int64)
+    nblk = (ctx + block - 1) // block
+    width = max(1, int(nblk.max()))
+    total = int(nblk.sum())
+    ids = rng.permutation(pool)[:total] if unique else rng.integers(0, pool, size=total)
+    tables = np.zeros((len(ctx), width), dtype=np.int32)
+    pos = 0
+    for b in range(len(ctx)):
+        n = int(nblk[b])
+        tables[b, :n] = ids[pos:pos + n]
+        tables[b, n:] = ids[pos] if n else 0
+        pos += n
+    return tables

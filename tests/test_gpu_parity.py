@@ -1,0 +1,448 @@
+"""GPU parity tests: the HIP kernels against the CPU oracle on the same seeded
+inputs. ReshapeAndCache, the slot scatter and the int8 quantised cache must be
+bit-exact; attention must be within rtol = atol = 1e-3 for fp16 and 2e-2 for
+bf16 / int8 caches of the fp32 oracle. Shapes follow the reference's own
+kernel-test matrix (tests/apitest/kernelstest/mix/test_paged_attention_common.py,
+test_paged_attention_mla.py, test_reshape_and_cache.py) plus the small
+benchmark configuration."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from pa_harness import assert_close, oracle_pa, pa_decode_cabi, random_tables, to_oracle
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float16: 1e-3, torch.bfloat16: 2e-2}
+INT8_TOL = 2e-2
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return torch.device("cuda:0")
+
+
+@pytest.fixture(scope="module")
+def stream(dev):
+    return torch.cuda.Stream(device=dev)
+
+
+def _rng(seed):
+    return np.random.Generator(np.random.PCG64(seed))
+
+
+# ------------------------------------------------------------------ ReshapeAndCache
+RAC_SHAPES = [
+    # tokens, heads, dk, dv, block, blocks, dtype   (reference test_reshape_and_cache.py:106-260, pool scaled down)
+    (100, 64, 576, 512, 128, 8, torch.int8),
+    (100, 64, 320, 256, 128, 8, torch.float16),
+    (100, 64, 400, 200, 128, 8, torch.bfloat16),
+    (100, 64, 576, 576, 128, 8, torch.int8),
+    (64, 8, 128, 128, 128, 80, torch.bfloat16),   # a decode step of the 8B-shaped config
+    (7, 3, 5, 3, 16, 4, torch.int8),              # odd row sizes: byte-granular copy path
+    (9, 1, 7, 9, 16, 4, torch.float16),           # 2-byte-granular copy path
+]
+
+
+def _rac_inputs(rng, dev, tokens, heads, dk, dv, block, blocks, dtype):
+    def mk(shape, lo, hi):
+        a = rng.integers(lo, hi, size=shape)
+        return torch.from_numpy(a.astype(np.float32)).to(dtype).to(dev) if dtype != torch.int8 else \
+            torch.from_numpy(a.astype(np.int8)).to(dev)
+    key = mk((tokens, heads, dk), 1, 11)
+    value = mk((tokens, heads, dv), 1, 11)
+    kc = mk((blocks, block, heads, dk), 20, 30)
+    vc = mk((blocks, block, heads, dv), 20, 30)
+    n = blocks * block
+    slots = rng.choice(np.arange(-n, n), size=tokens, replace=False).astype(np.int32)
+    return key, value, kc, vc, slots
+
+
+def _bits(t):
+    return t.view(torch.int16) if t.dtype in (torch.float16, torch.bfloat16) else t
+
+
+@pytest.mark.parametrize("shape", RAC_SHAPES, ids=lambda s: "x".join(str(v) for v in s[:6]) + str(s[6]).split(".")[-1])
+def test_reshape_and_cache_bit_exact(binding, oracle, dev, stream, shape):
+    rng = _rng(11)
+    key, value, kc, vc, slots = _rac_inputs(rng, dev, *shape)
+    want_k, want_v = oracle.reshape_and_cache(_bits(key).cpu().numpy(), _bits(value).cpu().numpy(),
+                                              _bits(kc).cpu().numpy(), _bits(vc).cpu().numpy(), slots)
+    ctx = binding.Context(stream)
+    runner = binding.OperationRunner("ReshapeAndCacheOperation", binding.ReshapeAndCacheParam(), ctx)
+    with torch.cuda.stream(stream):
+        slots_d = torch.from_numpy(slots).to(dev)
+        runner.run([key, value, kc, vc, slots_d], outputs=[kc, vc])
+    stream.synchronize()
+    assert np.array_equal(_bits(kc).cpu().numpy(), want_k)
+    assert np.array_equal(_bits(vc).cpu().numpy(), want_v)
+    assert (slots < 0).any()
+    runner.close()
+    ctx.close()
+
+
+def test_reshape_and_cache_single_cache_and_out_of_range_slots(binding, oracle, dev, stream):
+    rng = _rng(12)
+    key, _, kc, _, slots = _rac_inputs(rng, dev, 20, 1, 576, 576, 128, 2, torch.bfloat16)
+    want_k, _ = oracle.reshape_and_cache(_bits(key).cpu().numpy(), None, _bits(kc).cpu().numpy(), None, slots)
+    ctx = binding.Context(stream)
+    runner = binding.OperationRunner("ReshapeAndCacheOperation", binding.ReshapeAndCacheParam(kvCacheCfg=1), ctx)
+    with torch.cuda.stream(stream):
+        runner.run([key, kc, torch.from_numpy(slots).to(dev)], outputs=[kc])
+    stream.synchronize()
+    assert np.array_equal(_bits(kc).cpu().numpy(), want_k)
+    # slots past the end of the cache are undefined in the reference; here they are skipped
+    before = kc.clone()
+    k = binding.kernels()
+    with torch.cuda.stream(stream):
+        far = torch.full((20,), 2 * 128 + 5, dtype=torch.int32, device=dev)
+        rc = k.atbmi_reshape_and_cache(key.data_ptr(), None, kc.data_ptr(), None, far.data_ptr(), 20, 1, 576, 0,
+                                       2 * 128, 2, stream.cuda_stream)
+    stream.synchronize()
+    assert rc == 0 and torch.equal(_bits(kc), _bits(before))
+    runner.close()
+    ctx.close()
+
+
+# ------------------------------------------------------------------ quantiser
+def test_quant_all_fp16_patterns_bit_exact(binding, oracle, dev, stream):
+    k = binding.kernels()
+    x = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    scales = np.array([0.005, 0.0123, 0.02, 0.37, 1.0, 3.0, 1e-4, 7.3], dtype=np.float32)
+    x = x.reshape(8192, 8).to(dev)  # channel c = pattern % 8 sees scale c
+    offs = np.array([0, 3, -3, 100, -100, 0, 1, -1], dtype=np.int32)
+    for offset in (None, offs):
+        with torch.cuda.stream(stream):
+            out = torch.empty((8192, 8), dtype=torch.int8, device=dev)
+            s_d = torch.from_numpy(scales).to(dev)
+            o_d = torch.from_numpy(offset).to(dev) if offset is not None else None
+            rc = k.atbmi_quant_per_channel(x.data_ptr(), binding.ATBMI_F16, s_d.data_ptr(),
+                                           o_d.data_ptr() if o_d is not None else None, out.data_ptr(), 8192, 8,
+                                           stream.cuda_stream)
+        stream.synchronize()
+        assert rc == 0
+        want = oracle.quant_per_channel(x.float().cpu().numpy(), scales, offset)
+        assert np.array_equal(out.cpu().numpy(), want)
+
+
+def test_quant_bf16_bit_exact(binding, oracle, dev, stream):
+    k = binding.kernels()
+    x = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).reshape(4096, 16).to(dev)
+    scales = _rng(13).uniform(0.005, 0.02, size=16).astype(np.float32)
+    with torch.cuda.stream(stream):
+        out = torch.empty((4096, 16), dtype=torch.int8, device=dev)
+        s_d = torch.from_numpy(scales).to(dev)
+        rc = k.atbmi_quant_per_channel(x.data_ptr(), binding.ATBMI_BF16, s_d.data_ptr(), None, out.data_ptr(), 4096, 16,
+                                       stream.cuda_stream)
+    stream.synchronize()
+    assert rc == 0
+    assert np.array_equal(out.cpu().numpy(), oracle.quant_per_channel(x.float().cpu().numpy(), scales))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_reshape_and_cache_quant_bit_exact(binding, oracle, dev, stream, dtype):
+    """Fused quantise + cache write == quantiser followed by ReshapeAndCache."""
+    rng = _rng(14)
+    tokens, g, d, block, blocks = 128, 8, 128, 128, 6
+    k = binding.kernels()
+    key = torch.from_numpy(rng.standard_normal((tokens, g, d)).astype(np.float32) * 0.5).to(dtype).to(dev)
+    value = torch.from_numpy(rng.standard_normal((tokens, g, d)).astype(np.float32) * 0.5).to(dtype).to(dev)
+    ks = rng.uniform(0.005, 0.02, size=g * d).astype(np.float32)
+    vs = rng.uniform(0.005, 0.02, size=g * d).astype(np.float32)
+    kc = torch.from_numpy(rng.integers(-127, 128, size=(blocks, block, g, d)).astype(np.int8)).to(dev)
+    vc = torch.from_numpy(rng.integers(-127, 128, size=(blocks, block, g, d)).astype(np.int8)).to(dev)
+    n = blocks * block
+    slots = rng.choice(np.arange(-n, n), size=tokens, replace=False).astype(np.int32)
+    qk = oracle.quant_per_channel(key.float().cpu().numpy().reshape(tokens, -1), ks).reshape(tokens, g, d)
+    qv = oracle.quant_per_channel(value.float().cpu().numpy().reshape(tokens, -1), vs).reshape(tokens, g, d)
+    want_k, want_v = oracle.reshape_and_cache(qk, qv, kc.cpu().numpy(), vc.cpu().numpy(), slots)
+    with torch.cuda.stream(stream):
+        ks_d, vs_d, sl_d = torch.from_numpy(ks).to(dev), torch.from_numpy(vs).to(dev), torch.from_numpy(slots).to(dev)
+        rc = k.atbmi_reshape_and_cache_quant(key.data_ptr(), value.data_ptr(),
+                                             binding.ATBMI_BF16 if dtype == torch.bfloat16 else binding.ATBMI_F16,
+                                             ks_d.data_ptr(), vs_d.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+                                             sl_d.data_ptr(), tokens, g, d, d, n, stream.cuda_stream)
+    stream.synchronize()
+    assert rc == 0
+    assert np.array_equal(kc.cpu().numpy(), want_k) and np.array_equal(vc.cpu().numpy(), want_v)
+
+
+# ------------------------------------------------------------------ attention
+def _pa_inputs(rng, dev, batch, heads, kv_heads, block, d, dv, ctx, dtype, kv_int8=False, pool_extra=4, std=1.0,
+               unique=True):
+    ctx = np.asarray(ctx if hasattr(ctx, "__len__") else [ctx] * batch, dtype=np.int32)
+    need = int(((ctx.astype(np.int64) + block - 1) // block).sum())
+    pool = need + pool_extra
+    tables = random_tables(rng, ctx, block, pool, unique=unique)
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(int(rng.integers(1 << 30)))
+    q = (torch.rand((len(ctx), heads, d), generator=gen) * 2 - 1).to(dtype).to(dev)
+    if kv_int8:
+        kc = torch.randint(-4, 5, (pool, block, kv_heads, d), generator=gen, dtype=torch.int8).to(dev)
+        vc = torch.randint(-4, 5, (pool, block, kv_heads, dv), generator=gen, dtype=torch.int8).to(dev)
+    else:
+        kc = ((torch.rand((pool, block, kv_heads, d), generator=gen) * 2 - 1) * std).to(dtype).to(dev)
+        vc = ((torch.rand((pool, block, kv_heads, dv), generator=gen) * 2 - 1) * std).to(dtype).to(dev)
+    return q, kc, vc, torch.from_numpy(tables).to(dev), ctx
+
+
+# batch, heads, kv_heads, block, d, ctx, dtype  (reference test_paged_attention_common.py case list)
+PA_MATRIX = [
+    (6, 32, 32, 128, 128, 819, torch.float16),
+    (13, 32, 32, 128, 128, 200, torch.bfloat16),
+    (13, 8, 1, 128, 128, 88, torch.float16),
+    (20, 127, 1, 128, 128, 88, torch.float16),
+    (18, 30, 2, 128, 128, 88, torch.float16),
+    (20, 33, 33, 128, 128, 88, torch.float16),
+    (4, 32, 2, 128, 128, 2048, torch.float16),
+    (4, 24, 1, 16, 256, 3000, torch.float16),
+    (2, 24, 1, 16, 256, 30000, torch.float16),
+    (9, 40, 40, 16, 96, [3000, 300, 14000, 33, 65, 1, 16, 14000, 300], torch.float16),
+    (1, 12, 1, 128, 128, 16390, torch.float16),
+    (5, 8, 4, 128, 128, 13164, torch.bfloat16),
+    (3, 12, 1, 128, 128, 32768, torch.bfloat16),
+]
+
+
+def _kernels_for(binding, d, dv, block):
+    """Kernel selections to test: the scalar kernel always, the MFMA kernel where it is built."""
+    return [binding.ATBMI_PA_KERNEL_SCALAR, binding.ATBMI_PA_KERNEL_AUTO]
+
+
+@pytest.mark.parametrize("case", PA_MATRIX, ids=lambda c: "b%d_h%d_g%d_bs%d_d%d_%s" % (
+    c[0], c[1], c[2], c[3], c[4], str(c[6]).split(".")[-1]))
+def test_paged_attention_matrix(binding, oracle, dev, stream, case):
+    batch, heads, kv_heads, block, d, ctx, dtype = case
+    rng = _rng(hash(case[:5]) % 1000 + 20)
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, batch, heads, kv_heads, block, d, d, ctx, dtype)
+    scale = 1.0 / math.sqrt(d)
+    want = oracle_pa(oracle, q, kc, vc, tables, ctx, scale)
+    for kernel in _kernels_for(binding, d, d, block):
+        got = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, kernel=kernel)
+        assert_close(got, want, TOL[dtype], "kernel=%d" % kernel)
+
+
+def test_c1_decode_step_through_operation_api(binding, oracle, pkg, dev, stream):
+    """Benchmark configuration 1 end to end: ReshapeAndCache then PagedAttention
+    through atb::Operation, fp16, rtol = atol = 1e-3."""
+    w = pkg.workloads
+    cfg = w.config("c1")
+    step = w.make_step(cfg, dev)
+    scale = w.qk_scale(cfg)
+    kc0, vc0 = step["key_cache"].clone(), step["value_cache"].clone()
+    want_k, want_v = oracle.reshape_and_cache(_bits(step["k_new"]).cpu().numpy(), _bits(step["v_new"]).cpu().numpy(),
+                                              _bits(kc0).cpu().numpy(), _bits(vc0).cpu().numpy(),
+                                              step["layout"]["slots"])
+    ctx = binding.Context(stream)
+    rac = binding.OperationRunner("ReshapeAndCacheOperation", binding.ReshapeAndCacheParam(), ctx)
+    pa = binding.OperationRunner("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=cfg["heads"], kvHeadNum=cfg["kv_heads"], qkScale=scale), ctx)
+    with torch.cuda.stream(stream):
+        rac.run([step["k_new"], step["v_new"], step["key_cache"], step["value_cache"], step["slot_mapping"]],
+                outputs=[step["key_cache"], step["value_cache"]])
+        lens_dev = step["context_lens"].to(dev)
+        out, = pa.run([step["q"], step["key_cache"], step["value_cache"], step["block_tables"], lens_dev],
+                      host_inputs={4: step["context_lens"]})
+    stream.synchronize()
+    assert np.array_equal(_bits(step["key_cache"]).cpu().numpy(), want_k)
+    assert np.array_equal(_bits(step["value_cache"]).cpu().numpy(), want_v)
+    want = oracle.paged_attention(to_oracle(step["q"]), to_oracle(step["key_cache"]), to_oracle(step["value_cache"]),
+                                  step["layout"]["tables"], step["layout"]["ctx"], scale)
+    assert_close(out, want, 1e-3, "c1")
+    # the new token is part of the context: dropping it must change the result
+    short = oracle.paged_attention(to_oracle(step["q"]), to_oracle(kc0), to_oracle(vc0), step["layout"]["tables"],
+                                   step["layout"]["ctx"], scale)
+    assert np.abs(short - want).max() > 1e-3
+    rac.close()
+    pa.close()
+    ctx.close()
+
+
+# batch, heads, kv_heads, ctx, q dtype, with offsets   (reference :2179-2808)
+INT8_MATRIX = [
+    (24, 8, 8, 256, torch.float16, False),
+    (16, 8, 1, 256, torch.bfloat16, False),
+    (1, 24, 1, 513, torch.bfloat16, False),
+    (16, 8, 1, 256, torch.float16, True),
+    (1, 8, 8, 256, torch.float16, False),
+    (1, 8, 8, 1780, torch.float16, True),
+    (8, 64, 8, 1200, torch.float16, False),
+]
+
+
+@pytest.mark.parametrize("case", INT8_MATRIX, ids=lambda c: "b%d_h%d_g%d_ctx%d_%s_off%d" % (
+    c[0], c[1], c[2], c[3], str(c[4]).split(".")[-1], c[5]))
+def test_paged_attention_int8_cache(binding, oracle, dev, stream, case):
+    batch, heads, kv_heads, ctx, dtype, with_off = case
+    rng = _rng(30 + batch + heads)
+    d = 128
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, batch, heads, kv_heads, 128, d, d, ctx, dtype, kv_int8=True)
+    ks = torch.from_numpy(rng.uniform(0.05, 0.5, size=kv_heads * d).astype(np.float32)).to(dev)
+    vs = torch.from_numpy(rng.uniform(0.05, 0.5, size=kv_heads * d).astype(np.float32)).to(dev)
+    ko = torch.from_numpy(rng.integers(-20, 20, size=kv_heads * d).astype(np.int32)).to(dev) if with_off else None
+    vo = torch.from_numpy(rng.integers(-20, 20, size=kv_heads * d).astype(np.int32)).to(dev) if with_off else None
+    scale = 1.0 / math.sqrt(d)
+    want = oracle_pa(oracle, q, kc, vc, tables, ctx, scale, ks, ko, vs, vo)
+    for kernel in _kernels_for(binding, d, d, 128):
+        got = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, ks, ko, vs, vo, kernel=kernel)
+        assert_close(got, want, INT8_TOL, "kernel=%d" % kernel)
+
+
+def test_int8_through_operation_api_with_offsets(binding, oracle, dev, stream):
+    rng = _rng(41)
+    heads, kv_heads, d = 32, 16, 128
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, 4, heads, kv_heads, 64, d, d, [100, 2000, 64, 777], torch.float16,
+                                        kv_int8=True)
+    ks = torch.from_numpy(rng.uniform(0.01, 0.1, size=kv_heads * d).astype(np.float32)).to(dev)
+    vs = torch.from_numpy(rng.uniform(0.01, 0.1, size=kv_heads * d).astype(np.float32)).to(dev)
+    ko = torch.from_numpy(rng.integers(-20, 20, size=kv_heads * d).astype(np.int32)).to(dev)
+    vo = torch.from_numpy(rng.integers(-20, 20, size=kv_heads * d).astype(np.int32)).to(dev)
+    scale = 1.0 / math.sqrt(d)
+    c = binding.Context(stream)
+    pa = binding.OperationRunner("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=heads, kvHeadNum=kv_heads, qkScale=scale, quantType=1, hasQuantOffset=True), c)
+    lens = torch.from_numpy(ctx)
+    with torch.cuda.stream(stream):
+        out, = pa.run([q, kc, vc, tables, lens.to(dev), ks, ko, vs, vo], host_inputs={4: lens})
+    stream.synchronize()
+    assert_close(out, oracle_pa(oracle, q, kc, vc, tables, ctx, scale, ks, ko, vs, vo), INT8_TOL, "dequant api")
+    pa.close()
+    c.close()
+
+
+# batch, heads, d, dv, block, ctx, dtype   (reference test_paged_attention_mla.py:713-1137, op test :412-444)
+MLA_MATRIX = [
+    (20, 128, 576, 512, 128, 256, torch.float16),
+    (1, 8, 576, 512, 128, 256, torch.bfloat16),
+    (64, 32, 192, 128, 128, 256, torch.float16),
+    (32, 8, 576, 512, 128, 819, torch.float16),
+    (4, 128, 576, 512, 128, [3000, 17, 128, 1025], torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("case", MLA_MATRIX, ids=lambda c: "b%d_h%d_d%d_dv%d_%s" % (
+    c[0], c[1], c[2], c[3], str(c[6]).split(".")[-1]))
+def test_paged_attention_mla_combined_cache(binding, oracle, dev, stream, case):
+    batch, heads, d, dv, block, ctx, dtype = case
+    rng = _rng(50 + batch)
+    q, kc, _, tables, ctx = _pa_inputs(rng, dev, batch, heads, 1, block, d, dv, ctx, dtype, std=0.5)
+    scale = 1.0 / math.sqrt(d)
+    want = oracle_pa(oracle, q, kc, None, tables, ctx, scale, mla_dv=dv)
+    for kernel in _kernels_for(binding, d, dv, block):
+        got = pa_decode_cabi(binding, stream, q, kc, None, tables, ctx, scale, mla_dv=dv, kernel=kernel)
+        assert_close(got, want, TOL[dtype], "kernel=%d" % kernel)
+
+
+def test_mla_through_operation_api_and_split_head_sizes(binding, oracle, dev, stream):
+    rng = _rng(61)
+    c = binding.Context(stream)
+    # combined cache: 4 inputs, output width mlaVHeadSize
+    q, kc, _, tables, ctx = _pa_inputs(rng, dev, 5, 16, 1, 128, 576, 512, [300, 1, 129, 128, 640], torch.bfloat16,
+                                       std=0.5)
+    scale = 1.0 / math.sqrt(192)
+    pa = binding.OperationRunner("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=16, kvHeadNum=1, qkScale=scale, mlaVHeadSize=512), c)
+    lens = torch.from_numpy(ctx)
+    with torch.cuda.stream(stream):
+        out, = pa.run([q, kc, tables, lens.to(dev)], host_inputs={3: lens})
+    stream.synchronize()
+    assert tuple(out.shape) == (5, 16, 512)
+    assert_close(out, oracle_pa(oracle, q, kc, None, tables, ctx, scale, mla_dv=512), 2e-2, "mla api")
+    pa.close()
+    # separate caches with different K and V head sizes (reference CSV row "MLA": 128 / 96)
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, 4, 32, 16, 64, 128, 96, [64, 500, 33, 1000], torch.float16)
+    pa = binding.OperationRunner("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=32, kvHeadNum=16, qkScale=0.088), c)
+    lens = torch.from_numpy(ctx)
+    with torch.cuda.stream(stream):
+        out, = pa.run([q, kc, vc, tables, lens.to(dev)], host_inputs={4: lens})
+    stream.synchronize()
+    assert tuple(out.shape) == (4, 32, 96)
+    assert_close(out, oracle_pa(oracle, q, kc, vc, tables, ctx, 0.088), 1e-3, "dk!=dv")
+    pa.close()
+    c.close()
+
+
+# ------------------------------------------------------------------ edge semantics
+@pytest.mark.parametrize("kernel", [1, 0])
+def test_empty_sequences_garbage_rows_and_shared_blocks(binding, oracle, dev, stream, kernel):
+    rng = _rng(70)
+    heads, kv_heads, d, block = 16, 4, 128, 16
+    ctx = np.array([0, 37, 1, 0, 400, 16, 0], dtype=np.int32)
+    # blocks may be shared between sequences and repeat inside one (read-only)
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, len(ctx), heads, kv_heads, block, d, d, ctx, torch.float16,
+                                        unique=False)
+    # poison every cache row no sequence may read
+    used = np.zeros((kc.shape[0], block), dtype=bool)
+    t = tables.cpu().numpy()
+    for b, n in enumerate(ctx):
+        j = np.arange(n)
+        used[t[b][j // block], j % block] = True
+    mask = torch.from_numpy(~used).to(dev)
+    kc[mask] = float("nan")
+    vc[mask] = float("nan")
+    # block-table entries past the last used block must never be dereferenced
+    t2 = t.copy()
+    for b, n in enumerate(ctx):
+        t2[b, (n + block - 1) // block:] = 0x3FFFFFF
+    tables2 = torch.from_numpy(t2).to(dev)
+    scale = 1.0 / math.sqrt(d)
+    out = torch.full((len(ctx), heads, d), 0.1, dtype=torch.float16, device=dev)
+    got = pa_decode_cabi(binding, stream, q, kc, vc, tables2, ctx, scale, kernel=kernel, out=out)
+    kc_o, vc_o = kc.clone(), vc.clone()
+    kc_o[mask] = 0
+    vc_o[mask] = 0
+    want = oracle_pa(oracle, q, kc_o, vc_o, tables, ctx, scale, out_init=0.1)
+    # rows 0..3 belong to the four non-empty sequences, rows 4..6 are never written
+    assert_close(got, want, 1e-3, "edge")
+    assert torch.all(got[4:] == torch.tensor(0.1, dtype=torch.float16))
+
+
+@pytest.mark.parametrize("kernel", [1, 0])
+@pytest.mark.parametrize("chunk", [128, 256, 1024, 100000])
+def test_split_kv_chunking_does_not_change_the_result(binding, oracle, dev, stream, kernel, chunk):
+    rng = _rng(80)
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, 3, 32, 8, 128, 128, 128, [5000, 129, 2049], torch.bfloat16)
+    scale = 1.0 / math.sqrt(128)
+    got, info = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, kernel=kernel, chunk_tokens=chunk,
+                               return_plan_info=True)
+    assert_close(got, oracle_pa(oracle, q, kc, vc, tables, ctx, scale), 2e-2, "chunk=%d" % chunk)
+    if chunk == 128:
+        assert info["chunks"] >= 40 + 2 + 17
+    if chunk == 100000:
+        assert info["chunks"] == 3
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_q_scale_premultiply(binding, oracle, dev, stream, dtype):
+    rng = _rng(90)
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, 4, 8, 8, 128, 128, 128, [300, 64, 512, 9], dtype)
+    for kernel in (1, 0):
+        got = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, 0.2, q_scale=0.7, kernel=kernel)
+        assert_close(got, oracle_pa(oracle, q, kc, vc, tables, ctx, 0.2, q_scale=0.7), TOL[dtype], "qScale")
+
+
+def test_repeated_execute_and_changing_lengths(binding, oracle, dev, stream):
+    """One operation, Setup + Execute repeatedly with growing context lengths, no sync in between."""
+    rng = _rng(95)
+    heads, kv_heads, d, block = 32, 8, 128, 128
+    base = np.array([700, 1500, 128, 3000], dtype=np.int32)
+    q, kc, vc, tables, _ = _pa_inputs(rng, dev, 4, heads, kv_heads, block, d, d, base + 8, torch.float16)
+    scale = 1.0 / math.sqrt(d)
+    c = binding.Context(stream)
+    pa = binding.OperationRunner("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=heads, kvHeadNum=kv_heads, qkScale=scale), c)
+    outs = []
+    with torch.cuda.stream(stream):
+        for step in range(8):
+            lens = torch.from_numpy(base + step)
+            out, = pa.run([q, kc, vc, tables, lens.to(dev)], host_inputs={4: lens})
+            outs.append(out)
+    stream.synchronize()
+    for step in (0, 3, 7):
+        assert_close(outs[step], oracle_pa(oracle, q, kc, vc, tables, base + step, scale), 1e-3, "step %d" % step)
+    pa.close()
+    c.close()

@@ -1,0 +1,383 @@
+"""Host-side behaviour of the atb::Operation layer, without a GPU.
+
+The expected statuses come from the reference's own operator-API test tables
+(tests/golden/*_cases.json, extracted from the reference CSVs by
+tests/golden/make_csv_fixtures.py): one row = param + input/output
+descriptions + the status the reference returns, tagged with the stage
+(C: CreateOperation, I: InferShape, S: Setup). Setup never touches device
+memory, so fake device addresses are enough here.
+"""
+import ctypes
+import json
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+FAKE_DEVICE = 0x10000
+
+
+def _load(name):
+    with open(os.path.join(HERE, "golden", name + "_cases.json")) as f:
+        return json.load(f)["cases"]
+
+
+PA_CASES = _load("paged_attention")
+RAC_CASES = _load("reshape_and_cache")
+
+
+def _pa_unimplemented(p):
+    """Features of PagedAttentionParam the reference accepts but this library rejects at creation."""
+    return (p.get("maskType", 0) != 0 or p.get("batchRunStatusEnable", False) or p.get("compressType", 0) != 0 or
+            p.get("calcType", 0) != 0 or p.get("scaleType", 0) != 0 or p.get("inputLayout", 0) != 0 or
+            p.get("quantType", 0) >= 2)
+
+
+def _rac_unimplemented(p):
+    return p.get("compressType", 0) in (1, 2) or p.get("kvCacheCfg", 0) == 2
+
+
+def _make_param(binding, op, p):
+    if op == "PagedAttentionOperation":
+        return binding.PagedAttentionParam(**p)
+    return binding.ReshapeAndCacheParam(**p)
+
+
+def _tensors(binding, dtypes, formats, shapes, host_index=None, host_array=None):
+    out = []
+    for i, (dt, fmt, shape) in enumerate(zip(dtypes, formats, shapes)):
+        host = host_array.ctypes.data if (i == host_index and host_array is not None) else None
+        out.append(binding.make_tensor(dt, shape, device_ptr=FAKE_DEVICE, host_ptr=host, fmt=fmt))
+    return out
+
+
+def _run_case(binding, case, ctx):
+    """Returns (stage, status) of the first failing stage, or ("", 0)."""
+    op = binding.Operation(case["op"], _make_param(binding, case["op"], case["param"]))
+    if op.status != 0:
+        return "C", op.status, None
+    try:
+        ins = _tensors(binding, case["in_dtypes"], case["in_formats"], case["in_shapes"])
+        st, out_descs = op.infer_shape(ins)
+        if st != 0:
+            return "I", st, None
+        host = None
+        host_index = None
+        if case["op"] == "PagedAttentionOperation":
+            host_index = 3 if case["param"].get("mlaVHeadSize", 0) > 0 else 4
+            kc = case["in_shapes"][1]
+            tables = case["in_shapes"][host_index - 1]
+            host = np.full((case["in_shapes"][host_index][0],), min(kc[1] * tables[1], 7), dtype=np.int32)
+        ins = _tensors(binding, case["in_dtypes"], case["in_formats"], case["in_shapes"], host_index, host)
+        outs = _tensors(binding, case["out_dtypes"], case["out_formats"], case["out_shapes"])
+        st, _ = op.setup(ins, outs, ctx)
+        if st != 0:
+            return "S", st, out_descs
+        return "", 0, out_descs
+    finally:
+        op.close()
+
+
+@pytest.fixture(scope="module")
+def ctx(binding):
+    c = binding.Context(0x1)  # any non-null handle: Setup never uses the stream
+    yield c
+    c.close()
+
+
+def _check(binding, case, ctx, unimplemented):
+    stage, status, out_descs = _run_case(binding, case, ctx)
+    expected = case["expected"]
+    if unimplemented:
+        # documented deviation: rejected when the operation is created
+        assert (stage, status) == ("C", binding.ERROR_CODE["ERROR_INVALID_PARAM"])
+        return
+    if expected == "NO_ERROR":
+        assert (stage, status) == ("", 0), "%s: %s:%s" % (case["name"], stage, binding.ERROR_NAMES[status])
+        got = [[d.dims[i] for i in range(d.dimNum)] for d in out_descs]
+        assert got == case["out_shapes"]
+        return
+    want_stage, want_name = expected.split(":")
+    assert stage == want_stage and binding.ERROR_NAMES[status] == want_name, \
+        "%s: got %s:%s want %s" % (case["name"], stage, binding.ERROR_NAMES[status], expected)
+
+
+@pytest.mark.parametrize("case", PA_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
+def test_paged_attention_table(binding, ctx, case):
+    _check(binding, case, ctx, _pa_unimplemented(case["param"]) and not case["expected"].startswith("C:"))
+
+
+@pytest.mark.parametrize("case", RAC_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
+def test_reshape_and_cache_table(binding, ctx, case):
+    _check(binding, case, ctx, _rac_unimplemented(case["param"]) and not case["expected"].startswith("C:"))
+
+
+def test_table_coverage():
+    """Most rows of the reference tables must be checked at face value, not as deviations."""
+    pa_dev = [c for c in PA_CASES if _pa_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
+    rac_dev = [c for c in RAC_CASES if _rac_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
+    assert len(PA_CASES) == 81 and len(PA_CASES) - len(pa_dev) >= 55
+    assert len(RAC_CASES) == 37 and len(RAC_CASES) - len(rac_dev) >= 25
+
+
+def test_param_sizes(binding):
+    # reference tests/unittest/ops/test_op_param_size.cpp:47,51
+    assert binding.atb().atb_c_sizeof_paged_attention_param() == 120
+    assert binding.atb().atb_c_sizeof_reshape_and_cache_param() == 24
+    assert ctypes.sizeof(binding.PagedAttentionParam) == 120
+    assert ctypes.sizeof(binding.ReshapeAndCacheParam) == 24
+
+
+def test_reserved_bytes_must_be_zero(binding):
+    p = binding.PagedAttentionParam(headNum=8, kvHeadNum=8)
+    p.rsv[63] = 1
+    assert binding.Operation("PagedAttentionOperation", p).status == binding.ERROR_CODE["ERROR_INVALID_PARAM"]
+    r = binding.ReshapeAndCacheParam()
+    r.rsv[0] = 1
+    assert binding.Operation("ReshapeAndCacheOperation", r).status == binding.ERROR_CODE["ERROR_INVALID_PARAM"]
+
+
+def test_names_and_tensor_counts(binding):
+    cases = [
+        (binding.PagedAttentionParam(headNum=8, kvHeadNum=8), 5),
+        (binding.PagedAttentionParam(headNum=8, kvHeadNum=8, quantType=1), 7),
+        (binding.PagedAttentionParam(headNum=8, kvHeadNum=8, quantType=1, hasQuantOffset=True), 9),
+        (binding.PagedAttentionParam(headNum=8, kvHeadNum=1, mlaVHeadSize=512), 4),
+    ]
+    for p, n in cases:
+        op = binding.Operation("PagedAttentionOperation", p)
+        assert op.ok and op.get_name() == "PagedAttentionOperation"
+        assert (op.input_num(), op.output_num()) == (n, 1)
+        op.close()
+    op = binding.Operation("ReshapeAndCacheOperation", binding.ReshapeAndCacheParam())
+    assert op.get_name() == "ReshapeAndCacheOperation" and (op.input_num(), op.output_num()) == (5, 2)
+    op.close()
+    op = binding.Operation("ReshapeAndCacheOperation", binding.ReshapeAndCacheParam(kvCacheCfg=1))
+    assert (op.input_num(), op.output_num()) == (3, 1)
+    op.close()
+
+
+def _c1_pack(binding, lens_host, q_rows=4, tables_rows=4):
+    ins = [
+        binding.make_tensor("float16", [q_rows, 8, 128], FAKE_DEVICE),
+        binding.make_tensor("float16", [64, 128, 8, 128], FAKE_DEVICE),
+        binding.make_tensor("float16", [64, 128, 8, 128], FAKE_DEVICE),
+        binding.make_tensor("int32", [tables_rows, 4], FAKE_DEVICE),
+        binding.make_tensor("int32", [len(lens_host)], FAKE_DEVICE,
+                            host_ptr=lens_host.ctypes.data if lens_host is not None else None),
+    ]
+    outs = [binding.make_tensor("float16", [q_rows, 8, 128], FAKE_DEVICE)]
+    return ins, outs
+
+
+def test_setup_reads_host_context_lens(binding, ctx):
+    op = binding.Operation("PagedAttentionOperation",
+                           binding.PagedAttentionParam(headNum=8, kvHeadNum=8, qkScale=0.088))
+    lens = np.array([469, 339, 432, 71], dtype=np.int32)
+    ins, outs = _c1_pack(binding, lens)
+    st, ws = op.setup(ins, outs, ctx)
+    assert st == 0
+    # missing hostData: the lengths cannot be read (reference param.cpp:16-62)
+    ins[4].hostData = None
+    st, _ = op.setup(ins, outs, ctx)
+    assert binding.ERROR_NAMES[st] == "ERROR_INVALID_PARAM"
+    # a length beyond what the block table can address
+    bad = np.array([469, 339, 4 * 128 + 1, 71], dtype=np.int32)
+    ins, outs = _c1_pack(binding, bad)
+    st, _ = op.setup(ins, outs, ctx)
+    assert binding.ERROR_NAMES[st] == "ERROR_INVALID_PARAM"
+    op.close()
+
+
+def test_setup_workspace_grows_with_split_count(binding, ctx):
+    op = binding.Operation("PagedAttentionOperation",
+                           binding.PagedAttentionParam(headNum=32, kvHeadNum=8, qkScale=0.088))
+
+    def setup(lens):
+        lens = np.asarray(lens, dtype=np.int32)
+        ins = [
+            binding.make_tensor("bf16", [len(lens), 32, 128], FAKE_DEVICE),
+            binding.make_tensor("bf16", [4096, 128, 8, 128], FAKE_DEVICE),
+            binding.make_tensor("bf16", [4096, 128, 8, 128], FAKE_DEVICE),
+            binding.make_tensor("int32", [len(lens), 256], FAKE_DEVICE),
+            binding.make_tensor("int32", [len(lens)], FAKE_DEVICE, host_ptr=lens.ctypes.data),
+        ]
+        outs = [binding.make_tensor("bf16", [len(lens), 32, 128], FAKE_DEVICE)]
+        st, ws = op.setup(ins, outs, ctx)
+        assert st == 0
+        return ws
+
+    short = setup([100] * 4)
+    long = setup([32768] * 4)
+    assert long > short >= 0
+    op.close()
+
+
+def test_setup_and_execute_error_paths(binding, ctx):
+    e = binding.ERROR_CODE
+    op = binding.Operation("PagedAttentionOperation",
+                           binding.PagedAttentionParam(headNum=8, kvHeadNum=8, qkScale=0.088))
+    lens = np.array([469, 339, 432, 71], dtype=np.int32)
+    ins, outs = _c1_pack(binding, lens)
+    # Execute before any Setup
+    assert op.execute(ins, outs, FAKE_DEVICE, 1 << 20, ctx) == e["ERROR_INVALID_PARAM"]
+    # Setup without a context
+    st, _ = op.setup(ins, outs, None)
+    assert st == e["ERROR_INVALID_PARAM"]
+    # wrong tensor count
+    st, _ = op.setup(ins[:4], outs, ctx)
+    assert st == e["ERROR_INVALID_IN_TENSOR_NUM"]
+    st, _ = op.setup(ins, [], ctx)
+    assert st == e["ERROR_INVALID_IN_TENSOR_NUM"]
+    # a zero-sized dim is an invalid tensor size, 9 dims an invalid dim count
+    bad = list(ins)
+    bad[0] = binding.make_tensor("float16", [4, 0, 128], FAKE_DEVICE)
+    st, _ = op.setup(bad, outs, ctx)
+    assert st == e["ERROR_INVALID_TENSOR_SIZE"]
+    bad[0] = binding.make_tensor("float16", [4, 8, 128], FAKE_DEVICE)
+    bad[0].dimNum = 9
+    st, _ = op.setup(bad, outs, ctx)
+    assert st == e["ERROR_INVALID_TENSOR_DIM"]
+    # query head count differs from headNum: caught by the kernel-level checks
+    bad = list(ins)
+    bad[0] = binding.make_tensor("float16", [4, 16, 128], FAKE_DEVICE)
+    st, _ = op.setup(bad, [binding.make_tensor("float16", [4, 16, 128], FAKE_DEVICE)], ctx)
+    assert st == e["ERROR_INVALID_PARAM"]
+
+    st, ws = op.setup(ins, outs, ctx)
+    assert st == 0
+    # a failed Setup invalidates the previous one
+    st, _ = op.setup(ins[:4], outs, ctx)
+    assert st != 0
+    assert op.execute(ins, outs, FAKE_DEVICE, 1 << 20, ctx) == e["ERROR_INVALID_PARAM"]
+
+    st, ws = op.setup(ins, outs, ctx)
+    assert st == 0
+    # different context
+    other = binding.Context(0x2)
+    assert op.execute(ins, outs, FAKE_DEVICE, max(ws, 1), other) == e["ERROR_INVALID_PARAM"]
+    other.close()
+    # workspace too small / null
+    if ws > 0:
+        assert op.execute(ins, outs, FAKE_DEVICE, ws - 1, ctx) == e["ERROR_INVALID_PARAM"]
+        assert op.execute(ins, outs, None, ws, ctx) == e["ERROR_INVALID_PARAM"]
+    # dataSize changed since Setup
+    changed = list(ins)
+    changed[0] = binding.make_tensor("float16", [4, 8, 128], FAKE_DEVICE, data_size=17)
+    assert op.execute(changed, outs, FAKE_DEVICE, max(ws, 1), ctx) == e["ERROR_INVALID_PARAM"]
+    # tensor with no data pointer at all
+    nodata = list(ins)
+    nodata[1] = binding.make_tensor("float16", [64, 128, 8, 128], None)
+    assert op.execute(nodata, outs, FAKE_DEVICE, max(ws, 1), ctx) == e["ERROR_INVALID_PARAM"]
+    # null stream
+    nostream = binding.Context(None)
+    st, ws2 = op.setup(ins, outs, nostream)
+    assert st == 0
+    assert op.execute(ins, outs, FAKE_DEVICE, max(ws2, 1), nostream) == e["ERROR_INVALID_PARAM"]
+    nostream.close()
+    # split execute: LAUNCH without a PRELAUNCH
+    st, ws = op.setup(ins, outs, ctx)
+    ctx.set_execute_type(2)
+    try:
+        assert op.execute(ins, outs, FAKE_DEVICE, max(ws, 1), ctx) == e["ERROR_INVALID_PARAM"]
+    finally:
+        ctx.set_execute_type(0)
+    op.close()
+
+
+def test_dequant_vector_lengths(binding, ctx):
+    e = binding.ERROR_CODE
+    op = binding.Operation("PagedAttentionOperation",
+                           binding.PagedAttentionParam(headNum=32, kvHeadNum=16, quantType=1, qkScale=0.088))
+    lens = np.array([5, 6, 7, 8], dtype=np.int32)
+
+    def pack(n):
+        return [
+            binding.make_tensor("float16", [4, 32, 128], FAKE_DEVICE),
+            binding.make_tensor("int8", [4, 64, 16, 128], FAKE_DEVICE),
+            binding.make_tensor("int8", [4, 64, 16, 128], FAKE_DEVICE),
+            binding.make_tensor("int32", [4, 32], FAKE_DEVICE),
+            binding.make_tensor("int32", [4], FAKE_DEVICE, host_ptr=lens.ctypes.data),
+            binding.make_tensor("float", [n], FAKE_DEVICE),
+            binding.make_tensor("float", [2048], FAKE_DEVICE),
+        ]
+    outs = [binding.make_tensor("float16", [4, 32, 128], FAKE_DEVICE)]
+    assert op.setup(pack(2048), outs, ctx)[0] == 0
+    assert op.setup(pack(128), outs, ctx)[0] == e["ERROR_INVALID_PARAM"]
+    # int64-packed descales are a reference feature that is not implemented here
+    ins = pack(2048)
+    ins[5] = binding.make_tensor("int64", [2048], FAKE_DEVICE)
+    ins[6] = binding.make_tensor("int64", [2048], FAKE_DEVICE)
+    assert op.setup(ins, outs, ctx)[0] == e["ERROR_INVALID_TENSOR_INI_MATCH"]
+    op.close()
+
+
+def test_tensor_size_helper(binding):
+    t = binding.make_tensor("bf16", [3, 5, 7], FAKE_DEVICE)
+    assert t.dataSize == 3 * 5 * 7 * 2
+    assert binding.make_tensor("int64", [4], FAKE_DEVICE).dataSize == 32
+    assert binding.make_tensor("float", [2, 0], FAKE_DEVICE).dataSize == 0
+    t = binding.make_tensor("float", [2, 2], FAKE_DEVICE)
+    t.dimNum = 0
+    assert binding.atb().atb_c_tensor_size(ctypes.byref(t)) == 0
+
+
+def _declared_symbols(header):
+    import re
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(atbmi_[a-z0-9_]+|atb_c_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.mark.parametrize("header,lib", [("atbmi_kernels.h", "libatbmi_kernels.so"), ("atb_capi.h", "libatb.so")])
+def test_every_declared_symbol_is_exported(pkg, header, lib):
+    names = _declared_symbols(header)
+    assert len(names) >= 10
+    path = os.path.join(ROOT, "ascend-transformer-boost_amd", "lib", lib)
+    handle = ctypes.CDLL(path)
+    for n in names:
+        assert hasattr(handle, n), "%s does not export %s" % (lib, n)
+
+
+def test_cpp_api_symbols_are_exported(pkg):
+    """The C++ entry points an ATB caller links against."""
+    path = os.path.join(ROOT, "ascend-transformer-boost_amd", "lib", "libatb.so")
+    out = subprocess.run(["nm", "-DC", "--defined-only", path], stdout=subprocess.PIPE, text=True).stdout
+    for needle in [
+        "atb::CreateOperation<atb::infer::PagedAttentionParam>",
+        "atb::CreateOperation<atb::infer::ReshapeAndCacheParam>",
+        "atb::DestroyOperation(atb::Operation*)",
+        "atb::CreateContext(atb::Context**)",
+        "atb::DestroyContext(atb::Context*)",
+        "atb::Utils::GetTensorSize(atb::TensorDesc const&)",
+        "atb::Utils::GetTensorNumel(atb::Tensor const&)",
+        "atb::Utils::GetAtbVersion",
+    ]:
+        assert needle in out, needle
+
+
+def test_kernel_layer_validates_without_a_gpu(binding):
+    """Argument validation of the C ABI happens before any HIP call."""
+    k = binding.kernels()
+    assert k.atbmi_reshape_and_cache(None, None, None, None, None, 1, 1, 1, 1, 1, 2, None) == 1
+    assert b"non-null" in k.atbmi_last_error()
+    assert k.atbmi_reshape_and_cache(1, None, 1, None, 1, 1, 1, 1, 1, 1, 3, None) == 1
+    assert k.atbmi_quant_per_channel(1, 5, 1, None, 1, 1, 1, None) == 1
+    shape = binding.AtbmiPaShape(qDtype=0, kvDtype=0, numHeads=8, numKvHeads=3, headDimK=128, headDimV=128,
+                                 blockSize=128, numBlocks=4, maxBlocksPerSeq=4, numQueryRows=4, qkScale=1.0)
+    plan = ctypes.c_void_p()
+    assert k.atbmi_pa_plan_create(ctypes.byref(shape), ctypes.byref(plan)) == 1
+    shape.numKvHeads = 8
+    assert k.atbmi_pa_plan_create(ctypes.byref(shape), ctypes.byref(plan)) == 0
+    lens = np.array([100, 0, 512, 7], dtype=np.int32)
+    assert k.atbmi_pa_plan_update(plan, lens.ctypes.data, 4) == 0
+    assert k.atbmi_pa_plan_num_chunks(plan) >= 3
+    # bytes: valid rows * G*(D+Dv)*2 + 3 rows of q/out + table entries + lens
+    want = (100 + 512 + 7) * 8 * 256 * 2 + 3 * 8 * 256 * 2 + (1 + 4 + 1) * 4 + 4 * 4
+    assert k.atbmi_pa_plan_algorithmic_bytes(plan) == want
+    lens[2] = 513
+    assert k.atbmi_pa_plan_update(plan, lens.ctypes.data, 4) == 1
+    k.atbmi_pa_plan_destroy(plan)

@@ -1,0 +1,297 @@
+"""Pins the CPU oracle (oracle/atb_oracle.py) without running any reference code:
+closed forms, exact special cases, an independent float64 loop implementation,
+torch's scaled_dot_product_attention on densely gathered rows, and the
+invariants of paged attention. A plausible oracle mistake (wrong channel
+index for the descale, a missing scale, a transposed operand, advancing the
+query row over an empty sequence) fails at least one test here."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+
+def _rng(seed):
+    return np.random.Generator(np.random.PCG64(seed))
+
+
+def _paged_case(rng, batch=3, heads=4, kv_heads=2, d=16, dv=16, block=4, pool=24, max_ctx=14, dtype=np.float32):
+    ctx = rng.integers(1, max_ctx + 1, size=batch)
+    nblk = (ctx + block - 1) // block
+    perm = rng.permutation(pool)
+    tables = np.zeros((batch, int(nblk.max())), dtype=np.int32)
+    pos = 0
+    for b in range(batch):
+        tables[b, :nblk[b]] = perm[pos:pos + nblk[b]]
+        tables[b, nblk[b]:] = perm[pos]
+        pos += nblk[b]
+    q = rng.standard_normal((batch, heads, d)).astype(dtype)
+    kc = rng.standard_normal((pool, block, kv_heads, d)).astype(dtype)
+    vc = rng.standard_normal((pool, block, kv_heads, dv)).astype(dtype)
+    return q, kc, vc, tables, ctx.astype(np.int32)
+
+
+# ---------------------------------------------------------------- reshape_and_cache
+@pytest.mark.parametrize("dtype,dk,dv", [(np.float16, 8, 8), (np.int8, 12, 6), (np.float32, 5, 9)])
+def test_reshape_and_cache_closed_form(oracle, dtype, dk, dv):
+    rng = _rng(1)
+    tokens, heads, blocks, block = 10, 3, 6, 4
+    key = rng.integers(1, 11, size=(tokens, heads, dk)).astype(dtype)
+    value = rng.integers(1, 11, size=(tokens, heads, dv)).astype(dtype)
+    kc0 = rng.integers(20, 30, size=(blocks, block, heads, dk)).astype(dtype)
+    vc0 = rng.integers(20, 30, size=(blocks, block, heads, dv)).astype(dtype)
+    # unique slots drawn from [-N, N): negatives must be skipped
+    slots = rng.choice(np.arange(-blocks * block, blocks * block), size=tokens, replace=False).astype(np.int32)
+    kc, vc = oracle.reshape_and_cache(key, value, kc0, vc0, slots)
+    ek = kc0.copy().reshape(blocks * block, heads * dk)
+    ev = vc0.copy().reshape(blocks * block, heads * dv)
+    keep = slots >= 0
+    ek[slots[keep]] = key[keep].reshape(-1, heads * dk)
+    ev[slots[keep]] = value[keep].reshape(-1, heads * dv)
+    assert np.array_equal(kc.reshape(ek.shape), ek)
+    assert np.array_equal(vc.reshape(ev.shape), ev)
+    assert (slots < 0).any() and keep.any()
+    # inputs are not modified, untouched slots keep their content
+    untouched = np.setdiff1d(np.arange(blocks * block), slots[keep])
+    assert np.array_equal(kc.reshape(ek.shape)[untouched], kc0.reshape(ek.shape)[untouched])
+
+
+def test_reshape_and_cache_single_cache(oracle):
+    key = np.arange(2 * 1 * 4, dtype=np.float32).reshape(2, 1, 4)
+    kc0 = np.zeros((2, 2, 1, 4), dtype=np.float32)
+    kc, vc = oracle.reshape_and_cache(key, None, kc0, None, np.array([3, -1], dtype=np.int32))
+    assert vc is None
+    assert np.array_equal(kc[1, 1, 0], key[0, 0]) and kc.sum() == key[0].sum()
+
+
+# ---------------------------------------------------------------- quantiser
+def test_quant_special_cases(oracle):
+    s = np.float32(0.5)
+    x = np.array([0.25, 0.75, 1.25, -0.25, -0.75, -1.25, 0.0, -0.0, 1000.0, -1000.0, np.inf, -np.inf, np.nan,
+                  63.5, 63.75, -64.0, -64.25, 6e-8], dtype=np.float32)
+    #            0.5->0 1.5->2 2.5->2 -0.5->0 -1.5->-2 -2.5->-2
+    want = np.array([0, 2, 2, 0, -2, -2, 0, 0, 127, -128, 127, -128, 0, 127, 127, -128, -128, 0], dtype=np.int8)
+    assert np.array_equal(oracle.quant_per_channel(x, s), want)
+    # offset is added after rounding and before the clamp
+    assert np.array_equal(oracle.quant_per_channel(x[:3], s, np.array([3, -3, 126])), np.array([3, -1, 127], np.int8))
+
+
+def test_quant_exact_rational(oracle):
+    """x/s rounded to fp32 then to the nearest-even integer, checked against exact
+    rational arithmetic for every fp16 x on a few scales."""
+    from fractions import Fraction
+    bits = np.arange(0, 65536, 37, dtype=np.uint16)  # a stride through all patterns, both signs
+    x = bits.view(np.float16)
+    x = x[np.isfinite(x)]
+    for s in [np.float32(0.005), np.float32(0.0123), np.float32(0.02), np.float32(1.0), np.float32(3.0)]:
+        got = oracle.quant_per_channel(x.astype(np.float32), s)
+        for xi, gi in zip(x.tolist(), got.tolist()):
+            quot = Fraction(xi) / Fraction(float(s))
+            f32 = np.float32(float(quot))  # double then single: both roundings checked below
+            # guard against double rounding: the exact quotient must not sit on an fp32 tie
+            lo, hi = np.nextafter(f32, np.float32(-np.inf)), np.nextafter(f32, np.float32(np.inf))
+            assert abs(quot - Fraction(float(f32))) <= min(abs(quot - Fraction(float(lo))),
+                                                           abs(quot - Fraction(float(hi))))
+            fr = Fraction(float(f32))
+            fl = math.floor(fr)
+            rem = fr - fl
+            r = fl if rem < Fraction(1, 2) else fl + 1 if rem > Fraction(1, 2) else (fl if fl % 2 == 0 else fl + 1)
+            assert gi == max(-128, min(127, r)), (xi, float(s))
+
+
+def test_quant_all_fp16_patterns_vs_golden_dtype(oracle):
+    """The reference golden divides in fp16 and is accepted with atol=1; the fp32
+    form must stay within that band for every finite fp16 input, and be monotone."""
+    x = np.arange(65536, dtype=np.uint16).view(np.float16)
+    x = x[np.isfinite(x)]
+    for s in [0.1, 0.37, 1.0]:
+        a = oracle.quant_per_channel(x.astype(np.float32), np.float32(np.float16(s))).astype(np.int32)
+        b = oracle.quant_per_channel_golden_dtype(x, np.float16(s)).astype(np.int32)
+        assert np.abs(a - b).max() <= 1
+        order = np.argsort(x.astype(np.float32), kind="stable")
+        assert (np.diff(a[order]) >= 0).all()
+
+
+def test_quant_per_channel_axis(oracle):
+    x = np.ones((3, 4), dtype=np.float32)
+    s = np.array([1.0, 0.5, 0.25, 0.125], dtype=np.float32)
+    assert np.array_equal(oracle.quant_per_channel(x, s), np.tile(np.array([1, 2, 4, 8], np.int8), (3, 1)))
+
+
+# ---------------------------------------------------------------- attention
+def test_attention_matches_independent_loops(oracle):
+    rng = _rng(2)
+    q, kc, vc, tables, ctx = _paged_case(rng)
+    scale = 1.0 / math.sqrt(q.shape[2])
+    got = oracle.paged_attention(q, kc, vc, tables, ctx, scale)
+    want = oracle.paged_attention_loops(q, kc, vc, tables, ctx, scale)
+    np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-6)
+
+
+def test_attention_matches_torch_sdpa(oracle):
+    """Gathering the rows densely reduces the op to textbook attention."""
+    rng = _rng(3)
+    q, kc, vc, tables, ctx = _paged_case(rng, batch=4, heads=6, kv_heads=3, d=32, dv=24, block=8, pool=40, max_ctx=50)
+    scale = 0.37
+    got = oracle.paged_attention(q, kc, vc, tables, ctx, scale)
+    group = q.shape[1] // kc.shape[2]
+    for b in range(len(ctx)):
+        j = np.arange(ctx[b])
+        k = kc[tables[b][j // 8], j % 8]  # [ctx, G, D]
+        v = vc[tables[b][j // 8], j % 8]
+        kt = torch.from_numpy(np.repeat(k, group, axis=1)).double().permute(1, 0, 2)  # [H, ctx, D]
+        vt = torch.from_numpy(np.repeat(v, group, axis=1)).double().permute(1, 0, 2)
+        qt = torch.from_numpy(q[b]).double().unsqueeze(1)  # [H, 1, D]
+        ref = torch.nn.functional.scaled_dot_product_attention(qt, kt, vt, scale=scale).squeeze(1).numpy()
+        np.testing.assert_allclose(got[b], ref, rtol=2e-5, atol=2e-6)
+
+
+def test_attention_block_permutation_invariance(oracle):
+    rng = _rng(4)
+    q, kc, vc, tables, ctx = _paged_case(rng)
+    base = oracle.paged_attention(q, kc, vc, tables, ctx, 0.25)
+    perm = rng.permutation(kc.shape[0])
+    inv = np.empty_like(perm)
+    inv[perm] = np.arange(len(perm))
+    moved = oracle.paged_attention(q, kc[perm], vc[perm], inv[tables].astype(np.int32), ctx, 0.25)
+    assert np.array_equal(base, moved)
+
+
+def test_attention_ctx1_returns_value_row(oracle):
+    rng = _rng(5)
+    q, kc, vc, tables, _ = _paged_case(rng)
+    ctx = np.ones(len(tables), dtype=np.int32)
+    out = oracle.paged_attention(q, kc, vc, tables, ctx, 0.3)
+    group = q.shape[1] // kc.shape[2]
+    for b in range(len(ctx)):
+        assert np.array_equal(out[b], np.repeat(vc[tables[b, 0], 0], group, axis=0))
+
+
+def test_attention_equal_keys_gives_mean_of_values(oracle):
+    rng = _rng(6)
+    q, kc, vc, tables, ctx = _paged_case(rng)
+    kc[:] = kc[0, 0]
+    out = oracle.paged_attention(q, kc, vc, tables, ctx, 0.3)
+    group = q.shape[1] // kc.shape[2]
+    for b in range(len(ctx)):
+        j = np.arange(ctx[b])
+        mean = vc[tables[b][j // 4], j % 4].mean(axis=0)
+        np.testing.assert_allclose(out[b], np.repeat(mean, group, axis=0), rtol=1e-5, atol=1e-6)
+
+
+def test_attention_gqa_equals_replicated_mha(oracle):
+    rng = _rng(7)
+    q, kc, vc, tables, ctx = _paged_case(rng, heads=6, kv_heads=2)
+    gqa = oracle.paged_attention(q, kc, vc, tables, ctx, 0.2)
+    mha = oracle.paged_attention(q, np.repeat(kc, 3, axis=2), np.repeat(vc, 3, axis=2), tables, ctx, 0.2)
+    np.testing.assert_allclose(gqa, mha, rtol=1e-5, atol=1e-6)
+
+
+def test_attention_scale_is_applied_to_scores(oracle):
+    rng = _rng(8)
+    q, kc, vc, tables, ctx = _paged_case(rng)
+    a = oracle.paged_attention(q, kc, vc, tables, ctx, 0.5)
+    b = oracle.paged_attention(q * 0.5, kc, vc, tables, ctx, 1.0)
+    np.testing.assert_allclose(a, b, rtol=1e-5, atol=1e-6)
+    assert np.abs(a - oracle.paged_attention(q, kc, vc, tables, ctx, 1.0)).max() > 1e-3
+
+
+def test_attention_ignores_rows_past_context_and_unused_blocks(oracle):
+    rng = _rng(9)
+    q, kc, vc, tables, ctx = _paged_case(rng)
+    base = oracle.paged_attention(q, kc, vc, tables, ctx, 0.25)
+    kc2, vc2 = kc.copy(), vc.copy()
+    used = np.zeros(kc.shape[:2], dtype=bool)
+    for b in range(len(ctx)):
+        j = np.arange(ctx[b])
+        used[tables[b][j // 4], j % 4] = True
+    kc2[~used] = np.nan
+    vc2[~used] = np.nan
+    out = oracle.paged_attention(q, kc2, vc2, tables, ctx, 0.25)
+    assert np.array_equal(base, out) and (~used).any()
+
+
+def test_attention_empty_sequences_take_no_query_row(oracle):
+    rng = _rng(10)
+    q, kc, vc, tables, ctx = _paged_case(rng, batch=4)
+    dense = oracle.paged_attention(q, kc, vc, tables, ctx, 0.25)
+    ctx2 = ctx.copy()
+    ctx2[1] = 0
+    out = oracle.paged_attention(q, kc, vc, tables, ctx2, 0.25, out_init=0.1)
+    # sequences 0,2,3 use query rows 0,1,2; row 3 is never written
+    assert np.array_equal(out[0], dense[0])
+    want1 = oracle.paged_attention(q[1:2], kc, vc, tables[2:3], ctx[2:3], 0.25)[0]
+    assert np.array_equal(out[1], want1)
+    assert np.all(out[3] == np.float32(0.1))
+
+
+def test_int8_dequant_channel_indexing_and_identity(oracle):
+    rng = _rng(11)
+    q, _, _, tables, ctx = _paged_case(rng, heads=4, kv_heads=2, d=8, dv=8)
+    kc8 = rng.integers(-20, 21, size=(24, 4, 2, 8)).astype(np.int8)
+    vc8 = rng.integers(-20, 21, size=(24, 4, 2, 8)).astype(np.int8)
+    # scale 1, offset 0 equals the float path on integer-valued caches
+    ones = np.ones(16, dtype=np.float32)
+    a = oracle.paged_attention(q, kc8, vc8, tables, ctx, 0.1, ones, None, ones, None)
+    b = oracle.paged_attention(q, kc8.astype(np.float32), vc8.astype(np.float32), tables, ctx, 0.1)
+    assert np.array_equal(a, b)
+    # per-(kv head, channel) vectors: channel index is g*D + d
+    ks = rng.uniform(0.5, 2.0, size=16).astype(np.float32)
+    vs = rng.uniform(0.5, 2.0, size=16).astype(np.float32)
+    ko = rng.integers(-5, 6, size=16).astype(np.int32)
+    vo = rng.integers(-5, 6, size=16).astype(np.int32)
+    got = oracle.paged_attention(q, kc8, vc8, tables, ctx, 0.1, ks, ko, vs, vo)
+    kf = (kc8.astype(np.float32) + ko.reshape(2, 8)) * ks.reshape(2, 8)
+    vf = (vc8.astype(np.float32) + vo.reshape(2, 8)) * vs.reshape(2, 8)
+    want = oracle.paged_attention(q, kf, vf, tables, ctx, 0.1)
+    np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-6)
+    # a key offset shifts every score of a head equally and so cannot change the output
+    nok = oracle.paged_attention(q, kc8, vc8, tables, ctx, 0.1, ks, None, vs, vo)
+    np.testing.assert_allclose(got, nok, rtol=1e-4, atol=1e-5)
+
+
+def test_mla_equals_generic_with_materialised_values(oracle):
+    rng = _rng(12)
+    q, kc, _, tables, ctx = _paged_case(rng, heads=8, kv_heads=1, d=24, dv=16)
+    a = oracle.paged_attention(q, kc, None, tables, ctx, 0.2, mla_v_head_size=16)
+    b = oracle.paged_attention(q, kc, np.ascontiguousarray(kc[..., :16]), tables, ctx, 0.2)
+    assert np.array_equal(a, b) and a.shape == (3, 8, 16)
+
+
+def test_q_scale_rounds_in_query_dtype(oracle):
+    rng = _rng(13)
+    q, kc, vc, tables, ctx = _paged_case(rng)
+    q = q.astype(np.float16).astype(np.float32)
+    a = oracle.paged_attention(q, kc, vc, tables, ctx, 0.25, q_scale=0.3, q_dtype="float16")
+    b = oracle.paged_attention((q * np.float32(0.3)).astype(np.float16).astype(np.float32), kc, vc, tables, ctx, 0.25)
+    assert np.array_equal(a, b)
+    for noop in (0.0, 1.0):
+        assert np.array_equal(oracle.paged_attention(q, kc, vc, tables, ctx, 0.25, q_scale=noop),
+                              oracle.paged_attention(q, kc, vc, tables, ctx, 0.25))
+
+
+def test_split_kv_merge_equals_single_pass(oracle):
+    rng = _rng(14)
+    ctx = 53
+    q = rng.standard_normal((6, 16)).astype(np.float32)
+    keys = rng.standard_normal((ctx, 2, 16)).astype(np.float32) * 3
+    values = rng.standard_normal((ctx, 2, 8)).astype(np.float32)
+    full = oracle.attention_one(q, keys, values, 0.3)
+    for cuts in ([0, 53], [0, 1, 53], [0, 20, 21, 40, 53], list(range(0, 54))):
+        outs, lses = [], []
+        for a, b in zip(cuts[:-1], cuts[1:]):
+            o, l = oracle.partial_attention(q, keys[a:b], values[a:b], 0.3)
+            outs.append(o)
+            lses.append(l)
+        # an empty split contributes nothing
+        outs.append(np.full_like(outs[0], 7.0))
+        lses.append(np.full_like(lses[0], -np.inf))
+        np.testing.assert_allclose(oracle.merge_partials(outs, lses), full, rtol=2e-6, atol=2e-6)
+
+
+def test_bf16_round(oracle):
+    x = np.array([1.0, 1.00390625, 1.0 + 2 ** -8, 1.0 + 3 * 2 ** -8, -2.5, 3.0e38, 1e-40], dtype=np.float32)
+    want = torch.from_numpy(x).to(torch.bfloat16).float().numpy()
+    assert np.array_equal(oracle.bf16_round(x), want)
+    big = _rng(15).standard_normal(10000).astype(np.float32) * 100
+    assert np.array_equal(oracle.bf16_round(big), torch.from_numpy(big).to(torch.bfloat16).float().numpy())
