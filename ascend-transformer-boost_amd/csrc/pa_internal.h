@@ -24,6 +24,12 @@ int LaunchPaScalar(const AtbmiPaShape &shape, const PaArgs &args, int numItems, 
 // MFMA kernel: head sizes and block sizes listed by PaMfmaSupports.
 bool PaMfmaSupports(const AtbmiPaShape &shape);
 int LaunchPaMfma(const AtbmiPaShape &shape, const PaArgs &args, int numItems, hipStream_t stream);
+// Per-operand-type halves of LaunchPaMfma (one translation unit each, so the
+// instantiations compile in parallel). Return -1 when the shape has no
+// instantiation.
+int LaunchPaMfmaF16(const AtbmiPaShape &shape, const PaArgs &args, int numItems, hipStream_t stream);
+int LaunchPaMfmaBf16(const AtbmiPaShape &shape, const PaArgs &args, int numItems, hipStream_t stream);
+int LaunchPaMfmaInt8(const AtbmiPaShape &shape, const PaArgs &args, int numItems, hipStream_t stream);
 
 // Merges the partials of every sequence that has more than one.
 int LaunchPaReduce(const AtbmiPaShape &shape, const PaArgs &args, int numSeqs, hipStream_t stream);

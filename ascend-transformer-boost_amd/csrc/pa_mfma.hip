@@ -1,9 +1,41 @@
-// placeholder until the MFMA kernel lands
+// Shape coverage and dispatch of the MFMA decode-attention kernel.
 #include "pa_internal.h"
+
 namespace atbmi {
-bool PaMfmaSupports(const AtbmiPaShape &) { return false; }
-int LaunchPaMfma(const AtbmiPaShape &, const PaArgs &, int, hipStream_t)
+
+bool PaMfmaSupports(const AtbmiPaShape &s)
 {
-    return Fail(ERR_INVALID_PARAM, "pa_decode: MFMA kernel not built");
+    if (s.blockSize % 16 != 0) {
+        return false; // a 16-token sub-tile must not straddle cache blocks
+    }
+    const int d = s.headDimK;
+    const int dv = s.headDimV;
+    if (s.mlaCombined) {
+        return s.kvDtype != ATBMI_INT8 && ((d == 576 && dv == 512) || (d == 192 && dv == 128));
+    }
+    if (d != dv) {
+        return false;
+    }
+    if (s.kvDtype == ATBMI_INT8) {
+        return d == 64 || d == 128 || d == 256;
+    }
+    return d == 64 || d == 96 || d == 128 || d == 256;
 }
+
+int LaunchPaMfma(const AtbmiPaShape &s, const PaArgs &args, int numItems, hipStream_t stream)
+{
+    int rc;
+    if (s.kvDtype == ATBMI_INT8) {
+        rc = LaunchPaMfmaInt8(s, args, numItems, stream);
+    } else if (s.qDtype == ATBMI_BF16) {
+        rc = LaunchPaMfmaBf16(s, args, numItems, stream);
+    } else {
+        rc = LaunchPaMfmaF16(s, args, numItems, stream);
+    }
+    if (rc < 0) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: no MFMA kernel for head sizes %d/%d", s.headDimK, s.headDimV);
+    }
+    return rc;
+}
+
 } // namespace atbmi

@@ -1,0 +1,25 @@
+// MFMA decode-attention instantiations for int8 caches (fp16 or bf16 queries;
+// the matrix cores run in fp16 either way, int8 values are exact in fp16).
+#include "pa_mfma_kernel.h"
+
+namespace atbmi {
+
+int LaunchPaMfmaInt8(const AtbmiPaShape &s, const PaArgs &args, int numItems, hipStream_t stream)
+{
+    using namespace mfma;
+    if (s.mlaCombined || s.headDimK != s.headDimV) {
+        return -1;
+    }
+    switch (s.headDimK) {
+        case 64:
+            return Launch<false, true, 64, 64, false, true>(args, numItems, stream);
+        case 128:
+            return Launch<false, true, 128, 128, false, true>(args, numItems, stream);
+        case 256:
+            return Launch<false, true, 256, 256, false, true>(args, numItems, stream);
+        default:
+            return -1;
+    }
+}
+
+} // namespace atbmi
