@@ -77,6 +77,49 @@ struct PaArgs {
     int32_t finishV;     // 1: partial outputs are still in int8 units; the final write applies vScale/vOff
 };
 
+// ---- Plan of the MFMA kernel ------------------------------------------------
+// The KV rows of all non-empty sequences, cut into 32-token steps, form one
+// linear step space [0, totalSteps). It is divided evenly into numWaveRanges
+// contiguous ranges; one wave walks one range for one KV head (or one tile of
+// 16 query heads of it), crossing sequence boundaries where they fall. The
+// device only needs where each sequence starts in that space.
+constexpr int PA_INLINE_SEQS = 192;   // plans up to this many sequences travel in the kernel arguments
+constexpr int PA_INLINE_RANGES = 512; // workgroup ranges whose first sequence is tabulated inline
+
+struct PaSeq {
+    int32_t tableRow;  // row of blockTables (index of the sequence in the batch)
+    int32_t ctxLen;    // tokens
+    int32_t stepBegin; // first step of this sequence in the linear step space
+};
+
+struct PaStreamPlan {
+    const PaSeq *seqs;        // numSeqs + 1 entries (the last one only carries stepBegin = totalSteps);
+                              // null: use inlineSeqs
+    const uint16_t *firstSeq; // per workgroup range: sequence holding its first step; null: use inlineFirst
+    int32_t numSeqs;          // non-empty sequences; the i-th one uses query/output row i
+    int32_t totalSteps;
+    int32_t numWaveRanges;    // numWgRanges * tokenSlices
+    int32_t numWgRanges;
+    int32_t tokenSlices;      // consecutive wave ranges one workgroup covers (waves / headsPerWg)
+    int32_t headsPerWg;       // virtual heads (KV head x query-head tile) one workgroup covers
+    int32_t headGroups;       // virtual heads / headsPerWg
+    int32_t headTiles;        // query-head tiles per KV head
+    PaSeq inlineSeqs[PA_INLINE_SEQS + 1];
+    uint16_t inlineFirst[PA_INLINE_RANGES];
+};
+
+// First step of wave range `wr`: ranges differ by at most one step.
+__host__ __device__ __forceinline__ int32_t PaRangeBegin(int32_t wr, int32_t totalSteps, int32_t numWaveRanges)
+{
+    return static_cast<int32_t>(static_cast<int64_t>(wr) * totalSteps / numWaveRanges);
+}
+
+// The wave range that holds step `s`.
+__host__ __device__ __forceinline__ int32_t PaRangeOf(int32_t s, int32_t totalSteps, int32_t numWaveRanges)
+{
+    return static_cast<int32_t>(((static_cast<int64_t>(s) + 1) * numWaveRanges - 1) / totalSteps);
+}
+
 __device__ __forceinline__ float Bf16ToFloat(uint16_t v)
 {
     return __uint_as_float(static_cast<uint32_t>(v) << 16);

@@ -68,10 +68,19 @@ using namespace atbmi;
 struct AtbmiPaPlan {
     AtbmiPaShape shape;
     bool useMfma = false;
-    int headTile = 1;        // query heads per workgroup
-    int partialsPerItem = 1; // partial slots one work item writes
-    int tokenUnit = 1;       // chunk lengths are multiples of this
+    int headTile = 1;        // query heads per workgroup (scalar kernel) or wave (MFMA kernel)
+    int partialsPerItem = 1; // scalar kernel: partial slots one work item writes
+    int tokenUnit = 1;       // scalar kernel: chunk lengths are multiples of this
+    int mfmaWaves = 8;       // MFMA kernel: waves per workgroup
     int64_t chunkOverride = 0;
+    int64_t minStepsOverride = 0;
+
+    // MFMA kernel: the stream plan (see PaStreamPlan) and its host-side pieces
+    PaStreamPlan stream{};
+    std::vector<PaSeq> seqTable;       // numSeqs + 1 entries
+    std::vector<uint16_t> firstSeq;    // one per workgroup range
+    bool streamInline = true;          // the tables fit into the kernel arguments
+    bool streamNeedsReduce = false;
 
     std::vector<PaWorkItem> items;
     std::vector<PaSeqInfo> reduceSeqs;
@@ -158,17 +167,147 @@ extern "C" int atbmi_pa_plan_create(const AtbmiPaShape *shape, AtbmiPaPlan **pla
     p->useMfma = (kernel == ATBMI_PA_KERNEL_MFMA) || (kernel == ATBMI_PA_KERNEL_AUTO && mfmaOk);
     if (p->useMfma) {
         p->headTile = PA_MFMA_HEAD_TILE;
-        p->partialsPerItem = 1;
-        p->tokenUnit = PA_MFMA_STEP * PA_MFMA_WAVES;
+        p->mfmaWaves = PaMfmaWaves(s);
     } else {
         p->headTile = PA_SCALAR_HEAD_TILE;
         p->partialsPerItem = PA_SCALAR_WAVES;
         p->tokenUnit = PA_SCALAR_WAVES;
     }
     p->chunkOverride = EnvInt("ATBMI_PA_CHUNK_TOKENS", 0);
+    p->minStepsOverride = EnvInt("ATBMI_PA_MIN_STEPS", 0);
     *plan = p;
     return OK;
 }
+
+
+namespace {
+
+// Stream plan of the MFMA kernel: every wave gets an equal share of the linear
+// step space (32-token steps of all non-empty sequences, back to back).
+int PlanStream(AtbmiPaPlan *plan, const int32_t *ctx, int32_t batch)
+{
+    const AtbmiPaShape &s = plan->shape;
+    const int groupSize = s.numHeads / s.numKvHeads;
+    const int headTiles = (groupSize + PA_MFMA_HEAD_TILE - 1) / PA_MFMA_HEAD_TILE;
+    const int virtualHeads = s.numKvHeads * headTiles;
+    const int waves = plan->mfmaWaves;
+    // The waves of a workgroup take different heads of one token range when the
+    // head count allows it, so that the CU reads whole cache rows.
+    int headsPerWg = waves;
+    while (virtualHeads % headsPerWg != 0) {
+        headsPerWg >>= 1;
+    }
+    const int tokenSlices = waves / headsPerWg;
+    const int headGroups = virtualHeads / headsPerWg;
+    try {
+        plan->seqTable.clear();
+        int64_t steps = 0;
+        for (int32_t b = 0; b < batch; ++b) {
+            if (ctx[b] == 0) {
+                continue;
+            }
+            PaSeq sq{};
+            sq.tableRow = b;
+            sq.ctxLen = ctx[b];
+            sq.stepBegin = static_cast<int32_t>(steps);
+            plan->seqTable.push_back(sq);
+            steps += (ctx[b] + PA_MFMA_STEP - 1) / PA_MFMA_STEP;
+            if (steps > 0x3fffffff) {
+                return Fail(ERR_INVALID_PARAM, "pa_plan_update: too many KV tokens for one call");
+            }
+        }
+        PaSeq sentinel{};
+        sentinel.stepBegin = static_cast<int32_t>(steps);
+        plan->seqTable.push_back(sentinel);
+        const int numSeqs = static_cast<int>(plan->seqTable.size()) - 1;
+
+        // One workgroup per CU and head group is the most that runs at once;
+        // short batches use fewer so that a wave still has a few steps to do.
+        const int64_t minSteps = plan->minStepsOverride > 0 ? plan->minStepsOverride : 2;
+        int64_t wgRanges = std::max<int64_t>(1, NUM_CUS / headGroups);
+        if (plan->chunkOverride > 0) {
+            // test hook: ranges of about this many tokens
+            const int64_t per = std::max<int64_t>(1, plan->chunkOverride / PA_MFMA_STEP) * tokenSlices;
+            wgRanges = std::max<int64_t>(1, (steps + per - 1) / per);
+        } else {
+            const int64_t cap = std::max<int64_t>(1, steps / (minSteps * tokenSlices));
+            wgRanges = std::min(wgRanges, cap);
+        }
+        if (wgRanges * tokenSlices > 0x3fffffff / 2) {
+            return Fail(ERR_INVALID_PARAM, "pa_plan_update: too many ranges");
+        }
+        const int32_t waveRanges = static_cast<int32_t>(wgRanges * tokenSlices);
+
+        plan->firstSeq.assign(static_cast<size_t>(wgRanges), 0);
+        int cursor = 0;
+        for (int64_t r = 0; r < wgRanges; ++r) {
+            const int32_t begin = PaRangeBegin(static_cast<int32_t>(r * tokenSlices), static_cast<int32_t>(steps),
+                                               waveRanges);
+            while (cursor + 1 < numSeqs && plan->seqTable[cursor + 1].stepBegin <= begin) {
+                ++cursor;
+            }
+            plan->firstSeq[static_cast<size_t>(r)] = static_cast<uint16_t>(std::min(cursor, 0xffff));
+        }
+        plan->streamNeedsReduce = false;
+        for (int i = 0; i < numSeqs; ++i) {
+            const int32_t first = PaRangeOf(plan->seqTable[i].stepBegin, static_cast<int32_t>(steps), waveRanges);
+            const int32_t last = PaRangeOf(plan->seqTable[i + 1].stepBegin - 1, static_cast<int32_t>(steps), waveRanges);
+            if (first != last) {
+                plan->streamNeedsReduce = true;
+                break;
+            }
+        }
+
+        PaStreamPlan &sp = plan->stream;
+        sp = PaStreamPlan{};
+        sp.numSeqs = numSeqs;
+        sp.totalSteps = static_cast<int32_t>(steps);
+        sp.numWaveRanges = waveRanges;
+        sp.numWgRanges = static_cast<int32_t>(wgRanges);
+        sp.tokenSlices = tokenSlices;
+        sp.headsPerWg = headsPerWg;
+        sp.headGroups = headGroups;
+        sp.headTiles = headTiles;
+        // firstSeq is a 16-bit table: batches beyond 65535 sequences go through memory as 16-bit too,
+        // so they are refused here rather than silently truncated
+        if (numSeqs > 0xffff) {
+            return Fail(ERR_INVALID_PARAM, "pa_plan_update: more than 65535 non-empty sequences");
+        }
+        plan->streamInline = numSeqs <= PA_INLINE_SEQS && wgRanges <= PA_INLINE_RANGES;
+        const uint64_t seqBytes = plan->seqTable.size() * sizeof(PaSeq);
+        const uint64_t firstBytes = plan->firstSeq.size() * sizeof(uint16_t);
+        if (plan->streamInline) {
+            memcpy(sp.inlineSeqs, plan->seqTable.data(), seqBytes);
+            memcpy(sp.inlineFirst, plan->firstSeq.data(), firstBytes);
+            plan->blobBytes = 0;
+            plan->blob.clear();
+            plan->offItems = plan->offSeqs = 0;
+        } else {
+            plan->offItems = 0; // sequence table
+            plan->offSeqs = AlignUp(seqBytes, 16); // first-sequence table
+            plan->blobBytes = plan->offSeqs + firstBytes;
+            plan->blob.assign(plan->blobBytes, 0);
+            memcpy(plan->blob.data() + plan->offItems, plan->seqTable.data(), seqBytes);
+            memcpy(plan->blob.data() + plan->offSeqs, plan->firstSeq.data(), firstBytes);
+        }
+    } catch (const std::bad_alloc &) {
+        return Fail(ERR_OUT_OF_HOST_MEMORY, "pa_plan_update: out of host memory");
+    }
+    plan->items.clear();
+    plan->reduceSeqs.clear();
+    const uint64_t slots = plan->streamNeedsReduce ? 2ull * plan->stream.numWaveRanges : 0;
+    plan->numPartials = static_cast<int64_t>(slots);
+    plan->offPartO = AlignUp(plan->blobBytes, WS_ALIGN);
+    const uint64_t partOBytes = slots * s.numHeads * s.headDimV * sizeof(float);
+    plan->offPartLse = AlignUp(plan->offPartO + partOBytes, WS_ALIGN);
+    plan->wsBytes = AlignUp(plan->offPartLse + slots * s.numHeads * sizeof(float), WS_ALIGN);
+    if (plan->blobBytes == 0 && slots == 0) {
+        plan->wsBytes = 0;
+    }
+    return OK;
+}
+
+} // namespace
 
 extern "C" int atbmi_pa_plan_update(AtbmiPaPlan *plan, const int32_t *ctx, int32_t batch)
 {
@@ -203,6 +342,10 @@ extern "C" int atbmi_pa_plan_update(AtbmiPaPlan *plan, const int32_t *ctx, int32
     plan->nonEmpty = nonEmpty;
     plan->items.clear();
     plan->reduceSeqs.clear();
+
+    if (plan->useMfma) {
+        return PlanStream(plan, ctx, batch);
+    }
 
     // Chunk length: enough workgroups to load every CU several times over,
     // but chunks long enough that the per-chunk prologue/epilogue stays small.
@@ -290,7 +433,11 @@ extern "C" uint64_t atbmi_pa_plan_workspace_size(const AtbmiPaPlan *plan)
 
 extern "C" int64_t atbmi_pa_plan_num_chunks(const AtbmiPaPlan *plan)
 {
-    return plan ? static_cast<int64_t>(plan->items.size()) : 0;
+    if (!plan) {
+        return 0;
+    }
+    return plan->useMfma ? static_cast<int64_t>(plan->stream.numWaveRanges)
+                         : static_cast<int64_t>(plan->items.size());
 }
 
 extern "C" uint64_t atbmi_pa_plan_algorithmic_bytes(const AtbmiPaPlan *plan)
@@ -374,7 +521,7 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
         return Fail(ERR_INVALID_PARAM, "pa_decode: null argument");
     }
     const AtbmiPaShape &s = plan->shape;
-    if (plan->items.empty()) {
+    if (plan->nonEmpty == 0) {
         return OK; // every sequence is empty: nothing is written
     }
     if (!t->query || !t->keyCache || !t->blockTables || !t->out || (!s.mlaCombined && !t->valueCache)) {
@@ -390,7 +537,7 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
         return Fail(ERR_INVALID_PARAM, "pa_decode: workspace of %llu bytes, %llu needed",
                     (unsigned long long)workspaceBytes, (unsigned long long)plan->wsBytes);
     }
-    if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0) {
+    if (plan->wsBytes > 0 && reinterpret_cast<uintptr_t>(workspace) % 16 != 0) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: workspace must be 16-byte aligned");
     }
     hipStream_t stream = static_cast<hipStream_t>(streamHandle);
@@ -441,7 +588,14 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
         ATBMI_HIP_CHECK(hipEventRecord(rec.begin, stream));
     }
     const int numItems = static_cast<int>(plan->items.size());
-    rc = plan->useMfma ? LaunchPaMfma(s, a, numItems, stream) : LaunchPaScalar(s, a, numItems, stream);
+    PaStreamPlan &sp = plan->stream;
+    if (plan->useMfma) {
+        sp.seqs = plan->streamInline ? nullptr : reinterpret_cast<const PaSeq *>(ws + plan->offItems);
+        sp.firstSeq = plan->streamInline ? nullptr : reinterpret_cast<const uint16_t *>(ws + plan->offSeqs);
+        rc = LaunchPaMfma(s, a, sp, stream);
+    } else {
+        rc = LaunchPaScalar(s, a, numItems, stream);
+    }
     if (timed) {
         ATBMI_HIP_CHECK(hipEventRecord(rec.end, stream));
         std::lock_guard<std::mutex> lock(g_timingMutex);
@@ -449,6 +603,9 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
     }
     if (rc != OK) {
         return rc;
+    }
+    if (plan->useMfma) {
+        return plan->streamNeedsReduce ? LaunchPaStreamReduce(s, a, sp, stream) : OK;
     }
     return LaunchPaReduce(s, a, static_cast<int>(plan->reduceSeqs.size()), stream);
 }

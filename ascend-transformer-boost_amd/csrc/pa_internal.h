@@ -11,10 +11,9 @@ constexpr int PA_SCALAR_WAVES = 4;
 // Query heads one scalar-kernel workgroup handles.
 constexpr int PA_SCALAR_HEAD_TILE = 8;
 
-// Tokens one MFMA-kernel wave consumes per step, waves per workgroup, and
-// query heads per workgroup (the N extent of a 16x16 MFMA tile).
+// Tokens one MFMA-kernel wave consumes per step and query heads per wave
+// (the N extent of a 16x16 MFMA tile).
 constexpr int PA_MFMA_STEP = 32;
-constexpr int PA_MFMA_WAVES = 4;
 constexpr int PA_MFMA_HEAD_TILE = 16;
 
 // Scalar (VALU) kernel: any head size up to 576, any block size, any group.
@@ -23,16 +22,22 @@ int LaunchPaScalar(const AtbmiPaShape &shape, const PaArgs &args, int numItems, 
 
 // MFMA kernel: head sizes and block sizes listed by PaMfmaSupports.
 bool PaMfmaSupports(const AtbmiPaShape &shape);
-int LaunchPaMfma(const AtbmiPaShape &shape, const PaArgs &args, int numItems, hipStream_t stream);
+// Waves per workgroup of the instantiation that serves `shape` (8, or 4 when
+// the LDS tiles of eight waves would not fit).
+int PaMfmaWaves(const AtbmiPaShape &shape);
+int LaunchPaMfma(const AtbmiPaShape &shape, const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream);
 // Per-operand-type halves of LaunchPaMfma (one translation unit each, so the
 // instantiations compile in parallel). Return -1 when the shape has no
 // instantiation.
-int LaunchPaMfmaF16(const AtbmiPaShape &shape, const PaArgs &args, int numItems, hipStream_t stream);
-int LaunchPaMfmaBf16(const AtbmiPaShape &shape, const PaArgs &args, int numItems, hipStream_t stream);
-int LaunchPaMfmaInt8(const AtbmiPaShape &shape, const PaArgs &args, int numItems, hipStream_t stream);
+int LaunchPaMfmaF16(const AtbmiPaShape &shape, const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream);
+int LaunchPaMfmaBf16(const AtbmiPaShape &shape, const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream);
+int LaunchPaMfmaInt8(const AtbmiPaShape &shape, const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream);
 
-// Merges the partials of every sequence that has more than one.
+// Merges the partials of every sequence that has more than one (scalar-kernel plan).
 int LaunchPaReduce(const AtbmiPaShape &shape, const PaArgs &args, int numSeqs, hipStream_t stream);
+// Merges the partials the MFMA kernel left for sequences that span several wave ranges.
+int LaunchPaStreamReduce(const AtbmiPaShape &shape, const PaArgs &args, const PaStreamPlan &plan,
+                         hipStream_t stream);
 
 } // namespace atbmi
 #endif

@@ -22,15 +22,22 @@ bool PaMfmaSupports(const AtbmiPaShape &s)
     return d == 64 || d == 96 || d == 128 || d == 256;
 }
 
-int LaunchPaMfma(const AtbmiPaShape &s, const PaArgs &args, int numItems, hipStream_t stream)
+int PaMfmaWaves(const AtbmiPaShape &s)
+{
+    // eight waves' K/V tiles fit the 160 KB of LDS up to 128-channel rows
+    // (and for the 192/128 combined cache); wider rows run four waves
+    return (s.headDimK <= 128 || (s.mlaCombined && s.headDimK <= 192)) ? 8 : 4;
+}
+
+int LaunchPaMfma(const AtbmiPaShape &s, const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
 {
     int rc;
     if (s.kvDtype == ATBMI_INT8) {
-        rc = LaunchPaMfmaInt8(s, args, numItems, stream);
+        rc = LaunchPaMfmaInt8(s, args, plan, stream);
     } else if (s.qDtype == ATBMI_BF16) {
-        rc = LaunchPaMfmaBf16(s, args, numItems, stream);
+        rc = LaunchPaMfmaBf16(s, args, plan, stream);
     } else {
-        rc = LaunchPaMfmaF16(s, args, numItems, stream);
+        rc = LaunchPaMfmaF16(s, args, plan, stream);
     }
     if (rc < 0) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: no MFMA kernel for head sizes %d/%d", s.headDimK, s.headDimV);

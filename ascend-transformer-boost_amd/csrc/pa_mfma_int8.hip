@@ -4,7 +4,7 @@
 
 namespace atbmi {
 
-int LaunchPaMfmaInt8(const AtbmiPaShape &s, const PaArgs &args, int numItems, hipStream_t stream)
+int LaunchPaMfmaInt8(const AtbmiPaShape &s, const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
 {
     using namespace mfma;
     if (s.mlaCombined || s.headDimK != s.headDimV) {
@@ -12,11 +12,11 @@ int LaunchPaMfmaInt8(const AtbmiPaShape &s, const PaArgs &args, int numItems, hi
     }
     switch (s.headDimK) {
         case 64:
-            return Launch<false, true, 64, 64, false, true>(args, numItems, stream);
+            return Launch<false, true, 64, 64, false, true, 8>(args, plan, stream);
         case 128:
-            return Launch<false, true, 128, 128, false, true>(args, numItems, stream);
+            return Launch<false, true, 128, 128, false, true, 8>(args, plan, stream);
         case 256:
-            return Launch<false, true, 256, 256, false, true>(args, numItems, stream);
+            return Launch<false, true, 256, 256, false, true, 4>(args, plan, stream);
         default:
             return -1;
     }

@@ -1,11 +1,16 @@
 // MFMA paged decode-attention kernel for gfx950 (MI355X).
 //
-// Work decomposition
-//   One workgroup (4 waves) = one KV chunk of one sequence, one KV head, one
-//   tile of up to 16 query heads. The waves take 32-token steps of the chunk
-//   round-robin and never synchronise inside the loop: each wave keeps its own
-//   online-softmax state and its own K/V tile in LDS; the four states are
-//   merged once at the end.
+// Work decomposition ("stream" split-KV)
+//   The KV rows of all sequences, in 32-token steps, form one linear step
+//   space. It is cut into equal contiguous ranges, one per wave and KV head:
+//   every wave gets the same number of steps (+-1) whatever the length
+//   distribution of the batch, so there is no tail of half-empty rounds and no
+//   per-chunk workgroup launch. A range that crosses a sequence boundary makes
+//   the wave finish one (partial or complete) attention row and start the next.
+//   The waves of a workgroup cover the KV heads of the SAME token range, so a
+//   CU pulls whole contiguous [token][head][channel] cache rows out of HBM.
+//   Waves never synchronise: each owns its K/V tile in LDS and its softmax
+//   state; rows that span several ranges are merged by the reduce kernel.
 //
 // Data path per wave and step (32 tokens)
 //   HBM -> VGPR : the 32 K rows and 32 V rows of this KV head, 16 bytes per
@@ -46,7 +51,6 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int STEP = PA_MFMA_STEP;   // tokens per wave step
-constexpr int NW = PA_MFMA_WAVES;    // waves per workgroup
 constexpr int HT = PA_MFMA_HEAD_TILE;
 constexpr int K_PAD = 8;             // halves of padding per K tile row (16 B)
 constexpr int V_PAD = 16;            // halves of padding per V tile row (32 B)
@@ -109,21 +113,25 @@ __device__ __forceinline__ u32x4 LoadGlobal16(const void *p)
     return *reinterpret_cast<const u32x4 *>(p);
 }
 
-// LDS bytes one workgroup needs.
-template <bool KV8, int D, int DV, bool MLA> constexpr int LdsBytes()
+// LDS bytes one wave needs for its K and V tiles.
+template <int D, int DV, bool MLA> constexpr int WaveLdsBytes()
 {
     constexpr int kTile = STEP * (D + K_PAD) * 2;
     constexpr int vTile = MLA ? 0 : STEP * (DV + V_PAD) * 2;
-    constexpr int tiles = NW * (kTile + vTile);
-    constexpr int merge = NW * HT * (DV + 4) * 4 + 2 * NW * HT * 4;
-    return tiles > merge ? tiles : merge;
+    return kTile + vTile;
+}
+
+__device__ __forceinline__ PaSeq PlanSeq(const PaStreamPlan &p, int i)
+{
+    return p.seqs ? p.seqs[i] : p.inlineSeqs[i];
 }
 
 // BF16: MFMA operand type (bf16 when the cache is bf16, fp16 otherwise).
 // KV8 : int8 cache rows. MLA: V is the first DV channels of the K row.
 // PF  : keep the next step's rows in registers while computing this one.
-template <bool BF16, bool KV8, int D, int DV, bool MLA, bool PF>
-__global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const int numStreams)
+// NW  : waves per workgroup.
+template <bool BF16, bool KV8, int D, int DV, bool MLA, bool PF, int NW>
+__global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const PaStreamPlan p)
 {
     static_assert(D % 32 == 0 && DV % 16 == 0, "head sizes must fit the MFMA tiles");
     static_assert(!KV8 || DV % 32 == 0, "int8 rows are staged 16 channels at a time");
@@ -131,7 +139,6 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const i
     constexpr int KP = D + K_PAD;                 // K tile pitch in halves
     constexpr int VP = MLA ? KP : DV + V_PAD;     // V tile pitch in halves
     constexpr int K_TILE_BYTES = STEP * KP * 2;
-    constexpr int V_TILE_BYTES = MLA ? 0 : STEP * VP * 2;
     constexpr int NQ = D / 32;                    // QK MFMAs per 16-token sub-tile
     constexpr int NO = DV / 16;                   // PV MFMAs (output tiles of 16 channels)
     constexpr int ESZ = KV8 ? 1 : 2;              // bytes per cache element
@@ -143,387 +150,396 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const i
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
-    // blockIdx -> (stream = work item x KV head, head tile). The head tiles of
-    // one stream read the same K/V rows: they are placed 8 workgroups apart so
-    // that they run on the same XCD (workgroups go to XCDs round-robin) and
-    // share its L2.
-    const int headTiles = (a.groupSize + HT - 1) / HT;
-    const int bx = blockIdx.x;
-    const int octet = bx / (8 * headTiles);
-    const int within = bx % (8 * headTiles);
-    const int ht = within / 8;
-    const int stream = octet * 8 + (within % 8);
-    if (stream >= numStreams) {
-        return;
-    }
-    const int g = stream % a.G;
-    const PaWorkItem it = a.items[stream / a.G];
-
     const int lane = threadIdx.x % WAVE;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const int n = lane & 15;  // head (B operand / accumulator column), token or channel (A operand row)
     const int kg = lane >> 4; // k-group: which 8 contraction values / 4 accumulator rows this lane holds
     const bool qBf16 = a.qIsBf16 != 0;
+
+    // Workgroup -> (token range, group of virtual heads); wave -> (virtual head, slice of the range).
+    // Head groups vary fastest so that the workgroups reading one token range run together.
+    const int hgIdx = blockIdx.x % p.headGroups;
+    const int wgRange = blockIdx.x / p.headGroups;
+    const int vh = hgIdx * p.headsPerWg + wave % p.headsPerWg;
+    const int g = vh / p.headTiles;
+    const int ht = vh % p.headTiles;
+    const int wr = wgRange * p.tokenSlices + wave / p.headsPerWg;
+    if (wr >= p.numWaveRanges) {
+        return;
+    }
+    const int s0 = PaRangeBegin(wr, p.totalSteps, p.numWaveRanges);
+    const int s1 = PaRangeBegin(wr + 1, p.totalSteps, p.numWaveRanges);
+    if (s0 >= s1) {
+        return;
+    }
     const int h0 = g * a.groupSize + ht * HT;
     const int nh = min(HT, a.groupSize - ht * HT);
 
-    unsigned char *kTile = smem + wave * (K_TILE_BYTES + V_TILE_BYTES);
+    unsigned char *kTile = smem + wave * WaveLdsBytes<D, DV, MLA>();
     unsigned char *vTile = MLA ? kTile : kTile + K_TILE_BYTES;
-
-    // ---- Q^T as B operand: lane (n, kg) holds q[h0+n][32j + 8kg .. +8) for j < NQ
-    u32x4 qreg[NQ];
-    {
-        const bool plain = !KV8 && a.qScale == 0.0f; // raw bits are already the operand
-        const uint16_t *qrow =
-            reinterpret_cast<const uint16_t *>(a.q) + (static_cast<int64_t>(it.qRow) * a.H + h0 + n) * D;
-#pragma unroll
-        for (int j = 0; j < NQ; ++j) {
-            const int d0 = j * 32 + kg * 8;
-            u32x4 raw = {0u, 0u, 0u, 0u};
-            if (n < nh) {
-                raw = LoadGlobal16(qrow + d0);
-            }
-            if (!plain) {
-                float f[8];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    f[e] = Unpack(raw[e >> 1], e & 1, qBf16);
-                    if (a.qScale != 0.0f) {
-                        f[e] *= a.qScale;
-                        f[e] = qBf16 ? Bf16ToFloat(FloatToBf16(f[e])) : HalfBitsToFloat(FloatToHalfBits(f[e]));
-                    }
-                    if (KV8) {
-                        f[e] *= a.kScale[g * D + d0 + e];
-                    }
-                }
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    raw[e] = Pack2<BF16>(f[2 * e], f[2 * e + 1]);
-                }
-            }
-            qreg[j] = raw;
-        }
-    }
-
-    constexpr float LOG2E = 1.4426950408889634f;
-    const float scale2 = a.qkScale * LOG2E;
-    float m = -INFINITY; // running maximum (base-2 exponent units) of head n
-    float l = 0.0f;      // this lane's share of the running denominator
-    f32x4 acc[NO];
-#pragma unroll
-    for (int i = 0; i < NO; ++i) {
-        acc[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    }
-
-    const int32_t *table = a.tables + static_cast<int64_t>(it.seq) * a.maxBlocksPerSeq;
     const unsigned char *kcBase = reinterpret_cast<const unsigned char *>(a.kc);
     const unsigned char *vcBase = reinterpret_cast<const unsigned char *>(a.vc);
+    constexpr float LOG2E = 1.4426950408889634f;
+    const float scale2 = a.qkScale * LOG2E;
 
-    // Issues the loads of the 32 rows starting at token t; rows at or past
-    // tokEnd come back as zeros and their block-table entries are not read.
-    auto loadStep = [&](int t, u32x4 *kp, u32x4 *vp) {
-        int64_t rowBase[2];
+    int seqIdx = p.firstSeq ? p.firstSeq[wgRange] : p.inlineFirst[wgRange];
+    while (PlanSeq(p, seqIdx + 1).stepBegin <= s0) {
+        ++seqIdx;
+    }
+
+    for (; seqIdx < p.numSeqs; ++seqIdx) {
+        const PaSeq sq = PlanSeq(p, seqIdx);
+        if (sq.stepBegin >= s1) {
+            break;
+        }
+        const int seqEnd = PlanSeq(p, seqIdx + 1).stepBegin;
+        const int segBegin = max(s0, sq.stepBegin);
+        const int segEnd = min(s1, seqEnd);
+        const int tokBegin = (segBegin - sq.stepBegin) * STEP;
+        const int tokEnd = min(sq.ctxLen, (segEnd - sq.stepBegin) * STEP);
+        const bool complete = segBegin == sq.stepBegin && segEnd == seqEnd;
+        const int qRow = seqIdx; // the i-th non-empty sequence owns query/output row i
+
+        // ---- Q^T as B operand: lane (n, kg) holds q[h0+n][32j + 8kg .. +8) for j < NQ
+        u32x4 qreg[NQ];
+        {
+            const uint16_t *qrow =
+                reinterpret_cast<const uint16_t *>(a.q) + (static_cast<int64_t>(qRow) * a.H + h0 + n) * D;
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            const int ts = t + 16 * s;
-            rowBase[s] = 0;
-            if (ts < it.tokEnd) {
-                rowBase[s] = static_cast<int64_t>(table[ts / a.blockSize]) * a.blockSize + (ts % a.blockSize);
+            for (int j = 0; j < NQ; ++j) { // all loads first, so their latencies overlap
+                qreg[j] = u32x4{0u, 0u, 0u, 0u};
+                if (n < nh) {
+                    qreg[j] = LoadGlobal16(qrow + j * 32 + kg * 8);
+                }
+            }
+            const bool plain = !KV8 && a.qScale == 0.0f; // raw bits are already the operand
+            if (!plain) {
+#pragma unroll
+                for (int j = 0; j < NQ; ++j) {
+                    const int d0 = j * 32 + kg * 8;
+                    float f[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        f[e] = Unpack(qreg[j][e >> 1], e & 1, qBf16);
+                        if (a.qScale != 0.0f) {
+                            f[e] *= a.qScale;
+                            f[e] = qBf16 ? Bf16ToFloat(FloatToBf16(f[e])) : HalfBitsToFloat(FloatToHalfBits(f[e]));
+                        }
+                        if (KV8) {
+                            f[e] *= a.kScale[g * D + d0 + e];
+                        }
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        qreg[j][e] = Pack2<BF16>(f[2 * e], f[2 * e + 1]);
+                    }
+                }
             }
         }
+
+        float m = -INFINITY; // running maximum (base-2 exponent units) of head n
+        float l = 0.0f;      // this lane's share of the running denominator
+        f32x4 acc[NO];
 #pragma unroll
-        for (int i = 0; i < NKP; ++i) {
-            const int p = i * WAVE + lane;
-            const int row = p / KPR;
-            const int col = p % KPR;
+        for (int i = 0; i < NO; ++i) {
+            acc[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+
+        const int32_t *table = a.tables + static_cast<int64_t>(sq.tableRow) * a.maxBlocksPerSeq;
+
+        // Block ids of this segment, 64 at a time, one per lane: a step then gets
+        // its block id with a cross-lane read instead of a dependent memory load.
+        const int blocksNeeded = (tokEnd + a.blockSize - 1) / a.blockSize; // entries past this are never read
+        int cacheBase = tokBegin / a.blockSize;
+        int blkCache = (cacheBase + lane < blocksNeeded) ? table[cacheBase + lane] : 0;
+        // The load cursor: block index and offset inside the block of the next
+        // 16-token sub-tile to fetch (a sub-tile never straddles cache blocks).
+        int curBlk = cacheBase;
+        int curOff = tokBegin % a.blockSize;
+
+        // Cache row index (rows = [slot][head][channel]) of the next two sub-tiles; advances the cursor.
+        auto nextRows = [&](int64_t *rowBase) {
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub) {
+                if (curBlk >= cacheBase + WAVE) {
+                    cacheBase = curBlk;
+                    blkCache = (cacheBase + lane < blocksNeeded) ? table[cacheBase + lane] : 0;
+                }
+                const int blk = __builtin_amdgcn_readlane(blkCache, curBlk - cacheBase);
+                rowBase[sub] = static_cast<int64_t>(blk) * a.blockSize + curOff;
+                curOff += 16;
+                if (curOff >= a.blockSize) {
+                    curOff = 0;
+                    ++curBlk;
+                }
+            }
+        };
+        // `full`: all 32 rows of the step are inside the segment; otherwise rows
+        // at or past tokEnd are not touched and read as zeros.
+        auto loadK = [&](int t, const int64_t *rowBase, int i, bool full) -> u32x4 {
+            const int pc = i * WAVE + lane;
+            const int row = pc / KPR;
+            const int col = pc % KPR;
             u32x4 v = {0u, 0u, 0u, 0u};
-            if (t + row < it.tokEnd) {
+            if (full || t + row < tokEnd) {
                 const int64_t r = rowBase[row >> 4] + (row & 15);
                 v = LoadGlobal16(kcBase + (r * a.kRowStride + static_cast<int64_t>(g) * D) * ESZ + col * 16);
             }
-            kp[i] = v;
-        }
-#pragma unroll
-        for (int i = 0; i < NVP; ++i) {
-            const int p = i * WAVE + lane;
-            const int row = p / VPR;
-            const int col = p % VPR;
+            return v;
+        };
+        auto loadV = [&](int t, const int64_t *rowBase, int i, bool full) -> u32x4 {
+            const int pc = i * WAVE + lane;
+            const int row = pc / VPR;
+            const int col = pc % VPR;
             u32x4 v = {0u, 0u, 0u, 0u};
-            if (t + row < it.tokEnd) {
+            if (full || t + row < tokEnd) {
                 const int64_t r = rowBase[row >> 4] + (row & 15);
-                v = LoadGlobal16(vcBase + (r * a.vRowStride + static_cast<int64_t>(g) * a.vHeadStride) * ESZ + col * 16);
+                v = LoadGlobal16(vcBase + (r * a.vRowStride + static_cast<int64_t>(g) * a.vHeadStride) * ESZ +
+                                 col * 16);
             }
-            vp[i] = v;
-        }
-    };
-
-    // Writes staged rows into this wave's LDS tiles (int8 widened to fp16).
-    auto storeStep = [&](const u32x4 *kp, const u32x4 *vp) {
-#pragma unroll
-        for (int i = 0; i < NKP; ++i) {
-            const int p = i * WAVE + lane;
-            const int row = p / KPR;
-            const int col = p % KPR;
+            return v;
+        };
+        // Writes one staged 16-byte piece into an LDS tile (int8 widened to fp16).
+        auto storePiece = [&](unsigned char *tile, int pitchHalves, int piecesPerRow, int i, u32x4 piece) {
+            const int pc = i * WAVE + lane;
+            const int row = pc / piecesPerRow;
+            const int col = pc % piecesPerRow;
             if constexpr (KV8) {
                 u32x4 lo, hi;
-                WidenPiece(kp[i], lo, hi);
-                u32x4 *dst = reinterpret_cast<u32x4 *>(kTile + row * (KP * 2) + col * 32);
+                WidenPiece(piece, lo, hi);
+                u32x4 *dst = reinterpret_cast<u32x4 *>(tile + row * (pitchHalves * 2) + col * 32);
                 dst[0] = lo;
                 dst[1] = hi;
             } else {
-                *reinterpret_cast<u32x4 *>(kTile + row * (KP * 2) + col * 16) = kp[i];
+                *reinterpret_cast<u32x4 *>(tile + row * (pitchHalves * 2) + col * 16) = piece;
             }
-        }
-#pragma unroll
-        for (int i = 0; i < NVP; ++i) {
-            const int p = i * WAVE + lane;
-            const int row = p / VPR;
-            const int col = p % VPR;
-            if constexpr (KV8) {
-                u32x4 lo, hi;
-                WidenPiece(vp[i], lo, hi);
-                u32x4 *dst = reinterpret_cast<u32x4 *>(vTile + row * (VP * 2) + col * 32);
-                dst[0] = lo;
-                dst[1] = hi;
-            } else {
-                *reinterpret_cast<u32x4 *>(vTile + row * (VP * 2) + col * 16) = vp[i];
+        };
+
+        constexpr int NKR = PF ? NKP : 1;
+        constexpr int NVR = (PF && NVP > 0) ? NVP : 1;
+        u32x4 kStage[NKR];
+        u32x4 vStage[NVR];
+        // Issues the loads of the step at token t into the stage registers.
+        auto loadStage = [&](int t) {
+            if constexpr (PF) {
+                int64_t rowBase[2];
+                nextRows(rowBase);
+                if (t + STEP <= tokEnd) {
+    #pragma unroll
+                    for (int i = 0; i < NKP; ++i) {
+                        kStage[i] = loadK(t, rowBase, i, true);
+                    }
+    #pragma unroll
+                    for (int i = 0; i < NVP; ++i) {
+                        vStage[i] = loadV(t, rowBase, i, true);
+                    }
+                } else {
+    #pragma unroll
+                    for (int i = 0; i < NKP; ++i) {
+                        kStage[i] = loadK(t, rowBase, i, false);
+                    }
+    #pragma unroll
+                    for (int i = 0; i < NVP; ++i) {
+                        vStage[i] = loadV(t, rowBase, i, false);
+                    }
+                }
             }
-        }
-    };
-
-    constexpr int NKR = PF ? NKP : 1;
-    constexpr int NVR = PF ? (NVP > 0 ? NVP : 1) : 1;
-    u32x4 kStage[NKR];
-    u32x4 vStage[NVR];
-
-    const int tFirst = it.tokBegin + wave * STEP;
-    if constexpr (PF) {
-        if (tFirst < it.tokEnd) {
-            loadStep(tFirst, kStage, vStage);
-        }
-    }
-
-    for (int t = tFirst; t < it.tokEnd; t += NW * STEP) {
+        };
         if constexpr (PF) {
-            storeStep(kStage, vStage);
-            if (t + NW * STEP < it.tokEnd) {
-                loadStep(t + NW * STEP, kStage, vStage);
-            }
-        } else {
-            // Large rows: stage a few pieces at a time to bound register use.
-            int64_t rowBase[2];
+            loadStage(tokBegin);
+        }
+
+        for (int t = tokBegin; t < tokEnd; t += STEP) {
+            if constexpr (PF) {
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                const int ts = t + 16 * s;
-                rowBase[s] = 0;
-                if (ts < it.tokEnd) {
-                    rowBase[s] = static_cast<int64_t>(table[ts / a.blockSize]) * a.blockSize + (ts % a.blockSize);
+                for (int i = 0; i < NKP; ++i) {
+                    storePiece(kTile, KP, KPR, i, kStage[i]);
                 }
-            }
-            constexpr int BATCH = 6;
-            static_assert(!KV8, "the unstaged path handles 16-bit rows only");
 #pragma unroll
-            for (int i0 = 0; i0 < NKP; i0 += BATCH) {
-                u32x4 tmp[BATCH];
+                for (int i = 0; i < NVP; ++i) {
+                    storePiece(vTile, VP, VPR, i, vStage[i]);
+                }
+                if (t + STEP < tokEnd) {
+                    loadStage(t + STEP);
+                }
+            } else {
+                // Large rows: stage a few pieces at a time to bound register use.
+                constexpr int BATCH = 6;
+                int64_t rowBase[2];
+                nextRows(rowBase);
+                const bool full = t + STEP <= tokEnd;
 #pragma unroll
-                for (int b = 0; b < BATCH; ++b) {
-                    const int i = i0 + b;
-                    tmp[b] = u32x4{0u, 0u, 0u, 0u};
-                    if (i < NKP) {
-                        const int p = i * WAVE + lane;
-                        const int row = p / KPR;
-                        const int col = p % KPR;
-                        if (t + row < it.tokEnd) {
-                            const int64_t r = rowBase[row >> 4] + (row & 15);
-                            tmp[b] = LoadGlobal16(kcBase + (r * a.kRowStride + static_cast<int64_t>(g) * D) * 2 + col * 16);
+                for (int i0 = 0; i0 < NKP; i0 += BATCH) {
+                    u32x4 tmp[BATCH];
+#pragma unroll
+                    for (int b = 0; b < BATCH; ++b) {
+                        if (i0 + b < NKP) {
+                            tmp[b] = loadK(t, rowBase, i0 + b, full);
+                        }
+                    }
+#pragma unroll
+                    for (int b = 0; b < BATCH; ++b) {
+                        if (i0 + b < NKP) {
+                            storePiece(kTile, KP, KPR, i0 + b, tmp[b]);
                         }
                     }
                 }
 #pragma unroll
-                for (int b = 0; b < BATCH; ++b) {
-                    const int i = i0 + b;
-                    if (i < NKP) {
-                        const int p = i * WAVE + lane;
-                        *reinterpret_cast<u32x4 *>(kTile + (p / KPR) * (KP * 2) + (p % KPR) * 16) = tmp[b];
+                for (int i0 = 0; i0 < NVP; i0 += BATCH) {
+                    u32x4 tmp[BATCH];
+#pragma unroll
+                    for (int b = 0; b < BATCH; ++b) {
+                        if (i0 + b < NVP) {
+                            tmp[b] = loadV(t, rowBase, i0 + b, full);
+                        }
                     }
-                }
-            }
 #pragma unroll
-            for (int i0 = 0; i0 < NVP; i0 += BATCH) {
-                u32x4 tmp[BATCH];
-#pragma unroll
-                for (int b = 0; b < BATCH; ++b) {
-                    const int i = i0 + b;
-                    tmp[b] = u32x4{0u, 0u, 0u, 0u};
-                    if (i < NVP) {
-                        const int p = i * WAVE + lane;
-                        const int row = p / VPR;
-                        const int col = p % VPR;
-                        if (t + row < it.tokEnd) {
-                            const int64_t r = rowBase[row >> 4] + (row & 15);
-                            tmp[b] = LoadGlobal16(vcBase + (r * a.vRowStride + static_cast<int64_t>(g) * a.vHeadStride) * 2 + col * 16);
+                    for (int b = 0; b < BATCH; ++b) {
+                        if (i0 + b < NVP) {
+                            storePiece(vTile, VP, VPR, i0 + b, tmp[b]);
                         }
                     }
                 }
+            }
+            // The tile is private to this wave: LDS executes a wave's accesses in
+            // order, only the compiler has to be kept from moving reads above writes.
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+            // ---- S^T = K . Q^T for the two 16-token sub-tiles
+            f32x4 s[2];
 #pragma unroll
-                for (int b = 0; b < BATCH; ++b) {
-                    const int i = i0 + b;
-                    if (i < NVP) {
-                        const int p = i * WAVE + lane;
-                        *reinterpret_cast<u32x4 *>(vTile + (p / VPR) * (VP * 2) + (p % VPR) * 16) = tmp[b];
-                    }
+            for (int sub = 0; sub < 2; ++sub) {
+                s[sub] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                const unsigned char *krow = kTile + (sub * 16 + n) * (KP * 2) + kg * 16;
+#pragma unroll
+                for (int j = 0; j < NQ; ++j) {
+                    const u32x4 kop = *reinterpret_cast<const u32x4 *>(krow + j * 64);
+                    s[sub] = Mma<BF16>(kop, qreg[j], s[sub]);
                 }
             }
-        }
-        // The tile is private to this wave: LDS executes a wave's accesses in
-        // order, only the compiler has to be kept from moving reads above writes.
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        // ---- S^T = K . Q^T for the two 16-token sub-tiles
-        f32x4 s[2];
+            // ---- online softmax in base 2; lane holds tokens t + 16 sub + 4 kg + r of head n
+            float x[8];
+            float mloc = -INFINITY;
 #pragma unroll
-        for (int sub = 0; sub < 2; ++sub) {
-            s[sub] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-            const unsigned char *krow = kTile + (sub * 16 + n) * (KP * 2) + kg * 16;
+            for (int sub = 0; sub < 2; ++sub) {
 #pragma unroll
-            for (int j = 0; j < NQ; ++j) {
-                const u32x4 kop = *reinterpret_cast<const u32x4 *>(krow + j * 64);
-                s[sub] = Mma<BF16>(kop, qreg[j], s[sub]);
+                for (int r = 0; r < 4; ++r) {
+                    const int tok = t + sub * 16 + kg * 4 + r;
+                    const float v = tok < tokEnd ? s[sub][r] * scale2 : -INFINITY;
+                    x[sub * 4 + r] = v;
+                    mloc = fmaxf(mloc, v);
+                }
             }
-        }
-
-        // ---- online softmax in base 2; lane holds tokens t + 16 sub + 4 kg + r of head n
-        float x[8];
-        float mloc = -INFINITY;
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 16, WAVE));
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+            const float mNew = fmaxf(m, mloc); // finite: every step holds at least one valid token
+            const float corr = exp2f(m - mNew);
+            m = mNew;
+            float psum = 0.0f;
 #pragma unroll
-        for (int sub = 0; sub < 2; ++sub) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int tok = t + sub * 16 + kg * 4 + r;
-                const float v = tok < it.tokEnd ? s[sub][r] * scale2 : -INFINITY;
-                x[sub * 4 + r] = v;
-                mloc = fmaxf(mloc, v);
+            for (int e = 0; e < 8; ++e) {
+                x[e] = exp2f(x[e] - mNew);
+                psum += x[e];
             }
-        }
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 16, WAVE));
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
-        const float mNew = fmaxf(m, mloc); // finite: every step holds at least one valid token
-        const float corr = exp2f(m - mNew);
-        m = mNew;
-        float psum = 0.0f;
+            l = l * corr + psum;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            x[e] = exp2f(x[e] - mNew);
-            psum += x[e];
-        }
-        l = l * corr + psum;
-#pragma unroll
-        for (int i = 0; i < NO; ++i) {
-            acc[i] *= corr;
-        }
-        u32x4 pop; // P^T as B operand: k = {sub 0: r 0..3, sub 1: r 0..3}
-        pop[0] = Pack2<BF16>(x[0], x[1]);
-        pop[1] = Pack2<BF16>(x[2], x[3]);
-        pop[2] = Pack2<BF16>(x[4], x[5]);
-        pop[3] = Pack2<BF16>(x[6], x[7]);
-
-        // ---- O^T += V^T . P^T. The transposing read hands lane (n, kg) the four
-        // tokens 4kg..4kg+3 of channel 16 i + n when lane (n, kg) points at
-        // token 4kg + n/4, channels 16 i + 4 (n%4) .. +4.
-        const unsigned char *vrow = vTile + (kg * 4 + (n >> 2)) * (VP * 2) + (n & 3) * 8;
-#pragma unroll
-        for (int i = 0; i < NO; ++i) {
-            const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (__attribute__((address_space(3))) i16x4 *)(vrow + i * 32));
-            const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (__attribute__((address_space(3))) i16x4 *)(vrow + 16 * (VP * 2) + i * 32));
-            u32x4 vop;
-            const u32x2 lo2 = __builtin_bit_cast(u32x2, lo);
-            const u32x2 hi2 = __builtin_bit_cast(u32x2, hi);
-            vop[0] = lo2[0];
-            vop[1] = lo2[1];
-            vop[2] = hi2[0];
-            vop[3] = hi2[1];
-            acc[i] = Mma<BF16>(vop, pop, acc[i]);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-    }
-
-    // ---- merge the four waves
-    l += __shfl_xor(l, 16, WAVE);
-    l += __shfl_xor(l, 32, WAVE);
-    __syncthreads(); // every wave is done with its tiles; the space is reused
-    constexpr int OP = DV + 4; // floats per (wave, head) row of the merge area
-    float *mergeO = reinterpret_cast<float *>(smem);
-    float *mergeM = mergeO + NW * HT * OP;
-    float *mergeL = mergeM + NW * HT;
-#pragma unroll
-    for (int i = 0; i < NO; ++i) {
-        *reinterpret_cast<f32x4 *>(mergeO + (wave * HT + n) * OP + i * 16 + kg * 4) = acc[i];
-    }
-    if (kg == 0) {
-        mergeM[wave * HT + n] = m;
-        mergeL[wave * HT + n] = l;
-    }
-    __syncthreads();
-    for (int idx = threadIdx.x; idx < HT * DV; idx += NW * WAVE) {
-        const int hh = idx / DV;
-        const int d = idx % DV;
-        if (hh >= nh) {
-            continue;
-        }
-        float mx = -INFINITY;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) {
-            mx = fmaxf(mx, mergeM[w * HT + hh]);
-        }
-        float den = 0.0f;
-        float num = 0.0f;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) {
-            const float wgt = exp2f(mergeM[w * HT + hh] - mx); // 0 for a wave that saw no token
-            den += wgt * mergeL[w * HT + hh];
-            num += wgt * mergeO[(w * HT + hh) * OP + d];
-        }
-        float o = num / den;
-        const int h = h0 + hh;
-        if (it.direct) {
-            if (KV8) {
-                const int c = g * DV + d;
-                o = (o + (a.vOff ? static_cast<float>(a.vOff[c]) : 0.0f)) * a.vScale[c];
+            for (int i = 0; i < NO; ++i) {
+                acc[i] *= corr;
             }
-            Store16(a.out, (static_cast<int64_t>(it.qRow) * a.H + h) * DV + d, o, qBf16);
-        } else {
-            const int64_t ph = static_cast<int64_t>(it.partialBase) * a.H + h;
-            a.partO[ph * DV + d] = o;
-            if (d == 0) {
-                a.partLse[ph] = mx + log2f(den);
+            u32x4 pop; // P^T as B operand: k = {sub 0: r 0..3, sub 1: r 0..3}
+            pop[0] = Pack2<BF16>(x[0], x[1]);
+            pop[1] = Pack2<BF16>(x[2], x[3]);
+            pop[2] = Pack2<BF16>(x[4], x[5]);
+            pop[3] = Pack2<BF16>(x[6], x[7]);
+
+            // ---- O^T += V^T . P^T. The transposing read hands lane (n, kg) the four
+            // tokens 4kg..4kg+3 of channel 16 i + n when lane (n, kg) points at
+            // token 4kg + n/4, channels 16 i + 4 (n%4) .. +4.
+            const unsigned char *vrow = vTile + (kg * 4 + (n >> 2)) * (VP * 2) + (n & 3) * 8;
+#pragma unroll
+            for (int i = 0; i < NO; ++i) {
+                const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (__attribute__((address_space(3))) i16x4 *)(vrow + i * 32));
+                const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (__attribute__((address_space(3))) i16x4 *)(vrow + 16 * (VP * 2) + i * 32));
+                const u32x2 lo2 = __builtin_bit_cast(u32x2, lo);
+                const u32x2 hi2 = __builtin_bit_cast(u32x2, hi);
+                const u32x4 vop = {lo2[0], lo2[1], hi2[0], hi2[1]};
+                acc[i] = Mma<BF16>(vop, pop, acc[i]);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
+
+        // ---- finish the row (or this wave's share of it)
+        l += __shfl_xor(l, 16, WAVE);
+        l += __shfl_xor(l, 32, WAVE);
+        const float inv = 1.0f / l;
+        if (n < nh) {
+            const int h = h0 + n;
+            if (complete) {
+                uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) + (static_cast<int64_t>(qRow) * a.H + h) * DV;
+#pragma unroll
+                for (int i = 0; i < NO; ++i) {
+                    const int d = i * 16 + kg * 4;
+                    float o[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        o[r] = acc[i][r] * inv;
+                        if (KV8) {
+                            const int c = g * DV + d + r;
+                            o[r] = (o[r] + (a.vOff ? static_cast<float>(a.vOff[c]) : 0.0f)) * a.vScale[c];
+                        }
+                    }
+                    u32x2 packed;
+                    if (qBf16) {
+                        packed[0] = Pack2<true>(o[0], o[1]);
+                        packed[1] = Pack2<true>(o[2], o[3]);
+                    } else {
+                        packed[0] = Pack2<false>(o[0], o[1]);
+                        packed[1] = Pack2<false>(o[2], o[3]);
+                    }
+                    *reinterpret_cast<u32x2 *>(orow + d) = packed;
+                }
+            } else {
+                const int slot = 2 * wr + (segBegin == s0 ? 0 : 1);
+                const int64_t ph = static_cast<int64_t>(slot) * a.H + h;
+#pragma unroll
+                for (int i = 0; i < NO; ++i) {
+                    *reinterpret_cast<f32x4 *>(a.partO + ph * DV + i * 16 + kg * 4) = acc[i] * inv;
+                }
+                if (kg == 0) {
+                    a.partLse[ph] = m + log2f(l);
+                }
             }
         }
     }
 }
 
-template <bool BF16, bool KV8, int D, int DV, bool MLA, bool PF>
-int Launch(const PaArgs &args, int numItems, hipStream_t stream)
+template <bool BF16, bool KV8, int D, int DV, bool MLA, bool PF, int NW>
+int Launch(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
 {
-    auto kernel = PaMfmaKernel<BF16, KV8, D, DV, MLA, PF>;
-    constexpr int lds = LdsBytes<KV8, D, DV, MLA>();
+    auto kernel = PaMfmaKernel<BF16, KV8, D, DV, MLA, PF, NW>;
+    constexpr int lds = NW * WaveLdsBytes<D, DV, MLA>();
+    static_assert(lds <= 160 * 1024, "tiles exceed the 160 KB of LDS per CU");
     static bool configured = false; // one attribute call per instantiation and process
     if (!configured) {
         ATBMI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         configured = true;
     }
-    const int headTiles = (args.groupSize + HT - 1) / HT;
-    const int64_t streams = static_cast<int64_t>(numItems) * args.G;
-    const int64_t grid = (streams + 7) / 8 * 8 * headTiles;
+    if (plan.headsPerWg * plan.tokenSlices != NW) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: plan made for %d waves, kernel has %d",
+                    plan.headsPerWg * plan.tokenSlices, NW);
+    }
+    const int64_t grid = static_cast<int64_t>(plan.numWgRanges) * plan.headGroups;
     if (grid <= 0 || grid > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: grid of %lld workgroups is out of range", (long long)grid);
     }
-    kernel<<<static_cast<unsigned>(grid), NW * WAVE, lds, stream>>>(args, static_cast<int>(streams));
+    kernel<<<static_cast<unsigned>(grid), NW * WAVE, lds, stream>>>(args, plan);
     ATBMI_HIP_CHECK(hipGetLastError());
     return OK;
 }

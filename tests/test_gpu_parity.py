@@ -410,10 +410,11 @@ def test_split_kv_chunking_does_not_change_the_result(binding, oracle, dev, stre
     got, info = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, kernel=kernel, chunk_tokens=chunk,
                                return_plan_info=True)
     assert_close(got, oracle_pa(oracle, q, kc, vc, tables, ctx, scale), 2e-2, "chunk=%d" % chunk)
+    # scalar kernel: chunks per sequence; MFMA kernel: equal ranges of the whole batch
     if chunk == 128:
-        assert info["chunks"] >= 40 + 2 + 17
+        assert info["chunks"] >= (40 + 2 + 17 if kernel == 1 else 50)
     if chunk == 100000:
-        assert info["chunks"] == 3
+        assert info["chunks"] == (3 if kernel == 1 else 1)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
