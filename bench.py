@@ -92,6 +92,7 @@ def main():
     ap.add_argument("--config", default="c2", choices=sorted(DESCRIPTIONS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--attention-only", action="store_true", help="leave ReshapeAndCache out of the step")
+    ap.add_argument("--no-kernel-events", action="store_true", help="do not bracket the attention kernel with events")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU; --gpus %d is not supported" % args.gpus)
@@ -155,7 +156,7 @@ def main():
             one_step()
         stream.synchronize()
         torch.cuda.synchronize()
-        k.atbmi_timing_enable(1)
+        k.atbmi_timing_enable(0 if args.no_kernel_events else 1)
         t0 = time.perf_counter()
         for _ in range(args.steps):
             one_step()
