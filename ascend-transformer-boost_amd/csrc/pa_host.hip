@@ -57,7 +57,8 @@ struct TimingRecord {
     hipEvent_t end;
 };
 std::mutex g_timingMutex;
-bool g_timingEnabled = false;
+int g_timingEvery = 0;   // 0: off; n: bracket every n-th decode launch with events
+int64_t g_timingLaunch = 0;
 std::vector<TimingRecord> g_timingRecords;
 
 } // namespace
@@ -580,7 +581,7 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
     bool timed = false;
     {
         std::lock_guard<std::mutex> lock(g_timingMutex);
-        timed = g_timingEnabled;
+        timed = g_timingEvery > 0 && (g_timingLaunch++ % g_timingEvery) == 0;
     }
     if (timed) {
         ATBMI_HIP_CHECK(hipEventCreate(&rec.begin));
@@ -613,7 +614,8 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
 extern "C" int atbmi_timing_enable(int32_t enable)
 {
     std::lock_guard<std::mutex> lock(g_timingMutex);
-    g_timingEnabled = enable != 0;
+    g_timingEvery = enable > 0 ? enable : 0;
+    g_timingLaunch = 0;
     return OK;
 }
 

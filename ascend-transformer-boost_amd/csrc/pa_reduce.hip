@@ -53,9 +53,15 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaReduceKernel(const PaArgs a)
 
 // Stream plan: the partials of sequence b live in the slots of the wave
 // ranges that intersect its steps; a sequence inside one range was written
-// directly by that wave.
+// directly by that wave. One workgroup merges one (sequence, query head).
+// Slot 2wr holds the row a range starts in, slot 2wr+1 the row it ends in, so
+// only the first range of a sequence can use an odd slot.
+// The weights 2^(lse_k - max) are computed once, 128 ranges at a time by the
+// 128 threads, and kept in LDS; threads then own output channels.
 __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaArgs a, const PaStreamPlan p)
 {
+    __shared__ float weight[REDUCE_THREADS];
+    __shared__ float red[REDUCE_THREADS / WAVE];
     const int b = blockIdx.x / a.H;
     const int h = blockIdx.x % a.H;
     const int begin = (p.seqs ? p.seqs[b] : p.inlineSeqs[b]).stepBegin;
@@ -65,33 +71,84 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaA
     if (wrFirst == wrLast) {
         return;
     }
-    // slot 2wr holds the row a range starts in, slot 2wr+1 the row it ends in
-    auto slotOf = [&](int wr) {
-        return 2 * wr + (PaRangeBegin(wr, p.totalSteps, p.numWaveRanges) >= begin ? 0 : 1);
+    const int firstOdd = PaRangeBegin(wrFirst, p.totalSteps, p.numWaveRanges) >= begin ? 0 : 1;
+    const int64_t stride = 2 * static_cast<int64_t>(a.H);
+    const int64_t phEven = 2 * static_cast<int64_t>(wrFirst) * a.H + h; // partial row of the k-th range, k >= 1
+    const int64_t ph0 = phEven + static_cast<int64_t>(firstOdd) * a.H;
+    const int count = wrLast - wrFirst + 1;
+    const int tid = threadIdx.x;
+    auto rowOf = [&](int k) { return k == 0 ? ph0 : phEven + k * stride; };
+    auto blockMax = [&](float v) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            v = fmaxf(v, __shfl_xor(v, off, WAVE));
+        }
+        __syncthreads();
+        if (tid % WAVE == 0) {
+            red[tid / WAVE] = v;
+        }
+        __syncthreads();
+        return fmaxf(red[0], red[1]);
     };
+    auto blockSum = [&](float v) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            v += __shfl_xor(v, off, WAVE);
+        }
+        __syncthreads();
+        if (tid % WAVE == 0) {
+            red[tid / WAVE] = v;
+        }
+        __syncthreads();
+        return red[0] + red[1];
+    };
+
     float mx = -INFINITY;
-    for (int wr = wrFirst; wr <= wrLast; ++wr) {
-        mx = fmaxf(mx, a.partLse[static_cast<int64_t>(slotOf(wr)) * a.H + h]);
+    for (int k = tid; k < count; k += REDUCE_THREADS) {
+        mx = fmaxf(mx, a.partLse[rowOf(k)]);
     }
-    float total = 0.0f;
-    for (int wr = wrFirst; wr <= wrLast; ++wr) {
-        total += exp2f(a.partLse[static_cast<int64_t>(slotOf(wr)) * a.H + h] - mx);
-    }
-    const float inv = 1.0f / total;
+    mx = blockMax(mx);
+
     const int g = h / a.groupSize;
     const bool bf16 = a.qIsBf16 != 0;
-    for (int d = threadIdx.x; d < a.Dv; d += REDUCE_THREADS) {
-        float acc = 0.0f;
-        for (int wr = wrFirst; wr <= wrLast; ++wr) {
-            const int64_t ph = static_cast<int64_t>(slotOf(wr)) * a.H + h;
-            acc += exp2f(a.partLse[ph] - mx) * a.partO[ph * a.Dv + d];
+    // channels handled by this thread: tid, tid + 128, ... (at most 5 for Dv <= 576)
+    float acc[5] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    float total = 0.0f;
+    for (int k0 = 0; k0 < count; k0 += REDUCE_THREADS) {
+        const int kn = min(REDUCE_THREADS, count - k0);
+        __syncthreads();
+        float w = 0.0f;
+        if (tid < kn) {
+            w = exp2f(a.partLse[rowOf(k0 + tid)] - mx);
+            weight[tid] = w;
         }
-        acc *= inv;
-        if (a.finishV) {
-            const int c = g * a.Dv + d;
-            acc = (acc + (a.vOff ? static_cast<float>(a.vOff[c]) : 0.0f)) * a.vScale[c];
+        total += w;
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < 5; ++c) {
+            const int d = tid + c * REDUCE_THREADS;
+            if (d < a.Dv) {
+                float s = 0.0f;
+#pragma unroll 4
+                for (int k = 0; k < kn; ++k) {
+                    s += weight[k] * a.partO[rowOf(k0 + k) * a.Dv + d];
+                }
+                acc[c] += s;
+            }
         }
-        Store16(a.out, (static_cast<int64_t>(b) * a.H + h) * a.Dv + d, acc, bf16);
+    }
+    const float inv = 1.0f / blockSum(total);
+#pragma unroll
+    for (int c = 0; c < 5; ++c) {
+        const int d = tid + c * REDUCE_THREADS;
+        if (d < a.Dv) {
+            float o = acc[c] * inv;
+            if (a.finishV) {
+                const int ch = g * a.Dv + d;
+                o = (o + (a.vOff ? static_cast<float>(a.vOff[ch]) : 0.0f)) * a.vScale[ch];
+            }
+            Store16(a.out, (static_cast<int64_t>(b) * a.H + h) * a.Dv + d, o, bf16);
+        }
     }
 }
 

@@ -156,7 +156,8 @@ def main():
             one_step()
         stream.synchronize()
         torch.cuda.synchronize()
-        k.atbmi_timing_enable(0 if args.no_kernel_events else 1)
+        # every 4th attention launch is bracketed with HIP events on the launch stream
+        k.atbmi_timing_enable(0 if args.no_kernel_events else 4)
         t0 = time.perf_counter()
         for _ in range(args.steps):
             one_step()

@@ -156,10 +156,12 @@ int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *tensors, void *work
 void atbmi_pa_plan_destroy(AtbmiPaPlan *plan);
 
 /*
- * Kernel timing for benchmarks. When enabled, every atbmi_pa_decode brackets
- * its attention kernel with HIP events on the launch stream.
+ * Kernel timing for benchmarks. atbmi_timing_enable(n) with n > 0 makes every
+ * n-th atbmi_pa_decode bracket its attention kernel with HIP events on the
+ * launch stream (the events themselves cost a few microseconds of stream
+ * time, hence the sampling); 0 turns it off.
  * atbmi_timing_read waits for the recorded events, adds them up, returns the
- * sum in milliseconds and the number of launches, and clears the record.
+ * sum in milliseconds and the number of timed launches, and clears the record.
  */
 int atbmi_timing_enable(int32_t enable);
 int atbmi_timing_read(double *totalMs, int64_t *launches);

@@ -447,3 +447,17 @@ def test_repeated_execute_and_changing_lengths(binding, oracle, dev, stream):
         assert_close(outs[step], oracle_pa(oracle, q, kc, vc, tables, base + step, scale), 1e-3, "step %d" % step)
     pa.close()
     c.close()
+
+
+@pytest.mark.parametrize("heads,kv_heads", [(30, 2), (8, 2), (8, 4), (32, 8), (16, 1)])
+def test_rows_spanning_wave_ranges_merge_consistently(binding, oracle, dev, stream, heads, kv_heads):
+    """Rows cut across several wave ranges are merged inside the kernel by the wave
+    that finishes last; the partial rows travel between CUs of different XCDs.
+    Repeated launches on reused workspace addresses must all give the oracle's rows."""
+    rng = _rng(97)
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, 18, heads, kv_heads, 128, 128, 128, 88, torch.float16)
+    scale = 1.0 / math.sqrt(128)
+    want = oracle_pa(oracle, q, kc, vc, tables, ctx, scale)
+    for rep in range(12):
+        got = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, kernel=0)
+        assert_close(got, want, 1e-3, "repetition %d" % rep)
