@@ -23,6 +23,12 @@ if ROOT not in sys.path:
 PKG = "ascend-transformer-boost_amd"
 HBM_PEAK_GBPS = 8000.0
 
+# HBM bytes one attention launch moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this
+# script, scaled by what the same counters read for a 256 MiB copy (--calibrate-copy); the runs and the
+# scale factors are written up in profiles/pa_mfma_bf16_d128_c2_hbm_traffic.md. Keyed by workload and
+# its algorithmic bytes, so a changed workload reports null instead of a stale figure.
+MEASURED_TRAFFIC = {("c2", 651658484): 658.7e6}
+
 DESCRIPTIONS = {
     "c1": "C1 small fp16 decode: batch 4, 8 q heads, 8 kv heads, d128, block 128, ctx U[64,512]",
     "c2": "C2 Llama-3-8B-shaped bf16 decode: batch 64, 32 q heads, 8 kv heads, d128, block 128, ctx U[1024,4096]",
@@ -93,6 +99,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--attention-only", action="store_true", help="leave ReshapeAndCache out of the step")
     ap.add_argument("--no-kernel-events", action="store_true", help="do not bracket the attention kernel with events")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device copy, as the known-size reference for hardware counters")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU; --gpus %d is not supported" % args.gpus)
@@ -151,6 +159,12 @@ def main():
                 rac.run(rac_in, outputs=rac_out)
         pa.run(pa_in, outputs=[out], host_inputs={host_idx: lens_host})
 
+    if args.calibrate_copy:
+        with torch.cuda.stream(stream):
+            src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+            dst = torch.empty_like(src)
+            dst.copy_(src)
+        stream.synchronize()
     with torch.cuda.stream(stream):
         for _ in range(args.warmup):
             one_step()
@@ -191,7 +205,8 @@ def main():
                    "ReshapeAndCache + PagedAttention (Setup + Execute each)",
                    "context_tokens": int(step["layout"]["ctx"].sum())},
         "roofline": {"bound": "hbm", "kernel": "paged attention decode", "achieved": achieved,
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+                     "traffic": MEASURED_TRAFFIC.get((args.config, alg_bytes)),
                      "algorithmic_bytes": alg_bytes, "kernel_ms": kernel_ms, "launches": launches.value},
         "step_hbm_gbps": alg_bytes / (ms_per_step * 1e-3) / 1e9,
     }
