@@ -18,8 +18,8 @@
 //                 row is read as whole 128-byte lines exactly once. The loads
 //                 of step i+1 are issued before step i is computed.
 //   VGPR -> LDS : rows are written row-major with a padded pitch (int8 rows
-//                 are widened to fp16 on the way: x ^ 0x80 is spliced under
-//                 the exponent 0x6400 and 1152 is subtracted, which is exact).
+//                 are widened to fp16 on the way: x ^ 0x80 spliced under the
+//                 exponent byte 0x64, i.e. value + 1152, exactly).
 //   QK^T        : S^T[token, head] = K . Q^T on v_mfma_f32_16x16x32. K is the A
 //                 operand (ds_read_b128 per lane), Q^T stays in registers as B.
 //                 The accumulator then holds 4 consecutive tokens of one head
@@ -83,17 +83,22 @@ __device__ __forceinline__ float Unpack(uint32_t word, int half, bool bf16)
     return bf16 ? Bf16ToFloat(bits) : HalfBitsToFloat(bits);
 }
 
-// 4 int8 in one dword -> 4 fp16 in two dwords, exact.
+// int8 rows enter the matrix cores as fp16 numbers equal to value + INT8_BIAS:
+// x ^ 0x80 (value + 128 as an unsigned byte) spliced under the fp16 high byte
+// 0x64 reads as 1024 + (value + 128). The bias is never subtracted per element:
+// in Q.K^T it adds the same constant to every score of a head, which the
+// softmax cancels, and in P.V it adds INT8_BIAS times the sum of P, which is
+// removed once per output element after the normalisation.
+constexpr float INT8_BIAS = 1152.0f;
+
+// 4 int8 in one dword -> 4 biased fp16 in two dwords.
 __device__ __forceinline__ u32x2 Int8x4ToHalf(uint32_t w)
 {
-    const uint32_t x = w ^ 0x80808080u;                       // bytes now hold value + 128
-    const uint32_t e = 0x64646464u;                           // fp16 high byte 0x64: 0x64xx = 1024 + xx
-    const uint32_t a = __builtin_amdgcn_perm(e, x, 0x04010400u); // {x.b0, 0x64, x.b1, 0x64}
-    const uint32_t b = __builtin_amdgcn_perm(e, x, 0x04030402u); // {x.b2, 0x64, x.b3, 0x64}
-    const f16x2 bias = {static_cast<_Float16>(1152.0f), static_cast<_Float16>(1152.0f)};
+    const uint32_t x = w ^ 0x80808080u;
+    const uint32_t e = 0x64646464u;
     u32x2 r;
-    r[0] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, a) - bias);
-    r[1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, b) - bias);
+    r[0] = __builtin_amdgcn_perm(e, x, 0x04010400u); // {x.b0, 0x64, x.b1, 0x64}
+    r[1] = __builtin_amdgcn_perm(e, x, 0x04030402u); // {x.b2, 0x64, x.b3, 0x64}
     return r;
 }
 
@@ -106,6 +111,13 @@ __device__ __forceinline__ void WidenPiece(u32x4 piece, u32x4 &lo, u32x4 &hi)
     const u32x2 d = Int8x4ToHalf(piece[3]);
     lo = u32x4{a[0], a[1], b[0], b[1]};
     hi = u32x4{c[0], c[1], d[0], d[1]};
+}
+
+// 2^x on the hardware unit directly: arguments here are <= 0 (or -inf) and a
+// result below the normal range may flush to zero.
+__device__ __forceinline__ float Exp2(float x)
+{
+    return __builtin_amdgcn_exp2f(x);
 }
 
 __device__ __forceinline__ u32x4 LoadGlobal16(const void *p)
@@ -189,6 +201,8 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
     const unsigned char *vcBase = reinterpret_cast<const unsigned char *>(a.vc);
     constexpr float LOG2E = 1.4426950408889634f;
     const float scale2 = a.qkScale * LOG2E;
+    const uint32_t onePair = BF16 ? 0x3f803f80u : 0x3c003c00u; // {1.0, 1.0} in the operand type
+    const u32x4 ones = {onePair, onePair, onePair, onePair};
 
     int seqIdx = p.firstSeq ? p.firstSeq[wgRange] : p.inlineFirst[wgRange];
     while (PlanSeq(p, seqIdx + 1).stepBegin <= s0) {
@@ -246,7 +260,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
         }
 
         float m = -INFINITY; // running maximum (base-2 exponent units) of head n
-        float l = 0.0f;      // this lane's share of the running denominator
+        f32x4 accL = {0.0f, 0.0f, 0.0f, 0.0f}; // running denominator of head n (the same in all four entries)
         f32x4 acc[NO];
 #pragma unroll
         for (int i = 0; i < NO; ++i) {
@@ -282,9 +296,28 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                 }
             }
         };
-        // `full`: all 32 rows of the step are inside the segment; otherwise rows
-        // at or past tokEnd are not touched and read as zeros.
+        // Loads of a step. When the 16-byte pieces of a row divide the wave evenly,
+        // load i of a full step covers whole consecutive rows of one sub-tile: its
+        // address is a wave-uniform base plus a per-lane offset that never changes.
+        // Otherwise (or in the last, partial step, where rows at or past tokEnd are
+        // not touched and read as zeros) every lane computes its own row.
+        constexpr bool K_UNIFORM = WAVE % KPR == 0;
+        constexpr bool V_UNIFORM = !MLA && WAVE % VPR == 0;
+        constexpr int K_RPL = K_UNIFORM ? WAVE / KPR : 1; // rows per load
+        constexpr int V_RPL = V_UNIFORM ? WAVE / VPR : 1;
+        const uint32_t laneOffK = static_cast<uint32_t>(
+            (static_cast<int64_t>(lane / KPR) * a.kRowStride + static_cast<int64_t>(g) * D) * ESZ + (lane % KPR) * 16);
+        const uint32_t laneOffV = static_cast<uint32_t>(
+            (static_cast<int64_t>(lane / VPR) * a.vRowStride + static_cast<int64_t>(g) * a.vHeadStride) * ESZ +
+            (lane % VPR) * 16);
         auto loadK = [&](int t, const int64_t *rowBase, int i, bool full) -> u32x4 {
+            if constexpr (K_UNIFORM) {
+                if (full) {
+                    const int row0 = i * K_RPL;
+                    const unsigned char *base = kcBase + (rowBase[row0 >> 4] + (row0 & 15)) * a.kRowStride * ESZ;
+                    return LoadStream16(base + laneOffK);
+                }
+            }
             const int pc = i * WAVE + lane;
             const int row = pc / KPR;
             const int col = pc % KPR;
@@ -296,6 +329,13 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
             return v;
         };
         auto loadV = [&](int t, const int64_t *rowBase, int i, bool full) -> u32x4 {
+            if constexpr (V_UNIFORM) {
+                if (full) {
+                    const int row0 = i * V_RPL;
+                    const unsigned char *base = vcBase + (rowBase[row0 >> 4] + (row0 & 15)) * a.vRowStride * ESZ;
+                    return LoadStream16(base + laneOffV);
+                }
+            }
             const int pc = i * WAVE + lane;
             const int row = pc / VPR;
             const int col = pc % VPR;
@@ -430,38 +470,44 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
 
             // ---- online softmax in base 2; lane holds tokens t + 16 sub + 4 kg + r of head n
             float x[8];
-            float mloc = -INFINITY;
-#pragma unroll
-            for (int sub = 0; sub < 2; ++sub) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int tok = t + sub * 16 + kg * 4 + r;
-                    const float v = tok < tokEnd ? s[sub][r] * scale2 : -INFINITY;
-                    x[sub * 4 + r] = v;
-                    mloc = fmaxf(mloc, v);
-                }
-            }
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 16, WAVE));
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
-            const float mNew = fmaxf(m, mloc); // finite: every step holds at least one valid token
-            const float corr = exp2f(m - mNew);
-            m = mNew;
-            float psum = 0.0f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                x[e] = exp2f(x[e] - mNew);
-                psum += x[e];
+                x[e] = s[e >> 2][e & 3] * scale2;
             }
-            l = l * corr + psum;
+            if (t + STEP > tokEnd) { // last step of the segment: mask the tokens past its end
 #pragma unroll
-            for (int i = 0; i < NO; ++i) {
-                acc[i] *= corr;
+                for (int e = 0; e < 8; ++e) {
+                    const int tok = t + (e >> 2) * 16 + kg * 4 + (e & 3);
+                    x[e] = tok < tokEnd ? x[e] : -INFINITY;
+                }
+            }
+            float mloc = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 16, WAVE));
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+            // finite from the first step on: every step holds at least one valid token
+            if (__builtin_amdgcn_ballot_w64(mloc > m) != 0) { // some head's maximum grew: rescale
+                const float mNew = fmaxf(m, mloc);
+                const float corr = Exp2(m - mNew);
+                m = mNew;
+                accL *= corr;
+#pragma unroll
+                for (int i = 0; i < NO; ++i) {
+                    acc[i] *= corr;
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                x[e] = Exp2(x[e] - m);
             }
             u32x4 pop; // P^T as B operand: k = {sub 0: r 0..3, sub 1: r 0..3}
             pop[0] = Pack2<BF16>(x[0], x[1]);
             pop[1] = Pack2<BF16>(x[2], x[3]);
             pop[2] = Pack2<BF16>(x[4], x[5]);
             pop[3] = Pack2<BF16>(x[6], x[7]);
+            // The denominator is the sum of the rounded P that multiplies V, taken by
+            // the matrix core itself from a row of ones: numerator and denominator
+            // then see exactly the same weights.
+            accL = Mma<BF16>(ones, pop, accL);
 
             // ---- O^T += V^T . P^T. The transposing read hands lane (n, kg) the four
             // tokens 4kg..4kg+3 of channel 16 i + n when lane (n, kg) points at
@@ -483,9 +529,9 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
         }
 
         // ---- finish the row (or this wave's share of it)
-        l += __shfl_xor(l, 16, WAVE);
-        l += __shfl_xor(l, 32, WAVE);
+        const float l = accL[0];
         const float inv = 1.0f / l;
+        const float bias = KV8 ? INT8_BIAS : 0.0f; // see Int8x4ToHalf
         if (n < nh) {
             const int h = h0 + n;
             if (complete) {
@@ -496,7 +542,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                     float o[4];
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        o[r] = acc[i][r] * inv;
+                        o[r] = acc[i][r] * inv - bias;
                         if (KV8) {
                             const int c = g * DV + d + r;
                             o[r] = (o[r] + (a.vOff ? static_cast<float>(a.vOff[c]) : 0.0f)) * a.vScale[c];
@@ -517,7 +563,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                 const int64_t ph = static_cast<int64_t>(slot) * a.H + h;
 #pragma unroll
                 for (int i = 0; i < NO; ++i) {
-                    *reinterpret_cast<f32x4 *>(a.partO + ph * DV + i * 16 + kg * 4) = acc[i] * inv;
+                    *reinterpret_cast<f32x4 *>(a.partO + ph * DV + i * 16 + kg * 4) = acc[i] * inv - bias;
                 }
                 if (kg == 0) {
                     a.partLse[ph] = m + log2f(l);
