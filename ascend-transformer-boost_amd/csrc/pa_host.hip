@@ -198,6 +198,7 @@ int PlanStream(AtbmiPaPlan *plan, const int32_t *ctx, int32_t batch)
     while (virtualHeads % headsPerWg != 0) {
         headsPerWg >>= 1;
     }
+    // shared-tile instantiations: PaMfmaWaves already returned a divisor of the head-tile count
     const int tokenSlices = waves / headsPerWg;
     const int headGroups = virtualHeads / headsPerWg;
     try {

@@ -25,6 +25,10 @@ bool PaMfmaSupports(const AtbmiPaShape &shape);
 // Waves per workgroup of the instantiation that serves `shape` (8, or 4 when
 // the LDS tiles of eight waves would not fit).
 int PaMfmaWaves(const AtbmiPaShape &shape);
+// True when the instantiation for `shape` stages one K tile per workgroup and its waves are the
+// query-head tiles of one KV head (combined 576/512 cache with at least 64 query heads per KV head).
+// The plan must then use one token slice and four head tiles per workgroup.
+bool PaMfmaSharedTile(const AtbmiPaShape &shape);
 int LaunchPaMfma(const AtbmiPaShape &shape, const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream);
 // Per-operand-type halves of LaunchPaMfma (one translation unit each, so the
 // instantiations compile in parallel). Return -1 when the shape has no

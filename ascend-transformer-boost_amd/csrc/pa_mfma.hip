@@ -22,8 +22,22 @@ bool PaMfmaSupports(const AtbmiPaShape &s)
     return d == 64 || d == 96 || d == 128 || d == 256;
 }
 
+bool PaMfmaSharedTile(const AtbmiPaShape &s)
+{
+    if (!s.mlaCombined || s.headDimK != 576 || s.headDimV != 512 || s.numKvHeads <= 0) {
+        return false;
+    }
+    const int group = s.numHeads / s.numKvHeads;
+    const int headTiles = (group + PA_MFMA_HEAD_TILE - 1) / PA_MFMA_HEAD_TILE;
+    return (s.numKvHeads * headTiles) % 4 == 0;
+}
+
 int PaMfmaWaves(const AtbmiPaShape &s)
 {
+    if (PaMfmaSharedTile(s)) {
+        // 16 heads x (576 + 512) channels of Q and accumulators need a whole SIMD's registers
+        return 4;
+    }
     // eight waves' K/V tiles fit the 160 KB of LDS up to 128-channel rows
     // (and for the 192/128 combined cache); wider rows run four waves
     return (s.headDimK <= 128 || (s.mlaCombined && s.headDimK <= 192)) ? 8 : 4;

@@ -150,17 +150,21 @@ __device__ __forceinline__ PaSeq PlanSeq(const PaStreamPlan &p, int i)
 // KV8 : int8 cache rows. MLA: V is the first DV channels of the K row.
 // PF  : keep the next step's rows in registers while computing this one.
 // NW  : waves per workgroup.
-template <bool BF16, bool KV8, int D, int DV, bool MLA, bool PF, int NW>
+// SHARED: the waves of a workgroup are the query-head tiles of ONE KV head and token range (MLA with
+//       many heads): the K tile is staged once per workgroup, double-buffered, and read by all waves.
+template <bool BF16, bool KV8, int D, int DV, bool MLA, bool PF, int NW, bool SHARED>
 __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const PaStreamPlan p)
 {
     static_assert(D % 32 == 0 && DV % 16 == 0, "head sizes must fit the MFMA tiles");
     static_assert(!KV8 || DV % 32 == 0, "int8 rows are staged 16 channels at a time");
     static_assert(!(MLA && KV8), "combined cache is 16-bit only");
+    static_assert(!SHARED || MLA, "the shared-tile mode is built for the combined (MLA) cache");
     constexpr int KP = D + K_PAD;                 // K tile pitch in halves
     constexpr int VP = MLA ? KP : DV + V_PAD;     // V tile pitch in halves
     constexpr int K_TILE_BYTES = STEP * KP * 2;
     constexpr int NQ = D / 32;                    // QK MFMAs per 16-token sub-tile
     constexpr int NO = DV / 16;                   // PV MFMAs (output tiles of 16 channels)
+    constexpr bool BIG = NQ > 8 || NO > 16;       // wide rows: operand fetch is pipelined by hand
     constexpr int ESZ = KV8 ? 1 : 2;              // bytes per cache element
     constexpr int KPR = D * ESZ / 16;             // 16-byte pieces per K row
     constexpr int VPR = DV * ESZ / 16;
@@ -177,9 +181,15 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
     const bool qBf16 = a.qIsBf16 != 0;
 
     // Workgroup -> (token range, group of virtual heads); wave -> (virtual head, slice of the range).
-    // Head groups vary fastest so that the workgroups reading one token range run together.
-    const int hgIdx = blockIdx.x % p.headGroups;
-    const int wgRange = blockIdx.x / p.headGroups;
+    // Workgroups go to the 8 XCDs round-robin; the head groups of one token range read the
+    // same cache rows, so they sit 8 workgroup ids apart: same XCD, same L2, launched together.
+    const int octet = blockIdx.x / (8 * p.headGroups);
+    const int within = blockIdx.x % (8 * p.headGroups);
+    const int hgIdx = within / 8;
+    const int wgRange = octet * 8 + within % 8;
+    if (wgRange >= p.numWgRanges) {
+        return;
+    }
     const int vh = hgIdx * p.headsPerWg + wave % p.headsPerWg;
     const int g = vh / p.headTiles;
     const int ht = vh % p.headTiles;
@@ -195,7 +205,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
     const int h0 = g * a.groupSize + ht * HT;
     const int nh = min(HT, a.groupSize - ht * HT);
 
-    unsigned char *kTile = smem + wave * WaveLdsBytes<D, DV, MLA>();
+    unsigned char *kTile = SHARED ? smem : smem + wave * WaveLdsBytes<D, DV, MLA>();
     unsigned char *vTile = MLA ? kTile : kTile + K_TILE_BYTES;
     const unsigned char *kcBase = reinterpret_cast<const unsigned char *>(a.kc);
     const unsigned char *vcBase = reinterpret_cast<const unsigned char *>(a.vc);
@@ -393,139 +403,233 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                 }
             }
         };
-        if constexpr (PF) {
+        if constexpr (PF && !SHARED) {
             loadStage(tokBegin);
         }
 
-        for (int t = tokBegin; t < tokEnd; t += STEP) {
-            if constexpr (PF) {
+        // One 32-token step of attention for this wave's heads, on the tile at kT / vT.
+        auto computeStep = [&](int t, const unsigned char *kT, const unsigned char *vT) {
+                // ---- S^T = K . Q^T for the two 16-token sub-tiles
+                f32x4 s[2] = {f32x4{0.0f, 0.0f, 0.0f, 0.0f}, f32x4{0.0f, 0.0f, 0.0f, 0.0f}};
+                const unsigned char *krow = kT + n * (KP * 2) + kg * 16;
+                if constexpr (BIG) {
+                    // Wide rows: operands are fetched two MFMAs ahead and the order is pinned,
+                    // otherwise the scheduler hoists every LDS read and spills.
+                    u32x4 ka[3], kb[3];
+                    ka[0] = *reinterpret_cast<const u32x4 *>(krow);
+                    kb[0] = *reinterpret_cast<const u32x4 *>(krow + 16 * (KP * 2));
+                    ka[1] = *reinterpret_cast<const u32x4 *>(krow + 64);
+                    kb[1] = *reinterpret_cast<const u32x4 *>(krow + 16 * (KP * 2) + 64);
 #pragma unroll
-                for (int i = 0; i < NKP; ++i) {
-                    storePiece(kTile, KP, KPR, i, kStage[i]);
-                }
+                    for (int j = 0; j < NQ; ++j) {
+                        if (j + 2 < NQ) {
+                            ka[(j + 2) % 3] = *reinterpret_cast<const u32x4 *>(krow + (j + 2) * 64);
+                            kb[(j + 2) % 3] = *reinterpret_cast<const u32x4 *>(krow + 16 * (KP * 2) + (j + 2) * 64);
+                        }
+                        s[0] = Mma<BF16>(ka[j % 3], qreg[j], s[0]);
+                        s[1] = Mma<BF16>(kb[j % 3], qreg[j], s[1]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                } else {
 #pragma unroll
-                for (int i = 0; i < NVP; ++i) {
-                    storePiece(vTile, VP, VPR, i, vStage[i]);
+                    for (int sub = 0; sub < 2; ++sub) {
+#pragma unroll
+                        for (int j = 0; j < NQ; ++j) {
+                            const u32x4 kop = *reinterpret_cast<const u32x4 *>(krow + sub * 16 * (KP * 2) + j * 64);
+                            s[sub] = Mma<BF16>(kop, qreg[j], s[sub]);
+                        }
+                    }
                 }
-                if (t + STEP < tokEnd) {
-                    loadStage(t + STEP);
+
+                // ---- online softmax in base 2; lane holds tokens t + 16 sub + 4 kg + r of head n
+                float x[8];
+    #pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    x[e] = s[e >> 2][e & 3] * scale2;
                 }
-            } else {
-                // Large rows: stage a few pieces at a time to bound register use.
-                constexpr int BATCH = 6;
+                if (t + STEP > tokEnd) { // last step of the segment: mask the tokens past its end
+    #pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const int tok = t + (e >> 2) * 16 + kg * 4 + (e & 3);
+                        x[e] = tok < tokEnd ? x[e] : -INFINITY;
+                    }
+                }
+                float mloc = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+                mloc = fmaxf(mloc, __shfl_xor(mloc, 16, WAVE));
+                mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+                // finite from the first step on: every step holds at least one valid token
+                if (__builtin_amdgcn_ballot_w64(mloc > m) != 0) { // some head's maximum grew: rescale
+                    const float mNew = fmaxf(m, mloc);
+                    const float corr = Exp2(m - mNew);
+                    m = mNew;
+                    accL *= corr;
+    #pragma unroll
+                    for (int i = 0; i < NO; ++i) {
+                        acc[i] *= corr;
+                    }
+                }
+    #pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    x[e] = Exp2(x[e] - m);
+                }
+                u32x4 pop; // P^T as B operand: k = {sub 0: r 0..3, sub 1: r 0..3}
+                pop[0] = Pack2<BF16>(x[0], x[1]);
+                pop[1] = Pack2<BF16>(x[2], x[3]);
+                pop[2] = Pack2<BF16>(x[4], x[5]);
+                pop[3] = Pack2<BF16>(x[6], x[7]);
+                // The denominator is the sum of the rounded P that multiplies V, taken by
+                // the matrix core itself from a row of ones: numerator and denominator
+                // then see exactly the same weights.
+                accL = Mma<BF16>(ones, pop, accL);
+
+                // ---- O^T += V^T . P^T. The transposing read hands lane (n, kg) the four
+                // tokens 4kg..4kg+3 of channel 16 i + n when lane (n, kg) points at
+                // token 4kg + n/4, channels 16 i + 4 (n%4) .. +4.
+                const unsigned char *vrow = vT + (kg * 4 + (n >> 2)) * (VP * 2) + (n & 3) * 8;
+                auto readV = [&](int i) -> u32x4 {
+                    const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (__attribute__((address_space(3))) i16x4 *)(vrow + i * 32));
+                    const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (__attribute__((address_space(3))) i16x4 *)(vrow + 16 * (VP * 2) + i * 32));
+                    const u32x2 lo2 = __builtin_bit_cast(u32x2, lo);
+                    const u32x2 hi2 = __builtin_bit_cast(u32x2, hi);
+                    return u32x4{lo2[0], lo2[1], hi2[0], hi2[1]};
+                };
+                if constexpr (BIG) {
+                    u32x4 vop[4];
+                    vop[0] = readV(0);
+                    vop[1] = readV(1);
+                    vop[2] = readV(2);
+#pragma unroll
+                    for (int i = 0; i < NO; ++i) {
+                        if (i + 3 < NO) {
+                            vop[(i + 3) % 4] = readV(i + 3);
+                        }
+                        acc[i] = Mma<BF16>(vop[i % 4], pop, acc[i]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < NO; ++i) {
+                        acc[i] = Mma<BF16>(readV(i), pop, acc[i]);
+                    }
+                }
+        };
+
+        if constexpr (SHARED) {
+            // Cooperative staging: the NW*64 threads fetch the 32 latent rows of a step
+            // together (whole rows, consecutive threads on consecutive 16-byte pieces),
+            // one step ahead in registers, into the buffer the waves are not reading.
+            constexpr int NT = NW * WAVE;
+            constexpr int PIECES = STEP * KPR;
+            constexpr int NSP = (PIECES + NT - 1) / NT;
+            u32x4 stage[NSP];
+            const int tid = threadIdx.x;
+            auto coopLoad = [&](int t) {
                 int64_t rowBase[2];
                 nextRows(rowBase);
-                const bool full = t + STEP <= tokEnd;
 #pragma unroll
-                for (int i0 = 0; i0 < NKP; i0 += BATCH) {
-                    u32x4 tmp[BATCH];
-#pragma unroll
-                    for (int b = 0; b < BATCH; ++b) {
-                        if (i0 + b < NKP) {
-                            tmp[b] = loadK(t, rowBase, i0 + b, full);
-                        }
-                    }
-#pragma unroll
-                    for (int b = 0; b < BATCH; ++b) {
-                        if (i0 + b < NKP) {
-                            storePiece(kTile, KP, KPR, i0 + b, tmp[b]);
-                        }
+                for (int i = 0; i < NSP; ++i) {
+                    const int pc = i * NT + tid;
+                    const int row = pc / KPR;
+                    const int col = pc % KPR;
+                    stage[i] = u32x4{0u, 0u, 0u, 0u};
+                    if (pc < PIECES && t + row < tokEnd) {
+                        const int64_t r = rowBase[row >> 4] + (row & 15);
+                        // plain load: the other head groups of this range fetch the same rows from L2
+                        stage[i] = LoadGlobal16(kcBase + (r * a.kRowStride + static_cast<int64_t>(g) * D) * 2 + col * 16);
                     }
                 }
+            };
+            auto coopStore = [&](unsigned char *tile) {
 #pragma unroll
-                for (int i0 = 0; i0 < NVP; i0 += BATCH) {
-                    u32x4 tmp[BATCH];
-#pragma unroll
-                    for (int b = 0; b < BATCH; ++b) {
-                        if (i0 + b < NVP) {
-                            tmp[b] = loadV(t, rowBase, i0 + b, full);
-                        }
-                    }
-#pragma unroll
-                    for (int b = 0; b < BATCH; ++b) {
-                        if (i0 + b < NVP) {
-                            storePiece(vTile, VP, VPR, i0 + b, tmp[b]);
-                        }
+                for (int i = 0; i < NSP; ++i) {
+                    const int pc = i * NT + tid;
+                    if (pc < PIECES) {
+                        *reinterpret_cast<u32x4 *>(tile + (pc / KPR) * (KP * 2) + (pc % KPR) * 16) = stage[i];
                     }
                 }
+            };
+            int buf = 0;
+            coopLoad(tokBegin);
+            coopStore(smem);
+            __syncthreads();
+            for (int t = tokBegin; t < tokEnd; t += STEP) {
+                const bool more = t + STEP < tokEnd;
+                if (more) {
+                    coopLoad(t + STEP);
+                }
+                const unsigned char *cur = smem + buf * K_TILE_BYTES;
+                computeStep(t, cur, cur);
+                if (more) {
+                    coopStore(smem + (buf ^ 1) * K_TILE_BYTES);
+                }
+                __syncthreads(); // everyone is done with `cur`, the other buffer is complete
+                buf ^= 1;
             }
-            // The tile is private to this wave: LDS executes a wave's accesses in
-            // order, only the compiler has to be kept from moving reads above writes.
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        } else {
+            for (int t = tokBegin; t < tokEnd; t += STEP) {
+                if constexpr (PF) {
+#pragma unroll
+                    for (int i = 0; i < NKP; ++i) {
+                        storePiece(kTile, KP, KPR, i, kStage[i]);
+                    }
+#pragma unroll
+                    for (int i = 0; i < NVP; ++i) {
+                        storePiece(vTile, VP, VPR, i, vStage[i]);
+                    }
+                    if (t + STEP < tokEnd) {
+                        loadStage(t + STEP);
+                    }
+                } else {
+                    // Large rows: stage a few pieces at a time to bound register use.
+                    constexpr int BATCH = 6;
+                    int64_t rowBase[2];
+                    nextRows(rowBase);
+                    const bool full = t + STEP <= tokEnd;
+#pragma unroll
+                    for (int i0 = 0; i0 < NKP; i0 += BATCH) {
+                        u32x4 tmp[BATCH];
+#pragma unroll
+                        for (int b = 0; b < BATCH; ++b) {
+                            if (i0 + b < NKP) {
+                                tmp[b] = loadK(t, rowBase, i0 + b, full);
+                            }
+                        }
+#pragma unroll
+                        for (int b = 0; b < BATCH; ++b) {
+                            if (i0 + b < NKP) {
+                                storePiece(kTile, KP, KPR, i0 + b, tmp[b]);
+                            }
+                        }
+                    }
+#pragma unroll
+                    for (int i0 = 0; i0 < NVP; i0 += BATCH) {
+                        u32x4 tmp[BATCH];
+#pragma unroll
+                        for (int b = 0; b < BATCH; ++b) {
+                            if (i0 + b < NVP) {
+                                tmp[b] = loadV(t, rowBase, i0 + b, full);
+                            }
+                        }
+#pragma unroll
+                        for (int b = 0; b < BATCH; ++b) {
+                            if (i0 + b < NVP) {
+                                storePiece(vTile, VP, VPR, i0 + b, tmp[b]);
+                            }
+                        }
+                    }
+                }
+                // The tile is private to this wave: LDS executes a wave's accesses in
+                // order, only the compiler has to be kept from moving reads above writes.
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-            // ---- S^T = K . Q^T for the two 16-token sub-tiles
-            f32x4 s[2];
-#pragma unroll
-            for (int sub = 0; sub < 2; ++sub) {
-                s[sub] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-                const unsigned char *krow = kTile + (sub * 16 + n) * (KP * 2) + kg * 16;
-#pragma unroll
-                for (int j = 0; j < NQ; ++j) {
-                    const u32x4 kop = *reinterpret_cast<const u32x4 *>(krow + j * 64);
-                    s[sub] = Mma<BF16>(kop, qreg[j], s[sub]);
-                }
+                computeStep(t, kTile, vTile);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
             }
-
-            // ---- online softmax in base 2; lane holds tokens t + 16 sub + 4 kg + r of head n
-            float x[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                x[e] = s[e >> 2][e & 3] * scale2;
-            }
-            if (t + STEP > tokEnd) { // last step of the segment: mask the tokens past its end
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int tok = t + (e >> 2) * 16 + kg * 4 + (e & 3);
-                    x[e] = tok < tokEnd ? x[e] : -INFINITY;
-                }
-            }
-            float mloc = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 16, WAVE));
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
-            // finite from the first step on: every step holds at least one valid token
-            if (__builtin_amdgcn_ballot_w64(mloc > m) != 0) { // some head's maximum grew: rescale
-                const float mNew = fmaxf(m, mloc);
-                const float corr = Exp2(m - mNew);
-                m = mNew;
-                accL *= corr;
-#pragma unroll
-                for (int i = 0; i < NO; ++i) {
-                    acc[i] *= corr;
-                }
-            }
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                x[e] = Exp2(x[e] - m);
-            }
-            u32x4 pop; // P^T as B operand: k = {sub 0: r 0..3, sub 1: r 0..3}
-            pop[0] = Pack2<BF16>(x[0], x[1]);
-            pop[1] = Pack2<BF16>(x[2], x[3]);
-            pop[2] = Pack2<BF16>(x[4], x[5]);
-            pop[3] = Pack2<BF16>(x[6], x[7]);
-            // The denominator is the sum of the rounded P that multiplies V, taken by
-            // the matrix core itself from a row of ones: numerator and denominator
-            // then see exactly the same weights.
-            accL = Mma<BF16>(ones, pop, accL);
-
-            // ---- O^T += V^T . P^T. The transposing read hands lane (n, kg) the four
-            // tokens 4kg..4kg+3 of channel 16 i + n when lane (n, kg) points at
-            // token 4kg + n/4, channels 16 i + 4 (n%4) .. +4.
-            const unsigned char *vrow = vTile + (kg * 4 + (n >> 2)) * (VP * 2) + (n & 3) * 8;
-#pragma unroll
-            for (int i = 0; i < NO; ++i) {
-                const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (__attribute__((address_space(3))) i16x4 *)(vrow + i * 32));
-                const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (__attribute__((address_space(3))) i16x4 *)(vrow + 16 * (VP * 2) + i * 32));
-                const u32x2 lo2 = __builtin_bit_cast(u32x2, lo);
-                const u32x2 hi2 = __builtin_bit_cast(u32x2, hi);
-                const u32x4 vop = {lo2[0], lo2[1], hi2[0], hi2[1]};
-                acc[i] = Mma<BF16>(vop, pop, acc[i]);
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
         }
 
         // ---- finish the row (or this wave's share of it)
@@ -573,11 +677,11 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
     }
 }
 
-template <bool BF16, bool KV8, int D, int DV, bool MLA, bool PF, int NW>
+template <bool BF16, bool KV8, int D, int DV, bool MLA, bool PF, int NW, bool SHARED = false>
 int Launch(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
 {
-    auto kernel = PaMfmaKernel<BF16, KV8, D, DV, MLA, PF, NW>;
-    constexpr int lds = NW * WaveLdsBytes<D, DV, MLA>();
+    auto kernel = PaMfmaKernel<BF16, KV8, D, DV, MLA, PF, NW, SHARED>;
+    constexpr int lds = SHARED ? 2 * WaveLdsBytes<D, DV, MLA>() : NW * WaveLdsBytes<D, DV, MLA>();
     static_assert(lds <= 160 * 1024, "tiles exceed the 160 KB of LDS per CU");
     static bool configured = false; // one attribute call per instantiation and process
     if (!configured) {
@@ -585,11 +689,11 @@ int Launch(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
                                             hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         configured = true;
     }
-    if (plan.headsPerWg * plan.tokenSlices != NW) {
+    if (plan.headsPerWg * plan.tokenSlices != NW || (SHARED && plan.tokenSlices != 1)) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: plan made for %d waves, kernel has %d",
                     plan.headsPerWg * plan.tokenSlices, NW);
     }
-    const int64_t grid = static_cast<int64_t>(plan.numWgRanges) * plan.headGroups;
+    const int64_t grid = (static_cast<int64_t>(plan.numWgRanges) + 7) / 8 * 8 * plan.headGroups;
     if (grid <= 0 || grid > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: grid of %lld workgroups is out of range", (long long)grid);
     }
