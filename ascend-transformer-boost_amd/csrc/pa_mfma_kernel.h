@@ -165,6 +165,8 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
     constexpr int NQ = D / 32;                    // QK MFMAs per 16-token sub-tile
     constexpr int NO = DV / 16;                   // PV MFMAs (output tiles of 16 channels)
     constexpr bool BIG = NQ > 8 || NO > 16;       // wide rows: operand fetch is pipelined by hand
+    constexpr int KD = 2;                         // ... this many MFMA pairs ahead for K
+    constexpr int VD = 3;                         // ... and this many MFMAs ahead for V
     constexpr int ESZ = KV8 ? 1 : 2;              // bytes per cache element
     constexpr int KPR = D * ESZ / 16;             // 16-byte pieces per K row
     constexpr int VPR = DV * ESZ / 16;
@@ -415,19 +417,21 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                 if constexpr (BIG) {
                     // Wide rows: operands are fetched two MFMAs ahead and the order is pinned,
                     // otherwise the scheduler hoists every LDS read and spills.
-                    u32x4 ka[3], kb[3];
-                    ka[0] = *reinterpret_cast<const u32x4 *>(krow);
-                    kb[0] = *reinterpret_cast<const u32x4 *>(krow + 16 * (KP * 2));
-                    ka[1] = *reinterpret_cast<const u32x4 *>(krow + 64);
-                    kb[1] = *reinterpret_cast<const u32x4 *>(krow + 16 * (KP * 2) + 64);
+                    u32x4 ka[KD + 1], kb[KD + 1];
+#pragma unroll
+                    for (int j = 0; j < KD && j < NQ; ++j) {
+                        ka[j] = *reinterpret_cast<const u32x4 *>(krow + j * 64);
+                        kb[j] = *reinterpret_cast<const u32x4 *>(krow + 16 * (KP * 2) + j * 64);
+                    }
 #pragma unroll
                     for (int j = 0; j < NQ; ++j) {
-                        if (j + 2 < NQ) {
-                            ka[(j + 2) % 3] = *reinterpret_cast<const u32x4 *>(krow + (j + 2) * 64);
-                            kb[(j + 2) % 3] = *reinterpret_cast<const u32x4 *>(krow + 16 * (KP * 2) + (j + 2) * 64);
+                        if (j + KD < NQ) {
+                            ka[(j + KD) % (KD + 1)] = *reinterpret_cast<const u32x4 *>(krow + (j + KD) * 64);
+                            kb[(j + KD) % (KD + 1)] =
+                                *reinterpret_cast<const u32x4 *>(krow + 16 * (KP * 2) + (j + KD) * 64);
                         }
-                        s[0] = Mma<BF16>(ka[j % 3], qreg[j], s[0]);
-                        s[1] = Mma<BF16>(kb[j % 3], qreg[j], s[1]);
+                        s[0] = Mma<BF16>(ka[j % (KD + 1)], qreg[j], s[0]);
+                        s[1] = Mma<BF16>(kb[j % (KD + 1)], qreg[j], s[1]);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 } else {
@@ -496,16 +500,17 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                     return u32x4{lo2[0], lo2[1], hi2[0], hi2[1]};
                 };
                 if constexpr (BIG) {
-                    u32x4 vop[4];
-                    vop[0] = readV(0);
-                    vop[1] = readV(1);
-                    vop[2] = readV(2);
+                    u32x4 vop[VD + 1];
+#pragma unroll
+                    for (int i = 0; i < VD && i < NO; ++i) {
+                        vop[i] = readV(i);
+                    }
 #pragma unroll
                     for (int i = 0; i < NO; ++i) {
-                        if (i + 3 < NO) {
-                            vop[(i + 3) % 4] = readV(i + 3);
+                        if (i + VD < NO) {
+                            vop[(i + VD) % (VD + 1)] = readV(i + VD);
                         }
-                        acc[i] = Mma<BF16>(vop[i % 4], pop, acc[i]);
+                        acc[i] = Mma<BF16>(vop[i % (VD + 1)], pop, acc[i]);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 } else {
