@@ -199,7 +199,12 @@ int PlanStream(AtbmiPaPlan *plan, const int32_t *ctx, int32_t batch)
         headsPerWg >>= 1;
     }
     // shared-tile instantiations: PaMfmaWaves already returned a divisor of the head-tile count
-    const int tokenSlices = waves / headsPerWg;
+    int tokenSlices = waves / headsPerWg;
+    if (PaMlaWide(s)) {
+        // each wave takes two 16-head tiles: a workgroup covers 128 heads of one token range
+        headsPerWg = PA_MLA_HEADS_PER_WG / PA_MFMA_HEAD_TILE;
+        tokenSlices = 1;
+    }
     const int headGroups = virtualHeads / headsPerWg;
     try {
         plan->seqTable.clear();

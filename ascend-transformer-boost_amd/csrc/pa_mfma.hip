@@ -1,4 +1,5 @@
 // Shape coverage and dispatch of the MFMA decode-attention kernel.
+#include <cstdlib>
 #include "pa_internal.h"
 
 namespace atbmi {
@@ -22,8 +23,22 @@ bool PaMfmaSupports(const AtbmiPaShape &s)
     return d == 64 || d == 96 || d == 128 || d == 256;
 }
 
+bool PaMlaWide(const AtbmiPaShape &s)
+{
+    static const bool enabled = [] {
+        const char *v = getenv("ATBMI_PA_MLA_WIDE");
+        return !(v && v[0] == '0');
+    }();
+    return enabled && s.mlaCombined && s.kvDtype != ATBMI_INT8 && s.headDimK == 576 && s.headDimV == 512 &&
+           s.numKvHeads == 1 && s.numHeads % PA_MLA_HEADS_PER_WG == 0 && s.blockSize % 16 == 0 &&
+           (s.qScale == 0.0f || s.qScale == 1.0f); // a q pre-scale takes the 16-head kernel
+}
+
 bool PaMfmaSharedTile(const AtbmiPaShape &s)
 {
+    if (PaMlaWide(s)) {
+        return false;
+    }
     if (!s.mlaCombined || s.headDimK != 576 || s.headDimV != 512 || s.numKvHeads <= 0) {
         return false;
     }
@@ -34,6 +49,9 @@ bool PaMfmaSharedTile(const AtbmiPaShape &s)
 
 int PaMfmaWaves(const AtbmiPaShape &s)
 {
+    if (PaMlaWide(s)) {
+        return PA_MLA_WAVES;
+    }
     if (PaMfmaSharedTile(s)) {
         // 16 heads x (576 + 512) channels of Q and accumulators need a whole SIMD's registers
         return 4;
@@ -46,6 +64,9 @@ int PaMfmaWaves(const AtbmiPaShape &s)
 int LaunchPaMfma(const AtbmiPaShape &s, const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
 {
     int rc;
+    if (PaMlaWide(s)) {
+        return LaunchPaMlaWide(s, args, plan, stream);
+    }
     if (s.kvDtype == ATBMI_INT8) {
         rc = LaunchPaMfmaInt8(s, args, plan, stream);
     } else if (s.qDtype == ATBMI_BF16) {

@@ -1,0 +1,14 @@
+// Instantiations and dispatch of the 128-head decode-attention kernel for the combined MLA cache.
+#include "pa_mla_kernel.h"
+
+namespace atbmi {
+
+int LaunchPaMlaWide(const AtbmiPaShape &s, const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
+{
+    if (!PaMlaWide(s)) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: shape does not fit the 128-head MLA kernel");
+    }
+    return s.qDtype == ATBMI_BF16 ? mla::LaunchWide<true>(args, plan, stream) : mla::LaunchWide<false>(args, plan, stream);
+}
+
+} // namespace atbmi

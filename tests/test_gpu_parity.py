@@ -336,6 +336,39 @@ def test_paged_attention_mla_combined_cache(binding, oracle, dev, stream, case):
         assert_close(got, want, TOL[dtype], "kernel=%d" % kernel)
 
 
+# The 128-head kernel (combined 576/512 cache, heads a multiple of 128) has paths of its own:
+# batch, heads, block, ctx, dtype, chunk_tokens, what the case is for
+MLA_WIDE_MATRIX = [
+    (3, 256, 128, [700, 45, 1], torch.bfloat16, None, "two head groups of 128, ragged lengths, one token"),
+    (6, 128, 128, [333, 32, 31, 33, 64, 257], torch.float16, 64, "ranges of two steps: rows cut everywhere"),
+    (2, 128, 16, [18000, 500], torch.bfloat16, 32768, "block size 16, one range: more block ids than the LDS table holds"),
+    (2, 128, 16, [18000, 500], torch.bfloat16, None, "block size 16, many short ranges"),
+    (5, 128, 32, [96, 4100, 1, 160, 2047], torch.float16, 4096, "block size 32, ranges spanning sequences"),
+    (1, 128, 128, [12345], torch.float16, 320, "one long row merged from many ranges"),
+]
+
+
+@pytest.mark.parametrize("case", MLA_WIDE_MATRIX, ids=lambda c: "b%d_h%d_bs%d_%s" % (
+    c[0], c[1], c[2], str(c[4]).split(".")[-1]))
+def test_paged_attention_mla_128_head_kernel(binding, oracle, dev, stream, case):
+    """Checked against the oracle and, element by element, against the fp32 scalar kernel."""
+    batch, heads, block, ctx, dtype, chunk, _ = case
+    rng = _rng(300 + batch + block)
+    q, kc, _, tables, ctx = _pa_inputs(rng, dev, batch, heads, 1, block, 576, 512, ctx, dtype, std=0.5)
+    scale = 1.0 / math.sqrt(576)
+    want = oracle_pa(oracle, q, kc, None, tables, ctx, scale, mla_dv=512)
+    got, info = pa_decode_cabi(binding, stream, q, kc, None, tables, ctx, scale, mla_dv=512,
+                               kernel=binding.ATBMI_PA_KERNEL_MFMA, chunk_tokens=chunk, return_plan_info=True)
+    assert_close(got, want, TOL[dtype], "128-head kernel, %d ranges" % info["chunks"])
+    ref = pa_decode_cabi(binding, stream, q, kc, None, tables, ctx, scale, mla_dv=512,
+                         kernel=binding.ATBMI_PA_KERNEL_SCALAR)
+    assert_close(got, ref.float().cpu().numpy(), TOL[dtype], "128-head kernel vs scalar kernel")
+    for rep in range(3):  # same answer on relaunch: the tile buffers and the id table carry nothing over
+        again = pa_decode_cabi(binding, stream, q, kc, None, tables, ctx, scale, mla_dv=512,
+                               kernel=binding.ATBMI_PA_KERNEL_MFMA, chunk_tokens=chunk)
+        assert torch.equal(again, got), "relaunch %d differs" % rep
+
+
 def test_mla_through_operation_api_and_split_head_sizes(binding, oracle, dev, stream):
     rng = _rng(61)
     c = binding.Context(stream)
