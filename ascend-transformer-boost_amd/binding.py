@@ -89,14 +89,16 @@ class AtbmiPaShape(ctypes.Structure):
         ("numKvHeads", ctypes.c_int32), ("headDimK", ctypes.c_int32), ("headDimV", ctypes.c_int32),
         ("blockSize", ctypes.c_int32), ("numBlocks", ctypes.c_int32), ("maxBlocksPerSeq", ctypes.c_int32),
         ("numQueryRows", ctypes.c_int32), ("mlaCombined", ctypes.c_int32), ("hasOffset", ctypes.c_int32),
-        ("kernel", ctypes.c_int32), ("reserved", ctypes.c_int32), ("qkScale", ctypes.c_float),
-        ("qScale", ctypes.c_float),
+        ("kernel", ctypes.c_int32), ("hasMask", ctypes.c_int32), ("qkScale", ctypes.c_float),
+        ("qScale", ctypes.c_float), ("maskBatchStride", ctypes.c_int64), ("maskHeadStride", ctypes.c_int64),
+        ("maskLen", ctypes.c_int32), ("hasLogN", ctypes.c_int32),
     ]
 
 
 class AtbmiPaTensors(ctypes.Structure):
     _fields_ = [(n, ctypes.c_void_p) for n in
-                ("query", "keyCache", "valueCache", "blockTables", "kScale", "kOffset", "vScale", "vOffset", "out")]
+                ("query", "keyCache", "valueCache", "blockTables", "kScale", "kOffset", "vScale", "vOffset", "out",
+                 "mask", "logN")]
 
 
 _kernels = None

@@ -75,6 +75,14 @@ struct PaArgs {
     int64_t vRowStride; // same for the value cache (G*Dv, or G*D when V aliases K)
     int32_t vHeadStride; // elements between KV heads inside a value row (Dv, or D when V aliases K)
     int32_t finishV;     // 1: partial outputs are still in int8 units; the final write applies vScale/vOff
+    // Additive score bias (null: none), in the query's type: the score of the sequence in batch row b,
+    // head h, token t gets mask[b * maskBatchStride + h * maskHeadStride + t] added after scaling.
+    const void *mask;
+    int64_t maskBatchStride;
+    int64_t maskHeadStride;
+    int32_t maskLen;     // tokens per mask row
+    int32_t maskVec;     // 1: every mask row starts on an 8-byte boundary (4-token vector loads are legal)
+    const float *logN;   // per batch row factor on qkScale (null: none)
 };
 
 // ---- Plan of the MFMA kernel ------------------------------------------------

@@ -90,6 +90,7 @@ struct AtbmiPaPlan {
     int64_t totalCtx = 0;
     int64_t tableEntries = 0;
     int32_t nonEmpty = 0;
+    int32_t maxCtx = 0;
 
     uint64_t offItems = 0, offSeqs = 0, offPartO = 0, offPartLse = 0, blobBytes = 0, wsBytes = 0;
     std::vector<uint8_t> blob; // items then reduceSeqs, as uploaded
@@ -145,6 +146,10 @@ extern "C" int atbmi_pa_plan_create(const AtbmiPaShape *shape, AtbmiPaPlan **pla
     }
     if (s.hasOffset && s.kvDtype != ATBMI_INT8) {
         return Fail(ERR_INVALID_PARAM, "pa_plan_create: offsets only apply to an int8 cache");
+    }
+    if (s.hasMask && (s.maskLen <= 0 || s.maskBatchStride < 0 || s.maskHeadStride < 0)) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: mask row length %d, strides %lld / %lld", s.maskLen,
+                    (long long)s.maskBatchStride, (long long)s.maskHeadStride);
     }
     AtbmiPaPlan *p = new (std::nothrow) AtbmiPaPlan();
     if (!p) {
@@ -347,6 +352,7 @@ extern "C" int atbmi_pa_plan_update(AtbmiPaPlan *plan, const int32_t *ctx, int32
     plan->totalCtx = total;
     plan->tableEntries = tableEntries;
     plan->nonEmpty = nonEmpty;
+    plan->maxCtx = *std::max_element(ctx, ctx + batch);
     plan->items.clear();
     plan->reduceSeqs.clear();
 
@@ -463,6 +469,15 @@ extern "C" uint64_t atbmi_pa_plan_algorithmic_bytes(const AtbmiPaPlan *plan)
         const uint64_t vec = static_cast<uint64_t>(s.numKvHeads) * (s.headDimK + s.headDimV) * 4;
         bytes += vec * (s.hasOffset ? 2 : 1);
     }
+    if (s.hasMask) {
+        // each distinct mask row once, over the tokens attended to
+        const uint64_t tokens = s.maskBatchStride ? static_cast<uint64_t>(plan->totalCtx)
+                                                  : static_cast<uint64_t>(plan->maxCtx);
+        bytes += tokens * (s.maskHeadStride ? s.numHeads : 1) * 2;
+    }
+    if (s.hasLogN) {
+        bytes += static_cast<uint64_t>(plan->batch) * 4;
+    }
     return bytes;
 }
 
@@ -540,6 +555,9 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
     if (s.hasOffset && (!t->kOffset || !t->vOffset)) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: hasOffset needs kOffset and vOffset");
     }
+    if ((s.hasMask && !t->mask) || (s.hasLogN && !t->logN)) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: the plan was made with a mask / logN, none given");
+    }
     if (plan->wsBytes > 0 && (!workspace || workspaceBytes < plan->wsBytes)) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: workspace of %llu bytes, %llu needed",
                     (unsigned long long)workspaceBytes, (unsigned long long)plan->wsBytes);
@@ -582,6 +600,15 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
     a.vRowStride = s.mlaCombined ? a.kRowStride : static_cast<int64_t>(s.numKvHeads) * s.headDimV;
     a.vHeadStride = s.mlaCombined ? s.headDimK : s.headDimV;
     a.finishV = (plan->useMfma && s.kvDtype == ATBMI_INT8) ? 1 : 0;
+    if (s.hasMask) {
+        a.mask = t->mask;
+        a.maskBatchStride = s.maskBatchStride;
+        a.maskHeadStride = s.maskHeadStride;
+        a.maskLen = s.maskLen;
+        a.maskVec = (reinterpret_cast<uintptr_t>(t->mask) % 8 == 0 && s.maskBatchStride % 4 == 0 &&
+                     s.maskHeadStride % 4 == 0) ? 1 : 0;
+    }
+    a.logN = s.hasLogN ? t->logN : nullptr;
 
     TimingRecord rec{nullptr, nullptr};
     bool timed = false;

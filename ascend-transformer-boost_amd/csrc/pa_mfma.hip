@@ -31,7 +31,7 @@ bool PaMlaWide(const AtbmiPaShape &s)
     }();
     return enabled && s.mlaCombined && s.kvDtype != ATBMI_INT8 && s.headDimK == 576 && s.headDimV == 512 &&
            s.numKvHeads == 1 && s.numHeads % PA_MLA_HEADS_PER_WG == 0 && s.blockSize % 16 == 0 &&
-           (s.qScale == 0.0f || s.qScale == 1.0f); // a q pre-scale takes the 16-head kernel
+           (s.qScale == 0.0f || s.qScale == 1.0f) && !s.hasMask && !s.hasLogN; // those take the 16-head kernel
 }
 
 bool PaMfmaSharedTile(const AtbmiPaShape &s)

@@ -233,6 +233,14 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
         const int tokEnd = min(sq.ctxLen, (segEnd - sq.stepBegin) * STEP);
         const bool complete = segBegin == sq.stepBegin && segEnd == seqEnd;
         const int qRow = seqIdx; // the i-th non-empty sequence owns query/output row i
+        // SCALE_TYPE_LOGN: a per-sequence factor on the score scale, indexed like the block tables
+        const float scaleSeq = a.logN ? scale2 * a.logN[sq.tableRow] : scale2;
+        // additive score bias of head n of this sequence (heads past the tile's end borrow its last one)
+        const uint16_t *maskRow = nullptr;
+        if (a.mask) {
+            maskRow = reinterpret_cast<const uint16_t *>(a.mask) + static_cast<int64_t>(sq.tableRow) * a.maskBatchStride +
+                      static_cast<int64_t>(h0 + min(n, nh - 1)) * a.maskHeadStride;
+        }
 
         // ---- Q^T as B operand: lane (n, kg) holds q[h0+n][32j + 8kg .. +8) for j < NQ
         u32x4 qreg[NQ];
@@ -411,6 +419,24 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
 
         // One 32-token step of attention for this wave's heads, on the tile at kT / vT.
         auto computeStep = [&](int t, const unsigned char *kT, const unsigned char *vT) {
+                // The bias of this lane's 8 tokens is requested before the MFMAs and used after them.
+                u32x2 bias[2] = {u32x2{0u, 0u}, u32x2{0u, 0u}};
+                if (maskRow) {
+#pragma unroll
+                    for (int sub = 0; sub < 2; ++sub) {
+                        const int tok0 = t + sub * 16 + kg * 4;
+                        if (a.maskVec && tok0 + 4 <= a.maskLen) {
+                            bias[sub] = *reinterpret_cast<const u32x2 *>(maskRow + tok0);
+                        } else {
+                            uint32_t h[4];
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) {
+                                h[r] = tok0 + r < a.maskLen ? maskRow[tok0 + r] : 0u;
+                            }
+                            bias[sub] = u32x2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+                        }
+                    }
+                }
                 // ---- S^T = K . Q^T for the two 16-token sub-tiles
                 f32x4 s[2] = {f32x4{0.0f, 0.0f, 0.0f, 0.0f}, f32x4{0.0f, 0.0f, 0.0f, 0.0f}};
                 const unsigned char *krow = kT + n * (KP * 2) + kg * 16;
@@ -449,7 +475,13 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                 float x[8];
     #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    x[e] = s[e >> 2][e & 3] * scale2;
+                    x[e] = s[e >> 2][e & 3] * scaleSeq;
+                }
+                if (maskRow) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        x[e] += Unpack(bias[e >> 2][(e >> 1) & 1], e & 1, qBf16) * LOG2E;
+                    }
                 }
                 if (t + STEP > tokEnd) { // last step of the segment: mask the tokens past its end
     #pragma unroll
@@ -461,10 +493,11 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                 float mloc = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
                 mloc = fmaxf(mloc, __shfl_xor(mloc, 16, WAVE));
                 mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
-                // finite from the first step on: every step holds at least one valid token
+                // without a mask mloc is finite from the first step on (every step holds a valid token);
+                // a bias of -inf may leave a head without any token yet: m then stays -inf
                 if (__builtin_amdgcn_ballot_w64(mloc > m) != 0) { // some head's maximum grew: rescale
                     const float mNew = fmaxf(m, mloc);
-                    const float corr = Exp2(m - mNew);
+                    const float corr = mNew == -INFINITY ? 1.0f : Exp2(m - mNew);
                     m = mNew;
                     accL *= corr;
     #pragma unroll
@@ -472,9 +505,10 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                         acc[i] *= corr;
                     }
                 }
+                const float mRef = m == -INFINITY ? 0.0f : m; // (-inf) - (-inf) would be NaN
     #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    x[e] = Exp2(x[e] - m);
+                    x[e] = Exp2(x[e] - mRef);
                 }
                 u32x4 pop; // P^T as B operand: k = {sub 0: r 0..3, sub 1: r 0..3}
                 pop[0] = Pack2<BF16>(x[0], x[1]);
@@ -639,7 +673,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
 
         // ---- finish the row (or this wave's share of it)
         const float l = accL[0];
-        const float inv = 1.0f / l;
+        const float inv = l > 0.0f ? 1.0f / l : 0.0f; // l == 0: a -inf mask took every token out
         const float bias = KV8 ? INT8_BIAS : 0.0f; // see Int8x4ToHalf
         if (n < nh) {
             const int h = h0 + n;

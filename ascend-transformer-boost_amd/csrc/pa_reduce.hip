@@ -28,8 +28,10 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaReduceKernel(const PaArgs a)
         mx = fmaxf(mx, lse[static_cast<int64_t>(p) * a.H]);
     }
     float total = 0.0f;
+    // (a chunk a -inf mask emptied has lse == -inf and weighs nothing, even when every chunk is like that)
+    auto weightOf = [mx](float v) { return v == -INFINITY ? 0.0f : exp2f(v - mx); };
     for (int p = 0; p < np; ++p) {
-        total += exp2f(lse[static_cast<int64_t>(p) * a.H] - mx);
+        total += weightOf(lse[static_cast<int64_t>(p) * a.H]);
     }
     const float inv = total > 0.0f ? 1.0f / total : 0.0f;
     const int g = h / a.groupSize;
@@ -38,7 +40,7 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaReduceKernel(const PaArgs a)
     for (int d = threadIdx.x; d < a.Dv; d += REDUCE_THREADS) {
         float acc = 0.0f;
         for (int p = 0; p < np; ++p) {
-            const float w = exp2f(lse[static_cast<int64_t>(p) * a.H] - mx);
+            const float w = weightOf(lse[static_cast<int64_t>(p) * a.H]);
             const int64_t ph = (static_cast<int64_t>(s.firstPartial) + p) * a.H + h;
             acc += w * a.partO[ph * a.Dv + d];
         }
@@ -119,7 +121,8 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaA
         __syncthreads();
         float w = 0.0f;
         if (tid < kn) {
-            w = exp2f(a.partLse[rowOf(k0 + tid)] - mx);
+            const float lse = a.partLse[rowOf(k0 + tid)];
+            w = lse == -INFINITY ? 0.0f : exp2f(lse - mx); // a range a -inf mask emptied weighs nothing
             weight[tid] = w;
         }
         total += w;
@@ -137,7 +140,8 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaA
             }
         }
     }
-    const float inv = 1.0f / blockSum(total);
+    const float sum = blockSum(total);
+    const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
 #pragma unroll
     for (int c = 0; c < 5; ++c) {
         const int d = tid + c * REDUCE_THREADS;

@@ -43,7 +43,9 @@ __global__ __launch_bounds__(PA_SCALAR_WAVES * WAVE) void PaScalarKernel(const P
     const int h0 = g * a.groupSize + ht * HT;
     const int nh = min(HT, a.groupSize - ht * HT);
     constexpr float LOG2E = 1.4426950408889634f;
-    const float scale2 = a.qkScale * LOG2E;
+    const float scale2 = a.qkScale * LOG2E * (a.logN ? a.logN[it.seq] : 1.0f);
+    // additive score bias of this sequence and head tile (base-2 units once multiplied by LOG2E)
+    const int64_t maskRow = a.mask ? static_cast<int64_t>(it.seq) * a.maskBatchStride : 0;
 
     float q[HT][EPL];
 #pragma unroll
@@ -129,9 +131,13 @@ __global__ __launch_bounds__(PA_SCALAR_WAVES * WAVE) void PaScalarKernel(const P
                     s += q[hh][e] * k[e];
                 }
                 s = WaveSum(s) * scale2;
+                if (a.mask) {
+                    s += Load16(a.mask, maskRow + static_cast<int64_t>(h0 + hh) * a.maskHeadStride + t, bf16) * LOG2E;
+                }
                 const float mNew = fmaxf(m[hh], s);
-                const float corr = exp2f(m[hh] - mNew);
-                const float p = exp2f(s - mNew);
+                // (a bias of -inf takes the token out; nothing to rescale while the row is still empty)
+                const float corr = m[hh] == -INFINITY ? 0.0f : exp2f(m[hh] - mNew);
+                const float p = s == -INFINITY ? 0.0f : exp2f(s - mNew);
                 m[hh] = mNew;
                 l[hh] = l[hh] * corr + p;
 #pragma unroll

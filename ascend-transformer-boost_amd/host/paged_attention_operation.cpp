@@ -12,11 +12,12 @@
 // reference runner does (src/ops/ops_infer/paged_attention/param.cpp:16-62).
 //
 // Implemented feature set: fp16/bf16 caches, int8 caches with fp32 per-channel
-// descale (+ int32 offset), and the MLA combined cache (mlaVHeadSize > 0).
-// Masks, dynamic batch status, LogN scale, speculative (multi-token) queries,
-// head compression, BNSD layout, int8 queries and int64-packed descales are
-// legal in the reference but not implemented here; such params are rejected
-// at creation with ERROR_INVALID_PARAM.
+// descale (+ int32 offset), the MLA combined cache (mlaVHeadSize > 0), additive
+// NORM and ALIBI masks, the dynamic-batch status input and per-sequence LogN
+// scaling. Speculative (multi-token) queries with their masks, head
+// compression, BNSD layout, int8 queries and int64-packed descales are legal
+// in the reference but not implemented here; such params are rejected at
+// creation with ERROR_INVALID_PARAM.
 #include <cmath>
 #include <new>
 #include "atb/infer_op_params.h"
@@ -137,16 +138,13 @@ bool FeatureParamCheck(const Param &p)
 bool ImplementedCheck(const Param &p)
 {
     const char *what = nullptr;
-    if (p.maskType != Param::UNDEFINED) {
-        what = "attention masks";
-    } else if (p.batchRunStatusEnable) {
-        what = "batchRunStatus";
+    if (p.maskType != Param::UNDEFINED && p.maskType != Param::MASK_TYPE_NORM &&
+        p.maskType != Param::MASK_TYPE_ALIBI) {
+        what = "SPEC and MASK_FREE masks";
     } else if (p.compressType != Param::COMPRESS_TYPE_UNDEFINED) {
         what = "head compression";
     } else if (p.calcType != Param::CALC_TYPE_UNDEFINED) {
         what = "speculative (multi-token) queries";
-    } else if (p.scaleType != Param::SCALE_TYPE_TOR) {
-        what = "LogN scaling";
     } else if (p.inputLayout != infer::TYPE_BSND) {
         what = "BNSD layout";
     } else if (p.quantType == Param::TYPE_QUANT_QKV_OFFLINE || p.quantType == Param::TYPE_QUANT_QKV_ONLINE) {
@@ -167,10 +165,23 @@ OpIr MakeIr(const Param &p)
     const aclFormat nd = ACL_FORMAT_ND;
     for (aclDataType q : {ACL_FLOAT16, ACL_BF16}) {
         IrCombo c;
+        const bool dequant = p.quantType == Param::TYPE_DEQUANT_FUSION;
         if (p.mlaVHeadSize > 0) {
             c.inDtypes = {q, q, ACL_INT32, ACL_INT32};
-        } else if (p.quantType == Param::TYPE_DEQUANT_FUSION) {
-            c.inDtypes = {q, ACL_INT8, ACL_INT8, ACL_INT32, ACL_INT32, ACL_FLOAT};
+        } else if (dequant) {
+            c.inDtypes = {q, ACL_INT8, ACL_INT8, ACL_INT32, ACL_INT32};
+        } else {
+            c.inDtypes = {q, q, q, ACL_INT32, ACL_INT32};
+        }
+        // Optional inputs, in the reference's order (:408-444).
+        if (p.maskType != Param::UNDEFINED) {
+            c.inDtypes.push_back(q);
+        }
+        if (p.batchRunStatusEnable) {
+            c.inDtypes.push_back(ACL_INT32);
+        }
+        if (dequant) {
+            c.inDtypes.push_back(ACL_FLOAT);
             if (p.hasQuantOffset) {
                 c.inDtypes.push_back(ACL_INT32);
             }
@@ -178,8 +189,9 @@ OpIr MakeIr(const Param &p)
             if (p.hasQuantOffset) {
                 c.inDtypes.push_back(ACL_INT32);
             }
-        } else {
-            c.inDtypes = {q, q, q, ACL_INT32, ACL_INT32};
+        }
+        if (p.scaleType == Param::SCALE_TYPE_LOGN) {
+            c.inDtypes.push_back(ACL_FLOAT);
         }
         c.inFormats.assign(c.inDtypes.size(), nd);
         c.outDtypes = {q};
@@ -198,6 +210,27 @@ public:
         ir_ = &irTable_;
         tablesIdx_ = mla_ ? 2 : 3;
         lensIdx_ = mla_ ? 3 : 4;
+        size_t next = lensIdx_ + 1;
+        if (param.maskType != Param::UNDEFINED) {
+            maskIdx_ = next++;
+        }
+        if (param.batchRunStatusEnable) {
+            statusIdx_ = next++;
+        }
+        if (dequant_) {
+            kScaleIdx_ = next++;
+            if (param.hasQuantOffset) {
+                kOffsetIdx_ = next++;
+            }
+            vScaleIdx_ = next++;
+            if (param.hasQuantOffset) {
+                vOffsetIdx_ = next++;
+            }
+        }
+        if (param.scaleType == Param::SCALE_TYPE_LOGN) {
+            logNIdx_ = next++;
+        }
+        inputNum_ = static_cast<uint32_t>(next);
     }
 
     ~PagedAttentionOperation() override
@@ -207,17 +240,7 @@ public:
         }
     }
 
-    uint32_t GetInputNum() const override
-    {
-        uint32_t n = 5;
-        if (dequant_) {
-            n += param_.hasQuantOffset ? 4 : 2;
-        }
-        if (mla_) {
-            n -= 1;
-        }
-        return n;
-    }
+    uint32_t GetInputNum() const override { return inputNum_; }
     uint32_t GetOutputNum() const override { return 1; }
 
 protected:
@@ -241,6 +264,14 @@ protected:
             in.at(lensIdx_).shape.dimNum != 1) {
             ATB_LOG(ERROR) << "expected dims: query 3, keyCache 4, blockTables 2, contextLens 1";
             return ERROR_INVALID_TENSOR_DIM_NUM;
+        }
+        if (param_.batchRunStatusEnable) {
+            // reference :679-688: with a dynamic batch the query may hold fewer rows than the tables
+            const int64_t numTokens = in.at(0).shape.dims[0];
+            if (numTokens > in.at(tablesIdx_).shape.dims[0] || numTokens > in.at(lensIdx_).shape.dims[0]) {
+                ATB_LOG(ERROR) << "numTokens in q should be no greater than blockTables and contextLens";
+                return ERROR_INVALID_TENSOR_DIM;
+            }
         }
         const Dims &kc = in.at(1).shape;
         if (!mla_) {
@@ -277,6 +308,26 @@ protected:
         if (in.at(0).shape.dims[1] != out.dims[1]) {
             ATB_LOG(ERROR) << "query and output must have the same head count";
             return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (param_.batchRunStatusEnable && in.at(0).shape.dims[0] != out.dims[0]) {
+            ATB_LOG(ERROR) << "numTokens of the output should be the same as q";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (logNIdx_ != NONE) {
+            // reference :900-924 (LogNDimCheck)
+            const Dims &logN = in.at(logNIdx_).shape;
+            if (logN.dimNum != 1) {
+                ATB_LOG(ERROR) << "logN should have 1 dim";
+                return ERROR_INVALID_TENSOR_DIM;
+            }
+            if (in.at(lensIdx_).shape.dims[0] != logN.dims[0]) {
+                ATB_LOG(ERROR) << "contextLens and logN have different batch sizes";
+                return ERROR_INVALID_TENSOR_DIM;
+            }
+            if (statusIdx_ != NONE && in.at(statusIdx_).shape.dims[0] != logN.dims[0]) {
+                ATB_LOG(ERROR) << "batchRunStatus and logN have different batch sizes";
+                return ERROR_INVALID_TENSOR_DIM;
+            }
         }
         return NO_ERROR;
     }
@@ -332,19 +383,38 @@ protected:
             return ERROR_INVALID_PARAM;
         }
         if (dequant_) {
-            const size_t kScaleIdx = 5;
-            const size_t vScaleIdx = param_.hasQuantOffset ? 7 : 6;
             const int64_t kLen = kvHeads * d;
             const int64_t vLen = kvHeads * dv;
-            if (pack.inTensors.at(kScaleIdx).desc.shape.dims[0] != kLen ||
-                pack.inTensors.at(vScaleIdx).desc.shape.dims[0] != vLen) {
+            if (pack.inTensors.at(kScaleIdx_).desc.shape.dims[0] != kLen ||
+                pack.inTensors.at(vScaleIdx_).desc.shape.dims[0] != vLen) {
                 ATB_LOG(ERROR) << "descale vectors must have kvHeadNum * headSize elements";
                 return ERROR_INVALID_PARAM;
             }
-            if (param_.hasQuantOffset && (pack.inTensors.at(6).desc.shape.dims[0] != kLen ||
-                                          pack.inTensors.at(8).desc.shape.dims[0] != vLen)) {
+            if (param_.hasQuantOffset && (pack.inTensors.at(kOffsetIdx_).desc.shape.dims[0] != kLen ||
+                                          pack.inTensors.at(vOffsetIdx_).desc.shape.dims[0] != vLen)) {
                 ATB_LOG(ERROR) << "offset vectors must have kvHeadNum * headSize elements";
                 return ERROR_INVALID_PARAM;
+            }
+        }
+        if (statusIdx_ != NONE && !pack.inTensors.at(statusIdx_).hostData) {
+            // reference src/ops/ops_infer/paged_attention/param.cpp:39-49: the status vector is read on the
+            // host; its values do not reach the kernel, which skips a sequence by its zero context length
+            ATB_LOG(ERROR) << "batchRunStatus.hostData is null";
+            return ERROR_INVALID_PARAM;
+        }
+        if (logNIdx_ != NONE && pack.inTensors.at(logNIdx_).desc.shape.dims[0] < q.desc.shape.dims[0]) {
+            // reference kernel library paged_attention_operation.cpp:199-203
+            ATB_LOG(ERROR) << "logN has fewer elements than the query has rows";
+            return ERROR_INVALID_PARAM;
+        }
+        int64_t maskBatchStride = 0;
+        int64_t maskHeadStride = 0;
+        int64_t maskLen = 0;
+        if (maskIdx_ != NONE) {
+            Status st = MaskLayout(pack.inTensors.at(maskIdx_).desc.shape, lens, maskBatchStride, maskHeadStride,
+                                   maskLen);
+            if (st != NO_ERROR) {
+                return st;
             }
         }
 
@@ -364,6 +434,11 @@ protected:
         shape.kernel = ATBMI_PA_KERNEL_AUTO;
         shape.qkScale = param_.qkScale;
         shape.qScale = param_.qScale;
+        shape.hasMask = maskIdx_ != NONE ? 1 : 0;
+        shape.maskBatchStride = maskBatchStride;
+        shape.maskHeadStride = maskHeadStride;
+        shape.maskLen = static_cast<int32_t>(maskLen);
+        shape.hasLogN = logNIdx_ != NONE ? 1 : 0;
         if (!plan_ || !SameShape(shape, planShape_)) {
             if (plan_) {
                 atbmi_pa_plan_destroy(plan_);
@@ -396,15 +471,18 @@ protected:
         t.valueCache = mla_ ? nullptr : pack.inTensors.at(2).deviceData;
         t.blockTables = static_cast<const int32_t *>(pack.inTensors.at(tablesIdx_).deviceData);
         if (dequant_) {
-            size_t i = 5;
-            t.kScale = static_cast<const float *>(pack.inTensors.at(i++).deviceData);
+            t.kScale = static_cast<const float *>(pack.inTensors.at(kScaleIdx_).deviceData);
+            t.vScale = static_cast<const float *>(pack.inTensors.at(vScaleIdx_).deviceData);
             if (param_.hasQuantOffset) {
-                t.kOffset = static_cast<const int32_t *>(pack.inTensors.at(i++).deviceData);
+                t.kOffset = static_cast<const int32_t *>(pack.inTensors.at(kOffsetIdx_).deviceData);
+                t.vOffset = static_cast<const int32_t *>(pack.inTensors.at(vOffsetIdx_).deviceData);
             }
-            t.vScale = static_cast<const float *>(pack.inTensors.at(i++).deviceData);
-            if (param_.hasQuantOffset) {
-                t.vOffset = static_cast<const int32_t *>(pack.inTensors.at(i++).deviceData);
-            }
+        }
+        if (maskIdx_ != NONE) {
+            t.mask = pack.inTensors.at(maskIdx_).deviceData;
+        }
+        if (logNIdx_ != NONE) {
+            t.logN = static_cast<const float *>(pack.inTensors.at(logNIdx_).deviceData);
         }
         t.out = pack.outTensors.at(0).deviceData;
         int rc = atbmi_pa_decode(plan_, &t, workspace, workspaceSize, stream);
@@ -421,7 +499,59 @@ private:
                a.numKvHeads == b.numKvHeads && a.headDimK == b.headDimK && a.headDimV == b.headDimV &&
                a.blockSize == b.blockSize && a.numBlocks == b.numBlocks && a.maxBlocksPerSeq == b.maxBlocksPerSeq &&
                a.numQueryRows == b.numQueryRows && a.mlaCombined == b.mlaCombined && a.hasOffset == b.hasOffset &&
-               a.qkScale == b.qkScale && a.qScale == b.qScale;
+               a.qkScale == b.qkScale && a.qScale == b.qScale && a.hasMask == b.hasMask &&
+               a.maskBatchStride == b.maskBatchStride && a.maskHeadStride == b.maskHeadStride &&
+               a.maskLen == b.maskLen && a.hasLogN == b.hasLogN;
+    }
+
+    // Element strides of the additive mask, as the reference derives them from
+    // its shape (src/kernels/mixkernels/pagedattention/tiling/paged_attention_tiling.cpp:36-74),
+    // with the shapes its kernel library accepts for one query token per sequence
+    // (src/kernels/mixkernels/pagedattention/paged_attention_operation.cpp:728-763):
+    //   NORM  (1, maxS): one row for every sequence and head; (batch, 1, maxS): one row per sequence;
+    //   ALIBI (heads, 1, maxS): one row per head; (batch, 1 | heads, 1, maxS): per sequence (and head).
+    // maxS has to cover the longest context. The reference's shape check also lets
+    // through shapes with more than one query row, which its stride rules then
+    // ignore, and a 4-dim NORM mask, for which it derives no strides at all; those
+    // are refused here rather than read with strides that do not fit them.
+    Status MaskLayout(const Dims &m, const Tensor &lens, int64_t &batchStride, int64_t &headStride,
+                      int64_t &maskLen) const
+    {
+        const int64_t batch = lens.desc.shape.dims[0];
+        const int64_t heads = param_.headNum;
+        const bool alibi = param_.maskType == Param::MASK_TYPE_ALIBI;
+        bool ok = false;
+        if (!alibi && m.dimNum == 2) {
+            ok = m.dims[0] == 1;
+            batchStride = 0;
+            headStride = 0;
+        } else if (!alibi && m.dimNum == 3) {
+            ok = m.dims[0] == batch && m.dims[1] == 1;
+            batchStride = m.dims[2];
+            headStride = 0;
+        } else if (alibi && m.dimNum == 3) {
+            ok = m.dims[0] == heads && m.dims[1] == 1;
+            batchStride = 0;
+            headStride = m.dims[2];
+        } else if (alibi && m.dimNum == 4) {
+            ok = m.dims[0] == batch && (m.dims[1] == 1 || m.dims[1] == heads) && m.dims[2] == 1;
+            batchStride = m.dims[1] * m.dims[3];
+            headStride = m.dims[1] == 1 ? 0 : m.dims[3];
+        }
+        if (!ok) {
+            ATB_LOG(ERROR) << "mask shape is not one of NORM (1,maxS) / (batch,1,maxS), "
+                              "ALIBI (heads,1,maxS) / (batch,1|heads,1,maxS)";
+            return ERROR_INVALID_PARAM;
+        }
+        maskLen = m.dims[m.dimNum - 1];
+        const int32_t *ctx = static_cast<const int32_t *>(lens.hostData);
+        for (int64_t i = 0; i < batch; ++i) {
+            if (ctx[i] > maskLen) {
+                ATB_LOG(ERROR) << "mask covers " << maskLen << " positions but contextLens[" << i << "] is " << ctx[i];
+                return ERROR_INVALID_PARAM;
+            }
+        }
+        return NO_ERROR;
     }
 
     // Reference :585-632 (KVCacheDimCheck910B) with :561-572 (IsInMLAIncompatible).
@@ -474,8 +604,17 @@ private:
     bool mla_;
     bool dequant_;
     OpIr irTable_;
+    static constexpr size_t NONE = ~static_cast<size_t>(0);
     size_t tablesIdx_ = 3;
     size_t lensIdx_ = 4;
+    size_t maskIdx_ = NONE;
+    size_t statusIdx_ = NONE;
+    size_t kScaleIdx_ = NONE;
+    size_t kOffsetIdx_ = NONE;
+    size_t vScaleIdx_ = NONE;
+    size_t vOffsetIdx_ = NONE;
+    size_t logNIdx_ = NONE;
+    uint32_t inputNum_ = 5;
     AtbmiPaPlan *plan_ = nullptr;
     AtbmiPaShape planShape_{};
 };

@@ -19,6 +19,12 @@ CONFIGS = {
                kv="bf16", dist="uniform", std=0.5, pool=None),
     "c2_fp16": dict(batch=64, heads=32, kv_heads=8, d=128, dv=128, block=128, ctx=(1024, 4096), dtype="float16",
                     kv="float16", dist="uniform", std=0.5, pool=None),
+    # C2 with the additive masks of the reference's decode tests: ALiBi rows per (sequence, head),
+    # and a per-sequence NORM row that hides the first i positions of sequence i
+    "c2_alibi": dict(batch=64, heads=32, kv_heads=8, d=128, dv=128, block=128, ctx=(1024, 4096), dtype="bf16",
+                     kv="bf16", dist="uniform", std=0.5, pool=None, mask="alibi"),
+    "c2_norm": dict(batch=64, heads=32, kv_heads=8, d=128, dv=128, block=128, ctx=(1024, 4096), dtype="bf16",
+                    kv="bf16", dist="uniform", std=0.5, pool=None, mask="norm"),
     "c3": dict(batch=128, heads=64, kv_heads=8, d=128, dv=128, block=128, ctx=(2048, 8192), dtype="float16",
                kv="int8", dist="uniform", std=1.0, pool=None),
     "c4": dict(batch=16, heads=32, kv_heads=8, d=128, dv=128, block=128, ctx=(256, 32768), dtype="float16",
@@ -26,7 +32,7 @@ CONFIGS = {
     "c5": dict(batch=64, heads=128, kv_heads=1, d=576, dv=512, block=128, ctx=(2048, 4096), dtype="bf16",
                kv="bf16", dist="uniform", std=0.3, pool=None, mla=True),
 }
-SEEDS = {"c1": 1001, "c2": 1002, "c2_fp16": 1002, "c3": 1003, "c4": 1004, "c5": 1005}
+SEEDS = {"c1": 1001, "c2": 1002, "c2_fp16": 1002, "c2_alibi": 1002, "c2_norm": 1002, "c3": 1003, "c4": 1004, "c5": 1005}
 
 
 def config(name, **overrides):
@@ -79,11 +85,41 @@ def torch_dtype(name):
     return {"float16": torch.float16, "bf16": torch.bfloat16, "int8": torch.int8}[name]
 
 
+def alibi_slopes(heads):
+    """2^(-8 k / n), k = 1..n, n the largest power of two <= heads, then 2^(-4 k / n) for odd k
+    (reference tests/apitest/kernelstest/mix/test_paged_attention_common.py:74-83)."""
+    n = 1 << (int(heads).bit_length() - 1)
+    return [2.0 ** (-8.0 * k / n) for k in range(1, n + 1)] + \
+           [2.0 ** (-4.0 * k / n) for k in range(1, 1 + 2 * (heads - n), 2)]
+
+
+def make_mask(cfg, ctx, device):
+    """The additive mask of a masked workload, in the query dtype, rows padded to a
+    multiple of the block size. "alibi": [batch, heads, 1, maxS], slope_h * (j - ctx_i + 1)
+    on the valid positions (reference :489-499); "norm": [batch, 1, maxS], -10000 on the
+    first i positions of sequence i (reference :501-505)."""
+    import torch
+    bs = cfg["block"]
+    max_s = (int(max(ctx)) + bs - 1) // bs * bs
+    lens = torch.as_tensor(np.asarray(ctx), device=device, dtype=torch.float32)
+    pos = torch.arange(max_s, device=device, dtype=torch.float32)
+    if cfg["mask"] == "alibi":
+        slopes = torch.tensor(alibi_slopes(cfg["heads"]), device=device, dtype=torch.float32)
+        dist = pos[None, :] - lens[:, None] + 1.0                       # [batch, maxS]
+        m = slopes[None, :, None] * torch.where(dist <= 0, dist, torch.zeros_like(dist))[:, None, :]
+        return m[:, :, None, :].to(torch_dtype(cfg["dtype"])).contiguous()
+    row = torch.arange(len(ctx), device=device, dtype=torch.float32)
+    m = torch.where(pos[None, :] < row[:, None], torch.full((1, 1), -10000.0, device=device),
+                    torch.zeros((1, 1), device=device))
+    return m[:, None, :].to(torch_dtype(cfg["dtype"])).contiguous()
+
+
 def make_step(cfg, device, seed=None):
     """Tensors of one decode step on `device` (torch). Returns a dict:
     q, k_new, v_new (query dtype), key_cache, value_cache (kv dtype; value_cache
     is None for MLA), k_scale/v_scale (fp32, int8 caches only), block_tables,
-    slot_mapping (int32, device), context_lens (int32, CPU) and cfg/layout."""
+    slot_mapping (int32, device), context_lens (int32, CPU), mask (query dtype, or
+    None) and cfg/layout."""
     import torch
     lay = layout(cfg, seed)
     gen = torch.Generator(device=device)
@@ -128,12 +164,14 @@ def make_step(cfg, device, seed=None):
     out["block_tables"] = torch.from_numpy(lay["tables"]).to(device)
     out["slot_mapping"] = torch.from_numpy(lay["slots"]).to(device)
     out["context_lens"] = torch.from_numpy(lay["ctx"].copy())
+    out["mask"] = make_mask(cfg, lay["ctx"], device) if cfg.get("mask") else None
     return out
 
 
 def algorithmic_bytes(cfg, ctx):
     """HBM bytes a decode-attention call must move: valid K/V rows + q + out +
-    block-table entries + context lengths (+ scale vectors for an int8 cache)."""
+    block-table entries + context lengths (+ scale vectors for an int8 cache, + the
+    mask rows over the valid positions)."""
     kv = 1 if cfg["kv"] == "int8" else 2
     g, d, dv, h, bs = cfg["kv_heads"], cfg["d"], cfg["dv"], cfg["heads"], cfg["block"]
     ctx = np.asarray(ctx, dtype=np.int64)
@@ -143,4 +181,6 @@ def algorithmic_bytes(cfg, ctx):
     total += int(((ctx + bs - 1) // bs).sum()) * 4 + len(ctx) * 4
     if cfg["kv"] == "int8":
         total += g * (d + dv) * 4
+    if cfg.get("mask"):
+        total += int(ctx.sum()) * (h if cfg["mask"] == "alibi" else 1) * 2
     return total

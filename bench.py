@@ -33,15 +33,20 @@ DESCRIPTIONS = {
     "c1": "C1 small fp16 decode: batch 4, 8 q heads, 8 kv heads, d128, block 128, ctx U[64,512]",
     "c2": "C2 Llama-3-8B-shaped bf16 decode: batch 64, 32 q heads, 8 kv heads, d128, block 128, ctx U[1024,4096]",
     "c2_fp16": "C2 shape in fp16: batch 64, 32 q heads, 8 kv heads, d128, block 128, ctx U[1024,4096]",
+    "c2_alibi": "C2 with an ALiBi mask [batch, heads, 1, maxS]: batch 64, 32 q heads, 8 kv heads, d128, block 128, "
+                "ctx U[1024,4096], bf16",
+    "c2_norm": "C2 with a NORM mask [batch, 1, maxS]: batch 64, 32 q heads, 8 kv heads, d128, block 128, "
+               "ctx U[1024,4096], bf16",
     "c3": "C3 int8-KV 70B-shaped decode: batch 128, 64 q heads, 8 kv heads, d128, block 128, ctx U[2048,8192], fp16 q",
     "c4": "C4 skewed long-context fp16 decode: batch 16, 32 q heads, 8 kv heads, d128, ctx lognormal(median 8k) in [256,32768]",
     "c5": "C5 MLA bf16 decode: batch 64, 128 q heads, 1 latent kv head, d576/dv512, block 128, ctx U[2048,4096]",
 }
 
 
-def cpu_baseline(pkg, step, cfg, scale, budget_s=15.0):
-    """Times the numpy oracle on the first sequences of the batch until about
-    `budget_s` seconds of CPU work are spent; returns tokens/s on that sample."""
+def cpu_baseline(pkg, step, cfg, scale, budget_s=10.0):
+    """Times the numpy oracle on the sequences of the batch, taken in order and
+    again from the first once all are done, until about `budget_s` seconds of CPU
+    work are spent; returns tokens/s (one token per sequence) on that sample."""
     import numpy as np
     oracle = importlib.import_module("oracle.atb_oracle")
     try:
@@ -58,9 +63,11 @@ def cpu_baseline(pkg, step, cfg, scale, budget_s=15.0):
     vs = step.get("v_scale")
     ks = ks.cpu().numpy() if ks is not None else None
     vs = vs.cpu().numpy() if vs is not None else None
+    mask = step["mask"].float().cpu().numpy() if step.get("mask") is not None else None
     done, spent, tokens = 0, 0.0, 0
     import torch
-    for b in range(len(ctx)):
+    b = 0
+    while spent < budget_s:  # cycles over the batch until the budget is spent
         n = int(ctx[b])
         nblk = (n + cfg["block"] - 1) // cfg["block"]
         ids = torch.from_numpy(tables[b, :nblk].astype("int64")).to(kc.device)
@@ -74,19 +81,19 @@ def cpu_baseline(pkg, step, cfg, scale, budget_s=15.0):
         local = np.arange(nblk, dtype=np.int32)[None, :]
         t0 = time.perf_counter()
         oracle.paged_attention(q, kb, vb, local, np.array([n]), scale, ks, None, vs, None,
-                               mla_v_head_size=cfg["dv"] if cfg.get("mla") else 0)
+                               mla_v_head_size=cfg["dv"] if cfg.get("mla") else 0,
+                               mask=None if mask is None else mask[b:b + 1], mask_per_head=False)
         spent += time.perf_counter() - t0
         done += 1
         tokens += n
-        if spent >= budget_s:
-            break
+        b = (b + 1) % len(ctx)
     return {
         "value": done / spent if spent > 0 else 0.0,
         "unit": "tokens/s",
         "cores": threads,
         "kind": "port",
-        "sample": "numpy oracle on the first %d of %d sequences (%d context tokens), attention only, %.1f s" % (
-            done, len(ctx), tokens, spent),
+        "sample": "numpy oracle on %d sequences drawn in order from the batch of %d (%d context tokens), "
+                  "attention only, %.1f s" % (done, len(ctx), tokens, spent),
     }
 
 
@@ -119,8 +126,10 @@ def main():
     int8 = cfg["kv"] == "int8"
     mla = bool(cfg.get("mla"))
 
+    mask_type = {None: 0, "norm": 1, "alibi": 2}[cfg.get("mask")]
     pa_param = b.PagedAttentionParam(headNum=cfg["heads"], kvHeadNum=cfg["kv_heads"], qkScale=scale,
-                                     quantType=1 if int8 else 0, mlaVHeadSize=cfg["dv"] if mla else 0)
+                                     quantType=1 if int8 else 0, mlaVHeadSize=cfg["dv"] if mla else 0,
+                                     maskType=mask_type)
     pa = b.OperationRunner("PagedAttentionOperation", pa_param, ctx)
     rac = None
     k = b.kernels()
@@ -136,6 +145,8 @@ def main():
         else:
             pa_in = [step["q"], step["key_cache"], step["value_cache"], step["block_tables"], lens_dev]
             host_idx = 4
+            if mask_type:
+                pa_in.append(step["mask"])
             if int8:
                 pa_in += [step["k_scale"], step["v_scale"]]
             else:

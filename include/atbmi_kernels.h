@@ -102,9 +102,13 @@ typedef struct AtbmiPaShape {
     int32_t mlaCombined;     /* 1: no value cache; V = first Dv channels of the key cache row */
     int32_t hasOffset;       /* int8 KV: kOffset / vOffset are given */
     int32_t kernel;          /* AtbmiPaKernel */
-    int32_t reserved;
+    int32_t hasMask;         /* 1: an additive score bias (AtbmiPaTensors.mask) is given */
     float qkScale;           /* multiplies q.k before the softmax */
     float qScale;            /* pre-multiplies q (rounded to qDtype) unless 0 or 1 */
+    int64_t maskBatchStride; /* elements between the mask rows of consecutive sequences (0: shared) */
+    int64_t maskHeadStride;  /* elements between the mask rows of consecutive query heads (0: shared) */
+    int32_t maskLen;         /* tokens per mask row, >= every context length */
+    int32_t hasLogN;         /* 1: a per-sequence factor on qkScale (AtbmiPaTensors.logN) is given */
 } AtbmiPaShape;
 
 /* Device tensors of one decode call.
@@ -114,6 +118,13 @@ typedef struct AtbmiPaShape {
  *   blockTables [batch, maxBlocksPerSeq]            int32
  *   kScale/vScale [G*D] / [G*Dv] fp32, kOffset/vOffset same length int32 (int8 KV only)
  *   out         [numQueryRows, H, Dv]               qDtype
+ *   mask        qDtype, hasMask only: the score of sequence b (its index in hostContextLens), head h and
+ *               token t gets mask[b * maskBatchStride + h * maskHeadStride + t] added after the qkScale
+ *               multiplication. Covers the reference's MASK_TYPE_NORM ([batch, 1, maxLen]: batch stride
+ *               maxLen, head stride 0; [1, maxLen]: both 0) and MASK_TYPE_ALIBI ([heads, 1, maxLen]: batch
+ *               stride 0; [batch, heads | 1, 1, maxLen]) layouts of a decode step
+ *               (tiling/paged_attention_tiling.cpp:36-80).
+ *   logN        fp32 [batch], hasLogN only: sequence b uses qkScale * logN[b] (SCALE_TYPE_LOGN).
  */
 typedef struct AtbmiPaTensors {
     const void *query;
@@ -125,6 +136,8 @@ typedef struct AtbmiPaTensors {
     const float *vScale;
     const int32_t *vOffset;
     void *out;
+    const void *mask;
+    const float *logN;
 } AtbmiPaTensors;
 
 typedef struct AtbmiPaPlan AtbmiPaPlan; /* opaque; owned by the caller, not thread-safe */
@@ -145,7 +158,8 @@ uint64_t atbmi_pa_plan_workspace_size(const AtbmiPaPlan *plan);
 int64_t atbmi_pa_plan_num_chunks(const AtbmiPaPlan *plan);
 
 /* Algorithmic HBM bytes of one decode call with the current plan: valid K/V
- * rows + q + out + block-table entries + context lengths + scale vectors. */
+ * rows + q + out + block-table entries + context lengths + scale vectors +
+ * every distinct mask row over the tokens it biases + logN. */
 uint64_t atbmi_pa_plan_algorithmic_bytes(const AtbmiPaPlan *plan);
 
 /* Uploads the plan into the workspace and launches the attention kernel (and

@@ -17,8 +17,12 @@ the invariants of the mathematics (no function is left "parity unpinned"):
                       tests/apitest/kernelstest/elewise/test_quant_per_channel.py:22-40
   paged_attention     tests/apitest/kernelstest/mix/test_paged_attention_common.py:85-118 (grouped
                       matmul, int8 dequant (q + offset) * scale per channel g*D + d), :132-139
-                      (softmax), :229-276 (the fp32 "out_high" branch), :278-365 (paged gather,
-                      zero-length sequences are skipped and take no query row);
+                      (softmax), :229-276 (the fp32 "out_high" branch; :252-254 the mask is added
+                      in fp32 after the scale), :278-365 (paged gather, zero-length sequences are
+                      skipped and take no query row; :311-313,347-349 logN multiplies the scale of
+                      sequence i; :353-358 a 4-dim mask is sliced [i, :, :, :ctx], a 3-dim one
+                      [i, :, :ctx], with i the index into context_lens); :74-83 (ALiBi slopes),
+                      :488-505 (the masks the reference tests feed);
                       MLA: tests/apitest/opstest/python/operations/paged_attention/
                       test_paged_attention_operation_mla.py:229-262 (V = K[..., :head_size_vo])
   merge_partials      src/kernels/mixkernels/pagedattention/op_kernel/
@@ -114,10 +118,14 @@ def gather_rows(cache, block_table, context_len):
     return cache[np.asarray(block_table)[j // block_size], j % block_size]
 
 
-def attention_one(q, keys, values, scale, k_descale=None, k_offset=None, v_descale=None, v_offset=None):
+def attention_one(q, keys, values, scale, k_descale=None, k_offset=None, v_descale=None, v_offset=None,
+                  bias=None):
     """One query token against gathered rows. q [heads, D] float32; keys
-    [ctx, kv_heads, D]; values [ctx, kv_heads, Dv] (float32 or int8).
-    Returns float32 [heads, Dv]: softmax(scale * q k^T) v per GQA group."""
+    [ctx, kv_heads, D]; values [ctx, kv_heads, Dv] (float32 or int8); bias None
+    or broadcastable to [heads, ctx], added to the scaled scores.
+    Returns float32 [heads, Dv]: softmax(scale * q k^T + bias) v per GQA group."""
+    if bias is not None:
+        bias = np.broadcast_to(np.asarray(bias, dtype=np.float32), (q.shape[0], keys.shape[0]))
     heads = q.shape[0]
     kv_heads = keys.shape[1]
     group = heads // kv_heads
@@ -132,14 +140,44 @@ def attention_one(q, keys, values, scale, k_descale=None, k_offset=None, v_desca
         v = v.astype(np.float32)
         qg = q[g * group:(g + 1) * group].astype(np.float32)
         sim = (qg @ k.T) * np.float32(scale)
+        if bias is not None:
+            sim = sim + bias[g * group:(g + 1) * group]
         p = softmax_rows(sim)
         out[g * group:(g + 1) * group] = p @ v
     return out
 
 
+def alibi_slopes(n_heads):
+    """Per-head ALiBi slopes as the reference tests build them: 2^(-8 k / n) for
+    k = 1..n with n the largest power of two <= n_heads, then 2^(-4 k / n) for
+    odd k to fill up."""
+    n = 1 << (int(n_heads).bit_length() - 1)
+    slopes = [2.0 ** (-8.0 * k / n) for k in range(1, n + 1)]
+    slopes += [2.0 ** (-4.0 * k / n) for k in range(1, 1 + 2 * (n_heads - n), 2)]
+    return np.asarray(slopes, dtype=np.float32)
+
+
+def alibi_mask(context_lens, n_heads, max_len):
+    """[batch, heads, 1, max_len] float32: slope_h * (j - ctx_i + 1) for j < ctx_i, else 0."""
+    mask = np.zeros((len(context_lens), n_heads, 1, max_len), dtype=np.float32)
+    slopes = alibi_slopes(n_heads)
+    for i, ctx in enumerate(context_lens):
+        pos = np.arange(ctx, dtype=np.float32) - np.float32(ctx) + 1
+        mask[i, :, 0, :ctx] = slopes[:, None] * pos[None, :]
+    return mask
+
+
+def norm_mask(batch, max_len, value=-10000.0):
+    """[batch, 1, max_len] float32: row i hides its first i positions."""
+    mask = np.zeros((batch, 1, max_len), dtype=np.float32)
+    for i in range(batch):
+        mask[i, :, :i] = value
+    return mask
+
+
 def paged_attention(query, key_cache, value_cache, block_tables, context_lens, scale, k_descale=None,
                     k_offset=None, v_descale=None, v_offset=None, mla_v_head_size=0, q_scale=0.0,
-                    q_dtype="float32", out_init=0.0):
+                    q_dtype="float32", out_init=0.0, mask=None, logn=None, mask_per_head=None):
     """Decode attention over paged caches.
 
     query [rows, heads, D] float32; key_cache [blocks, block, kv_heads, D];
@@ -149,6 +187,12 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, s
     the n-th non-empty sequence uses query row n and writes output row n.
     Rows never written keep `out_init`. q_scale not in {0, 1} pre-multiplies the
     query and rounds it to q_dtype, as the reference's separate multiply node does.
+    mask (float32 values of the mask tensor's dtype) is added to the scaled scores
+    of sequence i (its index in context_lens, empty ones counted): a 4-dim mask
+    [batch, heads | 1, 1, max_len] is sliced [i, :, 0, :ctx], a 3-dim mask whose
+    first dim is the batch [i, 0, :ctx] for every head, a 3-dim mask
+    [heads, 1, max_len] (mask_per_head=True, or left to its size when heads !=
+    batch), or a 2-dim [1, max_len] one, is shared by all sequences. logn [batch] multiplies the scale of sequence i.
     Returns float32 [rows, heads, Dv]."""
     query = np.asarray(query, dtype=np.float32)
     if mla_v_head_size > 0:
@@ -164,15 +208,37 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, s
             continue
         keys = gather_rows(key_cache, block_tables[i], ctx)
         values = keys[..., :dv] if mla_v_head_size > 0 else gather_rows(value_cache, block_tables[i], ctx)
-        out[row] = attention_one(query[row], keys, values, scale, k_descale, k_offset, v_descale, v_offset)
+        bias = None if mask is None else mask_rows(mask, i, ctx, query.shape[1], len(context_lens),
+                                                      mask_per_head)
+        seq_scale = np.float32(scale) if logn is None else np.float32(scale) * np.float32(logn[i])
+        out[row] = attention_one(query[row], keys, values, seq_scale, k_descale, k_offset, v_descale, v_offset,
+                                 bias)
         row += 1
     return out
 
 
-def paged_attention_loops(query, key_cache, value_cache, block_tables, context_lens, scale):
+def mask_rows(mask, i, ctx, heads, batch, per_head=None):
+    """The [heads | 1, ctx] slice of `mask` that sequence i sees (see paged_attention).
+    per_head says whether a 3-dim mask's first dim counts heads (ALIBI) or
+    sequences (NORM); None decides by its size and refuses the ambiguous case."""
+    mask = np.asarray(mask, dtype=np.float32)
+    if mask.ndim == 4:
+        return mask[i, :, 0, :ctx]
+    if mask.ndim == 3:
+        if per_head is None:
+            if heads == batch and mask.shape[0] == batch:
+                raise ValueError("3-dim mask with heads == batch: say per_head")
+            per_head = mask.shape[0] != batch
+        return mask[:, 0, :ctx] if per_head else mask[i, :, :ctx]
+    return mask[:1, :ctx]
+
+
+def paged_attention_loops(query, key_cache, value_cache, block_tables, context_lens, scale, dense_bias=None,
+                          logn=None):
     """The same computation written as plain Python loops in float64, for tiny
     inputs only: an independent check of the vectorised version (no numpy
-    matmul, no broadcasting, no shared helper)."""
+    matmul, no broadcasting, no shared helper). dense_bias[i][h][j] is added to
+    the scaled score of sequence i, head h, token j; logn[i] multiplies the scale."""
     import math
     rows, heads, d = query.shape
     _, block_size, kv_heads, _ = key_cache.shape
@@ -193,7 +259,10 @@ def paged_attention_loops(query, key_cache, value_cache, block_tables, context_l
                 s = 0.0
                 for c in range(d):
                     s += float(query[row][h][c]) * float(key_cache[blk][off][g][c])
-                scores.append(s * float(scale))
+                s = s * float(scale) * (float(logn[i]) if logn is not None else 1.0)
+                if dense_bias is not None:
+                    s += float(dense_bias[i][h][j])
+                scores.append(s)
             m = max(scores)
             w = [math.exp(s - m) for s in scores]
             z = sum(w)

@@ -21,16 +21,22 @@ def dtype_code(binding, t):
 
 
 def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=None, v_scale=None,
-                   v_off=None, mla_dv=0, q_scale=0.0, kernel=0, chunk_tokens=None, out=None, return_plan_info=False):
-    """atbmi_pa_plan_* + atbmi_pa_decode on `stream`; returns the output tensor."""
+                   v_off=None, mla_dv=0, q_scale=0.0, kernel=0, chunk_tokens=None, out=None, return_plan_info=False,
+                   mask=None, mask_per_head=False, logn=None):
+    """atbmi_pa_plan_* + atbmi_pa_decode on `stream`; returns the output tensor.
+    mask: device tensor of q's dtype shaped like one of the reference's decode
+    masks; mask_per_head says that a 3-dim mask's first dim counts heads (ALIBI)."""
     k = binding.kernels()
     rows, heads, d = q.shape
     dv = mla_dv if mla_dv else vc.shape[3]
+    mask_batch_stride, mask_head_stride = mask_strides(mask, mask_per_head)
     shape = binding.AtbmiPaShape(
         qDtype=dtype_code(binding, q), kvDtype=dtype_code(binding, kc), numHeads=heads, numKvHeads=kc.shape[2],
         headDimK=d, headDimV=dv, blockSize=kc.shape[1], numBlocks=kc.shape[0], maxBlocksPerSeq=tables.shape[1],
         numQueryRows=rows, mlaCombined=1 if mla_dv else 0, hasOffset=1 if k_off is not None else 0, kernel=kernel,
-        qkScale=scale, qScale=q_scale)
+        qkScale=scale, qScale=q_scale, hasMask=0 if mask is None else 1, maskBatchStride=mask_batch_stride,
+        maskHeadStride=mask_head_stride, maskLen=0 if mask is None else mask.shape[-1],
+        hasLogN=0 if logn is None else 1)
     old = os.environ.get("ATBMI_PA_CHUNK_TOKENS")
     if chunk_tokens is not None:
         os.environ["ATBMI_PA_CHUNK_TOKENS"] = str(chunk_tokens)
@@ -65,6 +71,8 @@ def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=
             t.vScale = v_scale.data_ptr() if v_scale is not None else None
             t.vOffset = v_off.data_ptr() if v_off is not None else None
             t.out = out.data_ptr()
+            t.mask = mask.data_ptr() if mask is not None else None
+            t.logN = logn.data_ptr() if logn is not None else None
             rc = k.atbmi_pa_decode(plan, ctypes.byref(t), ws.data_ptr(), ws_bytes, stream.cuda_stream)
             if rc != 0:
                 raise RuntimeError("pa_decode: " + binding.last_kernel_error())
@@ -76,13 +84,30 @@ def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=
     return (out, info) if return_plan_info else out
 
 
+def mask_strides(mask, per_head):
+    """(batch stride, head stride) in elements of a decode mask, by the rules of
+    the reference tiling (tiling/paged_attention_tiling.cpp:36-74)."""
+    if mask is None:
+        return 0, 0
+    assert mask.is_contiguous()
+    if mask.dim() == 2:
+        assert mask.shape[0] == 1
+        return 0, 0
+    if mask.dim() == 3:
+        assert mask.shape[1] == 1
+        return (0, mask.shape[2]) if per_head else (mask.shape[2], 0)
+    assert mask.dim() == 4 and mask.shape[2] == 1
+    return mask.shape[1] * mask.shape[3], (0 if mask.shape[1] == 1 else mask.shape[3])
+
+
 def oracle_pa(oracle, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=None, v_scale=None, v_off=None,
-              mla_dv=0, q_scale=0.0, out_init=0.0):
+              mla_dv=0, q_scale=0.0, out_init=0.0, mask=None, mask_per_head=False, logn=None):
     qd = "bf16" if q.dtype == torch.bfloat16 else "float16"
     return oracle.paged_attention(
         to_oracle(q), to_oracle(kc), to_oracle(vc), tables.cpu().numpy(), np.asarray(ctx_host), scale,
         to_oracle(k_scale), to_oracle(k_off), to_oracle(v_scale), to_oracle(v_off), mla_v_head_size=mla_dv,
-        q_scale=q_scale, q_dtype=qd, out_init=out_init)
+        q_scale=q_scale, q_dtype=qd, out_init=out_init, mask=to_oracle(mask), logn=to_oracle(logn),
+        mask_per_head=mask_per_head if (mask is not None and mask.dim() == 3) else None)
 
 
 def assert_close(got, want, tol, what=""):

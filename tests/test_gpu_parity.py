@@ -399,6 +399,174 @@ def test_mla_through_operation_api_and_split_head_sizes(binding, oracle, dev, st
     c.close()
 
 
+# ------------------------------------------------------------------ masks, logN, dynamic batch
+def _mask_tensor(oracle, rng, dev, kind, ctx, heads, max_len, dtype):
+    """A decode mask of the given layout in q's dtype, plus whether a 3-dim one is per head.
+    NORM masks hide the first i positions of sequence i with -10000 like the reference
+    tests do (test_paged_attention_common.py:501-505) and carry small random values
+    elsewhere, so that a wrong row or column shows; ALIBI masks are the reference's
+    slope * distance rows (:489-499)."""
+    batch = len(ctx)
+    if kind == "norm2":
+        m = rng.standard_normal((1, max_len)).astype(np.float32)
+        m[0, :2] = -10000.0
+    elif kind == "norm3":
+        m = oracle.norm_mask(batch, max_len) + rng.standard_normal((batch, 1, max_len)).astype(np.float32)
+        for i, n in enumerate(ctx):  # never hide a whole sequence
+            m[i, 0, max(int(n) - 1, 0)] = 0.0
+    elif kind == "alibi4":
+        m = oracle.alibi_mask(ctx, heads, max_len)
+    elif kind == "alibi4_1":
+        m = oracle.alibi_mask(ctx, heads, max_len)[:, 3:4].copy()
+    elif kind == "alibi3":
+        m = oracle.alibi_mask([max_len], heads, max_len)[0]
+    else:
+        raise ValueError(kind)
+    return torch.from_numpy(m).to(dtype).to(dev).contiguous(), kind == "alibi3"
+
+
+# layout, batch, heads, kv_heads, block, d, ctx, mask row length, dtype, logN, int8 cache
+# (reference test_paged_attention_common.py:725-1100: logN, alibi multi batch, norm mask with
+#  long / small / ragged lengths; CSV rows PagedAttentionDequantNorm / DequantAlibi)
+MASK_MATRIX = [
+    ("norm3", 4, 32, 32, 128, 128, 15, 15, torch.float16, False, False),
+    ("norm3", 6, 32, 32, 128, 128, 200, 256, torch.float16, False, False),
+    ("norm3", 3, 40, 40, 128, 128, [30000, 77, 4099], 30001, torch.bfloat16, False, False),
+    ("norm2", 5, 8, 2, 16, 128, [33, 900, 64, 1, 3000], 3000, torch.float16, False, False),
+    ("alibi4", 2, 32, 32, 128, 128, 500, 500, torch.bfloat16, False, False),
+    ("alibi4", 7, 30, 2, 128, 128, [88, 1500, 3, 128, 129, 640, 2000], 2002, torch.float16, True, False),
+    ("alibi4_1", 4, 16, 4, 64, 96, [100, 2000, 64, 777], 2048, torch.float16, False, False),
+    ("alibi3", 5, 32, 8, 128, 128, [819, 12, 4000, 256, 300], 4000, torch.float16, False, False),
+    (None, 30, 32, 32, 128, 128, 69, 0, torch.bfloat16, True, False),
+    ("norm3", 30, 32, 32, 128, 128, 69, 72, torch.bfloat16, True, False),
+    ("norm3", 8, 64, 8, 128, 128, 1200, 1200, torch.float16, False, True),
+    ("alibi4", 4, 32, 16, 64, 128, [100, 2000, 64, 777], 2000, torch.float16, False, True),
+    ("norm3", 3, 24, 1, 16, 256, [3000, 5, 12000], 12000, torch.float16, False, False),
+]
+
+
+@pytest.mark.parametrize("case", MASK_MATRIX, ids=lambda c: "%s_b%d_h%d_g%d_d%d_%s%s%s" % (
+    c[0], c[1], c[2], c[3], c[5], str(c[8]).split(".")[-1], "_logn" if c[9] else "", "_int8" if c[10] else ""))
+def test_paged_attention_masks_and_logn(binding, oracle, dev, stream, case):
+    kind, batch, heads, kv_heads, block, d, ctx, max_len, dtype, with_logn, kv_int8 = case
+    rng = _rng(200 + batch + heads)
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, batch, heads, kv_heads, block, d, d, ctx, dtype, kv_int8=kv_int8)
+    mask, per_head = (None, False) if kind is None else _mask_tensor(oracle, rng, dev, kind, ctx, heads, max_len, dtype)
+    logn = torch.from_numpy(rng.uniform(1, 2, size=batch).astype(np.float32)).to(dev) if with_logn else None
+    ks = ko = vs = vo = None
+    if kv_int8:
+        ks = torch.from_numpy(rng.uniform(0.05, 0.5, size=kv_heads * d).astype(np.float32)).to(dev)
+        vs = torch.from_numpy(rng.uniform(0.05, 0.5, size=kv_heads * d).astype(np.float32)).to(dev)
+    scale = 1.0 / math.sqrt(d)
+    want = oracle_pa(oracle, q, kc, vc, tables, ctx, scale, ks, ko, vs, vo, mask=mask, mask_per_head=per_head,
+                     logn=logn)
+    plain = oracle_pa(oracle, q, kc, vc, tables, ctx, scale, ks, ko, vs, vo)
+    assert np.abs(want - plain).max() > 0.01  # the mask / logN matters in this case
+    tol = INT8_TOL if kv_int8 else TOL[dtype]
+    for kernel in _kernels_for(binding, d, d, block):
+        got = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, ks, ko, vs, vo, kernel=kernel,
+                             mask=mask, mask_per_head=per_head, logn=logn)
+        assert_close(got, want, tol, "kernel=%d" % kernel)
+
+
+@pytest.mark.parametrize("kernel", [1, 0])
+def test_mask_rows_follow_the_sequence_index_past_empty_sequences(binding, oracle, dev, stream, kernel):
+    """Empty sequences take no query row, but mask and logN rows stay indexed by
+    the position in contextLens (reference test_paged_attention_common.py:311-358)."""
+    rng = _rng(231)
+    heads, kv_heads, d, block = 16, 4, 128, 16
+    ctx = np.array([0, 37, 1, 0, 400, 16, 0], dtype=np.int32)
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, len(ctx), heads, kv_heads, block, d, d, ctx, torch.float16)
+    mask, _ = _mask_tensor(oracle, rng, dev, "alibi4", ctx, heads, 401, torch.float16)
+    mask += torch.from_numpy(rng.standard_normal((len(ctx), 1, 1, 401)).astype(np.float32)).to(dev).half()
+    logn = torch.from_numpy(rng.uniform(1, 2, size=len(ctx)).astype(np.float32)).to(dev)
+    scale = 1.0 / math.sqrt(d)
+    out = torch.full((len(ctx), heads, d), 0.1, dtype=torch.float16, device=dev)
+    got = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, kernel=kernel, out=out, mask=mask, logn=logn)
+    want = oracle_pa(oracle, q, kc, vc, tables, ctx, scale, out_init=0.1, mask=mask, logn=logn)
+    assert_close(got, want, 1e-3, "empty+mask")
+
+
+@pytest.mark.parametrize("kernel", [1, 0])
+@pytest.mark.parametrize("chunk", [64, 1024])
+def test_minus_infinity_mask_hides_whole_ranges(binding, oracle, dev, stream, kernel, chunk):
+    """A bf16 mask of -inf over the first 300 positions: ranges of the split that
+    lie wholly inside it contribute nothing, and the result is the attention over
+    the rest."""
+    rng = _rng(232)
+    heads, kv_heads, d, block = 8, 2, 128, 16
+    ctx = [1000, 301, 640]
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, 3, heads, kv_heads, block, d, d, ctx, torch.bfloat16)
+    m = np.zeros((3, 1, 1000), np.float32)
+    m[:, :, :300] = -np.inf
+    mask = torch.from_numpy(m).to(torch.bfloat16).to(dev)
+    scale = 1.0 / math.sqrt(d)
+    got = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, kernel=kernel, chunk_tokens=chunk, mask=mask)
+    want = oracle_pa(oracle, q, kc, vc, tables, ctx, scale, mask=mask, mask_per_head=False)
+    assert_close(got, want, TOL[torch.bfloat16], "-inf mask")
+
+
+def test_mla_with_norm_mask(binding, oracle, dev, stream):
+    """The combined-cache variant takes a NORM mask (not ALIBI, not logN) in the
+    reference; 128 heads, so the kernel choice with and without mask differs."""
+    rng = _rng(233)
+    batch, heads, d, dv, block = 3, 128, 576, 512, 128
+    ctx = np.array([700, 33, 1500], dtype=np.int32)
+    q, kc, _, tables, ctx = _pa_inputs(rng, dev, batch, heads, 1, block, d, d, ctx, torch.bfloat16, std=0.5)
+    mask, _ = _mask_tensor(oracle, rng, dev, "norm3", ctx, heads, 1500, torch.bfloat16)
+    want = oracle_pa(oracle, q, kc, None, tables, ctx, 0.05, mla_dv=dv, mask=mask, mask_per_head=False)
+    for kernel in (binding.ATBMI_PA_KERNEL_SCALAR, binding.ATBMI_PA_KERNEL_AUTO):
+        got = pa_decode_cabi(binding, stream, q, kc, None, tables, ctx, 0.05, mla_dv=dv, kernel=kernel, mask=mask)
+        assert_close(got, want, TOL[torch.bfloat16], "mla mask kernel=%d" % kernel)
+
+
+def test_masks_logn_and_dynamic_batch_through_operation_api(binding, oracle, dev, stream):
+    """Input order of the operation: q, caches, tables, lens, mask, batchRunStatus, ..., logN
+    (reference paged_attention_operation.cpp:408-444). With a dynamic batch the
+    query holds one row per running sequence only."""
+    rng = _rng(234)
+    heads, kv_heads, d, block = 32, 16, 128, 64
+    ctx = np.array([100, 0, 2000, 64, 0, 777], dtype=np.int32)
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, len(ctx), heads, kv_heads, block, d, d, ctx, torch.float16)
+    q = q[:4].contiguous()
+    status = torch.from_numpy((ctx > 0).astype(np.int32))
+    lens = torch.from_numpy(ctx)
+    logn = torch.from_numpy(rng.uniform(1, 2, size=len(ctx)).astype(np.float32)).to(dev)
+    scale = 1.0 / math.sqrt(d)
+    c = binding.Context(stream)
+    for kind, mask_type in (("norm3", 1), ("alibi4", 2), ("alibi3", 2)):
+        mask, per_head = _mask_tensor(oracle, rng, dev, kind, ctx, heads, 2048, torch.float16)
+        pa = binding.OperationRunner("PagedAttentionOperation", binding.PagedAttentionParam(
+            headNum=heads, kvHeadNum=kv_heads, qkScale=scale, maskType=mask_type, batchRunStatusEnable=True,
+            scaleType=1), c)
+        with torch.cuda.stream(stream):
+            out, = pa.run([q, kc, vc, tables, lens.to(dev), mask, status.to(dev), logn],
+                          host_inputs={4: lens, 6: status})
+        stream.synchronize()
+        assert tuple(out.shape) == (4, heads, d)
+        want = oracle_pa(oracle, q, kc, vc, tables, ctx, scale, mask=mask, mask_per_head=per_head, logn=logn)
+        assert_close(out, want, 1e-3, kind)
+        pa.close()
+    # int8 cache with offsets and a mask: the descale tensors follow the mask
+    q8, kc8, vc8, tables8, ctx8 = _pa_inputs(rng, dev, 4, heads, kv_heads, block, d, d, [100, 2000, 64, 777],
+                                             torch.float16, kv_int8=True)
+    ks = torch.from_numpy(rng.uniform(0.01, 0.1, size=kv_heads * d).astype(np.float32)).to(dev)
+    vs = torch.from_numpy(rng.uniform(0.01, 0.1, size=kv_heads * d).astype(np.float32)).to(dev)
+    ko = torch.from_numpy(rng.integers(-20, 20, size=kv_heads * d).astype(np.int32)).to(dev)
+    vo = torch.from_numpy(rng.integers(-20, 20, size=kv_heads * d).astype(np.int32)).to(dev)
+    mask, _ = _mask_tensor(oracle, rng, dev, "norm3", ctx8, heads, 2000, torch.float16)
+    pa = binding.OperationRunner("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=heads, kvHeadNum=kv_heads, qkScale=scale, quantType=1, hasQuantOffset=True, maskType=1), c)
+    lens8 = torch.from_numpy(ctx8)
+    with torch.cuda.stream(stream):
+        out, = pa.run([q8, kc8, vc8, tables8, lens8.to(dev), mask, ks, ko, vs, vo], host_inputs={4: lens8})
+    stream.synchronize()
+    assert_close(out, oracle_pa(oracle, q8, kc8, vc8, tables8, ctx8, scale, ks, ko, vs, vo, mask=mask,
+                                mask_per_head=False), INT8_TOL, "dequant + mask")
+    pa.close()
+    c.close()
+
+
 # ------------------------------------------------------------------ edge semantics
 @pytest.mark.parametrize("kernel", [1, 0])
 def test_empty_sequences_garbage_rows_and_shared_blocks(binding, oracle, dev, stream, kernel):

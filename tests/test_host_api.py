@@ -31,9 +31,21 @@ RAC_CASES = _load("reshape_and_cache")
 
 def _pa_unimplemented(p):
     """Features of PagedAttentionParam the reference accepts but this library rejects at creation."""
-    return (p.get("maskType", 0) != 0 or p.get("batchRunStatusEnable", False) or p.get("compressType", 0) != 0 or
-            p.get("calcType", 0) != 0 or p.get("scaleType", 0) != 0 or p.get("inputLayout", 0) != 0 or
-            p.get("quantType", 0) >= 2)
+    return (p.get("maskType", 0) >= 3 or p.get("compressType", 0) != 0 or p.get("calcType", 0) != 0 or
+            p.get("inputLayout", 0) != 0 or p.get("quantType", 0) >= 2)
+
+
+def _pa_mask_shape_refused(case):
+    """Mask shapes the reference operation lets through Setup but its tiling has no stride
+    rule for (tiling/paged_attention_tiling.cpp:36-74): a 4-dim NORM mask, and a 3-dim ALIBI
+    mask whose first dim is not the head count. Refused here during Setup."""
+    p = case["param"]
+    if p.get("maskType", 0) not in (1, 2) or _pa_unimplemented(p) or case["expected"] != "NO_ERROR":
+        return False
+    mask = case["in_shapes"][4 if p.get("mlaVHeadSize", 0) > 0 else 5]
+    if p["maskType"] == 1:
+        return len(mask) == 4
+    return len(mask) == 3 and mask[0] != p["headNum"]
 
 
 def _rac_unimplemented(p):
@@ -46,10 +58,12 @@ def _make_param(binding, op, p):
     return binding.ReshapeAndCacheParam(**p)
 
 
-def _tensors(binding, dtypes, formats, shapes, host_index=None, host_array=None):
+def _tensors(binding, dtypes, formats, shapes, host_arrays=None):
+    """host_arrays: {input index: numpy array bound as hostData}."""
     out = []
     for i, (dt, fmt, shape) in enumerate(zip(dtypes, formats, shapes)):
-        host = host_array.ctypes.data if (i == host_index and host_array is not None) else None
+        host = host_arrays[i].ctypes.data if host_arrays and i in host_arrays else None
+        dt = {"float32": "float"}.get(dt, dt)  # the reference table spells ACL_FLOAT both ways
         out.append(binding.make_tensor(dt, shape, device_ptr=FAKE_DEVICE, host_ptr=host, fmt=fmt))
     return out
 
@@ -64,14 +78,18 @@ def _run_case(binding, case, ctx):
         st, out_descs = op.infer_shape(ins)
         if st != 0:
             return "I", st, None
-        host = None
-        host_index = None
+        host = {}
         if case["op"] == "PagedAttentionOperation":
-            host_index = 3 if case["param"].get("mlaVHeadSize", 0) > 0 else 4
+            p = case["param"]
+            lens_index = 3 if p.get("mlaVHeadSize", 0) > 0 else 4
             kc = case["in_shapes"][1]
-            tables = case["in_shapes"][host_index - 1]
-            host = np.full((case["in_shapes"][host_index][0],), min(kc[1] * tables[1], 7), dtype=np.int32)
-        ins = _tensors(binding, case["in_dtypes"], case["in_formats"], case["in_shapes"], host_index, host)
+            tables = case["in_shapes"][lens_index - 1]
+            host[lens_index] = np.full((case["in_shapes"][lens_index][0],), min(kc[1] * tables[1], 7), dtype=np.int32)
+            if p.get("batchRunStatusEnable", False):
+                status_index = lens_index + (2 if p.get("maskType", 0) != 0 else 1)
+                if status_index < len(case["in_shapes"]):
+                    host[status_index] = np.ones((case["in_shapes"][status_index][0],), dtype=np.int32)
+        ins = _tensors(binding, case["in_dtypes"], case["in_formats"], case["in_shapes"], host)
         outs = _tensors(binding, case["out_dtypes"], case["out_formats"], case["out_shapes"])
         st, _ = op.setup(ins, outs, ctx)
         if st != 0:
@@ -88,12 +106,15 @@ def ctx(binding):
     c.close()
 
 
-def _check(binding, case, ctx, unimplemented):
+def _check(binding, case, ctx, unimplemented, refused_at_setup=False):
     stage, status, out_descs = _run_case(binding, case, ctx)
     expected = case["expected"]
     if unimplemented:
         # documented deviation: rejected when the operation is created
         assert (stage, status) == ("C", binding.ERROR_CODE["ERROR_INVALID_PARAM"])
+        return
+    if refused_at_setup:
+        assert (stage, status) == ("S", binding.ERROR_CODE["ERROR_INVALID_PARAM"])
         return
     if expected == "NO_ERROR":
         assert (stage, status) == ("", 0), "%s: %s:%s" % (case["name"], stage, binding.ERROR_NAMES[status])
@@ -107,7 +128,8 @@ def _check(binding, case, ctx, unimplemented):
 
 @pytest.mark.parametrize("case", PA_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
 def test_paged_attention_table(binding, ctx, case):
-    _check(binding, case, ctx, _pa_unimplemented(case["param"]) and not case["expected"].startswith("C:"))
+    _check(binding, case, ctx, _pa_unimplemented(case["param"]) and not case["expected"].startswith("C:"),
+           _pa_mask_shape_refused(case))
 
 
 @pytest.mark.parametrize("case", RAC_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
@@ -117,9 +139,10 @@ def test_reshape_and_cache_table(binding, ctx, case):
 
 def test_table_coverage():
     """Most rows of the reference tables must be checked at face value, not as deviations."""
-    pa_dev = [c for c in PA_CASES if _pa_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
+    pa_dev = [c for c in PA_CASES if (_pa_unimplemented(c["param"]) and not c["expected"].startswith("C:")) or
+              _pa_mask_shape_refused(c)]
     rac_dev = [c for c in RAC_CASES if _rac_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
-    assert len(PA_CASES) == 81 and len(PA_CASES) - len(pa_dev) >= 55
+    assert len(PA_CASES) == 81 and len(PA_CASES) - len(pa_dev) >= 68
     assert len(RAC_CASES) == 37 and len(RAC_CASES) - len(rac_dev) >= 25
 
 
@@ -146,6 +169,10 @@ def test_names_and_tensor_counts(binding):
         (binding.PagedAttentionParam(headNum=8, kvHeadNum=8, quantType=1), 7),
         (binding.PagedAttentionParam(headNum=8, kvHeadNum=8, quantType=1, hasQuantOffset=True), 9),
         (binding.PagedAttentionParam(headNum=8, kvHeadNum=1, mlaVHeadSize=512), 4),
+        (binding.PagedAttentionParam(headNum=8, kvHeadNum=8, maskType=1), 6),
+        (binding.PagedAttentionParam(headNum=8, kvHeadNum=8, maskType=2, batchRunStatusEnable=True, scaleType=1), 8),
+        (binding.PagedAttentionParam(headNum=8, kvHeadNum=8, maskType=1, quantType=1, hasQuantOffset=True), 10),
+        (binding.PagedAttentionParam(headNum=8, kvHeadNum=1, mlaVHeadSize=512, maskType=1), 5),
     ]
     for p, n in cases:
         op = binding.Operation("PagedAttentionOperation", p)
@@ -288,6 +315,72 @@ def test_setup_and_execute_error_paths(binding, ctx):
     op.close()
 
 
+def test_mask_status_and_logn_inputs(binding, ctx):
+    """Setup-time rules for the optional inputs: mask layouts (reference
+    tiling/paged_attention_tiling.cpp:36-74), the host-side status vector
+    (param.cpp:39-49), logN sizes (paged_attention_operation.cpp:900-924), and
+    the smaller query of a dynamic batch (:679-688, :935-941)."""
+    e = binding.ERROR_CODE
+    lens = np.array([5, 0, 7, 200], dtype=np.int32)
+    status = np.array([1, 0, 1, 1], dtype=np.int32)
+
+    def pack(mask_shape=None, q_rows=4, out_rows=None, status_host=True, logn=None, mask_dtype="float16"):
+        ins = [
+            binding.make_tensor("float16", [q_rows, 32, 128], FAKE_DEVICE),
+            binding.make_tensor("float16", [8, 64, 16, 128], FAKE_DEVICE),
+            binding.make_tensor("float16", [8, 64, 16, 128], FAKE_DEVICE),
+            binding.make_tensor("int32", [4, 4], FAKE_DEVICE),
+            binding.make_tensor("int32", [4], FAKE_DEVICE, host_ptr=lens.ctypes.data),
+        ]
+        if mask_shape is not None:
+            ins.append(binding.make_tensor(mask_dtype, mask_shape, FAKE_DEVICE))
+        if status_host is not None:
+            ins.append(binding.make_tensor("int32", [4], FAKE_DEVICE,
+                                           host_ptr=status.ctypes.data if status_host else None))
+        if logn is not None:
+            ins.append(binding.make_tensor("float", logn, FAKE_DEVICE))
+        outs = [binding.make_tensor("float16", [q_rows if out_rows is None else out_rows, 32, 128], FAKE_DEVICE)]
+        return ins, outs
+
+    def setup(op, *a, **k):
+        return op.setup(*pack(*a, **k), ctx)[0]
+
+    norm = binding.Operation("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=32, kvHeadNum=16, qkScale=0.088, maskType=1))
+    for shape, want in (([4, 1, 256], 0), ([1, 256], 0), ([4, 1, 200], 0), ([4, 1, 199], e["ERROR_INVALID_PARAM"]),
+                        ([3, 1, 256], e["ERROR_INVALID_PARAM"]), ([4, 2, 256], e["ERROR_INVALID_PARAM"]),
+                        ([4, 32, 1, 256], e["ERROR_INVALID_PARAM"]), ([2, 256], e["ERROR_INVALID_PARAM"])):
+        assert setup(norm, shape, status_host=None) == want, shape
+    # the mask has q's dtype
+    assert setup(norm, [4, 1, 256], status_host=None, mask_dtype="bf16") == e["ERROR_INVALID_TENSOR_INI_MATCH"]
+    norm.close()
+
+    alibi = binding.Operation("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=32, kvHeadNum=16, qkScale=0.088, maskType=2))
+    for shape, want in (([32, 1, 256], 0), ([4, 32, 1, 256], 0), ([4, 1, 1, 256], 0),
+                        ([4, 1, 256], e["ERROR_INVALID_PARAM"]), ([4, 16, 1, 256], e["ERROR_INVALID_PARAM"]),
+                        ([4, 32, 2, 256], e["ERROR_INVALID_PARAM"]), ([1, 256], e["ERROR_INVALID_PARAM"])):
+        assert setup(alibi, shape, status_host=None) == want, shape
+    alibi.close()
+
+    dyn = binding.Operation("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=32, kvHeadNum=16, qkScale=0.088, batchRunStatusEnable=True, scaleType=1))
+    assert setup(dyn, logn=[4]) == 0
+    assert setup(dyn, q_rows=3, logn=[4]) == 0                      # three running sequences, three query rows
+    assert setup(dyn, q_rows=2, logn=[4]) == e["ERROR_INVALID_PARAM"]  # fewer rows than non-empty sequences
+    assert setup(dyn, q_rows=5, logn=[4]) == e["ERROR_INVALID_TENSOR_DIM"]
+    assert setup(dyn, q_rows=3, out_rows=4, logn=[4]) == e["ERROR_INVALID_TENSOR_DIM"]
+    assert setup(dyn, status_host=False, logn=[4]) == e["ERROR_INVALID_PARAM"]
+    assert setup(dyn, logn=[5]) == e["ERROR_INVALID_TENSOR_DIM"]
+    assert setup(dyn, logn=[4, 1]) == e["ERROR_INVALID_TENSOR_DIM"]
+    dyn.close()
+    # without the dynamic batch the query must cover every sequence of contextLens
+    plain = binding.Operation("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=32, kvHeadNum=16, qkScale=0.088))
+    assert setup(plain, status_host=None) == 0
+    plain.close()
+
+
 def test_dequant_vector_lengths(binding, ctx):
     e = binding.ERROR_CODE
     op = binding.Operation("PagedAttentionOperation",
@@ -381,3 +474,15 @@ def test_kernel_layer_validates_without_a_gpu(binding):
     lens[2] = 513
     assert k.atbmi_pa_plan_update(plan, lens.ctypes.data, 4) == 1
     k.atbmi_pa_plan_destroy(plan)
+    # a mask needs a row length and non-negative strides; its bytes count per distinct row
+    lens[2] = 512
+    shape.hasMask = 1
+    assert k.atbmi_pa_plan_create(ctypes.byref(shape), ctypes.byref(plan)) == 1
+    for batch_stride, head_stride, extra in ((0, 0, 512), (512, 0, 619), (0, 512, 8 * 512), (8 * 512, 512, 8 * 619)):
+        shape.maskLen, shape.maskBatchStride, shape.maskHeadStride, shape.hasLogN = 512, batch_stride, head_stride, 1
+        assert k.atbmi_pa_plan_create(ctypes.byref(shape), ctypes.byref(plan)) == 0
+        assert k.atbmi_pa_plan_update(plan, lens.ctypes.data, 4) == 0
+        assert k.atbmi_pa_plan_algorithmic_bytes(plan) == want + extra * 2 + 4 * 4
+        k.atbmi_pa_plan_destroy(plan)
+    shape.maskBatchStride = -1
+    assert k.atbmi_pa_plan_create(ctypes.byref(shape), ctypes.byref(plan)) == 1

@@ -225,6 +225,126 @@ def test_attention_empty_sequences_take_no_query_row(oracle):
     assert np.all(out[3] == np.float32(0.1))
 
 
+# ---------------------------------------------------------------- masks and logN
+def _with_empty(ctx, at):
+    ctx = ctx.copy()
+    ctx[at] = 0
+    return ctx
+
+
+def test_masked_attention_matches_independent_loops(oracle):
+    """Every mask layout against the float64 loops on a densely expanded bias, with an
+    empty sequence in the middle: the mask and logN rows go by the index into
+    context_lens, the query rows by the count of non-empty sequences before."""
+    rng = _rng(30)
+    q, kc, vc, tables, ctx = _paged_case(rng, batch=5, heads=4, kv_heads=2, max_ctx=11)
+    ctx = _with_empty(ctx, 2)
+    batch, heads, max_len = 5, 4, 13
+    logn = rng.uniform(1, 2, size=batch).astype(np.float32)
+    layouts = {
+        "norm2": (rng.standard_normal((1, max_len)), None, lambda m, i, h: m[0]),
+        "norm3": (rng.standard_normal((batch, 1, max_len)), False, lambda m, i, h: m[i, 0]),
+        "alibi3": (rng.standard_normal((heads, 1, max_len)), True, lambda m, i, h: m[h, 0]),
+        "alibi4": (rng.standard_normal((batch, heads, 1, max_len)), None, lambda m, i, h: m[i, h, 0]),
+        "alibi4_1": (rng.standard_normal((batch, 1, 1, max_len)), None, lambda m, i, h: m[i, 0, 0]),
+    }
+    for name, (mask, per_head, row) in layouts.items():
+        mask = mask.astype(np.float32)
+        dense = np.stack([np.stack([row(mask, i, h) for h in range(heads)]) for i in range(batch)])
+        got = oracle.paged_attention(q, kc, vc, tables, ctx, 0.3, mask=mask, mask_per_head=per_head, logn=logn)
+        want = oracle.paged_attention_loops(q, kc, vc, tables, ctx, 0.3, dense_bias=dense, logn=logn)
+        np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-6, err_msg=name)
+
+
+def test_mask_matches_torch_sdpa_attn_mask(oracle):
+    rng = _rng(31)
+    q, kc, vc, tables, ctx = _paged_case(rng, batch=3, heads=6, kv_heads=6, d=32, dv=32, block=8, pool=30, max_ctx=40)
+    mask = rng.standard_normal((3, 6, 1, 40)).astype(np.float32)
+    out = oracle.paged_attention(q, kc, vc, tables, ctx, 0.21, mask=mask)
+    for i in range(3):
+        keys = oracle.gather_rows(kc, tables[i], ctx[i])
+        vals = oracle.gather_rows(vc, tables[i], ctx[i])
+        want = torch.nn.functional.scaled_dot_product_attention(
+            torch.from_numpy(q[i])[:, None, :].double(), torch.from_numpy(keys).permute(1, 0, 2).double(),
+            torch.from_numpy(vals).permute(1, 0, 2).double(),
+            attn_mask=torch.from_numpy(mask[i, :, :, :ctx[i]]).double(), scale=0.21)
+        np.testing.assert_allclose(out[i], want[:, 0, :].numpy(), rtol=2e-5, atol=2e-6)
+
+
+def test_mask_two_token_closed_form(oracle):
+    """q = 0: the weights are softmax(bias) alone, sigma(b0 - b1) for two tokens."""
+    kc = np.zeros((1, 4, 1, 4), np.float32)
+    vc = np.zeros((1, 4, 1, 2), np.float32)
+    vc[0, 0, 0] = [1.0, 10.0]
+    vc[0, 1, 0] = [3.0, -10.0]
+    q = np.zeros((1, 1, 4), np.float32)
+    mask = np.array([[[0.5, -1.5, 99.0, 99.0]]], np.float32)
+    out = oracle.paged_attention(q, kc, vc, np.zeros((1, 1), np.int32), np.array([2], np.int32), 1.0, mask=mask,
+                                 mask_per_head=False)
+    w = 1.0 / (1.0 + math.exp(-2.0))
+    np.testing.assert_allclose(out[0, 0], [w * 1 + (1 - w) * 3, w * 10 - (1 - w) * 10], rtol=1e-6)
+
+
+def test_mask_hiding_positions_equals_attention_over_the_rest(oracle):
+    """-inf, and the reference tests' -10000, on the first k positions leave exactly
+    the attention over the remaining tokens."""
+    rng = _rng(32)
+    q, kc, vc, tables, ctx = _paged_case(rng, batch=4, heads=4, kv_heads=2, block=4, max_ctx=14)
+    ctx = np.maximum(ctx, 5)
+    tables = np.tile(np.arange(4, dtype=np.int32), (4, 1)) + 4 * np.arange(4, dtype=np.int32)[:, None]
+    for value, tol in ((-np.inf, 1e-6), (-10000.0, 1e-6)):
+        mask = oracle.norm_mask(4, 16, value)
+        out = oracle.paged_attention(q, kc, vc, tables, ctx, 0.4, mask=mask, mask_per_head=False)
+        for i in range(4):
+            keys = oracle.gather_rows(kc, tables[i], ctx[i])[i:]
+            vals = oracle.gather_rows(vc, tables[i], ctx[i])[i:]
+            np.testing.assert_allclose(out[i], oracle.attention_one(q[i], keys, vals, 0.4), rtol=tol, atol=tol)
+
+
+def test_mask_constant_along_a_row_changes_nothing(oracle):
+    rng = _rng(33)
+    q, kc, vc, tables, ctx = _paged_case(rng, batch=3, heads=4, kv_heads=2)
+    base = oracle.paged_attention(q, kc, vc, tables, ctx, 0.25)
+    mask = np.broadcast_to(rng.standard_normal((3, 4, 1, 1)).astype(np.float32), (3, 4, 1, 14)).copy()
+    np.testing.assert_allclose(oracle.paged_attention(q, kc, vc, tables, ctx, 0.25, mask=mask), base,
+                               rtol=1e-5, atol=1e-6)
+    zero = np.zeros((4, 1, 14), np.float32)
+    assert np.array_equal(oracle.paged_attention(q, kc, vc, tables, ctx, 0.25, mask=zero, mask_per_head=True), base)
+
+
+def test_alibi_slopes_and_mask_closed_form(oracle):
+    # the published ALiBi slopes: 8 heads -> 1/2 .. 1/256; 12 heads add 2^-0.5, 2^-1.5, 2^-2.5, 2^-3.5
+    np.testing.assert_allclose(oracle.alibi_slopes(8), [2.0 ** -k for k in range(1, 9)], rtol=1e-7)
+    np.testing.assert_allclose(oracle.alibi_slopes(12)[8:], [2.0 ** -0.5, 2.0 ** -1.5, 2.0 ** -2.5, 2.0 ** -3.5],
+                               rtol=1e-7)
+    assert len(oracle.alibi_slopes(40)) == 40
+    m = oracle.alibi_mask([3, 0, 5], 8, 6)
+    assert m.shape == (3, 8, 1, 6)
+    assert np.array_equal(m[0, 0, 0], [-1.0, -0.5, 0.0, 0.0, 0.0, 0.0])   # slope 1/2, distances 2, 1, 0
+    assert np.array_equal(m[2, 1, 0], [-1.0, -0.75, -0.5, -0.25, 0.0, 0.0])  # slope 1/4
+    assert not m[1].any()
+    n = oracle.norm_mask(3, 4)
+    assert np.array_equal(n[:, 0], [[0, 0, 0, 0], [-10000, 0, 0, 0], [-10000, -10000, 0, 0]])
+
+
+def test_logn_is_a_per_sequence_factor_on_the_scale(oracle):
+    rng = _rng(34)
+    q, kc, vc, tables, ctx = _paged_case(rng, batch=4)
+    ctx = _with_empty(ctx, 1)
+    logn = np.array([1.25, 7.0, 1.5, 2.0], np.float32)
+    out = oracle.paged_attention(q, kc, vc, tables, ctx, 0.25, logn=logn)
+    row = 0
+    for i in range(4):
+        if ctx[i] == 0:
+            continue
+        want = oracle.paged_attention(q[row:row + 1], kc, vc, tables[i:i + 1], ctx[i:i + 1],
+                                      np.float32(0.25) * logn[i])
+        assert np.array_equal(out[row], want[0])
+        row += 1
+    assert np.array_equal(oracle.paged_attention(q, kc, vc, tables, ctx, 0.25, logn=np.ones(4, np.float32)),
+                          oracle.paged_attention(q, kc, vc, tables, ctx, 0.25))
+
+
 def test_int8_dequant_channel_indexing_and_identity(oracle):
     rng = _rng(11)
     q, _, _, tables, ctx = _paged_case(rng, heads=4, kv_heads=2, d=8, dv=8)
