@@ -92,6 +92,7 @@ class AtbmiPaShape(ctypes.Structure):
         ("kernel", ctypes.c_int32), ("hasMask", ctypes.c_int32), ("qkScale", ctypes.c_float),
         ("qScale", ctypes.c_float), ("maskBatchStride", ctypes.c_int64), ("maskHeadStride", ctypes.c_int64),
         ("maskLen", ctypes.c_int32), ("hasLogN", ctypes.c_int32),
+        ("descalePacked", ctypes.c_int32), ("reserved", ctypes.c_int32),
     ]
 
 
@@ -165,6 +166,8 @@ def atb():
         lib.atb_c_op_execute.argtypes = [vp, tp, u32, tp, u32, vp, u64, vp]
         lib.atb_c_tensor_size.argtypes = [tp]
         lib.atb_c_tensor_size.restype = u64
+        lib.atb_c_quant_param_convert.argtypes = [ctypes.c_void_p, ctypes.c_void_p, u64]
+        lib.atb_c_quant_param_convert.restype = None
         lib.atb_c_sizeof_paged_attention_param.restype = u64
         lib.atb_c_sizeof_reshape_and_cache_param.restype = u64
         _atb = lib

@@ -83,6 +83,7 @@ struct PaArgs {
     int32_t maskLen;     // tokens per mask row
     int32_t maskVec;     // 1: every mask row starts on an 8-byte boundary (4-token vector loads are legal)
     const float *logN;   // per batch row factor on qkScale (null: none)
+    int32_t scaleStride; // floats between consecutive kScale / vScale entries: 1, or 2 for uint64-packed ones
 };
 
 // ---- Plan of the MFMA kernel ------------------------------------------------

@@ -147,6 +147,9 @@ extern "C" int atbmi_pa_plan_create(const AtbmiPaShape *shape, AtbmiPaPlan **pla
     if (s.hasOffset && s.kvDtype != ATBMI_INT8) {
         return Fail(ERR_INVALID_PARAM, "pa_plan_create: offsets only apply to an int8 cache");
     }
+    if (s.descalePacked && s.kvDtype != ATBMI_INT8) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: packed descales only apply to an int8 cache");
+    }
     if (s.hasMask && (s.maskLen <= 0 || s.maskBatchStride < 0 || s.maskHeadStride < 0)) {
         return Fail(ERR_INVALID_PARAM, "pa_plan_create: mask row length %d, strides %lld / %lld", s.maskLen,
                     (long long)s.maskBatchStride, (long long)s.maskHeadStride);
@@ -609,6 +612,7 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
                      s.maskHeadStride % 4 == 0) ? 1 : 0;
     }
     a.logN = s.hasLogN ? t->logN : nullptr;
+    a.scaleStride = s.descalePacked ? 2 : 1; // little endian: the low half of each uint64 comes first
 
     TimingRecord rec{nullptr, nullptr};
     bool timed = false;

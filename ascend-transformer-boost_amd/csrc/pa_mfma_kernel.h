@@ -268,7 +268,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                             f[e] = qBf16 ? Bf16ToFloat(FloatToBf16(f[e])) : HalfBitsToFloat(FloatToHalfBits(f[e]));
                         }
                         if (KV8) {
-                            f[e] *= a.kScale[g * D + d0 + e];
+                            f[e] *= a.kScale[(g * D + d0 + e) * a.scaleStride];
                         }
                     }
 #pragma unroll
@@ -688,7 +688,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                         o[r] = acc[i][r] * inv - bias;
                         if (KV8) {
                             const int c = g * DV + d + r;
-                            o[r] = (o[r] + (a.vOff ? static_cast<float>(a.vOff[c]) : 0.0f)) * a.vScale[c];
+                            o[r] = (o[r] + (a.vOff ? static_cast<float>(a.vOff[c]) : 0.0f)) * a.vScale[c * a.scaleStride];
                         }
                     }
                     u32x2 packed;

@@ -47,7 +47,7 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaReduceKernel(const PaArgs a)
         acc *= inv;
         if (a.finishV) {
             const int c = g * a.Dv + d;
-            acc = (acc + (a.vOff ? static_cast<float>(a.vOff[c]) : 0.0f)) * a.vScale[c];
+            acc = (acc + (a.vOff ? static_cast<float>(a.vOff[c]) : 0.0f)) * a.vScale[c * a.scaleStride];
         }
         Store16(a.out, (static_cast<int64_t>(s.qRow) * a.H + h) * a.Dv + d, acc, bf16);
     }
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaA
             float o = acc[c] * inv;
             if (a.finishV) {
                 const int ch = g * a.Dv + d;
-                o = (o + (a.vOff ? static_cast<float>(a.vOff[ch]) : 0.0f)) * a.vScale[ch];
+                o = (o + (a.vOff ? static_cast<float>(a.vOff[ch]) : 0.0f)) * a.vScale[ch * a.scaleStride];
             }
             Store16(a.out, (static_cast<int64_t>(b) * a.H + h) * a.Dv + d, o, bf16);
         }

@@ -74,11 +74,11 @@ __global__ __launch_bounds__(PA_SCALAR_WAVES * WAVE) void PaScalarKernel(const P
         kS[e] = 1.0f; kO[e] = 0.0f; vS[e] = 1.0f; vO[e] = 0.0f;
         if (KV8) {
             if (d < a.D) {
-                kS[e] = a.kScale[g * a.D + d];
+                kS[e] = a.kScale[(g * a.D + d) * a.scaleStride];
                 kO[e] = a.kOff ? static_cast<float>(a.kOff[g * a.D + d]) : 0.0f;
             }
             if (d < a.Dv) {
-                vS[e] = a.vScale[g * a.Dv + d];
+                vS[e] = a.vScale[(g * a.Dv + d) * a.scaleStride];
                 vO[e] = a.vOff ? static_cast<float>(a.vOff[g * a.Dv + d]) : 0.0f;
             }
         }

@@ -197,6 +197,11 @@ uint64_t atb_c_tensor_size(const AtbCTensor *tensor)
     return tensor ? atb::Utils::GetTensorSize(ToTensor(*tensor).desc) : 0;
 }
 
+void atb_c_quant_param_convert(const float *src, uint64_t *dest, uint64_t itemCount)
+{
+    atb::Utils::QuantParamConvert(src, dest, itemCount);
+}
+
 uint64_t atb_c_sizeof_paged_attention_param(void)
 {
     return sizeof(atb::infer::PagedAttentionParam);

@@ -12,12 +12,12 @@
 // reference runner does (src/ops/ops_infer/paged_attention/param.cpp:16-62).
 //
 // Implemented feature set: fp16/bf16 caches, int8 caches with fp32 per-channel
-// descale (+ int32 offset), the MLA combined cache (mlaVHeadSize > 0), additive
+// descale, plain or uint64-packed, (+ int32 offset), the MLA combined cache (mlaVHeadSize > 0), additive
 // NORM and ALIBI masks, the dynamic-batch status input and per-sequence LogN
 // scaling. Speculative (multi-token) queries with their masks, head
-// compression, BNSD layout, int8 queries and int64-packed descales are legal
-// in the reference but not implemented here; such params are rejected at
-// creation with ERROR_INVALID_PARAM.
+// compression, BNSD layout and int8 queries are legal in the reference but not
+// implemented here; such params are rejected at creation with
+// ERROR_INVALID_PARAM.
 #include <cmath>
 #include <new>
 #include "atb/infer_op_params.h"
@@ -159,44 +159,53 @@ bool ImplementedCheck(const Param &p)
     return true;
 }
 
+// One row of the dtype table: query dtype q, and for an int8 cache the dtype of
+// its descales, fp32 or uint64-packed fp32 (Utils::QuantParamConvert). Optional
+// inputs follow in the reference's order (:408-444).
+IrCombo MakeCombo(const Param &p, aclDataType q, aclDataType descale)
+{
+    IrCombo c;
+    const bool dequant = p.quantType == Param::TYPE_DEQUANT_FUSION;
+    if (p.mlaVHeadSize > 0) {
+        c.inDtypes = {q, q, ACL_INT32, ACL_INT32};
+    } else if (dequant) {
+        c.inDtypes = {q, ACL_INT8, ACL_INT8, ACL_INT32, ACL_INT32};
+    } else {
+        c.inDtypes = {q, q, q, ACL_INT32, ACL_INT32};
+    }
+    if (p.maskType != Param::UNDEFINED) {
+        c.inDtypes.push_back(q);
+    }
+    if (p.batchRunStatusEnable) {
+        c.inDtypes.push_back(ACL_INT32);
+    }
+    if (dequant) {
+        c.inDtypes.push_back(descale);
+        if (p.hasQuantOffset) {
+            c.inDtypes.push_back(ACL_INT32);
+        }
+        c.inDtypes.push_back(descale);
+        if (p.hasQuantOffset) {
+            c.inDtypes.push_back(ACL_INT32);
+        }
+    }
+    if (p.scaleType == Param::SCALE_TYPE_LOGN) {
+        c.inDtypes.push_back(ACL_FLOAT);
+    }
+    c.inFormats.assign(c.inDtypes.size(), ACL_FORMAT_ND);
+    c.outDtypes = {q};
+    c.outFormats = {ACL_FORMAT_ND};
+    return c;
+}
+
 OpIr MakeIr(const Param &p)
 {
     OpIr ir;
-    const aclFormat nd = ACL_FORMAT_ND;
     for (aclDataType q : {ACL_FLOAT16, ACL_BF16}) {
-        IrCombo c;
-        const bool dequant = p.quantType == Param::TYPE_DEQUANT_FUSION;
-        if (p.mlaVHeadSize > 0) {
-            c.inDtypes = {q, q, ACL_INT32, ACL_INT32};
-        } else if (dequant) {
-            c.inDtypes = {q, ACL_INT8, ACL_INT8, ACL_INT32, ACL_INT32};
-        } else {
-            c.inDtypes = {q, q, q, ACL_INT32, ACL_INT32};
+        ir.push_back(MakeCombo(p, q, ACL_FLOAT));
+        if (p.quantType == Param::TYPE_DEQUANT_FUSION) {
+            ir.push_back(MakeCombo(p, q, ACL_INT64));
         }
-        // Optional inputs, in the reference's order (:408-444).
-        if (p.maskType != Param::UNDEFINED) {
-            c.inDtypes.push_back(q);
-        }
-        if (p.batchRunStatusEnable) {
-            c.inDtypes.push_back(ACL_INT32);
-        }
-        if (dequant) {
-            c.inDtypes.push_back(ACL_FLOAT);
-            if (p.hasQuantOffset) {
-                c.inDtypes.push_back(ACL_INT32);
-            }
-            c.inDtypes.push_back(ACL_FLOAT);
-            if (p.hasQuantOffset) {
-                c.inDtypes.push_back(ACL_INT32);
-            }
-        }
-        if (p.scaleType == Param::SCALE_TYPE_LOGN) {
-            c.inDtypes.push_back(ACL_FLOAT);
-        }
-        c.inFormats.assign(c.inDtypes.size(), nd);
-        c.outDtypes = {q};
-        c.outFormats = {nd};
-        ir.push_back(c);
     }
     return ir;
 }
@@ -439,6 +448,7 @@ protected:
         shape.maskHeadStride = maskHeadStride;
         shape.maskLen = static_cast<int32_t>(maskLen);
         shape.hasLogN = logNIdx_ != NONE ? 1 : 0;
+        shape.descalePacked = (dequant_ && pack.inTensors.at(kScaleIdx_).desc.dtype == ACL_INT64) ? 1 : 0;
         if (!plan_ || !SameShape(shape, planShape_)) {
             if (plan_) {
                 atbmi_pa_plan_destroy(plan_);
@@ -501,7 +511,7 @@ private:
                a.numQueryRows == b.numQueryRows && a.mlaCombined == b.mlaCombined && a.hasOffset == b.hasOffset &&
                a.qkScale == b.qkScale && a.qScale == b.qScale && a.hasMask == b.hasMask &&
                a.maskBatchStride == b.maskBatchStride && a.maskHeadStride == b.maskHeadStride &&
-               a.maskLen == b.maskLen && a.hasLogN == b.hasLogN;
+               a.maskLen == b.maskLen && a.hasLogN == b.hasLogN && a.descalePacked == b.descalePacked;
     }
 
     // Element strides of the additive mask, as the reference derives them from

@@ -64,6 +64,9 @@ int32_t atb_c_op_execute(void *operation, const AtbCTensor *inTensors, uint32_t 
 /* atb::Utils::GetTensorSize on the desc fields. */
 uint64_t atb_c_tensor_size(const AtbCTensor *tensor);
 
+/* atb::Utils::QuantParamConvert (reference include/atb/utils.h:82): fp32 bits into the low half of uint64. */
+void atb_c_quant_param_convert(const float *src, uint64_t *dest, uint64_t itemCount);
+
 /* sizeof(infer::PagedAttentionParam), sizeof(infer::ReshapeAndCacheParam). */
 uint64_t atb_c_sizeof_paged_attention_param(void);
 uint64_t atb_c_sizeof_reshape_and_cache_param(void);

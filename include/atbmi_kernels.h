@@ -109,6 +109,9 @@ typedef struct AtbmiPaShape {
     int64_t maskHeadStride;  /* elements between the mask rows of consecutive query heads (0: shared) */
     int32_t maskLen;         /* tokens per mask row, >= every context length */
     int32_t hasLogN;         /* 1: a per-sequence factor on qkScale (AtbmiPaTensors.logN) is given */
+    int32_t descalePacked;   /* 1: kScale / vScale are uint64 arrays whose low 32 bits hold the fp32 value,
+                                as atb::Utils::QuantParamConvert packs them (reference src/atb/utils/utils.cpp:153-164) */
+    int32_t reserved;        /* 0 */
 } AtbmiPaShape;
 
 /* Device tensors of one decode call.
@@ -116,7 +119,8 @@ typedef struct AtbmiPaShape {
  *   keyCache    [numBlocks, blockSize, G, D]        kvDtype
  *   valueCache  [numBlocks, blockSize, G, Dv]       kvDtype (NULL when mlaCombined)
  *   blockTables [batch, maxBlocksPerSeq]            int32
- *   kScale/vScale [G*D] / [G*Dv] fp32, kOffset/vOffset same length int32 (int8 KV only)
+ *   kScale/vScale [G*D] / [G*Dv] fp32 (or uint64-packed fp32, see descalePacked), kOffset/vOffset same
+ *               length int32 (int8 KV only)
  *   out         [numQueryRows, H, Dv]               qDtype
  *   mask        qDtype, hasMask only: the score of sequence b (its index in hostContextLens), head h and
  *               token t gets mask[b * maskBatchStride + h * maskHeadStride + t] added after the qkScale

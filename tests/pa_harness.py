@@ -36,7 +36,8 @@ def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=
         numQueryRows=rows, mlaCombined=1 if mla_dv else 0, hasOffset=1 if k_off is not None else 0, kernel=kernel,
         qkScale=scale, qScale=q_scale, hasMask=0 if mask is None else 1, maskBatchStride=mask_batch_stride,
         maskHeadStride=mask_head_stride, maskLen=0 if mask is None else mask.shape[-1],
-        hasLogN=0 if logn is None else 1)
+        hasLogN=0 if logn is None else 1,
+        descalePacked=1 if (k_scale is not None and k_scale.dtype == torch.int64) else 0)
     old = os.environ.get("ATBMI_PA_CHUNK_TOKENS")
     if chunk_tokens is not None:
         os.environ["ATBMI_PA_CHUNK_TOKENS"] = str(chunk_tokens)
@@ -82,6 +83,12 @@ def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=
     finally:
         k.atbmi_pa_plan_destroy(plan)
     return (out, info) if return_plan_info else out
+
+
+def pack_descale(scale):
+    """fp32 device vector -> int64 device vector with the float's bits in the low half
+    (what atb::Utils::QuantParamConvert produces on the host)."""
+    return scale.contiguous().view(torch.int32).to(torch.int64) & 0xFFFFFFFF
 
 
 def mask_strides(mask, per_head):

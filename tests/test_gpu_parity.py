@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from pa_harness import assert_close, oracle_pa, pa_decode_cabi, random_tables, to_oracle
+from pa_harness import assert_close, oracle_pa, pa_decode_cabi, pack_descale, random_tables, to_oracle
 
 pytestmark = pytest.mark.gpu
 
@@ -309,6 +309,18 @@ def test_int8_through_operation_api_with_offsets(binding, oracle, dev, stream):
         out, = pa.run([q, kc, vc, tables, lens.to(dev), ks, ko, vs, vo], host_inputs={4: lens})
     stream.synchronize()
     assert_close(out, oracle_pa(oracle, q, kc, vc, tables, ctx, scale, ks, ko, vs, vo), INT8_TOL, "dequant api")
+    # the same descales uint64-packed (Utils::QuantParamConvert; reference
+    # test_paged_attention_common.py:120-122,523-533): bit-identical output
+    ks64, vs64 = pack_descale(ks), pack_descale(vs)
+    assert ks64.dtype == torch.int64 and int(ks64.min()) >= 0
+    with torch.cuda.stream(stream):
+        out64, = pa.run([q, kc, vc, tables, lens.to(dev), ks64, ko, vs64, vo], host_inputs={4: lens})
+    stream.synchronize()
+    assert torch.equal(out64, out)
+    for kernel in (binding.ATBMI_PA_KERNEL_SCALAR, binding.ATBMI_PA_KERNEL_AUTO):
+        a = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, ks, ko, vs, vo, kernel=kernel)
+        b = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, ks64, ko, vs64, vo, kernel=kernel)
+        assert torch.equal(a, b)
     pa.close()
     c.close()
 

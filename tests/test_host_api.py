@@ -400,12 +400,27 @@ def test_dequant_vector_lengths(binding, ctx):
     outs = [binding.make_tensor("float16", [4, 32, 128], FAKE_DEVICE)]
     assert op.setup(pack(2048), outs, ctx)[0] == 0
     assert op.setup(pack(128), outs, ctx)[0] == e["ERROR_INVALID_PARAM"]
-    # int64-packed descales are a reference feature that is not implemented here
+    # uint64-packed descales (Utils::QuantParamConvert): both vectors or neither
     ins = pack(2048)
     ins[5] = binding.make_tensor("int64", [2048], FAKE_DEVICE)
-    ins[6] = binding.make_tensor("int64", [2048], FAKE_DEVICE)
     assert op.setup(ins, outs, ctx)[0] == e["ERROR_INVALID_TENSOR_INI_MATCH"]
+    ins[6] = binding.make_tensor("int64", [2048], FAKE_DEVICE)
+    assert op.setup(ins, outs, ctx)[0] == 0
+    ins[5] = binding.make_tensor("int64", [128], FAKE_DEVICE)
+    assert op.setup(ins, outs, ctx)[0] == e["ERROR_INVALID_PARAM"]
     op.close()
+
+
+def test_quant_param_convert(binding):
+    """reference tests/unittest/core/test_utils.cpp:37-50: the low 32 bits carry the float, the rest is 0;
+    null arguments are ignored."""
+    lib = binding.atb()
+    lib.atb_c_quant_param_convert(None, None, 0)
+    src = np.array([1.0, 2.3, 3.0, 4.0, 5.0, -0.0, np.inf], dtype=np.float32)
+    dest = np.full(len(src), 0xFFFFFFFFFFFFFFFF, dtype=np.uint64)
+    lib.atb_c_quant_param_convert(src.ctypes.data, dest.ctypes.data, len(src))
+    assert np.array_equal(dest, src.view(np.uint32).astype(np.uint64))
+    assert np.array_equal((dest & 0xFFFFFFFF).astype(np.uint32).view(np.float32), src)
 
 
 def test_tensor_size_helper(binding):
