@@ -41,6 +41,7 @@ ERROR_CODE = {n: i for i, n in enumerate(ERROR_NAMES)}
 
 ATBMI_F16, ATBMI_BF16, ATBMI_INT8 = 0, 1, 2
 ATBMI_PA_KERNEL_AUTO, ATBMI_PA_KERNEL_SCALAR, ATBMI_PA_KERNEL_MFMA = 0, 1, 2
+ATBMI_PA_MASK_ROW_SEQUENCE, ATBMI_PA_MASK_ROW_QUERY, ATBMI_PA_MASK_ROW_POSITION = 0, 1, 2
 
 
 class AtbCTensor(ctypes.Structure):
@@ -92,7 +93,7 @@ class AtbmiPaShape(ctypes.Structure):
         ("kernel", ctypes.c_int32), ("hasMask", ctypes.c_int32), ("qkScale", ctypes.c_float),
         ("qScale", ctypes.c_float), ("maskBatchStride", ctypes.c_int64), ("maskHeadStride", ctypes.c_int64),
         ("maskLen", ctypes.c_int32), ("hasLogN", ctypes.c_int32),
-        ("descalePacked", ctypes.c_int32), ("reserved", ctypes.c_int32),
+        ("descalePacked", ctypes.c_int32), ("maskRowBy", ctypes.c_int32), ("reserved", ctypes.c_int32),
     ]
 
 
@@ -127,6 +128,8 @@ def kernels():
         lib.atbmi_reshape_and_cache_quant.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]
         lib.atbmi_pa_plan_create.argtypes = [ctypes.POINTER(AtbmiPaShape), ctypes.POINTER(vp)]
         lib.atbmi_pa_plan_update.argtypes = [vp, vp, i32]
+        lib.atbmi_pa_plan_update_multi.argtypes = [vp, vp, vp, i32]
+        lib.atbmi_pa_plan_update_multi.restype = i32
         lib.atbmi_pa_plan_workspace_size.argtypes = [vp]
         lib.atbmi_pa_plan_workspace_size.restype = u64
         lib.atbmi_pa_plan_num_chunks.argtypes = [vp]

@@ -32,13 +32,13 @@ int Fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 // One physical work item of the split-K plan: the token range
 // [tokBegin, tokEnd) of one sequence, handled by one workgroup per KV head.
 struct PaWorkItem {
-    int32_t qRow;        // row of q / out this sequence uses
-    int32_t seq;         // row of blockTables
+    int32_t qRow;        // row of q / out
+    int32_t seq;         // row of blockTables (and of logN)
     int32_t tokBegin;
     int32_t tokEnd;
     int32_t partialBase; // first partial slot this item writes
     int32_t direct;      // 1: the only chunk of its sequence, write `out` directly
-    int32_t pad0;
+    int32_t maskRow;     // row of the mask (in units of maskBatchStride) this query row uses
     int32_t pad1;
 };
 
@@ -84,6 +84,7 @@ struct PaArgs {
     int32_t maskVec;     // 1: every mask row starts on an 8-byte boundary (4-token vector loads are legal)
     const float *logN;   // per batch row factor on qkScale (null: none)
     int32_t scaleStride; // floats between consecutive kScale / vScale entries: 1, or 2 for uint64-packed ones
+    int32_t maskRowStep; // mask rows between consecutive query tokens of one sequence (0: they share a row)
 };
 
 // ---- Plan of the MFMA kernel ------------------------------------------------
@@ -91,21 +92,29 @@ struct PaArgs {
 // linear step space [0, totalSteps). It is divided evenly into numWaveRanges
 // contiguous ranges; one wave walks one range for one KV head (or one tile of
 // 16 query heads of it), crossing sequence boundaries where they fall. The
-// device only needs where each sequence starts in that space.
-constexpr int PA_INLINE_SEQS = 192;   // plans up to this many sequences travel in the kernel arguments
+// device only needs where each sequence starts in that space. A sequence with
+// several query tokens appears once per token, each with the whole context.
+constexpr int PA_INLINE_SEQS = 160;   // plans up to this many query rows travel in the kernel arguments
 constexpr int PA_INLINE_RANGES = 512; // workgroup ranges whose first sequence is tabulated inline
 
+// One pass over a sequence's context: for its single decode token, or for up to
+// PaStreamPlan::foldTokens of its consecutive query tokens (speculative /
+// multi-token decoding), which share the pass as extra columns of the head tile.
+// A sequence with more query tokens than that appears once per such group.
 struct PaSeq {
-    int32_t tableRow;  // row of blockTables (index of the sequence in the batch)
+    int32_t tableRow;  // row of blockTables and of logN (index of the sequence in the batch)
     int32_t ctxLen;    // tokens
-    int32_t stepBegin; // first step of this sequence in the linear step space
+    int32_t stepBegin; // first step of this pass in the linear step space
+    int32_t maskRow;   // row of the mask (in units of maskBatchStride) of its first query token
+    int32_t qRow;      // row of q / out of its first query token
+    int32_t nTok;      // query tokens in this pass
 };
 
 struct PaStreamPlan {
     const PaSeq *seqs;        // numSeqs + 1 entries (the last one only carries stepBegin = totalSteps);
                               // null: use inlineSeqs
     const uint16_t *firstSeq; // per workgroup range: sequence holding its first step; null: use inlineFirst
-    int32_t numSeqs;          // non-empty sequences; the i-th one uses query/output row i
+    int32_t numSeqs;          // passes (PaSeq entries)
     int32_t totalSteps;
     int32_t numWaveRanges;    // numWgRanges * tokenSlices
     int32_t numWgRanges;
@@ -113,6 +122,8 @@ struct PaStreamPlan {
     int32_t headsPerWg;       // virtual heads (KV head x query-head tile) one workgroup covers
     int32_t headGroups;       // virtual heads / headsPerWg
     int32_t headTiles;        // query-head tiles per KV head
+    int32_t foldTokens;       // query tokens of one sequence that may share a head tile (1: none do);
+                              // a partial slot then holds foldTokens x H rows
     PaSeq inlineSeqs[PA_INLINE_SEQS + 1];
     uint16_t inlineFirst[PA_INLINE_RANGES];
 };

@@ -89,8 +89,11 @@ struct AtbmiPaPlan {
     int32_t batch = 0;
     int64_t totalCtx = 0;
     int64_t tableEntries = 0;
-    int32_t nonEmpty = 0;
+    int32_t nonEmpty = 0;    // query rows: one per non-empty sequence, or one per query token of it
     int32_t maxCtx = 0;
+    int64_t rowCtx = 0;      // sum over query rows of the context they attend to
+    int32_t maxQueryLen = 1; // most query tokens any sequence brings
+    std::vector<PaSeq> rows; // the query rows in query/output order (stepBegin unused here)
 
     uint64_t offItems = 0, offSeqs = 0, offPartO = 0, offPartLse = 0, blobBytes = 0, wsBytes = 0;
     std::vector<uint8_t> blob; // items then reduceSeqs, as uploaded
@@ -150,6 +153,9 @@ extern "C" int atbmi_pa_plan_create(const AtbmiPaShape *shape, AtbmiPaPlan **pla
     if (s.descalePacked && s.kvDtype != ATBMI_INT8) {
         return Fail(ERR_INVALID_PARAM, "pa_plan_create: packed descales only apply to an int8 cache");
     }
+    if (s.maskRowBy < ATBMI_PA_MASK_ROW_SEQUENCE || s.maskRowBy > ATBMI_PA_MASK_ROW_POSITION || s.reserved != 0) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: maskRowBy %d / reserved %d", s.maskRowBy, s.reserved);
+    }
     if (s.hasMask && (s.maskLen <= 0 || s.maskBatchStride < 0 || s.maskHeadStride < 0)) {
         return Fail(ERR_INVALID_PARAM, "pa_plan_create: mask row length %d, strides %lld / %lld", s.maskLen,
                     (long long)s.maskBatchStride, (long long)s.maskHeadStride);
@@ -193,7 +199,7 @@ namespace {
 
 // Stream plan of the MFMA kernel: every wave gets an equal share of the linear
 // step space (32-token steps of all non-empty sequences, back to back).
-int PlanStream(AtbmiPaPlan *plan, const int32_t *ctx, int32_t batch)
+int PlanStream(AtbmiPaPlan *plan)
 {
     const AtbmiPaShape &s = plan->shape;
     const int groupSize = s.numHeads / s.numKvHeads;
@@ -214,19 +220,28 @@ int PlanStream(AtbmiPaPlan *plan, const int32_t *ctx, int32_t batch)
         tokenSlices = 1;
     }
     const int headGroups = virtualHeads / headsPerWg;
+    // Several query tokens of one sequence share a pass over its context when a GQA group
+    // leaves columns of the 16-wide head tile free: 16 / group tokens per pass.
+    int fold = 1;
+    if (headTiles == 1 && !PaMlaWide(s) && plan->maxQueryLen > 1) {
+        fold = std::min(PA_MFMA_HEAD_TILE / groupSize, plan->maxQueryLen);
+    }
     try {
         plan->seqTable.clear();
         int64_t steps = 0;
-        for (int32_t b = 0; b < batch; ++b) {
-            if (ctx[b] == 0) {
-                continue;
+        for (size_t r = 0; r < plan->rows.size();) {
+            // consecutive rows of one sequence, `fold` at a time
+            size_t e = r + 1;
+            while (e < plan->rows.size() && e - r < static_cast<size_t>(fold) &&
+                   plan->rows[e].tableRow == plan->rows[r].tableRow) {
+                ++e;
             }
-            PaSeq sq{};
-            sq.tableRow = b;
-            sq.ctxLen = ctx[b];
+            PaSeq sq = plan->rows[r];
+            sq.nTok = static_cast<int32_t>(e - r);
             sq.stepBegin = static_cast<int32_t>(steps);
             plan->seqTable.push_back(sq);
-            steps += (ctx[b] + PA_MFMA_STEP - 1) / PA_MFMA_STEP;
+            steps += (sq.ctxLen + PA_MFMA_STEP - 1) / PA_MFMA_STEP;
+            r = e;
             if (steps > 0x3fffffff) {
                 return Fail(ERR_INVALID_PARAM, "pa_plan_update: too many KV tokens for one call");
             }
@@ -283,6 +298,7 @@ int PlanStream(AtbmiPaPlan *plan, const int32_t *ctx, int32_t batch)
         sp.headsPerWg = headsPerWg;
         sp.headGroups = headGroups;
         sp.headTiles = headTiles;
+        sp.foldTokens = fold;
         // firstSeq is a 16-bit table: batches beyond 65535 sequences go through memory as 16-bit too,
         // so they are refused here rather than silently truncated
         if (numSeqs > 0xffff) {
@@ -310,7 +326,8 @@ int PlanStream(AtbmiPaPlan *plan, const int32_t *ctx, int32_t batch)
     }
     plan->items.clear();
     plan->reduceSeqs.clear();
-    const uint64_t slots = plan->streamNeedsReduce ? 2ull * plan->stream.numWaveRanges : 0;
+    // a slot holds the partial rows of every query token of a pass
+    const uint64_t slots = plan->streamNeedsReduce ? 2ull * plan->stream.numWaveRanges * fold : 0;
     plan->numPartials = static_cast<int64_t>(slots);
     plan->offPartO = AlignUp(plan->blobBytes, WS_ALIGN);
     const uint64_t partOBytes = slots * s.numHeads * s.headDimV * sizeof(float);
@@ -326,6 +343,11 @@ int PlanStream(AtbmiPaPlan *plan, const int32_t *ctx, int32_t batch)
 
 extern "C" int atbmi_pa_plan_update(AtbmiPaPlan *plan, const int32_t *ctx, int32_t batch)
 {
+    return atbmi_pa_plan_update_multi(plan, ctx, nullptr, batch);
+}
+
+extern "C" int atbmi_pa_plan_update_multi(AtbmiPaPlan *plan, const int32_t *ctx, const int32_t *qLens, int32_t batch)
+{
     if (!plan || !ctx) {
         return Fail(ERR_INVALID_PARAM, "pa_plan_update: null argument");
     }
@@ -333,34 +355,64 @@ extern "C" int atbmi_pa_plan_update(AtbmiPaPlan *plan, const int32_t *ctx, int32
     if (batch <= 0) {
         return Fail(ERR_INVALID_PARAM, "pa_plan_update: batch %d", batch);
     }
-    int64_t total = 0, tableEntries = 0;
-    int32_t nonEmpty = 0;
+    int64_t total = 0, tableEntries = 0, rowCtx = 0;
+    int64_t nonEmpty = 0;
     const int64_t maxCtx = static_cast<int64_t>(s.maxBlocksPerSeq) * s.blockSize;
     for (int32_t b = 0; b < batch; ++b) {
         if (ctx[b] < 0 || ctx[b] > maxCtx) {
             return Fail(ERR_INVALID_PARAM, "pa_plan_update: contextLens[%d]=%d outside [0,%lld]", b, ctx[b],
                         (long long)maxCtx);
         }
-        if (ctx[b] > 0) {
-            ++nonEmpty;
+        if (qLens && (qLens[b] < 0 || (ctx[b] > 0 && qLens[b] > ctx[b]))) {
+            return Fail(ERR_INVALID_PARAM, "pa_plan_update: queryLens[%d]=%d outside [0, contextLens = %d]", b, qLens[b],
+                        ctx[b]);
+        }
+        const int32_t n = ctx[b] == 0 ? 0 : (qLens ? qLens[b] : 1);
+        if (n > 0) {
+            nonEmpty += n;
             total += ctx[b];
+            rowCtx += static_cast<int64_t>(n) * ctx[b];
             tableEntries += (ctx[b] + s.blockSize - 1) / s.blockSize;
         }
     }
     if (nonEmpty > s.numQueryRows) {
-        return Fail(ERR_INVALID_PARAM, "pa_plan_update: %d non-empty sequences but only %d query rows", nonEmpty,
-                    s.numQueryRows);
+        return Fail(ERR_INVALID_PARAM, "pa_plan_update: %lld query rows planned but the query holds %d",
+                    (long long)nonEmpty, s.numQueryRows);
+    }
+    try {
+        plan->rows.clear();
+        for (int32_t b = 0; b < batch; ++b) {
+            const int32_t n = ctx[b] == 0 ? 0 : (qLens ? qLens[b] : 1);
+            for (int32_t i = 0; i < n; ++i) {
+                PaSeq row{};
+                row.tableRow = b;
+                row.ctxLen = ctx[b];
+                row.nTok = 1;
+                const int32_t index = static_cast<int32_t>(plan->rows.size());
+                row.qRow = index;
+                row.maskRow = s.maskRowBy == ATBMI_PA_MASK_ROW_QUERY ? index
+                              : s.maskRowBy == ATBMI_PA_MASK_ROW_POSITION ? ctx[b] - n + i : b;
+                plan->rows.push_back(row);
+            }
+        }
+    } catch (const std::bad_alloc &) {
+        return Fail(ERR_OUT_OF_HOST_MEMORY, "pa_plan_update: out of host memory");
+    }
+    plan->rowCtx = rowCtx;
+    plan->maxQueryLen = 1;
+    for (int32_t b = 0; qLens && b < batch; ++b) {
+        plan->maxQueryLen = std::max(plan->maxQueryLen, ctx[b] > 0 ? qLens[b] : 0);
     }
     plan->batch = batch;
     plan->totalCtx = total;
     plan->tableEntries = tableEntries;
-    plan->nonEmpty = nonEmpty;
+    plan->nonEmpty = static_cast<int32_t>(nonEmpty);
     plan->maxCtx = *std::max_element(ctx, ctx + batch);
     plan->items.clear();
     plan->reduceSeqs.clear();
 
     if (plan->useMfma) {
-        return PlanStream(plan, ctx, batch);
+        return PlanStream(plan);
     }
 
     // Chunk length: enough workgroups to load every CU several times over,
@@ -373,7 +425,7 @@ extern "C" int atbmi_pa_plan_update(AtbmiPaPlan *plan, const int32_t *ctx, int32
     if (chunk <= 0) {
         const int64_t targetWgs = static_cast<int64_t>(NUM_CUS) * 8;
         const int64_t targetItems = std::max<int64_t>(1, targetWgs / wgPerItem);
-        chunk = (total + targetItems - 1) / std::max<int64_t>(1, targetItems);
+        chunk = (rowCtx + targetItems - 1) / std::max<int64_t>(1, targetItems);
         const int64_t minChunk = plan->useMfma ? 2 * unit : 64;
         chunk = std::min<int64_t>(std::max<int64_t>(chunk, minChunk), 4096);
     }
@@ -382,11 +434,8 @@ extern "C" int atbmi_pa_plan_update(AtbmiPaPlan *plan, const int32_t *ctx, int32
     int64_t partials = 0;
     int32_t qRow = 0;
     try {
-        for (int32_t b = 0; b < batch; ++b) {
-            const int64_t len = ctx[b];
-            if (len == 0) {
-                continue;
-            }
+        for (const PaSeq &row : plan->rows) {
+            const int64_t len = row.ctxLen;
             const int64_t n = (len + chunk - 1) / chunk;
             int64_t each = (len + n - 1) / n;
             each = (each + unit - 1) / unit * unit;
@@ -395,7 +444,8 @@ extern "C" int atbmi_pa_plan_update(AtbmiPaPlan *plan, const int32_t *ctx, int32
             for (int64_t i = 0; i * each < len; ++i) {
                 PaWorkItem it{};
                 it.qRow = qRow;
-                it.seq = b;
+                it.seq = row.tableRow;
+                it.maskRow = row.maskRow;
                 it.tokBegin = static_cast<int32_t>(i * each);
                 it.tokEnd = static_cast<int32_t>(std::min<int64_t>(len, (i + 1) * each));
                 it.direct = direct ? 1 : 0;
@@ -474,12 +524,15 @@ extern "C" uint64_t atbmi_pa_plan_algorithmic_bytes(const AtbmiPaPlan *plan)
     }
     if (s.hasMask) {
         // each distinct mask row once, over the tokens attended to
-        const uint64_t tokens = s.maskBatchStride ? static_cast<uint64_t>(plan->totalCtx)
+        const uint64_t tokens = s.maskBatchStride ? static_cast<uint64_t>(plan->rowCtx)
                                                   : static_cast<uint64_t>(plan->maxCtx);
         bytes += tokens * (s.maskHeadStride ? s.numHeads : 1) * 2;
     }
     if (s.hasLogN) {
         bytes += static_cast<uint64_t>(plan->batch) * 4;
+    }
+    if (plan->nonEmpty > 0 && plan->rows.size() > 0 && plan->rowCtx != plan->totalCtx) {
+        bytes += static_cast<uint64_t>(plan->batch) * 4; // the query lengths
     }
     return bytes;
 }
@@ -613,6 +666,7 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
     }
     a.logN = s.hasLogN ? t->logN : nullptr;
     a.scaleStride = s.descalePacked ? 2 : 1; // little endian: the low half of each uint64 comes first
+    a.maskRowStep = s.maskRowBy == ATBMI_PA_MASK_ROW_SEQUENCE ? 0 : 1;
 
     TimingRecord rec{nullptr, nullptr};
     bool timed = false;

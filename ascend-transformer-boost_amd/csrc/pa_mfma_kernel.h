@@ -205,7 +205,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
         return;
     }
     const int h0 = g * a.groupSize + ht * HT;
-    const int nh = min(HT, a.groupSize - ht * HT);
+    const int nhTile = min(HT, a.groupSize - ht * HT);
 
     unsigned char *kTile = SHARED ? smem : smem + wave * WaveLdsBytes<D, DV, MLA>();
     unsigned char *vTile = MLA ? kTile : kTile + K_TILE_BYTES;
@@ -232,21 +232,35 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
         const int tokBegin = (segBegin - sq.stepBegin) * STEP;
         const int tokEnd = min(sq.ctxLen, (segEnd - sq.stepBegin) * STEP);
         const bool complete = segBegin == sq.stepBegin && segEnd == seqEnd;
-        const int qRow = seqIdx; // the i-th non-empty sequence owns query/output row i
+        // Column n of the tile is head h0 + n of the pass's query token, or, when the plan folds
+        // several query tokens of a sequence into one tile (small GQA groups), head h0 + n % group
+        // of its query token n / group.
+        int nh = nhTile;
+        if (p.foldTokens > 1) {
+            nh = sq.nTok * a.groupSize;
+        }
+        const int nc = min(n, nh - 1); // columns past the tile's end borrow its last one where they must read
+        int colTok = 0, colHead = nc;
+        if (p.foldTokens > 1) {
+            colTok = nc / a.groupSize;
+            colHead = nc - colTok * a.groupSize;
+        }
+        const int qRow = sq.qRow + colTok;
         // SCALE_TYPE_LOGN: a per-sequence factor on the score scale, indexed like the block tables
         const float scaleSeq = a.logN ? scale2 * a.logN[sq.tableRow] : scale2;
-        // additive score bias of head n of this sequence (heads past the tile's end borrow its last one)
+        // additive score bias of this column's query token and head
         const uint16_t *maskRow = nullptr;
         if (a.mask) {
-            maskRow = reinterpret_cast<const uint16_t *>(a.mask) + static_cast<int64_t>(sq.tableRow) * a.maskBatchStride +
-                      static_cast<int64_t>(h0 + min(n, nh - 1)) * a.maskHeadStride;
+            maskRow = reinterpret_cast<const uint16_t *>(a.mask) +
+                      static_cast<int64_t>(sq.maskRow + colTok * a.maskRowStep) * a.maskBatchStride +
+                      static_cast<int64_t>(h0 + colHead) * a.maskHeadStride;
         }
 
-        // ---- Q^T as B operand: lane (n, kg) holds q[h0+n][32j + 8kg .. +8) for j < NQ
+        // ---- Q^T as B operand: lane (n, kg) holds q[column n][32j + 8kg .. +8) for j < NQ
         u32x4 qreg[NQ];
         {
             const uint16_t *qrow =
-                reinterpret_cast<const uint16_t *>(a.q) + (static_cast<int64_t>(qRow) * a.H + h0 + n) * D;
+                reinterpret_cast<const uint16_t *>(a.q) + (static_cast<int64_t>(qRow) * a.H + h0 + colHead) * D;
 #pragma unroll
             for (int j = 0; j < NQ; ++j) { // all loads first, so their latencies overlap
                 qreg[j] = u32x4{0u, 0u, 0u, 0u};
@@ -676,7 +690,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
         const float inv = l > 0.0f ? 1.0f / l : 0.0f; // l == 0: a -inf mask took every token out
         const float bias = KV8 ? INT8_BIAS : 0.0f; // see Int8x4ToHalf
         if (n < nh) {
-            const int h = h0 + n;
+            const int h = h0 + colHead;
             if (complete) {
                 uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) + (static_cast<int64_t>(qRow) * a.H + h) * DV;
 #pragma unroll
@@ -703,7 +717,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                 }
             } else {
                 const int slot = 2 * wr + (segBegin == s0 ? 0 : 1);
-                const int64_t ph = static_cast<int64_t>(slot) * a.H + h;
+                const int64_t ph = (static_cast<int64_t>(slot) * p.foldTokens + colTok) * a.H + h;
 #pragma unroll
                 for (int i = 0; i < NO; ++i) {
                     *reinterpret_cast<f32x4 *>(a.partO + ph * DV + i * 16 + kg * 4) = acc[i] * inv - bias;

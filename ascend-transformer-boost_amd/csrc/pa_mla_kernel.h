@@ -217,7 +217,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaWideKernel(const PaArgs a, cons
         const int tokBegin = (segBegin - sq.stepBegin) * STEP;
         const int tokEnd = min(sq.ctxLen, (segEnd - sq.stepBegin) * STEP);
         const bool complete = segBegin == sq.stepBegin && segEnd == seqEnd;
-        const int qRow = seqIdx; // the i-th non-empty sequence owns query/output row i
+        const int qRow = uniform(sq.qRow); // (128 heads fill the tile: a pass never holds a second query token)
 
         // ---- block ids of this segment sit in LDS (BLK_IDS at a time) and are read one tile ahead of
         // their use: the step loop then holds no memory instruction of the compiler's whose wait would

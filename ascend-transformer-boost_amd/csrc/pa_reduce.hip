@@ -64,9 +64,16 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaA
 {
     __shared__ float weight[REDUCE_THREADS];
     __shared__ float red[REDUCE_THREADS / WAVE];
-    const int b = blockIdx.x / a.H;
+    // one workgroup per (pass, query token of it, head); a slot holds foldTokens x H partial rows
+    const int rowsPerSlot = a.H * p.foldTokens;
+    const int b = blockIdx.x / rowsPerSlot;
+    const int tok = blockIdx.x % rowsPerSlot / a.H;
     const int h = blockIdx.x % a.H;
-    const int begin = (p.seqs ? p.seqs[b] : p.inlineSeqs[b]).stepBegin;
+    const PaSeq sq = p.seqs ? p.seqs[b] : p.inlineSeqs[b];
+    if (tok >= sq.nTok) {
+        return;
+    }
+    const int begin = sq.stepBegin;
     const int end = (p.seqs ? p.seqs[b + 1] : p.inlineSeqs[b + 1]).stepBegin;
     const int wrFirst = PaRangeOf(begin, p.totalSteps, p.numWaveRanges);
     const int wrLast = PaRangeOf(end - 1, p.totalSteps, p.numWaveRanges);
@@ -74,9 +81,10 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaA
         return;
     }
     const int firstOdd = PaRangeBegin(wrFirst, p.totalSteps, p.numWaveRanges) >= begin ? 0 : 1;
-    const int64_t stride = 2 * static_cast<int64_t>(a.H);
-    const int64_t phEven = 2 * static_cast<int64_t>(wrFirst) * a.H + h; // partial row of the k-th range, k >= 1
-    const int64_t ph0 = phEven + static_cast<int64_t>(firstOdd) * a.H;
+    const int64_t stride = 2 * static_cast<int64_t>(rowsPerSlot);
+    // partial row of the k-th range, k >= 1
+    const int64_t phEven = 2 * static_cast<int64_t>(wrFirst) * rowsPerSlot + static_cast<int64_t>(tok) * a.H + h;
+    const int64_t ph0 = phEven + static_cast<int64_t>(firstOdd) * rowsPerSlot;
     const int count = wrLast - wrFirst + 1;
     const int tid = threadIdx.x;
     auto rowOf = [&](int k) { return k == 0 ? ph0 : phEven + k * stride; };
@@ -151,7 +159,7 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaA
                 const int ch = g * a.Dv + d;
                 o = (o + (a.vOff ? static_cast<float>(a.vOff[ch]) : 0.0f)) * a.vScale[ch * a.scaleStride];
             }
-            Store16(a.out, (static_cast<int64_t>(b) * a.H + h) * a.Dv + d, o, bf16);
+            Store16(a.out, (static_cast<int64_t>(sq.qRow + tok) * a.H + h) * a.Dv + d, o, bf16);
         }
     }
 }
@@ -162,7 +170,7 @@ int LaunchPaStreamReduce(const AtbmiPaShape &shape, const PaArgs &args, const Pa
                          hipStream_t stream)
 {
     (void)shape;
-    const int64_t grid = static_cast<int64_t>(plan.numSeqs) * args.H;
+    const int64_t grid = static_cast<int64_t>(plan.numSeqs) * plan.foldTokens * args.H;
     if (grid <= 0) {
         return OK;
     }

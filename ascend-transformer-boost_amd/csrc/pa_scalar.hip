@@ -45,7 +45,7 @@ __global__ __launch_bounds__(PA_SCALAR_WAVES * WAVE) void PaScalarKernel(const P
     constexpr float LOG2E = 1.4426950408889634f;
     const float scale2 = a.qkScale * LOG2E * (a.logN ? a.logN[it.seq] : 1.0f);
     // additive score bias of this sequence and head tile (base-2 units once multiplied by LOG2E)
-    const int64_t maskRow = a.mask ? static_cast<int64_t>(it.seq) * a.maskBatchStride : 0;
+    const int64_t maskRow = a.mask ? static_cast<int64_t>(it.maskRow) * a.maskBatchStride : 0;
 
     float q[HT][EPL];
 #pragma unroll

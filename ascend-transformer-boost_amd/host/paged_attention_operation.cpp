@@ -11,13 +11,14 @@
 // Context lengths are read from contextLens.hostData during Setup, as the
 // reference runner does (src/ops/ops_infer/paged_attention/param.cpp:16-62).
 //
-// Implemented feature set: fp16/bf16 caches, int8 caches with fp32 per-channel
-// descale, plain or uint64-packed, (+ int32 offset), the MLA combined cache (mlaVHeadSize > 0), additive
-// NORM and ALIBI masks, the dynamic-batch status input and per-sequence LogN
-// scaling. Speculative (multi-token) queries with their masks, head
-// compression, BNSD layout and int8 queries are legal in the reference but not
-// implemented here; such params are rejected at creation with
-// ERROR_INVALID_PARAM.
+// Implemented feature set: fp16/bf16 caches; int8 caches with fp32 per-channel
+// descales, plain or uint64-packed, (+ int32 offsets); the MLA combined cache
+// (mlaVHeadSize > 0); additive NORM and ALIBI masks; the dynamic-batch status
+// input; per-sequence LogN scaling; several query tokens per sequence
+// (CALC_TYPE_SPEC) with the SPEC or the square NORM mask.
+// MASK_TYPE_MASK_FREE, head compression, BNSD layout and int8 queries are
+// legal in the reference but not implemented here; such params are rejected
+// at creation with ERROR_INVALID_PARAM.
 #include <cmath>
 #include <new>
 #include "atb/infer_op_params.h"
@@ -138,13 +139,12 @@ bool FeatureParamCheck(const Param &p)
 bool ImplementedCheck(const Param &p)
 {
     const char *what = nullptr;
-    if (p.maskType != Param::UNDEFINED && p.maskType != Param::MASK_TYPE_NORM &&
-        p.maskType != Param::MASK_TYPE_ALIBI) {
-        what = "SPEC and MASK_FREE masks";
+    if (p.maskType == Param::MASK_TYPE_MASK_FREE) {
+        what = "MASK_TYPE_MASK_FREE";
+    } else if (p.maskType == Param::MASK_TYPE_SPEC && p.calcType != Param::CALC_TYPE_SPEC) {
+        what = "MASK_TYPE_SPEC without CALC_TYPE_SPEC";
     } else if (p.compressType != Param::COMPRESS_TYPE_UNDEFINED) {
         what = "head compression";
-    } else if (p.calcType != Param::CALC_TYPE_UNDEFINED) {
-        what = "speculative (multi-token) queries";
     } else if (p.inputLayout != infer::TYPE_BSND) {
         what = "BNSD layout";
     } else if (p.quantType == Param::TYPE_QUANT_QKV_OFFLINE || p.quantType == Param::TYPE_QUANT_QKV_ONLINE) {
@@ -178,6 +178,9 @@ IrCombo MakeCombo(const Param &p, aclDataType q, aclDataType descale)
     }
     if (p.batchRunStatusEnable) {
         c.inDtypes.push_back(ACL_INT32);
+    }
+    if (p.calcType == Param::CALC_TYPE_SPEC) {
+        c.inDtypes.push_back(ACL_INT32); // qSeqLens; never together with the descales below
     }
     if (dequant) {
         c.inDtypes.push_back(descale);
@@ -225,6 +228,9 @@ public:
         }
         if (param.batchRunStatusEnable) {
             statusIdx_ = next++;
+        }
+        if (param.calcType == Param::CALC_TYPE_SPEC) {
+            qLensIdx_ = next++;
         }
         if (dequant_) {
             kScaleIdx_ = next++;
@@ -419,12 +425,27 @@ protected:
         int64_t maskBatchStride = 0;
         int64_t maskHeadStride = 0;
         int64_t maskLen = 0;
+        int32_t maskRowBy = ATBMI_PA_MASK_ROW_SEQUENCE;
         if (maskIdx_ != NONE) {
-            Status st = MaskLayout(pack.inTensors.at(maskIdx_).desc.shape, lens, maskBatchStride, maskHeadStride,
-                                   maskLen);
+            Status st = MaskLayout(pack.inTensors.at(maskIdx_).desc.shape, lens, q.desc.shape.dims[0], maskBatchStride,
+                                   maskHeadStride, maskLen, maskRowBy);
             if (st != NO_ERROR) {
                 return st;
             }
+        }
+        const int32_t *queryLens = nullptr;
+        if (qLensIdx_ != NONE) {
+            // reference param.cpp:96-110: the query lengths are read on the host, one per sequence
+            const Tensor &ql = pack.inTensors.at(qLensIdx_);
+            if (!ql.hostData) {
+                ATB_LOG(ERROR) << "qSeqLens.hostData is null";
+                return ERROR_INVALID_PARAM;
+            }
+            if (ql.desc.shape.dimNum != 1 || ql.desc.shape.dims[0] != lens.desc.shape.dims[0]) {
+                ATB_LOG(ERROR) << "qSeqLens should have one entry per sequence of contextLens";
+                return ERROR_INVALID_PARAM;
+            }
+            queryLens = static_cast<const int32_t *>(ql.hostData);
         }
 
         AtbmiPaShape shape{};
@@ -447,6 +468,7 @@ protected:
         shape.maskBatchStride = maskBatchStride;
         shape.maskHeadStride = maskHeadStride;
         shape.maskLen = static_cast<int32_t>(maskLen);
+        shape.maskRowBy = maskRowBy;
         shape.hasLogN = logNIdx_ != NONE ? 1 : 0;
         shape.descalePacked = (dequant_ && pack.inTensors.at(kScaleIdx_).desc.dtype == ACL_INT64) ? 1 : 0;
         if (!plan_ || !SameShape(shape, planShape_)) {
@@ -462,8 +484,8 @@ protected:
             planShape_ = shape;
         }
         // Lengths are re-read on every Setup, like the reference runner does.
-        int rc = atbmi_pa_plan_update(plan_, static_cast<const int32_t *>(lens.hostData),
-                                      static_cast<int32_t>(lens.desc.shape.dims[0]));
+        int rc = atbmi_pa_plan_update_multi(plan_, static_cast<const int32_t *>(lens.hostData), queryLens,
+                                            static_cast<int32_t>(lens.desc.shape.dims[0]));
         if (rc != 0) {
             ATB_LOG(ERROR) << "PagedAttention plan: " << atbmi_last_error();
             return rc;
@@ -511,7 +533,8 @@ private:
                a.numQueryRows == b.numQueryRows && a.mlaCombined == b.mlaCombined && a.hasOffset == b.hasOffset &&
                a.qkScale == b.qkScale && a.qScale == b.qScale && a.hasMask == b.hasMask &&
                a.maskBatchStride == b.maskBatchStride && a.maskHeadStride == b.maskHeadStride &&
-               a.maskLen == b.maskLen && a.hasLogN == b.hasLogN && a.descalePacked == b.descalePacked;
+               a.maskLen == b.maskLen && a.hasLogN == b.hasLogN && a.descalePacked == b.descalePacked &&
+               a.maskRowBy == b.maskRowBy;
     }
 
     // Element strides of the additive mask, as the reference derives them from
@@ -524,14 +547,34 @@ private:
     // through shapes with more than one query row, which its stride rules then
     // ignore, and a 4-dim NORM mask, for which it derives no strides at all; those
     // are refused here rather than read with strides that do not fit them.
-    Status MaskLayout(const Dims &m, const Tensor &lens, int64_t &batchStride, int64_t &headStride,
-                      int64_t &maskLen) const
+    //
+    // With several query tokens per sequence (CALC_TYPE_SPEC; reference
+    // tiling/paged_attention_tiling_dependency.cpp:557-569): MASK_TYPE_SPEC is
+    // (query rows, maxS), one row per query token; MASK_TYPE_NORM is the square
+    // causal (maxS, maxS), of which the i-th query token of a sequence uses row
+    // contextLen - queryLen + i. Other NORM shapes are refused under
+    // CALC_TYPE_SPEC: the reference would step from a sequence's row into its
+    // neighbour's for the second query token.
+    Status MaskLayout(const Dims &m, const Tensor &lens, int64_t queryRows, int64_t &batchStride,
+                      int64_t &headStride, int64_t &maskLen, int32_t &rowBy) const
     {
         const int64_t batch = lens.desc.shape.dims[0];
         const int64_t heads = param_.headNum;
         const bool alibi = param_.maskType == Param::MASK_TYPE_ALIBI;
+        const bool multi = param_.calcType == Param::CALC_TYPE_SPEC;
         bool ok = false;
-        if (!alibi && m.dimNum == 2) {
+        rowBy = ATBMI_PA_MASK_ROW_SEQUENCE;
+        if (multi) {
+            if (m.dimNum == 2 && param_.maskType == Param::MASK_TYPE_SPEC) {
+                ok = m.dims[0] == queryRows;
+                rowBy = ATBMI_PA_MASK_ROW_QUERY;
+            } else if (m.dimNum == 2 && param_.maskType == Param::MASK_TYPE_NORM) {
+                ok = m.dims[0] == m.dims[1];
+                rowBy = ATBMI_PA_MASK_ROW_POSITION;
+            }
+            batchStride = m.dimNum == 2 ? m.dims[1] : 0;
+            headStride = 0;
+        } else if (!alibi && m.dimNum == 2) {
             ok = m.dims[0] == 1;
             batchStride = 0;
             headStride = 0;
@@ -550,7 +593,8 @@ private:
         }
         if (!ok) {
             ATB_LOG(ERROR) << "mask shape is not one of NORM (1,maxS) / (batch,1,maxS), "
-                              "ALIBI (heads,1,maxS) / (batch,1|heads,1,maxS)";
+                              "ALIBI (heads,1,maxS) / (batch,1|heads,1,maxS), or with CALC_TYPE_SPEC "
+                              "SPEC (query rows,maxS) / NORM (maxS,maxS)";
             return ERROR_INVALID_PARAM;
         }
         maskLen = m.dims[m.dimNum - 1];
@@ -573,8 +617,10 @@ private:
             return ERROR_INVALID_TENSOR_DIM;
         }
         const int64_t blockSize = in.at(1).shape.dims[1];
-        if (dequant_) {
-            // strict regime: features that predate the split K/V head sizes
+        const bool strict = dequant_ || (param_.calcType == Param::CALC_TYPE_SPEC && !mla_) ||
+                            param_.scaleType == Param::SCALE_TYPE_LOGN;
+        if (strict) {
+            // strict regime (reference :561-572): features that predate the split K/V head sizes
             if (d != in.at(2).shape.dims[3]) {
                 ATB_LOG(ERROR) << "headSize of keyCache and valueCache should be same";
                 return ERROR_INVALID_TENSOR_DIM;
@@ -599,7 +645,8 @@ private:
             return ERROR_INVALID_TENSOR_DIM;
         }
         const bool blockSize256 = mla_ && blockSize == 256 && param_.kvHeadNum == 1 &&
-                                  (param_.headNum == 16 || param_.headNum == 32) && d == 576 && dv == 512;
+                                  (param_.headNum == 16 || param_.headNum == 32) && d == 576 && dv == 512 &&
+                                  param_.calcType != Param::CALC_TYPE_SPEC;
         if (blockSize256) {
             return NO_ERROR;
         }
@@ -624,6 +671,7 @@ private:
     size_t vScaleIdx_ = NONE;
     size_t vOffsetIdx_ = NONE;
     size_t logNIdx_ = NONE;
+    size_t qLensIdx_ = NONE;
     uint32_t inputNum_ = 5;
     AtbmiPaPlan *plan_ = nullptr;
     AtbmiPaShape planShape_{};

@@ -25,6 +25,10 @@ CONFIGS = {
                      kv="bf16", dist="uniform", std=0.5, pool=None, mask="alibi"),
     "c2_norm": dict(batch=64, heads=32, kv_heads=8, d=128, dv=128, block=128, ctx=(1024, 4096), dtype="bf16",
                     kv="bf16", dist="uniform", std=0.5, pool=None, mask="norm"),
+    # C2 as a multi-token (speculative / MTP) decode step: 4 query tokens per sequence, the last 4
+    # positions of its context, with the per-query-row causal mask of the reference's tests
+    "c2_mtp4": dict(batch=64, heads=32, kv_heads=8, d=128, dv=128, block=128, ctx=(1024, 4096), dtype="bf16",
+                    kv="bf16", dist="uniform", std=0.5, pool=None, mask="spec", q_len=4),
     "c3": dict(batch=128, heads=64, kv_heads=8, d=128, dv=128, block=128, ctx=(2048, 8192), dtype="float16",
                kv="int8", dist="uniform", std=1.0, pool=None),
     "c4": dict(batch=16, heads=32, kv_heads=8, d=128, dv=128, block=128, ctx=(256, 32768), dtype="float16",
@@ -32,7 +36,7 @@ CONFIGS = {
     "c5": dict(batch=64, heads=128, kv_heads=1, d=576, dv=512, block=128, ctx=(2048, 4096), dtype="bf16",
                kv="bf16", dist="uniform", std=0.3, pool=None, mla=True),
 }
-SEEDS = {"c1": 1001, "c2": 1002, "c2_fp16": 1002, "c2_alibi": 1002, "c2_norm": 1002, "c3": 1003, "c4": 1004, "c5": 1005}
+SEEDS = {"c1": 1001, "c2": 1002, "c2_fp16": 1002, "c2_alibi": 1002, "c2_norm": 1002, "c2_mtp4": 1002, "c3": 1003, "c4": 1004, "c5": 1005}
 
 
 def config(name, **overrides):
@@ -75,9 +79,13 @@ def layout(cfg, seed=None):
         tables[b, :n] = perm[pos:pos + n]
         tables[b, n:] = perm[pos]  # unused entries stay valid block ids
         pos += n
-    last = ctx.astype(np.int64) - 1
-    slots = (tables[np.arange(cfg["batch"]), last // bs].astype(np.int64) * bs + last % bs).astype(np.int32)
-    return dict(ctx=ctx, tables=tables, slots=slots, pool=pool, max_blocks=max_blocks)
+    # the new tokens are the last q_len positions of each context (one for a plain decode step)
+    n = int(cfg.get("q_len", 1))
+    pos = (ctx.astype(np.int64)[:, None] - n + np.arange(n)[None, :]).reshape(-1)
+    seq = np.repeat(np.arange(cfg["batch"]), n)
+    slots = (tables[seq, pos // bs].astype(np.int64) * bs + pos % bs).astype(np.int32)
+    return dict(ctx=ctx, tables=tables, slots=slots, pool=pool, max_blocks=max_blocks,
+                q_lens=np.full(cfg["batch"], n, dtype=np.int32))
 
 
 def torch_dtype(name):
@@ -97,7 +105,9 @@ def make_mask(cfg, ctx, device):
     """The additive mask of a masked workload, in the query dtype, rows padded to a
     multiple of the block size. "alibi": [batch, heads, 1, maxS], slope_h * (j - ctx_i + 1)
     on the valid positions (reference :489-499); "norm": [batch, 1, maxS], -10000 on the
-    first i positions of sequence i (reference :501-505)."""
+    first i positions of sequence i (reference :501-505); "spec": [batch * q_len, maxS], for
+    the t-th query token of a sequence -10000 on the q_len - 1 - t positions after its own
+    (reference tests/apitest/kernelstest/mix/test_paged_attention_mla_mtp.py:220-231)."""
     import torch
     bs = cfg["block"]
     max_s = (int(max(ctx)) + bs - 1) // bs * bs
@@ -108,6 +118,13 @@ def make_mask(cfg, ctx, device):
         dist = pos[None, :] - lens[:, None] + 1.0                       # [batch, maxS]
         m = slopes[None, :, None] * torch.where(dist <= 0, dist, torch.zeros_like(dist))[:, None, :]
         return m[:, :, None, :].to(torch_dtype(cfg["dtype"])).contiguous()
+    if cfg["mask"] == "spec":
+        n = int(cfg["q_len"])
+        own = (lens[:, None] - n + torch.arange(n, device=device, dtype=torch.float32)[None, :]).reshape(-1, 1)
+        end = lens.repeat_interleave(n)[:, None]
+        hidden = (pos[None, :] > own) & (pos[None, :] < end)
+        m = torch.where(hidden, torch.full((1, 1), -10000.0, device=device), torch.zeros((1, 1), device=device))
+        return m.to(torch_dtype(cfg["dtype"])).contiguous()
     row = torch.arange(len(ctx), device=device, dtype=torch.float32)
     m = torch.where(pos[None, :] < row[:, None], torch.full((1, 1), -10000.0, device=device),
                     torch.zeros((1, 1), device=device))
@@ -118,14 +135,15 @@ def make_step(cfg, device, seed=None):
     """Tensors of one decode step on `device` (torch). Returns a dict:
     q, k_new, v_new (query dtype), key_cache, value_cache (kv dtype; value_cache
     is None for MLA), k_scale/v_scale (fp32, int8 caches only), block_tables,
-    slot_mapping (int32, device), context_lens (int32, CPU), mask (query dtype, or
-    None) and cfg/layout."""
+    slot_mapping (int32, device), context_lens and q_lens (int32, CPU), mask (query
+    dtype, or None) and cfg/layout."""
     import torch
     lay = layout(cfg, seed)
     gen = torch.Generator(device=device)
     gen.manual_seed(SEEDS.get(cfg["name"], 1) if seed is None else seed)
     qdt = torch_dtype(cfg["dtype"])
     b, h, g, d, dv, bs = cfg["batch"], cfg["heads"], cfg["kv_heads"], cfg["d"], cfg["dv"], cfg["block"]
+    b *= int(cfg.get("q_len", 1))  # query / new K,V rows: one per query token
     pool = lay["pool"]
     std = cfg["std"]
 
@@ -165,22 +183,27 @@ def make_step(cfg, device, seed=None):
     out["slot_mapping"] = torch.from_numpy(lay["slots"]).to(device)
     out["context_lens"] = torch.from_numpy(lay["ctx"].copy())
     out["mask"] = make_mask(cfg, lay["ctx"], device) if cfg.get("mask") else None
+    out["q_lens"] = torch.from_numpy(lay["q_lens"].copy())
     return out
 
 
 def algorithmic_bytes(cfg, ctx):
     """HBM bytes a decode-attention call must move: valid K/V rows + q + out +
     block-table entries + context lengths (+ scale vectors for an int8 cache, + the
-    mask rows over the valid positions)."""
+    mask rows over the valid positions). With several query tokens per sequence K and V
+    still count once per sequence; q, out and the mask count per query row."""
     kv = 1 if cfg["kv"] == "int8" else 2
     g, d, dv, h, bs = cfg["kv_heads"], cfg["d"], cfg["dv"], cfg["heads"], cfg["block"]
     ctx = np.asarray(ctx, dtype=np.int64)
     per_tok = g * (d if cfg.get("mla") else d + dv) * kv
-    rows = int((ctx > 0).sum())
+    n = int(cfg.get("q_len", 1))
+    rows = int((ctx > 0).sum()) * n
     total = int(ctx.sum()) * per_tok + rows * h * (d + dv) * 2
     total += int(((ctx + bs - 1) // bs).sum()) * 4 + len(ctx) * 4
     if cfg["kv"] == "int8":
         total += g * (d + dv) * 4
     if cfg.get("mask"):
-        total += int(ctx.sum()) * (h if cfg["mask"] == "alibi" else 1) * 2
+        total += int(ctx.sum()) * n * (h if cfg["mask"] == "alibi" else 1) * 2
+    if n > 1:
+        total += len(ctx) * 4  # the query lengths
     return total

@@ -38,6 +38,8 @@ DESCRIPTIONS = {
                 "ctx U[1024,4096], bf16",
     "c2_norm": "C2 with a NORM mask [batch, 1, maxS]: batch 64, 32 q heads, 8 kv heads, d128, block 128, "
                "ctx U[1024,4096], bf16",
+    "c2_mtp4": "C2 with 4 query tokens per sequence (CALC_TYPE_SPEC, MASK_TYPE_SPEC mask [256, maxS]): batch 64, "
+               "32 q heads, 8 kv heads, d128, block 128, ctx U[1024,4096], bf16",
     "c3": "C3 int8-KV 70B-shaped decode: batch 128, 64 q heads, 8 kv heads, d128, block 128, ctx U[2048,8192], fp16 q",
     "c4": "C4 skewed long-context fp16 decode: batch 16, 32 q heads, 8 kv heads, d128, ctx lognormal(median 8k) in [256,32768]",
     "c5": "C5 MLA bf16 decode: batch 64, 128 q heads, 1 latent kv head, d576/dv512, block 128, ctx U[2048,4096]",
@@ -66,6 +68,7 @@ def cpu_baseline(pkg, step, cfg, scale, budget_s=10.0):
     vs = vs.cpu().numpy() if vs is not None else None
     mask = step["mask"].float().cpu().numpy() if step.get("mask") is not None else None
     done, spent, tokens = 0, 0.0, 0
+    q_len = int(cfg.get("q_len", 1))
     import torch
     b = 0
     while spent < budget_s:  # cycles over the batch until the budget is spent
@@ -78,14 +81,16 @@ def cpu_baseline(pkg, step, cfg, scale, budget_s=10.0):
         kb = kb.numpy() if kb.dtype == torch.int8 else kb.float().numpy()
         if vb is not None:
             vb = vb.numpy() if vb.dtype == torch.int8 else vb.float().numpy()
-        q = dev_q[b:b + 1].float().cpu().numpy()
+        q = dev_q[b * q_len:(b + 1) * q_len].float().cpu().numpy()
         local = np.arange(nblk, dtype=np.int32)[None, :]
+        rows_mask = None if mask is None else (mask[b * q_len:(b + 1) * q_len] if q_len > 1 else mask[b:b + 1])
         t0 = time.perf_counter()
         oracle.paged_attention(q, kb, vb, local, np.array([n]), scale, ks, None, vs, None,
-                               mla_v_head_size=cfg["dv"] if cfg.get("mla") else 0,
-                               mask=None if mask is None else mask[b:b + 1], mask_per_head=False)
+                               mla_v_head_size=cfg["dv"] if cfg.get("mla") else 0, mask=rows_mask,
+                               mask_per_head=False, q_lens=np.array([q_len]) if q_len > 1 else None,
+                               mask_rows="query" if q_len > 1 else "sequence")
         spent += time.perf_counter() - t0
-        done += 1
+        done += q_len
         tokens += n
         b = (b + 1) % len(ctx)
     return {
@@ -93,8 +98,8 @@ def cpu_baseline(pkg, step, cfg, scale, budget_s=10.0):
         "unit": "tokens/s",
         "cores": threads,
         "kind": "port",
-        "sample": "numpy oracle on %d sequences drawn in order from the batch of %d (%d context tokens), "
-                  "attention only, %.1f s" % (done, len(ctx), tokens, spent),
+        "sample": "numpy oracle on %d query tokens of sequences drawn in order from the batch of %d "
+                  "(%d context tokens), attention only, %.1f s" % (done, len(ctx), tokens, spent),
     }
 
 
@@ -127,14 +132,17 @@ def main():
     int8 = cfg["kv"] == "int8"
     mla = bool(cfg.get("mla"))
 
-    mask_type = {None: 0, "norm": 1, "alibi": 2}[cfg.get("mask")]
+    mask_type = {None: 0, "norm": 1, "alibi": 2, "spec": 3}[cfg.get("mask")]
+    q_len = int(cfg.get("q_len", 1))
+    rows = cfg["batch"] * q_len  # query tokens of one step
     pa_param = b.PagedAttentionParam(headNum=cfg["heads"], kvHeadNum=cfg["kv_heads"], qkScale=scale,
                                      quantType=1 if int8 else 0, mlaVHeadSize=cfg["dv"] if mla else 0,
-                                     maskType=mask_type)
+                                     maskType=mask_type, calcType=1 if q_len > 1 else 0)
     pa = b.OperationRunner("PagedAttentionOperation", pa_param, ctx)
     rac = None
     k = b.kernels()
     lens_host = step["context_lens"]
+    host_inputs = {}
     with torch.cuda.stream(stream):
         lens_dev = lens_host.to(dev)
         if mla:
@@ -148,13 +156,17 @@ def main():
             host_idx = 4
             if mask_type:
                 pa_in.append(step["mask"])
+            if q_len > 1:
+                host_inputs[len(pa_in)] = step["q_lens"]
+                pa_in.append(step["q_lens"].to(dev))
             if int8:
                 pa_in += [step["k_scale"], step["v_scale"]]
             else:
                 rac = b.OperationRunner("ReshapeAndCacheOperation", b.ReshapeAndCacheParam(), ctx)
                 rac_in = [step["k_new"], step["v_new"], step["key_cache"], step["value_cache"], step["slot_mapping"]]
                 rac_out = [step["key_cache"], step["value_cache"]]
-        out = torch.empty((cfg["batch"], cfg["heads"], cfg["dv"]), dtype=step["q"].dtype, device=dev)
+        host_inputs[host_idx] = lens_host
+        out = torch.empty((rows, cfg["heads"], cfg["dv"]), dtype=step["q"].dtype, device=dev)
     slots = cfg["block"] * step["layout"]["pool"]
 
     def one_step():
@@ -164,12 +176,12 @@ def main():
                 rc = k.atbmi_reshape_and_cache_quant(
                     step["k_new"].data_ptr(), step["v_new"].data_ptr(), b.ATBMI_F16, step["k_scale"].data_ptr(),
                     step["v_scale"].data_ptr(), step["key_cache"].data_ptr(), step["value_cache"].data_ptr(),
-                    step["slot_mapping"].data_ptr(), cfg["batch"], cfg["kv_heads"], cfg["d"], cfg["dv"], slots,
+                    step["slot_mapping"].data_ptr(), rows, cfg["kv_heads"], cfg["d"], cfg["dv"], slots,
                     stream.cuda_stream)
                 assert rc == 0, b.last_kernel_error()
             else:
                 rac.run(rac_in, outputs=rac_out)
-        pa.run(pa_in, outputs=[out], host_inputs={host_idx: lens_host})
+        pa.run(pa_in, outputs=[out], host_inputs=host_inputs)
 
     if args.calibrate_copy:
         with torch.cuda.stream(stream):
@@ -202,7 +214,7 @@ def main():
     achieved = alg_bytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
     result = {
         "metric": "paged_attention_decode_tokens_per_s",
-        "value": cfg["batch"] / (ms_per_step * 1e-3),
+        "value": rows / (ms_per_step * 1e-3),
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,

@@ -88,6 +88,18 @@ int atbmi_reshape_and_cache_quant(const void *keyDevice, const void *valueDevice
                                   void *stream);
 
 /* Static description of a paged decode-attention problem. */
+/* Row of the mask a query row uses, in units of maskBatchStride
+ * (reference tiling/paged_attention_tiling_dependency.cpp:557-569, GetLookaheadMaskOffset):
+ *   SEQUENCE  the index of its sequence in hostContextLens (one-token decode: NORM / ALIBI masks)
+ *   QUERY     its own index among the query rows (MASK_TYPE_SPEC: mask [numQueryRows, maxLen])
+ *   POSITION  its position in the sequence, contextLen - queryLen + i for the i-th query token
+ *             (a square causal NORM mask [maxLen, maxLen] under CALC_TYPE_SPEC) */
+typedef enum AtbmiPaMaskRow {
+    ATBMI_PA_MASK_ROW_SEQUENCE = 0,
+    ATBMI_PA_MASK_ROW_QUERY = 1,
+    ATBMI_PA_MASK_ROW_POSITION = 2
+} AtbmiPaMaskRow;
+
 typedef struct AtbmiPaShape {
     int32_t qDtype;          /* ATBMI_F16 or ATBMI_BF16; the output has the same type */
     int32_t kvDtype;         /* ATBMI_F16 / ATBMI_BF16 (== qDtype) or ATBMI_INT8 */
@@ -111,6 +123,7 @@ typedef struct AtbmiPaShape {
     int32_t hasLogN;         /* 1: a per-sequence factor on qkScale (AtbmiPaTensors.logN) is given */
     int32_t descalePacked;   /* 1: kScale / vScale are uint64 arrays whose low 32 bits hold the fp32 value,
                                 as atb::Utils::QuantParamConvert packs them (reference src/atb/utils/utils.cpp:153-164) */
+    int32_t maskRowBy;       /* AtbmiPaMaskRow: which mask row (in units of maskBatchStride) a query row uses */
     int32_t reserved;        /* 0 */
 } AtbmiPaShape;
 
@@ -154,6 +167,16 @@ int atbmi_pa_plan_create(const AtbmiPaShape *shape, AtbmiPaPlan **plan);
  * 0 is skipped and takes no query row: query/out row index = number of
  * non-empty sequences before it. Host only, O(batch + chunks). */
 int atbmi_pa_plan_update(AtbmiPaPlan *plan, const int32_t *hostContextLens, int32_t batch);
+
+/* The same with several query tokens per sequence (CALC_TYPE_SPEC: speculative / multi-token decoding;
+ * replaces the qSeqLen handling of the reference, src/ops/ops_infer/paged_attention/param.cpp:39-62 and
+ * tiling/paged_attention_tiling_dependency.cpp:580-620). Sequence b brings hostQueryLens[b] consecutive
+ * query rows (0 <= hostQueryLens[b] <= hostContextLens[b]; none when its context length is 0), each of
+ * which attends to all hostContextLens[b] tokens: which of them a row may see is the mask's business
+ * (AtbmiPaShape.maskRowBy). hostQueryLens == NULL means one row per sequence. Up to 16 / (numHeads /
+ * numKvHeads) query tokens of a sequence share one pass over its K and V rows. */
+int atbmi_pa_plan_update_multi(AtbmiPaPlan *plan, const int32_t *hostContextLens, const int32_t *hostQueryLens,
+                               int32_t batch);
 
 /* Device workspace bytes atbmi_pa_decode needs for the current plan. */
 uint64_t atbmi_pa_plan_workspace_size(const AtbmiPaPlan *plan);

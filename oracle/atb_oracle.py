@@ -23,6 +23,18 @@ the invariants of the mathematics (no function is left "parity unpinned"):
                       sequence i; :353-358 a 4-dim mask is sliced [i, :, :, :ctx], a 3-dim one
                       [i, :, :ctx], with i the index into context_lens); :74-83 (ALiBi slopes),
                       :488-505 (the masks the reference tests feed);
+                      several query tokens per sequence (calcType SPEC): tests/apitest/opstest/python/
+                      operations/paged_attention/test_paged_attention_operation_parallel_decoding_910B.py:
+                      75-121 (sequence i owns q_lens[i] consecutive query rows, every one attends to
+                      all k_lens[i] tokens; mask rows [k - q : k] of the square causal mask, or rows
+                      [cu : cu + q] of the per-query-row mask), tests/apitest/kernelstest/mix/
+                      test_paged_attention_mla_mtp.py:120-166 (the same for the MLA cache, fp32 branch);
+                      several query tokens per sequence (calcType SPEC): tests/apitest/opstest/python/
+                      operations/paged_attention/test_paged_attention_operation_parallel_decoding_910B.py:
+                      75-121 (sequence i owns q_lens[i] consecutive query rows, every one attends to
+                      all k_lens[i] tokens; mask rows [k - q : k] of the square causal mask, or rows
+                      [cu : cu + q] of the per-query-row mask), tests/apitest/kernelstest/mix/
+                      test_paged_attention_mla_mtp.py:120-166 (the same for the MLA cache, fp32 branch);
                       MLA: tests/apitest/opstest/python/operations/paged_attention/
                       test_paged_attention_operation_mla.py:229-262 (V = K[..., :head_size_vo])
   merge_partials      src/kernels/mixkernels/pagedattention/op_kernel/
@@ -177,7 +189,8 @@ def norm_mask(batch, max_len, value=-10000.0):
 
 def paged_attention(query, key_cache, value_cache, block_tables, context_lens, scale, k_descale=None,
                     k_offset=None, v_descale=None, v_offset=None, mla_v_head_size=0, q_scale=0.0,
-                    q_dtype="float32", out_init=0.0, mask=None, logn=None, mask_per_head=None):
+                    q_dtype="float32", out_init=0.0, mask=None, logn=None, mask_per_head=None, q_lens=None,
+                    mask_rows="sequence"):
     """Decode attention over paged caches.
 
     query [rows, heads, D] float32; key_cache [blocks, block, kv_heads, D];
@@ -192,7 +205,13 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, s
     [batch, heads | 1, 1, max_len] is sliced [i, :, 0, :ctx], a 3-dim mask whose
     first dim is the batch [i, 0, :ctx] for every head, a 3-dim mask
     [heads, 1, max_len] (mask_per_head=True, or left to its size when heads !=
-    batch), or a 2-dim [1, max_len] one, is shared by all sequences. logn [batch] multiplies the scale of sequence i.
+    batch), or a 2-dim [1, max_len] one, is shared by all sequences.
+    logn [batch] multiplies the scale of sequence i.
+    q_lens [batch] gives sequence i that many consecutive query rows (none when
+    its context is empty), each attending to all context_lens[i] tokens; the
+    2-dim mask then has one row per query row (mask_rows="query") or is the
+    square causal mask, of which the t-th query token of a sequence with n of
+    them uses row ctx - n + t (mask_rows="position").
     Returns float32 [rows, heads, Dv]."""
     query = np.asarray(query, dtype=np.float32)
     if mla_v_head_size > 0:
@@ -208,16 +227,23 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, s
             continue
         keys = gather_rows(key_cache, block_tables[i], ctx)
         values = keys[..., :dv] if mla_v_head_size > 0 else gather_rows(value_cache, block_tables[i], ctx)
-        bias = None if mask is None else mask_rows(mask, i, ctx, query.shape[1], len(context_lens),
-                                                      mask_per_head)
         seq_scale = np.float32(scale) if logn is None else np.float32(scale) * np.float32(logn[i])
-        out[row] = attention_one(query[row], keys, values, seq_scale, k_descale, k_offset, v_descale, v_offset,
-                                 bias)
-        row += 1
+        for t in range(1 if q_lens is None else int(q_lens[i])):
+            if mask is None:
+                bias = None
+            elif mask_rows == "query":
+                bias = np.asarray(mask, dtype=np.float32)[row:row + 1, :ctx]
+            elif mask_rows == "position":
+                bias = np.asarray(mask, dtype=np.float32)[ctx - int(q_lens[i]) + t][None, :ctx]
+            else:
+                bias = _mask_slice(mask, i, ctx, query.shape[1], len(context_lens), mask_per_head)
+            out[row] = attention_one(query[row], keys, values, seq_scale, k_descale, k_offset, v_descale,
+                                     v_offset, bias)
+            row += 1
     return out
 
 
-def mask_rows(mask, i, ctx, heads, batch, per_head=None):
+def _mask_slice(mask, i, ctx, heads, batch, per_head=None):
     """The [heads | 1, ctx] slice of `mask` that sequence i sees (see paged_attention).
     per_head says whether a 3-dim mask's first dim counts heads (ALIBI) or
     sequences (NORM); None decides by its size and refuses the ambiguous case."""

@@ -22,7 +22,7 @@ def dtype_code(binding, t):
 
 def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=None, v_scale=None,
                    v_off=None, mla_dv=0, q_scale=0.0, kernel=0, chunk_tokens=None, out=None, return_plan_info=False,
-                   mask=None, mask_per_head=False, logn=None):
+                   mask=None, mask_per_head=False, logn=None, q_lens=None, mask_rows="sequence"):
     """atbmi_pa_plan_* + atbmi_pa_decode on `stream`; returns the output tensor.
     mask: device tensor of q's dtype shaped like one of the reference's decode
     masks; mask_per_head says that a 3-dim mask's first dim counts heads (ALIBI)."""
@@ -30,6 +30,8 @@ def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=
     rows, heads, d = q.shape
     dv = mla_dv if mla_dv else vc.shape[3]
     mask_batch_stride, mask_head_stride = mask_strides(mask, mask_per_head)
+    if mask_rows != "sequence":
+        mask_batch_stride, mask_head_stride = (mask.shape[1], 0) if mask is not None else (0, 0)
     shape = binding.AtbmiPaShape(
         qDtype=dtype_code(binding, q), kvDtype=dtype_code(binding, kc), numHeads=heads, numKvHeads=kc.shape[2],
         headDimK=d, headDimV=dv, blockSize=kc.shape[1], numBlocks=kc.shape[0], maxBlocksPerSeq=tables.shape[1],
@@ -37,7 +39,8 @@ def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=
         qkScale=scale, qScale=q_scale, hasMask=0 if mask is None else 1, maskBatchStride=mask_batch_stride,
         maskHeadStride=mask_head_stride, maskLen=0 if mask is None else mask.shape[-1],
         hasLogN=0 if logn is None else 1,
-        descalePacked=1 if (k_scale is not None and k_scale.dtype == torch.int64) else 0)
+        descalePacked=1 if (k_scale is not None and k_scale.dtype == torch.int64) else 0,
+        maskRowBy={"sequence": 0, "query": 1, "position": 2}[mask_rows])
     old = os.environ.get("ATBMI_PA_CHUNK_TOKENS")
     if chunk_tokens is not None:
         os.environ["ATBMI_PA_CHUNK_TOKENS"] = str(chunk_tokens)
@@ -54,7 +57,11 @@ def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=
         raise RuntimeError("plan_create: " + binding.last_kernel_error())
     try:
         lens = np.ascontiguousarray(np.asarray(ctx_host, dtype=np.int32))
-        rc = k.atbmi_pa_plan_update(plan, lens.ctypes.data, len(lens))
+        if q_lens is None:
+            rc = k.atbmi_pa_plan_update(plan, lens.ctypes.data, len(lens))
+        else:
+            qn = np.ascontiguousarray(np.asarray(q_lens, dtype=np.int32))
+            rc = k.atbmi_pa_plan_update_multi(plan, lens.ctypes.data, qn.ctypes.data, len(lens))
         if rc != 0:
             raise RuntimeError("plan_update: " + binding.last_kernel_error())
         ws_bytes = k.atbmi_pa_plan_workspace_size(plan)
@@ -98,7 +105,6 @@ def mask_strides(mask, per_head):
         return 0, 0
     assert mask.is_contiguous()
     if mask.dim() == 2:
-        assert mask.shape[0] == 1
         return 0, 0
     if mask.dim() == 3:
         assert mask.shape[1] == 1
@@ -108,13 +114,15 @@ def mask_strides(mask, per_head):
 
 
 def oracle_pa(oracle, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=None, v_scale=None, v_off=None,
-              mla_dv=0, q_scale=0.0, out_init=0.0, mask=None, mask_per_head=False, logn=None):
+              mla_dv=0, q_scale=0.0, out_init=0.0, mask=None, mask_per_head=False, logn=None, q_lens=None,
+              mask_rows="sequence"):
     qd = "bf16" if q.dtype == torch.bfloat16 else "float16"
     return oracle.paged_attention(
         to_oracle(q), to_oracle(kc), to_oracle(vc), tables.cpu().numpy(), np.asarray(ctx_host), scale,
         to_oracle(k_scale), to_oracle(k_off), to_oracle(v_scale), to_oracle(v_off), mla_v_head_size=mla_dv,
         q_scale=q_scale, q_dtype=qd, out_init=out_init, mask=to_oracle(mask), logn=to_oracle(logn),
-        mask_per_head=mask_per_head if (mask is not None and mask.dim() == 3) else None)
+        mask_per_head=mask_per_head if (mask is not None and mask.dim() == 3) else None, q_lens=q_lens,
+        mask_rows=mask_rows)
 
 
 def assert_close(got, want, tol, what=""):

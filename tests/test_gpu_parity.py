@@ -579,6 +579,98 @@ def test_masks_logn_and_dynamic_batch_through_operation_api(binding, oracle, dev
     c.close()
 
 
+# ------------------------------------------------------------------ several query tokens per sequence
+def _spec_mask(rng, dev, kind, ctx, q_lens, dtype):
+    """The masks of the reference's multi-token tests: "query" — one row per query row, the
+    causal triangle of -10000 over the last q positions of its sequence
+    (test_paged_attention_mla_mtp.py:220-231); "position" — the square causal mask
+    (test_paged_attention_operation_parallel_decoding_910B.py:157-160); both with a random
+    bias added where they are zero."""
+    max_len = int(max(ctx))
+    if kind == "position":
+        m = np.triu(np.ones((max_len, max_len), np.float32), 1) * -10000.0
+    else:
+        rows = int(sum(n for n, c in zip(q_lens, ctx) if c > 0))
+        m = np.zeros((rows, max_len), np.float32)
+        row = 0
+        for n, c in zip(q_lens, ctx):
+            if c == 0:
+                continue
+            m[row:row + n, c - n:c] = np.triu(np.ones((n, n), np.float32), 1) * -10000.0
+            row += n
+    # a random bias on the visible positions, so that a wrong row shows even where the triangle is small
+    m = np.where(m == 0, rng.standard_normal(m.shape).astype(np.float32), m)
+    return torch.from_numpy(m).to(dtype).to(dev)
+
+
+# heads, kv_heads, block, d, dv (0: same as d; > 0 with kv_heads 1 and d 576: MLA), ctx, q_lens, mask, dtype
+# (reference parallel-decoding test: q [1, 15, 30, 6] over k [10, 64, 64, 64]; MLA MTP tests: 2..4 tokens)
+SPEC_MATRIX = [
+    (32, 32, 128, 128, 0, [10, 64, 64, 64], [1, 15, 30, 6], "query", torch.float16),
+    (32, 32, 128, 128, 0, [10, 64, 64, 64], [1, 15, 30, 6], "position", torch.float16),
+    (32, 8, 128, 128, 0, [1000, 0, 2300, 130, 4], [2, 3, 4, 1, 4], "query", torch.bfloat16),
+    (30, 2, 16, 128, 0, [700, 33, 1500], [3, 2, 4], "position", torch.float16),
+    (16, 4, 64, 96, 0, [513, 800], [4, 0], "query", torch.float16),
+    (128, 1, 128, 576, 512, [700, 33, 1500], [2, 1, 3], None, torch.bfloat16),
+    (32, 1, 128, 576, 512, [300, 1200], [2, 4], "query", torch.float16),
+]
+
+
+@pytest.mark.parametrize("case", SPEC_MATRIX, ids=lambda c: "h%d_g%d_d%d_%s_%s" % (
+    c[0], c[1], c[3], c[7], str(c[8]).split(".")[-1]))
+def test_paged_attention_several_query_tokens(binding, oracle, dev, stream, case):
+    heads, kv_heads, block, d, mla_dv, ctx, q_lens, kind, dtype = case
+    rng = _rng(300 + heads + len(ctx))
+    dv = mla_dv if mla_dv else d
+    _, kc, vc, tables, ctx = _pa_inputs(rng, dev, len(ctx), heads, kv_heads, block, d, d, ctx, dtype,
+                                        std=0.5 if mla_dv else 1.0)
+    if mla_dv:
+        vc = None
+    rows = int(sum(n for n, c in zip(q_lens, ctx) if c > 0))
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(int(rng.integers(1 << 30)))
+    q = (torch.rand((rows + 1, heads, d), generator=gen) * 2 - 1).to(dtype).to(dev)
+    mask = None if kind is None else _spec_mask(rng, dev, kind, ctx, q_lens, dtype)
+    scale = 1.0 / math.sqrt(d)
+    mode = kind or "sequence"
+    want = oracle_pa(oracle, q, kc, vc, tables, ctx, scale, mla_dv=mla_dv, out_init=0.25, mask=mask, q_lens=q_lens,
+                     mask_rows=mode)
+    if kind is not None:
+        unmasked = oracle_pa(oracle, q, kc, vc, tables, ctx, scale, mla_dv=mla_dv, out_init=0.25, q_lens=q_lens)
+        assert np.abs(want - unmasked).max() > 0.01
+    for kernel in (binding.ATBMI_PA_KERNEL_SCALAR, binding.ATBMI_PA_KERNEL_AUTO):
+        out = torch.full((rows + 1, heads, dv), 0.25, dtype=dtype, device=dev)
+        got = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, mla_dv=mla_dv, kernel=kernel, out=out,
+                             mask=mask, q_lens=q_lens, mask_rows=mode)
+        assert_close(got, want, TOL[dtype], "kernel=%d" % kernel)
+
+
+def test_several_query_tokens_through_operation_api(binding, oracle, dev, stream):
+    """calcType = CALC_TYPE_SPEC: inputs q, caches, tables, contextLens, mask, qSeqLens
+    (reference paged_attention_operation.cpp:408-426), both lengths with hostData."""
+    rng = _rng(320)
+    heads, kv_heads, d, block = 32, 8, 128, 128
+    ctx = np.array([10, 64, 640, 64], dtype=np.int32)
+    q_lens = np.array([1, 15, 30, 6], dtype=np.int32)
+    _, kc, vc, tables, ctx = _pa_inputs(rng, dev, 4, heads, kv_heads, block, d, d, ctx, torch.float16)
+    q = (torch.rand((52, heads, d)) * 2 - 1).half().to(dev)
+    scale = 1.0 / math.sqrt(d)
+    lens, qn = torch.from_numpy(ctx), torch.from_numpy(q_lens)
+    c = binding.Context(stream)
+    for kind, mask_type in (("query", 3), ("position", 1)):
+        mask = _spec_mask(rng, dev, kind, ctx, q_lens, torch.float16)
+        pa = binding.OperationRunner("PagedAttentionOperation", binding.PagedAttentionParam(
+            headNum=heads, kvHeadNum=kv_heads, qkScale=scale, maskType=mask_type, calcType=1), c)
+        with torch.cuda.stream(stream):
+            out, = pa.run([q, kc, vc, tables, lens.to(dev), mask, qn.to(dev)], host_inputs={4: lens, 6: qn})
+        stream.synchronize()
+        assert tuple(out.shape) == (52, heads, d)
+        want = oracle_pa(oracle, q, kc, vc, tables, ctx, scale, mask=mask, q_lens=q_lens, mask_rows=kind)
+        assert_close(out, want, 1e-3, kind)
+        pa.close()
+    c.close()
+
+
 # ------------------------------------------------------------------ edge semantics
 @pytest.mark.parametrize("kernel", [1, 0])
 def test_empty_sequences_garbage_rows_and_shared_blocks(binding, oracle, dev, stream, kernel):

@@ -31,18 +31,23 @@ RAC_CASES = _load("reshape_and_cache")
 
 def _pa_unimplemented(p):
     """Features of PagedAttentionParam the reference accepts but this library rejects at creation."""
-    return (p.get("maskType", 0) >= 3 or p.get("compressType", 0) != 0 or p.get("calcType", 0) != 0 or
-            p.get("inputLayout", 0) != 0 or p.get("quantType", 0) >= 2)
+    return (p.get("maskType", 0) >= 4 or (p.get("maskType", 0) == 3 and p.get("calcType", 0) != 1) or
+            p.get("compressType", 0) != 0 or p.get("inputLayout", 0) != 0 or p.get("quantType", 0) >= 2)
 
 
 def _pa_mask_shape_refused(case):
     """Mask shapes the reference operation lets through Setup but its tiling has no stride
     rule for (tiling/paged_attention_tiling.cpp:36-74): a 4-dim NORM mask, and a 3-dim ALIBI
-    mask whose first dim is not the head count. Refused here during Setup."""
+    mask whose first dim is not the head count; with several query tokens per sequence
+    (calcType 1) a NORM mask that is not the square causal one. Refused here during Setup."""
     p = case["param"]
-    if p.get("maskType", 0) not in (1, 2) or _pa_unimplemented(p) or case["expected"] != "NO_ERROR":
+    if p.get("maskType", 0) not in (1, 2, 3) or _pa_unimplemented(p) or case["expected"] != "NO_ERROR":
         return False
     mask = case["in_shapes"][4 if p.get("mlaVHeadSize", 0) > 0 else 5]
+    if p.get("calcType", 0) == 1:
+        if p["maskType"] == 3:
+            return not (len(mask) == 2 and mask[0] == case["in_shapes"][0][0])
+        return not (len(mask) == 2 and mask[0] == mask[1])
     if p["maskType"] == 1:
         return len(mask) == 4
     return len(mask) == 3 and mask[0] != p["headNum"]
@@ -89,6 +94,10 @@ def _run_case(binding, case, ctx):
                 status_index = lens_index + (2 if p.get("maskType", 0) != 0 else 1)
                 if status_index < len(case["in_shapes"]):
                     host[status_index] = np.ones((case["in_shapes"][status_index][0],), dtype=np.int32)
+            if p.get("calcType", 0) == 1:
+                qlens_index = lens_index + (2 if p.get("maskType", 0) != 0 else 1)
+                if qlens_index < len(case["in_shapes"]):
+                    host[qlens_index] = np.ones((case["in_shapes"][qlens_index][0],), dtype=np.int32)
         ins = _tensors(binding, case["in_dtypes"], case["in_formats"], case["in_shapes"], host)
         outs = _tensors(binding, case["out_dtypes"], case["out_formats"], case["out_shapes"])
         st, _ = op.setup(ins, outs, ctx)
@@ -381,6 +390,60 @@ def test_mask_status_and_logn_inputs(binding, ctx):
     plain.close()
 
 
+def test_several_query_tokens_inputs(binding, ctx):
+    """CALC_TYPE_SPEC: qSeqLens follows the mask, is read on the host (reference param.cpp:96-110)
+    and has one entry per sequence; masks are (query rows, maxS) for MASK_TYPE_SPEC and the
+    square (maxS, maxS) for MASK_TYPE_NORM; the query rows must cover the sum of the lengths."""
+    e = binding.ERROR_CODE
+    lens = np.array([10, 64, 0, 64], dtype=np.int32)
+    qlens = np.array([1, 15, 7, 6], dtype=np.int32)   # the empty sequence brings no rows: 22 in all
+
+    def setup(op, mask_shape, q_rows=22, qlens_host=qlens, qlens_shape=(4,)):
+        ins = [
+            binding.make_tensor("float16", [q_rows, 32, 128], FAKE_DEVICE),
+            binding.make_tensor("float16", [8, 64, 16, 128], FAKE_DEVICE),
+            binding.make_tensor("float16", [8, 64, 16, 128], FAKE_DEVICE),
+            binding.make_tensor("int32", [4, 2], FAKE_DEVICE),
+            binding.make_tensor("int32", [4], FAKE_DEVICE, host_ptr=lens.ctypes.data),
+            binding.make_tensor("float16", mask_shape, FAKE_DEVICE),
+            binding.make_tensor("int32", list(qlens_shape), FAKE_DEVICE,
+                                host_ptr=qlens_host.ctypes.data if qlens_host is not None else None),
+        ]
+        outs = [binding.make_tensor("float16", [q_rows, 32, 128], FAKE_DEVICE)]
+        return op.setup(ins, outs, ctx)[0]
+
+    spec = binding.Operation("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=32, kvHeadNum=16, qkScale=0.088, maskType=3, calcType=1))
+    assert spec.ok and spec.input_num() == 7
+    assert setup(spec, [22, 64]) == 0
+    assert setup(spec, [24, 64], q_rows=24) == 0                      # spare query rows are left alone
+    assert setup(spec, [21, 64], q_rows=21) == e["ERROR_INVALID_PARAM"]  # 22 rows planned
+    assert setup(spec, [20, 64]) == e["ERROR_INVALID_PARAM"]          # one mask row per query row
+    assert setup(spec, [22, 63]) == e["ERROR_INVALID_PARAM"]          # shorter than a context
+    assert setup(spec, [4, 1, 64]) == e["ERROR_INVALID_PARAM"]
+    assert setup(spec, [22, 64], qlens_host=None) == e["ERROR_INVALID_PARAM"]
+    assert setup(spec, [22, 64], qlens_shape=(3,)) == e["ERROR_INVALID_PARAM"]
+    too_long = np.array([11, 1, 0, 1], dtype=np.int32)              # more query tokens than context
+    assert setup(spec, [22, 64], qlens_host=too_long) == e["ERROR_INVALID_PARAM"]
+    spec.close()
+    norm = binding.Operation("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=32, kvHeadNum=16, qkScale=0.088, maskType=1, calcType=1))
+    assert setup(norm, [64, 64]) == 0
+    assert setup(norm, [128, 128]) == 0
+    assert setup(norm, [22, 64]) == e["ERROR_INVALID_PARAM"]
+    assert setup(norm, [4, 1, 64]) == e["ERROR_INVALID_PARAM"]
+    norm.close()
+    # the reference's creation rules: SPEC needs the NORM or SPEC mask, and neither dequant nor logN
+    for bad in (dict(maskType=0), dict(maskType=2), dict(maskType=1, quantType=1), dict(maskType=1, scaleType=1),
+                dict(maskType=1, batchRunStatusEnable=True)):
+        op = binding.Operation("PagedAttentionOperation", binding.PagedAttentionParam(
+            headNum=32, kvHeadNum=16, qkScale=0.088, calcType=1, **bad))
+        assert op.status == e["ERROR_INVALID_PARAM"], bad
+    # MASK_TYPE_SPEC without CALC_TYPE_SPEC has no defined rows
+    op = binding.Operation("PagedAttentionOperation", binding.PagedAttentionParam(headNum=32, kvHeadNum=16, maskType=3))
+    assert op.status == e["ERROR_INVALID_PARAM"]
+
+
 def test_dequant_vector_lengths(binding, ctx):
     e = binding.ERROR_CODE
     op = binding.Operation("PagedAttentionOperation",
@@ -500,4 +563,20 @@ def test_kernel_layer_validates_without_a_gpu(binding):
         assert k.atbmi_pa_plan_algorithmic_bytes(plan) == want + extra * 2 + 4 * 4
         k.atbmi_pa_plan_destroy(plan)
     shape.maskBatchStride = -1
+    assert k.atbmi_pa_plan_create(ctypes.byref(shape), ctypes.byref(plan)) == 1
+    # several query rows per sequence: K/V count once, q/out and the mask once per row
+    shape.maskBatchStride, shape.maskHeadStride, shape.maskRowBy, shape.hasLogN = 512, 0, 1, 0
+    shape.numQueryRows = 9
+    assert k.atbmi_pa_plan_create(ctypes.byref(shape), ctypes.byref(plan)) == 0
+    qlens = np.array([3, 5, 4, 2], dtype=np.int32)    # sequence 1 is empty: 3 + 4 + 2 rows
+    assert k.atbmi_pa_plan_update_multi(plan, lens.ctypes.data, qlens.ctypes.data, 4) == 0
+    rows_ctx = 3 * 100 + 4 * 512 + 2 * 7
+    want_multi = (100 + 512 + 7) * 8 * 256 * 2 + 9 * 8 * 256 * 2 + (1 + 4 + 1) * 4 + 4 * 4 + rows_ctx * 2 + 4 * 4
+    assert k.atbmi_pa_plan_algorithmic_bytes(plan) == want_multi
+    qlens[3] = 8                                       # more query tokens than the 7 of context
+    assert k.atbmi_pa_plan_update_multi(plan, lens.ctypes.data, qlens.ctypes.data, 4) == 1
+    qlens[3] = 3                                       # 10 rows, the query holds 9
+    assert k.atbmi_pa_plan_update_multi(plan, lens.ctypes.data, qlens.ctypes.data, 4) == 1
+    k.atbmi_pa_plan_destroy(plan)
+    shape.maskRowBy = 3
     assert k.atbmi_pa_plan_create(ctypes.byref(shape), ctypes.byref(plan)) == 1

@@ -345,6 +345,61 @@ def test_logn_is_a_per_sequence_factor_on_the_scale(oracle):
                           oracle.paged_attention(q, kc, vc, tables, ctx, 0.25))
 
 
+# ---------------------------------------------------------------- several query tokens per sequence
+def _expand_rows(tables, ctx, q_lens):
+    """One single-token sequence per query row: (tables, ctx, owner sequence, token index)."""
+    owner = [i for i, n in enumerate(q_lens) if ctx[i] > 0 for _ in range(n)]
+    token = [t for i, n in enumerate(q_lens) if ctx[i] > 0 for t in range(n)]
+    return tables[owner], ctx[owner], np.array(owner), np.array(token)
+
+
+@pytest.mark.parametrize("mode", ["query", "position", None])
+def test_multi_token_queries_match_loops_on_expanded_rows(oracle, mode):
+    """Sequence i owns q_lens[i] consecutive query rows that all see its whole context; the
+    float64 loops get one single-token sequence per query row and the mask rows spelled out."""
+    rng = _rng(40)
+    q, kc, vc, tables, ctx = _paged_case(rng, batch=5, heads=4, kv_heads=2, max_ctx=12)
+    ctx = np.maximum(ctx, 4)
+    ctx[3] = 0
+    q_lens = np.array([2, 1, 4, 3, 3], np.int32)
+    rows = int(q_lens[ctx > 0].sum())
+    query = rng.standard_normal((rows + 1, 4, 16)).astype(np.float32)
+    tables_x, ctx_x, owner, token = _expand_rows(tables, ctx, q_lens)
+    max_len = 12
+    if mode == "query":
+        mask = rng.standard_normal((rows, max_len)).astype(np.float32)
+        dense = np.repeat(mask[:, None, :], 4, axis=1)
+    elif mode == "position":
+        mask = rng.standard_normal((max_len, max_len)).astype(np.float32)
+        pick = ctx[owner] - q_lens[owner] + token
+        dense = np.repeat(mask[pick][:, None, :], 4, axis=1)
+    else:
+        mask, dense = None, None
+    got = oracle.paged_attention(query, kc, vc, tables, ctx, 0.3, mask=mask, q_lens=q_lens,
+                                 mask_rows=mode or "sequence", out_init=0.5)
+    want = oracle.paged_attention_loops(query[:rows], kc, vc, tables_x, ctx_x, 0.3, dense_bias=dense)
+    np.testing.assert_allclose(got[:rows], want, rtol=2e-5, atol=2e-6)
+    assert np.all(got[rows] == np.float32(0.5))
+
+
+def test_multi_token_causal_mask_equals_growing_contexts(oracle):
+    """With the square causal mask the t-th of n query tokens sees the first ctx - n + t + 1 tokens."""
+    rng = _rng(41)
+    q, kc, vc, tables, ctx = _paged_case(rng, batch=3, heads=4, kv_heads=2, max_ctx=14)
+    ctx = np.maximum(ctx, 5)
+    q_lens = np.array([3, 1, 5], np.int32)
+    query = rng.standard_normal((9, 4, 16)).astype(np.float32)
+    causal = np.triu(np.full((14, 14), -np.inf, np.float32), 1)
+    got = oracle.paged_attention(query, kc, vc, tables, ctx, 0.3, mask=causal, q_lens=q_lens, mask_rows="position")
+    tables_x, ctx_x, owner, token = _expand_rows(tables, ctx, q_lens)
+    seen = (ctx_x - q_lens[owner] + token + 1).astype(np.int32)
+    want = oracle.paged_attention(query, kc, vc, tables_x, seen, 0.3)
+    np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-6)
+    # one query token per sequence is the plain decode step
+    assert np.array_equal(oracle.paged_attention(q, kc, vc, tables, ctx, 0.3, q_lens=np.ones(3, np.int32)),
+                          oracle.paged_attention(q, kc, vc, tables, ctx, 0.3))
+
+
 def test_int8_dequant_channel_indexing_and_identity(oracle):
     rng = _rng(11)
     q, _, _, tables, ctx = _paged_case(rng, heads=4, kv_heads=2, d=8, dv=8)
