@@ -27,8 +27,8 @@ HBM_PEAK_GBPS = 8000.0
 # script, scaled by what the same counters read for a 256 MiB copy (--calibrate-copy); the runs and the
 # scale factors are written up in the profiles/ summaries of each workload. Keyed by workload and its
 # algorithmic bytes, so a changed workload reports null instead of a stale figure.
-MEASURED_TRAFFIC = {("c2", 651658484): 658.7e6, ("c2_alibi", 661824180): 669.5e6, ("c3", 1364204576): 1379.2e6,
-                    ("c5", 253384304): 388.7e6}
+MEASURED_TRAFFIC = {("c2", 651658484): 658.7e6, ("c2_alibi", 661824180): 669.5e6, ("c2_mtp4", 656075180): 683.6e6,
+                    ("c3", 1364204576): 1379.2e6, ("c5", 253384304): 388.7e6}
 
 DESCRIPTIONS = {
     "c1": "C1 small fp16 decode: batch 4, 8 q heads, 8 kv heads, d128, block 128, ctx U[64,512]",
