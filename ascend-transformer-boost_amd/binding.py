@@ -93,14 +93,14 @@ class AtbmiPaShape(ctypes.Structure):
         ("kernel", ctypes.c_int32), ("hasMask", ctypes.c_int32), ("qkScale", ctypes.c_float),
         ("qScale", ctypes.c_float), ("maskBatchStride", ctypes.c_int64), ("maskHeadStride", ctypes.c_int64),
         ("maskLen", ctypes.c_int32), ("hasLogN", ctypes.c_int32),
-        ("descalePacked", ctypes.c_int32), ("maskRowBy", ctypes.c_int32), ("reserved", ctypes.c_int32),
+        ("descalePacked", ctypes.c_int32), ("maskRowBy", ctypes.c_int32), ("ropeDim", ctypes.c_int32),
     ]
 
 
 class AtbmiPaTensors(ctypes.Structure):
     _fields_ = [(n, ctypes.c_void_p) for n in
                 ("query", "keyCache", "valueCache", "blockTables", "kScale", "kOffset", "vScale", "vOffset", "out",
-                 "mask", "logN")]
+                 "mask", "logN", "queryRope", "keyRopeCache", "lse")]
 
 
 _kernels = None

@@ -85,6 +85,15 @@ struct PaArgs {
     const float *logN;   // per batch row factor on qkScale (null: none)
     int32_t scaleStride; // floats between consecutive kScale / vScale entries: 1, or 2 for uint64-packed ones
     int32_t maskRowStep; // mask rows between consecutive query tokens of one sequence (0: they share a row)
+    // Split latent layout (null / 0: none): the last ropeDim of the D channels of every query row live in
+    // qRope [rows][H][ropeDim] and those of every key row in kRope [slots][G][ropeDim]; q and kc then
+    // hold rows of D - ropeDim channels.
+    const void *qRope;
+    const void *kRope;
+    int64_t ropeRowStride; // elements between consecutive tokens in kRope (G * ropeDim)
+    int32_t ropeDim;
+    int32_t pad0;
+    void *lse;           // [rows][H] in the query's type: natural-log log-sum-exp of the scaled scores (null: none)
 };
 
 // ---- Plan of the MFMA kernel ------------------------------------------------

@@ -153,8 +153,14 @@ extern "C" int atbmi_pa_plan_create(const AtbmiPaShape *shape, AtbmiPaPlan **pla
     if (s.descalePacked && s.kvDtype != ATBMI_INT8) {
         return Fail(ERR_INVALID_PARAM, "pa_plan_create: packed descales only apply to an int8 cache");
     }
-    if (s.maskRowBy < ATBMI_PA_MASK_ROW_SEQUENCE || s.maskRowBy > ATBMI_PA_MASK_ROW_POSITION || s.reserved != 0) {
-        return Fail(ERR_INVALID_PARAM, "pa_plan_create: maskRowBy %d / reserved %d", s.maskRowBy, s.reserved);
+    if (s.maskRowBy < ATBMI_PA_MASK_ROW_SEQUENCE || s.maskRowBy > ATBMI_PA_MASK_ROW_POSITION) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: maskRowBy %d", s.maskRowBy);
+    }
+    if (s.ropeDim != 0 && !(s.ropeDim == 64 && s.mlaCombined && s.headDimK == 576 && s.headDimV == 512 &&
+                            s.kvDtype != ATBMI_INT8)) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: the split latent layout is 512 + 64 channels of a 16-bit "
+                                       "combined cache, got ropeDim %d with head sizes %d / %d", s.ropeDim, s.headDimK,
+                    s.headDimV);
     }
     if (s.hasMask && (s.maskLen <= 0 || s.maskBatchStride < 0 || s.maskHeadStride < 0)) {
         return Fail(ERR_INVALID_PARAM, "pa_plan_create: mask row length %d, strides %lld / %lld", s.maskLen,
@@ -611,6 +617,12 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
     if (s.hasOffset && (!t->kOffset || !t->vOffset)) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: hasOffset needs kOffset and vOffset");
     }
+    if (s.ropeDim != 0 && (!t->queryRope || !t->keyRopeCache)) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: the split latent layout needs queryRope and keyRopeCache");
+    }
+    if (t->lse && s.kvDtype == ATBMI_INT8) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: no log-sum-exp output with an int8 cache");
+    }
     if ((s.hasMask && !t->mask) || (s.hasLogN && !t->logN)) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: the plan was made with a mask / logN, none given");
     }
@@ -652,9 +664,9 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
     a.groupSize = s.numHeads / s.numKvHeads;
     a.qkScale = s.qkScale;
     a.qScale = (s.qScale == 0.0f || s.qScale == 1.0f) ? 0.0f : s.qScale;
-    a.kRowStride = static_cast<int64_t>(s.numKvHeads) * s.headDimK;
+    a.kRowStride = static_cast<int64_t>(s.numKvHeads) * (s.headDimK - s.ropeDim);
     a.vRowStride = s.mlaCombined ? a.kRowStride : static_cast<int64_t>(s.numKvHeads) * s.headDimV;
-    a.vHeadStride = s.mlaCombined ? s.headDimK : s.headDimV;
+    a.vHeadStride = s.mlaCombined ? s.headDimK - s.ropeDim : s.headDimV;
     a.finishV = (plan->useMfma && s.kvDtype == ATBMI_INT8) ? 1 : 0;
     if (s.hasMask) {
         a.mask = t->mask;
@@ -667,6 +679,11 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
     a.logN = s.hasLogN ? t->logN : nullptr;
     a.scaleStride = s.descalePacked ? 2 : 1; // little endian: the low half of each uint64 comes first
     a.maskRowStep = s.maskRowBy == ATBMI_PA_MASK_ROW_SEQUENCE ? 0 : 1;
+    a.qRope = s.ropeDim ? t->queryRope : nullptr;
+    a.kRope = s.ropeDim ? t->keyRopeCache : nullptr;
+    a.ropeDim = s.ropeDim;
+    a.ropeRowStride = static_cast<int64_t>(s.numKvHeads) * s.ropeDim;
+    a.lse = t->lse;
 
     TimingRecord rec{nullptr, nullptr};
     bool timed = false;

@@ -211,6 +211,18 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
     unsigned char *vTile = MLA ? kTile : kTile + K_TILE_BYTES;
     const unsigned char *kcBase = reinterpret_cast<const unsigned char *>(a.kc);
     const unsigned char *vcBase = reinterpret_cast<const unsigned char *>(a.vc);
+    // Split latent layout (combined cache only): the last ropeDim channels of a key row come from a
+    // cache of their own, those of a query row from a tensor of their own.
+    const unsigned char *krBase = reinterpret_cast<const unsigned char *>(a.kRope);
+    const int dn = MLA ? D - a.ropeDim : D;  // channels per row of q and of the key cache itself
+    const int nopePieces = dn / 8;           // 16-byte pieces of a key row that the key cache holds
+    // Address of piece `col` of the key row at cache slot r.
+    auto keyPiece = [&](int64_t r, int col) -> const unsigned char * {
+        if (MLA && col >= nopePieces) {
+            return krBase + (r * a.ropeRowStride + static_cast<int64_t>(g) * a.ropeDim) * 2 + (col - nopePieces) * 16;
+        }
+        return kcBase + (r * a.kRowStride + static_cast<int64_t>(g) * dn) * ESZ + col * 16;
+    };
     constexpr float LOG2E = 1.4426950408889634f;
     const float scale2 = a.qkScale * LOG2E;
     const uint32_t onePair = BF16 ? 0x3f803f80u : 0x3c003c00u; // {1.0, 1.0} in the operand type
@@ -259,13 +271,14 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
         // ---- Q^T as B operand: lane (n, kg) holds q[column n][32j + 8kg .. +8) for j < NQ
         u32x4 qreg[NQ];
         {
-            const uint16_t *qrow =
-                reinterpret_cast<const uint16_t *>(a.q) + (static_cast<int64_t>(qRow) * a.H + h0 + colHead) * D;
+            const int64_t qh = static_cast<int64_t>(qRow) * a.H + h0 + colHead;
+            const uint16_t *qrow = reinterpret_cast<const uint16_t *>(a.q) + qh * dn;
+            const uint16_t *qrope = reinterpret_cast<const uint16_t *>(a.qRope) + qh * a.ropeDim - dn;
 #pragma unroll
             for (int j = 0; j < NQ; ++j) { // all loads first, so their latencies overlap
                 qreg[j] = u32x4{0u, 0u, 0u, 0u};
                 if (n < nh) {
-                    qreg[j] = LoadGlobal16(qrow + j * 32 + kg * 8);
+                    qreg[j] = LoadGlobal16((MLA && j * 32 >= dn ? qrope : qrow) + j * 32 + kg * 8);
                 }
             }
             const bool plain = !KV8 && a.qScale == 0.0f; // raw bits are already the operand
@@ -358,7 +371,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
             u32x4 v = {0u, 0u, 0u, 0u};
             if (full || t + row < tokEnd) {
                 const int64_t r = rowBase[row >> 4] + (row & 15);
-                v = LoadStream16(kcBase + (r * a.kRowStride + static_cast<int64_t>(g) * D) * ESZ + col * 16);
+                v = LoadStream16(keyPiece(r, col));
             }
             return v;
         };
@@ -590,7 +603,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                     if (pc < PIECES && t + row < tokEnd) {
                         const int64_t r = rowBase[row >> 4] + (row & 15);
                         // plain load: the other head groups of this range fetch the same rows from L2
-                        stage[i] = LoadGlobal16(kcBase + (r * a.kRowStride + static_cast<int64_t>(g) * D) * 2 + col * 16);
+                        stage[i] = LoadGlobal16(keyPiece(r, col));
                     }
                 }
             };
@@ -714,6 +727,9 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                         packed[1] = Pack2<false>(o[2], o[3]);
                     }
                     *reinterpret_cast<u32x2 *>(orow + d) = packed;
+                }
+                if (a.lse && kg == 0) {
+                    Store16(a.lse, static_cast<int64_t>(qRow) * a.H + h, (m + log2f(l)) * 0.6931471805599453f, qBf16);
                 }
             } else {
                 const int slot = 2 * wr + (segBegin == s0 ? 0 : 1);

@@ -163,7 +163,9 @@ __device__ __forceinline__ void DmaWait()
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-template <bool BF16>
+// SPLIT: the last 64 channels of every latent row live in a cache of their own (a.kRope), those of every
+// query row in a.qRope; a.kc and a.q then hold 512-channel rows.
+template <bool BF16, bool SPLIT>
 __global__ __launch_bounds__(NW *WAVE) void PaMlaWideKernel(const PaArgs a, const PaStreamPlan p)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -193,6 +195,9 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaWideKernel(const PaArgs a, cons
         reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char *)smem));
     const unsigned char *kcBase = reinterpret_cast<const unsigned char *>(a.kc);
     const int64_t rowBytes = a.kRowStride * 2;
+    const unsigned char *krBase = reinterpret_cast<const unsigned char *>(a.kRope);
+    const int64_t ropeRowBytes = a.ropeRowStride * 2;
+    constexpr int NOPE_PIECES = DV * 2 / 16; // 16-byte pieces of a latent row ahead of its rope channels
     constexpr float LOG2E = 1.4426950408889634f;
     const float scale2 = a.qkScale * LOG2E;
 
@@ -267,6 +272,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaWideKernel(const PaArgs a, cons
         // data (the padding slot of each row, everything past the 8 rows) fetch a neighbour's piece, so
         // every lane of every transfer is active and reads valid memory.
         const unsigned char *stSub0 = nullptr, *stSub1 = nullptr;
+        const unsigned char *stRope0 = nullptr, *stRope1 = nullptr; // SPLIT: the same rows of the rope cache
         int stLastRow = 0;
         uint32_t stDst = 0;
         auto prepare = [&](int t, uint32_t tileAddr) {
@@ -274,6 +280,10 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaWideKernel(const PaArgs a, cons
             const int64_t row1 = static_cast<int64_t>(__builtin_amdgcn_readfirstlane(pendBlk[1])) * a.blockSize + pendOff[1];
             stSub0 = kcBase + row0 * rowBytes;
             stSub1 = kcBase + row1 * rowBytes;
+            if constexpr (SPLIT) {
+                stRope0 = krBase + row0 * ropeRowBytes;
+                stRope1 = krBase + row1 * ropeRowBytes;
+            }
             lookAhead();
             stLastRow = min(tokEnd - 1 - t, STEP - 1);
             stDst = tileAddr + static_cast<uint32_t>(wave * REGION);
@@ -282,13 +292,25 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaWideKernel(const PaArgs a, cons
         // through a second one.
         auto transfer = [&](auto index) {
             constexpr int i = decltype(index)::value;
-            int slot = i * WAVE + lane;
+            int ln = lane;
+            if constexpr (SPLIT) {
+                // rederive the slot from the lane id at every transfer: hoisted out of the loop, the
+                // per-lane row, piece and cache choice of ten transfers would not fit the registers
+                asm volatile("" : "+v"(ln));
+            }
+            int slot = i * WAVE + ln;
             slot = slot < WAVE_SLOTS ? slot : slot - WAVE_SLOTS;
             const int rowIn = slot / SLOTS_PER_ROW;
             const int col = min(slot - rowIn * SLOTS_PER_ROW, SLOTS_PER_ROW - 2);
             const int row = min(ROWS_PER_WAVE * wave + rowIn, stLastRow);
             const unsigned char *src = ((row >> 4) ? stSub1 : stSub0) +
                                        static_cast<uint32_t>(row & 15) * static_cast<uint32_t>(rowBytes) + col * 16;
+            if constexpr (SPLIT) {
+                if (col >= NOPE_PIECES) {
+                    src = ((row >> 4) ? stRope1 : stRope0) +
+                          static_cast<uint32_t>(row & 15) * static_cast<uint32_t>(ropeRowBytes) + (col - NOPE_PIECES) * 16;
+                }
+            }
             if constexpr (i == 0) {
                 DmaBase(stDst + 4096);
             }
@@ -324,11 +346,12 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaWideKernel(const PaArgs a, cons
         // ---- Q^T as B operand: lane (n, kh) holds q[h0+n][16 j + 8 kh .. +8) for j < NQ
         u32x4 qreg[NQ];
         {
-            const uint16_t *qrow =
-                reinterpret_cast<const uint16_t *>(a.q) + (static_cast<int64_t>(qRow) * a.H + h0 + n) * D + kh * 8;
+            const int64_t qh = static_cast<int64_t>(qRow) * a.H + h0 + n;
+            const uint16_t *qrow = reinterpret_cast<const uint16_t *>(a.q) + qh * (SPLIT ? DV : D) + kh * 8;
+            const uint16_t *qrope = reinterpret_cast<const uint16_t *>(a.qRope) + qh * (D - DV) - DV + kh * 8;
 #pragma unroll
             for (int j = 0; j < NQ; ++j) {
-                qreg[j] = mfma::LoadGlobal16(qrow + j * 16);
+                qreg[j] = mfma::LoadGlobal16((SPLIT && j * 16 >= DV ? qrope : qrow) + j * 16);
             }
         }
 
@@ -514,6 +537,9 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaWideKernel(const PaArgs a, cons
                 }
                 __builtin_amdgcn_sched_barrier(0); // one tile at a time through the VGPRs
             }
+            if (a.lse && kh == 0) {
+                Store16(a.lse, static_cast<int64_t>(qRow) * a.H + h, (m + log2f(l)) * 0.6931471805599453f, qBf16);
+            }
         } else {
             const int slot = 2 * wr + (segBegin == s0 ? 0 : 1);
             const int64_t ph = static_cast<int64_t>(slot) * a.H + h;
@@ -534,9 +560,9 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaWideKernel(const PaArgs a, cons
     }
 }
 
-template <bool BF16> int LaunchWide(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
+template <bool BF16, bool SPLIT> int LaunchWide(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
 {
-    auto kernel = PaMlaWideKernel<BF16>;
+    auto kernel = PaMlaWideKernel<BF16, SPLIT>;
     constexpr int lds = 3 * TILE_BYTES + BLK_IDS * 4;
     static bool configured = false; // one attribute call per instantiation and process
     if (!configured) {
@@ -545,7 +571,8 @@ template <bool BF16> int LaunchWide(const PaArgs &args, const PaStreamPlan &plan
         configured = true;
     }
     if (plan.tokenSlices != 1 || plan.numWaveRanges != plan.numWgRanges ||
-        plan.headGroups * PA_MLA_HEADS_PER_WG != args.H || args.G != 1 || args.D != D || args.Dv != DV) {
+        plan.headGroups * PA_MLA_HEADS_PER_WG != args.H || args.G != 1 || args.D != D || args.Dv != DV ||
+        args.ropeDim != (SPLIT ? D - DV : 0)) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: plan or shape does not fit the 128-head MLA kernel");
     }
     const int64_t grid = (static_cast<int64_t>(plan.numWgRanges) + 7) / 8 * 8 * plan.headGroups;

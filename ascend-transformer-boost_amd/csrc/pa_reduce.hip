@@ -15,6 +15,7 @@ namespace atbmi {
 namespace {
 
 constexpr int REDUCE_THREADS = 128;
+constexpr float LN2 = 0.6931471805599453f; // the partial log-sum-exps are kept in base 2
 
 __global__ __launch_bounds__(REDUCE_THREADS) void PaReduceKernel(const PaArgs a)
 {
@@ -36,6 +37,9 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaReduceKernel(const PaArgs a)
     const float inv = total > 0.0f ? 1.0f / total : 0.0f;
     const int g = h / a.groupSize;
     const bool bf16 = a.qIsBf16 != 0;
+    if (a.lse && threadIdx.x == 0) {
+        Store16(a.lse, static_cast<int64_t>(s.qRow) * a.H + h, (mx + log2f(total)) * LN2, bf16);
+    }
 
     for (int d = threadIdx.x; d < a.Dv; d += REDUCE_THREADS) {
         float acc = 0.0f;
@@ -150,6 +154,9 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaA
     }
     const float sum = blockSum(total);
     const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
+    if (a.lse && tid == 0) {
+        Store16(a.lse, static_cast<int64_t>(sq.qRow + tok) * a.H + h, (mx + log2f(sum)) * LN2, a.qIsBf16 != 0);
+    }
 #pragma unroll
     for (int c = 0; c < 5; ++c) {
         const int d = tid + c * REDUCE_THREADS;

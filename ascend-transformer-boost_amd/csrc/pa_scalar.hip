@@ -47,6 +47,7 @@ __global__ __launch_bounds__(PA_SCALAR_WAVES * WAVE) void PaScalarKernel(const P
     // additive score bias of this sequence and head tile (base-2 units once multiplied by LOG2E)
     const int64_t maskRow = a.mask ? static_cast<int64_t>(it.maskRow) * a.maskBatchStride : 0;
 
+    const int dn = a.D - a.ropeDim; // channels held by q / kc themselves (all of them unless the layout is split)
     float q[HT][EPL];
 #pragma unroll
     for (int hh = 0; hh < HT; ++hh) {
@@ -55,8 +56,8 @@ __global__ __launch_bounds__(PA_SCALAR_WAVES * WAVE) void PaScalarKernel(const P
             const int d = lane + WAVE * e;
             float v = 0.0f;
             if (hh < nh && d < a.D) {
-                const int64_t idx = (static_cast<int64_t>(it.qRow) * a.H + h0 + hh) * a.D + d;
-                v = Load16(a.q, idx, bf16);
+                const int64_t qh = static_cast<int64_t>(it.qRow) * a.H + h0 + hh;
+                v = d < dn ? Load16(a.q, qh * dn + d, bf16) : Load16(a.qRope, qh * a.ropeDim + d - dn, bf16);
                 if (a.qScale != 0.0f) {
                     // the reference pre-multiplies Q in its own dtype
                     v *= a.qScale;
@@ -98,7 +99,8 @@ __global__ __launch_bounds__(PA_SCALAR_WAVES * WAVE) void PaScalarKernel(const P
     const int32_t *table = a.tables + static_cast<int64_t>(it.seq) * a.maxBlocksPerSeq;
     for (int t = it.tokBegin + wave; t < it.tokEnd; t += PA_SCALAR_WAVES) {
         const int64_t row = static_cast<int64_t>(table[t / a.blockSize]) * a.blockSize + (t % a.blockSize);
-        const int64_t kBase = row * a.kRowStride + static_cast<int64_t>(g) * a.D;
+        const int64_t kBase = row * a.kRowStride + static_cast<int64_t>(g) * dn;
+        const int64_t rBase = row * a.ropeRowStride + static_cast<int64_t>(g) * a.ropeDim - dn;
         const int64_t vBase = row * a.vRowStride + static_cast<int64_t>(g) * a.vHeadStride;
         float k[EPL], v[EPL];
 #pragma unroll
@@ -115,7 +117,7 @@ __global__ __launch_bounds__(PA_SCALAR_WAVES * WAVE) void PaScalarKernel(const P
                 }
             } else {
                 if (d < a.D) {
-                    k[e] = Load16(a.kc, kBase + d, bf16);
+                    k[e] = d < dn ? Load16(a.kc, kBase + d, bf16) : Load16(a.kRope, rBase + d, bf16);
                 }
                 if (d < a.Dv) {
                     v[e] = Load16(a.vc, vBase + d, bf16);

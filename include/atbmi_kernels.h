@@ -124,7 +124,10 @@ typedef struct AtbmiPaShape {
     int32_t descalePacked;   /* 1: kScale / vScale are uint64 arrays whose low 32 bits hold the fp32 value,
                                 as atb::Utils::QuantParamConvert packs them (reference src/atb/utils/utils.cpp:153-164) */
     int32_t maskRowBy;       /* AtbmiPaMaskRow: which mask row (in units of maskBatchStride) a query row uses */
-    int32_t reserved;        /* 0 */
+    int32_t ropeDim;         /* 0, or 64 with mlaCombined, headDimK 576 and headDimV 512: the split latent layout of
+                                MultiLatentAttentionParam::KROPE_CTKV (reference include/atb/infer_op_params.h:2949-2958):
+                                query and keyCache hold rows of headDimK - ropeDim channels, queryRope and
+                                keyRopeCache the remaining ropeDim channels of the same rows */
 } AtbmiPaShape;
 
 /* Device tensors of one decode call.
@@ -155,6 +158,11 @@ typedef struct AtbmiPaTensors {
     void *out;
     const void *mask;
     const float *logN;
+    const void *queryRope;    /* [numQueryRows, H, ropeDim] qDtype, ropeDim > 0 only */
+    const void *keyRopeCache; /* [numBlocks, blockSize, G, ropeDim] qDtype, ropeDim > 0 only */
+    void *lse;                /* NULL, or [numQueryRows, H] qDtype: receives the natural-log log-sum-exp of the
+                                 scaled (and masked) scores of every planned query row and head — the second
+                                 output of MultiLatentAttentionParam::CALC_TYPE_RING */
 } AtbmiPaTensors;
 
 typedef struct AtbmiPaPlan AtbmiPaPlan; /* opaque; owned by the caller, not thread-safe */

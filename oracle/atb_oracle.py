@@ -29,6 +29,9 @@ the invariants of the mathematics (no function is left "parity unpinned"):
                       all k_lens[i] tokens; mask rows [k - q : k] of the square causal mask, or rows
                       [cu : cu + q] of the per-query-row mask), tests/apitest/kernelstest/mix/
                       test_paged_attention_mla_mtp.py:120-166 (the same for the MLA cache, fp32 branch);
+                      MultiLatentAttention: tests/apitest/opstest/python/operations/multi_latent_attention/
+                      test_multi_latent_attention_lse.py:122-130 (lse = row max + log(row sum)), :148-182,
+                      :386-388 (query and cache split [512, 64] along the channels);
                       several query tokens per sequence (calcType SPEC): tests/apitest/opstest/python/
                       operations/paged_attention/test_paged_attention_operation_parallel_decoding_910B.py:
                       75-121 (sequence i owns q_lens[i] consecutive query rows, every one attends to
@@ -131,11 +134,13 @@ def gather_rows(cache, block_table, context_len):
 
 
 def attention_one(q, keys, values, scale, k_descale=None, k_offset=None, v_descale=None, v_offset=None,
-                  bias=None):
+                  bias=None, lse_out=None):
     """One query token against gathered rows. q [heads, D] float32; keys
     [ctx, kv_heads, D]; values [ctx, kv_heads, Dv] (float32 or int8); bias None
     or broadcastable to [heads, ctx], added to the scaled scores.
-    Returns float32 [heads, Dv]: softmax(scale * q k^T + bias) v per GQA group."""
+    Returns float32 [heads, Dv]: softmax(scale * q k^T + bias) v per GQA group.
+    lse_out, a float32 [heads] array, receives the natural-log log-sum-exp of the
+    scaled and biased scores (row max + log of the row sum of exp(score - max))."""
     if bias is not None:
         bias = np.broadcast_to(np.asarray(bias, dtype=np.float32), (q.shape[0], keys.shape[0]))
     heads = q.shape[0]
@@ -156,6 +161,9 @@ def attention_one(q, keys, values, scale, k_descale=None, k_offset=None, v_desca
             sim = sim + bias[g * group:(g + 1) * group]
         p = softmax_rows(sim)
         out[g * group:(g + 1) * group] = p @ v
+        if lse_out is not None:
+            row_max = np.max(sim, axis=-1)
+            lse_out[g * group:(g + 1) * group] = row_max + np.log(np.sum(np.exp(sim - row_max[:, None]), axis=-1))
     return out
 
 
@@ -190,7 +198,7 @@ def norm_mask(batch, max_len, value=-10000.0):
 def paged_attention(query, key_cache, value_cache, block_tables, context_lens, scale, k_descale=None,
                     k_offset=None, v_descale=None, v_offset=None, mla_v_head_size=0, q_scale=0.0,
                     q_dtype="float32", out_init=0.0, mask=None, logn=None, mask_per_head=None, q_lens=None,
-                    mask_rows="sequence"):
+                    mask_rows="sequence", lse_out=None):
     """Decode attention over paged caches.
 
     query [rows, heads, D] float32; key_cache [blocks, block, kv_heads, D];
@@ -212,6 +220,12 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, s
     2-dim mask then has one row per query row (mask_rows="query") or is the
     square causal mask, of which the t-th query token of a sequence with n of
     them uses row ctx - n + t (mask_rows="position").
+    lse_out, a float32 [rows, heads] array, receives the log-sum-exp of every
+    written row (see attention_one); other rows are left alone.
+    The split latent layout of MultiLatentAttention (query / cache rows given as
+    512 + 64 channels in two tensors) is the same computation on the rows
+    concatenated along the channel axis, which is what the reference golden
+    does the other way round (it splits the concatenated tensors).
     Returns float32 [rows, heads, Dv]."""
     query = np.asarray(query, dtype=np.float32)
     if mla_v_head_size > 0:
@@ -238,7 +252,7 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, s
             else:
                 bias = _mask_slice(mask, i, ctx, query.shape[1], len(context_lens), mask_per_head)
             out[row] = attention_one(query[row], keys, values, seq_scale, k_descale, k_offset, v_descale,
-                                     v_offset, bias)
+                                     v_offset, bias, None if lse_out is None else lse_out[row])
             row += 1
     return out
 

@@ -22,12 +22,17 @@ def dtype_code(binding, t):
 
 def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=None, v_scale=None,
                    v_off=None, mla_dv=0, q_scale=0.0, kernel=0, chunk_tokens=None, out=None, return_plan_info=False,
-                   mask=None, mask_per_head=False, logn=None, q_lens=None, mask_rows="sequence"):
+                   mask=None, mask_per_head=False, logn=None, q_lens=None, mask_rows="sequence", q_rope=None,
+                   k_rope=None, lse=None):
     """atbmi_pa_plan_* + atbmi_pa_decode on `stream`; returns the output tensor.
     mask: device tensor of q's dtype shaped like one of the reference's decode
-    masks; mask_per_head says that a 3-dim mask's first dim counts heads (ALIBI)."""
+    masks; mask_per_head says that a 3-dim mask's first dim counts heads (ALIBI).
+    q_rope / k_rope: the split latent layout (q and kc then hold the first 512
+    channels); lse: a [rows, heads] tensor of q's dtype that receives the log-sum-exp."""
     k = binding.kernels()
     rows, heads, d = q.shape
+    rope = 0 if q_rope is None else q_rope.shape[2]
+    d += rope
     dv = mla_dv if mla_dv else vc.shape[3]
     mask_batch_stride, mask_head_stride = mask_strides(mask, mask_per_head)
     if mask_rows != "sequence":
@@ -40,7 +45,7 @@ def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=
         maskHeadStride=mask_head_stride, maskLen=0 if mask is None else mask.shape[-1],
         hasLogN=0 if logn is None else 1,
         descalePacked=1 if (k_scale is not None and k_scale.dtype == torch.int64) else 0,
-        maskRowBy={"sequence": 0, "query": 1, "position": 2}[mask_rows])
+        maskRowBy={"sequence": 0, "query": 1, "position": 2}[mask_rows], ropeDim=rope)
     old = os.environ.get("ATBMI_PA_CHUNK_TOKENS")
     if chunk_tokens is not None:
         os.environ["ATBMI_PA_CHUNK_TOKENS"] = str(chunk_tokens)
@@ -81,6 +86,9 @@ def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=
             t.out = out.data_ptr()
             t.mask = mask.data_ptr() if mask is not None else None
             t.logN = logn.data_ptr() if logn is not None else None
+            t.queryRope = q_rope.data_ptr() if q_rope is not None else None
+            t.keyRopeCache = k_rope.data_ptr() if k_rope is not None else None
+            t.lse = lse.data_ptr() if lse is not None else None
             rc = k.atbmi_pa_decode(plan, ctypes.byref(t), ws.data_ptr(), ws_bytes, stream.cuda_stream)
             if rc != 0:
                 raise RuntimeError("pa_decode: " + binding.last_kernel_error())
@@ -115,14 +123,14 @@ def mask_strides(mask, per_head):
 
 def oracle_pa(oracle, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=None, v_scale=None, v_off=None,
               mla_dv=0, q_scale=0.0, out_init=0.0, mask=None, mask_per_head=False, logn=None, q_lens=None,
-              mask_rows="sequence"):
+              mask_rows="sequence", lse_out=None):
     qd = "bf16" if q.dtype == torch.bfloat16 else "float16"
     return oracle.paged_attention(
         to_oracle(q), to_oracle(kc), to_oracle(vc), tables.cpu().numpy(), np.asarray(ctx_host), scale,
         to_oracle(k_scale), to_oracle(k_off), to_oracle(v_scale), to_oracle(v_off), mla_v_head_size=mla_dv,
         q_scale=q_scale, q_dtype=qd, out_init=out_init, mask=to_oracle(mask), logn=to_oracle(logn),
         mask_per_head=mask_per_head if (mask is not None and mask.dim() == 3) else None, q_lens=q_lens,
-        mask_rows=mask_rows)
+        mask_rows=mask_rows, lse_out=lse_out)
 
 
 def assert_close(got, want, tol, what=""):

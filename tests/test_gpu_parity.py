@@ -579,6 +579,69 @@ def test_masks_logn_and_dynamic_batch_through_operation_api(binding, oracle, dev
     c.close()
 
 
+# ------------------------------------------------------------------ split latent layout, log-sum-exp output
+# batch, heads, ctx, q_lens (None: one token each), dtype, chunk override
+# (reference test_multi_latent_attention.py / _lse.py / _mtp.py: heads 8..128, block 128, 512 + 64 channels)
+SPLIT_MATRIX = [
+    (32, 32, 256, None, torch.float16, None),
+    (4, 128, [3000, 17, 128, 1025], None, torch.bfloat16, None),
+    (20, 128, 256, None, torch.float16, 64),
+    (3, 128, [700, 0, 1500], [2, 3, 4], torch.bfloat16, None),
+    (5, 8, [819, 12, 4000, 256, 300], None, torch.float16, None),
+    (6, 64, 515, [1, 2, 1, 3, 1, 1], torch.bfloat16, None),
+]
+
+
+@pytest.mark.parametrize("case", SPLIT_MATRIX, ids=lambda c: "b%d_h%d_%s%s%s" % (
+    c[0], c[1], str(c[4]).split(".")[-1], "_multi" if c[3] else "", "_chunk%d" % c[5] if c[5] else ""))
+def test_split_latent_layout_and_lse(binding, oracle, dev, stream, case):
+    """Query and cache rows given as 512 + 64 channels in two tensors each give bit-for-bit what the
+    576-channel rows give (same kernels, two sources), and both match the oracle; the log-sum-exp
+    output matches the oracle's within the output tolerance."""
+    batch, heads, ctx, q_lens, dtype, chunk = case
+    rng = _rng(400 + batch + heads)
+    d, dv, block = 576, 512, 128
+    _, kc, _, tables, ctx = _pa_inputs(rng, dev, batch, heads, 1, block, d, d, ctx, dtype, std=0.5)
+    rows = int(sum((1 if q_lens is None else q_lens[i]) for i in range(batch) if ctx[i] > 0))
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(int(rng.integers(1 << 30)))
+    q = (torch.rand((rows, heads, d), generator=gen) * 2 - 1).to(dtype).to(dev)
+    q_nope, q_rope = q[..., :dv].contiguous(), q[..., dv:].contiguous()
+    k_nope, k_rope = kc[..., :dv].contiguous(), kc[..., dv:].contiguous()
+    scale = 1.0 / math.sqrt(192.0)
+    want_lse = np.zeros((rows, heads), np.float32)
+    want = oracle_pa(oracle, q, kc, None, tables, ctx, scale, mla_dv=dv, q_lens=q_lens, lse_out=want_lse)
+    for kernel in (binding.ATBMI_PA_KERNEL_SCALAR, binding.ATBMI_PA_KERNEL_AUTO):
+        lse = torch.zeros((rows, heads), dtype=dtype, device=dev)
+        got = pa_decode_cabi(binding, stream, q_nope, k_nope, None, tables, ctx, scale, mla_dv=dv, kernel=kernel,
+                             q_lens=q_lens, q_rope=q_rope, k_rope=k_rope, lse=lse, chunk_tokens=chunk)
+        assert_close(got, want, TOL[dtype], "split kernel=%d" % kernel)
+        assert_close(lse, want_lse, TOL[dtype], "lse kernel=%d" % kernel)
+        lse2 = torch.zeros_like(lse)
+        combined = pa_decode_cabi(binding, stream, q, kc, None, tables, ctx, scale, mla_dv=dv, kernel=kernel,
+                                  q_lens=q_lens, lse=lse2, chunk_tokens=chunk)
+        assert torch.equal(got, combined) and torch.equal(lse, lse2)
+
+
+def test_lse_output_of_plain_and_masked_decode(binding, oracle, dev, stream):
+    """The log-sum-exp output is not tied to the latent layouts: separate K and V caches, a mask, rows
+    split over ranges and rows written directly."""
+    rng = _rng(420)
+    heads, kv_heads, d, block = 32, 8, 128, 128
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, 5, heads, kv_heads, block, d, d, [3000, 40, 0, 129, 1000],
+                                        torch.float16)
+    mask, _ = _mask_tensor(oracle, rng, dev, "alibi4", ctx, heads, 3000, torch.float16)
+    scale = 1.0 / math.sqrt(d)
+    want_lse = np.zeros((5, heads), np.float32)
+    want = oracle_pa(oracle, q, kc, vc, tables, ctx, scale, mask=mask, lse_out=want_lse)
+    for kernel in (binding.ATBMI_PA_KERNEL_SCALAR, binding.ATBMI_PA_KERNEL_AUTO):
+        lse = torch.zeros((5, heads), dtype=torch.float16, device=dev)
+        got = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, kernel=kernel, mask=mask, lse=lse)
+        assert_close(got, want, 1e-3, "out kernel=%d" % kernel)
+        assert_close(lse[:4], want_lse[:4], 2e-3, "lse kernel=%d" % kernel)  # |lse| ~ 8: fp16 spacing 4e-3..8e-3
+        assert torch.all(lse[4] == 0)
+
+
 # ------------------------------------------------------------------ several query tokens per sequence
 def _spec_mask(rng, dev, kind, ctx, q_lens, dtype):
     """The masks of the reference's multi-token tests: "query" — one row per query row, the

@@ -400,6 +400,49 @@ def test_multi_token_causal_mask_equals_growing_contexts(oracle):
                           oracle.paged_attention(q, kc, vc, tables, ctx, 0.3))
 
 
+# ---------------------------------------------------------------- log-sum-exp output
+def test_lse_closed_forms_and_logsumexp(oracle):
+    from scipy.special import logsumexp
+    rng = _rng(50)
+    q, kc, vc, tables, ctx = _paged_case(rng, batch=4, heads=4, kv_heads=2, max_ctx=13)
+    ctx[2] = 0
+    mask = rng.standard_normal((4, 4, 1, 13)).astype(np.float32)
+    lse = np.full((4, 4), 77.0, np.float32)
+    oracle.paged_attention(q, kc, vc, tables, ctx, 0.3, mask=mask, lse_out=lse)
+    row = 0
+    for i in range(4):
+        if ctx[i] == 0:
+            continue
+        keys = oracle.gather_rows(kc, tables[i], ctx[i]).astype(np.float64)
+        for h in range(4):
+            scores = keys[:, h // 2, :] @ q[row, h].astype(np.float64) * 0.3 + mask[i, h, 0, :ctx[i]]
+            assert abs(lse[row, h] - logsumexp(scores)) < 1e-5
+        row += 1
+    assert np.all(lse[3] == 77.0)  # only three rows are written
+    # one token: the score itself; n equal keys: the score plus log n
+    one = np.zeros(2, np.float32)
+    k1 = rng.standard_normal((1, 1, 8)).astype(np.float32)
+    q1 = rng.standard_normal((2, 8)).astype(np.float32)
+    oracle.attention_one(q1, k1, k1, 0.5, lse_out=one)
+    np.testing.assert_allclose(one, (q1 @ k1[0, 0]) * 0.5, rtol=1e-6)
+    oracle.attention_one(q1, np.repeat(k1, 7, axis=0), np.repeat(k1, 7, axis=0), 0.5, lse_out=one)
+    np.testing.assert_allclose(one, (q1 @ k1[0, 0]) * 0.5 + math.log(7.0), rtol=1e-6)
+
+
+def test_lse_of_a_split_context_is_logaddexp_of_the_parts(oracle):
+    rng = _rng(51)
+    qv = rng.standard_normal((4, 16)).astype(np.float32)
+    keys = rng.standard_normal((40, 2, 16)).astype(np.float32)
+    vals = rng.standard_normal((40, 2, 8)).astype(np.float32)
+    whole, a, b = (np.zeros(4, np.float32) for _ in range(3))
+    o = oracle.attention_one(qv, keys, vals, 0.3, lse_out=whole)
+    oa = oracle.attention_one(qv, keys[:17], vals[:17], 0.3, lse_out=a)
+    ob = oracle.attention_one(qv, keys[17:], vals[17:], 0.3, lse_out=b)
+    np.testing.assert_allclose(whole, np.logaddexp(a, b), rtol=1e-6)
+    wa = np.exp(a - whole)[:, None]
+    np.testing.assert_allclose(o, wa * oa + (1 - wa) * ob, rtol=1e-5, atol=1e-6)
+
+
 def test_int8_dequant_channel_indexing_and_identity(oracle):
     rng = _rng(11)
     q, _, _, tables, ctx = _paged_case(rng, heads=4, kv_heads=2, d=8, dv=8)
