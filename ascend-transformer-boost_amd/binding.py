@@ -84,6 +84,21 @@ class ReshapeAndCacheParam(ctypes.Structure):
             setattr(self, k, v)
 
 
+class MultiLatentAttentionParam(ctypes.Structure):
+    """Byte image of atb::infer::MultiLatentAttentionParam (64 bytes)."""
+    _fields_ = [("headNum", ctypes.c_int32), ("qkScale", ctypes.c_float), ("kvHeadNum", ctypes.c_int32),
+                ("maskType", ctypes.c_int32), ("calcType", ctypes.c_int32), ("cacheMode", ctypes.c_uint8),
+                ("windowSize", ctypes.c_uint32), ("maskUseStatusType", ctypes.c_int32), ("rsv", ctypes.c_uint8 * 32)]
+
+    def __init__(self, **kw):
+        super().__init__()
+        self.qkScale = 1.0
+        for k, v in kw.items():
+            if not hasattr(self, k):
+                raise AttributeError("MultiLatentAttentionParam has no field " + k)
+            setattr(self, k, v)
+
+
 class AtbmiPaShape(ctypes.Structure):
     _fields_ = [
         ("qDtype", ctypes.c_int32), ("kvDtype", ctypes.c_int32), ("numHeads", ctypes.c_int32),
@@ -173,6 +188,7 @@ def atb():
         lib.atb_c_quant_param_convert.restype = None
         lib.atb_c_sizeof_paged_attention_param.restype = u64
         lib.atb_c_sizeof_reshape_and_cache_param.restype = u64
+        lib.atb_c_sizeof_multi_latent_attention_param.restype = u64
         _atb = lib
     return _atb
 

@@ -95,6 +95,12 @@ int32_t atb_c_create_operation(const char *opName, const void *param, uint64_t p
         memcpy(static_cast<void *>(&p), param, sizeof(p));
         return atb::CreateOperation(p, out);
     }
+    if (!strcmp(opName, "MultiLatentAttentionOperation") &&
+        paramSize == sizeof(atb::infer::MultiLatentAttentionParam)) {
+        atb::infer::MultiLatentAttentionParam p;
+        memcpy(static_cast<void *>(&p), param, sizeof(p));
+        return atb::CreateOperation(p, out);
+    }
     return atb::ERROR_INVALID_PARAM;
 }
 
@@ -210,6 +216,11 @@ uint64_t atb_c_sizeof_paged_attention_param(void)
 uint64_t atb_c_sizeof_reshape_and_cache_param(void)
 {
     return sizeof(atb::infer::ReshapeAndCacheParam);
+}
+
+uint64_t atb_c_sizeof_multi_latent_attention_param(void)
+{
+    return sizeof(atb::infer::MultiLatentAttentionParam);
 }
 
 } // extern "C"

@@ -1,0 +1,470 @@
+// MultiLatentAttentionOperation on MI355X: decode attention over the split
+// latent cache (512 latent + 64 rotary channels per token, one KV head).
+//
+// Creation-time checks, tensor counts, InferShape and the dim checks follow the
+// reference operator (reference src/ops/ops_infer/multi_latent_attention/
+// multi_latent_attention_operation.cpp: 58-89 create, 91-148 decode param rules,
+// 150-173 ranges, 175-206 prefill rules, 245-293 counts and InferShape, 350-392
+// QKVDimCheck, 478-490 qSeqlen, 558-620 DimCheck). Context and query lengths are
+// read from hostData during Setup, as the reference runner does
+// (src/ops/ops_infer/multi_latent_attention/param.cpp).
+//
+// Implemented: cacheMode KROPE_CTKV with fp16/bf16 tensors; calcType UNDEFINED,
+// SPEC (qSeqlen, optionally with the MASK_TYPE_SPEC mask), RING and
+// SPEC_AND_RING (second output: log-sum-exp). The fractal-NZ cache modes, the
+// prefill calcType, the MASK_FREE / CAUSAL_MASK / SWA_NORM masks and
+// maskUseStatus are legal in the reference but not implemented here; such
+// params are rejected at creation with ERROR_INVALID_PARAM.
+//
+// The kernels are those of PagedAttention's combined-cache variant reading
+// each query and key row from two tensors.
+#include <new>
+#include "atb/infer_op_params.h"
+#include "atb/utils.h"
+#include "atbmi_kernels.h"
+#include "log.h"
+#include "operation_base.h"
+
+namespace atb {
+namespace {
+using Param = infer::MultiLatentAttentionParam;
+
+constexpr size_t QUERY = 0, QUERY_ROPE = 1, KV_CACHE = 2, KV_CACHE_ROPE = 3, BLOCK_TABLES = 4, CONTEXT_LENS = 5;
+constexpr int64_t LATENT_DIM = 512;
+constexpr int64_t ROPE_DIM = 64;
+constexpr int64_t DECODER_BLOCK_SIZE = 128;
+constexpr int64_t MAX_BATCH = 8192;
+
+bool IsSpec(const Param &p)
+{
+    return p.calcType == Param::CALC_TYPE_SPEC || p.calcType == Param::CALC_TYPE_SPEC_AND_RING;
+}
+
+bool IsRing(const Param &p)
+{
+    return p.calcType == Param::CALC_TYPE_RING || p.calcType == Param::CALC_TYPE_SPEC_AND_RING;
+}
+
+bool HasMaskInput(const Param &p)
+{
+    return p.maskType != Param::UNDEFINED && p.maskType != Param::MASK_TYPE_CAUSAL_MASK;
+}
+
+// Reference :150-173.
+bool ParamRangeCheck(const Param &p)
+{
+    if (p.qkScale <= 0 || p.qkScale > 1) {
+        ATB_LOG(ERROR) << "qkScale should be > 0 and <= 1";
+        return false;
+    }
+    if (p.maskType < Param::UNDEFINED || p.maskType > Param::MASK_TYPE_SWA_NORM) {
+        ATB_LOG(ERROR) << "invalid maskType";
+        return false;
+    }
+    if (p.calcType < Param::CALC_TYPE_UNDEFINED || p.calcType > Param::CALC_TYPE_PREFILL) {
+        ATB_LOG(ERROR) << "invalid calcType";
+        return false;
+    }
+    if (p.cacheMode > Param::NZCACHE) {
+        ATB_LOG(ERROR) << "invalid cacheMode";
+        return false;
+    }
+    return true;
+}
+
+// Reference :91-148 (decode).
+bool ParamCheck(const Param &p)
+{
+    if (p.headNum != 8 && p.headNum != 16 && p.headNum != 32 && p.headNum != 64 && p.headNum != 128) {
+        ATB_LOG(ERROR) << "headNum should be one of 8, 16, 32, 64, 128";
+        return false;
+    }
+    if (p.kvHeadNum != 1) {
+        ATB_LOG(ERROR) << "kvHeadNum should be 1, only MQA is supported";
+        return false;
+    }
+    if (p.cacheMode == Param::KVCACHE) {
+        ATB_LOG(ERROR) << "cacheMode KVCACHE is not supported";
+        return false;
+    }
+    if (!IsSpec(p) && p.maskType != Param::UNDEFINED) {
+        ATB_LOG(ERROR) << "only CALC_TYPE_SPEC takes a mask";
+        return false;
+    }
+    if (IsSpec(p) && p.maskType == Param::MASK_TYPE_SWA_NORM) {
+        ATB_LOG(ERROR) << "decode with CALC_TYPE_SPEC does not take the SWA_NORM mask";
+        return false;
+    }
+    if (p.cacheMode == Param::INT8_NZCACHE && IsRing(p) && p.maskType != Param::UNDEFINED) {
+        ATB_LOG(ERROR) << "int8 NZ cache with log-sum-exp output does not take a mask";
+        return false;
+    }
+    if (p.maskUseStatusType < Param::MASK_USE_STATUS_TYPE_UNDEFINED ||
+        p.maskUseStatusType >= Param::MASK_USE_STATUS_TYPE_MAX) {
+        ATB_LOG(ERROR) << "invalid maskUseStatusType";
+        return false;
+    }
+    if (p.maskUseStatusType == Param::MASK_USE_STATUS_TYPE_BATCH_MASK && p.calcType != Param::CALC_TYPE_SPEC_AND_RING) {
+        ATB_LOG(ERROR) << "maskUseStatus needs CALC_TYPE_SPEC_AND_RING";
+        return false;
+    }
+    if (p.maskType == Param::MASK_TYPE_SWA_NORM && p.windowSize <= 0) {
+        ATB_LOG(ERROR) << "windowSize in swa mode should be greater than 0";
+        return false;
+    }
+    return true;
+}
+
+// Reference :175-206 (prefill).
+bool ParamPrefillCheck(const Param &p)
+{
+    if (p.headNum < 1 || p.headNum > 128) {
+        ATB_LOG(ERROR) << "headNum should be >= 1 and <= 128";
+        return false;
+    }
+    if (p.maskType != Param::MASK_TYPE_CAUSAL_MASK && p.headNum != p.kvHeadNum) {
+        ATB_LOG(ERROR) << "prefill: headNum should equal kvHeadNum";
+        return false;
+    }
+    if (p.maskType != Param::UNDEFINED && p.maskType != Param::MASK_TYPE_MASK_FREE &&
+        p.maskType != Param::MASK_TYPE_CAUSAL_MASK && p.maskType != Param::MASK_TYPE_SWA_NORM) {
+        ATB_LOG(ERROR) << "prefill: maskType should be UNDEFINED, MASK_FREE, CAUSAL_MASK or SWA_NORM";
+        return false;
+    }
+    if (p.cacheMode != Param::KROPE_CTKV) {
+        ATB_LOG(ERROR) << "prefill: cacheMode should be KROPE_CTKV";
+        return false;
+    }
+    if (p.maskType == Param::MASK_TYPE_SWA_NORM && p.windowSize <= 0) {
+        ATB_LOG(ERROR) << "prefill: windowSize in swa mode should be greater than 0";
+        return false;
+    }
+    return true;
+}
+
+// Features that are legal in the reference but have no MI355X kernel yet.
+bool ImplementedCheck(const Param &p)
+{
+    const char *what = nullptr;
+    if (p.calcType == Param::CALC_TYPE_PREFILL) {
+        what = "the prefill calcType";
+    } else if (p.cacheMode != Param::KROPE_CTKV) {
+        what = "fractal-NZ caches";
+    } else if (p.maskType != Param::UNDEFINED && p.maskType != Param::MASK_TYPE_SPEC) {
+        what = "this maskType";
+    } else if (p.maskUseStatusType != Param::MASK_USE_STATUS_TYPE_UNDEFINED) {
+        what = "maskUseStatus";
+    }
+    if (what) {
+        ATB_LOG(ERROR) << "MultiLatentAttention: " << what << " not implemented on MI355X";
+        return false;
+    }
+    return true;
+}
+
+// The dtype table of the implemented sections of the reference
+// ops_configs/atb_ops_info.ini (:6669-6690 base, :6691-6715 Mask, :6716-6740 IsRing,
+// :6772-6824 Qlens / QlensIsRing, :6859-6917 MaskQlens / MaskQlensIsRing).
+OpIr MakeIr(const Param &p)
+{
+    OpIr ir;
+    for (aclDataType q : {ACL_FLOAT16, ACL_BF16}) {
+        IrCombo c;
+        c.inDtypes = {q, q, q, q, ACL_INT32, ACL_INT32};
+        if (HasMaskInput(p)) {
+            c.inDtypes.push_back(q);
+        }
+        if (IsSpec(p)) {
+            c.inDtypes.push_back(ACL_INT32);
+        }
+        c.inFormats.assign(c.inDtypes.size(), ACL_FORMAT_ND);
+        c.outDtypes = {q};
+        if (IsRing(p)) {
+            c.outDtypes.push_back(q);
+        }
+        c.outFormats.assign(c.outDtypes.size(), ACL_FORMAT_ND);
+        ir.push_back(c);
+    }
+    return ir;
+}
+
+class MultiLatentAttentionOperation : public OperationBase {
+public:
+    explicit MultiLatentAttentionOperation(const Param &param)
+        : OperationBase("MultiLatentAttentionOperation"), param_(param), irTable_(MakeIr(param))
+    {
+        ir_ = &irTable_;
+        size_t next = CONTEXT_LENS + 1;
+        if (HasMaskInput(param)) {
+            maskIdx_ = next++;
+        }
+        if (IsSpec(param)) {
+            qLensIdx_ = next++;
+        }
+        inputNum_ = static_cast<uint32_t>(next);
+    }
+
+    ~MultiLatentAttentionOperation() override
+    {
+        if (plan_) {
+            atbmi_pa_plan_destroy(plan_);
+        }
+    }
+
+    uint32_t GetInputNum() const override { return inputNum_; }
+    uint32_t GetOutputNum() const override { return IsRing(param_) ? 2 : 1; }
+
+protected:
+    // Reference :268-283.
+    Status InferShapeImpl(const SVector<TensorDesc> &in, SVector<TensorDesc> &out) const override
+    {
+        out.at(0) = in.at(QUERY);
+        out.at(0).dtype = in.at(QUERY_ROPE).dtype;
+        if (IsRing(param_)) {
+            out.at(1) = out.at(0);
+            out.at(1).shape.dims[2] = 1;
+        }
+        return NO_ERROR;
+    }
+
+    Status InferShapeCheckImpl(const SVector<TensorDesc> &in) const override { return DimCheck(in); }
+
+    Status SetupCheckImpl(const SVector<Tensor> &inTensors, const SVector<Tensor> &outTensors) const override
+    {
+        (void)outTensors;
+        SVector<TensorDesc> in;
+        for (size_t i = 0; i < inTensors.size(); ++i) {
+            in.push_back(inTensors.at(i).desc);
+        }
+        return DimCheck(in);
+    }
+
+    Status PlanImpl(const VariantPack &pack, uint64_t &workspaceSize) override
+    {
+        const Tensor &q = pack.inTensors.at(QUERY);
+        const Tensor &kv = pack.inTensors.at(KV_CACHE);
+        const Tensor &tables = pack.inTensors.at(BLOCK_TABLES);
+        const Tensor &lens = pack.inTensors.at(CONTEXT_LENS);
+        const Tensor &out = pack.outTensors.at(0);
+        if (!lens.hostData) {
+            ATB_LOG(ERROR) << "contextLens.hostData is null; the lengths are read on the host during Setup";
+            return ERROR_INVALID_PARAM;
+        }
+        const int32_t batch = static_cast<int32_t>(lens.desc.shape.dims[0]);
+        const int32_t *queryLens = nullptr;
+        if (qLensIdx_ != NONE) {
+            const Tensor &ql = pack.inTensors.at(qLensIdx_);
+            if (!ql.hostData) {
+                ATB_LOG(ERROR) << "qSeqlen.hostData is null; the lengths are read on the host during Setup";
+                return ERROR_INVALID_PARAM;
+            }
+            queryLens = static_cast<const int32_t *>(ql.hostData);
+        }
+        const Dims &o = out.desc.shape;
+        if (o.dimNum != 3 || o.dims[0] != q.desc.shape.dims[0] || o.dims[1] != param_.headNum ||
+            o.dims[2] != LATENT_DIM) {
+            ATB_LOG(ERROR) << "the output should be [numTokens, headNum, 512]";
+            return ERROR_INVALID_PARAM;
+        }
+        if (IsRing(param_)) {
+            const Dims &l = pack.outTensors.at(1).desc.shape;
+            if (l.dimNum != 3 || l.dims[0] != o.dims[0] || l.dims[1] != o.dims[1] || l.dims[2] != 1) {
+                ATB_LOG(ERROR) << "the log-sum-exp output should be [numTokens, headNum, 1]";
+                return ERROR_INVALID_PARAM;
+            }
+        }
+        int64_t maskLen = 0;
+        if (maskIdx_ != NONE) {
+            // one mask row per query token (reference tests/apitest/opstest/python/operations/
+            // multi_latent_attention/test_multi_latent_attention_mtp.py:262-274)
+            const Dims &m = pack.inTensors.at(maskIdx_).desc.shape;
+            if (m.dimNum != 2 || m.dims[0] != q.desc.shape.dims[0]) {
+                ATB_LOG(ERROR) << "the mask should be [numTokens, maxS]";
+                return ERROR_INVALID_PARAM;
+            }
+            maskLen = m.dims[1];
+            const int32_t *ctx = static_cast<const int32_t *>(lens.hostData);
+            for (int32_t i = 0; i < batch; ++i) {
+                if (ctx[i] > maskLen) {
+                    ATB_LOG(ERROR) << "mask covers " << maskLen << " positions but contextLens[" << i << "] is " << ctx[i];
+                    return ERROR_INVALID_PARAM;
+                }
+            }
+        }
+
+        AtbmiPaShape shape{};
+        shape.qDtype = q.desc.dtype == ACL_BF16 ? ATBMI_BF16 : ATBMI_F16;
+        shape.kvDtype = shape.qDtype;
+        shape.numHeads = param_.headNum;
+        shape.numKvHeads = 1;
+        shape.headDimK = static_cast<int32_t>(LATENT_DIM + ROPE_DIM);
+        shape.headDimV = static_cast<int32_t>(LATENT_DIM);
+        shape.blockSize = static_cast<int32_t>(kv.desc.shape.dims[1]);
+        shape.numBlocks = static_cast<int32_t>(kv.desc.shape.dims[0]);
+        shape.maxBlocksPerSeq = static_cast<int32_t>(tables.desc.shape.dims[1]);
+        shape.numQueryRows = static_cast<int32_t>(q.desc.shape.dims[0]);
+        shape.mlaCombined = 1;
+        shape.kernel = ATBMI_PA_KERNEL_AUTO;
+        shape.qkScale = param_.qkScale;
+        shape.ropeDim = static_cast<int32_t>(ROPE_DIM);
+        shape.hasMask = maskIdx_ != NONE ? 1 : 0;
+        shape.maskBatchStride = maskLen;
+        shape.maskLen = static_cast<int32_t>(maskLen);
+        shape.maskRowBy = maskIdx_ != NONE ? ATBMI_PA_MASK_ROW_QUERY : ATBMI_PA_MASK_ROW_SEQUENCE;
+        if (!plan_ || !SameShape(shape, planShape_)) {
+            if (plan_) {
+                atbmi_pa_plan_destroy(plan_);
+                plan_ = nullptr;
+            }
+            int rc = atbmi_pa_plan_create(&shape, &plan_);
+            if (rc != 0) {
+                ATB_LOG(ERROR) << "MultiLatentAttention plan: " << atbmi_last_error();
+                return rc;
+            }
+            planShape_ = shape;
+        }
+        int rc = atbmi_pa_plan_update_multi(plan_, static_cast<const int32_t *>(lens.hostData), queryLens, batch);
+        if (rc != 0) {
+            ATB_LOG(ERROR) << "MultiLatentAttention plan: " << atbmi_last_error();
+            return rc;
+        }
+        workspaceSize = atbmi_pa_plan_workspace_size(plan_);
+        return NO_ERROR;
+    }
+
+    Status LaunchImpl(const VariantPack &pack, uint8_t *workspace, uint64_t workspaceSize,
+                      aclrtStream stream) override
+    {
+        AtbmiPaTensors t{};
+        t.query = pack.inTensors.at(QUERY).deviceData;
+        t.queryRope = pack.inTensors.at(QUERY_ROPE).deviceData;
+        t.keyCache = pack.inTensors.at(KV_CACHE).deviceData;
+        t.keyRopeCache = pack.inTensors.at(KV_CACHE_ROPE).deviceData;
+        t.blockTables = static_cast<const int32_t *>(pack.inTensors.at(BLOCK_TABLES).deviceData);
+        if (maskIdx_ != NONE) {
+            t.mask = pack.inTensors.at(maskIdx_).deviceData;
+        }
+        t.out = pack.outTensors.at(0).deviceData;
+        if (IsRing(param_)) {
+            t.lse = pack.outTensors.at(1).deviceData;
+        }
+        int rc = atbmi_pa_decode(plan_, &t, workspace, workspaceSize, stream);
+        if (rc != 0) {
+            ATB_LOG(ERROR) << "MultiLatentAttention launch failed: " << atbmi_last_error();
+        }
+        return rc;
+    }
+
+private:
+    static constexpr size_t NONE = ~static_cast<size_t>(0);
+
+    static bool SameShape(const AtbmiPaShape &a, const AtbmiPaShape &b)
+    {
+        return a.qDtype == b.qDtype && a.numHeads == b.numHeads && a.blockSize == b.blockSize &&
+               a.numBlocks == b.numBlocks && a.maxBlocksPerSeq == b.maxBlocksPerSeq &&
+               a.numQueryRows == b.numQueryRows && a.qkScale == b.qkScale && a.hasMask == b.hasMask &&
+               a.maskBatchStride == b.maskBatchStride && a.maskLen == b.maskLen;
+    }
+
+    // Reference :558-620 (DimCheck) with :350-392 (QKVDimCheck) and :478-490 (DimCheckSpec).
+    Status DimCheck(const SVector<TensorDesc> &in) const
+    {
+        if (in.at(QUERY).shape.dimNum != 3 || in.at(QUERY_ROPE).shape.dimNum != 3 || in.at(KV_CACHE).shape.dimNum != 4 ||
+            in.at(KV_CACHE_ROPE).shape.dimNum != 4 || in.at(BLOCK_TABLES).shape.dimNum != 2 ||
+            in.at(CONTEXT_LENS).shape.dimNum != 1) {
+            ATB_LOG(ERROR) << "expected dims: query 3, queryRope 3, kvCache 4, kvCacheRope 4, blockTables 2, contextLens 1";
+            return ERROR_INVALID_TENSOR_DIM_NUM;
+        }
+        const int64_t numTokens = in.at(QUERY).shape.dims[0];
+        const int64_t batch = in.at(BLOCK_TABLES).shape.dims[0];
+        if (batch > MAX_BATCH) {
+            ATB_LOG(ERROR) << "batch should be <= " << MAX_BATCH;
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (param_.calcType == Param::CALC_TYPE_UNDEFINED && numTokens != batch) {
+            ATB_LOG(ERROR) << "numTokens and batch should be the same in the decode stage";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (in.at(CONTEXT_LENS).shape.dims[0] != batch) {
+            ATB_LOG(ERROR) << "dim 0 of blockTables and contextLens should be the same";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        const Dims &kv = in.at(KV_CACHE).shape;
+        const Dims &kr = in.at(KV_CACHE_ROPE).shape;
+        if (kv.dims[1] != DECODER_BLOCK_SIZE) {
+            ATB_LOG(ERROR) << "decoder blockSize should be " << DECODER_BLOCK_SIZE << ", got " << kv.dims[1];
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (in.at(QUERY_ROPE).shape.dims[0] != numTokens) {
+            ATB_LOG(ERROR) << "dim 0 of query and queryRope should be the same";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (kr.dims[0] != kv.dims[0] || kr.dims[1] != kv.dims[1]) {
+            ATB_LOG(ERROR) << "dim 0 and dim 1 of kvCache and kvCacheRope should be the same";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (kv.dims[2] != param_.kvHeadNum || kr.dims[2] != param_.kvHeadNum) {
+            ATB_LOG(ERROR) << "dim 2 of kvCache and kvCacheRope should equal kvHeadNum";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (in.at(QUERY).shape.dims[1] != param_.headNum || in.at(QUERY_ROPE).shape.dims[1] != param_.headNum) {
+            ATB_LOG(ERROR) << "dim 1 of query and queryRope should equal headNum";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (in.at(QUERY).shape.dims[2] != LATENT_DIM || kv.dims[3] != LATENT_DIM) {
+            ATB_LOG(ERROR) << "head size of query and kvCache should be 512";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (in.at(QUERY_ROPE).shape.dims[2] != ROPE_DIM || kr.dims[3] != ROPE_DIM) {
+            ATB_LOG(ERROR) << "head size of queryRope and kvCacheRope should be 64";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (qLensIdx_ != NONE) {
+            const Dims &ql = in.at(qLensIdx_).shape;
+            if (ql.dimNum != 1) {
+                ATB_LOG(ERROR) << "qSeqlen should have 1 dim";
+                return ERROR_INVALID_TENSOR_DIM_NUM;
+            }
+            if (ql.dims[0] != batch) {
+                ATB_LOG(ERROR) << "dim 0 of qSeqlen should equal dim 0 of contextLens";
+                return ERROR_INVALID_TENSOR_DIM;
+            }
+        }
+        return NO_ERROR;
+    }
+
+    Param param_;
+    OpIr irTable_;
+    size_t maskIdx_ = NONE;
+    size_t qLensIdx_ = NONE;
+    uint32_t inputNum_ = 6;
+    AtbmiPaPlan *plan_ = nullptr;
+    AtbmiPaShape planShape_{};
+};
+} // namespace
+
+template <> Status CreateOperation(const infer::MultiLatentAttentionParam &opParam, Operation **operation)
+{
+    if (operation == nullptr) {
+        return ERROR_INVALID_PARAM;
+    }
+    if (!ParamRangeCheck(opParam)) {
+        return ERROR_INVALID_PARAM;
+    }
+    if (opParam.calcType == Param::CALC_TYPE_PREFILL ? !ParamPrefillCheck(opParam) : !ParamCheck(opParam)) {
+        return ERROR_INVALID_PARAM;
+    }
+    if (!ReservedIsZero(opParam)) {
+        ATB_LOG(ERROR) << "MultiLatentAttentionParam rsv has a non-zero byte";
+        return ERROR_INVALID_PARAM;
+    }
+    if (!ImplementedCheck(opParam)) {
+        return ERROR_INVALID_PARAM;
+    }
+    *operation = new (std::nothrow) MultiLatentAttentionOperation(opParam);
+    if (*operation == nullptr) {
+        return ERROR_OUT_OF_HOST_MEMORY;
+    }
+    return NO_ERROR;
+}
+} // namespace atb

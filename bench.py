@@ -42,6 +42,8 @@ DESCRIPTIONS = {
                "32 q heads, 8 kv heads, d128, block 128, ctx U[1024,4096], bf16",
     "c3": "C3 int8-KV 70B-shaped decode: batch 128, 64 q heads, 8 kv heads, d128, block 128, ctx U[2048,8192], fp16 q",
     "c4": "C4 skewed long-context fp16 decode: batch 16, 32 q heads, 8 kv heads, d128, ctx lognormal(median 8k) in [256,32768]",
+    "c5_split": "C5 through MultiLatentAttentionOperation (cacheMode KROPE_CTKV: 512 latent + 64 rotary channels in "
+                "two caches): batch 64, 128 q heads, block 128, ctx U[2048,4096], bf16",
     "c5": "C5 MLA bf16 decode: batch 64, 128 q heads, 1 latent kv head, d576/dv512, block 128, ctx U[2048,4096]",
 }
 
@@ -138,14 +140,30 @@ def main():
     pa_param = b.PagedAttentionParam(headNum=cfg["heads"], kvHeadNum=cfg["kv_heads"], qkScale=scale,
                                      quantType=1 if int8 else 0, mlaVHeadSize=cfg["dv"] if mla else 0,
                                      maskType=mask_type, calcType=1 if q_len > 1 else 0)
-    pa = b.OperationRunner("PagedAttentionOperation", pa_param, ctx)
+    split = bool(cfg.get("split"))
+    if split:
+        pa = b.OperationRunner("MultiLatentAttentionOperation", b.MultiLatentAttentionParam(
+            headNum=cfg["heads"], kvHeadNum=1, qkScale=scale, cacheMode=1), ctx)
+    else:
+        pa = b.OperationRunner("PagedAttentionOperation", pa_param, ctx)
     rac = None
     k = b.kernels()
     lens_host = step["context_lens"]
     host_inputs = {}
     with torch.cuda.stream(stream):
         lens_dev = lens_host.to(dev)
-        if mla:
+        if split:
+            dv = cfg["dv"]
+            nope, rope = step["key_cache"][..., :dv].contiguous(), step["key_cache"][..., dv:].contiguous()
+            pa_in = [step["q"][..., :dv].contiguous(), step["q"][..., dv:].contiguous(), nope, rope,
+                     step["block_tables"], lens_dev]
+            host_idx = 5
+            # the latent and rotary rows of the new token go to their caches as the K and V of one cache write
+            rac = b.OperationRunner("ReshapeAndCacheOperation", b.ReshapeAndCacheParam(), ctx)
+            rac_in = [step["k_new"][..., :dv].contiguous(), step["k_new"][..., dv:].contiguous(), nope, rope,
+                      step["slot_mapping"]]
+            rac_out = [nope, rope]  # (the combined copy stays for the CPU baseline, which concatenates anyway)
+        elif mla:
             pa_in = [step["q"], step["key_cache"], step["block_tables"], lens_dev]
             host_idx = 3
             rac = b.OperationRunner("ReshapeAndCacheOperation", b.ReshapeAndCacheParam(kvCacheCfg=1), ctx)
@@ -225,8 +243,8 @@ def main():
         "vs_baseline": None,
         "dtype": "int8" if int8 else cfg["dtype"],
         "data": "synthetic",
-        "config": {"workload": DESCRIPTIONS[args.config], "step": "PagedAttention only" if args.attention_only else
-                   "ReshapeAndCache + PagedAttention (Setup + Execute each)",
+        "config": {"workload": DESCRIPTIONS[args.config], "step": ("%s only" if args.attention_only else "ReshapeAndCache + %s (Setup + Execute each)") % (
+                       "MultiLatentAttention" if split else "PagedAttention"),
                    "context_tokens": int(step["layout"]["ctx"].sum())},
         "roofline": {"bound": "hbm", "kernel": "paged attention decode", "achieved": achieved,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,

@@ -101,7 +101,55 @@ struct PagedAttentionParam {
     uint8_t rsv[64] = {0}; // must stay zero
 };
 
+// Decode attention over the compressed latent cache of multi-head latent
+// attention, with the query and the cache rows given as 512 latent channels
+// plus 64 rotary channels in two tensors each; V is the 512 latent channels.
+// (reference include/atb/infer_op_params.h:2899-2984)
+struct MultiLatentAttentionParam {
+    int32_t headNum = 0;   // query heads: 8, 16, 32, 64 or 128
+    float qkScale = 1.0;   // multiplies Q.K^T before the softmax, in (0, 1]
+    int32_t kvHeadNum = 0; // 1
+
+    enum MaskType : int {
+        UNDEFINED = 0,         // no mask input
+        MASK_TYPE_SPEC,        // one mask row per query token, with CALC_TYPE_SPEC
+        MASK_TYPE_MASK_FREE,   // compressed causal mask; not implemented on MI355X
+        MASK_TYPE_CAUSAL_MASK, // mask generated inside the kernel; not implemented on MI355X
+        MASK_TYPE_SWA_NORM     // sliding window (prefill); not implemented on MI355X
+    };
+    MaskType maskType = UNDEFINED;
+
+    enum CalcType : int {
+        CALC_TYPE_UNDEFINED = 0, // one query token per sequence
+        CALC_TYPE_SPEC,          // qSeqlen input: several query tokens per sequence
+        CALC_TYPE_RING,          // second output: the log-sum-exp of every row
+        CALC_TYPE_SPEC_AND_RING, // both
+        CALC_TYPE_PREFILL        // not implemented on MI355X
+    };
+    CalcType calcType = CALC_TYPE_UNDEFINED;
+
+    enum CacheMode : uint8_t {
+        KVCACHE = 0,  // one 576-channel cache; rejected by the reference itself
+        KROPE_CTKV,   // latent cache [blocks, 128, 1, 512] + rotary cache [blocks, 128, 1, 64]
+        INT8_NZCACHE, // int8 fractal-NZ caches; not implemented on MI355X
+        NZCACHE       // 16-bit fractal-NZ caches; not implemented on MI355X
+    };
+    CacheMode cacheMode = KVCACHE;
+
+    uint32_t windowSize = 0;
+
+    enum MaskUseStatusType : int {
+        MASK_USE_STATUS_TYPE_UNDEFINED = 0,
+        MASK_USE_STATUS_TYPE_BATCH_MASK, // per-sequence switch of the mask; not implemented on MI355X
+        MASK_USE_STATUS_TYPE_MAX
+    };
+    MaskUseStatusType maskUseStatusType = MASK_USE_STATUS_TYPE_UNDEFINED;
+
+    uint8_t rsv[32] = {0}; // must stay zero
+};
+
 static_assert(sizeof(ReshapeAndCacheParam) == 24, "ReshapeAndCacheParam ABI size");
+static_assert(sizeof(MultiLatentAttentionParam) == 64, "MultiLatentAttentionParam ABI size");
 static_assert(sizeof(PagedAttentionParam) == 120, "PagedAttentionParam ABI size");
 
 } // namespace infer

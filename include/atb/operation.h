@@ -34,7 +34,8 @@ public:
                            Context *context) = 0;
 };
 
-// Specialised for infer::PagedAttentionParam and infer::ReshapeAndCacheParam.
+// Specialised for infer::PagedAttentionParam, infer::ReshapeAndCacheParam and
+// infer::MultiLatentAttentionParam.
 template <typename OpParam> Status CreateOperation(const OpParam &opParam, Operation **operation);
 
 Status DestroyOperation(Operation *operation);

@@ -38,9 +38,10 @@ int32_t atb_c_context_set_execute_type(void *context, int32_t type);
 /* atb::DestroyContext. */
 int32_t atb_c_destroy_context(void *context);
 
-/* atb::CreateOperation<infer::PagedAttentionParam> / <infer::ReshapeAndCacheParam>.
- * opName is "PagedAttentionOperation" or "ReshapeAndCacheOperation"; param
- * points at the bytes of the matching C++ param struct (120 / 24 bytes). */
+/* atb::CreateOperation<infer::PagedAttentionParam> / <infer::ReshapeAndCacheParam> /
+ * <infer::MultiLatentAttentionParam>. opName is "PagedAttentionOperation",
+ * "ReshapeAndCacheOperation" or "MultiLatentAttentionOperation"; param points at
+ * the bytes of the matching C++ param struct (120 / 24 / 64 bytes). */
 int32_t atb_c_create_operation(const char *opName, const void *param, uint64_t paramSize, void **operation);
 /* atb::DestroyOperation. */
 int32_t atb_c_destroy_operation(void *operation);
@@ -67,9 +68,11 @@ uint64_t atb_c_tensor_size(const AtbCTensor *tensor);
 /* atb::Utils::QuantParamConvert (reference include/atb/utils.h:82): fp32 bits into the low half of uint64. */
 void atb_c_quant_param_convert(const float *src, uint64_t *dest, uint64_t itemCount);
 
-/* sizeof(infer::PagedAttentionParam), sizeof(infer::ReshapeAndCacheParam). */
+/* sizeof(infer::PagedAttentionParam), sizeof(infer::ReshapeAndCacheParam),
+ * sizeof(infer::MultiLatentAttentionParam). */
 uint64_t atb_c_sizeof_paged_attention_param(void);
 uint64_t atb_c_sizeof_reshape_and_cache_param(void);
+uint64_t atb_c_sizeof_multi_latent_attention_param(void);
 
 #ifdef __cplusplus
 }

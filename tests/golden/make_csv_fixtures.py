@@ -6,10 +6,12 @@ param JSON + input dtypes/formats/shapes + output dtype/shape + the expected
 status, tagged C: for CreateOperation, I: for InferShape, S: for Setup):
     tests/apitest/opstest/csv/paged_attention.csv
     tests/apitest/opstest/csv/reshape_and_cache.csv
+    tests/apitest/opstest/csv/multi_latent_attention.csv
 Those rows are data, not code. This script copies the rows written for the
 Ascend910B feature set (the one this library mirrors) into
     tests/golden/paged_attention_cases.json
     tests/golden/reshape_and_cache_cases.json
+    tests/golden/multi_latent_attention_cases.json
 so the parity tests can run where the reference tree is absent.
 
 Run from the repository root in a container that has /root/reference:
@@ -72,3 +74,4 @@ if __name__ == "__main__":
         sys.exit("reference tree not found at " + REF)
     convert("paged_attention")
     convert("reshape_and_cache")
+    convert("multi_latent_attention")

@@ -623,6 +623,50 @@ def test_split_latent_layout_and_lse(binding, oracle, dev, stream, case):
         assert torch.equal(got, combined) and torch.equal(lse, lse2)
 
 
+@pytest.mark.parametrize("heads,dtype", [(128, torch.bfloat16), (32, torch.float16), (8, torch.float16)])
+def test_multi_latent_attention_operation(binding, oracle, dev, stream, heads, dtype):
+    """MultiLatentAttentionOperation, cacheMode KROPE_CTKV, through Setup / Execute: plain decode, with
+    the log-sum-exp output (CALC_TYPE_RING), several query tokens with the SPEC mask (CALC_TYPE_SPEC) and
+    both (CALC_TYPE_SPEC_AND_RING). Inputs: query, queryRope, kvCache, kvCacheRope, blockTables,
+    contextLens, [mask], [qSeqlen] (reference multi_latent_attention_operation.cpp:245-266)."""
+    rng = _rng(440 + heads)
+    d, dv, block = 576, 512, 128
+    ctx = np.array([700, 33, 1500, 128], dtype=np.int32)
+    _, kc, _, tables, ctx = _pa_inputs(rng, dev, 4, heads, 1, block, d, d, ctx, dtype, std=0.5)
+    k_nope, k_rope = kc[..., :dv].contiguous(), kc[..., dv:].contiguous()
+    q_lens = np.array([2, 1, 3, 1], dtype=np.int32)
+    scale = 1.0 / math.sqrt(192.0)
+    lens, qn = torch.from_numpy(ctx), torch.from_numpy(q_lens)
+    c = binding.Context(stream)
+    for calc in (0, 2, 1, 3):
+        multi, ring = calc in (1, 3), calc in (2, 3)
+        rows = int(q_lens.sum()) if multi else 4
+        q = (torch.rand((rows, heads, d)) * 2 - 1).to(dtype).to(dev)
+        ins = [q[..., :dv].contiguous(), q[..., dv:].contiguous(), k_nope, k_rope, tables, lens.to(dev)]
+        host = {5: lens}
+        mask = None
+        if multi:
+            mask = _spec_mask(rng, dev, "query", ctx, q_lens, dtype)
+            ins += [mask, qn.to(dev)]
+            host[7] = qn
+        op = binding.OperationRunner("MultiLatentAttentionOperation", binding.MultiLatentAttentionParam(
+            headNum=heads, kvHeadNum=1, qkScale=scale, cacheMode=1, calcType=calc, maskType=1 if multi else 0), c)
+        with torch.cuda.stream(stream):
+            outs = op.run(ins, host_inputs=host)
+        stream.synchronize()
+        assert len(outs) == (2 if ring else 1) and tuple(outs[0].shape) == (rows, heads, dv)
+        want_lse = np.zeros((rows, heads), np.float32)
+        want = oracle_pa(oracle, q, kc, None, tables, ctx, scale, mla_dv=dv, mask=mask,
+                         q_lens=q_lens if multi else None, mask_rows="query" if multi else "sequence",
+                         lse_out=want_lse)
+        assert_close(outs[0], want, TOL[dtype], "calcType %d" % calc)
+        if ring:
+            assert tuple(outs[1].shape) == (rows, heads, 1) and outs[1].dtype == dtype
+            assert_close(outs[1][..., 0], want_lse, TOL[dtype], "lse calcType %d" % calc)
+        op.close()
+    c.close()
+
+
 def test_lse_output_of_plain_and_masked_decode(binding, oracle, dev, stream):
     """The log-sum-exp output is not tied to the latent layouts: separate K and V caches, a mask, rows
     split over ranges and rows written directly."""

@@ -27,6 +27,7 @@ def _load(name):
 
 PA_CASES = _load("paged_attention")
 RAC_CASES = _load("reshape_and_cache")
+MLA_CASES = _load("multi_latent_attention")
 
 
 def _pa_unimplemented(p):
@@ -57,9 +58,18 @@ def _rac_unimplemented(p):
     return p.get("compressType", 0) in (1, 2) or p.get("kvCacheCfg", 0) == 2
 
 
+def _mla_unimplemented(p):
+    """Features of MultiLatentAttentionParam the reference accepts but this library rejects at creation:
+    the prefill calcType, the fractal-NZ cache modes, masks other than MASK_TYPE_SPEC, maskUseStatus."""
+    return (p.get("calcType", 0) == 4 or p.get("cacheMode", 0) in (2, 3) or p.get("maskType", 0) >= 2 or
+            p.get("maskUseStatusType", 0) != 0)
+
+
 def _make_param(binding, op, p):
     if op == "PagedAttentionOperation":
         return binding.PagedAttentionParam(**p)
+    if op == "MultiLatentAttentionOperation":
+        return binding.MultiLatentAttentionParam(**p)
     return binding.ReshapeAndCacheParam(**p)
 
 
@@ -98,6 +108,10 @@ def _run_case(binding, case, ctx):
                 qlens_index = lens_index + (2 if p.get("maskType", 0) != 0 else 1)
                 if qlens_index < len(case["in_shapes"]):
                     host[qlens_index] = np.ones((case["in_shapes"][qlens_index][0],), dtype=np.int32)
+        if case["op"] == "MultiLatentAttentionOperation" and len(case["in_shapes"]) > 5:
+            host[5] = np.full((case["in_shapes"][5][0],), 7, dtype=np.int32)
+            if case["param"].get("calcType", 0) in (1, 3):
+                host[len(case["in_shapes"]) - 1] = np.ones((case["in_shapes"][-1][0],), dtype=np.int32)
         ins = _tensors(binding, case["in_dtypes"], case["in_formats"], case["in_shapes"], host)
         outs = _tensors(binding, case["out_dtypes"], case["out_formats"], case["out_shapes"])
         st, _ = op.setup(ins, outs, ctx)
@@ -141,6 +155,11 @@ def test_paged_attention_table(binding, ctx, case):
            _pa_mask_shape_refused(case))
 
 
+@pytest.mark.parametrize("case", MLA_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
+def test_multi_latent_attention_table(binding, ctx, case):
+    _check(binding, case, ctx, _mla_unimplemented(case["param"]) and not case["expected"].startswith("C:"))
+
+
 @pytest.mark.parametrize("case", RAC_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
 def test_reshape_and_cache_table(binding, ctx, case):
     _check(binding, case, ctx, _rac_unimplemented(case["param"]) and not case["expected"].startswith("C:"))
@@ -153,6 +172,9 @@ def test_table_coverage():
     rac_dev = [c for c in RAC_CASES if _rac_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
     assert len(PA_CASES) == 81 and len(PA_CASES) - len(pa_dev) >= 72
     assert len(RAC_CASES) == 37 and len(RAC_CASES) - len(rac_dev) >= 25
+    # most MultiLatentAttention rows exercise the prefill calcType and the fractal-NZ caches, which are not built
+    mla_dev = [c for c in MLA_CASES if _mla_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
+    assert len(MLA_CASES) == 147 and len(MLA_CASES) - len(mla_dev) == 45
 
 
 def test_param_sizes(binding):
@@ -161,6 +183,9 @@ def test_param_sizes(binding):
     assert binding.atb().atb_c_sizeof_reshape_and_cache_param() == 24
     assert ctypes.sizeof(binding.PagedAttentionParam) == 120
     assert ctypes.sizeof(binding.ReshapeAndCacheParam) == 24
+    # :68
+    assert binding.atb().atb_c_sizeof_multi_latent_attention_param() == 64
+    assert ctypes.sizeof(binding.MultiLatentAttentionParam) == 64
 
 
 def test_reserved_bytes_must_be_zero(binding):
@@ -442,6 +467,81 @@ def test_several_query_tokens_inputs(binding, ctx):
     # MASK_TYPE_SPEC without CALC_TYPE_SPEC has no defined rows
     op = binding.Operation("PagedAttentionOperation", binding.PagedAttentionParam(headNum=32, kvHeadNum=16, maskType=3))
     assert op.status == e["ERROR_INVALID_PARAM"]
+
+
+def test_multi_latent_attention_counts_shapes_and_setup(binding, ctx):
+    """Tensor counts and InferShape per calcType (reference multi_latent_attention_operation.cpp:245-283),
+    host-side lengths, and the output shapes Setup insists on."""
+    e = binding.ERROR_CODE
+    mk = binding.MultiLatentAttentionParam
+    for kw, n_in, n_out in ((dict(), 6, 1), (dict(calcType=1), 7, 1), (dict(calcType=1, maskType=1), 8, 1),
+                            (dict(calcType=2), 6, 2), (dict(calcType=3, maskType=1), 8, 2)):
+        op = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07,
+                                                                   cacheMode=1, **kw))
+        assert op.ok and (op.input_num(), op.output_num()) == (n_in, n_out), kw
+        op.close()
+    for bad in (dict(headNum=12), dict(kvHeadNum=2), dict(cacheMode=0), dict(maskType=1), dict(qkScale=1.5),
+                dict(qkScale=0.0), dict(calcType=5), dict(cacheMode=2), dict(cacheMode=3), dict(calcType=4),
+                dict(calcType=1, maskType=2), dict(calcType=1, maskType=3), dict(calcType=1, maskType=4),
+                dict(calcType=3, maskUseStatusType=1)):
+        kw = dict(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1)
+        kw.update(bad)
+        assert binding.Operation("MultiLatentAttentionOperation", mk(**kw)).status == e["ERROR_INVALID_PARAM"], bad
+    p = mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1)
+    p.rsv[31] = 1
+    assert binding.Operation("MultiLatentAttentionOperation", p).status == e["ERROR_INVALID_PARAM"]
+
+    lens = np.array([10, 300, 0, 64], dtype=np.int32)
+    qlens = np.array([1, 3, 2, 2], dtype=np.int32)   # 6 query rows
+
+    def pack(rows=4, mask=None, with_qlens=False, lens_host=True, qlens_host=True, dtype="float16", block=128):
+        ins = [
+            binding.make_tensor(dtype, [rows, 32, 512], FAKE_DEVICE),
+            binding.make_tensor(dtype, [rows, 32, 64], FAKE_DEVICE),
+            binding.make_tensor(dtype, [16, block, 1, 512], FAKE_DEVICE),
+            binding.make_tensor(dtype, [16, block, 1, 64], FAKE_DEVICE),
+            binding.make_tensor("int32", [4, 3], FAKE_DEVICE),
+            binding.make_tensor("int32", [4], FAKE_DEVICE, host_ptr=lens.ctypes.data if lens_host else None),
+        ]
+        if mask is not None:
+            ins.append(binding.make_tensor(dtype, mask, FAKE_DEVICE))
+        if with_qlens:
+            ins.append(binding.make_tensor("int32", [4], FAKE_DEVICE, host_ptr=qlens.ctypes.data if qlens_host else None))
+        return ins
+
+    def outs(rows=4, lse=False, dtype="float16", width=512):
+        o = [binding.make_tensor(dtype, [rows, 32, width], FAKE_DEVICE)]
+        if lse:
+            o.append(binding.make_tensor(dtype, [rows, 32, 1], FAKE_DEVICE))
+        return o
+
+    ring = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1,
+                                                                 calcType=2))
+    st, descs = ring.infer_shape(pack(dtype="bf16"))
+    assert st == 0 and [[d.dims[i] for i in range(d.dimNum)] for d in descs] == [[4, 32, 512], [4, 32, 1]]
+    assert all(d.dtype == binding.ACL_DTYPE_BY_NAME["bf16"] for d in descs)
+    assert ring.setup(pack(), outs(lse=True), ctx)[0] == 0
+    assert ring.setup(pack(lens_host=False), outs(lse=True), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    assert ring.setup(pack(), outs(lse=True, width=576), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    assert ring.setup(pack(block=64), outs(lse=True), ctx)[0] == e["ERROR_INVALID_TENSOR_DIM"]
+    # only the plain decode calcType ties the token count to the batch (reference :577-580)
+    assert ring.setup(pack(rows=5), outs(rows=5, lse=True), ctx)[0] == 0
+    plain = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1))
+    assert plain.setup(pack(), outs(), ctx)[0] == 0
+    assert plain.setup(pack(rows=5), outs(rows=5), ctx)[0] == e["ERROR_INVALID_TENSOR_DIM"]
+    plain.close()
+    assert ring.setup(pack(dtype="bf16"), outs(lse=True), ctx)[0] == e["ERROR_INVALID_TENSOR_INI_MATCH"]
+    ring.close()
+
+    spec = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1,
+                                                                 calcType=1, maskType=1))
+    assert spec.setup(pack(rows=6, mask=[6, 300], with_qlens=True), outs(rows=6), ctx)[0] == 0
+    assert spec.setup(pack(rows=6, mask=[6, 299], with_qlens=True), outs(rows=6), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    assert spec.setup(pack(rows=6, mask=[5, 300], with_qlens=True), outs(rows=6), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    assert spec.setup(pack(rows=5, mask=[5, 300], with_qlens=True), outs(rows=5), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    assert spec.setup(pack(rows=6, mask=[6, 300], with_qlens=True, qlens_host=False), outs(rows=6), ctx)[0] == \
+        e["ERROR_INVALID_PARAM"]
+    spec.close()
 
 
 def test_dequant_vector_lengths(binding, ctx):
