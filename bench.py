@@ -28,7 +28,8 @@ HBM_PEAK_GBPS = 8000.0
 # scale factors are written up in the profiles/ summaries of each workload. Keyed by workload and its
 # algorithmic bytes, so a changed workload reports null instead of a stale figure.
 MEASURED_TRAFFIC = {("c2", 651658484): 658.7e6, ("c2_alibi", 661824180): 669.5e6, ("c2_mtp4", 656075180): 683.6e6,
-                    ("c3", 1364204576): 1379.2e6, ("c5", 253384304): 388.7e6}
+                    ("c3", 1364204576): 1379.2e6, ("c5", 253384304): 388.7e6,
+                    ("c5_split", 253384304): 378.4e6}
 
 DESCRIPTIONS = {
     "c1": "C1 small fp16 decode: batch 4, 8 q heads, 8 kv heads, d128, block 128, ctx U[64,512]",
