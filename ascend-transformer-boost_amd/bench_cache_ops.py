@@ -1,0 +1,97 @@
+#!/usr/bin/env python3
+"""Times the cache-side operations at the size of benchmark workload C2 on one MI355X and
+prints one JSON line per operation: BlockCopy (512 blocks of 256 KB copied in each cache) and
+PagedCacheLoad (all 158 839 cached rows of the 64 sequences gathered), through atb::Operation
+(Setup + Execute per call). Both are HBM-bound byte movers; `roofline.achieved` is their
+algorithmic bytes (every source byte read once, every destination byte written once) over the
+mean kernel time between HIP events on the launch stream.
+
+    python3 ascend-transformer-boost_amd/bench_cache_ops.py [--steps 50] [--warmup 5]
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(HERE))
+HBM_PEAK_GBPS = 8000.0
+
+
+def timed(fn, stream, steps, warmup):
+    import torch
+    with torch.cuda.stream(stream):
+        for _ in range(warmup):
+            fn()
+        start = torch.cuda.Event(enable_timing=True)
+        stop = torch.cuda.Event(enable_timing=True)
+        start.record(stream)
+        for _ in range(steps):
+            fn()
+        stop.record(stream)
+    stream.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    args = ap.parse_args()
+    import torch
+    pkg = importlib.import_module(os.path.basename(HERE))
+    b, w = pkg.binding, pkg.workloads
+    if not torch.cuda.is_available():
+        sys.exit("bench_cache_ops.py: no GPU visible")
+    dev = torch.device("cuda:0")
+    cfg = w.config("c2")
+    lay = w.layout(cfg)
+    g, d, bs, pool = cfg["kv_heads"], cfg["d"], cfg["block"], lay["pool"]
+    stream = torch.cuda.Stream(device=dev)
+    ctx = b.Context(stream)
+    kc = torch.randn((pool, bs, g, d), device=dev).to(torch.bfloat16)
+    vc = torch.randn((pool, bs, g, d), device=dev).to(torch.bfloat16)
+    block_bytes = bs * g * d * 2
+
+    # ---- BlockCopy: 256 sources, two destinations each
+    rng = np.random.Generator(np.random.PCG64(11))
+    perm = rng.permutation(pool)
+    src, dst = perm[:256].astype(np.int32), perm[256:768].astype(np.int32)
+    cum = (np.arange(1, 257) * 2).astype(np.int32)
+    src_d, dst_d, cum_d = (torch.from_numpy(a).to(dev) for a in (src, dst, cum))
+    copy = b.OperationRunner("BlockCopyOperation", b.BlockCopyParam(), ctx)
+    ms = timed(lambda: copy.run([kc, vc, src_d, dst_d, cum_d], outputs=[]), stream, args.steps, args.warmup)
+    alg = 2 * (len(src) + len(dst)) * block_bytes
+    print(json.dumps({"operation": "BlockCopyOperation", "workload": "C2 caches: 256 source blocks of 256 KB to 512 "
+                      "destination blocks, in the key and in the value cache", "ms_per_call": ms,
+                      "roofline": {"bound": "hbm", "achieved": alg / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
+                                   "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                                   "algorithmic_bytes": alg}}))
+    copy.close()
+
+    # ---- PagedCacheLoad: every cached row of the batch
+    lens = lay["ctx"]
+    total = int(lens.sum())
+    key = torch.empty((total, g, d), dtype=torch.bfloat16, device=dev)
+    value = torch.empty_like(key)
+    tables_d = torch.from_numpy(lay["tables"]).to(dev)
+    lens_d = torch.from_numpy(lens).to(dev)
+    starts_d = torch.zeros(len(lens), dtype=torch.int32, device=dev)
+    load = b.OperationRunner("PagedCacheLoadOperation", b.PagedCacheLoadParam(kvCacheCfg=1), ctx)
+    ms = timed(lambda: load.run([kc, vc, tables_d, lens_d, key, value, starts_d], outputs=[key, value]), stream,
+               args.steps, args.warmup)
+    alg = 2 * 2 * total * g * d * 2
+    print(json.dumps({"operation": "PagedCacheLoadOperation", "workload": "C2: %d rows of %d B gathered from each "
+                      "cache into contiguous key / value" % (total, g * d * 2), "ms_per_call": ms,
+                      "roofline": {"bound": "hbm", "achieved": alg / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
+                                   "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                                   "algorithmic_bytes": alg}}))
+    load.close()
+    ctx.close()
+
+
+if __name__ == "__main__":
+    main()

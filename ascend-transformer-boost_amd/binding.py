@@ -84,6 +84,24 @@ class ReshapeAndCacheParam(ctypes.Structure):
             setattr(self, k, v)
 
 
+class BlockCopyParam(ctypes.Structure):
+    """Byte image of atb::infer::BlockCopyParam (16 bytes)."""
+    _fields_ = [("rsv", ctypes.c_uint8 * 16)]
+
+
+class PagedCacheLoadParam(ctypes.Structure):
+    """Byte image of atb::infer::PagedCacheLoadParam (64 bytes)."""
+    _fields_ = [("kvCacheCfg", ctypes.c_int8), ("isSeqLensCumsumMode", ctypes.c_bool), ("hasSeqStarts", ctypes.c_bool),
+                ("rsv", ctypes.c_uint8 * 61)]
+
+    def __init__(self, **kw):
+        super().__init__()
+        for k, v in kw.items():
+            if not hasattr(self, k):
+                raise AttributeError("PagedCacheLoadParam has no field " + k)
+            setattr(self, k, v)
+
+
 class MultiLatentAttentionParam(ctypes.Structure):
     """Byte image of atb::infer::MultiLatentAttentionParam (64 bytes)."""
     _fields_ = [("headNum", ctypes.c_int32), ("qkScale", ctypes.c_float), ("kvHeadNum", ctypes.c_int32),
@@ -141,6 +159,9 @@ def kernels():
         lib.atbmi_reshape_and_cache.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]
         lib.atbmi_quant_per_channel.argtypes = [vp, i32, vp, vp, vp, i64, i64, vp]
         lib.atbmi_reshape_and_cache_quant.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]
+        lib.atbmi_block_copy.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]
+        lib.atbmi_paged_cache_load.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64,
+                                               i32, vp]
         lib.atbmi_pa_plan_create.argtypes = [ctypes.POINTER(AtbmiPaShape), ctypes.POINTER(vp)]
         lib.atbmi_pa_plan_update.argtypes = [vp, vp, i32]
         lib.atbmi_pa_plan_update_multi.argtypes = [vp, vp, vp, i32]

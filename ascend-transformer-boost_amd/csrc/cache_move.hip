@@ -1,0 +1,293 @@
+// KV-cache block movement kernels for gfx950: BlockCopy (whole cache blocks
+// copied to other blocks of the same caches) and PagedCacheLoad (the rows of
+// every sequence gathered from the paged caches into contiguous tensors, the
+// reverse of ReshapeAndCache).
+//
+// Both are plain HBM-bound byte movers: every access is a full-width vector
+// access (16 bytes per lane when sizes and addresses allow it), consecutive
+// lanes touch consecutive addresses, and a launch has many more workgroups
+// than the chip has CUs.
+#include <algorithm>
+#include "atbmi_common.h"
+
+namespace atbmi {
+namespace {
+
+constexpr int MOVE_THREADS = 256;
+constexpr int PIECES_PER_THREAD = 4; // a workgroup moves 256 * 4 vectors: 16 KB with 16-byte vectors
+
+typedef uint32_t Vec16 __attribute__((ext_vector_type(4)));
+typedef uint32_t Vec8 __attribute__((ext_vector_type(2)));
+
+// Every byte is read once and written once: the non-temporal hints keep the stream from displacing
+// what the attention kernels want to find in the caches.
+template <typename VecT> __device__ __forceinline__ VecT LoadOnce(const VecT *p)
+{
+    return __builtin_nontemporal_load(p);
+}
+template <typename VecT> __device__ __forceinline__ void StoreOnce(VecT *p, VecT v)
+{
+    __builtin_nontemporal_store(v, p);
+}
+
+inline bool Aligned(const void *p, uintptr_t a)
+{
+    return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
+}
+
+// grid.x = piece of the block, grid.y = destination index, grid.z = 0 (key cache) / 1 (value cache).
+// Destination j takes the block of source i, the first i with cumSum[i] > j.
+template <typename VecT>
+__global__ __launch_bounds__(MOVE_THREADS) void BlockCopyKernel(uint8_t *__restrict__ keyCache,
+                                                                uint8_t *__restrict__ valueCache,
+                                                                const int32_t *__restrict__ srcBlocks,
+                                                                const int32_t *__restrict__ dstBlocks,
+                                                                const int32_t *__restrict__ cumSum, int32_t srcCount,
+                                                                int64_t numBlocks, int64_t kBlockBytes,
+                                                                int64_t vBlockBytes)
+{
+    const int j = blockIdx.y;
+    int lo = 0, hi = srcCount; // first i in [0, srcCount) with cumSum[i] > j
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (cumSum[mid] > j) {
+            hi = mid;
+        } else {
+            lo = mid + 1;
+        }
+    }
+    if (lo >= srcCount) {
+        return; // past the last source's share: nothing names this destination
+    }
+    const int64_t src = srcBlocks[lo];
+    const int64_t dst = dstBlocks[j];
+    if (src < 0 || src >= numBlocks || dst < 0 || dst >= numBlocks || src == dst) {
+        return;
+    }
+    const bool isValue = blockIdx.z == 1;
+    const int64_t blockBytes = isValue ? vBlockBytes : kBlockBytes;
+    uint8_t *cache = isValue ? valueCache : keyCache;
+    const VecT *from = reinterpret_cast<const VecT *>(cache + src * blockBytes);
+    VecT *to = reinterpret_cast<VecT *>(cache + dst * blockBytes);
+    const int64_t n = blockBytes / static_cast<int64_t>(sizeof(VecT));
+    const int64_t base = static_cast<int64_t>(blockIdx.x) * (MOVE_THREADS * PIECES_PER_THREAD) + threadIdx.x;
+    VecT v[PIECES_PER_THREAD];
+#pragma unroll
+    for (int p = 0; p < PIECES_PER_THREAD; ++p) { // all loads first
+        const int64_t i = base + p * MOVE_THREADS;
+        if (i < n) {
+            v[p] = from[i]; // (a source with several destinations is read again: let it stay cached)
+        }
+    }
+#pragma unroll
+    for (int p = 0; p < PIECES_PER_THREAD; ++p) {
+        const int64_t i = base + p * MOVE_THREADS;
+        if (i < n) {
+            StoreOnce(to + i, v[p]);
+        }
+    }
+}
+
+// grid.x = 64-token group of a sequence, grid.y = sequence, grid.z = 0 (key) / 1 (value).
+// Token t of sequence b sits in block tables[b][seqStarts[b] / blockSize + t / blockSize] at offset
+// t % blockSize and goes to output row (tokens of the sequences before b) + t. A negative block id
+// leaves the output row as it is.
+constexpr int LOAD_TOKENS = 64;
+
+template <typename VecT>
+__global__ __launch_bounds__(MOVE_THREADS) void PagedCacheLoadKernel(
+    const uint8_t *__restrict__ keyCache, const uint8_t *__restrict__ valueCache,
+    const int32_t *__restrict__ tables, const int32_t *__restrict__ lens, const int32_t *__restrict__ seqStarts,
+    uint8_t *__restrict__ key, uint8_t *__restrict__ value, int32_t maxBlocksPerSeq, int32_t blockSize,
+    int64_t numBlocks, int64_t kRowBytes, int64_t vRowBytes, int64_t outRows, int32_t cumsumMode)
+{
+    const int b = blockIdx.y;
+    int64_t begin; // first output row of this sequence
+    int32_t len;
+    if (cumsumMode) {
+        begin = lens[b];
+        len = lens[b + 1] - lens[b];
+    } else {
+        // the sequences before this one: summed by the first wave, 64 at a time
+        __shared__ int64_t total;
+        if (threadIdx.x < WAVE) {
+            int64_t s = 0;
+            for (int i = threadIdx.x; i < b; i += WAVE) {
+                s += lens[i];
+            }
+            for (int off = 32; off > 0; off >>= 1) {
+                s += __shfl_xor(s, off, WAVE);
+            }
+            if (threadIdx.x == 0) {
+                total = s;
+            }
+        }
+        __syncthreads();
+        begin = total;
+        len = lens[b];
+    }
+    const int t0 = blockIdx.x * LOAD_TOKENS;
+    if (t0 >= len) {
+        return;
+    }
+    const int firstBlock = seqStarts ? seqStarts[b] / blockSize : 0;
+    const bool isValue = blockIdx.z == 1;
+    const int64_t rowBytes = isValue ? vRowBytes : kRowBytes;
+    const uint8_t *cache = isValue ? valueCache : keyCache;
+    uint8_t *out = isValue ? value : key;
+    const int tokens = min(LOAD_TOKENS, len - t0);
+    // cache row of each of the group's tokens (-1: leave the output row alone)
+    __shared__ int64_t srcRow[LOAD_TOKENS];
+    if (threadIdx.x < LOAD_TOKENS) {
+        const int t = t0 + threadIdx.x;
+        int64_t r = -1;
+        const int tableIdx = firstBlock + t / blockSize;
+        if (static_cast<int>(threadIdx.x) < tokens && tableIdx < maxBlocksPerSeq && begin + t < outRows) {
+            const int64_t blk = tables[static_cast<int64_t>(b) * maxBlocksPerSeq + tableIdx];
+            if (blk >= 0 && blk < numBlocks) {
+                r = blk * blockSize + t % blockSize;
+            }
+        }
+        srcRow[threadIdx.x] = r;
+    }
+    __syncthreads();
+    const int perRow = static_cast<int>(rowBytes / static_cast<int64_t>(sizeof(VecT)));
+    const int n = perRow * tokens;
+    const VecT *from = reinterpret_cast<const VecT *>(cache);
+    VecT *to = reinterpret_cast<VecT *>(out + (begin + t0) * rowBytes);
+    constexpr int BATCH = 4;
+    for (int i0 = threadIdx.x; i0 < n; i0 += MOVE_THREADS * BATCH) {
+        VecT v[BATCH];
+        bool live[BATCH];
+#pragma unroll
+        for (int k = 0; k < BATCH; ++k) { // all loads first
+            const int i = i0 + k * MOVE_THREADS;
+            live[k] = false;
+            if (i < n) {
+                const int tok = i / perRow;
+                const int64_t r = srcRow[tok];
+                if (r >= 0) {
+                    live[k] = true;
+                    v[k] = LoadOnce(from + r * perRow + (i - tok * perRow));
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < BATCH; ++k) {
+            if (live[k]) {
+                StoreOnce(to + i0 + k * MOVE_THREADS, v[k]);
+            }
+        }
+    }
+}
+
+// Widest power-of-two vector (<= 16 bytes) that divides both sizes and that every pointer is aligned to.
+template <typename... Ptrs> uintptr_t CommonAlign(int64_t a, int64_t b, Ptrs... ptrs)
+{
+    uintptr_t align = 16;
+    const void *all[] = {ptrs...};
+    for (;;) {
+        bool ok = a % static_cast<int64_t>(align) == 0 && b % static_cast<int64_t>(align) == 0;
+        for (const void *p : all) {
+            ok = ok && (p == nullptr || Aligned(p, align));
+        }
+        if (ok || align == 1) {
+            return align;
+        }
+        align >>= 1;
+    }
+}
+
+} // namespace
+
+extern "C" int atbmi_block_copy(void *keyCache, void *valueCache, const int32_t *srcBlocks, const int32_t *dstBlocks,
+                                const int32_t *cumSum, int64_t srcCount, int64_t dstCount, int64_t numBlocks,
+                                int64_t keyBlockBytes, int64_t valueBlockBytes, void *stream)
+{
+    if (!keyCache || !srcBlocks || !dstBlocks || !cumSum) {
+        return Fail(ERR_INVALID_PARAM, "block_copy: keyCache, srcBlocks, dstBlocks and cumSum must be non-null");
+    }
+    if (srcCount < 0 || dstCount < 0 || numBlocks <= 0 || keyBlockBytes <= 0 || (valueCache && valueBlockBytes <= 0)) {
+        return Fail(ERR_INVALID_PARAM, "block_copy: bad extents");
+    }
+    if (srcCount == 0 || dstCount == 0) {
+        return OK;
+    }
+    if (srcCount > 0x7fffffffLL || dstCount > 65535) {
+        return Fail(ERR_INVALID_PARAM, "block_copy: %lld sources / %lld destinations are more than one launch takes",
+                    (long long)srcCount, (long long)dstCount);
+    }
+    const int64_t vBytes = valueCache ? valueBlockBytes : keyBlockBytes;
+    const uintptr_t align = CommonAlign(keyBlockBytes, vBytes, keyCache, valueCache);
+    const int64_t maxBytes = std::max(keyBlockBytes, vBytes);
+    const int64_t perWg = static_cast<int64_t>(MOVE_THREADS) * PIECES_PER_THREAD * static_cast<int64_t>(align);
+    const int64_t pieces = (maxBytes + perWg - 1) / perWg;
+    if (pieces > 0x7fffffffLL) {
+        return Fail(ERR_INVALID_PARAM, "block_copy: blocks of %lld bytes are too large", (long long)maxBytes);
+    }
+    dim3 grid(static_cast<unsigned>(pieces), static_cast<unsigned>(dstCount), valueCache ? 2 : 1);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    uint8_t *k8 = static_cast<uint8_t *>(keyCache);
+    uint8_t *v8 = static_cast<uint8_t *>(valueCache);
+    const int32_t n = static_cast<int32_t>(srcCount);
+#define ATBMI_LAUNCH_BLOCK_COPY(T) \
+    BlockCopyKernel<T><<<grid, MOVE_THREADS, 0, s>>>(k8, v8, srcBlocks, dstBlocks, cumSum, n, numBlocks, keyBlockBytes, vBytes)
+    switch (align) {
+        case 16: ATBMI_LAUNCH_BLOCK_COPY(Vec16); break;
+        case 8: ATBMI_LAUNCH_BLOCK_COPY(Vec8); break;
+        case 4: ATBMI_LAUNCH_BLOCK_COPY(uint32_t); break;
+        case 2: ATBMI_LAUNCH_BLOCK_COPY(uint16_t); break;
+        default: ATBMI_LAUNCH_BLOCK_COPY(uint8_t); break;
+    }
+#undef ATBMI_LAUNCH_BLOCK_COPY
+    ATBMI_HIP_CHECK(hipGetLastError());
+    return OK;
+}
+
+extern "C" int atbmi_paged_cache_load(const void *keyCache, const void *valueCache, const int32_t *blockTables,
+                                      const int32_t *seqLens, const int32_t *seqStarts, void *key, void *value,
+                                      int64_t batch, int64_t maxBlocksPerSeq, int64_t blockSize, int64_t numBlocks,
+                                      int64_t keyRowBytes, int64_t valueRowBytes, int64_t outRows,
+                                      int64_t maxSeqLen, int32_t cumsumMode, void *stream)
+{
+    if (!keyCache || !valueCache || !blockTables || !seqLens || !key || !value) {
+        return Fail(ERR_INVALID_PARAM, "paged_cache_load: caches, blockTables, seqLens, key and value must be non-null");
+    }
+    if (batch < 0 || maxBlocksPerSeq <= 0 || blockSize <= 0 || numBlocks <= 0 || keyRowBytes <= 0 ||
+        valueRowBytes <= 0 || outRows < 0 || maxSeqLen < 0) {
+        return Fail(ERR_INVALID_PARAM, "paged_cache_load: bad extents");
+    }
+    if (batch == 0 || outRows == 0 || maxSeqLen == 0) {
+        return OK;
+    }
+    const int64_t groups = (maxSeqLen + LOAD_TOKENS - 1) / LOAD_TOKENS;
+    if (batch > 65535 || groups > 0x7fffffffLL || maxBlocksPerSeq > 0x7fffffffLL || blockSize > 0x7fffffffLL ||
+        keyRowBytes > (1 << 24) || valueRowBytes > (1 << 24)) {
+        return Fail(ERR_INVALID_PARAM, "paged_cache_load: %lld sequences of up to %lld tokens are more than one "
+                                       "launch takes", (long long)batch, (long long)maxSeqLen);
+    }
+    const uintptr_t align = CommonAlign(keyRowBytes, valueRowBytes, keyCache, valueCache, key, value);
+    dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(batch), 2);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint8_t *kc8 = static_cast<const uint8_t *>(keyCache);
+    const uint8_t *vc8 = static_cast<const uint8_t *>(valueCache);
+    uint8_t *k8 = static_cast<uint8_t *>(key);
+    uint8_t *v8 = static_cast<uint8_t *>(value);
+#define ATBMI_LAUNCH_CACHE_LOAD(T)                                                                             \
+    PagedCacheLoadKernel<T><<<grid, MOVE_THREADS, 0, s>>>(kc8, vc8, blockTables, seqLens, seqStarts, k8, v8,   \
+                                                          static_cast<int32_t>(maxBlocksPerSeq),               \
+                                                          static_cast<int32_t>(blockSize), numBlocks, keyRowBytes, \
+                                                          valueRowBytes, outRows, cumsumMode)
+    switch (align) {
+        case 16: ATBMI_LAUNCH_CACHE_LOAD(Vec16); break;
+        case 8: ATBMI_LAUNCH_CACHE_LOAD(Vec8); break;
+        case 4: ATBMI_LAUNCH_CACHE_LOAD(uint32_t); break;
+        case 2: ATBMI_LAUNCH_CACHE_LOAD(uint16_t); break;
+        default: ATBMI_LAUNCH_CACHE_LOAD(uint8_t); break;
+    }
+#undef ATBMI_LAUNCH_CACHE_LOAD
+    ATBMI_HIP_CHECK(hipGetLastError());
+    return OK;
+}
+
+} // namespace atbmi

@@ -95,6 +95,16 @@ int32_t atb_c_create_operation(const char *opName, const void *param, uint64_t p
         memcpy(static_cast<void *>(&p), param, sizeof(p));
         return atb::CreateOperation(p, out);
     }
+    if (!strcmp(opName, "BlockCopyOperation") && paramSize == sizeof(atb::infer::BlockCopyParam)) {
+        atb::infer::BlockCopyParam p;
+        memcpy(static_cast<void *>(&p), param, sizeof(p));
+        return atb::CreateOperation(p, out);
+    }
+    if (!strcmp(opName, "PagedCacheLoadOperation") && paramSize == sizeof(atb::infer::PagedCacheLoadParam)) {
+        atb::infer::PagedCacheLoadParam p;
+        memcpy(static_cast<void *>(&p), param, sizeof(p));
+        return atb::CreateOperation(p, out);
+    }
     if (!strcmp(opName, "MultiLatentAttentionOperation") &&
         paramSize == sizeof(atb::infer::MultiLatentAttentionParam)) {
         atb::infer::MultiLatentAttentionParam p;

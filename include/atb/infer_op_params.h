@@ -148,7 +148,28 @@ struct MultiLatentAttentionParam {
     uint8_t rsv[32] = {0}; // must stay zero
 };
 
+// Copies whole blocks of the key and value caches onto other blocks of the same caches
+// (reference include/atb/infer_op_params.h:1208-1217).
+struct BlockCopyParam {
+    uint8_t rsv[16] = {0}; // must stay zero
+};
+
+// Gathers the cached rows of every sequence into contiguous key / value tensors, the
+// reverse of ReshapeAndCache (reference include/atb/infer_op_params.h:3070-3101).
+struct PagedCacheLoadParam {
+    enum KvCacheCfg : int8_t {
+        K_CACHE_V_CACHE_NZ = 0, // fractal-NZ caches; not implemented on MI355X
+        K_CACHE_V_CACHE_ND      // caches [blocks, blockSize, heads, headSize]
+    };
+    KvCacheCfg kvCacheCfg = K_CACHE_V_CACHE_NZ;
+    bool isSeqLensCumsumMode = false; // seqLens holds running sums [batch + 1] instead of lengths [batch]
+    bool hasSeqStarts = false;        // seqStarts gives the first cached position of every sequence
+    uint8_t rsv[61] = {0};            // must stay zero
+};
+
 static_assert(sizeof(ReshapeAndCacheParam) == 24, "ReshapeAndCacheParam ABI size");
+static_assert(sizeof(BlockCopyParam) == 16, "BlockCopyParam ABI size");
+static_assert(sizeof(PagedCacheLoadParam) == 64, "PagedCacheLoadParam ABI size");
 static_assert(sizeof(MultiLatentAttentionParam) == 64, "MultiLatentAttentionParam ABI size");
 static_assert(sizeof(PagedAttentionParam) == 120, "PagedAttentionParam ABI size");
 

@@ -34,8 +34,8 @@ public:
                            Context *context) = 0;
 };
 
-// Specialised for infer::PagedAttentionParam, infer::ReshapeAndCacheParam and
-// infer::MultiLatentAttentionParam.
+// Specialised for infer::PagedAttentionParam, ReshapeAndCacheParam,
+// MultiLatentAttentionParam, BlockCopyParam and PagedCacheLoadParam.
 template <typename OpParam> Status CreateOperation(const OpParam &opParam, Operation **operation);
 
 Status DestroyOperation(Operation *operation);

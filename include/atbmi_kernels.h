@@ -75,6 +75,40 @@ int atbmi_quant_per_channel(const void *xDevice, int32_t xDtype, const float *sc
                             void *stream);
 
 /*
+ * BlockCopy: copies whole cache blocks inside the key cache and the value cache. Source i
+ * (srcBlocks[i]) goes to the destinations dstBlocks[cumSum[i-1] .. cumSum[i]) (cumSum[-1] = 0).
+ * All index vectors are int32 device memory; keyBlockBytes / valueBlockBytes are the bytes of
+ * one block (blockSize * heads * headSize * sizeof element). valueCache may be NULL. Sources
+ * and destinations must be disjoint sets (the copies run in parallel); an index outside
+ * [0, numBlocks) skips that copy.
+ * Replaces: BlockCopyOperation's kernel (reference src/ops/ops_infer/block_copy/
+ * block_copy_operation.cpp:69-99 inputs, golden tests/apitest/opstest/python/operations/
+ * block_copy/test_block_copy.py golden_calc).
+ */
+int atbmi_block_copy(void *keyCacheDevice, void *valueCacheDevice, const int32_t *srcBlocksDevice,
+                     const int32_t *dstBlocksDevice, const int32_t *cumSumDevice, int64_t srcCount, int64_t dstCount,
+                     int64_t numBlocks, int64_t keyBlockBytes, int64_t valueBlockBytes, void *stream);
+
+/*
+ * PagedCacheLoad, ND caches: gathers the rows of every sequence from the paged caches into
+ * contiguous key / value tensors, the reverse of ReshapeAndCache. Token t of sequence b is
+ * the row at offset t % blockSize of block blockTables[b][seqStarts[b] / blockSize + t / blockSize]
+ * and lands in output row (tokens of the sequences before b) + t. seqLens (int32, device) holds
+ * the lengths [batch], or with cumsumMode their running sum [batch + 1] starting at 0; seqStarts
+ * may be NULL (all 0). A negative or out-of-range block id leaves its output rows untouched, as do
+ * rows at or past outRows. maxSeqLen bounds every length (the launch is sized by it; the lengths
+ * themselves are only known on the device).
+ * Replaces: PagedCacheLoadOperation's ND kernel (reference src/ops/ops_infer/paged_cache_load/
+ * paged_cache_load_operation.cpp:20-50 inputs, golden tests/apitest/opstest/python/operations/
+ * paged_cache_load/test_paged_cache_load_operation_nd.py:57-170).
+ */
+int atbmi_paged_cache_load(const void *keyCacheDevice, const void *valueCacheDevice, const int32_t *blockTablesDevice,
+                           const int32_t *seqLensDevice, const int32_t *seqStartsDevice, void *keyDevice,
+                           void *valueDevice, int64_t batch, int64_t maxBlocksPerSeq, int64_t blockSize,
+                           int64_t numBlocks, int64_t keyRowBytes, int64_t valueRowBytes, int64_t outRows,
+                           int64_t maxSeqLen, int32_t cumsumMode, void *stream);
+
+/*
  * Fused quantise + KV-cache write (extension; the reference runs the
  * quantiser and ReshapeAndCache as two operators): key/value are fp16/bf16
  * [numTokens, numKvHeads, headDim*], kScale/vScale are fp32 [numKvHeads*headDim*],

@@ -40,6 +40,14 @@ the invariants of the mathematics (no function is left "parity unpinned"):
                       test_paged_attention_mla_mtp.py:120-166 (the same for the MLA cache, fp32 branch);
                       MLA: tests/apitest/opstest/python/operations/paged_attention/
                       test_paged_attention_operation_mla.py:229-262 (V = K[..., :head_size_vo])
+  block_copy          tests/apitest/opstest/python/operations/block_copy/test_block_copy.py (golden_calc:
+                      source i goes to the destinations dst[cum_sum[i-1] : cum_sum[i]], one after the other)
+  paged_cache_load    tests/apitest/opstest/python/operations/paged_cache_load/
+                      test_paged_cache_load_operation_nd.py:57-170 (token j of sequence i comes from block
+                      table[i][seq_starts[i] // block_size + j // block_size], offset j % block_size; lengths
+                      or their running sums. The golden also skips negative block ids, moving later rows up;
+                      its own tests never draw one (ids come from [0, num_blocks)), so that branch fixes no
+                      behaviour of the kernel: here such rows are skipped in place, see paged_cache_load)
   merge_partials      src/kernels/mixkernels/pagedattention/op_kernel/
                       paged_attention_decoder_nd_common.cce:6568-6760,7959-7975 (split-KV combine)
 
@@ -82,6 +90,44 @@ def reshape_and_cache(key, value, key_cache, value_cache, slot_mapping):
         if vc is not None:
             vc[slot // block_size, slot % block_size] = value[i]
     return kc, vc
+
+
+def block_copy(key_cache, value_cache, src_blocks, dst_blocks, cum_sum):
+    """Returns copies of the caches in which block src_blocks[i] has been copied onto the blocks
+    dst_blocks[cum_sum[i-1] : cum_sum[i]] (cum_sum[-1] = 0), sources taken in order, as the
+    reference golden does: a destination written earlier is seen by a later copy that reads it."""
+    kc = np.array(key_cache, copy=True)
+    vc = np.array(value_cache, copy=True)
+    start = 0
+    for i, src in enumerate(np.asarray(src_blocks).tolist()):
+        end = int(cum_sum[i])
+        for j in range(start, end):
+            dst = int(dst_blocks[j])
+            kc[dst] = kc[src]
+            vc[dst] = vc[src]
+        start = end
+    return kc, vc
+
+
+def paged_cache_load(key_cache, value_cache, block_tables, seq_lens, key, value, seq_starts=None, cumsum_mode=False):
+    """Returns copies of key [tokens, heads, Dk] and value [tokens, heads, Dv] with the cached rows of
+    every sequence written one after the other. seq_lens holds the lengths, or with cumsum_mode their
+    running sums starting at 0 (one entry more). Token j of sequence i always owns output row
+    (tokens of the sequences before i) + j; where its block id is negative that row keeps its input."""
+    key = np.array(key, copy=True)
+    value = np.array(value, copy=True)
+    block_size = key_cache.shape[1]
+    lens = np.diff(np.asarray(seq_lens)) if cumsum_mode else np.asarray(seq_lens)
+    row = 0
+    for i, n in enumerate(lens.tolist()):
+        first = 0 if seq_starts is None else int(seq_starts[i]) // block_size
+        for j in range(int(n)):
+            block = int(block_tables[i][first + j // block_size])
+            if block >= 0:
+                key[row] = key_cache[block][j % block_size]
+                value[row] = value_cache[block][j % block_size]
+            row += 1
+    return key, value
 
 
 def quant_per_channel(x, scale, offset=None):

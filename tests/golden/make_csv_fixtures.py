@@ -7,11 +7,15 @@ status, tagged C: for CreateOperation, I: for InferShape, S: for Setup):
     tests/apitest/opstest/csv/paged_attention.csv
     tests/apitest/opstest/csv/reshape_and_cache.csv
     tests/apitest/opstest/csv/multi_latent_attention.csv
+    tests/apitest/opstest/csv/block_copy.csv
+    tests/apitest/opstest/csv/paged_cache_load.csv
 Those rows are data, not code. This script copies the rows written for the
 Ascend910B feature set (the one this library mirrors) into
     tests/golden/paged_attention_cases.json
     tests/golden/reshape_and_cache_cases.json
     tests/golden/multi_latent_attention_cases.json
+    tests/golden/block_copy_cases.json
+    tests/golden/paged_cache_load_cases.json
 so the parity tests can run where the reference tree is absent.
 
 Run from the repository root in a container that has /root/reference:
@@ -48,6 +52,8 @@ def convert(name):
         d = {h: v.strip() for h, v in zip(header, row)}
         if d.get("SocVersion") != "Ascend910B":
             continue
+        # OutNum is what the harness hands to the operation (BlockCopy lists two output columns but takes none)
+        n_out = int(d["OutNum"]) if d.get("OutNum", "").strip().isdigit() else None
         cases.append({
             "csv_line": line_no,
             "case": int(d["CaseNum"]),
@@ -57,9 +63,9 @@ def convert(name):
             "in_dtypes": split(d["InDType"]),
             "in_formats": split(d["InFormat"]),
             "in_shapes": shapes(d["InShape"]),
-            "out_dtypes": split(d["OutDType"]),
-            "out_formats": split(d["OutFormat"]),
-            "out_shapes": shapes(d["OutShape"]),
+            "out_dtypes": split(d["OutDType"])[:n_out],
+            "out_formats": split(d["OutFormat"])[:n_out],
+            "out_shapes": shapes(d["OutShape"])[:n_out],
             "expected": d["ExpectedError"],
         })
     out = os.path.join(HERE, name + "_cases.json")
@@ -75,3 +81,5 @@ if __name__ == "__main__":
     convert("paged_attention")
     convert("reshape_and_cache")
     convert("multi_latent_attention")
+    convert("block_copy")
+    convert("paged_cache_load")

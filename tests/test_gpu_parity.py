@@ -170,6 +170,131 @@ def test_reshape_and_cache_quant_bit_exact(binding, oracle, dev, stream, dtype):
     assert np.array_equal(kc.cpu().numpy(), want_k) and np.array_equal(vc.cpu().numpy(), want_v)
 
 
+# ------------------------------------------------------------------ block copy, paged cache load
+# blocks, block size, heads, head size, sources, destinations, dtype
+# (reference test_block_copy.py cases; an odd block size in bytes for the narrow-vector path; C2-sized blocks)
+BLOCK_COPY_SHAPES = [
+    (100, 2, 2, 2, 30, 30, torch.float16),
+    (64, 16, 8, 128, 5, 40, torch.bfloat16),
+    (37, 3, 1, 5, 4, 9, torch.int8),
+    (300, 128, 8, 128, 16, 64, torch.float16),
+]
+
+
+@pytest.mark.parametrize("shape", BLOCK_COPY_SHAPES, ids=lambda s: "x".join(str(v) for v in s[:6]) + str(s[6]).split(".")[-1])
+def test_block_copy_bit_exact(binding, oracle, dev, stream, shape):
+    blocks, block, heads, d, n_src, n_dst, dtype = shape
+    rng = _rng(500 + blocks)
+    if dtype == torch.int8:
+        kc = torch.from_numpy(rng.integers(-128, 128, size=(blocks, block, heads, d)).astype(np.int8)).to(dev)
+        vc = torch.from_numpy(rng.integers(-128, 128, size=(blocks, block, heads, d)).astype(np.int8)).to(dev)
+    else:
+        kc = torch.from_numpy(rng.standard_normal((blocks, block, heads, d)).astype(np.float32)).to(dtype).to(dev)
+        vc = torch.from_numpy(rng.standard_normal((blocks, block, heads, d)).astype(np.float32)).to(dtype).to(dev)
+    perm = rng.permutation(blocks)
+    src = perm[:n_src].astype(np.int32)
+    dst = perm[n_src:n_src + n_dst].astype(np.int32)
+    cuts = np.sort(rng.choice(np.arange(1, n_dst), size=n_src - 1, replace=False)) if n_src > 1 else np.array([], int)
+    cum = np.append(cuts, n_dst).astype(np.int32)
+    want_k, want_v = oracle.block_copy(_bits(kc).cpu().numpy(), _bits(vc).cpu().numpy(), src, dst, cum)
+    src_d, dst_d, cum_d = (torch.from_numpy(a).to(dev) for a in (src, dst, cum))
+    elem = kc.element_size()
+    # through the C ABI on copies, then through the operation on the tensors themselves
+    k2, v2 = kc.clone(), vc.clone()
+    with torch.cuda.stream(stream):
+        rc = binding.kernels().atbmi_block_copy(k2.data_ptr(), v2.data_ptr(), src_d.data_ptr(), dst_d.data_ptr(),
+                                                cum_d.data_ptr(), n_src, n_dst, blocks, block * heads * d * elem,
+                                                block * heads * d * elem, stream.cuda_stream)
+    assert rc == 0, binding.last_kernel_error()
+    stream.synchronize()
+    assert np.array_equal(_bits(k2).cpu().numpy(), want_k) and np.array_equal(_bits(v2).cpu().numpy(), want_v)
+    c = binding.Context(stream)
+    op = binding.OperationRunner("BlockCopyOperation", binding.BlockCopyParam(), c)
+    with torch.cuda.stream(stream):
+        assert op.run([kc, vc, src_d, dst_d, cum_d], outputs=[]) == []
+    stream.synchronize()
+    assert np.array_equal(_bits(kc).cpu().numpy(), want_k) and np.array_equal(_bits(vc).cpu().numpy(), want_v)
+    op.close()
+    c.close()
+
+
+# batch, heads, head size K, head size V, block size, blocks, dtype   (reference test_paged_cache_load_operation_nd.py:24-33)
+CACHE_LOAD_SHAPES = [
+    (16, 16, 144, 128, 128, 128, torch.float16),
+    (16, 16, 144, 128, 128, 128, torch.int8),
+    (32, 16, 192, 128, 64, 256, torch.bfloat16),
+    (5, 2, 24, 8, 16, 40, torch.float16),
+]
+
+
+@pytest.mark.parametrize("cumsum,starts", [(True, True), (False, True), (False, False), (True, False)])
+@pytest.mark.parametrize("shape", CACHE_LOAD_SHAPES, ids=lambda s: "x".join(str(v) for v in s[:6]) + str(s[6]).split(".")[-1])
+def test_paged_cache_load_bit_exact(binding, oracle, dev, stream, shape, cumsum, starts):
+    batch, heads, dk, dv, block, blocks, dtype = shape
+    rng = _rng(520 + batch + int(cumsum) * 2 + int(starts))
+    if dtype == torch.int8:
+        kc = torch.from_numpy(rng.integers(-128, 128, size=(blocks, block, heads, dk)).astype(np.int8)).to(dev)
+        vc = torch.from_numpy(rng.integers(-128, 128, size=(blocks, block, heads, dv)).astype(np.int8)).to(dev)
+    else:
+        kc = torch.from_numpy(rng.integers(1, 11, size=(blocks, block, heads, dk)).astype(np.float32)).to(dtype).to(dev)
+        vc = torch.from_numpy(rng.integers(1, 11, size=(blocks, block, heads, dv)).astype(np.float32)).to(dtype).to(dev)
+    lens = rng.integers(0, 1025, size=batch).astype(np.int32)
+    lens[rng.integers(batch)] = 0
+    max_blocks = (int(lens.max()) + block - 1) // block + 4
+    tables = rng.integers(0, blocks, size=(batch, max_blocks)).astype(np.int32)
+    seq_starts = (rng.integers(0, 5, size=batch) * block).astype(np.int32) if starts else np.zeros(batch, np.int32)
+    total = int(lens.sum())
+    key = torch.zeros((total, heads, dk), dtype=dtype, device=dev)
+    value = torch.zeros((total, heads, dv), dtype=dtype, device=dev)
+    arg = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32) if cumsum else lens
+    want_k, want_v = oracle.paged_cache_load(_bits(kc).cpu().numpy(), _bits(vc).cpu().numpy(), tables, arg,
+                                             _bits(key).cpu().numpy(), _bits(value).cpu().numpy(),
+                                             seq_starts if starts else None, cumsum)
+    c = binding.Context(stream)
+    op = binding.OperationRunner("PagedCacheLoadOperation", binding.PagedCacheLoadParam(
+        kvCacheCfg=1, isSeqLensCumsumMode=cumsum, hasSeqStarts=starts), c)
+    with torch.cuda.stream(stream):
+        op.run([kc, vc, torch.from_numpy(tables).to(dev), torch.from_numpy(arg).to(dev), key, value,
+                torch.from_numpy(seq_starts).to(dev)], outputs=[key, value])
+    stream.synchronize()
+    assert np.array_equal(_bits(key).cpu().numpy(), want_k) and np.array_equal(_bits(value).cpu().numpy(), want_v)
+    op.close()
+    c.close()
+
+
+def test_cache_write_then_load_round_trip_at_c2_size(binding, pkg, dev, stream):
+    """ReshapeAndCache followed by PagedCacheLoad returns the written rows in order (full C2 layout:
+    64 sequences, 158 839 rows of 8 x 128 bf16), and BlockCopy of a sequence's blocks preserves them."""
+    w = pkg.workloads
+    cfg = w.config("c2")
+    lay = w.layout(cfg)
+    ctx, tables = lay["ctx"], lay["tables"]
+    g, d, bs = cfg["kv_heads"], cfg["d"], cfg["block"]
+    total = int(ctx.sum())
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(7)
+    rows_k = torch.randn((total, g, d), generator=gen, device=dev).to(torch.bfloat16)
+    rows_v = torch.randn((total, g, d), generator=gen, device=dev).to(torch.bfloat16)
+    kc = torch.zeros((lay["pool"], bs, g, d), dtype=torch.bfloat16, device=dev)
+    vc = torch.zeros_like(kc)
+    slots = np.concatenate([tables[b][np.arange(n) // bs].astype(np.int64) * bs + np.arange(n) % bs
+                            for b, n in enumerate(ctx)]).astype(np.int32)
+    c = binding.Context(stream)
+    rac = binding.OperationRunner("ReshapeAndCacheOperation", binding.ReshapeAndCacheParam(), c)
+    load = binding.OperationRunner("PagedCacheLoadOperation", binding.PagedCacheLoadParam(kvCacheCfg=1), c)
+    out_k, out_v = torch.zeros_like(rows_k), torch.zeros_like(rows_v)
+    tables_d = torch.from_numpy(tables).to(dev)
+    with torch.cuda.stream(stream):
+        rac.run([rows_k, rows_v, kc, vc, torch.from_numpy(slots).to(dev)], outputs=[kc, vc])
+        load.run([kc, vc, tables_d, torch.from_numpy(ctx).to(dev), out_k, out_v,
+                  torch.zeros(len(ctx), dtype=torch.int32, device=dev)], outputs=[out_k, out_v])
+    stream.synchronize()
+    assert torch.equal(out_k, rows_k) and torch.equal(out_v, rows_v)
+    rac.close()
+    load.close()
+    c.close()
+
+
 # ------------------------------------------------------------------ attention
 def _pa_inputs(rng, dev, batch, heads, kv_heads, block, d, dv, ctx, dtype, kv_int8=False, pool_extra=4, std=1.0,
                unique=True):

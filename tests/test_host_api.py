@@ -28,6 +28,8 @@ def _load(name):
 PA_CASES = _load("paged_attention")
 RAC_CASES = _load("reshape_and_cache")
 MLA_CASES = _load("multi_latent_attention")
+BLOCK_COPY_CASES = _load("block_copy")
+CACHE_LOAD_CASES = _load("paged_cache_load")
 
 
 def _pa_unimplemented(p):
@@ -70,6 +72,10 @@ def _make_param(binding, op, p):
         return binding.PagedAttentionParam(**p)
     if op == "MultiLatentAttentionOperation":
         return binding.MultiLatentAttentionParam(**p)
+    if op == "BlockCopyOperation":
+        return binding.BlockCopyParam()
+    if op == "PagedCacheLoadOperation":
+        return binding.PagedCacheLoadParam(**p)
     return binding.ReshapeAndCacheParam(**p)
 
 
@@ -158,6 +164,18 @@ def test_paged_attention_table(binding, ctx, case):
 @pytest.mark.parametrize("case", MLA_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
 def test_multi_latent_attention_table(binding, ctx, case):
     _check(binding, case, ctx, _mla_unimplemented(case["param"]) and not case["expected"].startswith("C:"))
+
+
+@pytest.mark.parametrize("case", BLOCK_COPY_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
+def test_block_copy_table(binding, ctx, case):
+    _check(binding, case, ctx, False)
+
+
+@pytest.mark.parametrize("case", CACHE_LOAD_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
+def test_paged_cache_load_table(binding, ctx, case):
+    # the fractal-NZ cache layout (kvCacheCfg 0, the param's default) is rejected when the operation is created
+    nz = case["param"].get("kvCacheCfg", 0) == 0
+    _check(binding, case, ctx, nz and not case["expected"].startswith("C:"))
 
 
 @pytest.mark.parametrize("case", RAC_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))

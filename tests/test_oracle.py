@@ -118,6 +118,70 @@ def test_quant_per_channel_axis(oracle):
     assert np.array_equal(oracle.quant_per_channel(x, s), np.tile(np.array([1, 2, 4, 8], np.int8), (3, 1)))
 
 
+# ---------------------------------------------------------------- block_copy, paged_cache_load
+def test_block_copy_closed_form(oracle):
+    """With disjoint sources and destinations every destination j ends up holding the block of the
+    source whose cumSum interval contains j, and every other block is untouched."""
+    rng = _rng(60)
+    blocks = 40
+    kc = rng.integers(-100, 100, size=(blocks, 4, 2, 8)).astype(np.int8)
+    vc = rng.integers(-100, 100, size=(blocks, 4, 2, 8)).astype(np.int8)
+    perm = rng.permutation(blocks)
+    src, dst = perm[:5].astype(np.int32), perm[5:5 + 17].astype(np.int32)
+    cum = np.array([3, 3, 9, 10, 17], np.int32)   # source 1 has no destination
+    got_k, got_v = oracle.block_copy(kc, vc, src, dst, cum)
+    owner = np.searchsorted(cum, np.arange(17), side="right")
+    want_k, want_v = kc.copy(), vc.copy()
+    want_k[dst] = kc[src[owner]]
+    want_v[dst] = vc[src[owner]]
+    assert np.array_equal(got_k, want_k) and np.array_equal(got_v, want_v)
+    untouched = np.setdiff1d(np.arange(blocks), dst)
+    assert np.array_equal(got_k[untouched], kc[untouched])
+    # nothing to do
+    same_k, _ = oracle.block_copy(kc, vc, src[:0], dst[:0], cum[:0])
+    assert np.array_equal(same_k, kc)
+
+
+@pytest.mark.parametrize("cumsum,starts", [(False, False), (True, False), (False, True), (True, True)])
+def test_paged_cache_load_is_the_concatenation_of_gathered_rows(oracle, cumsum, starts):
+    rng = _rng(61)
+    blocks, block, heads, dk, dv = 30, 4, 2, 6, 3
+    kc = rng.standard_normal((blocks, block, heads, dk)).astype(np.float32)
+    vc = rng.standard_normal((blocks, block, heads, dv)).astype(np.float32)
+    lens = np.array([5, 0, 13, 4, 1], np.int32)
+    tables = rng.integers(0, blocks, size=(5, 8)).astype(np.int32)
+    seq_starts = (rng.integers(0, 4, size=5) * block).astype(np.int32) if starts else None
+    total = int(lens.sum())
+    key0 = np.full((total + 2, heads, dk), 9.0, np.float32)
+    val0 = np.full((total + 2, heads, dv), 9.0, np.float32)
+    arg = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32) if cumsum else lens
+    got_k, got_v = oracle.paged_cache_load(kc, vc, tables, arg, key0, val0, seq_starts, cumsum)
+    want_k, want_v = [], []
+    for i, n in enumerate(lens):
+        shift = 0 if seq_starts is None else seq_starts[i] // block
+        want_k.append(oracle.gather_rows(kc, tables[i][shift:], n))
+        want_v.append(oracle.gather_rows(vc, tables[i][shift:], n))
+    assert np.array_equal(got_k[:total], np.concatenate(want_k)) and np.array_equal(got_v[:total], np.concatenate(want_v))
+    assert np.all(got_k[total:] == 9.0) and np.all(got_v[total:] == 9.0)
+    # it undoes reshape_and_cache: rows written to their slots come back in order
+    slots = np.concatenate([tables[i][(0 if seq_starts is None else seq_starts[i] // block) + np.arange(n) // block]
+                            * block + np.arange(n) % block for i, n in enumerate(lens)])
+    if len(np.unique(slots)) == len(slots):
+        new_k = rng.standard_normal((total, heads, dk)).astype(np.float32)
+        new_v = rng.standard_normal((total, heads, dv)).astype(np.float32)
+        kc2, vc2 = oracle.reshape_and_cache(new_k, new_v, kc, vc, slots.astype(np.int32))
+        back_k, back_v = oracle.paged_cache_load(kc2, vc2, tables, arg, key0, val0, seq_starts, cumsum)
+        assert np.array_equal(back_k[:total], new_k) and np.array_equal(back_v[:total], new_v)
+
+
+def test_paged_cache_load_negative_block_ids_leave_their_rows(oracle):
+    kc = np.arange(2 * 2 * 1 * 1, dtype=np.float32).reshape(2, 2, 1, 1) + 1
+    tables = np.array([[1, -1, 0]], np.int32)
+    k, v = oracle.paged_cache_load(kc, kc, tables, np.array([5], np.int32), np.zeros((5, 1, 1), np.float32),
+                                   np.zeros((5, 1, 1), np.float32))
+    assert k[:, 0, 0].tolist() == [3.0, 4.0, 0.0, 0.0, 1.0] and np.array_equal(k, v)
+
+
 # ---------------------------------------------------------------- attention
 def test_attention_matches_independent_loops(oracle):
     rng = _rng(2)
