@@ -903,6 +903,32 @@ def test_several_query_tokens_through_operation_api(binding, oracle, dev, stream
     c.close()
 
 
+def test_decode_step_through_torch_atb(pkg, oracle, dev):
+    """A decode step the way a torch_atb user writes it: Operation(param).forward([...]) with the
+    context lengths as a CPU tensor, on torch's current stream."""
+    ta = pkg.torch_atb
+    rng = _rng(600)
+    heads, kv_heads, d, block = 32, 8, 128, 128
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, 4, heads, kv_heads, block, d, d, [300, 17, 1025, 128], torch.float16)
+    new_k = (torch.rand((4, kv_heads, d)) * 2 - 1).half().to(dev)
+    new_v = (torch.rand((4, kv_heads, d)) * 2 - 1).half().to(dev)
+    last = ctx.astype(np.int64) - 1
+    t = tables.cpu().numpy()
+    slots = torch.from_numpy((t[np.arange(4), last // block].astype(np.int64) * block + last % block).astype(np.int32))
+    want_k, want_v = oracle.reshape_and_cache(_bits(new_k).cpu().numpy(), _bits(new_v).cpu().numpy(),
+                                              _bits(kc).cpu().numpy(), _bits(vc).cpu().numpy(), slots.numpy())
+    rac = ta.Operation(ta.ReshapeAndCacheParam())
+    outs = rac.forward([new_k, new_v, kc, vc, slots.to(dev)])
+    assert outs[0] is kc and outs[1] is vc
+    assert np.array_equal(_bits(kc).cpu().numpy(), want_k) and np.array_equal(_bits(vc).cpu().numpy(), want_v)
+    scale = 1.0 / math.sqrt(d)
+    pa = ta.Operation(ta.PagedAttentionParam(head_num=heads, kv_head_num=kv_heads, qk_scale=scale))
+    out, = pa.forward([q, kc, vc, tables, torch.from_numpy(ctx)])
+    assert_close(out, oracle_pa(oracle, q, kc, vc, tables, ctx, scale), 1e-3, "torch_atb")
+    rac.close()
+    pa.close()
+
+
 # ------------------------------------------------------------------ edge semantics
 @pytest.mark.parametrize("kernel", [1, 0])
 def test_empty_sequences_garbage_rows_and_shared_blocks(binding, oracle, dev, stream, kernel):

@@ -562,6 +562,33 @@ def test_multi_latent_attention_counts_shapes_and_setup(binding, ctx):
     spec.close()
 
 
+def test_torch_atb_surface(pkg):
+    """The reference's torch binding surface: snake_case parameter fields, nested enums, name and
+    tensor counts (reference src/torch_atb/bindings.cpp:84-93, :520-590, :926-944)."""
+    ta = pkg.torch_atb
+    p = ta.PagedAttentionParam(head_num=32, qk_scale=0.088, kv_head_num=8,
+                               mask_type=ta.PagedAttentionParam.MaskType.MASK_TYPE_ALIBI, batch_run_status_enable=True,
+                               scale_type=ta.PagedAttentionParam.ScaleType.SCALE_TYPE_LOGN)
+    assert (p.head_num, p.kv_head_num, p.mask_type, p.batch_run_status_enable, p.scale_type) == (32, 8, 2, True, 1)
+    assert abs(p.qk_scale - 0.088) < 1e-7 and "head_num: 32" in repr(p)
+    op = ta.Operation(p)
+    assert (op.name, op.input_num, op.output_num) == ("PagedAttentionOperation", 8, 1)
+    assert repr(op) == "op name: PagedAttentionOperation, input_num: 8, output_num: 1"
+    op.close()
+    with pytest.raises(AttributeError):
+        ta.PagedAttentionParam(headNum=1)
+    with pytest.raises(RuntimeError):
+        ta.Operation(ta.PagedAttentionParam(head_num=0))
+    rac = ta.Operation(ta.ReshapeAndCacheParam(kv_cache_cfg=ta.ReshapeAndCacheParam.KvCacheCfg.K_CACHE_V_BYPASS))
+    assert (rac.name, rac.input_num, rac.output_num) == ("ReshapeAndCacheOperation", 3, 1)
+    rac.close()
+    mla = ta.Operation(ta.MultiLatentAttentionParam(head_num=128, kv_head_num=1, qk_scale=0.07,
+                                                    cache_mode=ta.MultiLatentAttentionParam.CacheMode.KROPE_CTKV,
+                                                    calc_type=ta.MultiLatentAttentionParam.CalcType.CALC_TYPE_RING))
+    assert (mla.input_num, mla.output_num) == (6, 2)
+    mla.close()
+
+
 def test_dequant_vector_lengths(binding, ctx):
     e = binding.ERROR_CODE
     op = binding.Operation("PagedAttentionOperation",
