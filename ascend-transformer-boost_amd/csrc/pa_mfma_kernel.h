@@ -55,6 +55,21 @@ constexpr int HT = PA_MFMA_HEAD_TILE;
 constexpr int K_PAD = 8;             // halves of padding per K tile row (16 B)
 constexpr int V_PAD = 16;            // halves of padding per V tile row (32 B)
 
+// Four consecutive per-channel descales from channel c on. stride 1: a plain float array; stride 2:
+// the low halves of 8-byte packed entries. Read as whole 16-byte vectors either way: one address per
+// four channels keeps the many descale loads of a row from crowding the register file.
+__device__ __forceinline__ f32x4 LoadScale4(const float *scales, int c, int stride)
+{
+    typedef float Vec4 __attribute__((ext_vector_type(4), aligned(4)));
+    if (stride == 1) {
+        const Vec4 v = *reinterpret_cast<const Vec4 *>(scales + c);
+        return f32x4{v[0], v[1], v[2], v[3]};
+    }
+    const Vec4 lo = *reinterpret_cast<const Vec4 *>(scales + 2 * c);
+    const Vec4 hi = *reinterpret_cast<const Vec4 *>(scales + 2 * c + 4);
+    return f32x4{lo[0], lo[2], hi[0], hi[2]};
+}
+
 template <bool BF16> __device__ __forceinline__ f32x4 Mma(u32x4 a, u32x4 b, f32x4 c)
 {
     if constexpr (BF16) {
@@ -152,7 +167,10 @@ __device__ __forceinline__ PaSeq PlanSeq(const PaStreamPlan &p, int i)
 // NW  : waves per workgroup.
 // SHARED: the waves of a workgroup are the query-head tiles of ONE KV head and token range (MLA with
 //       many heads): the K tile is staged once per workgroup, double-buffered, and read by all waves.
-template <bool BF16, bool KV8, int D, int DV, bool MLA, bool PF, int NW, bool SHARED>
+// EXT : with the additive mask, the per-sequence log-N scale and several query tokens folded into one
+//       tile. Calls that use none of them run the EXT = false build, which keeps those values out of
+//       its registers (the int8 builds sit at the register limit of their occupancy).
+template <bool BF16, bool KV8, int D, int DV, bool MLA, bool PF, int NW, bool SHARED, bool EXT>
 __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const PaStreamPlan p)
 {
     static_assert(D % 32 == 0 && DV % 16 == 0, "head sizes must fit the MFMA tiles");
@@ -247,22 +265,23 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
         // Column n of the tile is head h0 + n of the pass's query token, or, when the plan folds
         // several query tokens of a sequence into one tile (small GQA groups), head h0 + n % group
         // of its query token n / group.
+        const bool fold = EXT && p.foldTokens > 1;
         int nh = nhTile;
-        if (p.foldTokens > 1) {
+        if (fold) {
             nh = sq.nTok * a.groupSize;
         }
-        const int nc = min(n, nh - 1); // columns past the tile's end borrow its last one where they must read
+        const int nc = EXT ? min(n, nh - 1) : n; // columns past the tile's end borrow its last one where they must read
         int colTok = 0, colHead = nc;
-        if (p.foldTokens > 1) {
+        if (fold) {
             colTok = nc / a.groupSize;
             colHead = nc - colTok * a.groupSize;
         }
         const int qRow = sq.qRow + colTok;
         // SCALE_TYPE_LOGN: a per-sequence factor on the score scale, indexed like the block tables
-        const float scaleSeq = a.logN ? scale2 * a.logN[sq.tableRow] : scale2;
+        const float scaleSeq = EXT && a.logN ? scale2 * a.logN[sq.tableRow] : scale2;
         // additive score bias of this column's query token and head
         const uint16_t *maskRow = nullptr;
-        if (a.mask) {
+        if (EXT && a.mask) {
             maskRow = reinterpret_cast<const uint16_t *>(a.mask) +
                       static_cast<int64_t>(sq.maskRow + colTok * a.maskRowStep) * a.maskBatchStride +
                       static_cast<int64_t>(h0 + colHead) * a.maskHeadStride;
@@ -287,6 +306,11 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                 for (int j = 0; j < NQ; ++j) {
                     const int d0 = j * 32 + kg * 8;
                     float f[8];
+                    f32x4 ks[2] = {f32x4{1.0f, 1.0f, 1.0f, 1.0f}, f32x4{1.0f, 1.0f, 1.0f, 1.0f}};
+                    if (KV8) {
+                        ks[0] = LoadScale4(a.kScale, g * D + d0, a.scaleStride);
+                        ks[1] = LoadScale4(a.kScale, g * D + d0 + 4, a.scaleStride);
+                    }
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
                         f[e] = Unpack(qreg[j][e >> 1], e & 1, qBf16);
@@ -295,7 +319,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                             f[e] = qBf16 ? Bf16ToFloat(FloatToBf16(f[e])) : HalfBitsToFloat(FloatToHalfBits(f[e]));
                         }
                         if (KV8) {
-                            f[e] *= a.kScale[(g * D + d0 + e) * a.scaleStride];
+                            f[e] *= ks[e >> 2][e & 3];
                         }
                     }
 #pragma unroll
@@ -524,7 +548,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                 // a bias of -inf may leave a head without any token yet: m then stays -inf
                 if (__builtin_amdgcn_ballot_w64(mloc > m) != 0) { // some head's maximum grew: rescale
                     const float mNew = fmaxf(m, mloc);
-                    const float corr = mNew == -INFINITY ? 1.0f : Exp2(m - mNew);
+                    const float corr = EXT && mNew == -INFINITY ? 1.0f : Exp2(m - mNew);
                     m = mNew;
                     accL *= corr;
     #pragma unroll
@@ -532,7 +556,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                         acc[i] *= corr;
                     }
                 }
-                const float mRef = m == -INFINITY ? 0.0f : m; // (-inf) - (-inf) would be NaN
+                const float mRef = EXT && m == -INFINITY ? 0.0f : m; // (-inf) - (-inf) would be NaN
     #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     x[e] = Exp2(x[e] - mRef);
@@ -700,7 +724,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
 
         // ---- finish the row (or this wave's share of it)
         const float l = accL[0];
-        const float inv = l > 0.0f ? 1.0f / l : 0.0f; // l == 0: a -inf mask took every token out
+        const float inv = EXT && l == 0.0f ? 0.0f : 1.0f / l; // l == 0: a -inf mask took every token out
         const float bias = KV8 ? INT8_BIAS : 0.0f; // see Int8x4ToHalf
         if (n < nh) {
             const int h = h0 + colHead;
@@ -710,12 +734,16 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                 for (int i = 0; i < NO; ++i) {
                     const int d = i * 16 + kg * 4;
                     float o[4];
+                    f32x4 vs = {1.0f, 1.0f, 1.0f, 1.0f};
+                    if (KV8) {
+                        vs = LoadScale4(a.vScale, g * DV + d, a.scaleStride);
+                    }
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         o[r] = acc[i][r] * inv - bias;
                         if (KV8) {
                             const int c = g * DV + d + r;
-                            o[r] = (o[r] + (a.vOff ? static_cast<float>(a.vOff[c]) : 0.0f)) * a.vScale[c * a.scaleStride];
+                            o[r] = (o[r] + (a.vOff ? static_cast<float>(a.vOff[c]) : 0.0f)) * vs[r];
                         }
                     }
                     u32x2 packed;
@@ -733,7 +761,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                 }
             } else {
                 const int slot = 2 * wr + (segBegin == s0 ? 0 : 1);
-                const int64_t ph = (static_cast<int64_t>(slot) * p.foldTokens + colTok) * a.H + h;
+                const int64_t ph = (static_cast<int64_t>(slot) * (EXT ? p.foldTokens : 1) + colTok) * a.H + h;
 #pragma unroll
                 for (int i = 0; i < NO; ++i) {
                     *reinterpret_cast<f32x4 *>(a.partO + ph * DV + i * 16 + kg * 4) = acc[i] * inv - bias;
@@ -746,10 +774,10 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
     }
 }
 
-template <bool BF16, bool KV8, int D, int DV, bool MLA, bool PF, int NW, bool SHARED = false>
-int Launch(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
+template <bool BF16, bool KV8, int D, int DV, bool MLA, bool PF, int NW, bool SHARED, bool EXT>
+int LaunchBuild(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
 {
-    auto kernel = PaMfmaKernel<BF16, KV8, D, DV, MLA, PF, NW, SHARED>;
+    auto kernel = PaMfmaKernel<BF16, KV8, D, DV, MLA, PF, NW, SHARED, EXT>;
     constexpr int lds = SHARED ? 2 * WaveLdsBytes<D, DV, MLA>() : NW * WaveLdsBytes<D, DV, MLA>();
     static_assert(lds <= 160 * 1024, "tiles exceed the 160 KB of LDS per CU");
     static bool configured = false; // one attribute call per instantiation and process
@@ -769,6 +797,17 @@ int Launch(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
     kernel<<<static_cast<unsigned>(grid), NW * WAVE, lds, stream>>>(args, plan);
     ATBMI_HIP_CHECK(hipGetLastError());
     return OK;
+}
+
+// The combined-cache builds always carry the extensions (their callers use masks and several query
+// tokens routinely and they are not register-bound); the others come in both forms.
+template <bool BF16, bool KV8, int D, int DV, bool MLA, bool PF, int NW, bool SHARED = false>
+int Launch(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
+{
+    if (MLA || args.mask != nullptr || args.logN != nullptr || plan.foldTokens > 1) {
+        return LaunchBuild<BF16, KV8, D, DV, MLA, PF, NW, SHARED, true>(args, plan, stream);
+    }
+    return LaunchBuild<BF16, KV8, D, DV, MLA, PF, NW, SHARED, MLA>(args, plan, stream);
 }
 
 } // namespace mfma

@@ -57,22 +57,30 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaReduceKernel(const PaArgs a)
     }
 }
 
-// Stream plan: the partials of sequence b live in the slots of the wave
-// ranges that intersect its steps; a sequence inside one range was written
-// directly by that wave. One workgroup merges one (sequence, query head).
-// Slot 2wr holds the row a range starts in, slot 2wr+1 the row it ends in, so
-// only the first range of a sequence can use an odd slot.
-// The weights 2^(lse_k - max) are computed once, 128 ranges at a time by the
-// 128 threads, and kept in LDS; threads then own output channels.
+// Stream plan: the partials of a pass live in the slots of the wave ranges that
+// intersect its steps; a pass inside one range was written directly by that
+// wave. Slot 2wr holds the row a range starts in, slot 2wr+1 the row it ends
+// in, so only the first range of a pass can use an odd slot; a slot holds
+// foldTokens x H partial rows.
+// A thread owns four consecutive channels of one output row (pass, query token,
+// head): it takes the maximum of the row's log-sum-exps, then adds up the
+// weighted partial rows with 16-byte loads. A workgroup of 128 threads covers as
+// many whole rows as fit (four for 128 channels, one for 512).
+typedef float ReduceF4 __attribute__((ext_vector_type(4)));
+
 __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaArgs a, const PaStreamPlan p)
 {
-    __shared__ float weight[REDUCE_THREADS];
-    __shared__ float red[REDUCE_THREADS / WAVE];
-    // one workgroup per (pass, query token of it, head); a slot holds foldTokens x H partial rows
+    const int vecs = a.Dv / 4;                                        // threads per row
+    const int rowsPerWg = vecs >= REDUCE_THREADS ? 1 : REDUCE_THREADS / vecs;
     const int rowsPerSlot = a.H * p.foldTokens;
-    const int b = blockIdx.x / rowsPerSlot;
-    const int tok = blockIdx.x % rowsPerSlot / a.H;
-    const int h = blockIdx.x % a.H;
+    const int tid = threadIdx.x;
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * rowsPerWg + (vecs >= REDUCE_THREADS ? 0 : tid / vecs);
+    if (row >= static_cast<int64_t>(p.numSeqs) * rowsPerSlot || (vecs < REDUCE_THREADS && tid >= rowsPerWg * vecs)) {
+        return;
+    }
+    const int b = static_cast<int>(row / rowsPerSlot);
+    const int tok = static_cast<int>(row % rowsPerSlot) / a.H;
+    const int h = static_cast<int>(row % a.H);
     const PaSeq sq = p.seqs ? p.seqs[b] : p.inlineSeqs[b];
     if (tok >= sq.nTok) {
         return;
@@ -90,83 +98,46 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaA
     const int64_t phEven = 2 * static_cast<int64_t>(wrFirst) * rowsPerSlot + static_cast<int64_t>(tok) * a.H + h;
     const int64_t ph0 = phEven + static_cast<int64_t>(firstOdd) * rowsPerSlot;
     const int count = wrLast - wrFirst + 1;
-    const int tid = threadIdx.x;
     auto rowOf = [&](int k) { return k == 0 ? ph0 : phEven + k * stride; };
-    auto blockMax = [&](float v) {
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            v = fmaxf(v, __shfl_xor(v, off, WAVE));
-        }
-        __syncthreads();
-        if (tid % WAVE == 0) {
-            red[tid / WAVE] = v;
-        }
-        __syncthreads();
-        return fmaxf(red[0], red[1]);
-    };
-    auto blockSum = [&](float v) {
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            v += __shfl_xor(v, off, WAVE);
-        }
-        __syncthreads();
-        if (tid % WAVE == 0) {
-            red[tid / WAVE] = v;
-        }
-        __syncthreads();
-        return red[0] + red[1];
-    };
 
     float mx = -INFINITY;
-    for (int k = tid; k < count; k += REDUCE_THREADS) {
+    for (int k = 0; k < count; ++k) {
         mx = fmaxf(mx, a.partLse[rowOf(k)]);
     }
-    mx = blockMax(mx);
-
     const int g = h / a.groupSize;
     const bool bf16 = a.qIsBf16 != 0;
-    // channels handled by this thread: tid, tid + 128, ... (at most 5 for Dv <= 576)
-    float acc[5] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-    float total = 0.0f;
-    for (int k0 = 0; k0 < count; k0 += REDUCE_THREADS) {
-        const int kn = min(REDUCE_THREADS, count - k0);
-        __syncthreads();
-        float w = 0.0f;
-        if (tid < kn) {
-            const float lse = a.partLse[rowOf(k0 + tid)];
-            w = lse == -INFINITY ? 0.0f : exp2f(lse - mx); // a range a -inf mask emptied weighs nothing
-            weight[tid] = w;
-        }
-        total += w;
-        __syncthreads();
-#pragma unroll
-        for (int c = 0; c < 5; ++c) {
-            const int d = tid + c * REDUCE_THREADS;
-            if (d < a.Dv) {
-                float s = 0.0f;
+    const int64_t outRow = static_cast<int64_t>(sq.qRow + tok) * a.H + h;
+    for (int c4 = vecs >= REDUCE_THREADS ? tid : tid % vecs; c4 < vecs; c4 += REDUCE_THREADS) {
+        ReduceF4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        float sum = 0.0f;
 #pragma unroll 4
-                for (int k = 0; k < kn; ++k) {
-                    s += weight[k] * a.partO[rowOf(k0 + k) * a.Dv + d];
-                }
-                acc[c] += s;
+        for (int k = 0; k < count; ++k) {
+            const int64_t ph = rowOf(k);
+            const float lse = a.partLse[ph];
+            const float w = lse == -INFINITY ? 0.0f : exp2f(lse - mx); // a range a -inf mask emptied weighs nothing
+            sum += w;
+            acc += w * *reinterpret_cast<const ReduceF4 *>(a.partO + ph * a.Dv + c4 * 4);
+        }
+        const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
+        float o[4] = {acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv};
+        if (a.finishV) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int ch = g * a.Dv + c4 * 4 + e;
+                o[e] = (o[e] + (a.vOff ? static_cast<float>(a.vOff[ch]) : 0.0f)) * a.vScale[ch * a.scaleStride];
             }
         }
-    }
-    const float sum = blockSum(total);
-    const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
-    if (a.lse && tid == 0) {
-        Store16(a.lse, static_cast<int64_t>(sq.qRow + tok) * a.H + h, (mx + log2f(sum)) * LN2, a.qIsBf16 != 0);
-    }
+        uint16_t bits[4];
 #pragma unroll
-    for (int c = 0; c < 5; ++c) {
-        const int d = tid + c * REDUCE_THREADS;
-        if (d < a.Dv) {
-            float o = acc[c] * inv;
-            if (a.finishV) {
-                const int ch = g * a.Dv + d;
-                o = (o + (a.vOff ? static_cast<float>(a.vOff[ch]) : 0.0f)) * a.vScale[ch * a.scaleStride];
-            }
-            Store16(a.out, (static_cast<int64_t>(sq.qRow + tok) * a.H + h) * a.Dv + d, o, bf16);
+        for (int e = 0; e < 4; ++e) {
+            bits[e] = bf16 ? FloatToBf16(o[e]) : FloatToHalfBits(o[e]);
+        }
+        uint2 packed;
+        packed.x = static_cast<uint32_t>(bits[0]) | (static_cast<uint32_t>(bits[1]) << 16);
+        packed.y = static_cast<uint32_t>(bits[2]) | (static_cast<uint32_t>(bits[3]) << 16);
+        *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(a.out) + outRow * a.Dv + c4 * 4) = packed;
+        if (a.lse && c4 == 0) {
+            Store16(a.lse, outRow, (mx + log2f(sum)) * LN2, bf16);
         }
     }
 }
@@ -177,7 +148,10 @@ int LaunchPaStreamReduce(const AtbmiPaShape &shape, const PaArgs &args, const Pa
                          hipStream_t stream)
 {
     (void)shape;
-    const int64_t grid = static_cast<int64_t>(plan.numSeqs) * plan.foldTokens * args.H;
+    const int vecs = args.Dv / 4;
+    const int rowsPerWg = vecs >= REDUCE_THREADS ? 1 : REDUCE_THREADS / vecs;
+    const int64_t rows = static_cast<int64_t>(plan.numSeqs) * plan.foldTokens * args.H;
+    const int64_t grid = (rows + rowsPerWg - 1) / rowsPerWg;
     if (grid <= 0) {
         return OK;
     }
