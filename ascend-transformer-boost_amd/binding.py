@@ -84,6 +84,10 @@ class ReshapeAndCacheParam(ctypes.Structure):
             setattr(self, k, v)
 
 
+class ReshapeAndCacheWithStrideParam(ReshapeAndCacheParam):
+    """Byte image of atb::infer::ReshapeAndCacheWithStrideParam (24 bytes, the same fields)."""
+
+
 class BlockCopyParam(ctypes.Structure):
     """Byte image of atb::infer::BlockCopyParam (16 bytes)."""
     _fields_ = [("rsv", ctypes.c_uint8 * 16)]
@@ -157,6 +161,8 @@ def kernels():
         lib.atbmi_last_error.argtypes = []
         lib.atbmi_device_count.restype = ctypes.c_int
         lib.atbmi_reshape_and_cache.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]
+        lib.atbmi_reshape_and_cache_strided.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp, i64, vp,
+                                                        i64, vp]
         lib.atbmi_quant_per_channel.argtypes = [vp, i32, vp, vp, vp, i64, i64, vp]
         lib.atbmi_reshape_and_cache_quant.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]
         lib.atbmi_block_copy.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]
@@ -348,12 +354,13 @@ class OperationRunner:
         self.workspace = None
 
     def run(self, inputs, outputs=None, host_inputs=None):
-        """inputs: torch GPU tensors; host_inputs: {index: CPU tensor} bound as
+        """inputs: torch GPU tensors (or ready-made AtbCTensor descriptions, for a view whose shape
+        is not the tensor's own); host_inputs: {index: CPU tensor} bound as
         hostData; outputs: caller-owned output tensors (in-place cache update)
         or None to allocate from InferShape. Returns the output tensors."""
         import torch
         host_inputs = host_inputs or {}
-        ins = [tensor_of(t, host_inputs.get(i)) for i, t in enumerate(inputs)]
+        ins = [t if isinstance(t, AtbCTensor) else tensor_of(t, host_inputs.get(i)) for i, t in enumerate(inputs)]
         if outputs is None:
             st, descs = self.op.infer_shape(ins)
             if st != 0:

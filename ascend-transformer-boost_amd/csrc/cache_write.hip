@@ -38,6 +38,41 @@ __global__ __launch_bounds__(COPY_THREADS) void ReshapeAndCacheKernel(const uint
     }
 }
 
+// A key or value input that is a strided view: element (token, head, channel) sits
+// `offset + token * tokenStride + head * headStride + channel * chanStride` bytes from the base.
+struct StridedRows {
+    const uint8_t *base;
+    int64_t offset, tokenStride, headStride, chanStride;
+    int64_t headBytes; // headDim * element size: what one head contributes to a cache row
+};
+
+// grid.x = token, grid.y = 0 (key) / 1 (value). One workgroup gathers one strided row into its slot.
+// VecT is the widest type every head's start is aligned to when the channels are contiguous,
+// otherwise the element type (one element per access).
+template <typename VecT>
+__global__ __launch_bounds__(COPY_THREADS) void ReshapeAndCacheStridedKernel(StridedRows k, StridedRows v,
+                                                                             uint8_t *__restrict__ keyCache,
+                                                                             uint8_t *__restrict__ valueCache,
+                                                                             const int32_t *__restrict__ slots,
+                                                                             int64_t heads, int64_t numSlots)
+{
+    const int64_t token = blockIdx.x;
+    const int64_t slot = slots[token];
+    if (slot < 0 || slot >= numSlots) {
+        return;
+    }
+    const bool isValue = blockIdx.y == 1;
+    const StridedRows &r = isValue ? v : k;
+    const int64_t perHead = r.headBytes / static_cast<int64_t>(sizeof(VecT));
+    const uint8_t *src = r.base + r.offset + token * r.tokenStride;
+    uint8_t *dst = (isValue ? valueCache : keyCache) + slot * heads * r.headBytes;
+    for (int64_t i = threadIdx.x; i < heads * perHead; i += COPY_THREADS) {
+        const int64_t h = i / perHead;
+        const int64_t c = i - h * perHead;
+        reinterpret_cast<VecT *>(dst)[i] = *reinterpret_cast<const VecT *>(src + h * r.headStride + c * r.chanStride);
+    }
+}
+
 // q = clamp(rint(x / s) + offset, -128, 127); IEEE divide, ties to even.
 __device__ __forceinline__ int8_t QuantOne(float x, float s, int32_t offset)
 {
@@ -157,6 +192,83 @@ extern "C" int atbmi_reshape_and_cache(const void *key, const void *value, void 
         default:
             ReshapeAndCacheKernel<uint8_t><<<grid, COPY_THREADS, 0, s>>>(k8, v8, kc8, vc8, slotMapping, kRowBytes,
                                                                           vRowBytes, numSlots);
+            break;
+    }
+    ATBMI_HIP_CHECK(hipGetLastError());
+    return OK;
+}
+
+extern "C" int atbmi_reshape_and_cache_strided(const void *key, const void *value, void *keyCache, void *valueCache,
+                                               const int32_t *slotMapping, int64_t numTokens, int64_t numKvHeads,
+                                               int64_t headDimK, int64_t headDimV, int64_t numSlots,
+                                               int32_t elemBytes, const int64_t *keyStrides, int64_t keyOffset,
+                                               const int64_t *valueStrides, int64_t valueOffset, void *stream)
+{
+    if (!key || !keyCache || !slotMapping || !keyStrides) {
+        return Fail(ERR_INVALID_PARAM, "reshape_and_cache_strided: key, keyCache, slotMapping, keyStrides must be non-null");
+    }
+    if ((value == nullptr) != (valueCache == nullptr) || (value && !valueStrides)) {
+        return Fail(ERR_INVALID_PARAM, "reshape_and_cache_strided: value, valueCache and valueStrides go together");
+    }
+    if (numTokens < 0 || numTokens > 0x7fffffffLL || numKvHeads <= 0 || headDimK <= 0 || numSlots <= 0 ||
+        (value && headDimV <= 0)) {
+        return Fail(ERR_INVALID_PARAM, "reshape_and_cache_strided: bad extents");
+    }
+    if (elemBytes != 1 && elemBytes != 2) {
+        return Fail(ERR_INVALID_PARAM, "reshape_and_cache_strided: elemBytes must be 1 or 2, got %d", elemBytes);
+    }
+    if (numTokens == 0) {
+        return OK;
+    }
+    auto rows = [&](const void *base, const int64_t *strides, int64_t offset, int64_t headDim) {
+        StridedRows r;
+        r.base = static_cast<const uint8_t *>(base);
+        r.offset = offset * elemBytes;
+        r.tokenStride = strides[0] * elemBytes;
+        r.headStride = strides[1] * elemBytes;
+        r.chanStride = strides[2] * elemBytes;
+        r.headBytes = headDim * elemBytes;
+        return r;
+    };
+    const StridedRows k = rows(key, keyStrides, keyOffset, headDimK);
+    const StridedRows v = value ? rows(value, valueStrides, valueOffset, headDimV) : k;
+    // Widest access: whole vectors when the channels of a head are contiguous and every head of every
+    // token starts on the vector's alignment, single elements otherwise.
+    uintptr_t align = static_cast<uintptr_t>(elemBytes);
+    if (k.chanStride == elemBytes && v.chanStride == elemBytes) {
+        align = 16;
+        auto fits = [&](const StridedRows &r, const void *cache) {
+            return Aligned(r.base, align) && Aligned(cache, align) && r.offset % static_cast<int64_t>(align) == 0 &&
+                   r.tokenStride % static_cast<int64_t>(align) == 0 && r.headStride % static_cast<int64_t>(align) == 0 &&
+                   r.headBytes % static_cast<int64_t>(align) == 0;
+        };
+        while (align > static_cast<uintptr_t>(elemBytes) && !(fits(k, keyCache) && (!value || fits(v, valueCache)))) {
+            align >>= 1;
+        }
+    }
+    dim3 grid(static_cast<unsigned>(numTokens), value ? 2 : 1);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    uint8_t *kc8 = static_cast<uint8_t *>(keyCache);
+    uint8_t *vc8 = static_cast<uint8_t *>(valueCache);
+    StridedRows kk = k, vv = v;
+    if (align > static_cast<uintptr_t>(elemBytes)) { // contiguous channels: the step between accesses is the vector
+        kk.chanStride = vv.chanStride = static_cast<int64_t>(align);
+    }
+    switch (align) {
+        case 16:
+            ReshapeAndCacheStridedKernel<uint4><<<grid, COPY_THREADS, 0, s>>>(kk, vv, kc8, vc8, slotMapping, numKvHeads, numSlots);
+            break;
+        case 8:
+            ReshapeAndCacheStridedKernel<uint2><<<grid, COPY_THREADS, 0, s>>>(kk, vv, kc8, vc8, slotMapping, numKvHeads, numSlots);
+            break;
+        case 4:
+            ReshapeAndCacheStridedKernel<uint32_t><<<grid, COPY_THREADS, 0, s>>>(kk, vv, kc8, vc8, slotMapping, numKvHeads, numSlots);
+            break;
+        case 2:
+            ReshapeAndCacheStridedKernel<uint16_t><<<grid, COPY_THREADS, 0, s>>>(kk, vv, kc8, vc8, slotMapping, numKvHeads, numSlots);
+            break;
+        default:
+            ReshapeAndCacheStridedKernel<uint8_t><<<grid, COPY_THREADS, 0, s>>>(kk, vv, kc8, vc8, slotMapping, numKvHeads, numSlots);
             break;
     }
     ATBMI_HIP_CHECK(hipGetLastError());

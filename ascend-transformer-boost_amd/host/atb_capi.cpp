@@ -95,6 +95,12 @@ int32_t atb_c_create_operation(const char *opName, const void *param, uint64_t p
         memcpy(static_cast<void *>(&p), param, sizeof(p));
         return atb::CreateOperation(p, out);
     }
+    if (!strcmp(opName, "ReshapeAndCacheWithStrideOperation") &&
+        paramSize == sizeof(atb::infer::ReshapeAndCacheWithStrideParam)) {
+        atb::infer::ReshapeAndCacheWithStrideParam p;
+        memcpy(static_cast<void *>(&p), param, sizeof(p));
+        return atb::CreateOperation(p, out);
+    }
     if (!strcmp(opName, "BlockCopyOperation") && paramSize == sizeof(atb::infer::BlockCopyParam)) {
         atb::infer::BlockCopyParam p;
         memcpy(static_cast<void *>(&p), param, sizeof(p));

@@ -15,8 +15,10 @@ Differences from the reference module, all forced by the operators themselves: t
 device ("cuda" in torch); the work runs on torch's current stream of the first device tensor (on a side
 stream ordered after it when that is the null stream, which a Context does not take); operators
 whose outputs are their inputs updated in place (ReshapeAndCache, PagedCacheLoad) return those input
-tensors instead of fresh ones. MultiLatentAttentionParam, BlockCopyParam and PagedCacheLoadParam are
-not bound by the reference's module; they are offered here in the same style.
+tensors instead of fresh ones. ReshapeAndCacheWithStrideParam, MultiLatentAttentionParam, BlockCopyParam
+and PagedCacheLoadParam are not bound by the reference's module; they are offered here in the same style
+(for ReshapeAndCacheWithStride, key / value are [tokens, heads, head_size] tensors that start at the base
+of the storage which the strides and the offset index into).
 """
 import enum
 import re
@@ -106,6 +108,20 @@ class ReshapeAndCacheParam(_Param):
         K_CACHE_V_CACHE_NZ = 2
 
 
+class ReshapeAndCacheWithStrideParam(_Param):
+    _struct = _b.ReshapeAndCacheWithStrideParam
+    _op_name = "ReshapeAndCacheWithStrideOperation"
+
+    class CompressType(enum.IntEnum):
+        COMPRESS_TYPE_UNDEFINED = 0
+        COMPRESS_TYPE_KVHEAD = 1
+        COMPRESS_TYPE_KVHEAD_ROPE = 2
+
+    class KvCacheCfg(enum.IntEnum):
+        K_CACHE_V_CACHE = 0
+        K_CACHE_V_BYPASS = 1
+
+
 class MultiLatentAttentionParam(_Param):
     _struct = _b.MultiLatentAttentionParam
     _op_name = "MultiLatentAttentionOperation"
@@ -148,6 +164,7 @@ class PagedCacheLoadParam(_Param):
 # operation name -> indices of the inputs that its outputs are (updated in place), by input count
 _IN_PLACE = {
     "ReshapeAndCacheOperation": {5: [2, 3], 3: [1]},
+    "ReshapeAndCacheWithStrideOperation": {9: [2, 3], 5: [1]},
     "PagedCacheLoadOperation": {7: [4, 5]},
 }
 

@@ -37,6 +37,25 @@ struct ReshapeAndCacheParam {
     uint8_t rsv[16] = {0}; // must stay zero
 };
 
+// ReshapeAndCache whose key / value inputs are strided views: two (or one) more pairs of host
+// int64 inputs give the element strides [3] and the element offset [1] of each
+// (reference include/atb/infer_op_params.h:531-568).
+struct ReshapeAndCacheWithStrideParam {
+    enum CompressType : int {
+        COMPRESS_TYPE_UNDEFINED = 0,
+        COMPRESS_TYPE_KVHEAD,     // not implemented on MI355X
+        COMPRESS_TYPE_KVHEAD_ROPE // not implemented on MI355X
+    };
+    enum KvCacheCfg : int {
+        K_CACHE_V_CACHE = 0, // inputs: key, value, keyCache, valueCache, slotMapping, kStrides, vStrides, kOffset, vOffset
+        K_CACHE_V_BYPASS,    // inputs: key, keyCache, slotMapping, kStrides, kOffset
+    };
+
+    CompressType compressType = COMPRESS_TYPE_UNDEFINED;
+    KvCacheCfg kvCacheCfg = K_CACHE_V_CACHE;
+    uint8_t rsv[16] = {0}; // must stay zero
+};
+
 // Decode attention: one query token per sequence against that sequence's
 // cached keys/values, found through blockTables and bounded by contextLens.
 struct PagedAttentionParam {
@@ -168,6 +187,7 @@ struct PagedCacheLoadParam {
 };
 
 static_assert(sizeof(ReshapeAndCacheParam) == 24, "ReshapeAndCacheParam ABI size");
+static_assert(sizeof(ReshapeAndCacheWithStrideParam) == 24, "ReshapeAndCacheWithStrideParam ABI size");
 static_assert(sizeof(BlockCopyParam) == 16, "BlockCopyParam ABI size");
 static_assert(sizeof(PagedCacheLoadParam) == 64, "PagedCacheLoadParam ABI size");
 static_assert(sizeof(MultiLatentAttentionParam) == 64, "MultiLatentAttentionParam ABI size");

@@ -34,7 +34,7 @@ public:
                            Context *context) = 0;
 };
 
-// Specialised for infer::PagedAttentionParam, ReshapeAndCacheParam,
+// Specialised for infer::PagedAttentionParam, ReshapeAndCacheParam, ReshapeAndCacheWithStrideParam,
 // MultiLatentAttentionParam, BlockCopyParam and PagedCacheLoadParam.
 template <typename OpParam> Status CreateOperation(const OpParam &opParam, Operation **operation);
 

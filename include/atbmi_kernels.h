@@ -65,6 +65,22 @@ int atbmi_reshape_and_cache(const void *keyDevice, const void *valueDevice, void
                             int32_t elemBytes, void *stream);
 
 /*
+ * KV-cache write from strided views of key / value: element (token, head, channel) of key is read
+ * keyOffset + token * keyStrides[0] + head * keyStrides[1] + channel * keyStrides[2] ELEMENTS from
+ * keyDevice (the same for value); everything else as atbmi_reshape_and_cache. The stride arrays are
+ * host memory and are read before the call returns.
+ * Replaces: ReshapeAndCacheWithStrideOperation's kernel launch, which sets strides and offset on the
+ * key / value tensors of the ReshapeAndCache kernel (reference src/ops/ops_infer/
+ * reshape_and_cache_with_stride/reshape_and_cache_with_stride_ops_runner.cpp:78-104; golden
+ * tests/unittest/ops/reshape_and_cache_with_stride/test_reshape_and_cache_with_stride.cpp:219-245).
+ */
+int atbmi_reshape_and_cache_strided(const void *keyDevice, const void *valueDevice, void *keyCacheDevice,
+                                    void *valueCacheDevice, const int32_t *slotMappingDevice, int64_t numTokens,
+                                    int64_t numKvHeads, int64_t headDimK, int64_t headDimV, int64_t numSlots,
+                                    int32_t elemBytes, const int64_t *keyStridesHost, int64_t keyOffset,
+                                    const int64_t *valueStridesHost, int64_t valueOffset, void *stream);
+
+/*
  * Per-channel int8 quantiser: out[r][c] = clamp(rint(float(x[r][c]) / scale[c]) + offset[c], -128, 127),
  * IEEE fp32 divide, round-half-even, NaN -> 0. offset may be NULL.
  * Replaces: the ELEWISE_QUANT_PER_CHANNEL kernel (golden

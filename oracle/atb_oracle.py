@@ -13,6 +13,9 @@ pinned by tests/test_oracle.py against closed forms, fp64 brute force and
 the invariants of the mathematics (no function is left "parity unpinned"):
 
   reshape_and_cache   tests/apitest/kernelstest/mix/test_reshape_and_cache.py:45-65
+  strided_view        tests/unittest/ops/reshape_and_cache_with_stride/test_reshape_and_cache_with_stride.cpp:
+                      219-245 (element [i0, i1, i2] of the view is storage[offset + sum(i_k * stride_k)]),
+                      :411-433 (the view then goes through the plain reshape_and_cache golden)
   quant_per_channel   tests/apitest/opstest/python/operations/elewise/test_elewise_quant.py:24-32,
                       tests/apitest/kernelstest/elewise/test_quant_per_channel.py:22-40
   paged_attention     tests/apitest/kernelstest/mix/test_paged_attention_common.py:85-118 (grouped
@@ -32,12 +35,6 @@ the invariants of the mathematics (no function is left "parity unpinned"):
                       MultiLatentAttention: tests/apitest/opstest/python/operations/multi_latent_attention/
                       test_multi_latent_attention_lse.py:122-130 (lse = row max + log(row sum)), :148-182,
                       :386-388 (query and cache split [512, 64] along the channels);
-                      several query tokens per sequence (calcType SPEC): tests/apitest/opstest/python/
-                      operations/paged_attention/test_paged_attention_operation_parallel_decoding_910B.py:
-                      75-121 (sequence i owns q_lens[i] consecutive query rows, every one attends to
-                      all k_lens[i] tokens; mask rows [k - q : k] of the square causal mask, or rows
-                      [cu : cu + q] of the per-query-row mask), tests/apitest/kernelstest/mix/
-                      test_paged_attention_mla_mtp.py:120-166 (the same for the MLA cache, fp32 branch);
                       MLA: tests/apitest/opstest/python/operations/paged_attention/
                       test_paged_attention_operation_mla.py:229-262 (V = K[..., :head_size_vo])
   block_copy          tests/apitest/opstest/python/operations/block_copy/test_block_copy.py (golden_calc:
@@ -90,6 +87,19 @@ def reshape_and_cache(key, value, key_cache, value_cache, slot_mapping):
         if vc is not None:
             vc[slot // block_size, slot % block_size] = value[i]
     return kc, vc
+
+
+def strided_view(storage, shape, strides, offset):
+    """The [tokens, heads, head_size] view that ReshapeAndCacheWithStride reads: element
+    (t, h, d) is storage.flat[offset + t * strides[0] + h * strides[1] + d * strides[2]],
+    strides and offset in elements. Returns a contiguous copy."""
+    flat = np.asarray(storage).reshape(-1)
+    idx = np.full(tuple(shape), int(offset), dtype=np.int64)
+    for axis, (n, st) in enumerate(zip(shape, strides)):
+        ext = [1] * len(shape)
+        ext[axis] = n
+        idx += (np.arange(n, dtype=np.int64) * int(st)).reshape(ext)
+    return flat[idx]
 
 
 def block_copy(key_cache, value_cache, src_blocks, dst_blocks, cum_sum):

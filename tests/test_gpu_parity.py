@@ -107,6 +107,91 @@ def test_reshape_and_cache_single_cache_and_out_of_range_slots(binding, oracle, 
     ctx.close()
 
 
+# ------------------------------------------------------------------ ReshapeAndCacheWithStride
+STRIDED_CASES = [
+    # tokens, heads, d, view builder -> (storage elements, strides, offset) per input, what it exercises
+    ("unit_test_view", 2, 32, 128, lambda T, H, D: (T * H * D * 2, (H * D, D, 1), 5)),       # reference unit test: odd offset, 2-byte path
+    ("fused_qkv_k", 64, 8, 128, lambda T, H, D: (T * (32 + 2 * H) * D, ((32 + 2 * H) * D, D, 1), 32 * D)),  # K slice of [T, (32+8+8)*128]
+    ("padded_heads", 9, 3, 40, lambda T, H, D: (T * H * 48 + 8, (H * 48, 48, 1), 4)),        # 8-byte path
+    ("channel_stride", 5, 4, 16, lambda T, H, D: (T * H * D * 3 + 7, (H * D * 3, D * 3, 3), 7)),  # channels not contiguous
+    ("heads_major", 6, 4, 32, lambda T, H, D: (H * T * D, (D, T * D, 1), 0)),                # a [H, T, D] buffer viewed [T, H, D]
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", STRIDED_CASES, ids=lambda c: c[0])
+def test_reshape_and_cache_with_stride_bit_exact(binding, oracle, dev, stream, case, dtype):
+    """Strided key / value views through ReshapeAndCacheWithStrideOperation against the oracle's view
+    + cache write (reference tests/unittest/ops/reshape_and_cache_with_stride/
+    test_reshape_and_cache_with_stride.cpp:411-470: view by strides and offset, then the plain golden)."""
+    name, T, H, D, view = case
+    rng = _rng(31)
+    block, blocks = 16, 8
+    n_store, strides, offset = view(T, H, D)
+    mk = lambda n, lo, hi: torch.from_numpy(rng.integers(lo, hi, size=n).astype(np.float32)).to(dtype).to(dev)
+    k_store, v_store = mk(n_store, 1, 1000), mk(n_store + 16, 1, 1000)
+    v_offset = offset + 16 if name != "unit_test_view" else offset
+    kc = mk((blocks, block, H, D), 2000, 3000)
+    vc = mk((blocks, block, H, D), 2000, 3000)
+    slots = rng.choice(np.arange(-blocks * block, blocks * block), size=T, replace=False).astype(np.int32)
+    slots[0] = max(slots[0], 0)
+    key_view = oracle.strided_view(_bits(k_store).cpu().numpy(), (T, H, D), strides, offset)
+    value_view = oracle.strided_view(_bits(v_store).cpu().numpy(), (T, H, D), strides, v_offset)
+    want_k, want_v = oracle.reshape_and_cache(key_view, value_view, _bits(kc).cpu().numpy(), _bits(vc).cpu().numpy(), slots)
+
+    acl = binding.ACL_FLOAT16 if dtype == torch.float16 else binding.ACL_BF16
+    k_str, v_str = np.array(strides, dtype=np.int64), np.array(strides, dtype=np.int64)
+    k_off, v_off = np.array([offset], dtype=np.int64), np.array([v_offset], dtype=np.int64)
+    host = lambda a: binding.make_tensor(binding.ACL_INT64, list(a.shape), None, host_ptr=a.ctypes.data)
+    ctx = binding.Context(stream)
+    runner = binding.OperationRunner("ReshapeAndCacheWithStrideOperation", binding.ReshapeAndCacheWithStrideParam(), ctx)
+    with torch.cuda.stream(stream):
+        slots_d = torch.from_numpy(slots).to(dev)
+        ins = [binding.make_tensor(acl, [T, H, D], k_store.data_ptr()), binding.make_tensor(acl, [T, H, D], v_store.data_ptr()),
+               kc, vc, slots_d, host(k_str), host(v_str), host(k_off), host(v_off)]
+        runner.run(ins, outputs=[kc, vc])
+    stream.synchronize()
+    assert np.array_equal(_bits(kc).cpu().numpy(), want_k)
+    assert np.array_equal(_bits(vc).cpu().numpy(), want_v)
+    runner.close()
+
+    # single-cache form on the same view
+    kc2 = mk((blocks, block, H, D), 2000, 3000)
+    want_k2, _ = oracle.reshape_and_cache(key_view, None, _bits(kc2).cpu().numpy(), None, slots)
+    single = binding.OperationRunner("ReshapeAndCacheWithStrideOperation",
+                                     binding.ReshapeAndCacheWithStrideParam(kvCacheCfg=1), ctx)
+    with torch.cuda.stream(stream):
+        single.run([binding.make_tensor(acl, [T, H, D], k_store.data_ptr()), kc2, slots_d, host(k_str), host(k_off)],
+                   outputs=[kc2])
+    stream.synchronize()
+    assert np.array_equal(_bits(kc2).cpu().numpy(), want_k2)
+    single.close()
+    ctx.close()
+
+
+def test_reshape_and_cache_with_stride_equals_plain_on_contiguous_input(binding, dev, stream):
+    """With the strides of a contiguous tensor and offset 0 the operation is ReshapeAndCache."""
+    rng = _rng(32)
+    key, value, kc, vc, slots = _rac_inputs(rng, dev, 64, 8, 128, 128, 128, 80, torch.bfloat16)
+    kc2, vc2 = kc.clone(), vc.clone()
+    strides = np.array([8 * 128, 128, 1], dtype=np.int64)
+    zero = np.zeros(1, dtype=np.int64)
+    host = lambda a: binding.make_tensor(binding.ACL_INT64, list(a.shape), None, host_ptr=a.ctypes.data)
+    ctx = binding.Context(stream)
+    plain = binding.OperationRunner("ReshapeAndCacheOperation", binding.ReshapeAndCacheParam(), ctx)
+    strided = binding.OperationRunner("ReshapeAndCacheWithStrideOperation", binding.ReshapeAndCacheWithStrideParam(), ctx)
+    with torch.cuda.stream(stream):
+        slots_d = torch.from_numpy(slots).to(dev)
+        plain.run([key, value, kc, vc, slots_d], outputs=[kc, vc])
+        strided.run([key, value, kc2, vc2, slots_d, host(strides), host(strides), host(zero), host(zero)],
+                    outputs=[kc2, vc2])
+    stream.synchronize()
+    assert torch.equal(_bits(kc), _bits(kc2)) and torch.equal(_bits(vc), _bits(vc2))
+    plain.close()
+    strided.close()
+    ctx.close()
+
+
 # ------------------------------------------------------------------ quantiser
 def test_quant_all_fp16_patterns_bit_exact(binding, oracle, dev, stream):
     k = binding.kernels()

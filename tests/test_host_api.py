@@ -76,6 +76,8 @@ def _make_param(binding, op, p):
         return binding.BlockCopyParam()
     if op == "PagedCacheLoadOperation":
         return binding.PagedCacheLoadParam(**p)
+    if op == "ReshapeAndCacheWithStrideOperation":
+        return binding.ReshapeAndCacheWithStrideParam(**p)
     return binding.ReshapeAndCacheParam(**p)
 
 
@@ -236,6 +238,13 @@ def test_names_and_tensor_counts(binding):
     op.close()
     op = binding.Operation("ReshapeAndCacheOperation", binding.ReshapeAndCacheParam(kvCacheCfg=1))
     assert (op.input_num(), op.output_num()) == (3, 1)
+    op.close()
+    # reference reshape_and_cache_with_stride_operation.cpp:116-138
+    op = binding.Operation("ReshapeAndCacheWithStrideOperation", binding.ReshapeAndCacheWithStrideParam())
+    assert op.get_name() == "ReshapeAndCacheWithStrideOperation" and (op.input_num(), op.output_num()) == (9, 2)
+    op.close()
+    op = binding.Operation("ReshapeAndCacheWithStrideOperation", binding.ReshapeAndCacheWithStrideParam(kvCacheCfg=1))
+    assert (op.input_num(), op.output_num()) == (5, 1)
     op.close()
 
 
@@ -562,6 +571,72 @@ def test_multi_latent_attention_counts_shapes_and_setup(binding, ctx):
     spec.close()
 
 
+def test_reshape_and_cache_with_stride_checks(binding, ctx):
+    """Creation, tensor-count, dim and host-data checks of ReshapeAndCacheWithStrideOperation
+    (reference reshape_and_cache_with_stride_operation.cpp:51-88,163-299; the strides and offsets
+    are host tensors read at Setup, reshape_and_cache_with_stride_ops_runner.cpp:78-104)."""
+    E = binding.ERROR_CODE
+    P = binding.ReshapeAndCacheWithStrideParam
+    for bad in (P(compressType=1), P(compressType=2), P(compressType=3), P(kvCacheCfg=2), P(compressType=-1)):
+        assert binding.Operation("ReshapeAndCacheWithStrideOperation", bad).status == E["ERROR_INVALID_PARAM"]
+    r = P()
+    r.rsv[3] = 1
+    assert binding.Operation("ReshapeAndCacheWithStrideOperation", r).status == E["ERROR_INVALID_PARAM"]
+
+    k_strides = np.array([2 * 8 * 128, 128, 1], dtype=np.int64)
+    v_strides = np.array([2 * 8 * 128, 128, 1], dtype=np.int64)
+    k_off = np.array([0], dtype=np.int64)
+    v_off = np.array([8 * 128], dtype=np.int64)
+
+    def pack(dtype="float16", key=(4, 8, 128), value=(4, 8, 128), kc=(16, 32, 8, 128), vc=(16, 32, 8, 128), slots=(4,),
+             stride_shape=(3,), hosts=True, stride_dtype="int64"):
+        mk = binding.make_tensor
+        hp = lambda a: a.ctypes.data if hosts else None
+        return [mk(dtype, key, FAKE_DEVICE), mk(dtype, value, FAKE_DEVICE), mk(dtype, kc, FAKE_DEVICE),
+                mk(dtype, vc, FAKE_DEVICE), mk("int32", slots, FAKE_DEVICE),
+                mk(stride_dtype, stride_shape, None, host_ptr=hp(k_strides)),
+                mk(stride_dtype, stride_shape, None, host_ptr=hp(v_strides)),
+                mk("int64", (1,), None, host_ptr=hp(k_off)), mk("int64", (1,), None, host_ptr=hp(v_off))]
+
+    op = binding.Operation("ReshapeAndCacheWithStrideOperation", P())
+    st, descs = op.infer_shape(pack())
+    assert st == 0 and [descs[i].dims[j] for i in range(2) for j in range(4)] == [16, 32, 8, 128] * 2
+    outs = lambda: [binding.make_tensor("float16", (16, 32, 8, 128), FAKE_DEVICE) for _ in range(2)]
+    assert op.setup(pack(), outs(), ctx) == (0, 0)
+    assert op.infer_shape(pack(key=(4, 8)))[0] == E["ERROR_INVALID_TENSOR_DIM_NUM"]
+    assert op.infer_shape(pack(stride_shape=(3, 1)))[0] == E["ERROR_INVALID_TENSOR_DIM_NUM"]
+    assert op.infer_shape(pack(value=(5, 8, 128)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.infer_shape(pack(value=(4, 4, 128)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.infer_shape(pack(vc=(16, 64, 8, 128)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.infer_shape(pack(vc=(8, 32, 8, 128)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.infer_shape(pack(kc=(16, 32, 4, 128)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.infer_shape(pack(kc=(16, 32, 8, 64)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    # different head sizes of key and value are fine as long as each matches its cache
+    assert op.infer_shape(pack(value=(4, 8, 64), vc=(16, 32, 8, 64)))[0] == 0
+    assert op.infer_shape(pack(dtype="int8"))[0] == E["ERROR_INVALID_TENSOR_INI_MATCH"]
+    assert op.infer_shape(pack(stride_dtype="int32"))[0] == E["ERROR_INVALID_TENSOR_INI_MATCH"]
+    # outputs must describe the caches
+    wrong = [binding.make_tensor("float16", (16, 32, 8, 64), FAKE_DEVICE) for _ in range(2)]
+    assert op.setup(pack(), wrong, ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    # strides / offsets without host data, or not three strides
+    assert op.setup(pack(hosts=False), outs(), ctx)[0] == E["ERROR_INVALID_PARAM"]
+    assert op.setup(pack(stride_shape=(2,)), outs(), ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    op.close()
+
+    op = binding.Operation("ReshapeAndCacheWithStrideOperation", P(kvCacheCfg=1))
+    mk = binding.make_tensor
+    siso = lambda key=(4, 1, 576), kc=(16, 32, 1, 576), slots=(4,): [
+        mk("bf16", key, FAKE_DEVICE), mk("bf16", kc, FAKE_DEVICE), mk("int32", slots, FAKE_DEVICE),
+        mk("int64", (3,), None, host_ptr=k_strides.ctypes.data), mk("int64", (1,), None, host_ptr=k_off.ctypes.data)]
+    assert op.infer_shape(siso())[0] == 0
+    assert op.setup(siso(), [mk("bf16", (16, 32, 1, 576), FAKE_DEVICE)], ctx) == (0, 0)
+    assert op.infer_shape(siso(slots=(5,)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.infer_shape(siso(kc=(16, 32, 2, 576)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.infer_shape(siso(kc=(16, 32, 1, 512)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.infer_shape(siso(key=(4, 576)))[0] == E["ERROR_INVALID_TENSOR_DIM_NUM"]
+    op.close()
+
+
 def test_torch_atb_surface(pkg):
     """The reference's torch binding surface: snake_case parameter fields, nested enums, name and
     tensor counts (reference src/torch_atb/bindings.cpp:84-93, :520-590, :926-944)."""
@@ -665,6 +740,7 @@ def test_cpp_api_symbols_are_exported(pkg):
     for needle in [
         "atb::CreateOperation<atb::infer::PagedAttentionParam>",
         "atb::CreateOperation<atb::infer::ReshapeAndCacheParam>",
+        "atb::CreateOperation<atb::infer::ReshapeAndCacheWithStrideParam>",
         "atb::DestroyOperation(atb::Operation*)",
         "atb::CreateContext(atb::Context**)",
         "atb::DestroyContext(atb::Context*)",
@@ -682,6 +758,11 @@ def test_kernel_layer_validates_without_a_gpu(binding):
     assert b"non-null" in k.atbmi_last_error()
     assert k.atbmi_reshape_and_cache(1, None, 1, None, 1, 1, 1, 1, 1, 1, 3, None) == 1
     assert k.atbmi_quant_per_channel(1, 5, 1, None, 1, 1, 1, None) == 1
+    strides = np.array([256, 128, 1], dtype=np.int64)
+    assert k.atbmi_reshape_and_cache_strided(1, None, 1, None, 1, 1, 1, 1, 1, 1, 2, None, 0, None, 0, None) == 1
+    assert k.atbmi_reshape_and_cache_strided(1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 2, strides.ctypes.data, 0, None, 0, None) == 1
+    assert k.atbmi_reshape_and_cache_strided(1, None, 1, None, 1, 0, 1, 1, 1, 1, 2, strides.ctypes.data, 0, None, 0,
+                                             None) == 0
     shape = binding.AtbmiPaShape(qDtype=0, kvDtype=0, numHeads=8, numKvHeads=3, headDimK=128, headDimV=128,
                                  blockSize=128, numBlocks=4, maxBlocksPerSeq=4, numQueryRows=4, qkScale=1.0)
     plan = ctypes.c_void_p()

@@ -64,6 +64,33 @@ def test_reshape_and_cache_single_cache(oracle):
     assert np.array_equal(kc[1, 1, 0], key[0, 0]) and kc.sum() == key[0].sum()
 
 
+# ---------------------------------------------------------------- strided_view
+def test_strided_view_matches_library_views_and_loops(oracle):
+    """Against numpy's and torch's own strided views, against the element loop of the reference's unit
+    test, and on a closed form (storage[i] = i makes every element its own address)."""
+    import torch
+    rng = _rng(5)
+    storage = rng.standard_normal(9000).astype(np.float32)
+    cases = [((2, 32, 128), (32 * 128, 128, 1), 5),    # the reference unit test's view (overlapping tokens, odd offset)
+             ((3, 4, 8), (4 * 16 * 3, 16, 1), 16),     # the K slice of a fused [T, 3, H, D] projection
+             ((3, 4, 8), (100, 24, 3), 7),             # channels not contiguous
+             ((2, 3, 4), (12, 4, 1), 0)]               # a plain contiguous tensor
+    for shape, strides, offset in cases:
+        got = oracle.strided_view(storage, shape, strides, offset)
+        lib = np.lib.stride_tricks.as_strided(storage[offset:], shape=shape, strides=[4 * st for st in strides])
+        assert np.array_equal(got, lib)
+        assert np.array_equal(got, torch.as_strided(torch.from_numpy(storage), shape, strides, offset).numpy())
+        addr = oracle.strided_view(np.arange(9000), shape, strides, offset)
+        t, h, d = 1, shape[1] - 1, shape[2] - 2
+        assert addr[t, h, d] == offset + t * strides[0] + h * strides[1] + d * strides[2]
+    shape, strides, offset = cases[2]
+    got = oracle.strided_view(storage, shape, strides, offset)
+    for t in range(shape[0]):
+        for h in range(shape[1]):
+            for d in range(shape[2]):
+                assert got[t, h, d] == storage[offset + t * strides[0] + h * strides[1] + d * strides[2]]
+
+
 # ---------------------------------------------------------------- quantiser
 def test_quant_special_cases(oracle):
     s = np.float32(0.5)
