@@ -1,8 +1,9 @@
 #!/usr/bin/env python3
 """Times the cache-side operations at the size of benchmark workload C2 on one MI355X and
-prints one JSON line per operation: BlockCopy (512 blocks of 256 KB copied in each cache) and
-PagedCacheLoad (all 158 839 cached rows of the 64 sequences gathered), through atb::Operation
-(Setup + Execute per call). Both are HBM-bound byte movers; `roofline.achieved` is their
+prints one JSON line per operation: BlockCopy (512 blocks of 256 KB copied in each cache),
+PagedCacheLoad (all 158 839 cached rows of the 64 sequences gathered) and NormRopeReshape (the
+producer of the combined MLA cache, at the 65 536 tokens of the reference's kernel test), through
+atb::Operation (Setup + Execute per call; NormRopeReshape: Setup once). All are HBM-bound; `roofline.achieved` is their
 algorithmic bytes (every source byte read once, every destination byte written once) over the
 mean kernel time between HIP events on the launch stream.
 
@@ -90,6 +91,34 @@ def main():
                                    "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                                    "algorithmic_bytes": alg}}))
     load.close()
+
+    # ---- NormRopeReshape: 65 536 tokens of 512 + 64 channels into a cache of 512-token blocks
+    tokens, n, r, block = 65536, 512, 64, 512
+    blocks = (tokens + 100 + block - 1) // block
+    x = torch.rand((tokens, 1, n), device=dev).to(torch.float16)
+    gamma = torch.rand((n,), device=dev).to(torch.float16)
+    rope, cos, sin = (torch.rand((tokens, r), device=dev).to(torch.float16) for _ in range(3))
+    slots = torch.from_numpy(rng.permutation(tokens + 100)[:tokens].astype(np.int32)).to(dev)
+    cache = torch.zeros((blocks, block, 1, n + r), dtype=torch.float16, device=dev)
+    fused = b.OperationRunner("NormRopeReshapeOperation", b.NormRopeReshapeParam(epsilon=1e-5), ctx)
+    # The kernel takes less time than Setup + Execute take on the host from Python: Setup once, then Execute
+    # per call, so that the events bracket a stream the host keeps full.
+    ins = [b.tensor_of(t) for t in (x, gamma, rope, cos, sin, slots, cache)]
+    outs = [b.tensor_of(cache)]
+    st, ws = fused.op.setup(ins, outs, ctx)
+    assert st == 0 and ws == 0
+
+    def execute():
+        assert fused.op.execute(ins, outs, None, 0, ctx) == 0
+    ms = timed(execute, stream, args.steps, args.warmup)
+    alg = tokens * ((n + 3 * r) * 2 + 4 + (n + r) * 2) + n * 2
+    print(json.dumps({"operation": "NormRopeReshapeOperation", "workload": "%d tokens: RMSNorm of %d channels + rotary "
+                      "embedding of %d channels written into the combined cache, fp16 (Setup once, Execute per call)" % (tokens, n, r),
+                      "ms_per_call": ms,
+                      "roofline": {"bound": "hbm", "achieved": alg / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
+                                   "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                                   "algorithmic_bytes": alg}}))
+    fused.close()
     ctx.close()
 
 

@@ -88,6 +88,21 @@ class ReshapeAndCacheWithStrideParam(ReshapeAndCacheParam):
     """Byte image of atb::infer::ReshapeAndCacheWithStrideParam (24 bytes, the same fields)."""
 
 
+class NormRopeReshapeParam(ctypes.Structure):
+    """Byte image of atb::infer::NormRopeReshapeParam (28 bytes)."""
+    _fields_ = [("precisionMode", ctypes.c_uint32), ("rotaryCoeff", ctypes.c_uint32), ("epsilon", ctypes.c_float),
+                ("rsv", ctypes.c_uint8 * 16)]
+
+    def __init__(self, **kw):
+        super().__init__()
+        self.rotaryCoeff = 2
+        self.epsilon = 1e-5
+        for k, v in kw.items():
+            if not hasattr(self, k):
+                raise AttributeError("NormRopeReshapeParam has no field " + k)
+            setattr(self, k, v)
+
+
 class BlockCopyParam(ctypes.Structure):
     """Byte image of atb::infer::BlockCopyParam (16 bytes)."""
     _fields_ = [("rsv", ctypes.c_uint8 * 16)]
@@ -163,6 +178,8 @@ def kernels():
         lib.atbmi_reshape_and_cache.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]
         lib.atbmi_reshape_and_cache_strided.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp, i64, vp,
                                                         i64, vp]
+        lib.atbmi_norm_rope_reshape_and_cache.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32,
+                                                          ctypes.c_float, vp]
         lib.atbmi_quant_per_channel.argtypes = [vp, i32, vp, vp, vp, i64, i64, vp]
         lib.atbmi_reshape_and_cache_quant.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]
         lib.atbmi_block_copy.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]

@@ -5,6 +5,7 @@
 // row per sequence); the only hardware concern is that every HBM access is a
 // full-width vector access, so rows are moved as 16-byte pieces whenever the
 // row size and base addresses allow it.
+#include <algorithm>
 #include "atbmi_common.h"
 
 namespace atbmi {
@@ -122,6 +123,153 @@ __global__ __launch_bounds__(256) void ReshapeAndCacheQuantKernel(const void *__
     int8_t *dst = (isValue ? valueCache : keyCache) + slot * row;
     for (int64_t c = threadIdx.x; c < row; c += blockDim.x) {
         dst[c] = QuantOne(Load16(src, token * row + c, isBf16 != 0), scale[c], 0);
+    }
+}
+
+// RMSNorm of the latent row + rotary embedding of the rotary row, written side by side into the
+// token's slot of a single cache (the producer of the combined MLA cache). One wave per token, four
+// tokens per workgroup; fp32 arithmetic, one rounding to the 16-bit type at the end:
+//   cache[slot][0 : normDim]       = (x * (1 / sqrt(mean(x^2) + epsilon))) * gamma
+//   cache[slot][normDim + i]       = r[i] * cos[i] - r[i + half] * sin[i]            (i < half)
+//   cache[slot][normDim + half + i] = r[half + i] * cos[half + i] + r[i] * sin[half + i]
+constexpr int NORM_ROPE_WAVES = 4;
+typedef uint32_t RowVec __attribute__((ext_vector_type(4)));
+// A cache row is written once and read much later by another kernel: non-temporal, so that the write
+// stream does not claim cache lines on its way out.
+__device__ __forceinline__ void StoreRowPiece(uint16_t *p, uint4 v)
+{
+    __builtin_nontemporal_store(RowVec{v.x, v.y, v.z, v.w}, reinterpret_cast<RowVec *>(p));
+}
+
+__device__ __forceinline__ float Half16(uint32_t word, int hi, bool bf16)
+{
+    const uint16_t h = static_cast<uint16_t>(word >> (16 * hi));
+    return bf16 ? Bf16ToFloat(h) : HalfBitsToFloat(h);
+}
+__device__ __forceinline__ uint32_t PackPair(float lo, float hi, bool bf16)
+{
+    const uint32_t l = bf16 ? FloatToBf16(lo) : FloatToHalfBits(lo);
+    const uint32_t h = bf16 ? FloatToBf16(hi) : FloatToHalfBits(hi);
+    return l | (h << 16);
+}
+// (x * inv) * gamma for 8 channels, inv = 1 / rms: the order of the reference's golden
+__device__ __forceinline__ uint4 NormPiece(uint4 v, uint4 g, float inv, bool bf16)
+{
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        o[e] = PackPair(__fmul_rn(__fmul_rn(inv, Half16(w[e], 0, bf16)), Half16(gw[e], 0, bf16)),
+                        __fmul_rn(__fmul_rn(inv, Half16(w[e], 1, bf16)), Half16(gw[e], 1, bf16)), bf16);
+    }
+    return uint4{o[0], o[1], o[2], o[3]};
+}
+__device__ __forceinline__ float SumSquares(uint4 v, bool bf16)
+{
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    float sq = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float f = Half16(w[e >> 1], e & 1, bf16);
+        sq += f * f;
+    }
+    return sq;
+}
+
+// FAST: rows of at most 512 latent channels and at most 128 rotary channels: everything a lane needs is
+// requested up front (one 16-byte piece of the latent row and of gamma, one rotary pair) and the latent
+// row stays in registers between the two passes. Otherwise the row is read twice (the second time
+// from the caches). The kernel is bound by its vector instructions as much as by memory (a row is
+// only 2.5 KB): the element type is a template parameter and every lane has work in every phase.
+template <bool FAST, bool BF16>
+__global__ __launch_bounds__(NORM_ROPE_WAVES *WAVE) void NormRopeCacheKernel(
+    const uint16_t *__restrict__ x, const uint16_t *__restrict__ gamma, const uint16_t *__restrict__ rope,
+    const uint16_t *__restrict__ cosTab, const uint16_t *__restrict__ sinTab, const int32_t *__restrict__ slots,
+    uint16_t *__restrict__ cache, int64_t numTokens, int32_t normDim, int32_t ropeDim, int64_t numSlots,
+    float epsilon)
+{
+    const int lane = threadIdx.x % WAVE;
+    constexpr bool bf16 = BF16;
+    const int half = ropeDim / 2;
+    // a wave walks the tokens with the stride of the whole launch
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * NORM_ROPE_WAVES;
+    for (int64_t token = static_cast<int64_t>(blockIdx.x) * NORM_ROPE_WAVES + threadIdx.x / WAVE; token < numTokens;
+         token += stride) {
+        // The slot is asked for first and looked at last (FAST): a row's loads do not wait for it, and
+        // the few rows that turn out to be skipped cost their loads.
+        const int64_t slot = slots[token];
+        if (!FAST && (slot < 0 || slot >= numSlots)) {
+            continue;
+        }
+        const uint16_t *xr = x + token * normDim;
+        const uint16_t *rr = rope + token * ropeDim;
+        const uint16_t *cr = cosTab + token * ropeDim;
+        const uint16_t *sr = sinTab + token * ropeDim;
+        // Rotary pair (i, half + i): two products and a sum, each rounded, as the reference kernel's
+        // vector unit does them.
+        auto turn = [&](int i, uint16_t *out) {
+            const float a = Load16(rr, i, bf16), b = Load16(rr, i + half, bf16);
+            const float lo = __fadd_rn(__fmul_rn(a, Load16(cr, i, bf16)), __fmul_rn(-b, Load16(sr, i, bf16)));
+            const float hi = __fadd_rn(__fmul_rn(b, Load16(cr, i + half, bf16)), __fmul_rn(a, Load16(sr, i + half, bf16)));
+            Store16(out, normDim + i, lo, bf16);
+            Store16(out, normDim + half + i, hi, bf16);
+        };
+        // normDim is a multiple of 8 (checked by the host): a lane takes 8 consecutive channels at a time
+        if constexpr (FAST) {
+            const int c = lane * 8;
+            const bool mine = c < normDim;
+            const bool turns = lane < half;
+            uint4 xv = {0u, 0u, 0u, 0u}, gv = xv;
+            uint16_t ra = 0, rb = 0, ca = 0, cb = 0, sa = 0, sb = 0;
+            if (mine) {
+                xv = *reinterpret_cast<const uint4 *>(xr + c);
+                gv = *reinterpret_cast<const uint4 *>(gamma + c);
+            }
+            if (turns) {
+                ra = rr[lane]; rb = rr[half + lane];
+                ca = cr[lane]; cb = cr[half + lane];
+                sa = sr[lane]; sb = sr[half + lane];
+            }
+            float sq = SumSquares(xv, bf16);
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                sq += __shfl_xor(sq, off, WAVE);
+            }
+            const float inv = __fdiv_rn(1.0f, __fsqrt_rn(__fdiv_rn(sq, static_cast<float>(normDim)) + epsilon));
+            if (slot < 0 || slot >= numSlots) {
+                continue;
+            }
+            uint16_t *out = cache + slot * (static_cast<int64_t>(normDim) + ropeDim);
+            if (mine) {
+                StoreRowPiece(out + c, NormPiece(xv, gv, inv, bf16));
+            }
+            if (turns) {
+                const float a = Half16(ra, 0, bf16), b = Half16(rb, 0, bf16);
+                const float lo = __fadd_rn(__fmul_rn(a, Half16(ca, 0, bf16)), __fmul_rn(-b, Half16(sa, 0, bf16)));
+                const float hi = __fadd_rn(__fmul_rn(b, Half16(cb, 0, bf16)), __fmul_rn(a, Half16(sb, 0, bf16)));
+                Store16(out, normDim + lane, lo, bf16);
+                Store16(out, normDim + half + lane, hi, bf16);
+            }
+        } else {
+            uint16_t *out = cache + slot * (static_cast<int64_t>(normDim) + ropeDim);
+            float sq = 0.0f;
+            for (int c = lane * 8; c < normDim; c += WAVE * 8) {
+                sq += SumSquares(*reinterpret_cast<const uint4 *>(xr + c), bf16);
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                sq += __shfl_xor(sq, off, WAVE);
+            }
+            const float inv = __fdiv_rn(1.0f, __fsqrt_rn(__fdiv_rn(sq, static_cast<float>(normDim)) + epsilon));
+            for (int c = lane * 8; c < normDim; c += WAVE * 8) { // second pass: the row is still in the caches
+                StoreRowPiece(out + c, NormPiece(*reinterpret_cast<const uint4 *>(xr + c),
+                                                 *reinterpret_cast<const uint4 *>(gamma + c), inv, bf16));
+            }
+            for (int i = lane; i < half; i += WAVE) {
+                turn(i, out);
+            }
+        }
     }
 }
 
@@ -271,6 +419,50 @@ extern "C" int atbmi_reshape_and_cache_strided(const void *key, const void *valu
             ReshapeAndCacheStridedKernel<uint8_t><<<grid, COPY_THREADS, 0, s>>>(kk, vv, kc8, vc8, slotMapping, numKvHeads, numSlots);
             break;
     }
+    ATBMI_HIP_CHECK(hipGetLastError());
+    return OK;
+}
+
+extern "C" int atbmi_norm_rope_reshape_and_cache(const void *x, const void *gamma, const void *keyRope,
+                                                 const void *cosTable, const void *sinTable,
+                                                 const int32_t *slotMapping, void *keyCache, int64_t numTokens,
+                                                 int64_t normDim, int64_t ropeDim, int64_t numSlots, int32_t dtype,
+                                                 float epsilon, void *stream)
+{
+    if (!x || !gamma || !keyRope || !cosTable || !sinTable || !slotMapping || !keyCache) {
+        return Fail(ERR_INVALID_PARAM, "norm_rope_reshape_and_cache: every tensor must be non-null");
+    }
+    if (dtype != ATBMI_F16 && dtype != ATBMI_BF16) {
+        return Fail(ERR_INVALID_PARAM, "norm_rope_reshape_and_cache: tensors must be fp16 or bf16");
+    }
+    if (numTokens < 0 || numTokens > 0x7fffffffLL || normDim <= 0 || ropeDim <= 0 || numSlots <= 0 ||
+        normDim > (1 << 20) || ropeDim > (1 << 20)) {
+        return Fail(ERR_INVALID_PARAM, "norm_rope_reshape_and_cache: bad extents");
+    }
+    if (normDim % 8 != 0 || ropeDim % 2 != 0) {
+        return Fail(ERR_INVALID_PARAM, "norm_rope_reshape_and_cache: normDim must be a multiple of 8 and ropeDim even, "
+                                       "got %lld and %lld", (long long)normDim, (long long)ropeDim);
+    }
+    if (!Aligned(x, 16) || !Aligned(gamma, 16) || !Aligned(keyCache, 16) || (ropeDim * 2) % 16 != 0) {
+        return Fail(ERR_INVALID_PARAM, "norm_rope_reshape_and_cache: x, gamma and keyCache must be 16-byte aligned and "
+                                       "a rotary row a multiple of 16 bytes");
+    }
+    if (numTokens == 0) {
+        return OK;
+    }
+    // one wave per token up to 262 144 tokens (more waves in flight hide more of each row's load latency
+    // than longer-lived waves do); beyond that the waves loop over the tokens
+    const unsigned grid = static_cast<unsigned>(std::min<int64_t>((numTokens + NORM_ROPE_WAVES - 1) / NORM_ROPE_WAVES, 65536));
+    // the register-resident form: one 16-byte piece of the latent row and one rotary pair per lane
+    const bool fast = normDim <= WAVE * 8 && ropeDim <= WAVE * 2;
+    const bool bf16 = dtype == ATBMI_BF16;
+    auto kernel = fast ? (bf16 ? NormRopeCacheKernel<true, true> : NormRopeCacheKernel<true, false>)
+                       : (bf16 ? NormRopeCacheKernel<false, true> : NormRopeCacheKernel<false, false>);
+    kernel<<<grid, NORM_ROPE_WAVES * WAVE, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const uint16_t *>(x), static_cast<const uint16_t *>(gamma), static_cast<const uint16_t *>(keyRope),
+        static_cast<const uint16_t *>(cosTable), static_cast<const uint16_t *>(sinTable), slotMapping,
+        static_cast<uint16_t *>(keyCache), numTokens, static_cast<int32_t>(normDim), static_cast<int32_t>(ropeDim),
+        numSlots, epsilon);
     ATBMI_HIP_CHECK(hipGetLastError());
     return OK;
 }

@@ -167,6 +167,16 @@ struct MultiLatentAttentionParam {
     uint8_t rsv[32] = {0}; // must stay zero
 };
 
+// RMSNorm of the latent row, rotary embedding of the rotary row and the write of both, side by side,
+// into a single cache: the step that fills the combined MLA cache
+// (reference include/atb/infer_op_params.h:2697-2716).
+struct NormRopeReshapeParam {
+    uint32_t precisionMode = 0; // passed through to the kernel by the reference; the arithmetic here is fp32 always
+    uint32_t rotaryCoeff = 2;   // 2: rotate halves (the only form the reference's goldens define)
+    float epsilon = 1e-5;       // added to the mean square; |epsilon| must not be below FLT_MIN
+    uint8_t rsv[16] = {0};      // must stay zero
+};
+
 // Copies whole blocks of the key and value caches onto other blocks of the same caches
 // (reference include/atb/infer_op_params.h:1208-1217).
 struct BlockCopyParam {
@@ -188,6 +198,7 @@ struct PagedCacheLoadParam {
 
 static_assert(sizeof(ReshapeAndCacheParam) == 24, "ReshapeAndCacheParam ABI size");
 static_assert(sizeof(ReshapeAndCacheWithStrideParam) == 24, "ReshapeAndCacheWithStrideParam ABI size");
+static_assert(sizeof(NormRopeReshapeParam) == 28, "NormRopeReshapeParam ABI size");
 static_assert(sizeof(BlockCopyParam) == 16, "BlockCopyParam ABI size");
 static_assert(sizeof(PagedCacheLoadParam) == 64, "PagedCacheLoadParam ABI size");
 static_assert(sizeof(MultiLatentAttentionParam) == 64, "MultiLatentAttentionParam ABI size");

@@ -35,7 +35,7 @@ public:
 };
 
 // Specialised for infer::PagedAttentionParam, ReshapeAndCacheParam, ReshapeAndCacheWithStrideParam,
-// MultiLatentAttentionParam, BlockCopyParam and PagedCacheLoadParam.
+// NormRopeReshapeParam, MultiLatentAttentionParam, BlockCopyParam and PagedCacheLoadParam.
 template <typename OpParam> Status CreateOperation(const OpParam &opParam, Operation **operation);
 
 Status DestroyOperation(Operation *operation);

@@ -81,6 +81,24 @@ int atbmi_reshape_and_cache_strided(const void *keyDevice, const void *valueDevi
                                     const int64_t *valueStridesHost, int64_t valueOffset, void *stream);
 
 /*
+ * RMSNorm + rotary embedding + cache write in one kernel, the producer of the combined (MLA) cache:
+ * for token i with slot s = slotMapping[i] in [0, numSlots),
+ *   keyCache[s][0 : normDim]            = gamma * x[i] / sqrt(mean(x[i]^2) + epsilon)
+ *   keyCache[s][normDim : normDim+ropeDim] = r * cos[i] + rotate_half(r) * sin[i],  r = keyRope[i],
+ *   rotate_half(r) = concat(-r[ropeDim/2:], r[:ropeDim/2]),
+ * computed in fp32 and rounded once to dtype (fp16 or bf16, the type of every tensor). keyCache is
+ * viewed as [numSlots, normDim + ropeDim]; other slots keep their content.
+ * Replaces: the RmsNormAndRopeAndReshapeAndCache kernel behind NormRopeReshapeOperation (reference
+ * src/kernels/mixkernels/rms_norm_and_rope_and_reshape_and_cache/op_kernel/
+ * rms_norm_and_rope_and_reshape_and_cache.cpp:160-305; golden tests/apitest/opstest/python/operations/
+ * norm_rope_reshape/test_norm_rope_reshape.py:21-71).
+ */
+int atbmi_norm_rope_reshape_and_cache(const void *xDevice, const void *gammaDevice, const void *keyRopeDevice,
+                                      const void *cosDevice, const void *sinDevice, const int32_t *slotMappingDevice,
+                                      void *keyCacheDevice, int64_t numTokens, int64_t normDim, int64_t ropeDim,
+                                      int64_t numSlots, int32_t dtype, float epsilon, void *stream);
+
+/*
  * Per-channel int8 quantiser: out[r][c] = clamp(rint(float(x[r][c]) / scale[c]) + offset[c], -128, 127),
  * IEEE fp32 divide, round-half-even, NaN -> 0. offset may be NULL.
  * Replaces: the ELEWISE_QUANT_PER_CHANNEL kernel (golden

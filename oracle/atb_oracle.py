@@ -16,6 +16,10 @@ the invariants of the mathematics (no function is left "parity unpinned"):
   strided_view        tests/unittest/ops/reshape_and_cache_with_stride/test_reshape_and_cache_with_stride.cpp:
                       219-245 (element [i0, i1, i2] of the view is storage[offset + sum(i_k * stride_k)]),
                       :411-433 (the view then goes through the plain reshape_and_cache golden)
+  norm_rope_reshape   tests/apitest/opstest/python/operations/norm_rope_reshape/test_norm_rope_reshape.py:21-71
+                      and tests/apitest/kernelstest/mix/test_rms_norm_and_rope_and_reshape_and_cache_bf16.py:24-74
+                      (rms = 1 / sqrt(mean(x^2) + eps); x * rms * gamma; r * cos + rotate_half(r) * sin with
+                      rotate_half = concat(-second half, first half); both written side by side into the slot)
   quant_per_channel   tests/apitest/opstest/python/operations/elewise/test_elewise_quant.py:24-32,
                       tests/apitest/kernelstest/elewise/test_quant_per_channel.py:22-40
   paged_attention     tests/apitest/kernelstest/mix/test_paged_attention_common.py:85-118 (grouped
@@ -100,6 +104,30 @@ def strided_view(storage, shape, strides, offset):
         ext[axis] = n
         idx += (np.arange(n, dtype=np.int64) * int(st)).reshape(ext)
     return flat[idx]
+
+
+def norm_rope_reshape(x, gamma, key_rope, cos, sin, slot_mapping, key_cache, epsilon, out_dtype=np.float16):
+    """Returns an updated copy of key_cache [blocks, block, 1, norm_dim + rope_dim]: for token i with
+    slot s >= 0, the RMS-normalised x[i] (times gamma) followed by the rotated key_rope[i]. fp32
+    arithmetic, rounded once to out_dtype (np.float16, or "bf16" for round-to-nearest-even bfloat16 values
+    kept in float32)."""
+    xf = np.asarray(x, dtype=np.float32)
+    mean_sq = np.sum(np.square(xf), axis=-1, keepdims=True) / np.float32(xf.shape[-1])
+    rms = np.float32(1.0) / np.sqrt(mean_sq + np.float32(epsilon))
+    normed = rms * xf * np.asarray(gamma, dtype=np.float32)
+    r = np.asarray(key_rope, dtype=np.float32)
+    first, second = np.split(r, 2, axis=1)
+    rotated = np.concatenate((-second, first), axis=1)
+    roped = r * np.asarray(cos, dtype=np.float32) + rotated * np.asarray(sin, dtype=np.float32)
+    rows = np.concatenate((normed.reshape(normed.shape[0], -1), roped), axis=-1)
+    rows = bf16_round(rows) if out_dtype == "bf16" else rows.astype(out_dtype)
+    kc = np.array(key_cache, copy=True)
+    block_size = kc.shape[1]
+    for i, slot in enumerate(np.asarray(slot_mapping).tolist()):
+        if slot < 0:
+            continue
+        kc[slot // block_size, slot % block_size, 0] = rows[i]
+    return kc
 
 
 def block_copy(key_cache, value_cache, src_blocks, dst_blocks, cum_sum):

@@ -9,6 +9,7 @@ status, tagged C: for CreateOperation, I: for InferShape, S: for Setup):
     tests/apitest/opstest/csv/multi_latent_attention.csv
     tests/apitest/opstest/csv/block_copy.csv
     tests/apitest/opstest/csv/paged_cache_load.csv
+    tests/apitest/opstest/csv/norm_rope_reshape.csv
 Those rows are data, not code. This script copies the rows written for the
 Ascend910B feature set (the one this library mirrors) into
     tests/golden/paged_attention_cases.json
@@ -16,6 +17,7 @@ Ascend910B feature set (the one this library mirrors) into
     tests/golden/multi_latent_attention_cases.json
     tests/golden/block_copy_cases.json
     tests/golden/paged_cache_load_cases.json
+    tests/golden/norm_rope_reshape_cases.json
 so the parity tests can run where the reference tree is absent.
 
 Run from the repository root in a container that has /root/reference:
@@ -41,7 +43,7 @@ def shapes(field):
     return out
 
 
-def convert(name):
+def convert(name, also_untagged=False):
     path = os.path.join(REF, "tests/apitest/opstest/csv", name + ".csv")
     rows = list(csv.reader(open(path, newline=""), delimiter="|"))
     header = [h.strip() for h in rows[0]]
@@ -50,7 +52,8 @@ def convert(name):
         if not any(c.strip() for c in row):
             continue
         d = {h: v.strip() for h, v in zip(header, row)}
-        if d.get("SocVersion") != "Ascend910B":
+        # (a creation-only row may leave every column after the param empty, the product tag included)
+        if d.get("SocVersion") != "Ascend910B" and not (also_untagged and d.get("SocVersion", "") == ""):
             continue
         # OutNum is what the harness hands to the operation (BlockCopy lists two output columns but takes none)
         n_out = int(d["OutNum"]) if d.get("OutNum", "").strip().isdigit() else None
@@ -83,3 +86,4 @@ if __name__ == "__main__":
     convert("multi_latent_attention")
     convert("block_copy")
     convert("paged_cache_load")
+    convert("norm_rope_reshape", also_untagged=True)

@@ -192,6 +192,86 @@ def test_reshape_and_cache_with_stride_equals_plain_on_contiguous_input(binding,
     ctx.close()
 
 
+# ------------------------------------------------------------------ NormRopeReshape
+def _reference_standard(got, want, factor_max, factor_mean):
+    """The reference's own pass criterion for this operator (tests/apitest/opstest/python/operations/
+    norm_rope_reshape/test_norm_rope_reshape.py:74-85): |diff| <= factor_max * max(1, |golden|) everywhere
+    and |mean(diff / max(1, |golden|))| <= factor_mean."""
+    diff = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    scale = np.maximum(1.0, np.abs(want.astype(np.float64)))
+    assert np.all(diff <= factor_max * scale), float((diff / scale).max())
+    assert abs(np.mean(diff / scale)) <= factor_mean
+
+
+@pytest.mark.parametrize("lo,hi", [(0.0, 1.0), (-100.0, 100.0)])
+def test_norm_rope_reshape_operation_fp16(binding, oracle, dev, stream, lo, hi):
+    """The reference's operation test shape (64 tokens, 512 + 64 channels, 192 blocks of 128) with its
+    [0, 1) inputs, and the CSV rows' [-100, 100] range; fp16. Tolerance: the reference's fp16 standard
+    2^-8 / 2^-10; on top of it every element must be within one fp16 step of the fp32 oracle rounded once."""
+    rng = _rng(41)
+    T, n, r, blocks, block = 64, 512, 64, 192, 128
+    u = lambda *shape: torch.from_numpy(rng.uniform(lo, hi, size=shape).astype(np.float32)).to(torch.float16)
+    x, gamma, rope, cos, sin = u(T, 1, n), u(n), u(T, r), u(T, r), u(T, r)
+    cache = u(blocks, block, 1, n + r)
+    slots = rng.choice(np.arange(-50, blocks * block), size=T, replace=False).astype(np.int32)
+    slots[:3] = [-1, 0, blocks * block - 1]
+    want = oracle.norm_rope_reshape(x.float().numpy(), gamma.float().numpy(), rope.float().numpy(), cos.float().numpy(),
+                                    sin.float().numpy(), slots, cache.numpy(), 1e-5)
+    ctx = binding.Context(stream)
+    runner = binding.OperationRunner("NormRopeReshapeOperation", binding.NormRopeReshapeParam(epsilon=1e-5), ctx)
+    with torch.cuda.stream(stream):
+        cache_d = cache.to(dev)
+        ins = [t.to(dev) for t in (x, gamma, rope, cos, sin)] + [torch.from_numpy(slots).to(dev), cache_d]
+        runner.run(ins, outputs=[cache_d])
+    stream.synchronize()
+    got = cache_d.cpu().numpy()
+    _reference_standard(got, want, 2.0 ** -8, 2.0 ** -10)
+    # within one step of the 16-bit grid; rows of skipped and untouched slots are bit-identical
+    step = np.abs(np.nextafter(want, np.float16(np.inf)).astype(np.float32) - want.astype(np.float32))
+    assert np.all(np.abs(got.astype(np.float32) - want.astype(np.float32)) <= step)
+    assert np.mean(got.view(np.int16) != want.view(np.int16)) < 0.01
+    flat_got, flat_in = got.reshape(blocks * block, -1), cache.numpy().reshape(blocks * block, -1)
+    untouched = np.setdiff1d(np.arange(blocks * block), slots[slots >= 0])
+    assert np.array_equal(flat_got[untouched].view(np.int16), flat_in[untouched].view(np.int16))
+    runner.close()
+    ctx.close()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_norm_rope_reshape_kernel_many_tokens(binding, oracle, dev, stream, dtype):
+    """The kernel-level test of the reference (tests/apitest/kernelstest/mix/
+    test_rms_norm_and_rope_and_reshape_and_cache_bf16.py:91-130: tokens x 512 + 64 channels, inputs in
+    [-100, 100], slots a random permutation, blocks of 512) through the C ABI, with 8192 tokens and
+    odd row sizes as a second shape. Tolerance: the reference's standard, 2^-7 for bf16 and 2^-8 / 2^-10 for fp16."""
+    k = binding.kernels()
+    rng = _rng(42)
+    for T, n, r, block in ((8192, 512, 64, 512), (37, 48, 16, 16), (19, 1024, 40, 16)):
+        blocks = (T + 100 + block - 1) // block
+        u = lambda *shape: torch.from_numpy(rng.uniform(-100, 100, size=shape).astype(np.float32)).to(dtype)
+        x, gamma, rope, cos, sin = u(T, 1, n), u(n), u(T, r), u(T, r), u(T, r)
+        slots = rng.permutation(T + 100)[:T].astype(np.int32)
+        cache = torch.zeros((blocks, block, 1, n + r), dtype=dtype)
+        is_bf16 = dtype == torch.bfloat16
+        want = oracle.norm_rope_reshape(x.float().numpy(), gamma.float().numpy(), rope.float().numpy(),
+                                        cos.float().numpy(), sin.float().numpy(), slots, cache.float().numpy(), 1e-5,
+                                        out_dtype="bf16" if is_bf16 else np.float16)
+        with torch.cuda.stream(stream):
+            d = [t.to(dev) for t in (x, gamma, rope, cos, sin)]
+            slots_d = torch.from_numpy(slots).to(dev)
+            cache_d = cache.to(dev)
+            rc = k.atbmi_norm_rope_reshape_and_cache(d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(),
+                                                     d[4].data_ptr(), slots_d.data_ptr(), cache_d.data_ptr(), T, n, r,
+                                                     blocks * block, 1 if is_bf16 else 0, 1e-5, stream.cuda_stream)
+        stream.synchronize()
+        assert rc == 0, binding.last_kernel_error()
+        got = cache_d.float().cpu().numpy()
+        if is_bf16:
+            _reference_standard(got, want.astype(np.float32), 2.0 ** -7, 2.0 ** -7)
+        else:
+            _reference_standard(got, want.astype(np.float32), 2.0 ** -8, 2.0 ** -10)
+        assert np.mean(got != want.astype(np.float32)) < 0.01
+
+
 # ------------------------------------------------------------------ quantiser
 def test_quant_all_fp16_patterns_bit_exact(binding, oracle, dev, stream):
     k = binding.kernels()

@@ -30,6 +30,7 @@ RAC_CASES = _load("reshape_and_cache")
 MLA_CASES = _load("multi_latent_attention")
 BLOCK_COPY_CASES = _load("block_copy")
 CACHE_LOAD_CASES = _load("paged_cache_load")
+NORM_ROPE_CASES = _load("norm_rope_reshape")
 
 
 def _pa_unimplemented(p):
@@ -78,6 +79,11 @@ def _make_param(binding, op, p):
         return binding.PagedCacheLoadParam(**p)
     if op == "ReshapeAndCacheWithStrideOperation":
         return binding.ReshapeAndCacheWithStrideParam(**p)
+    if op == "NormRopeReshapeOperation":
+        param = binding.NormRopeReshapeParam(**{k: v for k, v in p.items() if k != "rsv"})
+        for i, v in enumerate(p.get("rsv", [])):
+            param.rsv[i] = v
+        return param
     return binding.ReshapeAndCacheParam(**p)
 
 
@@ -178,6 +184,11 @@ def test_paged_cache_load_table(binding, ctx, case):
     # the fractal-NZ cache layout (kvCacheCfg 0, the param's default) is rejected when the operation is created
     nz = case["param"].get("kvCacheCfg", 0) == 0
     _check(binding, case, ctx, nz and not case["expected"].startswith("C:"))
+
+
+@pytest.mark.parametrize("case", NORM_ROPE_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
+def test_norm_rope_reshape_table(binding, ctx, case):
+    _check(binding, case, ctx, False)
 
 
 @pytest.mark.parametrize("case", RAC_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
@@ -637,6 +648,57 @@ def test_reshape_and_cache_with_stride_checks(binding, ctx):
     op.close()
 
 
+def test_norm_rope_reshape_checks(binding, ctx):
+    """Creation, dim and output checks of NormRopeReshapeOperation (reference
+    norm_rope_reshape_operation.cpp:35-55,77-106,113-201; kernel-library checks
+    rms_norm_and_rope_and_reshape_and_cache_operation.cpp:63-117)."""
+    E = binding.ERROR_CODE
+    P = binding.NormRopeReshapeParam
+    assert binding.Operation("NormRopeReshapeOperation", P(epsilon=0.0)).status == E["ERROR_INVALID_PARAM"]
+    assert binding.Operation("NormRopeReshapeOperation", P(epsilon=1e-39)).status == E["ERROR_INVALID_PARAM"]
+    assert binding.Operation("NormRopeReshapeOperation", P(epsilon=-1e-5)).status == 0   # |epsilon| is what counts
+    assert binding.Operation("NormRopeReshapeOperation", P(rotaryCoeff=4)).status == E["ERROR_INVALID_PARAM"]
+    assert ctypes.sizeof(P) == 28
+    mk = binding.make_tensor
+
+    def pack(x=(64, 1, 512), gamma=(512,), rope=(64, 64), cos=(64, 64), sin=(64, 64), slots=(64,),
+             cache=(192, 128, 1, 576), gamma_dtype="float16"):
+        return [mk("float16", x, FAKE_DEVICE), mk(gamma_dtype, gamma, FAKE_DEVICE), mk("float16", rope, FAKE_DEVICE),
+                mk("float16", cos, FAKE_DEVICE), mk("float16", sin, FAKE_DEVICE), mk("int32", slots, FAKE_DEVICE),
+                mk("float16", cache, FAKE_DEVICE)]
+
+    op = binding.Operation("NormRopeReshapeOperation", P())
+    assert op.get_name() == "NormRopeReshapeOperation" and (op.input_num(), op.output_num()) == (7, 1)
+    st, descs = op.infer_shape(pack())
+    assert st == 0 and [descs[0].dims[i] for i in range(4)] == [192, 128, 1, 576]
+    out = lambda shape=(192, 128, 1, 576), dtype="float16", fmt="nd": [mk(dtype, shape, FAKE_DEVICE, fmt=fmt)]
+    assert op.setup(pack(), out(), ctx) == (0, 0)
+    assert op.infer_shape(pack(x=(64, 512)))[0] == E["ERROR_INVALID_TENSOR_DIM_NUM"]
+    assert op.infer_shape(pack(cache=(192, 128, 576)))[0] == E["ERROR_INVALID_TENSOR_DIM_NUM"]
+    assert op.infer_shape(pack(gamma=(496,)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.infer_shape(pack(rope=(63, 64)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.infer_shape(pack(cos=(63, 64)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.infer_shape(pack(cos=(64, 32)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.infer_shape(pack(sin=(64, 32)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.infer_shape(pack(cache=(192, 128, 1, 512)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.infer_shape(pack(x=(64, 1, 520), gamma=(520,), cache=(192, 128, 1, 584)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    # rows far beyond the reference's Ascend buffer bound are fine here
+    assert op.infer_shape(pack(x=(64, 1, 16384), gamma=(16384,), cache=(192, 128, 1, 16448)))[0] == 0
+    # the output against the cache: a dtype or format outside the operation's table is caught by the table
+    # check that runs first; then rank and dims
+    assert op.setup(pack(), out(dtype="bf16"), ctx)[0] == E["ERROR_INVALID_TENSOR_INI_MATCH"]
+    assert op.setup(pack(), out(fmt="fractal_nz"), ctx)[0] == E["ERROR_INVALID_TENSOR_INI_MATCH"]
+    assert op.setup(pack(), out(shape=(192, 128, 576)), ctx)[0] == E["ERROR_INVALID_TENSOR_SIZE"]
+    assert op.setup(pack(), out(shape=(192, 64, 1, 576)), ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    # the kernel library's own checks, met at Setup: one head, equal row counts, rows in units of 16
+    assert op.setup(pack(x=(64, 2, 512)), out(), ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.setup(pack(slots=(63,)), out(), ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.setup(pack(sin=(63, 64)), out(), ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.setup(pack(rope=(64, 8), cos=(64, 8), sin=(64, 8), cache=(192, 128, 1, 520)),
+                    out(shape=(192, 128, 1, 520)), ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    op.close()
+
+
 def test_torch_atb_surface(pkg):
     """The reference's torch binding surface: snake_case parameter fields, nested enums, name and
     tensor counts (reference src/torch_atb/bindings.cpp:84-93, :520-590, :926-944)."""
@@ -741,6 +803,7 @@ def test_cpp_api_symbols_are_exported(pkg):
         "atb::CreateOperation<atb::infer::PagedAttentionParam>",
         "atb::CreateOperation<atb::infer::ReshapeAndCacheParam>",
         "atb::CreateOperation<atb::infer::ReshapeAndCacheWithStrideParam>",
+        "atb::CreateOperation<atb::infer::NormRopeReshapeParam>",
         "atb::DestroyOperation(atb::Operation*)",
         "atb::CreateContext(atb::Context**)",
         "atb::DestroyContext(atb::Context*)",
@@ -758,6 +821,11 @@ def test_kernel_layer_validates_without_a_gpu(binding):
     assert b"non-null" in k.atbmi_last_error()
     assert k.atbmi_reshape_and_cache(1, None, 1, None, 1, 1, 1, 1, 1, 1, 3, None) == 1
     assert k.atbmi_quant_per_channel(1, 5, 1, None, 1, 1, 1, None) == 1
+    assert k.atbmi_norm_rope_reshape_and_cache(16, 16, 16, 16, 16, 16, None, 1, 512, 64, 128, 0, 1e-5, None) == 1
+    assert k.atbmi_norm_rope_reshape_and_cache(16, 16, 16, 16, 16, 16, 16, 1, 500, 64, 128, 0, 1e-5, None) == 1
+    assert k.atbmi_norm_rope_reshape_and_cache(16, 16, 16, 16, 16, 16, 16, 1, 512, 64, 128, 2, 1e-5, None) == 1
+    assert k.atbmi_norm_rope_reshape_and_cache(16, 8, 16, 16, 16, 16, 16, 1, 512, 64, 128, 0, 1e-5, None) == 1
+    assert k.atbmi_norm_rope_reshape_and_cache(16, 16, 16, 16, 16, 16, 16, 0, 512, 64, 128, 0, 1e-5, None) == 0
     strides = np.array([256, 128, 1], dtype=np.int64)
     assert k.atbmi_reshape_and_cache_strided(1, None, 1, None, 1, 1, 1, 1, 1, 1, 2, None, 0, None, 0, None) == 1
     assert k.atbmi_reshape_and_cache_strided(1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 2, strides.ctypes.data, 0, None, 0, None) == 1

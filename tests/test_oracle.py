@@ -91,6 +91,61 @@ def test_strided_view_matches_library_views_and_loops(oracle):
                 assert got[t, h, d] == storage[offset + t * strides[0] + h * strides[1] + d * strides[2]]
 
 
+# ---------------------------------------------------------------- norm_rope_reshape
+def test_norm_rope_reshape_closed_forms_and_library_routines(oracle):
+    """RMSNorm against torch's own rms_norm and two closed forms; the rotation against complex
+    multiplication (channel i and i + half are the real and imaginary part of one number turned by
+    the angle whose cosine / sine the tables hold); slot placement against direct indexing."""
+    import torch
+    rng = _rng(21)
+    T, n, r, blocks, block = 9, 64, 16, 3, 8
+    x = rng.standard_normal((T, 1, n)).astype(np.float32)
+    gamma = rng.standard_normal(n).astype(np.float32)
+    rope = rng.standard_normal((T, r)).astype(np.float32)
+    theta = rng.uniform(0, 2 * np.pi, size=(T, r // 2))
+    cos = np.concatenate([np.cos(theta), np.cos(theta)], axis=1).astype(np.float32)
+    sin = np.concatenate([np.sin(theta), np.sin(theta)], axis=1).astype(np.float32)
+    cache0 = rng.standard_normal((blocks, block, 1, n + r)).astype(np.float32)
+    slots = rng.choice(np.arange(-blocks * block, blocks * block), size=T, replace=False).astype(np.int32)
+    slots[:2] = [5, -3]
+    eps = 1e-5
+    got = oracle.norm_rope_reshape(x, gamma, rope, cos, sin, slots, cache0, eps, out_dtype=np.float32)
+    want_norm = torch.nn.functional.rms_norm(torch.from_numpy(x).double(), (n,), torch.from_numpy(gamma).double(),
+                                             eps).numpy().reshape(T, n)
+    z = (rope[:, :r // 2].astype(np.float64) + 1j * rope[:, r // 2:]) * np.exp(1j * theta)
+    want_rope = np.concatenate([z.real, z.imag], axis=1)
+    flat = got.reshape(blocks * block, n + r)
+    flat0 = cache0.reshape(blocks * block, n + r)
+    for i, s in enumerate(slots.tolist()):
+        if s >= 0:
+            np.testing.assert_allclose(flat[s, :n], want_norm[i], rtol=2e-6, atol=2e-6)
+            np.testing.assert_allclose(flat[s, n:], want_rope[i], rtol=2e-6, atol=2e-6)
+            # a rotation keeps the length of every (i, i + half) pair
+            np.testing.assert_allclose(flat[s, n:n + r // 2] ** 2 + flat[s, n + r // 2:] ** 2,
+                                       rope[i, :r // 2] ** 2 + rope[i, r // 2:] ** 2, rtol=1e-5)
+    untouched = np.setdiff1d(np.arange(blocks * block), slots[slots >= 0])
+    assert np.array_equal(flat[untouched], flat0[untouched]) and (slots < 0).any()
+    # closed forms: a constant row normalises to sign(c) * gamma (up to epsilon); a row with one non-zero
+    # channel a to a / sqrt(a^2 / n + eps) there; angle 0 leaves the rotary row alone, a quarter turn maps
+    # (first, second) to (-second, first)
+    xc = np.full((1, 1, n), -3.0, dtype=np.float32)
+    one = np.ones((1, r), np.float32)
+    zero = np.zeros((1, r), np.float32)
+    out = oracle.norm_rope_reshape(xc, gamma, rope[:1], one, zero, [0], cache0, eps, out_dtype=np.float32)
+    np.testing.assert_allclose(out[0, 0, 0, :n], -gamma / np.sqrt(1 + eps / 9), rtol=1e-6)
+    assert np.array_equal(out[0, 0, 0, n:], rope[0])
+    xh = np.zeros((1, 1, n), np.float32)
+    xh[0, 0, 7] = 4.0
+    out = oracle.norm_rope_reshape(xh, np.ones(n, np.float32), rope[:1], zero, one, [1], cache0, eps, out_dtype=np.float32)
+    assert abs(out[0, 1, 0, 7] - 4.0 / np.sqrt(16.0 / n + eps)) < 1e-5 and np.count_nonzero(out[0, 1, 0, :n]) == 1
+    assert np.array_equal(out[0, 1, 0, n:], np.concatenate([-rope[0, r // 2:], rope[0, :r // 2]]))
+    # the 16-bit results are the fp32 ones rounded once
+    h = oracle.norm_rope_reshape(x, gamma, rope, cos, sin, slots, cache0.astype(np.float16), eps)
+    assert h.dtype == np.float16 and np.array_equal(h[0, 5, 0], got[0, 5, 0].astype(np.float16))
+    b = oracle.norm_rope_reshape(x, gamma, rope, cos, sin, slots, cache0, eps, out_dtype="bf16")
+    assert np.array_equal(b[0, 5, 0], oracle.bf16_round(got[0, 5, 0]))
+
+
 # ---------------------------------------------------------------- quantiser
 def test_quant_special_cases(oracle):
     s = np.float32(0.5)
