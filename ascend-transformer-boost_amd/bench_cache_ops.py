@@ -2,8 +2,9 @@
 """Times the cache-side operations at the size of benchmark workload C2 on one MI355X and
 prints one JSON line per operation: BlockCopy (512 blocks of 256 KB copied in each cache),
 PagedCacheLoad (all 158 839 cached rows of the 64 sequences gathered) and NormRopeReshape (the
-producer of the combined MLA cache, at the 65 536 tokens of the reference's kernel test), through
-atb::Operation (Setup + Execute per call; NormRopeReshape: Setup once). All are HBM-bound; `roofline.achieved` is their
+producer of the combined MLA cache, at the 65 536 tokens of the reference's kernel test) and Rope
+(8 192 tokens of a Llama-3-8B-shaped layer), through
+atb::Operation (Setup + Execute per call; NormRopeReshape and Rope: Setup once). All are HBM-bound; `roofline.achieved` is their
 algorithmic bytes (every source byte read once, every destination byte written once) over the
 mean kernel time between HIP events on the launch stream.
 
@@ -119,6 +120,31 @@ def main():
                                    "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                                    "algorithmic_bytes": alg}}))
     fused.close()
+
+    # ---- Rope: 8 192 tokens of a Llama-3-8B-shaped layer (32 query heads, 8 KV heads, head size 128), bf16
+    tokens, hq, hk, d = 8192, 32 * 128, 8 * 128, 128
+    q = torch.rand((tokens, hq), device=dev).to(torch.bfloat16)
+    k = torch.rand((tokens, hk), device=dev).to(torch.bfloat16)
+    cos, sin = (torch.rand((tokens, d), device=dev).to(torch.bfloat16) for _ in range(2))
+    lens_r = torch.tensor([tokens], dtype=torch.int32, device=dev)
+    q_out, k_out = torch.empty_like(q), torch.empty_like(k)
+    rope = b.OperationRunner("RopeOperation", b.RopeParam(rotaryCoeff=2), ctx)
+    ins = [b.tensor_of(t) for t in (q, k, cos, sin, lens_r)]
+    outs = [b.tensor_of(q_out), b.tensor_of(k_out)]
+    st, ws = rope.op.setup(ins, outs, ctx)
+    assert st == 0 and ws == 0
+
+    def execute_rope():
+        assert rope.op.execute(ins, outs, None, 0, ctx) == 0
+    ms = timed(execute_rope, stream, args.steps, args.warmup)
+    alg = tokens * ((hq + hk) * 2 * 2 + 2 * d * 2)
+    print(json.dumps({"operation": "RopeOperation", "workload": "%d tokens, query rows of %d and key rows of %d channels, "
+                      "head size %d, rotaryCoeff 2, bf16 (Setup once, Execute per call)" % (tokens, hq, hk, d),
+                      "ms_per_call": ms,
+                      "roofline": {"bound": "hbm", "achieved": alg / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
+                                   "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                                   "algorithmic_bytes": alg}}))
+    rope.close()
     ctx.close()
 
 

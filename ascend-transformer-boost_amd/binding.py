@@ -88,6 +88,19 @@ class ReshapeAndCacheWithStrideParam(ReshapeAndCacheParam):
     """Byte image of atb::infer::ReshapeAndCacheWithStrideParam (24 bytes, the same fields)."""
 
 
+class RopeParam(ctypes.Structure):
+    """Byte image of atb::infer::RopeParam (16 bytes)."""
+    _fields_ = [("rotaryCoeff", ctypes.c_int32), ("cosFormat", ctypes.c_int32), ("rsv", ctypes.c_uint8 * 8)]
+
+    def __init__(self, **kw):
+        super().__init__()
+        self.rotaryCoeff = 4
+        for k, v in kw.items():
+            if not hasattr(self, k):
+                raise AttributeError("RopeParam has no field " + k)
+            setattr(self, k, v)
+
+
 class NormRopeReshapeParam(ctypes.Structure):
     """Byte image of atb::infer::NormRopeReshapeParam (28 bytes)."""
     _fields_ = [("precisionMode", ctypes.c_uint32), ("rotaryCoeff", ctypes.c_uint32), ("epsilon", ctypes.c_float),
@@ -180,6 +193,7 @@ def kernels():
                                                         i64, vp]
         lib.atbmi_norm_rope_reshape_and_cache.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32,
                                                           ctypes.c_float, vp]
+        lib.atbmi_rope.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i32, i32, i32, i32, vp]
         lib.atbmi_quant_per_channel.argtypes = [vp, i32, vp, vp, vp, i64, i64, vp]
         lib.atbmi_reshape_and_cache_quant.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]
         lib.atbmi_block_copy.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]

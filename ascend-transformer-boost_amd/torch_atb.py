@@ -122,6 +122,11 @@ class ReshapeAndCacheWithStrideParam(_Param):
         K_CACHE_V_BYPASS = 1
 
 
+class RopeParam(_Param):
+    _struct = _b.RopeParam
+    _op_name = "RopeOperation"
+
+
 class NormRopeReshapeParam(_Param):
     _struct = _b.NormRopeReshapeParam
     _op_name = "NormRopeReshapeOperation"

@@ -167,6 +167,13 @@ struct MultiLatentAttentionParam {
     uint8_t rsv[32] = {0}; // must stay zero
 };
 
+// Rotary position embedding of query and key rows (reference include/atb/infer_op_params.h:1605-1617).
+struct RopeParam {
+    int32_t rotaryCoeff = 4; // 2: rotate halves; 4: the two halves of a head separately; headDim: interleaved pairs
+    int32_t cosFormat = 0;   // 0: cos / sin hold a row per token; 1: a row per position of a sequence
+    uint8_t rsv[8] = {0};    // must stay zero
+};
+
 // RMSNorm of the latent row, rotary embedding of the rotary row and the write of both, side by side,
 // into a single cache: the step that fills the combined MLA cache
 // (reference include/atb/infer_op_params.h:2697-2716).
@@ -198,6 +205,7 @@ struct PagedCacheLoadParam {
 
 static_assert(sizeof(ReshapeAndCacheParam) == 24, "ReshapeAndCacheParam ABI size");
 static_assert(sizeof(ReshapeAndCacheWithStrideParam) == 24, "ReshapeAndCacheWithStrideParam ABI size");
+static_assert(sizeof(RopeParam) == 16, "RopeParam ABI size");
 static_assert(sizeof(NormRopeReshapeParam) == 28, "NormRopeReshapeParam ABI size");
 static_assert(sizeof(BlockCopyParam) == 16, "BlockCopyParam ABI size");
 static_assert(sizeof(PagedCacheLoadParam) == 64, "PagedCacheLoadParam ABI size");

@@ -99,6 +99,25 @@ int atbmi_norm_rope_reshape_and_cache(const void *xDevice, const void *gammaDevi
                                       int64_t numSlots, int32_t dtype, float epsilon, void *stream);
 
 /*
+ * Rotary position embedding of query and key rows (q [numTokens, hiddenQ], k [numTokens, hiddenK],
+ * fp16 or bf16). The cos / sin tables have rows of headDim entries (the type of q, or fp32 with
+ * fp16 rows when tableIsFloat); a row of q or k is cut into units of headDim channels, a unit into
+ * rotaryCoeff / 2 chunks of 2 * stride channels (stride = headDim / rotaryCoeff), and in a chunk
+ *   out[i]          = x[i] * cos[i'] - x[i + stride] * sin[i']
+ *   out[i + stride] = x[i + stride] * cos[i' + stride] + x[i] * sin[i' + stride]     (i' = i's offset in its unit)
+ * in fp32, rounded once. cosFormat 0: table row r belongs to token r. cosFormat 1: to position r of
+ * every sequence; seqLens (int32 [batch], device) then gives the tokens their positions; tokens past
+ * the last sequence, or with a row outside the table, are left alone. qOut / kOut may be q / k.
+ * Replaces: the Rope kernel behind RopeOperation (reference src/ops/ops_infer/rope/rope_ops_runner.cpp:43-72;
+ * golden tests/apitest/opstest/python/operations/rope/test_rope_operation2.py:120-218, cosFormat 1
+ * test_rope_operation3.py:29-55).
+ */
+int atbmi_rope(const void *qDevice, const void *kDevice, const void *cosDevice, const void *sinDevice,
+               const int32_t *seqLensDevice, void *qOutDevice, void *kOutDevice, int64_t numTokens, int64_t hiddenQ,
+               int64_t hiddenK, int64_t headDim, int64_t tableRows, int64_t batch, int32_t rotaryCoeff,
+               int32_t cosFormat, int32_t dtype, int32_t tableIsFloat, void *stream);
+
+/*
  * Per-channel int8 quantiser: out[r][c] = clamp(rint(float(x[r][c]) / scale[c]) + offset[c], -128, 127),
  * IEEE fp32 divide, round-half-even, NaN -> 0. offset may be NULL.
  * Replaces: the ELEWISE_QUANT_PER_CHANNEL kernel (golden

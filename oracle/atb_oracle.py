@@ -16,6 +16,11 @@ the invariants of the mathematics (no function is left "parity unpinned"):
   strided_view        tests/unittest/ops/reshape_and_cache_with_stride/test_reshape_and_cache_with_stride.cpp:
                       219-245 (element [i0, i1, i2] of the view is storage[offset + sum(i_k * stride_k)]),
                       :411-433 (the view then goes through the plain reshape_and_cache golden)
+  rope                tests/apitest/opstest/python/operations/rope/test_rope_operation2.py:120-218 (the general
+                      form: rows cut into units of the table row size, a unit into rotaryCoeff / 2 chunks, in a
+                      chunk first half <- -second half, second half <- first half, times sin, plus x times
+                      cos), :86-101 (fp32 arithmetic, one rounding), test_rope_operation3.py:29-55 (cosFormat 1:
+                      table row = position inside the token's sequence)
   norm_rope_reshape   tests/apitest/opstest/python/operations/norm_rope_reshape/test_norm_rope_reshape.py:21-71
                       and tests/apitest/kernelstest/mix/test_rms_norm_and_rope_and_reshape_and_cache_bf16.py:24-74
                       (rms = 1 / sqrt(mean(x^2) + eps); x * rms * gamma; r * cos + rotate_half(r) * sin with
@@ -104,6 +109,33 @@ def strided_view(storage, shape, strides, offset):
         ext[axis] = n
         idx += (np.arange(n, dtype=np.int64) * int(st)).reshape(ext)
     return flat[idx]
+
+
+def rope(q, k, cos, sin, seq_lens, rotary_coeff, cos_format=0, out_dtype=np.float16):
+    """Rotary embedding of q [tokens, hidden_q] and k [tokens, hidden_k] with tables [rows, head_dim]:
+    out = x * cos + rotated(x) * sin, where inside every chunk of 2 * (head_dim / rotary_coeff) channels
+    rotated(x) = concat(-second half, first half). Table row of token t: t itself (cos_format 0) or its
+    position inside its sequence (cos_format 1; seq_lens gives the sequences). fp32 arithmetic, rounded
+    once to out_dtype (np.float16, or "bf16" for bfloat16 values kept in float32). Returns (q_out, k_out)."""
+    cos = np.asarray(cos, dtype=np.float32)
+    sin = np.asarray(sin, dtype=np.float32)
+    head_dim = cos.shape[1]
+    stride = head_dim // rotary_coeff
+    tokens = np.asarray(q).shape[0]
+    if cos_format == 0:
+        rows = np.arange(tokens)
+    else:
+        rows = np.concatenate([np.arange(n) for n in np.asarray(seq_lens).tolist()])[:tokens]
+
+    def one(x):
+        x = np.asarray(x, dtype=np.float32)
+        units = x.reshape(tokens, -1, head_dim // (2 * stride), 2, stride)  # token, unit, chunk, half, channel
+        rotated = np.stack((-units[:, :, :, 1], units[:, :, :, 0]), axis=3).reshape(tokens, -1, head_dim)
+        c = cos[rows][:, None, :]
+        s_ = sin[rows][:, None, :]
+        out = (x.reshape(tokens, -1, head_dim) * c + rotated * s_).reshape(x.shape)
+        return bf16_round(out) if out_dtype == "bf16" else out.astype(out_dtype)
+    return one(q), one(k)
 
 
 def norm_rope_reshape(x, gamma, key_rope, cos, sin, slot_mapping, key_cache, epsilon, out_dtype=np.float16):

@@ -10,6 +10,7 @@ status, tagged C: for CreateOperation, I: for InferShape, S: for Setup):
     tests/apitest/opstest/csv/block_copy.csv
     tests/apitest/opstest/csv/paged_cache_load.csv
     tests/apitest/opstest/csv/norm_rope_reshape.csv
+    tests/apitest/opstest/csv/rope.csv
 Those rows are data, not code. This script copies the rows written for the
 Ascend910B feature set (the one this library mirrors) into
     tests/golden/paged_attention_cases.json
@@ -18,6 +19,7 @@ Ascend910B feature set (the one this library mirrors) into
     tests/golden/block_copy_cases.json
     tests/golden/paged_cache_load_cases.json
     tests/golden/norm_rope_reshape_cases.json
+    tests/golden/rope_cases.json
 so the parity tests can run where the reference tree is absent.
 
 Run from the repository root in a container that has /root/reference:
@@ -52,8 +54,10 @@ def convert(name, also_untagged=False):
         if not any(c.strip() for c in row):
             continue
         d = {h: v.strip() for h, v in zip(header, row)}
-        # (a creation-only row may leave every column after the param empty, the product tag included)
-        if d.get("SocVersion") != "Ascend910B" and not (also_untagged and d.get("SocVersion", "") == ""):
+        # (a creation-only row may leave every column after the param empty, the product tag included,
+        # and a row may name several products, or none when it holds for all of them)
+        tags = [t.strip() for t in d.get("SocVersion", "").split(",") if t.strip()]
+        if "Ascend910B" not in tags and not (also_untagged and not tags):
             continue
         # OutNum is what the harness hands to the operation (BlockCopy lists two output columns but takes none)
         n_out = int(d["OutNum"]) if d.get("OutNum", "").strip().isdigit() else None
@@ -87,3 +91,4 @@ if __name__ == "__main__":
     convert("block_copy")
     convert("paged_cache_load")
     convert("norm_rope_reshape", also_untagged=True)
+    convert("rope", also_untagged=True)

@@ -192,6 +192,79 @@ def test_reshape_and_cache_with_stride_equals_plain_on_contiguous_input(binding,
     ctx.close()
 
 
+# ------------------------------------------------------------------ Rope
+ROPE_CASES = [
+    # name, q shape, k shape, table rows, head_dim, rotaryCoeff, cosFormat, seq lens, x dtype, table dtype
+    ("glm_coeff4", (4, 4096), (4, 4096), 4, 128, 4, 0, [4], torch.float16, torch.float16),            # rope.csv row 1
+    ("interleaved_4d", (2, 256, 32, 64), (2, 256, 32, 64), 512, 64, 64, 0, [256, 256], torch.float16, torch.float16),  # row 2
+    ("gqa_half", (128, 1024), (128, 128), 128, 128, 2, 0, [128], torch.float16, torch.float16),        # row 3
+    ("fp32_tables", (128, 1024), (128, 128), 128, 128, 2, 0, [128], torch.float16, torch.float32),     # test_rope_operation2.py:103-117
+    ("deepseek", (3072, 8192), (3072, 64), 3072, 64, 2, 0, [3072], torch.float16, torch.float16),      # row 25
+    ("coeff16_bf16", (4, 448), (4, 448), 4, 16, 16, 0, [4], torch.bfloat16, torch.bfloat16),           # row 26
+    ("coeff4_positions", (9, 19264), (9, 19264), 4, 448, 4, 1, [4, 2, 3], torch.bfloat16, torch.bfloat16),  # row 40 (cosFormat 1)
+    ("positions_half", (2048, 1024), (2048, 1024), 700, 128, 2, 1, [700, 1, 647, 700], torch.float16, torch.float16),  # test_rope_operation3.py:57-74
+    ("llama3_8b_step", (64, 4096), (64, 1024), 64, 128, 2, 0, [1] * 64, torch.bfloat16, torch.bfloat16),  # the decode step before workload C2
+]
+
+
+@pytest.mark.parametrize("case", ROPE_CASES, ids=lambda c: c[0])
+def test_rope_operation(binding, oracle, dev, stream, case):
+    """RopeOperation against the fp32 oracle rounded once. Tolerance: one step of the 16-bit output grid
+    (the kernel rounds products and sum separately in fp32 like the oracle; what is left are the ties of the
+    final rounding), and under 0.1 % of the elements may differ at all."""
+    name, q_shape, k_shape, rows, d, coeff, fmt, lens, dtype, tab_dtype = case
+    rng = _rng(51)
+    u = lambda shape, dt: torch.from_numpy(rng.uniform(-2, 2, size=shape).astype(np.float32)).to(dt)
+    q, k = u(q_shape, dtype), u(k_shape, dtype)
+    cos, sin = u((rows, d), tab_dtype), u((rows, d), tab_dtype)
+    lens_t = torch.tensor(lens, dtype=torch.int32)
+    T = q_shape[0] if len(q_shape) == 2 else q_shape[0] * q_shape[1]
+    want_q, want_k = oracle.rope(q.float().numpy().reshape(T, -1), k.float().numpy().reshape(T, -1), cos.float().numpy(),
+                                 sin.float().numpy(), lens, coeff, fmt, out_dtype="bf16" if dtype == torch.bfloat16 else np.float16)
+    ctx = binding.Context(stream)
+    runner = binding.OperationRunner("RopeOperation", binding.RopeParam(rotaryCoeff=coeff, cosFormat=fmt), ctx)
+    with torch.cuda.stream(stream):
+        out_q, out_k = runner.run([t.to(dev) for t in (q, k, cos, sin, lens_t)])
+    stream.synchronize()
+    assert tuple(out_q.shape) == q_shape and tuple(out_k.shape) == k_shape
+    for got, want in ((out_q, want_q), (out_k, want_k)):
+        g = got.float().cpu().numpy().reshape(T, -1)
+        w = want.astype(np.float32)
+        step = np.abs(w) * (2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10) + 2.0 ** -24
+        assert np.all(np.abs(g - w) <= step), float(np.abs(g - w).max())
+        assert np.mean(g != w) < 1e-3
+    runner.close()
+    ctx.close()
+
+
+def test_rope_in_place_and_tokens_outside_the_sequences(binding, oracle, dev, stream):
+    """The C ABI with the outputs aliasing the inputs, and cosFormat 1 with more tokens than the sequences
+    hold and a sequence longer than the tables: those tokens keep their values."""
+    k_ = binding.kernels()
+    rng = _rng(52)
+    T, hq, hk, d, rows = 12, 256, 64, 64, 4
+    u = lambda *shape: torch.from_numpy(rng.uniform(-2, 2, size=shape).astype(np.float32)).to(torch.float16)
+    q, k, cos, sin = u(T, hq), u(T, hk), u(rows, d), u(rows, d)
+    lens = [3, 6, 1]   # 10 of the 12 tokens; positions 4 and 5 of the second sequence have no table row
+    pos = np.array([0, 1, 2, 0, 1, 2, 3, -1, -1, 0, -1, -1])
+    live = pos >= 0
+    want_q, want_k = q.numpy().copy(), k.numpy().copy()
+    lq, lk = oracle.rope(q.float().numpy()[live], k.float().numpy()[live], cos.float().numpy()[pos[live]],
+                         sin.float().numpy()[pos[live]], [int(live.sum())], 2, 0)
+    want_q[live], want_k[live] = lq, lk
+    with torch.cuda.stream(stream):
+        qd, kd, cd, sd = (t.to(dev) for t in (q, k, cos, sin))
+        ld = torch.tensor(lens, dtype=torch.int32, device=dev)
+        rc = k_.atbmi_rope(qd.data_ptr(), kd.data_ptr(), cd.data_ptr(), sd.data_ptr(), ld.data_ptr(), qd.data_ptr(),
+                           kd.data_ptr(), T, hq, hk, d, rows, len(lens), 2, 1, 0, 0, stream.cuda_stream)
+    stream.synchronize()
+    assert rc == 0, binding.last_kernel_error()
+    for got, want in ((qd, want_q), (kd, want_k)):
+        g = got.cpu().numpy().astype(np.float32)
+        assert np.all(np.abs(g - want.astype(np.float32)) <= np.abs(want.astype(np.float32)) * 2.0 ** -10 + 2.0 ** -24)
+        assert np.array_equal(got.cpu().numpy()[~live].view(np.int16), want[~live].view(np.int16))
+
+
 # ------------------------------------------------------------------ NormRopeReshape
 def _reference_standard(got, want, factor_max, factor_mean):
     """The reference's own pass criterion for this operator (tests/apitest/opstest/python/operations/

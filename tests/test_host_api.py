@@ -31,6 +31,7 @@ MLA_CASES = _load("multi_latent_attention")
 BLOCK_COPY_CASES = _load("block_copy")
 CACHE_LOAD_CASES = _load("paged_cache_load")
 NORM_ROPE_CASES = _load("norm_rope_reshape")
+ROPE_CASES = _load("rope")
 
 
 def _pa_unimplemented(p):
@@ -69,22 +70,19 @@ def _mla_unimplemented(p):
 
 
 def _make_param(binding, op, p):
-    if op == "PagedAttentionOperation":
-        return binding.PagedAttentionParam(**p)
-    if op == "MultiLatentAttentionOperation":
-        return binding.MultiLatentAttentionParam(**p)
-    if op == "BlockCopyOperation":
-        return binding.BlockCopyParam()
-    if op == "PagedCacheLoadOperation":
-        return binding.PagedCacheLoadParam(**p)
-    if op == "ReshapeAndCacheWithStrideOperation":
-        return binding.ReshapeAndCacheWithStrideParam(**p)
-    if op == "NormRopeReshapeOperation":
-        param = binding.NormRopeReshapeParam(**{k: v for k, v in p.items() if k != "rsv"})
-        for i, v in enumerate(p.get("rsv", [])):
-            param.rsv[i] = v
-        return param
-    return binding.ReshapeAndCacheParam(**p)
+    cls = {"PagedAttentionOperation": binding.PagedAttentionParam,
+           "MultiLatentAttentionOperation": binding.MultiLatentAttentionParam,
+           "BlockCopyOperation": binding.BlockCopyParam,
+           "PagedCacheLoadOperation": binding.PagedCacheLoadParam,
+           "ReshapeAndCacheWithStrideOperation": binding.ReshapeAndCacheWithStrideParam,
+           "NormRopeReshapeOperation": binding.NormRopeReshapeParam,
+           "RopeOperation": binding.RopeParam,
+           "ReshapeAndCacheOperation": binding.ReshapeAndCacheParam}[op]
+    fields = {k: v for k, v in p.items() if k != "rsv"}
+    param = cls(**fields) if fields else cls()
+    for i, v in enumerate(p.get("rsv", [])):  # a row may set reserved bytes to see them refused
+        param.rsv[i] = v
+    return param
 
 
 def _tensors(binding, dtypes, formats, shapes, host_arrays=None):
@@ -186,6 +184,11 @@ def test_paged_cache_load_table(binding, ctx, case):
     _check(binding, case, ctx, nz and not case["expected"].startswith("C:"))
 
 
+@pytest.mark.parametrize("case", ROPE_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
+def test_rope_table(binding, ctx, case):
+    _check(binding, case, ctx, False)
+
+
 @pytest.mark.parametrize("case", NORM_ROPE_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
 def test_norm_rope_reshape_table(binding, ctx, case):
     _check(binding, case, ctx, False)
@@ -202,7 +205,7 @@ def test_table_coverage():
               _pa_mask_shape_refused(c)]
     rac_dev = [c for c in RAC_CASES if _rac_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
     assert len(PA_CASES) == 81 and len(PA_CASES) - len(pa_dev) >= 72
-    assert len(RAC_CASES) == 37 and len(RAC_CASES) - len(rac_dev) >= 25
+    assert len(RAC_CASES) == 38 and len(RAC_CASES) - len(rac_dev) >= 26
     # most MultiLatentAttention rows exercise the prefill calcType and the fractal-NZ caches, which are not built
     mla_dev = [c for c in MLA_CASES if _mla_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
     assert len(MLA_CASES) == 147 and len(MLA_CASES) - len(mla_dev) == 45
@@ -804,6 +807,7 @@ def test_cpp_api_symbols_are_exported(pkg):
         "atb::CreateOperation<atb::infer::ReshapeAndCacheParam>",
         "atb::CreateOperation<atb::infer::ReshapeAndCacheWithStrideParam>",
         "atb::CreateOperation<atb::infer::NormRopeReshapeParam>",
+        "atb::CreateOperation<atb::infer::RopeParam>",
         "atb::DestroyOperation(atb::Operation*)",
         "atb::CreateContext(atb::Context**)",
         "atb::DestroyContext(atb::Context*)",

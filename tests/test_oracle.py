@@ -91,6 +91,67 @@ def test_strided_view_matches_library_views_and_loops(oracle):
                 assert got[t, h, d] == storage[offset + t * strides[0] + h * strides[1] + d * strides[2]]
 
 
+# ---------------------------------------------------------------- rope
+def _rotate_half(x):
+    x0, x1 = x.chunk(2, -1)
+    return __import__("torch").cat((-x1, x0), dim=-1)
+
+
+def test_rope_against_the_three_forms_the_reference_tests_use(oracle):
+    """rotaryCoeff 2 against x * cos + rotate_half(x) * sin over whole heads, 4 against the same applied to
+    the two halves of a head separately, rotaryCoeff = head size against the interleaved-pair form; then
+    the rotation as a complex multiplication, and the positions of cosFormat 1."""
+    import torch
+    rng = _rng(23)
+    T, heads_q, heads_k, d = 7, 6, 2, 16
+    q = torch.from_numpy(rng.standard_normal((T, heads_q * d)).astype(np.float32))
+    k = torch.from_numpy(rng.standard_normal((T, heads_k * d)).astype(np.float32))
+    cos = torch.from_numpy(rng.standard_normal((T, d)).astype(np.float32))
+    sin = torch.from_numpy(rng.standard_normal((T, d)).astype(np.float32))
+    lens = np.array([T], dtype=np.int32)
+    f32 = dict(out_dtype=np.float32)
+    # coefficient 2: whole heads
+    for x, got in zip((q, k), oracle.rope(q.numpy(), k.numpy(), cos.numpy(), sin.numpy(), lens, 2, **f32)):
+        xh = x.view(T, -1, d)
+        want = xh * cos[:, None] + _rotate_half(xh) * sin[:, None]
+        np.testing.assert_allclose(got, want.reshape(T, -1).numpy(), rtol=1e-6, atol=1e-6)
+    # coefficient 4: the halves of a head, each with its half of the tables
+    for x, got in zip((q, k), oracle.rope(q.numpy(), k.numpy(), cos.numpy(), sin.numpy(), lens, 4, **f32)):
+        x0, x1 = x.view(T, -1, d).chunk(2, -1)
+        c0, c1 = cos[:, None].chunk(2, -1)
+        s0, s1 = sin[:, None].chunk(2, -1)
+        want = torch.cat([x0 * c0 + _rotate_half(x0) * s0, x1 * c1 + _rotate_half(x1) * s1], dim=-1)
+        np.testing.assert_allclose(got, want.reshape(T, -1).numpy(), rtol=1e-6, atol=1e-6)
+    # coefficient = head size: neighbouring channels pair up; tables repeat every entry once
+    half = torch.from_numpy(rng.standard_normal((T, d // 2)).astype(np.float32))
+    half_s = torch.from_numpy(rng.standard_normal((T, d // 2)).astype(np.float32))
+    cos_r, sin_r = half.repeat_interleave(2, dim=1), half_s.repeat_interleave(2, dim=1)
+    for x, got in zip((q, k), oracle.rope(q.numpy(), k.numpy(), cos_r.numpy(), sin_r.numpy(), lens, d, **f32)):
+        xs = x.view(T, -1, d // 2, 2)
+        c, s_ = half[:, None], half_s[:, None]
+        want = torch.stack([xs[..., 0] * c - xs[..., 1] * s_, xs[..., 1] * c + xs[..., 0] * s_], -1)
+        np.testing.assert_allclose(got, want.reshape(T, -1).numpy(), rtol=1e-6, atol=1e-6)
+    # a rotation: with cos / sin of one angle per pair, (x[i] + j x[i + d/2]) turns by that angle
+    theta = rng.uniform(0, 2 * np.pi, size=(T, d // 2))
+    ct = np.concatenate([np.cos(theta), np.cos(theta)], axis=1).astype(np.float32)
+    st = np.concatenate([np.sin(theta), np.sin(theta)], axis=1).astype(np.float32)
+    got, _ = oracle.rope(q.numpy(), k.numpy(), ct, st, lens, 2, **f32)
+    qh = q.numpy().reshape(T, heads_q, d).astype(np.float64)
+    z = (qh[..., :d // 2] + 1j * qh[..., d // 2:]) * np.exp(1j * theta)[:, None]
+    np.testing.assert_allclose(got.reshape(T, heads_q, d), np.concatenate([z.real, z.imag], axis=-1), rtol=1e-5, atol=1e-5)
+    # cosFormat 1: row = position inside the sequence; the same as cosFormat 0 with the rows gathered by hand
+    seq = np.array([3, 1, 3], dtype=np.int32)
+    pos = np.array([0, 1, 2, 0, 0, 1, 2])
+    table_c, table_s = cos.numpy()[:4], sin.numpy()[:4]
+    a = oracle.rope(q.numpy(), k.numpy(), table_c, table_s, seq, 2, cos_format=1, **f32)
+    b = oracle.rope(q.numpy(), k.numpy(), table_c[pos], table_s[pos], seq, 2, cos_format=0, **f32)
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+    # 16-bit results are the fp32 ones rounded once
+    h = oracle.rope(q.numpy(), k.numpy(), cos.numpy(), sin.numpy(), lens, 2)
+    assert h[0].dtype == np.float16
+    assert np.array_equal(h[0], oracle.rope(q.numpy(), k.numpy(), cos.numpy(), sin.numpy(), lens, 2, **f32)[0].astype(np.float16))
+
+
 # ---------------------------------------------------------------- norm_rope_reshape
 def test_norm_rope_reshape_closed_forms_and_library_routines(oracle):
     """RMSNorm against torch's own rms_norm and two closed forms; the rotation against complex
