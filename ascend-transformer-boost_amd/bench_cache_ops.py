@@ -3,8 +3,9 @@
 prints one JSON line per operation: BlockCopy (512 blocks of 256 KB copied in each cache),
 PagedCacheLoad (all 158 839 cached rows of the 64 sequences gathered) and NormRopeReshape (the
 producer of the combined MLA cache, at the 65 536 tokens of the reference's kernel test) and Rope
-(8 192 tokens of a Llama-3-8B-shaped layer), through
-atb::Operation (Setup + Execute per call; NormRopeReshape and Rope: Setup once). All are HBM-bound; `roofline.achieved` is their
+(8 192 tokens of a Llama-3-8B-shaped layer) and the per-channel quantiser / dequantiser of
+ElewiseOperation (3 072 x 16 384), through
+atb::Operation (Setup + Execute per call; NormRopeReshape, Rope and Elewise: Setup once). All are HBM-bound; `roofline.achieved` is their
 algorithmic bytes (every source byte read once, every destination byte written once) over the
 mean kernel time between HIP events on the launch stream.
 
@@ -145,6 +146,33 @@ def main():
                                    "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                                    "algorithmic_bytes": alg}}))
     rope.close()
+
+    # ---- Elewise per-channel quantiser / dequantiser: 3 072 rows of 16 384 channels (a CSV row of the reference)
+    rows, ch = 3072, 16384
+    x = (torch.rand((rows, ch), device=dev) * 200 - 100).to(torch.float16)
+    scale = (torch.rand((ch,), device=dev) * 0.9 + 0.1).to(torch.float16)
+    offset = torch.randint(-10, 10, (ch,), dtype=torch.int8, device=dev)
+    xq = torch.empty((rows, ch), dtype=torch.int8, device=dev)
+    xd = torch.empty((rows, ch), dtype=torch.float16, device=dev)
+    for name, etype, src, dst in (("quantiser", b.ElewiseParam.ELEWISE_QUANT_PER_CHANNEL, x, xq),
+                                  ("dequantiser", b.ElewiseParam.ELEWISE_DEQUANT_PER_CHANNEL, xq, xd)):
+        op = b.OperationRunner("ElewiseOperation", b.ElewiseParam(elewiseType=etype), ctx)
+        ins = [b.tensor_of(t) for t in (src, scale, offset)]
+        outs = [b.tensor_of(dst)]
+        st, ws = op.op.setup(ins, outs, ctx)
+        assert st == 0 and ws == 0
+
+        def execute_elewise():
+            assert op.op.execute(ins, outs, None, 0, ctx) == 0
+        ms = timed(execute_elewise, stream, args.steps, args.warmup)
+        alg = rows * ch * 3 + ch * 3
+        print(json.dumps({"operation": "ElewiseOperation (per-channel %s)" % name,
+                          "workload": "%d x %d fp16 <-> int8, scale and offset per channel (Setup once, Execute per call)"
+                          % (rows, ch), "ms_per_call": ms,
+                          "roofline": {"bound": "hbm", "achieved": alg / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
+                                       "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                                       "algorithmic_bytes": alg}}))
+        op.close()
     ctx.close()
 
 

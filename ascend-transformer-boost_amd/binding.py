@@ -23,7 +23,7 @@ ACL_DTYPE_BY_NAME = {
     "float": 0, "float16": 1, "int8": 2, "int32": 3, "uint8": 4, "int16": 6, "uint16": 7, "uint32": 8,
     "int64": 9, "uint64": 10, "double": 11, "bool": 12, "bf16": 27,
 }
-ACL_FORMAT_BY_NAME = {"nchw": 0, "nhwc": 1, "nd": 2, "fractal_nz": 29}
+ACL_FORMAT_BY_NAME = {"nchw": 0, "nhwc": 1, "nd": 2, "fractal_nz": 29, "ncdhw": 30}
 
 # atb::ErrorType (include/atb/types.h)
 ERROR_NAMES = [
@@ -86,6 +86,23 @@ class ReshapeAndCacheParam(ctypes.Structure):
 
 class ReshapeAndCacheWithStrideParam(ReshapeAndCacheParam):
     """Byte image of atb::infer::ReshapeAndCacheWithStrideParam (24 bytes, the same fields)."""
+
+
+class ElewiseParam(ctypes.Structure):
+    """Byte image of atb::infer::ElewiseParam (64 bytes: type, QuantParam 32, MulsParam 16, out type, rsv)."""
+    _fields_ = [("elewiseType", ctypes.c_int32), ("inputScale", ctypes.c_float), ("asymmetric", ctypes.c_bool),
+                ("inputOffset", ctypes.c_int32), ("quantRsv", ctypes.c_uint8 * 20), ("varAttr", ctypes.c_float),
+                ("mulsRsv", ctypes.c_uint8 * 12), ("outTensorType", ctypes.c_int32), ("rsv", ctypes.c_uint8 * 8)]
+    ELEWISE_QUANT_PER_CHANNEL, ELEWISE_DEQUANT_PER_CHANNEL = 17, 18
+
+    def __init__(self, **kw):
+        super().__init__()
+        self.inputScale = 1.0
+        self.outTensorType = -1
+        for k, v in kw.items():
+            if not hasattr(self, k):
+                raise AttributeError("ElewiseParam has no field " + k)
+            setattr(self, k, v)
 
 
 class RopeParam(ctypes.Structure):
@@ -194,6 +211,8 @@ def kernels():
         lib.atbmi_norm_rope_reshape_and_cache.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32,
                                                           ctypes.c_float, vp]
         lib.atbmi_rope.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i32, i32, i32, i32, vp]
+        lib.atbmi_elewise_quant_per_channel.argtypes = [vp, vp, vp, vp, i64, i64, i32, vp]
+        lib.atbmi_elewise_dequant_per_channel.argtypes = [vp, vp, vp, vp, i64, i64, vp]
         lib.atbmi_quant_per_channel.argtypes = [vp, i32, vp, vp, vp, i64, i64, vp]
         lib.atbmi_reshape_and_cache_quant.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]
         lib.atbmi_block_copy.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]

@@ -273,6 +273,116 @@ __global__ __launch_bounds__(NORM_ROPE_WAVES *WAVE) void NormRopeCacheKernel(
     }
 }
 
+// ElewiseOperation's per-channel quantiser and dequantiser: the scale has the type of x (16-bit) and
+// the offset is int8; "channel" is the element's index modulo the number of scale entries (the scale
+// covers the trailing dimensions of x, or is a single value).
+//   quant:        clamp(rint(fp16(x / scale)) + offset, -128, 127): the quotient is rounded to fp16
+//                 before it is rounded to an integer, as the reference golden's fp16 division does
+//                 (for bf16 inputs too: the golden converts them to fp16 first)
+//   dequant:      fp16((x - offset) * scale), saturated at +-65504
+// VEC = 8: eight consecutive elements per thread with 16-byte accesses on the 16-bit side.
+__device__ __forceinline__ int8_t QuantOne16(float x, float s, int32_t offset, bool bf16)
+{
+    (void)bf16; // (bf16 inputs take the same route: the reference golden converts them to fp16 and divides there)
+    const float q = HalfBitsToFloat(FloatToHalfBits(__fdiv_rn(x, s)));
+    float r = rintf(q);
+    if (r != r) {
+        return 0;
+    }
+    r += static_cast<float>(offset);
+    r = fminf(fmaxf(r, -128.0f), 127.0f);
+    return static_cast<int8_t>(static_cast<int32_t>(r));
+}
+
+__device__ __forceinline__ uint16_t DequantOne(int8_t x, float s, int32_t offset)
+{
+    // The product is exact in fp32 (9 bits times 11). Its zero must keep the product's sign (0 * -s = -0
+    // in the golden): the compiler would otherwise merge the multiply and the conversion into one
+    // fused multiply-add with +0, which turns -0 into +0, so the product is made opaque first.
+    float p = static_cast<float>(static_cast<int32_t>(x) - offset) * s;
+    asm volatile("" : "+v"(p));
+    uint16_t h = FloatToHalfBits(p);
+    if ((h & 0x7fffu) == 0x7c00u) { // overflowed to infinity: the golden clips to the largest finite value
+        h = static_cast<uint16_t>((h & 0x8000u) | 0x7bffu);
+    }
+    return h;
+}
+
+template <int VEC, bool DEQUANT>
+__global__ __launch_bounds__(256) void ElewisePerChannelKernel(const void *__restrict__ x,
+                                                               const uint16_t *__restrict__ scale,
+                                                               const int8_t *__restrict__ offset,
+                                                               void *__restrict__ out, int64_t total,
+                                                               int64_t channels, int32_t isBf16)
+{
+    const bool bf16 = isBf16 != 0;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x * VEC;
+    for (int64_t i = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * VEC; i < total; i += stride) {
+        const int64_t c = i % channels;
+        if constexpr (VEC == 8) {
+            uint32_t sw[4] = {0u, 0u, 0u, 0u};
+            if (channels > 1) {
+                const uint4 sv = *reinterpret_cast<const uint4 *>(scale + c);
+                sw[0] = sv.x; sw[1] = sv.y; sw[2] = sv.z; sw[3] = sv.w;
+            }
+            int8_t off[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (offset) {
+                if (channels > 1) {
+                    const uint2 ov = *reinterpret_cast<const uint2 *>(offset + c);
+                    const uint32_t ow[2] = {ov.x, ov.y};
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        off[e] = static_cast<int8_t>(ow[e >> 2] >> (8 * (e & 3)));
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        off[e] = offset[0];
+                    }
+                }
+            }
+            float sf[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint16_t h = channels > 1 ? static_cast<uint16_t>(sw[e >> 1] >> (16 * (e & 1))) : scale[0];
+                sf[e] = bf16 ? Bf16ToFloat(h) : HalfBitsToFloat(h);
+            }
+            if constexpr (DEQUANT) {
+                const uint2 xv = *reinterpret_cast<const uint2 *>(static_cast<const int8_t *>(x) + i);
+                const uint32_t xw[2] = {xv.x, xv.y};
+                uint32_t o[4];
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) {
+                    const uint32_t lo = DequantOne(static_cast<int8_t>(xw[e >> 2] >> (8 * (e & 3))), sf[e], off[e]);
+                    const uint32_t hi = DequantOne(static_cast<int8_t>(xw[(e + 1) >> 2] >> (8 * ((e + 1) & 3))), sf[e + 1], off[e + 1]);
+                    o[e >> 1] = lo | (hi << 16);
+                }
+                *reinterpret_cast<uint4 *>(static_cast<uint16_t *>(out) + i) = uint4{o[0], o[1], o[2], o[3]};
+            } else {
+                const uint4 xv = *reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(x) + i);
+                const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+                uint32_t o[2] = {0u, 0u};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const uint16_t h = static_cast<uint16_t>(xw[e >> 1] >> (16 * (e & 1)));
+                    const float xf = bf16 ? Bf16ToFloat(h) : HalfBitsToFloat(h);
+                    const uint32_t q = static_cast<uint8_t>(QuantOne16(xf, sf[e], off[e], bf16));
+                    o[e >> 2] |= q << (8 * (e & 3));
+                }
+                *reinterpret_cast<uint2 *>(static_cast<int8_t *>(out) + i) = uint2{o[0], o[1]};
+            }
+        } else {
+            const float sf = Load16(scale, c, bf16);
+            const int32_t off = offset ? offset[c] : 0;
+            if constexpr (DEQUANT) {
+                static_cast<uint16_t *>(out)[i] = DequantOne(static_cast<const int8_t *>(x)[i], sf, off);
+            } else {
+                static_cast<int8_t *>(out)[i] = QuantOne16(Load16(x, i, bf16), sf, off, bf16);
+            }
+        }
+    }
+}
+
 bool Aligned(const void *p, uintptr_t a)
 {
     return (reinterpret_cast<uintptr_t>(p) % a) == 0;
@@ -465,6 +575,54 @@ extern "C" int atbmi_norm_rope_reshape_and_cache(const void *x, const void *gamm
         numSlots, epsilon);
     ATBMI_HIP_CHECK(hipGetLastError());
     return OK;
+}
+
+namespace {
+template <bool DEQUANT>
+int LaunchElewisePerChannel(const char *what, const void *x, const void *scale, const int8_t *offset, void *out,
+                            int64_t total, int64_t channels, int32_t dtype, void *stream)
+{
+    if (!x || !scale || !out) {
+        return Fail(ERR_INVALID_PARAM, "%s: x, scale and out must be non-null", what);
+    }
+    if (dtype != ATBMI_F16 && !(dtype == ATBMI_BF16 && !DEQUANT)) {
+        return Fail(ERR_INVALID_PARAM, "%s: unsupported element type %d", what, dtype);
+    }
+    if (total < 0 || channels <= 0 || (total % channels) != 0) {
+        return Fail(ERR_INVALID_PARAM, "%s: %lld elements do not divide into rows of %lld scale entries", what,
+                    (long long)total, (long long)channels);
+    }
+    if (total == 0) {
+        return OK;
+    }
+    const bool wide = total % 8 == 0 && (channels == 1 || channels % 8 == 0) && Aligned(x, 16) && Aligned(out, 16) &&
+                      Aligned(scale, 16) && (!offset || Aligned(offset, 8));
+    const int64_t items = wide ? total / 8 : total;
+    const unsigned grid = static_cast<unsigned>(std::min<int64_t>((items + 255) / 256, 1 << 20));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (wide) {
+        ElewisePerChannelKernel<8, DEQUANT><<<grid, 256, 0, s>>>(x, static_cast<const uint16_t *>(scale), offset, out, total,
+                                                                 channels, dtype == ATBMI_BF16);
+    } else {
+        ElewisePerChannelKernel<1, DEQUANT><<<grid, 256, 0, s>>>(x, static_cast<const uint16_t *>(scale), offset, out, total,
+                                                                 channels, dtype == ATBMI_BF16);
+    }
+    ATBMI_HIP_CHECK(hipGetLastError());
+    return OK;
+}
+} // namespace
+
+extern "C" int atbmi_elewise_quant_per_channel(const void *x, const void *scale, const int8_t *offset, int8_t *out,
+                                               int64_t total, int64_t channels, int32_t dtype, void *stream)
+{
+    return LaunchElewisePerChannel<false>("elewise_quant_per_channel", x, scale, offset, out, total, channels, dtype, stream);
+}
+
+extern "C" int atbmi_elewise_dequant_per_channel(const int8_t *x, const void *scale, const int8_t *offset, void *out,
+                                                 int64_t total, int64_t channels, void *stream)
+{
+    return LaunchElewisePerChannel<true>("elewise_dequant_per_channel", x, scale, offset, out, total, channels, ATBMI_F16,
+                                         stream);
 }
 
 extern "C" int atbmi_quant_per_channel(const void *x, int32_t xDtype, const float *scale, const int32_t *offset,

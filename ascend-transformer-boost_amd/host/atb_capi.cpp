@@ -111,6 +111,11 @@ int32_t atb_c_create_operation(const char *opName, const void *param, uint64_t p
         memcpy(static_cast<void *>(&p), param, sizeof(p));
         return atb::CreateOperation(p, out);
     }
+    if (!strcmp(opName, "ElewiseOperation") && paramSize == sizeof(atb::infer::ElewiseParam)) {
+        atb::infer::ElewiseParam p;
+        memcpy(static_cast<void *>(&p), param, sizeof(p));
+        return atb::CreateOperation(p, out);
+    }
     if (!strcmp(opName, "BlockCopyOperation") && paramSize == sizeof(atb::infer::BlockCopyParam)) {
         atb::infer::BlockCopyParam p;
         memcpy(static_cast<void *>(&p), param, sizeof(p));

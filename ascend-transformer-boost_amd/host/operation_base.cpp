@@ -9,13 +9,16 @@ namespace {
 constexpr uint64_t MAX_TENSOR_BYTES = 256ULL * 1024ULL * 1024ULL * 1024ULL;
 
 // Reference src/atb/utils/tensor_check.cpp:25-62.
-Status CheckOneShape(const TensorDesc &desc)
+Status CheckOneShape(const TensorDesc &desc, bool mayBeEmpty = false)
 {
     if (desc.shape.dimNum == 0 || desc.shape.dimNum > MAX_DIM) {
         ATB_LOG(ERROR) << "tensor dimNum " << desc.shape.dimNum << " is invalid, should be in (0, 8]";
         return ERROR_INVALID_TENSOR_DIM;
     }
     const uint64_t bytes = Utils::GetTensorSize(desc);
+    if (bytes == 0 && mayBeEmpty) {
+        return NO_ERROR;
+    }
     if (bytes == 0 || bytes > MAX_TENSOR_BYTES) {
         ATB_LOG(ERROR) << "tensor size " << bytes << " is invalid, should be in (0, 256 GiB]";
         return ERROR_INVALID_TENSOR_SIZE;
@@ -33,10 +36,10 @@ void DescsOf(const SVector<Tensor> &tensors, SVector<TensorDesc> &descs)
 }
 } // namespace
 
-Status OperationBase::CheckShapes(const SVector<Tensor> &tensors, const char *what) const
+Status OperationBase::CheckShapes(const SVector<Tensor> &tensors, const char *what, bool inputs) const
 {
     for (size_t i = 0; i < tensors.size(); ++i) {
-        Status st = CheckOneShape(tensors.at(i).desc);
+        Status st = CheckOneShape(tensors.at(i).desc, inputs && InputMayBeEmpty(i));
         if (st != NO_ERROR) {
             ATB_LOG(ERROR) << name_ << " " << what << "[" << i << "] shape check failed: " << st;
             return st;
@@ -56,6 +59,9 @@ bool OperationBase::IrMatch(const SVector<TensorDesc> &inDescs, const SVector<Te
         }
         bool ok = true;
         for (size_t i = 0; ok && i < inDescs.size(); ++i) {
+            if (InputMayBeEmpty(i) && Utils::GetTensorSize(inDescs.at(i)) == 0) {
+                continue; // an optional operand that is left out
+            }
             ok = inDescs.at(i).dtype == c.inDtypes[i] && inDescs.at(i).format == c.inFormats[i];
         }
         if (ok && outDescs && outDescs->size() != 0) {
@@ -80,7 +86,7 @@ Status OperationBase::InferShape(const SVector<TensorDesc> &inTensorDescs, SVect
             return ERROR_INVALID_IN_TENSOR_NUM;
         }
         for (size_t i = 0; i < inTensorDescs.size(); ++i) {
-            Status st = CheckOneShape(inTensorDescs.at(i));
+            Status st = CheckOneShape(inTensorDescs.at(i), InputMayBeEmpty(i));
             if (st != NO_ERROR) {
                 return st;
             }
@@ -117,11 +123,11 @@ Status OperationBase::Setup(const VariantPack &variantPack, uint64_t &workspaceS
                            << GetOutputNum();
             return ERROR_INVALID_IN_TENSOR_NUM;
         }
-        Status st = CheckShapes(variantPack.inTensors, "inTensor");
+        Status st = CheckShapes(variantPack.inTensors, "inTensor", true);
         if (st != NO_ERROR) {
             return st;
         }
-        st = CheckShapes(variantPack.outTensors, "outTensor");
+        st = CheckShapes(variantPack.outTensors, "outTensor", false);
         if (st != NO_ERROR) {
             return st;
         }
@@ -201,7 +207,7 @@ Status OperationBase::PreLaunch(const VariantPack &variantPack, uint8_t *workspa
             ATB_LOG(ERROR) << name_ << " Execute: inTensors(" << i << ").dataSize differs from the Setup size";
             return ERROR_INVALID_PARAM;
         }
-        if (!t.deviceData && !t.hostData) {
+        if (!t.deviceData && !t.hostData && !(t.dataSize == 0 && InputMayBeEmpty(i))) {
             ATB_LOG(ERROR) << name_ << " Execute: inTensors(" << i << ") has no data pointer";
             return ERROR_INVALID_PARAM;
         }

@@ -59,7 +59,10 @@ protected:
     const OpIr *ir_ = nullptr;
 
 private:
-    Status CheckShapes(const SVector<Tensor> &tensors, const char *what) const;
+    // Inputs an operation accepts as empty tensors (a dimension of 0): optional operands such as a
+    // quantiser's offset (reference Operation::GetEmptyInTensorPermissions).
+    virtual bool InputMayBeEmpty(size_t index) const { (void)index; return false; }
+    Status CheckShapes(const SVector<Tensor> &tensors, const char *what, bool inputs) const;
     bool IrMatch(const SVector<TensorDesc> &inDescs, const SVector<TensorDesc> *outDescs) const;
     Status PreLaunch(const VariantPack &variantPack, uint8_t *workspace, uint64_t workspaceSize, Context *context);
 

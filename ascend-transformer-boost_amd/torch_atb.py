@@ -122,6 +122,15 @@ class ReshapeAndCacheWithStrideParam(_Param):
         K_CACHE_V_BYPASS = 1
 
 
+class ElewiseParam(_Param):
+    _struct = _b.ElewiseParam
+    _op_name = "ElewiseOperation"
+
+    class ElewiseType(enum.IntEnum):
+        ELEWISE_QUANT_PER_CHANNEL = 17
+        ELEWISE_DEQUANT_PER_CHANNEL = 18
+
+
 class RopeParam(_Param):
     _struct = _b.RopeParam
     _op_name = "RopeOperation"

@@ -40,6 +40,7 @@ typedef enum {
     ACL_FORMAT_NC1HWC0 = 3,
     ACL_FORMAT_FRACTAL_Z = 4,
     ACL_FORMAT_FRACTAL_NZ = 29,
+    ACL_FORMAT_NCDHW = 30,
 } aclFormat;
 
 typedef void *aclrtStream;

@@ -167,6 +167,52 @@ struct MultiLatentAttentionParam {
     uint8_t rsv[32] = {0}; // must stay zero
 };
 
+// Elementwise operations (reference include/atb/infer_op_params.h:354-421). Built here: the two
+// per-channel forms that sit beside the int8 KV cache, ELEWISE_QUANT_PER_CHANNEL (x, scale, offset ->
+// int8) and ELEWISE_DEQUANT_PER_CHANNEL (int8 x, scale, offset -> fp16); the other types are
+// rejected when the operation is created.
+struct ElewiseParam {
+    enum ElewiseType : int {
+        ELEWISE_UNDEFINED = 0,
+        ELEWISE_CAST,
+        ELEWISE_MULS,
+        ELEWISE_COS,
+        ELEWISE_SIN,
+        ELEWISE_NEG,
+        ELEWISE_QUANT,
+        ELEWISE_LOGICAL_NOT,
+        ELEWISE_ADD,
+        ELEWISE_MUL,
+        ELEWISE_REALDIV,
+        ELEWISE_LOGICAL_AND,
+        ELEWISE_LOGICAL_OR,
+        ELEWISE_LESS,
+        ELEWISE_GREATER,
+        ELEWISE_SUB,
+        ELEWISE_EQUAL,
+        ELEWISE_QUANT_PER_CHANNEL,
+        ELEWISE_DEQUANT_PER_CHANNEL,
+        ELEWISE_DYNAMIC_QUANT,
+        ELEWISE_TANH,
+        ELEWISE_TYPE_MAX
+    };
+    struct QuantParam {
+        float inputScale = 1.0f;
+        bool asymmetric = false;
+        int inputOffset = 0;
+        uint8_t rsv[20] = {0}; // must stay zero
+    };
+    struct MulsParam {
+        float varAttr = 0.0f;
+        uint8_t rsv[12] = {0}; // must stay zero
+    };
+    ElewiseType elewiseType = ELEWISE_UNDEFINED;
+    QuantParam quantParam;
+    MulsParam mulsParam;
+    aclDataType outTensorType = ACL_DT_UNDEFINED;
+    uint8_t rsv[8] = {0}; // must stay zero
+};
+
 // Rotary position embedding of query and key rows (reference include/atb/infer_op_params.h:1605-1617).
 struct RopeParam {
     int32_t rotaryCoeff = 4; // 2: rotate halves; 4: the two halves of a head separately; headDim: interleaved pairs
@@ -205,6 +251,8 @@ struct PagedCacheLoadParam {
 
 static_assert(sizeof(ReshapeAndCacheParam) == 24, "ReshapeAndCacheParam ABI size");
 static_assert(sizeof(ReshapeAndCacheWithStrideParam) == 24, "ReshapeAndCacheWithStrideParam ABI size");
+static_assert(sizeof(ElewiseParam) == 64 && sizeof(ElewiseParam::QuantParam) == 32 && sizeof(ElewiseParam::MulsParam) == 16,
+              "ElewiseParam ABI size");
 static_assert(sizeof(RopeParam) == 16, "RopeParam ABI size");
 static_assert(sizeof(NormRopeReshapeParam) == 28, "NormRopeReshapeParam ABI size");
 static_assert(sizeof(BlockCopyParam) == 16, "BlockCopyParam ABI size");

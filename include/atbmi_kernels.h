@@ -118,6 +118,24 @@ int atbmi_rope(const void *qDevice, const void *kDevice, const void *cosDevice, 
                int32_t cosFormat, int32_t dtype, int32_t tableIsFloat, void *stream);
 
 /*
+ * ElewiseOperation's per-channel quantiser and dequantiser. x holds `total` elements, scale (the
+ * type of x for the quantiser, fp16 for the dequantiser) and offset (int8, may be NULL) hold
+ * `channels` entries each; element i uses entry i % channels (the scale covers the trailing
+ * dimensions of x, or is a single value).
+ *   quantiser:   out = clamp(rint(fp16(x / scale)) + offset, -128, 127) as int8: the quotient is
+ *                rounded to fp16 first (the reference golden divides in fp16, bf16 inputs included);
+ *                ties to even, NaN -> 0
+ *   dequantiser: out = fp16((x - offset) * scale), saturated at +-65504
+ * Replaces: the ELEWISE_QUANT_PER_CHANNEL / ELEWISE_DEQUANT_PER_CHANNEL kernels behind ElewiseOperation
+ * (reference src/ops/ops_infer/elewise/elewise_operation.cpp:451-472; goldens tests/apitest/opstest/
+ * python/operations/elewise/test_elewise_quant.py:24-32, test_elewise_dequant.py:23-31).
+ */
+int atbmi_elewise_quant_per_channel(const void *xDevice, const void *scaleDevice, const int8_t *offsetDevice,
+                                    int8_t *outDevice, int64_t total, int64_t channels, int32_t dtype, void *stream);
+int atbmi_elewise_dequant_per_channel(const int8_t *xDevice, const void *scaleDevice, const int8_t *offsetDevice,
+                                      void *outDevice, int64_t total, int64_t channels, void *stream);
+
+/*
  * Per-channel int8 quantiser: out[r][c] = clamp(rint(float(x[r][c]) / scale[c]) + offset[c], -128, 127),
  * IEEE fp32 divide, round-half-even, NaN -> 0. offset may be NULL.
  * Replaces: the ELEWISE_QUANT_PER_CHANNEL kernel (golden

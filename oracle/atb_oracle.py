@@ -13,6 +13,7 @@ pinned by tests/test_oracle.py against closed forms, fp64 brute force and
 the invariants of the mathematics (no function is left "parity unpinned"):
 
   reshape_and_cache   tests/apitest/kernelstest/mix/test_reshape_and_cache.py:45-65
+  dequant_per_channel tests/apitest/opstest/python/operations/elewise/test_elewise_dequant.py:23-31
   strided_view        tests/unittest/ops/reshape_and_cache_with_stride/test_reshape_and_cache_with_stride.cpp:
                       219-245 (element [i0, i1, i2] of the view is storage[offset + sum(i_k * stride_k)]),
                       :411-433 (the view then goes through the plain reshape_and_cache golden)
@@ -224,6 +225,19 @@ def quant_per_channel_golden_dtype(x_fp16, scale_fp16, offset=None):
         r = r + offset
     r = np.where(np.isnan(r), 0, r)
     return np.clip(r, -128, 127).astype(np.int8)
+
+
+def dequant_per_channel(x_int8, scale_fp16, offset=None):
+    """ElewiseOperation's per-channel dequantiser as the reference golden writes it (tests/apitest/opstest/
+    python/operations/elewise/test_elewise_dequant.py:23-31): (fp16(x) - fp16(offset)) * scale in fp16
+    arithmetic, clipped to the largest finite fp16 values. scale / offset broadcast over the trailing
+    dimensions of x."""
+    y = np.asarray(x_int8).astype(np.float16)
+    with np.errstate(over="ignore", invalid="ignore"):
+        if offset is not None:
+            y = y - np.asarray(offset).astype(np.float16)
+        out = y * np.asarray(scale_fp16, dtype=np.float16)
+    return np.clip(out, np.float16(-65504), np.float16(65504)).astype(np.float16)
 
 
 def softmax_rows(sim):

@@ -11,6 +11,7 @@ status, tagged C: for CreateOperation, I: for InferShape, S: for Setup):
     tests/apitest/opstest/csv/paged_cache_load.csv
     tests/apitest/opstest/csv/norm_rope_reshape.csv
     tests/apitest/opstest/csv/rope.csv
+    tests/apitest/opstest/csv/elewise.csv (the rows of the two per-channel quantiser types)
 Those rows are data, not code. This script copies the rows written for the
 Ascend910B feature set (the one this library mirrors) into
     tests/golden/paged_attention_cases.json
@@ -20,6 +21,7 @@ Ascend910B feature set (the one this library mirrors) into
     tests/golden/paged_cache_load_cases.json
     tests/golden/norm_rope_reshape_cases.json
     tests/golden/rope_cases.json
+    tests/golden/elewise_cases.json
 so the parity tests can run where the reference tree is absent.
 
 Run from the repository root in a container that has /root/reference:
@@ -45,7 +47,7 @@ def shapes(field):
     return out
 
 
-def convert(name, also_untagged=False):
+def convert(name, also_untagged=False, keep=None):
     path = os.path.join(REF, "tests/apitest/opstest/csv", name + ".csv")
     rows = list(csv.reader(open(path, newline=""), delimiter="|"))
     header = [h.strip() for h in rows[0]]
@@ -58,6 +60,8 @@ def convert(name, also_untagged=False):
         # and a row may name several products, or none when it holds for all of them)
         tags = [t.strip() for t in d.get("SocVersion", "").split(",") if t.strip()]
         if "Ascend910B" not in tags and not (also_untagged and not tags):
+            continue
+        if keep is not None and not keep(json.loads(d["OpParam"])):
             continue
         # OutNum is what the harness hands to the operation (BlockCopy lists two output columns but takes none)
         n_out = int(d["OutNum"]) if d.get("OutNum", "").strip().isdigit() else None
@@ -92,3 +96,4 @@ if __name__ == "__main__":
     convert("paged_cache_load")
     convert("norm_rope_reshape", also_untagged=True)
     convert("rope", also_untagged=True)
+    convert("elewise", also_untagged=True, keep=lambda p: p.get("elewiseType") in (17, 18))

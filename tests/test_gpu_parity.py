@@ -192,6 +192,76 @@ def test_reshape_and_cache_with_stride_equals_plain_on_contiguous_input(binding,
     ctx.close()
 
 
+# ------------------------------------------------------------------ ElewiseOperation (per-channel quantiser / dequantiser)
+def test_elewise_quant_per_channel_bit_exact(binding, oracle, dev, stream):
+    """ELEWISE_QUANT_PER_CHANNEL against the reference golden (fp16 division, round, offset, clamp), bit-exact:
+    every finite fp16 pattern as x, the shapes of the reference's tests (scale over the trailing dimensions,
+    a single scale, no offset), fp16 and bf16."""
+    rng = _rng(71)
+    ctx = binding.Context(stream)
+    runner = binding.OperationRunner("ElewiseOperation", binding.ElewiseParam(elewiseType=17), ctx)
+    bits = np.arange(65536, dtype=np.uint16).view(np.float16)
+    allx = bits[np.isfinite(bits)]
+    allx = np.concatenate([allx, allx[: (-len(allx)) % 1024]]).reshape(-1, 1024)
+    cases = [(torch.float16, torch.from_numpy(allx.copy()), (1024,), True),
+             (torch.float16, None, (32, 160), True), (torch.float16, None, (1,), True),
+             (torch.float16, None, (32, 32), False), (torch.bfloat16, None, (32, 160), True),
+             (torch.float16, None, (7, 9), True)]     # odd sizes: the element-wise path
+    for dtype, x, scale_shape, with_offset in cases:
+        if x is None:
+            lead = (27,) if len(scale_shape) == 2 else (64, 1024)
+            x = torch.from_numpy(rng.uniform(-300, 300, size=lead + (scale_shape if scale_shape != (1,) else ())).astype(np.float32)).to(dtype)
+        scale = torch.from_numpy(rng.uniform(0.1, 3.0, size=scale_shape).astype(np.float32)).to(dtype)
+        offset = torch.from_numpy(rng.integers(-10, 10, size=scale_shape).astype(np.int8)) if with_offset else \
+            torch.empty((0,), dtype=torch.int8)
+        # the golden converts bf16 inputs to fp16 first
+        want = oracle.quant_per_channel_golden_dtype(x.to(torch.float16).numpy(), scale.to(torch.float16).numpy(),
+                                                     offset.numpy() if with_offset else None)
+        with torch.cuda.stream(stream):
+            keep = [x.to(dev), scale.to(dev), offset.to(dev)]
+            ins = [binding.tensor_of(keep[0]), binding.tensor_of(keep[1]),
+                   binding.tensor_of(keep[2]) if with_offset else binding.make_tensor("int8", [0], None)]
+            out = torch.empty(x.shape, dtype=torch.int8, device=dev)
+            runner.run(ins, outputs=[out])
+        stream.synchronize()
+        assert np.array_equal(out.cpu().numpy(), want), (dtype, scale_shape, with_offset)
+    runner.close()
+    ctx.close()
+
+
+def test_elewise_dequant_per_channel_bit_exact(binding, oracle, dev, stream):
+    """ELEWISE_DEQUANT_PER_CHANNEL against the reference golden, bit-exact: every int8 value against every
+    offset for a set of scales that includes the saturating ones, and the shapes of the reference's tests."""
+    rng = _rng(72)
+    ctx = binding.Context(stream)
+    runner = binding.OperationRunner("ElewiseOperation", binding.ElewiseParam(elewiseType=18), ctx)
+    grid_x = np.repeat(np.arange(-128, 128, dtype=np.int8), 256).reshape(256, 256)      # row = x
+    grid_o = np.tile(np.arange(-128, 128, dtype=np.int8), 256).reshape(256, 256)[:1]    # column = offset
+    cases = []
+    for sc in (0.37, 1.0, 300.0, -512.0, 6e-5, 65504.0):
+        cases.append((torch.from_numpy(grid_x.copy()), np.full((256,), sc, np.float16), grid_o[0].copy()))
+    cases.append((torch.from_numpy(rng.integers(-128, 128, size=(27, 32, 160)).astype(np.int8)),
+                  rng.uniform(0.1, 1, size=(32, 160)).astype(np.float16), rng.integers(-128, 128, size=(32, 160)).astype(np.int8)))
+    cases.append((torch.from_numpy(rng.integers(-128, 128, size=(64, 1024)).astype(np.int8)),
+                  np.array([0.25], np.float16), np.array([-7], np.int8)))
+    cases.append((torch.from_numpy(rng.integers(-128, 128, size=(10, 8192)).astype(np.int8)),
+                  rng.uniform(0.1, 1, size=(8192,)).astype(np.float16), None))
+    cases.append((torch.from_numpy(rng.integers(-128, 128, size=(5, 7, 9)).astype(np.int8)),
+                  rng.uniform(0.1, 1, size=(7, 9)).astype(np.float16), rng.integers(-128, 128, size=(7, 9)).astype(np.int8)))
+    for x, scale, offset in cases:
+        want = oracle.dequant_per_channel(x.numpy(), scale, offset)
+        with torch.cuda.stream(stream):
+            keep = [x.to(dev), torch.from_numpy(scale).to(dev)] + ([torch.from_numpy(offset).to(dev)] if offset is not None else [])
+            ins = [binding.tensor_of(keep[0]), binding.tensor_of(keep[1]),
+                   binding.tensor_of(keep[2]) if offset is not None else binding.make_tensor("int8", [0], None)]
+            out = torch.empty(x.shape, dtype=torch.float16, device=dev)
+            runner.run(ins, outputs=[out])
+        stream.synchronize()
+        assert np.array_equal(out.cpu().numpy().view(np.int16), want.view(np.int16)), (tuple(x.shape), scale.shape)
+    runner.close()
+    ctx.close()
+
+
 # ------------------------------------------------------------------ Rope
 ROPE_CASES = [
     # name, q shape, k shape, table rows, head_dim, rotaryCoeff, cosFormat, seq lens, x dtype, table dtype

@@ -32,6 +32,7 @@ BLOCK_COPY_CASES = _load("block_copy")
 CACHE_LOAD_CASES = _load("paged_cache_load")
 NORM_ROPE_CASES = _load("norm_rope_reshape")
 ROPE_CASES = _load("rope")
+ELEWISE_CASES = _load("elewise")
 
 
 def _pa_unimplemented(p):
@@ -77,6 +78,7 @@ def _make_param(binding, op, p):
            "ReshapeAndCacheWithStrideOperation": binding.ReshapeAndCacheWithStrideParam,
            "NormRopeReshapeOperation": binding.NormRopeReshapeParam,
            "RopeOperation": binding.RopeParam,
+           "ElewiseOperation": binding.ElewiseParam,
            "ReshapeAndCacheOperation": binding.ReshapeAndCacheParam}[op]
     fields = {k: v for k, v in p.items() if k != "rsv"}
     param = cls(**fields) if fields else cls()
@@ -182,6 +184,51 @@ def test_paged_cache_load_table(binding, ctx, case):
     # the fractal-NZ cache layout (kvCacheCfg 0, the param's default) is rejected when the operation is created
     nz = case["param"].get("kvCacheCfg", 0) == 0
     _check(binding, case, ctx, nz and not case["expected"].startswith("C:"))
+
+
+@pytest.mark.parametrize("case", ELEWISE_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
+def test_elewise_per_channel_table(binding, ctx, case):
+    _check(binding, case, ctx, False)
+
+
+def test_elewise_checks(binding, ctx):
+    """Creation (reference elewise_operation.cpp:40-99), the optional offset (:474-486) and what the kernel
+    needs of the shapes."""
+    E = binding.ERROR_CODE
+    P = binding.ElewiseParam
+    assert ctypes.sizeof(P) == 64   # reference tests/unittest/ops/test_op_param_size.cpp:25
+    for t in (0, 21, 22, -1):       # out of range
+        assert binding.Operation("ElewiseOperation", P(elewiseType=t)).status == E["ERROR_INVALID_PARAM"]
+    for t in (1, 2, 6, 8, 19, 20):  # in range, not built here
+        assert binding.Operation("ElewiseOperation", P(elewiseType=t)).status == E["ERROR_INVALID_PARAM"]
+    for field in ("rsv", "quantRsv", "mulsRsv"):
+        p = P(elewiseType=17)
+        getattr(p, field)[1] = 1
+        assert binding.Operation("ElewiseOperation", p).status == E["ERROR_INVALID_PARAM"]
+    mk = binding.make_tensor
+    op = binding.Operation("ElewiseOperation", P(elewiseType=17))
+    assert op.get_name() == "ElewiseOperation" and (op.input_num(), op.output_num()) == (3, 1)
+    ins = lambda x=(10, 8192), s=(8192,), o=(8192,): [mk("float16", x, FAKE_DEVICE), mk("float16", s, FAKE_DEVICE),
+                                                     mk("int8", o, FAKE_DEVICE)]
+    out = lambda shape=(10, 8192): [mk("int8", shape, FAKE_DEVICE)]
+    st, descs = op.infer_shape(ins())
+    assert st == 0 and descs[0].dtype == binding.ACL_INT8 and [descs[0].dims[i] for i in range(2)] == [10, 8192]
+    assert op.setup(ins(), out(), ctx) == (0, 0)
+    # the offset may be an empty tensor; nothing else may
+    assert op.infer_shape(ins(o=(0,)))[0] == 0 and op.setup(ins(o=(0,)), out(), ctx) == (0, 0)
+    assert op.infer_shape(ins(s=(0,)))[0] == E["ERROR_INVALID_TENSOR_SIZE"]
+    # scale / offset must tile x, the output must have x's size
+    assert op.setup(ins(s=(100,), o=(100,)), out(), ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.setup(ins(o=(4096,)), out(), ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.setup(ins(), out((10, 4096)), ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    op.close()
+    op = binding.Operation("ElewiseOperation", P(elewiseType=18))
+    d_ins = [mk("int8", (10, 64), FAKE_DEVICE), mk("float16", (64,), FAKE_DEVICE), mk("int8", (64,), FAKE_DEVICE)]
+    st, descs = op.infer_shape(d_ins)
+    assert st == 0 and descs[0].dtype == binding.ACL_FLOAT16
+    bf = [mk("int8", (10, 64), FAKE_DEVICE), mk("bf16", (64,), FAKE_DEVICE), mk("int8", (64,), FAKE_DEVICE)]
+    assert op.infer_shape(bf)[0] == E["ERROR_INVALID_TENSOR_INI_MATCH"]
+    op.close()
 
 
 @pytest.mark.parametrize("case", ROPE_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
@@ -808,6 +855,7 @@ def test_cpp_api_symbols_are_exported(pkg):
         "atb::CreateOperation<atb::infer::ReshapeAndCacheWithStrideParam>",
         "atb::CreateOperation<atb::infer::NormRopeReshapeParam>",
         "atb::CreateOperation<atb::infer::RopeParam>",
+        "atb::CreateOperation<atb::infer::ElewiseParam>",
         "atb::DestroyOperation(atb::Operation*)",
         "atb::CreateContext(atb::Context**)",
         "atb::DestroyContext(atb::Context*)",

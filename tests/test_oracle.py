@@ -64,6 +64,65 @@ def test_reshape_and_cache_single_cache(oracle):
     assert np.array_equal(kc[1, 1, 0], key[0, 0]) and kc.sum() == key[0].sum()
 
 
+def test_quant_golden_dtype_exact_rational(oracle):
+    """The ElewiseOperation form (16-bit scale, quotient rounded to fp16, then to an integer) against exact
+    rational arithmetic: the fp16 nearest to x / s (ties to even), then the integer nearest to that."""
+    from fractions import Fraction
+    import math
+    bits = np.arange(0, 65536, 53, dtype=np.uint16)
+    x = bits.view(np.float16)
+    x = x[np.isfinite(x)]
+
+    def nearest_fp16(q):
+        f = np.float16(float(q))            # double -> fp16 rounds the double; the double of q may itself be rounded,
+        lo, hi = np.nextafter(f, np.float16(-np.inf)), np.nextafter(f, np.float16(np.inf))
+        best = min((c for c in (lo, f, hi) if np.isfinite(c)), key=lambda c: abs(Fraction(float(c)) - q), default=f)
+        return best                          # so take the closest of the neighbours by exact distance
+
+    for s in [np.float16(0.1), np.float16(0.337), np.float16(1.0), np.float16(3.0)]:
+        got = oracle.quant_per_channel_golden_dtype(x, s, np.int8(5))
+        for xi, gi in zip(x.tolist(), got.tolist()):
+            q = Fraction(xi) / Fraction(float(s))
+            h = nearest_fp16(q)
+            if not np.isfinite(h) or abs(q) >= 65520:
+                want = 127 if q > 0 else -128
+            else:
+                hf = Fraction(float(h))
+                r = math.floor(hf)
+                frac = hf - r
+                r = r + 1 if frac > Fraction(1, 2) or (frac == Fraction(1, 2) and r % 2 == 1) else r
+                want = max(-128, min(127, r + 5))
+            # (a quotient exactly between two fp16 values is the one case the neighbour search cannot order; skip it)
+            lo, hi = np.nextafter(h, np.float16(-np.inf)), np.nextafter(h, np.float16(np.inf))
+            if np.isfinite(lo) and np.isfinite(hi) and abs(Fraction(float(h)) - q) in (abs(Fraction(float(lo)) - q), abs(Fraction(float(hi)) - q)):
+                continue
+            assert gi == want, (xi, float(s), gi, want)
+
+
+# ---------------------------------------------------------------- dequant_per_channel
+def test_dequant_per_channel_exact_products_and_saturation(oracle):
+    """Every (x - offset) is an integer in [-255, 255] and a scale has 11 significant bits, so the exact
+    product fits a double: the fp16 result must be that product rounded once, or +-65504 past the range."""
+    from fractions import Fraction
+    rng = _rng(61)
+    x = rng.integers(-128, 128, size=(5, 4, 8)).astype(np.int8)
+    scale = rng.uniform(0.1, 1.0, size=(4, 8)).astype(np.float16)
+    scale[0, 0], scale[0, 1], scale[0, 2] = np.float16(300.0), np.float16(-512.0), np.float16(6e-5)
+    offset = rng.integers(-128, 128, size=(4, 8)).astype(np.int8)
+    got = oracle.dequant_per_channel(x, scale, offset)
+    assert got.dtype == np.float16 and got.shape == x.shape
+    exact = (x.astype(np.float64) - offset.astype(np.float64)) * scale.astype(np.float64)
+    want = np.clip(exact, -65504, 65504).astype(np.float16)   # float64 -> fp16 is one rounding of an exact value
+    assert np.array_equal(got.view(np.int16), want.view(np.int16))
+    assert np.isfinite(got).all() and (np.abs(exact) > 65504).any()
+    assert Fraction(float(got[1, 1, 3])) == Fraction(float(np.float16(float(
+        (int(x[1, 1, 3]) - int(offset[1, 3])) * Fraction(float(scale[1, 3]))))))
+    # no offset, and a single scale for everything
+    assert np.array_equal(oracle.dequant_per_channel(x, scale), np.clip(x.astype(np.float64) * scale.astype(np.float64), -65504, 65504).astype(np.float16))
+    one = oracle.dequant_per_channel(x, np.array([0.5], np.float16), np.array([3], np.int8))
+    assert np.array_equal(one, ((x.astype(np.float32) - 3) * 0.5).astype(np.float16))
+
+
 # ---------------------------------------------------------------- strided_view
 def test_strided_view_matches_library_views_and_loops(oracle):
     """Against numpy's and torch's own strided views, against the element loop of the reference's unit
