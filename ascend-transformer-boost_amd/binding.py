@@ -266,8 +266,42 @@ def atb():
         lib.atb_c_sizeof_paged_attention_param.restype = u64
         lib.atb_c_sizeof_reshape_and_cache_param.restype = u64
         lib.atb_c_sizeof_multi_latent_attention_param.restype = u64
+        # the aclnn-style tensor handle and the two-call wrappers of atb/atb_acl.h
+        i64p = ctypes.POINTER(ctypes.c_int64)
+        lib.aclCreateTensor.argtypes = [i64p, u64, i32, i64p, ctypes.c_int64, i32, i64p, u64, vp]
+        lib.aclCreateTensor.restype = vp
+        lib.aclDestroyTensor.argtypes = [vp]
+        lib.aclGetDataType.argtypes = [vp, ctypes.POINTER(i32)]
+        lib.aclGetFormat.argtypes = [vp, ctypes.POINTER(i32)]
+        lib.aclGetRawTensorAddr.argtypes = [vp, ctypes.POINTER(vp)]
+        lib.aclDataTypeSize.argtypes = [i32]
+        lib.aclDataTypeSize.restype = ctypes.c_size_t
+        lib.AtbMLAGetWorkspaceSize.argtypes = [vp] * 10 + [i32, ctypes.c_float, i32, ctypes.c_int, ctypes.c_int,
+                                                           ctypes.c_uint8, vp, vp, ctypes.POINTER(u64),
+                                                           ctypes.POINTER(vp), vp]
+        lib.AtbMLA.argtypes = [vp, u64, vp, vp]
+        lib.AtbPagedCacheLoadGetWorkspaceSize.argtypes = [vp] * 7 + [ctypes.c_int8, ctypes.c_bool, ctypes.c_bool,
+                                                                     ctypes.POINTER(u64), ctypes.POINTER(vp), vp]
+        lib.AtbPagedCacheLoad.argtypes = [vp, u64, vp, vp]
         _atb = lib
     return _atb
+
+
+def acl_tensor(dtype, shape, data_ptr, fmt=ACL_FORMAT_ND):
+    """aclCreateTensor for a contiguous tensor at data_ptr (device or host memory); release it with
+    atb().aclDestroyTensor."""
+    dims = (ctypes.c_int64 * len(shape))(*[int(d) for d in shape])
+    strides = [1] * len(shape)
+    for i in range(len(shape) - 2, -1, -1):
+        strides[i] = strides[i + 1] * int(shape[i + 1])
+    st = (ctypes.c_int64 * len(shape))(*strides)
+    code = ACL_DTYPE_BY_NAME[dtype] if isinstance(dtype, str) else int(dtype)
+    return atb().aclCreateTensor(dims, len(shape), code, st, 0, int(fmt), dims, len(shape), ctypes.c_void_p(data_ptr))
+
+
+def acl_tensor_of(t):
+    """aclTensor handle of a contiguous torch tensor (a CPU tensor gives a host address)."""
+    return acl_tensor(_torch_acl_dtype(t), list(t.shape), t.data_ptr())
 
 
 def last_kernel_error():

@@ -157,6 +157,7 @@ Status OperationBase::Setup(const VariantPack &variantPack, uint64_t &workspaceS
         context_ = impl;
         workspaceSize_ = ws;
         workspaceSize = ws;
+        setupPack_ = variantPack;
         setupInSizes_.clear();
         setupOutSizes_.clear();
         for (size_t i = 0; i < variantPack.inTensors.size(); ++i) {
@@ -234,6 +235,14 @@ Status OperationBase::Execute(const VariantPack &variantPack, uint8_t *workspace
         return ERROR_INVALID_PARAM;
     }
     const ExecuteType type = context->GetExecuteType();
+    // A pack without tensors stands for the one Setup was given: the two-call C wrappers
+    // (AtbMLAGetWorkspaceSize + AtbMLA, reference src/ops/ops_infer/multi_latent_attention/
+    // atb_acl_mla.cpp:118-124) run Execute that way.
+    if (variantPack.inTensors.size() == 0 && variantPack.outTensors.size() == 0 && setupOk_ &&
+        (type == EXECUTE_NORMAL || type == EXECUTE_PRELAUNCH)) {
+        const VariantPack kept = setupPack_;
+        return Execute(kept, workspace, workspaceSize, context);
+    }
     try {
         if (type == EXECUTE_NORMAL || type == EXECUTE_PRELAUNCH) {
             Status st = PreLaunch(variantPack, workspace, workspaceSize, context);

@@ -70,6 +70,7 @@ private:
     bool setupOk_ = false;
     ContextImpl *context_ = nullptr;
     uint64_t workspaceSize_ = 0;
+    VariantPack setupPack_;
     std::vector<uint64_t> setupInSizes_;
     std::vector<uint64_t> setupOutSizes_;
     // Captured by a pre-launch for the launch half.

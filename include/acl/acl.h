@@ -1,12 +1,16 @@
 // Minimal stand-in for the CANN runtime header that atb/types.h pulls in.
-// Only the three things the PagedAttention / ReshapeAndCache path touches are
-// declared: tensor element types, tensor formats and the stream handle.
+// Only what the PagedAttention / ReshapeAndCache path touches is declared: tensor
+// element types, tensor formats, the stream handle and the tensor handle of the
+// aclnn-style wrappers.
 // Enumerator values are the CANN ones, so packs built by existing callers
 // keep their meaning (value table: reference
 // tests/framework/python/CsvOpsTestTool/atb_csv_ops_test.py:33-40).
 // On MI355X an aclrtStream carries a hipStream_t.
 #ifndef ATB_MI_ACL_SHIM_H
 #define ATB_MI_ACL_SHIM_H
+
+#include <stddef.h>
+#include <stdint.h>
 
 #ifdef __cplusplus
 extern "C" {
@@ -44,6 +48,28 @@ typedef enum {
 } aclFormat;
 
 typedef void *aclrtStream;
+
+/* The tensor handle of CANN's aclnn-style interfaces (there: aclnn/acl_meta.h), as far as the
+ * two-call C wrappers of atb/atb_acl.h need it: a view shape, an element type, a format and the
+ * address of the data (device memory, or host memory for the operands the wrappers read on the
+ * host). stride, offset and the storage shape are accepted and kept, and must describe a
+ * contiguous tensor that starts at tensorData. */
+typedef struct aclTensor aclTensor;
+typedef int aclnnStatus;
+#define ACL_SUCCESS 0
+#define ACL_ERROR_INVALID_PARAM 100000
+
+aclTensor *aclCreateTensor(const int64_t *viewDims, uint64_t viewDimsNum, aclDataType dataType, const int64_t *stride,
+                           int64_t offset, aclFormat format, const int64_t *storageDims, uint64_t storageDimsNum,
+                           void *tensorData);
+aclnnStatus aclDestroyTensor(const aclTensor *tensor);
+/* *viewDims is allocated with new[]; the caller releases it with delete[] (as CANN's does). */
+aclnnStatus aclGetViewShape(const aclTensor *tensor, int64_t **viewDims, uint64_t *viewDimsNum);
+aclnnStatus aclGetDataType(const aclTensor *tensor, aclDataType *dataType);
+aclnnStatus aclGetFormat(const aclTensor *tensor, aclFormat *format);
+aclnnStatus aclGetRawTensorAddr(const aclTensor *tensor, void **addr);
+/* Bytes per element; 0 for a type without a fixed size. */
+size_t aclDataTypeSize(aclDataType dataType);
 
 #ifdef __cplusplus
 }

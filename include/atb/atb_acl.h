@@ -1,0 +1,41 @@
+// The aclnn-style two-call C wrappers of the reference (include/atb/atb_acl.h) for the operations
+// this library has: the first call creates the operation if *op is null, binds the tensors and
+// runs Setup (returning the workspace size), the second runs Execute on what the first bound.
+//   AtbMLAGetWorkspaceSize / AtbMLA                      reference include/atb/atb_acl.h:99-116
+//   AtbPagedCacheLoadGetWorkspaceSize / AtbPagedCacheLoad  reference include/atb/atb_acl.h:251-267
+// contextLens and qSeqLen are host tensors: their aclTensor carries a host address.
+#ifndef ATB_MI_ATB_ACL_H
+#define ATB_MI_ATB_ACL_H
+#include <acl/acl.h>
+#include "atb/context.h"
+#include "atb/infer_op_params.h"
+#include "atb/operation.h"
+#include "atb/types.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+// MultiLatentAttention (cacheMode KROPE_CTKV). mask is read when maskType is not UNDEFINED, qSeqLen
+// when calcType is CALC_TYPE_SPEC, lse when calcType is CALC_TYPE_RING; qkDescale / pvDescale belong
+// to the int8 cache mode, which this library does not have. Pointers that are not read may be null.
+atb::Status AtbMLAGetWorkspaceSize(const aclTensor *qNope, const aclTensor *qRope, const aclTensor *ctKV,
+                                   const aclTensor *kRope, const aclTensor *blockTables, const aclTensor *contextLens,
+                                   const aclTensor *mask, const aclTensor *qSeqLen, const aclTensor *qkDescale,
+                                   const aclTensor *pvDescale, int32_t headNum, float qkScale, int32_t kvHeadNum,
+                                   int maskType, int calcType, uint8_t cacheMode, aclTensor *attenOut, aclTensor *lse,
+                                   uint64_t *workspaceSize, atb::Operation **op, atb::Context *context);
+atb::Status AtbMLA(void *workspace, uint64_t workspaceSize, atb::Operation *op, atb::Context *context);
+
+// PagedCacheLoad. key and value are inputs and outputs at once; seqStarts is read when hasSeqStarts.
+atb::Status AtbPagedCacheLoadGetWorkspaceSize(const aclTensor *keyCache, const aclTensor *valueCache,
+                                              const aclTensor *blockTables, const aclTensor *contextLens,
+                                              const aclTensor *key, const aclTensor *value, const aclTensor *seqStarts,
+                                              int8_t kvCacheCfg, bool isSeqLensCumsumType, bool hasSeqStarts,
+                                              uint64_t *workspaceSize, atb::Operation **op, atb::Context *context);
+atb::Status AtbPagedCacheLoad(void *workspace, uint64_t workspaceSize, atb::Operation *op, atb::Context *context);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1100,6 +1100,82 @@ def test_multi_latent_attention_operation(binding, oracle, dev, stream, heads, d
     c.close()
 
 
+def test_two_call_c_wrappers_run_the_operations(binding, oracle, dev, stream):
+    """AtbMLAGetWorkspaceSize + AtbMLA and AtbPagedCacheLoadGetWorkspaceSize + AtbPagedCacheLoad on
+    aclTensor handles (reference include/atb/atb_acl.h:99-116,251-267): plain decode, the log-sum-exp
+    output, several query tokens with the mask; results against the oracle."""
+    import ctypes
+    lib = binding.atb()
+    rng = _rng(470)
+    heads, d, dv, block, dtype = 128, 576, 512, 128, torch.bfloat16
+    ctx_lens = np.array([700, 33, 1500, 128], dtype=np.int32)
+    _, kc, _, tables, ctx_lens = _pa_inputs(rng, dev, 4, heads, 1, block, d, d, ctx_lens, dtype, std=0.5)
+    k_nope, k_rope = kc[..., :dv].contiguous(), kc[..., dv:].contiguous()
+    q_lens = np.array([2, 1, 3, 1], dtype=np.int32)
+    scale = 1.0 / math.sqrt(192.0)
+    lens_host, qn_host = torch.from_numpy(ctx_lens), torch.from_numpy(q_lens)
+    c = binding.Context(stream)
+    A = binding.acl_tensor_of
+    for calc in (0, 2, 1):
+        multi, ring = calc == 1, calc == 2
+        rows = int(q_lens.sum()) if multi else 4
+        with torch.cuda.stream(stream):
+            q = (torch.rand((rows, heads, d)) * 2 - 1).to(dtype).to(dev)
+            qn_, qr_ = q[..., :dv].contiguous(), q[..., dv:].contiguous()
+            out = torch.zeros((rows, heads, dv), dtype=dtype, device=dev)
+            lse = torch.zeros((rows, heads, 1), dtype=dtype, device=dev)
+            mask = _spec_mask(rng, dev, "query", ctx_lens, q_lens, dtype) if multi else None
+        stream.synchronize()
+        handles = [A(qn_), A(qr_), A(k_nope), A(k_rope), A(tables), A(lens_host), A(mask) if multi else None,
+                   A(qn_host) if multi else None, A(out), A(lse) if ring else None]
+        ws, op = ctypes.c_uint64(0), ctypes.c_void_p()
+        st = lib.AtbMLAGetWorkspaceSize(*handles[:8], None, None, heads, scale, 1, 1 if multi else 0, calc, 1, handles[8],
+                                        handles[9], ctypes.byref(ws), ctypes.byref(op), c.ptr)
+        assert st == 0 and op.value, binding.ERROR_NAMES[st]
+        with torch.cuda.stream(stream):
+            work = torch.empty(max(int(ws.value), 1), dtype=torch.uint8, device=dev)
+            st = lib.AtbMLA(work.data_ptr(), ws.value, op, c.ptr)
+        stream.synchronize()
+        assert st == 0, binding.ERROR_NAMES[st]
+        want_lse = np.zeros((rows, heads), np.float32)
+        want = oracle_pa(oracle, q, kc, None, tables, ctx_lens, scale, mla_dv=dv, mask=mask,
+                         q_lens=q_lens if multi else None, mask_rows="query" if multi else "sequence", lse_out=want_lse)
+        assert_close(out, want, TOL[dtype], "AtbMLA calcType %d" % calc)
+        if ring:
+            assert_close(lse[..., 0], want_lse, TOL[dtype], "AtbMLA lse")
+        lib.atb_c_destroy_operation(op)
+        for h in handles:
+            if h:
+                lib.aclDestroyTensor(h)
+
+    # PagedCacheLoad through its wrapper
+    heads_kv, hd, blocks, bs = 4, 64, 12, 16
+    lens = np.array([20, 5, 33], dtype=np.int32)
+    tables_np = rng.permutation(blocks)[:9].reshape(3, 3).astype(np.int32)
+    with torch.cuda.stream(stream):
+        kcache = torch.from_numpy(rng.integers(-100, 100, size=(blocks, bs, heads_kv, hd)).astype(np.float32)).to(torch.float16).to(dev)
+        vcache = torch.from_numpy(rng.integers(-100, 100, size=(blocks, bs, heads_kv, hd)).astype(np.float32)).to(torch.float16).to(dev)
+        key = torch.zeros((int(lens.sum()), heads_kv, hd), dtype=torch.float16, device=dev)
+        value = torch.zeros_like(key)
+        t_d, l_d = torch.from_numpy(tables_np).to(dev), torch.from_numpy(lens).to(dev)
+        starts = torch.zeros(3, dtype=torch.int32, device=dev)
+    stream.synchronize()
+    want_k, want_v = oracle.paged_cache_load(_bits(kcache).cpu().numpy(), _bits(vcache).cpu().numpy(), tables_np, lens,
+                                             _bits(key).cpu().numpy(), _bits(value).cpu().numpy(), np.zeros(3, np.int32))
+    handles = [A(kcache), A(vcache), A(t_d), A(l_d), A(key), A(value), A(starts)]
+    ws, op = ctypes.c_uint64(0), ctypes.c_void_p()
+    st = lib.AtbPagedCacheLoadGetWorkspaceSize(*handles, 1, False, True, ctypes.byref(ws), ctypes.byref(op), c.ptr)
+    assert st == 0 and op.value, binding.ERROR_NAMES[st]
+    st = lib.AtbPagedCacheLoad(None, 0, op, c.ptr)
+    stream.synchronize()
+    assert st == 0, binding.ERROR_NAMES[st]
+    assert np.array_equal(_bits(key).cpu().numpy(), want_k) and np.array_equal(_bits(value).cpu().numpy(), want_v)
+    lib.atb_c_destroy_operation(op)
+    for h in handles:
+        lib.aclDestroyTensor(h)
+    c.close()
+
+
 def test_lse_output_of_plain_and_masked_decode(binding, oracle, dev, stream):
     """The log-sum-exp output is not tied to the latent layouts: separate K and V caches, a mask, rows
     split over ranges and rows written directly."""

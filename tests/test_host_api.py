@@ -845,6 +845,72 @@ def test_every_declared_symbol_is_exported(pkg, header, lib):
         assert hasattr(handle, n), "%s does not export %s" % (lib, n)
 
 
+def test_acl_tensor_handle_and_two_call_wrappers(binding, ctx):
+    """The aclnn-style tensor handle and AtbMLAGetWorkspaceSize / AtbPagedCacheLoadGetWorkspaceSize up to
+    Setup (reference include/atb/atb_acl.h:99-116,251-267; atb_acl_mla.cpp:25-116)."""
+    lib = binding.atb()
+    E = binding.ERROR_CODE
+    t = binding.acl_tensor("bf16", [4, 128, 512], FAKE_DEVICE)
+    assert t
+    dt, fmt, addr = ctypes.c_int32(), ctypes.c_int32(), ctypes.c_void_p()
+    assert lib.aclGetDataType(t, ctypes.byref(dt)) == 0 and dt.value == binding.ACL_BF16
+    assert lib.aclGetFormat(t, ctypes.byref(fmt)) == 0 and fmt.value == binding.ACL_FORMAT_ND
+    assert lib.aclGetRawTensorAddr(t, ctypes.byref(addr)) == 0 and addr.value == FAKE_DEVICE
+    assert lib.aclGetDataType(None, ctypes.byref(dt)) != 0
+    lib.aclDestroyTensor(t)
+    assert [lib.aclDataTypeSize(c) for c in (binding.ACL_INT8, binding.ACL_FLOAT16, binding.ACL_BF16, binding.ACL_FLOAT,
+                                             binding.ACL_INT64, -1)] == [1, 2, 2, 4, 8, 0]
+
+    lens = np.array([100, 7, 300, 1], dtype=np.int32)
+    mk = binding.acl_tensor
+    handles = dict(q=mk("float16", [4, 32, 512], FAKE_DEVICE), qr=mk("float16", [4, 32, 64], FAKE_DEVICE),
+                   kv=mk("float16", [16, 128, 1, 512], FAKE_DEVICE), kr=mk("float16", [16, 128, 1, 64], FAKE_DEVICE),
+                   tables=mk("int32", [4, 3], FAKE_DEVICE), lens=mk("int32", [4], lens.ctypes.data),
+                   out=mk("float16", [4, 32, 512], FAKE_DEVICE), lse=mk("float16", [4, 32, 1], FAKE_DEVICE))
+    ws, op = ctypes.c_uint64(0), ctypes.c_void_p()
+
+    def mla(calc_type, cache_mode=1, out="out", lse=None, op_ref=op):
+        h = handles
+        return lib.AtbMLAGetWorkspaceSize(h["q"], h["qr"], h["kv"], h["kr"], h["tables"], h["lens"], None, None, None, None,
+                                          32, 0.1, 1, 0, calc_type, cache_mode, h[out], h[lse] if lse else None,
+                                          ctypes.byref(ws), ctypes.byref(op_ref), ctx.ptr)
+    assert mla(0) == 0 and op.value and ws.value > 0
+    first = op.value
+    assert mla(0) == 0 and op.value == first          # an existing operation is reused
+    ring = ctypes.c_void_p()
+    assert mla(2, lse="lse", op_ref=ring) == 0 and ring.value and ring.value != first
+    nz = ctypes.c_void_p()
+    assert mla(0, cache_mode=2, op_ref=nz) == E["ERROR_INVALID_PARAM"] and not nz.value   # the int8 cache mode is not built
+    lens[2] = 3 * 128 + 1                              # longer than its block table: Setup refuses
+    assert mla(0) == E["ERROR_INVALID_PARAM"]
+    assert lib.AtbMLA(None, 0, None, ctx.ptr) == E["ERROR_INVALID_OPERATION_ADDR"]
+    for o in (op, ring):
+        lib.atb_c_destroy_operation(o)
+
+    load = ctypes.c_void_p()
+    hc = dict(kc=mk("float16", [16, 128, 8, 128], FAKE_DEVICE), vc=mk("float16", [16, 128, 8, 128], FAKE_DEVICE),
+              tables=mk("int32", [4, 3], FAKE_DEVICE), lens=mk("int32", [4], FAKE_DEVICE),
+              key=mk("float16", [400, 8, 128], FAKE_DEVICE), value=mk("float16", [400, 8, 128], FAKE_DEVICE),
+              starts=mk("int32", [4], FAKE_DEVICE))
+    assert lib.AtbPagedCacheLoadGetWorkspaceSize(hc["kc"], hc["vc"], hc["tables"], hc["lens"], hc["key"], hc["value"],
+                                                 hc["starts"], 1, False, True, ctypes.byref(ws), ctypes.byref(load),
+                                                 ctx.ptr) == 0 and load.value
+    lib.atb_c_destroy_operation(load)
+    # without seqStarts the wrapper binds six tensors, and the ND operation takes seven: refused, as in the reference
+    # (atb_acl_paged_cache_load.cpp:37-41 against paged_cache_load_operation.cpp:93-100)
+    six = ctypes.c_void_p()
+    assert lib.AtbPagedCacheLoadGetWorkspaceSize(hc["kc"], hc["vc"], hc["tables"], hc["lens"], hc["key"], hc["value"],
+                                                 None, 1, False, False, ctypes.byref(ws), ctypes.byref(six),
+                                                 ctx.ptr) == E["ERROR_INVALID_IN_TENSOR_NUM"]
+    lib.atb_c_destroy_operation(six)
+    nzload = ctypes.c_void_p()   # the fractal-NZ layout (kvCacheCfg 0) is not built
+    assert lib.AtbPagedCacheLoadGetWorkspaceSize(hc["kc"], hc["vc"], hc["tables"], hc["lens"], hc["key"], hc["value"],
+                                                 None, 0, False, False, ctypes.byref(ws), ctypes.byref(nzload),
+                                                 ctx.ptr) == E["ERROR_INVALID_PARAM"]
+    for h in list(handles.values()) + list(hc.values()):
+        lib.aclDestroyTensor(h)
+
+
 def test_cpp_api_symbols_are_exported(pkg):
     """The C++ entry points an ATB caller links against."""
     path = os.path.join(ROOT, "ascend-transformer-boost_amd", "lib", "libatb.so")
@@ -862,6 +928,8 @@ def test_cpp_api_symbols_are_exported(pkg):
         "atb::Utils::GetTensorSize(atb::TensorDesc const&)",
         "atb::Utils::GetTensorNumel(atb::Tensor const&)",
         "atb::Utils::GetAtbVersion",
+        "AtbMLAGetWorkspaceSize", "AtbMLA", "AtbPagedCacheLoadGetWorkspaceSize", "AtbPagedCacheLoad",
+        "aclCreateTensor", "aclDestroyTensor", "aclGetViewShape", "aclGetDataType", "aclGetFormat", "aclDataTypeSize",
     ]:
         assert needle in out, needle
 
