@@ -82,21 +82,22 @@ def test_quant_golden_dtype_exact_rational(oracle):
     for s in [np.float16(0.1), np.float16(0.337), np.float16(1.0), np.float16(3.0)]:
         got = oracle.quant_per_channel_golden_dtype(x, s, np.int8(5))
         for xi, gi in zip(x.tolist(), got.tolist()):
-            q = Fraction(xi) / Fraction(float(s))
-            h = nearest_fp16(q)
-            if not np.isfinite(h) or abs(q) >= 65520:
-                want = 127 if q > 0 else -128
-            else:
-                hf = Fraction(float(h))
-                r = math.floor(hf)
-                frac = hf - r
-                r = r + 1 if frac > Fraction(1, 2) or (frac == Fraction(1, 2) and r % 2 == 1) else r
-                want = max(-128, min(127, r + 5))
-            # (a quotient exactly between two fp16 values is the one case the neighbour search cannot order; skip it)
-            lo, hi = np.nextafter(h, np.float16(-np.inf)), np.nextafter(h, np.float16(np.inf))
-            if np.isfinite(lo) and np.isfinite(hi) and abs(Fraction(float(h)) - q) in (abs(Fraction(float(lo)) - q), abs(Fraction(float(hi)) - q)):
-                continue
-            assert gi == want, (xi, float(s), gi, want)
+          with np.errstate(over="ignore"):   # quotients past the fp16 range are meant to overflow here
+              q = Fraction(xi) / Fraction(float(s))
+              h = nearest_fp16(q)
+              if not np.isfinite(h) or abs(q) >= 65520:
+                  want = 127 if q > 0 else -128
+              else:
+                  hf = Fraction(float(h))
+                  r = math.floor(hf)
+                  frac = hf - r
+                  r = r + 1 if frac > Fraction(1, 2) or (frac == Fraction(1, 2) and r % 2 == 1) else r
+                  want = max(-128, min(127, r + 5))
+              # (a quotient exactly between two fp16 values is the one case the neighbour search cannot order; skip it)
+              lo, hi = np.nextafter(h, np.float16(-np.inf)), np.nextafter(h, np.float16(np.inf))
+              if np.isfinite(lo) and np.isfinite(hi) and abs(Fraction(float(h)) - q) in (abs(Fraction(float(lo)) - q), abs(Fraction(float(hi)) - q)):
+                  continue
+              assert gi == want, (xi, float(s), gi, want)
 
 
 # ---------------------------------------------------------------- dequant_per_channel
