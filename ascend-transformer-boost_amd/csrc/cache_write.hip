@@ -294,6 +294,31 @@ __device__ __forceinline__ int8_t QuantOne16(float x, float s, int32_t offset, b
     return static_cast<int8_t>(static_cast<int32_t>(r));
 }
 
+// The same result with the division replaced by a multiplication with y = RN(1 / s) and one correction step
+// (q = x y; r = x - s q exactly, by fused multiply-add; q' = q + r y): q' is the correctly rounded x / s
+// for finite non-zero s and 1 / s, because x and s carry at most 11 significant bits: q is within two
+// units of the quotient, the correction leaves an error below 2^-47 of it, and a quotient of two such
+// numbers that is not itself representable stays at least 2^-36 away from every rounding boundary.
+// Scales that are 0, infinite or NaN (special = true) take the division.
+__device__ __forceinline__ int8_t QuantOne16Fast(float x, float s, float y, float offset, bool special)
+{
+    float q;
+    if (__builtin_expect(special, 0)) {
+        q = __fdiv_rn(x, s);
+    } else {
+        const float q0 = __fmul_rn(x, y);
+        const float r = __fmaf_rn(-s, q0, x);
+        q = __fmaf_rn(r, y, q0);
+        q = fabsf(q0) < INFINITY ? q : q0; // x infinite or NaN: the product already is the answer
+    }
+    float v = rintf(HalfBitsToFloat(FloatToHalfBits(q)));
+    if (v != v) {
+        return 0;
+    }
+    v = fminf(fmaxf(v + offset, -128.0f), 127.0f);
+    return static_cast<int8_t>(static_cast<int32_t>(v));
+}
+
 __device__ __forceinline__ uint16_t DequantOne(int8_t x, float s, int32_t offset)
 {
     // The product is exact in fp32 (9 bits times 11). Its zero must keep the product's sign (0 * -s = -0
@@ -317,15 +342,26 @@ __global__ __launch_bounds__(256) void ElewisePerChannelKernel(const void *__res
 {
     const bool bf16 = isBf16 != 0;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x * VEC;
+    // per-channel values of the thread's current 8 channels (VEC == 8): they are looked up again only when
+    // the channels change, which with the launcher's grid they do not
+    int64_t cached = -1;
+    float sf[8], inv[8], offF[8];
+    int8_t off[8];
+    bool special = false;
     for (int64_t i = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * VEC; i < total; i += stride) {
         const int64_t c = i % channels;
         if constexpr (VEC == 8) {
+          if (c != cached) {
+            cached = c;
             uint32_t sw[4] = {0u, 0u, 0u, 0u};
             if (channels > 1) {
                 const uint4 sv = *reinterpret_cast<const uint4 *>(scale + c);
                 sw[0] = sv.x; sw[1] = sv.y; sw[2] = sv.z; sw[3] = sv.w;
             }
-            int8_t off[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                off[e] = 0;
+            }
             if (offset) {
                 if (channels > 1) {
                     const uint2 ov = *reinterpret_cast<const uint2 *>(offset + c);
@@ -341,12 +377,18 @@ __global__ __launch_bounds__(256) void ElewisePerChannelKernel(const void *__res
                     }
                 }
             }
-            float sf[8];
+            special = false;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const uint16_t h = channels > 1 ? static_cast<uint16_t>(sw[e >> 1] >> (16 * (e & 1))) : scale[0];
                 sf[e] = bf16 ? Bf16ToFloat(h) : HalfBitsToFloat(h);
+                if constexpr (!DEQUANT) {
+                    inv[e] = __fdiv_rn(1.0f, sf[e]);
+                    offF[e] = static_cast<float>(off[e]);
+                    special = special || !(fabsf(inv[e]) < INFINITY) || inv[e] == 0.0f;
+                }
             }
+          }
             if constexpr (DEQUANT) {
                 const uint2 xv = *reinterpret_cast<const uint2 *>(static_cast<const int8_t *>(x) + i);
                 const uint32_t xw[2] = {xv.x, xv.y};
@@ -366,7 +408,7 @@ __global__ __launch_bounds__(256) void ElewisePerChannelKernel(const void *__res
                 for (int e = 0; e < 8; ++e) {
                     const uint16_t h = static_cast<uint16_t>(xw[e >> 1] >> (16 * (e & 1)));
                     const float xf = bf16 ? Bf16ToFloat(h) : HalfBitsToFloat(h);
-                    const uint32_t q = static_cast<uint8_t>(QuantOne16(xf, sf[e], off[e], bf16));
+                    const uint32_t q = static_cast<uint8_t>(QuantOne16Fast(xf, sf[e], inv[e], offF[e], special));
                     o[e >> 2] |= q << (8 * (e & 3));
                 }
                 *reinterpret_cast<uint2 *>(static_cast<int8_t *>(out) + i) = uint2{o[0], o[1]};
@@ -598,7 +640,24 @@ int LaunchElewisePerChannel(const char *what, const void *x, const void *scale, 
     const bool wide = total % 8 == 0 && (channels == 1 || channels % 8 == 0) && Aligned(x, 16) && Aligned(out, 16) &&
                       Aligned(scale, 16) && (!offset || Aligned(offset, 8));
     const int64_t items = wide ? total / 8 : total;
-    const unsigned grid = static_cast<unsigned>(std::min<int64_t>((items + 255) / 256, 1 << 20));
+    int64_t blocks = std::min<int64_t>((items + 255) / 256, 1 << 20);
+    if (wide && channels > 1) {
+        // A thread keeps its 8 channels while it walks the rows if the launch's stride (blocks * 2048 elements)
+        // is a multiple of the channel count: round the grid to the next multiple that makes it one, unless
+        // that would leave most of it idle.
+        int64_t a = channels, b = 2048;
+        while (b != 0) {
+            const int64_t t = a % b;
+            a = b;
+            b = t;
+        }
+        const int64_t unit = channels / a; // blocks must be a multiple of this
+        if (unit <= blocks) {
+            blocks = blocks / unit * unit;
+            blocks = std::min<int64_t>(blocks, std::max<int64_t>(unit, 2048 / unit * unit));
+        }
+    }
+    const unsigned grid = static_cast<unsigned>(blocks);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (wide) {
         ElewisePerChannelKernel<8, DEQUANT><<<grid, 256, 0, s>>>(x, static_cast<const uint16_t *>(scale), offset, out, total,

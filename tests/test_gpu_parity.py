@@ -229,6 +229,29 @@ def test_elewise_quant_per_channel_bit_exact(binding, oracle, dev, stream):
     ctx.close()
 
 
+def test_elewise_quant_special_scales_and_inputs(binding, oracle, dev, stream):
+    """Scales of 0, infinity, NaN, the smallest subnormal and the largest fp16 beside ordinary ones, and x with
+    infinities, NaN and signed zeros: the multiply-and-correct path of the quantiser must hand these to the
+    plain division and agree with the golden (NaN quantises to 0)."""
+    ctx = binding.Context(stream)
+    runner = binding.OperationRunner("ElewiseOperation", binding.ElewiseParam(elewiseType=17), ctx)
+    special = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 6e-8, 65504.0, 1.0, 0.5, 3.0, -2.0, 0.33, 1e-3, 100.0, 7.0, 0.1],
+                       dtype=np.float16)
+    xs = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 6e-8, -6e-8, 65504.0, -65504.0, 1.0, -1.0, 0.5, 1.5, 2.5, -2.5, 126.5],
+                  dtype=np.float16)
+    x = torch.from_numpy(np.repeat(xs[:, None], 16, axis=1).copy())        # row = x value, column = scale
+    with np.errstate(all="ignore"):
+        want = oracle.quant_per_channel_golden_dtype(x.numpy(), special, np.zeros(16, np.int8))
+    with torch.cuda.stream(stream):
+        keep = [x.to(dev), torch.from_numpy(special).to(dev), torch.zeros(16, dtype=torch.int8, device=dev)]
+        out = torch.empty(x.shape, dtype=torch.int8, device=dev)
+        runner.run(keep, outputs=[out])
+    stream.synchronize()
+    assert np.array_equal(out.cpu().numpy(), want), (out.cpu().numpy(), want)
+    runner.close()
+    ctx.close()
+
+
 def test_elewise_dequant_per_channel_bit_exact(binding, oracle, dev, stream):
     """ELEWISE_DEQUANT_PER_CHANNEL against the reference golden, bit-exact: every int8 value against every
     offset for a set of scales that includes the saturating ones, and the shapes of the reference's tests."""
