@@ -100,23 +100,57 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaA
     const int count = wrLast - wrFirst + 1;
     auto rowOf = [&](int k) { return k == 0 ? ph0 : phEven + k * stride; };
 
-    float mx = -INFINITY;
-    for (int k = 0; k < count; ++k) {
-        mx = fmaxf(mx, a.partLse[rowOf(k)]);
-    }
     const int g = h / a.groupSize;
     const bool bf16 = a.qIsBf16 != 0;
     const int64_t outRow = static_cast<int64_t>(sq.qRow + tok) * a.H + h;
+    // Rows of up to MAX_HELD ranges (nearly all): the log-sum-exps and the thread's pieces of the partial
+    // rows are requested together and held in registers, one memory round trip; longer rows take the
+    // log-sum-exps first and the pieces in a second pass.
+    constexpr int MAX_HELD = 8;
+    const bool held = count <= MAX_HELD;
+    float lseHeld[MAX_HELD];
+    float mx = -INFINITY;
+    if (!held) {
+        for (int k = 0; k < count; ++k) {
+            mx = fmaxf(mx, a.partLse[rowOf(k)]);
+        }
+    }
     for (int c4 = vecs >= REDUCE_THREADS ? tid : tid % vecs; c4 < vecs; c4 += REDUCE_THREADS) {
         ReduceF4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
         float sum = 0.0f;
+        if (held) {
+            ReduceF4 piece[MAX_HELD];
+#pragma unroll
+            for (int k = 0; k < MAX_HELD; ++k) {
+                lseHeld[k] = -INFINITY;
+                piece[k] = ReduceF4{0.0f, 0.0f, 0.0f, 0.0f};
+                if (k < count) {
+                    const int64_t ph = rowOf(k);
+                    lseHeld[k] = a.partLse[ph];
+                    piece[k] = *reinterpret_cast<const ReduceF4 *>(a.partO + ph * a.Dv + c4 * 4);
+                }
+            }
+            mx = -INFINITY;
+#pragma unroll
+            for (int k = 0; k < MAX_HELD; ++k) {
+                mx = fmaxf(mx, lseHeld[k]);
+            }
+#pragma unroll
+            for (int k = 0; k < MAX_HELD; ++k) {
+                // a range that a -inf mask emptied (and a slot past the row's ranges) weighs nothing
+                const float w = lseHeld[k] == -INFINITY ? 0.0f : exp2f(lseHeld[k] - mx);
+                sum += w;
+                acc += w * piece[k];
+            }
+        } else {
 #pragma unroll 4
-        for (int k = 0; k < count; ++k) {
-            const int64_t ph = rowOf(k);
-            const float lse = a.partLse[ph];
-            const float w = lse == -INFINITY ? 0.0f : exp2f(lse - mx); // a range a -inf mask emptied weighs nothing
-            sum += w;
-            acc += w * *reinterpret_cast<const ReduceF4 *>(a.partO + ph * a.Dv + c4 * 4);
+            for (int k = 0; k < count; ++k) {
+                const int64_t ph = rowOf(k);
+                const float lse = a.partLse[ph];
+                const float w = lse == -INFINITY ? 0.0f : exp2f(lse - mx); // a range a -inf mask emptied weighs nothing
+                sum += w;
+                acc += w * *reinterpret_cast<const ReduceF4 *>(a.partO + ph * a.Dv + c4 * 4);
+            }
         }
         const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
         float o[4] = {acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv};
