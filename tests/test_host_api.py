@@ -911,6 +911,21 @@ def test_acl_tensor_handle_and_two_call_wrappers(binding, ctx):
         lib.aclDestroyTensor(h)
 
 
+def test_cpp_caller_builds_and_runs_against_the_public_headers(pkg, tmp_path):
+    """tests/cpp/atb_caller.cpp uses nothing but atb/atb_infer.h, the way a caller of the reference does
+    (context, CreateOperation, InferShape, Setup, the error paths); it is compiled with the host compiler
+    against include/ and the built libraries and run on the CPU."""
+    lib_dir = os.path.join(ROOT, "ascend-transformer-boost_amd", "lib")
+    exe = str(tmp_path / "atb_caller")
+    build = subprocess.run(["g++", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-I" + os.path.join(ROOT, "include"),
+                            os.path.join(HERE, "cpp", "atb_caller.cpp"), "-o", exe, "-L" + lib_dir, "-latb",
+                            "-latbmi_kernels", "-Wl,-rpath," + lib_dir], stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                           text=True)
+    assert build.returncode == 0, build.stdout
+    run = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=60)
+    assert run.returncode == 0 and run.stdout.strip().endswith("ok"), run.stdout + run.stderr
+
+
 def test_cpp_api_symbols_are_exported(pkg):
     """The C++ entry points an ATB caller links against."""
     path = os.path.join(ROOT, "ascend-transformer-boost_amd", "lib", "libatb.so")
