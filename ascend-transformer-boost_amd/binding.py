@@ -176,6 +176,7 @@ class AtbmiPaShape(ctypes.Structure):
         ("qScale", ctypes.c_float), ("maskBatchStride", ctypes.c_int64), ("maskHeadStride", ctypes.c_int64),
         ("maskLen", ctypes.c_int32), ("hasLogN", ctypes.c_int32),
         ("descalePacked", ctypes.c_int32), ("maskRowBy", ctypes.c_int32), ("ropeDim", ctypes.c_int32),
+        ("kvLayout", ctypes.c_int32),
     ]
 
 

@@ -71,9 +71,13 @@ struct PaArgs {
     int32_t groupSize; // H / G
     float qkScale;
     float qScale; // 0 when unused
-    int64_t kRowStride; // elements between consecutive tokens in the key cache (G*D)
-    int64_t vRowStride; // same for the value cache (G*Dv, or G*D when V aliases K)
-    int32_t vHeadStride; // elements between KV heads inside a value row (Dv, or D when V aliases K)
+    // Element (slot r, head g, channel c) of a cache sits at r * rowStride + g * headStride + c, where the
+    // slot of token `off` of block `blk` is blk * blockRows + off. Token-major blocks [blockSize][G][D]:
+    // rowStride G*D, headStride D, blockRows blockSize. Head-major blocks [G][blockSize][D]: rowStride D,
+    // headStride blockSize*D, blockRows G*blockSize.
+    int64_t kRowStride; // key cache
+    int64_t vRowStride; // value cache (the key cache's when V aliases K)
+    int32_t vHeadStride; // value cache (D - ropeDim when V aliases K)
     int32_t finishV;     // 1: partial outputs are still in int8 units; the final write applies vScale/vOff
     // Additive score bias (null: none), in the query's type: the score of the sequence in batch row b,
     // head h, token t gets mask[b * maskBatchStride + h * maskHeadStride + t] added after scaling.
@@ -92,6 +96,8 @@ struct PaArgs {
     const void *kRope;
     int64_t ropeRowStride; // elements between consecutive tokens in kRope (G * ropeDim)
     int32_t ropeDim;
+    int32_t blockRows;   // cache slots per block (see kRowStride)
+    int32_t kHeadStride; // elements between the KV heads of one key-cache slot (see kRowStride)
     int32_t pad0;
     void *lse;           // [rows][H] in the query's type: natural-log log-sum-exp of the scaled scores (null: none)
 };

@@ -162,6 +162,19 @@ extern "C" int atbmi_pa_plan_create(const AtbmiPaShape *shape, AtbmiPaPlan **pla
                                        "combined cache, got ropeDim %d with head sizes %d / %d", s.ropeDim, s.headDimK,
                     s.headDimV);
     }
+    if (s.kvLayout != ATBMI_PA_KV_TOKEN_MAJOR && s.kvLayout != ATBMI_PA_KV_HEAD_MAJOR) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: kvLayout %d", s.kvLayout);
+    }
+    if (s.kvLayout == ATBMI_PA_KV_HEAD_MAJOR) {
+        if (s.mlaCombined) {
+            return Fail(ERR_INVALID_PARAM, "pa_plan_create: a combined cache has one head; head-major blocks do not apply");
+        }
+        // the kernels keep a lane's offset inside one block in 32 bits
+        const int64_t width = s.headDimK > s.headDimV ? s.headDimK : s.headDimV;
+        if (static_cast<int64_t>(s.numKvHeads) * s.blockSize * width * 2 > 0x7fffffffLL) {
+            return Fail(ERR_INVALID_PARAM, "pa_plan_create: a head-major cache block exceeds 2 GiB");
+        }
+    }
     if (s.hasMask && (s.maskLen <= 0 || s.maskBatchStride < 0 || s.maskHeadStride < 0)) {
         return Fail(ERR_INVALID_PARAM, "pa_plan_create: mask row length %d, strides %lld / %lld", s.maskLen,
                     (long long)s.maskBatchStride, (long long)s.maskHeadStride);
@@ -664,9 +677,19 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
     a.groupSize = s.numHeads / s.numKvHeads;
     a.qkScale = s.qkScale;
     a.qScale = (s.qScale == 0.0f || s.qScale == 1.0f) ? 0.0f : s.qScale;
-    a.kRowStride = static_cast<int64_t>(s.numKvHeads) * (s.headDimK - s.ropeDim);
-    a.vRowStride = s.mlaCombined ? a.kRowStride : static_cast<int64_t>(s.numKvHeads) * s.headDimV;
-    a.vHeadStride = s.mlaCombined ? s.headDimK - s.ropeDim : s.headDimV;
+    if (s.kvLayout == ATBMI_PA_KV_HEAD_MAJOR) {
+        a.blockRows = s.blockSize * s.numKvHeads;
+        a.kRowStride = s.headDimK;
+        a.kHeadStride = s.blockSize * s.headDimK;
+        a.vRowStride = s.headDimV;
+        a.vHeadStride = s.blockSize * s.headDimV;
+    } else {
+        a.blockRows = s.blockSize;
+        a.kRowStride = static_cast<int64_t>(s.numKvHeads) * (s.headDimK - s.ropeDim);
+        a.kHeadStride = s.headDimK - s.ropeDim;
+        a.vRowStride = s.mlaCombined ? a.kRowStride : static_cast<int64_t>(s.numKvHeads) * s.headDimV;
+        a.vHeadStride = s.mlaCombined ? s.headDimK - s.ropeDim : s.headDimV;
+    }
     a.finishV = (plan->useMfma && s.kvDtype == ATBMI_INT8) ? 1 : 0;
     if (s.hasMask) {
         a.mask = t->mask;

@@ -239,7 +239,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
         if (MLA && col >= nopePieces) {
             return krBase + (r * a.ropeRowStride + static_cast<int64_t>(g) * a.ropeDim) * 2 + (col - nopePieces) * 16;
         }
-        return kcBase + (r * a.kRowStride + static_cast<int64_t>(g) * dn) * ESZ + col * 16;
+        return kcBase + (r * a.kRowStride + static_cast<int64_t>(g) * a.kHeadStride) * ESZ + col * 16;
     };
     constexpr float LOG2E = 1.4426950408889634f;
     const float scale2 = a.qkScale * LOG2E;
@@ -350,7 +350,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
         int curBlk = cacheBase;
         int curOff = tokBegin % a.blockSize;
 
-        // Cache row index (rows = [slot][head][channel]) of the next two sub-tiles; advances the cursor.
+        // Cache slot of the first token of the next two sub-tiles; advances the cursor.
         auto nextRows = [&](int64_t *rowBase) {
 #pragma unroll
             for (int sub = 0; sub < 2; ++sub) {
@@ -359,7 +359,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                     blkCache = (cacheBase + lane < blocksNeeded) ? table[cacheBase + lane] : 0;
                 }
                 const int blk = __builtin_amdgcn_readlane(blkCache, curBlk - cacheBase);
-                rowBase[sub] = static_cast<int64_t>(blk) * a.blockSize + curOff;
+                rowBase[sub] = static_cast<int64_t>(blk) * a.blockRows + curOff;
                 curOff += 16;
                 if (curOff >= a.blockSize) {
                     curOff = 0;
@@ -377,7 +377,8 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
         constexpr int K_RPL = K_UNIFORM ? WAVE / KPR : 1; // rows per load
         constexpr int V_RPL = V_UNIFORM ? WAVE / VPR : 1;
         const uint32_t laneOffK = static_cast<uint32_t>(
-            (static_cast<int64_t>(lane / KPR) * a.kRowStride + static_cast<int64_t>(g) * D) * ESZ + (lane % KPR) * 16);
+            (static_cast<int64_t>(lane / KPR) * a.kRowStride + static_cast<int64_t>(g) * a.kHeadStride) * ESZ +
+            (lane % KPR) * 16);
         const uint32_t laneOffV = static_cast<uint32_t>(
             (static_cast<int64_t>(lane / VPR) * a.vRowStride + static_cast<int64_t>(g) * a.vHeadStride) * ESZ +
             (lane % VPR) * 16);

@@ -98,8 +98,8 @@ __global__ __launch_bounds__(PA_SCALAR_WAVES * WAVE) void PaScalarKernel(const P
 
     const int32_t *table = a.tables + static_cast<int64_t>(it.seq) * a.maxBlocksPerSeq;
     for (int t = it.tokBegin + wave; t < it.tokEnd; t += PA_SCALAR_WAVES) {
-        const int64_t row = static_cast<int64_t>(table[t / a.blockSize]) * a.blockSize + (t % a.blockSize);
-        const int64_t kBase = row * a.kRowStride + static_cast<int64_t>(g) * dn;
+        const int64_t row = static_cast<int64_t>(table[t / a.blockSize]) * a.blockRows + (t % a.blockSize);
+        const int64_t kBase = row * a.kRowStride + static_cast<int64_t>(g) * a.kHeadStride;
         const int64_t rBase = row * a.ropeRowStride + static_cast<int64_t>(g) * a.ropeDim - dn;
         const int64_t vBase = row * a.vRowStride + static_cast<int64_t>(g) * a.vHeadStride;
         float k[EPL], v[EPL];

@@ -145,8 +145,6 @@ bool ImplementedCheck(const Param &p)
         what = "MASK_TYPE_SPEC without CALC_TYPE_SPEC";
     } else if (p.compressType != Param::COMPRESS_TYPE_UNDEFINED) {
         what = "head compression";
-    } else if (p.inputLayout != infer::TYPE_BSND) {
-        what = "BNSD layout";
     } else if (p.quantType == Param::TYPE_QUANT_QKV_OFFLINE || p.quantType == Param::TYPE_QUANT_QKV_ONLINE) {
         what = "int8 query quantisation";
     } else if (p.quantType != Param::TYPE_QUANT_UNQUANT && p.quantType != Param::TYPE_DEQUANT_FUSION) {
@@ -217,7 +215,8 @@ class PagedAttentionOperation : public OperationBase {
 public:
     explicit PagedAttentionOperation(const Param &param)
         : OperationBase("PagedAttentionOperation"), param_(param), mla_(param.mlaVHeadSize > 0),
-          dequant_(param.quantType == Param::TYPE_DEQUANT_FUSION), irTable_(MakeIr(param))
+          dequant_(param.quantType == Param::TYPE_DEQUANT_FUSION), bnsd_(param.inputLayout == infer::TYPE_BNSD),
+          irTable_(MakeIr(param))
     {
         ir_ = &irTable_;
         tablesIdx_ = mla_ ? 2 : 3;
@@ -271,6 +270,9 @@ protected:
     // Reference :697-726 (InferShapeDimCheck) + :634-661 (KVCacheDimCheck).
     Status InferShapeCheckImpl(const SVector<TensorDesc> &in) const override
     {
+        if (bnsd_) {
+            return BnsdDimCheck(in);
+        }
         if (!mla_ && in.at(2).shape.dimNum != 4) {
             ATB_LOG(ERROR) << "valueCache should have 4 dims";
             return ERROR_INVALID_TENSOR_DIM_NUM;
@@ -320,6 +322,9 @@ protected:
             ATB_LOG(ERROR) << "head size of the output should be " << dv;
             return ERROR_INVALID_TENSOR_DIM;
         }
+        if (bnsd_) {
+            return NO_ERROR; // reference :965-994 (SetupDimCheckBNSD910B) stops here
+        }
         if (in.at(0).shape.dims[1] != out.dims[1]) {
             ATB_LOG(ERROR) << "query and output must have the same head count";
             return ERROR_INVALID_TENSOR_DIM;
@@ -361,14 +366,15 @@ protected:
         const int64_t kvHeads = param_.kvHeadNum > 0 ? param_.kvHeadNum : param_.headNum;
         const int64_t d = kc.desc.shape.dims[3];
         const int64_t dv = mla_ ? static_cast<int64_t>(param_.mlaVHeadSize) : pack.inTensors.at(2).desc.shape.dims[3];
-        const int64_t blockSize = kc.desc.shape.dims[1];
+        const int64_t blockSize = kc.desc.shape.dims[bnsd_ ? 2 : 1];
         // Kernel-library level checks of the reference.
         if (q.desc.shape.dims[1] != param_.headNum) {
             ATB_LOG(ERROR) << "query head count " << q.desc.shape.dims[1] << " != headNum " << param_.headNum;
             return ERROR_INVALID_PARAM;
         }
-        if (kc.desc.shape.dims[2] != kvHeads) {
-            ATB_LOG(ERROR) << "cache head count " << kc.desc.shape.dims[2] << " != kvHeadNum " << kvHeads;
+        const int64_t cacheHeads = kc.desc.shape.dims[bnsd_ ? 1 : 2];
+        if (cacheHeads != kvHeads || (bnsd_ && pack.inTensors.at(2).desc.shape.dims[1] != kvHeads)) {
+            ATB_LOG(ERROR) << "cache head count " << cacheHeads << " != kvHeadNum " << kvHeads;
             return ERROR_INVALID_PARAM;
         }
         if (blockSize % 16 != 0) {
@@ -393,8 +399,8 @@ protected:
             ATB_LOG(ERROR) << "blockTables has fewer rows than contextLens";
             return ERROR_INVALID_PARAM;
         }
-        if (out.desc.shape.dims[0] != q.desc.shape.dims[0]) {
-            ATB_LOG(ERROR) << "output and query must have the same token count";
+        if (out.desc.shape.dims[0] != q.desc.shape.dims[0] || out.desc.shape.dims[1] != q.desc.shape.dims[1]) {
+            ATB_LOG(ERROR) << "output and query must have the same token and head counts";
             return ERROR_INVALID_PARAM;
         }
         if (dequant_) {
@@ -470,6 +476,7 @@ protected:
         shape.maskLen = static_cast<int32_t>(maskLen);
         shape.maskRowBy = maskRowBy;
         shape.hasLogN = logNIdx_ != NONE ? 1 : 0;
+        shape.kvLayout = bnsd_ ? ATBMI_PA_KV_HEAD_MAJOR : ATBMI_PA_KV_TOKEN_MAJOR;
         shape.descalePacked = (dequant_ && pack.inTensors.at(kScaleIdx_).desc.dtype == ACL_INT64) ? 1 : 0;
         if (!plan_ || !SameShape(shape, planShape_)) {
             if (plan_) {
@@ -534,7 +541,7 @@ private:
                a.qkScale == b.qkScale && a.qScale == b.qScale && a.hasMask == b.hasMask &&
                a.maskBatchStride == b.maskBatchStride && a.maskHeadStride == b.maskHeadStride &&
                a.maskLen == b.maskLen && a.hasLogN == b.hasLogN && a.descalePacked == b.descalePacked &&
-               a.maskRowBy == b.maskRowBy;
+               a.maskRowBy == b.maskRowBy && a.kvLayout == b.kvLayout;
     }
 
     // Element strides of the additive mask, as the reference derives them from
@@ -608,6 +615,30 @@ private:
         return NO_ERROR;
     }
 
+    // Reference :697-726 (InferShapeDimCheckBNSD910B): caches [numBlocks, kvHeads, blockSize, headSize].
+    Status BnsdDimCheck(const SVector<TensorDesc> &in) const
+    {
+        if (in.at(0).shape.dimNum != 3 || in.at(1).shape.dimNum != 4 || in.at(2).shape.dimNum != 4 ||
+            in.at(3).shape.dimNum != 2 || in.at(4).shape.dimNum != 1) {
+            ATB_LOG(ERROR) << "expected dims: query 3, keyCache 4, valueCache 4, blockTables 2, contextLens 1";
+            return ERROR_INVALID_TENSOR_DIM_NUM;
+        }
+        const int64_t headSize = in.at(0).shape.dims[2];
+        if (headSize != in.at(1).shape.dims[3] || headSize != in.at(2).shape.dims[3]) {
+            ATB_LOG(ERROR) << "headSize of query, keyCache and valueCache should be same";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (in.at(1).shape.dims[0] != in.at(2).shape.dims[0]) {
+            ATB_LOG(ERROR) << "numBlocks of keyCache and valueCache should be same";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (in.at(1).shape.dims[2] != in.at(2).shape.dims[2]) {
+            ATB_LOG(ERROR) << "blockSize of keyCache and valueCache should be same";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        return NO_ERROR;
+    }
+
     // Reference :585-632 (KVCacheDimCheck910B) with :561-572 (IsInMLAIncompatible).
     Status CacheDimCheck(const SVector<TensorDesc> &in) const
     {
@@ -660,6 +691,7 @@ private:
     Param param_;
     bool mla_;
     bool dequant_;
+    bool bnsd_;
     OpIr irTable_;
     static constexpr size_t NONE = ~static_cast<size_t>(0);
     size_t tablesIdx_ = 3;

@@ -15,7 +15,7 @@ namespace infer {
 
 enum InputLayout : int {
     TYPE_BSND = 0, // [tokens, heads, head_dim] queries, [blocks, block, heads, dim] caches
-    TYPE_BNSD      // head-major caches; not implemented on MI355X
+    TYPE_BNSD      // head-major caches [numBlocks, kvHeads, blockSize, headSize]
 };
 
 // Writes one K row and one V row per token into the paged caches at the

@@ -205,6 +205,15 @@ typedef enum AtbmiPaMaskRow {
     ATBMI_PA_MASK_ROW_POSITION = 2
 } AtbmiPaMaskRow;
 
+/* Order of the dimensions inside one cache block (reference include/atb/infer_op_params.h, InputLayout):
+ *   TOKEN_MAJOR  [numBlocks, blockSize, G, D]  TYPE_BSND
+ *   HEAD_MAJOR   [numBlocks, G, blockSize, D]  TYPE_BNSD (PagedAttentionParam::inputLayout; 16-bit
+ *                caches with separate key and value caches only) */
+typedef enum AtbmiPaKvLayout {
+    ATBMI_PA_KV_TOKEN_MAJOR = 0,
+    ATBMI_PA_KV_HEAD_MAJOR = 1
+} AtbmiPaKvLayout;
+
 typedef struct AtbmiPaShape {
     int32_t qDtype;          /* ATBMI_F16 or ATBMI_BF16; the output has the same type */
     int32_t kvDtype;         /* ATBMI_F16 / ATBMI_BF16 (== qDtype) or ATBMI_INT8 */
@@ -233,12 +242,13 @@ typedef struct AtbmiPaShape {
                                 MultiLatentAttentionParam::KROPE_CTKV (reference include/atb/infer_op_params.h:2949-2958):
                                 query and keyCache hold rows of headDimK - ropeDim channels, queryRope and
                                 keyRopeCache the remaining ropeDim channels of the same rows */
+    int32_t kvLayout;        /* AtbmiPaKvLayout of keyCache and valueCache */
 } AtbmiPaShape;
 
 /* Device tensors of one decode call.
  *   query       [numQueryRows, H, D]                qDtype
- *   keyCache    [numBlocks, blockSize, G, D]        kvDtype
- *   valueCache  [numBlocks, blockSize, G, Dv]       kvDtype (NULL when mlaCombined)
+ *   keyCache    [numBlocks, blockSize, G, D]        kvDtype ([numBlocks, G, blockSize, D] when head-major)
+ *   valueCache  [numBlocks, blockSize, G, Dv]       kvDtype (NULL when mlaCombined; head-major like keyCache)
  *   blockTables [batch, maxBlocksPerSeq]            int32
  *   kScale/vScale [G*D] / [G*Dv] fp32 (or uint64-packed fp32, see descalePacked), kOffset/vOffset same
  *               length int32 (int8 KV only)

@@ -328,7 +328,7 @@ def norm_mask(batch, max_len, value=-10000.0):
 def paged_attention(query, key_cache, value_cache, block_tables, context_lens, scale, k_descale=None,
                     k_offset=None, v_descale=None, v_offset=None, mla_v_head_size=0, q_scale=0.0,
                     q_dtype="float32", out_init=0.0, mask=None, logn=None, mask_per_head=None, q_lens=None,
-                    mask_rows="sequence", lse_out=None):
+                    mask_rows="sequence", lse_out=None, head_major=False):
     """Decode attention over paged caches.
 
     query [rows, heads, D] float32; key_cache [blocks, block, kv_heads, D];
@@ -356,8 +356,16 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, s
     512 + 64 channels in two tensors) is the same computation on the rows
     concatenated along the channel axis, which is what the reference golden
     does the other way round (it splits the concatenated tensors).
+    head_major: the caches are [blocks, kv_heads, block, D] (InputLayout TYPE_BNSD);
+    the reference golden computes on the token-major cache and hands the
+    operation its (0, 2, 1, 3) permutation
+    (tests/apitest/opstest/python/operations/paged_attention/test_paged_attention_operation_BNSD.py:369-373),
+    so this is the same computation after permuting back.
     Returns float32 [rows, heads, Dv]."""
     query = np.asarray(query, dtype=np.float32)
+    if head_major:
+        key_cache = np.transpose(key_cache, (0, 2, 1, 3))
+        value_cache = None if value_cache is None else np.transpose(value_cache, (0, 2, 1, 3))
     if mla_v_head_size > 0:
         dv = mla_v_head_size
     else:

@@ -23,7 +23,7 @@ def dtype_code(binding, t):
 def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=None, v_scale=None,
                    v_off=None, mla_dv=0, q_scale=0.0, kernel=0, chunk_tokens=None, out=None, return_plan_info=False,
                    mask=None, mask_per_head=False, logn=None, q_lens=None, mask_rows="sequence", q_rope=None,
-                   k_rope=None, lse=None):
+                   k_rope=None, lse=None, head_major=False):
     """atbmi_pa_plan_* + atbmi_pa_decode on `stream`; returns the output tensor.
     mask: device tensor of q's dtype shaped like one of the reference's decode
     masks; mask_per_head says that a 3-dim mask's first dim counts heads (ALIBI).
@@ -38,8 +38,9 @@ def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=
     if mask_rows != "sequence":
         mask_batch_stride, mask_head_stride = (mask.shape[1], 0) if mask is not None else (0, 0)
     shape = binding.AtbmiPaShape(
-        qDtype=dtype_code(binding, q), kvDtype=dtype_code(binding, kc), numHeads=heads, numKvHeads=kc.shape[2],
-        headDimK=d, headDimV=dv, blockSize=kc.shape[1], numBlocks=kc.shape[0], maxBlocksPerSeq=tables.shape[1],
+        qDtype=dtype_code(binding, q), kvDtype=dtype_code(binding, kc), numHeads=heads,
+        numKvHeads=kc.shape[1 if head_major else 2], kvLayout=1 if head_major else 0,
+        headDimK=d, headDimV=dv, blockSize=kc.shape[2 if head_major else 1], numBlocks=kc.shape[0], maxBlocksPerSeq=tables.shape[1],
         numQueryRows=rows, mlaCombined=1 if mla_dv else 0, hasOffset=1 if k_off is not None else 0, kernel=kernel,
         qkScale=scale, qScale=q_scale, hasMask=0 if mask is None else 1, maskBatchStride=mask_batch_stride,
         maskHeadStride=mask_head_stride, maskLen=0 if mask is None else mask.shape[-1],
@@ -123,14 +124,14 @@ def mask_strides(mask, per_head):
 
 def oracle_pa(oracle, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=None, v_scale=None, v_off=None,
               mla_dv=0, q_scale=0.0, out_init=0.0, mask=None, mask_per_head=False, logn=None, q_lens=None,
-              mask_rows="sequence", lse_out=None):
+              mask_rows="sequence", lse_out=None, head_major=False):
     qd = "bf16" if q.dtype == torch.bfloat16 else "float16"
     return oracle.paged_attention(
         to_oracle(q), to_oracle(kc), to_oracle(vc), tables.cpu().numpy(), np.asarray(ctx_host), scale,
         to_oracle(k_scale), to_oracle(k_off), to_oracle(v_scale), to_oracle(v_off), mla_v_head_size=mla_dv,
         q_scale=q_scale, q_dtype=qd, out_init=out_init, mask=to_oracle(mask), logn=to_oracle(logn),
         mask_per_head=mask_per_head if (mask is not None and mask.dim() == 3) else None, q_lens=q_lens,
-        mask_rows=mask_rows, lse_out=lse_out)
+        mask_rows=mask_rows, lse_out=lse_out, head_major=head_major)
 
 
 def assert_close(got, want, tol, what=""):

@@ -681,6 +681,70 @@ def test_paged_attention_matrix(binding, oracle, dev, stream, case):
         assert_close(got, want, TOL[dtype], "kernel=%d" % kernel)
 
 
+# batch, heads, kv_heads, block, d, ctx, dtype, mask kind
+HEAD_MAJOR_MATRIX = [
+    (16, 40, 10, 128, 128, 3000, torch.bfloat16, "norm3"),  # reference test_paged_attention_operation_BNSD.py:392-405
+    (4, 32, 16, 64, 128, [100, 2000, 64, 777], torch.float16, None),  # the reference table's PagedAttentionBNSD row
+    (5, 8, 8, 16, 64, [819, 12, 4000, 256, 300], torch.float16, "alibi4"),
+    (3, 12, 1, 128, 256, [700, 1, 5000], torch.bfloat16, None),
+    (4, 30, 2, 32, 96, [88, 1500, 3, 640], torch.float16, None),
+    (2, 9, 3, 16, 80, [300, 45], torch.float16, None),
+]
+
+
+@pytest.mark.parametrize("case", HEAD_MAJOR_MATRIX, ids=lambda c: "b%d_h%d_g%d_bs%d_d%d_%s_%s" % (
+    c[0], c[1], c[2], c[3], c[4], str(c[6]).split(".")[-1], c[7]))
+def test_paged_attention_head_major_blocks(binding, oracle, dev, stream, case):
+    """InputLayout TYPE_BNSD: caches [numBlocks, kvHeads, blockSize, headSize]. Against the oracle, and
+    bit for bit against the same kernel on the token-major cache (the rows and their order are the same)."""
+    batch, heads, kv_heads, block, d, ctx, dtype, kind = case
+    rng = _rng(700 + batch + heads)
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, batch, heads, kv_heads, block, d, d, ctx, dtype)
+    max_len = int(ctx.max())
+    mask, per_head = (None, False) if kind is None else _mask_tensor(oracle, rng, dev, kind, ctx, heads, max_len, dtype)
+    kc_hm = kc.permute(0, 2, 1, 3).contiguous()
+    vc_hm = vc.permute(0, 2, 1, 3).contiguous()
+    scale = 1.0 / math.sqrt(d)
+    want = oracle_pa(oracle, q, kc_hm, vc_hm, tables, ctx, scale, mask=mask, mask_per_head=per_head, head_major=True)
+    for kernel in _kernels_for(binding, d, d, block):
+        got = pa_decode_cabi(binding, stream, q, kc_hm, vc_hm, tables, ctx, scale, kernel=kernel, mask=mask,
+                             mask_per_head=per_head, head_major=True)
+        assert_close(got, want, TOL[dtype], "kernel=%d" % kernel)
+        same = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, kernel=kernel, mask=mask,
+                              mask_per_head=per_head)
+        assert torch.equal(_bits(got), _bits(same)), "kernel=%d differs from the token-major run" % kernel
+
+
+def test_head_major_blocks_through_operation_api(binding, oracle, dev, stream):
+    """PagedAttentionParam::inputLayout = TYPE_BNSD with and without a mask (reference
+    test_paged_attention_operation_BNSD.py:417-430: headNum 40, kvHeadNum 10, maskType 1, inputLayout 1)."""
+    rng = _rng(741)
+    heads, kv_heads, d, block = 40, 10, 128, 128
+    ctx = np.array([3000, 300, 17, 1024, 129], dtype=np.int32)
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, len(ctx), heads, kv_heads, block, d, d, ctx, torch.bfloat16)
+    kc_hm = kc.permute(0, 2, 1, 3).contiguous()
+    vc_hm = vc.permute(0, 2, 1, 3).contiguous()
+    lens = torch.from_numpy(ctx)
+    scale = 1.0 / math.sqrt(d)
+    c = binding.Context(stream)
+    mask, per_head = _mask_tensor(oracle, rng, dev, "norm3", ctx, heads, 3000, torch.bfloat16)
+    for mask_type, m in ((0, None), (1, mask)):
+        pa = binding.OperationRunner("PagedAttentionOperation", binding.PagedAttentionParam(
+            headNum=heads, kvHeadNum=kv_heads, qkScale=scale, maskType=mask_type, inputLayout=1), c)
+        ins = [q, kc_hm, vc_hm, tables, lens.to(dev)] + ([m] if m is not None else [])
+        with torch.cuda.stream(stream):
+            out, = pa.run(ins, host_inputs={4: lens})
+        stream.synchronize()
+        assert tuple(out.shape) == (5, heads, d)
+        want = oracle_pa(oracle, q, kc_hm, vc_hm, tables, ctx, scale, mask=m, mask_per_head=False, head_major=True)
+        assert_close(out, want, TOL[torch.bfloat16], "maskType=%d" % mask_type)
+        # the token-major reading of the same buffers is a different result
+        assert np.abs(oracle_pa(oracle, q, kc_hm.reshape(kc.shape), vc_hm.reshape(vc.shape), tables, ctx, scale, mask=m,
+                                mask_per_head=False) - want).max() > 1e-2
+        pa.close()
+    c.close()
+
+
 def test_c1_decode_step_through_operation_api(binding, oracle, pkg, dev, stream):
     """Benchmark configuration 1 end to end: ReshapeAndCache then PagedAttention
     through atb::Operation, fp16, rtol = atol = 1e-3."""

@@ -38,7 +38,7 @@ ELEWISE_CASES = _load("elewise")
 def _pa_unimplemented(p):
     """Features of PagedAttentionParam the reference accepts but this library rejects at creation."""
     return (p.get("maskType", 0) >= 4 or (p.get("maskType", 0) == 3 and p.get("calcType", 0) != 1) or
-            p.get("compressType", 0) != 0 or p.get("inputLayout", 0) != 0 or p.get("quantType", 0) >= 2)
+            p.get("compressType", 0) != 0 or p.get("quantType", 0) >= 2)
 
 
 def _pa_mask_shape_refused(case):
@@ -251,7 +251,7 @@ def test_table_coverage():
     pa_dev = [c for c in PA_CASES if (_pa_unimplemented(c["param"]) and not c["expected"].startswith("C:")) or
               _pa_mask_shape_refused(c)]
     rac_dev = [c for c in RAC_CASES if _rac_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
-    assert len(PA_CASES) == 81 and len(PA_CASES) - len(pa_dev) >= 72
+    assert len(PA_CASES) == 81 and len(PA_CASES) - len(pa_dev) >= 73
     assert len(RAC_CASES) == 38 and len(RAC_CASES) - len(rac_dev) >= 26
     # most MultiLatentAttention rows exercise the prefill calcType and the fractal-NZ caches, which are not built
     mla_dev = [c for c in MLA_CASES if _mla_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
@@ -630,6 +630,52 @@ def test_multi_latent_attention_counts_shapes_and_setup(binding, ctx):
     assert spec.setup(pack(rows=6, mask=[6, 300], with_qlens=True, qlens_host=False), outs(rows=6), ctx)[0] == \
         e["ERROR_INVALID_PARAM"]
     spec.close()
+
+
+def test_paged_attention_bnsd_checks(binding, ctx):
+    """inputLayout = TYPE_BNSD: caches [numBlocks, kvHeads, blockSize, headSize]. Parameter combinations
+    (reference paged_attention_operation.cpp:302-323), dim checks (:697-726, :965-994) and the head
+    counts, which the reference leaves to its kernel library."""
+    E = binding.ERROR_CODE
+    P = binding.PagedAttentionParam
+    base = dict(headNum=32, kvHeadNum=16, qkScale=0.088, inputLayout=1)
+    for extra in (dict(calcType=1), dict(compressType=1), dict(quantType=1), dict(scaleType=1),
+                  dict(mlaVHeadSize=512, kvHeadNum=1)):
+        assert binding.Operation("PagedAttentionOperation", P(**dict(base, **extra))).status == E["ERROR_INVALID_PARAM"]
+    lens = np.full((4,), 100, dtype=np.int32)
+    mk = binding.make_tensor
+
+    def pack(q=(4, 32, 128), kc=(9, 16, 64, 128), vc=(9, 16, 64, 128), tables=(4, 8), dtype="float16", mask=None):
+        t = [mk(dtype, q, FAKE_DEVICE), mk(dtype, kc, FAKE_DEVICE), mk(dtype, vc, FAKE_DEVICE),
+             mk("int32", tables, FAKE_DEVICE), mk("int32", (4,), FAKE_DEVICE, host_ptr=lens.ctypes.data)]
+        if mask:
+            t.append(mk(dtype, mask, FAKE_DEVICE))
+        return t
+
+    out = lambda shape=(4, 32, 128), dtype="float16": [mk(dtype, shape, FAKE_DEVICE)]
+    for mask_type, mask in ((0, None), (1, (4, 1, 512)), (2, (32, 1, 512))):
+        op = binding.Operation("PagedAttentionOperation", P(**dict(base, maskType=mask_type)))
+        assert op.status == 0
+        st, descs = op.infer_shape(pack(mask=mask))
+        assert st == 0 and [descs[0].dims[i] for i in range(3)] == [4, 32, 128]
+        assert op.setup(pack(mask=mask), out(), ctx)[0] == 0
+        assert op.setup(pack(mask=mask, dtype="bf16"), out(dtype="bf16"), ctx)[0] == 0
+        op.close()
+    op = binding.Operation("PagedAttentionOperation", P(**base))
+    assert op.infer_shape(pack(kc=(9, 16, 64)))[0] == E["ERROR_INVALID_TENSOR_DIM_NUM"]
+    assert op.infer_shape(pack(q=(4, 32 * 128)))[0] == E["ERROR_INVALID_TENSOR_DIM_NUM"]
+    assert op.infer_shape(pack(vc=(9, 16, 64, 64)))[0] == E["ERROR_INVALID_TENSOR_DIM"]    # head sizes
+    assert op.infer_shape(pack(q=(4, 32, 64)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.infer_shape(pack(vc=(8, 16, 64, 128)))[0] == E["ERROR_INVALID_TENSOR_DIM"]   # numBlocks
+    assert op.infer_shape(pack(vc=(9, 16, 32, 128)))[0] == E["ERROR_INVALID_TENSOR_DIM"]   # blockSize
+    assert op.setup(pack(), out((4, 32, 64)), ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    # what the reference's kernel library refuses: head counts of the caches and of the output
+    assert op.infer_shape(pack(kc=(9, 64, 16, 128), vc=(9, 64, 16, 128)))[0] == 0  # token-major caches fit the dim rules
+    assert op.setup(pack(kc=(9, 64, 16, 128), vc=(9, 64, 16, 128)), out(), ctx)[0] == E["ERROR_INVALID_PARAM"]
+    assert op.setup(pack(vc=(9, 8, 64, 128)), out(), ctx)[0] == E["ERROR_INVALID_PARAM"]
+    assert op.setup(pack(), out((4, 16, 128)), ctx)[0] == E["ERROR_INVALID_PARAM"]
+    assert op.setup(pack(kc=(9, 16, 24, 128), vc=(9, 16, 24, 128)), out(), ctx)[0] == E["ERROR_INVALID_PARAM"]  # 16-aligned
+    op.close()
 
 
 def test_reshape_and_cache_with_stride_checks(binding, ctx):

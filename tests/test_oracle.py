@@ -395,6 +395,37 @@ def test_attention_matches_independent_loops(oracle):
     np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-6)
 
 
+def test_attention_head_major_blocks_by_flat_addresses(oracle):
+    """TYPE_BNSD caches: element (block b, head g, offset o, channel c) sits at flat address
+    ((b * heads + g) * block + o) * D + c. The token-major cache is rebuilt from those addresses
+    one row at a time and run through the loop version."""
+    rng = _rng(23)
+    heads, kv_heads, d, dv, block, pool = 6, 3, 16, 8, 4, 19
+    ctx = np.array([9, 0, 4, 13], dtype=np.int32)
+    tables = rng.permutation(pool)[:16].reshape(4, 4).astype(np.int32)
+    q = rng.standard_normal((3, heads, d)).astype(np.float32)
+    kc_hm = rng.standard_normal((pool, kv_heads, block, d)).astype(np.float32)
+    vc_hm = rng.standard_normal((pool, kv_heads, block, dv)).astype(np.float32)
+
+    def token_major(hm, width):
+        flat = hm.ravel()
+        tm = np.empty((pool, block, kv_heads, width), dtype=np.float32)
+        for b in range(pool):
+            for o in range(block):
+                for g in range(kv_heads):
+                    at = ((b * kv_heads + g) * block + o) * width
+                    tm[b, o, g] = flat[at:at + width]
+        return tm
+
+    got = oracle.paged_attention(q, kc_hm, vc_hm, tables, ctx, 0.3, head_major=True)
+    want = oracle.paged_attention_loops(q, token_major(kc_hm, d), token_major(vc_hm, dv), tables, ctx, 0.3)
+    np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-6)
+    # and it is not the token-major reading of the same buffer
+    other = oracle.paged_attention(q, kc_hm.reshape(pool, block, kv_heads, d), vc_hm.reshape(pool, block, kv_heads, dv),
+                                   tables, ctx, 0.3)
+    assert np.abs(other - got).max() > 1e-2
+
+
 def test_attention_matches_torch_sdpa(oracle):
     """Gathering the rows densely reduces the op to textbook attention."""
     rng = _rng(3)
