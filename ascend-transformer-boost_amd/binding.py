@@ -176,14 +176,15 @@ class AtbmiPaShape(ctypes.Structure):
         ("qScale", ctypes.c_float), ("maskBatchStride", ctypes.c_int64), ("maskHeadStride", ctypes.c_int64),
         ("maskLen", ctypes.c_int32), ("hasLogN", ctypes.c_int32),
         ("descalePacked", ctypes.c_int32), ("maskRowBy", ctypes.c_int32), ("ropeDim", ctypes.c_int32),
-        ("kvLayout", ctypes.c_int32),
+        ("kvLayout", ctypes.c_int32), ("maskSeqDiv", ctypes.c_int32), ("maskSeqMod", ctypes.c_int32),
+        ("descaleHeads", ctypes.c_int32), ("hasRazorOffset", ctypes.c_int32),
     ]
 
 
 class AtbmiPaTensors(ctypes.Structure):
     _fields_ = [(n, ctypes.c_void_p) for n in
                 ("query", "keyCache", "valueCache", "blockTables", "kScale", "kOffset", "vScale", "vOffset", "out",
-                 "mask", "logN", "queryRope", "keyRopeCache", "lse")]
+                 "mask", "logN", "queryRope", "keyRopeCache", "razorOffset", "lse")]
 
 
 _kernels = None

@@ -98,7 +98,8 @@ struct PaArgs {
     int32_t ropeDim;
     int32_t blockRows;   // cache slots per block (see kRowStride)
     int32_t kHeadStride; // elements between the KV heads of one key-cache slot (see kRowStride)
-    int32_t pad0;
+    int32_t descaleHeads; // > 0: sequence b takes slice b % descaleHeads of the descale vectors instead of its KV head's
+    const float *razor;   // [slots] added to q.k before the score scale (null: none)
     void *lse;           // [rows][H] in the query's type: natural-log log-sum-exp of the scaled scores (null: none)
 };
 

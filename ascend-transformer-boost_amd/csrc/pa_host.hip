@@ -162,6 +162,18 @@ extern "C" int atbmi_pa_plan_create(const AtbmiPaShape *shape, AtbmiPaPlan **pla
                                        "combined cache, got ropeDim %d with head sizes %d / %d", s.ropeDim, s.headDimK,
                     s.headDimV);
     }
+    if (s.maskSeqDiv < 0 || s.maskSeqMod < 0 || s.descaleHeads < 0) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: maskSeqDiv %d, maskSeqMod %d, descaleHeads %d", s.maskSeqDiv,
+                    s.maskSeqMod, s.descaleHeads);
+    }
+    if ((s.descaleHeads > 0 || s.hasRazorOffset) &&
+        (s.numKvHeads != 1 || s.mlaCombined || s.kvLayout != ATBMI_PA_KV_TOKEN_MAJOR)) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: descale slices by sequence and per-slot score offsets belong to "
+                                       "head compression: one KV head, separate token-major caches");
+    }
+    if (s.descaleHeads > 0 && s.kvDtype != ATBMI_INT8) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: descaleHeads only applies to an int8 cache");
+    }
     if (s.kvLayout != ATBMI_PA_KV_TOKEN_MAJOR && s.kvLayout != ATBMI_PA_KV_HEAD_MAJOR) {
         return Fail(ERR_INVALID_PARAM, "pa_plan_create: kvLayout %d", s.kvLayout);
     }
@@ -409,8 +421,10 @@ extern "C" int atbmi_pa_plan_update_multi(AtbmiPaPlan *plan, const int32_t *ctx,
                 row.nTok = 1;
                 const int32_t index = static_cast<int32_t>(plan->rows.size());
                 row.qRow = index;
+                int32_t bySeq = s.maskSeqDiv > 1 ? b / s.maskSeqDiv : b;
+                bySeq = s.maskSeqMod > 0 ? bySeq % s.maskSeqMod : bySeq;
                 row.maskRow = s.maskRowBy == ATBMI_PA_MASK_ROW_QUERY ? index
-                              : s.maskRowBy == ATBMI_PA_MASK_ROW_POSITION ? ctx[b] - n + i : b;
+                              : s.maskRowBy == ATBMI_PA_MASK_ROW_POSITION ? ctx[b] - n + i : bySeq;
                 plan->rows.push_back(row);
             }
         }
@@ -550,6 +564,9 @@ extern "C" uint64_t atbmi_pa_plan_algorithmic_bytes(const AtbmiPaPlan *plan)
     if (s.hasLogN) {
         bytes += static_cast<uint64_t>(plan->batch) * 4;
     }
+    if (s.hasRazorOffset) {
+        bytes += static_cast<uint64_t>(plan->totalCtx) * 4; // one score offset per cache slot attended to
+    }
     if (plan->nonEmpty > 0 && plan->rows.size() > 0 && plan->rowCtx != plan->totalCtx) {
         bytes += static_cast<uint64_t>(plan->batch) * 4; // the query lengths
     }
@@ -627,6 +644,9 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
     if (s.kvDtype == ATBMI_INT8 && (!t->kScale || !t->vScale)) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: int8 cache needs kScale and vScale");
     }
+    if (s.hasRazorOffset && !t->razorOffset) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: hasRazorOffset needs razorOffset");
+    }
     if (s.hasOffset && (!t->kOffset || !t->vOffset)) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: hasOffset needs kOffset and vOffset");
     }
@@ -690,7 +710,10 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
         a.vRowStride = s.mlaCombined ? a.kRowStride : static_cast<int64_t>(s.numKvHeads) * s.headDimV;
         a.vHeadStride = s.mlaCombined ? s.headDimK - s.ropeDim : s.headDimV;
     }
-    a.finishV = (plan->useMfma && s.kvDtype == ATBMI_INT8) ? 1 : 0;
+    // (with per-sequence descale slices the attention kernel descales its partial rows itself)
+    a.finishV = (plan->useMfma && s.kvDtype == ATBMI_INT8 && s.descaleHeads == 0) ? 1 : 0;
+    a.descaleHeads = s.kvDtype == ATBMI_INT8 ? s.descaleHeads : 0;
+    a.razor = s.hasRazorOffset ? t->razorOffset : nullptr;
     if (s.hasMask) {
         a.mask = t->mask;
         a.maskBatchStride = s.maskBatchStride;

@@ -287,6 +287,9 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                       static_cast<int64_t>(h0 + colHead) * a.maskHeadStride;
         }
 
+        // descale slice of this sequence: its KV head's, or, under head compression, the model KV head it stands for
+        const int gs = EXT && a.descaleHeads > 0 ? sq.tableRow % a.descaleHeads : g;
+
         // ---- Q^T as B operand: lane (n, kg) holds q[column n][32j + 8kg .. +8) for j < NQ
         u32x4 qreg[NQ];
         {
@@ -308,8 +311,8 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                     float f[8];
                     f32x4 ks[2] = {f32x4{1.0f, 1.0f, 1.0f, 1.0f}, f32x4{1.0f, 1.0f, 1.0f, 1.0f}};
                     if (KV8) {
-                        ks[0] = LoadScale4(a.kScale, g * D + d0, a.scaleStride);
-                        ks[1] = LoadScale4(a.kScale, g * D + d0 + 4, a.scaleStride);
+                        ks[0] = LoadScale4(a.kScale, gs * D + d0, a.scaleStride);
+                        ks[1] = LoadScale4(a.kScale, gs * D + d0 + 4, a.scaleStride);
                     }
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
@@ -527,7 +530,27 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                 float x[8];
     #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    x[e] = s[e >> 2][e & 3] * scaleSeq;
+                    x[e] = s[e >> 2][e & 3];
+                }
+                if (EXT && a.razor) {
+                    // per-slot score offsets of this lane's 8 tokens, added before the scale (a 16-token
+                    // sub-tile lies in one block)
+#pragma unroll
+                    for (int sub = 0; sub < 2; ++sub) {
+                        const int tok0 = t + sub * 16;
+                        if (tok0 < tokEnd) {
+                            const int64_t slot = static_cast<int64_t>(table[tok0 / a.blockSize]) * a.blockSize +
+                                                 tok0 % a.blockSize + kg * 4;
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) {
+                                x[sub * 4 + r] += a.razor[slot + r];
+                            }
+                        }
+                    }
+                }
+    #pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    x[e] *= scaleSeq;
                 }
                 if (maskRow) {
 #pragma unroll
@@ -737,13 +760,13 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                     float o[4];
                     f32x4 vs = {1.0f, 1.0f, 1.0f, 1.0f};
                     if (KV8) {
-                        vs = LoadScale4(a.vScale, g * DV + d, a.scaleStride);
+                        vs = LoadScale4(a.vScale, gs * DV + d, a.scaleStride);
                     }
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         o[r] = acc[i][r] * inv - bias;
                         if (KV8) {
-                            const int c = g * DV + d + r;
+                            const int c = gs * DV + d + r;
                             o[r] = (o[r] + (a.vOff ? static_cast<float>(a.vOff[c]) : 0.0f)) * vs[r];
                         }
                     }
@@ -765,7 +788,18 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                 const int64_t ph = (static_cast<int64_t>(slot) * (EXT ? p.foldTokens : 1) + colTok) * a.H + h;
 #pragma unroll
                 for (int i = 0; i < NO; ++i) {
-                    *reinterpret_cast<f32x4 *>(a.partO + ph * DV + i * 16 + kg * 4) = acc[i] * inv - bias;
+                    f32x4 o = acc[i] * inv - bias;
+                    if (EXT && KV8 && a.descaleHeads > 0) {
+                        // the merge kernel cannot tell the slice: descale here (an affine map of rows whose
+                        // merge weights sum to one commutes with the merge)
+                        const int c = gs * DV + i * 16 + kg * 4;
+                        const f32x4 vs = LoadScale4(a.vScale, c, a.scaleStride);
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            o[r] = (o[r] + (a.vOff ? static_cast<float>(a.vOff[c + r]) : 0.0f)) * vs[r];
+                        }
+                    }
+                    *reinterpret_cast<f32x4 *>(a.partO + ph * DV + i * 16 + kg * 4) = o;
                 }
                 if (kg == 0) {
                     a.partLse[ph] = m + log2f(l);
@@ -805,7 +839,8 @@ int LaunchBuild(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream
 template <bool BF16, bool KV8, int D, int DV, bool MLA, bool PF, int NW, bool SHARED = false>
 int Launch(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
 {
-    if (MLA || args.mask != nullptr || args.logN != nullptr || plan.foldTokens > 1) {
+    if (MLA || args.mask != nullptr || args.logN != nullptr || plan.foldTokens > 1 || args.razor != nullptr ||
+        args.descaleHeads > 0) {
         return LaunchBuild<BF16, KV8, D, DV, MLA, PF, NW, SHARED, true>(args, plan, stream);
     }
     return LaunchBuild<BF16, KV8, D, DV, MLA, PF, NW, SHARED, MLA>(args, plan, stream);

@@ -47,6 +47,7 @@ __global__ __launch_bounds__(PA_SCALAR_WAVES * WAVE) void PaScalarKernel(const P
     // additive score bias of this sequence and head tile (base-2 units once multiplied by LOG2E)
     const int64_t maskRow = a.mask ? static_cast<int64_t>(it.maskRow) * a.maskBatchStride : 0;
 
+    const int gs = a.descaleHeads > 0 ? it.seq % a.descaleHeads : g; // descale slice (see PaArgs::descaleHeads)
     const int dn = a.D - a.ropeDim; // channels held by q / kc themselves (all of them unless the layout is split)
     float q[HT][EPL];
 #pragma unroll
@@ -75,12 +76,12 @@ __global__ __launch_bounds__(PA_SCALAR_WAVES * WAVE) void PaScalarKernel(const P
         kS[e] = 1.0f; kO[e] = 0.0f; vS[e] = 1.0f; vO[e] = 0.0f;
         if (KV8) {
             if (d < a.D) {
-                kS[e] = a.kScale[(g * a.D + d) * a.scaleStride];
-                kO[e] = a.kOff ? static_cast<float>(a.kOff[g * a.D + d]) : 0.0f;
+                kS[e] = a.kScale[(gs * a.D + d) * a.scaleStride];
+                kO[e] = a.kOff ? static_cast<float>(a.kOff[gs * a.D + d]) : 0.0f;
             }
             if (d < a.Dv) {
-                vS[e] = a.vScale[(g * a.Dv + d) * a.scaleStride];
-                vO[e] = a.vOff ? static_cast<float>(a.vOff[g * a.Dv + d]) : 0.0f;
+                vS[e] = a.vScale[(gs * a.Dv + d) * a.scaleStride];
+                vO[e] = a.vOff ? static_cast<float>(a.vOff[gs * a.Dv + d]) : 0.0f;
             }
         }
     }
@@ -102,6 +103,7 @@ __global__ __launch_bounds__(PA_SCALAR_WAVES * WAVE) void PaScalarKernel(const P
         const int64_t kBase = row * a.kRowStride + static_cast<int64_t>(g) * a.kHeadStride;
         const int64_t rBase = row * a.ropeRowStride + static_cast<int64_t>(g) * a.ropeDim - dn;
         const int64_t vBase = row * a.vRowStride + static_cast<int64_t>(g) * a.vHeadStride;
+        const float razor = a.razor ? a.razor[row] : 0.0f;
         float k[EPL], v[EPL];
 #pragma unroll
         for (int e = 0; e < EPL; ++e) {
@@ -132,7 +134,7 @@ __global__ __launch_bounds__(PA_SCALAR_WAVES * WAVE) void PaScalarKernel(const P
                 for (int e = 0; e < EPL; ++e) {
                     s += q[hh][e] * k[e];
                 }
-                s = WaveSum(s) * scale2;
+                s = (WaveSum(s) + razor) * scale2;
                 if (a.mask) {
                     s += Load16(a.mask, maskRow + static_cast<int64_t>(h0 + hh) * a.maskHeadStride + t, bf16) * LOG2E;
                 }

@@ -143,8 +143,6 @@ bool ImplementedCheck(const Param &p)
         what = "MASK_TYPE_MASK_FREE";
     } else if (p.maskType == Param::MASK_TYPE_SPEC && p.calcType != Param::CALC_TYPE_SPEC) {
         what = "MASK_TYPE_SPEC without CALC_TYPE_SPEC";
-    } else if (p.compressType != Param::COMPRESS_TYPE_UNDEFINED) {
-        what = "head compression";
     } else if (p.quantType == Param::TYPE_QUANT_QKV_OFFLINE || p.quantType == Param::TYPE_QUANT_QKV_ONLINE) {
         what = "int8 query quantisation";
     } else if (p.quantType != Param::TYPE_QUANT_UNQUANT && p.quantType != Param::TYPE_DEQUANT_FUSION) {
@@ -190,6 +188,9 @@ IrCombo MakeCombo(const Param &p, aclDataType q, aclDataType descale)
             c.inDtypes.push_back(ACL_INT32);
         }
     }
+    if (p.compressType == Param::COMPRESS_TYPE_KVHEAD_ROPE) {
+        c.inDtypes.push_back(ACL_FLOAT); // razorOffset (reference paged_attention_ops_runner.cpp:126-128)
+    }
     if (p.scaleType == Param::SCALE_TYPE_LOGN) {
         c.inDtypes.push_back(ACL_FLOAT);
     }
@@ -216,6 +217,7 @@ public:
     explicit PagedAttentionOperation(const Param &param)
         : OperationBase("PagedAttentionOperation"), param_(param), mla_(param.mlaVHeadSize > 0),
           dequant_(param.quantType == Param::TYPE_DEQUANT_FUSION), bnsd_(param.inputLayout == infer::TYPE_BNSD),
+          compress_(param.compressType != Param::COMPRESS_TYPE_UNDEFINED),
           irTable_(MakeIr(param))
     {
         ir_ = &irTable_;
@@ -240,6 +242,9 @@ public:
             if (param.hasQuantOffset) {
                 vOffsetIdx_ = next++;
             }
+        }
+        if (param.compressType == Param::COMPRESS_TYPE_KVHEAD_ROPE) {
+            razorIdx_ = next++;
         }
         if (param.scaleType == Param::SCALE_TYPE_LOGN) {
             logNIdx_ = next++;
@@ -333,6 +338,14 @@ protected:
             ATB_LOG(ERROR) << "numTokens of the output should be the same as q";
             return ERROR_INVALID_TENSOR_DIM;
         }
+        if (razorIdx_ != NONE) {
+            // reference :877-898 (RazorDimCheck): one score offset per cache slot
+            const Dims &razor = in.at(razorIdx_).shape;
+            if (razor.dimNum != 2 || razor.dims[0] != in.at(1).shape.dims[0] || razor.dims[1] != in.at(1).shape.dims[1]) {
+                ATB_LOG(ERROR) << "razorOffset should be [numBlocks, blockSize] of keyCache";
+                return ERROR_INVALID_TENSOR_DIM;
+            }
+        }
         if (logNIdx_ != NONE) {
             // reference :900-924 (LogNDimCheck)
             const Dims &logN = in.at(logNIdx_).shape;
@@ -373,7 +386,22 @@ protected:
             return ERROR_INVALID_PARAM;
         }
         const int64_t cacheHeads = kc.desc.shape.dims[bnsd_ ? 1 : 2];
-        if (cacheHeads != kvHeads || (bnsd_ && pack.inTensors.at(2).desc.shape.dims[1] != kvHeads)) {
+        if (compress_) {
+            // reference kernel library paged_attention_operation.cpp:316-325,342-354: the caches hold one head
+            // per block and contextLens / blockTables one row per (sequence, KV head)
+            if (cacheHeads != 1 || pack.inTensors.at(2).desc.shape.dims[2] != 1) {
+                ATB_LOG(ERROR) << "head compression: the caches should have one head, [numBlocks, blockSize, 1, headSize]";
+                return ERROR_INVALID_PARAM;
+            }
+            if (q.desc.shape.dims[0] * kvHeads != lens.desc.shape.dims[0]) {
+                ATB_LOG(ERROR) << "head compression: contextLens should have numTokens * kvHeadNum entries";
+                return ERROR_INVALID_PARAM;
+            }
+            if (dequant_ && q.desc.dtype != ACL_FLOAT16) {
+                ATB_LOG(ERROR) << "head compression with an int8 cache needs an fp16 query";
+                return ERROR_INVALID_PARAM;
+            }
+        } else if (cacheHeads != kvHeads || (bnsd_ && pack.inTensors.at(2).desc.shape.dims[1] != kvHeads)) {
             ATB_LOG(ERROR) << "cache head count " << cacheHeads << " != kvHeadNum " << kvHeads;
             return ERROR_INVALID_PARAM;
         }
@@ -432,9 +460,11 @@ protected:
         int64_t maskHeadStride = 0;
         int64_t maskLen = 0;
         int32_t maskRowBy = ATBMI_PA_MASK_ROW_SEQUENCE;
+        int32_t maskSeqDiv = 0;
+        int32_t maskSeqMod = 0;
         if (maskIdx_ != NONE) {
             Status st = MaskLayout(pack.inTensors.at(maskIdx_).desc.shape, lens, q.desc.shape.dims[0], maskBatchStride,
-                                   maskHeadStride, maskLen, maskRowBy);
+                                   maskHeadStride, maskLen, maskRowBy, maskSeqDiv, maskSeqMod);
             if (st != NO_ERROR) {
                 return st;
             }
@@ -457,14 +487,21 @@ protected:
         AtbmiPaShape shape{};
         shape.qDtype = q.desc.dtype == ACL_BF16 ? ATBMI_BF16 : ATBMI_F16;
         shape.kvDtype = kc.desc.dtype == ACL_INT8 ? ATBMI_INT8 : shape.qDtype;
-        shape.numHeads = param_.headNum;
-        shape.numKvHeads = static_cast<int32_t>(kvHeads);
+        // head compression: the kernels see one sequence per (sequence, KV head) pair, each with the query heads of
+        // that KV head; [tokens, heads, D] is the same memory as [tokens * kvHeads, heads / kvHeads, D]
+        // (reference tiling/paged_attention_tiling.cpp:217-226)
+        shape.numHeads = compress_ ? static_cast<int32_t>(param_.headNum / kvHeads) : param_.headNum;
+        shape.numKvHeads = compress_ ? 1 : static_cast<int32_t>(kvHeads);
+        shape.descaleHeads = (compress_ && dequant_) ? static_cast<int32_t>(kvHeads) : 0;
+        shape.maskSeqDiv = maskSeqDiv;
+        shape.maskSeqMod = maskSeqMod;
+        shape.hasRazorOffset = razorIdx_ != NONE ? 1 : 0;
         shape.headDimK = static_cast<int32_t>(d);
         shape.headDimV = static_cast<int32_t>(dv);
         shape.blockSize = static_cast<int32_t>(blockSize);
         shape.numBlocks = static_cast<int32_t>(kc.desc.shape.dims[0]);
         shape.maxBlocksPerSeq = static_cast<int32_t>(tables.desc.shape.dims[1]);
-        shape.numQueryRows = static_cast<int32_t>(q.desc.shape.dims[0]);
+        shape.numQueryRows = static_cast<int32_t>(q.desc.shape.dims[0] * (compress_ ? kvHeads : 1));
         shape.mlaCombined = mla_ ? 1 : 0;
         shape.hasOffset = (dequant_ && param_.hasQuantOffset) ? 1 : 0;
         shape.kernel = ATBMI_PA_KERNEL_AUTO;
@@ -523,6 +560,9 @@ protected:
         if (logNIdx_ != NONE) {
             t.logN = static_cast<const float *>(pack.inTensors.at(logNIdx_).deviceData);
         }
+        if (razorIdx_ != NONE) {
+            t.razorOffset = static_cast<const float *>(pack.inTensors.at(razorIdx_).deviceData);
+        }
         t.out = pack.outTensors.at(0).deviceData;
         int rc = atbmi_pa_decode(plan_, &t, workspace, workspaceSize, stream);
         if (rc != 0) {
@@ -541,7 +581,8 @@ private:
                a.qkScale == b.qkScale && a.qScale == b.qScale && a.hasMask == b.hasMask &&
                a.maskBatchStride == b.maskBatchStride && a.maskHeadStride == b.maskHeadStride &&
                a.maskLen == b.maskLen && a.hasLogN == b.hasLogN && a.descalePacked == b.descalePacked &&
-               a.maskRowBy == b.maskRowBy && a.kvLayout == b.kvLayout;
+               a.maskRowBy == b.maskRowBy && a.kvLayout == b.kvLayout && a.maskSeqDiv == b.maskSeqDiv &&
+               a.maskSeqMod == b.maskSeqMod && a.descaleHeads == b.descaleHeads && a.hasRazorOffset == b.hasRazorOffset;
     }
 
     // Element strides of the additive mask, as the reference derives them from
@@ -562,11 +603,21 @@ private:
     // contextLen - queryLen + i. Other NORM shapes are refused under
     // CALC_TYPE_SPEC: the reference would step from a sequence's row into its
     // neighbour's for the second query token.
+    //
+    // Under head compression the kernels' sequences are (sequence, KV head) pairs and their heads the
+    // query heads of one KV head (reference tiling :36-80, kernel library :754-758): a mask with one
+    // row per model sequence is indexed by pair / kvHeads, the ALIBI (heads, 1, maxS) mask by pair %
+    // kvHeads with a row group of heads / kvHeads rows, and (batch, heads, 1, maxS) reads as
+    // (pairs, heads / kvHeads, 1, maxS) as it lies.
     Status MaskLayout(const Dims &m, const Tensor &lens, int64_t queryRows, int64_t &batchStride,
-                      int64_t &headStride, int64_t &maskLen, int32_t &rowBy) const
+                      int64_t &headStride, int64_t &maskLen, int32_t &rowBy, int32_t &seqDiv, int32_t &seqMod) const
     {
-        const int64_t batch = lens.desc.shape.dims[0];
+        const int64_t kvHeads = param_.kvHeadNum > 0 ? param_.kvHeadNum : param_.headNum;
+        const int64_t pairs = compress_ ? kvHeads : 1; // kernel sequences per model sequence
+        const int64_t batch = lens.desc.shape.dims[0] / pairs;
         const int64_t heads = param_.headNum;
+        seqDiv = 0;
+        seqMod = 0;
         const bool alibi = param_.maskType == Param::MASK_TYPE_ALIBI;
         const bool multi = param_.calcType == Param::CALC_TYPE_SPEC;
         bool ok = false;
@@ -589,14 +640,17 @@ private:
             ok = m.dims[0] == batch && m.dims[1] == 1;
             batchStride = m.dims[2];
             headStride = 0;
+            seqDiv = static_cast<int32_t>(pairs);
         } else if (alibi && m.dimNum == 3) {
             ok = m.dims[0] == heads && m.dims[1] == 1;
-            batchStride = 0;
+            batchStride = compress_ ? heads / kvHeads * m.dims[2] : 0;
             headStride = m.dims[2];
+            seqMod = compress_ ? static_cast<int32_t>(kvHeads) : 0;
         } else if (alibi && m.dimNum == 4) {
             ok = m.dims[0] == batch && (m.dims[1] == 1 || m.dims[1] == heads) && m.dims[2] == 1;
-            batchStride = m.dims[1] * m.dims[3];
+            batchStride = m.dims[1] / (m.dims[1] == 1 ? 1 : pairs) * m.dims[3];
             headStride = m.dims[1] == 1 ? 0 : m.dims[3];
+            seqDiv = m.dims[1] == 1 ? static_cast<int32_t>(pairs) : 0;
         }
         if (!ok) {
             ATB_LOG(ERROR) << "mask shape is not one of NORM (1,maxS) / (batch,1,maxS), "
@@ -606,7 +660,7 @@ private:
         }
         maskLen = m.dims[m.dimNum - 1];
         const int32_t *ctx = static_cast<const int32_t *>(lens.hostData);
-        for (int64_t i = 0; i < batch; ++i) {
+        for (int64_t i = 0; i < lens.desc.shape.dims[0]; ++i) {
             if (ctx[i] > maskLen) {
                 ATB_LOG(ERROR) << "mask covers " << maskLen << " positions but contextLens[" << i << "] is " << ctx[i];
                 return ERROR_INVALID_PARAM;
@@ -649,7 +703,7 @@ private:
         }
         const int64_t blockSize = in.at(1).shape.dims[1];
         const bool strict = dequant_ || (param_.calcType == Param::CALC_TYPE_SPEC && !mla_) ||
-                            param_.scaleType == Param::SCALE_TYPE_LOGN;
+                            param_.scaleType == Param::SCALE_TYPE_LOGN || compress_;
         if (strict) {
             // strict regime (reference :561-572): features that predate the split K/V head sizes
             if (d != in.at(2).shape.dims[3]) {
@@ -692,8 +746,10 @@ private:
     bool mla_;
     bool dequant_;
     bool bnsd_;
+    bool compress_; // every (sequence, KV head) pair comes with its own context length and block-table row
     OpIr irTable_;
     static constexpr size_t NONE = ~static_cast<size_t>(0);
+    size_t razorIdx_ = NONE;
     size_t tablesIdx_ = 3;
     size_t lensIdx_ = 4;
     size_t maskIdx_ = NONE;

@@ -243,6 +243,18 @@ typedef struct AtbmiPaShape {
                                 query and keyCache hold rows of headDimK - ropeDim channels, queryRope and
                                 keyRopeCache the remaining ropeDim channels of the same rows */
     int32_t kvLayout;        /* AtbmiPaKvLayout of keyCache and valueCache */
+    /* Head compression (PagedAttentionParam::compressType, reference
+     * src/kernels/mixkernels/pagedattention/tiling/paged_attention_tiling.cpp:36-80,217-226): every (sequence,
+     * KV head) pair of the model becomes a sequence of its own here, with its own context length and block-table
+     * row, numKvHeads = 1 and numHeads = the model's heads per KV head; query / out rows are the same memory read
+     * as [tokens * kvHeads, numHeads, D]. Three things then still follow the model's indices: */
+    int32_t maskSeqDiv;      /* > 1 with maskRowBy SEQUENCE: sequence b uses mask row b / maskSeqDiv (a mask with one
+                                row per model sequence) */
+    int32_t maskSeqMod;      /* > 0 with maskRowBy SEQUENCE: ... row b % maskSeqMod (a mask with one row group per
+                                model KV head and none per sequence); applied after maskSeqDiv */
+    int32_t descaleHeads;    /* > 0, int8 KV: kScale / vScale (and the offsets) hold descaleHeads slices of D / Dv
+                                entries and sequence b uses slice b % descaleHeads; numKvHeads must be 1 */
+    int32_t hasRazorOffset;  /* 1: AtbmiPaTensors.razorOffset is given (COMPRESS_TYPE_KVHEAD_ROPE) */
 } AtbmiPaShape;
 
 /* Device tensors of one decode call.
@@ -275,6 +287,8 @@ typedef struct AtbmiPaTensors {
     const float *logN;
     const void *queryRope;    /* [numQueryRows, H, ropeDim] qDtype, ropeDim > 0 only */
     const void *keyRopeCache; /* [numBlocks, blockSize, G, ropeDim] qDtype, ropeDim > 0 only */
+    const float *razorOffset; /* hasRazorOffset only: fp32 [numBlocks, blockSize], added to q.k of the token in that
+                                 cache slot before the qkScale multiplication (numKvHeads 1, token-major caches) */
     void *lse;                /* NULL, or [numQueryRows, H] qDtype: receives the natural-log log-sum-exp of the
                                  scaled (and masked) scores of every planned query row and head — the second
                                  output of MultiLatentAttentionParam::CALC_TYPE_RING */

@@ -264,13 +264,16 @@ def gather_rows(cache, block_table, context_len):
 
 
 def attention_one(q, keys, values, scale, k_descale=None, k_offset=None, v_descale=None, v_offset=None,
-                  bias=None, lse_out=None):
+                  bias=None, lse_out=None, descale_head=None, score_offset=None):
     """One query token against gathered rows. q [heads, D] float32; keys
     [ctx, kv_heads, D]; values [ctx, kv_heads, Dv] (float32 or int8); bias None
     or broadcastable to [heads, ctx], added to the scaled scores.
     Returns float32 [heads, Dv]: softmax(scale * q k^T + bias) v per GQA group.
     lse_out, a float32 [heads] array, receives the natural-log log-sum-exp of the
-    scaled and biased scores (row max + log of the row sum of exp(score - max))."""
+    scaled and biased scores (row max + log of the row sum of exp(score - max)).
+    descale_head: the slice of the descale vectors to use instead of the KV head's
+    index (the reference golden's razor_mod, test_paged_attention_common.py:85-101,341-347).
+    score_offset: float32 [ctx], added to q k^T before the scale (its razor_offset_list, :249-252)."""
     if bias is not None:
         bias = np.broadcast_to(np.asarray(bias, dtype=np.float32), (q.shape[0], keys.shape[0]))
     heads = q.shape[0]
@@ -281,12 +284,15 @@ def attention_one(q, keys, values, scale, k_descale=None, k_offset=None, v_desca
         k = keys[:, g, :]
         v = values[:, g, :]
         if k.dtype == np.int8:
-            k = _dequant(k, k_descale, k_offset, g, keys.shape[2])
-            v = _dequant(v, v_descale, v_offset, g, values.shape[2])
+            k = _dequant(k, k_descale, k_offset, g if descale_head is None else descale_head, keys.shape[2])
+            v = _dequant(v, v_descale, v_offset, g if descale_head is None else descale_head, values.shape[2])
         k = k.astype(np.float32)
         v = v.astype(np.float32)
         qg = q[g * group:(g + 1) * group].astype(np.float32)
-        sim = (qg @ k.T) * np.float32(scale)
+        sim = qg @ k.T
+        if score_offset is not None:
+            sim = sim + np.asarray(score_offset, dtype=np.float32)[None, :]
+        sim = sim * np.float32(scale)
         if bias is not None:
             sim = sim + bias[g * group:(g + 1) * group]
         p = softmax_rows(sim)
@@ -328,7 +334,7 @@ def norm_mask(batch, max_len, value=-10000.0):
 def paged_attention(query, key_cache, value_cache, block_tables, context_lens, scale, k_descale=None,
                     k_offset=None, v_descale=None, v_offset=None, mla_v_head_size=0, q_scale=0.0,
                     q_dtype="float32", out_init=0.0, mask=None, logn=None, mask_per_head=None, q_lens=None,
-                    mask_rows="sequence", lse_out=None, head_major=False):
+                    mask_rows="sequence", lse_out=None, head_major=False, compress_kv_heads=0, razor_offset=None):
     """Decode attention over paged caches.
 
     query [rows, heads, D] float32; key_cache [blocks, block, kv_heads, D];
@@ -361,8 +367,37 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, s
     operation its (0, 2, 1, 3) permutation
     (tests/apitest/opstest/python/operations/paged_attention/test_paged_attention_operation_BNSD.py:369-373),
     so this is the same computation after permuting back.
+    compress_kv_heads = n > 0 (PagedAttentionParam::compressType; reference golden
+    test_paged_attention_common.py:292-360): the caches hold one head per block,
+    [blocks * n, block, 1, D], and block_tables / context_lens one row per
+    (sequence, KV head) pair; query [tokens, heads, D] is read as
+    [tokens * n, heads / n, D] and pair i takes the descale slices of KV head
+    i % n. A 4-dim mask [batch, heads, 1, max_len] is read as
+    [batch * n, heads / n, 1, max_len], a 3-dim mask has one row per sequence
+    (pair i uses row i // n). razor_offset, float32 [blocks * n, block], is added
+    to q k^T of the token in that cache slot before the scale.
     Returns float32 [rows, heads, Dv]."""
     query = np.asarray(query, dtype=np.float32)
+    if compress_kv_heads > 0:
+        n = compress_kv_heads
+        tokens, heads, d = query.shape
+        if mask is not None and np.ndim(mask) == 4:
+            mask = np.asarray(mask, dtype=np.float32)
+            if mask.shape[1] == 1:  # one row per sequence, shared by its heads
+                mask = np.repeat(mask, n, axis=0)
+            else:
+                mask = mask.reshape(mask.shape[0] * n, mask.shape[1] // n, 1, mask.shape[3])
+        elif mask is not None and np.ndim(mask) == 3 and mask_per_head:
+            # [heads, 1, max_len], shared by all sequences: the 4-dim form with the batch axis broadcast
+            mask = np.asarray(mask, dtype=np.float32)
+            pairs = len(context_lens)
+            mask = np.broadcast_to(mask[None], (pairs // n,) + mask.shape).reshape(pairs, heads // n, 1, mask.shape[2])
+        elif mask is not None and np.ndim(mask) == 3:
+            mask = np.repeat(np.asarray(mask, dtype=np.float32), n, axis=0)
+        out = _paged_attention_compressed(query.reshape(tokens * n, heads // n, d), key_cache, value_cache, block_tables,
+                                          context_lens, scale, k_descale, k_offset, v_descale, v_offset, out_init, mask,
+                                          n, razor_offset)
+        return out.reshape(tokens, heads, out.shape[2])
     if head_major:
         key_cache = np.transpose(key_cache, (0, 2, 1, 3))
         value_cache = None if value_cache is None else np.transpose(value_cache, (0, 2, 1, 3))
@@ -392,6 +427,32 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, s
             out[row] = attention_one(query[row], keys, values, seq_scale, k_descale, k_offset, v_descale,
                                      v_offset, bias, None if lse_out is None else lse_out[row])
             row += 1
+    return out
+
+
+def _paged_attention_compressed(query, key_cache, value_cache, block_tables, context_lens, scale, k_descale, k_offset,
+                                v_descale, v_offset, out_init, mask, n, razor_offset):
+    """paged_attention over (sequence, KV head) pairs; see its compress_kv_heads."""
+    out = np.full((query.shape[0], query.shape[1], value_cache.shape[3]), out_init, dtype=np.float32)
+    block_size = key_cache.shape[1]
+    row = 0
+    for i, ctx in enumerate(np.asarray(context_lens).tolist()):
+        if ctx == 0:
+            continue
+        keys = gather_rows(key_cache, block_tables[i], ctx)
+        values = gather_rows(value_cache, block_tables[i], ctx)
+        offsets = None
+        if razor_offset is not None:
+            j = np.arange(ctx)
+            offsets = np.asarray(razor_offset, dtype=np.float32)[np.asarray(block_tables[i])[j // block_size],
+                                                                  j % block_size]
+        bias = None
+        if mask is not None:
+            m = np.asarray(mask, dtype=np.float32)
+            bias = m[i, :, 0, :ctx] if m.ndim == 4 else (m[i, :, :ctx] if m.ndim == 3 else m[:1, :ctx])
+        out[row] = attention_one(query[row], keys, values, np.float32(scale), k_descale, k_offset, v_descale, v_offset,
+                                 bias, descale_head=i % n, score_offset=offsets)
+        row += 1
     return out
 
 

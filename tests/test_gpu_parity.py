@@ -745,6 +745,89 @@ def test_head_major_blocks_through_operation_api(binding, oracle, dev, stream):
     c.close()
 
 
+# name, model batch, heads, kv heads, block, d, dtype, mask kind, int8 cache (+ offsets), razor offsets, zero lengths
+COMPRESS_CASES = [
+    ("plain", 5, 32, 8, 128, 128, torch.float16, None, False, False, False),
+    ("norm3", 4, 32, 8, 128, 128, torch.bfloat16, "norm3", False, False, False),
+    ("alibi4", 3, 40, 2, 128, 128, torch.float16, "alibi4", False, False, False),   # 20 heads per KV head: two tiles
+    ("alibi4_1", 4, 16, 4, 16, 64, torch.float16, "alibi4_1", False, False, False),
+    ("alibi3", 4, 32, 2, 128, 128, torch.bfloat16, "alibi3", False, False, False),
+    ("int8", 6, 16, 4, 128, 128, torch.float16, None, True, False, False),
+    ("int8_norm3", 3, 32, 8, 64, 128, torch.float16, "norm3", True, False, False),
+    ("razor", 5, 32, 2, 128, 128, torch.bfloat16, None, False, True, False),
+    ("razor_int8", 4, 8, 8, 32, 128, torch.float16, None, True, True, False),        # reference CSV shape: 8 heads, 8 KV heads
+    ("zeros", 4, 32, 8, 128, 128, torch.float16, "alibi4", False, False, True),
+    ("d96", 3, 12, 3, 16, 96, torch.float16, "norm3", False, False, False),
+]
+
+
+@pytest.mark.parametrize("forced", ["scalar", None])
+@pytest.mark.parametrize("case", COMPRESS_CASES, ids=lambda c: c[0])
+def test_head_compression_through_operation_api(binding, oracle, dev, stream, case, forced, monkeypatch):
+    """PagedAttentionParam::compressType: caches [numBlocks, blockSize, 1, headSize], one context length and
+    block-table row per (sequence, KV head) pair (reference golden test_paged_attention_common.py:292-360 and
+    tiling/paged_attention_tiling.cpp:36-80,217-226); COMPRESS_TYPE_KVHEAD_ROPE adds the per-slot score offsets."""
+    name, batch, heads, n, block, d, dtype, kind, kv_int8, razor, zeros = case
+    rng = _rng(800 + batch + heads + n)
+    if forced:
+        monkeypatch.setenv("ATBMI_PA_KERNEL", forced)
+    group = heads // n
+    ctx = rng.integers(1, 1400, size=batch * n).astype(np.int32)
+    ctx[rng.integers(0, batch * n)] = 2500
+    if zeros:
+        ctx[[1, 2, batch * n - 1]] = 0
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, batch * n, group, 1, block, d, d, ctx, dtype, kv_int8=kv_int8)
+    q_model = q.view(batch, heads, d)
+    max_len = 2500
+    mask = per_head = None
+    if kind is not None:
+        mask, per_head = _mask_tensor(oracle, rng, dev, kind, np.full(batch, max_len), heads, max_len, dtype)
+    ks = ko = vs = vo = ro = None
+    if kv_int8:
+        ks = torch.from_numpy(rng.uniform(0.01, 0.1, size=n * d).astype(np.float32)).to(dev)
+        vs = torch.from_numpy(rng.uniform(0.01, 0.1, size=n * d).astype(np.float32)).to(dev)
+        ko = torch.from_numpy(rng.integers(-20, 20, size=n * d).astype(np.int32)).to(dev)
+        vo = torch.from_numpy(rng.integers(-20, 20, size=n * d).astype(np.int32)).to(dev)
+    if razor:
+        # like the reference generator (:469-478): mostly zero, values in [0, 20) at one offset of most blocks
+        r = np.zeros((kc.shape[0], block), dtype=np.float32)
+        rows = np.where(rng.random(kc.shape[0]) < 0.8)[0]
+        r[rows, rng.integers(0, block, size=len(rows))] = rng.uniform(0, 20, size=len(rows)).astype(np.float32)
+        ro = torch.from_numpy(r).to(dev)
+    scale = 1.0 / math.sqrt(d)
+    param = binding.PagedAttentionParam(
+        headNum=heads, kvHeadNum=n, qkScale=scale, compressType=2 if razor else 1,
+        maskType={None: 0, "norm3": 1}.get(kind, 2), quantType=1 if kv_int8 else 0, hasQuantOffset=kv_int8,
+        batchRunStatusEnable=zeros)
+    lens = torch.from_numpy(ctx)
+    ins = [q_model, kc, vc, tables, lens.to(dev)]
+    host = {4: lens}
+    if mask is not None:
+        ins.append(mask)
+    if zeros:
+        status = torch.from_numpy((ctx > 0).astype(np.int32))
+        host[len(ins)] = status
+        ins.append(status.to(dev))
+    if kv_int8:
+        ins += [ks, ko, vs, vo]
+    if razor:
+        ins.append(ro)
+    c = binding.Context(stream)
+    pa = binding.OperationRunner("PagedAttentionOperation", param, c)
+    out = torch.full((batch, heads, d), 7.0, dtype=dtype, device=dev)
+    with torch.cuda.stream(stream):
+        pa.run(ins, outputs=[out], host_inputs=host)
+    stream.synchronize()
+    pa.close()
+    c.close()
+    want = oracle_pa(oracle, q_model, kc, vc, tables, ctx, scale, ks, ko, vs, vo, mask=mask, mask_per_head=per_head,
+                     compress_kv_heads=n, razor_offset=ro, out_init=7.0)
+    assert_close(out, want, INT8_TOL if kv_int8 else TOL[dtype], name)
+    if razor or kind is not None:  # the offsets / the mask matter in this case
+        plain = oracle_pa(oracle, q_model, kc, vc, tables, ctx, scale, ks, ko, vs, vo, compress_kv_heads=n, out_init=7.0)
+        assert np.abs(want - plain).max() > 0.01
+
+
 def test_c1_decode_step_through_operation_api(binding, oracle, pkg, dev, stream):
     """Benchmark configuration 1 end to end: ReshapeAndCache then PagedAttention
     through atb::Operation, fp16, rtol = atol = 1e-3."""

@@ -38,7 +38,7 @@ ELEWISE_CASES = _load("elewise")
 def _pa_unimplemented(p):
     """Features of PagedAttentionParam the reference accepts but this library rejects at creation."""
     return (p.get("maskType", 0) >= 4 or (p.get("maskType", 0) == 3 and p.get("calcType", 0) != 1) or
-            p.get("compressType", 0) != 0 or p.get("quantType", 0) >= 2)
+            p.get("quantType", 0) >= 2)
 
 
 def _pa_mask_shape_refused(case):
@@ -251,7 +251,7 @@ def test_table_coverage():
     pa_dev = [c for c in PA_CASES if (_pa_unimplemented(c["param"]) and not c["expected"].startswith("C:")) or
               _pa_mask_shape_refused(c)]
     rac_dev = [c for c in RAC_CASES if _rac_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
-    assert len(PA_CASES) == 81 and len(PA_CASES) - len(pa_dev) >= 73
+    assert len(PA_CASES) == 81 and len(PA_CASES) - len(pa_dev) >= 75
     assert len(RAC_CASES) == 38 and len(RAC_CASES) - len(rac_dev) >= 26
     # most MultiLatentAttention rows exercise the prefill calcType and the fractal-NZ caches, which are not built
     mla_dev = [c for c in MLA_CASES if _mla_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
@@ -675,6 +675,67 @@ def test_paged_attention_bnsd_checks(binding, ctx):
     assert op.setup(pack(vc=(9, 8, 64, 128)), out(), ctx)[0] == E["ERROR_INVALID_PARAM"]
     assert op.setup(pack(), out((4, 16, 128)), ctx)[0] == E["ERROR_INVALID_PARAM"]
     assert op.setup(pack(kc=(9, 16, 24, 128), vc=(9, 16, 24, 128)), out(), ctx)[0] == E["ERROR_INVALID_PARAM"]  # 16-aligned
+    op.close()
+
+
+def test_paged_attention_head_compression_checks(binding, ctx):
+    """compressType KVHEAD / KVHEAD_ROPE: parameter combinations (reference paged_attention_operation.cpp:197-215,
+    225,266,294,309,339), the razorOffset input and its dims (:426-427,877-898), and what the reference's kernel
+    library asks of the shapes (mixkernels/pagedattention/paged_attention_operation.cpp:316-325,342-354,754-758)."""
+    E = binding.ERROR_CODE
+    P = binding.PagedAttentionParam
+    base = dict(headNum=32, kvHeadNum=8, qkScale=0.088)
+    for bad in (dict(compressType=3), dict(compressType=-1), dict(compressType=2, maskType=1),
+                dict(compressType=2, batchRunStatusEnable=True), dict(compressType=1, calcType=1, maskType=1),
+                dict(compressType=1, scaleType=1), dict(compressType=1, inputLayout=1),
+                dict(compressType=1, mlaVHeadSize=64, kvHeadNum=1), dict(compressType=1, quantType=2, outDataType=1)):
+        assert binding.Operation("PagedAttentionOperation", P(**dict(base, **bad))).status == E["ERROR_INVALID_PARAM"], bad
+    lens = np.full((32,), 100, dtype=np.int32)
+    mk = binding.make_tensor
+
+    def pack(q=(4, 32, 128), kc=(64, 128, 1, 128), vc=(64, 128, 1, 128), tables=(32, 8), n_lens=32, dtype="float16",
+             extra=()):
+        return [mk(dtype, q, FAKE_DEVICE), mk(dtype, kc, FAKE_DEVICE), mk(dtype, vc, FAKE_DEVICE),
+                mk("int32", tables, FAKE_DEVICE), mk("int32", (n_lens,), FAKE_DEVICE, host_ptr=lens.ctypes.data)] + [
+                    mk(dt, shape, FAKE_DEVICE) for dt, shape in extra]
+
+    out = lambda dtype="float16": [mk(dtype, (4, 32, 128), FAKE_DEVICE)]
+    op = binding.Operation("PagedAttentionOperation", P(**dict(base, compressType=1)))
+    assert op.status == 0 and op.infer_shape(pack())[0] == 0
+    assert op.setup(pack(), out(), ctx)[0] == 0
+    assert op.infer_shape(pack(vc=(64, 128, 1, 96)))[0] == E["ERROR_INVALID_TENSOR_DIM"]       # K and V head sizes
+    assert op.setup(pack(kc=(64, 128, 8, 128), vc=(64, 128, 8, 128)), out(), ctx)[0] == E["ERROR_INVALID_PARAM"]
+    assert op.setup(pack(tables=(4, 8), n_lens=4), out(), ctx)[0] == E["ERROR_INVALID_PARAM"]  # one length per pair
+    op.close()
+    # masks: one row per model sequence, per head of the model, or both
+    for mask_type, shape, ok in ((1, (1, 512), True), (1, (4, 1, 512), True), (1, (32, 1, 512), False),
+                                 (2, (32, 1, 512), True), (2, (4, 32, 1, 512), True), (2, (4, 1, 1, 512), True),
+                                 (2, (32, 32, 1, 512), False), (2, (4, 4, 1, 512), False)):
+        op = binding.Operation("PagedAttentionOperation", P(**dict(base, compressType=1, maskType=mask_type)))
+        st = op.setup(pack(extra=[("float16", shape)]), out(), ctx)[0]
+        assert st == (0 if ok else E["ERROR_INVALID_PARAM"]), (mask_type, shape)
+        op.close()
+    # int8 cache: descales of the model's KV heads; fp16 queries only
+    op = binding.Operation("PagedAttentionOperation", P(**dict(base, compressType=1, quantType=1)))
+    i8 = lambda dtype="float16", n=8 * 128: [
+        mk(dtype, (4, 32, 128), FAKE_DEVICE), mk("int8", (64, 128, 1, 128), FAKE_DEVICE),
+        mk("int8", (64, 128, 1, 128), FAKE_DEVICE), mk("int32", (32, 8), FAKE_DEVICE),
+        mk("int32", (32,), FAKE_DEVICE, host_ptr=lens.ctypes.data), mk("float", (n,), FAKE_DEVICE),
+        mk("float", (n,), FAKE_DEVICE)]
+    assert op.setup(i8(), out(), ctx)[0] == 0
+    assert op.setup(i8(n=128), out(), ctx)[0] == E["ERROR_INVALID_PARAM"]
+    assert op.setup(i8(dtype="bf16"), out("bf16"), ctx)[0] == E["ERROR_INVALID_PARAM"]
+    op.close()
+    # KVHEAD_ROPE: one more input, fp32 [numBlocks, blockSize]
+    op = binding.Operation("PagedAttentionOperation", P(**dict(base, compressType=2)))
+    assert op.status == 0 and op.input_num() == 6
+    assert op.setup(pack(extra=[("float", (64, 128))]), out(), ctx)[0] == 0
+    assert op.setup(pack(dtype="bf16", extra=[("float", (64, 128))]), out("bf16"), ctx)[0] == 0
+    assert op.setup(pack(extra=[("float", (64, 64))]), out(), ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.setup(pack(extra=[("float", (32, 128))]), out(), ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.setup(pack(extra=[("float", (64 * 128,))]), out(), ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.infer_shape(pack(extra=[("float16", (64, 128))]))[0] == E["ERROR_INVALID_TENSOR_INI_MATCH"]
+    assert op.infer_shape(pack())[0] == E["ERROR_INVALID_IN_TENSOR_NUM"]
     op.close()
 
 

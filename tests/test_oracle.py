@@ -426,6 +426,74 @@ def test_attention_head_major_blocks_by_flat_addresses(oracle):
     assert np.abs(other - got).max() > 1e-2
 
 
+def _compressed_twin(kc, vc, tables, ctx, n):
+    """The head-compressed form of an ordinary paged cache: block b * n + g holds head g of block b,
+    and pair (sequence s, head g) gets the table row of s mapped the same way."""
+    pool, block = kc.shape[:2]
+    kc_c = np.ascontiguousarray(kc.transpose(0, 2, 1, 3)).reshape(pool * n, block, 1, kc.shape[3])
+    vc_c = np.ascontiguousarray(vc.transpose(0, 2, 1, 3)).reshape(pool * n, block, 1, vc.shape[3])
+    tables_c = (np.repeat(tables, n, axis=0) * n + np.tile(np.arange(n), len(tables))[:, None]).astype(np.int32)
+    return kc_c, vc_c, tables_c, np.repeat(ctx, n).astype(np.int32)
+
+
+@pytest.mark.parametrize("mask_kind", [None, "norm3", "alibi4", "alibi4_1", "alibi3", "razor"])
+def test_head_compression_equals_ordinary_attention_on_the_twin_cache(oracle, mask_kind):
+    """With equal lengths for all KV heads of a sequence, attention over (sequence, KV head) pairs is
+    ordinary GQA attention on a rearranged cache: checked against the loop version on the ordinary
+    cache, masks and the per-slot score offsets (as a dense bias of offset * scale) included."""
+    rng = _rng(31)
+    heads, n, d, dv, block, pool = 6, 3, 16, 8, 4, 23
+    ctx = np.array([9, 0, 4, 13], dtype=np.int32)
+    tables = rng.permutation(pool)[:16].reshape(4, 4).astype(np.int32)
+    q = rng.standard_normal((3, heads, d)).astype(np.float32)
+    kc = rng.standard_normal((pool, block, n, d)).astype(np.float32)
+    vc = rng.standard_normal((pool, block, n, dv)).astype(np.float32)
+    kc_c, vc_c, tables_c, ctx_c = _compressed_twin(kc, vc, tables, ctx, n)
+    max_len, scale = 16, 0.3
+    mask = razor = None
+    dense = np.zeros((4, heads, max_len), dtype=np.float32)
+    per_head = None
+    if mask_kind == "norm3":
+        mask = rng.standard_normal((4, 1, max_len)).astype(np.float32)
+        dense[:] = mask
+    elif mask_kind == "alibi4":
+        mask = rng.standard_normal((4, heads, 1, max_len)).astype(np.float32)
+        dense[:] = mask[:, :, 0]
+    elif mask_kind == "alibi4_1":
+        mask = rng.standard_normal((4, 1, 1, max_len)).astype(np.float32)
+        dense[:] = mask[:, :, 0]
+    elif mask_kind == "alibi3":
+        mask = rng.standard_normal((heads, 1, max_len)).astype(np.float32)
+        dense[:] = mask[None, :, 0]
+        per_head = True
+    elif mask_kind == "razor":
+        razor = rng.uniform(0, 20, size=(pool * n, block)).astype(np.float32)
+        for i in range(4):
+            for h in range(heads):
+                for j in range(int(ctx[i])):
+                    dense[i, h, j] = razor[tables[i, j // block] * n + h // (heads // n), j % block] * scale
+    got = oracle.paged_attention(q, kc_c, vc_c, tables_c, ctx_c, scale, mask=mask, mask_per_head=per_head,
+                                 compress_kv_heads=n, razor_offset=razor)
+    want = oracle.paged_attention_loops(q, kc, vc, tables, ctx, scale, dense_bias=dense)
+    np.testing.assert_allclose(got, want, rtol=3e-5, atol=3e-6)
+
+
+def test_head_compression_int8_takes_the_descale_slice_of_its_kv_head(oracle):
+    rng = _rng(32)
+    heads, n, d, block, pool = 8, 2, 16, 4, 9
+    ctx = np.array([7, 16], dtype=np.int32)
+    tables = rng.permutation(pool)[:8].reshape(2, 4).astype(np.int32)
+    q = rng.standard_normal((2, heads, d)).astype(np.float32)
+    kc = rng.integers(-5, 6, size=(pool, block, n, d)).astype(np.int8)
+    vc = rng.integers(-5, 6, size=(pool, block, n, d)).astype(np.int8)
+    ks, vs = (rng.uniform(0.1, 1.0, size=n * d).astype(np.float32) for _ in range(2))
+    ko, vo = (rng.integers(-3, 4, size=n * d).astype(np.int32) for _ in range(2))
+    kc_c, vc_c, tables_c, ctx_c = _compressed_twin(kc, vc, tables, ctx, n)
+    got = oracle.paged_attention(q, kc_c, vc_c, tables_c, ctx_c, 0.25, ks, ko, vs, vo, compress_kv_heads=n)
+    want = oracle.paged_attention(q, kc, vc, tables, ctx, 0.25, ks, ko, vs, vo)  # pinned by its own tests
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5)
+
+
 def test_attention_matches_torch_sdpa(oracle):
     """Gathering the rows densely reduces the op to textbook attention."""
     rng = _rng(3)
