@@ -4,9 +4,10 @@
 // :124-158 tensor counts / InferShape, :176-319 dim checks), launching the
 // gfx950 copy kernel through the C ABI.
 //
-// Supported: COMPRESS_TYPE_UNDEFINED with K_CACHE_V_CACHE (key + value
-// caches) or K_CACHE_V_BYPASS (key cache only). Head compression and
-// fractal-NZ caches are Ascend-specific and rejected at creation.
+// Supported: K_CACHE_V_CACHE (key + value caches), also with head compression
+// (COMPRESS_TYPE_KVHEAD: + wins, seqLens; COMPRESS_TYPE_KVHEAD_ROPE: + wins,
+// seqLens, offsetIndex), and K_CACHE_V_BYPASS (key cache only). Fractal-NZ
+// caches are an Ascend cube-unit layout and rejected at creation.
 #include <new>
 #include "atb/infer_op_params.h"
 #include "atb/utils.h"
@@ -18,16 +19,21 @@ namespace atb {
 namespace {
 using Param = infer::ReshapeAndCacheParam;
 
-OpIr MakeIr(bool siso)
+// extra: the int32 inputs after slotMapping (reference ops_configs/atb_ops_info.ini:851-908)
+OpIr MakeIr(bool siso, int extra = 0)
 {
     OpIr ir;
     for (aclDataType t : {ACL_FLOAT16, ACL_INT8, ACL_BF16}) {
         IrCombo c;
+        if (extra == 3 && t == ACL_INT8) {
+            continue; // the window mean is built for 16-bit rows only
+        }
         if (siso) {
             c.inDtypes = {t, t, ACL_INT32};
             c.outDtypes = {t};
         } else {
             c.inDtypes = {t, t, t, t, ACL_INT32};
+            c.inDtypes.insert(c.inDtypes.end(), extra, ACL_INT32);
             c.outDtypes = {t, t};
         }
         c.inFormats.assign(c.inDtypes.size(), ACL_FORMAT_ND);
@@ -53,14 +59,19 @@ bool SameDesc(const TensorDesc &a, const TensorDesc &b)
 class ReshapeAndCacheOperation : public OperationBase {
 public:
     explicit ReshapeAndCacheOperation(const Param &param)
-        : OperationBase("ReshapeAndCacheOperation"), param_(param), siso_(param.kvCacheCfg == Param::K_CACHE_V_BYPASS)
+        : OperationBase("ReshapeAndCacheOperation"), param_(param), siso_(param.kvCacheCfg == Param::K_CACHE_V_BYPASS),
+          extra_(param.compressType == Param::COMPRESS_TYPE_KVHEAD ? 2
+                 : param.compressType == Param::COMPRESS_TYPE_KVHEAD_ROPE ? 3 : 0)
     {
         static const OpIr normal = MakeIr(false);
         static const OpIr single = MakeIr(true);
-        ir_ = siso_ ? &single : &normal;
+        static const OpIr keepLast = MakeIr(false, 2);
+        static const OpIr meanWindow = MakeIr(false, 3);
+        ir_ = siso_ ? &single : extra_ == 2 ? &keepLast : extra_ == 3 ? &meanWindow : &normal;
     }
 
-    uint32_t GetInputNum() const override { return siso_ ? 3 : 5; }
+    // reference :124-136: + wins, seqLens (+ offsetIndex) under head compression
+    uint32_t GetInputNum() const override { return siso_ ? 3 : 5 + extra_; }
     uint32_t GetOutputNum() const override { return siso_ ? 1 : 2; }
 
 protected:
@@ -105,6 +116,25 @@ protected:
         // (src/kernels/mixkernels/reshape_and_cache/reshape_and_cache_operation.cpp:95-196):
         // slot count equals token count.
         const Tensor &slots = pack.inTensors.at(siso_ ? 2 : 4);
+        if (extra_ > 0) {
+            // reference kernel library reshape_and_cache_operation.cpp:198-229,246-275: one slot, window (and
+            // offset) per (sequence, head) pair
+            const Tensor &seqLens = pack.inTensors.at(6);
+            if (pack.inTensors.at(5).desc.shape.dimNum != 1 || seqLens.desc.shape.dimNum != 1 ||
+                (extra_ == 3 && pack.inTensors.at(7).desc.shape.dimNum != 1)) {
+                ATB_LOG(ERROR) << "ReshapeAndCache: wins, seqLens and offsetIndex should have one dim";
+                return ERROR_INVALID_PARAM;
+            }
+            const int64_t pairs = seqLens.desc.shape.dims[0] * pack.inTensors.at(0).desc.shape.dims[1];
+            if (slots.desc.shape.dims[0] != pairs || pack.inTensors.at(5).desc.shape.dims[0] != pairs ||
+                (extra_ == 3 && pack.inTensors.at(7).desc.shape.dims[0] != pairs)) {
+                ATB_LOG(ERROR) << "ReshapeAndCache: slotMapping, wins and offsetIndex should have batch * numHeads = "
+                               << pairs << " entries";
+                return ERROR_INVALID_PARAM;
+            }
+            workspaceSize = 0;
+            return NO_ERROR;
+        }
         if (slots.desc.shape.dims[0] != pack.inTensors.at(0).desc.shape.dims[0]) {
             ATB_LOG(ERROR) << "ReshapeAndCache: slotMapping length must equal the token count";
             return ERROR_INVALID_PARAM;
@@ -143,6 +173,19 @@ protected:
             ATB_LOG(ERROR) << "ReshapeAndCache: key / keyCache / slotMapping device pointer is null";
             return ERROR_INVALID_PARAM;
         }
+        if (extra_ > 0) {
+            const int32_t dtype = key.desc.dtype == ACL_INT8 ? ATBMI_INT8 : key.desc.dtype == ACL_BF16 ? ATBMI_BF16 : ATBMI_F16;
+            int rc = atbmi_reshape_and_cache_compress(
+                key.deviceData, value, keyCacheOut.deviceData, valueCache, static_cast<const int32_t *>(slots.deviceData),
+                static_cast<const int32_t *>(pack.inTensors.at(5).deviceData),
+                static_cast<const int32_t *>(pack.inTensors.at(6).deviceData),
+                extra_ == 3 ? static_cast<const int32_t *>(pack.inTensors.at(7).deviceData) : nullptr,
+                pack.inTensors.at(6).desc.shape.dims[0], heads, dk, tokens, numSlots, dtype, stream);
+            if (rc != 0) {
+                ATB_LOG(ERROR) << "ReshapeAndCache launch failed: " << atbmi_last_error();
+            }
+            return rc;
+        }
         int rc = atbmi_reshape_and_cache(key.deviceData, value, keyCacheOut.deviceData, valueCache,
                                          static_cast<const int32_t *>(slots.deviceData), tokens, heads, dk, dv,
                                          numSlots, elemBytes, stream);
@@ -173,7 +216,21 @@ private:
             ATB_LOG(ERROR) << "ReshapeAndCache: caches must agree on numBlocks and blockSize";
             return ERROR_INVALID_TENSOR_DIM;
         }
-        if (k.dims[1] != kc.dims[2] || v.dims[1] != vc.dims[2]) {
+        if (extra_ > 0) {
+            // reference :286-305: one head per cache slot, equal head sizes, a multiple of 32
+            if (k.dims[2] != v.dims[2] || k.dims[2] != kc.dims[3] || k.dims[2] != vc.dims[3]) {
+                ATB_LOG(ERROR) << "ReshapeAndCache: head compress key, value and cache headSizes should be same";
+                return ERROR_INVALID_TENSOR_DIM;
+            }
+            if (kc.dims[2] != 1 || vc.dims[2] != 1) {
+                ATB_LOG(ERROR) << "ReshapeAndCache: dim 2 of head compress keyCache and valueCache should be 1";
+                return ERROR_INVALID_TENSOR_DIM;
+            }
+            if (k.dims[2] % 32 != 0) {
+                ATB_LOG(ERROR) << "ReshapeAndCache: head compress headSizes must be a multiple of 32";
+                return ERROR_INVALID_TENSOR_DIM;
+            }
+        } else if (k.dims[1] != kc.dims[2] || v.dims[1] != vc.dims[2]) {
             ATB_LOG(ERROR) << "ReshapeAndCache: head count of key/value must equal that of the caches";
             return ERROR_INVALID_TENSOR_DIM;
         }
@@ -202,6 +259,7 @@ private:
 
     Param param_;
     bool siso_;
+    uint32_t extra_; // int32 inputs after slotMapping: 2 (wins, seqLens) or 3 (+ offsetIndex) under head compression
 };
 } // namespace
 
@@ -223,8 +281,8 @@ template <> Status CreateOperation(const infer::ReshapeAndCacheParam &opParam, O
         ATB_LOG(ERROR) << "ReshapeAndCacheParam: compressType needs K_CACHE_V_CACHE";
         return ERROR_INVALID_PARAM;
     }
-    if (opParam.compressType != Param::COMPRESS_TYPE_UNDEFINED || opParam.kvCacheCfg == Param::K_CACHE_V_CACHE_NZ) {
-        ATB_LOG(ERROR) << "ReshapeAndCacheParam: head compression and NZ caches are not implemented on MI355X";
+    if (opParam.kvCacheCfg == Param::K_CACHE_V_CACHE_NZ) {
+        ATB_LOG(ERROR) << "ReshapeAndCacheParam: NZ caches are not implemented on MI355X";
         return ERROR_INVALID_PARAM;
     }
     *operation = new (std::nothrow) ReshapeAndCacheOperation(opParam);

@@ -65,6 +65,28 @@ int atbmi_reshape_and_cache(const void *keyDevice, const void *valueDevice, void
                             int32_t elemBytes, void *stream);
 
 /*
+ * KV-cache write under head compression (ReshapeAndCacheParam::compressType): the caches hold one head per
+ * slot, [numSlots, headSize], and pair i = b * numHeads + h (sequence b of `batch`, head h) owns the slots from
+ * slotMapping[i] on (slotMapping[i] < 0 skips the pair). Sequence b is the seqLens[b] rows of key / value
+ * [numTokens, numHeads, headSize] after those of the sequences before it. All index tensors are device memory.
+ *   offsetIndex == NULL (COMPRESS_TYPE_KVHEAD): the last wins[i] tokens of the sequence, head h, in order.
+ *   offsetIndex != NULL (COMPRESS_TYPE_KVHEAD_ROPE), o = offsetIndex[i]: o == -1 copies the whole sequence;
+ *     otherwise the tokens before o, then ONE slot with the mean of the wins[i] tokens from o on (fp32 sum in
+ *     token order, divided by wins[i], rounded to nearest even), then the tokens after the window; wins[i] == 0
+ *     copies everything. fp16 / bf16 only.
+ * Rows that would be read outside key / value or written outside the caches are left out.
+ * Replaces: reshape_and_cache_compress.cpp / reshape_and_cache_compress_rope.cpp of the reference
+ * (src/kernels/mixkernels/reshape_and_cache/op_kernel/; goldens tests/apitest/kernelstest/mix/
+ * test_reshape_and_cache_wins.py:61-88 and test_reshape_and_cache_wins_rope.py:78-131).
+ */
+int atbmi_reshape_and_cache_compress(const void *keyDevice, const void *valueDevice, void *keyCacheDevice,
+                                     void *valueCacheDevice, const int32_t *slotMappingDevice,
+                                     const int32_t *winsDevice, const int32_t *seqLensDevice,
+                                     const int32_t *offsetIndexDevice, int64_t batch, int64_t numHeads,
+                                     int64_t headSize, int64_t numTokens, int64_t numSlots, int32_t dtype,
+                                     void *stream);
+
+/*
  * KV-cache write from strided views of key / value: element (token, head, channel) of key is read
  * keyOffset + token * keyStrides[0] + head * keyStrides[1] + channel * keyStrides[2] ELEMENTS from
  * keyDevice (the same for value); everything else as atbmi_reshape_and_cache. The stride arrays are

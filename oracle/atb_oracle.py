@@ -99,6 +99,66 @@ def reshape_and_cache(key, value, key_cache, value_cache, slot_mapping):
     return kc, vc
 
 
+def reshape_and_cache_compress(key, value, key_cache, value_cache, slot_mapping, wins, seq_lens, offset_index=None,
+                               out_dtype=None):
+    """KV-cache write under head compression; caches [blocks, block, 1, D] (copied and returned).
+    Pair i = b * heads + h owns the slots from slot_mapping[i] on (negative: skipped); sequence b is
+    the seq_lens[b] rows of key / value [tokens, heads, D] after those of the sequences before it.
+    offset_index None (COMPRESS_TYPE_KVHEAD; reference golden
+    tests/apitest/kernelstest/mix/test_reshape_and_cache_wins.py:61-88): the last wins[i] tokens of
+    the sequence, head h, in order.
+    offset_index given (COMPRESS_TYPE_KVHEAD_ROPE; golden test_reshape_and_cache_wins_rope.py:78-131):
+    o = offset_index[i] == -1 copies the whole sequence; otherwise the tokens before o, one slot
+    with the mean of the wins[i] tokens from o on, then the tokens after the window (wins[i] == 0:
+    everything is copied). The mean is an fp32 sum in token order divided by wins[i]; the golden
+    keeps it in fp32, the reference's device kernel rounds it to the cache dtype, nearest even
+    (src/kernels/mixkernels/reshape_and_cache/op_kernel/reshape_and_cache_compress_rope.cpp:92-100):
+    out_dtype ("float16" / "bf16") applies that rounding, None leaves the fp32 value."""
+    kc = np.array(key_cache, copy=True)
+    vc = np.array(value_cache, copy=True)
+    heads = key.shape[1]
+    block = kc.shape[1]
+    ends = np.cumsum(np.asarray(seq_lens, dtype=np.int64))
+    starts = ends - np.asarray(seq_lens, dtype=np.int64)
+
+    def put(slot, k_row, v_row):
+        kc[slot // block, slot % block, 0] = k_row
+        vc[slot // block, slot % block, 0] = v_row
+
+    for i, slot in enumerate(np.asarray(slot_mapping).tolist()):
+        if slot < 0:
+            continue
+        b, h = divmod(i, heads)
+        win = int(wins[i])
+        if offset_index is None:
+            for j in range(win):
+                tok = int(ends[b]) - win + j
+                put(slot + j, key[tok, h], value[tok, h])
+            continue
+        off = int(offset_index[i])
+        for j in range(int(seq_lens[b])):
+            tok = int(starts[b]) + j
+            if off == -1 or j < off or (win == 0 and j >= off):
+                put(slot, key[tok, h], value[tok, h])
+                slot += 1
+            elif j == off:
+                k_sum = np.zeros(key.shape[2], dtype=np.float32)
+                v_sum = np.zeros(value.shape[2], dtype=np.float32)
+                for t in range(tok, tok + win):
+                    k_sum = k_sum + key[t, h].astype(np.float32)
+                    v_sum = v_sum + value[t, h].astype(np.float32)
+                k_mean = k_sum / np.float32(win)
+                v_mean = v_sum / np.float32(win)
+                if out_dtype is not None:
+                    k_mean, v_mean = round_to(k_mean, out_dtype), round_to(v_mean, out_dtype)
+                put(slot, k_mean, v_mean)
+                slot += 1
+            elif j >= off + win:
+                put(slot, key[tok, h], value[tok, h])
+                slot += 1
+    return kc, vc
+
+
 def strided_view(storage, shape, strides, offset):
     """The [tokens, heads, head_size] view that ReshapeAndCacheWithStride reads: element
     (t, h, d) is storage.flat[offset + t * strides[0] + h * strides[1] + d * strides[2]],

@@ -169,6 +169,77 @@ def test_reshape_and_cache_with_stride_bit_exact(binding, oracle, dev, stream, c
     ctx.close()
 
 
+# batch, heads, head size, block, dtype, sequence lengths (lo, hi)
+COMPRESS_WRITE_CASES = [
+    (2, 4, 128, 128, torch.float16, (300, 700)),     # reference test_reshape_and_cache_wins.py shapes, shorter
+    (5, 8, 128, 128, torch.bfloat16, (1, 400)),
+    (3, 2, 64, 16, torch.int8, (50, 200)),
+    (4, 8, 128, 128, torch.float16, (1024, 4096)),   # reference test_reshape_and_cache_wins_rope.py lengths
+    (1, 1, 32, 16, torch.bfloat16, (17, 18)),
+]
+
+
+@pytest.mark.parametrize("mean_window", [False, True], ids=["keep_last", "mean_window"])
+@pytest.mark.parametrize("case", COMPRESS_WRITE_CASES, ids=lambda c: "b%d_h%d_d%d_bs%d_%s" % (
+    c[0], c[1], c[2], c[3], str(c[4]).split(".")[-1]))
+def test_reshape_and_cache_head_compression_bit_exact(binding, oracle, dev, stream, case, mean_window):
+    """ReshapeAndCacheParam::compressType KVHEAD (the last wins[i] tokens of each (sequence, head) pair) and
+    KVHEAD_ROPE (a window of tokens replaced by its mean), bit for bit against the oracle; slots outside the
+    pairs' stretches keep their contents."""
+    batch, heads, d, block, dtype, (lo, hi) = case
+    if mean_window and dtype == torch.int8:
+        pytest.skip("the window mean is defined for 16-bit rows")
+    rng = _rng(900 + batch + heads + d)
+    seq = rng.integers(lo, hi, size=batch).astype(np.int32)
+    tokens = int(seq.sum())
+    pairs = batch * heads
+    per_seq = np.repeat(seq, heads)
+    wins = np.minimum(rng.integers(0, hi, size=pairs), per_seq).astype(np.int32)
+    offs = None
+    if mean_window:
+        offs = np.array([rng.integers(-1, n - w + 1) for n, w in zip(per_seq, wins)], dtype=np.int32)
+        offs[0] = -1
+        wins[min(1, pairs - 1)] = min(1, wins[min(1, pairs - 1)])
+        need = np.where((offs < 0) | (wins == 0), per_seq, per_seq - wins + 1)
+    else:
+        need = wins
+    # every pair gets whole blocks of its own, in shuffled order; one pair is skipped
+    order = rng.permutation(pairs)
+    nblocks = (need + block - 1) // block
+    first = np.zeros(pairs, dtype=np.int64)
+    first[order] = np.concatenate([[0], np.cumsum(nblocks[order])[:-1]])
+    slots = (first * block).astype(np.int32)
+    if pairs > 2:
+        slots[2] = -1
+    blocks = int(nblocks.sum()) + 2
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(int(rng.integers(1 << 30)))
+    if dtype == torch.int8:
+        mk = lambda *shape: torch.randint(-128, 128, shape, generator=gen, dtype=torch.int8)
+    else:
+        mk = lambda *shape: ((torch.rand(shape, generator=gen) * 10 - 5)).to(dtype)
+    key, value = mk(tokens, heads, d), mk(tokens, heads, d)
+    kc0, vc0 = mk(blocks, block, 1, d), mk(blocks, block, 1, d)
+    ins = [key.to(dev), value.to(dev), kc0.to(dev), vc0.to(dev), torch.from_numpy(slots).to(dev),
+           torch.from_numpy(wins).to(dev), torch.from_numpy(seq).to(dev)]
+    if mean_window:
+        ins.append(torch.from_numpy(offs).to(dev))
+    c = binding.Context(stream)
+    op = binding.OperationRunner("ReshapeAndCacheOperation",
+                                 binding.ReshapeAndCacheParam(compressType=2 if mean_window else 1), c)
+    with torch.cuda.stream(stream):
+        op.run(ins, outputs=[ins[2], ins[3]])
+    stream.synchronize()
+    op.close()
+    c.close()
+    od = {torch.float16: "float16", torch.bfloat16: "bf16", torch.int8: None}[dtype]
+    want_k, want_v = oracle.reshape_and_cache_compress(
+        to_oracle(key), to_oracle(value), to_oracle(kc0), to_oracle(vc0), slots, wins, seq, offs, out_dtype=od)
+    for got, want, what in ((ins[2], want_k, "key"), (ins[3], want_v, "value")):
+        want_t = torch.from_numpy(np.ascontiguousarray(want)).to(dtype)
+        assert torch.equal(_bits(got.cpu()), _bits(want_t)), what
+
+
 def test_reshape_and_cache_with_stride_equals_plain_on_contiguous_input(binding, dev, stream):
     """With the strides of a contiguous tensor and offset 0 the operation is ReshapeAndCache."""
     rng = _rng(32)
@@ -826,6 +897,53 @@ def test_head_compression_through_operation_api(binding, oracle, dev, stream, ca
     if razor or kind is not None:  # the offsets / the mask matter in this case
         plain = oracle_pa(oracle, q_model, kc, vc, tables, ctx, scale, ks, ko, vs, vo, compress_kv_heads=n, out_init=7.0)
         assert np.abs(want - plain).max() > 0.01
+
+
+def test_compressed_write_then_compressed_attention(binding, oracle, dev, stream):
+    """The two halves of head compression together: ReshapeAndCache (KVHEAD) keeps the last wins[i] tokens of
+    every (sequence, KV head) pair, PagedAttention (KVHEAD) attends over them; the result is plain attention
+    of each head group over its own window of the uncompressed keys and values."""
+    rng = _rng(955)
+    batch, heads, n, d, block = 3, 16, 4, 128, 128
+    seq = rng.integers(200, 600, size=batch).astype(np.int32)
+    wins = np.array([rng.integers(1, s + 1) for s in np.repeat(seq, n)], dtype=np.int32)
+    nblocks = (wins + block - 1) // block
+    first = np.concatenate([[0], np.cumsum(nblocks)[:-1]])
+    slots = (first * block).astype(np.int32)
+    blocks = int(nblocks.sum()) + 1
+    tables = np.zeros((batch * n, int(nblocks.max())), dtype=np.int32)
+    for i in range(batch * n):
+        tables[i, :nblocks[i]] = first[i] + np.arange(nblocks[i])
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(9)
+    mk = lambda *shape: (torch.rand(shape, generator=gen) * 2 - 1).to(torch.float16)
+    key, value, q = mk(int(seq.sum()), n, d), mk(int(seq.sum()), n, d), mk(batch, heads, d)
+    kc = torch.zeros((blocks, block, 1, d), dtype=torch.float16, device=dev)
+    vc = torch.zeros_like(kc)
+    c = binding.Context(stream)
+    rac = binding.OperationRunner("ReshapeAndCacheOperation", binding.ReshapeAndCacheParam(compressType=1), c)
+    scale = 1.0 / math.sqrt(d)
+    pa = binding.OperationRunner("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=heads, kvHeadNum=n, qkScale=scale, compressType=1), c)
+    lens = torch.from_numpy(wins)
+    with torch.cuda.stream(stream):
+        rac.run([key.to(dev), value.to(dev), kc, vc, torch.from_numpy(slots).to(dev), lens.to(dev),
+                 torch.from_numpy(seq).to(dev)], outputs=[kc, vc])
+        out, = pa.run([q.to(dev), kc, vc, torch.from_numpy(tables).to(dev), lens.to(dev)], host_inputs={4: lens})
+    stream.synchronize()
+    rac.close()
+    pa.close()
+    c.close()
+    group = heads // n
+    ends = np.cumsum(seq)
+    want = np.zeros((batch, heads, d), dtype=np.float32)
+    for i in range(batch * n):
+        b, g = divmod(i, n)
+        rows = slice(int(ends[b]) - int(wins[i]), int(ends[b]))
+        want[b, g * group:(g + 1) * group] = oracle.attention_one(
+            to_oracle(q)[b, g * group:(g + 1) * group], to_oracle(key)[rows, g:g + 1], to_oracle(value)[rows, g:g + 1],
+            np.float32(scale))
+    assert_close(out, want, TOL[torch.float16], "write + attention")
 
 
 def test_c1_decode_step_through_operation_api(binding, oracle, pkg, dev, stream):

@@ -60,7 +60,7 @@ def _pa_mask_shape_refused(case):
 
 
 def _rac_unimplemented(p):
-    return p.get("compressType", 0) in (1, 2) or p.get("kvCacheCfg", 0) == 2
+    return p.get("kvCacheCfg", 0) == 2
 
 
 def _mla_unimplemented(p):
@@ -252,7 +252,7 @@ def test_table_coverage():
               _pa_mask_shape_refused(c)]
     rac_dev = [c for c in RAC_CASES if _rac_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
     assert len(PA_CASES) == 81 and len(PA_CASES) - len(pa_dev) >= 75
-    assert len(RAC_CASES) == 38 and len(RAC_CASES) - len(rac_dev) >= 26
+    assert len(RAC_CASES) == 38 and len(RAC_CASES) - len(rac_dev) >= 29
     # most MultiLatentAttention rows exercise the prefill calcType and the fractal-NZ caches, which are not built
     mla_dev = [c for c in MLA_CASES if _mla_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
     assert len(MLA_CASES) == 147 and len(MLA_CASES) - len(mla_dev) == 45
@@ -737,6 +737,46 @@ def test_paged_attention_head_compression_checks(binding, ctx):
     assert op.infer_shape(pack(extra=[("float16", (64, 128))]))[0] == E["ERROR_INVALID_TENSOR_INI_MATCH"]
     assert op.infer_shape(pack())[0] == E["ERROR_INVALID_IN_TENSOR_NUM"]
     op.close()
+
+
+def test_reshape_and_cache_head_compression_checks(binding, ctx):
+    """ReshapeAndCacheParam::compressType (reference reshape_and_cache_operation.cpp:61-80 create, :124-136 input
+    counts, :286-305 dim rules; kernel library reshape_and_cache_operation.cpp:198-229,246-275 for the index tensors)."""
+    E = binding.ERROR_CODE
+    P = binding.ReshapeAndCacheParam
+    for bad in (P(compressType=3), P(compressType=-1), P(compressType=1, kvCacheCfg=1), P(compressType=2, kvCacheCfg=2)):
+        assert binding.Operation("ReshapeAndCacheOperation", bad).status == E["ERROR_INVALID_PARAM"]
+    mk = binding.make_tensor
+
+    def pack(n_extra, dtype="float16", key=(100, 4, 128), value=(100, 4, 128), kc=(32, 128, 1, 128), vc=(32, 128, 1, 128),
+             pairs=8, batch=2, extra_dtype="int32"):
+        t = [mk(dtype, key, FAKE_DEVICE), mk(dtype, value, FAKE_DEVICE), mk(dtype, kc, FAKE_DEVICE),
+             mk(dtype, vc, FAKE_DEVICE), mk("int32", (pairs,), FAKE_DEVICE), mk(extra_dtype, (pairs,), FAKE_DEVICE),
+             mk("int32", (batch,), FAKE_DEVICE)]
+        if n_extra == 3:
+            t.append(mk("int32", (pairs,), FAKE_DEVICE))
+        return t
+
+    outs = lambda dtype="float16": [mk(dtype, (32, 128, 1, 128), FAKE_DEVICE) for _ in range(2)]
+    for compress, n_extra in ((1, 2), (2, 3)):
+        op = binding.Operation("ReshapeAndCacheOperation", P(compressType=compress))
+        assert op.status == 0 and op.input_num() == 5 + n_extra and op.output_num() == 2
+        st, descs = op.infer_shape(pack(n_extra))
+        assert st == 0 and [descs[1].dims[i] for i in range(4)] == [32, 128, 1, 128]
+        assert op.setup(pack(n_extra), outs(), ctx) == (0, 0)
+        assert op.setup(pack(n_extra, dtype="bf16"), outs("bf16"), ctx) == (0, 0)
+        int8 = op.infer_shape(pack(n_extra, dtype="int8"))[0]
+        assert int8 == (0 if compress == 1 else E["ERROR_INVALID_TENSOR_INI_MATCH"])  # the window mean is 16-bit only
+        assert op.infer_shape(pack(n_extra, extra_dtype="int64"))[0] == E["ERROR_INVALID_TENSOR_INI_MATCH"]
+        assert op.infer_shape(pack(5 - n_extra))[0] == E["ERROR_INVALID_IN_TENSOR_NUM"]
+        assert op.infer_shape(pack(n_extra, kc=(32, 128, 4, 128), vc=(32, 128, 4, 128)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+        assert op.infer_shape(pack(n_extra, value=(100, 4, 64), vc=(32, 128, 1, 64)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+        assert op.infer_shape(pack(n_extra, key=(100, 4, 48), value=(100, 4, 48), kc=(32, 128, 1, 48),
+                                   vc=(32, 128, 1, 48)))[0] == E["ERROR_INVALID_TENSOR_DIM"]      # multiple of 32
+        assert op.infer_shape(pack(n_extra, value=(99, 4, 128)))[0] == E["ERROR_INVALID_TENSOR_DIM"]
+        assert op.setup(pack(n_extra, pairs=7), outs(), ctx)[0] == E["ERROR_INVALID_PARAM"]       # batch * heads entries
+        assert op.setup(pack(n_extra, batch=3), outs(), ctx)[0] == E["ERROR_INVALID_PARAM"]
+        op.close()
 
 
 def test_reshape_and_cache_with_stride_checks(binding, ctx):

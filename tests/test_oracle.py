@@ -385,6 +385,81 @@ def test_paged_cache_load_negative_block_ids_leave_their_rows(oracle):
     assert k[:, 0, 0].tolist() == [3.0, 4.0, 0.0, 0.0, 1.0] and np.array_equal(k, v)
 
 
+# ---------------------------------------------------------------- cache write under head compression
+def _compress_case(rng, batch=3, heads=4, d=32, block=16, dtype=np.float16):
+    seq = rng.integers(20, 60, size=batch).astype(np.int32)
+    tokens = int(seq.sum())
+    key = rng.integers(-8, 9, size=(tokens, heads, d)).astype(dtype)
+    value = rng.integers(-8, 9, size=(tokens, heads, d)).astype(dtype)
+    return seq, key, value
+
+
+def test_compress_keep_last_by_flat_addresses(oracle):
+    """COMPRESS_TYPE_KVHEAD against element-wise loops over flat addresses of key and cache."""
+    rng = _rng(41)
+    batch, heads, d, block = 3, 4, 32, 16
+    seq, key, value = _compress_case(rng, batch, heads, d, block)
+    wins = rng.integers(0, 20, size=batch * heads).astype(np.int32)
+    starts_of = np.concatenate([[0], np.cumsum((wins + block - 1) // block)[:-1]]) * block
+    slots = starts_of.astype(np.int32)
+    slots[5] = -1
+    blocks = int(((wins + block - 1) // block).sum()) + 1
+    kc0 = np.full((blocks, block, 1, d), 77, dtype=np.float16)
+    kc, vc = oracle.reshape_and_cache_compress(key, value, kc0, kc0, slots, wins, seq)
+    want_k, want_v = kc0.ravel().copy(), kc0.ravel().copy()
+    kf, vf = key.ravel(), value.ravel()
+    ends = np.cumsum(seq)
+    for i in range(batch * heads):
+        if slots[i] < 0:
+            continue
+        for j in range(int(wins[i])):
+            tok = int(ends[i // heads]) - int(wins[i]) + j
+            for c in range(d):
+                want_k[(slots[i] + j) * d + c] = kf[(tok * heads + i % heads) * d + c]
+                want_v[(slots[i] + j) * d + c] = vf[(tok * heads + i % heads) * d + c]
+    assert np.array_equal(kc.ravel(), want_k) and np.array_equal(vc.ravel(), want_v)
+    assert np.array_equal(kc0, np.full_like(kc0, 77))  # the inputs are not written
+
+
+def test_compress_mean_window_invariants(oracle):
+    """COMPRESS_TYPE_KVHEAD_ROPE: a pair fills seqLen - win + 1 slots (seqLen with no window); a window of one
+    token is that token, so the result equals the plain copy; the window's slot holds the mean of its
+    tokens (float64 mean as the yardstick) and its neighbours the tokens next to the window."""
+    rng = _rng(42)
+    batch, heads, d, block = 3, 2, 32, 16
+    seq, key, value = _compress_case(rng, batch, heads, d, block, np.float32)
+    key = key + rng.standard_normal(key.shape).astype(np.float32)
+    pairs = batch * heads
+    stride = 64  # slots per pair, generous
+    slots = (np.arange(pairs) * stride).astype(np.int32)
+    blocks = pairs * stride // block
+    marker = np.float32(-555.0)
+    kc0 = np.full((blocks, block, 1, d), marker, dtype=np.float32)
+    wins = np.array([5, 1, 0, 7, 20, 3], dtype=np.int32)
+    offs = np.array([3, 4, 2, -1, 0, int(seq[2]) - 3], dtype=np.int32)  # last: the window ends the sequence
+    kc, vc = oracle.reshape_and_cache_compress(key, value, kc0, kc0, slots, wins, seq, offs)
+    flat = kc.reshape(-1, d)
+    starts = np.cumsum(seq) - seq
+    for i in range(pairs):
+        b, h = divmod(i, heads)
+        n = int(seq[b]) if offs[i] == -1 or wins[i] == 0 else int(seq[b]) - int(wins[i]) + 1
+        used = flat[slots[i]:slots[i] + stride]
+        assert (used[:n] != marker).all() and (used[n:] == marker).all(), i
+        rows = key[starts[b]:starts[b] + seq[b], h]
+        if offs[i] == -1 or wins[i] <= 1:
+            assert np.array_equal(used[:n], rows), i
+            continue
+        o, w = int(offs[i]), int(wins[i])
+        assert np.array_equal(used[:o], rows[:o]) and np.array_equal(used[o + 1:n], rows[o + w:]), i
+        np.testing.assert_allclose(used[o], rows[o:o + w].astype(np.float64).mean(axis=0), rtol=1e-5, atol=1e-6)
+    # rounding to the cache dtype, nearest even, is what the device kernel stores
+    k16 = key.astype(np.float16)
+    kc16, _ = oracle.reshape_and_cache_compress(k16, k16, kc0.astype(np.float16), kc0.astype(np.float16), slots, wins,
+                                                seq, offs, out_dtype="float16")
+    kc32, _ = oracle.reshape_and_cache_compress(k16, k16, kc0, kc0, slots, wins, seq, offs)
+    assert np.array_equal(kc16, kc32.astype(np.float16))
+
+
 # ---------------------------------------------------------------- attention
 def test_attention_matches_independent_loops(oracle):
     rng = _rng(2)
