@@ -4,7 +4,8 @@ prints one JSON line per operation: BlockCopy (512 blocks of 256 KB copied in ea
 PagedCacheLoad (all 158 839 cached rows of the 64 sequences gathered) and NormRopeReshape (the
 producer of the combined MLA cache, at the 65 536 tokens of the reference's kernel test) and Rope
 (8 192 tokens of a Llama-3-8B-shaped layer) and the per-channel quantiser / dequantiser of
-ElewiseOperation (3 072 x 16 384), through
+ElewiseOperation (3 072 x 16 384) and the head-compressed forms of ReshapeAndCache (4 sequences of 4 000
+tokens, windows of 1 501), through
 atb::Operation (Setup + Execute per call; NormRopeReshape, Rope and Elewise: Setup once). All are HBM-bound; `roofline.achieved` is their
 algorithmic bytes (every source byte read once, every destination byte written once) over the
 mean kernel time between HIP events on the launch stream.
@@ -169,6 +170,40 @@ def main():
         print(json.dumps({"operation": "ElewiseOperation (per-channel %s)" % name,
                           "workload": "%d x %d fp16 <-> int8, scale and offset per channel (Setup once, Execute per call)"
                           % (rows, ch), "ms_per_call": ms,
+                          "roofline": {"bound": "hbm", "achieved": alg / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
+                                       "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                                       "algorithmic_bytes": alg}}))
+        op.close()
+    # ---- ReshapeAndCache under head compression: 4 sequences of 4 000 tokens, 8 KV heads of 128 channels, bf16;
+    # windows of 1 501 tokens per (sequence, head) pair (the sizes of the reference's kernel test)
+    batch, heads, d, block, length, win = 4, 8, 128, 128, 4000, 1501
+    pairs = batch * heads
+    key = torch.randn((batch * length, heads, d), device=dev).to(torch.bfloat16)
+    value = torch.randn_like(key)
+    seq_d = torch.full((batch,), length, dtype=torch.int32, device=dev)
+    wins_d = torch.full((pairs,), win, dtype=torch.int32, device=dev)
+    for name, compress, rows_out in (("keep-last windows", 1, win), ("mean windows", 2, length - win + 1)):
+        per_pair = (rows_out + block - 1) // block
+        cache_k = torch.zeros((pairs * per_pair, block, 1, d), dtype=torch.bfloat16, device=dev)
+        cache_v = torch.zeros_like(cache_k)
+        slots_d = (torch.arange(pairs, dtype=torch.int32, device=dev) * (per_pair * block)).contiguous()
+        tensors = [key, value, cache_k, cache_v, slots_d, wins_d, seq_d]
+        if compress == 2:
+            tensors.append(torch.from_numpy(rng.integers(0, length - win + 1, size=pairs).astype(np.int32)).to(dev))
+        op = b.OperationRunner("ReshapeAndCacheOperation", b.ReshapeAndCacheParam(compressType=compress), ctx)
+        ins = [b.tensor_of(t) for t in tensors]
+        outs = [b.tensor_of(cache_k), b.tensor_of(cache_v)]
+        st, ws = op.op.setup(ins, outs, ctx)
+        assert st == 0 and ws == 0
+
+        def execute_compress():
+            assert op.op.execute(ins, outs, None, 0, ctx) == 0
+        ms = timed(execute_compress, stream, args.steps, args.warmup)
+        rows_in = win if compress == 1 else length
+        alg = 2 * pairs * (rows_in + rows_out) * d * 2
+        print(json.dumps({"operation": "ReshapeAndCacheOperation (head compression, %s)" % name,
+                          "workload": "%d sequences of %d tokens, %d heads of %d channels, windows of %d tokens, bf16 "
+                          "(Setup once, Execute per call)" % (batch, length, heads, d, win), "ms_per_call": ms,
                           "roofline": {"bound": "hbm", "achieved": alg / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
                                        "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                                        "algorithmic_bytes": alg}}))

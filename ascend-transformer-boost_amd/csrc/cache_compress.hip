@@ -24,6 +24,8 @@ namespace atbmi {
 namespace {
 
 constexpr int CC_THREADS = 256;
+constexpr int MEAN_STAGE_BYTES = 32768; // token rows of a window staged in LDS at a time
+constexpr int MEAN_MAX_CHANNELS = 1024; // head size the window mean is built for
 
 bool Aligned(const void *p, uintptr_t a)
 {
@@ -64,15 +66,15 @@ __device__ __forceinline__ int64_t SequenceStart(const int32_t *seqLens, int b, 
     return total;
 }
 
-// Copies `count` token rows of head h, from token `srcTok` on, to slots `dstSlot` on; the workgroups
-// of one pair (gridDim.y of them) share the rows. Rows outside the tensors are left out.
+// Copies `count` token rows of head h, from token `srcTok` on, to slots `dstSlot` on; `workers`
+// workgroups of the pair share the rows, this one is number `worker`. Rows outside the tensors are left out.
 __device__ __forceinline__ void CopyRows(const CompressArgs &a, int which, int h, int64_t srcTok, int64_t dstSlot,
-                                         int64_t count)
+                                         int64_t count, int worker, int workers)
 {
     const int pieces = a.rowBytes / 16;
     const int64_t total = count * pieces;
-    for (int64_t at = static_cast<int64_t>(blockIdx.y) * CC_THREADS + threadIdx.x; at < total;
-         at += static_cast<int64_t>(gridDim.y) * CC_THREADS) {
+    for (int64_t at = static_cast<int64_t>(worker) * CC_THREADS + threadIdx.x; at < total;
+         at += static_cast<int64_t>(workers) * CC_THREADS) {
         const int64_t j = at / pieces;
         const int p = static_cast<int>(at % pieces);
         const int64_t tok = srcTok + j;
@@ -98,7 +100,7 @@ __global__ __launch_bounds__(CC_THREADS) void CompressKeepLastKernel(const Compr
     const int h = pair % a.heads;
     const int64_t end = SequenceStart(a.seqLens, b, scratch) + a.seqLens[b];
     const int64_t win = a.wins[pair];
-    CopyRows(a, blockIdx.z, h, end - win, slot, win);
+    CopyRows(a, blockIdx.z, h, end - win, slot, win, blockIdx.y, gridDim.y);
 }
 
 template <bool BF16>
@@ -117,36 +119,90 @@ __global__ __launch_bounds__(CC_THREADS) void CompressMeanWindowKernel(const Com
     const int64_t len = a.seqLens[b];
     const int64_t off = a.offsets[pair];
     const int64_t win = a.wins[pair];
-    if (off < 0) {
-        CopyRows(a, which, h, start, slot, len);
+    if (off < 0 || win <= 0 || off >= len) { // no window: the whole sequence as it is
+        CopyRows(a, which, h, start, slot, len, blockIdx.y, gridDim.y);
         return;
     }
-    CopyRows(a, which, h, start, slot, min(off, len));
-    if (win <= 0) {
-        CopyRows(a, which, h, start + off, slot + off, len - off);
+    // The first workgroup of the pair takes the mean (the long pole: it starts at once), the others copy.
+    const bool solo = gridDim.y == 1;
+    if (blockIdx.y != 0 || solo) {
+        const int worker = solo ? 0 : blockIdx.y - 1;
+        const int workers = solo ? 1 : gridDim.y - 1;
+        CopyRows(a, which, h, start, slot, off, worker, workers);
+        CopyRows(a, which, h, start + off + win, slot + off + 1, len - off - win, worker, workers);
+    }
+    if (blockIdx.y != 0 || slot + off >= a.numSlots) {
         return;
     }
-    CopyRows(a, which, h, start + off + win, slot + off + 1, len - off - win);
-    if (blockIdx.y != 0 || off >= len || slot + off >= a.numSlots) {
-        return;
-    }
-    // The mean of the window: a thread owns a channel and adds its values in token order.
+    // The mean of the window. The order of the fp32 additions is fixed (token order), so the work of a
+    // channel cannot be split: the workgroup stages a run of token rows in LDS with all its lanes (16-byte
+    // pieces, many loads in flight), then every thread adds up its channels from there.
+    __shared__ __align__(16) uint8_t stage[MEAN_STAGE_BYTES];
     const int channels = a.rowBytes / 2;
-    const uint16_t *src = reinterpret_cast<const uint16_t *>(a.src[which]);
-    uint16_t *dst = reinterpret_cast<uint16_t *>(a.dst[which]);
-    for (int c = threadIdx.x; c < channels; c += CC_THREADS) {
-        float sum = 0.0f;
-        const int64_t first = start + off;
-#pragma unroll 8
-        for (int64_t k = 0; k < win; ++k) {
-            const int64_t tok = first + k;
-            if (tok < a.numTokens) {
-                const uint16_t raw = src[(tok * a.heads + h) * channels + c];
-                sum += BF16 ? Bf16ToFloat(raw) : HalfBitsToFloat(raw);
+    const int pieces = a.rowBytes / 16;
+    const int chunkTokens = MEAN_STAGE_BYTES / a.rowBytes;
+    const int64_t first = start + off;
+    const int64_t inRange = a.numTokens - first < win ? a.numTokens - first : win;
+    const uint8_t *src = a.src[which];
+    const uint16_t *staged = reinterpret_cast<const uint16_t *>(stage);
+    float sum[MEAN_MAX_CHANNELS / CC_THREADS];
+#pragma unroll
+    for (int i = 0; i < MEAN_MAX_CHANNELS / CC_THREADS; ++i) {
+        sum[i] = 0.0f;
+    }
+    for (int64_t k0 = 0; k0 < inRange; k0 += chunkTokens) {
+        const int count = static_cast<int>(inRange - k0 < chunkTokens ? inRange - k0 : chunkTokens);
+        __syncthreads(); // the previous run has been added up
+        constexpr int HELD = MEAN_STAGE_BYTES / 16 / CC_THREADS; // 16-byte pieces per thread and run
+        uint4 held[HELD];
+#pragma unroll
+        for (int u = 0; u < HELD; ++u) { // all loads of the run first (lanes past its end repeat its last piece)
+            const int last = count * pieces - 1;
+            const int at = threadIdx.x + u * CC_THREADS < last ? threadIdx.x + u * CC_THREADS : last;
+            held[u] = *reinterpret_cast<const uint4 *>(
+                src + ((first + k0 + at / pieces) * a.heads + h) * a.rowBytes + (at % pieces) * 16);
+        }
+#pragma unroll
+        for (int u = 0; u < HELD; ++u) {
+            const int at = threadIdx.x + u * CC_THREADS;
+            if (at < count * pieces) {
+                *reinterpret_cast<uint4 *>(stage + static_cast<size_t>(at) * 16) = held[u];
             }
         }
-        const float mean = sum / static_cast<float>(static_cast<int32_t>(win));
-        dst[(slot + off) * channels + c] = BF16 ? FloatToBf16(mean) : FloatToHalfBits(mean);
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < MEAN_MAX_CHANNELS / CC_THREADS; ++i) {
+            const int c = threadIdx.x + i * CC_THREADS;
+            if (c < channels) {
+                float acc = sum[i];
+                int j = 0;
+                for (; j + 16 <= count; j += 16) { // sixteen LDS reads in flight, then the additions in order
+                    uint16_t raw[16];
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) {
+                        raw[u] = staged[(j + u) * channels + c];
+                    }
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) {
+                        acc += BF16 ? Bf16ToFloat(raw[u]) : HalfBitsToFloat(raw[u]);
+                    }
+                }
+                for (; j < count; ++j) {
+                    const uint16_t raw = staged[j * channels + c];
+                    acc += BF16 ? Bf16ToFloat(raw) : HalfBitsToFloat(raw);
+                }
+                sum[i] = acc;
+            }
+        }
+    }
+    uint16_t *dst = reinterpret_cast<uint16_t *>(a.dst[which]);
+#pragma unroll
+    for (int i = 0; i < MEAN_MAX_CHANNELS / CC_THREADS; ++i) {
+        const int c = threadIdx.x + i * CC_THREADS;
+        if (c < channels) {
+            const float mean = sum[i] / static_cast<float>(static_cast<int32_t>(win));
+            dst[(slot + off) * channels + c] = BF16 ? FloatToBf16(mean) : FloatToHalfBits(mean);
+        }
     }
 }
 
@@ -173,6 +229,10 @@ extern "C" int atbmi_reshape_and_cache_compress(const void *key, const void *val
     }
     if (batch < 0 || numHeads <= 0 || headSize <= 0 || numTokens < 0 || numSlots <= 0) {
         return Fail(ERR_INVALID_PARAM, "reshape_and_cache_compress: bad extents");
+    }
+    if (offsetIndex && headSize > MEAN_MAX_CHANNELS) {
+        return Fail(ERR_INVALID_PARAM, "reshape_and_cache_compress: the window mean is built for head sizes up to %d, "
+                                       "got %lld", MEAN_MAX_CHANNELS, (long long)headSize);
     }
     if (headSize % 32 != 0) {
         return Fail(ERR_INVALID_PARAM, "reshape_and_cache_compress: headSize %lld is not a multiple of 32",
@@ -207,6 +267,7 @@ extern "C" int atbmi_reshape_and_cache_compress(const void *key, const void *val
     const int64_t rowsPerPair = (numTokens + batch - 1) / batch;
     int64_t workers = (rowsPerPair + 63) / 64;
     workers = workers < 1 ? 1 : (workers > 64 ? 64 : workers);
+    workers += offsetIndex ? 1 : 0; // the one that takes the window's mean
     dim3 grid(static_cast<unsigned>(pairs), static_cast<unsigned>(workers), 2);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (!offsetIndex) {
