@@ -182,7 +182,7 @@ class PagedCacheLoadParam(_Param):
 
 # operation name -> indices of the inputs that its outputs are (updated in place), by input count
 _IN_PLACE = {
-    "ReshapeAndCacheOperation": {5: [2, 3], 3: [1]},
+    "ReshapeAndCacheOperation": {5: [2, 3], 3: [1], 7: [2, 3], 8: [2, 3]},  # 7 / 8: head compression
     "ReshapeAndCacheWithStrideOperation": {9: [2, 3], 5: [1]},
     "NormRopeReshapeOperation": {7: [6]},
     "PagedCacheLoadOperation": {7: [4, 5]},

@@ -1156,3 +1156,49 @@ def test_kernel_layer_validates_without_a_gpu(binding):
     k.atbmi_pa_plan_destroy(plan)
     shape.maskRowBy = 3
     assert k.atbmi_pa_plan_create(ctypes.byref(shape), ctypes.byref(plan)) == 1
+
+
+def test_pa_plan_refuses_inconsistent_layout_and_compression_fields(binding):
+    """AtbmiPaShape.kvLayout, maskSeqDiv / maskSeqMod, descaleHeads and hasRazorOffset are validated on the host
+    before any kernel sees them; the razor offsets add 4 bytes per attended slot to the algorithmic bytes."""
+    k = binding.kernels()
+    plan = ctypes.c_void_p()
+
+    def create(**kw):
+        base = dict(qDtype=0, kvDtype=0, numHeads=8, numKvHeads=1, headDimK=128, headDimV=128, blockSize=128,
+                    numBlocks=8, maxBlocksPerSeq=4, numQueryRows=4, qkScale=1.0)
+        base.update(kw)
+        rc = k.atbmi_pa_plan_create(ctypes.byref(binding.AtbmiPaShape(**base)), ctypes.byref(plan))
+        if rc == 0:
+            k.atbmi_pa_plan_destroy(plan)
+        return rc
+
+    assert create() == 0
+    assert create(kvLayout=1, numKvHeads=4) == 0
+    assert create(kvLayout=2) == 1
+    assert create(kvLayout=1, mlaCombined=1, headDimK=576, headDimV=512) == 1
+    assert create(maskSeqDiv=-1) == 1 and create(maskSeqMod=-2) == 1 and create(descaleHeads=-1) == 1
+    assert create(kvDtype=2, descaleHeads=4) == 0
+    assert create(kvDtype=0, descaleHeads=4) == 1                       # descale slices need an int8 cache
+    assert create(kvDtype=2, descaleHeads=4, numKvHeads=2) == 1         # ... and one KV head
+    assert create(hasRazorOffset=1) == 0
+    assert create(hasRazorOffset=1, numKvHeads=2) == 1
+    assert create(hasRazorOffset=1, kvLayout=1) == 1
+    shape = binding.AtbmiPaShape(qDtype=0, kvDtype=0, numHeads=8, numKvHeads=1, headDimK=128, headDimV=128,
+                                 blockSize=128, numBlocks=8, maxBlocksPerSeq=4, numQueryRows=4, qkScale=1.0)
+    lens = np.array([100, 0, 512, 7], dtype=np.int32)
+    sizes = []
+    for razor in (0, 1):
+        shape.hasRazorOffset = razor
+        assert k.atbmi_pa_plan_create(ctypes.byref(shape), ctypes.byref(plan)) == 0
+        assert k.atbmi_pa_plan_update(plan, lens.ctypes.data, 4) == 0
+        sizes.append(k.atbmi_pa_plan_algorithmic_bytes(plan))
+        k.atbmi_pa_plan_destroy(plan)
+    assert sizes[1] - sizes[0] == (100 + 512 + 7) * 4
+    # the compressed cache write refuses what its kernels do not cover
+    assert k.atbmi_reshape_and_cache_compress(16, 16, 16, 16, 16, 16, 16, None, 2, 4, 48, 100, 256, 0, None) == 1   # 32-aligned
+    assert k.atbmi_reshape_and_cache_compress(16, 16, 16, 16, 16, 16, 16, 16, 2, 4, 128, 100, 256, 2, None) == 1   # int8 mean
+    assert k.atbmi_reshape_and_cache_compress(16, 16, 16, 16, 16, 16, 16, 16, 2, 4, 2048, 100, 256, 0, None) == 1  # > 1024
+    assert k.atbmi_reshape_and_cache_compress(16, 16, 16, 16, 16, None, 16, None, 2, 4, 128, 100, 256, 0, None) == 1
+    assert k.atbmi_reshape_and_cache_compress(16, 8, 16, 16, 16, 16, 16, None, 2, 4, 128, 100, 256, 0, None) == 1   # alignment
+    assert k.atbmi_reshape_and_cache_compress(16, 16, 16, 16, 16, 16, 16, None, 0, 4, 128, 0, 256, 0, None) == 0    # nothing to do
