@@ -15,10 +15,12 @@
 // descales, plain or uint64-packed, (+ int32 offsets); the MLA combined cache
 // (mlaVHeadSize > 0); additive NORM and ALIBI masks; the dynamic-batch status
 // input; per-sequence LogN scaling; several query tokens per sequence
-// (CALC_TYPE_SPEC) with the SPEC or the square NORM mask.
-// MASK_TYPE_MASK_FREE, head compression, BNSD layout and int8 queries are
-// legal in the reference but not implemented here; such params are rejected
-// at creation with ERROR_INVALID_PARAM.
+// (CALC_TYPE_SPEC) with the SPEC or the square NORM mask; head-major (BNSD)
+// caches; head compression with its per-slot score offsets.
+// int8 queries (QKV quant) are legal in the reference but not implemented
+// here; such params are rejected at creation with ERROR_INVALID_PARAM.
+// MASK_TYPE_MASK_FREE can be created and fails InferShape / Setup with
+// ERROR_INVALID_TENSOR_DIM, as the reference does off Atlas 300I Duo.
 #include <cmath>
 #include <new>
 #include "atb/infer_op_params.h"
@@ -139,9 +141,7 @@ bool FeatureParamCheck(const Param &p)
 bool ImplementedCheck(const Param &p)
 {
     const char *what = nullptr;
-    if (p.maskType == Param::MASK_TYPE_MASK_FREE) {
-        what = "MASK_TYPE_MASK_FREE";
-    } else if (p.maskType == Param::MASK_TYPE_SPEC && p.calcType != Param::CALC_TYPE_SPEC) {
+    if (p.maskType == Param::MASK_TYPE_SPEC && p.calcType != Param::CALC_TYPE_SPEC) {
         what = "MASK_TYPE_SPEC without CALC_TYPE_SPEC";
     } else if (p.quantType == Param::TYPE_QUANT_QKV_OFFLINE || p.quantType == Param::TYPE_QUANT_QKV_ONLINE) {
         what = "int8 query quantisation";
@@ -275,9 +275,20 @@ protected:
     // Reference :697-726 (InferShapeDimCheck) + :634-661 (KVCacheDimCheck).
     Status InferShapeCheckImpl(const SVector<TensorDesc> &in) const override
     {
-        if (bnsd_) {
-            return BnsdDimCheck(in);
+        const Status st = bnsd_ ? BnsdDimCheck(in) : ShapeDimCheck(in);
+        if (st != NO_ERROR) {
+            return st;
         }
+        if (param_.maskType == Param::MASK_TYPE_MASK_FREE) {
+            // reference :769-791: the operation can be created anywhere, its shapes pass on Atlas 300I Duo only
+            ATB_LOG(ERROR) << "Only Atlas 300I Duo inference products support mask free";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        return NO_ERROR;
+    }
+
+    Status ShapeDimCheck(const SVector<TensorDesc> &in) const
+    {
         if (!mla_ && in.at(2).shape.dimNum != 4) {
             ATB_LOG(ERROR) << "valueCache should have 4 dims";
             return ERROR_INVALID_TENSOR_DIM_NUM;

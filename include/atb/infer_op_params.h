@@ -68,8 +68,8 @@ struct PagedAttentionParam {
         MASK_TYPE_NORM,
         MASK_TYPE_ALIBI,
         MASK_TYPE_SPEC,
-        MASK_TYPE_MASK_FREE,
-        MASK_TYPE_NORM_COMPRESS
+        MASK_TYPE_MASK_FREE,    // Atlas 300I Duo only: InferShape / Setup return ERROR_INVALID_TENSOR_DIM elsewhere
+        MASK_TYPE_NORM_COMPRESS // Atlas 300I Duo only: refused at creation elsewhere
     };
     MaskType maskType = UNDEFINED;
 

@@ -37,7 +37,7 @@ ELEWISE_CASES = _load("elewise")
 
 def _pa_unimplemented(p):
     """Features of PagedAttentionParam the reference accepts but this library rejects at creation."""
-    return (p.get("maskType", 0) >= 4 or (p.get("maskType", 0) == 3 and p.get("calcType", 0) != 1) or
+    return ((p.get("maskType", 0) == 3 and p.get("calcType", 0) != 1) or
             p.get("quantType", 0) >= 2)
 
 
@@ -1202,3 +1202,25 @@ def test_pa_plan_refuses_inconsistent_layout_and_compression_fields(binding):
     assert k.atbmi_reshape_and_cache_compress(16, 16, 16, 16, 16, None, 16, None, 2, 4, 128, 100, 256, 0, None) == 1
     assert k.atbmi_reshape_and_cache_compress(16, 8, 16, 16, 16, 16, 16, None, 2, 4, 128, 100, 256, 0, None) == 1   # alignment
     assert k.atbmi_reshape_and_cache_compress(16, 16, 16, 16, 16, 16, 16, None, 0, 4, 128, 0, 256, 0, None) == 0    # nothing to do
+
+
+def test_mask_free_is_created_and_refused_at_infer_shape(binding, ctx):
+    """MASK_TYPE_MASK_FREE off Atlas 300I Duo (reference paged_attention_operation.cpp:769-791,805-840): the
+    operation is created, InferShape and Setup return ERROR_INVALID_TENSOR_DIM; NORM_COMPRESS is refused at creation."""
+    E = binding.ERROR_CODE
+    P = binding.PagedAttentionParam
+    assert binding.Operation("PagedAttentionOperation", P(headNum=8, kvHeadNum=8, qkScale=1.0, maskType=5)).status == \
+        E["ERROR_INVALID_PARAM"]
+    op = binding.Operation("PagedAttentionOperation", P(headNum=8, kvHeadNum=8, qkScale=1.0, maskType=4))
+    assert op.status == 0 and op.input_num() == 6
+    mk = binding.make_tensor
+    lens = np.full((2,), 5, dtype=np.int32)
+    ins = [mk("float16", (2, 8, 128), FAKE_DEVICE), mk("float16", (4, 128, 8, 128), FAKE_DEVICE),
+           mk("float16", (4, 128, 8, 128), FAKE_DEVICE), mk("int32", (2, 2), FAKE_DEVICE),
+           mk("int32", (2,), FAKE_DEVICE, host_ptr=lens.ctypes.data), mk("float16", (1, 8, 128, 16), FAKE_DEVICE)]
+    assert op.infer_shape(ins)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.setup(ins, [mk("float16", (2, 8, 128), FAKE_DEVICE)], ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    # dim-number mistakes are still reported first
+    ins[1] = mk("float16", (4, 128, 8 * 128), FAKE_DEVICE)
+    assert op.infer_shape(ins)[0] == E["ERROR_INVALID_TENSOR_DIM_NUM"]
+    op.close()
