@@ -141,9 +141,7 @@ bool FeatureParamCheck(const Param &p)
 bool ImplementedCheck(const Param &p)
 {
     const char *what = nullptr;
-    if (p.maskType == Param::MASK_TYPE_SPEC && p.calcType != Param::CALC_TYPE_SPEC) {
-        what = "MASK_TYPE_SPEC without CALC_TYPE_SPEC";
-    } else if (p.quantType == Param::TYPE_QUANT_QKV_OFFLINE || p.quantType == Param::TYPE_QUANT_QKV_ONLINE) {
+    if (p.quantType == Param::TYPE_QUANT_QKV_OFFLINE || p.quantType == Param::TYPE_QUANT_QKV_ONLINE) {
         what = "int8 query quantisation";
     } else if (p.quantType != Param::TYPE_QUANT_UNQUANT && p.quantType != Param::TYPE_DEQUANT_FUSION) {
         what = "this quantType";
@@ -633,9 +631,10 @@ private:
         const bool multi = param_.calcType == Param::CALC_TYPE_SPEC;
         bool ok = false;
         rowBy = ATBMI_PA_MASK_ROW_SEQUENCE;
-        if (multi) {
+        if (multi || param_.maskType == Param::MASK_TYPE_SPEC) {
+            // (MASK_TYPE_SPEC without CALC_TYPE_SPEC: one query token per sequence, still one mask row per query row)
             if (m.dimNum == 2 && param_.maskType == Param::MASK_TYPE_SPEC) {
-                ok = m.dims[0] == queryRows;
+                ok = m.dims[0] == queryRows && !compress_; // (under head compression the rows are pairs, not tokens)
                 rowBy = ATBMI_PA_MASK_ROW_QUERY;
             } else if (m.dimNum == 2 && param_.maskType == Param::MASK_TYPE_NORM) {
                 ok = m.dims[0] == m.dims[1];

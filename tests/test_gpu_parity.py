@@ -946,6 +946,37 @@ def test_compressed_write_then_compressed_attention(binding, oracle, dev, stream
     assert_close(out, want, TOL[torch.float16], "write + attention")
 
 
+@pytest.mark.parametrize("forced", ["scalar", None])
+def test_spec_mask_with_one_query_token_per_sequence(binding, oracle, dev, stream, forced, monkeypatch):
+    """MASK_TYPE_SPEC without CALC_TYPE_SPEC: the mask [query rows, maxS] has one row per query row (the reference
+    kernel library's look-ahead shape, mixkernels/pagedattention/paged_attention_operation.cpp:742-751); a sequence
+    of length 0 takes neither a query row nor a mask row."""
+    if forced:
+        monkeypatch.setenv("ATBMI_PA_KERNEL", forced)
+    rng = _rng(977)
+    heads, kv_heads, d, block = 32, 8, 128, 128
+    ctx = np.array([700, 0, 33, 2048, 129], dtype=np.int32)
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, len(ctx), heads, kv_heads, block, d, d, ctx, torch.float16)
+    q = q[:4].contiguous()
+    mask = rng.standard_normal((4, 2048)).astype(np.float32)
+    mask[:, :5] = -10000.0
+    mask = torch.from_numpy(mask).to(torch.float16).to(dev)
+    scale = 1.0 / math.sqrt(d)
+    lens = torch.from_numpy(ctx)
+    status = torch.from_numpy((ctx > 0).astype(np.int32))
+    c = binding.Context(stream)
+    pa = binding.OperationRunner("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=heads, kvHeadNum=kv_heads, qkScale=scale, maskType=3, batchRunStatusEnable=True), c)
+    with torch.cuda.stream(stream):
+        out, = pa.run([q, kc, vc, tables, lens.to(dev), mask, status.to(dev)], host_inputs={4: lens, 6: status})
+    stream.synchronize()
+    pa.close()
+    c.close()
+    want = oracle_pa(oracle, q, kc, vc, tables, ctx, scale, mask=mask, mask_rows="query")
+    assert_close(out, want, TOL[torch.float16], "SPEC mask, one token per sequence")
+    assert np.abs(want - oracle_pa(oracle, q, kc, vc, tables, ctx, scale)).max() > 0.01
+
+
 def test_c1_decode_step_through_operation_api(binding, oracle, pkg, dev, stream):
     """Benchmark configuration 1 end to end: ReshapeAndCache then PagedAttention
     through atb::Operation, fp16, rtol = atol = 1e-3."""

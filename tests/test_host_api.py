@@ -37,8 +37,7 @@ ELEWISE_CASES = _load("elewise")
 
 def _pa_unimplemented(p):
     """Features of PagedAttentionParam the reference accepts but this library rejects at creation."""
-    return ((p.get("maskType", 0) == 3 and p.get("calcType", 0) != 1) or
-            p.get("quantType", 0) >= 2)
+    return p.get("quantType", 0) >= 2
 
 
 def _pa_mask_shape_refused(case):
@@ -552,9 +551,10 @@ def test_several_query_tokens_inputs(binding, ctx):
         op = binding.Operation("PagedAttentionOperation", binding.PagedAttentionParam(
             headNum=32, kvHeadNum=16, qkScale=0.088, calcType=1, **bad))
         assert op.status == e["ERROR_INVALID_PARAM"], bad
-    # MASK_TYPE_SPEC without CALC_TYPE_SPEC has no defined rows
+    # MASK_TYPE_SPEC without CALC_TYPE_SPEC: one query token per sequence, one mask row per query row
     op = binding.Operation("PagedAttentionOperation", binding.PagedAttentionParam(headNum=32, kvHeadNum=16, maskType=3))
-    assert op.status == e["ERROR_INVALID_PARAM"]
+    assert op.status == 0 and op.input_num() == 6
+    op.close()
 
 
 def test_multi_latent_attention_counts_shapes_and_setup(binding, ctx):
