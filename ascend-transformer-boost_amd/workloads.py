@@ -36,11 +36,14 @@ CONFIGS = {
     "c5": dict(batch=64, heads=128, kv_heads=1, d=576, dv=512, block=128, ctx=(2048, 4096), dtype="bf16",
                kv="bf16", dist="uniform", std=0.3, pool=None, mla=True),
 }
+# C2 over head-major caches [blocks, kv heads, block, d] (InputLayout TYPE_BNSD); attention only: the reference
+# has no cache write for this layout
+CONFIGS["c2_bnsd"] = dict(CONFIGS["c2"], bnsd=True)
 # C5 as MultiLatentAttentionOperation sees it: the same rows, 512 latent + 64 rotary channels in two
 # tensors each for the query and the cache.
 CONFIGS["c5_split"] = dict(CONFIGS["c5"], split=True)
 
-SEEDS = {"c1": 1001, "c2": 1002, "c2_fp16": 1002, "c2_alibi": 1002, "c2_norm": 1002, "c2_mtp4": 1002, "c3": 1003, "c4": 1004, "c5": 1005, "c5_split": 1005}
+SEEDS = {"c1": 1001, "c2": 1002, "c2_fp16": 1002, "c2_alibi": 1002, "c2_norm": 1002, "c2_mtp4": 1002, "c2_bnsd": 1002, "c3": 1003, "c4": 1004, "c5": 1005, "c5_split": 1005}
 
 
 def config(name, **overrides):

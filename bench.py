@@ -39,6 +39,8 @@ DESCRIPTIONS = {
                 "ctx U[1024,4096], bf16",
     "c2_norm": "C2 with a NORM mask [batch, 1, maxS]: batch 64, 32 q heads, 8 kv heads, d128, block 128, "
                "ctx U[1024,4096], bf16",
+    "c2_bnsd": "C2 over head-major caches [blocks, kv heads, block, d] (inputLayout TYPE_BNSD), attention only: batch 64, "
+               "32 q heads, 8 kv heads, d128, block 128, ctx U[1024,4096], bf16",
     "c2_mtp4": "C2 with 4 query tokens per sequence (CALC_TYPE_SPEC, MASK_TYPE_SPEC mask [256, maxS]): batch 64, "
                "32 q heads, 8 kv heads, d128, block 128, ctx U[1024,4096], bf16",
     "c3": "C3 int8-KV 70B-shaped decode: batch 128, 64 q heads, 8 kv heads, d128, block 128, ctx U[2048,8192], fp16 q",
@@ -140,7 +142,10 @@ def main():
     rows = cfg["batch"] * q_len  # query tokens of one step
     pa_param = b.PagedAttentionParam(headNum=cfg["heads"], kvHeadNum=cfg["kv_heads"], qkScale=scale,
                                      quantType=1 if int8 else 0, mlaVHeadSize=cfg["dv"] if mla else 0,
-                                     maskType=mask_type, calcType=1 if q_len > 1 else 0)
+                                     maskType=mask_type, calcType=1 if q_len > 1 else 0,
+                                     inputLayout=1 if cfg.get("bnsd") else 0)
+    if cfg.get("bnsd"):
+        args.attention_only = True
     split = bool(cfg.get("split"))
     if split:
         pa = b.OperationRunner("MultiLatentAttentionOperation", b.MultiLatentAttentionParam(
@@ -172,6 +177,9 @@ def main():
             rac_out = [step["key_cache"]]
         else:
             pa_in = [step["q"], step["key_cache"], step["value_cache"], step["block_tables"], lens_dev]
+            if cfg.get("bnsd"):
+                pa_in[1] = step["key_cache"].permute(0, 2, 1, 3).contiguous()
+                pa_in[2] = step["value_cache"].permute(0, 2, 1, 3).contiguous()
             host_idx = 4
             if mask_type:
                 pa_in.append(step["mask"])
