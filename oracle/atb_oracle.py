@@ -13,6 +13,11 @@ pinned by tests/test_oracle.py against closed forms, fp64 brute force and
 the invariants of the mathematics (no function is left "parity unpinned"):
 
   reshape_and_cache   tests/apitest/kernelstest/mix/test_reshape_and_cache.py:45-65
+  reshape_and_cache_compress
+                      tests/apitest/kernelstest/mix/test_reshape_and_cache_wins.py:61-88 (the last wins[i]
+                      tokens of every (sequence, head) pair) and test_reshape_and_cache_wins_rope.py:78-131 (a
+                      window replaced by its mean); pinned by element loops over flat addresses, the slot
+                      counts, a one-token window = plain copy, and the float64 mean
   dequant_per_channel tests/apitest/opstest/python/operations/elewise/test_elewise_dequant.py:23-31
   strided_view        tests/unittest/ops/reshape_and_cache_with_stride/test_reshape_and_cache_with_stride.cpp:
                       219-245 (element [i0, i1, i2] of the view is storage[offset + sum(i_k * stride_k)]),
@@ -36,6 +41,9 @@ the invariants of the mathematics (no function is left "parity unpinned"):
                       sequence i; :353-358 a 4-dim mask is sliced [i, :, :, :ctx], a 3-dim one
                       [i, :, :ctx], with i the index into context_lens); :74-83 (ALiBi slopes),
                       :488-505 (the masks the reference tests feed);
+                      head-major caches: test_paged_attention_operation_BNSD.py:369-373 (pinned by flat
+                      addresses); head compression: test_paged_attention_common.py:292-360 with :85-101 and
+                      :249-252 (pinned against ordinary attention on the rearranged cache, loop version);
                       several query tokens per sequence (calcType SPEC): tests/apitest/opstest/python/
                       operations/paged_attention/test_paged_attention_operation_parallel_decoding_910B.py:
                       75-121 (sequence i owns q_lens[i] consecutive query rows, every one attends to
