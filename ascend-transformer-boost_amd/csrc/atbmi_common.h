@@ -132,7 +132,7 @@ struct PaStreamPlan {
     const uint16_t *firstSeq; // per workgroup range: sequence holding its first step; null: use inlineFirst
     int32_t numSeqs;          // passes (PaSeq entries)
     int32_t totalSteps;
-    int32_t numWaveRanges;    // numWgRanges * tokenSlices
+    int32_t numWaveRanges;    // at most numWgRanges * tokenSlices and at most totalSteps: no range is empty
     int32_t numWgRanges;
     int32_t tokenSlices;      // consecutive wave ranges one workgroup covers (waves / headsPerWg)
     int32_t headsPerWg;       // virtual heads (KV head x query-head tile) one workgroup covers

@@ -297,7 +297,11 @@ int PlanStream(AtbmiPaPlan *plan)
         if (wgRanges * tokenSlices > 0x3fffffff / 2) {
             return Fail(ERR_INVALID_PARAM, "pa_plan_update: too many ranges");
         }
-        const int32_t waveRanges = static_cast<int32_t>(wgRanges * tokenSlices);
+        // A wave range must hold at least one step: an empty range writes no partial row, and the merge
+        // kernel reads the slot of every range between a row's first and last. Surplus waves of the last
+        // workgroup idle (their range index is past numWaveRanges).
+        const int32_t waveRanges = static_cast<int32_t>(std::max<int64_t>(1, std::min<int64_t>(wgRanges * tokenSlices, steps)));
+        wgRanges = (waveRanges + tokenSlices - 1) / tokenSlices;
 
         plan->firstSeq.assign(static_cast<size_t>(wgRanges), 0);
         int cursor = 0;
@@ -397,6 +401,11 @@ extern "C" int atbmi_pa_plan_update_multi(AtbmiPaPlan *plan, const int32_t *ctx,
         if (qLens && (qLens[b] < 0 || (ctx[b] > 0 && qLens[b] > ctx[b]))) {
             return Fail(ERR_INVALID_PARAM, "pa_plan_update: queryLens[%d]=%d outside [0, contextLens = %d]", b, qLens[b],
                         ctx[b]);
+        }
+        if (s.hasMask && ctx[b] > s.maskLen) {
+            // both kernels index a mask row by token without a bound of their own
+            return Fail(ERR_INVALID_PARAM, "pa_plan_update: contextLens[%d]=%d exceeds the mask's %d tokens per row", b,
+                        ctx[b], s.maskLen);
         }
         const int32_t n = ctx[b] == 0 ? 0 : (qLens ? qLens[b] : 1);
         if (n > 0) {

@@ -23,7 +23,7 @@ def dtype_code(binding, t):
 def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=None, v_scale=None,
                    v_off=None, mla_dv=0, q_scale=0.0, kernel=0, chunk_tokens=None, out=None, return_plan_info=False,
                    mask=None, mask_per_head=False, logn=None, q_lens=None, mask_rows="sequence", q_rope=None,
-                   k_rope=None, lse=None, head_major=False):
+                   k_rope=None, lse=None, head_major=False, poison_workspace=False):
     """atbmi_pa_plan_* + atbmi_pa_decode on `stream`; returns the output tensor.
     mask: device tensor of q's dtype shaped like one of the reference's decode
     masks; mask_per_head says that a 3-dim mask's first dim counts heads (ALIBI).
@@ -73,6 +73,8 @@ def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=
         ws_bytes = k.atbmi_pa_plan_workspace_size(plan)
         with torch.cuda.stream(stream):
             ws = torch.empty(max(int(ws_bytes), 16), dtype=torch.uint8, device=q.device)
+            if poison_workspace:
+                ws.fill_(0xFF)  # every fp32 in it reads as NaN until a kernel writes it
             if out is None:
                 out = torch.zeros((rows, heads, dv), dtype=q.dtype, device=q.device)
             t = binding.AtbmiPaTensors()

@@ -752,6 +752,34 @@ def test_paged_attention_matrix(binding, oracle, dev, stream, case):
         assert_close(got, want, TOL[dtype], "kernel=%d" % kernel)
 
 
+# Fewer 32-token steps than the waves of a workgroup: batch, heads, kv_heads, d, ctx, dtype
+TINY_PLANS = [
+    (1, 8, 1, 128, [96], torch.float16),
+    (1, 8, 2, 128, [64], torch.float16),
+    (1, 4, 1, 64, [224], torch.bfloat16),
+    (2, 16, 1, 128, [33, 70], torch.float16),
+    (1, 12, 1, 256, [97], torch.float16),
+    (3, 8, 1, 128, [1, 40, 129], torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("case", TINY_PLANS, ids=lambda c: "b%d_h%d_g%d_d%d_%s" % (
+    c[0], c[1], c[2], c[3], "_".join(str(n) for n in c[4])))
+def test_plans_with_fewer_steps_than_waves(binding, oracle, dev, stream, case):
+    """One short sequence and few KV heads: the step space is shorter than the ranges a workgroup's waves
+    could take, so some waves must idle and the merge must only see ranges that were written. The
+    workspace is filled with NaN first: an unwritten partial row that is read shows up."""
+    batch, heads, kv_heads, d, ctx, dtype = case
+    rng = _rng(900 + heads + d + ctx[0])
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, batch, heads, kv_heads, 128, d, d, ctx, dtype)
+    scale = 1.0 / math.sqrt(d)
+    want = oracle_pa(oracle, q, kc, vc, tables, ctx, scale)
+    for kernel in _kernels_for(binding, d, d, 128):
+        got, info = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, kernel=kernel, return_plan_info=True,
+                                   poison_workspace=True)
+        assert_close(got, want, TOL[dtype], "kernel=%d, %d ranges" % (kernel, info["chunks"]))
+
+
 # batch, heads, kv_heads, block, d, ctx, dtype, mask kind
 HEAD_MAJOR_MATRIX = [
     (16, 40, 10, 128, 128, 3000, torch.bfloat16, "norm3"),  # reference test_paged_attention_operation_BNSD.py:392-405

@@ -1224,3 +1224,43 @@ def test_mask_free_is_created_and_refused_at_infer_shape(binding, ctx):
     ins[1] = mk("float16", (4, 128, 8 * 128), FAKE_DEVICE)
     assert op.infer_shape(ins)[0] == E["ERROR_INVALID_TENSOR_DIM_NUM"]
     op.close()
+
+
+def test_no_wave_range_of_a_plan_is_empty(binding):
+    """A range without steps writes no partial row, yet the merge kernel reads the slot of every range
+    between a row's first and last: the planner must never make more ranges than 32-token steps."""
+    k = binding.kernels()
+    cases = []
+    for heads, kv, dk, dv, mla in ((8, 1, 128, 128, 0), (8, 2, 128, 128, 0), (4, 4, 64, 64, 0), (32, 8, 128, 128, 0),
+                                   (16, 1, 576, 512, 1), (128, 1, 576, 512, 1), (32, 1, 192, 128, 1), (12, 1, 256, 256, 0)):
+        for lens in ([96], [64], [33], [1], [224], [32, 32], [40, 1, 70], [129, 0, 31], [225, 17], [4096], [7] * 5):
+            cases.append((heads, kv, dk, dv, mla, lens))
+    for heads, kv, dk, dv, mla, lens in cases:
+        shape = binding.AtbmiPaShape(qDtype=0, kvDtype=0, numHeads=heads, numKvHeads=kv, headDimK=dk, headDimV=dv,
+                                     blockSize=128, numBlocks=64, maxBlocksPerSeq=32, numQueryRows=len(lens),
+                                     mlaCombined=mla, qkScale=1.0, kernel=binding.ATBMI_PA_KERNEL_MFMA)
+        plan = ctypes.c_void_p()
+        assert k.atbmi_pa_plan_create(ctypes.byref(shape), ctypes.byref(plan)) == 0, (heads, kv, dk)
+        arr = np.array(lens, dtype=np.int32)
+        assert k.atbmi_pa_plan_update(plan, arr.ctypes.data, len(lens)) == 0
+        steps = int(sum((n + 31) // 32 for n in lens))
+        ranges = k.atbmi_pa_plan_num_chunks(plan)
+        assert 1 <= ranges <= steps, (heads, kv, dk, lens, ranges, steps)
+        if steps == 1:
+            assert k.atbmi_pa_plan_workspace_size(plan) == 0
+        k.atbmi_pa_plan_destroy(plan)
+
+
+def test_plan_refuses_a_context_longer_than_the_mask_row(binding):
+    k = binding.kernels()
+    shape = binding.AtbmiPaShape(qDtype=0, kvDtype=0, numHeads=8, numKvHeads=8, headDimK=128, headDimV=128,
+                                 blockSize=128, numBlocks=8, maxBlocksPerSeq=8, numQueryRows=2, qkScale=1.0,
+                                 hasMask=1, maskLen=300, maskBatchStride=300)
+    plan = ctypes.c_void_p()
+    assert k.atbmi_pa_plan_create(ctypes.byref(shape), ctypes.byref(plan)) == 0
+    arr = np.array([300, 12], dtype=np.int32)
+    assert k.atbmi_pa_plan_update(plan, arr.ctypes.data, 2) == 0
+    arr[1] = 301
+    assert k.atbmi_pa_plan_update(plan, arr.ctypes.data, 2) == 1
+    assert b"mask" in k.atbmi_last_error()
+    k.atbmi_pa_plan_destroy(plan)
