@@ -232,6 +232,9 @@ def kernels():
         lib.atbmi_pa_plan_algorithmic_bytes.argtypes = [vp]
         lib.atbmi_pa_plan_algorithmic_bytes.restype = u64
         lib.atbmi_pa_decode.argtypes = [vp, ctypes.POINTER(AtbmiPaTensors), vp, u64, vp]
+        lib.atbmi_pa_decode_static.argtypes = [vp, ctypes.POINTER(AtbmiPaTensors), vp]
+        lib.atbmi_pa_static_scratch_bytes.argtypes = []
+        lib.atbmi_pa_static_scratch_bytes.restype = u64
         lib.atbmi_pa_plan_destroy.argtypes = [vp]
         lib.atbmi_pa_plan_destroy.restype = None
         lib.atbmi_timing_enable.argtypes = [i32]

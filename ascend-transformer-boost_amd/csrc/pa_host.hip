@@ -15,6 +15,9 @@
 #include <vector>
 #include "pa_internal.h"
 
+#define ATBMI_STATIC_SCRATCH_BYTES (32ull << 20)
+static __device__ __align__(256) unsigned char scratch[ATBMI_STATIC_SCRATCH_BYTES];
+
 namespace atbmi {
 
 namespace {
@@ -56,6 +59,36 @@ struct TimingRecord {
     hipEvent_t begin;
     hipEvent_t end;
 };
+// Scratch of the entry point that allocates nothing (atbmi_pa_decode_static): the partial rows and
+// log-sum-exps a plan would otherwise keep in the caller's workspace. Every device the library runs on
+// holds its own copy at its own address; host code only ever uses the address hipGetSymbolAddress gave
+// for the device that is current, never the array's name.
+constexpr uint64_t STATIC_SCRATCH_BYTES = ATBMI_STATIC_SCRATCH_BYTES;
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratchMutex;
+void *g_scratchPtr[MAX_DEVICES] = {};
+
+// Address of `scratch` on the current device, looked up once per device.
+int StaticScratch(void **ptr)
+{
+    int dev = -1;
+    ATBMI_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode_static: device %d outside [0, %d)", dev, MAX_DEVICES);
+    }
+    std::lock_guard<std::mutex> lock(g_scratchMutex);
+    if (!g_scratchPtr[dev]) {
+        void *p = nullptr;
+        ATBMI_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(::scratch)));
+        if (!p) {
+            return Fail(ERR_RT_FAIL, "pa_decode_static: no address for the scratch array on device %d", dev);
+        }
+        g_scratchPtr[dev] = p;
+    }
+    *ptr = g_scratchPtr[dev];
+    return OK;
+}
+
 std::mutex g_timingMutex;
 int g_timingEvery = 0;   // 0: off; n: bracket every n-th decode launch with events
 int64_t g_timingLaunch = 0;
@@ -637,16 +670,14 @@ int UploadPlan(AtbmiPaPlan *plan, void *workspace, hipStream_t stream)
 
 } // namespace
 
-extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void *workspace, uint64_t workspaceBytes,
-                               void *streamHandle)
+namespace {
+
+// Both decode entry points. `mayAllocate` false: no plan upload (its pinned staging ring is allocated on
+// demand) and no timing events.
+int DecodeImpl(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void *workspace, uint64_t workspaceBytes,
+               void *streamHandle, bool mayAllocate)
 {
-    if (!plan || !t) {
-        return Fail(ERR_INVALID_PARAM, "pa_decode: null argument");
-    }
     const AtbmiPaShape &s = plan->shape;
-    if (plan->nonEmpty == 0) {
-        return OK; // every sequence is empty: nothing is written
-    }
     if (!t->query || !t->keyCache || !t->blockTables || !t->out || (!s.mlaCombined && !t->valueCache)) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: a required tensor is null");
     }
@@ -676,7 +707,7 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
         return Fail(ERR_INVALID_PARAM, "pa_decode: workspace must be 16-byte aligned");
     }
     hipStream_t stream = static_cast<hipStream_t>(streamHandle);
-    int rc = UploadPlan(plan, workspace, stream);
+    int rc = mayAllocate ? UploadPlan(plan, workspace, stream) : OK;
     if (rc != OK) {
         return rc;
     }
@@ -744,7 +775,7 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
     bool timed = false;
     {
         std::lock_guard<std::mutex> lock(g_timingMutex);
-        timed = g_timingEvery > 0 && (g_timingLaunch++ % g_timingEvery) == 0;
+        timed = mayAllocate && g_timingEvery > 0 && (g_timingLaunch++ % g_timingEvery) == 0;
     }
     if (timed) {
         ATBMI_HIP_CHECK(hipEventCreate(&rec.begin));
@@ -772,6 +803,56 @@ extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void 
         return plan->streamNeedsReduce ? LaunchPaStreamReduce(s, a, sp, stream) : OK;
     }
     return LaunchPaReduce(s, a, static_cast<int>(plan->reduceSeqs.size()), stream);
+}
+
+} // namespace
+
+extern "C" int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void *workspace, uint64_t workspaceBytes,
+                               void *streamHandle)
+{
+    if (!plan || !t) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: null argument");
+    }
+    if (plan->nonEmpty == 0) {
+        return OK; // every sequence is empty: nothing is written
+    }
+    return DecodeImpl(plan, t, workspace, workspaceBytes, streamHandle, true);
+}
+
+extern "C" uint64_t atbmi_pa_static_scratch_bytes(void)
+{
+    return STATIC_SCRATCH_BYTES;
+}
+
+extern "C" int atbmi_pa_decode_static(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void *streamHandle)
+{
+    if (!plan || !t) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode_static: null argument");
+    }
+    if (plan->nonEmpty == 0) {
+        return OK;
+    }
+    if (plan->blobBytes != 0) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode_static: the plan's tables (%llu bytes) do not travel in the kernel "
+                                       "arguments (MFMA kernel, at most %d passes and %d workgroup ranges); use "
+                                       "atbmi_pa_decode", (unsigned long long)plan->blobBytes, PA_INLINE_SEQS,
+                    PA_INLINE_RANGES);
+    }
+    if (plan->wsBytes > STATIC_SCRATCH_BYTES) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode_static: the plan needs %llu bytes of partial rows, the static scratch "
+                                       "holds %llu; use atbmi_pa_decode with a workspace",
+                    (unsigned long long)plan->wsBytes, (unsigned long long)STATIC_SCRATCH_BYTES);
+    }
+    void *ptr = nullptr;
+    if (plan->wsBytes > 0) {
+        const int rc = StaticScratch(&ptr);
+        if (rc != OK) {
+            return rc;
+        }
+    }
+    // Nothing in the scratch has to start at zero: every partial row and log-sum-exp the merge kernel
+    // reads was written by the attention kernel of the same call.
+    return DecodeImpl(plan, t, ptr, plan->wsBytes, streamHandle, false);
 }
 
 extern "C" int atbmi_timing_enable(int32_t enable)

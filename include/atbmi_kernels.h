@@ -353,6 +353,21 @@ uint64_t atbmi_pa_plan_algorithmic_bytes(const AtbmiPaPlan *plan);
 int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *tensors, void *workspaceDevice,
                     uint64_t workspaceBytes, void *stream);
 
+/*
+ * atbmi_pa_decode without a workspace and without any allocation. No counterpart in the reference: it is
+ * for callers that cannot allocate device or pinned memory around the call (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc). The partial rows of the split go into a static
+ * device array of atbmi_pa_static_scratch_bytes() bytes (32 MiB) that every GPU the library runs on holds
+ * until the process ends. Refused with 1 (invalid parameter) when the current plan needs more than that
+ * (atbmi_pa_plan_workspace_size), or when its tables do not travel in the kernel arguments (scalar-kernel
+ * plans; more than 160 passes or 512 workgroup ranges): use atbmi_pa_decode then. Kernel timing
+ * (atbmi_timing_enable) does not cover it. All calls on one GPU share the array: calls that may overlap on
+ * one GPU (different streams, different threads) race; calls on one stream are safe. Results are those of
+ * atbmi_pa_decode, bit for bit.
+ */
+int atbmi_pa_decode_static(AtbmiPaPlan *plan, const AtbmiPaTensors *tensors, void *stream);
+uint64_t atbmi_pa_static_scratch_bytes(void);
+
 void atbmi_pa_plan_destroy(AtbmiPaPlan *plan);
 
 /*
