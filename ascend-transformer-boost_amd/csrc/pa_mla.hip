@@ -9,11 +9,11 @@ int LaunchPaMlaWide(const AtbmiPaShape &s, const PaArgs &args, const PaStreamPla
         return Fail(ERR_INVALID_PARAM, "pa_decode: shape does not fit the 128-head MLA kernel");
     }
     if (s.ropeDim != 0) {
-        return s.qDtype == ATBMI_BF16 ? mla::LaunchWide<true, true>(args, plan, stream)
-                                      : mla::LaunchWide<false, true>(args, plan, stream);
+        return s.qDtype == ATBMI_BF16 ? mla::LaunchAsm<true, true>(args, plan, stream)
+                                      : mla::LaunchAsm<false, true>(args, plan, stream);
     }
-    return s.qDtype == ATBMI_BF16 ? mla::LaunchWide<true, false>(args, plan, stream)
-                                  : mla::LaunchWide<false, false>(args, plan, stream);
+    return s.qDtype == ATBMI_BF16 ? mla::LaunchAsm<true, false>(args, plan, stream)
+                                  : mla::LaunchAsm<false, false>(args, plan, stream);
 }
 
 } // namespace atbmi

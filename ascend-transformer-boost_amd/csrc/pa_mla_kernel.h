@@ -1,182 +1,803 @@
-// Decode attention over the combined MLA cache (key row 576 channels, value =
-// its first 512) for 128 query heads per workgroup, gfx950 (MI355X).
+// Decode attention over the combined MLA cache (key row 576 channels, value = its first 512), 128 query
+// heads per workgroup, with every register of the step loop assigned by hand (gfx950 assembly).
 //
-// Why a kernel of its own: at 576/512 channels the arithmetic intensity is
-// 128 heads x 2 flop per cache byte-pair, close to the machine's ridge, and the
-// bound is no longer HBM but how fast the latent tile can be fed from LDS into
-// the matrix cores. What matters then is how many query heads share one LDS
-// operand read, and that a single wave per SIMD (all the registers: the 32-head
-// accumulators alone are 256 of them) keeps its matrix pipe busy. Hence:
-//   - v_mfma_f32_32x32x16: 32 query heads per wave, so every K / V^T operand
-//     read from LDS feeds 32 heads, and one wave issuing these 8-pass
-//     instructions back to back saturates its SIMD's matrix pipe (16x16x32
-//     from a single wave reaches two thirds of that).
-//   - 4 waves x 32 heads = all 128 heads of one token range in one workgroup:
-//     the latent tile is fetched from HBM once and staged once.
-//   - HBM -> LDS directly (global_load_lds_dwordx4), no staging registers, no
-//     LDS store instructions. Three tile buffers: while a step computes on
-//     one, the next tile has landed or is landing in the second and the
-//     transfers of the tile after it are issued into the third, a few MFMAs
-//     apart. Each wave stages 8 of the 32 rows into its own region of the
-//     tile; rows keep the cache's order at a pitch of 1168 bytes (292 dwords
-//     = 36 mod 64 banks) and odd regions start half the banks further, which
-//     makes both the 32-row operand reads and the transposing reads
-//     conflict-free.
+// One wave per SIMD owns 32 heads: their 32 x 512 fp32 outputs are the 256 accumulation registers, their
+// 32 x 576 query the upper 144 vector registers. The step loop is software-pipelined so that the matrix
+// pipe does not wait for the vector unit:
+//     step i:   S(i+1) = K(i+1) . Q^T   (36 MFMAs)   with the softmax of S(i) between them
+//               O     += V(i)^T . P(i)^T (32 MFMAs)  with the HBM -> LDS transfers of tile i+3 between them
+// Four tile buffers: PV reads tile i, QK tile i+1, tile i+2 has landed or is landing, tile i+3 is being
+// requested. A register allocator does not hold this working set (it spills the query or moves the
+// accumulators through scratch), so the loop is one asm statement; the C++ around it only walks the plan
+// and hands over wave-uniform values.
 //
-// Layouts (lane = 32 kh + n):
+// Operand layouts are those of v_mfma_f32_32x32x16 (lane = 32 kh + n):
 //   S^T = K . Q^T   A = K tile: lane reads token row n, channels 16 j + 8 kh .. +8 (ds_read_b128)
-//                   B = Q^T in registers: head n, same channels; 36 k-steps
-//                   accumulator element e of lane (n, kh): token 8 (e/4) + 4 kh + e%4, head n
-//   O^T += V^T.P^T  contraction over 16 tokens per MFMA, two per 32-token step (kb = 0, 1). The k index
-//                   8 kh + e stands for token 16 kb + 8 (e/4) + 4 kh + e%4, which is exactly the token of
-//                   accumulator element 8 kb + e: P goes from the softmax into the B operand without
-//                   leaving its lane. V^T (A operand, channel 32 i + n) is read with two transposing
-//                   ds_read_b64_tr_b16 per MFMA, each lane pointing at the token row the permutation asks for.
+//                   B = Q^T: head n, same channels; element e of the result is token 8 (e/4) + 4 kh + e%4
+//   O^T += V^T.P^T  contraction over 16 tokens per MFMA (kb = 0, 1); the k index 8 kh + e stands for token
+//                   16 kb + 8 (e/4) + 4 kh + e%4, the token of score element 8 kb + e, so P never leaves its
+//                   lane; V^T (channel 32 i + n) comes from two transposing ds_read_b64_tr_b16.
 //
-// The plan is the "stream" plan of the 16-bit kernels with one wave range per
-// workgroup: ranges that cross a sequence boundary finish one row and start
-// the next, rows spanning several ranges leave partials for the merge kernel.
+// Tile in LDS: the 32 token rows at a pitch of 1168 bytes; wave w stages rows 8 w .. 8 w + 7 with ten
+// global_load_lds_dwordx4 (the last one on 8 lanes). 37 376 bytes a tile, four tiles.
+//
+// Hazards the assembler does not check and the code keeps by construction:
+//   - a result of an MFMA is read by the vector unit no sooner than 18 wait states after the MFMA was
+//     issued (S: a whole PV phase lies between; accumulators: s_nop before the epilogue / the rescale runs
+//     ten QK MFMAs after the last PV MFMA);
+//   - an operand register of the K / V^T rings is rewritten by an LDS read issued after the MFMA that read
+//     it last, and LDS latency exceeds the MFMA's operand fetch;
+//   - counted lgkmcnt waits only ever count LDS instructions (no scalar loads anywhere in the loop);
+//   - M0 (LDS base of the transfers) is only written when no LDS read of the wave is in flight.
 #ifndef ATBMI_PA_MLA_KERNEL_H
 #define ATBMI_PA_MLA_KERNEL_H
-#include <type_traits>
 #include "pa_mfma_kernel.h"
 
 namespace atbmi {
 namespace mla {
 
-using mfma::f16x8;
-using mfma::bf16x8;
-using mfma::i16x4;
-using mfma::u32x2;
-using mfma::u32x4;
-using mfma::f32x4;
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-
 constexpr int D = 576;
 constexpr int DV = 512;
-constexpr int STEP = PA_MFMA_STEP;           // tokens per step
-constexpr int NW = PA_MLA_WAVES;             // waves per workgroup
-constexpr int HPW = PA_MLA_HEADS_PER_WG / NW; // query heads per wave (the N extent of the 32x32 tile)
-constexpr int PITCH = D * 2 + 16;            // tile row pitch in bytes
-constexpr int ROWS_PER_WAVE = STEP / NW;     // tile rows each wave stages: one region of the tile
-constexpr int CHUNKS = (ROWS_PER_WAVE * PITCH + 1023) / 1024; // 1 KB transfer instructions per wave and step
-// A region is written by whole-wave transfers only (no lane is ever masked off): CHUNKS KB, of which the
-// 8 rows use 9344 bytes and the rest is padding; 128 more bytes shift odd regions by half the LDS banks, so
-// that the 16 rows a quarter-wave reads together (two regions) fall on 16 different bank groups.
-constexpr int REGION = CHUNKS * 1024 + 128;
-constexpr int TILE_BYTES = NW * REGION;
-constexpr int SLOTS_PER_ROW = PITCH / 16;    // 16-byte slots per tile row, the last one padding
-constexpr int WAVE_SLOTS = ROWS_PER_WAVE * SLOTS_PER_ROW;
-// LDS byte offset of tile row `row`
-__device__ __forceinline__ constexpr int RowOffset(int row)
-{
-    return (row / ROWS_PER_WAVE) * REGION + (row % ROWS_PER_WAVE) * PITCH;
-}
-constexpr int NQ = D / 16;                   // QK MFMAs per step
-constexpr int NO = DV / 32;                  // output tiles of 32 channels
-constexpr int KD = 5;                        // K operands in flight ahead of the MFMA that uses them
-constexpr int VD = 5;                        // V^T operands in flight
-constexpr int QK_PER_TRANSFER = NQ / (CHUNKS / 2);          // QK MFMAs between transfers
-constexpr int PV_PER_TRANSFER = 2 * NO / (CHUNKS - CHUNKS / 2); // PV MFMAs between transfers
-constexpr int BLK_IDS = 1024;                // block ids of a segment held in LDS at a time
-static_assert(HPW == 32 && STEP == 32 && ROWS_PER_WAVE == 8, "built around the 32x32x16 tile");
+constexpr int STEP = PA_MFMA_STEP;
+constexpr int NW = PA_MLA_WAVES;
+constexpr int HPW = PA_MLA_HEADS_PER_WG / NW;
+constexpr int PITCH = D * 2 + 16;
+constexpr int TILE_BYTES = 32 * PITCH;
+constexpr int NBUF = 4;
+constexpr int LDS_BYTES = NBUF * TILE_BYTES;
+static_assert(PITCH == 1168 && TILE_BYTES == 37376 && HPW == 32 && STEP == 32, "constants repeated in the assembly");
 
-// The three MFMA forms the kernel uses, written as assembly so that the register file is split the one
-// way that fits: the 16 output accumulators are the 256 AGPRs, everything else (Q, scores, operands)
-// lives in the 256 VGPRs. Left to the register allocator the two halves get mixed and the loop spills.
-// The compiler cannot see the latency of these instructions: MmaFence() must separate the last of a
-// chain from the first ordinary instruction that reads the chain's result, and MmaOperandFence() an
-// ordinary instruction that writes an operand from the MFMA that reads it (the forms that start a
-// chain carry that wait themselves).
-#define ATBMI_MFMA32(type) "v_mfma_f32_32x32x16_" type " %0, %1, %2, "
-template <bool BF16> __device__ __forceinline__ void MmaScoreFirst(f32x16 &s, u32x4 a, u32x4 b)
-{
-    if constexpr (BF16) {
-        asm volatile("s_nop 15\n\t" ATBMI_MFMA32("bf16") "0" : "=v"(s) : "v"(a), "v"(b));
-    } else {
-        asm volatile("s_nop 15\n\t" ATBMI_MFMA32("f16") "0" : "=v"(s) : "v"(a), "v"(b));
-    }
-}
-template <bool BF16> __device__ __forceinline__ void MmaScore(f32x16 &s, u32x4 a, u32x4 b)
-{
-    if constexpr (BF16) {
-        asm volatile(ATBMI_MFMA32("bf16") "%0" : "+v"(s) : "v"(a), "v"(b));
-    } else {
-        asm volatile(ATBMI_MFMA32("f16") "%0" : "+v"(s) : "v"(a), "v"(b));
-    }
-}
-template <bool BF16> __device__ __forceinline__ void MmaOut(f32x16 &acc, u32x4 a, u32x4 b)
-{
-    if constexpr (BF16) {
-        asm volatile(ATBMI_MFMA32("bf16") "%0" : "+a"(acc) : "v"(a), "v"(b));
-    } else {
-        asm volatile(ATBMI_MFMA32("f16") "%0" : "+a"(acc) : "v"(a), "v"(b));
-    }
-}
-// acc = 0 (a product of zero operands), without staging 256 zeros in VGPRs.
-template <bool BF16> __device__ __forceinline__ void MmaOutZero(f32x16 &acc)
-{
-    const u32x4 z = {0u, 0u, 0u, 0u};
-    if constexpr (BF16) {
-        asm volatile("s_nop 15\n\t" ATBMI_MFMA32("bf16") "0" : "=a"(acc) : "v"(z), "v"(z));
-    } else {
-        asm volatile("s_nop 15\n\t" ATBMI_MFMA32("f16") "0" : "=a"(acc) : "v"(z), "v"(z));
-    }
-}
-#undef ATBMI_MFMA32
-__device__ __forceinline__ void MmaOperandFence(u32x4 &b0, u32x4 &b1)
-{
-    // the operands pass through the statement, so the compiler cannot move their last write below it
-    asm volatile("s_nop 15" : "+v"(b0), "+v"(b1));
-}
-// 18 idle cycles: more than the wait an 8-pass MFMA result needs before another unit may read it.
-__device__ __forceinline__ void MmaFence(f32x16 &v)
-{
-    asm volatile("s_nop 15\n\ts_nop 1" : "+v"(v));
-}
-__device__ __forceinline__ void MmaFenceOut(f32x16 (&acc)[NO])
-{
-    static_assert(NO == 16, "operand list below");
-    asm volatile("s_nop 15\n\ts_nop 1"
-                 : "+a"(acc[0]), "+a"(acc[1]), "+a"(acc[2]), "+a"(acc[3]), "+a"(acc[4]), "+a"(acc[5]), "+a"(acc[6]),
-                   "+a"(acc[7]), "+a"(acc[8]), "+a"(acc[9]), "+a"(acc[10]), "+a"(acc[11]), "+a"(acc[12]),
-                   "+a"(acc[13]), "+a"(acc[14]), "+a"(acc[15]));
-}
+#define ATBMI_REGS_0_99(X) X"0", X"1", X"2", X"3", X"4", X"5", X"6", X"7", X"8", X"9", X"10", X"11", X"12", X"13", X"14", X"15", \
+    X"16", X"17", X"18", X"19", X"20", X"21", X"22", X"23", X"24", X"25", X"26", X"27", X"28", X"29", X"30", X"31", X"32", X"33", \
+    X"34", X"35", X"36", X"37", X"38", X"39", X"40", X"41", X"42", X"43", X"44", X"45", X"46", X"47", X"48", X"49", X"50", X"51", \
+    X"52", X"53", X"54", X"55", X"56", X"57", X"58", X"59", X"60", X"61", X"62", X"63", X"64", X"65", X"66", X"67", X"68", X"69", \
+    X"70", X"71", X"72", X"73", X"74", X"75", X"76", X"77", X"78", X"79", X"80", X"81", X"82", X"83", X"84", X"85", X"86", X"87", \
+    X"88", X"89", X"90", X"91", X"92", X"93", X"94", X"95", X"96", X"97", X"98", X"99"
+#define ATBMI_REGS_100_111(X) X"100", X"101", X"102", X"103", X"104", X"105", X"106", X"107", X"108", X"109", X"110", X"111"
+#define ATBMI_REGS_112_255(X) X"112", X"113", X"114", X"115", X"116", X"117", X"118", X"119", X"120", X"121", X"122", X"123", \
+    X"124", X"125", X"126", X"127", X"128", X"129", X"130", X"131", X"132", X"133", X"134", X"135", X"136", X"137", X"138", X"139", \
+    X"140", X"141", X"142", X"143", X"144", X"145", X"146", X"147", X"148", X"149", X"150", X"151", X"152", X"153", X"154", X"155", \
+    X"156", X"157", X"158", X"159", X"160", X"161", X"162", X"163", X"164", X"165", X"166", X"167", X"168", X"169", X"170", X"171", \
+    X"172", X"173", X"174", X"175", X"176", X"177", X"178", X"179", X"180", X"181", X"182", X"183", X"184", X"185", X"186", X"187", \
+    X"188", X"189", X"190", X"191", X"192", X"193", X"194", X"195", X"196", X"197", X"198", X"199", X"200", X"201", X"202", X"203", \
+    X"204", X"205", X"206", X"207", X"208", X"209", X"210", X"211", X"212", X"213", X"214", X"215", X"216", X"217", X"218", X"219", \
+    X"220", X"221", X"222", X"223", X"224", X"225", X"226", X"227", X"228", X"229", X"230", X"231", X"232", X"233", X"234", X"235", \
+    X"236", X"237", X"238", X"239", X"240", X"241", X"242", X"243", X"244", X"245", X"246", X"247", X"248", X"249", X"250", X"251", \
+    X"252", X"253", X"254", X"255"
+#define ATBMI_SREGS_36_69(X) X"36", X"37", X"38", X"39", X"40", X"41", X"42", X"43", X"44", X"45", X"46", X"47", X"48", X"49", X"50", \
+    X"51", X"52", X"53", X"54", X"55", X"56", X"57", X"58", X"59", X"60", X"61", X"62", X"63", X"64", X"65", X"66", X"67", X"68", X"69"
 
-// HBM -> LDS transfers that pass through no register. DmaBase sets the LDS base (register M0) for a run
-// of them; DmaPieceAt then moves, for every lane, 16 bytes from src + OFFSET to LDS base + OFFSET +
-// 16 * lane (the instruction's immediate offset, -4096 .. 4095, moves both addresses). The compiler
-// neither sees the transfers nor knows that M0 is in use: no code of its own between DmaBase and the
-// last DmaPieceAt of a run may use M0 (nothing this kernel is compiled to does), and DmaWait() or a
-// counted wait must come before the barrier that publishes a tile.
-__device__ __forceinline__ void DmaBase(uint32_t ldsBase)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(ldsBase) : "memory");
-}
-template <int OFFSET> __device__ __forceinline__ void DmaPieceAt(const void *src)
-{
-    asm volatile("global_load_lds_dwordx4 %0, off offset:%1" : : "v"(src), "n"(OFFSET) : "memory");
-}
+// Wave-uniform description of one segment: the part of a sequence's context that one workgroup range
+// holds, for the 32 heads of one wave.
+struct Segment {
+    const void *cache;    // key cache
+    const int32_t *table; // block ids of the sequence
+    const void *q;        // q[qRow][h0]: the first of this wave's 32 heads
+    const void *qRope;    // split layout: the last 64 channels of the same rows
+    const void *ropeCache; // split layout: the last 64 channels of the cache rows
+    void *out;            // out[qRow][h0] (complete) or partO[slot][h0]
+    void *lse;            // lse[qRow][h0] (complete; may be null) or partLse[slot][h0]
+    uint32_t rowBytes;    // bytes between consecutive cache rows
+    uint32_t ropeRowBytes; // ... of the rope cache
+    uint32_t blockShift;  // log2 of the block size
+    uint32_t tokBegin;    // multiple of 32
+    uint32_t tokEnd;      // > tokBegin
+    uint32_t complete;    // 1: the segment is the whole row, write the final output
+};
 
-__device__ __forceinline__ void DmaWait()
-{
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-}
-
-// SPLIT: the last 64 channels of every latent row live in a cache of their own (a.kRope), those of every
-// query row in a.qRope; a.kc and a.q then hold 512-channel rows.
+// One segment from start to finish: stages the first tiles, loads Q, runs the pipelined step loop, writes
+// the (partial) row. All four waves of a workgroup call it with the same token range and block table.
 template <bool BF16, bool SPLIT>
-__global__ __launch_bounds__(NW *WAVE) void PaMlaWideKernel(const PaArgs a, const PaStreamPlan p)
+__device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, uint32_t wave, float scale2)
+{
+    // Every input is wave-uniform; saying so value by value keeps each of them in scalar registers, which
+    // is where the statement's "s" operands must be.
+    auto uni = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(v))); };
+    auto uni64 = [&](const void *ptr) {
+        const uint64_t v = reinterpret_cast<uintptr_t>(ptr);
+        return (static_cast<uint64_t>(uni(static_cast<uint32_t>(v >> 32))) << 32) | uni(static_cast<uint32_t>(v));
+    };
+    const uint64_t cache = uni64(sg.cache);
+    const uint32_t cacheLo = static_cast<uint32_t>(cache);
+    const uint32_t cacheHi = static_cast<uint32_t>(cache >> 32);
+    const uint64_t table = uni64(sg.table), q = uni64(sg.q), out = uni64(sg.out), lse = uni64(sg.lse);
+    const uint64_t qRope = uni64(sg.qRope), rope = uni64(sg.ropeCache);
+    const uint32_t ropeLo = static_cast<uint32_t>(rope), ropeHi = static_cast<uint32_t>(rope >> 32);
+    const uint32_t ropeRowBytes = uni(sg.ropeRowBytes);
+    const uint32_t rowBytes = uni(sg.rowBytes), blockShift = uni(sg.blockShift), tokBegin = uni(sg.tokBegin);
+    const uint32_t tokEnd = uni(sg.tokEnd), complete = uni(sg.complete);
+    ldsBase = uni(ldsBase);
+    wave = uni(wave);
+    scale2 = __builtin_bit_cast(float, uni(__builtin_bit_cast(uint32_t, scale2)));
+    asm volatile(R"ASM(
+    // ---------------------------------------------------------------- register map
+    // v[0:15] S_A   v[16:31] S_B           scores of two consecutive steps
+    // v[32:47] K operand ring (4 x 4)      v[48:63] V^T operand ring (4 x 4)
+    // v[64:71] P operands (kb 0: 64..67, kb 1: 68..71)
+    // v[72:81] per-lane source offsets of the ten tile transfers
+    // v82 m   v83 lsum   v84 mloc   v85 corr   v86 ds_bpermute address of lane ^ 32   v87 4 kh
+    // v[88:93] temporaries   v94 K operand address of the QK tile   v95 V^T operand address of the PV tile
+    // v96 K operand address in buffer 0   v97 V^T operand address in buffer 0
+    // v98 block ids (lane k: block s42 + k)   v99 row (less 8 wave) of each transfer's slot, 3 bits each
+    // v[112:255] Q, piece j in v[112+4j : 115+4j];   a[16 i : 16 i + 15] output tile i
+    // s36 token of the PV tile   s37 end of the segment   s38 / s39 / s41 buffer offset of the PV / QK / fetched tile
+    // s40 steps done   s42 first block index in v98   s43 last block index   s44 8 wave   s45 block size - 1
+    // s[46:55] temporaries   s[56:57] transfer source base   s58 LDS address of this wave's rows in buffer 0
+    // s59 token of the tile to fetch   s[60:61] saved exec   s62 rows of this wave inside the segment
+    .set BF16, %[bf16]
+    .set SPLIT, %[split]
+    // SPLIT: the last 64 channels of every cache row come from a cache of their own (rows of 128 bytes) and
+    // those of every query row from a tensor of their own. A transfer then takes its lanes from two sources:
+    // lanes whose slot (64 i + lane, 73 slots a row, the last one padding) holds one of the first 64 pieces
+    // of a row, and lanes whose slot holds piece 64 .. 71 (or the padding). The lane masks of both kinds:
+    .set NOPE_LO_0, 0xffffffff
+    .set NOPE_HI_0, 0xffffffff
+    .set ROPE_LO_0, 0x00000000
+    .set ROPE_HI_0, 0x00000000
+    .set NOPE_LO_1, 0xfffffe00
+    .set NOPE_HI_1, 0xffffffff
+    .set ROPE_LO_1, 0x000001ff
+    .set ROPE_HI_1, 0x00000000
+    .set NOPE_LO_2, 0xfffc01ff
+    .set NOPE_HI_2, 0xffffffff
+    .set ROPE_LO_2, 0x0003fe00
+    .set ROPE_HI_2, 0x00000000
+    .set NOPE_LO_3, 0xf803ffff
+    .set NOPE_HI_3, 0xffffffff
+    .set ROPE_LO_3, 0x07fc0000
+    .set ROPE_HI_3, 0x00000000
+    .set NOPE_LO_4, 0x07ffffff
+    .set NOPE_HI_4, 0xfffffff0
+    .set ROPE_LO_4, 0xf8000000
+    .set ROPE_HI_4, 0x0000000f
+    .set NOPE_LO_5, 0xffffffff
+    .set NOPE_HI_5, 0xffffe00f
+    .set ROPE_LO_5, 0x00000000
+    .set ROPE_HI_5, 0x00001ff0
+    .set NOPE_LO_6, 0xffffffff
+    .set NOPE_HI_6, 0xffc01fff
+    .set ROPE_LO_6, 0x00000000
+    .set ROPE_HI_6, 0x003fe000
+    .set NOPE_LO_7, 0xffffffff
+    .set NOPE_HI_7, 0x803fffff
+    .set ROPE_LO_7, 0x00000000
+    .set ROPE_HI_7, 0x7fc00000
+    .set NOPE_LO_8, 0xffffffff
+    .set NOPE_HI_8, 0x7fffffff
+    .set ROPE_LO_8, 0x00000000
+    .set ROPE_HI_8, 0x80000000
+    .set NOPE_LO_9, 0x00000000
+    .set NOPE_HI_9, 0x00000000
+    .set ROPE_LO_9, 0x000000ff
+    .set ROPE_HI_9, 0x00000000
+    .if SPLIT
+      .set NDMA, 18                       // transfer instructions of a tile (empty lane masks issue none)
+    .else
+      .set NDMA, 10
+    .endif
+    .set PITCH, 1168
+    .set ROW8, 9344
+    .set ROW16, 18688
+    .set REGION, 9344
+    .set TILE, 37376
+
+    .macro LDK slot, j
+      ds_read_b128 v[32+4*(\slot):35+4*(\slot)], v94 offset:32*(\j)
+    .endm
+    .macro LDV slot, idx
+      ds_read_b64_tr_b16 v[48+4*(\slot):49+4*(\slot)], v95 offset:((\idx)/2)*64+((\idx)%%2)*ROW16
+      ds_read_b64_tr_b16 v[50+4*(\slot):51+4*(\slot)], v95 offset:((\idx)/2)*64+((\idx)%%2)*ROW16+ROW8
+    .endm
+
+    // ---- softmax slice k (k = the QK slot it rides on) of the scores at v[SO : SO+15]; P goes to v[64:71]
+    .macro SM_SLICE k, SO
+      .if \k == 0
+        v_max3_f32 v84, v[\SO+0], v[\SO+1], v[\SO+2]
+      .elseif \k == 1
+        v_max3_f32 v88, v[\SO+3], v[\SO+4], v[\SO+5]
+      .elseif \k == 2
+        v_max3_f32 v89, v[\SO+6], v[\SO+7], v[\SO+8]
+      .elseif \k == 3
+        v_max3_f32 v90, v[\SO+9], v[\SO+10], v[\SO+11]
+      .elseif \k == 4
+        v_max3_f32 v91, v[\SO+12], v[\SO+13], v[\SO+14]
+      .elseif \k == 5
+        v_max3_f32 v84, v84, v88, v89
+        v_max3_f32 v90, v90, v91, v[\SO+15]
+      .elseif \k == 6
+        v_max_f32 v84, v84, v90
+        s_nop 0
+        ds_bpermute_b32 v88, v86, v84
+      .elseif \k == 10
+        // (the exchange was issued before K piece 10 was requested: the wait for that piece covers it)
+        v_max_f32 v84, v84, v88
+        v_mul_f32 v84, %[scale], v84
+        v_add_f32 v89, 0x41000000, v82
+        v_cmp_gt_f32 vcc, v84, v89
+        s_cbranch_vccz 10f
+        // some head's maximum grew by more than 2^8: move the reference point of the exponentials
+        v_max_f32 v89, v82, v84
+        v_sub_f32 v90, v82, v89
+        v_exp_f32 v85, v90
+        v_mov_b32 v82, v89
+        s_nop 1
+        v_mul_f32 v83, v83, v85
+        s_cmp_eq_u32 s40, 0
+        s_cbranch_scc1 10f               // first step: the accumulators are still zero
+        .irp r,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15
+          .irp c,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15
+            v_accvgpr_read_b32 v90, a[16*\r+\c]
+            s_nop 0
+            v_mul_f32 v90, v90, v85
+            s_nop 0
+            v_accvgpr_write_b32 a[16*\r+\c], v90
+          .endr
+        .endr
+        10:
+      .elseif (\k >= 11) && (\k <= 26)
+        v_fma_f32 v[88+(\k%%2)], v[\SO+\k-11], %[scale], -v82
+        s_nop 0
+        v_exp_f32 v[\SO+\k-11], v[88+(\k%%2)]
+      .elseif (\k >= 27) && (\k <= 34)
+        .if BF16
+          v_cvt_pk_bf16_f32 v[64+\k-27], v[\SO+2*(\k-27)], v[\SO+2*(\k-27)+1]
+          s_nop 0
+          v_lshlrev_b32 v90, 16, v[64+\k-27]
+          v_and_b32 v91, 0xffff0000, v[64+\k-27]
+        .else
+          v_cvt_f16_f32 v90, v[\SO+2*(\k-27)]
+          v_cvt_f16_f32 v91, v[\SO+2*(\k-27)+1]
+          s_nop 0
+          v_pack_b32_f16 v[64+\k-27], v90, v91
+          v_cvt_f32_f16 v90, v90
+          v_cvt_f32_f16 v91, v91
+        .endif
+        // the denominator adds up the rounded weights, the ones that multiply V
+        v_add_f32 v83, v83, v90
+        v_add_f32 v83, v83, v91
+      .endif
+    .endm
+
+    // ---- QK slot j: S_new (v[SN : SN+15]) += K piece j . Q piece j; with SO >= 0 softmax slice j of S_old rides along
+    .macro QK_SLOT j, SN, SO
+      .if \j + 3 < 36
+        LDK ((\j+3)%%4), (\j+3)
+      .endif
+      .if \j >= 33
+        s_waitcnt lgkmcnt(35-\j)
+      .elseif (\SO >= 0) && (\j >= 7) && (\j <= 9)
+        s_waitcnt lgkmcnt(4)
+      .else
+        s_waitcnt lgkmcnt(3)
+      .endif
+      .if \j == 0
+        .if BF16
+          v_mfma_f32_32x32x16_bf16 v[\SN:\SN+15], v[32+4*(\j%%4):35+4*(\j%%4)], v[112+4*\j:115+4*\j], 0
+        .else
+          v_mfma_f32_32x32x16_f16 v[\SN:\SN+15], v[32+4*(\j%%4):35+4*(\j%%4)], v[112+4*\j:115+4*\j], 0
+        .endif
+      .else
+        .if BF16
+          v_mfma_f32_32x32x16_bf16 v[\SN:\SN+15], v[32+4*(\j%%4):35+4*(\j%%4)], v[112+4*\j:115+4*\j], v[\SN:\SN+15]
+        .else
+          v_mfma_f32_32x32x16_f16 v[\SN:\SN+15], v[32+4*(\j%%4):35+4*(\j%%4)], v[112+4*\j:115+4*\j], v[\SN:\SN+15]
+        .endif
+      .endif
+      .if \SO >= 0
+        SM_SLICE \j, \SO
+      .endif
+    .endm
+    .macro QK_PHASE SN, SO
+      LDK 0, 0
+      LDK 1, 1
+      LDK 2, 2
+      .irp j,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15,16,17,18,19,20,21,22,23,24,25,26,27,28,29,30,31,32,33,34,35
+        QK_SLOT \j, \SN, \SO
+      .endr
+    .endm
+
+    // ---- softmax of the scores at v[SO : SO+15] on its own: the last step of a segment, whose tokens at or
+    // past the end of the segment get a score of -inf
+    .macro SM_ALONE SO
+      s_sub_u32 s46, s37, s36              // tokens of this tile inside the segment
+      s_cmp_ge_u32 s46, 32
+      s_cbranch_scc1 11f
+      v_mov_b32 v88, 0xff800000
+      .irp e,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15
+        s_sub_i32 s47, s46, 8*(\e/4)+(\e%%4)
+        v_cmp_gt_i32 vcc, s47, v87
+        s_nop 1
+        v_cndmask_b32 v[\SO+\e], v88, v[\SO+\e], vcc
+      .endr
+      11:
+      .irp k,0,1,2,3,4,5,6
+        SM_SLICE \k, \SO
+      .endr
+      s_waitcnt lgkmcnt(0)
+      .irp k,10,11,12,13,14,15,16,17,18,19,20,21,22,23,24,25,26,27,28,29,30,31,32,33,34
+        SM_SLICE \k, \SO
+      .endr
+    .endm
+
+    // ---- source of the transfers of the tile at token s59 for this wave: s[56:57] = address of the cache row
+    // of token s59 + 8 wave, less 4096; s62 = tile rows of this wave that lie inside the segment (<= 0: none).
+    // Refills the block ids when the row's block is past the 64 held (waits for everything in flight then).
+    .macro DMA_PREP
+      s_add_u32 s46, s59, s44              // token of this wave's first row
+      s_sub_i32 s62, s37, s46              // rows left from there
+      s_lshr_b32 s47, s46, %[bshift]
+      s_min_u32 s47, s47, s43              // (a wave wholly past the end looks at the last block; it moves nothing)
+      s_sub_u32 s48, s47, s42
+      s_cmp_lt_u32 s48, 64
+      s_cbranch_scc1 12f
+      s_mov_b32 s42, s47
+      v_mbcnt_lo_u32_b32 v88, -1, 0
+      v_mbcnt_hi_u32_b32 v88, -1, v88
+      v_add_u32 v88, s42, v88
+      v_min_u32 v88, s43, v88
+      v_lshlrev_b32 v88, 2, v88
+      global_load_dword v98, v88, %[table]
+      s_waitcnt vmcnt(0)
+      s_mov_b32 s48, 0
+      12:
+      s_nop 0
+      v_readlane_b32 s49, v98, s48         // block id
+      s_and_b32 s50, s46, s45              // row inside the block
+      s_nop 3
+      s_lshl_b32 s49, s49, %[bshift]
+      s_add_u32 s49, s49, s50              // cache row
+      s_mul_i32 s56, s49, %[rowbytes]
+      s_mul_hi_u32 s57, s49, %[rowbytes]
+      s_add_u32 s56, s56, %[cache_lo]
+      s_addc_u32 s57, s57, %[cache_hi]
+      s_sub_u32 s56, s56, 4096
+      s_subb_u32 s57, s57, 0
+      .if SPLIT
+        s_mul_i32 s64, s49, %[roperowbytes]
+        s_mul_hi_u32 s65, s49, %[roperowbytes]
+        s_add_u32 s64, s64, %[rope_lo]
+        s_addc_u32 s65, s65, %[rope_hi]
+        s_sub_u32 s64, s64, 4096
+        s_subb_u32 s65, s65, 0
+      .endif
+    .endm
+    // the instruction of transfer i from the source base in s[base : base+1]; M0 = region + 4096 for i < 8,
+    // region + 8192 after
+    .macro DMA_LOAD i, base
+      .if \i < 8
+        global_load_lds_dwordx4 v[72+\i], s[\base:\base+1] offset:(\i-4)*1024
+      .else
+        global_load_lds_dwordx4 v[72+\i], s[\base:\base+1] offset:(\i-8)*1024
+      .endif
+    .endm
+    // transfer i of a tile whose rows all lie inside the segment
+    .macro DMA_ONE i
+      .if SPLIT
+        .if (NOPE_LO_\i != 0) || (NOPE_HI_\i != 0)
+          s_mov_b32 exec_lo, NOPE_LO_\i
+          s_mov_b32 exec_hi, NOPE_HI_\i
+          DMA_LOAD \i, 56
+        .endif
+        .if (ROPE_LO_\i != 0) || (ROPE_HI_\i != 0)
+          s_mov_b32 exec_lo, ROPE_LO_\i
+          s_mov_b32 exec_hi, ROPE_HI_\i
+          DMA_LOAD \i, 64
+        .endif
+        s_mov_b64 exec, -1
+      .else
+        .if \i == 9
+          s_mov_b64 exec, 0xff
+        .endif
+        DMA_LOAD \i, 56
+        .if \i == 9
+          s_mov_b64 exec, -1
+        .endif
+      .endif
+    .endm
+    // all ten transfers of a tile in a row, into the buffer at offset s41; slots of rows past the segment's
+    // end (s62 rows are inside) are filled with zeros instead. Not while LDS reads are being counted.
+    .macro DMA_ANY
+      s_add_u32 s53, s58, s41
+      s_mov_b64 s[60:61], exec
+      v_mov_b32 v88, 0
+      v_mov_b32 v89, 0
+      v_mov_b32 v90, 0
+      v_mov_b32 v91, 0
+      v_mbcnt_lo_u32_b32 v92, -1, 0
+      v_mbcnt_hi_u32_b32 v92, -1, v92
+      v_lshlrev_b32 v92, 4, v92
+      v_add_u32 v92, s53, v92              // LDS address of this lane's slot in transfer 0
+      .irp i,0,1,2,3,4,5,6,7,8,9
+        .if \i == 0
+          s_add_u32 s54, s53, 4096
+          s_mov_b32 m0, s54
+        .elseif \i == 8
+          s_add_u32 s54, s53, 8192
+          s_mov_b32 m0, s54
+        .endif
+        v_bfe_u32 v93, v99, 3*\i, 3
+        v_cmp_gt_i32 vcc, s62, v93         // the row of this slot lies inside the segment
+        s_nop 1
+        .if SPLIT
+          .if (NOPE_LO_\i != 0) || (NOPE_HI_\i != 0)
+            s_and_b32 exec_lo, vcc_lo, NOPE_LO_\i
+            s_and_b32 exec_hi, vcc_hi, NOPE_HI_\i
+            DMA_LOAD \i, 56
+          .endif
+          .if (ROPE_LO_\i != 0) || (ROPE_HI_\i != 0)
+            s_and_b32 exec_lo, vcc_lo, ROPE_LO_\i
+            s_and_b32 exec_hi, vcc_hi, ROPE_HI_\i
+            DMA_LOAD \i, 64
+          .endif
+        .else
+          .if \i == 9
+            s_and_b64 vcc, vcc, 0xff
+          .endif
+          s_mov_b64 exec, vcc
+          DMA_LOAD \i, 56
+        .endif
+        .if \i == 9
+          s_andn2_b64 exec, 0xff, vcc
+        .else
+          s_andn2_b64 exec, s[60:61], vcc
+        .endif
+        ds_write_b128 v92, v[88:91] offset:1024*\i
+        s_mov_b64 exec, s[60:61]
+      .endr
+    .endm
+
+    // ---- PV slot i: O tile i/2 += V^T piece i . P (kb = i mod 2); with DMA transfers of the fetched tile ride along
+    .macro PV_SLOT i, DMA
+      .if \i + 3 < 32
+        LDV ((\i+3)%%4), (\i+3)
+      .endif
+      .if \i >= 29
+        s_waitcnt lgkmcnt(2*(31-\i))
+      .else
+        s_waitcnt lgkmcnt(6)
+      .endif
+      .if BF16
+        v_mfma_f32_32x32x16_bf16 a[16*(\i/2):16*(\i/2)+15], v[48+4*(\i%%4):51+4*(\i%%4)], v[64+4*(\i%%2):67+4*(\i%%2)], a[16*(\i/2):16*(\i/2)+15]
+      .else
+        v_mfma_f32_32x32x16_f16 a[16*(\i/2):16*(\i/2)+15], v[48+4*(\i%%4):51+4*(\i%%4)], v[64+4*(\i%%2):67+4*(\i%%2)], a[16*(\i/2):16*(\i/2)+15]
+      .endif
+      .if \DMA
+        .if \i == 1
+          DMA_ONE 0
+        .elseif \i == 5
+          DMA_ONE 1
+        .elseif \i == 9
+          DMA_ONE 2
+        .elseif \i == 13
+          DMA_ONE 3
+        .elseif \i == 17
+          DMA_ONE 4
+        .elseif \i == 21
+          DMA_ONE 5
+        .elseif \i == 25
+          DMA_ONE 6
+        .elseif \i == 29
+          DMA_ONE 7
+        .endif
+      .endif
+    .endm
+    .macro PV_PHASE DMA
+      .if \DMA
+        // both LDS bases are set while none of the wave's LDS reads is in flight
+        s_add_u32 s53, s58, s41
+        s_add_u32 s54, s53, 8192
+        s_mov_b32 m0, s54
+        s_nop 0
+        DMA_ONE 8
+        DMA_ONE 9
+        s_add_u32 s54, s53, 4096
+        s_mov_b32 m0, s54
+      .endif
+      LDV 0, 0
+      LDV 1, 1
+      LDV 2, 2
+      s_nop 7
+      .irp i,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15,16,17,18,19,20,21,22,23,24,25,26,27,28,29,30,31
+        PV_SLOT \i, \DMA
+      .endr
+    .endm
+
+    // ---- one step: QK of the next tile into S_new with the softmax of S_old riding along, then PV of
+    // this tile; leaves to \tail when this tile is the segment's last
+    .macro BODY SN, SO, tail
+      s_add_u32 s46, s36, 32
+      s_cmp_ge_u32 s46, s37
+      s_cbranch_scc1 \tail
+      v_add_u32 v94, s39, v96
+      v_add_u32 v95, s38, v97
+      s_add_u32 s46, s59, 32
+      s_cmp_le_u32 s46, s37
+      s_cbranch_scc0 5f
+      // a whole tile three steps ahead: its transfers ride along
+      DMA_PREP
+      QK_PHASE \SN, \SO
+      PV_PHASE 1
+      s_waitcnt vmcnt(NDMA)                // all but the tile just requested have landed
+      s_branch 6f
+      5:
+      QK_PHASE \SN, \SO
+      PV_PHASE 0
+      s_cmp_lt_u32 s59, s37
+      s_cbranch_scc0 7f
+      DMA_PREP                             // the segment's last, partial tile
+      DMA_ANY
+      7:
+      s_waitcnt vmcnt(0) lgkmcnt(0)
+      6:
+      s_barrier
+      s_mov_b32 s38, s39
+      s_add_u32 s39, s39, TILE
+      s_cmp_eq_u32 s39, 4*TILE
+      s_cselect_b32 s39, 0, s39
+      s_add_u32 s41, s41, TILE
+      s_cmp_eq_u32 s41, 4*TILE
+      s_cselect_b32 s41, 0, s41
+      s_add_u32 s36, s36, 32
+      s_add_u32 s59, s59, 32
+      s_add_u32 s40, s40, 1
+    .endm
+
+    // ================================================================ the segment
+    s_barrier                              // every wave has left the tiles of the segment before
+    // ---- lane constants
+    v_mbcnt_lo_u32_b32 v88, -1, 0
+    v_mbcnt_hi_u32_b32 v88, -1, v88        // lane
+    v_and_b32 v89, 31, v88                 // n
+    v_lshrrev_b32 v90, 5, v88              // kh
+    v_mul_u32_u24 v96, PITCH, v89
+    v_lshl_add_u32 v96, v90, 4, v96
+    v_add_u32 v96, %[lds], v96             // K operand: row n, 16 bytes per kh
+    v_bfe_u32 v91, v88, 2, 2
+    v_lshl_add_u32 v91, v90, 2, v91        // 4 kh + (lane / 4) mod 4
+    v_mul_u32_u24 v97, PITCH, v91
+    v_bfe_u32 v91, v88, 4, 1
+    v_lshlrev_b32 v91, 5, v91
+    v_and_b32 v92, 3, v88
+    v_lshlrev_b32 v92, 3, v92
+    v_add3_u32 v97, v97, v91, v92
+    v_add_u32 v97, %[lds], v97             // V^T operand
+    v_xor_b32 v86, 32, v88
+    v_lshlrev_b32 v86, 2, v86
+    v_lshlrev_b32 v87, 2, v90
+    v_mov_b32 v99, 0
+    .irp i,0,1,2,3,4,5,6,7,8,9
+      // slot 64 i + lane of this wave's rows: row = slot / 73, piece = min(slot mod 73, 71)
+      v_add_u32 v91, 64*\i, v88
+      v_mul_u32_u24 v92, 449, v91
+      v_lshrrev_b32 v92, 15, v92
+      v_mul_u32_u24 v93, 73, v92
+      v_sub_u32 v93, v91, v93
+      v_min_u32 v93, 71, v93
+      v_mul_lo_u32 v91, v92, %[rowbytes]
+      v_lshl_add_u32 v91, v93, 4, v91
+      .if SPLIT
+        // pieces 64 .. 71 of a row: piece - 64 of the same row of the rope cache
+        v_mul_lo_u32 v94, v92, %[roperowbytes]
+        v_add_u32 v95, -64, v93
+        v_lshl_add_u32 v94, v95, 4, v94
+        v_cmp_lt_u32 vcc, 63, v93
+        s_nop 1
+        v_cndmask_b32 v91, v91, v94, vcc
+      .endif
+      .if \i < 8
+        v_add_u32 v[72+\i], 8192-1024*\i, v91
+      .else
+        v_add_u32 v[72+\i], 4096-1024*(\i-8), v91
+      .endif
+      v_and_b32 v92, 7, v92
+      v_lshl_or_b32 v99, v92, 3*\i, v99
+    .endr
+    // ---- segment state
+    s_mov_b32 s36, %[tokbegin]
+    s_mov_b32 s37, %[tokend]
+    s_mov_b32 s38, 0
+    s_mov_b32 s39, TILE
+    s_mov_b32 s40, 0
+    s_mov_b32 s42, 0x80000000
+    s_sub_u32 s43, s37, 1
+    s_lshr_b32 s43, s43, %[bshift]
+    s_lshl_b32 s44, %[wave], 3
+    s_lshl_b32 s45, 1, %[bshift]
+    s_sub_u32 s45, s45, 1
+    s_mul_i32 s58, %[wave], REGION
+    s_add_u32 s58, s58, %[lds]
+    // ---- the first three tiles
+    s_mov_b32 s59, s36
+    s_mov_b32 s41, 0
+    DMA_PREP
+    DMA_ANY
+    s_add_u32 s59, s59, 32
+    s_mov_b32 s41, TILE
+    s_cmp_lt_u32 s59, s37
+    s_cbranch_scc0 8f
+    DMA_PREP
+    DMA_ANY
+    8:
+    s_add_u32 s59, s59, 32
+    s_mov_b32 s41, 2*TILE
+    s_cmp_lt_u32 s59, s37
+    s_cbranch_scc0 9f
+    DMA_PREP
+    DMA_ANY
+    9:
+    s_add_u32 s59, s59, 32
+    s_mov_b32 s41, 3*TILE
+    // ---- Q: lane (n, kh) holds q[h0 + n][16 j + 8 kh .. +8) for the 36 pieces j
+    v_mbcnt_lo_u32_b32 v88, -1, 0
+    v_mbcnt_hi_u32_b32 v88, -1, v88
+    v_and_b32 v89, 31, v88
+    v_lshrrev_b32 v90, 5, v88
+    .if SPLIT
+      v_lshlrev_b32 v88, 10, v89
+      v_lshl_add_u32 v88, v90, 4, v88      // rows of 512 channels
+      v_lshlrev_b32 v91, 7, v89
+      v_lshl_add_u32 v91, v90, 4, v91      // rows of 64 channels
+      .irp j,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15,16,17,18,19,20,21,22,23,24,25,26,27,28,29,30,31
+        global_load_dwordx4 v[112+4*\j:115+4*\j], v88, %[q] offset:32*\j
+      .endr
+      .irp j,32,33,34,35
+        global_load_dwordx4 v[112+4*\j:115+4*\j], v91, %[qrope] offset:32*(\j-32)
+      .endr
+    .else
+      v_mul_u32_u24 v88, 1152, v89
+      v_lshl_add_u32 v88, v90, 4, v88
+      .irp j,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15,16,17,18,19,20,21,22,23,24,25,26,27,28,29,30,31,32,33,34,35
+        global_load_dwordx4 v[112+4*\j:115+4*\j], v88, %[q] offset:32*\j
+      .endr
+    .endif
+    // ---- O = 0, written by the matrix pipe itself
+    v_mov_b32 v64, 0
+    v_mov_b32 v65, 0
+    v_mov_b32 v66, 0
+    v_mov_b32 v67, 0
+    s_nop 4
+    .irp i,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15
+      .if BF16
+        v_mfma_f32_32x32x16_bf16 a[16*\i:16*\i+15], v[64:67], v[64:67], 0
+      .else
+        v_mfma_f32_32x32x16_f16 a[16*\i:16*\i+15], v[64:67], v[64:67], 0
+      .endif
+    .endr
+    v_mov_b32 v82, 0xff800000
+    v_mov_b32 v83, 0
+    s_waitcnt vmcnt(0) lgkmcnt(0)
+    s_barrier
+    // ---- scores of the first tile
+    v_add_u32 v94, s38, v96
+    QK_PHASE 0, -1
+    s_nop 15
+    s_nop 1
+    1:
+    BODY 16, 0, 2f
+    BODY 0, 16, 3f
+    s_branch 1b
+    2:
+    v_add_u32 v95, s38, v97
+    SM_ALONE 0
+    PV_PHASE 0
+    s_branch 4f
+    3:
+    v_add_u32 v95, s38, v97
+    SM_ALONE 16
+    PV_PHASE 0
+    4:
+    // ================================================================ the row, or this range's share of it
+    s_nop 15
+    s_nop 1
+    ds_bpermute_b32 v88, v86, v83
+    v_mbcnt_lo_u32_b32 v92, -1, 0
+    v_mbcnt_hi_u32_b32 v92, -1, v92        // lane
+    v_and_b32 v89, 31, v92                 // n
+    v_lshrrev_b32 v90, 5, v92              // kh
+    s_waitcnt lgkmcnt(0)
+    v_add_f32 v83, v83, v88                // l: both halves of the head's tokens
+    s_nop 0
+    v_rcp_f32 v84, v83
+    v_log_f32 v85, v83
+    s_nop 1
+    v_add_f32 v85, v85, v82                // log2 of the sum of 2^score
+    s_cmp_eq_u32 %[complete], 0
+    s_cbranch_scc1 13f
+    // ---- final row: out[h0 + n][32 i + 8 r + 4 kh .. +4) in the query's type
+    v_lshlrev_b32 v91, 10, v89
+    v_lshl_add_u32 v91, v90, 3, v91
+    .irp i,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15
+      .irp c,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15
+        v_accvgpr_read_b32 v[16*(\i%%2)+\c], a[16*\i+\c]
+      .endr
+      .irp c,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15
+        v_mul_f32 v[16*(\i%%2)+\c], v[16*(\i%%2)+\c], v84
+      .endr
+      .irp p,0,1,2,3,4,5,6,7
+        .if BF16
+          v_cvt_pk_bf16_f32 v[32+8*(\i%%2)+\p], v[16*(\i%%2)+2*\p], v[16*(\i%%2)+2*\p+1]
+        .else
+          v_cvt_f16_f32 v[16*(\i%%2)+2*\p], v[16*(\i%%2)+2*\p]
+          v_cvt_f16_f32 v[16*(\i%%2)+2*\p+1], v[16*(\i%%2)+2*\p+1]
+          s_nop 0
+          v_pack_b32_f16 v[32+8*(\i%%2)+\p], v[16*(\i%%2)+2*\p], v[16*(\i%%2)+2*\p+1]
+        .endif
+      .endr
+      s_nop 1
+      .irp r,0,1,2,3
+        global_store_dwordx2 v91, v[32+8*(\i%%2)+2*\r:33+8*(\i%%2)+2*\r], %[out] offset:(32*\i+8*\r)*2
+      .endr
+    .endr
+    s_cmp_eq_u64 %[lse], 0
+    s_cbranch_scc1 14f
+    // natural-log log-sum-exp of the row, by the kh = 0 lanes
+    v_mul_f32 v85, 0x3f317218, v85
+    v_lshlrev_b32 v91, 1, v89
+    .if BF16
+      v_cvt_pk_bf16_f32 v85, v85, v85
+    .else
+      v_cvt_f16_f32 v85, v85
+    .endif
+    s_mov_b64 s[60:61], exec
+    s_mov_b64 exec, 0xffffffff
+    s_nop 1
+    global_store_short v91, v85, %[lse]
+    s_mov_b64 exec, s[60:61]
+    s_branch 14f
+    13:
+    // ---- partial row: normalised fp32 channels and the base-2 log-sum-exp
+    v_lshlrev_b32 v91, 11, v89
+    v_lshl_add_u32 v91, v90, 4, v91
+    .irp i,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15
+      .irp c,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15
+        v_accvgpr_read_b32 v[16*(\i%%2)+\c], a[16*\i+\c]
+      .endr
+      .irp c,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15
+        v_mul_f32 v[16*(\i%%2)+\c], v[16*(\i%%2)+\c], v84
+      .endr
+      s_nop 1
+      .irp r,0,1,2,3
+        global_store_dwordx4 v91, v[16*(\i%%2)+4*\r:16*(\i%%2)+4*\r+3], %[out] offset:(32*\i+8*\r)*4
+      .endr
+    .endr
+    v_lshlrev_b32 v91, 2, v89
+    s_mov_b64 s[60:61], exec
+    s_mov_b64 exec, 0xffffffff
+    s_nop 1
+    global_store_dword v91, v85, %[lse]
+    s_mov_b64 exec, s[60:61]
+    14:
+    .purgem LDK
+    .purgem LDV
+    .purgem SM_SLICE
+    .purgem QK_SLOT
+    .purgem QK_PHASE
+    .purgem SM_ALONE
+    .purgem DMA_PREP
+    .purgem DMA_LOAD
+    .purgem DMA_ONE
+    .purgem DMA_ANY
+    .purgem PV_SLOT
+    .purgem PV_PHASE
+    .purgem BODY
+    )ASM"
+                 :
+                 : [bf16] "n"(BF16 ? 1 : 0), [split] "n"(SPLIT ? 1 : 0), [qrope] "s"(qRope), [rope_lo] "s"(ropeLo),
+                   [rope_hi] "s"(ropeHi), [roperowbytes] "s"(ropeRowBytes), [scale] "s"(scale2), [bshift] "s"(blockShift), [table] "s"(table),
+                   [rowbytes] "s"(rowBytes), [cache_lo] "s"(cacheLo), [cache_hi] "s"(cacheHi), [q] "s"(q), [out] "s"(out),
+                   [lse] "s"(lse), [tokbegin] "s"(tokBegin), [tokend] "s"(tokEnd), [lds] "s"(ldsBase), [wave] "s"(wave),
+                   [complete] "s"(complete)
+                 : "memory", "vcc", "scc", "m0", ATBMI_REGS_0_99("v"), ATBMI_REGS_112_255("v"), ATBMI_REGS_0_99("a"),
+                   ATBMI_REGS_100_111("a"), ATBMI_REGS_112_255("a"), ATBMI_SREGS_36_69("s"));
+}
+
+// Grid and plan as the 128-head kernel of pa_mla_kernel.h: one wave range per workgroup, the head groups of
+// one range 8 workgroup ids apart.
+template <bool BF16, bool SPLIT>
+__global__ __launch_bounds__(NW *WAVE) void PaMlaAsmKernel(const PaArgs a, const PaStreamPlan p)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-
-    const int lane = threadIdx.x % WAVE;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
-    const int n = lane & 31; // head (B operand / accumulator column); token or channel (A operand row)
-    const int kh = lane >> 5; // which 8 of the 16 contraction values this lane holds
-    const bool qBf16 = a.qIsBf16 != 0;
-
-    // Workgroup -> (token range, group of 128 heads): the groups of one range sit 8 ids apart (same XCD).
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const int octet = blockIdx.x / (8 * p.headGroups);
     const int within = blockIdx.x % (8 * p.headGroups);
     const int hgIdx = within / 8;
@@ -189,397 +810,76 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaWideKernel(const PaArgs a, cons
     if (s0 >= s1) {
         return;
     }
-    const int h0 = hgIdx * PA_MLA_HEADS_PER_WG + wave * HPW;
-
     const uint32_t ldsBase = static_cast<uint32_t>(
         reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char *)smem));
-    const unsigned char *kcBase = reinterpret_cast<const unsigned char *>(a.kc);
-    const int64_t rowBytes = a.kRowStride * 2;
-    const unsigned char *krBase = reinterpret_cast<const unsigned char *>(a.kRope);
-    const int64_t ropeRowBytes = a.ropeRowStride * 2;
-    constexpr int NOPE_PIECES = DV * 2 / 16; // 16-byte pieces of a latent row ahead of its rope channels
+    const int h0 = hgIdx * PA_MLA_HEADS_PER_WG + static_cast<int>(wave) * HPW;
     constexpr float LOG2E = 1.4426950408889634f;
     const float scale2 = a.qkScale * LOG2E;
+    const uint32_t blockShift = static_cast<uint32_t>(__builtin_ctz(static_cast<unsigned>(a.blockSize)));
 
-    // The plan is the same for every lane: say so, and the loop control below runs on the scalar unit.
     auto uniform = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
     int seqIdx = uniform(p.firstSeq ? p.firstSeq[wr] : p.inlineFirst[wr]);
     while (uniform(mfma::PlanSeq(p, seqIdx + 1).stepBegin) <= s0) {
         ++seqIdx;
     }
-
     for (; seqIdx < p.numSeqs; ++seqIdx) {
-        PaSeq sq = mfma::PlanSeq(p, seqIdx);
-        sq.tableRow = uniform(sq.tableRow);
-        sq.ctxLen = uniform(sq.ctxLen);
-        sq.stepBegin = uniform(sq.stepBegin);
-        if (sq.stepBegin >= s1) {
+        const PaSeq sq = mfma::PlanSeq(p, seqIdx);
+        const int tableRow = uniform(sq.tableRow);
+        const int ctxLen = uniform(sq.ctxLen);
+        const int stepBegin = uniform(sq.stepBegin);
+        const int qRow = uniform(sq.qRow);
+        if (stepBegin >= s1) {
             break;
         }
         const int seqEnd = uniform(mfma::PlanSeq(p, seqIdx + 1).stepBegin);
-        const int segBegin = max(s0, sq.stepBegin);
+        const int segBegin = max(s0, stepBegin);
         const int segEnd = min(s1, seqEnd);
-        const int tokBegin = (segBegin - sq.stepBegin) * STEP;
-        const int tokEnd = min(sq.ctxLen, (segEnd - sq.stepBegin) * STEP);
-        const bool complete = segBegin == sq.stepBegin && segEnd == seqEnd;
-        const int qRow = uniform(sq.qRow); // (128 heads fill the tile: a pass never holds a second query token)
-
-        // ---- block ids of this segment sit in LDS (BLK_IDS at a time) and are read one tile ahead of
-        // their use: the step loop then holds no memory instruction of the compiler's whose wait would
-        // also wait for the tile transfers in flight (vector loads), or stall every LDS wait behind an
-        // HBM round trip (scalar loads return out of order).
-        const int32_t *table = a.tables + static_cast<int64_t>(sq.tableRow) * a.maxBlocksPerSeq;
-        const int lastBlk = (tokEnd - 1) / a.blockSize; // entries past this one are never read
-        int curBlk = tokBegin / a.blockSize;            // cursor: the next 16-token sub-tile to look up
-        int curOff = tokBegin % a.blockSize;
-        int idBase = curBlk;                            // block index of blkIds[0]
-        int32_t *blkIds = reinterpret_cast<int32_t *>(smem + 3 * TILE_BYTES);
-        auto fillIds = [&]() { // all waves together
-            __syncthreads(); // nobody still reads the old ids
-            for (int i = threadIdx.x; i < BLK_IDS && idBase + i <= lastBlk; i += NW * WAVE) {
-                blkIds[i] = table[idBase + i];
-            }
-            __syncthreads();
-        };
-        fillIds();
-        int pendBlk[2]; // (still in flight from LDS) block ids of the two sub-tiles of the next tile
-        int pendOff[2]; // and the row offsets inside those blocks
-        auto lookAhead = [&]() {
-#pragma unroll
-            for (int sub = 0; sub < 2; ++sub) {
-                const int blkIdx = min(curBlk, lastBlk);
-                if (blkIdx >= idBase + BLK_IDS) {
-                    idBase = blkIdx;
-                    fillIds();
-                }
-                pendBlk[sub] = blkIds[blkIdx - idBase];
-                pendOff[sub] = curOff;
-                curOff += 16;
-                if (curOff >= a.blockSize) {
-                    curOff = 0;
-                    ++curBlk;
-                }
-            }
-        };
-        lookAhead();
-
-        // Transfer of the 32 latent rows at token t into the tile at LDS address tileAddr: prepare() once,
-        // then transfer(0 .. CHUNKS-1), exactly CHUNKS instructions per wave whatever the tile (the waits
-        // below count them). Wave w moves tile rows 8w .. 8w+7; the rows of a 16-token sub-tile are
-        // consecutive cache rows (a sub-tile never straddles cache blocks). Tile rows at or past the end
-        // of the segment get a copy of its last row: they only have to be finite, their weights are
-        // exact zeros. Lane l of transfer i fills slot 64 i + l of the wave's region; slots that hold no
-        // data (the padding slot of each row, everything past the 8 rows) fetch a neighbour's piece, so
-        // every lane of every transfer is active and reads valid memory.
-        const unsigned char *stSub0 = nullptr, *stSub1 = nullptr;
-        const unsigned char *stRope0 = nullptr, *stRope1 = nullptr; // SPLIT: the same rows of the rope cache
-        int stLastRow = 0;
-        uint32_t stDst = 0;
-        auto prepare = [&](int t, uint32_t tileAddr) {
-            const int64_t row0 = static_cast<int64_t>(__builtin_amdgcn_readfirstlane(pendBlk[0])) * a.blockSize + pendOff[0];
-            const int64_t row1 = static_cast<int64_t>(__builtin_amdgcn_readfirstlane(pendBlk[1])) * a.blockSize + pendOff[1];
-            stSub0 = kcBase + row0 * rowBytes;
-            stSub1 = kcBase + row1 * rowBytes;
-            if constexpr (SPLIT) {
-                stRope0 = krBase + row0 * ropeRowBytes;
-                stRope1 = krBase + row1 * ropeRowBytes;
-            }
-            lookAhead();
-            stLastRow = min(tokEnd - 1 - t, STEP - 1);
-            stDst = tileAddr + static_cast<uint32_t>(wave * REGION);
-        };
-        // Transfers 0 .. 7 go through one setting of the LDS base (the middle of their 8 KB), 8 and 9
-        // through a second one.
-        auto transfer = [&](auto index) {
-            constexpr int i = decltype(index)::value;
-            int ln = lane;
-            if constexpr (SPLIT) {
-                // rederive the slot from the lane id at every transfer: hoisted out of the loop, the
-                // per-lane row, piece and cache choice of ten transfers would not fit the registers
-                asm volatile("" : "+v"(ln));
-            }
-            int slot = i * WAVE + ln;
-            slot = slot < WAVE_SLOTS ? slot : slot - WAVE_SLOTS;
-            const int rowIn = slot / SLOTS_PER_ROW;
-            const int col = min(slot - rowIn * SLOTS_PER_ROW, SLOTS_PER_ROW - 2);
-            const int row = min(ROWS_PER_WAVE * wave + rowIn, stLastRow);
-            const unsigned char *src = ((row >> 4) ? stSub1 : stSub0) +
-                                       static_cast<uint32_t>(row & 15) * static_cast<uint32_t>(rowBytes) + col * 16;
-            if constexpr (SPLIT) {
-                if (col >= NOPE_PIECES) {
-                    src = ((row >> 4) ? stRope1 : stRope0) +
-                          static_cast<uint32_t>(row & 15) * static_cast<uint32_t>(ropeRowBytes) + (col - NOPE_PIECES) * 16;
-                }
-            }
-            if constexpr (i == 0) {
-                DmaBase(stDst + 4096);
-            }
-            if constexpr (i == 8) {
-                DmaBase(stDst + 8192);
-            }
-            constexpr int imm = i < 8 ? (i - 4) * 1024 : (i - 8) * 1024;
-            DmaPieceAt<imm>(src - imm);
-        };
-        auto transferAll = [&]() {
-            transfer(std::integral_constant<int, 0>{});
-            transfer(std::integral_constant<int, 1>{});
-            transfer(std::integral_constant<int, 2>{});
-            transfer(std::integral_constant<int, 3>{});
-            transfer(std::integral_constant<int, 4>{});
-            transfer(std::integral_constant<int, 5>{});
-            transfer(std::integral_constant<int, 6>{});
-            transfer(std::integral_constant<int, 7>{});
-            transfer(std::integral_constant<int, 8>{});
-            transfer(std::integral_constant<int, 9>{});
-        };
-        static_assert(CHUNKS == 10, "transfer schedule");
-
-        // The first two tiles are on their way while Q is fetched; from then on the transfers of the tile
-        // two steps ahead are issued during each step, one every few MFMAs.
-        prepare(tokBegin, ldsBase);
-        transferAll();
-        if (tokBegin + STEP < tokEnd) {
-            prepare(tokBegin + STEP, ldsBase + TILE_BYTES);
-            transferAll();
-        }
-
-        // ---- Q^T as B operand: lane (n, kh) holds q[h0+n][16 j + 8 kh .. +8) for j < NQ
-        u32x4 qreg[NQ];
-        {
-            const int64_t qh = static_cast<int64_t>(qRow) * a.H + h0 + n;
-            const uint16_t *qrow = reinterpret_cast<const uint16_t *>(a.q) + qh * (SPLIT ? DV : D) + kh * 8;
-            const uint16_t *qrope = reinterpret_cast<const uint16_t *>(a.qRope) + qh * (D - DV) - DV + kh * 8;
-#pragma unroll
-            for (int j = 0; j < NQ; ++j) {
-                qreg[j] = mfma::LoadGlobal16((SPLIT && j * 16 >= DV ? qrope : qrow) + j * 16);
-            }
-        }
-
-        float m = -INFINITY; // running maximum of head n, base-2 exponent units
-        float lsum = 0.0f;   // this lane's share (its 16 tokens of every step) of the denominator of head n
-        f32x16 acc[NO];
-#pragma unroll
-        for (int i = 0; i < NO; ++i) {
-            MmaOutZero<BF16>(acc[i]); // zeros written by the matrix core, straight into the AGPRs
-        }
-
-        DmaWait();
-        // Touch Q here so that the compiler's own wait for the Q loads lands before the loop and not,
-        // counting down, inside it, where it would also wait for the tile transfers in flight.
-#pragma unroll
-        for (int j = 0; j < NQ; ++j) {
-            asm volatile("" : "+v"(qreg[j]));
-        }
-        __syncthreads();
-
-        int buf = 0;
-        for (int t = tokBegin; t < tokEnd; t += STEP) {
-            const unsigned char *tile = smem + buf * TILE_BYTES;
-            // Operand read offsets inside the tile, rederived from the lane id every step (two
-            // instructions each) rather than kept live across the whole kernel.
-            int ln = lane;
-            asm volatile("" : "+v"(ln));
-            const int kOff = RowOffset(ln & 31) + (ln >> 5) * 16;
-            const int vOff = (4 * (ln >> 5) + ((ln >> 2) & 3)) * PITCH + (16 * ((ln >> 4) & 1) + 4 * (ln & 3)) * 2;
-
-            const bool fetch = t + 2 * STEP < tokEnd; // a tile two steps ahead exists: fetch it during this step
-            if (fetch) {
-                prepare(t + 2 * STEP, ldsBase + (buf == 0 ? 2 : buf - 1) * TILE_BYTES);
-            }
-
-            // ---- S^T = K . Q^T, operands fetched KD MFMAs ahead
-            f32x16 s;
-            {
-                const unsigned char *krow = tile + kOff;
-                u32x4 kop[KD + 1];
-#pragma unroll
-                for (int j = 0; j < KD; ++j) {
-                    kop[j] = *reinterpret_cast<const u32x4 *>(krow + j * 32);
-                }
-#pragma unroll
-                for (int j = 0; j < NQ; ++j) {
-                    if (j + KD < NQ) {
-                        kop[(j + KD) % (KD + 1)] = *reinterpret_cast<const u32x4 *>(krow + (j + KD) * 32);
-                    }
-                    if (j == 0) {
-                        MmaScoreFirst<BF16>(s, kop[0], qreg[0]);
-                    } else {
-                        MmaScore<BF16>(s, kop[j % (KD + 1)], qreg[j]);
-                    }
-                    if (j % QK_PER_TRANSFER == QK_PER_TRANSFER / 2 && j / QK_PER_TRANSFER < CHUNKS / 2 && fetch) {
-                        switch (j / QK_PER_TRANSFER) {
-                            case 0: transfer(std::integral_constant<int, 0>{}); break;
-                            case 1: transfer(std::integral_constant<int, 1>{}); break;
-                            case 2: transfer(std::integral_constant<int, 2>{}); break;
-                            case 3: transfer(std::integral_constant<int, 3>{}); break;
-                            default: transfer(std::integral_constant<int, 4>{}); break;
-                        }
-                    }
-                }
-                MmaFence(s);
-            }
-
-            // ---- online softmax in base 2; element e is token t + 8 (e/4) + 4 kh + e%4 of head n
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                s[e] *= scale2;
-            }
-            if (t + STEP > tokEnd) { // last step of the segment: mask the tokens past its end
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const int tok = t + 8 * (e >> 2) + 4 * kh + (e & 3);
-                    s[e] = tok < tokEnd ? s[e] : -INFINITY;
-                }
-            }
-            float mloc = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
-            mloc = fmaxf(mloc, fmaxf(fmaxf(fmaxf(s[8], s[9]), fmaxf(s[10], s[11])),
-                                     fmaxf(fmaxf(s[12], s[13]), fmaxf(s[14], s[15]))));
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
-            // The reference point of the exponentials only has to stay within 2^RESCALE_SLACK of the true
-            // running maximum (weights then reach at most 2^RESCALE_SLACK, harmless in fp32 accumulators
-            // and in the 16-bit P); numerator and denominator share it, so the result is the same. Moving
-            // it means a pass over all 256 accumulator registers, which this makes rare. mloc is finite:
-            // every step holds at least one valid token.
-            constexpr float RESCALE_SLACK = 8.0f;
-            if (__builtin_amdgcn_ballot_w64(mloc > m + RESCALE_SLACK) != 0) {
-                const float mNew = fmaxf(m, mloc);
-                const float corr = mfma::Exp2(m - mNew);
-                m = mNew;
-                lsum *= corr;
-                if (t != tokBegin) { // (the first step starts from zeros)
-                    MmaFenceOut(acc);
-#pragma unroll
-                    for (int i = 0; i < NO; ++i) { // one tile at a time through the VGPRs
-                        acc[i] *= corr;
-                        asm volatile("" : "+a"(acc[i])); // back into its AGPRs before the next tile is touched
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                }
-            }
-            u32x4 pop[2]; // P^T as B operand of the two 16-token contractions
-#pragma unroll
-            for (int e = 0; e < 16; e += 2) {
-                const uint32_t pair = mfma::Pack2<BF16>(mfma::Exp2(s[e] - m), mfma::Exp2(s[e + 1] - m));
-                pop[e >> 3][(e >> 1) & 3] = pair;
-                // the denominator adds up the rounded weights, the ones that multiply V
-                lsum += mfma::Unpack(pair, 0, BF16) + mfma::Unpack(pair, 1, BF16);
-            }
-
-            // ---- O^T += V^T . P^T, operands fetched VD MFMAs ahead
-            {
-                const unsigned char *vrow = tile + vOff;
-                auto readV = [&](int idx) -> u32x4 { // idx = 2 * channel tile + kb
-                    const unsigned char *ptr = vrow + (idx >> 1) * 64 + (idx & 1) * RowOffset(16);
-                    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) i16x4 *)(ptr)));
-                    const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) i16x4 *)(ptr + RowOffset(8))));
-                    return u32x4{lo[0], lo[1], hi[0], hi[1]};
-                };
-                u32x4 vop[VD + 1];
-#pragma unroll
-                for (int i = 0; i < VD; ++i) {
-                    vop[i] = readV(i);
-                }
-                MmaOperandFence(pop[0], pop[1]); // P was packed by ordinary instructions just above
-#pragma unroll
-                for (int i = 0; i < 2 * NO; ++i) {
-                    if (i + VD < 2 * NO) {
-                        vop[(i + VD) % (VD + 1)] = readV(i + VD);
-                    }
-                    MmaOut<BF16>(acc[i >> 1], vop[i % (VD + 1)], pop[i & 1]);
-                    if (i % PV_PER_TRANSFER == PV_PER_TRANSFER / 2 && i / PV_PER_TRANSFER < CHUNKS - CHUNKS / 2 && fetch) {
-                        switch (i / PV_PER_TRANSFER) {
-                            case 0: transfer(std::integral_constant<int, 5>{}); break;
-                            case 1: transfer(std::integral_constant<int, 6>{}); break;
-                            case 2: transfer(std::integral_constant<int, 7>{}); break;
-                            case 3: transfer(std::integral_constant<int, 8>{}); break;
-                            default: transfer(std::integral_constant<int, 9>{}); break;
-                        }
-                    }
-                }
-            }
-
-            // Transfers in flight, oldest first: the next step's tile (started during the previous step),
-            // then the one started during this step. The first must be in (for this wave's pieces; the
-            // barrier makes it everyone's), the second may stay in flight. After the barrier this step's
-            // buffer is free for the tile the next step will start to fetch.
-            if (fetch) {
-                asm volatile("s_waitcnt vmcnt(%0)" : : "n"(CHUNKS) : "memory");
-            } else {
-                DmaWait();
-            }
-            __syncthreads();
-            buf = buf == 2 ? 0 : buf + 1;
-        }
-
-        // ---- finish the row (or this range's share of it)
-        MmaFenceOut(acc);
-        const float l = lsum + __shfl_xor(lsum, 32, WAVE);
-        const float inv = 1.0f / l;
-        const int h = h0 + n;
-        if (complete) {
-            uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) + (static_cast<int64_t>(qRow) * a.H + h) * DV;
-#pragma unroll
-            for (int i = 0; i < NO; ++i) {
-#pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4) {
-                    const int d = 32 * i + 8 * r4 + 4 * kh;
-                    u32x2 packed;
-                    if (qBf16) {
-                        packed[0] = mfma::Pack2<true>(acc[i][4 * r4] * inv, acc[i][4 * r4 + 1] * inv);
-                        packed[1] = mfma::Pack2<true>(acc[i][4 * r4 + 2] * inv, acc[i][4 * r4 + 3] * inv);
-                    } else {
-                        packed[0] = mfma::Pack2<false>(acc[i][4 * r4] * inv, acc[i][4 * r4 + 1] * inv);
-                        packed[1] = mfma::Pack2<false>(acc[i][4 * r4 + 2] * inv, acc[i][4 * r4 + 3] * inv);
-                    }
-                    *reinterpret_cast<u32x2 *>(orow + d) = packed;
-                }
-                __builtin_amdgcn_sched_barrier(0); // one tile at a time through the VGPRs
-            }
-            if (a.lse && kh == 0) {
-                Store16(a.lse, static_cast<int64_t>(qRow) * a.H + h, (m + log2f(l)) * 0.6931471805599453f, qBf16);
-            }
+        Segment sg;
+        sg.cache = a.kc;
+        sg.table = a.tables + static_cast<int64_t>(tableRow) * a.maxBlocksPerSeq;
+        sg.rowBytes = static_cast<uint32_t>(a.kRowStride * 2);
+        sg.blockShift = blockShift;
+        sg.tokBegin = static_cast<uint32_t>((segBegin - stepBegin) * STEP);
+        sg.tokEnd = static_cast<uint32_t>(min(ctxLen, (segEnd - stepBegin) * STEP));
+        sg.complete = (segBegin == stepBegin && segEnd == seqEnd) ? 1u : 0u;
+        const int64_t rowHead = static_cast<int64_t>(qRow) * a.H + h0;
+        sg.q = reinterpret_cast<const uint16_t *>(a.q) + rowHead * (SPLIT ? DV : D);
+        sg.qRope = SPLIT ? reinterpret_cast<const uint16_t *>(a.qRope) + rowHead * (D - DV) : nullptr;
+        sg.ropeCache = SPLIT ? a.kRope : nullptr;
+        sg.ropeRowBytes = SPLIT ? static_cast<uint32_t>(a.ropeRowStride * 2) : 0u;
+        if (sg.complete) {
+            sg.out = reinterpret_cast<uint16_t *>(a.out) + rowHead * DV;
+            sg.lse = a.lse ? reinterpret_cast<uint16_t *>(a.lse) + rowHead : nullptr;
         } else {
             const int slot = 2 * wr + (segBegin == s0 ? 0 : 1);
-            const int64_t ph = static_cast<int64_t>(slot) * a.H + h;
-#pragma unroll
-            for (int i = 0; i < NO; ++i) {
-#pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4) {
-                    const f32x4 v = {acc[i][4 * r4] * inv, acc[i][4 * r4 + 1] * inv, acc[i][4 * r4 + 2] * inv,
-                                     acc[i][4 * r4 + 3] * inv};
-                    *reinterpret_cast<f32x4 *>(a.partO + ph * DV + 32 * i + 8 * r4 + 4 * kh) = v;
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            if (kh == 0) {
-                a.partLse[ph] = m + log2f(l);
-            }
+            const int64_t ph = static_cast<int64_t>(slot) * a.H + h0;
+            sg.out = a.partO + ph * DV;
+            sg.lse = a.partLse + ph;
         }
+        RunSegment<BF16, SPLIT>(sg, ldsBase, wave, scale2);
     }
 }
 
-template <bool BF16, bool SPLIT> int LaunchWide(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
+template <bool BF16, bool SPLIT> int LaunchAsm(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
 {
-    auto kernel = PaMlaWideKernel<BF16, SPLIT>;
-    constexpr int lds = 3 * TILE_BYTES + BLK_IDS * 4;
+    auto kernel = PaMlaAsmKernel<BF16, SPLIT>;
     static bool configured = false; // one attribute call per instantiation and process
     if (!configured) {
         ATBMI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES));
         configured = true;
     }
     if (plan.tokenSlices != 1 || plan.numWaveRanges != plan.numWgRanges ||
         plan.headGroups * PA_MLA_HEADS_PER_WG != args.H || args.G != 1 || args.D != D || args.Dv != DV ||
-        args.ropeDim != (SPLIT ? D - DV : 0)) {
+        args.ropeDim != (SPLIT ? D - DV : 0) || args.blockSize < 16 || (args.blockSize & (args.blockSize - 1)) != 0 ||
+        args.kRowStride * 2 > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: plan or shape does not fit the 128-head MLA kernel");
     }
     const int64_t grid = (static_cast<int64_t>(plan.numWgRanges) + 7) / 8 * 8 * plan.headGroups;
     if (grid <= 0 || grid > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: grid of %lld workgroups is out of range", (long long)grid);
     }
-    kernel<<<static_cast<unsigned>(grid), NW * WAVE, lds, stream>>>(args, plan);
+    kernel<<<static_cast<unsigned>(grid), NW * WAVE, LDS_BYTES, stream>>>(args, plan);
     ATBMI_HIP_CHECK(hipGetLastError());
     return OK;
 }
