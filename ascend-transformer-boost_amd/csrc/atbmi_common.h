@@ -63,7 +63,7 @@ struct PaArgs {
     void *out;
     const PaWorkItem *items;
     const PaSeqInfo *seqs;
-    float *partO;   // [numPartials][H][Dv] normalised partial outputs
+    float *partO;   // [numPartials][H][Dv] normalised partial outputs: fp32, or the query's 16-bit type when partHalf
     float *partLse; // [numPartials][H] log2-domain log-sum-exp
     int32_t H, G, D, Dv;
     int32_t blockSize, maxBlocksPerSeq;
@@ -101,6 +101,8 @@ struct PaArgs {
     int32_t descaleHeads; // > 0: sequence b takes slice b % descaleHeads of the descale vectors instead of its KV head's
     const float *razor;   // [slots] added to q.k before the score scale (null: none)
     void *lse;           // [rows][H] in the query's type: natural-log log-sum-exp of the scaled scores (null: none)
+    int32_t partHalf;    // 1: partO holds 16-bit values (the 128-head MLA kernel: its partial rows are a third of
+                         // what a segment moves, and a normalised row loses nothing the final rounding would keep)
 };
 
 // ---- Plan of the MFMA kernel ------------------------------------------------

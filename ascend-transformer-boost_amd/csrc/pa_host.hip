@@ -398,7 +398,7 @@ int PlanStream(AtbmiPaPlan *plan)
     const uint64_t slots = plan->streamNeedsReduce ? 2ull * plan->stream.numWaveRanges * fold : 0;
     plan->numPartials = static_cast<int64_t>(slots);
     plan->offPartO = AlignUp(plan->blobBytes, WS_ALIGN);
-    const uint64_t partOBytes = slots * s.numHeads * s.headDimV * sizeof(float);
+    const uint64_t partOBytes = slots * s.numHeads * s.headDimV * (PaMlaWide(s) ? sizeof(uint16_t) : sizeof(float));
     plan->offPartLse = AlignUp(plan->offPartO + partOBytes, WS_ALIGN);
     plan->wsBytes = AlignUp(plan->offPartLse + slots * s.numHeads * sizeof(float), WS_ALIGN);
     if (plan->blobBytes == 0 && slots == 0) {
@@ -770,6 +770,7 @@ int DecodeImpl(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void *workspace, uint
     a.ropeDim = s.ropeDim;
     a.ropeRowStride = static_cast<int64_t>(s.numKvHeads) * s.ropeDim;
     a.lse = t->lse;
+    a.partHalf = (plan->useMfma && PaMlaWide(s)) ? 1 : 0;
 
     TimingRecord rec{nullptr, nullptr};
     bool timed = false;

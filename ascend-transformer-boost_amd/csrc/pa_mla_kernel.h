@@ -75,7 +75,7 @@ struct Segment {
     const void *q;        // q[qRow][h0]: the first of this wave's 32 heads
     const void *qRope;    // split layout: the last 64 channels of the same rows
     const void *ropeCache; // split layout: the last 64 channels of the cache rows
-    void *out;            // out[qRow][h0] (complete) or partO[slot][h0]
+    void *out;            // out[qRow][h0] (complete) or partO[slot][h0], both in the query's type
     void *lse;            // lse[qRow][h0] (complete; may be null) or partLse[slot][h0]
     uint32_t rowBytes;    // bytes between consecutive cache rows
     uint32_t ropeRowBytes; // ... of the rope cache
@@ -598,7 +598,6 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     s_mov_b32 s38, 0
     s_mov_b32 s39, TILE
     s_mov_b32 s40, 0
-    s_mov_b32 s42, 0x80000000
     s_sub_u32 s43, s37, 1
     s_lshr_b32 s43, s43, %[bshift]
     s_lshl_b32 s44, %[wave], 3
@@ -606,6 +605,35 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     s_sub_u32 s45, s45, 1
     s_mul_i32 s58, %[wave], REGION
     s_add_u32 s58, s58, %[lds]
+    // ---- the block ids of this wave's first rows, then Q behind them: the ids are back (and the tile
+    // transfers can start) while Q is still on its way
+    s_add_u32 s46, s36, s44
+    s_lshr_b32 s42, s46, %[bshift]
+    s_min_u32 s42, s42, s43
+    v_add_u32 v91, s42, v88
+    v_min_u32 v91, s43, v91
+    v_lshlrev_b32 v91, 2, v91
+    global_load_dword v98, v91, %[table]
+    // ---- Q: lane (n, kh) holds q[h0 + n][16 j + 8 kh .. +8) for the 36 pieces j
+    .if SPLIT
+      v_lshlrev_b32 v88, 10, v89
+      v_lshl_add_u32 v88, v90, 4, v88      // rows of 512 channels
+      v_lshlrev_b32 v91, 7, v89
+      v_lshl_add_u32 v91, v90, 4, v91      // rows of 64 channels
+      .irp j,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15,16,17,18,19,20,21,22,23,24,25,26,27,28,29,30,31
+        global_load_dwordx4 v[112+4*\j:115+4*\j], v88, %[q] offset:32*\j
+      .endr
+      .irp j,32,33,34,35
+        global_load_dwordx4 v[112+4*\j:115+4*\j], v91, %[qrope] offset:32*(\j-32)
+      .endr
+    .else
+      v_mul_u32_u24 v88, 1152, v89
+      v_lshl_add_u32 v88, v90, 4, v88
+      .irp j,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15,16,17,18,19,20,21,22,23,24,25,26,27,28,29,30,31,32,33,34,35
+        global_load_dwordx4 v[112+4*\j:115+4*\j], v88, %[q] offset:32*\j
+      .endr
+    .endif
+    s_waitcnt vmcnt(36)
     // ---- the first three tiles
     s_mov_b32 s59, s36
     s_mov_b32 s41, 0
@@ -627,29 +655,6 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     9:
     s_add_u32 s59, s59, 32
     s_mov_b32 s41, 3*TILE
-    // ---- Q: lane (n, kh) holds q[h0 + n][16 j + 8 kh .. +8) for the 36 pieces j
-    v_mbcnt_lo_u32_b32 v88, -1, 0
-    v_mbcnt_hi_u32_b32 v88, -1, v88
-    v_and_b32 v89, 31, v88
-    v_lshrrev_b32 v90, 5, v88
-    .if SPLIT
-      v_lshlrev_b32 v88, 10, v89
-      v_lshl_add_u32 v88, v90, 4, v88      // rows of 512 channels
-      v_lshlrev_b32 v91, 7, v89
-      v_lshl_add_u32 v91, v90, 4, v91      // rows of 64 channels
-      .irp j,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15,16,17,18,19,20,21,22,23,24,25,26,27,28,29,30,31
-        global_load_dwordx4 v[112+4*\j:115+4*\j], v88, %[q] offset:32*\j
-      .endr
-      .irp j,32,33,34,35
-        global_load_dwordx4 v[112+4*\j:115+4*\j], v91, %[qrope] offset:32*(\j-32)
-      .endr
-    .else
-      v_mul_u32_u24 v88, 1152, v89
-      v_lshl_add_u32 v88, v90, 4, v88
-      .irp j,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15,16,17,18,19,20,21,22,23,24,25,26,27,28,29,30,31,32,33,34,35
-        global_load_dwordx4 v[112+4*\j:115+4*\j], v88, %[q] offset:32*\j
-      .endr
-    .endif
     // ---- O = 0, written by the matrix pipe itself
     v_mov_b32 v64, 0
     v_mov_b32 v65, 0
@@ -701,9 +706,7 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     v_log_f32 v85, v83
     s_nop 1
     v_add_f32 v85, v85, v82                // log2 of the sum of 2^score
-    s_cmp_eq_u32 %[complete], 0
-    s_cbranch_scc1 13f
-    // ---- final row: out[h0 + n][32 i + 8 r + 4 kh .. +4) in the query's type
+    // ---- the row in the query's type: out[h0 + n][32 i + 8 r + 4 kh .. +4); a partial row has the same form
     v_lshlrev_b32 v91, 10, v89
     v_lshl_add_u32 v91, v90, 3, v91
     .irp i,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15
@@ -728,6 +731,9 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
         global_store_dwordx2 v91, v[32+8*(\i%%2)+2*\r:33+8*(\i%%2)+2*\r], %[out] offset:(32*\i+8*\r)*2
       .endr
     .endr
+    s_mov_b64 s[60:61], exec
+    s_cmp_eq_u32 %[complete], 0
+    s_cbranch_scc1 13f
     s_cmp_eq_u64 %[lse], 0
     s_cbranch_scc1 14f
     // natural-log log-sum-exp of the row, by the kh = 0 lanes
@@ -738,30 +744,14 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     .else
       v_cvt_f16_f32 v85, v85
     .endif
-    s_mov_b64 s[60:61], exec
     s_mov_b64 exec, 0xffffffff
     s_nop 1
     global_store_short v91, v85, %[lse]
     s_mov_b64 exec, s[60:61]
     s_branch 14f
     13:
-    // ---- partial row: normalised fp32 channels and the base-2 log-sum-exp
-    v_lshlrev_b32 v91, 11, v89
-    v_lshl_add_u32 v91, v90, 4, v91
-    .irp i,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15
-      .irp c,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15
-        v_accvgpr_read_b32 v[16*(\i%%2)+\c], a[16*\i+\c]
-      .endr
-      .irp c,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15
-        v_mul_f32 v[16*(\i%%2)+\c], v[16*(\i%%2)+\c], v84
-      .endr
-      s_nop 1
-      .irp r,0,1,2,3
-        global_store_dwordx4 v91, v[16*(\i%%2)+4*\r:16*(\i%%2)+4*\r+3], %[out] offset:(32*\i+8*\r)*4
-      .endr
-    .endr
+    // partial row: its base-2 log-sum-exp, fp32
     v_lshlrev_b32 v91, 2, v89
-    s_mov_b64 s[60:61], exec
     s_mov_b64 exec, 0xffffffff
     s_nop 1
     global_store_dword v91, v85, %[lse]
@@ -853,7 +843,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaAsmKernel(const PaArgs a, const
         } else {
             const int slot = 2 * wr + (segBegin == s0 ? 0 : 1);
             const int64_t ph = static_cast<int64_t>(slot) * a.H + h0;
-            sg.out = a.partO + ph * DV;
+            sg.out = reinterpret_cast<uint16_t *>(a.partO) + ph * DV;
             sg.lse = a.partLse + ph;
         }
         RunSegment<BF16, SPLIT>(sg, ldsBase, wave, scale2);

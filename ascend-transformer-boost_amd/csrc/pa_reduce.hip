@@ -66,11 +66,45 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaReduceKernel(const PaArgs a)
 // head): it takes the maximum of the row's log-sum-exps, then adds up the
 // weighted partial rows with 16-byte loads. A workgroup of 128 threads covers as
 // many whole rows as fit (four for 128 channels, one for 512).
+// HALF: the partial rows are 16-bit values of the query's type and a thread owns eight channels.
 typedef float ReduceF4 __attribute__((ext_vector_type(4)));
 
+// A thread's piece of one partial row, kept as loaded (16 bytes) until it is accumulated.
+template <bool HALF> struct PartialPiece;
+template <> struct PartialPiece<false> {
+    static constexpr int CH = 4;
+    ReduceF4 raw;
+    __device__ __forceinline__ void Clear() { raw = ReduceF4{0.0f, 0.0f, 0.0f, 0.0f}; }
+    __device__ __forceinline__ void Load(const float *partO, int64_t elem)
+    {
+        raw = *reinterpret_cast<const ReduceF4 *>(partO + elem);
+    }
+    __device__ __forceinline__ float Get(int e, bool) const { return raw[e]; }
+};
+template <> struct PartialPiece<true> {
+    static constexpr int CH = 8;
+    uint32_t raw[4];
+    __device__ __forceinline__ void Clear() { raw[0] = raw[1] = raw[2] = raw[3] = 0u; }
+    __device__ __forceinline__ void Load(const float *partO, int64_t elem)
+    {
+        const uint4 x = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(partO) + elem);
+        raw[0] = x.x; raw[1] = x.y; raw[2] = x.z; raw[3] = x.w;
+    }
+    __device__ __forceinline__ float Get(int e, bool bf16) const
+    {
+        const uint32_t w = raw[e >> 1];
+        if (bf16) {
+            return __uint_as_float((e & 1) ? (w & 0xffff0000u) : (w << 16));
+        }
+        return HalfBitsToFloat(static_cast<uint16_t>((e & 1) ? (w >> 16) : (w & 0xffffu)));
+    }
+};
+
+template <bool HALF, bool BF16>
 __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaArgs a, const PaStreamPlan p)
 {
-    const int vecs = a.Dv / 4;                                        // threads per row
+    constexpr int CH = PartialPiece<HALF>::CH;                        // channels per thread
+    const int vecs = a.Dv / CH;                                       // threads per row
     const int rowsPerWg = vecs >= REDUCE_THREADS ? 1 : REDUCE_THREADS / vecs;
     const int rowsPerSlot = a.H * p.foldTokens;
     const int tid = threadIdx.x;
@@ -101,76 +135,85 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaA
     auto rowOf = [&](int k) { return k == 0 ? ph0 : phEven + k * stride; };
 
     const int g = h / a.groupSize;
-    const bool bf16 = a.qIsBf16 != 0;
+    constexpr bool bf16 = BF16;
     const int64_t outRow = static_cast<int64_t>(sq.qRow + tok) * a.H + h;
-    // Rows of up to MAX_HELD ranges (nearly all): the log-sum-exps and the thread's pieces of the partial
-    // rows are requested together and held in registers, one memory round trip; longer rows take the
-    // log-sum-exps first and the pieces in a second pass.
+    // 2^x on the hardware unit: -inf gives 0, which is what an empty range must weigh
+    auto pow2 = [](float x) { return __builtin_amdgcn_exp2f(x); };
+    // The ranges of a row are taken MAX_HELD at a time: their log-sum-exps and the thread's pieces of their
+    // partial rows are requested together and held as loaded, one memory round trip for nearly every row;
+    // a longer row carries its running maximum and sums from one group of ranges to the next.
     constexpr int MAX_HELD = 8;
-    const bool held = count <= MAX_HELD;
-    float lseHeld[MAX_HELD];
-    float mx = -INFINITY;
-    if (!held) {
-        for (int k = 0; k < count; ++k) {
-            mx = fmaxf(mx, a.partLse[rowOf(k)]);
+#pragma unroll 1
+    for (int c = vecs >= REDUCE_THREADS ? tid : tid % vecs; c < vecs; c += REDUCE_THREADS) {
+        float acc[CH];
+#pragma unroll
+        for (int e = 0; e < CH; ++e) {
+            acc[e] = 0.0f;
         }
-    }
-    for (int c4 = vecs >= REDUCE_THREADS ? tid : tid % vecs; c4 < vecs; c4 += REDUCE_THREADS) {
-        ReduceF4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
         float sum = 0.0f;
-        if (held) {
-            ReduceF4 piece[MAX_HELD];
+        float mx = -INFINITY;
+#pragma unroll 1
+        for (int k0 = 0; k0 < count; k0 += MAX_HELD) {
+            float lseHeld[MAX_HELD];
+            PartialPiece<HALF> piece[MAX_HELD];
 #pragma unroll
             for (int k = 0; k < MAX_HELD; ++k) {
                 lseHeld[k] = -INFINITY;
-                piece[k] = ReduceF4{0.0f, 0.0f, 0.0f, 0.0f};
-                if (k < count) {
-                    const int64_t ph = rowOf(k);
+                piece[k].Clear();
+                if (k0 + k < count) {
+                    const int64_t ph = rowOf(k0 + k);
                     lseHeld[k] = a.partLse[ph];
-                    piece[k] = *reinterpret_cast<const ReduceF4 *>(a.partO + ph * a.Dv + c4 * 4);
+                    piece[k].Load(a.partO, ph * a.Dv + c * CH);
                 }
             }
-            mx = -INFINITY;
+            float mNew = mx;
 #pragma unroll
             for (int k = 0; k < MAX_HELD; ++k) {
-                mx = fmaxf(mx, lseHeld[k]);
+                mNew = fmaxf(mNew, lseHeld[k]);
             }
+            if (k0 > 0 && mNew > mx) { // (mx is finite here or everything so far weighed nothing)
+                const float keep = pow2(mx - mNew);
+                sum *= keep;
+#pragma unroll
+                for (int e = 0; e < CH; ++e) {
+                    acc[e] *= keep;
+                }
+            }
+            mx = mNew;
 #pragma unroll
             for (int k = 0; k < MAX_HELD; ++k) {
                 // a range that a -inf mask emptied (and a slot past the row's ranges) weighs nothing
-                const float w = lseHeld[k] == -INFINITY ? 0.0f : exp2f(lseHeld[k] - mx);
+                const float w = mx == -INFINITY ? 0.0f : pow2(lseHeld[k] - mx);
                 sum += w;
-                acc += w * piece[k];
-            }
-        } else {
-#pragma unroll 4
-            for (int k = 0; k < count; ++k) {
-                const int64_t ph = rowOf(k);
-                const float lse = a.partLse[ph];
-                const float w = lse == -INFINITY ? 0.0f : exp2f(lse - mx); // a range a -inf mask emptied weighs nothing
-                sum += w;
-                acc += w * *reinterpret_cast<const ReduceF4 *>(a.partO + ph * a.Dv + c4 * 4);
+#pragma unroll
+                for (int e = 0; e < CH; ++e) {
+                    acc[e] += w * piece[k].Get(e, bf16);
+                }
             }
         }
         const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
-        float o[4] = {acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv};
-        if (a.finishV) {
+        uint16_t bits[CH];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int ch = g * a.Dv + c4 * 4 + e;
-                o[e] = (o[e] + (a.vOff ? static_cast<float>(a.vOff[ch]) : 0.0f)) * a.vScale[ch * a.scaleStride];
+        for (int e = 0; e < CH; ++e) {
+            float o = acc[e] * inv;
+            if (a.finishV) {
+                const int ch = g * a.Dv + c * CH + e;
+                o = (o + (a.vOff ? static_cast<float>(a.vOff[ch]) : 0.0f)) * a.vScale[ch * a.scaleStride];
             }
+            bits[e] = bf16 ? FloatToBf16(o) : FloatToHalfBits(o);
         }
-        uint16_t bits[4];
+        uint32_t packed[CH / 2];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            bits[e] = bf16 ? FloatToBf16(o[e]) : FloatToHalfBits(o[e]);
+        for (int e = 0; e < CH / 2; ++e) {
+            packed[e] = static_cast<uint32_t>(bits[2 * e]) | (static_cast<uint32_t>(bits[2 * e + 1]) << 16);
         }
-        uint2 packed;
-        packed.x = static_cast<uint32_t>(bits[0]) | (static_cast<uint32_t>(bits[1]) << 16);
-        packed.y = static_cast<uint32_t>(bits[2]) | (static_cast<uint32_t>(bits[3]) << 16);
-        *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(a.out) + outRow * a.Dv + c4 * 4) = packed;
-        if (a.lse && c4 == 0) {
+        uint16_t *dst = reinterpret_cast<uint16_t *>(a.out) + outRow * a.Dv + c * CH;
+        if constexpr (HALF) {
+            *reinterpret_cast<uint4 *>(dst) = uint4{packed[0], packed[1], packed[2], packed[3]};
+        } else {
+            *reinterpret_cast<uint2 *>(dst) = uint2{packed[0], packed[1]};
+        }
+        if (a.lse && c == 0) {
             Store16(a.lse, outRow, (mx + log2f(sum)) * LN2, bf16);
         }
     }
@@ -182,7 +225,7 @@ int LaunchPaStreamReduce(const AtbmiPaShape &shape, const PaArgs &args, const Pa
                          hipStream_t stream)
 {
     (void)shape;
-    const int vecs = args.Dv / 4;
+    const int vecs = args.Dv / (args.partHalf ? 8 : 4);
     const int rowsPerWg = vecs >= REDUCE_THREADS ? 1 : REDUCE_THREADS / vecs;
     const int64_t rows = static_cast<int64_t>(plan.numSeqs) * plan.foldTokens * args.H;
     const int64_t grid = (rows + rowsPerWg - 1) / rowsPerWg;
@@ -192,7 +235,18 @@ int LaunchPaStreamReduce(const AtbmiPaShape &shape, const PaArgs &args, const Pa
     if (grid > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "pa_reduce: grid of %lld workgroups is out of range", (long long)grid);
     }
-    PaStreamReduceKernel<<<static_cast<unsigned>(grid), REDUCE_THREADS, 0, stream>>>(args, plan);
+    const unsigned blocks = static_cast<unsigned>(grid);
+    if (args.partHalf) {
+        if (args.qIsBf16) {
+            PaStreamReduceKernel<true, true><<<blocks, REDUCE_THREADS, 0, stream>>>(args, plan);
+        } else {
+            PaStreamReduceKernel<true, false><<<blocks, REDUCE_THREADS, 0, stream>>>(args, plan);
+        }
+    } else if (args.qIsBf16) {
+        PaStreamReduceKernel<false, true><<<blocks, REDUCE_THREADS, 0, stream>>>(args, plan);
+    } else {
+        PaStreamReduceKernel<false, false><<<blocks, REDUCE_THREADS, 0, stream>>>(args, plan);
+    }
     ATBMI_HIP_CHECK(hipGetLastError());
     return OK;
 }
