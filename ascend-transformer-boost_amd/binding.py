@@ -239,6 +239,8 @@ def kernels():
         lib.atbmi_pa_plan_destroy.restype = None
         lib.atbmi_timing_enable.argtypes = [i32]
         lib.atbmi_timing_read.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(i64)]
+        lib.atbmi_timing_read_split.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
+                                                ctypes.POINTER(i64)]
         _kernels = lib
     return _kernels
 

@@ -57,7 +57,8 @@ int64_t EnvInt(const char *name, int64_t fallback)
 
 struct TimingRecord {
     hipEvent_t begin;
-    hipEvent_t end;
+    hipEvent_t end;    // after the attention kernel
+    hipEvent_t merged; // after the merge kernel (null when the call needs none)
 };
 // Scratch of the entry point that allocates nothing (atbmi_pa_decode_static): the partial rows and
 // log-sum-exps a plan would otherwise keep in the caller's workspace. Every device the library runs on
@@ -772,7 +773,7 @@ int DecodeImpl(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void *workspace, uint
     a.lse = t->lse;
     a.partHalf = (plan->useMfma && PaMlaWide(s)) ? 1 : 0;
 
-    TimingRecord rec{nullptr, nullptr};
+    TimingRecord rec{nullptr, nullptr, nullptr};
     bool timed = false;
     {
         std::lock_guard<std::mutex> lock(g_timingMutex);
@@ -794,16 +795,25 @@ int DecodeImpl(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void *workspace, uint
     }
     if (timed) {
         ATBMI_HIP_CHECK(hipEventRecord(rec.end, stream));
+    }
+    bool merged = false;
+    if (rc == OK) {
+        if (plan->useMfma) {
+            merged = plan->streamNeedsReduce;
+            rc = merged ? LaunchPaStreamReduce(s, a, sp, stream) : OK;
+        } else {
+            merged = !plan->reduceSeqs.empty();
+            rc = LaunchPaReduce(s, a, static_cast<int>(plan->reduceSeqs.size()), stream);
+        }
+    }
+    if (timed) {
+        if (merged && rc == OK && hipEventCreate(&rec.merged) == hipSuccess) {
+            (void)hipEventRecord(rec.merged, stream);
+        }
         std::lock_guard<std::mutex> lock(g_timingMutex);
         g_timingRecords.push_back(rec);
     }
-    if (rc != OK) {
-        return rc;
-    }
-    if (plan->useMfma) {
-        return plan->streamNeedsReduce ? LaunchPaStreamReduce(s, a, sp, stream) : OK;
-    }
-    return LaunchPaReduce(s, a, static_cast<int>(plan->reduceSeqs.size()), stream);
+    return rc;
 }
 
 } // namespace
@@ -864,27 +874,41 @@ extern "C" int atbmi_timing_enable(int32_t enable)
     return OK;
 }
 
-extern "C" int atbmi_timing_read(double *totalMs, int64_t *launches)
+extern "C" int atbmi_timing_read_split(double *kernelMs, double *withMergeMs, int64_t *launches)
 {
     std::vector<TimingRecord> records;
     {
         std::lock_guard<std::mutex> lock(g_timingMutex);
         records.swap(g_timingRecords);
     }
-    double sum = 0.0;
+    double sum = 0.0, sumMerged = 0.0;
     for (const TimingRecord &r : records) {
-        ATBMI_HIP_CHECK(hipEventSynchronize(r.end));
-        float ms = 0.0f;
+        hipEvent_t last = r.merged ? r.merged : r.end;
+        ATBMI_HIP_CHECK(hipEventSynchronize(last));
+        float ms = 0.0f, msMerged = 0.0f;
         ATBMI_HIP_CHECK(hipEventElapsedTime(&ms, r.begin, r.end));
+        ATBMI_HIP_CHECK(hipEventElapsedTime(&msMerged, r.begin, last));
         sum += ms;
+        sumMerged += msMerged;
         (void)hipEventDestroy(r.begin);
         (void)hipEventDestroy(r.end);
+        if (r.merged) {
+            (void)hipEventDestroy(r.merged);
+        }
     }
-    if (totalMs) {
-        *totalMs = sum;
+    if (kernelMs) {
+        *kernelMs = sum;
+    }
+    if (withMergeMs) {
+        *withMergeMs = sumMerged;
     }
     if (launches) {
         *launches = static_cast<int64_t>(records.size());
     }
     return OK;
+}
+
+extern "C" int atbmi_timing_read(double *totalMs, int64_t *launches)
+{
+    return atbmi_timing_read_split(totalMs, nullptr, launches);
 }

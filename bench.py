@@ -7,10 +7,14 @@ on one MI355X, synthetic data of the named configuration.
 Prints ONE JSON line: whole-step throughput (tokens/s = sequences decoded per
 second, inputs resident in HBM), the attention kernel's achieved HBM bandwidth
 against the 8 TB/s roofline (algorithmic bytes / mean kernel time from HIP
-events on the launch stream), and the CPU oracle timed on a bounded sample of
-the same workload.
+events on the launch stream; `frac_with_merge` counts the merge kernel that
+follows it as well), and the CPU oracle timed on a bounded sample of the same
+workload. Run without --config, the line describes the bf16 8B-shaped step (C2)
+and carries, under "configs", the same measurements of the other workloads of
+the benchmark (C2 in fp16, C3 int8-KV, C4 skewed, C5 MLA), fewer steps each.
 """
 import argparse
+import hashlib
 import importlib
 import json
 import os
@@ -23,13 +27,40 @@ if ROOT not in sys.path:
 PKG = "ascend-transformer-boost_amd"
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes one attention launch moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this
-# script, scaled by what the same counters read for a 256 MiB copy (--calibrate-copy); the runs and the
-# scale factors are written up in the profiles/ summaries of each workload. Keyed by workload and its
-# algorithmic bytes, so a changed workload reports null instead of a stale figure.
-MEASURED_TRAFFIC = {("c2", 651658484): 658.7e6, ("c2_alibi", 661824180): 669.5e6, ("c2_mtp4", 656075180): 683.6e6,
-                    ("c3", 1364204576): 1379.2e6, ("c5", 253384304): 388.7e6,
-                    ("c5_split", 253384304): 378.4e6}
+# HBM bytes one attention launch moves (attention kernel + its merge kernel), from rocprofv3 FETCH_SIZE /
+# WRITE_SIZE counter runs of this script, scaled by what the same counters read for a 256 MiB copy
+# (--calibrate-copy). Each figure names the profile summary it comes from and the hash of the attention
+# kernel sources it was measured on: a changed workload or changed kernels report null, not a stale figure.
+MEASURED_TRAFFIC = {
+    # (workload, algorithmic bytes): (HBM bytes, summary under profiles/, kernel source hash)
+}
+KERNEL_SOURCES = ["atbmi_common.h", "pa_internal.h", "pa_host.hip", "pa_mfma_kernel.h", "pa_mfma.hip",
+                  "pa_mfma_dispatch.inc", "pa_mla_kernel.h", "pa_mla.hip", "pa_reduce.hip"]
+OTHER_WORKLOADS = ["c2_fp16", "c3", "c4", "c5"]  # timed in the same run as the headline workload
+
+
+def kernel_source_hash():
+    """Short hash of the attention kernels' sources (what MEASURED_TRAFFIC figures are tied to)."""
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, PKG, "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:12]
+
+
+def cpu_description():
+    """(logical cores of the host, model string) as the kernel reports them."""
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return os.cpu_count() or 1, model
+
 
 DESCRIPTIONS = {
     "c1": "C1 small fp16 decode: batch 4, 8 q heads, 8 kv heads, d128, block 128, ctx U[64,512]",
@@ -57,11 +88,13 @@ def cpu_baseline(pkg, step, cfg, scale, budget_s=10.0):
     work are spent; returns tokens/s (one token per sequence) on that sample."""
     import numpy as np
     oracle = importlib.import_module("oracle.atb_oracle")
+    # threads numpy's BLAS may use (the oracle's matrix products are the only parallel part)
     try:
         from threadpoolctl import threadpool_info
         threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
-    except Exception:
-        threads = 1
+    except ImportError:
+        threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    host_cores, cpu_model = cpu_description()
     ctx = step["layout"]["ctx"]
     tables = step["layout"]["tables"]
     dev_q = step["q"]
@@ -102,34 +135,23 @@ def cpu_baseline(pkg, step, cfg, scale, budget_s=10.0):
         "value": done / spent if spent > 0 else 0.0,
         "unit": "tokens/s",
         "cores": threads,
+        "host_cores": host_cores,
+        "cpu_model": cpu_model,
         "kind": "port",
         "sample": "numpy oracle on %d query tokens of sequences drawn in order from the batch of %d "
                   "(%d context tokens), attention only, %.1f s" % (done, len(ctx), tokens, spent),
     }
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", default="c2", choices=sorted(DESCRIPTIONS))
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--attention-only", action="store_true", help="leave ReshapeAndCache out of the step")
-    ap.add_argument("--no-kernel-events", action="store_true", help="do not bracket the attention kernel with events")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run one 256 MiB device copy, as the known-size reference for hardware counters")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build runs on exactly one GPU; --gpus %d is not supported" % args.gpus)
-
+def run_workload(pkg, name, steps, warmup, attention_only=False, kernel_events=True, calibrate_copy=False,
+                 want_cpu_baseline=False):
+    """Sets one workload up on cuda:0, times `steps` decode steps after `warmup` untimed ones and returns
+    the measurements (and, on request, the CPU baseline on the same inputs)."""
+    import ctypes
     import torch
-    pkg = importlib.import_module(PKG)
     b, w = pkg.binding, pkg.workloads
-    if not torch.cuda.is_available():
-        sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
-    cfg = w.config(args.config)
+    cfg = w.config(name)
     step = w.make_step(cfg, dev)
     scale = w.qk_scale(cfg)
     stream = torch.cuda.Stream(device=dev)
@@ -145,7 +167,7 @@ def main():
                                      maskType=mask_type, calcType=1 if q_len > 1 else 0,
                                      inputLayout=1 if cfg.get("bnsd") else 0)
     if cfg.get("bnsd"):
-        args.attention_only = True
+        attention_only = True
     split = bool(cfg.get("split"))
     if split:
         pa = b.OperationRunner("MultiLatentAttentionOperation", b.MultiLatentAttentionParam(
@@ -197,7 +219,7 @@ def main():
     slots = cfg["block"] * step["layout"]["pool"]
 
     def one_step():
-        if not args.attention_only:
+        if not attention_only:
             if int8:
                 # the quantised cache write: fp16 rows -> int8 slots
                 rc = k.atbmi_reshape_and_cache_quant(
@@ -210,59 +232,124 @@ def main():
                 rac.run(rac_in, outputs=rac_out)
         pa.run(pa_in, outputs=[out], host_inputs=host_inputs)
 
-    if args.calibrate_copy:
+    if calibrate_copy:
         with torch.cuda.stream(stream):
             src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
             dst = torch.empty_like(src)
             dst.copy_(src)
         stream.synchronize()
     with torch.cuda.stream(stream):
-        for _ in range(args.warmup):
+        for _ in range(warmup):
             one_step()
         stream.synchronize()
         torch.cuda.synchronize()
         # every 4th attention launch is bracketed with HIP events on the launch stream
-        k.atbmi_timing_enable(0 if args.no_kernel_events else 4)
+        k.atbmi_timing_enable(4 if kernel_events else 0)
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(steps):
             one_step()
         stream.synchronize()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
-    import ctypes
-    total_ms = ctypes.c_double(0)
+    kernel_total = ctypes.c_double(0)
+    merged_total = ctypes.c_double(0)
     launches = ctypes.c_int64(0)
-    k.atbmi_timing_read(ctypes.byref(total_ms), ctypes.byref(launches))
+    k.atbmi_timing_read_split(ctypes.byref(kernel_total), ctypes.byref(merged_total), ctypes.byref(launches))
     k.atbmi_timing_enable(0)
 
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    ms_per_step = (t1 - t0) * 1e3 / steps
     alg_bytes = w.algorithmic_bytes(cfg, step["layout"]["ctx"])
-    kernel_ms = total_ms.value / max(1, launches.value)
+    kernel_ms = kernel_total.value / max(1, launches.value)
+    with_merge_ms = merged_total.value / max(1, launches.value)
     achieved = alg_bytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
+    with_merge = alg_bytes / (with_merge_ms * 1e-3) / 1e9 if with_merge_ms > 0 else 0.0
+    traffic, source = None, None
+    entry = MEASURED_TRAFFIC.get((name, alg_bytes))
+    if entry is not None:
+        if entry[2] == kernel_source_hash():
+            traffic, source = entry[0], "profiles/" + entry[1]
+        else:
+            source = "none: the attention kernels changed since profiles/%s was taken" % entry[1]
+    measured = {
+        "workload": DESCRIPTIONS[name],
+        "step": ("%s only" if attention_only else "ReshapeAndCache + %s (Setup + Execute each)") % (
+            "MultiLatentAttention" if split else "PagedAttention"),
+        "context_tokens": int(step["layout"]["ctx"].sum()),
+        "rows": rows,
+        "dtype": "int8" if int8 else cfg["dtype"],
+        "steps": steps,
+        "ms_per_step": ms_per_step,
+        "tokens_per_s": rows / (ms_per_step * 1e-3),
+        "roofline": {"bound": "hbm", "kernel": "paged attention decode", "achieved": achieved,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+                     "frac_with_merge": with_merge / HBM_PEAK_GBPS, "traffic": traffic, "traffic_source": source,
+                     "algorithmic_bytes": alg_bytes, "kernel_ms": kernel_ms, "kernel_with_merge_ms": with_merge_ms,
+                     "launches": launches.value},
+        "step_hbm_gbps": alg_bytes / (ms_per_step * 1e-3) / 1e9,
+    }
+    baseline = cpu_baseline(pkg, step, cfg, scale) if want_cpu_baseline else None
+    if rac is not None:
+        rac.close()
+    pa.close()
+    ctx.close()
+    del step, out, pa_in
+    torch.cuda.empty_cache()
+    return measured, baseline
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default=None, choices=sorted(DESCRIPTIONS),
+                    help="time this workload alone (default: c2, followed by the benchmark's other workloads)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--attention-only", action="store_true", help="leave ReshapeAndCache out of the step")
+    ap.add_argument("--no-kernel-events", action="store_true", help="do not bracket the attention kernel with events")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device copy, as the known-size reference for hardware counters")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU; --gpus %d is not supported" % args.gpus)
+
+    import torch
+    pkg = importlib.import_module(PKG)
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    headline = args.config or "c2"
+    m, baseline = run_workload(pkg, headline, args.steps, args.warmup, attention_only=args.attention_only,
+                               kernel_events=not args.no_kernel_events, calibrate_copy=args.calibrate_copy,
+                               want_cpu_baseline=not args.no_cpu_baseline)
     result = {
         "metric": "paged_attention_decode_tokens_per_s",
-        "value": rows / (ms_per_step * 1e-3),
+        "value": m["tokens_per_s"],
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
+        "ms_per_step": m["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int8" if int8 else cfg["dtype"],
+        "dtype": m["dtype"],
         "data": "synthetic",
-        "config": {"workload": DESCRIPTIONS[args.config], "step": ("%s only" if args.attention_only else "ReshapeAndCache + %s (Setup + Execute each)") % (
-                       "MultiLatentAttention" if split else "PagedAttention"),
-                   "context_tokens": int(step["layout"]["ctx"].sum())},
-        "roofline": {"bound": "hbm", "kernel": "paged attention decode", "achieved": achieved,
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": MEASURED_TRAFFIC.get((args.config, alg_bytes)),
-                     "algorithmic_bytes": alg_bytes, "kernel_ms": kernel_ms, "launches": launches.value},
-        "step_hbm_gbps": alg_bytes / (ms_per_step * 1e-3) / 1e9,
+        "config": {"workload": m["workload"], "step": m["step"], "context_tokens": m["context_tokens"]},
+        "roofline": m["roofline"],
+        "step_hbm_gbps": m["step_hbm_gbps"],
+        "kernel_source_hash": kernel_source_hash(),
     }
-    if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(pkg, step, cfg, scale)
+    if baseline is not None:
+        result["cpu_baseline"] = baseline
+    if args.config is None:
+        # the other workloads of the benchmark, same procedure; the timed steps are capped so that the
+        # whole run stays within a few minutes whatever --steps asks of the headline workload
+        others = {}
+        for name in OTHER_WORKLOADS:
+            om, _ = run_workload(pkg, name, min(args.steps, 100), min(args.warmup, 10),
+                                 kernel_events=not args.no_kernel_events)
+            others[name] = om
+        result["configs"] = others
     print(json.dumps(result))
 
 

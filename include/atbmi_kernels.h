@@ -380,6 +380,9 @@ void atbmi_pa_plan_destroy(AtbmiPaPlan *plan);
  */
 int atbmi_timing_enable(int32_t enable);
 int atbmi_timing_read(double *totalMs, int64_t *launches);
+/* The same, and also the sum from the start of the attention kernel to the end of the merge kernel that
+ * follows it (equal to the first sum for calls that need no merge). Any pointer may be NULL. */
+int atbmi_timing_read_split(double *kernelMs, double *withMergeMs, int64_t *launches);
 
 #ifdef __cplusplus
 }
