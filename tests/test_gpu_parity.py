@@ -1112,6 +1112,9 @@ MLA_MATRIX = [
     (64, 32, 192, 128, 128, 256, torch.float16),
     (32, 8, 576, 512, 128, 819, torch.float16),
     (4, 128, 576, 512, 128, [3000, 17, 128, 1025], torch.bfloat16),
+    (1, 16, 576, 512, 256, 256, torch.float16),      # block size 256: reference test_paged_attention_mla.py:1137-1152
+    (3, 16, 576, 512, 256, [700, 256, 257], torch.bfloat16),
+    (2, 128, 576, 512, 256, [2000, 511], torch.float16),  # ... and on the 128-head kernel
 ]
 
 
@@ -1234,6 +1237,9 @@ MASK_MATRIX = [
     ("norm3", 8, 64, 8, 128, 128, 1200, 1200, torch.float16, False, True),
     ("alibi4", 4, 32, 16, 64, 128, [100, 2000, 64, 777], 2000, torch.float16, False, True),
     ("norm3", 3, 24, 1, 16, 256, [3000, 5, 12000], 12000, torch.float16, False, False),
+    # reference test_paged_attention_common.py:2660-2671 (bf16, ALiBi mask, 32 768 tokens, split over many ranges);
+    # three of its twelve sequences, one of them at the full length
+    ("alibi4", 3, 12, 1, 128, 128, [32768, 2049, 700], 32768, torch.bfloat16, False, False),
 ]
 
 
