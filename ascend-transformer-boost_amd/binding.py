@@ -14,7 +14,8 @@ import ctypes
 import os
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-_LIB = os.path.join(_PKG, "lib")
+# ATB_MI_LIB_DIR names another build of the two libraries (the sanitizer build, lib_sanitize)
+_LIB = os.environ.get("ATB_MI_LIB_DIR") or os.path.join(_PKG, "lib")
 
 # aclDataType / aclFormat values (include/acl/acl.h)
 ACL_FLOAT, ACL_FLOAT16, ACL_INT8, ACL_INT32, ACL_INT64, ACL_BF16 = 0, 1, 2, 3, 9, 27

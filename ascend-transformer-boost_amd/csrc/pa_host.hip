@@ -10,6 +10,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <mutex>
 #include <new>
 #include <vector>
@@ -22,6 +23,42 @@ namespace atbmi {
 
 namespace {
 thread_local char g_lastError[512] = "";
+std::mutex g_deviceMutex;
+std::map<std::pair<const void *, int>, int> g_ldsConfigured; // (kernel, device) -> bytes set
+std::map<int, int> g_computeUnits;                            // device -> compute units
+}
+
+int ConfigureKernelLds(const void *kernel, int ldsBytes)
+{
+    int dev = 0;
+    ATBMI_HIP_CHECK(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_deviceMutex);
+    int &have = g_ldsConfigured[std::make_pair(kernel, dev)];
+    if (have < ldsBytes) {
+        ATBMI_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes));
+        have = ldsBytes;
+    }
+    return OK;
+}
+
+int DeviceComputeUnits()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    std::lock_guard<std::mutex> lock(g_deviceMutex);
+    int &cus = g_computeUnits[dev];
+    if (cus <= 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            n = 256;
+        }
+        cus = n;
+    }
+    return cus;
 }
 
 int Fail(int code, const char *fmt, ...)
@@ -37,7 +74,7 @@ namespace {
 
 constexpr uint64_t WS_ALIGN = 256;
 constexpr int RING = 4;
-constexpr int NUM_CUS = 256;
+constexpr int DEFAULT_CUS = 256;
 
 uint64_t AlignUp(uint64_t v, uint64_t a)
 {
@@ -107,6 +144,7 @@ struct AtbmiPaPlan {
     int partialsPerItem = 1; // scalar kernel: partial slots one work item writes
     int tokenUnit = 1;       // scalar kernel: chunk lengths are multiples of this
     int mfmaWaves = 8;       // MFMA kernel: waves per workgroup
+    int numCus = DEFAULT_CUS; // compute units of the device the plan was created on
     int64_t chunkOverride = 0;
     int64_t minStepsOverride = 0;
 
@@ -253,6 +291,7 @@ extern "C" int atbmi_pa_plan_create(const AtbmiPaShape *shape, AtbmiPaPlan **pla
         p->partialsPerItem = PA_SCALAR_WAVES;
         p->tokenUnit = PA_SCALAR_WAVES;
     }
+    p->numCus = DeviceComputeUnits();
     p->chunkOverride = EnvInt("ATBMI_PA_CHUNK_TOKENS", 0);
     p->minStepsOverride = EnvInt("ATBMI_PA_MIN_STEPS", 0);
     *plan = p;
@@ -319,7 +358,7 @@ int PlanStream(AtbmiPaPlan *plan)
         // One workgroup per CU and head group is the most that runs at once;
         // short batches use fewer so that a wave still has a few steps to do.
         const int64_t minSteps = plan->minStepsOverride > 0 ? plan->minStepsOverride : 2;
-        int64_t wgRanges = std::max<int64_t>(1, NUM_CUS / headGroups);
+        int64_t wgRanges = std::max<int64_t>(1, plan->numCus / headGroups);
         if (plan->chunkOverride > 0) {
             // test hook: ranges of about this many tokens
             const int64_t per = std::max<int64_t>(1, plan->chunkOverride / PA_MFMA_STEP) * tokenSlices;
@@ -499,7 +538,7 @@ extern "C" int atbmi_pa_plan_update_multi(AtbmiPaPlan *plan, const int32_t *ctx,
     const int64_t unit = plan->tokenUnit;
     int64_t chunk = plan->chunkOverride;
     if (chunk <= 0) {
-        const int64_t targetWgs = static_cast<int64_t>(NUM_CUS) * 8;
+        const int64_t targetWgs = static_cast<int64_t>(plan->numCus) * 8;
         const int64_t targetItems = std::max<int64_t>(1, targetWgs / wgPerItem);
         chunk = (rowCtx + targetItems - 1) / std::max<int64_t>(1, targetItems);
         const int64_t minChunk = plan->useMfma ? 2 * unit : 64;

@@ -45,6 +45,11 @@ int LaunchPaMfmaF16(const AtbmiPaShape &shape, const PaArgs &args, const PaStrea
 int LaunchPaMfmaBf16(const AtbmiPaShape &shape, const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream);
 int LaunchPaMfmaInt8(const AtbmiPaShape &shape, const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream);
 
+// Raises a kernel's dynamic LDS limit to `ldsBytes` on the current device, once per kernel and device.
+int ConfigureKernelLds(const void *kernel, int ldsBytes);
+// Compute units of the current device (256 when no device can be asked: plans are also made on hosts without a GPU).
+int DeviceComputeUnits();
+
 // Merges the partials of every sequence that has more than one (scalar-kernel plan).
 int LaunchPaReduce(const AtbmiPaShape &shape, const PaArgs &args, int numSeqs, hipStream_t stream);
 // Merges the partials the MFMA kernel left for sequences that span several wave ranges.

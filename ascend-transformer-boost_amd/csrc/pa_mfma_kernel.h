@@ -815,11 +815,9 @@ int LaunchBuild(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream
     auto kernel = PaMfmaKernel<BF16, KV8, D, DV, MLA, PF, NW, SHARED, EXT>;
     constexpr int lds = SHARED ? 2 * WaveLdsBytes<D, DV, MLA>() : NW * WaveLdsBytes<D, DV, MLA>();
     static_assert(lds <= 160 * 1024, "tiles exceed the 160 KB of LDS per CU");
-    static bool configured = false; // one attribute call per instantiation and process
-    if (!configured) {
-        ATBMI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        configured = true;
+    const int configured = ConfigureKernelLds(reinterpret_cast<const void *>(kernel), lds);
+    if (configured != OK) {
+        return configured;
     }
     if (plan.headsPerWg * plan.tokenSlices != NW || (SHARED && plan.tokenSlices != 1)) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: plan made for %d waves, kernel has %d",

@@ -853,11 +853,9 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaAsmKernel(const PaArgs a, const
 template <bool BF16, bool SPLIT> int LaunchAsm(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
 {
     auto kernel = PaMlaAsmKernel<BF16, SPLIT>;
-    static bool configured = false; // one attribute call per instantiation and process
-    if (!configured) {
-        ATBMI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES));
-        configured = true;
+    const int configured = ConfigureKernelLds(reinterpret_cast<const void *>(kernel), LDS_BYTES);
+    if (configured != OK) {
+        return configured;
     }
     if (plan.tokenSlices != 1 || plan.numWaveRanges != plan.numWgRanges ||
         plan.headGroups * PA_MLA_HEADS_PER_WG != args.H || args.G != 1 || args.D != D || args.Dv != DV ||

@@ -55,6 +55,16 @@ atb::Status RunExecute(const char *what, void *workspace, uint64_t workspaceSize
 }
 } // namespace
 
+// A handle that does not convert (more than 8 dims) ends the call with the conversion's own
+// status, as the reference's wrappers do (src/atb/atb_acl/atb_acl_mla.cpp:69-96).
+#define ATB_ACL_CONVERT(expr)               \
+    do {                                    \
+        const atb::Status converted_ = (expr); \
+        if (converted_ != atb::NO_ERROR) {  \
+            return converted_;              \
+        }                                   \
+    } while (0)
+
 extern "C" {
 
 aclTensor *aclCreateTensor(const int64_t *viewDims, uint64_t viewDimsNum, aclDataType dataType, const int64_t *stride,
@@ -178,26 +188,26 @@ atb::Status AtbMLAGetWorkspaceSize(const aclTensor *qNope, const aclTensor *qRop
     atb::VariantPack pack;
     pack.inTensors.resize(6 + (hasMask ? 1 : 0) + (hasQLens ? 1 : 0) + (int8Cache ? 2 : 0));
     size_t i = 0;
-    ToAtbTensor(qNope, &pack.inTensors[i++], true);
-    ToAtbTensor(qRope, &pack.inTensors[i++], true);
-    ToAtbTensor(ctKV, &pack.inTensors[i++], true);
-    ToAtbTensor(kRope, &pack.inTensors[i++], true);
-    ToAtbTensor(blockTables, &pack.inTensors[i++], true);
-    ToAtbTensor(contextLens, &pack.inTensors[i++], false);
+    ATB_ACL_CONVERT(ToAtbTensor(qNope, &pack.inTensors[i++], true));
+    ATB_ACL_CONVERT(ToAtbTensor(qRope, &pack.inTensors[i++], true));
+    ATB_ACL_CONVERT(ToAtbTensor(ctKV, &pack.inTensors[i++], true));
+    ATB_ACL_CONVERT(ToAtbTensor(kRope, &pack.inTensors[i++], true));
+    ATB_ACL_CONVERT(ToAtbTensor(blockTables, &pack.inTensors[i++], true));
+    ATB_ACL_CONVERT(ToAtbTensor(contextLens, &pack.inTensors[i++], false));
     if (hasMask) {
-        ToAtbTensor(mask, &pack.inTensors[i++], true);
+        ATB_ACL_CONVERT(ToAtbTensor(mask, &pack.inTensors[i++], true));
     }
     if (hasQLens) {
-        ToAtbTensor(qSeqLen, &pack.inTensors[i++], false);
+        ATB_ACL_CONVERT(ToAtbTensor(qSeqLen, &pack.inTensors[i++], false));
     }
     if (int8Cache) {
-        ToAtbTensor(qkDescale, &pack.inTensors[i++], true);
-        ToAtbTensor(pvDescale, &pack.inTensors[i++], true);
+        ATB_ACL_CONVERT(ToAtbTensor(qkDescale, &pack.inTensors[i++], true));
+        ATB_ACL_CONVERT(ToAtbTensor(pvDescale, &pack.inTensors[i++], true));
     }
     pack.outTensors.resize(hasLse ? 2 : 1);
-    ToAtbTensor(attenOut, &pack.outTensors[0], true);
+    ATB_ACL_CONVERT(ToAtbTensor(attenOut, &pack.outTensors[0], true));
     if (hasLse) {
-        ToAtbTensor(lse, &pack.outTensors[1], true);
+        ATB_ACL_CONVERT(ToAtbTensor(lse, &pack.outTensors[1], true));
     }
     return (*op)->Setup(pack, *workspaceSize, context);
 }
@@ -231,18 +241,18 @@ atb::Status AtbPagedCacheLoadGetWorkspaceSize(const aclTensor *keyCache, const a
     atb::VariantPack pack;
     pack.inTensors.resize(hasSeqStarts ? 7 : 6);
     size_t i = 0;
-    ToAtbTensor(keyCache, &pack.inTensors[i++], true);
-    ToAtbTensor(valueCache, &pack.inTensors[i++], true);
-    ToAtbTensor(blockTables, &pack.inTensors[i++], true);
-    ToAtbTensor(contextLens, &pack.inTensors[i++], true);
-    ToAtbTensor(key, &pack.inTensors[i++], true);
-    ToAtbTensor(value, &pack.inTensors[i++], true);
+    ATB_ACL_CONVERT(ToAtbTensor(keyCache, &pack.inTensors[i++], true));
+    ATB_ACL_CONVERT(ToAtbTensor(valueCache, &pack.inTensors[i++], true));
+    ATB_ACL_CONVERT(ToAtbTensor(blockTables, &pack.inTensors[i++], true));
+    ATB_ACL_CONVERT(ToAtbTensor(contextLens, &pack.inTensors[i++], true));
+    ATB_ACL_CONVERT(ToAtbTensor(key, &pack.inTensors[i++], true));
+    ATB_ACL_CONVERT(ToAtbTensor(value, &pack.inTensors[i++], true));
     if (hasSeqStarts) {
-        ToAtbTensor(seqStarts, &pack.inTensors[i++], true);
+        ATB_ACL_CONVERT(ToAtbTensor(seqStarts, &pack.inTensors[i++], true));
     }
     pack.outTensors.resize(2);
-    ToAtbTensor(key, &pack.outTensors[0], true);
-    ToAtbTensor(value, &pack.outTensors[1], true);
+    ATB_ACL_CONVERT(ToAtbTensor(key, &pack.outTensors[0], true));
+    ATB_ACL_CONVERT(ToAtbTensor(value, &pack.outTensors[1], true));
     return (*op)->Setup(pack, *workspaceSize, context);
 }
 

@@ -42,15 +42,15 @@ constexpr int64_t MAX_MLA_BATCH = 8192;
 bool CommonParamCheck(const Param &p)
 {
     if (p.headNum <= 0) {
-        ATB_LOG(ERROR) << "headNum should be greater than zero";
+        ATB_LOG(ERROR) << "PagedAttentionParam: headNum = " << p.headNum << ", a positive head count is required";
         return false;
     }
     if (p.kvHeadNum < 0) {
-        ATB_LOG(ERROR) << "kvHeadNum should be no less than zero";
+        ATB_LOG(ERROR) << "PagedAttentionParam: kvHeadNum = " << p.kvHeadNum << " is negative (0 means one KV head per query head)";
         return false;
     }
     if (p.kvHeadNum != 0 && p.headNum % p.kvHeadNum != 0) {
-        ATB_LOG(ERROR) << "headNum mod kvHeadNum should be zero";
+        ATB_LOG(ERROR) << "PagedAttentionParam: " << p.headNum << " query heads do not divide into " << p.kvHeadNum << " KV heads";
         return false;
     }
     return true;

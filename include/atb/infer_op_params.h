@@ -23,8 +23,8 @@ enum InputLayout : int {
 struct ReshapeAndCacheParam {
     enum CompressType : int {
         COMPRESS_TYPE_UNDEFINED = 0,
-        COMPRESS_TYPE_KVHEAD,     // head compression (alibi); not implemented on MI355X
-        COMPRESS_TYPE_KVHEAD_ROPE // head compression (rope); not implemented on MI355X
+        COMPRESS_TYPE_KVHEAD,     // head compression (alibi): inputs + wins, seqLens
+        COMPRESS_TYPE_KVHEAD_ROPE // head compression (rope): inputs + wins, seqLens, offsetIndex
     };
     enum KvCacheCfg : int {
         K_CACHE_V_CACHE = 0, // inputs: key, value, keyCache, valueCache, slotMapping
@@ -43,8 +43,8 @@ struct ReshapeAndCacheParam {
 struct ReshapeAndCacheWithStrideParam {
     enum CompressType : int {
         COMPRESS_TYPE_UNDEFINED = 0,
-        COMPRESS_TYPE_KVHEAD,     // not implemented on MI355X
-        COMPRESS_TYPE_KVHEAD_ROPE // not implemented on MI355X
+        COMPRESS_TYPE_KVHEAD,     // rejected at creation with strided inputs
+        COMPRESS_TYPE_KVHEAD_ROPE // rejected at creation with strided inputs
     };
     enum KvCacheCfg : int {
         K_CACHE_V_CACHE = 0, // inputs: key, value, keyCache, valueCache, slotMapping, kStrides, vStrides, kOffset, vOffset

@@ -1751,9 +1751,9 @@ def test_repeated_execute_and_changing_lengths(binding, oracle, dev, stream):
 
 @pytest.mark.parametrize("heads,kv_heads", [(30, 2), (8, 2), (8, 4), (32, 8), (16, 1)])
 def test_rows_spanning_wave_ranges_merge_consistently(binding, oracle, dev, stream, heads, kv_heads):
-    """Rows cut across several wave ranges are merged inside the kernel by the wave
-    that finishes last; the partial rows travel between CUs of different XCDs.
-    Repeated launches on reused workspace addresses must all give the oracle's rows."""
+    """Rows cut across several wave ranges leave partial rows in the workspace, written by CUs of
+    different XCDs and read back by the merge kernel that follows on the stream. Repeated launches
+    on reused workspace addresses must all give the oracle's rows."""
     rng = _rng(97)
     q, kc, vc, tables, ctx = _pa_inputs(rng, dev, 18, heads, kv_heads, 128, 128, 128, 88, torch.float16)
     scale = 1.0 / math.sqrt(128)

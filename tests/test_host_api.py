@@ -1031,6 +1031,15 @@ def test_acl_tensor_handle_and_two_call_wrappers(binding, ctx):
     lens[2] = 3 * 128 + 1                              # longer than its block table: Setup refuses
     assert mla(0) == E["ERROR_INVALID_PARAM"]
     assert lib.AtbMLA(None, 0, None, ctx.ptr) == E["ERROR_INVALID_OPERATION_ADDR"]
+    # a handle with more than 8 dims does not convert: the wrapper returns that status, not Setup's
+    # (reference atb_acl_mla.cpp:69-96 checks every conversion)
+    lens[2] = 300
+    wide = mk("float16", [1] * 9, FAKE_DEVICE)
+    good = handles["out"]
+    handles["out"] = wide
+    assert mla(0) == E["ERROR_INVALID_TENSOR_DIM"]
+    handles["out"] = good
+    lib.aclDestroyTensor(wide)
     for o in (op, ring):
         lib.atb_c_destroy_operation(o)
 
