@@ -21,6 +21,9 @@ constexpr int WAVE = 64;
 // Records the message atbmi_last_error() hands back and returns `code`.
 int Fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 
+// Compute units of the current device (256 when no device can be asked: plans are also made on hosts without a GPU).
+int DeviceComputeUnits();
+
 #define ATBMI_HIP_CHECK(expr)                                                                       \
     do {                                                                                            \
         hipError_t e_ = (expr);                                                                     \
@@ -146,16 +149,26 @@ struct PaStreamPlan {
     uint16_t inlineFirst[PA_INLINE_RANGES];
 };
 
-// First step of wave range `wr`: ranges differ by at most one step.
+// First step of wave range `wr`: ranges differ by at most one step. (The products fit 32 bits for all but
+// enormous plans, and a 32-bit division is a fraction of the instructions of a 64-bit one on the GPU; both
+// forms give the same quotient.)
 __host__ __device__ __forceinline__ int32_t PaRangeBegin(int32_t wr, int32_t totalSteps, int32_t numWaveRanges)
 {
-    return static_cast<int32_t>(static_cast<int64_t>(wr) * totalSteps / numWaveRanges);
+    const int64_t product = static_cast<int64_t>(wr) * totalSteps;
+    if (product < 0x7fffffffLL) {
+        return static_cast<int32_t>(static_cast<uint32_t>(product) / static_cast<uint32_t>(numWaveRanges));
+    }
+    return static_cast<int32_t>(product / numWaveRanges);
 }
 
 // The wave range that holds step `s`.
 __host__ __device__ __forceinline__ int32_t PaRangeOf(int32_t s, int32_t totalSteps, int32_t numWaveRanges)
 {
-    return static_cast<int32_t>(((static_cast<int64_t>(s) + 1) * numWaveRanges - 1) / totalSteps);
+    const int64_t product = (static_cast<int64_t>(s) + 1) * numWaveRanges - 1;
+    if (product < 0x7fffffffLL) {
+        return static_cast<int32_t>(static_cast<uint32_t>(product) / static_cast<uint32_t>(totalSteps));
+    }
+    return static_cast<int32_t>(product / totalSteps);
 }
 
 __device__ __forceinline__ float Bf16ToFloat(uint16_t v)

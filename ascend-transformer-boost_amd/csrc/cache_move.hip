@@ -90,7 +90,7 @@ __global__ __launch_bounds__(MOVE_THREADS) void BlockCopyKernel(uint8_t *__restr
 // Token t of sequence b sits in block tables[b][seqStarts[b] / blockSize + t / blockSize] at offset
 // t % blockSize and goes to output row (tokens of the sequences before b) + t. A negative block id
 // leaves the output row as it is.
-constexpr int LOAD_TOKENS = 16;
+constexpr int LOAD_TOKENS = 32;
 
 template <typename VecT>
 __global__ __launch_bounds__(MOVE_THREADS) void PagedCacheLoadKernel(
@@ -100,80 +100,119 @@ __global__ __launch_bounds__(MOVE_THREADS) void PagedCacheLoadKernel(
     int64_t numBlocks, int64_t kRowBytes, int64_t vRowBytes, int64_t outRows, int32_t cumsumMode)
 {
     const int b = blockIdx.y;
-    int64_t begin; // first output row of this sequence
+    const int t0 = blockIdx.x * LOAD_TOKENS;
+    // Everything the workgroup has to look up is requested at once: the lengths before this sequence
+    // (their sum is its first output row), its own length and the block ids of this group's tokens; one
+    // memory round trip instead of three in a row, which is most of what a group of this size costs.
+    __shared__ int64_t total;
+    __shared__ int64_t srcRow[LOAD_TOKENS]; // cache row of each of the group's tokens (-1: leave the output row alone)
+    const int firstBlock = seqStarts ? seqStarts[b] / blockSize : 0;
+    int64_t before = 0; // this lane's share of the lengths before sequence b
     int32_t len;
     if (cumsumMode) {
-        begin = lens[b];
-        len = lens[b + 1] - lens[b];
+        before = lens[b];
+        len = lens[b + 1] - static_cast<int32_t>(before);
     } else {
-        // the sequences before this one: summed by the first wave, 64 at a time
-        __shared__ int64_t total;
         if (threadIdx.x < WAVE) {
-            int64_t s = 0;
             for (int i = threadIdx.x; i < b; i += WAVE) {
-                s += lens[i];
-            }
-            for (int off = 32; off > 0; off >>= 1) {
-                s += __shfl_xor(s, off, WAVE);
-            }
-            if (threadIdx.x == 0) {
-                total = s;
+                before += lens[i];
             }
         }
-        __syncthreads();
-        begin = total;
         len = lens[b];
     }
-    const int t0 = blockIdx.x * LOAD_TOKENS;
+    int64_t blk = -1;
+    if (threadIdx.x < LOAD_TOKENS) {
+        const int tableIdx = firstBlock + (t0 + static_cast<int>(threadIdx.x)) / blockSize;
+        if (tableIdx < maxBlocksPerSeq) {
+            blk = tables[static_cast<int64_t>(b) * maxBlocksPerSeq + tableIdx];
+        }
+    }
     if (t0 >= len) {
         return;
     }
-    const int firstBlock = seqStarts ? seqStarts[b] / blockSize : 0;
-    const bool isValue = blockIdx.z == 1;
-    const int64_t rowBytes = isValue ? vRowBytes : kRowBytes;
-    const uint8_t *cache = isValue ? valueCache : keyCache;
-    uint8_t *out = isValue ? value : key;
+    if (!cumsumMode && threadIdx.x < WAVE) {
+        for (int off = 32; off > 0; off >>= 1) {
+            before += __shfl_xor(before, off, WAVE);
+        }
+    }
+    const int64_t begin = cumsumMode ? before : __shfl(before, 0, WAVE); // (valid in the first wave; the others read `total`)
+    if (threadIdx.x == 0) {
+        total = begin;
+    }
     const int tokens = min(LOAD_TOKENS, len - t0);
-    // cache row of each of the group's tokens (-1: leave the output row alone)
-    __shared__ int64_t srcRow[LOAD_TOKENS];
     if (threadIdx.x < LOAD_TOKENS) {
         const int t = t0 + threadIdx.x;
         int64_t r = -1;
-        const int tableIdx = firstBlock + t / blockSize;
-        if (static_cast<int>(threadIdx.x) < tokens && tableIdx < maxBlocksPerSeq && begin + t < outRows) {
-            const int64_t blk = tables[static_cast<int64_t>(b) * maxBlocksPerSeq + tableIdx];
-            if (blk >= 0 && blk < numBlocks) {
-                r = blk * blockSize + t % blockSize;
-            }
+        if (static_cast<int>(threadIdx.x) < tokens && blk >= 0 && blk < numBlocks && begin + t < outRows) {
+            r = blk * blockSize + t % blockSize;
         }
         srcRow[threadIdx.x] = r;
     }
     __syncthreads();
+    const int64_t firstRow = total;
+    const bool isValue = blockIdx.z == 1;
+    const int64_t rowBytes = isValue ? vRowBytes : kRowBytes;
+    const uint8_t *cache = isValue ? valueCache : keyCache;
+    uint8_t *out = isValue ? value : key;
     const int perRow = static_cast<int>(rowBytes / static_cast<int64_t>(sizeof(VecT)));
-    const int n = perRow * tokens;
     const VecT *from = reinterpret_cast<const VecT *>(cache);
-    VecT *to = reinterpret_cast<VecT *>(out + (begin + t0) * rowBytes);
+    VecT *to = reinterpret_cast<VecT *>(out + (firstRow + t0) * rowBytes);
+    // A thread keeps its column and walks down the rows: the division that finds (row, column) is done once,
+    // not per vector moved. Short rows: several rows per pass of the workgroup; long rows: several passes a row.
     constexpr int BATCH = 4;
-    for (int i0 = threadIdx.x; i0 < n; i0 += MOVE_THREADS * BATCH) {
-        VecT v[BATCH];
-        bool live[BATCH];
+    if (perRow <= MOVE_THREADS) {
+        const int rowsPerPass = MOVE_THREADS / perRow;
+        const int col = threadIdx.x % perRow;
+        const int row0 = threadIdx.x / perRow;
+        if (row0 >= rowsPerPass) {
+            return; // (threads past the last whole row of a pass)
+        }
+        for (int tok0 = row0; tok0 < tokens; tok0 += rowsPerPass * BATCH) {
+            VecT v[BATCH];
+            bool live[BATCH];
 #pragma unroll
-        for (int k = 0; k < BATCH; ++k) { // all loads first
-            const int i = i0 + k * MOVE_THREADS;
-            live[k] = false;
-            if (i < n) {
-                const int tok = i / perRow;
-                const int64_t r = srcRow[tok];
-                if (r >= 0) {
-                    live[k] = true;
-                    v[k] = from[r * perRow + (i - tok * perRow)];
+            for (int k = 0; k < BATCH; ++k) { // all loads first
+                const int tok = tok0 + k * rowsPerPass;
+                live[k] = false;
+                if (tok < tokens) {
+                    const int64_t r = srcRow[tok];
+                    if (r >= 0) {
+                        live[k] = true;
+                        v[k] = from[r * perRow + col];
+                    }
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < BATCH; ++k) {
+                if (live[k]) {
+                    StoreOnce(to + static_cast<int64_t>(tok0 + k * rowsPerPass) * perRow + col, v[k]);
                 }
             }
         }
+        return;
+    }
+    for (int tok = 0; tok < tokens; ++tok) {
+        const int64_t r = srcRow[tok];
+        if (r < 0) {
+            continue;
+        }
+        const VecT *src = from + r * perRow;
+        VecT *dst = to + static_cast<int64_t>(tok) * perRow;
+        for (int c0 = threadIdx.x; c0 < perRow; c0 += MOVE_THREADS * BATCH) {
+            VecT v[BATCH];
 #pragma unroll
-        for (int k = 0; k < BATCH; ++k) {
-            if (live[k]) {
-                StoreOnce(to + i0 + k * MOVE_THREADS, v[k]);
+            for (int k = 0; k < BATCH; ++k) {
+                const int c = c0 + k * MOVE_THREADS;
+                if (c < perRow) {
+                    v[k] = src[c];
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < BATCH; ++k) {
+                const int c = c0 + k * MOVE_THREADS;
+                if (c < perRow) {
+                    StoreOnce(dst + c, v[k]);
+                }
             }
         }
     }

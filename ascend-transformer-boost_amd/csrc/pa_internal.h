@@ -47,8 +47,6 @@ int LaunchPaMfmaInt8(const AtbmiPaShape &shape, const PaArgs &args, const PaStre
 
 // Raises a kernel's dynamic LDS limit to `ldsBytes` on the current device, once per kernel and device.
 int ConfigureKernelLds(const void *kernel, int ldsBytes);
-// Compute units of the current device (256 when no device can be asked: plans are also made on hosts without a GPU).
-int DeviceComputeUnits();
 
 // Merges the partials of every sequence that has more than one (scalar-kernel plan).
 int LaunchPaReduce(const AtbmiPaShape &shape, const PaArgs &args, int numSeqs, hipStream_t stream);
