@@ -104,6 +104,9 @@ struct PaArgs {
     int32_t descaleHeads; // > 0: sequence b takes slice b % descaleHeads of the descale vectors instead of its KV head's
     const float *razor;   // [slots] added to q.k before the score scale (null: none)
     void *lse;           // [rows][H] in the query's type: natural-log log-sum-exp of the scaled scores (null: none)
+    int32_t nzShift;     // > 0: fractal-NZ caches of the split latent layout, log2 of the block size; channel c of
+                         // the token at offset t of block b sits at ((b * (dn / 16) + c / 16) << nzShift) * 16 + t * 16 +
+                         // c % 16 (dn channels per row of that cache)
     int32_t partHalf;    // 1: partO holds 16-bit values (the 128-head MLA kernel: its partial rows are a third of
                          // what a segment moves, and a normalised row loses nothing the final rounding would keep)
 };

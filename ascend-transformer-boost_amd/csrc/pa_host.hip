@@ -246,8 +246,14 @@ extern "C" int atbmi_pa_plan_create(const AtbmiPaShape *shape, AtbmiPaPlan **pla
     if (s.descaleHeads > 0 && s.kvDtype != ATBMI_INT8) {
         return Fail(ERR_INVALID_PARAM, "pa_plan_create: descaleHeads only applies to an int8 cache");
     }
-    if (s.kvLayout != ATBMI_PA_KV_TOKEN_MAJOR && s.kvLayout != ATBMI_PA_KV_HEAD_MAJOR) {
+    if (s.kvLayout != ATBMI_PA_KV_TOKEN_MAJOR && s.kvLayout != ATBMI_PA_KV_HEAD_MAJOR &&
+        s.kvLayout != ATBMI_PA_KV_FRACTAL_NZ) {
         return Fail(ERR_INVALID_PARAM, "pa_plan_create: kvLayout %d", s.kvLayout);
+    }
+    if (s.kvLayout == ATBMI_PA_KV_FRACTAL_NZ &&
+        !(s.ropeDim == 64 && s.numKvHeads == 1 && s.blockSize >= 16 && (s.blockSize & (s.blockSize - 1)) == 0)) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_create: fractal-NZ caches come with the split latent layout (ropeDim 64, "
+                                       "one KV head) and a power-of-two block size of at least 16");
     }
     if (s.kvLayout == ATBMI_PA_KV_HEAD_MAJOR) {
         if (s.mlaCombined) {
@@ -810,6 +816,7 @@ int DecodeImpl(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void *workspace, uint
     a.ropeDim = s.ropeDim;
     a.ropeRowStride = static_cast<int64_t>(s.numKvHeads) * s.ropeDim;
     a.lse = t->lse;
+    a.nzShift = s.kvLayout == ATBMI_PA_KV_FRACTAL_NZ ? __builtin_ctz(static_cast<unsigned>(s.blockSize)) : 0;
     a.partHalf = (plan->useMfma && PaMlaWide(s)) ? 1 : 0;
 
     TimingRecord rec{nullptr, nullptr, nullptr};

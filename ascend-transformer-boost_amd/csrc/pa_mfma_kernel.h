@@ -236,6 +236,16 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
     const int nopePieces = dn / 8;           // 16-byte pieces of a key row that the key cache holds
     // Address of piece `col` of the key row at cache slot r.
     auto keyPiece = [&](int64_t r, int col) -> const unsigned char * {
+        if (MLA && a.nzShift > 0) {
+            // fractal-NZ: slabs of blockSize x 16 channels; a 16-byte piece is half a slab row
+            const int64_t blk = r >> a.nzShift;
+            const int64_t off = r & ((1 << a.nzShift) - 1);
+            if (col >= nopePieces) {
+                const int c = col - nopePieces;
+                return krBase + ((((blk * (a.ropeDim >> 4) + (c >> 1)) << a.nzShift) + off) * 16 + (c & 1) * 8) * 2;
+            }
+            return kcBase + ((((blk * (dn >> 4) + (col >> 1)) << a.nzShift) + off) * 16 + (col & 1) * 8) * 2;
+        }
         if (MLA && col >= nopePieces) {
             return krBase + (r * a.ropeRowStride + static_cast<int64_t>(g) * a.ropeDim) * 2 + (col - nopePieces) * 16;
         }

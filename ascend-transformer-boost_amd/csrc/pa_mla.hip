@@ -8,6 +8,10 @@ int LaunchPaMlaWide(const AtbmiPaShape &s, const PaArgs &args, const PaStreamPla
     if (!PaMlaWide(s)) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: shape does not fit the 128-head MLA kernel");
     }
+    if (s.kvLayout == ATBMI_PA_KV_FRACTAL_NZ) {
+        return s.qDtype == ATBMI_BF16 ? mla::LaunchAsm<true, true, true>(args, plan, stream)
+                                      : mla::LaunchAsm<false, true, true>(args, plan, stream);
+    }
     if (s.ropeDim != 0) {
         return s.qDtype == ATBMI_BF16 ? mla::LaunchAsm<true, true>(args, plan, stream)
                                       : mla::LaunchAsm<false, true>(args, plan, stream);

@@ -87,7 +87,7 @@ struct Segment {
 
 // One segment from start to finish: stages the first tiles, loads Q, runs the pipelined step loop, writes
 // the (partial) row. All four waves of a workgroup call it with the same token range and block table.
-template <bool BF16, bool SPLIT>
+template <bool BF16, bool SPLIT, bool NZ>
 __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, uint32_t wave, float scale2)
 {
     // Every input is wave-uniform; saying so value by value keeps each of them in scalar registers, which
@@ -126,6 +126,7 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     // s59 token of the tile to fetch   s[60:61] saved exec   s62 rows of this wave inside the segment
     .set BF16, %[bf16]
     .set SPLIT, %[split]
+    .set NZ, %[nz]
     // SPLIT: the last 64 channels of every cache row come from a cache of their own (rows of 128 bytes) and
     // those of every query row from a tensor of their own. A transfer then takes its lanes from two sources:
     // lanes whose slot (64 i + lane, 73 slots a row, the last one padding) holds one of the first 64 pieces
@@ -344,6 +345,31 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
       v_readlane_b32 s49, v98, s48         // block id
       s_and_b32 s50, s46, s45              // row inside the block
       s_nop 3
+      .if NZ
+        // fractal-NZ blocks: slabs of (block size) x 16 channels, 32 channel slabs in the latent cache and
+        // 4 in the rope cache; a token's 32 bytes of a slab follow those of the token before
+        s_lshl_b32 s50, s50, 5
+        s_add_u32 s52, %[bshift], 10
+        s_mov_b32 s56, s49
+        s_mov_b32 s57, 0
+        s_lshl_b64 s[56:57], s[56:57], s52 // block id x block size x 1024 bytes
+        s_add_u32 s56, s56, s50
+        s_addc_u32 s57, s57, 0
+        s_add_u32 s56, s56, %[cache_lo]
+        s_addc_u32 s57, s57, %[cache_hi]
+        s_sub_u32 s56, s56, 4096
+        s_subb_u32 s57, s57, 0
+        s_add_u32 s52, %[bshift], 7
+        s_mov_b32 s64, s49
+        s_mov_b32 s65, 0
+        s_lshl_b64 s[64:65], s[64:65], s52 // block id x block size x 128 bytes
+        s_add_u32 s64, s64, s50
+        s_addc_u32 s65, s65, 0
+        s_add_u32 s64, s64, %[rope_lo]
+        s_addc_u32 s65, s65, %[rope_hi]
+        s_sub_u32 s64, s64, 4096
+        s_subb_u32 s65, s65, 0
+      .else
       s_lshl_b32 s49, s49, %[bshift]
       s_add_u32 s49, s49, s50              // cache row
       s_mul_i32 s56, s49, %[rowbytes]
@@ -359,6 +385,7 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
         s_addc_u32 s65, s65, %[rope_hi]
         s_sub_u32 s64, s64, 4096
         s_subb_u32 s65, s65, 0
+      .endif
       .endif
     .endm
     // the instruction of transfer i from the source base in s[base : base+1]; M0 = region + 4096 for i < 8,
@@ -573,9 +600,25 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
       v_mul_u32_u24 v93, 73, v92
       v_sub_u32 v93, v91, v93
       v_min_u32 v93, 71, v93
+      .if NZ
+        // piece p of tile row r: r x 32 + (p / 2) x 32 x block size + (p mod 2) x 16 past the token of the
+        // tile's first row; pieces 64 .. 71 the same with p - 64, in the rope cache
+        v_cmp_lt_u32 vcc, 63, v93
+        v_add_u32 v95, -64, v93
+        s_nop 1
+        v_cndmask_b32 v94, v93, v95, vcc
+        v_lshrrev_b32 v95, 1, v94
+        v_and_b32 v94, 1, v94
+        v_lshlrev_b32 v94, 4, v94
+        s_add_u32 s46, %[bshift], 5
+        v_lshlrev_b32 v95, s46, v95
+        v_lshl_add_u32 v91, v92, 5, v94
+        v_add_u32 v91, v91, v95
+      .else
       v_mul_lo_u32 v91, v92, %[rowbytes]
       v_lshl_add_u32 v91, v93, 4, v91
-      .if SPLIT
+      .endif
+      .if SPLIT && !NZ
         // pieces 64 .. 71 of a row: piece - 64 of the same row of the rope cache
         v_mul_lo_u32 v94, v92, %[roperowbytes]
         v_add_u32 v95, -64, v93
@@ -772,7 +815,7 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     .purgem BODY
     )ASM"
                  :
-                 : [bf16] "n"(BF16 ? 1 : 0), [split] "n"(SPLIT ? 1 : 0), [qrope] "s"(qRope), [rope_lo] "s"(ropeLo),
+                 : [bf16] "n"(BF16 ? 1 : 0), [split] "n"(SPLIT ? 1 : 0), [nz] "n"(NZ ? 1 : 0), [qrope] "s"(qRope), [rope_lo] "s"(ropeLo),
                    [rope_hi] "s"(ropeHi), [roperowbytes] "s"(ropeRowBytes), [scale] "s"(scale2), [bshift] "s"(blockShift), [table] "s"(table),
                    [rowbytes] "s"(rowBytes), [cache_lo] "s"(cacheLo), [cache_hi] "s"(cacheHi), [q] "s"(q), [out] "s"(out),
                    [lse] "s"(lse), [tokbegin] "s"(tokBegin), [tokend] "s"(tokEnd), [lds] "s"(ldsBase), [wave] "s"(wave),
@@ -783,7 +826,7 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
 
 // Grid and plan as the 128-head kernel of pa_mla_kernel.h: one wave range per workgroup, the head groups of
 // one range 8 workgroup ids apart.
-template <bool BF16, bool SPLIT>
+template <bool BF16, bool SPLIT, bool NZ>
 __global__ __launch_bounds__(NW *WAVE) void PaMlaAsmKernel(const PaArgs a, const PaStreamPlan p)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -846,20 +889,21 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaAsmKernel(const PaArgs a, const
             sg.out = reinterpret_cast<uint16_t *>(a.partO) + ph * DV;
             sg.lse = a.partLse + ph;
         }
-        RunSegment<BF16, SPLIT>(sg, ldsBase, wave, scale2);
+        RunSegment<BF16, SPLIT, NZ>(sg, ldsBase, wave, scale2);
     }
 }
 
-template <bool BF16, bool SPLIT> int LaunchAsm(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
+template <bool BF16, bool SPLIT, bool NZ = false> int LaunchAsm(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
 {
-    auto kernel = PaMlaAsmKernel<BF16, SPLIT>;
+    static_assert(SPLIT || !NZ, "fractal-NZ caches come with the split layout");
+    auto kernel = PaMlaAsmKernel<BF16, SPLIT, NZ>;
     const int configured = ConfigureKernelLds(reinterpret_cast<const void *>(kernel), LDS_BYTES);
     if (configured != OK) {
         return configured;
     }
     if (plan.tokenSlices != 1 || plan.numWaveRanges != plan.numWgRanges ||
         plan.headGroups * PA_MLA_HEADS_PER_WG != args.H || args.G != 1 || args.D != D || args.Dv != DV ||
-        args.ropeDim != (SPLIT ? D - DV : 0) || args.blockSize < 16 || (args.blockSize & (args.blockSize - 1)) != 0 ||
+        args.ropeDim != (SPLIT ? D - DV : 0) || (args.nzShift > 0) != NZ || args.blockSize < 16 || (args.blockSize & (args.blockSize - 1)) != 0 ||
         args.kRowStride * 2 > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: plan or shape does not fit the 128-head MLA kernel");
     }

@@ -99,10 +99,21 @@ __global__ __launch_bounds__(PA_SCALAR_WAVES * WAVE) void PaScalarKernel(const P
 
     const int32_t *table = a.tables + static_cast<int64_t>(it.seq) * a.maxBlocksPerSeq;
     for (int t = it.tokBegin + wave; t < it.tokEnd; t += PA_SCALAR_WAVES) {
-        const int64_t row = static_cast<int64_t>(table[t / a.blockSize]) * a.blockRows + (t % a.blockSize);
-        const int64_t kBase = row * a.kRowStride + static_cast<int64_t>(g) * a.kHeadStride;
-        const int64_t rBase = row * a.ropeRowStride + static_cast<int64_t>(g) * a.ropeDim - dn;
-        const int64_t vBase = row * a.vRowStride + static_cast<int64_t>(g) * a.vHeadStride;
+        const int64_t blk = table[t / a.blockSize];
+        const int off = t % a.blockSize;
+        const int64_t row = blk * a.blockRows + off;
+        int64_t kBase = row * a.kRowStride + static_cast<int64_t>(g) * a.kHeadStride;
+        int64_t rBase = row * a.ropeRowStride + static_cast<int64_t>(g) * a.ropeDim - dn;
+        int64_t vBase = row * a.vRowStride + static_cast<int64_t>(g) * a.vHeadStride;
+        // Fractal-NZ caches: a block is (channels / 16) slabs of blockSize x 16; element d then sits
+        // ((d / 16) << nzShift) * 16 + d % 16 past the token's place in the first slab.
+        const bool nz = a.nzShift > 0;
+        if (nz) {
+            kBase = blk * a.blockSize * dn + off * 16;
+            vBase = kBase;
+            rBase = blk * a.blockSize * a.ropeDim + off * 16;
+        }
+        auto nzOff = [&](int d) { return (static_cast<int64_t>(d >> 4) << a.nzShift) * 16 + (d & 15); };
         const float razor = a.razor ? a.razor[row] : 0.0f;
         float k[EPL], v[EPL];
 #pragma unroll
@@ -119,10 +130,14 @@ __global__ __launch_bounds__(PA_SCALAR_WAVES * WAVE) void PaScalarKernel(const P
                 }
             } else {
                 if (d < a.D) {
-                    k[e] = d < dn ? Load16(a.kc, kBase + d, bf16) : Load16(a.kRope, rBase + d, bf16);
+                    if (nz) {
+                        k[e] = d < dn ? Load16(a.kc, kBase + nzOff(d), bf16) : Load16(a.kRope, rBase + nzOff(d - dn), bf16);
+                    } else {
+                        k[e] = d < dn ? Load16(a.kc, kBase + d, bf16) : Load16(a.kRope, rBase + d, bf16);
+                    }
                 }
                 if (d < a.Dv) {
-                    v[e] = Load16(a.vc, vBase + d, bf16);
+                    v[e] = Load16(a.vc, nz ? vBase + nzOff(d) : vBase + d, bf16);
                 }
             }
         }

@@ -9,9 +9,11 @@
 // read from hostData during Setup, as the reference runner does
 // (src/ops/ops_infer/multi_latent_attention/param.cpp).
 //
-// Implemented: cacheMode KROPE_CTKV with fp16/bf16 tensors; calcType UNDEFINED,
+// Implemented: cacheMode KROPE_CTKV and NZCACHE (the same 16-bit caches in the
+// fractal-NZ layout, [blocks, 512 / 16, 128, 16] and [blocks, 64 / 16, 128, 16];
+// reference :394-425 QKVDimCheckNz) with fp16/bf16 tensors; calcType UNDEFINED,
 // SPEC (qSeqlen, optionally with the MASK_TYPE_SPEC mask), RING and
-// SPEC_AND_RING (second output: log-sum-exp). The fractal-NZ cache modes, the
+// SPEC_AND_RING (second output: log-sum-exp). The int8 NZ cache mode, the
 // prefill calcType, the MASK_FREE / CAUSAL_MASK / SWA_NORM masks and
 // maskUseStatus are legal in the reference but not implemented here; such
 // params are rejected at creation with ERROR_INVALID_PARAM.
@@ -34,6 +36,7 @@ constexpr int64_t LATENT_DIM = 512;
 constexpr int64_t ROPE_DIM = 64;
 constexpr int64_t DECODER_BLOCK_SIZE = 128;
 constexpr int64_t MAX_BATCH = 8192;
+constexpr int64_t NZ_CHANNELS = 16; // channels of one fractal-NZ slab row (16-bit elements)
 
 bool IsSpec(const Param &p)
 {
@@ -148,8 +151,8 @@ bool ImplementedCheck(const Param &p)
     const char *what = nullptr;
     if (p.calcType == Param::CALC_TYPE_PREFILL) {
         what = "the prefill calcType";
-    } else if (p.cacheMode != Param::KROPE_CTKV) {
-        what = "fractal-NZ caches";
+    } else if (p.cacheMode == Param::INT8_NZCACHE) {
+        what = "the int8 fractal-NZ cache";
     } else if (p.maskType != Param::UNDEFINED && p.maskType != Param::MASK_TYPE_SPEC) {
         what = "this maskType";
     } else if (p.maskUseStatusType != Param::MASK_USE_STATUS_TYPE_UNDEFINED) {
@@ -164,10 +167,19 @@ bool ImplementedCheck(const Param &p)
 
 // The dtype table of the implemented sections of the reference
 // ops_configs/atb_ops_info.ini (:6669-6690 base, :6691-6715 Mask, :6716-6740 IsRing,
-// :6772-6824 Qlens / QlensIsRing, :6859-6917 MaskQlens / MaskQlensIsRing).
+// :6772-6824 Qlens / QlensIsRing, :6859-6917 MaskQlens / MaskQlensIsRing, :6946-6967 Nz).
+// The reference builds the section name from the param (:208-240); NZCACHE together with a mask,
+// qSeqlen or the log-sum-exp output names a section that does not exist, and an operation without
+// a table skips the check (reference operation_base.cpp:229-233): HasIr() says which.
+bool HasIr(const Param &p)
+{
+    return p.cacheMode != Param::NZCACHE || (!HasMaskInput(p) && !IsSpec(p) && !IsRing(p));
+}
+
 OpIr MakeIr(const Param &p)
 {
     OpIr ir;
+    const aclFormat cacheFormat = p.cacheMode == Param::NZCACHE ? ACL_FORMAT_FRACTAL_NZ : ACL_FORMAT_ND;
     for (aclDataType q : {ACL_FLOAT16, ACL_BF16}) {
         IrCombo c;
         c.inDtypes = {q, q, q, q, ACL_INT32, ACL_INT32};
@@ -178,6 +190,8 @@ OpIr MakeIr(const Param &p)
             c.inDtypes.push_back(ACL_INT32);
         }
         c.inFormats.assign(c.inDtypes.size(), ACL_FORMAT_ND);
+        c.inFormats[KV_CACHE] = cacheFormat;
+        c.inFormats[KV_CACHE_ROPE] = cacheFormat;
         c.outDtypes = {q};
         if (IsRing(p)) {
             c.outDtypes.push_back(q);
@@ -193,7 +207,7 @@ public:
     explicit MultiLatentAttentionOperation(const Param &param)
         : OperationBase("MultiLatentAttentionOperation"), param_(param), irTable_(MakeIr(param))
     {
-        ir_ = &irTable_;
+        ir_ = HasIr(param) ? &irTable_ : nullptr;
         size_t next = CONTEXT_LENS + 1;
         if (HasMaskInput(param)) {
             maskIdx_ = next++;
@@ -299,7 +313,9 @@ protected:
         shape.numKvHeads = 1;
         shape.headDimK = static_cast<int32_t>(LATENT_DIM + ROPE_DIM);
         shape.headDimV = static_cast<int32_t>(LATENT_DIM);
-        shape.blockSize = static_cast<int32_t>(kv.desc.shape.dims[1]);
+        const bool nz = param_.cacheMode == Param::NZCACHE;
+        shape.blockSize = static_cast<int32_t>(kv.desc.shape.dims[nz ? 2 : 1]);
+        shape.kvLayout = nz ? ATBMI_PA_KV_FRACTAL_NZ : ATBMI_PA_KV_TOKEN_MAJOR;
         shape.numBlocks = static_cast<int32_t>(kv.desc.shape.dims[0]);
         shape.maxBlocksPerSeq = static_cast<int32_t>(tables.desc.shape.dims[1]);
         shape.numQueryRows = static_cast<int32_t>(q.desc.shape.dims[0]);
@@ -363,7 +379,7 @@ private:
         return a.qDtype == b.qDtype && a.numHeads == b.numHeads && a.blockSize == b.blockSize &&
                a.numBlocks == b.numBlocks && a.maxBlocksPerSeq == b.maxBlocksPerSeq &&
                a.numQueryRows == b.numQueryRows && a.qkScale == b.qkScale && a.hasMask == b.hasMask &&
-               a.maskBatchStride == b.maskBatchStride && a.maskLen == b.maskLen;
+               a.maskBatchStride == b.maskBatchStride && a.maskLen == b.maskLen && a.kvLayout == b.kvLayout;
     }
 
     // Reference :558-620 (DimCheck) with :350-392 (QKVDimCheck) and :478-490 (DimCheckSpec).
@@ -391,19 +407,28 @@ private:
         }
         const Dims &kv = in.at(KV_CACHE).shape;
         const Dims &kr = in.at(KV_CACHE_ROPE).shape;
-        if (kv.dims[1] != DECODER_BLOCK_SIZE) {
-            ATB_LOG(ERROR) << "decoder blockSize should be " << DECODER_BLOCK_SIZE << ", got " << kv.dims[1];
+        // token-major caches [blocks, blockSize, kvHeads, channels] (reference :350-392) or fractal-NZ
+        // caches [blocks, channels / 16, blockSize, 16] (reference :394-425)
+        const bool nz = param_.cacheMode == Param::NZCACHE;
+        const int blockDim = nz ? 2 : 1;
+        if (kv.dims[blockDim] != DECODER_BLOCK_SIZE) {
+            ATB_LOG(ERROR) << "decoder blockSize should be " << DECODER_BLOCK_SIZE << ", got " << kv.dims[blockDim];
             return ERROR_INVALID_TENSOR_DIM;
         }
         if (in.at(QUERY_ROPE).shape.dims[0] != numTokens) {
             ATB_LOG(ERROR) << "dim 0 of query and queryRope should be the same";
             return ERROR_INVALID_TENSOR_DIM;
         }
-        if (kr.dims[0] != kv.dims[0] || kr.dims[1] != kv.dims[1]) {
-            ATB_LOG(ERROR) << "dim 0 and dim 1 of kvCache and kvCacheRope should be the same";
+        if (kr.dims[0] != kv.dims[0] || kr.dims[blockDim] != kv.dims[blockDim]) {
+            ATB_LOG(ERROR) << "block count and block size of kvCache and kvCacheRope should be the same";
             return ERROR_INVALID_TENSOR_DIM;
         }
-        if (kv.dims[2] != param_.kvHeadNum || kr.dims[2] != param_.kvHeadNum) {
+        if (nz) {
+            if (kv.dims[3] != NZ_CHANNELS || kr.dims[3] != NZ_CHANNELS) {
+                ATB_LOG(ERROR) << "dim 3 of kvCache and kvCacheRope should be " << NZ_CHANNELS;
+                return ERROR_INVALID_TENSOR_DIM;
+            }
+        } else if (kv.dims[2] != param_.kvHeadNum || kr.dims[2] != param_.kvHeadNum) {
             ATB_LOG(ERROR) << "dim 2 of kvCache and kvCacheRope should equal kvHeadNum";
             return ERROR_INVALID_TENSOR_DIM;
         }
@@ -411,11 +436,11 @@ private:
             ATB_LOG(ERROR) << "dim 1 of query and queryRope should equal headNum";
             return ERROR_INVALID_TENSOR_DIM;
         }
-        if (in.at(QUERY).shape.dims[2] != LATENT_DIM || kv.dims[3] != LATENT_DIM) {
+        if (in.at(QUERY).shape.dims[2] != LATENT_DIM || (nz ? kv.dims[1] * NZ_CHANNELS : kv.dims[3]) != LATENT_DIM) {
             ATB_LOG(ERROR) << "head size of query and kvCache should be 512";
             return ERROR_INVALID_TENSOR_DIM;
         }
-        if (in.at(QUERY_ROPE).shape.dims[2] != ROPE_DIM || kr.dims[3] != ROPE_DIM) {
+        if (in.at(QUERY_ROPE).shape.dims[2] != ROPE_DIM || (nz ? kr.dims[1] * NZ_CHANNELS : kr.dims[3]) != ROPE_DIM) {
             ATB_LOG(ERROR) << "head size of queryRope and kvCacheRope should be 64";
             return ERROR_INVALID_TENSOR_DIM;
         }

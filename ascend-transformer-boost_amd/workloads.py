@@ -42,8 +42,9 @@ CONFIGS["c2_bnsd"] = dict(CONFIGS["c2"], bnsd=True)
 # C5 as MultiLatentAttentionOperation sees it: the same rows, 512 latent + 64 rotary channels in two
 # tensors each for the query and the cache.
 CONFIGS["c5_split"] = dict(CONFIGS["c5"], split=True)
+CONFIGS["c5_nz"] = dict(CONFIGS["c5"], split=True, nz=True)
 
-SEEDS = {"c1": 1001, "c2": 1002, "c2_fp16": 1002, "c2_alibi": 1002, "c2_norm": 1002, "c2_mtp4": 1002, "c2_bnsd": 1002, "c3": 1003, "c4": 1004, "c5": 1005, "c5_split": 1005}
+SEEDS = {"c1": 1001, "c2": 1002, "c2_fp16": 1002, "c2_alibi": 1002, "c2_norm": 1002, "c2_mtp4": 1002, "c2_bnsd": 1002, "c3": 1003, "c4": 1004, "c5": 1005, "c5_split": 1005, "c5_nz": 1005}
 
 
 def config(name, **overrides):

@@ -78,6 +78,8 @@ DESCRIPTIONS = {
     "c4": "C4 skewed long-context fp16 decode: batch 16, 32 q heads, 8 kv heads, d128, ctx lognormal(median 8k) in [256,32768]",
     "c5_split": "C5 through MultiLatentAttentionOperation (cacheMode KROPE_CTKV: 512 latent + 64 rotary channels in "
                 "two caches): batch 64, 128 q heads, block 128, ctx U[2048,4096], bf16",
+    "c5_nz": "C5 through MultiLatentAttentionOperation with cacheMode NZCACHE (fractal-NZ caches [blocks, 32 | 4, 128, 16]), "
+             "attention only: batch 64, 128 q heads, block 128, ctx U[2048,4096], bf16",
     "c5": "C5 MLA bf16 decode: batch 64, 128 q heads, 1 latent kv head, d576/dv512, block 128, ctx U[2048,4096]",
 }
 
@@ -166,12 +168,13 @@ def run_workload(pkg, name, steps, warmup, attention_only=False, kernel_events=T
                                      quantType=1 if int8 else 0, mlaVHeadSize=cfg["dv"] if mla else 0,
                                      maskType=mask_type, calcType=1 if q_len > 1 else 0,
                                      inputLayout=1 if cfg.get("bnsd") else 0)
-    if cfg.get("bnsd"):
+    nz = bool(cfg.get("nz"))
+    if cfg.get("bnsd") or nz:
         attention_only = True
     split = bool(cfg.get("split"))
     if split:
         pa = b.OperationRunner("MultiLatentAttentionOperation", b.MultiLatentAttentionParam(
-            headNum=cfg["heads"], kvHeadNum=1, qkScale=scale, cacheMode=1), ctx)
+            headNum=cfg["heads"], kvHeadNum=1, qkScale=scale, cacheMode=3 if nz else 1), ctx)
     else:
         pa = b.OperationRunner("PagedAttentionOperation", pa_param, ctx)
     rac = None
@@ -191,6 +194,12 @@ def run_workload(pkg, name, steps, warmup, attention_only=False, kernel_events=T
             rac_in = [step["k_new"][..., :dv].contiguous(), step["k_new"][..., dv:].contiguous(), nope, rope,
                       step["slot_mapping"]]
             rac_out = [nope, rope]  # (the combined copy stays for the CPU baseline, which concatenates anyway)
+            if nz:
+                # [blocks, block, 1, channels] -> [blocks, channels / 16, block, 16], described in the fractal-NZ format
+                nz_caches = [t[:, :, 0, :].reshape(t.shape[0], t.shape[1], -1, 16).permute(0, 2, 1, 3).contiguous()
+                             for t in (nope, rope)]
+                pa_in[2:4] = [b.make_tensor(b._torch_acl_dtype(t), list(t.shape), device_ptr=t.data_ptr(),
+                                            fmt="fractal_nz") for t in nz_caches]
         elif mla:
             pa_in = [step["q"], step["key_cache"], step["block_tables"], lens_dev]
             host_idx = 3

@@ -230,10 +230,16 @@ typedef enum AtbmiPaMaskRow {
 /* Order of the dimensions inside one cache block (reference include/atb/infer_op_params.h, InputLayout):
  *   TOKEN_MAJOR  [numBlocks, blockSize, G, D]  TYPE_BSND
  *   HEAD_MAJOR   [numBlocks, G, blockSize, D]  TYPE_BNSD (PagedAttentionParam::inputLayout; 16-bit
- *                caches with separate key and value caches only) */
+ *                caches with separate key and value caches only)
+ *   FRACTAL_NZ   [numBlocks, D / 16, blockSize, 16]: channel c of the token at offset t of a block sits at
+ *                (c / 16) * blockSize * 16 + t * 16 + c % 16 of the block (MultiLatentAttentionParam::NZCACHE,
+ *                reference include/atb/infer_op_params.h:2949-2955; only the split latent layout, ropeDim 64,
+ *                16-bit, with a power-of-two block size: keyCache [numBlocks, 32, blockSize, 16] and
+ *                keyRopeCache [numBlocks, 4, blockSize, 16]) */
 typedef enum AtbmiPaKvLayout {
     ATBMI_PA_KV_TOKEN_MAJOR = 0,
-    ATBMI_PA_KV_HEAD_MAJOR = 1
+    ATBMI_PA_KV_HEAD_MAJOR = 1,
+    ATBMI_PA_KV_FRACTAL_NZ = 2
 } AtbmiPaKvLayout;
 
 typedef struct AtbmiPaShape {

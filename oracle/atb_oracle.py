@@ -55,6 +55,12 @@ the invariants of the mathematics (no function is left "parity unpinned"):
                       :386-388 (query and cache split [512, 64] along the channels);
                       MLA: tests/apitest/opstest/python/operations/paged_attention/
                       test_paged_attention_operation_mla.py:229-262 (V = K[..., :head_size_vo])
+  nd_to_nz, nz_to_nd  tests/apitest/opstest/python/operations/multi_latent_attention/
+                      test_multi_latent_attention_int8nz.py:24-44 (shape_nd_to_nz, convert_nd_to_nz),
+                      :633-636 (a cache [blocks, block_size, channels] becomes [blocks, channels / 16,
+                      block_size, 16]); the NZCACHE operator is paged_attention over nz_to_nd of its
+                      caches (:767-797 feed the same golden as the ND test); pinned by flat addresses,
+                      the round trip and the reference's two-step reshape / permute written with torch
   block_copy          tests/apitest/opstest/python/operations/block_copy/test_block_copy.py (golden_calc:
                       source i goes to the destinations dst[cum_sum[i-1] : cum_sum[i]], one after the other)
   paged_cache_load    tests/apitest/opstest/python/operations/paged_cache_load/
@@ -321,6 +327,25 @@ def _dequant(rows_i8, scale, offset, g, dim):
     if offset is not None:
         f = f + np.asarray(offset[g * dim:(g + 1) * dim], dtype=np.float32)
     return f * np.asarray(scale[g * dim:(g + 1) * dim], dtype=np.float32)
+
+
+def nd_to_nz(x, n0=16):
+    """[..., rows, channels] -> [..., channels / n0, rows, n0]: the fractal-NZ layout of a matrix whose
+    row count is a multiple of 16 and whose channel count is a multiple of n0 (16 for 16-bit elements,
+    32 for int8). Channel c of row r moves to [c // n0, r, c % n0]."""
+    x = np.asarray(x)
+    rows, channels = x.shape[-2], x.shape[-1]
+    if rows % 16 or channels % n0:
+        raise ValueError("fractal-NZ needs rows % 16 == 0 and channels % n0 == 0")
+    lead = x.shape[:-2]
+    return np.ascontiguousarray(np.moveaxis(x.reshape(lead + (rows, channels // n0, n0)), -2, -3))
+
+
+def nz_to_nd(x):
+    """Inverse of nd_to_nz: [..., channels / n0, rows, n0] -> [..., rows, channels]."""
+    x = np.asarray(x)
+    n1, rows, n0 = x.shape[-3:]
+    return np.ascontiguousarray(np.moveaxis(x, -3, -2)).reshape(x.shape[:-3] + (rows, n1 * n0))
 
 
 def gather_rows(cache, block_table, context_len):

@@ -23,12 +23,13 @@ def dtype_code(binding, t):
 def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=None, v_scale=None,
                    v_off=None, mla_dv=0, q_scale=0.0, kernel=0, chunk_tokens=None, out=None, return_plan_info=False,
                    mask=None, mask_per_head=False, logn=None, q_lens=None, mask_rows="sequence", q_rope=None,
-                   k_rope=None, lse=None, head_major=False, poison_workspace=False):
+                   k_rope=None, lse=None, head_major=False, poison_workspace=False, fractal_nz=False):
     """atbmi_pa_plan_* + atbmi_pa_decode on `stream`; returns the output tensor.
     mask: device tensor of q's dtype shaped like one of the reference's decode
     masks; mask_per_head says that a 3-dim mask's first dim counts heads (ALIBI).
     q_rope / k_rope: the split latent layout (q and kc then hold the first 512
-    channels); lse: a [rows, heads] tensor of q's dtype that receives the log-sum-exp."""
+    channels); lse: a [rows, heads] tensor of q's dtype that receives the log-sum-exp;
+    fractal_nz: kc and k_rope are [blocks, channels / 16, block size, 16]."""
     k = binding.kernels()
     rows, heads, d = q.shape
     rope = 0 if q_rope is None else q_rope.shape[2]
@@ -39,8 +40,9 @@ def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=
         mask_batch_stride, mask_head_stride = (mask.shape[1], 0) if mask is not None else (0, 0)
     shape = binding.AtbmiPaShape(
         qDtype=dtype_code(binding, q), kvDtype=dtype_code(binding, kc), numHeads=heads,
-        numKvHeads=kc.shape[1 if head_major else 2], kvLayout=1 if head_major else 0,
-        headDimK=d, headDimV=dv, blockSize=kc.shape[2 if head_major else 1], numBlocks=kc.shape[0], maxBlocksPerSeq=tables.shape[1],
+        numKvHeads=1 if fractal_nz else kc.shape[1 if head_major else 2],
+        kvLayout=2 if fractal_nz else (1 if head_major else 0),
+        headDimK=d, headDimV=dv, blockSize=kc.shape[2 if (head_major or fractal_nz) else 1], numBlocks=kc.shape[0], maxBlocksPerSeq=tables.shape[1],
         numQueryRows=rows, mlaCombined=1 if mla_dv else 0, hasOffset=1 if k_off is not None else 0, kernel=kernel,
         qkScale=scale, qScale=q_scale, hasMask=0 if mask is None else 1, maskBatchStride=mask_batch_stride,
         maskHeadStride=mask_head_stride, maskLen=0 if mask is None else mask.shape[-1],

@@ -1407,6 +1407,15 @@ def test_split_latent_layout_and_lse(binding, oracle, dev, stream, case):
         combined = pa_decode_cabi(binding, stream, q, kc, None, tables, ctx, scale, mla_dv=dv, kernel=kernel,
                                   q_lens=q_lens, lse=lse2, chunk_tokens=chunk)
         assert torch.equal(got, combined) and torch.equal(lse, lse2)
+        # the same caches in the fractal-NZ layout [blocks, channels / 16, block, 16]: other addresses, same values
+        nz_nope = torch.from_numpy(oracle.nd_to_nz(k_nope.view(torch.int16).cpu().numpy()[:, :, 0, :])).to(dev).view(dtype)
+        nz_rope = torch.from_numpy(oracle.nd_to_nz(k_rope.view(torch.int16).cpu().numpy()[:, :, 0, :])).to(dev).view(dtype)
+        assert tuple(nz_nope.shape) == (kc.shape[0], 32, block, 16) and tuple(nz_rope.shape) == (kc.shape[0], 4, block, 16)
+        lse3 = torch.zeros_like(lse)
+        from_nz = pa_decode_cabi(binding, stream, q_nope, nz_nope, None, tables, ctx, scale, mla_dv=dv, kernel=kernel,
+                                 q_lens=q_lens, q_rope=q_rope, k_rope=nz_rope, lse=lse3, chunk_tokens=chunk,
+                                 fractal_nz=True)
+        assert torch.equal(got, from_nz) and torch.equal(lse, lse3), "fractal-NZ caches, kernel=%d" % kernel
 
 
 @pytest.mark.parametrize("heads,dtype", [(128, torch.bfloat16), (32, torch.float16), (8, torch.float16)])
@@ -1449,6 +1458,19 @@ def test_multi_latent_attention_operation(binding, oracle, dev, stream, heads, d
         if ring:
             assert tuple(outs[1].shape) == (rows, heads, 1) and outs[1].dtype == dtype
             assert_close(outs[1][..., 0], want_lse, TOL[dtype], "lse calcType %d" % calc)
+        op.close()
+        # cacheMode NZCACHE: the caches as [blocks, channels / 16, 128, 16] in the fractal-NZ format
+        # (reference test_multi_latent_attention_int8nz.py:633-636,767-797)
+        nz = [torch.from_numpy(oracle.nd_to_nz(t.view(torch.int16).cpu().numpy()[:, :, 0, :])).to(dev).view(dtype)
+              for t in (k_nope, k_rope)]
+        ins[2:4] = [binding.make_tensor(binding._torch_acl_dtype(t), list(t.shape), device_ptr=t.data_ptr(),
+                                        fmt="fractal_nz") for t in nz]
+        op = binding.OperationRunner("MultiLatentAttentionOperation", binding.MultiLatentAttentionParam(
+            headNum=heads, kvHeadNum=1, qkScale=scale, cacheMode=3, calcType=calc, maskType=1 if multi else 0), c)
+        with torch.cuda.stream(stream):
+            outs_nz = op.run(ins, host_inputs=host)
+        stream.synchronize()
+        assert len(outs_nz) == len(outs) and all(torch.equal(a, b) for a, b in zip(outs, outs_nz)), "NZCACHE %d" % calc
         op.close()
     c.close()
 

@@ -64,8 +64,8 @@ def _rac_unimplemented(p):
 
 def _mla_unimplemented(p):
     """Features of MultiLatentAttentionParam the reference accepts but this library rejects at creation:
-    the prefill calcType, the fractal-NZ cache modes, masks other than MASK_TYPE_SPEC, maskUseStatus."""
-    return (p.get("calcType", 0) == 4 or p.get("cacheMode", 0) in (2, 3) or p.get("maskType", 0) >= 2 or
+    the prefill calcType, the int8 fractal-NZ cache mode, masks other than MASK_TYPE_SPEC, maskUseStatus."""
+    return (p.get("calcType", 0) == 4 or p.get("cacheMode", 0) == 2 or p.get("maskType", 0) >= 2 or
             p.get("maskUseStatusType", 0) != 0)
 
 
@@ -252,9 +252,9 @@ def test_table_coverage():
     rac_dev = [c for c in RAC_CASES if _rac_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
     assert len(PA_CASES) == 81 and len(PA_CASES) - len(pa_dev) >= 75
     assert len(RAC_CASES) == 38 and len(RAC_CASES) - len(rac_dev) >= 29
-    # most MultiLatentAttention rows exercise the prefill calcType and the fractal-NZ caches, which are not built
+    # most MultiLatentAttention rows exercise the prefill calcType and the int8 fractal-NZ cache, which are not built
     mla_dev = [c for c in MLA_CASES if _mla_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
-    assert len(MLA_CASES) == 147 and len(MLA_CASES) - len(mla_dev) == 45
+    assert len(MLA_CASES) == 147 and len(MLA_CASES) - len(mla_dev) == 46
 
 
 def test_param_sizes(binding):
@@ -569,7 +569,7 @@ def test_multi_latent_attention_counts_shapes_and_setup(binding, ctx):
         assert op.ok and (op.input_num(), op.output_num()) == (n_in, n_out), kw
         op.close()
     for bad in (dict(headNum=12), dict(kvHeadNum=2), dict(cacheMode=0), dict(maskType=1), dict(qkScale=1.5),
-                dict(qkScale=0.0), dict(calcType=5), dict(cacheMode=2), dict(cacheMode=3), dict(calcType=4),
+                dict(qkScale=0.0), dict(calcType=5), dict(cacheMode=2), dict(cacheMode=4), dict(calcType=4),
                 dict(calcType=1, maskType=2), dict(calcType=1, maskType=3), dict(calcType=1, maskType=4),
                 dict(calcType=3, maskUseStatusType=1)):
         kw = dict(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1)
@@ -629,6 +629,63 @@ def test_multi_latent_attention_counts_shapes_and_setup(binding, ctx):
     assert spec.setup(pack(rows=5, mask=[5, 300], with_qlens=True), outs(rows=5), ctx)[0] == e["ERROR_INVALID_PARAM"]
     assert spec.setup(pack(rows=6, mask=[6, 300], with_qlens=True, qlens_host=False), outs(rows=6), ctx)[0] == \
         e["ERROR_INVALID_PARAM"]
+    spec.close()
+
+
+def test_multi_latent_attention_nz_cache_checks(binding, ctx):
+    """cacheMode NZCACHE: caches [blocks, channels / 16, 128, 16] in the fractal-NZ format (reference
+    multi_latent_attention_operation.cpp:394-425). Only the plain decode has a dtype / format table in the
+    reference (ops_configs/atb_ops_info.ini:6946-6967); with qSeqlen, a mask or the log-sum-exp output the
+    section name it builds does not exist and the table check is skipped (operation_base.cpp:229-233)."""
+    e = binding.ERROR_CODE
+    mk = binding.MultiLatentAttentionParam
+    lens = np.array([10, 300, 0, 64], dtype=np.int32)
+    qlens = np.array([1, 3, 2, 2], dtype=np.int32)
+
+    def pack(kv=(16, 32, 128, 16), kr=(16, 4, 128, 16), fmt="fractal_nz", dtype="float16", rows=4, with_qlens=False):
+        ins = [binding.make_tensor(dtype, [rows, 32, 512], FAKE_DEVICE),
+               binding.make_tensor(dtype, [rows, 32, 64], FAKE_DEVICE),
+               binding.make_tensor(dtype, list(kv), FAKE_DEVICE, fmt=fmt),
+               binding.make_tensor(dtype, list(kr), FAKE_DEVICE, fmt=fmt),
+               binding.make_tensor("int32", [4, 3], FAKE_DEVICE),
+               binding.make_tensor("int32", [4], FAKE_DEVICE, host_ptr=lens.ctypes.data)]
+        if with_qlens:
+            ins.append(binding.make_tensor("int32", [4], FAKE_DEVICE, host_ptr=qlens.ctypes.data))
+        return ins
+
+    def outs(rows=4, lse=False, dtype="float16"):
+        o = [binding.make_tensor(dtype, [rows, 32, 512], FAKE_DEVICE)]
+        if lse:
+            o.append(binding.make_tensor(dtype, [rows, 32, 1], FAKE_DEVICE))
+        return o
+
+    op = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=3))
+    assert op.ok and (op.input_num(), op.output_num()) == (6, 1)
+    st, descs = op.infer_shape(pack())
+    assert st == 0 and [[d.dims[i] for i in range(d.dimNum)] for d in descs] == [[4, 32, 512]]
+    assert op.setup(pack(), outs(), ctx)[0] == 0
+    assert op.setup(pack(dtype="bf16"), outs(dtype="bf16"), ctx)[0] == 0
+    assert op.setup(pack(fmt="nd"), outs(), ctx)[0] == e["ERROR_INVALID_TENSOR_INI_MATCH"]
+    for bad in (dict(kv=(16, 32, 64, 16), kr=(16, 4, 64, 16)),      # block size is 128
+                dict(kr=(16, 4, 256, 16)), dict(kr=(15, 4, 128, 16)),
+                dict(kv=(16, 16, 128, 32)), dict(kr=(16, 2, 128, 32)),  # 16 channels per slab row
+                dict(kv=(16, 31, 128, 16)), dict(kr=(16, 8, 128, 16)),  # 512 and 64 channels
+                dict(kv=(16, 128, 1, 512), kr=(16, 128, 1, 64))):       # the token-major shapes
+        assert op.setup(pack(**bad), outs(), ctx)[0] == e["ERROR_INVALID_TENSOR_DIM"], bad
+    assert op.setup(pack(rows=5), outs(rows=5), ctx)[0] == e["ERROR_INVALID_TENSOR_DIM"]
+    op.close()
+    # with the log-sum-exp output or qSeqlen no table is checked; the dim checks are the same
+    ring = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=3,
+                                                                 calcType=2))
+    assert ring.ok and ring.output_num() == 2
+    assert ring.setup(pack(), outs(lse=True), ctx)[0] == 0
+    assert ring.setup(pack(fmt="nd"), outs(lse=True), ctx)[0] == 0
+    assert ring.setup(pack(kv=(16, 31, 128, 16)), outs(lse=True), ctx)[0] == e["ERROR_INVALID_TENSOR_DIM"]
+    ring.close()
+    spec = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=3,
+                                                                 calcType=1))
+    assert spec.ok and spec.input_num() == 7
+    assert spec.setup(pack(rows=6, with_qlens=True), outs(rows=6), ctx)[0] == 0
     spec.close()
 
 

@@ -917,6 +917,28 @@ def test_mla_equals_generic_with_materialised_values(oracle):
     assert np.array_equal(a, b) and a.shape == (3, 8, 16)
 
 
+@pytest.mark.parametrize("n0", [16, 32])
+def test_fractal_nz_layout_by_flat_addresses_and_round_trip(oracle, n0):
+    """Channel c of row r of block b lands at flat element b*rows*channels + (c // n0)*rows*n0 + r*n0 + c % n0;
+    the permutation written the reference's way (rows cut into 16s first, then the four axes permuted,
+    test_multi_latent_attention_int8nz.py:38-44) gives the same array; nz_to_nd undoes it."""
+    rng = _rng(120 + n0)
+    blocks, rows, channels = 3, 32, 4 * n0
+    x = rng.integers(-1000, 1000, size=(blocks, rows, channels)).astype(np.int16)
+    nz = oracle.nd_to_nz(x, n0)
+    assert nz.shape == (blocks, channels // n0, rows, n0) and nz.flags["C_CONTIGUOUS"]
+    flat = nz.reshape(-1)
+    for b in range(blocks):
+        for r in range(rows):
+            for c in range(channels):
+                assert flat[b * rows * channels + (c // n0) * rows * n0 + r * n0 + c % n0] == x[b, r, c]
+    t = torch.from_numpy(x).reshape(blocks, rows // 16, 16, channels // n0, n0).permute(0, 3, 1, 2, 4)
+    assert np.array_equal(t.reshape(blocks, channels // n0, rows, n0).numpy(), nz)
+    assert np.array_equal(oracle.nz_to_nd(nz), x)
+    with pytest.raises(ValueError):
+        oracle.nd_to_nz(x[:, :8], n0)
+
+
 def test_q_scale_rounds_in_query_dtype(oracle):
     rng = _rng(13)
     q, kc, vc, tables, ctx = _paged_case(rng)
