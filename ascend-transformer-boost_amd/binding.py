@@ -188,6 +188,18 @@ class AtbmiPaTensors(ctypes.Structure):
                  "mask", "logN", "queryRope", "keyRopeCache", "razorOffset", "lse")]
 
 
+class AtbmiMlaPrefillCall(ctypes.Structure):
+    """One atbmi_mla_prefill call (include/atbmi_kernels.h)."""
+    _fields_ = [("dtype", ctypes.c_int32), ("numHeads", ctypes.c_int32), ("numKvHeads", ctypes.c_int32),
+                ("mask", ctypes.c_int32), ("windowSize", ctypes.c_int32), ("qkScale", ctypes.c_float),
+                ("batch", ctypes.c_int32), ("reserved", ctypes.c_int32), ("kvPaddedRows", ctypes.c_int64),
+                ("hostQLens", ctypes.c_void_p), ("hostKvLens", ctypes.c_void_p), ("query", ctypes.c_void_p),
+                ("queryRope", ctypes.c_void_p), ("key", ctypes.c_void_p), ("keyRope", ctypes.c_void_p),
+                ("value", ctypes.c_void_p), ("out", ctypes.c_void_p)]
+
+
+ATBMI_MLA_PREFILL_MASK_NONE, ATBMI_MLA_PREFILL_MASK_CAUSAL, ATBMI_MLA_PREFILL_MASK_WINDOW = 0, 1, 2
+
 _kernels = None
 _atb = None
 
@@ -236,6 +248,8 @@ def kernels():
         lib.atbmi_pa_decode_static.argtypes = [vp, ctypes.POINTER(AtbmiPaTensors), vp]
         lib.atbmi_pa_static_scratch_bytes.argtypes = []
         lib.atbmi_pa_static_scratch_bytes.restype = u64
+        lib.atbmi_mla_prefill_workspace_size.argtypes = [ctypes.POINTER(AtbmiMlaPrefillCall), ctypes.POINTER(u64)]
+        lib.atbmi_mla_prefill.argtypes = [ctypes.POINTER(AtbmiMlaPrefillCall), vp, u64, vp]
         lib.atbmi_pa_plan_destroy.argtypes = [vp]
         lib.atbmi_pa_plan_destroy.restype = None
         lib.atbmi_timing_enable.argtypes = [i32]
@@ -289,6 +303,9 @@ def atb():
                                                            ctypes.c_uint8, vp, vp, ctypes.POINTER(u64),
                                                            ctypes.POINTER(vp), vp]
         lib.AtbMLA.argtypes = [vp, u64, vp, vp]
+        lib.AtbMLAPreFillGetWorkspaceSize.argtypes = [vp] * 8 + [i32, ctypes.c_float, i32, ctypes.c_int, ctypes.c_uint8,
+                                                                 vp, ctypes.POINTER(u64), ctypes.POINTER(vp), vp]
+        lib.AtbMLAPreFill.argtypes = [vp, u64, vp, vp]
         lib.AtbPagedCacheLoadGetWorkspaceSize.argtypes = [vp] * 7 + [ctypes.c_int8, ctypes.c_bool, ctypes.c_bool,
                                                                      ctypes.POINTER(u64), ctypes.POINTER(vp), vp]
         lib.AtbPagedCacheLoad.argtypes = [vp, u64, vp, vp]

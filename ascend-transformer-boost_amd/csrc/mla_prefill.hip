@@ -1,0 +1,514 @@
+// Prefill attention of MultiLatentAttention (calcType PREFILL) for gfx950: variable-length flash attention
+// with 128 + 64 key channels and 128 value channels per head (reference operator
+// src/ops/ops_infer/multi_latent_attention/multi_latent_attention_ops_runner_prefill.cpp, device kernels
+// src/kernels/mixkernels/multi_latent_attention/op_kernel/mla_prefill*.cce).
+//
+// A workgroup owns 128 consecutive queries of one sequence and one head: four waves of 32 queries each
+// walk the keys the block may see in 32-token steps over tiles that the workgroup stages in LDS once.
+//   HBM -> VGPR -> LDS : K rows (128 + 64 channels from two tensors) and V rows of the next step are
+//                        requested before this step's arithmetic and written after it (two tile buffers,
+//                        one barrier per step);
+//   S^T = K . Q^T      : v_mfma_f32_32x32x16, K from LDS as A (ds_read_b128), Q^T resident in registers as B;
+//                        lane (n, kh) then holds 16 tokens of query n: 8 (e / 4) + 4 kh + e % 4;
+//   softmax            : base 2, online; the row maximum needs one exchange between lanes n and n + 32;
+//   O^T += V^T . P^T   : the score registers are the B operand as they stand (k index 8 kh + e of the
+//                        half-step kb is token 16 kb + 8 (e / 4) + 4 kh + e % 4), V^T comes from the
+//                        row-major tile through the transposing ds_read_b64_tr_b16.
+// Steps that a mask hides completely are not visited (causal: keys past the block's last query; window:
+// keys before the first query's window); inside a visited step hidden scores are -inf.
+#include <algorithm>
+#include <mutex>
+#include <vector>
+#include <cstring>
+#include "atbmi_common.h"
+
+namespace atbmi {
+namespace prefill {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int DN = 128;               // channels of query / key
+constexpr int DR = 64;                // channels of queryRope / keyRope
+constexpr int D = DN + DR;
+constexpr int DV = 128;
+constexpr int QW = 32;                // queries per wave
+constexpr int NWAVES = 4;
+constexpr int QB = QW * NWAVES;       // queries per workgroup
+constexpr int STEP = 32;              // keys per step
+constexpr int K_PITCH = D * 2 + 16;   // 400 bytes: 16 lanes x 16 bytes of one operand read touch every bank once
+constexpr int V_PITCH = DV * 2 + 64;  // 320 bytes: four rows x 64 bytes of one transposing read likewise
+constexpr int K_TILE = STEP * K_PITCH;
+constexpr int V_TILE = STEP * V_PITCH;
+constexpr int BUF = K_TILE + V_TILE;
+constexpr int LDS_BYTES = 2 * BUF;
+constexpr int K_PIECES = STEP * (D / 8) / (NWAVES * WAVE);  // 16-byte pieces of a K tile per thread
+constexpr int V_PIECES = STEP * (DV / 8) / (NWAVES * WAVE);
+static_assert(K_PIECES == 3 && V_PIECES == 2 && LDS_BYTES == 46080, "tile staging assumes these sizes");
+
+// One block of queries: rows [qRow0, qRow0 + nQ) of the query tensors, positions [qPos0, qPos0 + nQ) of
+// a sequence whose keys are rows [kRow0, kRow0 + kvLen) of the key / value tensors.
+struct Item {
+    int32_t qRow0;
+    int32_t nQ;
+    int32_t kRow0;
+    int32_t kvLen;
+    int32_t qPos0;
+    int32_t pad[3];
+};
+
+struct Args {
+    const void *q;
+    const void *qRope;
+    const void *k;
+    const void *kRope;
+    const void *v;
+    void *out;
+    const Item *items;
+    int32_t H;
+    int32_t G;
+    int32_t group;   // H / G
+    int32_t mask;    // AtbmiMlaPrefillMask
+    int32_t window;
+    float scale2;    // qkScale * log2(e)
+};
+
+template <bool BF16> __device__ __forceinline__ f32x16 Mma(u32x4 a, u32x4 b, f32x16 c)
+{
+    if constexpr (BF16) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
+                                                       c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c,
+                                                      0, 0, 0);
+    }
+}
+
+template <bool BF16> __device__ __forceinline__ uint32_t Pack2(float lo, float hi)
+{
+    if constexpr (BF16) {
+        bf16x2 v = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};
+        return __builtin_bit_cast(uint32_t, v);
+    } else {
+        f16x2 v = {static_cast<_Float16>(lo), static_cast<_Float16>(hi)};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+}
+
+__device__ __forceinline__ float Exp2(float x)
+{
+    return __builtin_amdgcn_exp2f(x);
+}
+
+template <bool BF16> __global__ __launch_bounds__(NWAVES *WAVE) void MlaPrefillKernel(const Args a)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char smem[LDS_BYTES];
+    const int tid = threadIdx.x;
+    const int lane = tid & (WAVE - 1);
+    const int wave = tid / WAVE;
+    const int n = lane & 31;  // query column of this lane
+    const int kh = lane >> 5; // which half of an MFMA's contraction values this lane holds
+    const Item it = a.items[blockIdx.x / a.H];
+    const int h = blockIdx.x % a.H;
+    const int g = h / a.group;
+
+    const int qLocal = wave * QW + n;
+    const bool qValid = qLocal < it.nQ;
+    const int qPos = it.qPos0 + qLocal;
+    const bool waveHasWork = wave * QW < it.nQ;
+    const int qFirstW = it.qPos0 + wave * QW;                       // first and last query position of this wave
+    const int qLastW = it.qPos0 + min(it.nQ, wave * QW + QW) - 1;
+
+    // ---- Q^T as B operand: lane (n, kh) holds q[n][16 j + 8 kh .. +8) for the 12 pieces j
+    u32x4 qreg[D / 16];
+    {
+        const int64_t rowHead = (static_cast<int64_t>(it.qRow0) + (qValid ? qLocal : 0)) * a.H + h;
+        const uint16_t *qn = reinterpret_cast<const uint16_t *>(a.q) + rowHead * DN + kh * 8;
+        const uint16_t *qr = reinterpret_cast<const uint16_t *>(a.qRope) + rowHead * DR + kh * 8;
+#pragma unroll
+        for (int j = 0; j < D / 16; ++j) {
+            qreg[j] = *reinterpret_cast<const u32x4 *>(j < DN / 16 ? qn + 16 * j : qr + 16 * (j - DN / 16));
+            if (!qValid) {
+                qreg[j] = u32x4{0u, 0u, 0u, 0u};
+            }
+        }
+    }
+
+    // ---- the keys this block visits
+    int tBegin = 0;
+    int tEnd = it.kvLen;
+    if (a.mask != ATBMI_MLA_PREFILL_MASK_NONE) {
+        tEnd = min(tEnd, it.qPos0 + it.nQ);
+    }
+    if (a.mask == ATBMI_MLA_PREFILL_MASK_WINDOW) {
+        tBegin = max(0, it.qPos0 - a.window + 1) & ~(STEP - 1);
+    }
+
+    const unsigned char *kBase = reinterpret_cast<const unsigned char *>(a.k);
+    const unsigned char *krBase = reinterpret_cast<const unsigned char *>(a.kRope);
+    const unsigned char *vBase = reinterpret_cast<const unsigned char *>(a.v);
+    u32x4 kStage[K_PIECES];
+    u32x4 vStage[V_PIECES];
+    // Requests this thread's pieces of the tile at key t (rows at or past kvLen read as zeros).
+    auto loadTile = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < K_PIECES; ++i) {
+            const int p = tid + i * NWAVES * WAVE;
+            const int row = p / (D / 8);
+            const int col = p % (D / 8);
+            kStage[i] = u32x4{0u, 0u, 0u, 0u};
+            if (t + row < it.kvLen) {
+                const int64_t rg = (static_cast<int64_t>(it.kRow0) + t + row) * a.G + g;
+                kStage[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(
+                    col < DN / 8 ? kBase + rg * (DN * 2) + col * 16 : krBase + rg * (DR * 2) + (col - DN / 8) * 16));
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < V_PIECES; ++i) {
+            const int p = tid + i * NWAVES * WAVE;
+            const int row = p / (DV / 8);
+            const int col = p % (DV / 8);
+            vStage[i] = u32x4{0u, 0u, 0u, 0u};
+            if (t + row < it.kvLen) {
+                const int64_t rg = (static_cast<int64_t>(it.kRow0) + t + row) * a.G + g;
+                vStage[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(vBase + rg * (DV * 2) + col * 16));
+            }
+        }
+    };
+    auto storeTile = [&](unsigned char *buf) {
+#pragma unroll
+        for (int i = 0; i < K_PIECES; ++i) {
+            const int p = tid + i * NWAVES * WAVE;
+            *reinterpret_cast<u32x4 *>(buf + (p / (D / 8)) * K_PITCH + (p % (D / 8)) * 16) = kStage[i];
+        }
+#pragma unroll
+        for (int i = 0; i < V_PIECES; ++i) {
+            const int p = tid + i * NWAVES * WAVE;
+            *reinterpret_cast<u32x4 *>(buf + K_TILE + (p / (DV / 8)) * V_PITCH + (p % (DV / 8)) * 16) = vStage[i];
+        }
+    };
+
+    float m = -INFINITY; // running maximum of query n, base-2 exponent units
+    float l = 0.0f;      // this lane's share of the running denominator
+    f32x16 acc[DV / 32];
+#pragma unroll
+    for (int i = 0; i < DV / 32; ++i) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            acc[i][e] = 0.0f;
+        }
+    }
+
+    const int l16 = lane & 15;
+    const int kOperand = n * K_PITCH + kh * 16;
+    const int vOperand = K_TILE + (4 * kh + (l16 >> 2)) * V_PITCH + (((lane >> 4) & 1) * 16 + (l16 & 3) * 4) * 2;
+
+    auto computeStep = [&](int t, const unsigned char *buf) {
+        f32x16 s;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            s[e] = 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < D / 16; ++j) {
+            const u32x4 kk = *reinterpret_cast<const u32x4 *>(buf + kOperand + j * 32);
+            s = Mma<BF16>(kk, qreg[j], s);
+        }
+        // every key of the step visible to every query of the wave: no comparisons
+        const bool open = t + STEP <= it.kvLen &&
+                          (a.mask == ATBMI_MLA_PREFILL_MASK_NONE ||
+                           (t + STEP - 1 <= qFirstW &&
+                            (a.mask != ATBMI_MLA_PREFILL_MASK_WINDOW || t > qLastW - a.window)));
+        float mLoc = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            float x = s[e] * a.scale2;
+            if (!open) {
+                const int tok = t + 8 * (e >> 2) + 4 * kh + (e & 3);
+                bool hidden = tok >= it.kvLen;
+                if (a.mask != ATBMI_MLA_PREFILL_MASK_NONE) {
+                    hidden = hidden || tok > qPos;
+                }
+                if (a.mask == ATBMI_MLA_PREFILL_MASK_WINDOW) {
+                    hidden = hidden || tok <= qPos - a.window;
+                }
+                x = hidden ? -INFINITY : x;
+            }
+            s[e] = x;
+            mLoc = fmaxf(mLoc, x);
+        }
+        mLoc = fmaxf(mLoc, __shfl_xor(mLoc, 32));
+        const float mNew = fmaxf(m, mLoc);
+        const float mRef = mNew == -INFINITY ? 0.0f : mNew; // nothing visible so far: every weight is 0
+        const float corr = Exp2(m - mRef);
+        m = mNew;
+        float sum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            s[e] = Exp2(s[e] - mRef);
+            sum += s[e];
+        }
+        l = l * corr + sum;
+        if (__any(corr != 1.0f)) {
+#pragma unroll
+            for (int i = 0; i < DV / 32; ++i) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    acc[i][e] *= corr;
+                }
+            }
+        }
+        u32x4 pop[2]; // P^T as B operand of the two half-steps
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                pop[kb][w] = Pack2<BF16>(s[8 * kb + 2 * w], s[8 * kb + 2 * w + 1]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < DV / 32; ++i) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                const unsigned char *vp = buf + vOperand + kb * 16 * V_PITCH + i * 64;
+                const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4 *)(vp));
+                const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (__attribute__((address_space(3))) i16x4 *)(vp + 8 * V_PITCH));
+                const u32x2 lo2 = __builtin_bit_cast(u32x2, lo);
+                const u32x2 hi2 = __builtin_bit_cast(u32x2, hi);
+                acc[i] = Mma<BF16>(u32x4{lo2[0], lo2[1], hi2[0], hi2[1]}, pop[kb], acc[i]);
+            }
+        }
+    };
+
+    if (tBegin < tEnd) {
+        loadTile(tBegin);
+        storeTile(smem);
+    }
+    __syncthreads();
+    int cur = 0;
+    for (int t = tBegin; t < tEnd; t += STEP) {
+        const bool more = t + STEP < tEnd;
+        if (more) {
+            loadTile(t + STEP);
+        }
+        // a wave skips the steps that its own queries cannot see
+        bool visit = waveHasWork;
+        if (a.mask != ATBMI_MLA_PREFILL_MASK_NONE) {
+            visit = visit && t <= qLastW;
+        }
+        if (a.mask == ATBMI_MLA_PREFILL_MASK_WINDOW) {
+            visit = visit && t + STEP - 1 > qFirstW - a.window;
+        }
+        if (visit) {
+            computeStep(t, smem + cur * BUF);
+        }
+        if (more) {
+            storeTile(smem + (cur ^ 1) * BUF);
+        }
+        __syncthreads();
+        cur ^= 1;
+    }
+
+    // ---- out[q][h][32 i + 8 r + 4 kh .. +4) = acc / l
+    l += __shfl_xor(l, 32);
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f; // a query that sees no key yields zeros
+    if (qValid) {
+        uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) +
+                         ((static_cast<int64_t>(it.qRow0) + qLocal) * a.H + h) * DV + 4 * kh;
+#pragma unroll
+        for (int i = 0; i < DV / 32; ++i) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                u32x2 w;
+                w[0] = Pack2<BF16>(acc[i][4 * r] * inv, acc[i][4 * r + 1] * inv);
+                w[1] = Pack2<BF16>(acc[i][4 * r + 2] * inv, acc[i][4 * r + 3] * inv);
+                *reinterpret_cast<u32x2 *>(orow + 32 * i + 8 * r) = w;
+            }
+        }
+    }
+}
+
+// Pinned staging for the asynchronous upload of the block list: a slot is reused only after the copy that
+// last read it has finished. One ring per process, taken under a lock for the length of a launch call.
+constexpr int RING = 4;
+struct UploadRing {
+    std::mutex lock;
+    void *pinned[RING] = {nullptr, nullptr, nullptr, nullptr};
+    size_t cap[RING] = {0, 0, 0, 0};
+    hipEvent_t copied[RING] = {nullptr, nullptr, nullptr, nullptr};
+    bool inFlight[RING] = {false, false, false, false};
+    int pos = 0;
+};
+UploadRing g_ring;
+
+int Upload(const void *src, size_t bytes, void *dst, hipStream_t stream)
+{
+    std::lock_guard<std::mutex> hold(g_ring.lock);
+    const int slot = g_ring.pos;
+    g_ring.pos = (g_ring.pos + 1) % RING;
+    if (g_ring.inFlight[slot]) {
+        ATBMI_HIP_CHECK(hipEventSynchronize(g_ring.copied[slot]));
+        g_ring.inFlight[slot] = false;
+    }
+    if (g_ring.cap[slot] < bytes) {
+        if (g_ring.pinned[slot]) {
+            ATBMI_HIP_CHECK(hipHostFree(g_ring.pinned[slot]));
+            g_ring.pinned[slot] = nullptr;
+            g_ring.cap[slot] = 0;
+        }
+        const size_t cap = (bytes * 2 + 4095) / 4096 * 4096;
+        ATBMI_HIP_CHECK(hipHostMalloc(&g_ring.pinned[slot], cap, hipHostMallocDefault));
+        g_ring.cap[slot] = cap;
+    }
+    if (!g_ring.copied[slot]) {
+        ATBMI_HIP_CHECK(hipEventCreateWithFlags(&g_ring.copied[slot], hipEventDisableTiming));
+    }
+    memcpy(g_ring.pinned[slot], src, bytes);
+    ATBMI_HIP_CHECK(hipMemcpyAsync(dst, g_ring.pinned[slot], bytes, hipMemcpyHostToDevice, stream));
+    ATBMI_HIP_CHECK(hipEventRecord(g_ring.copied[slot], stream));
+    g_ring.inFlight[slot] = true;
+    return OK;
+}
+
+// Checks the call and lists its query blocks, longest key walk first.
+int BuildItems(const AtbmiMlaPrefillCall *c, std::vector<Item> *items)
+{
+    if (!c || !c->hostQLens || !c->hostKvLens) {
+        return Fail(ERR_INVALID_PARAM, "mla_prefill: null call or length arrays");
+    }
+    if (c->dtype != ATBMI_F16 && c->dtype != ATBMI_BF16) {
+        return Fail(ERR_INVALID_PARAM, "mla_prefill: dtype %d (fp16 or bf16)", c->dtype);
+    }
+    if (c->numHeads <= 0 || c->numKvHeads <= 0 || c->numHeads % c->numKvHeads != 0) {
+        return Fail(ERR_INVALID_PARAM, "mla_prefill: %d heads over %d KV heads", c->numHeads, c->numKvHeads);
+    }
+    if (c->mask < ATBMI_MLA_PREFILL_MASK_NONE || c->mask > ATBMI_MLA_PREFILL_MASK_WINDOW) {
+        return Fail(ERR_INVALID_PARAM, "mla_prefill: mask %d", c->mask);
+    }
+    if (c->mask == ATBMI_MLA_PREFILL_MASK_WINDOW && c->windowSize <= 0) {
+        return Fail(ERR_INVALID_PARAM, "mla_prefill: a window mask needs windowSize > 0, got %d", c->windowSize);
+    }
+    if (c->batch < 0 || c->kvPaddedRows < 0 || !(c->qkScale > 0.0f)) {
+        return Fail(ERR_INVALID_PARAM, "mla_prefill: batch %d, kvPaddedRows %lld, qkScale %g", c->batch,
+                    (long long)c->kvPaddedRows, c->qkScale);
+    }
+    int64_t qRow = 0, kRow = 0;
+    for (int32_t b = 0; b < c->batch; ++b) {
+        const int32_t nq = c->hostQLens[b];
+        const int32_t nk = c->hostKvLens[b];
+        if (nq < 0 || nk < 0) {
+            return Fail(ERR_INVALID_PARAM, "mla_prefill: sequence %d has lengths %d / %d", b, nq, nk);
+        }
+        if (c->mask != ATBMI_MLA_PREFILL_MASK_NONE && nq != nk) {
+            return Fail(ERR_INVALID_PARAM, "mla_prefill: with a mask, query and key lengths must agree (sequence %d: %d / %d)",
+                        b, nq, nk);
+        }
+        if (c->kvPaddedRows > 0) {
+            if (nk > c->kvPaddedRows) {
+                return Fail(ERR_INVALID_PARAM, "mla_prefill: sequence %d has %d keys in %lld padded rows", b, nk,
+                            (long long)c->kvPaddedRows);
+            }
+            kRow = static_cast<int64_t>(b) * c->kvPaddedRows;
+        }
+        if (qRow + nq > 0x7fffffffLL || kRow + nk > 0x7fffffffLL) {
+            return Fail(ERR_INVALID_PARAM, "mla_prefill: more than 2^31 rows");
+        }
+        for (int32_t q0 = 0; q0 < nq; q0 += QB) {
+            Item it{};
+            it.qRow0 = static_cast<int32_t>(qRow + q0);
+            it.nQ = nq - q0 < QB ? nq - q0 : QB;
+            it.kRow0 = static_cast<int32_t>(kRow);
+            it.kvLen = nk;
+            it.qPos0 = q0;
+            if (items) {
+                items->push_back(it);
+            }
+        }
+        qRow += nq;
+        kRow += nk;
+    }
+    if (items && c->mask != ATBMI_MLA_PREFILL_MASK_NONE) {
+        // blocks late in a sequence walk the most keys: start them first
+        std::stable_sort(items->begin(), items->end(), [](const Item &x, const Item &y) { return x.qPos0 > y.qPos0; });
+    } else if (items) {
+        std::stable_sort(items->begin(), items->end(), [](const Item &x, const Item &y) { return x.kvLen > y.kvLen; });
+    }
+    return OK;
+}
+
+} // namespace prefill
+} // namespace atbmi
+
+using namespace atbmi;
+
+extern "C" int atbmi_mla_prefill_workspace_size(const AtbmiMlaPrefillCall *call, uint64_t *bytes)
+{
+    if (!bytes) {
+        return Fail(ERR_INVALID_PARAM, "mla_prefill_workspace_size: null result pointer");
+    }
+    std::vector<prefill::Item> items;
+    const int rc = prefill::BuildItems(call, &items);
+    if (rc != OK) {
+        return rc;
+    }
+    *bytes = items.size() * sizeof(prefill::Item);
+    return OK;
+}
+
+extern "C" int atbmi_mla_prefill(const AtbmiMlaPrefillCall *call, void *workspaceDevice, uint64_t workspaceBytes,
+                                 void *stream)
+{
+    std::vector<prefill::Item> items;
+    int rc = prefill::BuildItems(call, &items);
+    if (rc != OK) {
+        return rc;
+    }
+    if (items.empty()) {
+        return OK;
+    }
+    if (!call->query || !call->queryRope || !call->key || !call->keyRope || !call->value || !call->out) {
+        return Fail(ERR_INVALID_PARAM, "mla_prefill: null tensor pointer");
+    }
+    const size_t bytes = items.size() * sizeof(prefill::Item);
+    if (!workspaceDevice || workspaceBytes < bytes) {
+        return Fail(ERR_INVALID_PARAM, "mla_prefill: workspace of %llu bytes, %llu needed",
+                    (unsigned long long)workspaceBytes, (unsigned long long)bytes);
+    }
+    const int64_t grid = static_cast<int64_t>(items.size()) * call->numHeads;
+    if (grid > 0x7fffffffLL) {
+        return Fail(ERR_INVALID_PARAM, "mla_prefill: %lld workgroups", (long long)grid);
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    rc = prefill::Upload(items.data(), bytes, workspaceDevice, s);
+    if (rc != OK) {
+        return rc;
+    }
+    prefill::Args a{};
+    a.q = call->query;
+    a.qRope = call->queryRope;
+    a.k = call->key;
+    a.kRope = call->keyRope;
+    a.v = call->value;
+    a.out = call->out;
+    a.items = static_cast<const prefill::Item *>(workspaceDevice);
+    a.H = call->numHeads;
+    a.G = call->numKvHeads;
+    a.group = call->numHeads / call->numKvHeads;
+    a.mask = call->mask;
+    a.window = call->windowSize;
+    a.scale2 = call->qkScale * 1.4426950408889634f;
+    if (call->dtype == ATBMI_BF16) {
+        prefill::MlaPrefillKernel<true><<<static_cast<unsigned>(grid), prefill::NWAVES * WAVE, 0, s>>>(a);
+    } else {
+        prefill::MlaPrefillKernel<false><<<static_cast<unsigned>(grid), prefill::NWAVES * WAVE, 0, s>>>(a);
+    }
+    ATBMI_HIP_CHECK(hipGetLastError());
+    return OK;
+}

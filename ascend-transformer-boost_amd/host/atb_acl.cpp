@@ -217,6 +217,58 @@ atb::Status AtbMLA(void *workspace, uint64_t workspaceSize, atb::Operation *op, 
     return RunExecute("AtbMLA", workspace, workspaceSize, op, context);
 }
 
+atb::Status AtbMLAPreFillGetWorkspaceSize(const aclTensor *q, const aclTensor *qRope, const aclTensor *k,
+                                          const aclTensor *kRope, const aclTensor *v, const aclTensor *qSeqLen,
+                                          const aclTensor *kvSeqLen, const aclTensor *mask, int32_t headNum,
+                                          float qkScale, int32_t kvHeadNum, int maskType, uint8_t cacheMode,
+                                          aclTensor *attenOut, uint64_t *workspaceSize, atb::Operation **op,
+                                          atb::Context *context)
+{
+    using Param = atb::infer::MultiLatentAttentionParam;
+    Param param;
+    param.headNum = headNum;
+    param.qkScale = qkScale;
+    param.kvHeadNum = kvHeadNum;
+    param.maskType = Param::MaskType(maskType);
+    param.calcType = Param::CALC_TYPE_PREFILL;
+    param.cacheMode = Param::CacheMode(cacheMode);
+    if (op == nullptr || workspaceSize == nullptr) {
+        ATB_LOG(ERROR) << "AtbMLAPreFillGetWorkspaceSize: op and workspaceSize must not be null";
+        return atb::ERROR_INVALID_OPERATION_ADDR;
+    }
+    if (*op == nullptr) {
+        atb::Status st = atb::CreateOperation(param, op);
+        if (st != atb::NO_ERROR) {
+            ATB_LOG(ERROR) << "AtbMLAPreFillGetWorkspaceSize: creating the operation failed";
+            return st;
+        }
+    }
+    // The mask travels with the mask types whose operation takes one (MASK_FREE; this wrapper has no
+    // windowSize argument, so SWA_NORM never gets past creation); both length tensors are host tensors.
+    const bool hasMask = param.maskType != Param::UNDEFINED && param.maskType != Param::MASK_TYPE_CAUSAL_MASK;
+    atb::VariantPack pack;
+    pack.inTensors.resize(hasMask ? 8 : 7);
+    size_t i = 0;
+    ATB_ACL_CONVERT(ToAtbTensor(q, &pack.inTensors[i++], true));
+    ATB_ACL_CONVERT(ToAtbTensor(qRope, &pack.inTensors[i++], true));
+    ATB_ACL_CONVERT(ToAtbTensor(k, &pack.inTensors[i++], true));
+    ATB_ACL_CONVERT(ToAtbTensor(kRope, &pack.inTensors[i++], true));
+    ATB_ACL_CONVERT(ToAtbTensor(v, &pack.inTensors[i++], true));
+    ATB_ACL_CONVERT(ToAtbTensor(qSeqLen, &pack.inTensors[i++], false));
+    ATB_ACL_CONVERT(ToAtbTensor(kvSeqLen, &pack.inTensors[i++], false));
+    if (hasMask) {
+        ATB_ACL_CONVERT(ToAtbTensor(mask, &pack.inTensors[i++], true));
+    }
+    pack.outTensors.resize(1);
+    ATB_ACL_CONVERT(ToAtbTensor(attenOut, &pack.outTensors[0], true));
+    return (*op)->Setup(pack, *workspaceSize, context);
+}
+
+atb::Status AtbMLAPreFill(void *workspace, uint64_t workspaceSize, atb::Operation *op, atb::Context *context)
+{
+    return RunExecute("AtbMLAPreFill", workspace, workspaceSize, op, context);
+}
+
 atb::Status AtbPagedCacheLoadGetWorkspaceSize(const aclTensor *keyCache, const aclTensor *valueCache,
                                               const aclTensor *blockTables, const aclTensor *contextLens,
                                               const aclTensor *key, const aclTensor *value, const aclTensor *seqStarts,

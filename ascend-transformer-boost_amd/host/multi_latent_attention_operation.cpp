@@ -13,8 +13,9 @@
 // fractal-NZ layout, [blocks, 512 / 16, 128, 16] and [blocks, 64 / 16, 128, 16];
 // reference :394-425 QKVDimCheckNz) with fp16/bf16 tensors; calcType UNDEFINED,
 // SPEC (qSeqlen, optionally with the MASK_TYPE_SPEC mask), RING and
-// SPEC_AND_RING (second output: log-sum-exp). The int8 NZ cache mode, the
-// prefill calcType, the MASK_FREE / CAUSAL_MASK / SWA_NORM masks and
+// SPEC_AND_RING (second output: log-sum-exp). calcType PREFILL is an operation
+// class of its own (multi_latent_attention_prefill_operation.cpp). The int8 NZ
+// cache mode, the MASK_FREE / CAUSAL_MASK masks of the decode calcTypes and
 // maskUseStatus are legal in the reference but not implemented here; such
 // params are rejected at creation with ERROR_INVALID_PARAM.
 //
@@ -150,8 +151,9 @@ bool ImplementedCheck(const Param &p)
 {
     const char *what = nullptr;
     if (p.calcType == Param::CALC_TYPE_PREFILL) {
-        what = "the prefill calcType";
-    } else if (p.cacheMode == Param::INT8_NZCACHE) {
+        return true; // every param that passes ParamPrefillCheck is built
+    }
+    if (p.cacheMode == Param::INT8_NZCACHE) {
         what = "the int8 fractal-NZ cache";
     } else if (p.maskType != Param::UNDEFINED && p.maskType != Param::MASK_TYPE_SPEC) {
         what = "this maskType";
@@ -202,6 +204,11 @@ OpIr MakeIr(const Param &p)
     return ir;
 }
 
+} // namespace
+
+Operation *NewMultiLatentAttentionPrefillOperation(const infer::MultiLatentAttentionParam &param);
+
+namespace {
 class MultiLatentAttentionOperation : public OperationBase {
 public:
     explicit MultiLatentAttentionOperation(const Param &param)
@@ -486,7 +493,9 @@ template <> Status CreateOperation(const infer::MultiLatentAttentionParam &opPar
     if (!ImplementedCheck(opParam)) {
         return ERROR_INVALID_PARAM;
     }
-    *operation = new (std::nothrow) MultiLatentAttentionOperation(opParam);
+    *operation = opParam.calcType == Param::CALC_TYPE_PREFILL
+                     ? NewMultiLatentAttentionPrefillOperation(opParam)
+                     : new (std::nothrow) MultiLatentAttentionOperation(opParam);
     if (*operation == nullptr) {
         return ERROR_OUT_OF_HOST_MEMORY;
     }

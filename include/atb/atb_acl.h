@@ -2,6 +2,7 @@
 // this library has: the first call creates the operation if *op is null, binds the tensors and
 // runs Setup (returning the workspace size), the second runs Execute on what the first bound.
 //   AtbMLAGetWorkspaceSize / AtbMLA                      reference include/atb/atb_acl.h:99-116
+//   AtbMLAPreFillGetWorkspaceSize / AtbMLAPreFill        reference include/atb/atb_acl.h:141-156
 //   AtbPagedCacheLoadGetWorkspaceSize / AtbPagedCacheLoad  reference include/atb/atb_acl.h:251-267
 // contextLens and qSeqLen are host tensors: their aclTensor carries a host address.
 #ifndef ATB_MI_ATB_ACL_H
@@ -16,7 +17,7 @@
 extern "C" {
 #endif
 
-// MultiLatentAttention (cacheMode KROPE_CTKV). mask is read when maskType is not UNDEFINED, qSeqLen
+// MultiLatentAttention (cacheMode KROPE_CTKV or NZCACHE). mask is read when maskType is not UNDEFINED, qSeqLen
 // when calcType is CALC_TYPE_SPEC, lse when calcType is CALC_TYPE_RING; qkDescale / pvDescale belong
 // to the int8 cache mode, which this library does not have. Pointers that are not read may be null.
 atb::Status AtbMLAGetWorkspaceSize(const aclTensor *qNope, const aclTensor *qRope, const aclTensor *ctKV,
@@ -26,6 +27,16 @@ atb::Status AtbMLAGetWorkspaceSize(const aclTensor *qNope, const aclTensor *qRop
                                    int maskType, int calcType, uint8_t cacheMode, aclTensor *attenOut, aclTensor *lse,
                                    uint64_t *workspaceSize, atb::Operation **op, atb::Context *context);
 atb::Status AtbMLA(void *workspace, uint64_t workspaceSize, atb::Operation *op, atb::Context *context);
+
+// MultiLatentAttention, calcType PREFILL (cacheMode KROPE_CTKV): attention of whole prompts over key / keyRope /
+// value tensors. qSeqLen and kvSeqLen are host tensors; mask is read when maskType is MASK_TYPE_MASK_FREE.
+atb::Status AtbMLAPreFillGetWorkspaceSize(const aclTensor *q, const aclTensor *qRope, const aclTensor *k,
+                                          const aclTensor *kRope, const aclTensor *v, const aclTensor *qSeqLen,
+                                          const aclTensor *kvSeqLen, const aclTensor *mask, int32_t headNum,
+                                          float qkScale, int32_t kvHeadNum, int maskType, uint8_t cacheMode,
+                                          aclTensor *attenOut, uint64_t *workspaceSize, atb::Operation **op,
+                                          atb::Context *context);
+atb::Status AtbMLAPreFill(void *workspace, uint64_t workspaceSize, atb::Operation *op, atb::Context *context);
 
 // PagedCacheLoad. key and value are inputs and outputs at once; seqStarts is read when hasSeqStarts.
 atb::Status AtbPagedCacheLoadGetWorkspaceSize(const aclTensor *keyCache, const aclTensor *valueCache,

@@ -377,6 +377,53 @@ uint64_t atbmi_pa_static_scratch_bytes(void);
 void atbmi_pa_plan_destroy(AtbmiPaPlan *plan);
 
 /*
+ * Prefill attention of MultiLatentAttention (MultiLatentAttentionParam::CALC_TYPE_PREFILL; reference
+ * src/ops/ops_infer/multi_latent_attention/multi_latent_attention_ops_runner_prefill.cpp:33-131, kernel library
+ * src/kernels/mixkernels/multi_latent_attention/mla_operation.cpp:184-235 and tiling/mla_tiling.cpp:286-327):
+ * flash attention over variable-length sequences with 128 + 64 key channels and 128 value channels per head.
+ * Sequence b owns hostQLens[b] consecutive rows of query / queryRope / out and hostKvLens[b] rows of key /
+ * keyRope / value: consecutive as well (kvPaddedRows 0, tensors [tokens, kvHeads, channels]), or rows
+ * [b * kvPaddedRows, b * kvPaddedRows + hostKvLens[b]) (tensors [batch, kvPaddedRows, kvHeads * channels]).
+ * Query head h attends over KV head h / (numHeads / numKvHeads).
+ *   mask NONE    every query sees every key of its sequence (MaskType UNDEFINED)
+ *        CAUSAL  query i sees keys j <= i (MASK_TYPE_CAUSAL_MASK, and MASK_TYPE_MASK_FREE, whose 512 x 512 mask
+ *                input is the strictly upper triangular matrix that says the same; its values are not read)
+ *        WINDOW  j <= i and j > i - windowSize (MASK_TYPE_SWA_NORM; the mask input is not read either)
+ * With a mask the two lengths of a sequence must agree. The lengths are host arrays, read during the call.
+ */
+typedef enum AtbmiMlaPrefillMask {
+    ATBMI_MLA_PREFILL_MASK_NONE = 0,
+    ATBMI_MLA_PREFILL_MASK_CAUSAL = 1,
+    ATBMI_MLA_PREFILL_MASK_WINDOW = 2
+} AtbmiMlaPrefillMask;
+
+typedef struct AtbmiMlaPrefillCall {
+    int32_t dtype;             /* AtbmiDtype of every tensor: ATBMI_F16 or ATBMI_BF16 */
+    int32_t numHeads;
+    int32_t numKvHeads;        /* divides numHeads */
+    int32_t mask;              /* AtbmiMlaPrefillMask */
+    int32_t windowSize;        /* WINDOW only, > 0 */
+    float qkScale;
+    int32_t batch;
+    int32_t reserved;
+    int64_t kvPaddedRows;      /* 0: key rows of the sequences follow each other */
+    const int32_t *hostQLens;  /* [batch], host memory */
+    const int32_t *hostKvLens; /* [batch], host memory */
+    const void *query;         /* [sum qLens, numHeads, 128] */
+    const void *queryRope;     /* [sum qLens, numHeads, 64] */
+    const void *key;           /* [key rows, numKvHeads, 128] */
+    const void *keyRope;       /* [key rows, numKvHeads, 64] */
+    const void *value;         /* [key rows, numKvHeads, 128] */
+    void *out;                 /* [sum qLens, numHeads, 128] */
+} AtbmiMlaPrefillCall;
+
+/* Validates the call (pointers aside) and reports the device workspace it needs: 32 bytes per block of
+ * 128 queries. Host only. */
+int atbmi_mla_prefill_workspace_size(const AtbmiMlaPrefillCall *call, uint64_t *bytes);
+/* Uploads the block list into the workspace and launches the kernel on `stream`; does not wait. */
+int atbmi_mla_prefill(const AtbmiMlaPrefillCall *call, void *workspaceDevice, uint64_t workspaceBytes, void *stream);
+
+/*
  * Kernel timing for benchmarks. atbmi_timing_enable(n) with n > 0 makes every
  * n-th atbmi_pa_decode bracket its attention kernel with HIP events on the
  * launch stream (the events themselves cost a few microseconds of stream

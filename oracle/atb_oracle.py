@@ -61,6 +61,14 @@ the invariants of the mathematics (no function is left "parity unpinned"):
                       block_size, 16]); the NZCACHE operator is paged_attention over nz_to_nd of its
                       caches (:767-797 feed the same golden as the ND test); pinned by flat addresses,
                       the round trip and the reference's two-step reshape / permute written with torch
+  mla_prefill         tests/apitest/opstest/python/operations/multi_latent_attention/
+                      test_multi_latent_attention_prefill.py:519-700 (gen_out_tensor: per sequence and head
+                      score = q . k^T * tor over the 128 + 64 channels, + mask, fp32 softmax over the keys,
+                      times v; the fp32 "out_true" branch), :301-316 and :373-391 (the masks: strictly upper
+                      triangle hidden, with a window also everything at or below the diagonal shifted down
+                      by the window), :707-716 (query and key split [128, 64] along the channels);
+                      pinned by torch's scaled_dot_product_attention (plain, is_causal, explicit band
+                      mask), float64 loops and closed forms
   block_copy          tests/apitest/opstest/python/operations/block_copy/test_block_copy.py (golden_calc:
                       source i goes to the destinations dst[cum_sum[i-1] : cum_sum[i]], one after the other)
   paged_cache_load    tests/apitest/opstest/python/operations/paged_cache_load/
@@ -607,6 +615,43 @@ def paged_attention_loops(query, key_cache, value_cache, block_tables, context_l
                 out[row][h][c] = acc / z
         row += 1
     return np.array(out, dtype=np.float64)
+
+
+def mla_prefill(q_nope, q_rope, k_nope, k_rope, value, q_lens, kv_lens, scale, mask="none", window=0,
+                kv_padded_rows=0):
+    """Prefill attention of MultiLatentAttention (calcType PREFILL): sequence b owns q_lens[b] consecutive
+    query rows and kv_lens[b] key / value rows (consecutive, or rows [b * kv_padded_rows, ...) when the keys
+    come padded per sequence); head h of a query attends over KV head h // (heads // kv_heads).
+    q_nope [T, H, 128], q_rope [T, H, 64], k_nope [Tk, G, 128], k_rope [Tk, G, 64], value [Tk, G, 128].
+    mask: "none" (every query sees every key), "causal" (query i sees keys j <= i) or "window" (j <= i and
+    j > i - window). Returns float32 [T, H, 128]."""
+    q = np.concatenate([np.asarray(q_nope, np.float32), np.asarray(q_rope, np.float32)], axis=-1)
+    k = np.concatenate([np.asarray(k_nope, np.float32), np.asarray(k_rope, np.float32)], axis=-1)
+    v = np.asarray(value, np.float32)
+    heads, kv_heads = q.shape[1], k.shape[1]
+    group = heads // kv_heads
+    out = np.zeros((q.shape[0], heads, v.shape[2]), np.float32)
+    q0 = k0 = 0
+    for b, (nq, nk) in enumerate(zip(q_lens, kv_lens)):
+        nq, nk = int(nq), int(nk)
+        if kv_padded_rows:
+            k0 = b * kv_padded_rows
+        if nq > 0 and nk > 0:
+            i = np.arange(nq)[:, None]
+            j = np.arange(nk)[None, :]
+            hidden = np.zeros((nq, nk), bool)
+            if mask in ("causal", "window"):
+                hidden |= j > i
+            if mask == "window":
+                hidden |= j <= i - window
+            for h in range(heads):
+                g = h // group
+                score = (q[q0:q0 + nq, h] @ k[k0:k0 + nk, g].T) * np.float32(scale)
+                score = np.where(hidden, -np.inf, score).astype(np.float32)
+                out[q0:q0 + nq, h] = softmax_rows(score) @ v[k0:k0 + nk, g]
+        q0 += nq
+        k0 += nk
+    return out
 
 
 def partial_attention(q, keys, values, scale):

@@ -64,9 +64,10 @@ def _rac_unimplemented(p):
 
 def _mla_unimplemented(p):
     """Features of MultiLatentAttentionParam the reference accepts but this library rejects at creation:
-    the prefill calcType, the int8 fractal-NZ cache mode, masks other than MASK_TYPE_SPEC, maskUseStatus."""
-    return (p.get("calcType", 0) == 4 or p.get("cacheMode", 0) == 2 or p.get("maskType", 0) >= 2 or
-            p.get("maskUseStatusType", 0) != 0)
+    the int8 fractal-NZ cache mode, decode masks other than MASK_TYPE_SPEC, maskUseStatus."""
+    if p.get("calcType", 0) == 4:
+        return False
+    return p.get("cacheMode", 0) == 2 or p.get("maskType", 0) >= 2 or p.get("maskUseStatusType", 0) != 0
 
 
 def _make_param(binding, op, p):
@@ -121,7 +122,12 @@ def _run_case(binding, case, ctx):
                 qlens_index = lens_index + (2 if p.get("maskType", 0) != 0 else 1)
                 if qlens_index < len(case["in_shapes"]):
                     host[qlens_index] = np.ones((case["in_shapes"][qlens_index][0],), dtype=np.int32)
-        if case["op"] == "MultiLatentAttentionOperation" and len(case["in_shapes"]) > 5:
+        if case["op"] == "MultiLatentAttentionOperation" and case["param"].get("calcType", 0) == 4:
+            # prefill: qSeqLen and kvSeqLen are host tensors; one sequence that fills the query
+            for i in (5, 6):
+                if i < len(case["in_shapes"]) and len(case["in_shapes"][i]) == 1:
+                    host[i] = np.full((case["in_shapes"][i][0],), 1, dtype=np.int32)
+        elif case["op"] == "MultiLatentAttentionOperation" and len(case["in_shapes"]) > 5:
             host[5] = np.full((case["in_shapes"][5][0],), 7, dtype=np.int32)
             if case["param"].get("calcType", 0) in (1, 3):
                 host[len(case["in_shapes"]) - 1] = np.ones((case["in_shapes"][-1][0],), dtype=np.int32)
@@ -252,9 +258,10 @@ def test_table_coverage():
     rac_dev = [c for c in RAC_CASES if _rac_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
     assert len(PA_CASES) == 81 and len(PA_CASES) - len(pa_dev) >= 75
     assert len(RAC_CASES) == 38 and len(RAC_CASES) - len(rac_dev) >= 29
-    # most MultiLatentAttention rows exercise the prefill calcType and the int8 fractal-NZ cache, which are not built
+    # the MultiLatentAttention rows replayed as "rejected at creation" exercise the int8 fractal-NZ cache, the
+    # decode masks other than MASK_TYPE_SPEC and maskUseStatus
     mla_dev = [c for c in MLA_CASES if _mla_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
-    assert len(MLA_CASES) == 147 and len(MLA_CASES) - len(mla_dev) == 46
+    assert len(MLA_CASES) == 147 and len(MLA_CASES) - len(mla_dev) == 114
 
 
 def test_param_sizes(binding):
@@ -569,7 +576,7 @@ def test_multi_latent_attention_counts_shapes_and_setup(binding, ctx):
         assert op.ok and (op.input_num(), op.output_num()) == (n_in, n_out), kw
         op.close()
     for bad in (dict(headNum=12), dict(kvHeadNum=2), dict(cacheMode=0), dict(maskType=1), dict(qkScale=1.5),
-                dict(qkScale=0.0), dict(calcType=5), dict(cacheMode=2), dict(cacheMode=4), dict(calcType=4),
+                dict(qkScale=0.0), dict(calcType=5), dict(cacheMode=2), dict(cacheMode=4), dict(calcType=4, headNum=32),
                 dict(calcType=1, maskType=2), dict(calcType=1, maskType=3), dict(calcType=1, maskType=4),
                 dict(calcType=3, maskUseStatusType=1)):
         kw = dict(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1)
@@ -630,6 +637,85 @@ def test_multi_latent_attention_counts_shapes_and_setup(binding, ctx):
     assert spec.setup(pack(rows=6, mask=[6, 300], with_qlens=True, qlens_host=False), outs(rows=6), ctx)[0] == \
         e["ERROR_INVALID_PARAM"]
     spec.close()
+
+
+def test_multi_latent_attention_prefill_checks(binding, ctx):
+    """calcType PREFILL: creation rules (reference multi_latent_attention_operation.cpp:175-206), tensor counts
+    (:245-266), output shaped like the query (:268-283, :306-320), both key layouts (:718-737), lengths read from
+    hostData and equal per sequence (multi_latent_attention_ops_runner_prefill.cpp:98-110)."""
+    e = binding.ERROR_CODE
+    mk = binding.MultiLatentAttentionParam
+    base = dict(headNum=4, kvHeadNum=4, qkScale=0.07, cacheMode=1, calcType=4)
+    for kw, n_in in ((dict(), 7), (dict(maskType=2), 8), (dict(maskType=3), 7), (dict(maskType=4, windowSize=100), 8),
+                     (dict(maskType=3, kvHeadNum=2), 7), (dict(headNum=1, kvHeadNum=1), 7),
+                     (dict(headNum=128, kvHeadNum=128), 7)):
+        op = binding.Operation("MultiLatentAttentionOperation", mk(**dict(base, **kw)))
+        assert op.ok and (op.input_num(), op.output_num()) == (n_in, 1), kw
+        assert op.get_name() == "MultiLatentAttentionOperation"
+        op.close()
+    for bad in (dict(headNum=0, kvHeadNum=0), dict(headNum=129, kvHeadNum=129), dict(kvHeadNum=2), dict(maskType=1),
+                dict(cacheMode=3), dict(cacheMode=0), dict(maskType=4), dict(qkScale=2.0)):
+        assert binding.Operation("MultiLatentAttentionOperation", mk(**dict(base, **bad))).status == \
+            e["ERROR_INVALID_PARAM"], bad
+
+    q_lens = np.array([100, 0, 28], dtype=np.int32)
+    kv_lens = q_lens.copy()
+
+    def pack(q=(128, 4, 128), qr=(128, 4, 64), k=(128, 4, 128), kr=(128, 4, 64), v=(128, 4, 128), mask=None,
+             ql=q_lens, kl=kv_lens, dtype="float16", host=True):
+        ins = [binding.make_tensor(dtype, list(s), FAKE_DEVICE) for s in (q, qr, k, kr, v)]
+        ins.append(binding.make_tensor("int32", [len(ql)], FAKE_DEVICE, host_ptr=ql.ctypes.data if host else None))
+        ins.append(binding.make_tensor("int32", [len(kl)], FAKE_DEVICE, host_ptr=kl.ctypes.data if host else None))
+        if mask is not None:
+            ins.append(binding.make_tensor(dtype, list(mask), FAKE_DEVICE))
+        return ins
+
+    def out(shape=(128, 4, 128), dtype="float16"):
+        return [binding.make_tensor(dtype, list(shape), FAKE_DEVICE)]
+
+    op = binding.Operation("MultiLatentAttentionOperation", mk(**base))
+    st, descs = op.infer_shape(pack(dtype="bf16"))
+    assert st == 0 and [[d.dims[i] for i in range(d.dimNum)] for d in descs] == [[128, 4, 128]]
+    assert descs[0].dtype == binding.ACL_DTYPE_BY_NAME["bf16"]
+    st, ws = op.setup(pack(), out(), ctx)
+    assert st == 0 and ws == 2 * 32   # one block of 128 queries per non-empty sequence, 32 bytes each
+    # 2-dim query and output, keys padded per sequence as [batch, maxSeqLen, kvHeads * channels]
+    flat = dict(q=(128, 512), qr=(128, 256), k=(3, 100, 512), kr=(3, 100, 256), v=(3, 100, 512))
+    st, descs = op.infer_shape(pack(**flat))
+    assert st == 0 and [[d.dims[i] for i in range(d.dimNum)] for d in descs] == [[128, 512]]
+    assert op.setup(pack(**flat), out((128, 512)), ctx)[0] == 0
+    short = dict(flat, k=(3, 99, 512), kr=(3, 99, 256), v=(3, 99, 512))
+    assert op.setup(pack(**short), out((128, 512)), ctx)[0] == e["ERROR_INVALID_PARAM"]      # 100 keys in 99 rows
+    assert op.setup(pack(host=False), out(), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    assert op.setup(pack(kl=np.array([100, 0, 27], dtype=np.int32)), out(), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    assert op.setup(pack(ql=np.array([100, 1, 28], dtype=np.int32), kl=np.array([100, 1, 28], dtype=np.int32)), out(),
+                    ctx)[0] == e["ERROR_INVALID_PARAM"]                                          # 129 rows of 128
+    assert op.setup(pack(), out((128, 4, 64)), ctx)[0] == e["ERROR_INVALID_TENSOR_DIM"]
+    assert op.setup(pack(), out((128, 512)), ctx)[0] == e["ERROR_INVALID_TENSOR_DIM_NUM"]
+    assert op.setup(pack(mask=(512, 512)), out(), ctx)[0] == e["ERROR_INVALID_IN_TENSOR_NUM"]
+    assert op.setup(pack(dtype="bf16"), out(), ctx)[0] == e["ERROR_INVALID_TENSOR_INI_MATCH"]
+    for bad in (dict(q=(128, 4, 127)), dict(qr=(128, 4, 32)), dict(qr=(127, 4, 64)), dict(k=(128, 3, 128)),
+                dict(kr=(128, 4, 32)), dict(v=(128, 4, 64)), dict(v=(127, 4, 128))):
+        assert op.setup(pack(**bad), out(), ctx)[0] == e["ERROR_INVALID_TENSOR_DIM"], bad
+    op.close()
+
+    free = binding.Operation("MultiLatentAttentionOperation", mk(**dict(base, maskType=2)))
+    assert free.setup(pack(mask=(512, 512)), out(), ctx)[0] == 0
+    assert free.setup(pack(mask=(512, 511)), out(), ctx)[0] == e["ERROR_INVALID_TENSOR_DIM"]
+    assert free.setup(pack(mask=(1, 512, 512)), out(), ctx)[0] == 0
+    assert free.setup(pack(), out(), ctx)[0] == e["ERROR_INVALID_IN_TENSOR_NUM"]
+    free.close()
+    # CAUSAL_MASK takes no mask tensor, keys only in the padded layout, and may group query heads over KV heads
+    causal = binding.Operation("MultiLatentAttentionOperation", mk(**dict(base, maskType=3, kvHeadNum=2)))
+    padded = dict(k=(3, 100, 256), kr=(3, 100, 128), v=(3, 100, 256))
+    assert causal.setup(pack(**padded), out(), ctx)[0] == 0
+    assert causal.setup(pack(k=(128, 2, 128), kr=(128, 2, 64), v=(128, 2, 128)), out(), ctx)[0] == \
+        e["ERROR_INVALID_TENSOR_DIM"]
+    causal.close()
+    swa = binding.Operation("MultiLatentAttentionOperation", mk(**dict(base, maskType=4, windowSize=50)))
+    assert swa.setup(pack(mask=(100, 100)), out(), ctx)[0] == 0
+    assert swa.setup(pack(mask=(99, 100)), out(), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    swa.close()
 
 
 def test_multi_latent_attention_nz_cache_checks(binding, ctx):

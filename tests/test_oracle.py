@@ -939,6 +939,80 @@ def test_fractal_nz_layout_by_flat_addresses_and_round_trip(oracle, n0):
         oracle.nd_to_nz(x[:, :8], n0)
 
 
+def _prefill_case(rng, q_lens, kv_lens, heads, kv_heads):
+    tq, tk = int(sum(q_lens)), int(sum(kv_lens))
+    mk = lambda *shape: rng.standard_normal(shape).astype(np.float32)
+    return mk(tq, heads, 128), mk(tq, heads, 64), mk(tk, kv_heads, 128), mk(tk, kv_heads, 64), mk(tk, kv_heads, 128)
+
+
+@pytest.mark.parametrize("mask", ["none", "causal", "window"])
+def test_mla_prefill_matches_torch_sdpa_per_sequence(oracle, mask):
+    """Every sequence and head on its own through torch's scaled_dot_product_attention over the concatenated
+    128 + 64 channels: no mask, is_causal, and an explicit boolean band for the window."""
+    rng = _rng(130)
+    lens = [37, 1, 0, 64, 130]
+    heads, window = 3, 20
+    qn, qr, kn, kr, v = _prefill_case(rng, lens, lens, heads, heads)
+    got = oracle.mla_prefill(qn, qr, kn, kr, v, lens, lens, 0.11, mask=mask, window=window)
+    assert got.shape == (sum(lens), heads, 128)
+    pos = 0
+    for n in lens:
+        if n == 0:
+            continue
+        q = torch.from_numpy(np.concatenate([qn[pos:pos + n], qr[pos:pos + n]], -1)).permute(1, 0, 2).double()
+        k = torch.from_numpy(np.concatenate([kn[pos:pos + n], kr[pos:pos + n]], -1)).permute(1, 0, 2).double()
+        vv = torch.from_numpy(v[pos:pos + n]).permute(1, 0, 2).double()
+        if mask == "none":
+            want = torch.nn.functional.scaled_dot_product_attention(q, k, vv, scale=0.11)
+        elif mask == "causal":
+            want = torch.nn.functional.scaled_dot_product_attention(q, k, vv, is_causal=True, scale=0.11)
+        else:
+            i, j = torch.arange(n)[:, None], torch.arange(n)[None, :]
+            want = torch.nn.functional.scaled_dot_product_attention(q, k, vv, attn_mask=(j <= i) & (j > i - window),
+                                                                    scale=0.11)
+        np.testing.assert_allclose(got[pos:pos + n], want.permute(1, 0, 2).numpy(), rtol=2e-5, atol=2e-5)
+        pos += n
+
+
+def test_mla_prefill_closed_forms_grouping_and_padded_keys(oracle):
+    rng = _rng(131)
+    lens = [5, 9]
+    qn, qr, kn, kr, v = _prefill_case(rng, lens, lens, 4, 2)
+    # a window of one key: every query sees only its own position
+    one = oracle.mla_prefill(qn, qr, kn, kr, v, lens, lens, 0.3, mask="window", window=1)
+    for h in range(4):
+        np.testing.assert_allclose(one[:, h], v[:, h // 2], rtol=1e-6, atol=1e-6)
+    # causal: the first query of a sequence sees one key; the last one sees them all, like an unmasked query
+    causal = oracle.mla_prefill(qn, qr, kn, kr, v, lens, lens, 0.3, mask="causal")
+    plain = oracle.mla_prefill(qn, qr, kn, kr, v, lens, lens, 0.3)
+    np.testing.assert_allclose(causal[0, 3], v[0, 1], rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(causal[5, 0], v[5, 0], rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(causal[4], plain[4], rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(causal[13], plain[13], rtol=1e-6, atol=1e-6)
+    # query head h reads KV head h // 2: the same as replicated KV heads
+    rep = oracle.mla_prefill(qn, qr, np.repeat(kn, 2, 1), np.repeat(kr, 2, 1), np.repeat(v, 2, 1), lens, lens, 0.3,
+                             mask="causal")
+    assert np.array_equal(rep, causal)
+    # a float64 loop over one (query, head): softmax over the visible keys of the 192 channels
+    b0, i, h = 5, 6, 2
+    sc = np.array([0.3 * (np.dot(qn[b0 + i, h].astype(np.float64), kn[b0 + j, 1]) +
+                          np.dot(qr[b0 + i, h].astype(np.float64), kr[b0 + j, 1])) for j in range(i + 1)])
+    w = np.exp(sc - sc.max())
+    w /= w.sum()
+    np.testing.assert_allclose(causal[b0 + i, h], (w[:, None] * v[b0:b0 + i + 1, 1]).sum(0), rtol=1e-5, atol=1e-5)
+    # keys padded per sequence to 12 rows, garbage in the padding
+    pad = lambda t: np.concatenate([np.concatenate([t[:5], np.full((7,) + t.shape[1:], np.nan, np.float32)]),
+                                    np.concatenate([t[5:], np.full((3,) + t.shape[1:], np.nan, np.float32)])])
+    padded = oracle.mla_prefill(qn, qr, pad(kn), pad(kr), pad(v), lens, lens, 0.3, mask="causal", kv_padded_rows=12)
+    assert np.array_equal(padded, causal)
+    # more keys than queries without a mask: every query sees them all
+    qn2, qr2, kn2, kr2, v2 = _prefill_case(rng, [2], [7], 1, 1)
+    cross = oracle.mla_prefill(qn2, qr2, kn2, kr2, v2, [2], [7], 1.0)
+    sc = np.concatenate([qn2[1, 0], qr2[1, 0]]) @ np.concatenate([kn2[:, 0], kr2[:, 0]], -1).T
+    w = np.exp(sc - sc.max())
+    np.testing.assert_allclose(cross[1, 0], (w / w.sum()) @ v2[:, 0], rtol=1e-5, atol=1e-5)
+
+
 def test_q_scale_rounds_in_query_dtype(oracle):
     rng = _rng(13)
     q, kc, vc, tables, ctx = _paged_case(rng)
