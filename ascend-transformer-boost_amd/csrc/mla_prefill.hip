@@ -5,9 +5,11 @@
 //
 // A workgroup owns 128 consecutive queries of one sequence and one head: four waves of 32 queries each
 // walk the keys the block may see in 32-token steps over tiles that the workgroup stages in LDS once.
-//   HBM -> VGPR -> LDS : K rows (128 + 64 channels from two tensors) and V rows of the next step are
-//                        requested before this step's arithmetic and written after it (two tile buffers,
-//                        one barrier per step);
+//   HBM -> LDS         : global_load_lds_dwordx4, no staging registers: wave w moves rows 8 w .. 8 w + 7 of
+//                        the K tile (128 + 64 channels from two tensors) and of the V tile with seven
+//                        transfers; three tile buffers, the tile two steps ahead is requested before this
+//                        step's arithmetic (a step is shorter than a round trip to L2 or HBM), one barrier
+//                        per step;
 //   S^T = K . Q^T      : v_mfma_f32_32x32x16, K from LDS as A (ds_read_b128), Q^T resident in registers as B;
 //                        lane (n, kh) then holds 16 tokens of query n: 8 (e / 4) + 4 kh + e % 4;
 //   softmax            : base 2, online; the row maximum needs one exchange between lanes n and n + 32;
@@ -15,12 +17,17 @@
 //                        half-step kb is token 16 kb + 8 (e / 4) + 4 kh + e % 4), V^T comes from the
 //                        row-major tile through the transposing ds_read_b64_tr_b16.
 // Steps that a mask hides completely are not visited (causal: keys past the block's last query; window:
-// keys before the first query's window); inside a visited step hidden scores are -inf.
+// keys before the first query's window); inside a visited step hidden scores are -inf. Tile rows past the
+// end of a sequence repeat its last row: their scores are hidden and their value rows finite.
+//
+// The transfers are inline assembly, so the compiler neither sees their LDS writes nor counts them: every
+// wait for them is written out (vmcnt counts loads in issue order; the loop issues no other load), and the
+// barrier that follows a wait makes the landed rows of all four waves visible to all.
 #include <algorithm>
 #include <mutex>
 #include <vector>
 #include <cstring>
-#include "atbmi_common.h"
+#include "pa_internal.h"
 
 namespace atbmi {
 namespace prefill {
@@ -47,10 +54,17 @@ constexpr int V_PITCH = DV * 2 + 64;  // 320 bytes: four rows x 64 bytes of one 
 constexpr int K_TILE = STEP * K_PITCH;
 constexpr int V_TILE = STEP * V_PITCH;
 constexpr int BUF = K_TILE + V_TILE;
-constexpr int LDS_BYTES = 2 * BUF;
-constexpr int K_PIECES = STEP * (D / 8) / (NWAVES * WAVE);  // 16-byte pieces of a K tile per thread
-constexpr int V_PIECES = STEP * (DV / 8) / (NWAVES * WAVE);
-static_assert(K_PIECES == 3 && V_PIECES == 2 && LDS_BYTES == 46080, "tile staging assumes these sizes");
+constexpr int NBUF = 3;
+constexpr int LDS_BYTES = NBUF * BUF;
+// A transfer fills 64 consecutive 16-byte slots of LDS, one per lane. A wave's 8 rows are 200 slots of the K
+// tile (25 a row, the last one padding) and 160 of the V tile (20 a row, four of them padding).
+constexpr int ROWS_PER_WAVE = STEP / NWAVES;
+constexpr int K_SLOTS = K_PITCH / 16;
+constexpr int V_SLOTS = V_PITCH / 16;
+constexpr int K_DMA = (ROWS_PER_WAVE * K_SLOTS + WAVE - 1) / WAVE;
+constexpr int V_DMA = (ROWS_PER_WAVE * V_SLOTS + WAVE - 1) / WAVE;
+constexpr int DMA_PER_TILE = K_DMA + V_DMA;
+static_assert(K_DMA == 4 && V_DMA == 3 && LDS_BYTES == 69120, "the waits below count seven transfers a tile");
 
 // One block of queries: rows [qRow0, qRow0 + nQ) of the query tensors, positions [qPos0, qPos0 + nQ) of
 // a sequence whose keys are rows [kRow0, kRow0 + kvLen) of the key / value tensors.
@@ -71,6 +85,7 @@ struct Args {
     const void *v;
     void *out;
     const Item *items;
+    int32_t numItems;
     int32_t H;
     int32_t G;
     int32_t group;   // H / G
@@ -106,16 +121,34 @@ __device__ __forceinline__ float Exp2(float x)
     return __builtin_amdgcn_exp2f(x);
 }
 
-template <bool BF16> __global__ __launch_bounds__(NWAVES *WAVE) void MlaPrefillKernel(const Args a)
+// 16 bytes per active lane from `src` to LDS address ldsBase + 16 x lane (ldsBase wave-uniform).
+__device__ __forceinline__ void TransferToLds(uint32_t ldsBase, const void *src)
 {
-    __shared__ __attribute__((aligned(16))) unsigned char smem[LDS_BYTES];
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(ldsBase), "v"(src)
+                 : "memory", "m0");
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(NWAVES *WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) void MlaPrefillKernel(const Args a)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x;
     const int lane = tid & (WAVE - 1);
-    const int wave = tid / WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
     const int n = lane & 31;  // query column of this lane
     const int kh = lane >> 5; // which half of an MFMA's contraction values this lane holds
-    const Item it = a.items[blockIdx.x / a.H];
-    const int h = blockIdx.x % a.H;
+    // Workgroups go to the 8 XCDs round-robin, and every XCD has an L2 of its own: XCD x takes the x-th
+    // eighth of the work list, which runs head by head, sequence by sequence, query block by query block, so
+    // that the blocks of one (sequence, head) pair, which read the same keys, run side by side on one XCD.
+    const int chunk = gridDim.x / 8;
+    const int work = (blockIdx.x % 8) * chunk + blockIdx.x / 8;
+    if (work >= a.numItems * a.H) {
+        return;
+    }
+    const int h = work / a.numItems;
+    const Item it = a.items[work % a.numItems];
     const int g = h / a.group;
 
     const int qLocal = wave * QW + n;
@@ -124,6 +157,69 @@ template <bool BF16> __global__ __launch_bounds__(NWAVES *WAVE) void MlaPrefillK
     const bool waveHasWork = wave * QW < it.nQ;
     const int qFirstW = it.qPos0 + wave * QW;                       // first and last query position of this wave
     const int qLastW = it.qPos0 + min(it.nQ, wave * QW + QW) - 1;
+
+    // ---- the keys this block visits
+    int tBegin = 0;
+    int tEnd = it.kvLen;
+    if (a.mask != ATBMI_MLA_PREFILL_MASK_NONE) {
+        tEnd = min(tEnd, it.qPos0 + it.nQ);
+    }
+    if (a.mask == ATBMI_MLA_PREFILL_MASK_WINDOW) {
+        tBegin = max(0, it.qPos0 - a.window + 1) & ~(STEP - 1);
+    }
+    const int numTiles = tEnd > tBegin ? (tEnd - tBegin + STEP - 1) / STEP : 0;
+
+    // ---- sources of this lane's slot in each of the wave's seven transfers: the address of its piece in
+    // row 0 of the tensor, the bytes between rows of that tensor, and the slot's row inside the wave's eight
+    const unsigned char *srcBase[DMA_PER_TILE];
+    uint32_t srcStride[DMA_PER_TILE];
+    uint32_t srcRows = 0; // 3 bits per transfer
+#pragma unroll
+    for (int i = 0; i < K_DMA; ++i) {
+        const int slot = min(i * WAVE + lane, ROWS_PER_WAVE * K_SLOTS - 1);
+        const int row = slot / K_SLOTS;
+        const int piece = min(slot % K_SLOTS, D / 8 - 1);
+        const bool rope = piece >= DN / 8;
+        srcBase[i] = rope ? reinterpret_cast<const unsigned char *>(a.kRope) + (g * DR + (piece - DN / 8) * 8) * 2
+                          : reinterpret_cast<const unsigned char *>(a.k) + (g * DN + piece * 8) * 2;
+        srcStride[i] = static_cast<uint32_t>(a.G) * (rope ? DR * 2 : DN * 2);
+        srcRows |= static_cast<uint32_t>(row) << (3 * i);
+    }
+#pragma unroll
+    for (int i = 0; i < V_DMA; ++i) {
+        const int slot = min(i * WAVE + lane, ROWS_PER_WAVE * V_SLOTS - 1);
+        const int row = slot / V_SLOTS;
+        const int piece = min(slot % V_SLOTS, DV / 8 - 1);
+        srcBase[K_DMA + i] = reinterpret_cast<const unsigned char *>(a.v) + (g * DV + piece * 8) * 2;
+        srcStride[K_DMA + i] = static_cast<uint32_t>(a.G) * (DV * 2);
+        srcRows |= static_cast<uint32_t>(row) << (3 * (K_DMA + i));
+    }
+    const uint32_t ldsBase = static_cast<uint32_t>(
+        reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char *)smem));
+    const uint32_t ldsWaveK = ldsBase + wave * (ROWS_PER_WAVE * K_PITCH);
+    const uint32_t ldsWaveV = ldsBase + K_TILE + wave * (ROWS_PER_WAVE * V_PITCH);
+    // Requests this wave's rows of the tile at key t into tile buffer `buf`: seven transfers, always.
+    auto requestTile = [&](int t, int buf) {
+        const int row0 = t + wave * ROWS_PER_WAVE;
+#pragma unroll
+        for (int i = 0; i < DMA_PER_TILE; ++i) {
+            const int row = min(row0 + static_cast<int>((srcRows >> (3 * i)) & 7u), it.kvLen - 1);
+            const unsigned char *src = srcBase[i] + static_cast<uint64_t>(it.kRow0 + row) * srcStride[i];
+            const bool isK = i < K_DMA;
+            const int j = isK ? i : i - K_DMA;
+            const uint32_t dst = (isK ? ldsWaveK : ldsWaveV) + static_cast<uint32_t>(buf * BUF + j * (WAVE * 16));
+            const int slots = isK ? ROWS_PER_WAVE * K_SLOTS : ROWS_PER_WAVE * V_SLOTS;
+            if (j * WAVE + lane < slots) {
+                TransferToLds(__builtin_amdgcn_readfirstlane(dst), src);
+            }
+        }
+    };
+    if (numTiles > 0) {
+        requestTile(tBegin, 0);
+    }
+    if (numTiles > 1) {
+        requestTile(tBegin + STEP, 1);
+    }
 
     // ---- Q^T as B operand: lane (n, kh) holds q[n][16 j + 8 kh .. +8) for the 12 pieces j
     u32x4 qreg[D / 16];
@@ -139,60 +235,6 @@ template <bool BF16> __global__ __launch_bounds__(NWAVES *WAVE) void MlaPrefillK
             }
         }
     }
-
-    // ---- the keys this block visits
-    int tBegin = 0;
-    int tEnd = it.kvLen;
-    if (a.mask != ATBMI_MLA_PREFILL_MASK_NONE) {
-        tEnd = min(tEnd, it.qPos0 + it.nQ);
-    }
-    if (a.mask == ATBMI_MLA_PREFILL_MASK_WINDOW) {
-        tBegin = max(0, it.qPos0 - a.window + 1) & ~(STEP - 1);
-    }
-
-    const unsigned char *kBase = reinterpret_cast<const unsigned char *>(a.k);
-    const unsigned char *krBase = reinterpret_cast<const unsigned char *>(a.kRope);
-    const unsigned char *vBase = reinterpret_cast<const unsigned char *>(a.v);
-    u32x4 kStage[K_PIECES];
-    u32x4 vStage[V_PIECES];
-    // Requests this thread's pieces of the tile at key t (rows at or past kvLen read as zeros).
-    auto loadTile = [&](int t) {
-#pragma unroll
-        for (int i = 0; i < K_PIECES; ++i) {
-            const int p = tid + i * NWAVES * WAVE;
-            const int row = p / (D / 8);
-            const int col = p % (D / 8);
-            kStage[i] = u32x4{0u, 0u, 0u, 0u};
-            if (t + row < it.kvLen) {
-                const int64_t rg = (static_cast<int64_t>(it.kRow0) + t + row) * a.G + g;
-                kStage[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(
-                    col < DN / 8 ? kBase + rg * (DN * 2) + col * 16 : krBase + rg * (DR * 2) + (col - DN / 8) * 16));
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < V_PIECES; ++i) {
-            const int p = tid + i * NWAVES * WAVE;
-            const int row = p / (DV / 8);
-            const int col = p % (DV / 8);
-            vStage[i] = u32x4{0u, 0u, 0u, 0u};
-            if (t + row < it.kvLen) {
-                const int64_t rg = (static_cast<int64_t>(it.kRow0) + t + row) * a.G + g;
-                vStage[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(vBase + rg * (DV * 2) + col * 16));
-            }
-        }
-    };
-    auto storeTile = [&](unsigned char *buf) {
-#pragma unroll
-        for (int i = 0; i < K_PIECES; ++i) {
-            const int p = tid + i * NWAVES * WAVE;
-            *reinterpret_cast<u32x4 *>(buf + (p / (D / 8)) * K_PITCH + (p % (D / 8)) * 16) = kStage[i];
-        }
-#pragma unroll
-        for (int i = 0; i < V_PIECES; ++i) {
-            const int p = tid + i * NWAVES * WAVE;
-            *reinterpret_cast<u32x4 *>(buf + K_TILE + (p / (DV / 8)) * V_PITCH + (p % (DV / 8)) * 16) = vStage[i];
-        }
-    };
 
     float m = -INFINITY; // running maximum of query n, base-2 exponent units
     float l = 0.0f;      // this lane's share of the running denominator
@@ -215,21 +257,28 @@ template <bool BF16> __global__ __launch_bounds__(NWAVES *WAVE) void MlaPrefillK
         for (int e = 0; e < 16; ++e) {
             s[e] = 0.0f;
         }
+        // K operands are requested four pieces ahead of the MFMA that takes them
+        constexpr int AHEAD = 4;
+        u32x4 kk[AHEAD];
+#pragma unroll
+        for (int j = 0; j < AHEAD; ++j) {
+            kk[j] = *reinterpret_cast<const u32x4 *>(buf + kOperand + j * 32);
+        }
 #pragma unroll
         for (int j = 0; j < D / 16; ++j) {
-            const u32x4 kk = *reinterpret_cast<const u32x4 *>(buf + kOperand + j * 32);
-            s = Mma<BF16>(kk, qreg[j], s);
+            s = Mma<BF16>(kk[j % AHEAD], qreg[j], s);
+            if (j + AHEAD < D / 16) {
+                kk[j % AHEAD] = *reinterpret_cast<const u32x4 *>(buf + kOperand + (j + AHEAD) * 32);
+            }
         }
         // every key of the step visible to every query of the wave: no comparisons
         const bool open = t + STEP <= it.kvLen &&
                           (a.mask == ATBMI_MLA_PREFILL_MASK_NONE ||
                            (t + STEP - 1 <= qFirstW &&
                             (a.mask != ATBMI_MLA_PREFILL_MASK_WINDOW || t > qLastW - a.window)));
-        float mLoc = -INFINITY;
+        if (!open) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            float x = s[e] * a.scale2;
-            if (!open) {
+            for (int e = 0; e < 16; ++e) {
                 const int tok = t + 8 * (e >> 2) + 4 * kh + (e & 3);
                 bool hidden = tok >= it.kvLen;
                 if (a.mask != ATBMI_MLA_PREFILL_MASK_NONE) {
@@ -238,12 +287,18 @@ template <bool BF16> __global__ __launch_bounds__(NWAVES *WAVE) void MlaPrefillK
                 if (a.mask == ATBMI_MLA_PREFILL_MASK_WINDOW) {
                     hidden = hidden || tok <= qPos - a.window;
                 }
-                x = hidden ? -INFINITY : x;
+                s[e] = hidden ? -INFINITY : s[e];
             }
-            s[e] = x;
-            mLoc = fmaxf(mLoc, x);
         }
-        mLoc = fmaxf(mLoc, __shfl_xor(mLoc, 32));
+        // the maximum is taken over the raw scores (the scale is positive) and the scale multiplies inside the
+        // exponent's fused multiply-add
+        float mLoc = fmaxf(fmaxf(s[0], s[1]), s[2]);
+#pragma unroll
+        for (int e = 3; e < 15; e += 2) {
+            mLoc = fmaxf(fmaxf(mLoc, s[e]), s[e + 1]);
+        }
+        mLoc = fmaxf(mLoc, s[15]);
+        mLoc = fmaxf(mLoc, __shfl_xor(mLoc, 32)) * a.scale2;
         const float mNew = fmaxf(m, mLoc);
         const float mRef = mNew == -INFINITY ? 0.0f : mNew; // nothing visible so far: every weight is 0
         const float corr = Exp2(m - mRef);
@@ -251,7 +306,7 @@ template <bool BF16> __global__ __launch_bounds__(NWAVES *WAVE) void MlaPrefillK
         float sum = 0.0f;
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            s[e] = Exp2(s[e] - mRef);
+            s[e] = Exp2(__builtin_fmaf(s[e], a.scale2, -mRef));
             sum += s[e];
         }
         l = l * corr + sum;
@@ -272,31 +327,43 @@ template <bool BF16> __global__ __launch_bounds__(NWAVES *WAVE) void MlaPrefillK
                 pop[kb][w] = Pack2<BF16>(s[8 * kb + 2 * w], s[8 * kb + 2 * w + 1]);
             }
         }
+        auto readV = [&](int idx) -> u32x4 { // V^T operand of output tile idx / 2, half-step idx % 2
+            const unsigned char *vp = buf + vOperand + (idx & 1) * 16 * V_PITCH + (idx >> 1) * 64;
+            const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4 *)(vp));
+            const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) i16x4 *)(vp + 8 * V_PITCH));
+            const u32x2 lo2 = __builtin_bit_cast(u32x2, lo);
+            const u32x2 hi2 = __builtin_bit_cast(u32x2, hi);
+            return u32x4{lo2[0], lo2[1], hi2[0], hi2[1]};
+        };
+        constexpr int NV = 2 * (DV / 32);
+        u32x4 vv[AHEAD];
 #pragma unroll
-        for (int i = 0; i < DV / 32; ++i) {
+        for (int i = 0; i < AHEAD; ++i) {
+            vv[i] = readV(i);
+        }
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                const unsigned char *vp = buf + vOperand + kb * 16 * V_PITCH + i * 64;
-                const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4 *)(vp));
-                const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (__attribute__((address_space(3))) i16x4 *)(vp + 8 * V_PITCH));
-                const u32x2 lo2 = __builtin_bit_cast(u32x2, lo);
-                const u32x2 hi2 = __builtin_bit_cast(u32x2, hi);
-                acc[i] = Mma<BF16>(u32x4{lo2[0], lo2[1], hi2[0], hi2[1]}, pop[kb], acc[i]);
+        for (int i = 0; i < NV; ++i) {
+            acc[i >> 1] = Mma<BF16>(vv[i % AHEAD], pop[i & 1], acc[i >> 1]);
+            if (i + AHEAD < NV) {
+                vv[i % AHEAD] = readV(i + AHEAD);
             }
         }
     };
 
-    if (tBegin < tEnd) {
-        loadTile(tBegin);
-        storeTile(smem);
-    }
-    __syncthreads();
-    int cur = 0;
-    for (int t = tBegin; t < tEnd; t += STEP) {
-        const bool more = t + STEP < tEnd;
-        if (more) {
-            loadTile(t + STEP);
+    int buf = 0;
+    for (int i = 0; i < numTiles; ++i) {
+        const int t = tBegin + i * STEP;
+        // this wave's rows of tile i have landed (the transfers of tile i + 1 may still be on their way) ...
+        if (i + 1 < numTiles) {
+            asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        // ... and so have everybody else's, and everybody has left tile i - 1, whose buffer tile i + 2 takes
+        __syncthreads();
+        if (i + 2 < numTiles) {
+            requestTile(t + 2 * STEP, buf == 0 ? 2 : buf - 1);
         }
         // a wave skips the steps that its own queries cannot see
         bool visit = waveHasWork;
@@ -307,13 +374,9 @@ template <bool BF16> __global__ __launch_bounds__(NWAVES *WAVE) void MlaPrefillK
             visit = visit && t + STEP - 1 > qFirstW - a.window;
         }
         if (visit) {
-            computeStep(t, smem + cur * BUF);
+            computeStep(t, smem + buf * BUF);
         }
-        if (more) {
-            storeTile(smem + (cur ^ 1) * BUF);
-        }
-        __syncthreads();
-        cur ^= 1;
+        buf = buf == NBUF - 1 ? 0 : buf + 1;
     }
 
     // ---- out[q][h][32 i + 8 r + 4 kh .. +4) = acc / l
@@ -377,7 +440,7 @@ int Upload(const void *src, size_t bytes, void *dst, hipStream_t stream)
     return OK;
 }
 
-// Checks the call and lists its query blocks, longest key walk first.
+// Checks the call and lists its query blocks.
 int BuildItems(const AtbmiMlaPrefillCall *c, std::vector<Item> *items)
 {
     if (!c || !c->hostQLens || !c->hostKvLens) {
@@ -420,7 +483,9 @@ int BuildItems(const AtbmiMlaPrefillCall *c, std::vector<Item> *items)
         if (qRow + nq > 0x7fffffffLL || kRow + nk > 0x7fffffffLL) {
             return Fail(ERR_INVALID_PARAM, "mla_prefill: more than 2^31 rows");
         }
-        for (int32_t q0 = 0; q0 < nq; q0 += QB) {
+        // the blocks of a sequence follow each other, the one that walks the most keys (under a mask: the
+        // last one) first
+        for (int32_t q0 = (nq - 1) / QB * QB; nq > 0 && q0 >= 0; q0 -= QB) {
             Item it{};
             it.qRow0 = static_cast<int32_t>(qRow + q0);
             it.nQ = nq - q0 < QB ? nq - q0 : QB;
@@ -433,12 +498,6 @@ int BuildItems(const AtbmiMlaPrefillCall *c, std::vector<Item> *items)
         }
         qRow += nq;
         kRow += nk;
-    }
-    if (items && c->mask != ATBMI_MLA_PREFILL_MASK_NONE) {
-        // blocks late in a sequence walk the most keys: start them first
-        std::stable_sort(items->begin(), items->end(), [](const Item &x, const Item &y) { return x.qPos0 > y.qPos0; });
-    } else if (items) {
-        std::stable_sort(items->begin(), items->end(), [](const Item &x, const Item &y) { return x.kvLen > y.kvLen; });
     }
     return OK;
 }
@@ -481,7 +540,7 @@ extern "C" int atbmi_mla_prefill(const AtbmiMlaPrefillCall *call, void *workspac
         return Fail(ERR_INVALID_PARAM, "mla_prefill: workspace of %llu bytes, %llu needed",
                     (unsigned long long)workspaceBytes, (unsigned long long)bytes);
     }
-    const int64_t grid = static_cast<int64_t>(items.size()) * call->numHeads;
+    const int64_t grid = (static_cast<int64_t>(items.size()) * call->numHeads + 7) / 8 * 8;
     if (grid > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "mla_prefill: %lld workgroups", (long long)grid);
     }
@@ -498,17 +557,19 @@ extern "C" int atbmi_mla_prefill(const AtbmiMlaPrefillCall *call, void *workspac
     a.v = call->value;
     a.out = call->out;
     a.items = static_cast<const prefill::Item *>(workspaceDevice);
+    a.numItems = static_cast<int32_t>(items.size());
     a.H = call->numHeads;
     a.G = call->numKvHeads;
     a.group = call->numHeads / call->numKvHeads;
     a.mask = call->mask;
     a.window = call->windowSize;
     a.scale2 = call->qkScale * 1.4426950408889634f;
-    if (call->dtype == ATBMI_BF16) {
-        prefill::MlaPrefillKernel<true><<<static_cast<unsigned>(grid), prefill::NWAVES * WAVE, 0, s>>>(a);
-    } else {
-        prefill::MlaPrefillKernel<false><<<static_cast<unsigned>(grid), prefill::NWAVES * WAVE, 0, s>>>(a);
+    auto kernel = call->dtype == ATBMI_BF16 ? prefill::MlaPrefillKernel<true> : prefill::MlaPrefillKernel<false>;
+    rc = ConfigureKernelLds(reinterpret_cast<const void *>(kernel), prefill::LDS_BYTES);
+    if (rc != OK) {
+        return rc;
     }
+    kernel<<<static_cast<unsigned>(grid), prefill::NWAVES * WAVE, prefill::LDS_BYTES, s>>>(a);
     ATBMI_HIP_CHECK(hipGetLastError());
     return OK;
 }
