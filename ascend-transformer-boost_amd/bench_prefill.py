@@ -6,7 +6,7 @@ call). The kernel is bound by the matrix cores: `roofline.achieved` is the algor
 per visible (query, key) pair and head) over the mean time of a call between HIP events on the launch stream,
 against the dense bf16 MFMA peak.
 
-    python3 ascend-transformer-boost_amd/bench_prefill.py [--steps 20] [--warmup 3]
+    python3 ascend-transformer-boost_amd/bench_prefill.py [--steps 20] [--warmup 3] [--only INDEX]
 """
 import argparse
 import importlib
@@ -44,6 +44,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--only", type=int, default=None, help="time only the workload with this index")
     args = ap.parse_args()
     import torch
     pkg = importlib.import_module(os.path.basename(HERE))
@@ -54,7 +55,7 @@ def main():
     stream = torch.cuda.Stream(device=dev)
     ctx = b.Context(stream)
     scale = 1.0 / (192.0 ** 0.5)
-    for name, lens, heads, mask_type, window in WORKLOADS:
+    for name, lens, heads, mask_type, window in (WORKLOADS if args.only is None else [WORKLOADS[args.only]]):
         tokens, longest = sum(lens), max(lens)
         with torch.cuda.stream(stream):
             mk = lambda *shape: (torch.randn(shape, device=dev) * 0.5).to(torch.bfloat16)

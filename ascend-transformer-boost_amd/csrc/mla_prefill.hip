@@ -271,6 +271,15 @@ __global__ __launch_bounds__(NWAVES *WAVE) __attribute__((amdgpu_waves_per_eu(2,
                 kk[j % AHEAD] = *reinterpret_cast<const u32x4 *>(buf + kOperand + (j + AHEAD) * 32);
             }
         }
+        // keep that order: four reads, then one MFMA and one read in turn (the scheduler would otherwise
+        // hold only two reads in flight and wait for each pair)
+        __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
+#pragma unroll
+        for (int j = 0; j + AHEAD < D / 16; ++j) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 0);
         // every key of the step visible to every query of the wave: no comparisons
         const bool open = t + STEP <= it.kvLen &&
                           (a.mask == ATBMI_MLA_PREFILL_MASK_NONE ||
