@@ -824,17 +824,21 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
                    ATBMI_REGS_100_111("a"), ATBMI_REGS_112_255("a"), ATBMI_SREGS_36_69("s"));
 }
 
-// Grid and plan as the 128-head kernel of pa_mla_kernel.h: one wave range per workgroup, the head groups of
-// one range 8 workgroup ids apart.
+// One wave range per workgroup; the grid is a multiple of 8 x head groups.
 template <bool BF16, bool SPLIT, bool NZ>
 __global__ __launch_bounds__(NW *WAVE) void PaMlaAsmKernel(const PaArgs a, const PaStreamPlan p)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
-    const int octet = blockIdx.x / (8 * p.headGroups);
-    const int within = blockIdx.x % (8 * p.headGroups);
-    const int hgIdx = within / 8;
-    const int wr = octet * 8 + within % 8;
+    // Workgroups go to the 8 XCDs round-robin and every XCD has an L2 of its own. XCD x takes the x-th eighth
+    // of the ranges: consecutive ranges walk the same sequences, so the (three to five) ranges of a sequence
+    // fetch its 147 KB of query rows from HBM once and from their common L2 after that; the head groups of a
+    // range, which read the same cache rows, sit on one XCD as well.
+    const int perXcd = gridDim.x / (8 * p.headGroups);
+    const int xcd = blockIdx.x % 8;
+    const int slot = blockIdx.x / 8;
+    const int hgIdx = slot % p.headGroups;
+    const int wr = xcd * perXcd + slot / p.headGroups;
     if (wr >= p.numWgRanges) {
         return;
     }
