@@ -200,6 +200,16 @@ class AtbmiMlaPrefillCall(ctypes.Structure):
 
 ATBMI_MLA_PREFILL_MASK_NONE, ATBMI_MLA_PREFILL_MASK_CAUSAL, ATBMI_MLA_PREFILL_MASK_WINDOW = 0, 1, 2
 
+
+class AtbmiMlaInt8Call(ctypes.Structure):
+    """One atbmi_mla_int8_decode call (include/atbmi_kernels.h)."""
+    _fields_ = [("outDtype", ctypes.c_int32), ("numHeads", ctypes.c_int32), ("blockSize", ctypes.c_int32),
+                ("numBlocks", ctypes.c_int32), ("maxBlocksPerSeq", ctypes.c_int32), ("batch", ctypes.c_int32),
+                ("numQueryRows", ctypes.c_int32), ("hasMask", ctypes.c_int32), ("maskLen", ctypes.c_int32),
+                ("qkScale", ctypes.c_float)] + [(n, ctypes.c_void_p) for n in (
+                    "hostContextLens", "hostQueryLens", "query", "queryRope", "kvCache", "kRopeCache", "blockTables",
+                    "qkDescale", "pvDescale", "mask", "out", "lse")]
+
 _kernels = None
 _atb = None
 
@@ -250,6 +260,8 @@ def kernels():
         lib.atbmi_pa_static_scratch_bytes.restype = u64
         lib.atbmi_mla_prefill_workspace_size.argtypes = [ctypes.POINTER(AtbmiMlaPrefillCall), ctypes.POINTER(u64)]
         lib.atbmi_mla_prefill.argtypes = [ctypes.POINTER(AtbmiMlaPrefillCall), vp, u64, vp]
+        lib.atbmi_mla_int8_workspace_size.argtypes = [ctypes.POINTER(AtbmiMlaInt8Call), ctypes.POINTER(u64)]
+        lib.atbmi_mla_int8_decode.argtypes = [ctypes.POINTER(AtbmiMlaInt8Call), vp, u64, vp]
         lib.atbmi_pa_plan_destroy.argtypes = [vp]
         lib.atbmi_pa_plan_destroy.restype = None
         lib.atbmi_timing_enable.argtypes = [i32]
@@ -475,7 +487,7 @@ class OperationRunner:
             st, descs = self.op.infer_shape(ins)
             if st != 0:
                 raise RuntimeError("InferShape failed: %s" % ERROR_NAMES[st])
-            rev = {ACL_FLOAT16: torch.float16, ACL_BF16: torch.bfloat16, ACL_INT8: torch.int8}
+            rev = {ACL_FLOAT16: torch.float16, ACL_BF16: torch.bfloat16, ACL_INT8: torch.int8, ACL_FLOAT: torch.float32}
             outputs = [torch.empty([d.dims[i] for i in range(d.dimNum)], dtype=rev[d.dtype], device=inputs[0].device)
                        for d in descs]
         outs = [tensor_of(t) for t in outputs]

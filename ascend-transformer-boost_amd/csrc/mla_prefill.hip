@@ -24,10 +24,9 @@
 // wait for them is written out (vmcnt counts loads in issue order; the loop issues no other load), and the
 // barrier that follows a wait makes the landed rows of all four waves visible to all.
 #include <algorithm>
-#include <mutex>
 #include <vector>
-#include <cstring>
 #include "pa_internal.h"
+#include "upload_ring.h"
 
 namespace atbmi {
 namespace prefill {
@@ -407,48 +406,6 @@ __global__ __launch_bounds__(NWAVES *WAVE) __attribute__((amdgpu_waves_per_eu(2,
     }
 }
 
-// Pinned staging for the asynchronous upload of the block list: a slot is reused only after the copy that
-// last read it has finished. One ring per process, taken under a lock for the length of a launch call.
-constexpr int RING = 4;
-struct UploadRing {
-    std::mutex lock;
-    void *pinned[RING] = {nullptr, nullptr, nullptr, nullptr};
-    size_t cap[RING] = {0, 0, 0, 0};
-    hipEvent_t copied[RING] = {nullptr, nullptr, nullptr, nullptr};
-    bool inFlight[RING] = {false, false, false, false};
-    int pos = 0;
-};
-UploadRing g_ring;
-
-int Upload(const void *src, size_t bytes, void *dst, hipStream_t stream)
-{
-    std::lock_guard<std::mutex> hold(g_ring.lock);
-    const int slot = g_ring.pos;
-    g_ring.pos = (g_ring.pos + 1) % RING;
-    if (g_ring.inFlight[slot]) {
-        ATBMI_HIP_CHECK(hipEventSynchronize(g_ring.copied[slot]));
-        g_ring.inFlight[slot] = false;
-    }
-    if (g_ring.cap[slot] < bytes) {
-        if (g_ring.pinned[slot]) {
-            ATBMI_HIP_CHECK(hipHostFree(g_ring.pinned[slot]));
-            g_ring.pinned[slot] = nullptr;
-            g_ring.cap[slot] = 0;
-        }
-        const size_t cap = (bytes * 2 + 4095) / 4096 * 4096;
-        ATBMI_HIP_CHECK(hipHostMalloc(&g_ring.pinned[slot], cap, hipHostMallocDefault));
-        g_ring.cap[slot] = cap;
-    }
-    if (!g_ring.copied[slot]) {
-        ATBMI_HIP_CHECK(hipEventCreateWithFlags(&g_ring.copied[slot], hipEventDisableTiming));
-    }
-    memcpy(g_ring.pinned[slot], src, bytes);
-    ATBMI_HIP_CHECK(hipMemcpyAsync(dst, g_ring.pinned[slot], bytes, hipMemcpyHostToDevice, stream));
-    ATBMI_HIP_CHECK(hipEventRecord(g_ring.copied[slot], stream));
-    g_ring.inFlight[slot] = true;
-    return OK;
-}
-
 // Checks the call and lists its query blocks.
 int BuildItems(const AtbmiMlaPrefillCall *c, std::vector<Item> *items)
 {
@@ -554,7 +511,7 @@ extern "C" int atbmi_mla_prefill(const AtbmiMlaPrefillCall *call, void *workspac
         return Fail(ERR_INVALID_PARAM, "mla_prefill: %lld workgroups", (long long)grid);
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    rc = prefill::Upload(items.data(), bytes, workspaceDevice, s);
+    rc = UploadTable(items.data(), bytes, workspaceDevice, s);
     if (rc != OK) {
         return rc;
     }

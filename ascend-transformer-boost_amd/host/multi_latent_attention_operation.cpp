@@ -13,15 +13,19 @@
 // fractal-NZ layout, [blocks, 512 / 16, 128, 16] and [blocks, 64 / 16, 128, 16];
 // reference :394-425 QKVDimCheckNz) with fp16/bf16 tensors; calcType UNDEFINED,
 // SPEC (qSeqlen, optionally with the MASK_TYPE_SPEC mask), RING and
-// SPEC_AND_RING (second output: log-sum-exp). calcType PREFILL is an operation
-// class of its own (multi_latent_attention_prefill_operation.cpp). The int8 NZ
-// cache mode, the MASK_FREE / CAUSAL_MASK masks of the decode calcTypes and
-// maskUseStatus are legal in the reference but not implemented here; such
-// params are rejected at creation with ERROR_INVALID_PARAM.
+// SPEC_AND_RING (second output: log-sum-exp). cacheMode INT8_NZCACHE (int8 query and
+// latent cache [blocks, 512 / 32, 128, 32] with a descale per head for the scores and
+// one for the values, the rotary parts 16-bit; reference :427-476, :493-511, :513-541)
+// runs on a kernel of its own (csrc/mla_int8.hip); its log-sum-exp output is fp32.
+// calcType PREFILL is an operation class of its own
+// (multi_latent_attention_prefill_operation.cpp). The MASK_FREE / CAUSAL_MASK masks
+// of the decode calcTypes and maskUseStatus are legal in the reference but not
+// implemented here; such params are rejected at creation with ERROR_INVALID_PARAM.
 //
 // The kernels are those of PagedAttention's combined-cache variant reading
 // each query and key row from two tensors.
 #include <new>
+#include <vector>
 #include "atb/infer_op_params.h"
 #include "atb/utils.h"
 #include "atbmi_kernels.h"
@@ -38,6 +42,7 @@ constexpr int64_t ROPE_DIM = 64;
 constexpr int64_t DECODER_BLOCK_SIZE = 128;
 constexpr int64_t MAX_BATCH = 8192;
 constexpr int64_t NZ_CHANNELS = 16; // channels of one fractal-NZ slab row (16-bit elements)
+constexpr int64_t NZ_CHANNELS_INT8 = 32;
 
 bool IsSpec(const Param &p)
 {
@@ -153,9 +158,7 @@ bool ImplementedCheck(const Param &p)
     if (p.calcType == Param::CALC_TYPE_PREFILL) {
         return true; // every param that passes ParamPrefillCheck is built
     }
-    if (p.cacheMode == Param::INT8_NZCACHE) {
-        what = "the int8 fractal-NZ cache";
-    } else if (p.maskType != Param::UNDEFINED && p.maskType != Param::MASK_TYPE_SPEC) {
+    if (p.maskType != Param::UNDEFINED && p.maskType != Param::MASK_TYPE_SPEC) {
         what = "this maskType";
     } else if (p.maskUseStatusType != Param::MASK_USE_STATUS_TYPE_UNDEFINED) {
         what = "maskUseStatus";
@@ -175,28 +178,37 @@ bool ImplementedCheck(const Param &p)
 // a table skips the check (reference operation_base.cpp:229-233): HasIr() says which.
 bool HasIr(const Param &p)
 {
+    if (p.cacheMode == Param::INT8_NZCACHE) {
+        // sections Int8Nz, IsRingInt8Nz and QlensIsRingInt8Nz (:6918-6945, :6741-6771, :6825-6858)
+        return !HasMaskInput(p) && (!IsSpec(p) || IsRing(p));
+    }
     return p.cacheMode != Param::NZCACHE || (!HasMaskInput(p) && !IsSpec(p) && !IsRing(p));
 }
 
 OpIr MakeIr(const Param &p)
 {
     OpIr ir;
-    const aclFormat cacheFormat = p.cacheMode == Param::NZCACHE ? ACL_FORMAT_FRACTAL_NZ : ACL_FORMAT_ND;
+    const bool int8 = p.cacheMode == Param::INT8_NZCACHE;
+    const aclFormat cacheFormat = p.cacheMode == Param::KROPE_CTKV ? ACL_FORMAT_ND : ACL_FORMAT_FRACTAL_NZ;
     for (aclDataType q : {ACL_FLOAT16, ACL_BF16}) {
         IrCombo c;
-        c.inDtypes = {q, q, q, q, ACL_INT32, ACL_INT32};
+        c.inDtypes = {int8 ? ACL_INT8 : q, q, int8 ? ACL_INT8 : q, q, ACL_INT32, ACL_INT32};
         if (HasMaskInput(p)) {
             c.inDtypes.push_back(q);
         }
         if (IsSpec(p)) {
             c.inDtypes.push_back(ACL_INT32);
         }
+        if (int8) {
+            c.inDtypes.push_back(ACL_FLOAT);
+            c.inDtypes.push_back(ACL_FLOAT);
+        }
         c.inFormats.assign(c.inDtypes.size(), ACL_FORMAT_ND);
         c.inFormats[KV_CACHE] = cacheFormat;
         c.inFormats[KV_CACHE_ROPE] = cacheFormat;
         c.outDtypes = {q};
         if (IsRing(p)) {
-            c.outDtypes.push_back(q);
+            c.outDtypes.push_back(int8 ? ACL_FLOAT : q);
         }
         c.outFormats.assign(c.outDtypes.size(), ACL_FORMAT_ND);
         ir.push_back(c);
@@ -222,6 +234,10 @@ public:
         if (IsSpec(param)) {
             qLensIdx_ = next++;
         }
+        if (param.cacheMode == Param::INT8_NZCACHE) {
+            descaleIdx_ = next;
+            next += 2; // qkDescale, pvDescale
+        }
         inputNum_ = static_cast<uint32_t>(next);
     }
 
@@ -243,6 +259,9 @@ protected:
         out.at(0).dtype = in.at(QUERY_ROPE).dtype;
         if (IsRing(param_)) {
             out.at(1) = out.at(0);
+            if (param_.cacheMode == Param::INT8_NZCACHE) {
+                out.at(1).dtype = ACL_FLOAT;
+            }
             out.at(1).shape.dims[2] = 1;
         }
         return NO_ERROR;
@@ -252,12 +271,30 @@ protected:
 
     Status SetupCheckImpl(const SVector<Tensor> &inTensors, const SVector<Tensor> &outTensors) const override
     {
-        (void)outTensors;
         SVector<TensorDesc> in;
         for (size_t i = 0; i < inTensors.size(); ++i) {
             in.push_back(inTensors.at(i).desc);
         }
-        return DimCheck(in);
+        Status st = DimCheck(in);
+        if (st != NO_ERROR) {
+            return st;
+        }
+        if (IsRing(param_) && param_.maskType == Param::UNDEFINED && param_.cacheMode == Param::INT8_NZCACHE) {
+            // reference :513-541
+            const Dims &q = inTensors.at(QUERY).desc.shape;
+            for (size_t i = 0; i < 2; ++i) {
+                const Dims &o = outTensors.at(i).desc.shape;
+                if (o.dimNum != q.dimNum) {
+                    ATB_LOG(ERROR) << "outputs should have as many dims as query";
+                    return ERROR_INVALID_TENSOR_DIM_NUM;
+                }
+                if (o.dims[0] != q.dims[0] || o.dims[1] != q.dims[1] || o.dims[2] != (i == 0 ? q.dims[2] : 1)) {
+                    ATB_LOG(ERROR) << "attenOut should be shaped like query, lse like query with a last dim of 1";
+                    return ERROR_INVALID_TENSOR_DIM;
+                }
+            }
+        }
+        return NO_ERROR;
     }
 
     Status PlanImpl(const VariantPack &pack, uint64_t &workspaceSize) override
@@ -313,6 +350,28 @@ protected:
             }
         }
 
+        if (param_.cacheMode == Param::INT8_NZCACHE) {
+            for (size_t i = descaleIdx_; i < descaleIdx_ + 2; ++i) {
+                const Dims &d = pack.inTensors.at(i).desc.shape;
+                if (d.dimNum != 1 || d.dims[0] != param_.headNum) {
+                    ATB_LOG(ERROR) << "qkDescale and pvDescale should be [headNum]";
+                    return ERROR_INVALID_PARAM;
+                }
+            }
+            lens_.assign(static_cast<const int32_t *>(lens.hostData), static_cast<const int32_t *>(lens.hostData) + batch);
+            qLens_.clear();
+            if (queryLens) {
+                qLens_.assign(queryLens, queryLens + batch);
+            }
+            maskLen_ = maskLen;
+            AtbmiMlaInt8Call call = MakeInt8Call(pack);
+            int rc = atbmi_mla_int8_workspace_size(&call, &workspaceSize);
+            if (rc != 0) {
+                ATB_LOG(ERROR) << "MultiLatentAttention int8 plan: " << atbmi_last_error();
+                return rc;
+            }
+            return NO_ERROR;
+        }
         AtbmiPaShape shape{};
         shape.qDtype = q.desc.dtype == ACL_BF16 ? ATBMI_BF16 : ATBMI_F16;
         shape.kvDtype = shape.qDtype;
@@ -358,6 +417,14 @@ protected:
     Status LaunchImpl(const VariantPack &pack, uint8_t *workspace, uint64_t workspaceSize,
                       aclrtStream stream) override
     {
+        if (param_.cacheMode == Param::INT8_NZCACHE) {
+            AtbmiMlaInt8Call call = MakeInt8Call(pack);
+            int rc = atbmi_mla_int8_decode(&call, workspace, workspaceSize, stream);
+            if (rc != 0) {
+                ATB_LOG(ERROR) << "MultiLatentAttention int8 launch failed: " << atbmi_last_error();
+            }
+            return rc;
+        }
         AtbmiPaTensors t{};
         t.query = pack.inTensors.at(QUERY).deviceData;
         t.queryRope = pack.inTensors.at(QUERY_ROPE).deviceData;
@@ -380,6 +447,35 @@ protected:
 
 private:
     static constexpr size_t NONE = ~static_cast<size_t>(0);
+
+    AtbmiMlaInt8Call MakeInt8Call(const VariantPack &pack) const
+    {
+        const Tensor &kv = pack.inTensors.at(KV_CACHE);
+        AtbmiMlaInt8Call c{};
+        c.outDtype = pack.inTensors.at(QUERY_ROPE).desc.dtype == ACL_BF16 ? ATBMI_BF16 : ATBMI_F16;
+        c.numHeads = param_.headNum;
+        c.blockSize = static_cast<int32_t>(kv.desc.shape.dims[2]);
+        c.numBlocks = static_cast<int32_t>(kv.desc.shape.dims[0]);
+        c.maxBlocksPerSeq = static_cast<int32_t>(pack.inTensors.at(BLOCK_TABLES).desc.shape.dims[1]);
+        c.batch = static_cast<int32_t>(lens_.size());
+        c.numQueryRows = static_cast<int32_t>(pack.inTensors.at(QUERY).desc.shape.dims[0]);
+        c.hasMask = maskIdx_ != NONE ? 1 : 0;
+        c.maskLen = static_cast<int32_t>(maskLen_);
+        c.qkScale = param_.qkScale;
+        c.hostContextLens = lens_.data();
+        c.hostQueryLens = qLens_.empty() ? nullptr : qLens_.data();
+        c.query = pack.inTensors.at(QUERY).deviceData;
+        c.queryRope = pack.inTensors.at(QUERY_ROPE).deviceData;
+        c.kvCache = kv.deviceData;
+        c.kRopeCache = pack.inTensors.at(KV_CACHE_ROPE).deviceData;
+        c.blockTables = static_cast<const int32_t *>(pack.inTensors.at(BLOCK_TABLES).deviceData);
+        c.qkDescale = static_cast<const float *>(pack.inTensors.at(descaleIdx_).deviceData);
+        c.pvDescale = static_cast<const float *>(pack.inTensors.at(descaleIdx_ + 1).deviceData);
+        c.mask = maskIdx_ != NONE ? pack.inTensors.at(maskIdx_).deviceData : nullptr;
+        c.out = pack.outTensors.at(0).deviceData;
+        c.lse = IsRing(param_) ? static_cast<float *>(pack.outTensors.at(1).deviceData) : nullptr;
+        return c;
+    }
 
     static bool SameShape(const AtbmiPaShape &a, const AtbmiPaShape &b)
     {
@@ -416,7 +512,9 @@ private:
         const Dims &kr = in.at(KV_CACHE_ROPE).shape;
         // token-major caches [blocks, blockSize, kvHeads, channels] (reference :350-392) or fractal-NZ
         // caches [blocks, channels / 16, blockSize, 16] (reference :394-425)
-        const bool nz = param_.cacheMode == Param::NZCACHE;
+        const bool int8 = param_.cacheMode == Param::INT8_NZCACHE;
+        const bool nz = param_.cacheMode == Param::NZCACHE || int8;
+        const int64_t nzLatent = int8 ? NZ_CHANNELS_INT8 : NZ_CHANNELS; // slab width of the latent cache
         const int blockDim = nz ? 2 : 1;
         if (kv.dims[blockDim] != DECODER_BLOCK_SIZE) {
             ATB_LOG(ERROR) << "decoder blockSize should be " << DECODER_BLOCK_SIZE << ", got " << kv.dims[blockDim];
@@ -431,8 +529,8 @@ private:
             return ERROR_INVALID_TENSOR_DIM;
         }
         if (nz) {
-            if (kv.dims[3] != NZ_CHANNELS || kr.dims[3] != NZ_CHANNELS) {
-                ATB_LOG(ERROR) << "dim 3 of kvCache and kvCacheRope should be " << NZ_CHANNELS;
+            if (kv.dims[3] != nzLatent || kr.dims[3] != NZ_CHANNELS) {
+                ATB_LOG(ERROR) << "dim 3 of kvCache should be " << nzLatent << ", of kvCacheRope " << NZ_CHANNELS;
                 return ERROR_INVALID_TENSOR_DIM;
             }
         } else if (kv.dims[2] != param_.kvHeadNum || kr.dims[2] != param_.kvHeadNum) {
@@ -443,7 +541,7 @@ private:
             ATB_LOG(ERROR) << "dim 1 of query and queryRope should equal headNum";
             return ERROR_INVALID_TENSOR_DIM;
         }
-        if (in.at(QUERY).shape.dims[2] != LATENT_DIM || (nz ? kv.dims[1] * NZ_CHANNELS : kv.dims[3]) != LATENT_DIM) {
+        if (in.at(QUERY).shape.dims[2] != LATENT_DIM || (nz ? kv.dims[1] * nzLatent : kv.dims[3]) != LATENT_DIM) {
             ATB_LOG(ERROR) << "head size of query and kvCache should be 512";
             return ERROR_INVALID_TENSOR_DIM;
         }
@@ -462,6 +560,19 @@ private:
                 return ERROR_INVALID_TENSOR_DIM;
             }
         }
+        if (int8 && IsRing(param_) && param_.maskType == Param::UNDEFINED) {
+            // reference :493-511 (only this combination checks the descales there)
+            const Dims &d0 = in.at(descaleIdx_).shape;
+            const Dims &d1 = in.at(descaleIdx_ + 1).shape;
+            if (d0.dimNum != 1 || d1.dimNum != 1) {
+                ATB_LOG(ERROR) << "qkDescale and pvDescale should have 1 dim";
+                return ERROR_INVALID_TENSOR_DIM_NUM;
+            }
+            if (d0.dims[0] != param_.headNum || d1.dims[0] != param_.headNum) {
+                ATB_LOG(ERROR) << "qkDescale and pvDescale should be [headNum]";
+                return ERROR_INVALID_TENSOR_DIM;
+            }
+        }
         return NO_ERROR;
     }
 
@@ -469,6 +580,10 @@ private:
     OpIr irTable_;
     size_t maskIdx_ = NONE;
     size_t qLensIdx_ = NONE;
+    size_t descaleIdx_ = NONE;
+    std::vector<int32_t> lens_;   // (int8 cache mode: the lengths of the last Setup)
+    std::vector<int32_t> qLens_;
+    int64_t maskLen_ = 0;
     uint32_t inputNum_ = 6;
     AtbmiPaPlan *plan_ = nullptr;
     AtbmiPaShape planShape_{};

@@ -17,9 +17,9 @@
 extern "C" {
 #endif
 
-// MultiLatentAttention (cacheMode KROPE_CTKV or NZCACHE). mask is read when maskType is not UNDEFINED, qSeqLen
-// when calcType is CALC_TYPE_SPEC, lse when calcType is CALC_TYPE_RING; qkDescale / pvDescale belong
-// to the int8 cache mode, which this library does not have. Pointers that are not read may be null.
+// MultiLatentAttention (cacheMode KROPE_CTKV, NZCACHE or INT8_NZCACHE). mask is read when maskType is not
+// UNDEFINED, qSeqLen when calcType is CALC_TYPE_SPEC, lse when calcType is CALC_TYPE_RING, qkDescale /
+// pvDescale with the int8 cache mode. Pointers that are not read may be null.
 atb::Status AtbMLAGetWorkspaceSize(const aclTensor *qNope, const aclTensor *qRope, const aclTensor *ctKV,
                                    const aclTensor *kRope, const aclTensor *blockTables, const aclTensor *contextLens,
                                    const aclTensor *mask, const aclTensor *qSeqLen, const aclTensor *qkDescale,

@@ -424,6 +424,54 @@ int atbmi_mla_prefill_workspace_size(const AtbmiMlaPrefillCall *call, uint64_t *
 int atbmi_mla_prefill(const AtbmiMlaPrefillCall *call, void *workspaceDevice, uint64_t workspaceBytes, void *stream);
 
 /*
+ * Decode attention of MultiLatentAttention over the int8 fractal-NZ cache (MultiLatentAttentionParam::INT8_NZCACHE;
+ * reference src/ops/ops_infer/multi_latent_attention/multi_latent_attention_operation.cpp:427-476 for the shapes,
+ * kernel library src/kernels/mixkernels/multi_latent_attention/op_kernel/mla_int8.cce, golden
+ * tests/apitest/opstest/python/operations/multi_latent_attention/test_multi_latent_attention_int8nz.py:115-121,179-262):
+ * the 512 latent channels of queries and cache rows are int8 with one fp32 descale per head for the scores
+ * (qkDescale) and one for the values (pvDescale), the 64 rotary channels stay 16-bit, and the softmax weights
+ * of every cache block (128 tokens) are quantised to int8 against the block's largest weight before they
+ * multiply the int8 value rows; all integer products are exact.
+ *   query       int8 [numQueryRows, numHeads, 512]       queryRope  16-bit [numQueryRows, numHeads, 64]
+ *   kvCache     int8 [numBlocks, 512 / 32, 128, 32]      kRopeCache 16-bit [numBlocks, 64 / 16, 128, 16]
+ *   blockTables int32 [batch, maxBlocksPerSeq] (device)  qkDescale, pvDescale fp32 [numHeads]
+ *   mask        NULL, or 16-bit [numQueryRows, maskLen] added to the scaled scores of its query row
+ *   out         16-bit [numQueryRows, numHeads, 512]     lse        NULL, or fp32 [numQueryRows, numHeads]
+ * Sequence b attends to hostContextLens[b] tokens with hostQueryLens[b] consecutive query rows (NULL: one
+ * each; a sequence of length 0 takes none). numHeads must be a multiple of 8. The lengths are host arrays,
+ * read during the call.
+ */
+typedef struct AtbmiMlaInt8Call {
+    int32_t outDtype;          /* ATBMI_F16 or ATBMI_BF16: type of queryRope, kRopeCache, mask and out */
+    int32_t numHeads;
+    int32_t blockSize;         /* 128 */
+    int32_t numBlocks;
+    int32_t maxBlocksPerSeq;
+    int32_t batch;
+    int32_t numQueryRows;
+    int32_t hasMask;
+    int32_t maskLen;
+    float qkScale;
+    const int32_t *hostContextLens; /* [batch], host memory */
+    const int32_t *hostQueryLens;   /* NULL or [batch], host memory */
+    const void *query;
+    const void *queryRope;
+    const void *kvCache;
+    const void *kRopeCache;
+    const int32_t *blockTables;
+    const float *qkDescale;
+    const float *pvDescale;
+    const void *mask;
+    void *out;
+    float *lse;
+} AtbmiMlaInt8Call;
+
+/* Validates the call (pointers aside) and reports the device workspace it needs (16 bytes per query row). */
+int atbmi_mla_int8_workspace_size(const AtbmiMlaInt8Call *call, uint64_t *bytes);
+/* Uploads the row list into the workspace and launches the kernel on `stream`; does not wait. */
+int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspaceDevice, uint64_t workspaceBytes, void *stream);
+
+/*
  * Kernel timing for benchmarks. atbmi_timing_enable(n) with n > 0 makes every
  * n-th atbmi_pa_decode bracket its attention kernel with HIP events on the
  * launch stream (the events themselves cost a few microseconds of stream

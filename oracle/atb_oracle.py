@@ -61,6 +61,20 @@ the invariants of the mathematics (no function is left "parity unpinned"):
                       block_size, 16]); the NZCACHE operator is paged_attention over nz_to_nd of its
                       caches (:767-797 feed the same golden as the ND test); pinned by flat addresses,
                       the round trip and the reference's two-step reshape / permute written with torch
+  mla_int8_decode     tests/apitest/opstest/python/operations/multi_latent_attention/
+                      test_multi_latent_attention_int8nz.py:115-121 (exact int32 products of the int8 query and
+                      cache, times a per-head descale), :276-286 (the 64 rotary channels in fp32, added before
+                      the scale; mask after it), :179-196 (softmax_quant_torch: weights exp(s - running max)
+                      quantised to int8 against the largest weight of the tile: rint(fp16(w / (wmax / 127)))),
+                      :198-262 (softmax_quant_numpy_online: per tile, exact int32 products of the int8 weights
+                      and the int8 values times pvDescale * wmax / 127, tiles joined by the usual online
+                      rescaling; lse = log(sum) + max). The tile length is a parameter of the golden, not a
+                      property of the operator: its own tests run 128 tokens for 32 and for 128 heads
+                      (:668-766) and 512 for 128 heads (:845-1104), and compare by the double-golden
+                      criterion of tests/apitest/opstest/python/operations/precision_calcu.py:111-140 against
+                      the whole context as one tile. Pinned by an independent float64 loop version, by the
+                      limit of fine descales (-> ordinary attention over the dequantised tensors), and by
+                      closed forms of the quantiser
   mla_prefill         tests/apitest/opstest/python/operations/multi_latent_attention/
                       test_multi_latent_attention_prefill.py:519-700 (gen_out_tensor: per sequence and head
                       score = q . k^T * tor over the 128 + 64 channels, + mask, fp32 softmax over the keys,
@@ -615,6 +629,67 @@ def paged_attention_loops(query, key_cache, value_cache, block_tables, context_l
                 out[row][h][c] = acc / z
         row += 1
     return np.array(out, dtype=np.float64)
+
+
+def quantise_weights(w):
+    """int8 weights of one tile and head (reference softmax_quant_torch): w / (max(w) / 127) in fp32, rounded
+    to fp16, then to the nearest integer (ties to even). Returns (int8 array, max(w))."""
+    w = np.asarray(w, np.float32)
+    wmax = np.float32(w.max()) if w.size else np.float32(0)
+    if not wmax > 0:
+        return np.zeros(w.shape, np.int8), np.float32(0)
+    step = np.float32(wmax / np.float32(127.0))
+    return np.rint((w / step).astype(np.float16)).astype(np.int8), wmax
+
+
+def mla_int8_decode(q_int8, q_rope, kv_int8, k_rope, block_tables, context_lens, qk_descale, pv_descale, scale,
+                    tile=128, mask=None, q_lens=None, lse_out=None):
+    """Decode attention of MultiLatentAttention's int8 cache mode over token-major views of the caches:
+    q_int8 [T, H, 512] int8, q_rope [T, H, 64] float, kv_int8 [blocks, block_size, 1, 512] int8 (keys and
+    values), k_rope [blocks, block_size, 1, 64] float, qk_descale / pv_descale [H] float32. The weights of
+    every `tile` consecutive tokens are quantised to int8 on their own. mask: None or [T, >= max context]
+    added to the scaled scores of its query row; q_lens: query rows per sequence (default one). Returns
+    float32 [T, H, 512]; lse_out [T, H] receives log(sum exp) of the scaled scores."""
+    q_int8 = np.asarray(q_int8)
+    rows, heads = q_int8.shape[0], q_int8.shape[1]
+    out = np.zeros((rows, heads, 512), np.float32)
+    qk_descale = np.asarray(qk_descale, np.float32)
+    pv_descale = np.asarray(pv_descale, np.float32)
+    row = 0
+    for b, ctx in enumerate(np.asarray(context_lens)):
+        ctx = int(ctx)
+        if ctx == 0:
+            continue
+        n_rows = 1 if q_lens is None else int(q_lens[b])
+        keys = gather_rows(np.asarray(kv_int8), block_tables[b], ctx)[:, 0].astype(np.int32)     # [ctx, 512]
+        rope = gather_rows(np.asarray(k_rope, np.float32), block_tables[b], ctx)[:, 0]             # [ctx, 64]
+        for r in range(row, row + n_rows):
+            prod = (q_int8[r].astype(np.int32) @ keys.T).astype(np.float32) * qk_descale[:, None]  # [H, ctx]
+            s = (prod + np.asarray(q_rope[r], np.float32) @ rope.T) * np.float32(scale)
+            if mask is not None:
+                s = s + np.asarray(mask[r, :ctx], np.float32)[None, :]
+            s = s.astype(np.float32)
+            for h in range(heads):
+                gm = gl = go = None
+                for t0 in range(0, ctx, tile):
+                    st = s[h, t0:t0 + tile]
+                    hm = np.float32(st.max()) if gm is None else np.maximum(gm, np.float32(st.max()))
+                    w = np.exp(st - hm).astype(np.float32) if np.isfinite(hm) else np.zeros_like(st)
+                    p8, wmax = quantise_weights(w)
+                    lo = (p8.astype(np.int32) @ keys[t0:t0 + tile]).astype(np.float32) * \
+                        np.float32(pv_descale[h] * wmax / np.float32(127.0))
+                    ll = np.float32(w.sum(dtype=np.float32))
+                    if gm is None:
+                        gl, go = ll, lo
+                    else:
+                        keep = np.float32(np.exp(gm - hm)) if np.isfinite(gm) else np.float32(0)
+                        gl, go = gl * keep + ll, go * keep + lo
+                    gm = hm
+                out[r, h] = go / gl if gl > 0 else 0
+                if lse_out is not None:
+                    lse_out[r, h] = np.log(gl) + gm if gl > 0 else -np.inf
+        row += n_rows
+    return out
 
 
 def mla_prefill(q_nope, q_rope, k_nope, k_rope, value, q_lens, kv_lens, scale, mask="none", window=0,

@@ -64,10 +64,10 @@ def _rac_unimplemented(p):
 
 def _mla_unimplemented(p):
     """Features of MultiLatentAttentionParam the reference accepts but this library rejects at creation:
-    the int8 fractal-NZ cache mode, decode masks other than MASK_TYPE_SPEC, maskUseStatus."""
+    decode masks other than MASK_TYPE_SPEC, maskUseStatus."""
     if p.get("calcType", 0) == 4:
         return False
-    return p.get("cacheMode", 0) == 2 or p.get("maskType", 0) >= 2 or p.get("maskUseStatusType", 0) != 0
+    return p.get("maskType", 0) >= 2 or p.get("maskUseStatusType", 0) != 0
 
 
 def _make_param(binding, op, p):
@@ -258,10 +258,10 @@ def test_table_coverage():
     rac_dev = [c for c in RAC_CASES if _rac_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
     assert len(PA_CASES) == 81 and len(PA_CASES) - len(pa_dev) >= 75
     assert len(RAC_CASES) == 38 and len(RAC_CASES) - len(rac_dev) >= 29
-    # the MultiLatentAttention rows replayed as "rejected at creation" exercise the int8 fractal-NZ cache, the
-    # decode masks other than MASK_TYPE_SPEC and maskUseStatus
+    # the MultiLatentAttention rows replayed as "rejected at creation" exercise decode masks other than
+    # MASK_TYPE_SPEC and maskUseStatus
     mla_dev = [c for c in MLA_CASES if _mla_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
-    assert len(MLA_CASES) == 147 and len(MLA_CASES) - len(mla_dev) == 114
+    assert len(MLA_CASES) == 147 and len(MLA_CASES) - len(mla_dev) == 144
 
 
 def test_param_sizes(binding):
@@ -576,7 +576,8 @@ def test_multi_latent_attention_counts_shapes_and_setup(binding, ctx):
         assert op.ok and (op.input_num(), op.output_num()) == (n_in, n_out), kw
         op.close()
     for bad in (dict(headNum=12), dict(kvHeadNum=2), dict(cacheMode=0), dict(maskType=1), dict(qkScale=1.5),
-                dict(qkScale=0.0), dict(calcType=5), dict(cacheMode=2), dict(cacheMode=4), dict(calcType=4, headNum=32),
+                dict(qkScale=0.0), dict(calcType=5), dict(cacheMode=4), dict(calcType=4, headNum=32),
+                dict(cacheMode=2, calcType=2, maskType=1),
                 dict(calcType=1, maskType=2), dict(calcType=1, maskType=3), dict(calcType=1, maskType=4),
                 dict(calcType=3, maskUseStatusType=1)):
         kw = dict(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1)
@@ -636,6 +637,74 @@ def test_multi_latent_attention_counts_shapes_and_setup(binding, ctx):
     assert spec.setup(pack(rows=5, mask=[5, 300], with_qlens=True), outs(rows=5), ctx)[0] == e["ERROR_INVALID_PARAM"]
     assert spec.setup(pack(rows=6, mask=[6, 300], with_qlens=True, qlens_host=False), outs(rows=6), ctx)[0] == \
         e["ERROR_INVALID_PARAM"]
+    spec.close()
+
+
+def test_multi_latent_attention_int8_nz_cache_checks(binding, ctx):
+    """cacheMode INT8_NZCACHE: int8 query [T, H, 512] and latent cache [blocks, 16, 128, 32], 16-bit rotary parts,
+    qkDescale / pvDescale fp32 [H] after the mask and qSeqlen, fp32 log-sum-exp (reference
+    multi_latent_attention_operation.cpp:245-283 counts and InferShape, :427-476 shapes, :493-541 descales and
+    outputs; ops_configs/atb_ops_info.ini:6741-6771, 6825-6858, 6918-6945)."""
+    e = binding.ERROR_CODE
+    mk = binding.MultiLatentAttentionParam
+    lens = np.array([10, 300, 0, 64], dtype=np.int32)
+    qlens = np.array([1, 3, 2, 2], dtype=np.int32)
+
+    def pack(rows=4, kv=(16, 16, 128, 32), kr=(16, 4, 128, 16), dtype="float16", with_qlens=False, q_dtype="int8",
+             descale=(32,), fmt="fractal_nz", mask=None):
+        ins = [binding.make_tensor(q_dtype, [rows, 32, 512], FAKE_DEVICE),
+               binding.make_tensor(dtype, [rows, 32, 64], FAKE_DEVICE),
+               binding.make_tensor("int8", list(kv), FAKE_DEVICE, fmt=fmt),
+               binding.make_tensor(dtype, list(kr), FAKE_DEVICE, fmt=fmt),
+               binding.make_tensor("int32", [4, 3], FAKE_DEVICE),
+               binding.make_tensor("int32", [4], FAKE_DEVICE, host_ptr=lens.ctypes.data)]
+        if mask is not None:
+            ins.append(binding.make_tensor(dtype, list(mask), FAKE_DEVICE))
+        if with_qlens:
+            ins.append(binding.make_tensor("int32", [4], FAKE_DEVICE, host_ptr=qlens.ctypes.data))
+        ins += [binding.make_tensor("float", list(descale), FAKE_DEVICE) for _ in range(2)]
+        return ins
+
+    def outs(rows=4, lse=None, dtype="float16"):
+        o = [binding.make_tensor(dtype, [rows, 32, 512], FAKE_DEVICE)]
+        if lse:
+            o.append(binding.make_tensor(lse, [rows, 32, 1], FAKE_DEVICE))
+        return o
+
+    plain = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=2))
+    assert plain.ok and (plain.input_num(), plain.output_num()) == (8, 1)
+    st, descs = plain.infer_shape(pack(dtype="bf16"))
+    assert st == 0 and descs[0].dtype == binding.ACL_DTYPE_BY_NAME["bf16"]      # the rotary query's type, not int8
+    st, ws = plain.setup(pack(), outs(), ctx)
+    assert st == 0 and ws == 3 * 16                                             # 16 bytes per query row
+    assert plain.setup(pack(q_dtype="float16"), outs(), ctx)[0] == e["ERROR_INVALID_TENSOR_INI_MATCH"]
+    assert plain.setup(pack(fmt="nd"), outs(), ctx)[0] == e["ERROR_INVALID_TENSOR_INI_MATCH"]
+    for bad in (dict(kv=(16, 32, 128, 16)), dict(kv=(16, 16, 64, 32), kr=(16, 4, 64, 16)), dict(kr=(16, 2, 128, 32)),
+                dict(kv=(16, 8, 128, 32))):
+        assert plain.setup(pack(**bad), outs(), ctx)[0] == e["ERROR_INVALID_TENSOR_DIM"], bad
+    assert plain.setup(pack(descale=(31,)), outs(), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    plain.close()
+    ring = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=2,
+                                                                 calcType=2))
+    assert ring.ok and (ring.input_num(), ring.output_num()) == (8, 2)
+    st, descs = ring.infer_shape(pack())
+    assert st == 0 and descs[1].dtype == binding.ACL_DTYPE_BY_NAME["float"]
+    assert [d.dims[i] for d in descs for i in range(d.dimNum)] == [4, 32, 512, 4, 32, 1]
+    assert ring.setup(pack(), outs(lse="float"), ctx)[0] == 0
+    assert ring.setup(pack(), outs(lse="float16"), ctx)[0] == e["ERROR_INVALID_TENSOR_INI_MATCH"]
+    assert ring.setup(pack(descale=(31,)), outs(lse="float"), ctx)[0] == e["ERROR_INVALID_TENSOR_DIM"]
+    assert ring.setup(pack(descale=(4, 8)), outs(lse="float"), ctx)[0] == e["ERROR_INVALID_TENSOR_DIM_NUM"]
+    ring.close()
+    both = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=2,
+                                                                 calcType=3))
+    assert both.ok and (both.input_num(), both.output_num()) == (9, 2)
+    assert both.setup(pack(rows=6, with_qlens=True), outs(rows=6, lse="float"), ctx)[0] == 0
+    both.close()
+    spec = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=2,
+                                                                 calcType=1, maskType=1))
+    assert spec.ok and spec.input_num() == 10
+    assert spec.setup(pack(rows=6, with_qlens=True, mask=(6, 300)), outs(rows=6), ctx)[0] == 0
+    assert spec.setup(pack(rows=6, with_qlens=True, mask=(6, 299)), outs(rows=6), ctx)[0] == e["ERROR_INVALID_PARAM"]
     spec.close()
 
 
@@ -1170,7 +1239,7 @@ def test_acl_tensor_handle_and_two_call_wrappers(binding, ctx):
     ring = ctypes.c_void_p()
     assert mla(2, lse="lse", op_ref=ring) == 0 and ring.value and ring.value != first
     nz = ctypes.c_void_p()
-    assert mla(0, cache_mode=2, op_ref=nz) == E["ERROR_INVALID_PARAM"] and not nz.value   # the int8 cache mode is not built
+    assert mla(0, cache_mode=4, op_ref=nz) == E["ERROR_INVALID_PARAM"] and not nz.value   # no such cache mode
     lens[2] = 3 * 128 + 1                              # longer than its block table: Setup refuses
     assert mla(0) == E["ERROR_INVALID_PARAM"]
     assert lib.AtbMLA(None, 0, None, ctx.ptr) == E["ERROR_INVALID_OPERATION_ADDR"]

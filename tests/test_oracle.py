@@ -939,6 +939,101 @@ def test_fractal_nz_layout_by_flat_addresses_and_round_trip(oracle, n0):
         oracle.nd_to_nz(x[:, :8], n0)
 
 
+def _int8_case(rng, ctx, heads=4, block=16, q_lens=None):
+    ctx = np.asarray(ctx, np.int32)
+    nblk = (ctx + block - 1) // block
+    pool = int(nblk.sum()) + 2
+    perm = rng.permutation(pool)
+    tables = np.zeros((len(ctx), max(1, int(nblk.max()))), np.int32)
+    pos = 0
+    for b in range(len(ctx)):
+        tables[b, :nblk[b]] = perm[pos:pos + nblk[b]]
+        pos += nblk[b]
+    rows = int(sum((1 if q_lens is None else q_lens[b]) for b in range(len(ctx)) if ctx[b] > 0))
+    q8 = rng.integers(-5, 6, size=(rows, heads, 512)).astype(np.int8)
+    qr = rng.uniform(-5, 5, size=(rows, heads, 64)).astype(np.float16).astype(np.float32)
+    kv8 = rng.integers(-5, 6, size=(pool, block, 1, 512)).astype(np.int8)
+    kr = rng.uniform(-5, 5, size=(pool, block, 1, 64)).astype(np.float16).astype(np.float32)
+    qd = rng.uniform(1 / 127, 5 / 127, size=heads).astype(np.float32)
+    pd = rng.uniform(-5 / 127, 5 / 127, size=heads).astype(np.float32)
+    return q8, qr, kv8, kr, tables, ctx, qd, pd
+
+
+def test_int8_weight_quantiser_closed_forms(oracle):
+    """w / (max / 127) rounded to fp16, then to the nearest integer, ties to even (reference
+    test_multi_latent_attention_int8nz.py:191-194)."""
+    p8, wmax = oracle.quantise_weights(np.array([1.0, 0.5, 0.25, 0.0, 3 / 254], np.float32))
+    assert wmax == 1.0 and p8.tolist() == [127, 64, 32, 0, 2]      # 63.5 -> 64, 31.75 -> 32, 1.5 -> 2
+    p8, wmax = oracle.quantise_weights(np.array([0.02, 0.01, 0.02], np.float32))
+    assert p8.tolist() == [127, 64, 127] and wmax == np.float32(0.02)
+    # fp16 keeps 11 bits: 2047 / 2048 of the maximum is 126.94 -> fp16 126.9375 -> 127
+    assert oracle.quantise_weights(np.array([1.0, 2047 / 2048], np.float32))[0].tolist() == [127, 127]
+    assert oracle.quantise_weights(np.zeros(3, np.float32))[0].tolist() == [0, 0, 0]
+
+
+@pytest.mark.parametrize("tile", [16, 48, 1000])
+def test_int8_decode_matches_independent_loops(oracle, tile):
+    """Token by token in Python integers and float64, every tile's weights quantised by their own maximum."""
+    rng = _rng(140 + tile)
+    q8, qr, kv8, kr, tables, ctx, qd, pd = _int8_case(rng, [37, 0, 5, 96], heads=3, q_lens=[2, 1, 1, 1])
+    mask = (rng.standard_normal((5, 96)) * 2).astype(np.float32)
+    lse = np.zeros((5, 3), np.float32)
+    got = oracle.mla_int8_decode(q8, qr, kv8, kr, tables, ctx, qd, pd, 0.04, tile=tile, mask=mask, q_lens=[2, 1, 1, 1],
+                                 lse_out=lse)
+    row = 0
+    for b, n in enumerate(ctx):
+        for _ in range([2, 1, 1, 1][b] if n > 0 else 0):
+            for h in range(3):
+                s = []
+                for t in range(n):
+                    blk, off = tables[b, t // 16], t % 16
+                    prod = sum(int(a) * int(c) for a, c in zip(q8[row, h], kv8[blk, off, 0]))
+                    rope = float(np.dot(qr[row, h].astype(np.float64), kr[blk, off, 0]))
+                    s.append(np.float32((np.float32(np.float32(prod) * qd[h]) + np.float32(rope)) * np.float32(0.04)) +
+                             mask[row, t])
+                s = np.array(s, np.float64)
+                num, den, ref = np.zeros(512), 0.0, None
+                for t0 in range(0, n, tile):
+                    st = s[t0:t0 + tile]
+                    new = st.max() if ref is None else max(ref, st.max())
+                    if ref is not None:
+                        num, den = num * math.exp(ref - new), den * math.exp(ref - new)
+                    ref = new
+                    w = np.exp(st - ref)
+                    p8 = np.rint((w.astype(np.float32) / np.float32(np.float32(w.max()) / np.float32(127))).astype(np.float16))
+                    for i, t in enumerate(range(t0, min(n, t0 + tile))):
+                        blk, off = tables[b, t // 16], t % 16
+                        num += p8[i] * kv8[blk, off, 0].astype(np.float64) * (float(pd[h]) * float(np.float32(w.max())) / 127)
+                    den += w.sum()
+                np.testing.assert_allclose(got[row, h], num / den, rtol=2e-5, atol=2e-6)
+                np.testing.assert_allclose(lse[row, h], math.log(den) + ref, rtol=1e-5, atol=1e-5)
+            row += 1
+
+
+def test_int8_decode_limits_and_closed_forms(oracle):
+    rng = _rng(150)
+    q8, qr, kv8, kr, tables, ctx, qd, pd = _int8_case(rng, [1, 64, 33], heads=2)
+    lse = np.zeros((3, 2), np.float32)
+    got = oracle.mla_int8_decode(q8, qr, kv8, kr, tables, ctx, qd, pd, 0.05, tile=16, lse_out=lse)
+    # one token: its weight is 127 of 127, the output is its value row times the head's descale
+    np.testing.assert_allclose(got[0], kv8[tables[0, 0], 0, 0][None, :] * pd[:, None], rtol=1e-6)
+    # 127 levels per tile: within about half a level of ordinary attention over the dequantised tensors, and
+    # the log-sum-exp (which adds up the unquantised weights) agrees to float precision
+    q = np.concatenate([q8.astype(np.float32) * qd[None, :, None], qr], -1)
+    kc = np.concatenate([kv8.astype(np.float32), kr], -1)
+    plain_lse = np.zeros((3, 2), np.float32)
+    plain = oracle.paged_attention(q, kc, None, tables, ctx, 0.05, mla_v_head_size=512, lse_out=plain_lse)
+    plain = plain * pd[None, :, None]
+    assert np.abs(got - plain).max() <= 0.012 * np.abs(kv8).max() * np.abs(pd).max() * 4
+    assert np.abs(got - plain).max() > 0                     # (it is not the unquantised computation)
+    np.testing.assert_allclose(lse, plain_lse, rtol=1e-5, atol=1e-5)
+    # equal scores: every weight is 127, the output is the mean of the value rows
+    q0 = np.zeros_like(q8[:1])
+    flat = oracle.mla_int8_decode(q0, np.zeros_like(qr[:1]), kv8, kr, tables[1:2], ctx[1:2], qd, pd, 0.05, tile=16)
+    rows = kv8[tables[1, np.arange(64) // 16], np.arange(64) % 16, 0].astype(np.float64)
+    np.testing.assert_allclose(flat[0], rows.mean(0)[None, :] * pd[:, None], rtol=1e-5, atol=1e-6)
+
+
 def _prefill_case(rng, q_lens, kv_lens, heads, kv_heads):
     tq, tk = int(sum(q_lens)), int(sum(kv_lens))
     mk = lambda *shape: rng.standard_normal(shape).astype(np.float32)
