@@ -14,15 +14,15 @@
 //             denominator adds up the unquantised weights.
 // Every integer product is exact (v_dot4_i32_i8 into int32; a tile's sums stay below 2^24).
 //
-// A workgroup owns one query row and eight heads and walks the row's context block by block:
+// A workgroup of eight waves owns one query row and 16 heads (8 when there are no more) and walks the row's context block by block:
 //   load    the block's int8 rows and rotary rows from the NZ layout into row-major LDS tiles;
-//   scores  thread (token, half of the heads): its row against four query heads, each cache dword reused for
-//           the four heads;
-//   softmax wave w for heads 2 w and 2 w + 1, two tokens a lane;
-//   values  thread (4 channels, half of the heads): four cache rows at a time, their bytes transposed in
+//   scores  thread (token, quarter of the heads): its row against its query heads, each cache dword reused for
+//           all of them;
+//   softmax one wave per head (or per two), two tokens a lane;
+//   values  thread (4 channels, quarter of the heads): four cache rows at a time, their bytes transposed in
 //           registers so that one dot4 covers four tokens.
 // Four barriers a block and no overlap of the load with the arithmetic: built for exact agreement with the
-// golden first; at the sizes of benchmark workload C5 it runs at about a third of the 16-bit kernel's rate.
+// golden first.
 #include <vector>
 #include "pa_internal.h"
 #include "upload_ring.h"
@@ -35,19 +35,22 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 constexpr int TILE = 128;            // tokens per tile = the block size of the cache
 constexpr int DN = 512;              // int8 channels (keys and values)
 constexpr int DR = 64;               // rotary channels (16-bit)
-constexpr int HT = 8;                // heads per workgroup
-constexpr int THREADS = 256;
+constexpr int THREADS = 512;         // eight waves, two a SIMD: one's LDS round trips hide behind the other's arithmetic
 constexpr int K_PITCH = DN + 16;     // bytes; 16-byte reads of 16 consecutive rows touch every bank once
 constexpr int R_PITCH = DR * 2 + 16;
-constexpr int LDS_K = 0;
-constexpr int LDS_R = LDS_K + TILE * K_PITCH;
-constexpr int LDS_Q8 = LDS_R + TILE * R_PITCH;          // [HT][512] int8
-constexpr int LDS_QR = LDS_Q8 + HT * DN;                // [HT][64] fp32
-constexpr int LDS_S = LDS_QR + HT * DR * 4;             // [HT][TILE] fp32 scores
-constexpr int LDS_P = LDS_S + HT * TILE * 4;            // [HT][TILE] int8 weights
-constexpr int LDS_STAT = LDS_P + HT * TILE;             // [HT] {keep, value scale, 1 / sum, lse}
-constexpr int LDS_BYTES = LDS_STAT + HT * 16;
-static_assert(LDS_BYTES <= 160 * 1024 && LDS_R % 16 == 0 && LDS_Q8 % 16 == 0 && LDS_S % 16 == 0, "LDS layout");
+// LDS of a workgroup with HT heads: the two tiles, the query (int8 rows, fp32 rotary rows), the tile's scores,
+// its int8 weights and four numbers per head {keep, value scale, 1 / sum, lse}.
+template <int HT> struct Lds {
+    static constexpr int K = 0;
+    static constexpr int R = K + TILE * K_PITCH;
+    static constexpr int Q8 = R + TILE * R_PITCH;
+    static constexpr int QR = Q8 + HT * DN;
+    static constexpr int S = QR + HT * DR * 4;
+    static constexpr int P = S + HT * TILE * 4;
+    static constexpr int STAT = P + HT * TILE;
+    static constexpr int BYTES = STAT + HT * 16;
+    static_assert(BYTES <= 160 * 1024 && R % 16 == 0 && Q8 % 16 == 0 && S % 16 == 0, "LDS layout");
+};
 
 // One query row: its sequence's block-table row and context length, the row of query / out, the mask row.
 struct Row {
@@ -81,8 +84,15 @@ __device__ __forceinline__ float Load16AsFloat(uint32_t bits, bool bf16)
     return bf16 ? Bf16ToFloat(static_cast<uint16_t>(bits)) : HalfBitsToFloat(static_cast<uint16_t>(bits));
 }
 
-__global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
+// HT heads per workgroup (8 or 16): a thread takes HT / 4 heads in the score and value phases, a wave HT / 8
+// in the softmax.
+template <int HT> __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
 {
+    using L = Lds<HT>;
+    constexpr int LDS_K = L::K, LDS_R = L::R, LDS_Q8 = L::Q8, LDS_QR = L::QR, LDS_S = L::S, LDS_P = L::P,
+                  LDS_STAT = L::STAT;
+    constexpr int HPT = HT / 4; // heads per thread
+    constexpr int HPW = HT / 8; // heads per wave
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x;
     const int lane = tid & (WAVE - 1);
@@ -96,7 +106,9 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
     // ---- the query of the eight heads: int8 rows as they are, rotary rows as fp32
     {
         const int8_t *q8 = a.q8 + (static_cast<int64_t>(row.qRow) * a.H + h0) * DN;
-        *reinterpret_cast<u32x4 *>(smem + LDS_Q8 + tid * 16) = *reinterpret_cast<const u32x4 *>(q8 + tid * 16);
+        if (tid < HT * DN / 16) {
+            *reinterpret_cast<u32x4 *>(smem + LDS_Q8 + tid * 16) = *reinterpret_cast<const u32x4 *>(q8 + tid * 16);
+        }
         const uint16_t *qr = reinterpret_cast<const uint16_t *>(a.qRope) + (static_cast<int64_t>(row.qRow) * a.H + h0) * DR;
         float *dst = reinterpret_cast<float *>(smem + LDS_QR);
         for (int i = tid; i < HT * DR; i += THREADS) {
@@ -106,23 +118,27 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
 
     // scores: thread (token, group of four heads)
     const int tok = tid & (TILE - 1);
-    const int hs = (tid / TILE) * (HT / 2);
+    const int hs = (tid / TILE) * HPT;
     // softmax: this wave's two heads; the running maximum, sum and per-tile factors live in its lanes
-    float runMax[2] = {-INFINITY, -INFINITY};
-    float runSum[2] = {0.0f, 0.0f};
+    float runMax[HPW], runSum[HPW];
+#pragma unroll
+    for (int i = 0; i < HPW; ++i) {
+        runMax[i] = -INFINITY;
+        runSum[i] = 0.0f;
+    }
     // values: thread (4 channels, group of four heads)
     const int col = tid & (TILE - 1); // dword column of a cache row
-    float acc[HT / 2][4];
+    float acc[HPT][4];
 #pragma unroll
-    for (int h = 0; h < HT / 2; ++h) {
+    for (int h = 0; h < HPT; ++h) {
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
             acc[h][b] = 0.0f;
         }
     }
-    float descale[HT / 2];
+    float descale[HPT];
 #pragma unroll
-    for (int h = 0; h < HT / 2; ++h) {
+    for (int h = 0; h < HPT; ++h) {
         descale[h] = a.qkDescale[h0 + hs + h];
     }
     const uint16_t *maskRow = a.mask ? reinterpret_cast<const uint16_t *>(a.mask) + static_cast<int64_t>(row.qRow) * a.maskLen
@@ -153,13 +169,13 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
         __syncthreads();
         // ---- scores of token `tok` for heads hs .. hs + 3
         {
-            int dot[HT / 2] = {0, 0, 0, 0};
+            int dot[HPT] = {};
             const unsigned char *krow = smem + LDS_K + tok * K_PITCH;
 #pragma unroll 4
             for (int j = 0; j < DN / 16; ++j) {
                 const u32x4 kk = *reinterpret_cast<const u32x4 *>(krow + j * 16);
 #pragma unroll
-                for (int h = 0; h < HT / 2; ++h) {
+                for (int h = 0; h < HPT; ++h) {
                     const u32x4 qq = *reinterpret_cast<const u32x4 *>(smem + LDS_Q8 + (hs + h) * DN + j * 16);
 #pragma unroll
                     for (int d = 0; d < 4; ++d) {
@@ -167,7 +183,7 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
                     }
                 }
             }
-            float rope[HT / 2] = {0.0f, 0.0f, 0.0f, 0.0f};
+            float rope[HPT] = {};
             const unsigned char *rrow = smem + LDS_R + tok * R_PITCH;
 #pragma unroll 2
             for (int j = 0; j < DR / 8; ++j) {
@@ -178,7 +194,7 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
                     kf[e] = Load16AsFloat((e & 1) ? (rr[e >> 1] >> 16) : (rr[e >> 1] & 0xffffu), bf16);
                 }
 #pragma unroll
-                for (int h = 0; h < HT / 2; ++h) {
+                for (int h = 0; h < HPT; ++h) {
                     const float *qf = reinterpret_cast<const float *>(smem + LDS_QR) + (hs + h) * DR + j * 8;
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
@@ -189,7 +205,7 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
             const bool live = t0 + tok < row.ctxLen;
             const float bias = (maskRow && live) ? Load16AsFloat(maskRow[t0 + tok], bf16) : 0.0f;
 #pragma unroll
-            for (int h = 0; h < HT / 2; ++h) {
+            for (int h = 0; h < HPT; ++h) {
                 float s = (static_cast<float>(dot[h]) * descale[h] + rope[h]) * a.qkScale + bias;
                 reinterpret_cast<float *>(smem + LDS_S)[(hs + h) * TILE + tok] = live ? s : -INFINITY;
             }
@@ -197,8 +213,8 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
         __syncthreads();
         // ---- weights of the tile for heads 2 wave, 2 wave + 1
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int h = 2 * wave + i;
+        for (int i = 0; i < HPW; ++i) {
+            const int h = HPW * wave + i;
             const float *srow = reinterpret_cast<const float *>(smem + LDS_S) + h * TILE;
             const float s0 = srow[lane], s1 = srow[lane + WAVE];
             float tileMax = fmaxf(s0, s1);
@@ -235,9 +251,9 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
         __syncthreads();
         // ---- values: channels 4 col .. 4 col + 3 for heads hs .. hs + 3
         {
-            int iacc[HT / 2][4];
+            int iacc[HPT][4];
 #pragma unroll
-            for (int h = 0; h < HT / 2; ++h) {
+            for (int h = 0; h < HPT; ++h) {
 #pragma unroll
                 for (int b = 0; b < 4; ++b) {
                     iacc[h][b] = 0;
@@ -262,7 +278,7 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
                 kt[2] = __builtin_amdgcn_perm(x23hi, x01hi, 0x05040100u);
                 kt[3] = __builtin_amdgcn_perm(x23hi, x01hi, 0x07060302u);
 #pragma unroll
-                for (int h = 0; h < HT / 2; ++h) {
+                for (int h = 0; h < HPT; ++h) {
                     const uint32_t pw = *reinterpret_cast<const uint32_t *>(smem + LDS_P + (hs + h) * TILE + t4 * 4);
 #pragma unroll
                     for (int b = 0; b < 4; ++b) {
@@ -271,7 +287,7 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
                 }
             }
 #pragma unroll
-            for (int h = 0; h < HT / 2; ++h) {
+            for (int h = 0; h < HPT; ++h) {
                 const float *stat = reinterpret_cast<const float *>(smem + LDS_STAT) + (hs + h) * 4;
                 const float keep = stat[0], vscale = stat[1];
 #pragma unroll
@@ -285,15 +301,15 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
     __syncthreads();
     if (lane == 0) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            float *stat = reinterpret_cast<float *>(smem + LDS_STAT) + (2 * wave + i) * 4;
+        for (int i = 0; i < HPW; ++i) {
+            float *stat = reinterpret_cast<float *>(smem + LDS_STAT) + (HPW * wave + i) * 4;
             stat[2] = runSum[i] > 0.0f ? 1.0f / runSum[i] : 0.0f;
             stat[3] = runSum[i] > 0.0f ? logf(runSum[i]) + runMax[i] : -INFINITY;
         }
     }
     __syncthreads();
 #pragma unroll
-    for (int h = 0; h < HT / 2; ++h) {
+    for (int h = 0; h < HPT; ++h) {
         const float inv = reinterpret_cast<const float *>(smem + LDS_STAT)[(hs + h) * 4 + 2];
         uint16_t bits[4];
 #pragma unroll
@@ -321,8 +337,8 @@ int BuildRows(const AtbmiMlaInt8Call *c, std::vector<Row> *rows)
     if (c->outDtype != ATBMI_F16 && c->outDtype != ATBMI_BF16) {
         return Fail(ERR_INVALID_PARAM, "mla_int8: the 16-bit tensors are fp16 or bf16, got %d", c->outDtype);
     }
-    if (c->numHeads <= 0 || c->numHeads % HT != 0) {
-        return Fail(ERR_INVALID_PARAM, "mla_int8: %d heads (a multiple of %d)", c->numHeads, HT);
+    if (c->numHeads <= 0 || c->numHeads % 8 != 0) {
+        return Fail(ERR_INVALID_PARAM, "mla_int8: %d heads (a multiple of 8)", c->numHeads);
     }
     if (c->blockSize != TILE) {
         return Fail(ERR_INVALID_PARAM, "mla_int8: block size %d (the int8 cache has blocks of %d tokens)", c->blockSize, TILE);
@@ -406,7 +422,8 @@ extern "C" int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspa
         return Fail(ERR_INVALID_PARAM, "mla_int8: workspace of %llu bytes, %llu needed", (unsigned long long)workspaceBytes,
                     (unsigned long long)bytes);
     }
-    const int64_t grid = static_cast<int64_t>(rows.size()) * (call->numHeads / mlaint8::HT);
+    const int ht = call->numHeads % 16 == 0 ? 16 : 8;
+    const int64_t grid = static_cast<int64_t>(rows.size()) * (call->numHeads / ht);
     if (grid > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "mla_int8: %lld workgroups", (long long)grid);
     }
@@ -432,11 +449,13 @@ extern "C" int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspa
     a.maskLen = call->maskLen;
     a.bf16 = call->outDtype == ATBMI_BF16 ? 1 : 0;
     a.qkScale = call->qkScale;
-    rc = ConfigureKernelLds(reinterpret_cast<const void *>(mlaint8::MlaInt8Kernel), mlaint8::LDS_BYTES);
+    auto kernel = ht == 16 ? mlaint8::MlaInt8Kernel<16> : mlaint8::MlaInt8Kernel<8>;
+    const int ldsBytes = ht == 16 ? mlaint8::Lds<16>::BYTES : mlaint8::Lds<8>::BYTES;
+    rc = ConfigureKernelLds(reinterpret_cast<const void *>(kernel), ldsBytes);
     if (rc != OK) {
         return rc;
     }
-    mlaint8::MlaInt8Kernel<<<static_cast<unsigned>(grid), mlaint8::THREADS, mlaint8::LDS_BYTES, s>>>(a);
+    kernel<<<static_cast<unsigned>(grid), mlaint8::THREADS, ldsBytes, s>>>(a);
     ATBMI_HIP_CHECK(hipGetLastError());
     return OK;
 }

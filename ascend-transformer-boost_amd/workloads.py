@@ -43,8 +43,9 @@ CONFIGS["c2_bnsd"] = dict(CONFIGS["c2"], bnsd=True)
 # tensors each for the query and the cache.
 CONFIGS["c5_split"] = dict(CONFIGS["c5"], split=True)
 CONFIGS["c5_nz"] = dict(CONFIGS["c5"], split=True, nz=True)
+CONFIGS["c5_int8"] = dict(CONFIGS["c5"], split=True, nz=True, int8nz=True)
 
-SEEDS = {"c1": 1001, "c2": 1002, "c2_fp16": 1002, "c2_alibi": 1002, "c2_norm": 1002, "c2_mtp4": 1002, "c2_bnsd": 1002, "c3": 1003, "c4": 1004, "c5": 1005, "c5_split": 1005, "c5_nz": 1005}
+SEEDS = {"c1": 1001, "c2": 1002, "c2_fp16": 1002, "c2_alibi": 1002, "c2_norm": 1002, "c2_mtp4": 1002, "c2_bnsd": 1002, "c3": 1003, "c4": 1004, "c5": 1005, "c5_split": 1005, "c5_nz": 1005, "c5_int8": 1005}
 
 
 def config(name, **overrides):
@@ -207,6 +208,8 @@ def algorithmic_bytes(cfg, ctx):
     n = int(cfg.get("q_len", 1))
     rows = int((ctx > 0).sum()) * n
     total = int(ctx.sum()) * per_tok + rows * h * (d + dv) * 2
+    if cfg.get("int8nz"):  # 512 int8 + 64 16-bit channels per cache row; 512 int8 + 64 16-bit per query row and head
+        total = int(ctx.sum()) * (512 + 64 * 2) + rows * h * (512 + 64 * 2 + dv * 2) + 2 * h * 4
     total += int(((ctx + bs - 1) // bs).sum()) * 4 + len(ctx) * 4
     if cfg["kv"] == "int8":
         total += g * (d + dv) * 4

@@ -80,6 +80,9 @@ DESCRIPTIONS = {
                 "two caches): batch 64, 128 q heads, block 128, ctx U[2048,4096], bf16",
     "c5_nz": "C5 through MultiLatentAttentionOperation with cacheMode NZCACHE (fractal-NZ caches [blocks, 32 | 4, 128, 16]), "
              "attention only: batch 64, 128 q heads, block 128, ctx U[2048,4096], bf16",
+    "c5_int8": "C5 through MultiLatentAttentionOperation with cacheMode INT8_NZCACHE (int8 query and latent cache, "
+               "fractal-NZ, bf16 rotary parts; random int8 contents), attention only: batch 64, 128 q heads, block 128, "
+               "ctx U[2048,4096]",
     "c5": "C5 MLA bf16 decode: batch 64, 128 q heads, 1 latent kv head, d576/dv512, block 128, ctx U[2048,4096]",
 }
 
@@ -174,7 +177,8 @@ def run_workload(pkg, name, steps, warmup, attention_only=False, kernel_events=T
     split = bool(cfg.get("split"))
     if split:
         pa = b.OperationRunner("MultiLatentAttentionOperation", b.MultiLatentAttentionParam(
-            headNum=cfg["heads"], kvHeadNum=1, qkScale=scale, cacheMode=3 if nz else 1), ctx)
+            headNum=cfg["heads"], kvHeadNum=1, qkScale=scale,
+            cacheMode=2 if cfg.get("int8nz") else (3 if nz else 1)), ctx)
     else:
         pa = b.OperationRunner("PagedAttentionOperation", pa_param, ctx)
     rac = None
@@ -198,6 +202,13 @@ def run_workload(pkg, name, steps, warmup, attention_only=False, kernel_events=T
                 # [blocks, block, 1, channels] -> [blocks, channels / 16, block, 16], described in the fractal-NZ format
                 nz_caches = [t[:, :, 0, :].reshape(t.shape[0], t.shape[1], -1, 16).permute(0, 2, 1, 3).contiguous()
                              for t in (nope, rope)]
+                if cfg.get("int8nz"):
+                    # int8 latent parts with random contents, slabs of 32 channels; one descale per head each
+                    nz_caches[0] = torch.randint(-5, 6, (nope.shape[0], dv // 32, nope.shape[1], 32), dtype=torch.int8,
+                                                 device=dev)
+                    pa_in[0] = torch.randint(-5, 6, tuple(pa_in[0].shape), dtype=torch.int8, device=dev)
+                    descales = [torch.rand(cfg["heads"], device=dev) * 0.04 + 0.001 for _ in range(2)]
+                    pa_in += descales
                 pa_in[2:4] = [b.make_tensor(b._torch_acl_dtype(t), list(t.shape), device_ptr=t.data_ptr(),
                                             fmt="fractal_nz") for t in nz_caches]
         elif mla:
