@@ -12,17 +12,21 @@
 //   values  = int32 dot of the int8 weights and the int8 cache rows (the first 512 channels are the values),
 //             times pvDescale[head] x wmax / 127; tiles are joined by the usual online rescaling, the
 //             denominator adds up the unquantised weights.
-// Every integer product is exact (v_dot4_i32_i8 into int32; a tile's sums stay below 2^24).
+// Every integer product is exact (v_mfma_i32_16x16x64_i8; a tile's sums stay below 2^24).
 //
-// A workgroup of eight waves owns one query row and 16 heads (8 when there are no more) and walks the row's context block by block:
+// A workgroup of eight waves owns one query row and 16 heads and walks the row's context block by block:
 //   load    the block's int8 rows and rotary rows from the NZ layout into row-major LDS tiles;
-//   scores  thread (token, quarter of the heads): its row against its query heads, each cache dword reused for
-//           all of them;
-//   softmax one wave per head (or per two), two tokens a lane;
-//   values  thread (4 channels, quarter of the heads): four cache rows at a time, their bytes transposed in
-//           registers so that one dot4 covers four tokens.
-// Four barriers a block and no overlap of the load with the arithmetic: built for exact agreement with the
-// golden first.
+//   scores  wave w for tokens 16 w .. 16 w + 15: S^T[token, head] = K . Q^T, eight int8 MFMAs over the 512
+//           latent channels (K rows from LDS as A, the query resident in registers as B) and two 16-bit MFMAs
+//           over the rotary channels;
+//   softmax wave w for heads 2 w and 2 w + 1, two tokens a lane; int8 weights P[head][token] go to LDS;
+//   values  wave w for channels 64 w .. 64 w + 63: O^T[channel, head] += V^T . P^T, V^T read from the row-major
+//           tile by the transposing ds_read_b64_tr_b8 (lane (channel, kg) gets the bytes of 8 consecutive
+//           tokens), P^T as 16 consecutive bytes of a head's weights.
+// Operand layout of v_mfma_i32_16x16x64_i8 (checked with a probe on the device): lane (n = lane % 16, kg =
+// lane / 16) supplies the 16 contraction values 16 kg .. 16 kg + 15 of row n (A) / column n (B) and receives
+// D[4 kg + e][n], e = 0 .. 3.
+// Four barriers a block, one pass per query row (no split over the context).
 #include <vector>
 #include "pa_internal.h"
 #include "upload_ring.h"
@@ -31,26 +35,28 @@ namespace atbmi {
 namespace mlaint8 {
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int TILE = 128;            // tokens per tile = the block size of the cache
 constexpr int DN = 512;              // int8 channels (keys and values)
 constexpr int DR = 64;               // rotary channels (16-bit)
-constexpr int THREADS = 512;         // eight waves, two a SIMD: one's LDS round trips hide behind the other's arithmetic
+constexpr int HT = 16;               // heads per workgroup (the N extent of the MFMA)
+constexpr int THREADS = 512;         // eight waves, two a SIMD
+constexpr int NWAVES = THREADS / WAVE;
 constexpr int K_PITCH = DN + 16;     // bytes; 16-byte reads of 16 consecutive rows touch every bank once
 constexpr int R_PITCH = DR * 2 + 16;
-// LDS of a workgroup with HT heads: the two tiles, the query (int8 rows, fp32 rotary rows), the tile's scores,
-// its int8 weights and four numbers per head {keep, value scale, 1 / sum, lse}.
-template <int HT> struct Lds {
-    static constexpr int K = 0;
-    static constexpr int R = K + TILE * K_PITCH;
-    static constexpr int Q8 = R + TILE * R_PITCH;
-    static constexpr int QR = Q8 + HT * DN;
-    static constexpr int S = QR + HT * DR * 4;
-    static constexpr int P = S + HT * TILE * 4;
-    static constexpr int STAT = P + HT * TILE;
-    static constexpr int BYTES = STAT + HT * 16;
-    static_assert(BYTES <= 160 * 1024 && R % 16 == 0 && Q8 % 16 == 0 && S % 16 == 0, "LDS layout");
-};
+constexpr int LDS_K = 0;
+constexpr int LDS_R = LDS_K + TILE * K_PITCH;
+constexpr int LDS_S = LDS_R + TILE * R_PITCH;          // [HT][TILE] fp32 scores
+constexpr int LDS_P = LDS_S + HT * TILE * 4;           // [HT][TILE] int8 weights
+constexpr int LDS_STAT = LDS_P + HT * TILE;            // [HT] {keep, value scale, 1 / sum, lse}
+constexpr int LDS_BYTES = LDS_STAT + HT * 16;
+static_assert(LDS_BYTES <= 160 * 1024 && LDS_R % 16 == 0 && LDS_S % 16 == 0 && LDS_P % 16 == 0, "LDS layout");
+static_assert(TILE == NWAVES * 16 && DN == NWAVES * 64 && HT == 2 * NWAVES, "eight waves share a tile this way");
 
 // One query row: its sequence's block-table row and context length, the row of query / out, the mask row.
 struct Row {
@@ -75,7 +81,6 @@ struct Args {
     int32_t H;
     int32_t maxBlocksPerSeq;
     int32_t maskLen;
-    int32_t bf16;
     float qkScale;
 };
 
@@ -84,69 +89,69 @@ __device__ __forceinline__ float Load16AsFloat(uint32_t bits, bool bf16)
     return bf16 ? Bf16ToFloat(static_cast<uint16_t>(bits)) : HalfBitsToFloat(static_cast<uint16_t>(bits));
 }
 
-// HT heads per workgroup (8 or 16): a thread takes HT / 4 heads in the score and value phases, a wave HT / 8
-// in the softmax.
-template <int HT> __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
+template <bool BF16> __device__ __forceinline__ f32x4 Mma16(u32x4 a, u32x4 b, f32x4 c)
 {
-    using L = Lds<HT>;
-    constexpr int LDS_K = L::K, LDS_R = L::R, LDS_Q8 = L::Q8, LDS_QR = L::QR, LDS_S = L::S, LDS_P = L::P,
-                  LDS_STAT = L::STAT;
-    constexpr int HPT = HT / 4; // heads per thread
-    constexpr int HPW = HT / 8; // heads per wave
+    if constexpr (BF16) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
+                                                       c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c,
+                                                      0, 0, 0);
+    }
+}
+
+template <bool BF16> __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
+{
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x;
     const int lane = tid & (WAVE - 1);
     const int wave = tid / WAVE;
-    const int headTiles = a.H / HT;
+    const int n = lane & 15;  // MFMA row (A) / column (B, D) of this lane
+    const int kg = lane >> 4; // which 16 contraction values / 4 result rows this lane holds
+    const int headTiles = (a.H + HT - 1) / HT;
     const Row row = a.rows[blockIdx.x / headTiles];
     const int h0 = (blockIdx.x % headTiles) * HT;
-    const bool bf16 = a.bf16 != 0;
+    const int nh = min(HT, a.H - h0);                 // heads past the last one compute on zeros and store nothing
+    const int hn = h0 + min(n, nh - 1);               // a head this lane may read the descale of
     const int32_t *table = a.tables + static_cast<int64_t>(row.tableRow) * a.maxBlocksPerSeq;
 
-    // ---- the query of the eight heads: int8 rows as they are, rotary rows as fp32
+    // ---- Q^T as B operands: lane (n, kg) holds q8[head n][64 j + 16 kg .. +16) and qRope[head n][32 m + 8 kg .. +8)
+    i32x4 q8[DN / 64];
+    u32x4 qr[DR / 32];
     {
-        const int8_t *q8 = a.q8 + (static_cast<int64_t>(row.qRow) * a.H + h0) * DN;
-        if (tid < HT * DN / 16) {
-            *reinterpret_cast<u32x4 *>(smem + LDS_Q8 + tid * 16) = *reinterpret_cast<const u32x4 *>(q8 + tid * 16);
+        const int64_t rowHead = static_cast<int64_t>(row.qRow) * a.H + hn;
+#pragma unroll
+        for (int j = 0; j < DN / 64; ++j) {
+            q8[j] = *reinterpret_cast<const i32x4 *>(a.q8 + rowHead * DN + j * 64 + kg * 16);
+            if (n >= nh) {
+                q8[j] = i32x4{0, 0, 0, 0};
+            }
         }
-        const uint16_t *qr = reinterpret_cast<const uint16_t *>(a.qRope) + (static_cast<int64_t>(row.qRow) * a.H + h0) * DR;
-        float *dst = reinterpret_cast<float *>(smem + LDS_QR);
-        for (int i = tid; i < HT * DR; i += THREADS) {
-            dst[i] = Load16AsFloat(qr[i], bf16);
-        }
-    }
-
-    // scores: thread (token, group of four heads)
-    const int tok = tid & (TILE - 1);
-    const int hs = (tid / TILE) * HPT;
-    // softmax: this wave's two heads; the running maximum, sum and per-tile factors live in its lanes
-    float runMax[HPW], runSum[HPW];
 #pragma unroll
-    for (int i = 0; i < HPW; ++i) {
-        runMax[i] = -INFINITY;
-        runSum[i] = 0.0f;
-    }
-    // values: thread (4 channels, group of four heads)
-    const int col = tid & (TILE - 1); // dword column of a cache row
-    float acc[HPT][4];
-#pragma unroll
-    for (int h = 0; h < HPT; ++h) {
-#pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            acc[h][b] = 0.0f;
+        for (int m = 0; m < DR / 32; ++m) {
+            qr[m] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const uint16_t *>(a.qRope) + rowHead * DR + m * 32 + kg * 8);
+            if (n >= nh) {
+                qr[m] = u32x4{0u, 0u, 0u, 0u};
+            }
         }
     }
-    float descale[HPT];
-#pragma unroll
-    for (int h = 0; h < HPT; ++h) {
-        descale[h] = a.qkDescale[h0 + hs + h];
-    }
+    const float descale = a.qkDescale[hn];
     const uint16_t *maskRow = a.mask ? reinterpret_cast<const uint16_t *>(a.mask) + static_cast<int64_t>(row.qRow) * a.maskLen
                                      : nullptr;
+    // softmax: this wave's two heads; the running maximum and sum live in its lanes
+    float runMax[2] = {-INFINITY, -INFINITY};
+    float runSum[2] = {0.0f, 0.0f};
+    // values: channels 64 wave + 16 cs + 4 kg + e of head n
+    f32x4 acc[4];
+#pragma unroll
+    for (int cs = 0; cs < 4; ++cs) {
+        acc[cs] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    const int l16 = lane & 15;
 
     for (int t0 = 0; t0 < row.ctxLen; t0 += TILE) {
         const int64_t blk = table[t0 / TILE];
-        __syncthreads(); // the tiles (and, the first time, the query) are free / written
+        __syncthreads(); // everybody has left the tiles of the block before
         // ---- the block, NZ [channels / 32][128][32] int8 and [4][128][16] 16-bit, into row-major tiles
         {
             const u32x4 *src = reinterpret_cast<const u32x4 *>(a.kv8 + blk * (TILE * DN));
@@ -154,67 +159,49 @@ template <int HT> __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const
             for (int v = tid; v < TILE * DN / 16; v += THREADS) {
                 const int slab = v / (TILE * 2);
                 const int r = (v % (TILE * 2)) / 2;
-                *reinterpret_cast<u32x4 *>(smem + LDS_K + r * K_PITCH + slab * 32 + (v & 1) * 16) =
-                    src[v];
+                *reinterpret_cast<u32x4 *>(smem + LDS_K + r * K_PITCH + slab * 32 + (v & 1) * 16) = src[v];
             }
             const u32x4 *srcR = reinterpret_cast<const u32x4 *>(reinterpret_cast<const unsigned char *>(a.kRope) +
                                                                 blk * (TILE * DR * 2));
             for (int v = tid; v < TILE * DR * 2 / 16; v += THREADS) {
                 const int slab = v / (TILE * 2);
                 const int r = (v % (TILE * 2)) / 2;
-                *reinterpret_cast<u32x4 *>(smem + LDS_R + r * R_PITCH + slab * 32 + (v & 1) * 16) =
-                    srcR[v];
+                *reinterpret_cast<u32x4 *>(smem + LDS_R + r * R_PITCH + slab * 32 + (v & 1) * 16) = srcR[v];
             }
         }
         __syncthreads();
-        // ---- scores of token `tok` for heads hs .. hs + 3
+        // ---- scores of tokens 16 wave .. + 15 for the 16 heads
         {
-            int dot[HPT] = {};
-            const unsigned char *krow = smem + LDS_K + tok * K_PITCH;
-#pragma unroll 4
-            for (int j = 0; j < DN / 16; ++j) {
-                const u32x4 kk = *reinterpret_cast<const u32x4 *>(krow + j * 16);
+            i32x4 dot = {0, 0, 0, 0};
+            const unsigned char *krow = smem + LDS_K + (wave * 16 + n) * K_PITCH + kg * 16;
 #pragma unroll
-                for (int h = 0; h < HPT; ++h) {
-                    const u32x4 qq = *reinterpret_cast<const u32x4 *>(smem + LDS_Q8 + (hs + h) * DN + j * 16);
-#pragma unroll
-                    for (int d = 0; d < 4; ++d) {
-                        dot[h] = __builtin_amdgcn_sdot4(static_cast<int>(kk[d]), static_cast<int>(qq[d]), dot[h], false);
-                    }
-                }
+            for (int j = 0; j < DN / 64; ++j) {
+                const i32x4 kk = *reinterpret_cast<const i32x4 *>(krow + j * 64);
+                dot = __builtin_amdgcn_mfma_i32_16x16x64_i8(kk, q8[j], dot, 0, 0, 0);
             }
-            float rope[HPT] = {};
-            const unsigned char *rrow = smem + LDS_R + tok * R_PITCH;
-#pragma unroll 2
-            for (int j = 0; j < DR / 8; ++j) {
-                const u32x4 rr = *reinterpret_cast<const u32x4 *>(rrow + j * 16);
-                float kf[8];
+            f32x4 rope = {0.0f, 0.0f, 0.0f, 0.0f};
+            const unsigned char *rrow = smem + LDS_R + (wave * 16 + n) * R_PITCH + kg * 16;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    kf[e] = Load16AsFloat((e & 1) ? (rr[e >> 1] >> 16) : (rr[e >> 1] & 0xffffu), bf16);
-                }
-#pragma unroll
-                for (int h = 0; h < HPT; ++h) {
-                    const float *qf = reinterpret_cast<const float *>(smem + LDS_QR) + (hs + h) * DR + j * 8;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        rope[h] = __builtin_fmaf(qf[e], kf[e], rope[h]);
-                    }
-                }
+            for (int m = 0; m < DR / 32; ++m) {
+                rope = Mma16<BF16>(*reinterpret_cast<const u32x4 *>(rrow + m * 64), qr[m], rope);
             }
-            const bool live = t0 + tok < row.ctxLen;
-            const float bias = (maskRow && live) ? Load16AsFloat(maskRow[t0 + tok], bf16) : 0.0f;
+            // lane (head n, kg) holds tokens 16 wave + 4 kg + e
+            const int tok = t0 + wave * 16 + kg * 4;
+            f32x4 sc;
 #pragma unroll
-            for (int h = 0; h < HPT; ++h) {
-                float s = (static_cast<float>(dot[h]) * descale[h] + rope[h]) * a.qkScale + bias;
-                reinterpret_cast<float *>(smem + LDS_S)[(hs + h) * TILE + tok] = live ? s : -INFINITY;
+            for (int e = 0; e < 4; ++e) {
+                const bool live = tok + e < row.ctxLen;
+                const float bias = (maskRow && live) ? Load16AsFloat(maskRow[tok + e], BF16) : 0.0f;
+                const float x = (static_cast<float>(dot[e]) * descale + rope[e]) * a.qkScale + bias;
+                sc[e] = live ? x : -INFINITY;
             }
+            *reinterpret_cast<f32x4 *>(smem + LDS_S + (n * TILE + wave * 16 + kg * 4) * 4) = sc;
         }
         __syncthreads();
         // ---- weights of the tile for heads 2 wave, 2 wave + 1
 #pragma unroll
-        for (int i = 0; i < HPW; ++i) {
-            const int h = HPW * wave + i;
+        for (int i = 0; i < 2; ++i) {
+            const int h = 2 * wave + i;
             const float *srow = reinterpret_cast<const float *>(smem + LDS_S) + h * TILE;
             const float s0 = srow[lane], s1 = srow[lane + WAVE];
             float tileMax = fmaxf(s0, s1);
@@ -245,54 +232,33 @@ template <int HT> __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const
             if (lane == 0) {
                 float *stat = reinterpret_cast<float *>(smem + LDS_STAT) + h * 4;
                 stat[0] = keep;
-                stat[1] = a.pvDescale[h0 + h] * wmax / 127.0f;
+                stat[1] = a.pvDescale[h0 + min(h, nh - 1)] * wmax / 127.0f;
             }
         }
         __syncthreads();
-        // ---- values: channels 4 col .. 4 col + 3 for heads hs .. hs + 3
+        // ---- values: O^T[channel, head] += V^T . P^T for channels 64 wave .. + 63
         {
-            int iacc[HPT][4];
+            const float keep = reinterpret_cast<const float *>(smem + LDS_STAT)[n * 4];
+            const float vscale = reinterpret_cast<const float *>(smem + LDS_STAT)[n * 4 + 1];
+            // the transposing read hands lane (channel l16, kg) the bytes of tokens r .. r + 7 when lane l16 of the
+            // group points at token r + l16 / 2, channels (l16 % 2) * 8 .. + 8
+            const unsigned char *vbase = smem + LDS_K + (kg * 16 + (l16 >> 1)) * K_PITCH + wave * 64 + (l16 & 1) * 8;
+            const unsigned char *pbase = smem + LDS_P + n * TILE + kg * 16;
 #pragma unroll
-            for (int h = 0; h < HPT; ++h) {
+            for (int cs = 0; cs < 4; ++cs) {
+                i32x4 iacc = {0, 0, 0, 0};
 #pragma unroll
-                for (int b = 0; b < 4; ++b) {
-                    iacc[h][b] = 0;
+                for (int hh = 0; hh < TILE / 64; ++hh) {
+                    const unsigned char *vp = vbase + hh * 64 * K_PITCH + cs * 16;
+                    const i32x2 lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2 *)(vp));
+                    const i32x2 hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                        (__attribute__((address_space(3))) i32x2 *)(vp + 8 * K_PITCH));
+                    const i32x4 pw = *reinterpret_cast<const i32x4 *>(pbase + hh * 64);
+                    iacc = __builtin_amdgcn_mfma_i32_16x16x64_i8(i32x4{lo[0], lo[1], hi[0], hi[1]}, pw, iacc, 0, 0, 0);
                 }
-            }
-            const unsigned char *kcol = smem + LDS_K + col * 4;
-#pragma unroll 2
-            for (int t4 = 0; t4 < TILE / 4; ++t4) {
-                uint32_t r[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    r[i] = *reinterpret_cast<const uint32_t *>(kcol + (t4 * 4 + i) * K_PITCH);
-                }
-                // bytes of four rows transposed: kt[b] = {r0.b, r1.b, r2.b, r3.b}
-                const uint32_t x01lo = __builtin_amdgcn_perm(r[1], r[0], 0x05010400u);
-                const uint32_t x01hi = __builtin_amdgcn_perm(r[1], r[0], 0x07030602u);
-                const uint32_t x23lo = __builtin_amdgcn_perm(r[3], r[2], 0x05010400u);
-                const uint32_t x23hi = __builtin_amdgcn_perm(r[3], r[2], 0x07030602u);
-                uint32_t kt[4];
-                kt[0] = __builtin_amdgcn_perm(x23lo, x01lo, 0x05040100u);
-                kt[1] = __builtin_amdgcn_perm(x23lo, x01lo, 0x07060302u);
-                kt[2] = __builtin_amdgcn_perm(x23hi, x01hi, 0x05040100u);
-                kt[3] = __builtin_amdgcn_perm(x23hi, x01hi, 0x07060302u);
-#pragma unroll
-                for (int h = 0; h < HPT; ++h) {
-                    const uint32_t pw = *reinterpret_cast<const uint32_t *>(smem + LDS_P + (hs + h) * TILE + t4 * 4);
-#pragma unroll
-                    for (int b = 0; b < 4; ++b) {
-                        iacc[h][b] = __builtin_amdgcn_sdot4(static_cast<int>(kt[b]), static_cast<int>(pw), iacc[h][b], false);
-                    }
-                }
-            }
-#pragma unroll
-            for (int h = 0; h < HPT; ++h) {
-                const float *stat = reinterpret_cast<const float *>(smem + LDS_STAT) + (hs + h) * 4;
-                const float keep = stat[0], vscale = stat[1];
-#pragma unroll
-                for (int b = 0; b < 4; ++b) {
-                    acc[h][b] = acc[h][b] * keep + static_cast<float>(iacc[h][b]) * vscale;
+                for (int e = 0; e < 4; ++e) {
+                    acc[cs][e] = acc[cs][e] * keep + static_cast<float>(iacc[e]) * vscale;
                 }
             }
         }
@@ -301,29 +267,32 @@ template <int HT> __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const
     __syncthreads();
     if (lane == 0) {
 #pragma unroll
-        for (int i = 0; i < HPW; ++i) {
-            float *stat = reinterpret_cast<float *>(smem + LDS_STAT) + (HPW * wave + i) * 4;
+        for (int i = 0; i < 2; ++i) {
+            float *stat = reinterpret_cast<float *>(smem + LDS_STAT) + (2 * wave + i) * 4;
             stat[2] = runSum[i] > 0.0f ? 1.0f / runSum[i] : 0.0f;
             stat[3] = runSum[i] > 0.0f ? logf(runSum[i]) + runMax[i] : -INFINITY;
         }
     }
     __syncthreads();
+    if (n < nh) {
+        const float inv = reinterpret_cast<const float *>(smem + LDS_STAT)[n * 4 + 2];
+        uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) + (static_cast<int64_t>(row.qRow) * a.H + h0 + n) * DN +
+                         wave * 64 + kg * 4;
 #pragma unroll
-    for (int h = 0; h < HPT; ++h) {
-        const float inv = reinterpret_cast<const float *>(smem + LDS_STAT)[(hs + h) * 4 + 2];
-        uint16_t bits[4];
+        for (int cs = 0; cs < 4; ++cs) {
+            uint16_t bits[4];
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            const float o = acc[h][b] * inv;
-            bits[b] = bf16 ? FloatToBf16(o) : FloatToHalfBits(o);
+            for (int e = 0; e < 4; ++e) {
+                const float o = acc[cs][e] * inv;
+                bits[e] = BF16 ? FloatToBf16(o) : FloatToHalfBits(o);
+            }
+            uint2 w;
+            w.x = static_cast<uint32_t>(bits[0]) | (static_cast<uint32_t>(bits[1]) << 16);
+            w.y = static_cast<uint32_t>(bits[2]) | (static_cast<uint32_t>(bits[3]) << 16);
+            *reinterpret_cast<uint2 *>(orow + cs * 16) = w;
         }
-        uint2 w;
-        w.x = static_cast<uint32_t>(bits[0]) | (static_cast<uint32_t>(bits[1]) << 16);
-        w.y = static_cast<uint32_t>(bits[2]) | (static_cast<uint32_t>(bits[3]) << 16);
-        uint16_t *dst = reinterpret_cast<uint16_t *>(a.out) + (static_cast<int64_t>(row.qRow) * a.H + h0 + hs + h) * DN + col * 4;
-        *reinterpret_cast<uint2 *>(dst) = w;
     }
-    if (a.lse && tid < HT) {
+    if (a.lse && tid < nh) {
         a.lse[static_cast<int64_t>(row.qRow) * a.H + h0 + tid] = reinterpret_cast<const float *>(smem + LDS_STAT)[tid * 4 + 3];
     }
 }
@@ -337,8 +306,8 @@ int BuildRows(const AtbmiMlaInt8Call *c, std::vector<Row> *rows)
     if (c->outDtype != ATBMI_F16 && c->outDtype != ATBMI_BF16) {
         return Fail(ERR_INVALID_PARAM, "mla_int8: the 16-bit tensors are fp16 or bf16, got %d", c->outDtype);
     }
-    if (c->numHeads <= 0 || c->numHeads % 8 != 0) {
-        return Fail(ERR_INVALID_PARAM, "mla_int8: %d heads (a multiple of 8)", c->numHeads);
+    if (c->numHeads <= 0) {
+        return Fail(ERR_INVALID_PARAM, "mla_int8: %d heads", c->numHeads);
     }
     if (c->blockSize != TILE) {
         return Fail(ERR_INVALID_PARAM, "mla_int8: block size %d (the int8 cache has blocks of %d tokens)", c->blockSize, TILE);
@@ -422,8 +391,7 @@ extern "C" int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspa
         return Fail(ERR_INVALID_PARAM, "mla_int8: workspace of %llu bytes, %llu needed", (unsigned long long)workspaceBytes,
                     (unsigned long long)bytes);
     }
-    const int ht = call->numHeads % 16 == 0 ? 16 : 8;
-    const int64_t grid = static_cast<int64_t>(rows.size()) * (call->numHeads / ht);
+    const int64_t grid = static_cast<int64_t>(rows.size()) * ((call->numHeads + mlaint8::HT - 1) / mlaint8::HT);
     if (grid > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "mla_int8: %lld workgroups", (long long)grid);
     }
@@ -447,15 +415,19 @@ extern "C" int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspa
     a.H = call->numHeads;
     a.maxBlocksPerSeq = call->maxBlocksPerSeq;
     a.maskLen = call->maskLen;
-    a.bf16 = call->outDtype == ATBMI_BF16 ? 1 : 0;
     a.qkScale = call->qkScale;
-    auto kernel = ht == 16 ? mlaint8::MlaInt8Kernel<16> : mlaint8::MlaInt8Kernel<8>;
-    const int ldsBytes = ht == 16 ? mlaint8::Lds<16>::BYTES : mlaint8::Lds<8>::BYTES;
+    auto kernel = call->outDtype == ATBMI_BF16 ? mlaint8::MlaInt8Kernel<true> : mlaint8::MlaInt8Kernel<false>;
+    const int ldsBytes = mlaint8::LDS_BYTES;
     rc = ConfigureKernelLds(reinterpret_cast<const void *>(kernel), ldsBytes);
+    if (rc != OK) {
+        return rc;
+    }
+    TimedLaunch timed;
+    rc = TimedLaunchBegin(s, &timed);
     if (rc != OK) {
         return rc;
     }
     kernel<<<static_cast<unsigned>(grid), mlaint8::THREADS, ldsBytes, s>>>(a);
     ATBMI_HIP_CHECK(hipGetLastError());
-    return OK;
+    return TimedLaunchEnd(s, timed);
 }

@@ -133,6 +133,33 @@ int64_t g_timingLaunch = 0;
 std::vector<TimingRecord> g_timingRecords;
 
 } // namespace
+
+int TimedLaunchBegin(hipStream_t stream, TimedLaunch *launch)
+{
+    *launch = TimedLaunch{};
+    {
+        std::lock_guard<std::mutex> lock(g_timingMutex);
+        if (g_timingEvery <= 0 || (g_timingLaunch++ % g_timingEvery) != 0) {
+            return OK;
+        }
+    }
+    ATBMI_HIP_CHECK(hipEventCreate(&launch->begin));
+    ATBMI_HIP_CHECK(hipEventCreate(&launch->end));
+    ATBMI_HIP_CHECK(hipEventRecord(launch->begin, stream));
+    return OK;
+}
+
+int TimedLaunchEnd(hipStream_t stream, const TimedLaunch &launch)
+{
+    if (!launch.begin) {
+        return OK;
+    }
+    ATBMI_HIP_CHECK(hipEventRecord(launch.end, stream));
+    std::lock_guard<std::mutex> lock(g_timingMutex);
+    g_timingRecords.push_back(TimingRecord{launch.begin, launch.end, nullptr});
+    return OK;
+}
+
 } // namespace atbmi
 
 using namespace atbmi;
