@@ -14,19 +14,21 @@
 //             denominator adds up the unquantised weights.
 // Every integer product is exact (v_mfma_i32_16x16x64_i8; a tile's sums stay below 2^24).
 //
-// A workgroup of eight waves owns one query row and 16 heads and walks the row's context block by block:
-//   load    the block's int8 rows and rotary rows from the NZ layout into row-major LDS tiles;
+// A workgroup of eight waves owns one query row and 32 heads (16 when the call has no more) and walks the
+// row's context block by block. The int8 rows of a block go from the cache to LDS without passing through
+// registers (global_load_lds_dwordx4), one block ahead of the arithmetic, into one of two 64 KiB buffers; the
+// rotary rows, which only the wave that scores their tokens needs, are prefetched into that wave's registers.
 //   scores  wave w for tokens 16 w .. 16 w + 15: S^T[token, head] = K . Q^T, eight int8 MFMAs over the 512
 //           latent channels (K rows from LDS as A, the query resident in registers as B) and two 16-bit MFMAs
-//           over the rotary channels;
-//   softmax wave w for heads 2 w and 2 w + 1, two tokens a lane; int8 weights P[head][token] go to LDS;
-//   values  wave w for channels 64 w .. 64 w + 63: O^T[channel, head] += V^T . P^T, V^T read from the row-major
-//           tile by the transposing ds_read_b64_tr_b8 (lane (channel, kg) gets the bytes of 8 consecutive
+//           over the rotary channels, per tile of 16 heads;
+//   softmax 16 (32) lanes a head, 8 (4) tokens a lane; int8 weights P[head][token] go to LDS;
+//   values  wave w for channels 64 w .. 64 w + 63: O^T[channel, head] += V^T . P^T, V^T read from the token-major
+//           buffer by the transposing ds_read_b64_tr_b8 (lane (channel, kg) gets the bytes of 8 consecutive
 //           tokens), P^T as 16 consecutive bytes of a head's weights.
 // Operand layout of v_mfma_i32_16x16x64_i8 (checked with a probe on the device): lane (n = lane % 16, kg =
 // lane / 16) supplies the 16 contraction values 16 kg .. 16 kg + 15 of row n (A) / column n (B) and receives
 // D[4 kg + e][n], e = 0 .. 3.
-// Four barriers a block, one pass per query row (no split over the context).
+// Three barriers a block, one pass per query row (no split over the context).
 #include <vector>
 #include "pa_internal.h"
 #include "upload_ring.h"
@@ -44,19 +46,28 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 constexpr int TILE = 128;            // tokens per tile = the block size of the cache
 constexpr int DN = 512;              // int8 channels (keys and values)
 constexpr int DR = 64;               // rotary channels (16-bit)
-constexpr int HT = 16;               // heads per workgroup (the N extent of the MFMA)
+constexpr int HT = 16;               // heads per head tile (the N extent of the MFMA)
 constexpr int THREADS = 512;         // eight waves, two a SIMD
 constexpr int NWAVES = THREADS / WAVE;
-constexpr int K_PITCH = DN + 16;     // bytes; 16-byte reads of 16 consecutive rows touch every bank once
-constexpr int R_PITCH = DR * 2 + 16;
-constexpr int LDS_K = 0;
-constexpr int LDS_R = LDS_K + TILE * K_PITCH;
-constexpr int LDS_S = LDS_R + TILE * R_PITCH;          // [HT][TILE] fp32 scores
-constexpr int LDS_P = LDS_S + HT * TILE * 4;           // [HT][TILE] int8 weights
-constexpr int LDS_STAT = LDS_P + HT * TILE;            // [HT] {keep, value scale, 1 / sum, lse}
-constexpr int LDS_BYTES = LDS_STAT + HT * 16;
-static_assert(LDS_BYTES <= 160 * 1024 && LDS_R % 16 == 0 && LDS_S % 16 == 0 && LDS_P % 16 == 0, "LDS layout");
-static_assert(TILE == NWAVES * 16 && DN == NWAVES * 64 && HT == 2 * NWAVES, "eight waves share a tile this way");
+// A block in LDS: the 1 KiB pieces of the NZ block ([channels / 32][128 tokens][32 bytes]: piece c = 32 tokens of
+// one 32-channel slab) keep their order, and inside a piece the 16-byte halves of the 32 tokens are parted: the
+// low halves first, 16 bytes a token, then the high halves. Sixteen tokens' reads of one half are then 256
+// contiguous bytes (every bank once), and so are the eight tokens x 16 channels of a transposing read.
+constexpr int K_BYTES = TILE * DN;
+constexpr int PIECE = 1024;
+constexpr int PIECES_PER_WAVE = K_BYTES / PIECE / NWAVES;
+constexpr int S_PITCH = (TILE + 4) * 4; // 16 heads' 16-byte writes touch every bank once
+constexpr int P_PITCH = TILE + 16;      // likewise for 16 heads' 16-byte reads
+template <int NT> struct Lds {
+    static constexpr int K = 0;                          // two blocks
+    static constexpr int S = 2 * K_BYTES;                // [16 NT] fp32 scores
+    static constexpr int P = S + NT * HT * S_PITCH;      // [16 NT] int8 weights
+    static constexpr int STAT = P + NT * HT * P_PITCH;   // [16 NT] {keep, value scale, 1 / sum, lse}
+    static constexpr int BYTES = STAT + NT * HT * 16;
+    static_assert(BYTES <= 160 * 1024 && S % 16 == 0 && P % 16 == 0 && STAT % 16 == 0, "LDS layout");
+};
+static_assert(TILE == NWAVES * 16 && DN == NWAVES * 64 && K_BYTES % (PIECE * NWAVES) == 0,
+              "eight waves share a tile this way");
 
 // One query row: its sequence's block-table row and context length, the row of query / out, the mask row.
 struct Row {
@@ -79,6 +90,7 @@ struct Args {
     float *lse;
     const Row *rows;
     int32_t H;
+    int32_t numRows;
     int32_t maxBlocksPerSeq;
     int32_t maskLen;
     float qkScale;
@@ -100,200 +112,326 @@ template <bool BF16> __device__ __forceinline__ f32x4 Mma16(u32x4 a, u32x4 b, f3
     }
 }
 
-template <bool BF16> __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
+// 16 bytes per lane from `src` to LDS address ldsBase + 16 x lane (ldsBase wave-uniform). The compiler does not
+// count these loads: the kernel waits for them with WaitForLoads.
+__device__ __forceinline__ void TransferToLds(uint32_t ldsBase, const void *src)
 {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(ldsBase), "v"(src) : "memory", "m0");
+}
+
+__device__ __forceinline__ void WaitForLoads()
+{
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+}
+
+// Makes the compiler treat a loaded value as used here, so that the wait it inserts for the load lands here
+// (next to WaitForLoads) and not later, behind transfers that were requested in between.
+template <typename T> __device__ __forceinline__ void Pin(T &v)
+{
+    asm volatile("" : "+v"(v));
+}
+
+template <bool BF16, int NT>
+__global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
+{
+    using L = Lds<NT>;
+    constexpr int HW = NT * HT;          // heads of the workgroup
+    constexpr int CH = THREADS / HW;     // softmax: lanes a head
+    constexpr int TPL = TILE / CH;       // softmax: tokens a lane
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x;
     const int lane = tid & (WAVE - 1);
-    const int wave = tid / WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
     const int n = lane & 15;  // MFMA row (A) / column (B, D) of this lane
     const int kg = lane >> 4; // which 16 contraction values / 4 result rows this lane holds
-    const int headTiles = (a.H + HT - 1) / HT;
-    const Row row = a.rows[blockIdx.x / headTiles];
-    const int h0 = (blockIdx.x % headTiles) * HT;
-    const int nh = min(HT, a.H - h0);                 // heads past the last one compute on zeros and store nothing
-    const int hn = h0 + min(n, nh - 1);               // a head this lane may read the descale of
+    const int headTiles = (a.H + HW - 1) / HW;
+    // workgroups go round the eight XCDs: the head tiles of a row, which read the same cache blocks, take
+    // neighbouring places on one XCD and share its L2
+    const int work = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
+    if (work >= a.numRows * headTiles) {
+        return;
+    }
+    const Row row = a.rows[work / headTiles];
+    const int h0 = (work % headTiles) * HW;
+    const int nh = min(HW, a.H - h0); // heads past the last one compute on zeros and store nothing
     const int32_t *table = a.tables + static_cast<int64_t>(row.tableRow) * a.maxBlocksPerSeq;
+    const int numBlocks = (row.ctxLen + TILE - 1) / TILE;
+    const uint32_t ldsBase =
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char *)smem));
+
+    // ---- requests for a block: this wave's eight pieces of the int8 rows, and its tokens' rotary rows
+    const int pieceLane = (lane & 31) * 32 + (lane >> 5) * 16; // token lane % 32, half lane / 32
+    auto requestBlock = [&](int64_t blk, int buf) {
+        const unsigned char *src = reinterpret_cast<const unsigned char *>(a.kv8) + blk * K_BYTES +
+                                   wave * (PIECES_PER_WAVE * PIECE) + pieceLane;
+        const uint32_t dst = ldsBase + L::K + buf * K_BYTES + wave * (PIECES_PER_WAVE * PIECE);
+#pragma unroll
+        for (int i = 0; i < PIECES_PER_WAVE; ++i) {
+            TransferToLds(__builtin_amdgcn_readfirstlane(dst + i * PIECE), src + i * PIECE);
+        }
+    };
+    // lane (token n of the wave's 16, kg): rotary channels 32 m + 8 kg .. + 8, NZ [4][128][16]
+    const int ropeLane = (kg >> 1) * (TILE * 32) + (wave * 16 + n) * 32 + (kg & 1) * 16;
+    auto loadRope = [&](int64_t blk, u32x4(&r)[DR / 32]) {
+        const unsigned char *src = reinterpret_cast<const unsigned char *>(a.kRope) + blk * (TILE * DR * 2) + ropeLane;
+#pragma unroll
+        for (int m = 0; m < DR / 32; ++m) {
+            r[m] = *reinterpret_cast<const u32x4 *>(src + m * (2 * TILE * 32));
+        }
+    };
+    u32x4 ropeNext[DR / 32] = {};
+    if (numBlocks > 0) {
+        const int64_t blk = table[0];
+        loadRope(blk, ropeNext);
+        requestBlock(blk, 0);
+    }
 
     // ---- Q^T as B operands: lane (n, kg) holds q8[head n][64 j + 16 kg .. +16) and qRope[head n][32 m + 8 kg .. +8)
-    i32x4 q8[DN / 64];
-    u32x4 qr[DR / 32];
-    {
+    i32x4 q8[NT][DN / 64];
+    u32x4 qr[NT][DR / 32];
+    float descale[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const bool live = nt * HT + n < nh;
+        const int hn = h0 + min(nt * HT + n, nh - 1);
         const int64_t rowHead = static_cast<int64_t>(row.qRow) * a.H + hn;
 #pragma unroll
         for (int j = 0; j < DN / 64; ++j) {
-            q8[j] = *reinterpret_cast<const i32x4 *>(a.q8 + rowHead * DN + j * 64 + kg * 16);
-            if (n >= nh) {
-                q8[j] = i32x4{0, 0, 0, 0};
+            q8[nt][j] = *reinterpret_cast<const i32x4 *>(a.q8 + rowHead * DN + j * 64 + kg * 16);
+            if (!live) {
+                q8[nt][j] = i32x4{0, 0, 0, 0};
             }
         }
 #pragma unroll
         for (int m = 0; m < DR / 32; ++m) {
-            qr[m] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const uint16_t *>(a.qRope) + rowHead * DR + m * 32 + kg * 8);
-            if (n >= nh) {
-                qr[m] = u32x4{0u, 0u, 0u, 0u};
+            qr[nt][m] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const uint16_t *>(a.qRope) + rowHead * DR +
+                                                          m * 32 + kg * 8);
+            if (!live) {
+                qr[nt][m] = u32x4{0u, 0u, 0u, 0u};
             }
         }
+        descale[nt] = a.qkDescale[hn];
     }
-    const float descale = a.qkDescale[hn];
     const uint16_t *maskRow = a.mask ? reinterpret_cast<const uint16_t *>(a.mask) + static_cast<int64_t>(row.qRow) * a.maskLen
                                      : nullptr;
-    // softmax: this wave's two heads; the running maximum and sum live in its lanes
-    float runMax[2] = {-INFINITY, -INFINITY};
-    float runSum[2] = {0.0f, 0.0f};
-    // values: channels 64 wave + 16 cs + 4 kg + e of head n
-    f32x4 acc[4];
+    // softmax: lane (head tid / CH, tokens TPL (tid % CH) .. + TPL); a head's lanes all hold its running maximum and sum
+    const int smHead = tid / CH;
+    const int smTok = (tid % CH) * TPL;
+    const float smPvDescale = a.pvDescale[h0 + min(smHead, nh - 1)];
+    float runMax = -INFINITY;
+    float runSum = 0.0f;
+    // values: channels 64 wave + 16 cs + 4 kg + e of head 16 nt + n
+    f32x4 acc[NT][4];
 #pragma unroll
-    for (int cs = 0; cs < 4; ++cs) {
-        acc[cs] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    }
-    const int l16 = lane & 15;
-
-    for (int t0 = 0; t0 < row.ctxLen; t0 += TILE) {
-        const int64_t blk = table[t0 / TILE];
-        __syncthreads(); // everybody has left the tiles of the block before
-        // ---- the block, NZ [channels / 32][128][32] int8 and [4][128][16] 16-bit, into row-major tiles
-        {
-            const u32x4 *src = reinterpret_cast<const u32x4 *>(a.kv8 + blk * (TILE * DN));
-#pragma unroll 4
-            for (int v = tid; v < TILE * DN / 16; v += THREADS) {
-                const int slab = v / (TILE * 2);
-                const int r = (v % (TILE * 2)) / 2;
-                *reinterpret_cast<u32x4 *>(smem + LDS_K + r * K_PITCH + slab * 32 + (v & 1) * 16) = src[v];
-            }
-            const u32x4 *srcR = reinterpret_cast<const u32x4 *>(reinterpret_cast<const unsigned char *>(a.kRope) +
-                                                                blk * (TILE * DR * 2));
-            for (int v = tid; v < TILE * DR * 2 / 16; v += THREADS) {
-                const int slab = v / (TILE * 2);
-                const int r = (v % (TILE * 2)) / 2;
-                *reinterpret_cast<u32x4 *>(smem + LDS_R + r * R_PITCH + slab * 32 + (v & 1) * 16) = srcR[v];
-            }
+    for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+        for (int cs = 0; cs < 4; ++cs) {
+            acc[nt][cs] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
         }
-        __syncthreads();
-        // ---- scores of tokens 16 wave .. + 15 for the 16 heads
-        {
-            i32x4 dot = {0, 0, 0, 0};
-            const unsigned char *krow = smem + LDS_K + (wave * 16 + n) * K_PITCH + kg * 16;
-#pragma unroll
-            for (int j = 0; j < DN / 64; ++j) {
-                const i32x4 kk = *reinterpret_cast<const i32x4 *>(krow + j * 64);
-                dot = __builtin_amdgcn_mfma_i32_16x16x64_i8(kk, q8[j], dot, 0, 0, 0);
-            }
-            f32x4 rope = {0.0f, 0.0f, 0.0f, 0.0f};
-            const unsigned char *rrow = smem + LDS_R + (wave * 16 + n) * R_PITCH + kg * 16;
-#pragma unroll
-            for (int m = 0; m < DR / 32; ++m) {
-                rope = Mma16<BF16>(*reinterpret_cast<const u32x4 *>(rrow + m * 64), qr[m], rope);
-            }
-            // lane (head n, kg) holds tokens 16 wave + 4 kg + e
-            const int tok = t0 + wave * 16 + kg * 4;
-            f32x4 sc;
+    }
+    // byte offsets into a block in LDS
+    const int scoreLane = (kg >> 1) * 4096 + (wave >> 1) * PIECE + (kg & 1) * 512 + ((wave & 1) * 16 + n) * 16;
+    // the transposing read hands lane (channel n, kg) the bytes of tokens r .. r + 7 when lane n of the group
+    // points at token r + n / 2, channels (n % 2) * 8 .. + 8
+    const int valueLane = wave * 8192 + (kg >> 1) * PIECE + ((kg & 1) * 16 + (n >> 1)) * 16 + (n & 1) * 8;
+
+    for (int i = 0; i < numBlocks; ++i) {
+        const int t0 = i * TILE;
+        const int tok = t0 + wave * 16 + kg * 4; // scores: this lane's four tokens
+        uint32_t maskBits[4] = {0u, 0u, 0u, 0u};
+        if (maskRow) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const bool live = tok + e < row.ctxLen;
-                const float bias = (maskRow && live) ? Load16AsFloat(maskRow[tok + e], BF16) : 0.0f;
-                const float x = (static_cast<float>(dot[e]) * descale + rope[e]) * a.qkScale + bias;
-                sc[e] = live ? x : -INFINITY;
+                maskBits[e] = maskRow[min(tok + e, row.ctxLen - 1)];
             }
-            *reinterpret_cast<f32x4 *>(smem + LDS_S + (n * TILE + wave * 16 + kg * 4) * 4) = sc;
+        }
+        const bool more = i + 1 < numBlocks;
+        const int64_t nextBlk = more ? table[i + 1] : 0;
+        WaitForLoads(); // this wave's pieces of block i are in LDS, its rotary rows and mask values in registers
+        u32x4 rope[DR / 32];
+#pragma unroll
+        for (int m = 0; m < DR / 32; ++m) {
+            Pin(ropeNext[m]);
+            rope[m] = ropeNext[m];
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            Pin(maskBits[e]);
+        }
+        __syncthreads(); // block i is complete; everybody has left block i - 1, the scores and the weights
+        if (more) {
+            loadRope(nextBlk, ropeNext);
+            requestBlock(nextBlk, (i + 1) & 1);
+        }
+        const unsigned char *kbuf = smem + L::K + (i & 1) * K_BYTES;
+        // ---- scores of tokens 16 wave .. + 15
+        {
+            i32x4 kk[DN / 64];
+#pragma unroll
+            for (int j = 0; j < DN / 64; ++j) {
+                kk[j] = *reinterpret_cast<const i32x4 *>(kbuf + scoreLane + j * 8192);
+            }
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                i32x4 dot = {0, 0, 0, 0};
+#pragma unroll
+                for (int j = 0; j < DN / 64; ++j) {
+                    dot = __builtin_amdgcn_mfma_i32_16x16x64_i8(kk[j], q8[nt][j], dot, 0, 0, 0);
+                }
+                f32x4 rdot = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int m = 0; m < DR / 32; ++m) {
+                    rdot = Mma16<BF16>(rope[m], qr[nt][m], rdot);
+                }
+                f32x4 sc;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const bool live = tok + e < row.ctxLen;
+                    const float bias = maskRow ? Load16AsFloat(maskBits[e], BF16) : 0.0f;
+                    const float x = (static_cast<float>(dot[e]) * descale[nt] + rdot[e]) * a.qkScale + bias;
+                    sc[e] = live ? x : -INFINITY;
+                }
+                *reinterpret_cast<f32x4 *>(smem + L::S + (nt * HT + n) * S_PITCH + (wave * 16 + kg * 4) * 4) = sc;
+            }
         }
         __syncthreads();
-        // ---- weights of the tile for heads 2 wave, 2 wave + 1
+        // ---- weights of the tile
+        {
+            float w[TPL];
+            const float *srow = reinterpret_cast<const float *>(smem + L::S + smHead * S_PITCH) + smTok;
+            float tileMax = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int h = 2 * wave + i;
-            const float *srow = reinterpret_cast<const float *>(smem + LDS_S) + h * TILE;
-            const float s0 = srow[lane], s1 = srow[lane + WAVE];
-            float tileMax = fmaxf(s0, s1);
-            for (int off = 32; off > 0; off >>= 1) {
+            for (int k = 0; k < TPL; k += 4) {
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(srow + k);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    w[k + e] = v[e];
+                    tileMax = fmaxf(tileMax, v[e]);
+                }
+            }
+#pragma unroll
+            for (int off = CH / 2; off > 0; off >>= 1) {
                 tileMax = fmaxf(tileMax, __shfl_xor(tileMax, off));
             }
-            const float newMax = fmaxf(runMax[i], tileMax);
+            const float newMax = fmaxf(runMax, tileMax);
             const bool any = newMax > -INFINITY; // (a mask of -inf can hide everything seen so far)
-            const float w0 = any ? __expf(s0 - newMax) : 0.0f;
-            const float w1 = any ? __expf(s1 - newMax) : 0.0f;
-            float sum = w0 + w1;
-            float wmax = fmaxf(w0, w1);
-            for (int off = 32; off > 0; off >>= 1) {
+            float sum = 0.0f, wmax = 0.0f;
+#pragma unroll
+            for (int k = 0; k < TPL; ++k) {
+                w[k] = any ? __expf(w[k] - newMax) : 0.0f;
+                sum += w[k];
+                wmax = fmaxf(wmax, w[k]);
+            }
+#pragma unroll
+            for (int off = CH / 2; off > 0; off >>= 1) {
                 sum += __shfl_xor(sum, off);
                 wmax = fmaxf(wmax, __shfl_xor(wmax, off));
             }
-            const float keep = (any && runMax[i] > -INFINITY) ? __expf(runMax[i] - newMax) : 0.0f;
-            runSum[i] = runSum[i] * keep + sum;
-            runMax[i] = newMax;
+            const float keep = (any && runMax > -INFINITY) ? __expf(runMax - newMax) : 0.0f;
+            runSum = runSum * keep + sum;
+            runMax = newMax;
             const float step = wmax / 127.0f;
-            int p0 = 0, p1 = 0;
-            if (wmax > 0.0f) {
-                p0 = static_cast<int>(rintf(static_cast<float>(static_cast<_Float16>(__fdiv_rn(w0, step)))));
-                p1 = static_cast<int>(rintf(static_cast<float>(static_cast<_Float16>(__fdiv_rn(w1, step)))));
+            uint32_t packed[TPL / 4];
+#pragma unroll
+            for (int k = 0; k < TPL; k += 4) {
+                uint32_t word = 0;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    int p = 0;
+                    if (wmax > 0.0f) {
+                        p = static_cast<int>(rintf(static_cast<float>(static_cast<_Float16>(__fdiv_rn(w[k + e], step)))));
+                    }
+                    word |= static_cast<uint32_t>(p & 0xff) << (8 * e);
+                }
+                packed[k / 4] = word;
             }
-            reinterpret_cast<int8_t *>(smem + LDS_P)[h * TILE + lane] = static_cast<int8_t>(p0);
-            reinterpret_cast<int8_t *>(smem + LDS_P)[h * TILE + lane + WAVE] = static_cast<int8_t>(p1);
-            if (lane == 0) {
-                float *stat = reinterpret_cast<float *>(smem + LDS_STAT) + h * 4;
+            unsigned char *prow = smem + L::P + smHead * P_PITCH + smTok;
+            if constexpr (TPL == 8) {
+                *reinterpret_cast<uint2 *>(prow) = uint2{packed[0], packed[1]};
+            } else {
+                *reinterpret_cast<uint32_t *>(prow) = packed[0];
+            }
+            if (tid % CH == 0) {
+                float *stat = reinterpret_cast<float *>(smem + L::STAT) + smHead * 4;
                 stat[0] = keep;
-                stat[1] = a.pvDescale[h0 + min(h, nh - 1)] * wmax / 127.0f;
+                stat[1] = smPvDescale * wmax / 127.0f;
             }
         }
         __syncthreads();
         // ---- values: O^T[channel, head] += V^T . P^T for channels 64 wave .. + 63
         {
-            const float keep = reinterpret_cast<const float *>(smem + LDS_STAT)[n * 4];
-            const float vscale = reinterpret_cast<const float *>(smem + LDS_STAT)[n * 4 + 1];
-            // the transposing read hands lane (channel l16, kg) the bytes of tokens r .. r + 7 when lane l16 of the
-            // group points at token r + l16 / 2, channels (l16 % 2) * 8 .. + 8
-            const unsigned char *vbase = smem + LDS_K + (kg * 16 + (l16 >> 1)) * K_PITCH + wave * 64 + (l16 & 1) * 8;
-            const unsigned char *pbase = smem + LDS_P + n * TILE + kg * 16;
+            float keep[NT], vscale[NT];
 #pragma unroll
-            for (int cs = 0; cs < 4; ++cs) {
-                i32x4 iacc = {0, 0, 0, 0};
+            for (int nt = 0; nt < NT; ++nt) {
+                const float *stat = reinterpret_cast<const float *>(smem + L::STAT) + (nt * HT + n) * 4;
+                keep[nt] = stat[0];
+                vscale[nt] = stat[1];
+            }
+            i32x4 pw[NT][TILE / 64];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
                 for (int hh = 0; hh < TILE / 64; ++hh) {
-                    const unsigned char *vp = vbase + hh * 64 * K_PITCH + cs * 16;
+                    pw[nt][hh] = *reinterpret_cast<const i32x4 *>(smem + L::P + (nt * HT + n) * P_PITCH + hh * 64 + kg * 16);
+                }
+            }
+#pragma unroll
+            for (int cs = 0; cs < 4; ++cs) {
+                i32x4 vt[TILE / 64];
+#pragma unroll
+                for (int hh = 0; hh < TILE / 64; ++hh) {
+                    const unsigned char *vp = kbuf + valueLane + (cs >> 1) * 4096 + (cs & 1) * 512 + hh * 2048;
                     const i32x2 lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2 *)(vp));
-                    const i32x2 hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-                        (__attribute__((address_space(3))) i32x2 *)(vp + 8 * K_PITCH));
-                    const i32x4 pw = *reinterpret_cast<const i32x4 *>(pbase + hh * 64);
-                    iacc = __builtin_amdgcn_mfma_i32_16x16x64_i8(i32x4{lo[0], lo[1], hi[0], hi[1]}, pw, iacc, 0, 0, 0);
+                    const i32x2 hi =
+                        __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2 *)(vp + 8 * 16));
+                    vt[hh] = i32x4{lo[0], lo[1], hi[0], hi[1]};
                 }
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    acc[cs][e] = acc[cs][e] * keep + static_cast<float>(iacc[e]) * vscale;
+                for (int nt = 0; nt < NT; ++nt) {
+                    i32x4 iacc = {0, 0, 0, 0};
+#pragma unroll
+                    for (int hh = 0; hh < TILE / 64; ++hh) {
+                        iacc = __builtin_amdgcn_mfma_i32_16x16x64_i8(vt[hh], pw[nt][hh], iacc, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        acc[nt][cs][e] = acc[nt][cs][e] * keep[nt] + static_cast<float>(iacc[e]) * vscale[nt];
+                    }
                 }
             }
         }
     }
     // ---- the rows: acc / sum, and log(sum) + max
     __syncthreads();
-    if (lane == 0) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            float *stat = reinterpret_cast<float *>(smem + LDS_STAT) + (2 * wave + i) * 4;
-            stat[2] = runSum[i] > 0.0f ? 1.0f / runSum[i] : 0.0f;
-            stat[3] = runSum[i] > 0.0f ? logf(runSum[i]) + runMax[i] : -INFINITY;
-        }
+    if (tid % CH == 0) {
+        float *stat = reinterpret_cast<float *>(smem + L::STAT) + smHead * 4;
+        stat[2] = runSum > 0.0f ? 1.0f / runSum : 0.0f;
+        stat[3] = runSum > 0.0f ? logf(runSum) + runMax : -INFINITY;
     }
     __syncthreads();
-    if (n < nh) {
-        const float inv = reinterpret_cast<const float *>(smem + LDS_STAT)[n * 4 + 2];
-        uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) + (static_cast<int64_t>(row.qRow) * a.H + h0 + n) * DN +
-                         wave * 64 + kg * 4;
 #pragma unroll
-        for (int cs = 0; cs < 4; ++cs) {
-            uint16_t bits[4];
+    for (int nt = 0; nt < NT; ++nt) {
+        if (nt * HT + n < nh) {
+            const float inv = reinterpret_cast<const float *>(smem + L::STAT)[(nt * HT + n) * 4 + 2];
+            uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) +
+                             (static_cast<int64_t>(row.qRow) * a.H + h0 + nt * HT + n) * DN + wave * 64 + kg * 4;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float o = acc[cs][e] * inv;
-                bits[e] = BF16 ? FloatToBf16(o) : FloatToHalfBits(o);
+            for (int cs = 0; cs < 4; ++cs) {
+                uint16_t bits[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float o = acc[nt][cs][e] * inv;
+                    bits[e] = BF16 ? FloatToBf16(o) : FloatToHalfBits(o);
+                }
+                uint2 w;
+                w.x = static_cast<uint32_t>(bits[0]) | (static_cast<uint32_t>(bits[1]) << 16);
+                w.y = static_cast<uint32_t>(bits[2]) | (static_cast<uint32_t>(bits[3]) << 16);
+                *reinterpret_cast<uint2 *>(orow + cs * 16) = w;
             }
-            uint2 w;
-            w.x = static_cast<uint32_t>(bits[0]) | (static_cast<uint32_t>(bits[1]) << 16);
-            w.y = static_cast<uint32_t>(bits[2]) | (static_cast<uint32_t>(bits[3]) << 16);
-            *reinterpret_cast<uint2 *>(orow + cs * 16) = w;
         }
     }
     if (a.lse && tid < nh) {
-        a.lse[static_cast<int64_t>(row.qRow) * a.H + h0 + tid] = reinterpret_cast<const float *>(smem + LDS_STAT)[tid * 4 + 3];
+        a.lse[static_cast<int64_t>(row.qRow) * a.H + h0 + tid] = reinterpret_cast<const float *>(smem + L::STAT)[tid * 4 + 3];
     }
 }
 
@@ -391,7 +529,9 @@ extern "C" int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspa
         return Fail(ERR_INVALID_PARAM, "mla_int8: workspace of %llu bytes, %llu needed", (unsigned long long)workspaceBytes,
                     (unsigned long long)bytes);
     }
-    const int64_t grid = static_cast<int64_t>(rows.size()) * ((call->numHeads + mlaint8::HT - 1) / mlaint8::HT);
+    const int nt = call->numHeads > mlaint8::HT ? 2 : 1; // head tiles of 16 a workgroup
+    const int headsPerWg = nt * mlaint8::HT;
+    const int64_t grid = (static_cast<int64_t>(rows.size()) * ((call->numHeads + headsPerWg - 1) / headsPerWg) + 7) / 8 * 8;
     if (grid > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "mla_int8: %lld workgroups", (long long)grid);
     }
@@ -413,11 +553,14 @@ extern "C" int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspa
     a.lse = call->lse;
     a.rows = static_cast<const mlaint8::Row *>(workspaceDevice);
     a.H = call->numHeads;
+    a.numRows = static_cast<int32_t>(rows.size());
     a.maxBlocksPerSeq = call->maxBlocksPerSeq;
     a.maskLen = call->maskLen;
     a.qkScale = call->qkScale;
-    auto kernel = call->outDtype == ATBMI_BF16 ? mlaint8::MlaInt8Kernel<true> : mlaint8::MlaInt8Kernel<false>;
-    const int ldsBytes = mlaint8::LDS_BYTES;
+    const bool bf16 = call->outDtype == ATBMI_BF16;
+    auto kernel = nt == 2 ? (bf16 ? mlaint8::MlaInt8Kernel<true, 2> : mlaint8::MlaInt8Kernel<false, 2>)
+                          : (bf16 ? mlaint8::MlaInt8Kernel<true, 1> : mlaint8::MlaInt8Kernel<false, 1>);
+    const int ldsBytes = nt == 2 ? mlaint8::Lds<2>::BYTES : mlaint8::Lds<1>::BYTES;
     rc = ConfigureKernelLds(reinterpret_cast<const void *>(kernel), ldsBytes);
     if (rc != OK) {
         return rc;
