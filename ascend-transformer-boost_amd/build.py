@@ -33,7 +33,7 @@ CXX = os.environ.get("CXX", "g++")
 
 # -packed-fp32-ops off: the compiler must not form v_pk_*_f32 instructions.
 HIP_FLAGS = [
-    "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Wall", "-Wno-unused-function",
+    "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Wall", "-Wno-unused-function", "-Wno-inline-asm",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-I" + INCLUDE, "-I" + CSRC,
 ]

@@ -51,11 +51,17 @@ constexpr int THREADS = 512;         // eight waves, two a SIMD
 constexpr int NWAVES = THREADS / WAVE;
 // A block in LDS: the 1 KiB pieces of the NZ block ([channels / 32][128 tokens][32 bytes]: piece c = 32 tokens of
 // one 32-channel slab) keep their order, and inside a piece the 16-byte halves of the 32 tokens are parted: the
-// low halves first, 16 bytes a token, then the high halves. Sixteen tokens' reads of one half are then 256
-// contiguous bytes (every bank once), and so are the eight tokens x 16 channels of a transposing read.
+// low halves first, 16 bytes a token, then the high halves; tokens 16 .. 31 of the 32 swap their two groups of
+// eight (place = token ^ 8). Sixteen tokens' reads of one half are then 256 contiguous bytes (every bank once),
+// and the 32 lanes a transposing read serves together (eight tokens x 16 channels twice, 16 tokens apart) touch
+// every bank once as well.
 constexpr int K_BYTES = TILE * DN;
 constexpr int PIECE = 1024;
 constexpr int PIECES_PER_WAVE = K_BYTES / PIECE / NWAVES;
+__host__ __device__ constexpr int PlaceOfToken(int t) // among the 32 tokens of a piece; its own inverse
+{
+    return t ^ ((t & 16) >> 1);
+}
 constexpr int S_PITCH = (TILE + 4) * 4; // 16 heads' 16-byte writes touch every bank once
 constexpr int P_PITCH = TILE + 16;      // likewise for 16 heads' 16-byte reads
 template <int NT> struct Lds {
@@ -66,7 +72,7 @@ template <int NT> struct Lds {
     static constexpr int BYTES = STAT + NT * HT * 16;
     static_assert(BYTES <= 160 * 1024 && S % 16 == 0 && P % 16 == 0 && STAT % 16 == 0, "LDS layout");
 };
-static_assert(TILE == NWAVES * 16 && DN == NWAVES * 64 && K_BYTES % (PIECE * NWAVES) == 0,
+static_assert(TILE == NWAVES * 16 && DN == NWAVES * 64 && PIECES_PER_WAVE == 8,
               "eight waves share a tile this way");
 
 // One query row: its sequence's block-table row and context length, the row of query / out, the mask row.
@@ -112,11 +118,28 @@ template <bool BF16> __device__ __forceinline__ f32x4 Mma16(u32x4 a, u32x4 b, f3
     }
 }
 
-// 16 bytes per lane from `src` to LDS address ldsBase + 16 x lane (ldsBase wave-uniform). The compiler does not
-// count these loads: the kernel waits for them with WaitForLoads.
-__device__ __forceinline__ void TransferToLds(uint32_t ldsBase, const void *src)
+// Eight transfers of 16 bytes per lane, cache to LDS without passing through registers: transfer i reads
+// base + laneOffset + 1024 i and writes LDS address ldsBase + 1024 i + 16 x lane (the instruction's offset field
+// moves both ends, so both bases are given 4096 bytes in). base and ldsBase are wave-uniform. The compiler does
+// not count these loads: the kernel waits for them with WaitForLoads.
+__device__ __forceinline__ void TransferPiecesToLds(uint32_t ldsBase, const void *base, uint32_t laneOffset)
 {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(ldsBase), "v"(src) : "memory", "m0");
+    const uint64_t src = reinterpret_cast<uint64_t>(base) + 4096u;
+    const uint64_t srcUniform =
+        (static_cast<uint64_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(src >> 32))) << 32) |
+        static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(src)));
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %1, %2 offset:-4096\n\t"
+                 "global_load_lds_dwordx4 %1, %2 offset:-3072\n\t"
+                 "global_load_lds_dwordx4 %1, %2 offset:-2048\n\t"
+                 "global_load_lds_dwordx4 %1, %2 offset:-1024\n\t"
+                 "global_load_lds_dwordx4 %1, %2\n\t"
+                 "global_load_lds_dwordx4 %1, %2 offset:1024\n\t"
+                 "global_load_lds_dwordx4 %1, %2 offset:2048\n\t"
+                 "global_load_lds_dwordx4 %1, %2 offset:3072"
+                 :
+                 : "s"(ldsBase + 4096u), "v"(laneOffset), "s"(srcUniform)
+                 : "memory", "m0");
 }
 
 __device__ __forceinline__ void WaitForLoads()
@@ -129,6 +152,35 @@ __device__ __forceinline__ void WaitForLoads()
 template <typename T> __device__ __forceinline__ void Pin(T &v)
 {
     asm volatile("" : "+v"(v));
+}
+
+// All-reduce over the 16 lanes of a row (lanes 16 r .. 16 r + 15) by rotations inside the row.
+template <int ROR> __device__ __forceinline__ float RowRotate(float x)
+{
+    const int v = __builtin_bit_cast(int, x);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(v, v, 0x120 + ROR, 0xf, 0xf, true));
+}
+template <int LANES> __device__ __forceinline__ float GroupMax(float x)
+{
+    x = fmaxf(x, RowRotate<8>(x));
+    x = fmaxf(x, RowRotate<4>(x));
+    x = fmaxf(x, RowRotate<2>(x));
+    x = fmaxf(x, RowRotate<1>(x));
+    if constexpr (LANES == 32) {
+        x = fmaxf(x, __shfl_xor(x, 16));
+    }
+    return x;
+}
+template <int LANES> __device__ __forceinline__ float GroupSum(float x)
+{
+    x += RowRotate<8>(x);
+    x += RowRotate<4>(x);
+    x += RowRotate<2>(x);
+    x += RowRotate<1>(x);
+    if constexpr (LANES == 32) {
+        x += __shfl_xor(x, 16);
+    }
+    return x;
 }
 
 template <bool BF16, int NT>
@@ -160,15 +212,12 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
         static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char *)smem));
 
     // ---- requests for a block: this wave's eight pieces of the int8 rows, and its tokens' rotary rows
-    const int pieceLane = (lane & 31) * 32 + (lane >> 5) * 16; // token lane % 32, half lane / 32
+    const uint32_t pieceLane = PlaceOfToken(lane & 31) * 32 + (lane >> 5) * 16; // place lane % 32, half lane / 32
     auto requestBlock = [&](int64_t blk, int buf) {
-        const unsigned char *src = reinterpret_cast<const unsigned char *>(a.kv8) + blk * K_BYTES +
-                                   wave * (PIECES_PER_WAVE * PIECE) + pieceLane;
+        const unsigned char *src =
+            reinterpret_cast<const unsigned char *>(a.kv8) + blk * K_BYTES + wave * (PIECES_PER_WAVE * PIECE);
         const uint32_t dst = ldsBase + L::K + buf * K_BYTES + wave * (PIECES_PER_WAVE * PIECE);
-#pragma unroll
-        for (int i = 0; i < PIECES_PER_WAVE; ++i) {
-            TransferToLds(__builtin_amdgcn_readfirstlane(dst + i * PIECE), src + i * PIECE);
-        }
+        TransferPiecesToLds(__builtin_amdgcn_readfirstlane(dst), src, pieceLane);
     };
     // lane (token n of the wave's 16, kg): rotary channels 32 m + 8 kg .. + 8, NZ [4][128][16]
     const int ropeLane = (kg >> 1) * (TILE * 32) + (wave * 16 + n) * 32 + (kg & 1) * 16;
@@ -214,9 +263,10 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
     }
     const uint16_t *maskRow = a.mask ? reinterpret_cast<const uint16_t *>(a.mask) + static_cast<int64_t>(row.qRow) * a.maskLen
                                      : nullptr;
-    // softmax: lane (head tid / CH, tokens TPL (tid % CH) .. + TPL); a head's lanes all hold its running maximum and sum
+    // softmax: lane (head tid / CH, tokens 4 (tid % CH + CH k) .. + 4 for k < TPL / 4); a head's lanes all hold its
+    // running maximum and sum
     const int smHead = tid / CH;
-    const int smTok = (tid % CH) * TPL;
+    const int smTok = (tid % CH) * 4;
     const float smPvDescale = a.pvDescale[h0 + min(smHead, nh - 1)];
     float runMax = -INFINITY;
     float runSum = 0.0f;
@@ -230,10 +280,11 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
         }
     }
     // byte offsets into a block in LDS
-    const int scoreLane = (kg >> 1) * 4096 + (wave >> 1) * PIECE + (kg & 1) * 512 + ((wave & 1) * 16 + n) * 16;
+    const int scoreLane = (kg >> 1) * 4096 + (wave >> 1) * PIECE + (kg & 1) * 512 + PlaceOfToken((wave & 1) * 16 + n) * 16;
     // the transposing read hands lane (channel n, kg) the bytes of tokens r .. r + 7 when lane n of the group
     // points at token r + n / 2, channels (n % 2) * 8 .. + 8
-    const int valueLane = wave * 8192 + (kg >> 1) * PIECE + ((kg & 1) * 16 + (n >> 1)) * 16 + (n & 1) * 8;
+    const int valueLane = wave * 8192 + (kg >> 1) * PIECE + PlaceOfToken((kg & 1) * 16 + (n >> 1)) * 16 + (n & 1) * 8;
+    const int valueHigh = (kg & 1) ? -128 : 128; // to the tokens eight further on
 
     for (int i = 0; i < numBlocks; ++i) {
         const int t0 = i * TILE;
@@ -302,17 +353,14 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
             float tileMax = -INFINITY;
 #pragma unroll
             for (int k = 0; k < TPL; k += 4) {
-                const f32x4 v = *reinterpret_cast<const f32x4 *>(srow + k);
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(srow + k * CH);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     w[k + e] = v[e];
                     tileMax = fmaxf(tileMax, v[e]);
                 }
             }
-#pragma unroll
-            for (int off = CH / 2; off > 0; off >>= 1) {
-                tileMax = fmaxf(tileMax, __shfl_xor(tileMax, off));
-            }
+            tileMax = GroupMax<CH>(tileMax);
             const float newMax = fmaxf(runMax, tileMax);
             const bool any = newMax > -INFINITY; // (a mask of -inf can hide everything seen so far)
             float sum = 0.0f, wmax = 0.0f;
@@ -322,34 +370,36 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
                 sum += w[k];
                 wmax = fmaxf(wmax, w[k]);
             }
-#pragma unroll
-            for (int off = CH / 2; off > 0; off >>= 1) {
-                sum += __shfl_xor(sum, off);
-                wmax = fmaxf(wmax, __shfl_xor(wmax, off));
-            }
+            sum = GroupSum<CH>(sum);
+            wmax = GroupMax<CH>(wmax);
             const float keep = (any && runMax > -INFINITY) ? __expf(runMax - newMax) : 0.0f;
             runSum = runSum * keep + sum;
             runMax = newMax;
+            // rint(fp16(w / step)), 0 .. 127. The quotient by a multiplication with 1 / step and one fused
+            // correction (the division's own sequence without its rescaling); a step too small for that takes
+            // the division.
             const float step = wmax / 127.0f;
-            uint32_t packed[TPL / 4];
+            uint32_t packed[TPL / 4] = {};
+            if (step >= 1.0e-30f) {
+                const float y = __builtin_amdgcn_rcpf(step);
 #pragma unroll
-            for (int k = 0; k < TPL; k += 4) {
-                uint32_t word = 0;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    int p = 0;
-                    if (wmax > 0.0f) {
-                        p = static_cast<int>(rintf(static_cast<float>(static_cast<_Float16>(__fdiv_rn(w[k + e], step)))));
-                    }
-                    word |= static_cast<uint32_t>(p & 0xff) << (8 * e);
+                for (int k = 0; k < TPL; ++k) {
+                    const float q0 = w[k] * y;
+                    const float q = __builtin_fmaf(__builtin_fmaf(-q0, step, w[k]), y, q0);
+                    const float p = rintf(static_cast<float>(static_cast<_Float16>(q)));
+                    packed[k / 4] = __builtin_amdgcn_cvt_pk_u8_f32(p, k % 4, packed[k / 4]);
                 }
-                packed[k / 4] = word;
+            } else if (wmax > 0.0f) {
+#pragma unroll
+                for (int k = 0; k < TPL; ++k) {
+                    const float p = rintf(static_cast<float>(static_cast<_Float16>(__fdiv_rn(w[k], step))));
+                    packed[k / 4] = __builtin_amdgcn_cvt_pk_u8_f32(p, k % 4, packed[k / 4]);
+                }
             }
             unsigned char *prow = smem + L::P + smHead * P_PITCH + smTok;
-            if constexpr (TPL == 8) {
-                *reinterpret_cast<uint2 *>(prow) = uint2{packed[0], packed[1]};
-            } else {
-                *reinterpret_cast<uint32_t *>(prow) = packed[0];
+#pragma unroll
+            for (int k = 0; k < TPL / 4; ++k) {
+                *reinterpret_cast<uint32_t *>(prow + k * CH * 4) = packed[k];
             }
             if (tid % CH == 0) {
                 float *stat = reinterpret_cast<float *>(smem + L::STAT) + smHead * 4;
@@ -383,7 +433,7 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
                     const unsigned char *vp = kbuf + valueLane + (cs >> 1) * 4096 + (cs & 1) * 512 + hh * 2048;
                     const i32x2 lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2 *)(vp));
                     const i32x2 hi =
-                        __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2 *)(vp + 8 * 16));
+                        __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2 *)(vp + valueHigh));
                     vt[hh] = i32x4{lo[0], lo[1], hi[0], hi[1]};
                 }
 #pragma unroll
