@@ -622,5 +622,6 @@ extern "C" int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspa
     }
     kernel<<<static_cast<unsigned>(grid), mlaint8::THREADS, ldsBytes, s>>>(a);
     ATBMI_HIP_CHECK(hipGetLastError());
-    return TimedLaunchEnd(s, timed);
+    rc = TimedLaunchKernelDone(s, timed);
+    return rc != OK ? rc : TimedLaunchEnd(s, timed, false);
 }

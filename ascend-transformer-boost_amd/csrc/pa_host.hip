@@ -149,14 +149,25 @@ int TimedLaunchBegin(hipStream_t stream, TimedLaunch *launch)
     return OK;
 }
 
-int TimedLaunchEnd(hipStream_t stream, const TimedLaunch &launch)
+int TimedLaunchKernelDone(hipStream_t stream, const TimedLaunch &launch)
+{
+    if (launch.begin) {
+        ATBMI_HIP_CHECK(hipEventRecord(launch.end, stream));
+    }
+    return OK;
+}
+
+int TimedLaunchEnd(hipStream_t stream, const TimedLaunch &launch, bool merged)
 {
     if (!launch.begin) {
         return OK;
     }
-    ATBMI_HIP_CHECK(hipEventRecord(launch.end, stream));
+    TimingRecord rec{launch.begin, launch.end, nullptr};
+    if (merged && hipEventCreate(&rec.merged) == hipSuccess) {
+        (void)hipEventRecord(rec.merged, stream);
+    }
     std::lock_guard<std::mutex> lock(g_timingMutex);
-    g_timingRecords.push_back(TimingRecord{launch.begin, launch.end, nullptr});
+    g_timingRecords.push_back(rec);
     return OK;
 }
 

@@ -46,14 +46,16 @@ int LaunchPaMfmaBf16(const AtbmiPaShape &shape, const PaArgs &args, const PaStre
 int LaunchPaMfmaInt8(const AtbmiPaShape &shape, const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream);
 
 // Event brackets around the attention kernel of a call while atbmi_timing_enable is on (every n-th launch).
-// TimedLaunchBegin records the first event on `stream` when this launch is one to time and returns a token
-// (0 otherwise); TimedLaunchEnd records the closing event and queues the pair for atbmi_timing_read.
+// TimedLaunchBegin records the first event on `stream` when this launch is one to time (launch->begin stays null
+// otherwise); TimedLaunchKernelDone records the event after the attention kernel; TimedLaunchEnd records a third
+// event when a merge kernel followed and queues the record for atbmi_timing_read_split.
 struct TimedLaunch {
     hipEvent_t begin = nullptr;
     hipEvent_t end = nullptr;
 };
 int TimedLaunchBegin(hipStream_t stream, TimedLaunch *launch);
-int TimedLaunchEnd(hipStream_t stream, const TimedLaunch &launch);
+int TimedLaunchKernelDone(hipStream_t stream, const TimedLaunch &launch);
+int TimedLaunchEnd(hipStream_t stream, const TimedLaunch &launch, bool merged);
 
 // Raises a kernel's dynamic LDS limit to `ldsBytes` on the current device, once per kernel and device.
 int ConfigureKernelLds(const void *kernel, int ldsBytes);
