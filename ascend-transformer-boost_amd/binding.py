@@ -206,9 +206,10 @@ class AtbmiMlaInt8Call(ctypes.Structure):
     _fields_ = [("outDtype", ctypes.c_int32), ("numHeads", ctypes.c_int32), ("blockSize", ctypes.c_int32),
                 ("numBlocks", ctypes.c_int32), ("maxBlocksPerSeq", ctypes.c_int32), ("batch", ctypes.c_int32),
                 ("numQueryRows", ctypes.c_int32), ("hasMask", ctypes.c_int32), ("maskLen", ctypes.c_int32),
-                ("qkScale", ctypes.c_float)] + [(n, ctypes.c_void_p) for n in (
-                    "hostContextLens", "hostQueryLens", "query", "queryRope", "kvCache", "kRopeCache", "blockTables",
-                    "qkDescale", "pvDescale", "mask", "out", "lse")]
+                ("qkScale", ctypes.c_float), ("hostContextLens", ctypes.c_void_p), ("hostQueryLens", ctypes.c_void_p),
+                ("causalRows", ctypes.c_int32), ("hostCausalUse", ctypes.c_void_p)] + [(n, ctypes.c_void_p) for n in (
+                    "query", "queryRope", "kvCache", "kRopeCache", "blockTables", "qkDescale", "pvDescale", "mask", "out",
+                    "lse")]
 
 _kernels = None
 _atb = None
@@ -248,6 +249,8 @@ def kernels():
         lib.atbmi_pa_plan_update.argtypes = [vp, vp, i32]
         lib.atbmi_pa_plan_update_multi.argtypes = [vp, vp, vp, i32]
         lib.atbmi_pa_plan_update_multi.restype = i32
+        lib.atbmi_pa_plan_set_causal_rows.argtypes = [vp, i32, vp, i32]
+        lib.atbmi_pa_plan_set_causal_rows.restype = i32
         lib.atbmi_pa_plan_workspace_size.argtypes = [vp]
         lib.atbmi_pa_plan_workspace_size.restype = u64
         lib.atbmi_pa_plan_num_chunks.argtypes = [vp]

@@ -512,6 +512,10 @@ int BuildRows(const AtbmiMlaInt8Call *c, std::vector<Row> *rows)
         if (ctx < 0 || nq < 0) {
             return Fail(ERR_INVALID_PARAM, "mla_int8: sequence %d has context %d and %d query tokens", b, ctx, nq);
         }
+        const bool causal = c->causalRows && (!c->hostCausalUse || c->hostCausalUse[b] != 0);
+        if (causal && ctx > 0 && nq > ctx) {
+            return Fail(ERR_INVALID_PARAM, "mla_int8: sequence %d has %d query tokens but a context of %d", b, nq, ctx);
+        }
         if (ctx > static_cast<int64_t>(c->maxBlocksPerSeq) * c->blockSize) {
             return Fail(ERR_INVALID_PARAM, "mla_int8: context %d of sequence %d exceeds its %d blocks", ctx, b,
                         c->maxBlocksPerSeq);
@@ -528,7 +532,7 @@ int BuildRows(const AtbmiMlaInt8Call *c, std::vector<Row> *rows)
                 return Fail(ERR_INVALID_PARAM, "mla_int8: more than 2^31 query rows");
             }
             if (rows) {
-                rows->push_back(Row{b, ctx, static_cast<int32_t>(qRow), 0});
+                rows->push_back(Row{b, causal ? ctx - nq + i + 1 : ctx, static_cast<int32_t>(qRow), 0});
             }
             ++qRow;
         }

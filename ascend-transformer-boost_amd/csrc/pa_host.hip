@@ -204,6 +204,8 @@ struct AtbmiPaPlan {
     int64_t rowCtx = 0;      // sum over query rows of the context they attend to
     int32_t maxQueryLen = 1; // most query tokens any sequence brings
     std::vector<PaSeq> rows; // the query rows in query/output order (stepBegin unused here)
+    bool causalRows = false;            // a sequence's query rows see growing prefixes of its context
+    std::vector<int32_t> causalUse;     // empty: every sequence; else one flag per sequence
 
     uint64_t offItems = 0, offSeqs = 0, offPartO = 0, offPartLse = 0, blobBytes = 0, wsBytes = 0;
     std::vector<uint8_t> blob; // items then reduceSeqs, as uploaded
@@ -371,7 +373,7 @@ int PlanStream(AtbmiPaPlan *plan)
     // Several query tokens of one sequence share a pass over its context when a GQA group
     // leaves columns of the 16-wide head tile free: 16 / group tokens per pass.
     int fold = 1;
-    if (headTiles == 1 && !PaMlaWide(s) && plan->maxQueryLen > 1) {
+    if (headTiles == 1 && !PaMlaWide(s) && plan->maxQueryLen > 1 && !plan->causalRows) {
         fold = std::min(PA_MFMA_HEAD_TILE / groupSize, plan->maxQueryLen);
     }
     try {
@@ -493,6 +495,24 @@ int PlanStream(AtbmiPaPlan *plan)
 
 } // namespace
 
+extern "C" int atbmi_pa_plan_set_causal_rows(AtbmiPaPlan *plan, int32_t enable, const int32_t *perSequence,
+                                             int32_t count)
+{
+    if (!plan || (perSequence && count <= 0)) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_set_causal_rows: null plan or %d flags", count);
+    }
+    try {
+        plan->causalRows = enable != 0;
+        plan->causalUse.clear();
+        if (plan->causalRows && perSequence) {
+            plan->causalUse.assign(perSequence, perSequence + count);
+        }
+    } catch (const std::bad_alloc &) {
+        return Fail(ERR_OUT_OF_HOST_MEMORY, "pa_plan_set_causal_rows: out of host memory");
+    }
+    return OK;
+}
+
 extern "C" int atbmi_pa_plan_update(AtbmiPaPlan *plan, const int32_t *ctx, int32_t batch)
 {
     return atbmi_pa_plan_update_multi(plan, ctx, nullptr, batch);
@@ -519,6 +539,10 @@ extern "C" int atbmi_pa_plan_update_multi(AtbmiPaPlan *plan, const int32_t *ctx,
             return Fail(ERR_INVALID_PARAM, "pa_plan_update: queryLens[%d]=%d outside [0, contextLens = %d]", b, qLens[b],
                         ctx[b]);
         }
+        if (plan->causalRows && !plan->causalUse.empty() && static_cast<int32_t>(plan->causalUse.size()) != batch) {
+            return Fail(ERR_INVALID_PARAM, "pa_plan_update: causal-row flags for %d sequences, batch %d",
+                        static_cast<int>(plan->causalUse.size()), batch);
+        }
         if (s.hasMask && ctx[b] > s.maskLen) {
             // both kernels index a mask row by token without a bound of their own
             return Fail(ERR_INVALID_PARAM, "pa_plan_update: contextLens[%d]=%d exceeds the mask's %d tokens per row", b,
@@ -544,6 +568,9 @@ extern "C" int atbmi_pa_plan_update_multi(AtbmiPaPlan *plan, const int32_t *ctx,
                 PaSeq row{};
                 row.tableRow = b;
                 row.ctxLen = ctx[b];
+                if (plan->causalRows && (plan->causalUse.empty() || plan->causalUse[static_cast<size_t>(b)] != 0)) {
+                    row.ctxLen = ctx[b] - n + i + 1; // (>= 1: n <= ctx[b] was checked above)
+                }
                 row.nTok = 1;
                 const int32_t index = static_cast<int32_t>(plan->rows.size());
                 row.qRow = index;

@@ -18,12 +18,25 @@
 // one for the values, the rotary parts 16-bit; reference :427-476, :493-511, :513-541)
 // runs on a kernel of its own (csrc/mla_int8.hip); its log-sum-exp output is fp32.
 // calcType PREFILL is an operation class of its own
-// (multi_latent_attention_prefill_operation.cpp). The MASK_FREE / CAUSAL_MASK masks
-// of the decode calcTypes and maskUseStatus are legal in the reference but not
-// implemented here; such params are rejected at creation with ERROR_INVALID_PARAM.
+// (multi_latent_attention_prefill_operation.cpp).
+//
+// Several query tokens per sequence (SPEC, SPEC_AND_RING). The reference's tiling runs one
+// job per query token, each over the context up to that token, when headNum is 128 or
+// the cache is int8 with more than one query token, and drops the mask type in that
+// case (src/kernels/mixkernels/multi_latent_attention/tiling/mla_tiling.cpp:139-144,
+// mla_tiling_dependency.cpp:292-316): the t-th of n query rows sees the first
+// contextLens - n + t + 1 tokens whatever mask tensor came with the call, and a
+// sequence whose maskUseStatus entry is 0 keeps the whole context for every row. The
+// same rule applies here (kernel layer: causal rows). With fewer heads the
+// MASK_TYPE_SPEC mask [numTokens, maxS] is added to the scores as given;
+// MASK_TYPE_CAUSAL_MASK (no mask tensor) is causal rows for any head count, and
+// MASK_TYPE_MASK_FREE, whose [125 + 2 q, 128] template the reference's other kernel
+// path indexes by the last two 128-token tiles (op_kernel/mla.cce:3719-3750), is
+// built for the 128-head / int8 path only: with fewer heads Setup refuses it.
 //
 // The kernels are those of PagedAttention's combined-cache variant reading
 // each query and key row from two tensors.
+#include <algorithm>
 #include <new>
 #include <vector>
 #include "atb/infer_op_params.h"
@@ -43,6 +56,7 @@ constexpr int64_t DECODER_BLOCK_SIZE = 128;
 constexpr int64_t MAX_BATCH = 8192;
 constexpr int64_t NZ_CHANNELS = 16; // channels of one fractal-NZ slab row (16-bit elements)
 constexpr int64_t NZ_CHANNELS_INT8 = 32;
+constexpr int32_t JOB_PER_TOKEN_HEADS = 128; // reference tiling/mla_tiling_dependency.h:31 (M_LIMIT)
 
 bool IsSpec(const Param &p)
 {
@@ -151,23 +165,9 @@ bool ParamPrefillCheck(const Param &p)
     return true;
 }
 
-// Features that are legal in the reference but have no MI355X kernel yet.
-bool ImplementedCheck(const Param &p)
+bool HasMaskUseStatus(const Param &p)
 {
-    const char *what = nullptr;
-    if (p.calcType == Param::CALC_TYPE_PREFILL) {
-        return true; // every param that passes ParamPrefillCheck is built
-    }
-    if (p.maskType != Param::UNDEFINED && p.maskType != Param::MASK_TYPE_SPEC) {
-        what = "this maskType";
-    } else if (p.maskUseStatusType != Param::MASK_USE_STATUS_TYPE_UNDEFINED) {
-        what = "maskUseStatus";
-    }
-    if (what) {
-        ATB_LOG(ERROR) << "MultiLatentAttention: " << what << " not implemented on MI355X";
-        return false;
-    }
-    return true;
+    return p.maskUseStatusType == Param::MASK_USE_STATUS_TYPE_BATCH_MASK;
 }
 
 // The dtype table of the implemented sections of the reference
@@ -178,6 +178,11 @@ bool ImplementedCheck(const Param &p)
 // a table skips the check (reference operation_base.cpp:229-233): HasIr() says which.
 bool HasIr(const Param &p)
 {
+    if (HasMaskUseStatus(p)) {
+        // (always SPEC_AND_RING) sections MaskQlensIsRingMaskUseStatus and QlensIsRingInt8NzMaskUseStatus
+        // (:7021-7055, :7091-7126)
+        return p.cacheMode == Param::INT8_NZCACHE ? !HasMaskInput(p) : p.cacheMode == Param::KROPE_CTKV && HasMaskInput(p);
+    }
     if (p.cacheMode == Param::INT8_NZCACHE) {
         // sections Int8Nz, IsRingInt8Nz and QlensIsRingInt8Nz (:6918-6945, :6741-6771, :6825-6858)
         return !HasMaskInput(p) && (!IsSpec(p) || IsRing(p));
@@ -202,6 +207,9 @@ OpIr MakeIr(const Param &p)
         if (int8) {
             c.inDtypes.push_back(ACL_FLOAT);
             c.inDtypes.push_back(ACL_FLOAT);
+        }
+        if (HasMaskUseStatus(p)) {
+            c.inDtypes.push_back(ACL_INT32);
         }
         c.inFormats.assign(c.inDtypes.size(), ACL_FORMAT_ND);
         c.inFormats[KV_CACHE] = cacheFormat;
@@ -238,6 +246,9 @@ public:
             descaleIdx_ = next;
             next += 2; // qkDescale, pvDescale
         }
+        if (HasMaskUseStatus(param)) {
+            maskUseIdx_ = next++;
+        }
         inputNum_ = static_cast<uint32_t>(next);
     }
 
@@ -250,6 +261,7 @@ public:
 
     uint32_t GetInputNum() const override { return inputNum_; }
     uint32_t GetOutputNum() const override { return IsRing(param_) ? 2 : 1; }
+    bool InputMayBeEmpty(size_t index) const override { return index == maskUseIdx_; } // reference ini: optional
 
 protected:
     // Reference :268-283.
@@ -318,6 +330,35 @@ protected:
             }
             queryLens = static_cast<const int32_t *>(ql.hostData);
         }
+        // One job per query token, each over the context up to its token, and no mask: the reference's tiling
+        // for 128 heads and for an int8 cache with several query tokens (mla_tiling.cpp:139-144,
+        // mla_tiling_dependency.cpp:292-316); MASK_TYPE_CAUSAL_MASK asks for the same.
+        const bool int8 = param_.cacheMode == Param::INT8_NZCACHE;
+        int32_t maxQuery = 1;
+        for (int32_t i = 0; queryLens && i < batch; ++i) {
+            maxQuery = std::max(maxQuery, queryLens[i]);
+        }
+        const bool jobPerToken = param_.headNum == JOB_PER_TOKEN_HEADS || (int8 && maxQuery > 1);
+        const bool causalRows = IsSpec(param_) && (jobPerToken || param_.maskType == Param::MASK_TYPE_CAUSAL_MASK);
+        useMask_ = maskIdx_ != NONE && !jobPerToken && !int8; // (the int8 kernels of the reference never read it)
+        if (useMask_ && param_.maskType == Param::MASK_TYPE_MASK_FREE) {
+            ATB_LOG(ERROR) << "MASK_TYPE_MASK_FREE with fewer than " << JOB_PER_TOKEN_HEADS
+                           << " heads is not implemented on MI355X (use MASK_TYPE_SPEC or MASK_TYPE_CAUSAL_MASK)";
+            return ERROR_INVALID_PARAM;
+        }
+        causalUse_.clear();
+        if (causalRows && maskUseIdx_ != NONE && Utils::GetTensorSize(pack.inTensors.at(maskUseIdx_).desc) != 0) {
+            const Tensor &use = pack.inTensors.at(maskUseIdx_);
+            if (!use.hostData) {
+                ATB_LOG(ERROR) << "maskUseStatus.hostData is null; the flags are read on the host during Setup";
+                return ERROR_INVALID_PARAM;
+            }
+            if (use.desc.shape.dimNum != 1 || use.desc.shape.dims[0] != batch) {
+                ATB_LOG(ERROR) << "maskUseStatus should be [batch]";
+                return ERROR_INVALID_PARAM;
+            }
+            causalUse_.assign(static_cast<const int32_t *>(use.hostData), static_cast<const int32_t *>(use.hostData) + batch);
+        }
         const Dims &o = out.desc.shape;
         if (o.dimNum != 3 || o.dims[0] != q.desc.shape.dims[0] || o.dims[1] != param_.headNum ||
             o.dims[2] != LATENT_DIM) {
@@ -332,7 +373,7 @@ protected:
             }
         }
         int64_t maskLen = 0;
-        if (maskIdx_ != NONE) {
+        if (useMask_) {
             // one mask row per query token (reference tests/apitest/opstest/python/operations/
             // multi_latent_attention/test_multi_latent_attention_mtp.py:262-274)
             const Dims &m = pack.inTensors.at(maskIdx_).desc.shape;
@@ -363,7 +404,7 @@ protected:
             if (queryLens) {
                 qLens_.assign(queryLens, queryLens + batch);
             }
-            maskLen_ = maskLen;
+            causalRows_ = causalRows;
             AtbmiMlaInt8Call call = MakeInt8Call(pack);
             int rc = atbmi_mla_int8_workspace_size(&call, &workspaceSize);
             if (rc != 0) {
@@ -389,10 +430,10 @@ protected:
         shape.kernel = ATBMI_PA_KERNEL_AUTO;
         shape.qkScale = param_.qkScale;
         shape.ropeDim = static_cast<int32_t>(ROPE_DIM);
-        shape.hasMask = maskIdx_ != NONE ? 1 : 0;
+        shape.hasMask = useMask_ ? 1 : 0;
         shape.maskBatchStride = maskLen;
         shape.maskLen = static_cast<int32_t>(maskLen);
-        shape.maskRowBy = maskIdx_ != NONE ? ATBMI_PA_MASK_ROW_QUERY : ATBMI_PA_MASK_ROW_SEQUENCE;
+        shape.maskRowBy = useMask_ ? ATBMI_PA_MASK_ROW_QUERY : ATBMI_PA_MASK_ROW_SEQUENCE;
         if (!plan_ || !SameShape(shape, planShape_)) {
             if (plan_) {
                 atbmi_pa_plan_destroy(plan_);
@@ -405,7 +446,11 @@ protected:
             }
             planShape_ = shape;
         }
-        int rc = atbmi_pa_plan_update_multi(plan_, static_cast<const int32_t *>(lens.hostData), queryLens, batch);
+        int rc = atbmi_pa_plan_set_causal_rows(plan_, causalRows ? 1 : 0, causalUse_.empty() ? nullptr : causalUse_.data(),
+                                               static_cast<int32_t>(causalUse_.size()));
+        if (rc == 0) {
+            rc = atbmi_pa_plan_update_multi(plan_, static_cast<const int32_t *>(lens.hostData), queryLens, batch);
+        }
         if (rc != 0) {
             ATB_LOG(ERROR) << "MultiLatentAttention plan: " << atbmi_last_error();
             return rc;
@@ -431,7 +476,7 @@ protected:
         t.keyCache = pack.inTensors.at(KV_CACHE).deviceData;
         t.keyRopeCache = pack.inTensors.at(KV_CACHE_ROPE).deviceData;
         t.blockTables = static_cast<const int32_t *>(pack.inTensors.at(BLOCK_TABLES).deviceData);
-        if (maskIdx_ != NONE) {
+        if (useMask_) {
             t.mask = pack.inTensors.at(maskIdx_).deviceData;
         }
         t.out = pack.outTensors.at(0).deviceData;
@@ -459,8 +504,10 @@ private:
         c.maxBlocksPerSeq = static_cast<int32_t>(pack.inTensors.at(BLOCK_TABLES).desc.shape.dims[1]);
         c.batch = static_cast<int32_t>(lens_.size());
         c.numQueryRows = static_cast<int32_t>(pack.inTensors.at(QUERY).desc.shape.dims[0]);
-        c.hasMask = maskIdx_ != NONE ? 1 : 0;
-        c.maskLen = static_cast<int32_t>(maskLen_);
+        c.hasMask = 0; // (the reference's int8 kernels never read the mask: mla_tiling.cpp:142-144)
+        c.maskLen = 0;
+        c.causalRows = causalRows_ ? 1 : 0;
+        c.hostCausalUse = causalUse_.empty() ? nullptr : causalUse_.data();
         c.qkScale = param_.qkScale;
         c.hostContextLens = lens_.data();
         c.hostQueryLens = qLens_.empty() ? nullptr : qLens_.data();
@@ -471,7 +518,7 @@ private:
         c.blockTables = static_cast<const int32_t *>(pack.inTensors.at(BLOCK_TABLES).deviceData);
         c.qkDescale = static_cast<const float *>(pack.inTensors.at(descaleIdx_).deviceData);
         c.pvDescale = static_cast<const float *>(pack.inTensors.at(descaleIdx_ + 1).deviceData);
-        c.mask = maskIdx_ != NONE ? pack.inTensors.at(maskIdx_).deviceData : nullptr;
+        c.mask = nullptr;
         c.out = pack.outTensors.at(0).deviceData;
         c.lse = IsRing(param_) ? static_cast<float *>(pack.outTensors.at(1).deviceData) : nullptr;
         return c;
@@ -560,6 +607,20 @@ private:
                 return ERROR_INVALID_TENSOR_DIM;
             }
         }
+        if (IsSpec(param_) && maskUseIdx_ != NONE && (param_.headNum == JOB_PER_TOKEN_HEADS || int8)) {
+            // reference :536-551 with :569-575
+            const Dims &u = in.at(maskUseIdx_).shape;
+            if (u.dimNum != 0 && Utils::GetTensorSize(in.at(maskUseIdx_)) != 0) { // (an empty tensor: left out)
+                if (u.dimNum != 1) {
+                    ATB_LOG(ERROR) << "maskUseStatus should have 1 dim";
+                    return ERROR_INVALID_TENSOR_DIM_NUM;
+                }
+                if (u.dims[0] != batch) {
+                    ATB_LOG(ERROR) << "dim 0 of maskUseStatus should equal dim 0 of contextLens";
+                    return ERROR_INVALID_TENSOR_DIM;
+                }
+            }
+        }
         if (int8 && IsRing(param_) && param_.maskType == Param::UNDEFINED) {
             // reference :493-511 (only this combination checks the descales there)
             const Dims &d0 = in.at(descaleIdx_).shape;
@@ -581,9 +642,12 @@ private:
     size_t maskIdx_ = NONE;
     size_t qLensIdx_ = NONE;
     size_t descaleIdx_ = NONE;
+    size_t maskUseIdx_ = NONE;
     std::vector<int32_t> lens_;   // (int8 cache mode: the lengths of the last Setup)
     std::vector<int32_t> qLens_;
-    int64_t maskLen_ = 0;
+    std::vector<int32_t> causalUse_; // the maskUseStatus flags of the last Setup (empty: every sequence)
+    bool useMask_ = false;           // the mask tensor is added to the scores
+    bool causalRows_ = false;
     uint32_t inputNum_ = 6;
     AtbmiPaPlan *plan_ = nullptr;
     AtbmiPaShape planShape_{};
@@ -603,9 +667,6 @@ template <> Status CreateOperation(const infer::MultiLatentAttentionParam &opPar
     }
     if (!ReservedIsZero(opParam)) {
         ATB_LOG(ERROR) << "MultiLatentAttentionParam rsv has a non-zero byte";
-        return ERROR_INVALID_PARAM;
-    }
-    if (!ImplementedCheck(opParam)) {
         return ERROR_INVALID_PARAM;
     }
     *operation = opParam.calcType == Param::CALC_TYPE_PREFILL

@@ -343,6 +343,15 @@ int atbmi_pa_plan_update(AtbmiPaPlan *plan, const int32_t *hostContextLens, int3
 int atbmi_pa_plan_update_multi(AtbmiPaPlan *plan, const int32_t *hostContextLens, const int32_t *hostQueryLens,
                                int32_t batch);
 
+/* Causal query rows for the updates that follow: the t-th of a sequence's n query rows then attends to its
+ * first hostContextLens[b] - n + t + 1 tokens only, with no mask involved. This is how the reference's MLA
+ * tiling makes several query tokens causal when it runs one job per query token (128 heads, or an int8 cache:
+ * src/kernels/mixkernels/multi_latent_attention/tiling/mla_tiling.cpp:139-144,
+ * mla_tiling_dependency.cpp:292-316). perSequence, NULL or a host array of `count` flags that is copied,
+ * exempts the sequences whose flag is 0 (the reference's maskUseStatus); an update with another batch than
+ * `count` is refused. enable == 0 returns to whole contexts. Query tokens of a sequence then take a pass each. */
+int atbmi_pa_plan_set_causal_rows(AtbmiPaPlan *plan, int32_t enable, const int32_t *perSequence, int32_t count);
+
 /* Device workspace bytes atbmi_pa_decode needs for the current plan. */
 uint64_t atbmi_pa_plan_workspace_size(const AtbmiPaPlan *plan);
 
@@ -438,8 +447,10 @@ int atbmi_mla_prefill(const AtbmiMlaPrefillCall *call, void *workspaceDevice, ui
  *   mask        NULL, or 16-bit [numQueryRows, maskLen] added to the scaled scores of its query row
  *   out         16-bit [numQueryRows, numHeads, 512]     lse        NULL, or fp32 [numQueryRows, numHeads]
  * Sequence b attends to hostContextLens[b] tokens with hostQueryLens[b] consecutive query rows (NULL: one
- * each; a sequence of length 0 takes none). numHeads must be a multiple of 8. The lengths are host arrays,
- * read during the call.
+ * each; a sequence of length 0 takes none). With causalRows != 0 the t-th of a sequence's n query rows
+ * attends to its first hostContextLens[b] - n + t + 1 tokens only, unless hostCausalUse (NULL, or [batch])
+ * holds 0 for the sequence: the reference golden's handling of several query tokens in this mode
+ * (test_multi_latent_attention_int8nz.py:356-364). The lengths and flags are host arrays, read during the call.
  */
 typedef struct AtbmiMlaInt8Call {
     int32_t outDtype;          /* ATBMI_F16 or ATBMI_BF16: type of queryRope, kRopeCache, mask and out */
@@ -454,6 +465,8 @@ typedef struct AtbmiMlaInt8Call {
     float qkScale;
     const int32_t *hostContextLens; /* [batch], host memory */
     const int32_t *hostQueryLens;   /* NULL or [batch], host memory */
+    int32_t causalRows;
+    const int32_t *hostCausalUse;   /* NULL or [batch], host memory */
     const void *query;
     const void *queryRope;
     const void *kvCache;

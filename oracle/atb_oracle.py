@@ -449,7 +449,8 @@ def norm_mask(batch, max_len, value=-10000.0):
 def paged_attention(query, key_cache, value_cache, block_tables, context_lens, scale, k_descale=None,
                     k_offset=None, v_descale=None, v_offset=None, mla_v_head_size=0, q_scale=0.0,
                     q_dtype="float32", out_init=0.0, mask=None, logn=None, mask_per_head=None, q_lens=None,
-                    mask_rows="sequence", lse_out=None, head_major=False, compress_kv_heads=0, razor_offset=None):
+                    mask_rows="sequence", lse_out=None, head_major=False, compress_kv_heads=0, razor_offset=None,
+                    causal_rows=None):
     """Decode attention over paged caches.
 
     query [rows, heads, D] float32; key_cache [blocks, block, kv_heads, D];
@@ -471,6 +472,13 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, s
     2-dim mask then has one row per query row (mask_rows="query") or is the
     square causal mask, of which the t-th query token of a sequence with n of
     them uses row ctx - n + t (mask_rows="position").
+    causal_rows (True, or a [batch] array of flags): the t-th of a sequence's n
+    query rows attends to its first ctx - n + t + 1 tokens only, which is how
+    the reference's MLA kernel makes several query tokens causal when it runs
+    one job per query token (128 heads, or an int8 cache with more than one
+    query token: src/kernels/mixkernels/multi_latent_attention/tiling/
+    mla_tiling.cpp:139-144, mla_tiling_dependency.cpp:292-316; a sequence whose
+    maskUseStatus entry is 0 keeps the whole context for every row).
     lse_out, a float32 [rows, heads] array, receives the log-sum-exp of every
     written row (see attention_one); other rows are left alone.
     The split latent layout of MultiLatentAttention (query / cache rows given as
@@ -530,7 +538,8 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, s
         keys = gather_rows(key_cache, block_tables[i], ctx)
         values = keys[..., :dv] if mla_v_head_size > 0 else gather_rows(value_cache, block_tables[i], ctx)
         seq_scale = np.float32(scale) if logn is None else np.float32(scale) * np.float32(logn[i])
-        for t in range(1 if q_lens is None else int(q_lens[i])):
+        n_rows = 1 if q_lens is None else int(q_lens[i])
+        for t in range(n_rows):
             if mask is None:
                 bias = None
             elif mask_rows == "query":
@@ -539,10 +548,21 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, s
                 bias = np.asarray(mask, dtype=np.float32)[ctx - int(q_lens[i]) + t][None, :ctx]
             else:
                 bias = _mask_slice(mask, i, ctx, query.shape[1], len(context_lens), mask_per_head)
-            out[row] = attention_one(query[row], keys, values, seq_scale, k_descale, k_offset, v_descale,
-                                     v_offset, bias, None if lse_out is None else lse_out[row])
+            seen = _causal_row_length(ctx, n_rows, t, i, causal_rows)
+            out[row] = attention_one(query[row], keys[:seen], values[:seen], seq_scale, k_descale, k_offset, v_descale,
+                                     v_offset, None if bias is None else bias[..., :seen],
+                                     None if lse_out is None else lse_out[row])
             row += 1
     return out
+
+
+def _causal_row_length(ctx, n_rows, t, seq, causal_rows):
+    """Tokens the t-th of a sequence's n_rows query rows attends to (see paged_attention's causal_rows)."""
+    if causal_rows is None or causal_rows is False:
+        return ctx
+    if causal_rows is not True and not int(np.asarray(causal_rows)[seq]):
+        return ctx
+    return ctx - n_rows + t + 1
 
 
 def _paged_attention_compressed(query, key_cache, value_cache, block_tables, context_lens, scale, k_descale, k_offset,
@@ -643,11 +663,13 @@ def quantise_weights(w):
 
 
 def mla_int8_decode(q_int8, q_rope, kv_int8, k_rope, block_tables, context_lens, qk_descale, pv_descale, scale,
-                    tile=128, mask=None, q_lens=None, lse_out=None):
+                    tile=128, mask=None, q_lens=None, lse_out=None, causal_rows=None):
     """Decode attention of MultiLatentAttention's int8 cache mode over token-major views of the caches:
     q_int8 [T, H, 512] int8, q_rope [T, H, 64] float, kv_int8 [blocks, block_size, 1, 512] int8 (keys and
     values), k_rope [blocks, block_size, 1, 64] float, qk_descale / pv_descale [H] float32. The weights of
-    every `tile` consecutive tokens are quantised to int8 on their own. mask: None or [T, >= max context]
+    every `tile` consecutive tokens are quantised to int8 on their own. causal_rows as in paged_attention: the
+    reference golden gives the j-th of q query rows context + j - q + 1 tokens unless the sequence's entry of
+    batch_list is 0 (test_multi_latent_attention_int8nz.py:356-364). mask: None or [T, >= max context]
     added to the scaled scores of its query row; q_lens: query rows per sequence (default one). Returns
     float32 [T, H, 512]; lse_out [T, H] receives log(sum exp) of the scaled scores."""
     q_int8 = np.asarray(q_int8)
@@ -663,7 +685,10 @@ def mla_int8_decode(q_int8, q_rope, kv_int8, k_rope, block_tables, context_lens,
         n_rows = 1 if q_lens is None else int(q_lens[b])
         keys = gather_rows(np.asarray(kv_int8), block_tables[b], ctx)[:, 0].astype(np.int32)     # [ctx, 512]
         rope = gather_rows(np.asarray(k_rope, np.float32), block_tables[b], ctx)[:, 0]             # [ctx, 64]
+        all_keys, all_rope, whole = keys, rope, ctx
         for r in range(row, row + n_rows):
+            ctx = _causal_row_length(whole, n_rows, r - row, b, causal_rows)
+            keys, rope = all_keys[:ctx], all_rope[:ctx]
             prod = (q_int8[r].astype(np.int32) @ keys.T).astype(np.float32) * qk_descale[:, None]  # [H, ctx]
             s = (prod + np.asarray(q_rope[r], np.float32) @ rope.T) * np.float32(scale)
             if mask is not None:

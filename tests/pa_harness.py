@@ -23,13 +23,14 @@ def dtype_code(binding, t):
 def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=None, v_scale=None,
                    v_off=None, mla_dv=0, q_scale=0.0, kernel=0, chunk_tokens=None, out=None, return_plan_info=False,
                    mask=None, mask_per_head=False, logn=None, q_lens=None, mask_rows="sequence", q_rope=None,
-                   k_rope=None, lse=None, head_major=False, poison_workspace=False, fractal_nz=False):
+                   k_rope=None, lse=None, head_major=False, poison_workspace=False, fractal_nz=False, causal_rows=None):
     """atbmi_pa_plan_* + atbmi_pa_decode on `stream`; returns the output tensor.
     mask: device tensor of q's dtype shaped like one of the reference's decode
     masks; mask_per_head says that a 3-dim mask's first dim counts heads (ALIBI).
     q_rope / k_rope: the split latent layout (q and kc then hold the first 512
     channels); lse: a [rows, heads] tensor of q's dtype that receives the log-sum-exp;
-    fractal_nz: kc and k_rope are [blocks, channels / 16, block size, 16]."""
+    fractal_nz: kc and k_rope are [blocks, channels / 16, block size, 16]; causal_rows: True or a
+    list of flags per sequence (atbmi_pa_plan_set_causal_rows)."""
     k = binding.kernels()
     rows, heads, d = q.shape
     rope = 0 if q_rope is None else q_rope.shape[2]
@@ -65,6 +66,12 @@ def pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx_host, scale, k_scale=
         raise RuntimeError("plan_create: " + binding.last_kernel_error())
     try:
         lens = np.ascontiguousarray(np.asarray(ctx_host, dtype=np.int32))
+        if causal_rows is not None:
+            flags = None if causal_rows is True else np.ascontiguousarray(np.asarray(causal_rows, dtype=np.int32))
+            rc = k.atbmi_pa_plan_set_causal_rows(plan, 1, None if flags is None else flags.ctypes.data,
+                                                 0 if flags is None else len(flags))
+            if rc != 0:
+                raise RuntimeError("plan_set_causal_rows: " + binding.last_kernel_error())
         if q_lens is None:
             rc = k.atbmi_pa_plan_update(plan, lens.ctypes.data, len(lens))
         else:
@@ -128,7 +135,8 @@ def mask_strides(mask, per_head):
 
 def oracle_pa(oracle, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=None, v_scale=None, v_off=None,
               mla_dv=0, q_scale=0.0, out_init=0.0, mask=None, mask_per_head=False, logn=None, q_lens=None,
-              mask_rows="sequence", lse_out=None, head_major=False, compress_kv_heads=0, razor_offset=None):
+              mask_rows="sequence", lse_out=None, head_major=False, compress_kv_heads=0, razor_offset=None,
+              causal_rows=None):
     qd = "bf16" if q.dtype == torch.bfloat16 else "float16"
     return oracle.paged_attention(
         to_oracle(q), to_oracle(kc), to_oracle(vc), tables.cpu().numpy(), np.asarray(ctx_host), scale,
@@ -136,7 +144,7 @@ def oracle_pa(oracle, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=No
         q_scale=q_scale, q_dtype=qd, out_init=out_init, mask=to_oracle(mask), logn=to_oracle(logn),
         mask_per_head=mask_per_head if (mask is not None and mask.dim() == 3) else None, q_lens=q_lens,
         mask_rows=mask_rows, lse_out=lse_out, head_major=head_major, compress_kv_heads=compress_kv_heads,
-        razor_offset=to_oracle(razor_offset))
+        razor_offset=to_oracle(razor_offset), causal_rows=causal_rows)
 
 
 def assert_close(got, want, tol, what=""):

@@ -31,7 +31,7 @@ def stream(dev):
     return torch.cuda.Stream(device=dev)
 
 
-def _case(seed, dev, ctx, heads, dtype, q_lens=None, with_mask=False):
+def _case(seed, dev, ctx, heads, dtype, q_lens=None, with_mask=False, causal=None):
     """Inputs drawn the way the reference test draws them (:478-506: uniform in [-5, 5], descales in +-5/127)."""
     rng = np.random.Generator(np.random.PCG64(seed))
     ctx = np.asarray(ctx, np.int32)
@@ -57,7 +57,7 @@ def _case(seed, dev, ctx, heads, dtype, q_lens=None, with_mask=False):
                 r += 1
         mask = torch.from_numpy(m).to(dtype)
     return dict(q8=q8, qr=qr, kv8=kv8, kr=kr, tables=torch.from_numpy(tables), ctx=ctx, qd=qd, pd=pd, mask=mask,
-                q_lens=q_lens, rows=rows, heads=heads, dtype=dtype)
+                q_lens=q_lens, rows=rows, heads=heads, dtype=dtype, causal=causal)
 
 
 def _nz(oracle, t, n0):
@@ -71,7 +71,7 @@ def _oracle(oracle, c, scale, tile, lse=None):
     return oracle.mla_int8_decode(c["q8"].numpy(), c["qr"].float().numpy(), c["kv8"].numpy(), c["kr"].float().numpy(),
                                   c["tables"].numpy(), c["ctx"], c["qd"].numpy(), c["pd"].numpy(), scale, tile=tile,
                                   mask=None if c["mask"] is None else c["mask"].float().numpy(), q_lens=c["q_lens"],
-                                  lse_out=lse)
+                                  lse_out=lse, causal_rows=c["causal"])
 
 
 def int8_cabi(binding, oracle, stream, dev, c, scale, want_lse=False):
@@ -82,11 +82,13 @@ def int8_cabi(binding, oracle, stream, dev, c, scale, want_lse=False):
     mask = c["mask"].to(dev) if c["mask"] is not None else None
     lens = np.ascontiguousarray(c["ctx"], dtype=np.int32)
     ql = None if c["q_lens"] is None else np.ascontiguousarray(np.asarray(c["q_lens"], dtype=np.int32))
+    use = None if c["causal"] in (None, True) else np.ascontiguousarray(np.asarray(c["causal"], dtype=np.int32))
     call = binding.AtbmiMlaInt8Call(
         outDtype=dtype_code(binding, c["qr"]), numHeads=c["heads"], blockSize=128, numBlocks=kv_nz.shape[0],
         maxBlocksPerSeq=c["tables"].shape[1], batch=len(lens), numQueryRows=c["rows"], hasMask=0 if mask is None else 1,
         maskLen=0 if mask is None else mask.shape[1], qkScale=scale, hostContextLens=lens.ctypes.data,
-        hostQueryLens=None if ql is None else ql.ctypes.data)
+        hostQueryLens=None if ql is None else ql.ctypes.data, causalRows=0 if c["causal"] is None else 1,
+        hostCausalUse=None if use is None else use.ctypes.data)
     ws_bytes = ctypes.c_uint64(0)
     if k.atbmi_mla_int8_workspace_size(ctypes.byref(call), ctypes.byref(ws_bytes)) != 0:
         raise RuntimeError("mla_int8_workspace_size: " + binding.last_kernel_error())
@@ -121,23 +123,27 @@ def _double_golden(true_out, golden, got, dtype):
     return rates[0] < 10 and rates[1] < 2 and rates[2] < 2, rates
 
 
-# ctx, heads, dtype, q_lens, mask    (reference :668-766: 32 sequences of 256 tokens, 32 / 128 heads; :845-1104 the
-# several-query-token cases with their look-ahead mask)
+# ctx, heads, dtype, q_lens, mask, causal rows    (reference :668-766: 32 sequences of 256 tokens, 32 / 128 heads;
+# :1270-1367 several query tokens: row j of q sees context + j - q + 1 tokens (:356-364), per sequence with
+# batch_list. The mask cases exercise the kernel layer's own mask input, which the operation does not use.)
 INT8_MATRIX = [
-    ([256] * 32, 32, torch.float16, None, False),
-    ([256] * 8, 128, torch.float16, None, False),
-    ([256] * 32, 32, torch.bfloat16, None, False),
-    ([700, 0, 1, 128, 129, 1500], 8, torch.float16, None, False),
-    ([515, 33, 2048], 64, torch.bfloat16, [2, 1, 3], True),
-    ([300, 1000, 0, 77], 16, torch.float16, [2, 2, 1, 4], True),
+    ([256] * 32, 32, torch.float16, None, False, None),
+    ([256] * 8, 128, torch.float16, None, False, None),
+    ([256] * 32, 32, torch.bfloat16, None, False, None),
+    ([700, 0, 1, 128, 129, 1500], 8, torch.float16, None, False, None),
+    ([515, 33, 2048], 64, torch.bfloat16, [2, 1, 3], True, None),
+    ([300, 1000, 0, 77], 16, torch.float16, [2, 2, 1, 4], True, None),
+    ([256, 256], 128, torch.float16, [2, 2], False, True),
+    ([515, 129, 2048, 4], 64, torch.bfloat16, [2, 1, 3, 4], False, True),
+    ([300, 1000, 0, 130], 16, torch.float16, [2, 2, 1, 4], False, [1, 0, 1, 1]),
 ]
 
 
 @pytest.mark.parametrize("case", INT8_MATRIX, ids=lambda c: "b%d_h%d_%s%s" % (
-    len(c[0]), c[1], str(c[2]).split(".")[-1], "_multi" if c[3] else ""))
+    len(c[0]), c[1], str(c[2]).split(".")[-1], ("_multi" if c[3] else "") + ("_causal" if c[5] is not None else "")))
 def test_mla_int8_nz_kernel(binding, oracle, dev, stream, case):
-    ctx, heads, dtype, q_lens, with_mask = case
-    c = _case(600 + heads + len(ctx), dev, ctx, heads, dtype, q_lens, with_mask)
+    ctx, heads, dtype, q_lens, with_mask, causal = case
+    c = _case(600 + heads + len(ctx), dev, ctx, heads, dtype, q_lens, with_mask, causal)
     scale = 1.0 / math.sqrt(576.0)
     want_lse = np.zeros((c["rows"], heads), np.float32)
     want = _oracle(oracle, c, scale, 128, want_lse)
@@ -154,17 +160,22 @@ def test_mla_int8_nz_kernel(binding, oracle, dev, stream, case):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_mla_int8_nz_through_operation_api(binding, oracle, dev, stream, dtype):
     """MultiLatentAttentionOperation with cacheMode INT8_NZCACHE through InferShape / Setup / Execute: plain decode,
-    log-sum-exp output (fp32), several query tokens with their mask, and both. Inputs: query (int8), queryRope,
-    kvCache (int8, fractal-NZ), kvCacheRope (fractal-NZ), blockTables, contextLens, [mask], [qSeqlen], qkDescale,
-    pvDescale (reference multi_latent_attention_operation.cpp:245-266)."""
+    log-sum-exp output (fp32), several query tokens (each sees the context up to itself, with or without a mask
+    tensor, which the reference's int8 kernels do not read: tiling/mla_tiling.cpp:139-144; golden :356-364), and
+    maskUseStatus, which exempts sequences from that (golden batch_list, :1348-1367). Inputs: query (int8),
+    queryRope, kvCache (int8, fractal-NZ), kvCacheRope (fractal-NZ), blockTables, contextLens, [mask], [qSeqlen],
+    qkDescale, pvDescale, [maskUseStatus] (reference multi_latent_attention_operation.cpp:245-266)."""
     heads = 32
     scale = 1.0 / math.sqrt(576.0)
     ctx = [700, 33, 1500, 128]
     q_lens = [2, 1, 3, 1]
     c = binding.Context(stream)
-    for calc, mask_type in ((0, 0), (2, 0), (1, 1), (3, 0), (1, 0)):
+    for calc, mask_type, use in ((0, 0, None), (2, 0, None), (1, 1, None), (3, 0, None), (1, 0, None),
+                                 (3, 0, [1, 1, 0, 1]), (3, 0, [])):
         multi, ring = calc in (1, 3), calc in (2, 3)
-        case = _case(700 + calc, dev, ctx, heads, dtype, q_lens if multi else None, mask_type == 1)
+        causal = None if not multi else (use if use else True)
+        case = _case(700 + calc, dev, ctx, heads, dtype, q_lens if multi else None, mask_type == 1, causal)
+        mask_tensor, case["mask"] = case["mask"], None   # (handed to the operation, not used by it)
         kv_nz = _nz(oracle, case["kv8"], 32).to(dev)
         kr_nz = _nz(oracle, case["kr"], 16).to(dev)
         lens = torch.from_numpy(case["ctx"])
@@ -173,14 +184,20 @@ def test_mla_int8_nz_through_operation_api(binding, oracle, dev, stream, dtype):
         ins = [case["q8"].to(dev), case["qr"].to(dev), nz_desc(kv_nz), nz_desc(kr_nz), case["tables"].to(dev), lens.to(dev)]
         host = {5: lens}
         if mask_type == 1:
-            ins.append(case["mask"].to(dev))
+            ins.append(mask_tensor.to(dev))
         if multi:
             qn = torch.tensor(q_lens, dtype=torch.int32)
             host[len(ins)] = qn
             ins.append(qn.to(dev))
         ins += [case["qd"].to(dev), case["pd"].to(dev)]
+        if use is not None:
+            flags = torch.tensor(use, dtype=torch.int32)
+            if use:
+                host[len(ins)] = flags
+            ins.append(flags.to(dev) if use else binding.make_tensor("int32", [0], device_ptr=0))
         op = binding.OperationRunner("MultiLatentAttentionOperation", binding.MultiLatentAttentionParam(
-            headNum=heads, kvHeadNum=1, qkScale=scale, cacheMode=2, calcType=calc, maskType=mask_type), c)
+            headNum=heads, kvHeadNum=1, qkScale=scale, cacheMode=2, calcType=calc, maskType=mask_type,
+            maskUseStatusType=0 if use is None else 1), c)
         with torch.cuda.stream(stream):
             outs = op.run(ins, host_inputs=host)
         stream.synchronize()

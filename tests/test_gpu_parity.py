@@ -1423,7 +1423,10 @@ def test_multi_latent_attention_operation(binding, oracle, dev, stream, heads, d
     """MultiLatentAttentionOperation, cacheMode KROPE_CTKV, through Setup / Execute: plain decode, with
     the log-sum-exp output (CALC_TYPE_RING), several query tokens with the SPEC mask (CALC_TYPE_SPEC) and
     both (CALC_TYPE_SPEC_AND_RING). Inputs: query, queryRope, kvCache, kvCacheRope, blockTables,
-    contextLens, [mask], [qSeqlen] (reference multi_latent_attention_operation.cpp:245-266)."""
+    contextLens, [mask], [qSeqlen] (reference multi_latent_attention_operation.cpp:245-266). With 128 heads the
+    reference runs a job per query token over the context up to that token and does not read the mask
+    (tiling/mla_tiling.cpp:139-144, mla_tiling_dependency.cpp:292-316): the oracle then takes causal rows and no
+    mask, although the (randomly biased) mask tensor is handed over."""
     rng = _rng(440 + heads)
     d, dv, block = 576, 512, 128
     ctx = np.array([700, 33, 1500, 128], dtype=np.int32)
@@ -1451,9 +1454,10 @@ def test_multi_latent_attention_operation(binding, oracle, dev, stream, heads, d
         stream.synchronize()
         assert len(outs) == (2 if ring else 1) and tuple(outs[0].shape) == (rows, heads, dv)
         want_lse = np.zeros((rows, heads), np.float32)
-        want = oracle_pa(oracle, q, kc, None, tables, ctx, scale, mla_dv=dv, mask=mask,
+        per_token = multi and heads == 128
+        want = oracle_pa(oracle, q, kc, None, tables, ctx, scale, mla_dv=dv, mask=None if per_token else mask,
                          q_lens=q_lens if multi else None, mask_rows="query" if multi else "sequence",
-                         lse_out=want_lse)
+                         lse_out=want_lse, causal_rows=True if per_token else None)
         assert_close(outs[0], want, TOL[dtype], "calcType %d" % calc)
         if ring:
             assert tuple(outs[1].shape) == (rows, heads, 1) and outs[1].dtype == dtype
@@ -1471,6 +1475,76 @@ def test_multi_latent_attention_operation(binding, oracle, dev, stream, heads, d
             outs_nz = op.run(ins, host_inputs=host)
         stream.synchronize()
         assert len(outs_nz) == len(outs) and all(torch.equal(a, b) for a, b in zip(outs, outs_nz)), "NZCACHE %d" % calc
+        op.close()
+    c.close()
+
+
+@pytest.mark.parametrize("kernel", [1, 2])
+def test_causal_rows_through_the_c_abi(binding, oracle, dev, stream, kernel):
+    """atbmi_pa_plan_set_causal_rows: the t-th of n query rows attends to the first ctx - n + t + 1 tokens, per
+    sequence when flags are given; on the generic kernels (GQA, where query tokens would otherwise share a pass)
+    and on the MLA kernels (16 and 128 heads), whole rows and rows cut into ranges."""
+    rng = _rng(480 + kernel)
+    for heads, kv_heads, d, dv, ctx, q_lens, flags, dtype, chunk in (
+            (32, 8, 128, 0, [1000, 0, 2300, 130, 4], [2, 3, 4, 1, 4], None, torch.bfloat16, None),
+            (32, 8, 128, 0, [1000, 0, 2300, 130, 4], [2, 3, 4, 1, 4], [1, 1, 0, 1, 0], torch.float16, 256),
+            (16, 1, 576, 512, [300, 1200], [2, 4], None, torch.float16, None),
+            (128, 1, 576, 512, [700, 33, 1500], [2, 1, 3], [0, 1, 1], torch.bfloat16, None)):
+        q_lens_np = np.asarray(q_lens, np.int32)
+        _, kc, vc, tables, ctx = _pa_inputs(rng, dev, len(ctx), heads, kv_heads, 128, d, dv or d, ctx, dtype, std=0.5)
+        rows = int(sum(n for n, c in zip(q_lens, ctx) if c > 0))
+        q = (torch.rand((rows, heads, d)) * 2 - 1).to(dtype).to(dev)
+        scale = 1.0 / math.sqrt(d)
+        lse = torch.zeros((rows, heads), dtype=dtype, device=dev)
+        got = pa_decode_cabi(binding, stream, q, kc, None if dv else vc, tables, ctx, scale, mla_dv=dv, kernel=kernel,
+                             q_lens=q_lens_np, lse=lse, chunk_tokens=chunk,
+                             causal_rows=True if flags is None else flags)
+        want_lse = np.zeros((rows, heads), np.float32)
+        want = oracle_pa(oracle, q, kc, None if dv else vc, tables, ctx, scale, mla_dv=dv, q_lens=q_lens_np,
+                         lse_out=want_lse, causal_rows=True if flags is None else flags)
+        assert_close(got, want, TOL[dtype], "causal rows heads=%d kernel=%d" % (heads, kernel))
+        assert_close(lse, want_lse, TOL[dtype], "causal rows lse heads=%d kernel=%d" % (heads, kernel))
+
+
+def test_multi_latent_attention_causal_mask_types(binding, oracle, dev, stream):
+    """MultiLatentAttentionOperation with several query tokens and no mask tensor to read: MASK_TYPE_CAUSAL_MASK (any
+    head count), MASK_TYPE_MASK_FREE on 128 heads with maskUseStatus flags per sequence (reference golden
+    test_multi_latent_attention_mtp.py:160-180,582-633: the look-ahead rows, or the whole context where the flag
+    is 0), and 128 heads with no mask type at all (the reference's job per query token)."""
+    rng = _rng(490)
+    d, dv, block, dtype = 576, 512, 128, torch.float16
+    ctx = np.array([700, 33, 1500, 128], dtype=np.int32)
+    q_lens = np.array([2, 1, 3, 2], dtype=np.int32)
+    rows = int(q_lens.sum())
+    scale = 1.0 / math.sqrt(192.0)
+    lens, qn = torch.from_numpy(ctx), torch.from_numpy(q_lens)
+    c = binding.Context(stream)
+    for heads, calc, mask_type, flags in ((32, 1, 3, None), (128, 3, 2, [1, 0, 1, 1]), (128, 3, 2, None),
+                                          (128, 1, 0, None)):
+        _, kc, _, tables, _ = _pa_inputs(rng, dev, 4, heads, 1, block, d, d, ctx, dtype, std=0.5)
+        k_nope, k_rope = kc[..., :dv].contiguous(), kc[..., dv:].contiguous()
+        q = (torch.rand((rows, heads, d)) * 2 - 1).to(dtype).to(dev)
+        ins = [q[..., :dv].contiguous(), q[..., dv:].contiguous(), k_nope, k_rope, tables, lens.to(dev)]
+        host = {5: lens}
+        if mask_type == 2:   # the template of the reference's mask-free tests ([125 + 2 q, 128]); not read on this path
+            ins.append(torch.from_numpy(np.triu(np.full((131, 128), -10000.0, np.float32), -1)).to(dtype).to(dev))
+        host[len(ins)] = qn
+        ins.append(qn.to(dev))
+        if flags is not None:
+            host[len(ins)] = torch.tensor(flags, dtype=torch.int32)
+            ins.append(host[len(ins)].to(dev))
+        op = binding.OperationRunner("MultiLatentAttentionOperation", binding.MultiLatentAttentionParam(
+            headNum=heads, kvHeadNum=1, qkScale=scale, cacheMode=1, calcType=calc, maskType=mask_type,
+            maskUseStatusType=0 if flags is None else 1), c)
+        with torch.cuda.stream(stream):
+            outs = op.run(ins, host_inputs=host)
+        stream.synchronize()
+        want_lse = np.zeros((rows, heads), np.float32)
+        want = oracle_pa(oracle, q, kc, None, tables, ctx, scale, mla_dv=dv, q_lens=q_lens, lse_out=want_lse,
+                         causal_rows=True if flags is None else flags)
+        assert_close(outs[0], want, TOL[dtype], "heads %d calcType %d maskType %d" % (heads, calc, mask_type))
+        if calc == 3:
+            assert_close(outs[1][..., 0], want_lse, TOL[dtype], "lse heads %d" % heads)
         op.close()
     c.close()
 
@@ -1513,8 +1587,9 @@ def test_two_call_c_wrappers_run_the_operations(binding, oracle, dev, stream):
         stream.synchronize()
         assert st == 0, binding.ERROR_NAMES[st]
         want_lse = np.zeros((rows, heads), np.float32)
-        want = oracle_pa(oracle, q, kc, None, tables, ctx_lens, scale, mla_dv=dv, mask=mask,
-                         q_lens=q_lens if multi else None, mask_rows="query" if multi else "sequence", lse_out=want_lse)
+        # (128 heads: a job per query token, the mask tensor is not read)
+        want = oracle_pa(oracle, q, kc, None, tables, ctx_lens, scale, mla_dv=dv, mask=None,
+                         q_lens=q_lens if multi else None, lse_out=want_lse, causal_rows=True if multi else None)
         assert_close(out, want, TOL[dtype], "AtbMLA calcType %d" % calc)
         if ring:
             assert_close(lse[..., 0], want_lse, TOL[dtype], "AtbMLA lse")

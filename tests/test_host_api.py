@@ -63,11 +63,9 @@ def _rac_unimplemented(p):
 
 
 def _mla_unimplemented(p):
-    """Features of MultiLatentAttentionParam the reference accepts but this library rejects at creation:
-    decode masks other than MASK_TYPE_SPEC, maskUseStatus."""
-    if p.get("calcType", 0) == 4:
-        return False
-    return p.get("maskType", 0) >= 2 or p.get("maskUseStatusType", 0) != 0
+    """Features of MultiLatentAttentionParam the reference accepts but this library rejects at creation: none
+    (MASK_TYPE_MASK_FREE with fewer than 128 heads is refused at Setup, which no table row reaches)."""
+    return False
 
 
 def _make_param(binding, op, p):
@@ -162,6 +160,10 @@ def _check(binding, case, ctx, unimplemented, refused_at_setup=False):
         assert (stage, status) == ("", 0), "%s: %s:%s" % (case["name"], stage, binding.ERROR_NAMES[status])
         got = [[d.dims[i] for i in range(d.dimNum)] for d in out_descs]
         assert got == case["out_shapes"]
+        return
+    if expected == "I:NO_ERROR":
+        # the row only asks InferShape to succeed (its output shapes are not the operation's)
+        assert stage not in ("C", "I"), "%s: %s:%s" % (case["name"], stage, binding.ERROR_NAMES[status])
         return
     want_stage, want_name = expected.split(":")
     assert stage == want_stage and binding.ERROR_NAMES[status] == want_name, \
@@ -258,10 +260,9 @@ def test_table_coverage():
     rac_dev = [c for c in RAC_CASES if _rac_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
     assert len(PA_CASES) == 81 and len(PA_CASES) - len(pa_dev) >= 75
     assert len(RAC_CASES) == 38 and len(RAC_CASES) - len(rac_dev) >= 29
-    # the MultiLatentAttention rows replayed as "rejected at creation" exercise decode masks other than
-    # MASK_TYPE_SPEC and maskUseStatus
+    # every MultiLatentAttention row is replayed at face value
     mla_dev = [c for c in MLA_CASES if _mla_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
-    assert len(MLA_CASES) == 147 and len(MLA_CASES) - len(mla_dev) == 144
+    assert len(MLA_CASES) == 147 and len(mla_dev) == 0
 
 
 def test_param_sizes(binding):
@@ -570,16 +571,21 @@ def test_multi_latent_attention_counts_shapes_and_setup(binding, ctx):
     e = binding.ERROR_CODE
     mk = binding.MultiLatentAttentionParam
     for kw, n_in, n_out in ((dict(), 6, 1), (dict(calcType=1), 7, 1), (dict(calcType=1, maskType=1), 8, 1),
-                            (dict(calcType=2), 6, 2), (dict(calcType=3, maskType=1), 8, 2)):
-        op = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07,
-                                                                   cacheMode=1, **kw))
+                            (dict(calcType=2), 6, 2), (dict(calcType=3, maskType=1), 8, 2),
+                            (dict(calcType=1, maskType=2), 8, 1),       # MASK_FREE brings its template
+                            (dict(calcType=1, maskType=3), 7, 1),       # CAUSAL_MASK has no mask tensor
+                            (dict(calcType=3, maskUseStatusType=1), 8, 2),
+                            (dict(calcType=3, maskType=2, maskUseStatusType=1), 9, 2),
+                            (dict(calcType=3, cacheMode=2, maskUseStatusType=1), 10, 2)):
+        op = binding.Operation("MultiLatentAttentionOperation", mk(**dict(dict(headNum=32, kvHeadNum=1, qkScale=0.07,
+                                                                             cacheMode=1), **kw)))
         assert op.ok and (op.input_num(), op.output_num()) == (n_in, n_out), kw
         op.close()
     for bad in (dict(headNum=12), dict(kvHeadNum=2), dict(cacheMode=0), dict(maskType=1), dict(qkScale=1.5),
                 dict(qkScale=0.0), dict(calcType=5), dict(cacheMode=4), dict(calcType=4, headNum=32),
                 dict(cacheMode=2, calcType=2, maskType=1),
-                dict(calcType=1, maskType=2), dict(calcType=1, maskType=3), dict(calcType=1, maskType=4),
-                dict(calcType=3, maskUseStatusType=1)):
+                dict(calcType=1, maskType=4), dict(calcType=1, maskUseStatusType=1), dict(maskUseStatusType=1),
+                dict(calcType=3, maskUseStatusType=2), dict(calcType=3, maskUseStatusType=-1)):
         kw = dict(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1)
         kw.update(bad)
         assert binding.Operation("MultiLatentAttentionOperation", mk(**kw)).status == e["ERROR_INVALID_PARAM"], bad
@@ -638,6 +644,61 @@ def test_multi_latent_attention_counts_shapes_and_setup(binding, ctx):
     assert spec.setup(pack(rows=6, mask=[6, 300], with_qlens=True, qlens_host=False), outs(rows=6), ctx)[0] == \
         e["ERROR_INVALID_PARAM"]
     spec.close()
+
+
+def test_multi_latent_attention_causal_rows_and_mask_use_status(binding, ctx):
+    """Several query tokens on the reference's job-per-token path (128 heads, or the int8 cache): the mask tensor is
+    not read, maskUseStatus is an optional host tensor [batch] (reference multi_latent_attention_operation.cpp:
+    536-575, ops_runner :117-131, tiling mla_tiling.cpp:139-144); MASK_TYPE_MASK_FREE with fewer heads is refused
+    at Setup."""
+    e = binding.ERROR_CODE
+    mk = binding.MultiLatentAttentionParam
+    lens = np.array([10, 300, 0, 64], dtype=np.int32)
+    qlens = np.array([1, 3, 2, 2], dtype=np.int32)   # 6 query rows
+    use = np.array([1, 0, 1, 1], dtype=np.int32)
+
+    def pack(heads, mask=None, use_shape=None, use_host=True, qlens_host=qlens):
+        ins = [binding.make_tensor("float16", [6, heads, 512], FAKE_DEVICE),
+               binding.make_tensor("float16", [6, heads, 64], FAKE_DEVICE),
+               binding.make_tensor("float16", [16, 128, 1, 512], FAKE_DEVICE),
+               binding.make_tensor("float16", [16, 128, 1, 64], FAKE_DEVICE),
+               binding.make_tensor("int32", [4, 3], FAKE_DEVICE),
+               binding.make_tensor("int32", [4], FAKE_DEVICE, host_ptr=lens.ctypes.data)]
+        if mask is not None:
+            ins.append(binding.make_tensor("float16", mask, FAKE_DEVICE))
+        ins.append(binding.make_tensor("int32", [4], FAKE_DEVICE, host_ptr=qlens_host.ctypes.data))
+        if use_shape is not None:
+            ins.append(binding.make_tensor("int32", use_shape, FAKE_DEVICE, host_ptr=use.ctypes.data if use_host else None))
+        return ins
+
+    def outs(heads, lse=True):
+        o = [binding.make_tensor("float16", [6, heads, 512], FAKE_DEVICE)]
+        return o + ([binding.make_tensor("float16", [6, heads, 1], FAKE_DEVICE)] if lse else [])
+
+    # 128 heads: any mask shape passes, because the tensor is not read; the flags come from the host
+    op = binding.Operation("MultiLatentAttentionOperation", mk(headNum=128, kvHeadNum=1, qkScale=0.07, cacheMode=1,
+                                                               calcType=3, maskType=2, maskUseStatusType=1))
+    assert op.ok and op.input_num() == 9
+    assert op.setup(pack(128, mask=[129, 128], use_shape=[4]), outs(128), ctx)[0] == 0
+    assert op.setup(pack(128, mask=[4, 129, 128], use_shape=[4]), outs(128), ctx)[0] == 0
+    assert op.setup(pack(128, mask=[129, 128], use_shape=[0]), outs(128), ctx)[0] == 0        # optional: left out
+    assert op.setup(pack(128, mask=[129, 128], use_shape=[4], use_host=False), outs(128), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    assert op.setup(pack(128, mask=[129, 128], use_shape=[3]), outs(128), ctx)[0] == e["ERROR_INVALID_TENSOR_DIM"]
+    assert op.setup(pack(128, mask=[129, 128], use_shape=[4, 1]), outs(128), ctx)[0] == e["ERROR_INVALID_TENSOR_DIM_NUM"]
+    # more query tokens than context cannot be made causal
+    assert op.setup(pack(128, mask=[129, 128], use_shape=[4], qlens_host=np.array([11, 3, 0, 2], np.int32)),
+                    outs(128), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    op.close()
+    # fewer heads: the reference's other kernel path reads the template; not built here
+    op = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1,
+                                                               calcType=1, maskType=2))
+    assert op.ok and op.setup(pack(32, mask=[129, 128]), outs(32, lse=False), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    op.close()
+    # CAUSAL_MASK: no mask tensor, any head count
+    op = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1,
+                                                               calcType=1, maskType=3))
+    assert op.ok and op.setup(pack(32), outs(32, lse=False), ctx)[0] == 0
+    op.close()
 
 
 def test_multi_latent_attention_int8_nz_cache_checks(binding, ctx):
@@ -704,7 +765,8 @@ def test_multi_latent_attention_int8_nz_cache_checks(binding, ctx):
                                                                  calcType=1, maskType=1))
     assert spec.ok and spec.input_num() == 10
     assert spec.setup(pack(rows=6, with_qlens=True, mask=(6, 300)), outs(rows=6), ctx)[0] == 0
-    assert spec.setup(pack(rows=6, with_qlens=True, mask=(6, 299)), outs(rows=6), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    # the int8 kernels of the reference never read the mask (tiling/mla_tiling.cpp:142-144): its shape is not looked at
+    assert spec.setup(pack(rows=6, with_qlens=True, mask=(6, 299)), outs(rows=6), ctx)[0] == 0
     spec.close()
 
 

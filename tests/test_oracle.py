@@ -841,6 +841,36 @@ def test_multi_token_causal_mask_equals_growing_contexts(oracle):
                           oracle.paged_attention(q, kc, vc, tables, ctx, 0.3))
 
 
+def test_causal_rows_equal_the_look_ahead_mask_and_growing_contexts(oracle):
+    """causal_rows: the t-th of n query rows sees ctx - n + t + 1 tokens. Pinned three ways: against every row
+    run as a sequence of its own with the shortened context (what the reference's per-token jobs are), against
+    the -inf look-ahead mask, and per sequence (a flag of 0 keeps the whole context)."""
+    rng = _rng(43)
+    q, kc, vc, tables, ctx = _paged_case(rng, batch=3, heads=4, kv_heads=2, max_ctx=14)
+    ctx = np.maximum(ctx, 5)
+    q_lens = np.array([3, 1, 5], np.int32)
+    query = rng.standard_normal((9, 4, 16)).astype(np.float32)
+    lse = np.zeros((9, 4), np.float32)
+    got = oracle.paged_attention(query, kc, vc, tables, ctx, 0.3, q_lens=q_lens, causal_rows=True, lse_out=lse)
+    tables_x, ctx_x, owner, token = _expand_rows(tables, ctx, q_lens)
+    seen = (ctx_x - q_lens[owner] + token + 1).astype(np.int32)
+    lse_x = np.zeros((9, 4), np.float32)
+    want = oracle.paged_attention(query, kc, vc, tables_x, seen, 0.3, lse_out=lse_x)
+    assert np.array_equal(got, want) and np.array_equal(lse, lse_x)
+    look_ahead = np.zeros((9, 14), np.float32)
+    for r in range(9):
+        look_ahead[r, seen[r]:] = -np.inf
+    masked = oracle.paged_attention(query, kc, vc, tables, ctx, 0.3, q_lens=q_lens, mask=look_ahead, mask_rows="query")
+    np.testing.assert_allclose(got, masked, rtol=1e-6, atol=1e-6)
+    # flags per sequence: sequence 0 keeps its whole context, the others are cut
+    flags = np.array([0, 1, 1], np.int32)
+    part = oracle.paged_attention(query, kc, vc, tables, ctx, 0.3, q_lens=q_lens, causal_rows=flags)
+    full = oracle.paged_attention(query, kc, vc, tables, ctx, 0.3, q_lens=q_lens)
+    assert np.array_equal(part[:3], full[:3]) and np.array_equal(part[3:], got[3:])
+    assert not np.array_equal(got[:2], full[:2])           # (the cut changes rows that lose tokens)
+    assert np.array_equal(got[2], full[2])                 # (the last row of a sequence loses none)
+
+
 # ---------------------------------------------------------------- log-sum-exp output
 def test_lse_closed_forms_and_logsumexp(oracle):
     from scipy.special import logsumexp
@@ -1008,6 +1038,31 @@ def test_int8_decode_matches_independent_loops(oracle, tile):
                 np.testing.assert_allclose(got[row, h], num / den, rtol=2e-5, atol=2e-6)
                 np.testing.assert_allclose(lse[row, h], math.log(den) + ref, rtol=1e-5, atol=1e-5)
             row += 1
+
+
+def test_int8_decode_causal_rows_are_shortened_contexts(oracle):
+    """The reference golden runs the j-th of q query rows over context + j - q + 1 tokens
+    (test_multi_latent_attention_int8nz.py:356-364): causal_rows equals that row run alone as a sequence with the
+    shortened context (tiles and all), and a sequence flagged 0 keeps the whole context."""
+    rng = _rng(147)
+    q_lens = [3, 1, 2]
+    q8, qr, kv8, kr, tables, ctx, qd, pd = _int8_case(rng, [37, 5, 96], heads=3, q_lens=q_lens)
+    lse = np.zeros((6, 3), np.float32)
+    got = oracle.mla_int8_decode(q8, qr, kv8, kr, tables, ctx, qd, pd, 0.04, tile=16, q_lens=q_lens, causal_rows=True,
+                                 lse_out=lse)
+    row = 0
+    for b, n in enumerate(q_lens):
+        for j in range(n):
+            one_lse = np.zeros((1, 3), np.float32)
+            alone = oracle.mla_int8_decode(q8[row:row + 1], qr[row:row + 1], kv8, kr, tables[b:b + 1],
+                                           [ctx[b] + j - n + 1], qd, pd, 0.04, tile=16, lse_out=one_lse)
+            assert np.array_equal(got[row], alone[0]) and np.array_equal(lse[row], one_lse[0])
+            row += 1
+    full = oracle.mla_int8_decode(q8, qr, kv8, kr, tables, ctx, qd, pd, 0.04, tile=16, q_lens=q_lens)
+    part = oracle.mla_int8_decode(q8, qr, kv8, kr, tables, ctx, qd, pd, 0.04, tile=16, q_lens=q_lens,
+                                  causal_rows=[0, 1, 1])
+    assert np.array_equal(part[:3], full[:3]) and np.array_equal(part[3:], got[3:])
+    assert not np.array_equal(got[0], full[0]) and np.array_equal(got[2], full[2])
 
 
 def test_int8_decode_limits_and_closed_forms(oracle):
