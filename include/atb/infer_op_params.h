@@ -132,9 +132,9 @@ struct MultiLatentAttentionParam {
     enum MaskType : int {
         UNDEFINED = 0,         // no mask input
         MASK_TYPE_SPEC,        // one mask row per query token, with CALC_TYPE_SPEC
-        MASK_TYPE_MASK_FREE,   // compressed causal mask; not implemented on MI355X
-        MASK_TYPE_CAUSAL_MASK, // mask generated inside the kernel; not implemented on MI355X
-        MASK_TYPE_SWA_NORM     // sliding window (prefill); not implemented on MI355X
+        MASK_TYPE_MASK_FREE,   // compressed causal mask (decode: 128 heads or int8 cache only; prefill)
+        MASK_TYPE_CAUSAL_MASK, // causal, no mask tensor
+        MASK_TYPE_SWA_NORM     // sliding window of windowSize tokens (prefill only)
     };
     MaskType maskType = UNDEFINED;
 
@@ -143,15 +143,15 @@ struct MultiLatentAttentionParam {
         CALC_TYPE_SPEC,          // qSeqlen input: several query tokens per sequence
         CALC_TYPE_RING,          // second output: the log-sum-exp of every row
         CALC_TYPE_SPEC_AND_RING, // both
-        CALC_TYPE_PREFILL        // not implemented on MI355X
+        CALC_TYPE_PREFILL        // prompt attention over key / value tensors instead of the caches
     };
     CalcType calcType = CALC_TYPE_UNDEFINED;
 
     enum CacheMode : uint8_t {
         KVCACHE = 0,  // one 576-channel cache; rejected by the reference itself
         KROPE_CTKV,   // latent cache [blocks, 128, 1, 512] + rotary cache [blocks, 128, 1, 64]
-        INT8_NZCACHE, // int8 fractal-NZ caches; not implemented on MI355X
-        NZCACHE       // 16-bit fractal-NZ caches; not implemented on MI355X
+        INT8_NZCACHE, // int8 latent cache [blocks, 16, 128, 32] + 16-bit rotary cache, fractal-NZ; int8 query
+        NZCACHE       // the 16-bit caches in fractal-NZ: [blocks, 32, 128, 16] + [blocks, 4, 128, 16]
     };
     CacheMode cacheMode = KVCACHE;
 
@@ -159,7 +159,7 @@ struct MultiLatentAttentionParam {
 
     enum MaskUseStatusType : int {
         MASK_USE_STATUS_TYPE_UNDEFINED = 0,
-        MASK_USE_STATUS_TYPE_BATCH_MASK, // per-sequence switch of the mask; not implemented on MI355X
+        MASK_USE_STATUS_TYPE_BATCH_MASK, // input maskUseStatus [batch]: 0 lets a sequence's query tokens see its whole context
         MASK_USE_STATUS_TYPE_MAX
     };
     MaskUseStatusType maskUseStatusType = MASK_USE_STATUS_TYPE_UNDEFINED;
