@@ -197,13 +197,26 @@ __global__ __launch_bounds__(NWAVES *WAVE) __attribute__((amdgpu_waves_per_eu(2,
         reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char *)smem));
     const uint32_t ldsWaveK = ldsBase + wave * (ROWS_PER_WAVE * K_PITCH);
     const uint32_t ldsWaveV = ldsBase + K_TILE + wave * (ROWS_PER_WAVE * V_PITCH);
+    // Tiles are requested in order: a cursor per transfer walks this lane's source row from tile to tile, and only
+    // a tile that reaches past the last key computes (and clamps) its rows anew.
+    const unsigned char *cursor[DMA_PER_TILE];
+#pragma unroll
+    for (int i = 0; i < DMA_PER_TILE; ++i) {
+        const int row = tBegin + wave * ROWS_PER_WAVE + static_cast<int>((srcRows >> (3 * i)) & 7u);
+        cursor[i] = srcBase[i] + static_cast<uint64_t>(it.kRow0 + row) * srcStride[i];
+    }
     // Requests this wave's rows of the tile at key t into tile buffer `buf`: seven transfers, always.
     auto requestTile = [&](int t, int buf) {
         const int row0 = t + wave * ROWS_PER_WAVE;
+        const bool whole = t + STEP <= it.kvLen;
 #pragma unroll
         for (int i = 0; i < DMA_PER_TILE; ++i) {
-            const int row = min(row0 + static_cast<int>((srcRows >> (3 * i)) & 7u), it.kvLen - 1);
-            const unsigned char *src = srcBase[i] + static_cast<uint64_t>(it.kRow0 + row) * srcStride[i];
+            const unsigned char *src = cursor[i];
+            if (!whole) {
+                const int row = min(row0 + static_cast<int>((srcRows >> (3 * i)) & 7u), it.kvLen - 1);
+                src = srcBase[i] + static_cast<uint64_t>(it.kRow0 + row) * srcStride[i];
+            }
+            cursor[i] += STEP * srcStride[i];
             const bool isK = i < K_DMA;
             const int j = isK ? i : i - K_DMA;
             const uint32_t dst = (isK ? ldsWaveK : ldsWaveV) + static_cast<uint32_t>(buf * BUF + j * (WAVE * 16));
@@ -250,6 +263,7 @@ __global__ __launch_bounds__(NWAVES *WAVE) __attribute__((amdgpu_waves_per_eu(2,
     const int kOperand = n * K_PITCH + kh * 16;
     const int vOperand = K_TILE + (4 * kh + (l16 >> 2)) * V_PITCH + (((lane >> 4) & 1) * 16 + (l16 & 3) * 4) * 2;
 
+    constexpr float SLACK = 8.0f;
     auto computeStep = [&](int t, const unsigned char *buf) {
         f32x16 s;
 #pragma unroll
@@ -307,7 +321,10 @@ __global__ __launch_bounds__(NWAVES *WAVE) __attribute__((amdgpu_waves_per_eu(2,
         }
         mLoc = fmaxf(mLoc, s[15]);
         mLoc = fmaxf(mLoc, __shfl_xor(mLoc, 32)) * a.scale2;
-        const float mNew = fmaxf(m, mLoc);
+        // The reference point of the exponents moves only when the step's maximum is more than 2^SLACK above
+        // it: weights may then reach 2^SLACK, which the 16-bit P and the fp32 sums hold with the same relative
+        // precision, and the 64 accumulators are rescaled on a few steps instead of most.
+        const float mNew = mLoc > m + SLACK ? mLoc : m; // (m = -inf: the first visible key sets it)
         const float mRef = mNew == -INFINITY ? 0.0f : mNew; // nothing visible so far: every weight is 0
         const float corr = Exp2(m - mRef);
         m = mNew;
