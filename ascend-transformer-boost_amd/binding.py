@@ -211,6 +211,13 @@ class AtbmiMlaInt8Call(ctypes.Structure):
                     "query", "queryRope", "kvCache", "kRopeCache", "blockTables", "qkDescale", "pvDescale", "mask", "out",
                     "lse")]
 
+class AtbmiMlaMaskFreeCall(ctypes.Structure):
+    """One atbmi_mla_mask_free_expand call (include/atbmi_kernels.h)."""
+    _fields_ = [("batch", ctypes.c_int32), ("numQueryRows", ctypes.c_int32), ("templateBatch", ctypes.c_int32),
+                ("templateRows", ctypes.c_int32), ("maskLen", ctypes.c_int32), ("hostContextLens", ctypes.c_void_p),
+                ("hostQueryLens", ctypes.c_void_p), ("maskTemplate", ctypes.c_void_p), ("outMask", ctypes.c_void_p)]
+
+
 _kernels = None
 _atb = None
 
@@ -249,6 +256,8 @@ def kernels():
         lib.atbmi_pa_plan_update.argtypes = [vp, vp, i32]
         lib.atbmi_pa_plan_update_multi.argtypes = [vp, vp, vp, i32]
         lib.atbmi_pa_plan_update_multi.restype = i32
+        lib.atbmi_mla_mask_free_workspace_size.argtypes = [vp, vp]
+        lib.atbmi_mla_mask_free_expand.argtypes = [vp, vp, u64, vp]
         lib.atbmi_pa_plan_set_causal_rows.argtypes = [vp, i32, vp, i32]
         lib.atbmi_pa_plan_set_causal_rows.restype = i32
         lib.atbmi_pa_plan_workspace_size.argtypes = [vp]

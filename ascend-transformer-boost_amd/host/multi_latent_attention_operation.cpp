@@ -29,10 +29,11 @@
 // sequence whose maskUseStatus entry is 0 keeps the whole context for every row. The
 // same rule applies here (kernel layer: causal rows). With fewer heads the
 // MASK_TYPE_SPEC mask [numTokens, maxS] is added to the scores as given;
-// MASK_TYPE_CAUSAL_MASK (no mask tensor) is causal rows for any head count, and
-// MASK_TYPE_MASK_FREE, whose [125 + 2 q, 128] template the reference's other kernel
-// path indexes by the last two 128-token tiles (op_kernel/mla.cce:3719-3750), is
-// built for the 128-head / int8 path only: with fewer heads Setup refuses it.
+// MASK_TYPE_CAUSAL_MASK (no mask tensor) is causal rows for any head count.
+// MASK_TYPE_MASK_FREE with fewer heads: the [125 + 2 q, 128] template (or one per
+// sequence), which the reference's other kernel path indexes by the last two 128-token
+// tiles (op_kernel/mla.cce:3719-3750), is expanded on the device into one mask row per
+// query token (atbmi_mla_mask_free_expand, in the workspace) and added like a SPEC mask.
 //
 // The kernels are those of PagedAttention's combined-cache variant reading
 // each query and key row from two tensors.
@@ -341,11 +342,7 @@ protected:
         const bool jobPerToken = param_.headNum == JOB_PER_TOKEN_HEADS || (int8 && maxQuery > 1);
         const bool causalRows = IsSpec(param_) && (jobPerToken || param_.maskType == Param::MASK_TYPE_CAUSAL_MASK);
         useMask_ = maskIdx_ != NONE && !jobPerToken && !int8; // (the int8 kernels of the reference never read it)
-        if (useMask_ && param_.maskType == Param::MASK_TYPE_MASK_FREE) {
-            ATB_LOG(ERROR) << "MASK_TYPE_MASK_FREE with fewer than " << JOB_PER_TOKEN_HEADS
-                           << " heads is not implemented on MI355X (use MASK_TYPE_SPEC or MASK_TYPE_CAUSAL_MASK)";
-            return ERROR_INVALID_PARAM;
-        }
+        maskFree_ = useMask_ && param_.maskType == Param::MASK_TYPE_MASK_FREE;
         causalUse_.clear();
         if (causalRows && maskUseIdx_ != NONE && Utils::GetTensorSize(pack.inTensors.at(maskUseIdx_).desc) != 0) {
             const Tensor &use = pack.inTensors.at(maskUseIdx_);
@@ -373,7 +370,33 @@ protected:
             }
         }
         int64_t maskLen = 0;
-        if (useMask_) {
+        uint64_t maskFreeTableBytes = 0;
+        if (maskFree_) {
+            // the template [rows, 128] or [batch, rows, 128] (reference tiling/mla_tiling.cpp:156-166) becomes a
+            // mask of one row per query token in the workspace
+            const Dims &m = pack.inTensors.at(maskIdx_).desc.shape;
+            if ((m.dimNum != 2 && m.dimNum != 3) || m.dims[m.dimNum - 1] != DECODER_BLOCK_SIZE ||
+                (m.dimNum == 3 && m.dims[0] != batch)) {
+                ATB_LOG(ERROR) << "the MASK_FREE mask should be [rows, 128] or [batch, rows, 128]";
+                return ERROR_INVALID_PARAM;
+            }
+            const int32_t *ctx = static_cast<const int32_t *>(lens.hostData);
+            lens_.assign(ctx, ctx + batch);
+            qLens_.assign(queryLens, queryLens + batch);
+            for (int32_t i = 0; i < batch; ++i) {
+                maskLen = std::max<int64_t>(maskLen, ctx[i]);
+            }
+            maskLen = std::max<int64_t>(8, (maskLen + 7) / 8 * 8);
+            maskFreeRows_ = static_cast<int32_t>(m.dims[m.dimNum - 2]);
+            maskFreeBatch_ = m.dimNum == 3 ? batch : 0;
+            maskLen_ = maskLen;
+            AtbmiMlaMaskFreeCall call = MakeMaskFreeCall(pack, nullptr);
+            int rc = atbmi_mla_mask_free_workspace_size(&call, &maskFreeTableBytes);
+            if (rc != 0) {
+                ATB_LOG(ERROR) << "MultiLatentAttention mask-free plan: " << atbmi_last_error();
+                return rc;
+            }
+        } else if (useMask_) {
             // one mask row per query token (reference tests/apitest/opstest/python/operations/
             // multi_latent_attention/test_multi_latent_attention_mtp.py:262-274)
             const Dims &m = pack.inTensors.at(maskIdx_).desc.shape;
@@ -456,6 +479,13 @@ protected:
             return rc;
         }
         workspaceSize = atbmi_pa_plan_workspace_size(plan_);
+        if (maskFree_) {
+            planBytes_ = workspaceSize;
+            maskFreeTableOff_ = (workspaceSize + 255) / 256 * 256;
+            maskFreeTableBytes_ = maskFreeTableBytes;
+            maskFreeMaskOff_ = (maskFreeTableOff_ + maskFreeTableBytes + 255) / 256 * 256;
+            workspaceSize = maskFreeMaskOff_ + static_cast<uint64_t>(q.desc.shape.dims[0]) * static_cast<uint64_t>(maskLen) * 2;
+        }
         return NO_ERROR;
     }
 
@@ -476,14 +506,28 @@ protected:
         t.keyCache = pack.inTensors.at(KV_CACHE).deviceData;
         t.keyRopeCache = pack.inTensors.at(KV_CACHE_ROPE).deviceData;
         t.blockTables = static_cast<const int32_t *>(pack.inTensors.at(BLOCK_TABLES).deviceData);
-        if (useMask_) {
+        uint64_t planBytes = workspaceSize;
+        if (maskFree_) {
+            if (!workspace || workspaceSize < maskFreeMaskOff_) {
+                ATB_LOG(ERROR) << "MultiLatentAttention: the workspace is smaller than Setup asked for";
+                return ERROR_INVALID_PARAM;
+            }
+            AtbmiMlaMaskFreeCall call = MakeMaskFreeCall(pack, workspace + maskFreeMaskOff_);
+            int rc = atbmi_mla_mask_free_expand(&call, workspace + maskFreeTableOff_, maskFreeTableBytes_, stream);
+            if (rc != 0) {
+                ATB_LOG(ERROR) << "MultiLatentAttention mask-free launch failed: " << atbmi_last_error();
+                return rc;
+            }
+            t.mask = workspace + maskFreeMaskOff_;
+            planBytes = planBytes_;
+        } else if (useMask_) {
             t.mask = pack.inTensors.at(maskIdx_).deviceData;
         }
         t.out = pack.outTensors.at(0).deviceData;
         if (IsRing(param_)) {
             t.lse = pack.outTensors.at(1).deviceData;
         }
-        int rc = atbmi_pa_decode(plan_, &t, workspace, workspaceSize, stream);
+        int rc = atbmi_pa_decode(plan_, &t, workspace, planBytes, stream);
         if (rc != 0) {
             ATB_LOG(ERROR) << "MultiLatentAttention launch failed: " << atbmi_last_error();
         }
@@ -521,6 +565,21 @@ private:
         c.mask = nullptr;
         c.out = pack.outTensors.at(0).deviceData;
         c.lse = IsRing(param_) ? static_cast<float *>(pack.outTensors.at(1).deviceData) : nullptr;
+        return c;
+    }
+
+    AtbmiMlaMaskFreeCall MakeMaskFreeCall(const VariantPack &pack, void *outMask) const
+    {
+        AtbmiMlaMaskFreeCall c{};
+        c.batch = static_cast<int32_t>(lens_.size());
+        c.numQueryRows = static_cast<int32_t>(pack.inTensors.at(QUERY).desc.shape.dims[0]);
+        c.templateBatch = maskFreeBatch_;
+        c.templateRows = maskFreeRows_;
+        c.maskLen = static_cast<int32_t>(maskLen_);
+        c.hostContextLens = lens_.data();
+        c.hostQueryLens = qLens_.data();
+        c.maskTemplate = pack.inTensors.at(maskIdx_).deviceData;
+        c.outMask = outMask;
         return c;
     }
 
@@ -647,7 +706,11 @@ private:
     std::vector<int32_t> qLens_;
     std::vector<int32_t> causalUse_; // the maskUseStatus flags of the last Setup (empty: every sequence)
     bool useMask_ = false;           // the mask tensor is added to the scores
+    bool maskFree_ = false;          // ... after its expansion from the MASK_FREE template
     bool causalRows_ = false;
+    int64_t maskLen_ = 0;
+    int32_t maskFreeRows_ = 0, maskFreeBatch_ = 0;
+    uint64_t planBytes_ = 0, maskFreeTableOff_ = 0, maskFreeTableBytes_ = 0, maskFreeMaskOff_ = 0;
     uint32_t inputNum_ = 6;
     AtbmiPaPlan *plan_ = nullptr;
     AtbmiPaShape planShape_{};

@@ -132,7 +132,7 @@ struct MultiLatentAttentionParam {
     enum MaskType : int {
         UNDEFINED = 0,         // no mask input
         MASK_TYPE_SPEC,        // one mask row per query token, with CALC_TYPE_SPEC
-        MASK_TYPE_MASK_FREE,   // compressed causal mask (decode: 128 heads or int8 cache only; prefill)
+        MASK_TYPE_MASK_FREE,   // compressed causal mask: a [125 + 2 q, 128] template (decode), [512, 512] (prefill)
         MASK_TYPE_CAUSAL_MASK, // causal, no mask tensor
         MASK_TYPE_SWA_NORM     // sliding window of windowSize tokens (prefill only)
     };

@@ -485,6 +485,34 @@ int atbmi_mla_int8_workspace_size(const AtbmiMlaInt8Call *call, uint64_t *bytes)
 int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspaceDevice, uint64_t workspaceBytes, void *stream);
 
 /*
+ * MultiLatentAttention with maskType MASK_TYPE_MASK_FREE and several query tokens (decode calcTypes; replaces the
+ * mask handling of the reference's device kernel, src/kernels/mixkernels/multi_latent_attention/op_kernel/
+ * mla.cce:3719-3750 with 2581-2592, and the shape rule of tiling/mla_tiling.cpp:156-166): expands the compressed
+ * mask, a template [templateRows, 128] (templateBatch == 0) or [templateBatch = batch, templateRows, 128] of 16-bit
+ * values, into one mask row per query token, outMask 16-bit [numQueryRows, maskLen], to be handed to the decode
+ * plan as a mask with one row per query row (AtbmiPaShape.maskRowBy = ATBMI_PA_MASK_ROW_QUERY). Sequence b has
+ * hostContextLens[b] tokens and hostQueryLens[b] query rows (none when its context is empty), as in
+ * atbmi_pa_plan_update_multi; both are host arrays read during the call.
+ */
+typedef struct AtbmiMlaMaskFreeCall {
+    int32_t batch;
+    int32_t numQueryRows;
+    int32_t templateBatch; /* 0, or batch */
+    int32_t templateRows;  /* 125 + 2 q in the reference's tests */
+    int32_t maskLen;       /* elements per row of outMask, >= every context length */
+    const int32_t *hostContextLens;
+    const int32_t *hostQueryLens;
+    const void *maskTemplate;
+    void *outMask;
+} AtbmiMlaMaskFreeCall;
+
+/* Validates the call (pointers aside) and reports the device workspace it needs (16 bytes per query row). */
+int atbmi_mla_mask_free_workspace_size(const AtbmiMlaMaskFreeCall *call, uint64_t *bytes);
+/* Uploads the row list into the workspace and launches the expansion on `stream`; does not wait. */
+int atbmi_mla_mask_free_expand(const AtbmiMlaMaskFreeCall *call, void *workspaceDevice, uint64_t workspaceBytes,
+                               void *stream);
+
+/*
  * Kernel timing for benchmarks. atbmi_timing_enable(n) with n > 0 makes every
  * n-th atbmi_pa_decode bracket its attention kernel with HIP events on the
  * launch stream (the events themselves cost a few microseconds of stream

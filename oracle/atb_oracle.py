@@ -75,6 +75,17 @@ the invariants of the mathematics (no function is left "parity unpinned"):
                       the whole context as one tile. Pinned by an independent float64 loop version, by the
                       limit of fine descales (-> ordinary attention over the dequantised tensors), and by
                       closed forms of the quantiser
+  causal_rows (paged_attention, mla_int8_decode)
+                      src/kernels/mixkernels/multi_latent_attention/tiling/mla_tiling.cpp:139-144 and
+                      mla_tiling_dependency.cpp:292-316 (128 heads, or an int8 cache with several query tokens: one
+                      job per query token over kvSeqlen - qSeqLen + its index + 1 tokens, the mask type dropped, a
+                      maskUseStatus of 0 keeping the whole context), test_multi_latent_attention_int8nz.py:356-364
+                      (the golden does the same); pinned against every row run alone on its shortened context,
+                      against the -inf look-ahead mask, and per sequence
+  mla_mask_free_rows  src/kernels/mixkernels/multi_latent_attention/op_kernel/mla.cce:3719-3750 with 2581-2592 (which
+                      rows of the compressed mask the kernel adds to the last two 128-token tiles),
+                      test_multi_latent_attention_mtp.py:342-368 (the template); pinned by the closed form: the
+                      reference's template read this way is "token > k - q + i" for every context length and q
   mla_prefill         tests/apitest/opstest/python/operations/multi_latent_attention/
                       test_multi_latent_attention_prefill.py:519-700 (gen_out_tensor: per sequence and head
                       score = q . k^T * tor over the 128 + 64 channels, + mask, fp32 softmax over the keys,
@@ -649,6 +660,31 @@ def paged_attention_loops(query, key_cache, value_cache, block_tables, context_l
                 out[row][h][c] = acc / z
         row += 1
     return np.array(out, dtype=np.float64)
+
+
+def mla_mask_free_rows(template, context_lens, q_lens, mask_len):
+    """One mask row per query token from MultiLatentAttention's compressed decode mask (MASK_TYPE_MASK_FREE), as
+    the reference's kernel reads it (src/kernels/mixkernels/multi_latent_attention/op_kernel/mla.cce:3719-3750,
+    2581-2592): template [rows, 128] or [batch, rows, 128]; for a sequence of k tokens whose last 128-token tile
+    holds n of them, query token i of q adds template row n - 1 + i to the last tile and, when n < q - 1 and there
+    is a tile before it, row n + 127 + i to that one. Sequences of length 0 take no row. Returns float32
+    [query rows, mask_len]; rows the template lacks read as 0."""
+    template = np.asarray(template, np.float32)
+    rows = []
+    for b, (k, q) in enumerate(zip(np.asarray(context_lens).tolist(), np.asarray(q_lens).tolist())):
+        if k == 0:
+            continue
+        tmpl = template[b] if template.ndim == 3 else template
+        last = (k - 1) // 128
+        n = k - last * 128
+        for i in range(q):
+            row = np.zeros(mask_len, np.float32)
+            if n - 1 + i < tmpl.shape[0]:
+                row[last * 128:k] = tmpl[n - 1 + i, :n]
+            if last >= 1 and n < q - 1 and n + 127 + i < tmpl.shape[0]:
+                row[(last - 1) * 128:last * 128] = tmpl[n + 127 + i, :]
+            rows.append(row)
+    return np.stack(rows) if rows else np.zeros((0, mask_len), np.float32)
 
 
 def quantise_weights(w):

@@ -1549,6 +1549,79 @@ def test_multi_latent_attention_causal_mask_types(binding, oracle, dev, stream):
     c.close()
 
 
+def test_mask_free_template_expansion_and_operation(binding, oracle, dev, stream):
+    """MASK_TYPE_MASK_FREE with fewer than 128 heads: atbmi_mla_mask_free_expand reproduces the oracle's reading of the
+    template bit for bit (the reference's template, a random one, one per sequence; contexts that end early in a
+    128-token tile, so that the triangle reaches into the tile before), and MultiLatentAttentionOperation run on it
+    equals the oracle with those mask rows."""
+    import ctypes
+    k = binding.kernels()
+    rng = _rng(495)
+    ctx = np.array([700, 33, 1500, 128, 129, 258, 0, 5], dtype=np.int32)
+    q_lens = np.array([2, 1, 3, 2, 4, 4, 2, 5], dtype=np.int32)
+    rows = int(sum(n for n, c in zip(q_lens, ctx) if c > 0))
+    mask_len = 1504
+    for dtype in (torch.float16, torch.bfloat16):
+        standard = np.triu(np.full((125 + 2 * 5, 128), -10000.0, np.float32), 2 - 5)
+        random = (rng.standard_normal((135, 128)) * 3).astype(np.float32)
+        per_seq = np.stack([standard if b % 2 == 0 else random for b in range(len(ctx))])
+        for template in (standard, random, per_seq):
+            tmpl = torch.from_numpy(template).to(dtype).to(dev)
+            call = binding.AtbmiMlaMaskFreeCall(
+                batch=len(ctx), numQueryRows=rows, templateBatch=len(ctx) if template.ndim == 3 else 0,
+                templateRows=template.shape[-2], maskLen=mask_len, hostContextLens=ctx.ctypes.data,
+                hostQueryLens=q_lens.ctypes.data)
+            ws_bytes = ctypes.c_uint64(0)
+            assert k.atbmi_mla_mask_free_workspace_size(ctypes.byref(call), ctypes.byref(ws_bytes)) == 0
+            assert ws_bytes.value == rows * 16
+            with torch.cuda.stream(stream):
+                ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=dev)
+                out = torch.full((rows, mask_len), 7.0, dtype=dtype, device=dev)
+                call.maskTemplate, call.outMask = tmpl.data_ptr(), out.data_ptr()
+                rc = k.atbmi_mla_mask_free_expand(ctypes.byref(call), ws.data_ptr(), ws_bytes.value, stream.cuda_stream)
+                assert rc == 0, binding.last_kernel_error()
+            stream.synchronize()
+            want = oracle.mla_mask_free_rows(tmpl.float().cpu().numpy(), ctx, q_lens, mask_len)
+            assert np.array_equal(out.float().cpu().numpy(), want)
+    # a template without the rows a sequence reads is refused
+    call = binding.AtbmiMlaMaskFreeCall(batch=len(ctx), numQueryRows=rows, templateBatch=0, templateRows=100, maskLen=mask_len,
+                                        hostContextLens=ctx.ctypes.data, hostQueryLens=q_lens.ctypes.data)
+    assert k.atbmi_mla_mask_free_workspace_size(ctypes.byref(call), ctypes.byref(ws_bytes)) != 0
+
+    # through the operation: 32 and 16 heads, the reference's template and a template per sequence with one all-zero
+    d, dv, block, dtype = 576, 512, 128, torch.float16
+    ctx, q_lens = ctx[:6].copy(), np.full(6, 4, dtype=np.int32)   # (the reference's template is made for one q)
+    rows = int(q_lens.sum())
+    scale = 1.0 / math.sqrt(192.0)
+    lens, qn = torch.from_numpy(ctx), torch.from_numpy(q_lens)
+    c = binding.Context(stream)
+    standard = np.triu(np.full((125 + 2 * 4, 128), -10000.0, np.float32), 2 - 4)
+    per_seq = np.stack([standard if b != 2 else np.zeros_like(standard) for b in range(6)])
+    for heads, calc, template in ((32, 1, standard), (16, 3, per_seq)):
+        _, kc, _, tables, _ = _pa_inputs(rng, dev, 6, heads, 1, block, d, d, ctx, dtype, std=0.5)
+        q = (torch.rand((rows, heads, d)) * 2 - 1).to(dtype).to(dev)
+        tmpl = torch.from_numpy(template).to(dtype).to(dev)
+        ins = [q[..., :dv].contiguous(), q[..., dv:].contiguous(), kc[..., :dv].contiguous(), kc[..., dv:].contiguous(),
+               tables, lens.to(dev), tmpl, qn.to(dev)]
+        op = binding.OperationRunner("MultiLatentAttentionOperation", binding.MultiLatentAttentionParam(
+            headNum=heads, kvHeadNum=1, qkScale=scale, cacheMode=1, calcType=calc, maskType=2), c)
+        with torch.cuda.stream(stream):
+            outs = op.run(ins, host_inputs={5: lens, 7: qn})
+        stream.synchronize()
+        mask = torch.from_numpy(oracle.mla_mask_free_rows(tmpl.float().cpu().numpy(), ctx, q_lens, int(ctx.max())))
+        want_lse = np.zeros((rows, heads), np.float32)
+        want = oracle_pa(oracle, q, kc, None, tables, ctx, scale, mla_dv=dv, q_lens=q_lens, mask=mask, mask_rows="query",
+                         lse_out=want_lse)
+        assert_close(outs[0], want, TOL[dtype], "mask-free heads %d" % heads)
+        if calc == 3:
+            assert_close(outs[1][..., 0], want_lse, TOL[dtype], "mask-free lse heads %d" % heads)
+        if template.ndim == 2:   # the reference's template is the causal rule
+            causal = oracle_pa(oracle, q, kc, None, tables, ctx, scale, mla_dv=dv, q_lens=q_lens, causal_rows=True)
+            assert_close(outs[0], causal, TOL[dtype], "mask-free equals causal rows, heads %d" % heads)
+        op.close()
+    c.close()
+
+
 def test_two_call_c_wrappers_run_the_operations(binding, oracle, dev, stream):
     """AtbMLAGetWorkspaceSize + AtbMLA and AtbPagedCacheLoadGetWorkspaceSize + AtbPagedCacheLoad on
     aclTensor handles (reference include/atb/atb_acl.h:99-116,251-267): plain decode, the log-sum-exp

@@ -689,11 +689,24 @@ def test_multi_latent_attention_causal_rows_and_mask_use_status(binding, ctx):
     assert op.setup(pack(128, mask=[129, 128], use_shape=[4], qlens_host=np.array([11, 3, 0, 2], np.int32)),
                     outs(128), ctx)[0] == e["ERROR_INVALID_PARAM"]
     op.close()
-    # fewer heads: the reference's other kernel path reads the template; not built here
+    # fewer heads: the template is expanded into the workspace, one row of 304 (300 rounded up to 8) 16-bit values per
+    # query token, after the plan's own bytes and the 16-byte row records
     op = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1,
                                                                calcType=1, maskType=2))
-    assert op.ok and op.setup(pack(32, mask=[129, 128]), outs(32, lse=False), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    plain = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1,
+                                                                  calcType=1, maskType=3))
+    st, ws = op.setup(pack(32, mask=[131, 128]), outs(32, lse=False), ctx)
+    st0, ws0 = plain.setup(pack(32), outs(32, lse=False), ctx)
+    assert (st, st0) == (0, 0) and ws >= ws0 + 6 * 16 + 6 * 304 * 2 and ws <= ws0 + 6 * 16 + 6 * 304 * 2 + 1024
+    assert op.setup(pack(32, mask=[4, 131, 128]), outs(32, lse=False), ctx)[0] == 0           # a template per sequence
+    assert op.setup(pack(32, mask=[3, 131, 128]), outs(32, lse=False), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    assert op.setup(pack(32, mask=[131, 64]), outs(32, lse=False), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    assert op.setup(pack(32, mask=[131]), outs(32, lse=False), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    # the 300-token sequence with 3 query tokens reads template rows up to 44 - 1 + 2; 64 tokens, 2 query tokens: 64
+    assert op.setup(pack(32, mask=[65, 128]), outs(32, lse=False), ctx)[0] == 0
+    assert op.setup(pack(32, mask=[64, 128]), outs(32, lse=False), ctx)[0] == e["ERROR_INVALID_PARAM"]
     op.close()
+    plain.close()
     # CAUSAL_MASK: no mask tensor, any head count
     op = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1,
                                                                calcType=1, maskType=3))

@@ -871,6 +871,28 @@ def test_causal_rows_equal_the_look_ahead_mask_and_growing_contexts(oracle):
     assert np.array_equal(got[2], full[2])                 # (the last row of a sequence loses none)
 
 
+def test_mask_free_template_rows_are_the_look_ahead_triangle(oracle):
+    """The reference's mask-free template (test_multi_latent_attention_mtp.py:342-358: -10000 where column - row >=
+    2 - q, 125 + 2 q rows) read the way the kernel reads it gives query token i of q the mask "token > k - q + i",
+    whatever the context length: last tile only, or reaching back into the tile before it; a template per sequence
+    masks only the sequences whose template does."""
+    for q in (1, 2, 3, 5):
+        template = np.triu(np.full((125 + 2 * q, 128), -10000.0, np.float32), 2 - q)
+        ctx = [k for k in (q, q + 1, 7, 127, 128, 129, 130, 131, 255, 256, 257, 260, 1000) if k >= q]
+        got = oracle.mla_mask_free_rows(template, ctx, [q] * len(ctx), 1024)
+        row = 0
+        for k in ctx:
+            for i in range(q):
+                want = np.where(np.arange(1024) > k - q + i, -10000.0, 0.0).astype(np.float32)
+                want[k:] = 0.0   # (past the context nothing is read)
+                assert np.array_equal(got[row], want), (q, k, i)
+                row += 1
+    per_seq = np.stack([np.triu(np.full((129, 128), -10000.0, np.float32), 0), np.zeros((129, 128), np.float32)])
+    got = oracle.mla_mask_free_rows(per_seq, [130, 130], [2, 2], 256)
+    assert got[0, 129] == -10000.0 and got[1, 129] == 0.0 and not got[2:].any()
+    assert oracle.mla_mask_free_rows(per_seq, [0, 5], [2, 1], 8).shape == (1, 8)   # an empty sequence takes no row
+
+
 # ---------------------------------------------------------------- log-sum-exp output
 def test_lse_closed_forms_and_logsumexp(oracle):
     from scipy.special import logsumexp
