@@ -749,9 +749,17 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     v_log_f32 v85, v83
     s_nop 1
     v_add_f32 v85, v85, v82                // log2 of the sum of 2^score
-    // ---- the row in the query's type: out[h0 + n][32 i + 8 r + 4 kh .. +4); a partial row has the same form
-    v_lshlrev_b32 v91, 10, v89
+    // ---- the rows in the query's type, out[h0 + n][0 .. 512) (a partial row has the same form). A lane holds
+    // four channels at a time (32 i + 8 r + 4 kh ..): stored from there, a row would reach memory in 64 pieces of
+    // 16 bytes. The rows go through LDS instead (the tile buffers are idle now: buffer `wave` holds this wave's
+    // 32 rows at a pitch of 1040 bytes) and leave as whole rows, 1 KiB an instruction.
+    s_barrier                                // every wave has left the tiles
+    s_movk_i32 s46, 1040
+    s_mul_i32 s48, %[wave], TILE
+    s_add_u32 s48, s48, %[lds]               // this wave's staging rows
+    v_mul_u32_u24 v91, s46, v89
     v_lshl_add_u32 v91, v90, 3, v91
+    v_add_u32 v91, s48, v91                  // row n, byte 8 kh
     .irp i,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15
       .irp c,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15
         v_accvgpr_read_b32 v[16*(\i%%2)+\c], a[16*\i+\c]
@@ -771,9 +779,30 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
       .endr
       s_nop 1
       .irp r,0,1,2,3
-        global_store_dwordx2 v91, v[32+8*(\i%%2)+2*\r:33+8*(\i%%2)+2*\r], %[out] offset:(32*\i+8*\r)*2
+        ds_write_b64 v91, v[32+8*(\i%%2)+2*\r:33+8*(\i%%2)+2*\r] offset:(32*\i+8*\r)*2
       .endr
     .endr
+    v_lshlrev_b32 v92, 4, v92                // 16 lane: this lane's piece of every row
+    v_add_u32 v93, s48, v92
+    s_mov_b64 s[50:51], %[out]
+    s_waitcnt lgkmcnt(0)
+    .irp b,0,1,2,3
+      .irp k,0,1,2,3,4,5,6,7
+        ds_read_b128 v[4*\k:4*\k+3], v93 offset:(8*\b+\k)*1040
+      .endr
+      s_waitcnt lgkmcnt(0)
+      .irp k,0,1,2,3
+        global_store_dwordx4 v92, v[4*\k:4*\k+3], s[50:51] offset:1024*\k
+      .endr
+      s_add_u32 s50, s50, 4096
+      s_addc_u32 s51, s51, 0
+      .irp k,4,5,6,7
+        global_store_dwordx4 v92, v[4*\k:4*\k+3], s[50:51] offset:1024*(\k-4)
+      .endr
+      s_add_u32 s50, s50, 4096
+      s_addc_u32 s51, s51, 0
+    .endr
+    s_barrier                                // the next segment's transfers may take the buffers
     s_mov_b64 s[60:61], exec
     s_cmp_eq_u32 %[complete], 0
     s_cbranch_scc1 13f
