@@ -95,6 +95,43 @@ def main():
                                    "algorithmic_bytes": alg}}))
     load.close()
 
+    # ---- the same rows through fractal-NZ caches [blocks, channels / 16, blockSize, 16]: written by
+    # ReshapeAndCache (kvCacheCfg 2) from contiguous rows, gathered back by PagedCacheLoad (kvCacheCfg 0)
+    chans = g * d
+    nz_caches = [torch.zeros((pool, chans // 16, bs, 16), dtype=torch.bfloat16, device=dev) for _ in range(2)]
+    nz_desc = [b.make_tensor(b._torch_acl_dtype(t), list(t.shape), device_ptr=t.data_ptr(), fmt="fractal_nz")
+               for t in nz_caches]
+    slots = np.concatenate([lay["tables"][i][np.arange(n) // bs].astype(np.int64) * bs + np.arange(n) % bs
+                            for i, n in enumerate(lens)]).astype(np.int32)
+    slots_d = torch.from_numpy(slots).to(dev)
+    rows_k = torch.randn((total, g, d), device=dev).to(torch.bfloat16)
+    rows_v = torch.randn((total, g, d), device=dev).to(torch.bfloat16)
+    write = b.OperationRunner("ReshapeAndCacheOperation", b.ReshapeAndCacheParam(kvCacheCfg=2), ctx)
+    ms = timed(lambda: write.run([rows_k, rows_v, nz_desc[0], nz_desc[1], slots_d], outputs=nz_desc), stream, args.steps,
+               args.warmup)
+    print(json.dumps({"operation": "ReshapeAndCacheOperation (fractal-NZ caches)", "workload": "C2 as a prefill: %d rows "
+                      "of %d B scattered into each cache in 32-byte pieces" % (total, chans * 2), "ms_per_call": ms,
+                      "roofline": {"bound": "hbm", "achieved": alg / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
+                                   "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                                   "algorithmic_bytes": alg}}))
+    write.close()
+    key2 = torch.empty((total, chans), dtype=torch.bfloat16, device=dev)
+    value2 = torch.empty_like(key2)
+    load = b.OperationRunner("PagedCacheLoadOperation", b.PagedCacheLoadParam(), ctx)
+    ms = timed(lambda: load.run([nz_desc[0], nz_desc[1], tables_d, lens_d, key2, value2], outputs=[key2, value2]), stream,
+               args.steps, args.warmup)
+    stream.synchronize()
+    if not (torch.equal(key2.view(total, g, d), rows_k) and torch.equal(value2.view(total, g, d), rows_v)):
+        sys.exit("bench_cache_ops.py: rows written to the fractal-NZ caches did not come back")
+    print(json.dumps({"operation": "PagedCacheLoadOperation (fractal-NZ caches)", "workload": "C2: %d rows of %d B "
+                      "gathered from each cache (32-byte pieces) into contiguous key / value" % (total, chans * 2),
+                      "ms_per_call": ms,
+                      "roofline": {"bound": "hbm", "achieved": alg / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
+                                   "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                                   "algorithmic_bytes": alg}}))
+    load.close()
+    del nz_caches, rows_k, rows_v, key2, value2
+
     # ---- NormRopeReshape: 65 536 tokens of 512 + 64 channels into a cache of 512-token blocks
     tokens, n, r, block = 65536, 512, 64, 512
     blocks = (tokens + 100 + block - 1) // block

@@ -239,6 +239,7 @@ def kernels():
         lib.atbmi_last_error.argtypes = []
         lib.atbmi_device_count.restype = ctypes.c_int
         lib.atbmi_reshape_and_cache.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]
+        lib.atbmi_reshape_and_cache_nz.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, i32, vp]
         lib.atbmi_reshape_and_cache_strided.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp, i64, vp,
                                                         i64, vp]
         lib.atbmi_reshape_and_cache_compress.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]
@@ -252,6 +253,8 @@ def kernels():
         lib.atbmi_block_copy.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp]
         lib.atbmi_paged_cache_load.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64,
                                                i32, vp]
+        lib.atbmi_paged_cache_load_nz.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64,
+                                                  vp]
         lib.atbmi_pa_plan_create.argtypes = [ctypes.POINTER(AtbmiPaShape), ctypes.POINTER(vp)]
         lib.atbmi_pa_plan_update.argtypes = [vp, vp, i32]
         lib.atbmi_pa_plan_update_multi.argtypes = [vp, vp, vp, i32]
@@ -490,8 +493,8 @@ class OperationRunner:
     def run(self, inputs, outputs=None, host_inputs=None):
         """inputs: torch GPU tensors (or ready-made AtbCTensor descriptions, for a view whose shape
         is not the tensor's own); host_inputs: {index: CPU tensor} bound as
-        hostData; outputs: caller-owned output tensors (in-place cache update)
-        or None to allocate from InferShape. Returns the output tensors."""
+        hostData; outputs: caller-owned output tensors (in-place cache update; torch tensors or
+        ready-made AtbCTensor descriptions) or None to allocate from InferShape. Returns the output tensors."""
         import torch
         host_inputs = host_inputs or {}
         ins = [t if isinstance(t, AtbCTensor) else tensor_of(t, host_inputs.get(i)) for i, t in enumerate(inputs)]
@@ -502,7 +505,7 @@ class OperationRunner:
             rev = {ACL_FLOAT16: torch.float16, ACL_BF16: torch.bfloat16, ACL_INT8: torch.int8, ACL_FLOAT: torch.float32}
             outputs = [torch.empty([d.dims[i] for i in range(d.dimNum)], dtype=rev[d.dtype], device=inputs[0].device)
                        for d in descs]
-        outs = [tensor_of(t) for t in outputs]
+        outs = [t if isinstance(t, AtbCTensor) else tensor_of(t) for t in outputs]
         st, ws = self.op.setup(ins, outs, self.context)
         if st != 0:
             raise RuntimeError("Setup failed: %s" % ERROR_NAMES[st])

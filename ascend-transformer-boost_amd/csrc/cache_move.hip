@@ -95,12 +95,28 @@ __global__ __launch_bounds__(MOVE_THREADS) void BlockCopyKernel(uint8_t *__restr
 // leaves the output row as it is.
 constexpr int LOAD_TOKENS = 8;
 
-template <typename VecT>
+// Where vector `col` of cache row `r` (= block * blockSize + offset) sits, in vectors from the cache's base.
+// Token-major caches: rows follow each other. Fractal-NZ caches [blocks, pieces, blockSize, piece]: the row is cut
+// into pieces of perPiece vectors, and a block holds piece 0 of all its rows, then piece 1, ...
+template <bool NZ>
+__device__ __forceinline__ int64_t CacheVector(int64_t r, int col, int perRow, int perPiece, int blockSize)
+{
+    if (!NZ) {
+        return r * perRow + col;
+    }
+    const int64_t blk = r / blockSize;
+    const int64_t off = r - blk * blockSize;
+    const int piece = col / perPiece;
+    return ((blk * (perRow / perPiece) + piece) * blockSize + off) * perPiece + (col - piece * perPiece);
+}
+
+template <typename VecT, bool NZ>
 __global__ __launch_bounds__(MOVE_THREADS) void PagedCacheLoadKernel(
     const uint8_t *__restrict__ keyCache, const uint8_t *__restrict__ valueCache,
     const int32_t *__restrict__ tables, const int32_t *__restrict__ lens, const int32_t *__restrict__ seqStarts,
     uint8_t *__restrict__ key, uint8_t *__restrict__ value, int32_t maxBlocksPerSeq, int32_t blockSize,
-    int64_t numBlocks, int64_t kRowBytes, int64_t vRowBytes, int64_t outRows, int32_t cumsumMode)
+    int64_t numBlocks, int64_t kRowBytes, int64_t vRowBytes, int64_t outRows, int32_t cumsumMode,
+    int32_t kPieceBytes, int32_t vPieceBytes)
 {
     const int b = blockIdx.y;
     const int t0 = blockIdx.x * LOAD_TOKENS;
@@ -158,6 +174,7 @@ __global__ __launch_bounds__(MOVE_THREADS) void PagedCacheLoadKernel(
     const uint8_t *cache = isValue ? valueCache : keyCache;
     uint8_t *out = isValue ? value : key;
     const int perRow = static_cast<int>(rowBytes / static_cast<int64_t>(sizeof(VecT)));
+    const int perPiece = NZ ? (isValue ? vPieceBytes : kPieceBytes) / static_cast<int>(sizeof(VecT)) : perRow;
     const VecT *from = reinterpret_cast<const VecT *>(cache);
     VecT *to = reinterpret_cast<VecT *>(out + (firstRow + t0) * rowBytes);
     // A thread keeps its column and walks down the rows: the division that finds (row, column) is done once,
@@ -181,7 +198,7 @@ __global__ __launch_bounds__(MOVE_THREADS) void PagedCacheLoadKernel(
                     const int64_t r = srcRow[tok];
                     if (r >= 0) {
                         live[k] = true;
-                        v[k] = from[r * perRow + col];
+                        v[k] = from[CacheVector<NZ>(r, col, perRow, perPiece, blockSize)];
                     }
                 }
             }
@@ -199,7 +216,6 @@ __global__ __launch_bounds__(MOVE_THREADS) void PagedCacheLoadKernel(
         if (r < 0) {
             continue;
         }
-        const VecT *src = from + r * perRow;
         VecT *dst = to + static_cast<int64_t>(tok) * perRow;
         for (int c0 = threadIdx.x; c0 < perRow; c0 += MOVE_THREADS * BATCH) {
             VecT v[BATCH];
@@ -207,7 +223,7 @@ __global__ __launch_bounds__(MOVE_THREADS) void PagedCacheLoadKernel(
             for (int k = 0; k < BATCH; ++k) {
                 const int c = c0 + k * MOVE_THREADS;
                 if (c < perRow) {
-                    v[k] = src[c];
+                    v[k] = from[CacheVector<NZ>(r, c, perRow, perPiece, blockSize)];
                 }
             }
 #pragma unroll
@@ -284,18 +300,26 @@ extern "C" int atbmi_block_copy(void *keyCache, void *valueCache, const int32_t 
     return OK;
 }
 
-extern "C" int atbmi_paged_cache_load(const void *keyCache, const void *valueCache, const int32_t *blockTables,
-                                      const int32_t *seqLens, const int32_t *seqStarts, void *key, void *value,
-                                      int64_t batch, int64_t maxBlocksPerSeq, int64_t blockSize, int64_t numBlocks,
-                                      int64_t keyRowBytes, int64_t valueRowBytes, int64_t outRows,
-                                      int64_t maxSeqLen, int32_t cumsumMode, void *stream)
+// Shared by the token-major and the fractal-NZ entry points: piece sizes of 0 mean token-major caches.
+static int LaunchPagedCacheLoad(const char *who, const void *keyCache, const void *valueCache,
+                                const int32_t *blockTables, const int32_t *seqLens, const int32_t *seqStarts,
+                                void *key, void *value, int64_t batch, int64_t maxBlocksPerSeq, int64_t blockSize,
+                                int64_t numBlocks, int64_t keyRowBytes, int64_t valueRowBytes, int64_t keyPieceBytes,
+                                int64_t valuePieceBytes, int64_t outRows, int64_t maxSeqLen, int32_t cumsumMode,
+                                void *stream)
 {
     if (!keyCache || !valueCache || !blockTables || !seqLens || !key || !value) {
-        return Fail(ERR_INVALID_PARAM, "paged_cache_load: caches, blockTables, seqLens, key and value must be non-null");
+        return Fail(ERR_INVALID_PARAM, "%s: caches, blockTables, seqLens, key and value must be non-null", who);
     }
     if (batch < 0 || maxBlocksPerSeq <= 0 || blockSize <= 0 || numBlocks <= 0 || keyRowBytes <= 0 ||
         valueRowBytes <= 0 || outRows < 0 || maxSeqLen < 0) {
-        return Fail(ERR_INVALID_PARAM, "paged_cache_load: bad extents");
+        return Fail(ERR_INVALID_PARAM, "%s: bad extents", who);
+    }
+    const bool nz = keyPieceBytes > 0;
+    if (nz && (valuePieceBytes <= 0 || keyRowBytes % keyPieceBytes != 0 || valueRowBytes % valuePieceBytes != 0)) {
+        return Fail(ERR_INVALID_PARAM, "%s: rows of %lld / %lld bytes are not whole pieces of %lld / %lld bytes", who,
+                    (long long)keyRowBytes, (long long)valueRowBytes, (long long)keyPieceBytes,
+                    (long long)valuePieceBytes);
     }
     if (batch == 0 || outRows == 0 || maxSeqLen == 0) {
         return OK;
@@ -303,21 +327,29 @@ extern "C" int atbmi_paged_cache_load(const void *keyCache, const void *valueCac
     const int64_t groups = (maxSeqLen + LOAD_TOKENS - 1) / LOAD_TOKENS;
     if (batch > 65535 || groups > 0x7fffffffLL || maxBlocksPerSeq > 0x7fffffffLL || blockSize > 0x7fffffffLL ||
         keyRowBytes > (1 << 24) || valueRowBytes > (1 << 24)) {
-        return Fail(ERR_INVALID_PARAM, "paged_cache_load: %lld sequences of up to %lld tokens are more than one "
-                                       "launch takes", (long long)batch, (long long)maxSeqLen);
+        return Fail(ERR_INVALID_PARAM, "%s: %lld sequences of up to %lld tokens are more than one launch takes", who,
+                    (long long)batch, (long long)maxSeqLen);
     }
-    const uintptr_t align = CommonAlign(keyRowBytes, valueRowBytes, keyCache, valueCache, key, value);
+    // a vector never straddles two pieces
+    const uintptr_t align = nz ? CommonAlign(keyPieceBytes, valuePieceBytes, keyCache, valueCache, key, value)
+                               : CommonAlign(keyRowBytes, valueRowBytes, keyCache, valueCache, key, value);
     dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(batch), 2);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const uint8_t *kc8 = static_cast<const uint8_t *>(keyCache);
     const uint8_t *vc8 = static_cast<const uint8_t *>(valueCache);
     uint8_t *k8 = static_cast<uint8_t *>(key);
     uint8_t *v8 = static_cast<uint8_t *>(value);
-#define ATBMI_LAUNCH_CACHE_LOAD(T)                                                                             \
-    PagedCacheLoadKernel<T><<<grid, MOVE_THREADS, 0, s>>>(kc8, vc8, blockTables, seqLens, seqStarts, k8, v8,   \
-                                                          static_cast<int32_t>(maxBlocksPerSeq),               \
-                                                          static_cast<int32_t>(blockSize), numBlocks, keyRowBytes, \
-                                                          valueRowBytes, outRows, cumsumMode)
+#define ATBMI_LAUNCH_CACHE_LOAD_AS(T, NZ)                                                                         \
+    PagedCacheLoadKernel<T, NZ><<<grid, MOVE_THREADS, 0, s>>>(                                                    \
+        kc8, vc8, blockTables, seqLens, seqStarts, k8, v8, static_cast<int32_t>(maxBlocksPerSeq),                 \
+        static_cast<int32_t>(blockSize), numBlocks, keyRowBytes, valueRowBytes, outRows, cumsumMode,              \
+        static_cast<int32_t>(keyPieceBytes), static_cast<int32_t>(valuePieceBytes))
+#define ATBMI_LAUNCH_CACHE_LOAD(T)              \
+    if (nz) {                                   \
+        ATBMI_LAUNCH_CACHE_LOAD_AS(T, true);    \
+    } else {                                    \
+        ATBMI_LAUNCH_CACHE_LOAD_AS(T, false);   \
+    }
     switch (align) {
         case 16: ATBMI_LAUNCH_CACHE_LOAD(Vec16); break;
         case 8: ATBMI_LAUNCH_CACHE_LOAD(Vec8); break;
@@ -326,8 +358,34 @@ extern "C" int atbmi_paged_cache_load(const void *keyCache, const void *valueCac
         default: ATBMI_LAUNCH_CACHE_LOAD(uint8_t); break;
     }
 #undef ATBMI_LAUNCH_CACHE_LOAD
+#undef ATBMI_LAUNCH_CACHE_LOAD_AS
     ATBMI_HIP_CHECK(hipGetLastError());
     return OK;
+}
+
+extern "C" int atbmi_paged_cache_load(const void *keyCache, const void *valueCache, const int32_t *blockTables,
+                                      const int32_t *seqLens, const int32_t *seqStarts, void *key, void *value,
+                                      int64_t batch, int64_t maxBlocksPerSeq, int64_t blockSize, int64_t numBlocks,
+                                      int64_t keyRowBytes, int64_t valueRowBytes, int64_t outRows,
+                                      int64_t maxSeqLen, int32_t cumsumMode, void *stream)
+{
+    return LaunchPagedCacheLoad("paged_cache_load", keyCache, valueCache, blockTables, seqLens, seqStarts, key, value,
+                                batch, maxBlocksPerSeq, blockSize, numBlocks, keyRowBytes, valueRowBytes, 0, 0, outRows,
+                                maxSeqLen, cumsumMode, stream);
+}
+
+extern "C" int atbmi_paged_cache_load_nz(const void *keyCache, const void *valueCache, const int32_t *blockTables,
+                                         const int32_t *seqLens, void *key, void *value, int64_t batch,
+                                         int64_t maxBlocksPerSeq, int64_t blockSize, int64_t numBlocks,
+                                         int64_t keyRowBytes, int64_t valueRowBytes, int64_t keyPieceBytes,
+                                         int64_t valuePieceBytes, int64_t outRows, int64_t maxSeqLen, void *stream)
+{
+    if (keyPieceBytes <= 0 || valuePieceBytes <= 0) {
+        return Fail(ERR_INVALID_PARAM, "paged_cache_load_nz: piece sizes must be positive");
+    }
+    return LaunchPagedCacheLoad("paged_cache_load_nz", keyCache, valueCache, blockTables, seqLens, nullptr, key, value,
+                                batch, maxBlocksPerSeq, blockSize, numBlocks, keyRowBytes, valueRowBytes, keyPieceBytes,
+                                valuePieceBytes, outRows, maxSeqLen, 0, stream);
 }
 
 } // namespace atbmi

@@ -39,6 +39,71 @@ __global__ __launch_bounds__(COPY_THREADS) void ReshapeAndCacheKernel(const uint
     }
 }
 
+// Fractal-NZ caches: a cache row of C elements is cut into pieces of `lastDim` elements and a block of blockSize
+// slots is stored piece-major, [numBlocks, C / lastDim, blockSize, lastDim]. grid.x = group of NZ_TOKENS tokens,
+// grid.y = 0 (key) / 1 (value). Neighbouring lanes take the same piece of neighbouring tokens: tokens of a
+// prompt sit in consecutive slots, so a piece of the group lands in one contiguous run of the cache
+// (NZ_TOKENS * pieceBytes), and the lanes that share a token read consecutive pieces of its row.
+constexpr int NZ_TOKENS = 8;
+typedef uint32_t NzVec16 __attribute__((ext_vector_type(4))); // (plain vector types: the non-temporal store takes no structs)
+typedef uint32_t NzVec8 __attribute__((ext_vector_type(2)));
+
+struct NzRows {
+    const uint8_t *src;
+    uint8_t *cache;
+    int64_t rowBytes;   // bytes of one token's row
+    int64_t pieceBytes; // lastDim * element size: 16 or 32
+};
+
+template <typename VecT>
+__global__ __launch_bounds__(COPY_THREADS) void ReshapeAndCacheNzKernel(NzRows k, NzRows v,
+                                                                        const int32_t *__restrict__ slots,
+                                                                        int64_t numTokens, int64_t blockSize,
+                                                                        int64_t numSlots)
+{
+    const NzRows &r = blockIdx.y == 1 ? v : k;
+    const int perPiece = static_cast<int>(r.pieceBytes / static_cast<int64_t>(sizeof(VecT)));
+    const int lanesPerPiece = perPiece * NZ_TOKENS; // divides COPY_THREADS for every VecT and piece size
+    const int sub = threadIdx.x % lanesPerPiece;
+    const int tok = sub / perPiece;
+    const int within = sub - tok * perPiece;
+    const int64_t token = static_cast<int64_t>(blockIdx.x) * NZ_TOKENS + tok;
+    if (token >= numTokens) {
+        return;
+    }
+    const int64_t slot = slots[token];
+    if (slot < 0 || slot >= numSlots) {
+        return;
+    }
+    const int64_t block = slot / blockSize;
+    const int64_t offset = slot - block * blockSize;
+    const VecT *src = reinterpret_cast<const VecT *>(r.src + token * r.rowBytes) + within;
+    uint8_t *dst = r.cache + block * blockSize * r.rowBytes + offset * r.pieceBytes +
+                   within * static_cast<int64_t>(sizeof(VecT));
+    const int pieces = static_cast<int>(r.rowBytes / r.pieceBytes);
+    const int step = COPY_THREADS / lanesPerPiece;
+    const int64_t pieceStride = blockSize * r.pieceBytes;
+    // all loads of a batch before its stores (the compiler cannot reorder them itself: the caches may alias the rows)
+    constexpr int BATCH = 4;
+    for (int p0 = threadIdx.x / lanesPerPiece; p0 < pieces; p0 += step * BATCH) {
+        VecT held[BATCH];
+#pragma unroll
+        for (int i = 0; i < BATCH; ++i) {
+            const int p = p0 + i * step;
+            if (p < pieces) {
+                held[i] = src[p * perPiece];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < BATCH; ++i) {
+            const int p = p0 + i * step;
+            if (p < pieces) {
+                __builtin_nontemporal_store(held[i], reinterpret_cast<VecT *>(dst + p * pieceStride));
+            }
+        }
+    }
+}
+
 // A key or value input that is a strided view: element (token, head, channel) sits
 // `offset + token * tokenStride + head * headStride + channel * chanStride` bytes from the base.
 struct StridedRows {
@@ -493,6 +558,65 @@ extern "C" int atbmi_reshape_and_cache(const void *key, const void *value, void 
             ReshapeAndCacheKernel<uint8_t><<<grid, COPY_THREADS, 0, s>>>(k8, v8, kc8, vc8, slotMapping, kRowBytes,
                                                                           vRowBytes, numSlots);
             break;
+    }
+    ATBMI_HIP_CHECK(hipGetLastError());
+    return OK;
+}
+
+template <typename VecT>
+static void LaunchNz(const NzRows &k, const NzRows &v, const int32_t *slots, int64_t numTokens, int64_t blockSize,
+                     int64_t numSlots, hipStream_t s)
+{
+    dim3 grid(static_cast<unsigned>((numTokens + NZ_TOKENS - 1) / NZ_TOKENS), 2);
+    ReshapeAndCacheNzKernel<VecT><<<grid, COPY_THREADS, 0, s>>>(k, v, slots, numTokens, blockSize, numSlots);
+}
+
+extern "C" int atbmi_reshape_and_cache_nz(const void *key, const void *value, void *keyCache, void *valueCache,
+                                          const int32_t *slotMapping, int64_t numTokens, int64_t keyRowElems,
+                                          int64_t valueRowElems, int64_t blockSize, int64_t numBlocks,
+                                          int32_t keyElemBytes, int32_t valueElemBytes, void *stream)
+{
+    if (!key || !value || !keyCache || !valueCache || !slotMapping) {
+        return Fail(ERR_INVALID_PARAM, "reshape_and_cache_nz: key, value, the caches and slotMapping must be non-null");
+    }
+    if ((keyElemBytes != 1 && keyElemBytes != 2) || (valueElemBytes != 1 && valueElemBytes != 2)) {
+        return Fail(ERR_INVALID_PARAM, "reshape_and_cache_nz: element sizes must be 1 or 2, got %d and %d", keyElemBytes,
+                    valueElemBytes);
+    }
+    // a piece is 32 int8 or 16 two-byte elements of a key row, 16 elements of a value row
+    const int64_t keyLast = keyElemBytes == 1 ? 32 : 16;
+    const int64_t valueLast = 16;
+    if (numTokens < 0 || keyRowElems <= 0 || valueRowElems <= 0 || blockSize <= 0 || numBlocks <= 0 ||
+        keyRowElems % keyLast != 0 || valueRowElems % valueLast != 0) {
+        return Fail(ERR_INVALID_PARAM,
+                    "reshape_and_cache_nz: bad extents (key row %lld must be a multiple of %lld, value row %lld of 16)",
+                    static_cast<long long>(keyRowElems), static_cast<long long>(keyLast),
+                    static_cast<long long>(valueRowElems));
+    }
+    if (numTokens == 0) {
+        return OK;
+    }
+    if (numTokens > 0x7fffffffLL) {
+        return Fail(ERR_INVALID_PARAM, "reshape_and_cache_nz: too many tokens");
+    }
+    const NzRows k{static_cast<const uint8_t *>(key), static_cast<uint8_t *>(keyCache), keyRowElems * keyElemBytes,
+                   keyLast * keyElemBytes};
+    const NzRows v{static_cast<const uint8_t *>(value), static_cast<uint8_t *>(valueCache),
+                   valueRowElems * valueElemBytes, valueLast * valueElemBytes};
+    // pieces are 32 or 16 bytes, so the widest access is set by the base addresses
+    uintptr_t align = 16;
+    while (align > 1 && !(k.pieceBytes % align == 0 && v.pieceBytes % align == 0 && Aligned(key, align) &&
+                          Aligned(value, align) && Aligned(keyCache, align) && Aligned(valueCache, align))) {
+        align >>= 1;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t numSlots = numBlocks * blockSize;
+    switch (align) {
+        case 16: LaunchNz<NzVec16>(k, v, slotMapping, numTokens, blockSize, numSlots, s); break;
+        case 8: LaunchNz<NzVec8>(k, v, slotMapping, numTokens, blockSize, numSlots, s); break;
+        case 4: LaunchNz<uint32_t>(k, v, slotMapping, numTokens, blockSize, numSlots, s); break;
+        case 2: LaunchNz<uint16_t>(k, v, slotMapping, numTokens, blockSize, numSlots, s); break;
+        default: LaunchNz<uint8_t>(k, v, slotMapping, numTokens, blockSize, numSlots, s); break;
     }
     ATBMI_HIP_CHECK(hipGetLastError());
     return OK;

@@ -6,8 +6,9 @@
 //
 // Supported: K_CACHE_V_CACHE (key + value caches), also with head compression
 // (COMPRESS_TYPE_KVHEAD: + wins, seqLens; COMPRESS_TYPE_KVHEAD_ROPE: + wins,
-// seqLens, offsetIndex), and K_CACHE_V_BYPASS (key cache only). Fractal-NZ
-// caches are an Ascend cube-unit layout and rejected at creation.
+// seqLens, offsetIndex), K_CACHE_V_BYPASS (key cache only) and K_CACHE_V_CACHE_NZ
+// (fractal-NZ caches, the layout MultiLatentAttention's NZCACHE / INT8_NZCACHE
+// modes read; reference :321-377 KVCacheDimCheck910BNZ).
 #include <new>
 #include "atb/infer_op_params.h"
 #include "atb/utils.h"
@@ -43,6 +44,24 @@ OpIr MakeIr(bool siso, int extra = 0)
     return ir;
 }
 
+// Fractal-NZ caches (reference ops_configs/atb_ops_info.ini:829-850): int8 or 16-bit key rows with 16-bit value
+// rows of either type.
+OpIr MakeNzIr()
+{
+    OpIr ir;
+    const aclDataType pairs[6][2] = {{ACL_INT8, ACL_FLOAT16}, {ACL_INT8, ACL_BF16},  {ACL_FLOAT16, ACL_FLOAT16},
+                                     {ACL_BF16, ACL_BF16},    {ACL_FLOAT16, ACL_BF16}, {ACL_BF16, ACL_FLOAT16}};
+    for (const auto &p : pairs) {
+        IrCombo c;
+        c.inDtypes = {p[0], p[1], p[0], p[1], ACL_INT32};
+        c.outDtypes = {p[0], p[1]};
+        c.inFormats = {ACL_FORMAT_ND, ACL_FORMAT_ND, ACL_FORMAT_FRACTAL_NZ, ACL_FORMAT_FRACTAL_NZ, ACL_FORMAT_ND};
+        c.outFormats = {ACL_FORMAT_FRACTAL_NZ, ACL_FORMAT_FRACTAL_NZ};
+        ir.push_back(c);
+    }
+    return ir;
+}
+
 bool SameDesc(const TensorDesc &a, const TensorDesc &b)
 {
     if (a.dtype != b.dtype || a.format != b.format || a.shape.dimNum != b.shape.dimNum) {
@@ -60,6 +79,7 @@ class ReshapeAndCacheOperation : public OperationBase {
 public:
     explicit ReshapeAndCacheOperation(const Param &param)
         : OperationBase("ReshapeAndCacheOperation"), param_(param), siso_(param.kvCacheCfg == Param::K_CACHE_V_BYPASS),
+          nz_(param.kvCacheCfg == Param::K_CACHE_V_CACHE_NZ),
           extra_(param.compressType == Param::COMPRESS_TYPE_KVHEAD ? 2
                  : param.compressType == Param::COMPRESS_TYPE_KVHEAD_ROPE ? 3 : 0)
     {
@@ -67,7 +87,8 @@ public:
         static const OpIr single = MakeIr(true);
         static const OpIr keepLast = MakeIr(false, 2);
         static const OpIr meanWindow = MakeIr(false, 3);
-        ir_ = siso_ ? &single : extra_ == 2 ? &keepLast : extra_ == 3 ? &meanWindow : &normal;
+        static const OpIr fractal = MakeNzIr();
+        ir_ = nz_ ? &fractal : siso_ ? &single : extra_ == 2 ? &keepLast : extra_ == 3 ? &meanWindow : &normal;
     }
 
     // reference :124-136: + wins, seqLens (+ offsetIndex) under head compression
@@ -88,7 +109,7 @@ protected:
 
     Status InferShapeCheckImpl(const SVector<TensorDesc> &in) const override
     {
-        return siso_ ? DimCheckSiso(in) : DimCheck(in);
+        return siso_ ? DimCheckSiso(in) : nz_ ? DimCheckNz(in) : DimCheck(in);
     }
 
     Status SetupCheckImpl(const SVector<Tensor> &inTensors, const SVector<Tensor> &outTensors) const override
@@ -155,7 +176,7 @@ protected:
         const int64_t tokens = key.desc.shape.dims[0];
         const int64_t heads = key.desc.shape.dims[1];
         const int64_t dk = key.desc.shape.dims[2];
-        const int64_t numSlots = keyCacheIn.desc.shape.dims[0] * keyCacheIn.desc.shape.dims[1];
+        const int64_t numSlots = keyCacheIn.desc.shape.dims[0] * keyCacheIn.desc.shape.dims[nz_ ? 2 : 1];
         const int32_t elemBytes = key.desc.dtype == ACL_INT8 ? 1 : 2;
         const void *value = nullptr;
         void *valueCache = nullptr;
@@ -172,6 +193,18 @@ protected:
         if (!key.deviceData || !keyCacheOut.deviceData || !slots.deviceData) {
             ATB_LOG(ERROR) << "ReshapeAndCache: key / keyCache / slotMapping device pointer is null";
             return ERROR_INVALID_PARAM;
+        }
+        if (nz_) {
+            const Tensor &valueIn = pack.inTensors.at(1);
+            int rc = atbmi_reshape_and_cache_nz(key.deviceData, value, keyCacheOut.deviceData, valueCache,
+                                                static_cast<const int32_t *>(slots.deviceData), tokens, heads * dk,
+                                                valueIn.desc.shape.dims[1] * dv, keyCacheIn.desc.shape.dims[2],
+                                                keyCacheIn.desc.shape.dims[0], elemBytes,
+                                                valueIn.desc.dtype == ACL_INT8 ? 1 : 2, stream);
+            if (rc != 0) {
+                ATB_LOG(ERROR) << "ReshapeAndCache launch failed: " << atbmi_last_error();
+            }
+            return rc;
         }
         if (extra_ > 0) {
             const int32_t dtype = key.desc.dtype == ACL_INT8 ? ATBMI_INT8 : key.desc.dtype == ACL_BF16 ? ATBMI_BF16 : ATBMI_F16;
@@ -257,8 +290,52 @@ private:
         return NO_ERROR;
     }
 
+    // Reference reshape_and_cache_operation.cpp:321-377 (KVCacheDimCheck910BNZ): caches
+    // [numBlocks, heads * headSize / lastDim, blockSize, lastDim], lastDim 32 for an int8 key cache, else 16.
+    Status DimCheckNz(const SVector<TensorDesc> &in) const
+    {
+        if (in.at(0).shape.dimNum != 3 || in.at(1).shape.dimNum != 3 || in.at(2).shape.dimNum != 4 ||
+            in.at(3).shape.dimNum != 4 || in.at(4).shape.dimNum != 1) {
+            ATB_LOG(ERROR) << "ReshapeAndCache: expected dims 3/3/4/4/1";
+            return ERROR_INVALID_TENSOR_DIM_NUM;
+        }
+        const Dims &k = in.at(0).shape;
+        const Dims &v = in.at(1).shape;
+        const Dims &kc = in.at(2).shape;
+        const Dims &vc = in.at(3).shape;
+        if (k.dims[0] != v.dims[0] || k.dims[1] != v.dims[1]) {
+            ATB_LOG(ERROR) << "ReshapeAndCache: key and value must agree on tokens and heads";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (kc.dims[2] != vc.dims[2]) {
+            ATB_LOG(ERROR) << "ReshapeAndCache: blockSizes should be same";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (kc.dims[2] % 16 != 0) {
+            ATB_LOG(ERROR) << "ReshapeAndCache: the blockSize of keyCache and valueCache should be 16-aligned";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        const int64_t keyLast = in.at(0).dtype == ACL_INT8 ? 32 : 16;
+        if (k.dims[1] * k.dims[2] != kc.dims[1] * keyLast || kc.dims[3] != keyLast) {
+            ATB_LOG(ERROR) << "ReshapeAndCache: NZ keyCache should be [blocks, heads * headSize / " << keyLast
+                           << ", blockSize, " << keyLast << "]";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        if (v.dims[1] * v.dims[2] != vc.dims[1] * 16 || vc.dims[3] != 16) {
+            ATB_LOG(ERROR) << "ReshapeAndCache: NZ valueCache should be [blocks, heads * headSize / 16, blockSize, 16]";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        // the kernel addresses both caches by one slot number (block = slot / blockSize)
+        if (kc.dims[0] != vc.dims[0]) {
+            ATB_LOG(ERROR) << "ReshapeAndCache: caches must agree on numBlocks";
+            return ERROR_INVALID_TENSOR_DIM;
+        }
+        return NO_ERROR;
+    }
+
     Param param_;
     bool siso_;
+    bool nz_;
     uint32_t extra_; // int32 inputs after slotMapping: 2 (wins, seqLens) or 3 (+ offsetIndex) under head compression
 };
 } // namespace
@@ -279,10 +356,6 @@ template <> Status CreateOperation(const infer::ReshapeAndCacheParam &opParam, O
     }
     if (opParam.kvCacheCfg != Param::K_CACHE_V_CACHE && opParam.compressType != Param::COMPRESS_TYPE_UNDEFINED) {
         ATB_LOG(ERROR) << "ReshapeAndCacheParam: compressType needs K_CACHE_V_CACHE";
-        return ERROR_INVALID_PARAM;
-    }
-    if (opParam.kvCacheCfg == Param::K_CACHE_V_CACHE_NZ) {
-        ATB_LOG(ERROR) << "ReshapeAndCacheParam: NZ caches are not implemented on MI355X";
         return ERROR_INVALID_PARAM;
     }
     *operation = new (std::nothrow) ReshapeAndCacheOperation(opParam);

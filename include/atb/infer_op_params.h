@@ -29,7 +29,7 @@ struct ReshapeAndCacheParam {
     enum KvCacheCfg : int {
         K_CACHE_V_CACHE = 0, // inputs: key, value, keyCache, valueCache, slotMapping
         K_CACHE_V_BYPASS,    // inputs: key, keyCache, slotMapping (single cache, e.g. MLA latent)
-        K_CACHE_V_CACHE_NZ   // fractal-NZ caches; not implemented on MI355X
+        K_CACHE_V_CACHE_NZ   // fractal-NZ caches [blocks, heads*headSize/L, blockSize, L], L = 32 (int8 key) or 16
     };
 
     CompressType compressType = COMPRESS_TYPE_UNDEFINED;
@@ -240,7 +240,7 @@ struct BlockCopyParam {
 // reverse of ReshapeAndCache (reference include/atb/infer_op_params.h:3070-3101).
 struct PagedCacheLoadParam {
     enum KvCacheCfg : int8_t {
-        K_CACHE_V_CACHE_NZ = 0, // fractal-NZ caches; not implemented on MI355X
+        K_CACHE_V_CACHE_NZ = 0, // fractal-NZ caches [blocks, heads*headSize/L, blockSize, L], L = 32 (int8) or 16
         K_CACHE_V_CACHE_ND      // caches [blocks, blockSize, heads, headSize]
     };
     KvCacheCfg kvCacheCfg = K_CACHE_V_CACHE_NZ;

@@ -87,6 +87,22 @@ int atbmi_reshape_and_cache_compress(const void *keyDevice, const void *valueDev
                                      void *stream);
 
 /*
+ * KV-cache write into fractal-NZ caches (ReshapeAndCacheParam::K_CACHE_V_CACHE_NZ), the writer of the caches
+ * MultiLatentAttention reads with cacheMode NZCACHE / INT8_NZCACHE. keyCache is
+ * [numBlocks, keyRowElems / L, blockSize, L] with L = 32 for one-byte and 16 for two-byte keys, valueCache
+ * [numBlocks, valueRowElems / 16, blockSize, 16]: element c of token i's key row (numKvHeads * headDimK elements)
+ * goes to block s / blockSize, piece c / L, row s % blockSize, place c % L, s = slotMapping[i]; s < 0 (or
+ * s >= numBlocks * blockSize) skips the token. Key and value may differ in element size (int8 latent rows with
+ * 16-bit rotary rows). A byte copy.
+ * Replaces: reshape_and_cache_nz.cpp:85-178 of the reference (src/kernels/mixkernels/reshape_and_cache/op_kernel/;
+ * golden tests/apitest/kernelstest/mix/test_reshape_and_cache_nz.py:45-66).
+ */
+int atbmi_reshape_and_cache_nz(const void *keyDevice, const void *valueDevice, void *keyCacheDevice,
+                               void *valueCacheDevice, const int32_t *slotMappingDevice, int64_t numTokens,
+                               int64_t keyRowElems, int64_t valueRowElems, int64_t blockSize, int64_t numBlocks,
+                               int32_t keyElemBytes, int32_t valueElemBytes, void *stream);
+
+/*
  * KV-cache write from strided views of key / value: element (token, head, channel) of key is read
  * keyOffset + token * keyStrides[0] + head * keyStrides[1] + channel * keyStrides[2] ELEMENTS from
  * keyDevice (the same for value); everything else as atbmi_reshape_and_cache. The stride arrays are
@@ -200,6 +216,21 @@ int atbmi_paged_cache_load(const void *keyCacheDevice, const void *valueCacheDev
                            void *valueDevice, int64_t batch, int64_t maxBlocksPerSeq, int64_t blockSize,
                            int64_t numBlocks, int64_t keyRowBytes, int64_t valueRowBytes, int64_t outRows,
                            int64_t maxSeqLen, int32_t cumsumMode, void *stream);
+
+/*
+ * PagedCacheLoad, fractal-NZ caches (PagedCacheLoadParam::K_CACHE_V_CACHE_NZ): the same gather from caches
+ * [numBlocks, rowBytes / pieceBytes, blockSize, piece], where a row is cut into pieces of keyPieceBytes /
+ * valuePieceBytes (32 int8 or 16 two-byte elements) and a block holds piece 0 of all its rows, then piece 1, ...
+ * The outputs are plain rows [outRows, rowBytes]. seqLens holds the lengths [batch]; there are no sequence starts
+ * and no running-sum form in this layout (reference paged_cache_load_operation.cpp:63-67).
+ * Replaces: PagedCacheLoadOperation's NZ kernel (golden tests/apitest/kernelstest/mix/
+ * test_paged_cache_load_nz.py:72-131).
+ */
+int atbmi_paged_cache_load_nz(const void *keyCacheDevice, const void *valueCacheDevice,
+                              const int32_t *blockTablesDevice, const int32_t *seqLensDevice, void *keyDevice,
+                              void *valueDevice, int64_t batch, int64_t maxBlocksPerSeq, int64_t blockSize,
+                              int64_t numBlocks, int64_t keyRowBytes, int64_t valueRowBytes, int64_t keyPieceBytes,
+                              int64_t valuePieceBytes, int64_t outRows, int64_t maxSeqLen, void *stream);
 
 /*
  * Fused quantise + KV-cache write (extension; the reference runs the

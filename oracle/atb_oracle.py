@@ -13,6 +13,10 @@ pinned by tests/test_oracle.py against closed forms, fp64 brute force and
 the invariants of the mathematics (no function is left "parity unpinned"):
 
   reshape_and_cache   tests/apitest/kernelstest/mix/test_reshape_and_cache.py:45-65
+  reshape_and_cache_nz
+                      tests/apitest/kernelstest/mix/test_reshape_and_cache_nz.py:45-66 (fractal-NZ caches
+                      [blocks, channels / last, block_size, last], last = 32 for int8 keys, else 16); pinned by
+                      element loops over flat addresses and by nz_to_nd of the result = the plain write
   reshape_and_cache_compress
                       tests/apitest/kernelstest/mix/test_reshape_and_cache_wins.py:61-88 (the last wins[i]
                       tokens of every (sequence, head) pair) and test_reshape_and_cache_wins_rope.py:78-131 (a
@@ -102,6 +106,10 @@ the invariants of the mathematics (no function is left "parity unpinned"):
                       or their running sums. The golden also skips negative block ids, moving later rows up;
                       its own tests never draw one (ids come from [0, num_blocks)), so that branch fixes no
                       behaviour of the kernel: here such rows are skipped in place, see paged_cache_load)
+  paged_cache_load_nz tests/apitest/kernelstest/mix/test_paged_cache_load_nz.py:72-131 (the same gather from
+                      fractal-NZ caches, the pieces of a row put back side by side); pinned by flat addresses,
+                      by paged_cache_load over nz_to_nd of the caches and by the round trip through
+                      reshape_and_cache_nz
   merge_partials      src/kernels/mixkernels/pagedattention/op_kernel/
                       paged_attention_decoder_nd_common.cce:6568-6760,7959-7975 (split-KV combine)
 
@@ -143,6 +151,25 @@ def reshape_and_cache(key, value, key_cache, value_cache, slot_mapping):
         kc[slot // block_size, slot % block_size] = key[i]
         if vc is not None:
             vc[slot // block_size, slot % block_size] = value[i]
+    return kc, vc
+
+
+def reshape_and_cache_nz(key, value, key_cache, value_cache, slot_mapping):
+    """KV-cache write into fractal-NZ caches [blocks, heads * head_size / last, block_size, last] (copies are
+    returned): token i's key row, flattened to heads * head_size elements, is cut into pieces of `last` elements
+    (the cache's last dim: 32 for int8 keys, 16 otherwise; 16 for values) and piece k lands in
+    key_cache[s // block_size, k, s % block_size, :], s = slot_mapping[i]; negative slots are skipped. Follows the
+    reference golden tests/apitest/kernelstest/mix/test_reshape_and_cache_nz.py:45-66 (also
+    tests/framework/python/CsvOpsTestTool/data_generation.py:4385-4420). Pure data movement."""
+    kc = np.array(key_cache, copy=True)
+    vc = np.array(value_cache, copy=True)
+    block_size = kc.shape[2]
+    for i, slot in enumerate(np.asarray(slot_mapping).tolist()):
+        if slot < 0:
+            continue
+        for cache, row in ((kc, key[i]), (vc, value[i])):
+            last = cache.shape[3]
+            cache[slot // block_size, :, slot % block_size, :] = np.asarray(row).reshape(-1, last)
     return kc, vc
 
 
@@ -304,6 +331,26 @@ def paged_cache_load(key_cache, value_cache, block_tables, seq_lens, key, value,
             if block >= 0:
                 key[row] = key_cache[block][j % block_size]
                 value[row] = value_cache[block][j % block_size]
+            row += 1
+    return key, value
+
+
+def paged_cache_load_nz(key_cache, value_cache, block_tables, seq_lens, key, value):
+    """The gather from fractal-NZ caches [blocks, channels / last, block_size, last]: returns copies of key
+    [tokens, channels_k] and value [tokens, channels_v] where row (tokens of the sequences before i) + j is the
+    cache row of token j of sequence i, its pieces put back side by side (reference golden
+    tests/apitest/kernelstest/mix/test_paged_cache_load_nz.py:72-131). A negative block id leaves its row as it
+    is (the golden would move the later rows up; its tests draw ids from [0, num_blocks) only)."""
+    key = np.array(key, copy=True)
+    value = np.array(value, copy=True)
+    block_size = key_cache.shape[2]
+    row = 0
+    for i, n in enumerate(np.asarray(seq_lens).tolist()):
+        for j in range(int(n)):
+            block = int(block_tables[i][j // block_size])
+            if block >= 0:
+                key[row] = key_cache[block, :, j % block_size, :].reshape(-1)
+                value[row] = value_cache[block, :, j % block_size, :].reshape(-1)
             row += 1
     return key, value
 

@@ -107,6 +107,131 @@ def test_reshape_and_cache_single_cache_and_out_of_range_slots(binding, oracle, 
     ctx.close()
 
 
+# ------------------------------------------------------------------ ReshapeAndCache, fractal-NZ caches
+NZ_RAC_SHAPES = [
+    # tokens, heads, dk, dv, block, blocks, key dtype, value dtype
+    (6144, 1, 512, 64, 128, 64, torch.int8, torch.float16),      # reference test_reshape_and_cache_nz.py:99-108
+    (8192, 1, 128, 128, 128, 96, torch.int8, torch.float16),     # :110-119
+    (6144, 1, 512, 64, 128, 64, torch.float16, torch.float16),   # :121-130
+    (8192, 1, 128, 128, 128, 96, torch.float16, torch.float16),  # :132-141
+    (4, 6, 64, 128, 64, 4, torch.int8, torch.bfloat16),          # CSV row 46: int8 key, heads * 64 / 32 pieces
+    (4, 6, 128, 128, 128, 4, torch.bfloat16, torch.float16),     # CSV row 43: mixed 16-bit types
+    (64, 1, 512, 64, 128, 34, torch.int8, torch.bfloat16),       # a decode step of the MLA int8 cache
+    (33, 3, 32, 16, 16, 5, torch.float16, torch.bfloat16),       # smallest pieces, block size 16
+]
+
+
+def _nz_rac_inputs(rng, dev, tokens, heads, dk, dv, block, blocks, kdt, vdt):
+    def mk(shape, dtype, lo, hi):
+        a = rng.integers(lo, hi, size=shape)
+        return torch.from_numpy(a.astype(np.int8)).to(dev) if dtype == torch.int8 else \
+            torch.from_numpy(a.astype(np.float32)).to(dtype).to(dev)
+    kl = 32 if kdt == torch.int8 else 16
+    key, value = mk((tokens, heads, dk), kdt, -100, 100), mk((tokens, heads, dv), vdt, -100, 100)
+    kc, vc = mk((blocks, heads * dk // kl, block, kl), kdt, 101, 120), mk((blocks, heads * dv // 16, block, 16), vdt, 101, 120)
+    n = blocks * block
+    # as the reference's test: unique slots from [-n, n), the negative ones are skipped, token 0 in slot 0
+    slots = rng.choice(np.delete(np.arange(-n, n), n), size=tokens, replace=False).astype(np.int32)
+    slots[0] = 0
+    return key, value, kc, vc, slots
+
+
+@pytest.mark.parametrize("shape", NZ_RAC_SHAPES, ids=lambda s: "x".join(str(v) for v in s[:6]) + "".join(
+    "_" + str(t).split(".")[-1] for t in s[6:]))
+def test_reshape_and_cache_nz_bit_exact(binding, oracle, dev, stream, shape):
+    """kvCacheCfg K_CACHE_V_CACHE_NZ through the operation and through the C ABI, against the oracle."""
+    rng = _rng(14)
+    tokens, heads, dk, dv, block, blocks = shape[:6]
+    key, value, kc, vc, slots = _nz_rac_inputs(rng, dev, *shape)
+    kc2, vc2 = kc.clone(), vc.clone()
+    want_k, want_v = oracle.reshape_and_cache_nz(_bits(key).cpu().numpy(), _bits(value).cpu().numpy(),
+                                                 _bits(kc).cpu().numpy(), _bits(vc).cpu().numpy(), slots)
+    ctx = binding.Context(stream)
+    runner = binding.OperationRunner("ReshapeAndCacheOperation", binding.ReshapeAndCacheParam(kvCacheCfg=2), ctx)
+    nz = [binding.make_tensor(binding._torch_acl_dtype(t), list(t.shape), device_ptr=t.data_ptr(), fmt="fractal_nz")
+          for t in (kc, vc)]
+    with torch.cuda.stream(stream):
+        slots_d = torch.from_numpy(slots).to(dev)
+        runner.run([key, value, nz[0], nz[1], slots_d], outputs=nz)
+        rc = binding.kernels().atbmi_reshape_and_cache_nz(
+            key.data_ptr(), value.data_ptr(), kc2.data_ptr(), vc2.data_ptr(), slots_d.data_ptr(), tokens, heads * dk,
+            heads * dv, block, blocks, key.element_size(), value.element_size(), stream.cuda_stream)
+    stream.synchronize()
+    assert rc == 0, binding.last_kernel_error()
+    for got in ((kc, vc), (kc2, vc2)):
+        assert np.array_equal(_bits(got[0]).cpu().numpy(), want_k)
+        assert np.array_equal(_bits(got[1]).cpu().numpy(), want_v)
+    assert (slots < 0).any() and not np.array_equal(want_k, 0 * want_k)
+    runner.close()
+    ctx.close()
+
+
+def test_reshape_and_cache_nz_feeds_multi_latent_attention(binding, oracle, dev, stream):
+    """The step as a model runs it: latent and rotary rows written by ReshapeAndCache, read by
+    MultiLatentAttention. Fractal-NZ caches (kvCacheCfg 2 -> cacheMode NZCACHE) must give the same bits as
+    the token-major pair (kvCacheCfg 0 -> cacheMode KROPE_CTKV) on the same rows, and unaligned bases and
+    slots past the end of the cache are handled by the C ABI as documented."""
+    rng = _rng(15)
+    heads, dv, dr, block, dtype = 32, 512, 64, 128, torch.float16
+    ctx_lens = np.array([300, 129, 17], dtype=np.int32)
+    blocks_per = 3
+    blocks = 3 * blocks_per + 1
+    tables = torch.from_numpy(rng.permutation(blocks)[:9].reshape(3, blocks_per).astype(np.int32)).to(dev)
+    tokens = int(ctx_lens.sum())
+    latent = ((torch.rand((tokens, 1, dv)) - 0.5)).to(dtype).to(dev)
+    rotary = ((torch.rand((tokens, 1, dr)) - 0.5)).to(dtype).to(dev)
+    slots = np.concatenate([tables.cpu().numpy()[b, np.arange(n) // block] * block + np.arange(n) % block
+                            for b, n in enumerate(ctx_lens)]).astype(np.int32)
+    nd = [torch.zeros((blocks, block, 1, dv), dtype=dtype, device=dev), torch.zeros((blocks, block, 1, dr), dtype=dtype, device=dev)]
+    nz = [torch.zeros((blocks, dv // 16, block, 16), dtype=dtype, device=dev), torch.zeros((blocks, dr // 16, block, 16), dtype=dtype, device=dev)]
+    nz_desc = [binding.make_tensor(binding._torch_acl_dtype(t), list(t.shape), device_ptr=t.data_ptr(), fmt="fractal_nz")
+               for t in nz]
+    c = binding.Context(stream)
+    write_nd = binding.OperationRunner("ReshapeAndCacheOperation", binding.ReshapeAndCacheParam(), c)
+    write_nz = binding.OperationRunner("ReshapeAndCacheOperation", binding.ReshapeAndCacheParam(kvCacheCfg=2), c)
+    q = ((torch.rand((3, heads, dv + dr)) - 0.5)).to(dtype).to(dev)
+    lens = torch.from_numpy(ctx_lens)
+    scale = 1.0 / math.sqrt(192.0)
+    outs = []
+    with torch.cuda.stream(stream):
+        slots_d = torch.from_numpy(slots).to(dev)
+        write_nd.run([latent, rotary, nd[0], nd[1], slots_d], outputs=nd)
+        write_nz.run([latent, rotary, nz_desc[0], nz_desc[1], slots_d], outputs=nz_desc)
+        for mode, caches in ((1, nd), (3, nz_desc)):
+            op = binding.OperationRunner("MultiLatentAttentionOperation", binding.MultiLatentAttentionParam(
+                headNum=heads, kvHeadNum=1, qkScale=scale, cacheMode=mode), c)
+            outs.append(op.run([q[..., :dv].contiguous(), q[..., dv:].contiguous(), caches[0], caches[1], tables,
+                                lens.to(dev)], host_inputs={5: lens})[0])
+            op.close()
+    stream.synchronize()
+    assert torch.equal(outs[0], outs[1]) and float(outs[0].float().abs().max()) > 0
+    for a, b in zip(nd, nz):
+        assert np.array_equal(oracle.nd_to_nz(_bits(a).cpu().numpy()[:, :, 0, :]), _bits(b).cpu().numpy())
+    # the C ABI alone: bases aligned to 2 bytes only (element-wide accesses), slots past the cache skipped
+    k = binding.kernels()
+    store = torch.zeros(blocks * block * (dv + dr) + 64, dtype=dtype, device=dev)
+    odd_k = store[1:1 + nz[0].numel()]
+    odd_v = store[nz[0].numel() + 3:nz[0].numel() + 3 + nz[1].numel()]
+    with torch.cuda.stream(stream):
+        far = slots_d.clone()
+        far[::7] = blocks * block + 5
+        rc = k.atbmi_reshape_and_cache_nz(latent.data_ptr(), rotary.data_ptr(), odd_k.data_ptr(), odd_v.data_ptr(),
+                                          far.data_ptr(), tokens, dv, dr, block, blocks, 2, 2, stream.cuda_stream)
+    stream.synchronize()
+    assert rc == 0, binding.last_kernel_error()
+    kept = slots.copy()
+    kept[::7] = -1
+    want_k, want_v = oracle.reshape_and_cache_nz(_bits(latent).cpu().numpy(), _bits(rotary).cpu().numpy(),
+                                                 np.zeros(nz[0].shape, np.int16), np.zeros(nz[1].shape, np.int16), kept)
+    assert np.array_equal(_bits(odd_k).cpu().numpy().reshape(want_k.shape), want_k)
+    assert np.array_equal(_bits(odd_v).cpu().numpy().reshape(want_v.shape), want_v)
+    assert k.atbmi_reshape_and_cache_nz(latent.data_ptr(), rotary.data_ptr(), odd_k.data_ptr(), odd_v.data_ptr(),
+                                        far.data_ptr(), tokens, dv + 8, dr, block, blocks, 2, 2, stream.cuda_stream) != 0
+    write_nd.close()
+    write_nz.close()
+    c.close()
+
+
 # ------------------------------------------------------------------ ReshapeAndCacheWithStride
 STRIDED_CASES = [
     # tokens, heads, d, view builder -> (storage elements, strides, offset) per input, what it exercises
@@ -660,6 +785,61 @@ def test_paged_cache_load_bit_exact(binding, oracle, dev, stream, shape, cumsum,
                 torch.from_numpy(seq_starts).to(dev)], outputs=[key, value])
     stream.synchronize()
     assert np.array_equal(_bits(key).cpu().numpy(), want_k) and np.array_equal(_bits(value).cpu().numpy(), want_v)
+    op.close()
+    c.close()
+
+
+# batch, channels K, channels V, block size, blocks, key dtype, value dtype
+# (reference test_paged_cache_load_nz.py:150-260: 128-channel rows of every dtype pair; the MLA int8 cache)
+NZ_LOAD_SHAPES = [
+    (16, 128, 128, 128, 128, torch.float16, torch.float16),
+    (16, 128, 128, 128, 128, torch.int8, torch.int8),
+    (16, 128, 128, 128, 128, torch.bfloat16, torch.bfloat16),
+    (16, 128, 128, 128, 128, torch.int8, torch.float16),
+    (8, 512, 64, 128, 290, torch.int8, torch.bfloat16),    # CSV row 13 ("modelcase"): int8 latent + 16-bit rotary rows
+    (5, 64, 32, 16, 40, torch.float16, torch.float16),
+]
+
+
+@pytest.mark.parametrize("shape", NZ_LOAD_SHAPES, ids=lambda s: "x".join(str(v) for v in s[:5]) + "".join(
+    "_" + str(t).split(".")[-1] for t in s[5:]))
+def test_paged_cache_load_nz_bit_exact(binding, oracle, dev, stream, shape):
+    """kvCacheCfg K_CACHE_V_CACHE_NZ (the param's default) through the operation and the C ABI."""
+    batch, ck, cv, block, blocks, kdt, vdt = shape
+    rng = _rng(560 + batch + ck)
+
+    def cache(chans, dtype):
+        last = 32 if dtype == torch.int8 else 16
+        a = rng.integers(-100, 100, size=(blocks, chans // last, block, last))
+        return torch.from_numpy(a.astype(np.int8)).to(dev) if dtype == torch.int8 else \
+            torch.from_numpy(a.astype(np.float32)).to(dtype).to(dev)
+    kc, vc = cache(ck, kdt), cache(cv, vdt)
+    lens = rng.integers(1, 1025, size=batch).astype(np.int32)
+    lens[rng.integers(batch)] = 0
+    max_blocks = (int(lens.max()) + block - 1) // block + 2
+    tables = rng.integers(0, blocks, size=(batch, max_blocks)).astype(np.int32)
+    total = int(lens.sum())
+    key = torch.zeros((total, ck), dtype=kdt, device=dev)
+    value = torch.zeros((total, cv), dtype=vdt, device=dev)
+    key2, value2 = key.clone(), value.clone()
+    want_k, want_v = oracle.paged_cache_load_nz(_bits(kc).cpu().numpy(), _bits(vc).cpu().numpy(), tables, lens,
+                                                _bits(key).cpu().numpy(), _bits(value).cpu().numpy())
+    c = binding.Context(stream)
+    op = binding.OperationRunner("PagedCacheLoadOperation", binding.PagedCacheLoadParam(), c)
+    nz = [binding.make_tensor(binding._torch_acl_dtype(t), list(t.shape), device_ptr=t.data_ptr(), fmt="fractal_nz")
+          for t in (kc, vc)]
+    with torch.cuda.stream(stream):
+        tables_d, lens_d = torch.from_numpy(tables).to(dev), torch.from_numpy(lens).to(dev)
+        op.run([nz[0], nz[1], tables_d, lens_d, key, value], outputs=[key, value])
+        rc = binding.kernels().atbmi_paged_cache_load_nz(
+            kc.data_ptr(), vc.data_ptr(), tables_d.data_ptr(), lens_d.data_ptr(), key2.data_ptr(), value2.data_ptr(),
+            batch, max_blocks, block, blocks, ck * kc.element_size(), cv * vc.element_size(), 32, 32, total,
+            int(lens.max()), stream.cuda_stream)
+    stream.synchronize()
+    assert rc == 0, binding.last_kernel_error()
+    for got_k, got_v in ((key, value), (key2, value2)):
+        assert np.array_equal(_bits(got_k).cpu().numpy(), want_k) and np.array_equal(_bits(got_v).cpu().numpy(), want_v)
+    assert total > 0 and np.any(want_k != 0)
     op.close()
     c.close()
 

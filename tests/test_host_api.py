@@ -59,7 +59,8 @@ def _pa_mask_shape_refused(case):
 
 
 def _rac_unimplemented(p):
-    return p.get("kvCacheCfg", 0) == 2
+    """Features of ReshapeAndCacheParam the reference accepts but this library rejects at creation: none."""
+    return False
 
 
 def _mla_unimplemented(p):
@@ -188,9 +189,7 @@ def test_block_copy_table(binding, ctx, case):
 
 @pytest.mark.parametrize("case", CACHE_LOAD_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
 def test_paged_cache_load_table(binding, ctx, case):
-    # the fractal-NZ cache layout (kvCacheCfg 0, the param's default) is rejected when the operation is created
-    nz = case["param"].get("kvCacheCfg", 0) == 0
-    _check(binding, case, ctx, nz and not case["expected"].startswith("C:"))
+    _check(binding, case, ctx, False)
 
 
 @pytest.mark.parametrize("case", ELEWISE_CASES, ids=lambda c: "%d-%s" % (c["case"], c["name"]))
@@ -259,7 +258,7 @@ def test_table_coverage():
               _pa_mask_shape_refused(c)]
     rac_dev = [c for c in RAC_CASES if _rac_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
     assert len(PA_CASES) == 81 and len(PA_CASES) - len(pa_dev) >= 75
-    assert len(RAC_CASES) == 38 and len(RAC_CASES) - len(rac_dev) >= 29
+    assert len(RAC_CASES) == 38 and len(rac_dev) == 0
     # every MultiLatentAttention row is replayed at face value
     mla_dev = [c for c in MLA_CASES if _mla_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
     assert len(MLA_CASES) == 147 and len(mla_dev) == 0
@@ -1346,10 +1345,20 @@ def test_acl_tensor_handle_and_two_call_wrappers(binding, ctx):
                                                  None, 1, False, False, ctypes.byref(ws), ctypes.byref(six),
                                                  ctx.ptr) == E["ERROR_INVALID_IN_TENSOR_NUM"]
     lib.atb_c_destroy_operation(six)
-    nzload = ctypes.c_void_p()   # the fractal-NZ layout (kvCacheCfg 0) is not built
+    # the fractal-NZ layout (kvCacheCfg 0): six tensors, caches [blocks, channels / 16, blockSize, 16], rows [tokens, channels]
+    nzf = binding.ACL_FORMAT_BY_NAME["fractal_nz"]
+    hn = dict(kc=mk("float16", [16, 64, 128, 16], FAKE_DEVICE, nzf), vc=mk("float16", [16, 64, 128, 16], FAKE_DEVICE, nzf),
+              key=mk("float16", [400, 1024], FAKE_DEVICE), value=mk("float16", [400, 1024], FAKE_DEVICE))
+    nzload = ctypes.c_void_p()
+    assert lib.AtbPagedCacheLoadGetWorkspaceSize(hn["kc"], hn["vc"], hc["tables"], hc["lens"], hn["key"], hn["value"],
+                                                 None, 0, False, False, ctypes.byref(ws), ctypes.byref(nzload),
+                                                 ctx.ptr) == 0 and nzload.value
+    # token-major handles do not match that operation's dtype / format table
     assert lib.AtbPagedCacheLoadGetWorkspaceSize(hc["kc"], hc["vc"], hc["tables"], hc["lens"], hc["key"], hc["value"],
                                                  None, 0, False, False, ctypes.byref(ws), ctypes.byref(nzload),
-                                                 ctx.ptr) == E["ERROR_INVALID_PARAM"]
+                                                 ctx.ptr) == E["ERROR_INVALID_TENSOR_INI_MATCH"]
+    lib.atb_c_destroy_operation(nzload)
+    hc.update({"nz_" + k: v for k, v in hn.items()})
     for h in list(handles.values()) + list(hc.values()):
         lib.aclDestroyTensor(h)
 

@@ -64,6 +64,38 @@ def test_reshape_and_cache_single_cache(oracle):
     assert np.array_equal(kc[1, 1, 0], key[0, 0]) and kc.sum() == key[0].sum()
 
 
+@pytest.mark.parametrize("key_dtype,value_dtype,heads,dk,dv", [(np.int8, np.float16, 1, 64, 32),
+                                                              (np.float16, np.float16, 3, 32, 16),
+                                                              (np.int8, np.float32, 2, 48, 24)])
+def test_reshape_and_cache_nz_by_flat_addresses(oracle, key_dtype, value_dtype, heads, dk, dv):
+    """Element c of token i's flattened row must sit at flat address
+    ((block * pieces + c // last) * block_size + offset) * last + c % last of the cache (reference
+    test_reshape_and_cache_nz.py:45-66 spelled out per element), and un-tiling the result must give the
+    plain token-major write."""
+    rng = _rng(7)
+    tokens, blocks, block = 9, 3, 16
+    kl = 32 if key_dtype == np.int8 else 16
+    key = rng.integers(-100, 100, size=(tokens, heads, dk)).astype(key_dtype)
+    value = rng.integers(-100, 100, size=(tokens, heads, dv)).astype(value_dtype)
+    kc0 = rng.integers(-9, 9, size=(blocks, heads * dk // kl, block, kl)).astype(key_dtype)
+    vc0 = rng.integers(-9, 9, size=(blocks, heads * dv // 16, block, 16)).astype(value_dtype)
+    slots = rng.choice(np.arange(-blocks * block, blocks * block), size=tokens, replace=False).astype(np.int32)
+    slots[0] = 5
+    kc, vc = oracle.reshape_and_cache_nz(key, value, kc0, vc0, slots)
+    for cache, cache0, rows, last in ((kc, kc0, key.reshape(tokens, -1), kl), (vc, vc0, value.reshape(tokens, -1), 16)):
+        expect = cache0.copy().reshape(-1)
+        pieces = rows.shape[1] // last
+        for i, s in enumerate(slots.tolist()):
+            if s < 0:
+                continue
+            for c in range(rows.shape[1]):
+                expect[((s // block * pieces + c // last) * block + s % block) * last + c % last] = rows[i, c]
+        assert np.array_equal(cache.reshape(-1), expect)
+        plain, _ = oracle.reshape_and_cache(rows[:, None, :], None, oracle.nz_to_nd(cache0)[:, :, None, :], None, slots)
+        assert np.array_equal(oracle.nz_to_nd(cache), plain[:, :, 0, :])
+    assert (slots < 0).any() and not np.array_equal(kc, kc0) and np.array_equal(kc0, kc0.copy())
+
+
 def test_quant_golden_dtype_exact_rational(oracle):
     """The ElewiseOperation form (16-bit scale, quotient rounded to fp16, then to an integer) against exact
     rational arithmetic: the fp16 nearest to x / s (ties to even), then the integer nearest to that."""
@@ -383,6 +415,45 @@ def test_paged_cache_load_negative_block_ids_leave_their_rows(oracle):
     k, v = oracle.paged_cache_load(kc, kc, tables, np.array([5], np.int32), np.zeros((5, 1, 1), np.float32),
                                    np.zeros((5, 1, 1), np.float32))
     assert k[:, 0, 0].tolist() == [3.0, 4.0, 0.0, 0.0, 1.0] and np.array_equal(k, v)
+
+
+@pytest.mark.parametrize("key_dtype,value_dtype", [(np.int8, np.int8), (np.int8, np.float16), (np.float16, np.float16)])
+def test_paged_cache_load_nz_by_flat_addresses_and_round_trip(oracle, key_dtype, value_dtype):
+    rng = _rng(62)
+    blocks, block, ck, cv = 7, 16, 64, 32
+    kl, vl = (32 if key_dtype == np.int8 else 16), (32 if value_dtype == np.int8 else 16)
+    kc = rng.integers(-100, 100, size=(blocks, ck // kl, block, kl)).astype(key_dtype)
+    vc = rng.integers(-100, 100, size=(blocks, cv // vl, block, vl)).astype(value_dtype)
+    lens = np.array([17, 0, 40, 1], np.int32)
+    tables = rng.integers(0, blocks, size=(4, 3)).astype(np.int32)
+    total = int(lens.sum())
+    key0 = np.full((total + 1, ck), 9, key_dtype)
+    val0 = np.full((total + 1, cv), 9, value_dtype)
+    got_k, got_v = oracle.paged_cache_load_nz(kc, vc, tables, lens, key0, val0)
+    # element by element over the flat cache
+    for cache, got, last in ((kc, got_k, kl), (vc, got_v, vl)):
+        flat, chans, row = cache.reshape(-1), got.shape[1], 0
+        for i, n in enumerate(lens):
+            for j in range(n):
+                blk = tables[i][j // block]
+                for c in range(chans):
+                    assert got[row, c] == flat[((blk * (chans // last) + c // last) * block + j % block) * last + c % last]
+                row += 1
+        assert row == total and np.all(got[total:] == 9)
+    # the token-major gather over the un-tiled caches
+    nd_k, nd_v = oracle.paged_cache_load(oracle.nz_to_nd(kc)[:, :, None, :], oracle.nz_to_nd(vc)[:, :, None, :], tables, lens,
+                                         key0[:, None, :], val0[:, None, :])
+    assert np.array_equal(nd_k[:, 0, :], got_k) and np.array_equal(nd_v[:, 0, :], got_v)
+    # it undoes reshape_and_cache_nz (value caches written by that operator are 16-bit, pieces of 16)
+    if vl == 16:
+        tables = rng.permutation(blocks)[:6].reshape(2, 3).astype(np.int32)
+        lens = np.array([33, 48], np.int32)
+        slots = np.concatenate([tables[i][np.arange(n) // block] * block + np.arange(n) % block for i, n in enumerate(lens)])
+        new_k = rng.integers(-100, 100, size=(81, 1, ck)).astype(key_dtype)
+        new_v = rng.integers(-100, 100, size=(81, 1, cv)).astype(value_dtype)
+        kc2, vc2 = oracle.reshape_and_cache_nz(new_k, new_v, kc, vc, slots.astype(np.int32))
+        back_k, back_v = oracle.paged_cache_load_nz(kc2, vc2, tables, lens, np.zeros((81, ck), key_dtype), np.zeros((81, cv), value_dtype))
+        assert np.array_equal(back_k, new_k[:, 0, :]) and np.array_equal(back_v, new_v[:, 0, :])
 
 
 # ---------------------------------------------------------------- cache write under head compression
