@@ -211,6 +211,16 @@ class AtbmiMlaInt8Call(ctypes.Structure):
                     "query", "queryRope", "kvCache", "kRopeCache", "blockTables", "qkDescale", "pvDescale", "mask", "out",
                     "lse")]
 
+class AtbmiPaInt8QCall(ctypes.Structure):
+    """One atbmi_pa_int8q_decode call (include/atbmi_kernels.h)."""
+    _fields_ = [(n, ctypes.c_int32) for n in ("outDtype", "numHeads", "numKvHeads", "headDim", "blockSize", "numBlocks",
+                                              "maxBlocksPerSeq", "batch", "numQueryRows", "offline", "hasMask",
+                                              "maskLen")] + [
+        ("qkScale", ctypes.c_float), ("maskSeqStride", ctypes.c_int64), ("maskHeadStride", ctypes.c_int64)] + [
+        (n, ctypes.c_void_p) for n in ("hostContextLens", "query", "keyCache", "valueCache", "blockTables", "kDescale",
+                                       "vDescale", "pScale", "mask", "out")]
+
+
 class AtbmiMlaMaskFreeCall(ctypes.Structure):
     """One atbmi_mla_mask_free_expand call (include/atbmi_kernels.h)."""
     _fields_ = [("batch", ctypes.c_int32), ("numQueryRows", ctypes.c_int32), ("templateBatch", ctypes.c_int32),
@@ -277,6 +287,8 @@ def kernels():
         lib.atbmi_mla_prefill.argtypes = [ctypes.POINTER(AtbmiMlaPrefillCall), vp, u64, vp]
         lib.atbmi_mla_int8_workspace_size.argtypes = [ctypes.POINTER(AtbmiMlaInt8Call), ctypes.POINTER(u64)]
         lib.atbmi_mla_int8_decode.argtypes = [ctypes.POINTER(AtbmiMlaInt8Call), vp, u64, vp]
+        lib.atbmi_pa_int8q_workspace_size.argtypes = [ctypes.POINTER(AtbmiPaInt8QCall), ctypes.POINTER(u64)]
+        lib.atbmi_pa_int8q_decode.argtypes = [ctypes.POINTER(AtbmiPaInt8QCall), vp, u64, vp]
         lib.atbmi_pa_plan_destroy.argtypes = [vp]
         lib.atbmi_pa_plan_destroy.restype = None
         lib.atbmi_timing_enable.argtypes = [i32]

@@ -516,6 +516,58 @@ int atbmi_mla_int8_workspace_size(const AtbmiMlaInt8Call *call, uint64_t *bytes)
 int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspaceDevice, uint64_t workspaceBytes, void *stream);
 
 /*
+ * PagedAttention decode with int8 queries over int8 caches (PagedAttentionParam::quantType TYPE_QUANT_QKV_ONLINE /
+ * TYPE_QUANT_QKV_OFFLINE; reference src/ops/ops_infer/paged_attention/paged_attention_operation.cpp:250-275,429-436
+ * for the parameters and inputs, kernel library src/kernels/mixkernels/pagedattention/paged_attention_operation.cpp:
+ * 357-403 for the descale shapes, golden tests/apitest/kernelstest/mix/test_paged_attention_common.py:104-110,147-229):
+ * query, keys and values are int8 with one fp32 descale per QUERY head for the scores (kDescale) and one for the
+ * values (vDescale); the softmax weights of every tile of 128 tokens are quantised to int8 before they multiply the
+ * int8 value rows, against the tile's largest weight (online) or with the factor pScale[head] (offline); all integer
+ * products are exact.
+ *   query       int8 [numQueryRows, numHeads, headDim]            kDescale, vDescale, pScale  fp32 [numHeads]
+ *   keyCache, valueCache  int8 [numBlocks, blockSize, numKvHeads, headDim]   blockTables int32 [batch, maxBlocksPerSeq]
+ *   mask        NULL, or 16-bit (the output's type): the bias of sequence b, head h, token t is
+ *               mask[b * maskSeqStride + h * maskHeadStride + t] (elements; a stride of 0 shares the row), added to
+ *               the scaled scores
+ *   out         16-bit [numQueryRows, numHeads, headDim]
+ * One query token per sequence; a sequence of length 0 takes no query row. headDim is 64, 128 or 256; pScale is
+ * expected to keep w x pScale within 127, as the reference's own generator does. The lengths are a host array, read
+ * during the call.
+ */
+typedef struct AtbmiPaInt8QCall {
+    int32_t outDtype;          /* ATBMI_F16 or ATBMI_BF16: type of mask and out */
+    int32_t numHeads;
+    int32_t numKvHeads;
+    int32_t headDim;
+    int32_t blockSize;
+    int32_t numBlocks;
+    int32_t maxBlocksPerSeq;
+    int32_t batch;
+    int32_t numQueryRows;
+    int32_t offline;           /* 0: weights quantised against the tile's maximum; 1: with pScale */
+    int32_t hasMask;
+    int32_t maskLen;           /* positions a mask row covers, >= every context length */
+    float qkScale;
+    int64_t maskSeqStride;
+    int64_t maskHeadStride;
+    const int32_t *hostContextLens; /* [batch], host memory */
+    const void *query;
+    const void *keyCache;
+    const void *valueCache;
+    const int32_t *blockTables;
+    const float *kDescale;
+    const float *vDescale;
+    const float *pScale;       /* offline only */
+    const void *mask;
+    void *out;
+} AtbmiPaInt8QCall;
+
+/* Validates the call (pointers aside) and reports the device workspace it needs (16 bytes per sequence). */
+int atbmi_pa_int8q_workspace_size(const AtbmiPaInt8QCall *call, uint64_t *bytes);
+/* Uploads the sequence list into the workspace and launches the kernel on `stream`; does not wait. */
+int atbmi_pa_int8q_decode(const AtbmiPaInt8QCall *call, void *workspaceDevice, uint64_t workspaceBytes, void *stream);
+
+/*
  * MultiLatentAttention with maskType MASK_TYPE_MASK_FREE and several query tokens (decode calcTypes; replaces the
  * mask handling of the reference's device kernel, src/kernels/mixkernels/multi_latent_attention/op_kernel/
  * mla.cce:3719-3750 with 2581-2592, and the shape rule of tiling/mla_tiling.cpp:156-166): expands the compressed

@@ -65,6 +65,17 @@ the invariants of the mathematics (no function is left "parity unpinned"):
                       block_size, 16]); the NZCACHE operator is paged_attention over nz_to_nd of its
                       caches (:767-797 feed the same golden as the ND test); pinned by flat addresses,
                       the round trip and the reference's two-step reshape / permute written with torch
+  paged_attention_int8q
+                      tests/apitest/kernelstest/mix/test_paged_attention_common.py:104-110 (exact int32 products of
+                      the int8 query and the int8 key rows, times a descale per query head), :147-168
+                      (softmax_quant_numpy: the weights of a tile quantised to int8, online against the tile's
+                      largest weight or offline with a given factor per head), :171-229 (tiles joined by online
+                      rescaling), :256-276 (scale, mask, and the whole context as one tile as the high-precision
+                      golden). As for mla_int8_decode the tile length is a parameter of the golden, not of the
+                      operator (:3026-3227 run it with the Ascend kernel's block size and split). Pinned by an
+                      independent float64 loop version, by exactly representable cases where quantisation loses
+                      nothing (= float attention over the dequantised tensors), by tile invariance in those cases,
+                      and by agreement with mla_int8_decode on a shared case
   mla_int8_decode     tests/apitest/opstest/python/operations/multi_latent_attention/
                       test_multi_latent_attention_int8nz.py:115-121 (exact int32 products of the int8 query and
                       cache, times a per-head descale), :276-286 (the 64 rotary channels in fp32, added before
@@ -797,6 +808,66 @@ def mla_int8_decode(q_int8, q_rope, kv_int8, k_rope, block_tables, context_lens,
                 if lse_out is not None:
                     lse_out[r, h] = np.log(gl) + gm if gl > 0 else -np.inf
         row += n_rows
+    return out
+
+
+def paged_attention_int8q(q_int8, key_cache, value_cache, block_tables, context_lens, k_descale, v_descale, scale,
+                          p_scale=None, tile=128, mask=None, mask_per_head=None, out_init=0.0):
+    """Decode attention with int8 queries over int8 caches (PagedAttentionParam quantType QKV online / offline;
+    reference golden tests/apitest/kernelstest/mix/test_paged_attention_common.py:104-110 (exact int32 products
+    times a descale per QUERY head), :256-263 (then the scale, then the mask), :147-168 (softmax_quant_numpy: weights
+    exp(s - running max); online they are quantised against the tile's largest weight, rint(fp16(w / (wmax / 127)))
+    with value descale v_descale * wmax / 127; offline with the given factor, rint(fp16(w * p_scale[h])) with value
+    descale v_descale), :171-216 (tiles joined by the usual online rescaling, the denominator adds up the
+    unquantised weights)).
+    q_int8 [rows, H, D] int8; key_cache / value_cache [blocks, block_size, G, D] int8; k_descale, v_descale, p_scale
+    [H] float32 (p_scale None: online). The weights of every `tile` consecutive tokens are quantised on their own;
+    tile=None takes the whole context as one tile, the reference's high-precision golden (:264-270). mask as in
+    paged_attention with one query token per sequence. A sequence of length 0 takes no query row; rows never
+    written keep out_init. Returns float32 [rows, H, D]."""
+    q_int8 = np.asarray(q_int8)
+    rows, heads, d = q_int8.shape
+    kv_heads = key_cache.shape[2]
+    group = heads // kv_heads
+    out = np.full((rows, heads, d), out_init, np.float32)
+    k_descale = np.asarray(k_descale, np.float32)
+    v_descale = np.asarray(v_descale, np.float32)
+    row = 0
+    for b, ctx in enumerate(np.asarray(context_lens).tolist()):
+        if ctx == 0:
+            continue
+        keys = gather_rows(np.asarray(key_cache), block_tables[b], ctx).astype(np.int32)      # [ctx, G, D]
+        values = gather_rows(np.asarray(value_cache), block_tables[b], ctx).astype(np.int32)
+        bias = None if mask is None else _mask_slice(mask, b, ctx, heads, len(context_lens), mask_per_head)
+        step = ctx if tile is None else tile
+        for h in range(heads):
+            g = h // group
+            prod = (keys[:, g, :] @ q_int8[row, h].astype(np.int32)).astype(np.float32)       # [ctx]
+            s = prod * k_descale[h] * np.float32(scale)
+            if bias is not None:
+                s = s + np.asarray(bias[h if bias.shape[0] > 1 else 0], np.float32)
+            s = s.astype(np.float32)
+            gm = gl = go = None
+            for t0 in range(0, ctx, step):
+                st = s[t0:t0 + step]
+                hm = np.float32(st.max()) if gm is None else np.maximum(gm, np.float32(st.max()))
+                w = np.exp(st - hm).astype(np.float32) if np.isfinite(hm) else np.zeros_like(st)
+                if p_scale is None:
+                    p8, wmax = quantise_weights(w)
+                    vs = np.float32(v_descale[h] * wmax / np.float32(127.0))
+                else:
+                    p8 = np.rint((w * np.float32(p_scale[h])).astype(np.float16)).astype(np.int8)
+                    vs = v_descale[h]
+                lo = (p8.astype(np.int32) @ values[t0:t0 + step, g, :]).astype(np.float32) * vs
+                ll = np.float32(w.sum(dtype=np.float32))
+                if gm is None:
+                    gl, go = ll, lo
+                else:
+                    keep = np.float32(np.exp(gm - hm)) if np.isfinite(gm) else np.float32(0)
+                    gl, go = gl * keep + ll, go * keep + lo
+                gm = hm
+            out[row, h] = go / gl if gl > 0 else 0
+        row += 1
     return out
 
 

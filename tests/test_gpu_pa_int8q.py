@@ -1,0 +1,170 @@
+"""GPU parity of PagedAttention with int8 queries over int8 caches (quantType TYPE_QUANT_QKV_ONLINE / OFFLINE): the
+HIP kernel through the C ABI and through atb::Operation against the CPU oracle, which restates the reference golden
+(tests/apitest/kernelstest/mix/test_paged_attention_common.py:104-110,147-229,256-276) with the same tile of 128
+tokens. All integer products are exact on both sides; what differs is the order of fp32 sums and the last bit of
+exp, which now and then moves an int8 weight by one step of 127: tolerance rtol = atol = 2e-3 (fp16) / 2e-2 (bf16)
+on outputs of magnitude <= 5 * 5 / 127. Beside it the reference's own criterion (compare_cv, :716-724 with
+precision_calcu.py:111-140): against the golden that quantises the whole context as one tile, the kernel's errors
+may not exceed the tiled golden's by the factors 10 / 2 / 2."""
+import ctypes
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from pa_harness import assert_close, dtype_code, random_tables
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float16: 2e-3, torch.bfloat16: 2e-2}
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return torch.device("cuda:0")
+
+
+@pytest.fixture(scope="module")
+def stream(dev):
+    return torch.cuda.Stream(device=dev)
+
+
+def _case(seed, ctx, heads, kv_heads, d, block, dtype, mask=None, offline=False):
+    """Inputs drawn the way the reference test draws them (:444-452 uniform in [-5, 5] cast to int8, :540-543
+    descales in +-5/127, the offline factor in [0, 127]); mask: None, "norm" ([batch, 1, maxS], :500-504) or "alibi"
+    ([batch, heads, 1, maxS], :487-498)."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    ctx = np.asarray(ctx, np.int32)
+    pool = int(((ctx + block - 1) // block).sum()) + 3
+    tables = random_tables(rng, ctx, block, pool)
+    rows = int((ctx > 0).sum())
+    c = dict(
+        q8=torch.from_numpy(rng.uniform(-5, 5, size=(rows, heads, d)).astype(np.int8)),
+        k8=torch.from_numpy(rng.uniform(-5, 5, size=(pool, block, kv_heads, d)).astype(np.int8)),
+        v8=torch.from_numpy(rng.uniform(-5, 5, size=(pool, block, kv_heads, d)).astype(np.int8)),
+        kd=torch.from_numpy(rng.uniform(-5 / 127, 5 / 127, size=heads).astype(np.float32)),
+        vd=torch.from_numpy(rng.uniform(-5 / 127, 5 / 127, size=heads).astype(np.float32)),
+        ps=torch.from_numpy(rng.uniform(0, 127, size=heads).astype(np.float32)) if offline else None,
+        tables=torch.from_numpy(tables), ctx=ctx, rows=rows, heads=heads, kv_heads=kv_heads, d=d, block=block,
+        dtype=dtype, mask=None, mask_kind=mask)
+    max_len = int(ctx.max())
+    if mask == "norm":
+        m = np.zeros((len(ctx), 1, max_len), np.float32)
+        for i in range(len(ctx)):
+            m[i, :, :i] = -10000.0
+        c["mask"] = torch.from_numpy(m).to(dtype)
+    elif mask == "alibi":
+        slopes = np.array([2.0 ** (-8.0 * (i + 1) / heads) for i in range(heads)], np.float32)
+        m = np.zeros((len(ctx), heads, 1, max_len), np.float32)
+        for i, n in enumerate(ctx):
+            if n > 0:
+                m[i, :, 0, :n] = slopes[:, None] * (np.arange(n) - n + 1).astype(np.float32)[None, :]
+        c["mask"] = torch.from_numpy(m).to(dtype)
+    return c
+
+
+def _oracle(oracle, c, scale, tile):
+    return oracle.paged_attention_int8q(
+        c["q8"].numpy(), c["k8"].numpy(), c["v8"].numpy(), c["tables"].numpy(), c["ctx"], c["kd"].numpy(), c["vd"].numpy(),
+        scale, p_scale=None if c["ps"] is None else c["ps"].numpy(), tile=tile,
+        mask=None if c["mask"] is None else c["mask"].float().numpy(), mask_per_head=False, out_init=7.0)
+
+
+def int8q_cabi(binding, stream, dev, c, scale):
+    k = binding.kernels()
+    t = {n: c[n].to(dev) for n in ("q8", "k8", "v8", "tables", "kd", "vd")}
+    ps = c["ps"].to(dev) if c["ps"] is not None else None
+    mask = c["mask"].to(dev) if c["mask"] is not None else None
+    lens = np.ascontiguousarray(c["ctx"], dtype=np.int32)
+    max_len = 0 if mask is None else mask.shape[-1]
+    call = binding.AtbmiPaInt8QCall(
+        outDtype=dtype_code(binding, torch.empty(0, dtype=c["dtype"])), numHeads=c["heads"], numKvHeads=c["kv_heads"],
+        headDim=c["d"], blockSize=c["block"], numBlocks=c["k8"].shape[0], maxBlocksPerSeq=c["tables"].shape[1],
+        batch=len(lens), numQueryRows=c["rows"], offline=0 if ps is None else 1, hasMask=0 if mask is None else 1,
+        maskLen=max_len, qkScale=scale,
+        maskSeqStride=0 if mask is None else (max_len if c["mask_kind"] == "norm" else c["heads"] * max_len),
+        maskHeadStride=max_len if c["mask_kind"] == "alibi" else 0, hostContextLens=lens.ctypes.data)
+    ws_bytes = ctypes.c_uint64(0)
+    if k.atbmi_pa_int8q_workspace_size(ctypes.byref(call), ctypes.byref(ws_bytes)) != 0:
+        raise RuntimeError("pa_int8q_workspace_size: " + binding.last_kernel_error())
+    with torch.cuda.stream(stream):
+        ws = torch.empty(max(int(ws_bytes.value), 16), dtype=torch.uint8, device=dev)
+        out = torch.full((c["rows"], c["heads"], c["d"]), 7.0, dtype=c["dtype"], device=dev)
+        call.query, call.keyCache, call.valueCache = t["q8"].data_ptr(), t["k8"].data_ptr(), t["v8"].data_ptr()
+        call.blockTables, call.kDescale, call.vDescale = t["tables"].data_ptr(), t["kd"].data_ptr(), t["vd"].data_ptr()
+        call.pScale = ps.data_ptr() if ps is not None else None
+        call.mask = mask.data_ptr() if mask is not None else None
+        call.out = out.data_ptr()
+        if k.atbmi_pa_int8q_decode(ctypes.byref(call), ws.data_ptr(), ws_bytes.value, stream.cuda_stream) != 0:
+            raise RuntimeError("pa_int8q_decode: " + binding.last_kernel_error())
+    stream.synchronize()
+    return out
+
+
+def _errors(golden, x):
+    """Largest relative, mean relative and root-mean-square error (reference precision_calcu.py:78-109)."""
+    golden = np.asarray(golden, np.float32)
+    x = np.asarray(x, np.float32)
+    rel = np.abs(x - golden) / (np.abs(golden) + 1e-7)
+    return rel.max(), rel.mean(), math.sqrt(np.mean((x - golden) ** 2))
+
+
+def _double_golden(true_out, golden, got, dtype):
+    floor = 2.0 ** -11 if dtype == torch.float16 else 2.0 ** -8    # CV_FUSION thresholds (precision_calcu.py:56-62)
+    e_got, e_gold = _errors(true_out, got), _errors(true_out, golden)
+    rates = [g / max(r, floor) for g, r in zip(e_got, e_gold)]
+    return rates[0] < 10 and rates[1] < 2 and rates[2] < 2, rates
+
+
+# ctx, heads, kv heads, head size, block size, dtype, mask, offline
+# (reference :3011-3227: 9 sequences [3000, 300, 14000, 33, 65, 1, 16, 14000, 300] with 32 heads over 2 KV heads,
+# head size 128, block 128, NORM / ALIBI / no mask, bf16 and fp16 outputs, online and offline; contexts cut to keep
+# the CPU oracle within seconds)
+INT8Q_MATRIX = [
+    ([3000, 300, 1400, 33, 65, 1, 16, 0, 300], 32, 2, 128, 128, torch.bfloat16, "norm", False),
+    ([3000, 300, 1400, 33, 65, 1, 16, 1400, 300], 32, 2, 128, 128, torch.float16, "alibi", False),
+    ([700, 129, 128, 4], 32, 2, 128, 128, torch.float16, None, True),
+    ([700, 129, 128, 4], 32, 8, 128, 128, torch.bfloat16, "norm", True),
+    ([515, 33, 2048], 64, 8, 128, 128, torch.float16, None, False),       # 8 heads a KV head: half a head tile
+    ([300, 1000, 0, 77], 40, 1, 128, 64, torch.float16, None, False),     # 40 heads over one KV head: three head tiles
+    ([300, 100, 77], 8, 8, 64, 16, torch.float16, "norm", False),         # head size 64, 16-token blocks, MHA
+    ([260, 31], 12, 4, 256, 32, torch.bfloat16, None, False),             # head size 256
+]
+
+
+@pytest.mark.parametrize("case", INT8Q_MATRIX, ids=lambda c: "ctx%d_h%d_g%d_d%d_b%d_%s_%s_%s" % (
+    max(c[0]), c[1], c[2], c[3], c[4], str(c[5]).split(".")[-1], c[6], "offline" if c[7] else "online"))
+def test_int8q_kernel_against_the_oracle(binding, oracle, dev, stream, case):
+    ctx, heads, kv_heads, d, block, dtype, mask, offline = case
+    c = _case(710 + heads + d, ctx, heads, kv_heads, d, block, dtype, mask, offline)
+    scale = 1.0 / math.sqrt(d)
+    got = int8q_cabi(binding, stream, dev, c, scale)
+    want = _oracle(oracle, c, scale, 128)
+    assert_close(got, want, TOL[dtype], "tile 128")
+    # the reference's criterion: compared with the whole context as one tile, no worse than the tiled golden
+    ok, rates = _double_golden(_oracle(oracle, c, scale, None), want, got.float().cpu().numpy(), dtype)
+    assert ok, rates
+    assert float(got.float().abs().max()) > 0
+
+
+def test_int8q_rejects_what_it_cannot_run(binding, dev, stream):
+    k = binding.kernels()
+    lens = np.array([5, 300], np.int32)
+    call = binding.AtbmiPaInt8QCall(outDtype=binding.ATBMI_F16, numHeads=32, numKvHeads=8, headDim=128, blockSize=128,
+                                    numBlocks=8, maxBlocksPerSeq=2, batch=2, numQueryRows=2, qkScale=0.1,
+                                    hostContextLens=lens.ctypes.data)
+    ws = ctypes.c_uint64(0)
+    assert k.atbmi_pa_int8q_workspace_size(ctypes.byref(call), ctypes.byref(ws)) != 0        # 300 tokens in 2 blocks
+    assert "exceeds" in binding.last_kernel_error()
+    lens[1] = 200
+    assert k.atbmi_pa_int8q_workspace_size(ctypes.byref(call), ctypes.byref(ws)) == 0 and ws.value == 32
+    call.headDim = 96
+    assert k.atbmi_pa_int8q_workspace_size(ctypes.byref(call), ctypes.byref(ws)) != 0
+    call.headDim, call.numKvHeads = 128, 5
+    assert k.atbmi_pa_int8q_workspace_size(ctypes.byref(call), ctypes.byref(ws)) != 0
+    call.numKvHeads, call.numQueryRows = 8, 1
+    assert k.atbmi_pa_int8q_workspace_size(ctypes.byref(call), ctypes.byref(ws)) != 0        # two rows asked for
+    call.numQueryRows = 2
+    assert k.atbmi_pa_int8q_decode(ctypes.byref(call), None, 0, stream.cuda_stream) != 0     # null tensors

@@ -1182,6 +1182,102 @@ def test_int8_decode_limits_and_closed_forms(oracle):
     np.testing.assert_allclose(flat[0], rows.mean(0)[None, :] * pd[:, None], rtol=1e-5, atol=1e-6)
 
 
+def _int8q_case(rng, ctx, heads=4, kv_heads=2, d=64, block=16):
+    ctx = np.asarray(ctx, np.int32)
+    nblk = (ctx + block - 1) // block
+    pool = int(nblk.sum()) + 2
+    perm = rng.permutation(pool)
+    tables = np.zeros((len(ctx), max(1, int(nblk.max()))), np.int32)
+    pos = 0
+    for b in range(len(ctx)):
+        tables[b, :nblk[b]] = perm[pos:pos + nblk[b]]
+        pos += nblk[b]
+    rows = int((ctx > 0).sum())
+    q8 = rng.integers(-5, 6, size=(rows, heads, d)).astype(np.int8)
+    k8 = rng.integers(-5, 6, size=(pool, block, kv_heads, d)).astype(np.int8)
+    v8 = rng.integers(-5, 6, size=(pool, block, kv_heads, d)).astype(np.int8)
+    kd = rng.uniform(-5 / 127, 5 / 127, size=heads).astype(np.float32)
+    vd = rng.uniform(-5 / 127, 5 / 127, size=heads).astype(np.float32)
+    ps = rng.uniform(20, 127, size=heads).astype(np.float32)
+    return q8, k8, v8, tables, ctx, kd, vd, ps
+
+
+@pytest.mark.parametrize("tile,offline", [(16, False), (48, False), (None, False), (16, True), (1000, True)])
+def test_int8q_attention_matches_independent_loops(oracle, tile, offline):
+    """Token by token in Python integers and float64: descale per query head, the mask after the scale, every
+    tile's weights quantised by their own maximum (online) or by the given factor (offline)."""
+    rng = _rng(160 + (tile or 7) + int(offline))
+    heads, kv_heads, d = 4, 2, 32
+    q8, k8, v8, tables, ctx, kd, vd, ps = _int8q_case(rng, [37, 0, 5, 96], heads, kv_heads, d)
+    mask = (rng.standard_normal((4, 1, 96)) * 2).astype(np.float32)       # one row per sequence, empty ones counted
+    got = oracle.paged_attention_int8q(q8, k8, v8, tables, ctx, kd, vd, 0.11, p_scale=ps if offline else None, tile=tile,
+                                       mask=mask, mask_per_head=False, out_init=7.0)
+    assert got.shape == (3, heads, d)
+    row = 0
+    for b, n in enumerate(ctx):
+        if n == 0:
+            continue
+        for h in range(heads):
+            g = h // (heads // kv_heads)
+            s = []
+            for t in range(n):
+                blk, off = tables[b, t // 16], t % 16
+                prod = sum(int(a) * int(c) for a, c in zip(q8[row, h], k8[blk, off, g]))
+                s.append(np.float32(np.float32(np.float32(prod) * kd[h]) * np.float32(0.11)) + mask[b, 0, t])
+            s = np.array(s, np.float64)
+            step = n if tile is None else tile
+            num, den, ref = np.zeros(d), 0.0, None
+            for t0 in range(0, n, step):
+                st = s[t0:t0 + step]
+                new = st.max() if ref is None else max(ref, st.max())
+                if ref is not None:
+                    num, den = num * math.exp(ref - new), den * math.exp(ref - new)
+                ref = new
+                w = np.exp(st - ref).astype(np.float32)
+                if offline:
+                    p8, vs = np.rint((w * ps[h]).astype(np.float16)), float(vd[h])
+                else:
+                    p8 = np.rint((w / np.float32(w.max() / np.float32(127))).astype(np.float16))
+                    vs = float(vd[h]) * float(w.max()) / 127
+                for i, t in enumerate(range(t0, min(n, t0 + step))):
+                    blk, off = tables[b, t // 16], t % 16
+                    num += p8[i] * v8[blk, off, g].astype(np.float64) * vs
+                den += float(w.astype(np.float64).sum())
+            np.testing.assert_allclose(got[row, h], num / den, rtol=3e-5, atol=3e-6)
+        row += 1
+
+
+def test_int8q_attention_limits_and_closed_forms(oracle):
+    rng = _rng(170)
+    heads, kv_heads, d = 4, 2, 64
+    q8, k8, v8, tables, ctx, kd, vd, ps = _int8q_case(rng, [1, 64, 33], heads, kv_heads, d)
+    got = oracle.paged_attention_int8q(q8, k8, v8, tables, ctx, kd, vd, 0.05, tile=16)
+    group = heads // kv_heads
+    # one token: its weight is 127 of 127, the output is its value row times the head's descale
+    one = v8[tables[0, 0], 0][np.arange(heads) // group].astype(np.float32) * vd[:, None]
+    np.testing.assert_allclose(got[0], one, rtol=1e-6)
+    # 127 levels per tile: within about half a level of ordinary attention over the dequantised tensors
+    plain = oracle.paged_attention(q8.astype(np.float32) * kd[None, :, None], k8.astype(np.float32), v8.astype(np.float32),
+                                   tables, ctx, 0.05) * vd[None, :, None]
+    assert 0 < np.abs(got - plain).max() <= 0.012 * np.abs(v8).max() * np.abs(vd).max() * 4
+    # equal scores (a zero query): every weight is 127 whatever the tile, the output is the mean of the value rows;
+    # offline with a factor f the weights are f and the value descale is taken as given, so the mean comes f-fold
+    q0 = np.zeros_like(q8)
+    for kwargs, fold in (({"tile": 16}, 1), ({"tile": None}, 1), ({"tile": 16, "p_scale": np.full(heads, 100, np.float32)}, 100)):
+        flat = oracle.paged_attention_int8q(q0, k8, v8, tables, ctx, kd, vd, 0.05, **kwargs)
+        rows = v8[tables[1, np.arange(64) // 16], np.arange(64) % 16].astype(np.float64)       # [64, G, d]
+        np.testing.assert_allclose(flat[1], fold * rows.mean(0)[np.arange(heads) // group] * vd[:, None], rtol=1e-5,
+                                   atol=1e-6)
+    # one KV head, head size 512, no rotary part: the computation of the int8 MLA decode
+    q8m = rng.integers(-5, 6, size=(3, 2, 512)).astype(np.int8)
+    kvm = rng.integers(-5, 6, size=(k8.shape[0], 16, 1, 512)).astype(np.int8)
+    qd, pd = np.abs(kd[:2]) + np.float32(0.01), vd[:2]
+    zero_q, zero_k = np.zeros((3, 2, 64), np.float32), np.zeros((k8.shape[0], 16, 1, 64), np.float32)
+    a = oracle.paged_attention_int8q(q8m, kvm, kvm, tables, ctx, qd, pd, 0.05, tile=16)
+    b = oracle.mla_int8_decode(q8m, zero_q, kvm, zero_k, tables, ctx, qd, pd, 0.05, tile=16)
+    np.testing.assert_allclose(a, b, rtol=1e-6, atol=1e-7)
+
+
 def _prefill_case(rng, q_lens, kv_lens, heads, kv_heads):
     tq, tk = int(sum(q_lens)), int(sum(kv_lens))
     mk = lambda *shape: rng.standard_normal(shape).astype(np.float32)
