@@ -215,7 +215,7 @@ class AtbmiPaInt8QCall(ctypes.Structure):
     """One atbmi_pa_int8q_decode call (include/atbmi_kernels.h)."""
     _fields_ = [(n, ctypes.c_int32) for n in ("outDtype", "numHeads", "numKvHeads", "headDim", "blockSize", "numBlocks",
                                               "maxBlocksPerSeq", "batch", "numQueryRows", "offline", "hasMask",
-                                              "maskLen")] + [
+                                              "maskLen", "pieceTiles")] + [
         ("qkScale", ctypes.c_float), ("maskSeqStride", ctypes.c_int64), ("maskHeadStride", ctypes.c_int64)] + [
         (n, ctypes.c_void_p) for n in ("hostContextLens", "query", "keyCache", "valueCache", "blockTables", "kDescale",
                                        "vDescale", "pScale", "mask", "out")]

@@ -16,8 +16,9 @@
 // property of the operator.) Every integer product is exact (v_mfma_i32_16x16x64_i8; sums stay below 2^24).
 //
 // A workgroup of four waves owns one sequence, one KV head and up to 16 of its query heads and walks the context
-// tile by tile. Key and value rows of tile i + 1 are requested into registers before the arithmetic of tile i and
-// stored to LDS after it, token-major with a padded pitch.
+// tile by tile. Key and value rows of tile i + 1 are requested into registers before the arithmetic of tile i. One
+// LDS buffer (token-major, padded pitch) serves both: it holds the key rows while they are scored, then the value
+// rows of the same tile, which wait in registers until then; that keeps a workgroup at 29 KB of LDS (D = 128).
 //   scores  wave w for tokens 32 w .. 32 w + 31: S^T[token, head] = K . Q^T (K rows from LDS as A, the query
 //           resident in registers as B);
 //   softmax 16 lanes a head, 8 tokens a lane; int8 weights P[head][token] go to LDS;
@@ -25,7 +26,10 @@
 //           the transposing ds_read_b64_tr_b8, P^T as 16 consecutive bytes of a head's weights.
 // Operand layout of v_mfma_i32_16x16x64_i8: lane (n = lane % 16, kg = lane / 16) supplies the 16 contraction values
 // 16 kg .. 16 kg + 15 of row n (A) / column n (B) and receives D[4 kg + e][n], e = 0 .. 3.
-// One pass per sequence (no split over the context): the launch has batch x kvHeads x ceil(group / 16) workgroups.
+// Long contexts are cut into pieces of whole tiles, sized so that the launch has a few workgroups per place on the
+// chip; a sequence in one piece is written directly, the others leave normalised fp32 rows and natural-log
+// log-sum-exps for a merge kernel (the golden cuts and merges the same way, :171-229).
+#include <algorithm>
 #include <vector>
 #include "pa_internal.h"
 #include "upload_ring.h"
@@ -50,21 +54,33 @@ static_assert(CH == 16 && TPL == 8 && TILE == NWAVES * 32, "four waves share a t
 
 template <int D> struct Lds {
     static constexpr int PITCH = D + 16; // row pitch of the key and value tiles: 16 rows' 16-byte reads touch every bank once
-    static constexpr int K = 0;
-    static constexpr int V = K + TILE * PITCH;
-    static constexpr int S = V + TILE * PITCH;   // [16] fp32 scores
+    static constexpr int KV = 0;                 // the key rows of a tile, then (once they are scored) its value rows
+    static constexpr int S = KV + TILE * PITCH;  // [16] fp32 scores
     static constexpr int P = S + HT * S_PITCH;   // [16] int8 weights
     static constexpr int STAT = P + HT * P_PITCH; // [16] {keep, value scale, 1 / sum, -}
     static constexpr int BYTES = STAT + HT * 16;
     static_assert(BYTES <= 160 * 1024 && S % 16 == 0 && P % 16 == 0 && STAT % 16 == 0, "LDS layout");
 };
 
-// One sequence with a non-empty context: its block-table row, context length, row of query / out, mask row.
+// One piece of a sequence with a non-empty context: its block-table row, the tokens [tokBegin, tokEnd) of its
+// context (tokBegin a multiple of the tile; an empty range pads the table), row of query / out, mask row, and the
+// first of its partial rows (-1: the piece is the whole sequence and writes the output itself).
 struct Row {
     int32_t tableRow;
-    int32_t ctxLen;
+    int32_t tokBegin;
+    int32_t tokEnd;
     int32_t qRow;
     int32_t maskRow;
+    int32_t partial;
+    int32_t pad[2];
+};
+
+// A sequence that was cut: row of out, its first partial row and how many pieces it has.
+struct MergeRow {
+    int32_t qRow;
+    int32_t firstPartial;
+    int32_t numPartials;
+    int32_t pad;
 };
 
 struct Args {
@@ -78,6 +94,9 @@ struct Args {
     const void *mask;
     void *out;
     const Row *rows;
+    const MergeRow *mergeRows;
+    float *partO;   // [partial rows][kvHeads x headTiles][16 heads][D], normalised
+    float *partLse; // [partial rows][kvHeads x headTiles][16 heads]
     int64_t maskSeqStride;  // elements between the mask rows of two sequences (0: shared)
     int64_t maskHeadStride; // elements between the mask rows of two heads (0: shared)
     int32_t H;
@@ -125,44 +144,71 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
     const int kg = lane >> 4; // which 16 contraction values / 4 result rows this lane holds
     const int group = a.H / a.G;
     const int headTiles = (group + HT - 1) / HT;
-    // workgroups go round the eight XCDs: the workgroups of a sequence, whose KV heads lie side by side in the
-    // cache rows, take neighbouring places on one XCD and share its L2
+    // workgroups go round the eight XCDs: XCD x takes the x-th eighth of the row table, so the workgroups of a
+    // sequence, whose KV heads lie side by side in the cache rows, share one L2 (the host deals the sequences out to
+    // the eighths longest first, see OrderRows)
     const int work = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
-    if (work >= a.numRows * a.G * headTiles) {
-        return;
-    }
     const Row row = a.rows[work / (a.G * headTiles)];
+    if (row.tokEnd <= row.tokBegin) {
+        return; // padding of an eighth
+    }
     const int g = (work / headTiles) % a.G;
     const int ht = work % headTiles;
     const int nh = min(HT, group - ht * HT); // heads past the last one compute on zeros and store nothing
     const int h0 = g * group + ht * HT;
     const int32_t *table = a.tables + static_cast<int64_t>(row.tableRow) * a.maxBlocksPerSeq;
-    const int numTiles = (row.ctxLen + TILE - 1) / TILE;
+    const int numTiles = (row.tokEnd - row.tokBegin + TILE - 1) / TILE;
     const int64_t slotBytes = static_cast<int64_t>(a.G) * D; // one token's rows of all KV heads
 
     // ---- requests for a tile: this thread's pieces of the key and value rows (tokens past the context repeat the last one)
     const int ldTok = tid / PPR;
     const int ldPiece = tid % PPR;
+    // When a block holds whole tiles (block sizes 128, 256, ..) a tile lies in one block and its first slot is the
+    // same for the whole workgroup; otherwise every token looks its block up.
+    // In that case the block ids come from a per-lane cache of 64 table entries (lane l holds entry cacheBase + l),
+    // so that a tile's rows can be requested without waiting for a table entry first.
+    const bool wholeTiles = a.blockSize % TILE == 0;
+    const int64_t laneAt = static_cast<int64_t>(g) * D + ldPiece * 16;
+    int cacheBase = wholeTiles ? row.tokBegin / a.blockSize : 0;
+    int cachedIds = table[min(cacheBase + lane, a.maxBlocksPerSeq - 1)];
     auto requestTile = [&](int t0, u32x4(&kr)[PASSES], u32x4(&vr)[PASSES]) {
+        if (wholeTiles) {
+            const int blk = __builtin_amdgcn_readfirstlane(t0 / a.blockSize);
+            if (blk - cacheBase >= WAVE) {
+                cacheBase = blk;
+                cachedIds = table[min(cacheBase + lane, a.maxBlocksPerSeq - 1)];
+            }
+            const int id = __builtin_amdgcn_readlane(cachedIds, blk - cacheBase);
+            const int64_t first = static_cast<int64_t>(id) * a.blockSize + (t0 - blk * a.blockSize);
+            const int last = row.tokEnd - 1 - t0; // (tokens past the piece repeat its last one)
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p) {
+                const int64_t at = (first + min(p * ROWS_PER_PASS + ldTok, last)) * slotBytes + laneAt;
+                kr[p] = *reinterpret_cast<const u32x4 *>(a.k8 + at);
+                vr[p] = *reinterpret_cast<const u32x4 *>(a.v8 + at);
+            }
+            return;
+        }
 #pragma unroll
         for (int p = 0; p < PASSES; ++p) {
-            const int tok = min(t0 + p * ROWS_PER_PASS + ldTok, row.ctxLen - 1);
-            const int64_t slot = static_cast<int64_t>(table[tok / a.blockSize]) * a.blockSize + tok % a.blockSize;
-            const int64_t at = slot * slotBytes + g * D + ldPiece * 16;
+            const int tok = min(t0 + p * ROWS_PER_PASS + ldTok, row.tokEnd - 1);
+            const int blk = tok / a.blockSize;
+            const int64_t slot = static_cast<int64_t>(table[blk]) * a.blockSize + (tok - blk * a.blockSize);
+            const int64_t at = slot * slotBytes + laneAt;
             kr[p] = *reinterpret_cast<const u32x4 *>(a.k8 + at);
             vr[p] = *reinterpret_cast<const u32x4 *>(a.v8 + at);
         }
     };
-    auto storeTile = [&](const u32x4(&kr)[PASSES], const u32x4(&vr)[PASSES]) {
+    auto storeRows = [&](const u32x4(&r)[PASSES]) {
 #pragma unroll
         for (int p = 0; p < PASSES; ++p) {
-            const int at = (p * ROWS_PER_PASS + ldTok) * L::PITCH + ldPiece * 16;
-            *reinterpret_cast<u32x4 *>(smem + L::K + at) = kr[p];
-            *reinterpret_cast<u32x4 *>(smem + L::V + at) = vr[p];
+            *reinterpret_cast<u32x4 *>(smem + L::KV + (p * ROWS_PER_PASS + ldTok) * L::PITCH + ldPiece * 16) = r[p];
         }
     };
-    u32x4 kNext[PASSES], vNext[PASSES];
-    requestTile(0, kNext, vNext);
+    // the rows of tile i + 1 are on their way while tile i is worked on; the value rows of tile i wait in registers
+    // until its key rows are scored
+    u32x4 kNext[PASSES], vNext[PASSES], vCur[PASSES];
+    requestTile(row.tokBegin, kNext, vCur);
 
     // ---- Q^T as B operands: lane (n, kg) holds q8[head n][64 j + 16 kg .. + 16)
     i32x4 q8[D / 64];
@@ -196,11 +242,11 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
     for (int ct = 0; ct < CT; ++ct) {
         acc[ct] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     }
-    storeTile(kNext, vNext);
+    storeRows(kNext);
     __syncthreads();
 
     for (int i = 0; i < numTiles; ++i) {
-        const int t0 = i * TILE;
+        const int t0 = row.tokBegin + i * TILE;
         const bool more = i + 1 < numTiles;
         if (more) {
             requestTile(t0 + TILE, kNext, vNext);
@@ -214,30 +260,35 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
             if (maskRow) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    maskBits[e] = maskRow[min(tok + e, row.ctxLen - 1)];
+                    maskBits[e] = maskRow[min(tok + e, row.tokEnd - 1)];
                 }
             }
             i32x4 dot = {0, 0, 0, 0};
 #pragma unroll
             for (int j = 0; j < D / 64; ++j) {
-                const i32x4 kk = *reinterpret_cast<const i32x4 *>(smem + L::K + (tokBase + n) * L::PITCH + j * 64 + kg * 16);
+                const i32x4 kk = *reinterpret_cast<const i32x4 *>(smem + L::KV + (tokBase + n) * L::PITCH + j * 64 + kg * 16);
                 dot = __builtin_amdgcn_mfma_i32_16x16x64_i8(kk, q8[j], dot, 0, 0, 0);
             }
             f32x4 sc;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const bool live = tok + e < row.ctxLen;
                 float bias = 0.0f;
                 if (maskRow) {
                     bias = BF16 ? Bf16ToFloat(static_cast<uint16_t>(maskBits[e]))
                                 : HalfBitsToFloat(static_cast<uint16_t>(maskBits[e]));
                 }
-                const float x = static_cast<float>(dot[e]) * descale * a.qkScale + bias;
-                sc[e] = live ? x : -INFINITY;
+                sc[e] = static_cast<float>(dot[e]) * descale * a.qkScale + bias;
+            }
+            if (t0 + TILE > row.tokEnd) { // the last tile of the piece: tokens past its end weigh nothing
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    sc[e] = tok + e < row.tokEnd ? sc[e] : -INFINITY;
+                }
             }
             *reinterpret_cast<f32x4 *>(smem + L::S + n * S_PITCH + (tokBase + kg * 4) * 4) = sc;
         }
-        __syncthreads();
+        __syncthreads(); // the key rows are scored: their place takes the value rows
+        storeRows(vCur);
         // ---- weights of the tile
         {
             float w[TPL];
@@ -331,7 +382,7 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
                     // the transposing read hands lane (channel n, kg) the bytes of tokens r .. r + 7 when lane n of
                     // the group points at token r + n / 2, channels (n % 2) * 8 .. + 8
                     const unsigned char *vp =
-                        smem + L::V + (hh * 64 + kg * 16 + (n >> 1)) * L::PITCH + cb + (n & 1) * 8;
+                        smem + L::KV + (hh * 64 + kg * 16 + (n >> 1)) * L::PITCH + cb + (n & 1) * 8;
                     const i32x2 lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2 *)(vp));
                     const i32x2 hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
                         (__attribute__((address_space(3))) i32x2 *)(vp + 8 * L::PITCH));
@@ -346,18 +397,33 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
         }
         __syncthreads(); // everybody has left the tile
         if (more) {
-            storeTile(kNext, vNext);
+            storeRows(kNext);
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p) {
+                vCur[p] = vNext[p];
+            }
             __syncthreads();
         }
     }
-    // ---- the rows: acc / sum
+    // ---- the rows: acc / sum, to the output or, for a piece of a sequence, to its partial row with log(sum) + max
     if (tid % CH == 0) {
         float *stat = reinterpret_cast<float *>(smem + L::STAT) + smHead * 4;
         stat[2] = runSum > 0.0f ? 1.0f / runSum : 0.0f;
+        stat[3] = runSum > 0.0f ? __logf(runSum) + runMax : -INFINITY;
     }
     __syncthreads();
-    if (liveHead) {
-        const float inv = reinterpret_cast<const float *>(smem + L::STAT)[n * 4 + 2];
+    const float inv = reinterpret_cast<const float *>(smem + L::STAT)[n * 4 + 2];
+    if (row.partial >= 0) {
+        const int64_t slot = (static_cast<int64_t>(row.partial) * a.G + g) * headTiles + ht;
+        float *prow = a.partO + (slot * HT + n) * D + kg * 4;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            *reinterpret_cast<f32x4 *>(prow + (wave * CT + ct) * 16) = acc[ct] * inv;
+        }
+        if (tid < HT) {
+            a.partLse[slot * HT + tid] = reinterpret_cast<const float *>(smem + L::STAT)[tid * 4 + 3];
+        }
+    } else if (liveHead) {
         uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) + (static_cast<int64_t>(row.qRow) * a.H + h0 + n) * D + kg * 4;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
@@ -372,6 +438,43 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
             w.y = static_cast<uint32_t>(bits[2]) | (static_cast<uint32_t>(bits[3]) << 16);
             *reinterpret_cast<uint2 *>(orow + (wave * CT + ct) * 16) = w;
         }
+    }
+}
+
+// Joins the pieces of a cut sequence: out = sum_p exp(lse_p - L) O_p, L = log sum_p exp(lse_p) (reference golden
+// test_paged_attention_common.py:217-228). grid.x = (cut sequence, head); a thread takes channels of the row.
+constexpr int MERGE_THREADS = 128;
+template <bool BF16>
+__global__ __launch_bounds__(MERGE_THREADS) void PaInt8QMergeKernel(const Args a, int D)
+{
+    const MergeRow m = a.mergeRows[blockIdx.x / a.H];
+    const int h = blockIdx.x % a.H;
+    const int group = a.H / a.G;
+    const int headTiles = (group + HT - 1) / HT;
+    const int g = h / group;
+    const int ht = (h % group) / HT;
+    const int n = (h % group) % HT;
+    const int64_t perPartial = static_cast<int64_t>(a.G) * headTiles * HT; // head rows of one partial row
+    const int64_t first = (static_cast<int64_t>(m.firstPartial) * a.G + g) * headTiles * HT + ht * HT + n;
+    float mx = -INFINITY;
+    for (int p = 0; p < m.numPartials; ++p) {
+        mx = fmaxf(mx, a.partLse[first + p * perPartial]);
+    }
+    // (a piece a -inf mask emptied has lse == -inf and weighs nothing, even when every piece is like that)
+    auto weightOf = [mx](float v) { return v == -INFINITY ? 0.0f : __expf(v - mx); };
+    float total = 0.0f;
+    for (int p = 0; p < m.numPartials; ++p) {
+        total += weightOf(a.partLse[first + p * perPartial]);
+    }
+    const float inv = total > 0.0f ? 1.0f / total : 0.0f;
+    uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) + (static_cast<int64_t>(m.qRow) * a.H + h) * D;
+    for (int d = threadIdx.x; d < D; d += MERGE_THREADS) {
+        float acc = 0.0f;
+        for (int p = 0; p < m.numPartials; ++p) {
+            acc += weightOf(a.partLse[first + p * perPartial]) * a.partO[(first + p * perPartial) * D + d];
+        }
+        const float o = acc * inv;
+        orow[d] = BF16 ? FloatToBf16(o) : FloatToHalfBits(o);
     }
 }
 
@@ -391,7 +494,7 @@ int BuildRows(const AtbmiPaInt8QCall *c, std::vector<Row> *rows)
         return Fail(ERR_INVALID_PARAM, "pa_int8q: head size %d (64, 128 and 256 are built)", c->headDim);
     }
     if (c->batch < 0 || c->numBlocks <= 0 || c->maxBlocksPerSeq <= 0 || c->blockSize <= 0 || !(c->qkScale > 0.0f) ||
-        (c->hasMask && c->maskLen <= 0) || c->maskSeqStride < 0 || c->maskHeadStride < 0) {
+        (c->hasMask && c->maskLen <= 0) || c->maskSeqStride < 0 || c->maskHeadStride < 0 || c->pieceTiles < 0) {
         return Fail(ERR_INVALID_PARAM,
                     "pa_int8q: batch %d, %d blocks of %d tokens, %d blocks a sequence, qkScale %g, mask length %d",
                     c->batch, c->numBlocks, c->blockSize, c->maxBlocksPerSeq, c->qkScale, c->maskLen);
@@ -417,7 +520,7 @@ int BuildRows(const AtbmiPaInt8QCall *c, std::vector<Row> *rows)
             return Fail(ERR_INVALID_PARAM, "pa_int8q: more than 2^31 query rows");
         }
         if (rows) {
-            rows->push_back(Row{b, ctx, static_cast<int32_t>(qRow), b});
+            rows->push_back(Row{b, 0, ctx, static_cast<int32_t>(qRow), b, -1, {0, 0}});
         }
         ++qRow;
     }
@@ -428,7 +531,67 @@ int BuildRows(const AtbmiPaInt8QCall *c, std::vector<Row> *rows)
     return OK;
 }
 
-template <int D> int Launch(const AtbmiPaInt8QCall *call, const Args &a, int64_t grid, hipStream_t s)
+// What a call lays out in its workspace: the piece table as the kernel walks it, the table of cut sequences, and the
+// partial rows.
+struct Layout {
+    std::vector<Row> pieces;     // eight equal parts, one per XCD, padded with empty pieces
+    std::vector<MergeRow> merges;
+    int64_t numPartials = 0;     // partial rows (each holds kvHeads x headTiles x 16 head rows)
+    uint64_t mergeOffset = 0, partOOffset = 0, partLseOffset = 0, bytes = 0;
+};
+
+// Cuts the sequences into pieces of whole tiles and deals them out to the eight parts of the table in turn from the
+// longest to the shortest (every part starts with its longest piece, and the parts carry about the same number of
+// tokens). The piece length aims at four workgroups for each of the 1024 places the chip has for them (256 CUs, four
+// workgroups of this kernel each), and at no less than four tiles.
+Layout PlanPieces(const AtbmiPaInt8QCall *c, const std::vector<Row> &seqs)
+{
+    Layout lay;
+    const int64_t headTiles = (c->numHeads / c->numKvHeads + HT - 1) / HT;
+    const int64_t perPiece = static_cast<int64_t>(c->numKvHeads) * headTiles; // workgroups of one piece
+    int64_t tiles = 0;
+    for (const Row &r : seqs) {
+        tiles += (r.tokEnd + TILE - 1) / TILE;
+    }
+    const int64_t target = 4 * 1024;
+    const int64_t chunk = c->pieceTiles > 0 ? c->pieceTiles : std::max<int64_t>(4, (tiles * perPiece + target - 1) / target);
+    for (const Row &r : seqs) {
+        const int64_t n = (r.tokEnd + TILE - 1) / TILE;
+        const int64_t parts = (n + chunk - 1) / chunk;
+        const int64_t each = (n + parts - 1) / parts;
+        if (parts > 1) {
+            lay.merges.push_back(MergeRow{r.qRow, static_cast<int32_t>(lay.numPartials), 0, 0});
+        }
+        for (int64_t i = 0; i * each < n; ++i) {
+            Row piece = r;
+            piece.tokBegin = static_cast<int32_t>(i * each * TILE);
+            piece.tokEnd = static_cast<int32_t>(std::min<int64_t>(r.tokEnd, (i + 1) * each * TILE));
+            piece.partial = parts > 1 ? static_cast<int32_t>(lay.numPartials++) : -1;
+            if (parts > 1) {
+                ++lay.merges.back().numPartials;
+            }
+            lay.pieces.push_back(piece);
+        }
+    }
+    std::stable_sort(lay.pieces.begin(), lay.pieces.end(), [](const Row &x, const Row &y) {
+        return x.tokEnd - x.tokBegin > y.tokEnd - y.tokBegin;
+    });
+    const size_t each = (lay.pieces.size() + 7) / 8;
+    std::vector<Row> table(each * 8, Row{0, 0, 0, 0, 0, -1, {0, 0}});
+    for (size_t i = 0; i < lay.pieces.size(); ++i) {
+        table[(i % 8) * each + i / 8] = lay.pieces[i];
+    }
+    lay.pieces.swap(table);
+    auto align = [](uint64_t v) { return (v + 255) / 256 * 256; };
+    lay.mergeOffset = align(lay.pieces.size() * sizeof(Row));
+    lay.partOOffset = align(lay.mergeOffset + lay.merges.size() * sizeof(MergeRow));
+    const uint64_t headRows = static_cast<uint64_t>(lay.numPartials) * perPiece * HT;
+    lay.partLseOffset = align(lay.partOOffset + headRows * c->headDim * sizeof(float));
+    lay.bytes = lay.partLseOffset + headRows * sizeof(float);
+    return lay;
+}
+
+template <int D> int Launch(const AtbmiPaInt8QCall *call, const Args &a, int64_t grid, int64_t numMerges, hipStream_t s)
 {
     const bool bf16 = call->outDtype == ATBMI_BF16;
     const bool offline = call->offline != 0;
@@ -446,7 +609,19 @@ template <int D> int Launch(const AtbmiPaInt8QCall *call, const Args &a, int64_t
     kernel<<<static_cast<unsigned>(grid), THREADS, Lds<D>::BYTES, s>>>(a);
     ATBMI_HIP_CHECK(hipGetLastError());
     rc = TimedLaunchKernelDone(s, timed);
-    return rc != OK ? rc : TimedLaunchEnd(s, timed, false);
+    if (rc != OK) {
+        return rc;
+    }
+    if (numMerges > 0) {
+        const unsigned mergeGrid = static_cast<unsigned>(numMerges * a.H);
+        if (bf16) {
+            PaInt8QMergeKernel<true><<<mergeGrid, MERGE_THREADS, 0, s>>>(a, D);
+        } else {
+            PaInt8QMergeKernel<false><<<mergeGrid, MERGE_THREADS, 0, s>>>(a, D);
+        }
+        ATBMI_HIP_CHECK(hipGetLastError());
+    }
+    return TimedLaunchEnd(s, timed, numMerges > 0);
 }
 
 } // namespace int8q
@@ -464,7 +639,7 @@ extern "C" int atbmi_pa_int8q_workspace_size(const AtbmiPaInt8QCall *call, uint6
     if (rc != OK) {
         return rc;
     }
-    *bytes = rows.size() * sizeof(int8q::Row);
+    *bytes = int8q::PlanPieces(call, rows).bytes;
     return OK;
 }
 
@@ -483,19 +658,23 @@ extern "C" int atbmi_pa_int8q_decode(const AtbmiPaInt8QCall *call, void *workspa
         !call->vDescale || !call->out || (call->hasMask && !call->mask) || (call->offline && !call->pScale)) {
         return Fail(ERR_INVALID_PARAM, "pa_int8q: null tensor pointer");
     }
-    const size_t bytes = rows.size() * sizeof(int8q::Row);
-    if (!workspaceDevice || workspaceBytes < bytes) {
+    const int8q::Layout lay = int8q::PlanPieces(call, rows);
+    if (!workspaceDevice || workspaceBytes < lay.bytes) {
         return Fail(ERR_INVALID_PARAM, "pa_int8q: workspace of %llu bytes, %llu needed", (unsigned long long)workspaceBytes,
-                    (unsigned long long)bytes);
+                    (unsigned long long)lay.bytes);
     }
     const int group = call->numHeads / call->numKvHeads;
     const int headTiles = (group + int8q::HT - 1) / int8q::HT;
-    const int64_t grid = (static_cast<int64_t>(rows.size()) * call->numKvHeads * headTiles + 7) / 8 * 8;
-    if (grid > 0x7fffffffLL) {
+    const int64_t grid = static_cast<int64_t>(lay.pieces.size()) * call->numKvHeads * headTiles; // (a multiple of 8)
+    if (grid > 0x7fffffffLL || static_cast<int64_t>(lay.merges.size()) * call->numHeads > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "pa_int8q: %lld workgroups", (long long)grid);
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    rc = UploadTable(rows.data(), bytes, workspaceDevice, s);
+    unsigned char *ws = static_cast<unsigned char *>(workspaceDevice);
+    rc = UploadTable(lay.pieces.data(), lay.pieces.size() * sizeof(int8q::Row), ws, s);
+    if (rc == OK && !lay.merges.empty()) {
+        rc = UploadTable(lay.merges.data(), lay.merges.size() * sizeof(int8q::MergeRow), ws + lay.mergeOffset, s);
+    }
     if (rc != OK) {
         return rc;
     }
@@ -509,18 +688,21 @@ extern "C" int atbmi_pa_int8q_decode(const AtbmiPaInt8QCall *call, void *workspa
     a.pScale = call->offline ? call->pScale : nullptr;
     a.mask = call->hasMask ? call->mask : nullptr;
     a.out = call->out;
-    a.rows = static_cast<const int8q::Row *>(workspaceDevice);
+    a.rows = reinterpret_cast<const int8q::Row *>(ws);
+    a.mergeRows = reinterpret_cast<const int8q::MergeRow *>(ws + lay.mergeOffset);
+    a.partO = reinterpret_cast<float *>(ws + lay.partOOffset);
+    a.partLse = reinterpret_cast<float *>(ws + lay.partLseOffset);
     a.maskSeqStride = call->maskSeqStride;
     a.maskHeadStride = call->maskHeadStride;
     a.H = call->numHeads;
     a.G = call->numKvHeads;
-    a.numRows = static_cast<int32_t>(rows.size());
+    a.numRows = static_cast<int32_t>(lay.pieces.size());
     a.maxBlocksPerSeq = call->maxBlocksPerSeq;
     a.blockSize = call->blockSize;
     a.qkScale = call->qkScale;
     switch (call->headDim) {
-        case 64: return int8q::Launch<64>(call, a, grid, s);
-        case 128: return int8q::Launch<128>(call, a, grid, s);
-        default: return int8q::Launch<256>(call, a, grid, s);
+        case 64: return int8q::Launch<64>(call, a, grid, static_cast<int64_t>(lay.merges.size()), s);
+        case 128: return int8q::Launch<128>(call, a, grid, static_cast<int64_t>(lay.merges.size()), s);
+        default: return int8q::Launch<256>(call, a, grid, static_cast<int64_t>(lay.merges.size()), s);
     }
 }

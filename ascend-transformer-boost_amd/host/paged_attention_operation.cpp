@@ -17,7 +17,8 @@
 // input; per-sequence LogN scaling; several query tokens per sequence
 // (CALC_TYPE_SPEC) with the SPEC or the square NORM mask; head-major (BNSD)
 // caches; head compression with its per-slot score offsets.
-// int8 queries (QKV quant) are legal in the reference but not implemented
+// int8 queries over int8 caches (quantType QKV online / offline) run on a kernel of their own
+// (csrc/pa_int8q.hip); combined with the MLA cache they are legal in the reference but not implemented
 // here; such params are rejected at creation with ERROR_INVALID_PARAM.
 // MASK_TYPE_MASK_FREE can be created and fails InferShape / Setup with
 // ERROR_INVALID_TENSOR_DIM, as the reference does off Atlas 300I Duo.
@@ -141,9 +142,10 @@ bool FeatureParamCheck(const Param &p)
 bool ImplementedCheck(const Param &p)
 {
     const char *what = nullptr;
-    if (p.quantType == Param::TYPE_QUANT_QKV_OFFLINE || p.quantType == Param::TYPE_QUANT_QKV_ONLINE) {
-        what = "int8 query quantisation";
-    } else if (p.quantType != Param::TYPE_QUANT_UNQUANT && p.quantType != Param::TYPE_DEQUANT_FUSION) {
+    if ((p.quantType == Param::TYPE_QUANT_QKV_OFFLINE || p.quantType == Param::TYPE_QUANT_QKV_ONLINE) &&
+        p.mlaVHeadSize > 0) {
+        what = "int8 query quantisation over the MLA cache";
+    } else if (p.quantType < Param::TYPE_QUANT_UNQUANT || p.quantType > Param::TYPE_QUANT_QKV_ONLINE) {
         what = "this quantType";
     }
     if (what) {
@@ -198,9 +200,37 @@ IrCombo MakeCombo(const Param &p, aclDataType q, aclDataType descale)
     return c;
 }
 
+// int8 query, keys and values; the mask and the output in outDataType; one fp32 descale per query head for the
+// scores and one for the values, offline also the factor of the weights (reference ops_configs/atb_ops_info.ini,
+// sections PagedAttentionOperationQKVQuantOnline.. / ..Offline.., their int8 columns; inputs :429-436).
+IrCombo MakeQkvCombo(const Param &p, aclDataType o)
+{
+    IrCombo c;
+    c.inDtypes = {ACL_INT8, ACL_INT8, ACL_INT8, ACL_INT32, ACL_INT32};
+    if (p.maskType != Param::UNDEFINED) {
+        c.inDtypes.push_back(o);
+    }
+    if (p.batchRunStatusEnable) {
+        c.inDtypes.push_back(ACL_INT32);
+    }
+    c.inDtypes.push_back(ACL_FLOAT);
+    c.inDtypes.push_back(ACL_FLOAT);
+    if (p.quantType == Param::TYPE_QUANT_QKV_OFFLINE) {
+        c.inDtypes.push_back(ACL_FLOAT);
+    }
+    c.inFormats.assign(c.inDtypes.size(), ACL_FORMAT_ND);
+    c.outDtypes = {o};
+    c.outFormats = {ACL_FORMAT_ND};
+    return c;
+}
+
 OpIr MakeIr(const Param &p)
 {
     OpIr ir;
+    if (p.quantType == Param::TYPE_QUANT_QKV_OFFLINE || p.quantType == Param::TYPE_QUANT_QKV_ONLINE) {
+        ir.push_back(MakeQkvCombo(p, p.outDataType));
+        return ir;
+    }
     for (aclDataType q : {ACL_FLOAT16, ACL_BF16}) {
         ir.push_back(MakeCombo(p, q, ACL_FLOAT));
         if (p.quantType == Param::TYPE_DEQUANT_FUSION) {
@@ -216,6 +246,7 @@ public:
         : OperationBase("PagedAttentionOperation"), param_(param), mla_(param.mlaVHeadSize > 0),
           dequant_(param.quantType == Param::TYPE_DEQUANT_FUSION), bnsd_(param.inputLayout == infer::TYPE_BNSD),
           compress_(param.compressType != Param::COMPRESS_TYPE_UNDEFINED),
+          qkv_(param.quantType == Param::TYPE_QUANT_QKV_OFFLINE || param.quantType == Param::TYPE_QUANT_QKV_ONLINE),
           irTable_(MakeIr(param))
     {
         ir_ = &irTable_;
@@ -241,8 +272,16 @@ public:
                 vOffsetIdx_ = next++;
             }
         }
+        if (qkv_) {
+            // reference paged_attention_ops_runner.cpp:118-131: kDescale, vDescale, then (offline) pScale
+            kScaleIdx_ = next++;
+            vScaleIdx_ = next++;
+        }
         if (param.compressType == Param::COMPRESS_TYPE_KVHEAD_ROPE) {
             razorIdx_ = next++;
+        }
+        if (param.quantType == Param::TYPE_QUANT_QKV_OFFLINE) {
+            pScaleIdx_ = next++;
         }
         if (param.scaleType == Param::SCALE_TYPE_LOGN) {
             logNIdx_ = next++;
@@ -264,6 +303,9 @@ protected:
     Status InferShapeImpl(const SVector<TensorDesc> &in, SVector<TensorDesc> &out) const override
     {
         out.at(0) = in.at(0);
+        if (qkv_) {
+            out.at(0).dtype = param_.outDataType; // reference :455-459
+        }
         const int64_t dv = mla_ ? static_cast<int64_t>(param_.mlaVHeadSize)
                                 : in.at(2).shape.dims[in.at(2).shape.dimNum - 1];
         out.at(0).shape.dims[out.at(0).shape.dimNum - 1] = dv;
@@ -478,6 +520,9 @@ protected:
                 return st;
             }
         }
+        if (qkv_) {
+            return PlanQkv(pack, maskBatchStride, maskHeadStride, maskLen, workspaceSize);
+        }
         const int32_t *queryLens = nullptr;
         if (qLensIdx_ != NONE) {
             // reference param.cpp:96-110: the query lengths are read on the host, one per sequence
@@ -550,6 +595,14 @@ protected:
     Status LaunchImpl(const VariantPack &pack, uint8_t *workspace, uint64_t workspaceSize,
                       aclrtStream stream) override
     {
+        if (qkv_) {
+            AtbmiPaInt8QCall call = MakeQkvCall(pack);
+            int rc = atbmi_pa_int8q_decode(&call, workspace, workspaceSize, stream);
+            if (rc != 0) {
+                ATB_LOG(ERROR) << "PagedAttention launch failed: " << atbmi_last_error();
+            }
+            return rc;
+        }
         AtbmiPaTensors t{};
         t.query = pack.inTensors.at(0).deviceData;
         t.keyCache = pack.inTensors.at(1).deviceData;
@@ -581,6 +634,72 @@ protected:
     }
 
 private:
+    // int8 queries: the kernel-library checks of the reference (src/kernels/mixkernels/pagedattention/
+    // paged_attention_operation.cpp:357-403: one descale per query head, fp32) and the call of the kernel layer.
+    Status PlanQkv(const VariantPack &pack, int64_t maskSeqStride, int64_t maskHeadStride, int64_t maskLen,
+                   uint64_t &workspaceSize)
+    {
+        const int64_t d = pack.inTensors.at(1).desc.shape.dims[3];
+        if (d != 64 && d != 128 && d != 256) {
+            ATB_LOG(ERROR) << "int8 queries: head size " << d << " (64, 128 and 256 are built)";
+            return ERROR_INVALID_PARAM;
+        }
+        for (size_t idx : {kScaleIdx_, vScaleIdx_, pScaleIdx_}) {
+            if (idx == NONE) {
+                continue;
+            }
+            const Dims &shape = pack.inTensors.at(idx).desc.shape;
+            if (shape.dimNum != 1 || shape.dims[0] != param_.headNum) {
+                ATB_LOG(ERROR) << "int8 queries: kDescale, vDescale and pScale should be [headNum]";
+                return ERROR_INVALID_PARAM;
+            }
+        }
+        qkvMaskSeqStride_ = maskSeqStride;
+        qkvMaskHeadStride_ = maskHeadStride;
+        qkvMaskLen_ = maskLen;
+        AtbmiPaInt8QCall call = MakeQkvCall(pack);
+        int rc = atbmi_pa_int8q_workspace_size(&call, &workspaceSize);
+        if (rc != 0) {
+            ATB_LOG(ERROR) << "PagedAttention plan: " << atbmi_last_error();
+        }
+        return rc;
+    }
+
+    AtbmiPaInt8QCall MakeQkvCall(const VariantPack &pack) const
+    {
+        const Tensor &q = pack.inTensors.at(0);
+        const Tensor &kc = pack.inTensors.at(1);
+        const Tensor &tables = pack.inTensors.at(tablesIdx_);
+        const Tensor &lens = pack.inTensors.at(lensIdx_);
+        AtbmiPaInt8QCall c{};
+        c.outDtype = param_.outDataType == ACL_BF16 ? ATBMI_BF16 : ATBMI_F16;
+        c.numHeads = param_.headNum;
+        c.numKvHeads = param_.kvHeadNum > 0 ? param_.kvHeadNum : param_.headNum;
+        c.headDim = static_cast<int32_t>(kc.desc.shape.dims[3]);
+        c.blockSize = static_cast<int32_t>(kc.desc.shape.dims[1]);
+        c.numBlocks = static_cast<int32_t>(kc.desc.shape.dims[0]);
+        c.maxBlocksPerSeq = static_cast<int32_t>(tables.desc.shape.dims[1]);
+        c.batch = static_cast<int32_t>(lens.desc.shape.dims[0]);
+        c.numQueryRows = static_cast<int32_t>(q.desc.shape.dims[0]);
+        c.offline = param_.quantType == Param::TYPE_QUANT_QKV_OFFLINE ? 1 : 0;
+        c.hasMask = maskIdx_ != NONE ? 1 : 0;
+        c.maskLen = static_cast<int32_t>(qkvMaskLen_);
+        c.qkScale = param_.qkScale;
+        c.maskSeqStride = qkvMaskSeqStride_;
+        c.maskHeadStride = qkvMaskHeadStride_;
+        c.hostContextLens = static_cast<const int32_t *>(lens.hostData);
+        c.query = q.deviceData;
+        c.keyCache = kc.deviceData;
+        c.valueCache = pack.inTensors.at(2).deviceData;
+        c.blockTables = static_cast<const int32_t *>(tables.deviceData);
+        c.kDescale = static_cast<const float *>(pack.inTensors.at(kScaleIdx_).deviceData);
+        c.vDescale = static_cast<const float *>(pack.inTensors.at(vScaleIdx_).deviceData);
+        c.pScale = pScaleIdx_ != NONE ? static_cast<const float *>(pack.inTensors.at(pScaleIdx_).deviceData) : nullptr;
+        c.mask = maskIdx_ != NONE ? pack.inTensors.at(maskIdx_).deviceData : nullptr;
+        c.out = pack.outTensors.at(0).deviceData;
+        return c;
+    }
+
     static bool SameShape(const AtbmiPaShape &a, const AtbmiPaShape &b)
     {
         return a.qDtype == b.qDtype && a.kvDtype == b.kvDtype && a.numHeads == b.numHeads &&
@@ -712,7 +831,7 @@ private:
             return ERROR_INVALID_TENSOR_DIM;
         }
         const int64_t blockSize = in.at(1).shape.dims[1];
-        const bool strict = dequant_ || (param_.calcType == Param::CALC_TYPE_SPEC && !mla_) ||
+        const bool strict = dequant_ || qkv_ || (param_.calcType == Param::CALC_TYPE_SPEC && !mla_) ||
                             param_.scaleType == Param::SCALE_TYPE_LOGN || compress_;
         if (strict) {
             // strict regime (reference :561-572): features that predate the split K/V head sizes
@@ -757,6 +876,7 @@ private:
     bool dequant_;
     bool bnsd_;
     bool compress_; // every (sequence, KV head) pair comes with its own context length and block-table row
+    bool qkv_;      // int8 queries over int8 caches (quantType QKV online / offline)
     OpIr irTable_;
     static constexpr size_t NONE = ~static_cast<size_t>(0);
     size_t razorIdx_ = NONE;
@@ -770,6 +890,10 @@ private:
     size_t vOffsetIdx_ = NONE;
     size_t logNIdx_ = NONE;
     size_t qLensIdx_ = NONE;
+    size_t pScaleIdx_ = NONE;
+    int64_t qkvMaskSeqStride_ = 0;
+    int64_t qkvMaskHeadStride_ = 0;
+    int64_t qkvMaskLen_ = 0;
     uint32_t inputNum_ = 5;
     AtbmiPaPlan *plan_ = nullptr;
     AtbmiPaShape planShape_{};

@@ -44,8 +44,10 @@ CONFIGS["c2_bnsd"] = dict(CONFIGS["c2"], bnsd=True)
 CONFIGS["c5_split"] = dict(CONFIGS["c5"], split=True)
 CONFIGS["c5_nz"] = dict(CONFIGS["c5"], split=True, nz=True)
 CONFIGS["c5_int8"] = dict(CONFIGS["c5"], split=True, nz=True, int8nz=True)
+# C3 with int8 queries as well (PagedAttentionParam quantType QKV online): the same int8 caches, one descale per query head
+CONFIGS["c3_int8q"] = dict(CONFIGS["c3"], int8q=True)
 
-SEEDS = {"c1": 1001, "c2": 1002, "c2_fp16": 1002, "c2_alibi": 1002, "c2_norm": 1002, "c2_mtp4": 1002, "c2_bnsd": 1002, "c3": 1003, "c4": 1004, "c5": 1005, "c5_split": 1005, "c5_nz": 1005, "c5_int8": 1005}
+SEEDS = {"c1": 1001, "c2": 1002, "c2_fp16": 1002, "c2_alibi": 1002, "c2_norm": 1002, "c2_mtp4": 1002, "c2_bnsd": 1002, "c3": 1003, "c4": 1004, "c5": 1005, "c5_split": 1005, "c5_nz": 1005, "c5_int8": 1005, "c3_int8q": 1003}
 
 
 def config(name, **overrides):
@@ -208,6 +210,8 @@ def algorithmic_bytes(cfg, ctx):
     n = int(cfg.get("q_len", 1))
     rows = int((ctx > 0).sum()) * n
     total = int(ctx.sum()) * per_tok + rows * h * (d + dv) * 2
+    if cfg.get("int8q"):  # int8 query rows, 16-bit output rows, two descales per query head instead of per channel
+        total = int(ctx.sum()) * per_tok + rows * h * (d + dv * 2) + 2 * h * 4 - g * (d + dv) * 4
     if cfg.get("int8nz"):  # 512 int8 + 64 16-bit channels per cache row; 512 int8 + 64 16-bit per query row and head
         total = int(ctx.sum()) * (512 + 64 * 2) + rows * h * (512 + 64 * 2 + dv * 2) + 2 * h * 4
     total += int(((ctx + bs - 1) // bs).sum()) * 4 + len(ctx) * 4

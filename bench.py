@@ -82,6 +82,9 @@ DESCRIPTIONS = {
     "c2_mtp4": "C2 with 4 query tokens per sequence (CALC_TYPE_SPEC, MASK_TYPE_SPEC mask [256, maxS]): batch 64, "
                "32 q heads, 8 kv heads, d128, block 128, ctx U[1024,4096], bf16",
     "c3": "C3 int8-KV 70B-shaped decode: batch 128, 64 q heads, 8 kv heads, d128, block 128, ctx U[2048,8192], fp16 q",
+    "c3_int8q": "C3 with int8 queries (quantType TYPE_QUANT_QKV_ONLINE: int8 q, k, v, one descale per query head; random "
+                "int8 contents), attention only: batch 128, 64 q heads, 8 kv heads, d128, block 128, ctx U[2048,8192], "
+                "fp16 out",
     "c4": "C4 skewed long-context fp16 decode: batch 16, 32 q heads, 8 kv heads, d128, ctx lognormal(median 8k) in [256,32768]",
     "c5_split": "C5 through MultiLatentAttentionOperation (cacheMode KROPE_CTKV: 512 latent + 64 rotary channels in "
                 "two caches): batch 64, 128 q heads, block 128, ctx U[2048,4096], bf16",
@@ -174,12 +177,14 @@ def run_workload(pkg, name, steps, warmup, attention_only=False, kernel_events=T
     mask_type = {None: 0, "norm": 1, "alibi": 2, "spec": 3}[cfg.get("mask")]
     q_len = int(cfg.get("q_len", 1))
     rows = cfg["batch"] * q_len  # query tokens of one step
+    int8q = bool(cfg.get("int8q"))
     pa_param = b.PagedAttentionParam(headNum=cfg["heads"], kvHeadNum=cfg["kv_heads"], qkScale=scale,
-                                     quantType=1 if int8 else 0, mlaVHeadSize=cfg["dv"] if mla else 0,
+                                     quantType=3 if int8q else (1 if int8 else 0),
+                                     outDataType=b.ACL_FLOAT16 if int8q else 0, mlaVHeadSize=cfg["dv"] if mla else 0,
                                      maskType=mask_type, calcType=1 if q_len > 1 else 0,
                                      inputLayout=1 if cfg.get("bnsd") else 0)
     nz = bool(cfg.get("nz"))
-    if cfg.get("bnsd") or nz:
+    if cfg.get("bnsd") or nz or int8q:
         attention_only = True
     split = bool(cfg.get("split"))
     if split:
@@ -235,7 +240,10 @@ def run_workload(pkg, name, steps, warmup, attention_only=False, kernel_events=T
             if q_len > 1:
                 host_inputs[len(pa_in)] = step["q_lens"]
                 pa_in.append(step["q_lens"].to(dev))
-            if int8:
+            if int8q:
+                pa_in[0] = torch.randint(-5, 6, tuple(step["q"].shape), dtype=torch.int8, device=dev)
+                pa_in += [torch.rand(cfg["heads"], device=dev) * 0.04 + 0.001 for _ in range(2)]
+            elif int8:
                 pa_in += [step["k_scale"], step["v_scale"]]
             else:
                 rac = b.OperationRunner("ReshapeAndCacheOperation", b.ReshapeAndCacheParam(), ctx)

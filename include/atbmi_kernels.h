@@ -531,7 +531,10 @@ int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspaceDevice, u
  *               the scaled scores
  *   out         16-bit [numQueryRows, numHeads, headDim]
  * One query token per sequence; a sequence of length 0 takes no query row. headDim is 64, 128 or 256; pScale is
- * expected to keep w x pScale within 127, as the reference's own generator does. The lengths are a host array, read
+ * expected to keep w x pScale within 127, as the reference's own generator does. Long contexts are cut into pieces
+ * that are worked on side by side and merged, as the reference's kernel and golden do (:171-229); offline the weights
+ * are taken against the running maximum, which starts anew in every piece, so the result depends on the cut in its
+ * last digits (pieceTiles fixes it). The lengths are a host array, read
  * during the call.
  */
 typedef struct AtbmiPaInt8QCall {
@@ -547,6 +550,8 @@ typedef struct AtbmiPaInt8QCall {
     int32_t offline;           /* 0: weights quantised against the tile's maximum; 1: with pScale */
     int32_t hasMask;
     int32_t maskLen;           /* positions a mask row covers, >= every context length */
+    int32_t pieceTiles;        /* 0: the library chooses; c > 0: a context of n tiles of 128 tokens is cut into
+                                  ceil(n / c) pieces of ceil(n / pieces) tiles, merged by their log-sum-exps */
     float qkScale;
     int64_t maskSeqStride;
     int64_t maskHeadStride;
@@ -562,9 +567,11 @@ typedef struct AtbmiPaInt8QCall {
     void *out;
 } AtbmiPaInt8QCall;
 
-/* Validates the call (pointers aside) and reports the device workspace it needs (16 bytes per sequence). */
+/* Validates the call (pointers aside) and reports the device workspace it needs: the table of context pieces
+ * (32 bytes each) and, for sequences cut into several pieces, their fp32 partial rows. */
 int atbmi_pa_int8q_workspace_size(const AtbmiPaInt8QCall *call, uint64_t *bytes);
-/* Uploads the sequence list into the workspace and launches the kernel on `stream`; does not wait. */
+/* Uploads the tables into the workspace and launches the kernel (and the merge of cut sequences) on `stream`;
+ * does not wait. */
 int atbmi_pa_int8q_decode(const AtbmiPaInt8QCall *call, void *workspaceDevice, uint64_t workspaceBytes, void *stream);
 
 /*

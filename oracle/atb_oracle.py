@@ -812,19 +812,23 @@ def mla_int8_decode(q_int8, q_rope, kv_int8, k_rope, block_tables, context_lens,
 
 
 def paged_attention_int8q(q_int8, key_cache, value_cache, block_tables, context_lens, k_descale, v_descale, scale,
-                          p_scale=None, tile=128, mask=None, mask_per_head=None, out_init=0.0):
+                          p_scale=None, tile=128, mask=None, mask_per_head=None, out_init=0.0, piece_tiles=None):
     """Decode attention with int8 queries over int8 caches (PagedAttentionParam quantType QKV online / offline;
     reference golden tests/apitest/kernelstest/mix/test_paged_attention_common.py:104-110 (exact int32 products
     times a descale per QUERY head), :256-263 (then the scale, then the mask), :147-168 (softmax_quant_numpy: weights
     exp(s - running max); online they are quantised against the tile's largest weight, rint(fp16(w / (wmax / 127)))
     with value descale v_descale * wmax / 127; offline with the given factor, rint(fp16(w * p_scale[h])) with value
     descale v_descale), :171-216 (tiles joined by the usual online rescaling, the denominator adds up the
-    unquantised weights)).
+    unquantised weights), :176-229 (the context cut into pieces that start from scratch and are joined by their
+    log-sum-exps: out = sum_p exp(lse_p - L) out_p, L = log sum_p exp(lse_p)).
     q_int8 [rows, H, D] int8; key_cache / value_cache [blocks, block_size, G, D] int8; k_descale, v_descale, p_scale
     [H] float32 (p_scale None: online). The weights of every `tile` consecutive tokens are quantised on their own;
-    tile=None takes the whole context as one tile, the reference's high-precision golden (:264-270). mask as in
-    paged_attention with one query token per sequence. A sequence of length 0 takes no query row; rows never
-    written keep out_init. Returns float32 [rows, H, D]."""
+    tile=None takes the whole context as one tile, the reference's high-precision golden (:264-270). piece_tiles = c
+    cuts a context of n tiles into ceil(n / c) pieces of ceil(n / pieces) tiles each. (Online the cut changes nothing
+    but the order of a few fp32 operations; offline the weights are taken against the running maximum, which starts
+    anew in every piece, so the int8 weights themselves depend on the cut.) mask as in paged_attention with one query
+    token per sequence. A sequence of length 0 takes no query row; rows never written keep out_init. Returns float32
+    [rows, H, D]."""
     q_int8 = np.asarray(q_int8)
     rows, heads, d = q_int8.shape
     kv_heads = key_cache.shape[2]
@@ -840,6 +844,12 @@ def paged_attention_int8q(q_int8, key_cache, value_cache, block_tables, context_
         values = gather_rows(np.asarray(value_cache), block_tables[b], ctx).astype(np.int32)
         bias = None if mask is None else _mask_slice(mask, b, ctx, heads, len(context_lens), mask_per_head)
         step = ctx if tile is None else tile
+        bounds = [0, ctx]
+        if piece_tiles is not None and tile is not None:
+            n = (ctx + tile - 1) // tile
+            parts = (n + piece_tiles - 1) // piece_tiles
+            each = (n + parts - 1) // parts
+            bounds = [min(ctx, i * each * tile) for i in range(parts)] + [ctx]
         for h in range(heads):
             g = h // group
             prod = (keys[:, g, :] @ q_int8[row, h].astype(np.int32)).astype(np.float32)       # [ctx]
@@ -847,26 +857,38 @@ def paged_attention_int8q(q_int8, key_cache, value_cache, block_tables, context_
             if bias is not None:
                 s = s + np.asarray(bias[h if bias.shape[0] > 1 else 0], np.float32)
             s = s.astype(np.float32)
-            gm = gl = go = None
-            for t0 in range(0, ctx, step):
-                st = s[t0:t0 + step]
-                hm = np.float32(st.max()) if gm is None else np.maximum(gm, np.float32(st.max()))
-                w = np.exp(st - hm).astype(np.float32) if np.isfinite(hm) else np.zeros_like(st)
-                if p_scale is None:
-                    p8, wmax = quantise_weights(w)
-                    vs = np.float32(v_descale[h] * wmax / np.float32(127.0))
-                else:
-                    p8 = np.rint((w * np.float32(p_scale[h])).astype(np.float16)).astype(np.int8)
-                    vs = v_descale[h]
-                lo = (p8.astype(np.int32) @ values[t0:t0 + step, g, :]).astype(np.float32) * vs
-                ll = np.float32(w.sum(dtype=np.float32))
-                if gm is None:
-                    gl, go = ll, lo
-                else:
-                    keep = np.float32(np.exp(gm - hm)) if np.isfinite(gm) else np.float32(0)
-                    gl, go = gl * keep + ll, go * keep + lo
-                gm = hm
-            out[row, h] = go / gl if gl > 0 else 0
+            outs, lses = [], []
+            for lo_tok, hi_tok in zip(bounds[:-1], bounds[1:]):
+                gm = gl = go = None
+                for t0 in range(lo_tok, hi_tok, step):
+                    st = s[t0:min(t0 + step, hi_tok)]
+                    hm = np.float32(st.max()) if gm is None else np.maximum(gm, np.float32(st.max()))
+                    w = np.exp(st - hm).astype(np.float32) if np.isfinite(hm) else np.zeros_like(st)
+                    if p_scale is None:
+                        p8, wmax = quantise_weights(w)
+                        vs = np.float32(v_descale[h] * wmax / np.float32(127.0))
+                    else:
+                        p8 = np.rint((w * np.float32(p_scale[h])).astype(np.float16)).astype(np.int8)
+                        vs = v_descale[h]
+                    lo = (p8.astype(np.int32) @ values[t0:t0 + len(st), g, :]).astype(np.float32) * vs
+                    ll = np.float32(w.sum(dtype=np.float32))
+                    if gm is None:
+                        gl, go = ll, lo
+                    else:
+                        keep = np.float32(np.exp(gm - hm)) if np.isfinite(gm) else np.float32(0)
+                        gl, go = gl * keep + ll, go * keep + lo
+                    gm = hm
+                outs.append(go / gl if gl > 0 else np.zeros(d, np.float32))
+                lses.append(np.float32(np.log(gl) + gm) if gl > 0 else np.float32(-np.inf))
+            if len(outs) == 1:
+                out[row, h] = outs[0]
+            else:
+                lses = np.array(lses, np.float32)
+                top = lses.max()
+                wts = np.where(np.isfinite(lses), np.exp(lses - top), 0).astype(np.float32) if np.isfinite(top) \
+                    else np.zeros_like(lses)
+                total = np.float32(wts.sum(dtype=np.float32))
+                out[row, h] = (wts[:, None] * np.array(outs, np.float32)).sum(0) / total if total > 0 else 0
         row += 1
     return out
 

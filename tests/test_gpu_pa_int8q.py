@@ -65,14 +65,18 @@ def _case(seed, ctx, heads, kv_heads, d, block, dtype, mask=None, offline=False)
     return c
 
 
-def _oracle(oracle, c, scale, tile):
+PIECE_TILES = 6   # contexts of more than 6 tiles are cut, in the C-ABI tests and in their oracle alike
+
+
+def _oracle(oracle, c, scale, tile, piece_tiles=PIECE_TILES):
     return oracle.paged_attention_int8q(
         c["q8"].numpy(), c["k8"].numpy(), c["v8"].numpy(), c["tables"].numpy(), c["ctx"], c["kd"].numpy(), c["vd"].numpy(),
         scale, p_scale=None if c["ps"] is None else c["ps"].numpy(), tile=tile,
-        mask=None if c["mask"] is None else c["mask"].float().numpy(), mask_per_head=False, out_init=7.0)
+        mask=None if c["mask"] is None else c["mask"].float().numpy(), mask_per_head=False, out_init=7.0,
+        piece_tiles=piece_tiles)
 
 
-def int8q_cabi(binding, stream, dev, c, scale):
+def int8q_cabi(binding, stream, dev, c, scale, piece_tiles=PIECE_TILES):
     k = binding.kernels()
     t = {n: c[n].to(dev) for n in ("q8", "k8", "v8", "tables", "kd", "vd")}
     ps = c["ps"].to(dev) if c["ps"] is not None else None
@@ -83,7 +87,7 @@ def int8q_cabi(binding, stream, dev, c, scale):
         outDtype=dtype_code(binding, torch.empty(0, dtype=c["dtype"])), numHeads=c["heads"], numKvHeads=c["kv_heads"],
         headDim=c["d"], blockSize=c["block"], numBlocks=c["k8"].shape[0], maxBlocksPerSeq=c["tables"].shape[1],
         batch=len(lens), numQueryRows=c["rows"], offline=0 if ps is None else 1, hasMask=0 if mask is None else 1,
-        maskLen=max_len, qkScale=scale,
+        maskLen=max_len, pieceTiles=piece_tiles, qkScale=scale,
         maskSeqStride=0 if mask is None else (max_len if c["mask_kind"] == "norm" else c["heads"] * max_len),
         maskHeadStride=max_len if c["mask_kind"] == "alibi" else 0, hostContextLens=lens.ctypes.data)
     ws_bytes = ctypes.c_uint64(0)
@@ -159,7 +163,7 @@ def test_int8q_rejects_what_it_cannot_run(binding, dev, stream):
     assert k.atbmi_pa_int8q_workspace_size(ctypes.byref(call), ctypes.byref(ws)) != 0        # 300 tokens in 2 blocks
     assert "exceeds" in binding.last_kernel_error()
     lens[1] = 200
-    assert k.atbmi_pa_int8q_workspace_size(ctypes.byref(call), ctypes.byref(ws)) == 0 and ws.value == 32
+    assert k.atbmi_pa_int8q_workspace_size(ctypes.byref(call), ctypes.byref(ws)) == 0 and ws.value == 256
     call.headDim = 96
     assert k.atbmi_pa_int8q_workspace_size(ctypes.byref(call), ctypes.byref(ws)) != 0
     call.headDim, call.numKvHeads = 128, 5
@@ -168,3 +172,44 @@ def test_int8q_rejects_what_it_cannot_run(binding, dev, stream):
     assert k.atbmi_pa_int8q_workspace_size(ctypes.byref(call), ctypes.byref(ws)) != 0        # two rows asked for
     call.numQueryRows = 2
     assert k.atbmi_pa_int8q_decode(ctypes.byref(call), None, 0, stream.cuda_stream) != 0     # null tensors
+
+
+@pytest.mark.parametrize("offline,mask,dtype", [(False, "norm", torch.bfloat16), (True, None, torch.float16),
+                                                (False, "alibi", torch.float16)])
+def test_paged_attention_operation_with_int8_queries(binding, oracle, dev, stream, offline, mask, dtype):
+    """PagedAttentionOperation, quantType TYPE_QUANT_QKV_ONLINE (3) / OFFLINE (2), through Setup / Execute. Inputs:
+    query, keyCache, valueCache, blockTables, contextLens, [mask], kDescale, vDescale, [pScale] (reference
+    paged_attention_operation.cpp:408-444); the output comes in outDataType."""
+    heads, kv_heads, d, block = 32, 2, 128, 128
+    c = _case(750 + int(offline), [3000, 300, 0, 33, 65, 1, 16, 1400, 300], heads, kv_heads, d, block, dtype, mask, offline)
+    scale = 1.0 / math.sqrt(d)
+    lens = torch.from_numpy(c["ctx"])
+    ctx = binding.Context(stream)
+    op = binding.OperationRunner("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=heads, kvHeadNum=kv_heads, qkScale=scale, quantType=2 if offline else 3,
+        maskType={None: 0, "norm": 1, "alibi": 2}[mask],
+        outDataType=binding.ACL_BF16 if dtype == torch.bfloat16 else binding.ACL_FLOAT16), ctx)
+    ins = [c["q8"].to(dev), c["k8"].to(dev), c["v8"].to(dev), c["tables"].to(dev), lens.to(dev)]
+    if mask is not None:
+        ins.append(c["mask"].to(dev))
+    ins += [c["kd"].to(dev), c["vd"].to(dev)]
+    if offline:
+        ins.append(c["ps"].to(dev))
+    with torch.cuda.stream(stream):
+        out = torch.full((c["rows"], heads, d), 7.0, dtype=dtype, device=dev)
+        op.run(ins, outputs=[out], host_inputs={4: lens})
+    stream.synchronize()
+    # the operation leaves the cut of long contexts to the library (pieces of at least four tiles here): online that
+    # moves no int8 weight, offline it does (the weights are taken against each piece's own running maximum)
+    want = _oracle(oracle, c, scale, 128, piece_tiles=4)
+    assert_close(out, want, TOL[dtype], "operation")
+    assert torch.equal(out, int8q_cabi(binding, stream, dev, c, scale, piece_tiles=0))
+    ok, rates = _double_golden(_oracle(oracle, c, scale, None), want, out.float().cpu().numpy(), dtype)
+    assert ok, rates
+    # allocated from InferShape the output has the type outDataType names
+    with torch.cuda.stream(stream):
+        fresh = op.run(ins, host_inputs={4: lens})[0]
+    stream.synchronize()
+    assert fresh.dtype == dtype and torch.equal(fresh, out)
+    op.close()
+    ctx.close()

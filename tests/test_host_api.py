@@ -36,8 +36,9 @@ ELEWISE_CASES = _load("elewise")
 
 
 def _pa_unimplemented(p):
-    """Features of PagedAttentionParam the reference accepts but this library rejects at creation."""
-    return p.get("quantType", 0) >= 2
+    """Features of PagedAttentionParam the reference accepts but this library rejects at creation: int8 queries
+    (quantType QKV online / offline) together with the MLA cache."""
+    return p.get("quantType", 0) >= 2 and p.get("mlaVHeadSize", 0) > 0
 
 
 def _pa_mask_shape_refused(case):
@@ -1237,6 +1238,49 @@ def test_dequant_vector_lengths(binding, ctx):
     ins[5] = binding.make_tensor("int64", [128], FAKE_DEVICE)
     assert op.setup(ins, outs, ctx)[0] == e["ERROR_INVALID_PARAM"]
     op.close()
+
+
+def test_int8_query_quantisation_param_and_tensor_rules(binding, ctx):
+    """quantType TYPE_QUANT_QKV_OFFLINE / ONLINE (reference paged_attention_operation.cpp:250-275 parameter rules,
+    :429-436 inputs kDescale, vDescale (+ pScale offline), :455-459 the output takes outDataType; kernel library
+    paged_attention_operation.cpp:357-403: one fp32 descale per query head)."""
+    e = binding.ERROR_CODE
+    P = binding.PagedAttentionParam
+    for bad in (dict(outDataType=0), dict(outDataType=binding.ACL_FLOAT16, hasQuantOffset=True),
+                dict(outDataType=binding.ACL_FLOAT16, calcType=1, maskType=1),
+                dict(outDataType=binding.ACL_FLOAT16, compressType=1),
+                dict(outDataType=binding.ACL_FLOAT16, scaleType=1),
+                dict(outDataType=binding.ACL_FLOAT16, mlaVHeadSize=512, kvHeadNum=1)):
+        kw = dict(headNum=32, kvHeadNum=2, quantType=3, qkScale=0.088)
+        kw.update(bad)
+        op = binding.Operation("PagedAttentionOperation", P(**kw))
+        assert op.status == e["ERROR_INVALID_PARAM"], bad
+    lens = np.array([5, 0, 700, 8], dtype=np.int32)
+
+    def pack(offline, heads=32, mask="bf16", q="int8"):
+        ins = [binding.make_tensor(q, [4, 32, 128], FAKE_DEVICE), binding.make_tensor("int8", [9, 128, 2, 128], FAKE_DEVICE),
+               binding.make_tensor("int8", [9, 128, 2, 128], FAKE_DEVICE), binding.make_tensor("int32", [4, 6], FAKE_DEVICE),
+               binding.make_tensor("int32", [4], FAKE_DEVICE, host_ptr=lens.ctypes.data),
+               binding.make_tensor(mask, [4, 1, 768], FAKE_DEVICE),
+               binding.make_tensor("float", [heads], FAKE_DEVICE), binding.make_tensor("float", [32], FAKE_DEVICE)]
+        return ins + ([binding.make_tensor("float", [32], FAKE_DEVICE)] if offline else [])
+    for quant, offline in ((3, False), (2, True)):
+        op = binding.Operation("PagedAttentionOperation", P(headNum=32, kvHeadNum=2, quantType=quant, qkScale=0.088,
+                                                            maskType=1, outDataType=binding.ACL_BF16))
+        assert op.ok and op.input_num() == (9 if offline else 8) and op.output_num() == 1
+        st, descs = op.infer_shape(pack(offline))
+        assert st == 0 and descs[0].dtype == binding.ACL_BF16 and [descs[0].dims[i] for i in range(3)] == [4, 32, 128]
+        outs = [binding.make_tensor("bf16", [4, 32, 128], FAKE_DEVICE)]
+        st, ws = op.setup(pack(offline), outs, ctx)
+        assert st == 0 and ws == 33536                        # the piece table, one cut sequence, its two partial rows
+        assert op.setup(pack(offline, heads=2), outs, ctx)[0] == e["ERROR_INVALID_PARAM"]        # descales per query head
+        assert op.setup(pack(offline, mask="float16"), outs, ctx)[0] == e["ERROR_INVALID_TENSOR_INI_MATCH"]
+        assert op.setup(pack(offline, q="float16"), outs, ctx)[0] == e["ERROR_INVALID_TENSOR_INI_MATCH"]
+        assert op.setup(pack(not offline), outs, ctx)[0] == e["ERROR_INVALID_IN_TENSOR_NUM"]
+        lens[2] = 6 * 128 + 1                                   # longer than its block-table row
+        assert op.setup(pack(offline), outs, ctx)[0] == e["ERROR_INVALID_PARAM"]
+        lens[2] = 700
+        op.close()
 
 
 def test_quant_param_convert(binding):
