@@ -30,6 +30,7 @@
 // chip; a sequence in one piece is written directly, the others leave normalised fp32 rows and natural-log
 // log-sum-exps for a merge kernel (the golden cuts and merges the same way, :171-229).
 #include <algorithm>
+#include <type_traits>
 #include <vector>
 #include "pa_internal.h"
 #include "upload_ring.h"
@@ -46,11 +47,9 @@ constexpr int TILE = 128;    // tokens per tile
 constexpr int HT = 16;       // query heads per workgroup (the N extent of the MFMA)
 constexpr int THREADS = 256; // four waves
 constexpr int NWAVES = THREADS / WAVE;
-constexpr int CH = THREADS / HT;  // softmax: lanes a head
-constexpr int TPL = TILE / CH;    // softmax: tokens a lane
 constexpr int S_PITCH = (TILE + 4) * 4; // 16 heads' 16-byte writes touch every bank once
 constexpr int P_PITCH = TILE + 16;      // likewise for 16 heads' 16-byte reads
-static_assert(CH == 16 && TPL == 8 && TILE == NWAVES * 32, "four waves share a tile this way");
+static_assert(TILE == NWAVES * 32, "four waves share a tile this way");
 
 template <int D> struct Lds {
     static constexpr int PITCH = D + 16; // row pitch of the key and value tiles: 16 rows' 16-byte reads touch every bank once
@@ -127,11 +126,43 @@ __device__ __forceinline__ float RowSum(float x)
     x += RowRotate<2>(x);
     return x + RowRotate<1>(x);
 }
+// Both rows of a pair (rows 0 and 1, 2 and 3) of a value: the lane's own and, through the cross-lane network, that of
+// the lane 16 further on or back.
+__device__ __forceinline__ void PairOfRows(float x, float &a, float &b)
+{
+    a = x;
+    b = __shfl_xor(x, 16);
+}
+// All-reduce over the LANES (16 or 32) lanes of a head.
+template <int LANES> __device__ __forceinline__ float HeadMax(float x)
+{
+    x = RowMax(x);
+    if constexpr (LANES == 32) {
+        float a, b;
+        PairOfRows(x, a, b);
+        x = fmaxf(a, b);
+    }
+    return x;
+}
+template <int LANES> __device__ __forceinline__ float HeadSum(float x)
+{
+    x = RowSum(x);
+    if constexpr (LANES == 32) {
+        float a, b;
+        PairOfRows(x, a, b);
+        x = a + b;
+    }
+    return x;
+}
 
-template <int D, bool BF16, bool OFFLINE>
+// NARROW: no KV head has more than 8 query heads; the softmax then gives a head 32 lanes with 4 tokens each instead of
+// 16 lanes with 8, and the rows of heads 8 .. 15 stay zero.
+template <int D, bool BF16, bool OFFLINE, bool MASK, bool NARROW>
 __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
 {
     using L = Lds<D>;
+    constexpr int CH = NARROW ? 32 : 16; // softmax: lanes a head
+    constexpr int TPL = TILE / CH;       // softmax: tokens a lane
     constexpr int PPR = D / 16;              // 16-byte pieces per row
     constexpr int ROWS_PER_PASS = THREADS / PPR;
     constexpr int PASSES = TILE / ROWS_PER_PASS;
@@ -223,12 +254,12 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
     }
     const float descale = a.kDescale[hn];
     const uint16_t *maskRow = nullptr;
-    if (a.mask) {
+    if constexpr (MASK) {
         maskRow = reinterpret_cast<const uint16_t *>(a.mask) + static_cast<int64_t>(row.maskRow) * a.maskSeqStride +
                   static_cast<int64_t>(hn) * a.maskHeadStride;
     }
-    // softmax: lane (head tid / 16, tokens 4 (tid % 16) .. + 4 and 64 more on); a head's lanes all hold its running
-    // maximum and sum
+    // softmax: lane (head tid / CH, tokens 4 (tid % CH) .. + 4, and with 16 lanes a head 64 more on); a head's lanes
+    // all hold its running maximum and sum
     const int smHead = tid / CH;
     const int smTok = (tid % CH) * 4;
     const int smH = h0 + min(smHead, nh - 1);
@@ -242,13 +273,52 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
     for (int ct = 0; ct < CT; ++ct) {
         acc[ct] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     }
+    // this lane's mask values of a tile: tokens 32 wave + 16 rt + 4 kg + e of head n. What is loaded is the aligned
+    // 32-bit word that holds the value; the half is taken out where the value is used, so that nothing has to wait
+    // for the load before then.
+    uint32_t maskNext[2][4] = {};
+    auto maskAddress = [&](int t0, int rt, int e) {
+        return reinterpret_cast<uintptr_t>(maskRow + min(t0 + wave * 32 + rt * 16 + kg * 4 + e, row.tokEnd - 1));
+    };
+    auto requestMask = [&](int t0) {
+        if constexpr (MASK) {
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    maskNext[rt][e] = *reinterpret_cast<const uint32_t *>(maskAddress(t0, rt, e) & ~static_cast<uintptr_t>(3));
+                }
+            }
+        }
+    };
+    requestMask(row.tokBegin);
     storeRows(kNext);
+    if constexpr (NARROW) { // the weights and factors of heads 8 .. 15, which the softmax never writes
+        for (int i = tid; i < (HT / 2) * (P_PITCH / 4); i += THREADS) {
+            reinterpret_cast<uint32_t *>(smem + L::P + (HT / 2) * P_PITCH)[i] = 0u;
+        }
+        if (tid < (HT / 2) * 4) {
+            reinterpret_cast<float *>(smem + L::STAT)[(HT / 2) * 4 + tid] = 0.0f;
+        }
+    }
     __syncthreads();
 
     for (int i = 0; i < numTiles; ++i) {
         const int t0 = row.tokBegin + i * TILE;
         const bool more = i + 1 < numTiles;
+        // the mask values travel with the rows: those of tile i + 1 are asked for here, together with its rows, and
+        // have arrived when the rows are stored at the end of this pass (waiting for them any earlier would mean
+        // waiting for the rows, which were asked for in between: loads come back in order)
+        uint32_t maskBits[2][4];
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                maskBits[rt][e] = maskNext[rt][e];
+            }
+        }
         if (more) {
+            requestMask(t0 + TILE);
             requestTile(t0 + TILE, kNext, vNext);
         }
         // ---- scores of tokens 32 wave .. + 31
@@ -256,13 +326,6 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
         for (int rt = 0; rt < 2; ++rt) {
             const int tokBase = wave * 32 + rt * 16;
             const int tok = t0 + tokBase + kg * 4; // this lane's four tokens
-            uint32_t maskBits[4] = {0u, 0u, 0u, 0u};
-            if (maskRow) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    maskBits[e] = maskRow[min(tok + e, row.tokEnd - 1)];
-                }
-            }
             i32x4 dot = {0, 0, 0, 0};
 #pragma unroll
             for (int j = 0; j < D / 64; ++j) {
@@ -273,9 +336,9 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 float bias = 0.0f;
-                if (maskRow) {
-                    bias = BF16 ? Bf16ToFloat(static_cast<uint16_t>(maskBits[e]))
-                                : HalfBitsToFloat(static_cast<uint16_t>(maskBits[e]));
+                if constexpr (MASK) {
+                    const uint16_t half = static_cast<uint16_t>(maskBits[rt][e] >> ((maskAddress(t0, rt, e) & 2) * 8));
+                    bias = BF16 ? Bf16ToFloat(half) : HalfBitsToFloat(half);
                 }
                 sc[e] = static_cast<float>(dot[e]) * descale * a.qkScale + bias;
             }
@@ -303,7 +366,7 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
                     tileMax = fmaxf(tileMax, v[e]);
                 }
             }
-            tileMax = RowMax(tileMax);
+            tileMax = HeadMax<CH>(tileMax);
             const float newMax = fmaxf(runMax, tileMax);
             const bool any = newMax > -INFINITY; // (a mask of -inf can hide everything seen so far)
             float sum = 0.0f, wmax = 0.0f;
@@ -313,8 +376,8 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
                 sum += w[k];
                 wmax = fmaxf(wmax, w[k]);
             }
-            sum = RowSum(sum);
-            wmax = RowMax(wmax);
+            sum = HeadSum<CH>(sum);
+            wmax = HeadMax<CH>(wmax);
             const float keep = (any && runMax > -INFINITY) ? __expf(runMax - newMax) : 0.0f;
             runSum = runSum * keep + sum;
             runMax = newMax;
@@ -595,8 +658,16 @@ template <int D> int Launch(const AtbmiPaInt8QCall *call, const Args &a, int64_t
 {
     const bool bf16 = call->outDtype == ATBMI_BF16;
     const bool offline = call->offline != 0;
-    auto kernel = bf16 ? (offline ? PaInt8QKernel<D, true, true> : PaInt8QKernel<D, true, false>)
-                       : (offline ? PaInt8QKernel<D, false, true> : PaInt8QKernel<D, false, false>);
+    const bool mask = a.mask != nullptr;
+    const bool narrow = call->numHeads / call->numKvHeads <= HT / 2;
+    auto pick = [&](auto withMask, auto isNarrow) {
+        constexpr bool M = decltype(withMask)::value;
+        constexpr bool N = decltype(isNarrow)::value;
+        return bf16 ? (offline ? PaInt8QKernel<D, true, true, M, N> : PaInt8QKernel<D, true, false, M, N>)
+                    : (offline ? PaInt8QKernel<D, false, true, M, N> : PaInt8QKernel<D, false, false, M, N>);
+    };
+    auto kernel = mask ? (narrow ? pick(std::true_type{}, std::true_type{}) : pick(std::true_type{}, std::false_type{}))
+                       : (narrow ? pick(std::false_type{}, std::true_type{}) : pick(std::false_type{}, std::false_type{}));
     int rc = ConfigureKernelLds(reinterpret_cast<const void *>(kernel), Lds<D>::BYTES);
     if (rc != OK) {
         return rc;
