@@ -15,19 +15,20 @@
 // tests compare against the whole context as one tile by the double-golden criterion, so the tile is not a
 // property of the operator.) Every integer product is exact (v_mfma_i32_16x16x64_i8; sums stay below 2^24).
 //
-// A workgroup of four waves owns one sequence, one KV head and up to 16 of its query heads and walks the context
-// tile by tile. Key and value rows of tile i + 1 are requested into registers before the arithmetic of tile i. One
-// LDS buffer (token-major, padded pitch) serves both: it holds the key rows while they are scored, then the value
-// rows of the same tile, which wait in registers until then; that keeps a workgroup at 29 KB of LDS (D = 128).
+// A workgroup of four waves owns one piece of a sequence, one KV head and up to 16 of its query heads and walks the
+// piece tile by tile. Key rows are requested into registers two tiles ahead of their scores, value rows one tile ahead, and
+// both are stored to LDS (token-major, padded pitch) right after the scores of a tile: the key rows of the next tile
+// and the value rows of this one. A tile then needs two workgroup barriers, after the scores and after the weights.
 //   scores  wave w for tokens 32 w .. 32 w + 31: S^T[token, head] = K . Q^T (K rows from LDS as A, the query
 //           resident in registers as B);
-//   softmax 16 lanes a head, 8 tokens a lane; int8 weights P[head][token] go to LDS;
+//   softmax 16 lanes a head, 8 tokens a lane (32 lanes with 4 tokens when a KV head has at most 8 query heads);
+//           int8 weights P[head][token] go to LDS;
 //   values  wave w for channels (D / 4) w .. : O^T[channel, head] += V^T . P^T, V^T read from the token-major rows by
 //           the transposing ds_read_b64_tr_b8, P^T as 16 consecutive bytes of a head's weights.
 // Operand layout of v_mfma_i32_16x16x64_i8: lane (n = lane % 16, kg = lane / 16) supplies the 16 contraction values
 // 16 kg .. 16 kg + 15 of row n (A) / column n (B) and receives D[4 kg + e][n], e = 0 .. 3.
-// Long contexts are cut into pieces of whole tiles, sized so that the launch has a few workgroups per place on the
-// chip; a sequence in one piece is written directly, the others leave normalised fp32 rows and natural-log
+// Long contexts are cut into pieces of whole tiles (64 at most), sized so that the launch has a few workgroups per
+// place on the chip; a sequence in one piece is written directly, the others leave normalised fp32 rows and natural-log
 // log-sum-exps for a merge kernel (the golden cuts and merges the same way, :171-229).
 #include <algorithm>
 #include <type_traits>
@@ -47,14 +48,16 @@ constexpr int TILE = 128;    // tokens per tile
 constexpr int HT = 16;       // query heads per workgroup (the N extent of the MFMA)
 constexpr int THREADS = 256; // four waves
 constexpr int NWAVES = THREADS / WAVE;
+constexpr int MAX_PIECE_TILES = 64; // a piece's block ids fit one register of a wave (see the kernel)
 constexpr int S_PITCH = (TILE + 4) * 4; // 16 heads' 16-byte writes touch every bank once
 constexpr int P_PITCH = TILE + 16;      // likewise for 16 heads' 16-byte reads
 static_assert(TILE == NWAVES * 32, "four waves share a tile this way");
 
 template <int D> struct Lds {
     static constexpr int PITCH = D + 16; // row pitch of the key and value tiles: 16 rows' 16-byte reads touch every bank once
-    static constexpr int KV = 0;                 // the key rows of a tile, then (once they are scored) its value rows
-    static constexpr int S = KV + TILE * PITCH;  // [16] fp32 scores
+    static constexpr int K = 0;                  // the key rows of a tile
+    static constexpr int V = K + TILE * PITCH;   // the value rows of a tile
+    static constexpr int S = V + TILE * PITCH;   // [16] fp32 scores
     static constexpr int P = S + HT * S_PITCH;   // [16] int8 weights
     static constexpr int STAT = P + HT * P_PITCH; // [16] {keep, value scale, 1 / sum, -}
     static constexpr int BYTES = STAT + HT * 16;
@@ -103,8 +106,16 @@ struct Args {
     int32_t numRows;
     int32_t maxBlocksPerSeq;
     int32_t blockSize;
+    int32_t bf16; // outputs (and mask values) are bf16 instead of fp16
     float qkScale;
 };
+
+// Cache rows are read once per call: the non-temporal hint keeps them from displacing anything in L2 / the
+// memory-side cache.
+__device__ __forceinline__ u32x4 LoadStream16(const void *p)
+{
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+}
 
 // All-reduce over the 16 lanes of a row (lanes 16 r .. 16 r + 15) by rotations inside the row.
 template <int ROR> __device__ __forceinline__ float RowRotate(float x)
@@ -157,7 +168,7 @@ template <int LANES> __device__ __forceinline__ float HeadSum(float x)
 
 // NARROW: no KV head has more than 8 query heads; the softmax then gives a head 32 lanes with 4 tokens each instead of
 // 16 lanes with 8, and the rows of heads 8 .. 15 stay zero.
-template <int D, bool BF16, bool OFFLINE, bool MASK, bool NARROW>
+template <int D, bool OFFLINE, bool MASK, bool NARROW, bool WHOLE>
 __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
 {
     using L = Lds<D>;
@@ -194,52 +205,51 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
     // ---- requests for a tile: this thread's pieces of the key and value rows (tokens past the context repeat the last one)
     const int ldTok = tid / PPR;
     const int ldPiece = tid % PPR;
-    // When a block holds whole tiles (block sizes 128, 256, ..) a tile lies in one block and its first slot is the
-    // same for the whole workgroup; otherwise every token looks its block up.
-    // In that case the block ids come from a per-lane cache of 64 table entries (lane l holds entry cacheBase + l),
-    // so that a tile's rows can be requested without waiting for a table entry first.
-    const bool wholeTiles = a.blockSize % TILE == 0;
+    // WHOLE: a block holds whole tiles (block sizes 128, 256, ..), so a tile lies in one block and its first slot is
+    // the same for the whole workgroup; otherwise every token looks its block up. With WHOLE the block ids of the
+    // piece are read once, before the loop: lane l keeps table entry firstBlock + l (the host cuts pieces of at most
+    // 64 tiles), and a request takes its id out of that register. No load and no branch then stands between the row
+    // requests of one pass and of the next. Requests are never skipped either: past the last tile of the piece every
+    // lane asks for its piece of one row of the last tile again (a few cache lines that are in L2), so that the
+    // number of loads in flight at any point of the loop is known when the kernel is compiled and the waits in front
+    // of the LDS stores name exactly the loads they need, instead of draining everything that is on its way.
     const int64_t laneAt = static_cast<int64_t>(g) * D + ldPiece * 16;
-    int cacheBase = wholeTiles ? row.tokBegin / a.blockSize : 0;
-    int cachedIds = table[min(cacheBase + lane, a.maxBlocksPerSeq - 1)];
-    auto requestTile = [&](int t0, u32x4(&kr)[PASSES], u32x4(&vr)[PASSES]) {
-        if (wholeTiles) {
+    const int firstBlock = WHOLE ? row.tokBegin / a.blockSize : 0;
+    const int cachedIds = table[min(firstBlock + lane, a.maxBlocksPerSeq - 1)];
+    const int lastTile = row.tokBegin + (numTiles - 1) * TILE;
+    auto requestRows = [&](const int8_t *cache, int tile0, u32x4(&r)[PASSES]) {
+        const bool live = tile0 <= lastTile;
+        const int t0 = min(tile0, lastTile);
+        if constexpr (WHOLE) {
             const int blk = __builtin_amdgcn_readfirstlane(t0 / a.blockSize);
-            if (blk - cacheBase >= WAVE) {
-                cacheBase = blk;
-                cachedIds = table[min(cacheBase + lane, a.maxBlocksPerSeq - 1)];
-            }
-            const int id = __builtin_amdgcn_readlane(cachedIds, blk - cacheBase);
+            const int id = __builtin_amdgcn_readlane(cachedIds, blk - firstBlock);
             const int64_t first = static_cast<int64_t>(id) * a.blockSize + (t0 - blk * a.blockSize);
-            const int last = row.tokEnd - 1 - t0; // (tokens past the piece repeat its last one)
+            const int last = live ? row.tokEnd - 1 - t0 : 0; // (tokens past the piece repeat its last one)
 #pragma unroll
             for (int p = 0; p < PASSES; ++p) {
-                const int64_t at = (first + min(p * ROWS_PER_PASS + ldTok, last)) * slotBytes + laneAt;
-                kr[p] = *reinterpret_cast<const u32x4 *>(a.k8 + at);
-                vr[p] = *reinterpret_cast<const u32x4 *>(a.v8 + at);
+                r[p] = LoadStream16(cache + (first + min(p * ROWS_PER_PASS + ldTok, last)) * slotBytes + laneAt);
             }
-            return;
-        }
+        } else {
 #pragma unroll
-        for (int p = 0; p < PASSES; ++p) {
-            const int tok = min(t0 + p * ROWS_PER_PASS + ldTok, row.tokEnd - 1);
-            const int blk = tok / a.blockSize;
-            const int64_t slot = static_cast<int64_t>(table[blk]) * a.blockSize + (tok - blk * a.blockSize);
-            const int64_t at = slot * slotBytes + laneAt;
-            kr[p] = *reinterpret_cast<const u32x4 *>(a.k8 + at);
-            vr[p] = *reinterpret_cast<const u32x4 *>(a.v8 + at);
+            for (int p = 0; p < PASSES; ++p) {
+                const int tok = live ? min(t0 + p * ROWS_PER_PASS + ldTok, row.tokEnd - 1) : t0;
+                const int blk = tok / a.blockSize;
+                const int64_t slot = static_cast<int64_t>(table[blk]) * a.blockSize + (tok - blk * a.blockSize);
+                r[p] = LoadStream16(cache + slot * slotBytes + laneAt);
+            }
         }
     };
-    auto storeRows = [&](const u32x4(&r)[PASSES]) {
+    auto storeRows = [&](int buffer, const u32x4(&r)[PASSES]) {
 #pragma unroll
         for (int p = 0; p < PASSES; ++p) {
-            *reinterpret_cast<u32x4 *>(smem + L::KV + (p * ROWS_PER_PASS + ldTok) * L::PITCH + ldPiece * 16) = r[p];
+            *reinterpret_cast<u32x4 *>(smem + buffer + (p * ROWS_PER_PASS + ldTok) * L::PITCH + ldPiece * 16) = r[p];
         }
     };
-    // the rows of tile i + 1 are on their way while tile i is worked on; the value rows of tile i wait in registers
-    // until its key rows are scored
-    u32x4 kNext[PASSES], vNext[PASSES], vCur[PASSES];
-    requestTile(row.tokBegin, kNext, vCur);
+    // Rows are asked for a tile and a half ahead: while tile i is worked on, set A holds the key rows of tile i + 1
+    // and the value rows of tile i (both stored to LDS once the scores of tile i are done), set B takes the key rows
+    // of tile i + 2 and the value rows of tile i + 1; the sets swap roles every tile.
+    u32x4 kA[PASSES], vA[PASSES], kB[PASSES], vB[PASSES];
+    requestRows(a.k8, row.tokBegin, kA);
 
     // ---- Q^T as B operands: lane (n, kg) holds q8[head n][64 j + 16 kg .. + 16)
     i32x4 q8[D / 64];
@@ -292,7 +302,9 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
         }
     };
     requestMask(row.tokBegin);
-    storeRows(kNext);
+    storeRows(L::K, kA);
+    requestRows(a.v8, row.tokBegin, vA);
+    requestRows(a.k8, row.tokBegin + TILE, kA);
     if constexpr (NARROW) { // the weights and factors of heads 8 .. 15, which the softmax never writes
         for (int i = tid; i < (HT / 2) * (P_PITCH / 4); i += THREADS) {
             reinterpret_cast<uint32_t *>(smem + L::P + (HT / 2) * P_PITCH)[i] = 0u;
@@ -303,24 +315,23 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
     }
     __syncthreads();
 
-    for (int i = 0; i < numTiles; ++i) {
+    // the mask values of the tile being worked on (see the end of a pass)
+    uint32_t maskBits[2][4];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            maskBits[rt][e] = maskNext[rt][e];
+        }
+    }
+    // One tile: LDS holds its key rows; kNow are the key rows of the next tile and vNow its own value rows, on their
+    // way since the pass before; kLater / vLater take what the pass after this one will store. Two barriers a tile:
+    // whatever a phase overwrites was last read two phases earlier.
+    auto pass = [&](const int i, u32x4(&kNow)[PASSES], u32x4(&vNow)[PASSES], u32x4(&kLater)[PASSES], u32x4(&vLater)[PASSES]) {
         const int t0 = row.tokBegin + i * TILE;
-        const bool more = i + 1 < numTiles;
-        // the mask values travel with the rows: those of tile i + 1 are asked for here, together with its rows, and
-        // have arrived when the rows are stored at the end of this pass (waiting for them any earlier would mean
-        // waiting for the rows, which were asked for in between: loads come back in order)
-        uint32_t maskBits[2][4];
-#pragma unroll
-        for (int rt = 0; rt < 2; ++rt) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                maskBits[rt][e] = maskNext[rt][e];
-            }
-        }
-        if (more) {
-            requestMask(t0 + TILE);
-            requestTile(t0 + TILE, kNext, vNext);
-        }
+        requestMask(t0 + TILE);
+        requestRows(a.v8, t0 + TILE, vLater);
+        requestRows(a.k8, t0 + 2 * TILE, kLater);
         // ---- scores of tokens 32 wave .. + 31
 #pragma unroll
         for (int rt = 0; rt < 2; ++rt) {
@@ -329,7 +340,7 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
             i32x4 dot = {0, 0, 0, 0};
 #pragma unroll
             for (int j = 0; j < D / 64; ++j) {
-                const i32x4 kk = *reinterpret_cast<const i32x4 *>(smem + L::KV + (tokBase + n) * L::PITCH + j * 64 + kg * 16);
+                const i32x4 kk = *reinterpret_cast<const i32x4 *>(smem + L::K + (tokBase + n) * L::PITCH + j * 64 + kg * 16);
                 dot = __builtin_amdgcn_mfma_i32_16x16x64_i8(kk, q8[j], dot, 0, 0, 0);
             }
             f32x4 sc;
@@ -338,7 +349,7 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
                 float bias = 0.0f;
                 if constexpr (MASK) {
                     const uint16_t half = static_cast<uint16_t>(maskBits[rt][e] >> ((maskAddress(t0, rt, e) & 2) * 8));
-                    bias = BF16 ? Bf16ToFloat(half) : HalfBitsToFloat(half);
+                    bias = a.bf16 ? Bf16ToFloat(half) : HalfBitsToFloat(half);
                 }
                 sc[e] = static_cast<float>(dot[e]) * descale * a.qkScale + bias;
             }
@@ -350,8 +361,9 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
             }
             *reinterpret_cast<f32x4 *>(smem + L::S + n * S_PITCH + (tokBase + kg * 4) * 4) = sc;
         }
-        __syncthreads(); // the key rows are scored: their place takes the value rows
-        storeRows(vCur);
+        __syncthreads(); // the key rows are scored, and everybody is done with the values of the tile before
+        storeRows(L::K, kNow); // (after the last tile: rows nobody reads)
+        storeRows(L::V, vNow);
         // ---- weights of the tile
         {
             float w[TPL];
@@ -445,7 +457,7 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
                     // the transposing read hands lane (channel n, kg) the bytes of tokens r .. r + 7 when lane n of
                     // the group points at token r + n / 2, channels (n % 2) * 8 .. + 8
                     const unsigned char *vp =
-                        smem + L::KV + (hh * 64 + kg * 16 + (n >> 1)) * L::PITCH + cb + (n & 1) * 8;
+                        smem + L::V + (hh * 64 + kg * 16 + (n >> 1)) * L::PITCH + cb + (n & 1) * 8;
                     const i32x2 lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2 *)(vp));
                     const i32x2 hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
                         (__attribute__((address_space(3))) i32x2 *)(vp + 8 * L::PITCH));
@@ -458,15 +470,29 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
                 }
             }
         }
-        __syncthreads(); // everybody has left the tile
-        if (more) {
-            storeRows(kNext);
+        // The mask values of the next tile were asked for at the top of this pass, before its rows; they are taken
+        // over here, a whole pass later, so that waiting for them does not hold anything up (loads come back in
+        // order: earlier in the pass this wait would have been a wait for the rows asked for after them).
+        if constexpr (MASK) {
 #pragma unroll
-            for (int p = 0; p < PASSES; ++p) {
-                vCur[p] = vNext[p];
+            for (int rt = 0; rt < 2; ++rt) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    maskBits[rt][e] = maskNext[rt][e];
+                    asm volatile("" : "+v"(maskBits[rt][e]));
+                }
             }
-            __syncthreads();
         }
+    };
+    // (pairs of tiles without a way round the second one: a path that skips it would reach the loop's head with the
+    // first one's requests still on their way, and the compiler would wait for them there on every round)
+    int tile = 0;
+    for (; tile + 1 < numTiles; tile += 2) {
+        pass(tile, kA, vA, kB, vB);
+        pass(tile + 1, kB, vB, kA, vA);
+    }
+    if (tile < numTiles) {
+        pass(tile, kA, vA, kB, vB);
     }
     // ---- the rows: acc / sum, to the output or, for a piece of a sequence, to its partial row with log(sum) + max
     if (tid % CH == 0) {
@@ -494,7 +520,7 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const float o = acc[ct][e] * inv;
-                bits[e] = BF16 ? FloatToBf16(o) : FloatToHalfBits(o);
+                bits[e] = a.bf16 ? FloatToBf16(o) : FloatToHalfBits(o);
             }
             uint2 w;
             w.x = static_cast<uint32_t>(bits[0]) | (static_cast<uint32_t>(bits[1]) << 16);
@@ -507,7 +533,6 @@ __global__ __launch_bounds__(THREADS) void PaInt8QKernel(const Args a)
 // Joins the pieces of a cut sequence: out = sum_p exp(lse_p - L) O_p, L = log sum_p exp(lse_p) (reference golden
 // test_paged_attention_common.py:217-228). grid.x = (cut sequence, head); a thread takes channels of the row.
 constexpr int MERGE_THREADS = 128;
-template <bool BF16>
 __global__ __launch_bounds__(MERGE_THREADS) void PaInt8QMergeKernel(const Args a, int D)
 {
     const MergeRow m = a.mergeRows[blockIdx.x / a.H];
@@ -537,7 +562,7 @@ __global__ __launch_bounds__(MERGE_THREADS) void PaInt8QMergeKernel(const Args a
             acc += weightOf(a.partLse[first + p * perPartial]) * a.partO[(first + p * perPartial) * D + d];
         }
         const float o = acc * inv;
-        orow[d] = BF16 ? FloatToBf16(o) : FloatToHalfBits(o);
+        orow[d] = a.bf16 ? FloatToBf16(o) : FloatToHalfBits(o);
     }
 }
 
@@ -606,7 +631,7 @@ struct Layout {
 // Cuts the sequences into pieces of whole tiles and deals them out to the eight parts of the table in turn from the
 // longest to the shortest (every part starts with its longest piece, and the parts carry about the same number of
 // tokens). The piece length aims at four workgroups for each of the 1024 places the chip has for them (256 CUs, four
-// workgroups of this kernel each), and at no less than four tiles.
+// workgroups of this kernel each), at no less than four tiles and at no more than MAX_PIECE_TILES.
 Layout PlanPieces(const AtbmiPaInt8QCall *c, const std::vector<Row> &seqs)
 {
     Layout lay;
@@ -617,7 +642,8 @@ Layout PlanPieces(const AtbmiPaInt8QCall *c, const std::vector<Row> &seqs)
         tiles += (r.tokEnd + TILE - 1) / TILE;
     }
     const int64_t target = 4 * 1024;
-    const int64_t chunk = c->pieceTiles > 0 ? c->pieceTiles : std::max<int64_t>(4, (tiles * perPiece + target - 1) / target);
+    const int64_t chunk = std::min<int64_t>(
+        MAX_PIECE_TILES, c->pieceTiles > 0 ? c->pieceTiles : std::max<int64_t>(4, (tiles * perPiece + target - 1) / target));
     for (const Row &r : seqs) {
         const int64_t n = (r.tokEnd + TILE - 1) / TILE;
         const int64_t parts = (n + chunk - 1) / chunk;
@@ -656,18 +682,25 @@ Layout PlanPieces(const AtbmiPaInt8QCall *c, const std::vector<Row> &seqs)
 
 template <int D> int Launch(const AtbmiPaInt8QCall *call, const Args &a, int64_t grid, int64_t numMerges, hipStream_t s)
 {
-    const bool bf16 = call->outDtype == ATBMI_BF16;
-    const bool offline = call->offline != 0;
-    const bool mask = a.mask != nullptr;
     const bool narrow = call->numHeads / call->numKvHeads <= HT / 2;
-    auto pick = [&](auto withMask, auto isNarrow) {
-        constexpr bool M = decltype(withMask)::value;
-        constexpr bool N = decltype(isNarrow)::value;
-        return bf16 ? (offline ? PaInt8QKernel<D, true, true, M, N> : PaInt8QKernel<D, true, false, M, N>)
-                    : (offline ? PaInt8QKernel<D, false, true, M, N> : PaInt8QKernel<D, false, false, M, N>);
+    // the kernel variant, one compile-time switch after the other
+    void (*kernel)(Args) = nullptr;
+    auto with = [](bool flag, auto &&next) {
+        if (flag) {
+            next(std::true_type{});
+        } else {
+            next(std::false_type{});
+        }
     };
-    auto kernel = mask ? (narrow ? pick(std::true_type{}, std::true_type{}) : pick(std::true_type{}, std::false_type{}))
-                       : (narrow ? pick(std::false_type{}, std::true_type{}) : pick(std::false_type{}, std::false_type{}));
+    with(call->offline != 0, [&](auto off) {
+        with(a.mask != nullptr, [&](auto msk) {
+            with(narrow, [&](auto nar) {
+                with(call->blockSize % TILE == 0, [&](auto who) {
+                    kernel = PaInt8QKernel<D, decltype(off)::value, decltype(msk)::value, decltype(nar)::value, decltype(who)::value>;
+                });
+            });
+        });
+    });
     int rc = ConfigureKernelLds(reinterpret_cast<const void *>(kernel), Lds<D>::BYTES);
     if (rc != OK) {
         return rc;
@@ -685,11 +718,7 @@ template <int D> int Launch(const AtbmiPaInt8QCall *call, const Args &a, int64_t
     }
     if (numMerges > 0) {
         const unsigned mergeGrid = static_cast<unsigned>(numMerges * a.H);
-        if (bf16) {
-            PaInt8QMergeKernel<true><<<mergeGrid, MERGE_THREADS, 0, s>>>(a, D);
-        } else {
-            PaInt8QMergeKernel<false><<<mergeGrid, MERGE_THREADS, 0, s>>>(a, D);
-        }
+        PaInt8QMergeKernel<<<mergeGrid, MERGE_THREADS, 0, s>>>(a, D);
         ATBMI_HIP_CHECK(hipGetLastError());
     }
     return TimedLaunchEnd(s, timed, numMerges > 0);
@@ -770,6 +799,7 @@ extern "C" int atbmi_pa_int8q_decode(const AtbmiPaInt8QCall *call, void *workspa
     a.numRows = static_cast<int32_t>(lay.pieces.size());
     a.maxBlocksPerSeq = call->maxBlocksPerSeq;
     a.blockSize = call->blockSize;
+    a.bf16 = call->outDtype == ATBMI_BF16 ? 1 : 0;
     a.qkScale = call->qkScale;
     switch (call->headDim) {
         case 64: return int8q::Launch<64>(call, a, grid, static_cast<int64_t>(lay.merges.size()), s);

@@ -551,7 +551,8 @@ typedef struct AtbmiPaInt8QCall {
     int32_t hasMask;
     int32_t maskLen;           /* positions a mask row covers, >= every context length */
     int32_t pieceTiles;        /* 0: the library chooses; c > 0: a context of n tiles of 128 tokens is cut into
-                                  ceil(n / c) pieces of ceil(n / pieces) tiles, merged by their log-sum-exps */
+                                  ceil(n / c) pieces of ceil(n / pieces) tiles, merged by their log-sum-exps; values
+                                  above 64 count as 64 */
     float qkScale;
     int64_t maskSeqStride;
     int64_t maskHeadStride;

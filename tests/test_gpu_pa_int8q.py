@@ -153,6 +153,21 @@ def test_int8q_kernel_against_the_oracle(binding, oracle, dev, stream, case):
     assert float(got.float().abs().max()) > 0
 
 
+def test_int8q_pieces_are_capped_at_64_tiles(binding, oracle, dev, stream):
+    """A piece never has more than 64 tiles, whatever pieceTiles asks for (a wave keeps a piece's block ids in one
+    register): a context of 71 tiles with pieceTiles = 100 is cut like pieceTiles = 64 cuts it, into 36 + 35 tiles.
+    Offline quantisation shows the cut in the int8 weights, so the oracle with one piece must differ where the
+    oracle with the capped cut matches."""
+    ctx, heads, kv_heads, d, block, dtype = [9000, 130], 4, 1, 64, 128, torch.float16
+    c = _case(911, ctx, heads, kv_heads, d, block, dtype, None, True)
+    scale = 1.0 / math.sqrt(d)
+    got = int8q_cabi(binding, stream, dev, c, scale, piece_tiles=100)
+    assert torch.equal(got, int8q_cabi(binding, stream, dev, c, scale, piece_tiles=64))
+    assert_close(got, _oracle(oracle, c, scale, 128, piece_tiles=64), TOL[dtype], "capped pieces")
+    whole = _oracle(oracle, c, scale, 128, piece_tiles=100)
+    assert np.abs(whole - _oracle(oracle, c, scale, 128, piece_tiles=64)).max() > 0
+
+
 def test_int8q_rejects_what_it_cannot_run(binding, dev, stream):
     k = binding.kernels()
     lens = np.array([5, 300], np.int32)
