@@ -521,7 +521,7 @@ int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspaceDevice, u
  * for the parameters and inputs, kernel library src/kernels/mixkernels/pagedattention/paged_attention_operation.cpp:
  * 357-403 for the descale shapes, golden tests/apitest/kernelstest/mix/test_paged_attention_common.py:104-110,147-229):
  * query, keys and values are int8 with one fp32 descale per QUERY head for the scores (kDescale) and one for the
- * values (vDescale); the softmax weights of every tile of 128 tokens are quantised to int8 before they multiply the
+ * values (vDescale); the softmax weights of every tile of 64 tokens are quantised to int8 before they multiply the
  * int8 value rows, against the tile's largest weight (online) or with the factor pScale[head] (offline); all integer
  * products are exact.
  *   query       int8 [numQueryRows, numHeads, headDim]            kDescale, vDescale, pScale  fp32 [numHeads]
@@ -550,9 +550,12 @@ typedef struct AtbmiPaInt8QCall {
     int32_t offline;           /* 0: weights quantised against the tile's maximum; 1: with pScale */
     int32_t hasMask;
     int32_t maskLen;           /* positions a mask row covers, >= every context length */
-    int32_t pieceTiles;        /* 0: the library chooses; c > 0: a context of n tiles of 128 tokens is cut into
-                                  ceil(n / c) pieces of ceil(n / pieces) tiles, merged by their log-sum-exps; values
-                                  above 64 count as 64 */
+    int32_t pieceTiles;        /* c > 0: a context of n units of 128 tokens is cut into ceil(n / c) pieces of
+                                  ceil(n / pieces) units, merged by their log-sum-exps. 0: the library cuts: the
+                                  64-token tiles of all sequences, in order, are one list cut into equal shares,
+                                  share w beginning at tile floor(tiles x w / shares), with shares = min(tiles / 4,
+                                  workgroups the chip holds at once); a sequence is cut where a share begins
+                                  inside it */
     float qkScale;
     int64_t maskSeqStride;
     int64_t maskHeadStride;

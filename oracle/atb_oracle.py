@@ -812,7 +812,8 @@ def mla_int8_decode(q_int8, q_rope, kv_int8, k_rope, block_tables, context_lens,
 
 
 def paged_attention_int8q(q_int8, key_cache, value_cache, block_tables, context_lens, k_descale, v_descale, scale,
-                          p_scale=None, tile=128, mask=None, mask_per_head=None, out_init=0.0, piece_tiles=None):
+                          p_scale=None, tile=128, mask=None, mask_per_head=None, out_init=0.0, piece_tiles=None, piece_unit=None,
+                          piece_cuts=None):
     """Decode attention with int8 queries over int8 caches (PagedAttentionParam quantType QKV online / offline;
     reference golden tests/apitest/kernelstest/mix/test_paged_attention_common.py:104-110 (exact int32 products
     times a descale per QUERY head), :256-263 (then the scale, then the mask), :147-168 (softmax_quant_numpy: weights
@@ -824,7 +825,9 @@ def paged_attention_int8q(q_int8, key_cache, value_cache, block_tables, context_
     q_int8 [rows, H, D] int8; key_cache / value_cache [blocks, block_size, G, D] int8; k_descale, v_descale, p_scale
     [H] float32 (p_scale None: online). The weights of every `tile` consecutive tokens are quantised on their own;
     tile=None takes the whole context as one tile, the reference's high-precision golden (:264-270). piece_tiles = c
-    cuts a context of n tiles into ceil(n / c) pieces of ceil(n / pieces) tiles each. (Online the cut changes nothing
+    cuts a context of n units into ceil(n / c) pieces of ceil(n / pieces) units each, a unit being piece_unit tokens
+    (a multiple of the tile; by default the tile itself); piece_cuts = {sequence: [tokens]} names the cuts of a
+    sequence outright (multiples of the tile). (Online the cut changes nothing
     but the order of a few fp32 operations; offline the weights are taken against the running maximum, which starts
     anew in every piece, so the int8 weights themselves depend on the cut.) mask as in paged_attention with one query
     token per sequence. A sequence of length 0 takes no query row; rows never written keep out_init. Returns float32
@@ -846,10 +849,16 @@ def paged_attention_int8q(q_int8, key_cache, value_cache, block_tables, context_
         step = ctx if tile is None else tile
         bounds = [0, ctx]
         if piece_tiles is not None and tile is not None:
-            n = (ctx + tile - 1) // tile
+            unit = tile if piece_unit is None else piece_unit
+            assert unit % tile == 0
+            n = (ctx + unit - 1) // unit
             parts = (n + piece_tiles - 1) // piece_tiles
             each = (n + parts - 1) // parts
-            bounds = [min(ctx, i * each * tile) for i in range(parts)] + [ctx]
+            bounds = [min(ctx, i * each * unit) for i in range(parts)] + [ctx]
+        if piece_cuts is not None and tile is not None:
+            cuts = sorted(piece_cuts.get(b, []))
+            assert all(0 < t < ctx and t % tile == 0 for t in cuts)
+            bounds = [0] + cuts + [ctx]
         for h in range(heads):
             g = h // group
             prod = (keys[:, g, :] @ q_int8[row, h].astype(np.int32)).astype(np.float32)       # [ctx]

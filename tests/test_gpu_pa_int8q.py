@@ -68,12 +68,45 @@ def _case(seed, ctx, heads, kv_heads, d, block, dtype, mask=None, offline=False)
 PIECE_TILES = 6   # contexts of more than 6 tiles are cut, in the C-ABI tests and in their oracle alike
 
 
-def _oracle(oracle, c, scale, tile, piece_tiles=PIECE_TILES):
+TILE = 64   # tokens whose weights the library quantises together
+
+
+def library_cuts(c, compute_units):
+    """Where the library cuts the sequences of a call with pieceTiles = 0: the tiles of 64 tokens of all sequences, in
+    order, are one list cut into equal shares (share w starts at tile floor(tiles * w / shares)); shares =
+    min(tiles // 4, workgroups the chip holds at once), a workgroup being up to 8 waves (4 for head size 256), one
+    per (KV head, tile of 16 query heads) pair, with 2 * 64 * (D + 16) bytes of the CU's 160 KiB each. Returns
+    {sequence: [tokens]}."""
+    pairs = c["kv_heads"] * -(-(c["heads"] // c["kv_heads"]) // 16)
+    most = 8 if c["d"] <= 128 else 4
+    groups = -(-pairs // most)
+    waves = -(-pairs // groups)
+    per_cu = max(1, min(8 // waves, 160 * 1024 // (waves * 2 * 64 * (c["d"] + 16))))
+    tiles = [-(-int(n) // 64) for n in c["ctx"]]
+    total = sum(tiles)
+    shares = max(1, min(total // 4, compute_units * per_cu // groups))
+    starts = [total * w // shares for w in range(1, shares)]
+    cuts, at = {}, 0
+    for b, n in enumerate(tiles):
+        here = [(s - at) * 64 for s in starts if at < s < at + n]
+        assert all(y - x <= min(8192, 64 * c["block"]) for x, y in zip([0] + here, here + [int(c["ctx"][b])]))
+        if here:
+            cuts[b] = here
+        at += n
+    return cuts
+
+
+def _oracle(oracle, c, scale, tile, piece_tiles=PIECE_TILES, piece_cuts=None):
+    """tile: "own" for the library's tile, None for the whole context as one tile; piece_tiles counts tiles of 128
+    tokens, as the C ABI does."""
+    if tile == "own":
+        tile = TILE
     return oracle.paged_attention_int8q(
         c["q8"].numpy(), c["k8"].numpy(), c["v8"].numpy(), c["tables"].numpy(), c["ctx"], c["kd"].numpy(), c["vd"].numpy(),
         scale, p_scale=None if c["ps"] is None else c["ps"].numpy(), tile=tile,
         mask=None if c["mask"] is None else c["mask"].float().numpy(), mask_per_head=False, out_init=7.0,
-        piece_tiles=piece_tiles)
+        piece_tiles=None if piece_cuts is not None else piece_tiles, piece_unit=None if tile is None else 128,
+        piece_cuts=piece_cuts)
 
 
 def int8q_cabi(binding, stream, dev, c, scale, piece_tiles=PIECE_TILES):
@@ -135,6 +168,13 @@ INT8Q_MATRIX = [
     ([300, 1000, 0, 77], 40, 1, 128, 64, torch.float16, None, False),     # 40 heads over one KV head: three head tiles
     ([300, 100, 77], 8, 8, 64, 16, torch.float16, "norm", False),         # head size 64, 16-token blocks, MHA
     ([260, 31], 12, 4, 256, 32, torch.bfloat16, None, False),             # head size 256
+    ([700, 260, 31], 24, 12, 256, 64, torch.float16, "norm", True),       # head size 256: 12 KV heads in workgroups of 4 waves
+    ([330, 64, 1100], 16, 4, 64, 64, torch.bfloat16, "alibi", False),     # head size 64, blocks of 64 tokens = a wave's tile
+    # one KV head with at most 16 query heads: workgroups of one wave
+    ([700, 129, 128, 4, 1500], 8, 1, 128, 128, torch.float16, "norm", False),
+    ([700, 129, 128, 4, 1500], 16, 1, 128, 128, torch.bfloat16, "alibi", True),
+    ([300, 100, 77], 4, 1, 64, 16, torch.float16, None, False),
+    ([260, 31], 12, 1, 256, 32, torch.bfloat16, None, False),
 ]
 
 
@@ -145,27 +185,28 @@ def test_int8q_kernel_against_the_oracle(binding, oracle, dev, stream, case):
     c = _case(710 + heads + d, ctx, heads, kv_heads, d, block, dtype, mask, offline)
     scale = 1.0 / math.sqrt(d)
     got = int8q_cabi(binding, stream, dev, c, scale)
-    want = _oracle(oracle, c, scale, 128)
-    assert_close(got, want, TOL[dtype], "tile 128")
+    want = _oracle(oracle, c, scale, "own")
+    assert_close(got, want, TOL[dtype], "the library's tile")
     # the reference's criterion: compared with the whole context as one tile, no worse than the tiled golden
     ok, rates = _double_golden(_oracle(oracle, c, scale, None), want, got.float().cpu().numpy(), dtype)
     assert ok, rates
     assert float(got.float().abs().max()) > 0
 
 
-def test_int8q_pieces_are_capped_at_64_tiles(binding, oracle, dev, stream):
-    """A piece never has more than 64 tiles, whatever pieceTiles asks for (a wave keeps a piece's block ids in one
-    register): a context of 71 tiles with pieceTiles = 100 is cut like pieceTiles = 64 cuts it, into 36 + 35 tiles.
-    Offline quantisation shows the cut in the int8 weights, so the oracle with one piece must differ where the
-    oracle with the capped cut matches."""
+def test_int8q_long_pieces_and_small_blocks(binding, oracle, dev, stream):
+    """A context of 71 units of 128 tokens in one piece (pieceTiles = 100) and in two (pieceTiles = 64: 36 + 35 units),
+    offline, where the cut shows in the int8 weights; then blocks of 64 tokens with two KV heads."""
     ctx, heads, kv_heads, d, block, dtype = [9000, 130], 4, 1, 64, 128, torch.float16
     c = _case(911, ctx, heads, kv_heads, d, block, dtype, None, True)
     scale = 1.0 / math.sqrt(d)
-    got = int8q_cabi(binding, stream, dev, c, scale, piece_tiles=100)
-    assert torch.equal(got, int8q_cabi(binding, stream, dev, c, scale, piece_tiles=64))
-    assert_close(got, _oracle(oracle, c, scale, 128, piece_tiles=64), TOL[dtype], "capped pieces")
-    whole = _oracle(oracle, c, scale, 128, piece_tiles=100)
-    assert np.abs(whole - _oracle(oracle, c, scale, 128, piece_tiles=64)).max() > 0
+    whole = _oracle(oracle, c, scale, "own", piece_tiles=100)
+    halves = _oracle(oracle, c, scale, "own", piece_tiles=64)
+    assert np.abs(whole - halves).max() > 0
+    assert_close(int8q_cabi(binding, stream, dev, c, scale, piece_tiles=100), whole, TOL[dtype], "one piece")
+    assert_close(int8q_cabi(binding, stream, dev, c, scale, piece_tiles=64), halves, TOL[dtype], "two pieces")
+    c = _case(912, ctx, 4, 2, d, 64, dtype, None, True)
+    got = int8q_cabi(binding, stream, dev, c, scale, piece_tiles=32)
+    assert_close(got, _oracle(oracle, c, scale, "own", piece_tiles=32), TOL[dtype], "blocks of 64 tokens")
 
 
 def test_int8q_rejects_what_it_cannot_run(binding, dev, stream):
@@ -214,9 +255,12 @@ def test_paged_attention_operation_with_int8_queries(binding, oracle, dev, strea
         out = torch.full((c["rows"], heads, d), 7.0, dtype=dtype, device=dev)
         op.run(ins, outputs=[out], host_inputs={4: lens})
     stream.synchronize()
-    # the operation leaves the cut of long contexts to the library (pieces of at least four tiles here): online that
-    # moves no int8 weight, offline it does (the weights are taken against each piece's own running maximum)
-    want = _oracle(oracle, c, scale, 128, piece_tiles=4)
+    # the operation leaves the cut of long contexts to the library (equal shares of the list of tiles, see
+    # library_cuts): online that moves no int8 weight, offline it does (the weights are taken against each piece's own
+    # running maximum)
+    cuts = library_cuts(c, torch.cuda.get_device_properties(dev).multi_processor_count)
+    assert cuts
+    want = _oracle(oracle, c, scale, "own", piece_cuts=cuts)
     assert_close(out, want, TOL[dtype], "operation")
     assert torch.equal(out, int8q_cabi(binding, stream, dev, c, scale, piece_tiles=0))
     ok, rates = _double_golden(_oracle(oracle, c, scale, None), want, out.float().cpu().numpy(), dtype)
