@@ -97,7 +97,6 @@ struct Args {
     int64_t maskHeadStride; // elements between the mask rows of two heads (0: shared)
     int32_t H;
     int32_t G;
-    int32_t numRows;
     int32_t maxBlocksPerSeq;
     int32_t blockSize;
     int32_t bf16; // outputs (and mask values) are bf16 instead of fp16
@@ -809,7 +808,6 @@ extern "C" int atbmi_pa_int8q_decode(const AtbmiPaInt8QCall *call, void *workspa
     a.maskHeadStride = call->maskHeadStride;
     a.H = call->numHeads;
     a.G = call->numKvHeads;
-    a.numRows = static_cast<int32_t>(lay.pieces.size());
     a.maxBlocksPerSeq = call->maxBlocksPerSeq;
     a.blockSize = call->blockSize;
     a.bf16 = call->outDtype == ATBMI_BF16 ? 1 : 0;

@@ -193,6 +193,24 @@ def test_int8q_kernel_against_the_oracle(binding, oracle, dev, stream, case):
     assert float(got.float().abs().max()) > 0
 
 
+@pytest.mark.parametrize("offline", [False, True])
+def test_int8q_library_cut_on_many_short_and_one_long_sequence(binding, oracle, dev, stream, offline):
+    """pieceTiles = 0 on shapes that stress the walk over pieces: 200 sequences of 0 .. 150 tokens (pieces of one to
+    three tiles, so the requests run one or two pieces ahead of the arithmetic), workgroups of six waves (12 KV
+    heads); then one sequence of 20 000 tokens, which every share boundary cuts."""
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    rng = np.random.Generator(np.random.PCG64(77))
+    ctx = rng.integers(0, 151, size=200).astype(np.int32)
+    ctx[:4] = [0, 1, 64, 65]
+    for case_ctx, heads, kv_heads, d, block, mask in ((ctx, 12, 12, 128, 32, "norm"), ([20000], 8, 2, 128, 128, None)):
+        c = _case(930 + len(case_ctx), case_ctx, heads, kv_heads, d, block, torch.float16, mask, offline)
+        scale = 1.0 / math.sqrt(d)
+        cuts = library_cuts(c, cus)
+        assert cuts
+        got = int8q_cabi(binding, stream, dev, c, scale, piece_tiles=0)
+        assert_close(got, _oracle(oracle, c, scale, "own", piece_cuts=cuts), TOL[torch.float16], "the library's cut")
+
+
 def test_int8q_long_pieces_and_small_blocks(binding, oracle, dev, stream):
     """A context of 71 units of 128 tokens in one piece (pieceTiles = 100) and in two (pieceTiles = 64: 36 + 35 units),
     offline, where the cut shows in the int8 weights; then blocks of 64 tokens with two KV heads."""
