@@ -20,9 +20,9 @@ typedef uint32_t Vec16 __attribute__((ext_vector_type(4)));
 typedef uint32_t Vec8 __attribute__((ext_vector_type(2)));
 
 // Every byte is written once: the non-temporal hint keeps the stream from displacing what the
-// attention kernels want to find in the caches. (Loads stay ordinary: a source block with several
-// destinations is then fetched from HBM once; with the hint on the loads BlockCopy ran at less than
-// half the rate, PagedCacheLoad the same.)
+// attention kernels want to find in the caches. (BlockCopy's loads stay ordinary: a source block with
+// several destinations is then fetched from HBM once; with the hint on the loads it ran at less than
+// half the rate.)
 template <typename VecT> __device__ __forceinline__ void StoreOnce(VecT *p, VecT v)
 {
     __builtin_nontemporal_store(v, p);
@@ -198,7 +198,10 @@ __global__ __launch_bounds__(MOVE_THREADS) void PagedCacheLoadKernel(
                     const int64_t r = srcRow[tok];
                     if (r >= 0) {
                         live[k] = true;
-                        v[k] = from[CacheVector<NZ>(r, col, perRow, perPiece, blockSize)];
+                        // (token-major rows are read once, in whole cache lines: the non-temporal hint is worth 3 %;
+                        // on the 32-byte pieces of the fractal layout it costs 40 %)
+                        const VecT *at = from + CacheVector<NZ>(r, col, perRow, perPiece, blockSize);
+                        v[k] = NZ ? *at : __builtin_nontemporal_load(at);
                     }
                 }
             }
