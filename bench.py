@@ -44,7 +44,7 @@ MEASURED_TRAFFIC = {
 }
 KERNEL_SOURCES = ["atbmi_common.h", "pa_internal.h", "pa_host.hip", "pa_mfma_kernel.h", "pa_mfma.hip",
                   "pa_mfma_dispatch.inc", "pa_mla_kernel.h", "pa_mla.hip", "pa_reduce.hip", "mla_int8.hip", "pa_int8q.hip"]
-OTHER_WORKLOADS = ["c2_fp16", "c3", "c4", "c5"]  # timed in the same run as the headline workload
+OTHER_WORKLOADS = ["c2_fp16", "c3", "c3_int8q", "c4", "c5"]  # timed in the same run as the headline workload
 
 
 def kernel_source_hash():
