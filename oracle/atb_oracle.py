@@ -75,7 +75,9 @@ the invariants of the mathematics (no function is left "parity unpinned"):
                       operator (:3026-3227 run it with the Ascend kernel's block size and split). Pinned by an
                       independent float64 loop version, by exactly representable cases where quantisation loses
                       nothing (= float attention over the dequantised tensors), by tile invariance in those cases,
-                      and by agreement with mla_int8_decode on a shared case
+                      by agreement with mla_int8_decode on a shared case, and, for contexts cut into pieces
+                      (:176-229), by running every piece as a sequence of its own and joining them in float64
+                      by their log-sum-exps
   mla_int8_decode     tests/apitest/opstest/python/operations/multi_latent_attention/
                       test_multi_latent_attention_int8nz.py:115-121 (exact int32 products of the int8 query and
                       cache, times a per-head descale), :276-286 (the 64 rotary channels in fp32, added before

@@ -1247,6 +1247,50 @@ def test_int8q_attention_matches_independent_loops(oracle, tile, offline):
         row += 1
 
 
+@pytest.mark.parametrize("offline", [False, True])
+def test_int8q_pieces_start_from_scratch_and_merge_by_log_sum_exp(oracle, offline):
+    """A context cut into pieces: every piece is the attention over its own tokens (computed here as a sequence of its
+    own, from the block-table entries of its tokens), and the pieces are joined as out = sum_p exp(lse_p - L) out_p
+    with lse_p = log sum exp(score) over the piece, in float64. piece_tiles with piece_unit and piece_cuts name the
+    same cuts; online the cut moves nothing but rounding."""
+    rng = _rng(180 + int(offline))
+    heads, kv_heads, d, block, tile = 4, 2, 32, 16, 16
+    q8, k8, v8, tables, ctx, kd, vd, ps = _int8q_case(rng, [300, 70, 5], heads, kv_heads, d, block)
+    kw = dict(p_scale=ps if offline else None, tile=tile)
+    # units of 64 tokens, at most 2 a piece: the 5 units of the first sequence become 2 + 2 + 1, the others stay whole
+    same = oracle.paged_attention_int8q(q8, k8, v8, tables, ctx, kd, vd, 0.09, piece_tiles=2, piece_unit=64, **kw)
+    assert np.array_equal(same, oracle.paged_attention_int8q(q8, k8, v8, tables, ctx, kd, vd, 0.09,
+                                                             piece_cuts={0: [128, 256]}, **kw))
+    cuts = {0: [128, 256], 1: [64]}
+    got = oracle.paged_attention_int8q(q8, k8, v8, tables, ctx, kd, vd, 0.09, piece_cuts=cuts, **kw)
+    assert np.array_equal(got[0], same[0]) and np.array_equal(got[2], same[2])
+    uncut = oracle.paged_attention_int8q(q8, k8, v8, tables, ctx, kd, vd, 0.09, **kw)
+    if not offline:
+        np.testing.assert_allclose(got, uncut, rtol=2e-5, atol=2e-6)
+    else:
+        assert np.abs(got - uncut).max() > 1e-4          # the weights of a piece are taken against its own maximum
+    group = heads // kv_heads
+    for b, row in ((0, 0), (1, 1)):
+        bounds = [0] + cuts[b] + [int(ctx[b])]
+        outs, lses = [], []
+        for lo, hi in zip(bounds[:-1], bounds[1:]):
+            # the piece as a sequence of its own: its blocks, its length, the same query row
+            piece = oracle.paged_attention_int8q(q8[row:row + 1], k8, v8, tables[b:b + 1, lo // block:], np.array([hi - lo]),
+                                                 kd, vd, 0.09, **kw)[0]
+            keys = np.concatenate([k8[tables[b, t // block], t % block][None] for t in range(lo, hi)]).astype(np.int64)
+            lse = []
+            for h in range(heads):
+                prod = keys[:, h // group, :] @ q8[row, h].astype(np.int64)
+                sc = (prod.astype(np.float32) * kd[h] * np.float32(0.09)).astype(np.float64)
+                lse.append(sc.max() + math.log(np.exp(sc - sc.max()).sum()))
+            outs.append(piece.astype(np.float64))
+            lses.append(np.array(lse))
+        lses = np.array(lses)                                   # [pieces, heads]
+        total = lses.max(0) + np.log(np.exp(lses - lses.max(0)).sum(0))
+        want = sum(np.exp(l - total)[:, None] * o for l, o in zip(lses, outs))
+        np.testing.assert_allclose(got[row], want, rtol=2e-5, atol=2e-6)
+
+
 def test_int8q_attention_limits_and_closed_forms(oracle):
     rng = _rng(170)
     heads, kv_heads, d = 4, 2, 64
