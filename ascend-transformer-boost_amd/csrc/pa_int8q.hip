@@ -460,12 +460,21 @@ __global__ __launch_bounds__(MaxWaves<D>() * WAVE) void PaInt8QKernel(const Args
 }
 
 // Joins the pieces of a cut sequence: out = sum_p exp(lse_p - L) O_p, L = log sum_p exp(lse_p) (reference golden
-// test_paged_attention_common.py:217-228). grid.x = (cut sequence, head); a thread takes channels of the row.
-constexpr int MERGE_THREADS = 128;
+// test_paged_attention_common.py:217-228). A thread takes four channels of one head's row (16-byte loads of the
+// partial rows, one 8-byte store); a workgroup of 256 threads takes as many heads of one cut sequence as fit (eight
+// for 128 channels); grid.x = cut sequences x ceil(heads / heads a workgroup).
+constexpr int MERGE_THREADS = 256;
 __global__ __launch_bounds__(MERGE_THREADS) void PaInt8QMergeKernel(const Args a, int D)
 {
-    const MergeRow m = a.mergeRows[blockIdx.x / a.H];
-    const int h = blockIdx.x % a.H;
+    const int perHead = D / 4;                      // threads a head
+    const int headsPerWg = MERGE_THREADS / perHead; // 16, 8 or 4
+    const int wgsPerRow = (a.H + headsPerWg - 1) / headsPerWg;
+    const MergeRow m = a.mergeRows[blockIdx.x / wgsPerRow];
+    const int h = (blockIdx.x % wgsPerRow) * headsPerWg + static_cast<int>(threadIdx.x) / perHead;
+    if (h >= a.H) {
+        return;
+    }
+    const int d = (static_cast<int>(threadIdx.x) % perHead) * 4;
     const int group = a.H / a.G;
     const int headTiles = (group + HT - 1) / HT;
     const int g = h / group;
@@ -480,19 +489,23 @@ __global__ __launch_bounds__(MERGE_THREADS) void PaInt8QMergeKernel(const Args a
     // (a piece a -inf mask emptied has lse == -inf and weighs nothing, even when every piece is like that)
     auto weightOf = [mx](float v) { return v == -INFINITY ? 0.0f : __expf(v - mx); };
     float total = 0.0f;
+    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
     for (int p = 0; p < m.numPartials; ++p) {
-        total += weightOf(a.partLse[first + p * perPartial]);
+        const float w = weightOf(a.partLse[first + p * perPartial]);
+        total += w;
+        acc += *reinterpret_cast<const f32x4 *>(a.partO + (first + p * perPartial) * D + d) * w;
     }
     const float inv = total > 0.0f ? 1.0f / total : 0.0f;
-    uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) + (static_cast<int64_t>(m.qRow) * a.H + h) * D;
-    for (int d = threadIdx.x; d < D; d += MERGE_THREADS) {
-        float acc = 0.0f;
-        for (int p = 0; p < m.numPartials; ++p) {
-            acc += weightOf(a.partLse[first + p * perPartial]) * a.partO[(first + p * perPartial) * D + d];
-        }
-        const float o = acc * inv;
-        orow[d] = a.bf16 ? FloatToBf16(o) : FloatToHalfBits(o);
+    uint16_t bits[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float o = acc[e] * inv;
+        bits[e] = a.bf16 ? FloatToBf16(o) : FloatToHalfBits(o);
     }
+    uint2 out2;
+    out2.x = static_cast<uint32_t>(bits[0]) | (static_cast<uint32_t>(bits[1]) << 16);
+    out2.y = static_cast<uint32_t>(bits[2]) | (static_cast<uint32_t>(bits[3]) << 16);
+    *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(a.out) + (static_cast<int64_t>(m.qRow) * a.H + h) * D + d) = out2;
 }
 
 // Checks the call and lists its sequences (those of length 0, or switched off, take no query row).
@@ -732,7 +745,8 @@ template <int D> int Launch(const AtbmiPaInt8QCall *call, const Args &a, const L
         return rc;
     }
     if (numMerges > 0) {
-        const unsigned mergeGrid = static_cast<unsigned>(numMerges * a.H);
+        const int headsPerWg = MERGE_THREADS / (D / 4);
+        const unsigned mergeGrid = static_cast<unsigned>(numMerges * ((a.H + headsPerWg - 1) / headsPerWg));
         PaInt8QMergeKernel<<<mergeGrid, MERGE_THREADS, 0, s>>>(a, D);
         ATBMI_HIP_CHECK(hipGetLastError());
     }

