@@ -211,6 +211,27 @@ def test_int8q_library_cut_on_many_short_and_one_long_sequence(binding, oracle, 
         assert_close(got, _oracle(oracle, c, scale, "own", piece_cuts=cuts), TOL[torch.float16], "the library's cut")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_int8q_masks_of_minus_infinity(binding, oracle, dev, stream, dtype):
+    """A mask of -inf over the first 130 tokens of a sequence (its first two tiles see nothing, and with pieces of
+    one unit its first piece reaches the merge with a log-sum-exp of -inf), over all of another (its output is
+    zero), and over a tile in the middle of a third."""
+    ctx, heads, kv_heads, d, block = [300, 70, 400], 8, 2, 128, 128
+    c = _case(940, ctx, heads, kv_heads, d, block, dtype, "norm", False)
+    m = np.zeros((3, 1, 400), np.float32)
+    m[0, 0, :130] = -np.inf
+    m[1, 0, :] = -np.inf
+    m[2, 0, 128:192] = -np.inf
+    c["mask"] = torch.from_numpy(m).to(dtype)
+    scale = 1.0 / math.sqrt(d)
+    for piece_tiles in (1, 100):
+        got = int8q_cabi(binding, stream, dev, c, scale, piece_tiles=piece_tiles)
+        want = _oracle(oracle, c, scale, "own", piece_tiles=piece_tiles)
+        assert np.isfinite(want).all() and np.abs(want[1]).max() == 0
+        assert_close(got, want, TOL[dtype], "pieces of %d units" % piece_tiles)
+        assert float(got[1].float().abs().max()) == 0
+
+
 def test_int8q_long_pieces_and_small_blocks(binding, oracle, dev, stream):
     """A context of 71 units of 128 tokens in one piece (pieceTiles = 100) and in two (pieceTiles = 64: 36 + 35 units),
     offline, where the cut shows in the int8 weights; then blocks of 64 tokens with two KV heads."""
