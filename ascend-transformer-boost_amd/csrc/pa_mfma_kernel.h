@@ -193,6 +193,9 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
     static_assert((STEP * KPR) % WAVE == 0 && (MLA || (STEP * VPR) % WAVE == 0), "pieces must split evenly");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    // eight private-tile waves: the steps each wave has left, behind the tiles (see the step loop)
+    constexpr bool BALANCED = NW == 8 && !SHARED;
+    volatile int *stepsLeft = reinterpret_cast<volatile int *>(smem + NW * WaveLdsBytes<D, DV, MLA>());
 
     const int lane = threadIdx.x % WAVE;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
@@ -693,6 +696,23 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
             }
         } else {
             for (int t = tokBegin; t < tokEnd; t += STEP) {
+                if constexpr (BALANCED) {
+                    // Two waves share a SIMD (wave w and w ^ 4), and its arbiter lets the older one issue first
+                    // whenever both are ready. With the memory system saturated that is worth 15 % more rows per
+                    // microsecond to waves 0-3, which then leave 13 us before their siblings and the launch ends with
+                    // half its requests in flight. Each wave publishes the steps it still has to do and takes the
+                    // higher issue priority while it has more left than its sibling (ties go to the younger wave).
+                    const int left = __builtin_amdgcn_readfirstlane(s1 - segBegin - (t - tokBegin) / STEP);
+                    if (lane == 0) {
+                        stepsLeft[wave] = left;
+                    }
+                    const int sibling = __builtin_amdgcn_readfirstlane(stepsLeft[wave ^ 4]);
+                    if (left > sibling || (left == sibling && wave >= 4)) {
+                        __builtin_amdgcn_s_setprio(1);
+                    } else {
+                        __builtin_amdgcn_s_setprio(0);
+                    }
+                }
                 if constexpr (PF) {
 #pragma unroll
                     for (int i = 0; i < NKP; ++i) {
@@ -817,13 +837,16 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
             }
         }
     }
+    if (BALANCED && lane == 0) {
+        stepsLeft[wave] = 0; // the sibling keeps the higher priority from here on
+    }
 }
 
 template <bool BF16, bool KV8, int D, int DV, bool MLA, bool PF, int NW, bool SHARED, bool EXT>
 int LaunchBuild(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
 {
     auto kernel = PaMfmaKernel<BF16, KV8, D, DV, MLA, PF, NW, SHARED, EXT>;
-    constexpr int lds = SHARED ? 2 * WaveLdsBytes<D, DV, MLA>() : NW * WaveLdsBytes<D, DV, MLA>();
+    constexpr int lds = SHARED ? 2 * WaveLdsBytes<D, DV, MLA>() : NW * WaveLdsBytes<D, DV, MLA>() + 64; // + stepsLeft
     static_assert(lds <= 160 * 1024, "tiles exceed the 160 KB of LDS per CU");
     const int configured = ConfigureKernelLds(reinterpret_cast<const void *>(kernel), lds);
     if (configured != OK) {
