@@ -295,6 +295,9 @@ def kernels():
         lib.atbmi_timing_read.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(i64)]
         lib.atbmi_timing_read_split.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
                                                 ctypes.POINTER(i64)]
+        lib.atbmi_timing_read_samples.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float), i64,
+                                                  ctypes.POINTER(i64)]
+        lib.atbmi_timing_whole_calls.argtypes = [i32]
         _kernels = lib
     return _kernels
 

@@ -129,6 +129,7 @@ int StaticScratch(void **ptr)
 
 std::mutex g_timingMutex;
 int g_timingEvery = 0;   // 0: off; n: bracket every n-th decode launch with events
+bool g_timingWhole = false; // no event between the attention kernel and its merge kernel: the call as one interval
 int64_t g_timingLaunch = 0;
 std::vector<TimingRecord> g_timingRecords;
 
@@ -142,6 +143,7 @@ int TimedLaunchBegin(hipStream_t stream, TimedLaunch *launch)
         if (g_timingEvery <= 0 || (g_timingLaunch++ % g_timingEvery) != 0) {
             return OK;
         }
+        launch->whole = g_timingWhole;
     }
     ATBMI_HIP_CHECK(hipEventCreate(&launch->begin));
     ATBMI_HIP_CHECK(hipEventCreate(&launch->end));
@@ -151,7 +153,7 @@ int TimedLaunchBegin(hipStream_t stream, TimedLaunch *launch)
 
 int TimedLaunchKernelDone(hipStream_t stream, const TimedLaunch &launch)
 {
-    if (launch.begin) {
+    if (launch.begin && !launch.whole) {
         ATBMI_HIP_CHECK(hipEventRecord(launch.end, stream));
     }
     return OK;
@@ -163,7 +165,10 @@ int TimedLaunchEnd(hipStream_t stream, const TimedLaunch &launch, bool merged)
         return OK;
     }
     TimingRecord rec{launch.begin, launch.end, nullptr};
-    if (merged && hipEventCreate(&rec.merged) == hipSuccess) {
+    if (launch.whole) {
+        // one interval for the whole call: its only closing event goes behind the last kernel
+        (void)hipEventRecord(rec.end, stream);
+    } else if (merged && hipEventCreate(&rec.merged) == hipSuccess) {
         (void)hipEventRecord(rec.merged, stream);
     }
     std::lock_guard<std::mutex> lock(g_timingMutex);
@@ -884,16 +889,12 @@ int DecodeImpl(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void *workspace, uint
     a.nzShift = s.kvLayout == ATBMI_PA_KV_FRACTAL_NZ ? __builtin_ctz(static_cast<unsigned>(s.blockSize)) : 0;
     a.partHalf = (plan->useMfma && PaMlaWide(s)) ? 1 : 0;
 
-    TimingRecord rec{nullptr, nullptr, nullptr};
-    bool timed = false;
-    {
-        std::lock_guard<std::mutex> lock(g_timingMutex);
-        timed = mayAllocate && g_timingEvery > 0 && (g_timingLaunch++ % g_timingEvery) == 0;
-    }
-    if (timed) {
-        ATBMI_HIP_CHECK(hipEventCreate(&rec.begin));
-        ATBMI_HIP_CHECK(hipEventCreate(&rec.end));
-        ATBMI_HIP_CHECK(hipEventRecord(rec.begin, stream));
+    TimedLaunch timed;
+    if (mayAllocate) {
+        rc = TimedLaunchBegin(stream, &timed);
+        if (rc != OK) {
+            return rc;
+        }
     }
     const int numItems = static_cast<int>(plan->items.size());
     PaStreamPlan &sp = plan->stream;
@@ -904,8 +905,8 @@ int DecodeImpl(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void *workspace, uint
     } else {
         rc = LaunchPaScalar(s, a, numItems, stream);
     }
-    if (timed) {
-        ATBMI_HIP_CHECK(hipEventRecord(rec.end, stream));
+    if (rc == OK) {
+        rc = TimedLaunchKernelDone(stream, timed);
     }
     bool merged = false;
     if (rc == OK) {
@@ -917,14 +918,8 @@ int DecodeImpl(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void *workspace, uint
             rc = LaunchPaReduce(s, a, static_cast<int>(plan->reduceSeqs.size()), stream);
         }
     }
-    if (timed) {
-        if (merged && rc == OK && hipEventCreate(&rec.merged) == hipSuccess) {
-            (void)hipEventRecord(rec.merged, stream);
-        }
-        std::lock_guard<std::mutex> lock(g_timingMutex);
-        g_timingRecords.push_back(rec);
-    }
-    return rc;
+    const int closed = TimedLaunchEnd(stream, timed, merged && rc == OK);
+    return rc != OK ? rc : closed;
 }
 
 } // namespace
@@ -985,27 +980,71 @@ extern "C" int atbmi_timing_enable(int32_t enable)
     return OK;
 }
 
-extern "C" int atbmi_timing_read_split(double *kernelMs, double *withMergeMs, int64_t *launches)
+extern "C" int atbmi_timing_whole_calls(int32_t whole)
+{
+    std::lock_guard<std::mutex> lock(g_timingMutex);
+    g_timingWhole = whole != 0;
+    return OK;
+}
+
+extern "C" int atbmi_timing_read_samples(float *kernelMs, float *withMergeMs, int64_t capacity, int64_t *launches)
 {
     std::vector<TimingRecord> records;
     {
         std::lock_guard<std::mutex> lock(g_timingMutex);
         records.swap(g_timingRecords);
     }
-    double sum = 0.0, sumMerged = 0.0;
+    int64_t count = 0;
     for (const TimingRecord &r : records) {
         hipEvent_t last = r.merged ? r.merged : r.end;
         ATBMI_HIP_CHECK(hipEventSynchronize(last));
         float ms = 0.0f, msMerged = 0.0f;
         ATBMI_HIP_CHECK(hipEventElapsedTime(&ms, r.begin, r.end));
         ATBMI_HIP_CHECK(hipEventElapsedTime(&msMerged, r.begin, last));
-        sum += ms;
-        sumMerged += msMerged;
+        if (count < capacity) {
+            if (kernelMs) {
+                kernelMs[count] = ms;
+            }
+            if (withMergeMs) {
+                withMergeMs[count] = msMerged;
+            }
+            ++count;
+        }
         (void)hipEventDestroy(r.begin);
         (void)hipEventDestroy(r.end);
         if (r.merged) {
             (void)hipEventDestroy(r.merged);
         }
+    }
+    if (launches) {
+        *launches = count;
+    }
+    return OK;
+}
+
+extern "C" int atbmi_timing_read_split(double *kernelMs, double *withMergeMs, int64_t *launches)
+{
+    std::vector<float> kernel, merged;
+    size_t pending = 0;
+    {
+        std::lock_guard<std::mutex> lock(g_timingMutex);
+        pending = g_timingRecords.size();
+    }
+    try {
+        kernel.resize(pending);
+        merged.resize(pending);
+    } catch (const std::bad_alloc &) {
+        return Fail(ERR_OUT_OF_HOST_MEMORY, "timing_read: out of host memory");
+    }
+    int64_t count = 0;
+    const int rc = atbmi_timing_read_samples(kernel.data(), merged.data(), static_cast<int64_t>(pending), &count);
+    if (rc != OK) {
+        return rc;
+    }
+    double sum = 0.0, sumMerged = 0.0;
+    for (int64_t i = 0; i < count; ++i) {
+        sum += kernel[static_cast<size_t>(i)];
+        sumMerged += merged[static_cast<size_t>(i)];
     }
     if (kernelMs) {
         *kernelMs = sum;
@@ -1014,7 +1053,7 @@ extern "C" int atbmi_timing_read_split(double *kernelMs, double *withMergeMs, in
         *withMergeMs = sumMerged;
     }
     if (launches) {
-        *launches = static_cast<int64_t>(records.size());
+        *launches = count;
     }
     return OK;
 }

@@ -52,6 +52,7 @@ int LaunchPaMfmaInt8(const AtbmiPaShape &shape, const PaArgs &args, const PaStre
 struct TimedLaunch {
     hipEvent_t begin = nullptr;
     hipEvent_t end = nullptr;
+    bool whole = false; // atbmi_timing_whole_calls: no event between the attention kernel and its merge kernel
 };
 int TimedLaunchBegin(hipStream_t stream, TimedLaunch *launch);
 int TimedLaunchKernelDone(hipStream_t stream, const TimedLaunch &launch);

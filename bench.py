@@ -5,13 +5,19 @@ on one MI355X, synthetic data of the named configuration.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2]
 
 Prints ONE JSON line: whole-step throughput (tokens/s = sequences decoded per
-second, inputs resident in HBM), the attention kernel's achieved HBM bandwidth
-against the 8 TB/s roofline (algorithmic bytes / mean kernel time from HIP
-events on the launch stream; `frac_with_merge` counts the merge kernel that
-follows it as well), and the CPU oracle timed on a bounded sample of the same
-workload. Run without --config, the line describes the bf16 8B-shaped step (C2)
-and carries, under "configs", the same measurements of the other workloads of
-the benchmark (C2 in fp16, C3 int8-KV, C4 skewed, C5 MLA), fewer steps each.
+second, inputs resident in HBM; --warmup untimed steps, then exactly --steps
+timed ones between two synchronisations, no events inside), the attention
+kernel's achieved HBM bandwidth against the 8 TB/s roofline, and the CPU oracle
+timed on a bounded sample of the same workload. The kernel figures come from two
+more passes over the same inputs, attention only, at least 100 launches each:
+one with HIP events on the launch stream around every attention kernel (mean,
+median, 10th and 90th percentile of its duration), one with events around every
+whole call, attention kernel + merge kernel, nothing between them
+(`frac_with_merge`). Run without --config, the line describes the bf16
+8B-shaped step (C2) and carries, under "configs", the same measurements of the
+other workloads of the benchmark (C2 in fp16, C3 int8-KV, C4 skewed, C5 MLA) and,
+under "reference_perf_rows", the three shapes the reference publishes its own
+timings for.
 """
 import argparse
 import hashlib
@@ -27,30 +33,36 @@ if ROOT not in sys.path:
 PKG = "ascend-transformer-boost_amd"
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes one attention launch moves (attention kernel + its merge kernel), from rocprofv3 FETCH_SIZE /
-# WRITE_SIZE counter runs of this script, scaled by what the same counters read for a 256 MiB copy
-# (--calibrate-copy). Each figure names the profile summary it comes from and the hash of the attention
-# kernel sources it was measured on: a changed workload or changed kernels report null, not a stale figure.
-MEASURED_TRAFFIC = {
-    # (workload, algorithmic bytes): (HBM bytes, summary under profiles/, kernel source hash)
-    ("c2", 651658484): (664832843, "pa_mfma_bf16_d128_c2_hbm_traffic.md", "ca02ccf6b798"),
-    ("c3", 1364204576): (1394523909, "pa_mfma_int8_d128_c3_kernel_trace_and_traffic.md", "ca02ccf6b798"),
-    ("c2_mtp4", 656075180): (707806638, "pa_mfma_bf16_d128_c2_four_query_tokens_trace_and_traffic.md", "ca02ccf6b798"),
-    ("c2_alibi", 661824180): (675676309, "pa_mfma_bf16_d128_c2_alibi_mask_trace_and_traffic.md", "ca02ccf6b798"),
-    ("c5", 253384304): (349335962, "pa_mla_wide_bf16_d576_c5_trace_mfma_traffic.md", "ca02ccf6b798"),
-    ("c5_split", 253384304): (349366477, "pa_mla_wide_split_bf16_c5_trace_and_traffic.md", "ca02ccf6b798"),
-    ("c5_int8", 144501360): (147183002, "mla_int8_nz_cache_c5_sizes_trace_counters_traffic.md", "ca02ccf6b798"),
-    ("c3_int8q", 1363148320): (1394160128, "pa_int8q_d128_c3_sizes_trace_counters_traffic.md", "ca02ccf6b798"),
+# The sources each workload's attention and merge kernels are compiled from: a traffic figure is tied to the hash
+# of exactly these, so an edit elsewhere leaves it standing and an edit here withdraws it.
+_COMMON = ["atbmi_common.h", "pa_internal.h", "pa_host.hip", "pa_reduce.hip"]
+_MFMA = _COMMON + ["pa_mfma_kernel.h", "pa_mfma.hip", "pa_mfma_dispatch.inc"]
+_MLA = _MFMA + ["pa_mla_kernel.h", "pa_mla.hip"]
+WORKLOAD_SOURCES = {
+    "c2": _MFMA + ["pa_mfma_bf16.hip"], "c2_alibi": _MFMA + ["pa_mfma_bf16.hip"], "c2_norm": _MFMA + ["pa_mfma_bf16.hip"],
+    "c2_mtp4": _MFMA + ["pa_mfma_bf16.hip"], "c2_bnsd": _MFMA + ["pa_mfma_bf16.hip"],
+    "c1": _MFMA + ["pa_mfma_f16.hip"], "c2_fp16": _MFMA + ["pa_mfma_f16.hip"], "c4": _MFMA + ["pa_mfma_f16.hip"],
+    "c3": _MFMA + ["pa_mfma_int8.hip"],
+    "c5": _MLA, "c5_split": _MLA, "c5_nz": _MLA,
+    "c5_int8": ["atbmi_common.h", "pa_internal.h", "mla_int8.hip"],
+    "c3_int8q": ["atbmi_common.h", "pa_internal.h", "pa_int8q.hip"],
 }
-KERNEL_SOURCES = ["atbmi_common.h", "pa_internal.h", "pa_host.hip", "pa_mfma_kernel.h", "pa_mfma.hip",
-                  "pa_mfma_dispatch.inc", "pa_mla_kernel.h", "pa_mla.hip", "pa_reduce.hip", "mla_int8.hip", "pa_int8q.hip"]
+
+# HBM bytes one attention call moves (attention kernel + its merge kernel), from rocprofv3 FETCH_SIZE /
+# WRITE_SIZE counter runs of this script, scaled by what the same counters read for a 256 MiB copy
+# (--calibrate-copy). Each figure names the profile summary it comes from and the hash of its workload's kernel
+# sources at the time it was measured: a changed workload or changed kernels report null, not a stale figure.
+MEASURED_TRAFFIC = {
+    # (workload, algorithmic bytes): (HBM bytes, summary under profiles/, source hash of the workload)
+}
 OTHER_WORKLOADS = ["c2_fp16", "c3", "c3_int8q", "c4", "c5"]  # timed in the same run as the headline workload
+MIN_KERNEL_LAUNCHES = 100  # launches behind every kernel figure, whatever --steps says
 
 
-def kernel_source_hash():
-    """Short hash of the attention kernels' sources (what MEASURED_TRAFFIC figures are tied to)."""
+def kernel_source_hash(workload):
+    """Short hash of the sources `workload`'s attention and merge kernels are built from."""
     h = hashlib.sha256()
-    for name in KERNEL_SOURCES:
+    for name in WORKLOAD_SOURCES[workload]:
         with open(os.path.join(ROOT, PKG, "csrc", name), "rb") as f:
             h.update(f.read())
     return h.hexdigest()[:12]
@@ -274,38 +286,62 @@ def run_workload(pkg, name, steps, warmup, attention_only=False, kernel_events=T
             dst = torch.empty_like(src)
             dst.copy_(src)
         stream.synchronize()
+    import numpy as np
+
+    def timed_pass(count, whole):
+        """`count` attention calls on the same inputs, every one bracketed with HIP events on the launch stream:
+        around the attention kernel (whole = False) or around attention + merge as one interval (whole = True).
+        Returns the durations in milliseconds."""
+        k.atbmi_timing_whole_calls(1 if whole else 0)
+        k.atbmi_timing_enable(1)
+        for _ in range(count):
+            pa.run(pa_in, outputs=[out], host_inputs=host_inputs)
+        stream.synchronize()
+        first = (ctypes.c_float * count)()
+        second = (ctypes.c_float * count)()
+        got = ctypes.c_int64(0)
+        rc = k.atbmi_timing_read_samples(first, second, count, ctypes.byref(got))
+        k.atbmi_timing_enable(0)
+        k.atbmi_timing_whole_calls(0)
+        assert rc == 0, b.last_kernel_error()
+        return np.array((second if whole else first)[:got.value], dtype=np.float64)
+
     with torch.cuda.stream(stream):
         for _ in range(warmup):
             one_step()
         stream.synchronize()
         torch.cuda.synchronize()
-        # every 4th attention launch is bracketed with HIP events on the launch stream
-        k.atbmi_timing_enable(4 if kernel_events else 0)
         t0 = time.perf_counter()
         for _ in range(steps):
             one_step()
         stream.synchronize()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
-    kernel_total = ctypes.c_double(0)
-    merged_total = ctypes.c_double(0)
-    launches = ctypes.c_int64(0)
-    k.atbmi_timing_read_split(ctypes.byref(kernel_total), ctypes.byref(merged_total), ctypes.byref(launches))
-    k.atbmi_timing_enable(0)
+        kernel_samples = with_merge_samples = np.zeros(0)
+        if kernel_events:
+            launches_wanted = max(steps, MIN_KERNEL_LAUNCHES)
+            kernel_samples = timed_pass(launches_wanted, whole=False)
+            with_merge_samples = timed_pass(launches_wanted, whole=True)
+
+    def spread(samples):
+        if len(samples) == 0:
+            return {"mean": 0.0, "median": 0.0, "p10": 0.0, "p90": 0.0}
+        return {"mean": float(samples.mean()), "median": float(np.median(samples)),
+                "p10": float(np.percentile(samples, 10)), "p90": float(np.percentile(samples, 90))}
 
     ms_per_step = (t1 - t0) * 1e3 / steps
     alg_bytes = w.algorithmic_bytes(cfg, step["layout"]["ctx"])
-    kernel_ms = kernel_total.value / max(1, launches.value)
-    with_merge_ms = merged_total.value / max(1, launches.value)
+    kernel_stats, with_merge_stats = spread(kernel_samples), spread(with_merge_samples)
+    kernel_ms, with_merge_ms = kernel_stats["mean"], with_merge_stats["mean"]
     achieved = alg_bytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
     with_merge = alg_bytes / (with_merge_ms * 1e-3) / 1e9 if with_merge_ms > 0 else 0.0
     traffic, source = None, None
     entry = MEASURED_TRAFFIC.get((name, alg_bytes))
     if entry is not None:
-        if entry[2] == kernel_source_hash():
+        if entry[2] == kernel_source_hash(name):
             traffic, source = entry[0], "profiles/" + entry[1]
         else:
-            source = "none: the attention kernels changed since profiles/%s was taken" % entry[1]
+            source = "none: the kernels of this workload changed since profiles/%s was taken" % entry[1]
     measured = {
         "workload": DESCRIPTIONS[name],
         "step": ("%s only" if attention_only else "ReshapeAndCache + %s (Setup + Execute each)") % (
@@ -319,9 +355,14 @@ def run_workload(pkg, name, steps, warmup, attention_only=False, kernel_events=T
         "roofline": {"bound": "hbm", "kernel": "paged attention decode", "achieved": achieved,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
                      "frac_with_merge": with_merge / HBM_PEAK_GBPS, "traffic": traffic, "traffic_source": source,
-                     "algorithmic_bytes": alg_bytes, "kernel_ms": kernel_ms, "kernel_with_merge_ms": with_merge_ms,
-                     "launches": launches.value},
+                     "algorithmic_bytes": alg_bytes, "kernel_ms": kernel_ms, "kernel_ms_spread": kernel_stats,
+                     "kernel_with_merge_ms": with_merge_ms, "kernel_with_merge_ms_spread": with_merge_stats,
+                     "launches": int(len(kernel_samples)),
+                     "method": "HIP events on the launch stream around every attention kernel of %d attention-only calls; "
+                               "frac_with_merge from a second pass of as many calls with one interval around attention + "
+                               "merge kernel" % len(kernel_samples)},
         "step_hbm_gbps": alg_bytes / (ms_per_step * 1e-3) / 1e9,
+        "kernel_source_hash": kernel_source_hash(name),
     }
     baseline = cpu_baseline(pkg, step, cfg, scale) if want_cpu_baseline else None
     if rac is not None:
@@ -331,6 +372,69 @@ def run_workload(pkg, name, steps, warmup, attention_only=False, kernel_events=T
     del step, out, pa_in
     torch.cuda.empty_cache()
     return measured, baseline
+
+
+def reference_perf_rows(pkg, calls=200, warmup=20):
+    """The three shapes the reference keeps timings for (its QA baselines: one whole operator call each, on an
+    Ascend NPU it does not name): Setup + Execute + stream synchronisation per call here, microseconds. Reference:
+    tests/high_level_test/PagedAttentionOperation/Performance/PagedAttentionOperation_Perf_TestCase.csv:2 with
+    PagedAttentionOperation_BaseLine.csv:2, and tests/high_level_test/ReshapeAndCacheOperation/Performance/
+    ReshapeAndCacheOperation_Perf_TestCase.csv:2-3 with ReshapeAndCacheOperation_BaseLine.csv:2-3."""
+    import numpy as np
+    import torch
+    b = pkg.binding
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.Stream(device=dev)
+    ctx = b.Context(stream)
+    gen = torch.Generator(device=dev).manual_seed(7)
+    rows = []
+
+    def time_calls(call):
+        with torch.cuda.stream(stream):
+            for _ in range(warmup):
+                call()
+                stream.synchronize()
+            samples = []
+            for _ in range(calls):
+                t0 = time.perf_counter()
+                call()
+                stream.synchronize()
+                samples.append((time.perf_counter() - t0) * 1e6)
+        samples = np.array(samples)
+        return {"median_us": float(np.median(samples)), "p10_us": float(np.percentile(samples, 10)),
+                "p90_us": float(np.percentile(samples, 90)), "calls": calls}
+
+    with torch.cuda.stream(stream):
+        caches = [torch.randn((4, 128, 1, 128), generator=gen, device=dev, dtype=torch.float16) for _ in range(2)]
+        # PagedAttentionOperation1: q [1, 8, 128], caches [4, 128, 1, 128], block table [1, 4], 8 heads over 1 KV head
+        q = torch.randn((1, 8, 128), generator=gen, device=dev, dtype=torch.float16)
+        tables = torch.arange(4, dtype=torch.int32, device=dev).reshape(1, 4)
+        lens = torch.tensor([512], dtype=torch.int32)
+        out = torch.empty((1, 8, 128), dtype=torch.float16, device=dev)
+        pa = b.OperationRunner("PagedAttentionOperation",
+                               b.PagedAttentionParam(headNum=8, kvHeadNum=1, qkScale=0.0883883461356163), ctx)
+        pa_in = [q, caches[0], caches[1], tables, lens.to(dev)]
+    measured = time_calls(lambda: pa.run(pa_in, outputs=[out], host_inputs={4: lens}))
+    rows.append(dict(measured, case="PagedAttentionOperation1", shape="q [1,8,128], caches [4,128,1,128], table [1,4], "
+                     "context 512 (the dump's own length is not in the table: the longest the block table holds)",
+                     reference_us=200.555))
+    pa.close()
+    for case, tokens, ref_us in (("ReshapeAndCacheOperation1", 256, 206.315), ("ReshapeAndCacheOperation2", 1, 187.805)):
+        with torch.cuda.stream(stream):
+            key = torch.randn((tokens, 1, 128), generator=gen, device=dev, dtype=torch.float16)
+            value = torch.randn((tokens, 1, 128), generator=gen, device=dev, dtype=torch.float16)
+            slots = torch.randperm(512, generator=gen, device=dev)[:tokens].to(torch.int32)
+            rac = b.OperationRunner("ReshapeAndCacheOperation", b.ReshapeAndCacheParam(), ctx)
+            rac_in = [key, value, caches[0], caches[1], slots]
+        measured = time_calls(lambda: rac.run(rac_in, outputs=[caches[0], caches[1]]))
+        rows.append(dict(measured, case=case, shape="key / value [%d,1,128], caches [4,128,1,128]" % tokens,
+                         reference_us=ref_us))
+        rac.close()
+    ctx.close()
+    return {"what": "Setup + Execute + stream synchronisation of one operator call, host clock, fp16; reference_us is the "
+                    "reference's own QA baseline for the same shape on an unnamed Ascend NPU (context, not a comparison "
+                    "on equal hardware)",
+            "rows": rows}
 
 
 def main():
@@ -373,7 +477,7 @@ def main():
         "config": {"workload": m["workload"], "step": m["step"], "context_tokens": m["context_tokens"]},
         "roofline": m["roofline"],
         "step_hbm_gbps": m["step_hbm_gbps"],
-        "kernel_source_hash": kernel_source_hash(),
+        "kernel_source_hash": m["kernel_source_hash"],
     }
     if baseline is not None:
         result["cpu_baseline"] = baseline
@@ -386,6 +490,7 @@ def main():
                                  kernel_events=not args.no_kernel_events)
             others[name] = om
         result["configs"] = others
+        result["reference_perf_rows"] = reference_perf_rows(pkg)
     print(json.dumps(result))
 
 

@@ -621,6 +621,12 @@ int atbmi_timing_read(double *totalMs, int64_t *launches);
 /* The same, and also the sum from the start of the attention kernel to the end of the merge kernel that
  * follows it (equal to the first sum for calls that need no merge). Any pointer may be NULL. */
 int atbmi_timing_read_split(double *kernelMs, double *withMergeMs, int64_t *launches);
+/* The same record launch by launch (milliseconds), at most `capacity` launches; clears the record. */
+int atbmi_timing_read_samples(float *kernelMs, float *withMergeMs, int64_t capacity, int64_t *launches);
+/* whole != 0: a timed call is bracketed as ONE interval, from in front of the attention kernel to behind its merge
+ * kernel, with no event between the two (an event there costs the merge kernel about a microsecond of stream time);
+ * both figures of a read are then that interval. 0 (the default): three events, as described above. */
+int atbmi_timing_whole_calls(int32_t whole);
 
 #ifdef __cplusplus
 }
