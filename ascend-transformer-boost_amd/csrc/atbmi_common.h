@@ -148,6 +148,7 @@ struct PaStreamPlan {
     int32_t headTiles;        // query-head tiles per KV head
     int32_t foldTokens;       // query tokens of one sequence that may share a head tile (1: none do);
                               // a partial slot then holds foldTokens x H rows
+    int32_t maxRangesPerRow;  // most wave ranges any one pass spans (the merge kernel sizes itself by it)
     PaSeq inlineSeqs[PA_INLINE_SEQS + 1];
     uint16_t inlineFirst[PA_INLINE_RANGES];
 };

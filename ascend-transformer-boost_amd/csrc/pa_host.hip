@@ -438,13 +438,14 @@ int PlanStream(AtbmiPaPlan *plan)
             plan->firstSeq[static_cast<size_t>(r)] = static_cast<uint16_t>(std::min(cursor, 0xffff));
         }
         plan->streamNeedsReduce = false;
+        int32_t maxRanges = 1;
         for (int i = 0; i < numSeqs; ++i) {
             const int32_t first = PaRangeOf(plan->seqTable[i].stepBegin, static_cast<int32_t>(steps), waveRanges);
             const int32_t last = PaRangeOf(plan->seqTable[i + 1].stepBegin - 1, static_cast<int32_t>(steps), waveRanges);
             if (first != last) {
                 plan->streamNeedsReduce = true;
-                break;
             }
+            maxRanges = std::max(maxRanges, last - first + 1);
         }
 
         PaStreamPlan &sp = plan->stream;
@@ -458,6 +459,7 @@ int PlanStream(AtbmiPaPlan *plan)
         sp.headGroups = headGroups;
         sp.headTiles = headTiles;
         sp.foldTokens = fold;
+        sp.maxRangesPerRow = maxRanges;
         // firstSeq is a 16-bit table: batches beyond 65535 sequences go through memory as 16-bit too,
         // so they are refused here rather than silently truncated
         if (numSeqs > 0xffff) {

@@ -219,6 +219,139 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaA
     }
 }
 
+// The same merge for plans whose rows span many ranges (a few long sequences in a batch): SLICES threads share each
+// piece of an output row, thread s taking the ranges s, s + SLICES, ... eight at a time; each ends with a maximum, a
+// sum of weights and a weighted sum of its own, and the first of them joins these through LDS. A row of 40 ranges is
+// then two memory round trips, not five. fp32 partial rows of up to 128 channels.
+constexpr int SLICES = 4;
+template <bool BF16>
+__global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceSlicedKernel(const PaArgs a, const PaStreamPlan p)
+{
+    constexpr int CH = 4;
+    constexpr int MAX_HELD = 8;
+    __shared__ float joined[REDUCE_THREADS * (CH + 2)];
+    const int vecs = a.Dv / CH;                  // pieces per row
+    const int rowThreads = vecs * SLICES;
+    const int rowsPerWg = REDUCE_THREADS / rowThreads; // (>= 1: the launcher sends wider rows to the other kernel)
+    const int rowsPerSlot = a.H * p.foldTokens;
+    const int tid = threadIdx.x;
+    const int slice = (tid / vecs) % SLICES;
+    const int c = tid % vecs;
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * rowsPerWg + tid / rowThreads;
+    // (every thread stays to the barrier; a thread without a row to merge works on nothing)
+    bool active = tid < rowsPerWg * rowThreads && row < static_cast<int64_t>(p.numSeqs) * rowsPerSlot;
+    const int b = active ? static_cast<int>(row / rowsPerSlot) : 0;
+    const int tok = active ? static_cast<int>(row % rowsPerSlot) / a.H : 0;
+    const int h = active ? static_cast<int>(row % a.H) : 0;
+    const PaSeq sq = p.seqs ? p.seqs[b] : p.inlineSeqs[b];
+    const int begin = sq.stepBegin;
+    const int end = (p.seqs ? p.seqs[b + 1] : p.inlineSeqs[b + 1]).stepBegin;
+    const int wrFirst = PaRangeOf(begin, p.totalSteps, p.numWaveRanges);
+    const int wrLast = PaRangeOf(end - 1, p.totalSteps, p.numWaveRanges);
+    active = active && tok < sq.nTok && wrFirst != wrLast;
+    const int firstOdd = PaRangeBegin(wrFirst, p.totalSteps, p.numWaveRanges) >= begin ? 0 : 1;
+    const int64_t stride = 2 * static_cast<int64_t>(rowsPerSlot);
+    const int64_t phEven = 2 * static_cast<int64_t>(wrFirst) * rowsPerSlot + static_cast<int64_t>(tok) * a.H + h;
+    const int64_t ph0 = phEven + static_cast<int64_t>(firstOdd) * rowsPerSlot;
+    const int count = active ? wrLast - wrFirst + 1 : 0;
+    auto rowOf = [&](int k) { return k == 0 ? ph0 : phEven + k * stride; };
+    auto pow2 = [](float x) { return __builtin_amdgcn_exp2f(x); };
+
+    float acc[CH] = {0.0f, 0.0f, 0.0f, 0.0f};
+    float sum = 0.0f;
+    float mx = -INFINITY;
+#pragma unroll 1
+    for (int k0 = slice; k0 < count; k0 += MAX_HELD * SLICES) {
+        float lseHeld[MAX_HELD];
+        PartialPiece<false> piece[MAX_HELD];
+#pragma unroll
+        for (int k = 0; k < MAX_HELD; ++k) {
+            lseHeld[k] = -INFINITY;
+            piece[k].Clear();
+            if (k0 + k * SLICES < count) {
+                const int64_t ph = rowOf(k0 + k * SLICES);
+                lseHeld[k] = a.partLse[ph];
+                piece[k].Load(a.partO, ph * a.Dv + c * CH);
+            }
+        }
+        float mNew = mx;
+#pragma unroll
+        for (int k = 0; k < MAX_HELD; ++k) {
+            mNew = fmaxf(mNew, lseHeld[k]);
+        }
+        if (k0 > slice && mNew > mx) {
+            const float keep = pow2(mx - mNew);
+            sum *= keep;
+#pragma unroll
+            for (int e = 0; e < CH; ++e) {
+                acc[e] *= keep;
+            }
+        }
+        mx = mNew;
+#pragma unroll
+        for (int k = 0; k < MAX_HELD; ++k) {
+            const float w = mx == -INFINITY ? 0.0f : pow2(lseHeld[k] - mx);
+            sum += w;
+#pragma unroll
+            for (int e = 0; e < CH; ++e) {
+                acc[e] += w * piece[k].Get(e, false);
+            }
+        }
+    }
+    float *mine = joined + tid * (CH + 2);
+    mine[0] = mx;
+    mine[1] = sum;
+#pragma unroll
+    for (int e = 0; e < CH; ++e) {
+        mine[2 + e] = acc[e];
+    }
+    __syncthreads();
+    if (!active || slice != 0) {
+        return;
+    }
+    // join the slices: the usual rescaling to the common maximum
+    float top = mx;
+#pragma unroll
+    for (int s = 1; s < SLICES; ++s) {
+        top = fmaxf(top, joined[(tid + s * vecs) * (CH + 2)]);
+    }
+    const float own = top == -INFINITY ? 0.0f : pow2(mx - top);
+    sum *= own;
+#pragma unroll
+    for (int e = 0; e < CH; ++e) {
+        acc[e] *= own;
+    }
+#pragma unroll
+    for (int s = 1; s < SLICES; ++s) {
+        const float *other = joined + (tid + s * vecs) * (CH + 2);
+        const float w = top == -INFINITY ? 0.0f : pow2(other[0] - top);
+        sum += w * other[1];
+#pragma unroll
+        for (int e = 0; e < CH; ++e) {
+            acc[e] += w * other[2 + e];
+        }
+    }
+    const int g = h / a.groupSize;
+    const int64_t outRow = static_cast<int64_t>(sq.qRow + tok) * a.H + h;
+    const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
+    uint16_t bits[CH];
+#pragma unroll
+    for (int e = 0; e < CH; ++e) {
+        float o = acc[e] * inv;
+        if (a.finishV) {
+            const int ch = g * a.Dv + c * CH + e;
+            o = (o + (a.vOff ? static_cast<float>(a.vOff[ch]) : 0.0f)) * a.vScale[ch * a.scaleStride];
+        }
+        bits[e] = BF16 ? FloatToBf16(o) : FloatToHalfBits(o);
+    }
+    uint16_t *dst = reinterpret_cast<uint16_t *>(a.out) + outRow * a.Dv + c * CH;
+    *reinterpret_cast<uint2 *>(dst) = uint2{static_cast<uint32_t>(bits[0]) | (static_cast<uint32_t>(bits[1]) << 16),
+                                            static_cast<uint32_t>(bits[2]) | (static_cast<uint32_t>(bits[3]) << 16)};
+    if (a.lse && c == 0) {
+        Store16(a.lse, outRow, (top + log2f(sum)) * LN2, BF16);
+    }
+}
+
 } // namespace
 
 int LaunchPaStreamReduce(const AtbmiPaShape &shape, const PaArgs &args, const PaStreamPlan &plan,
@@ -234,6 +367,19 @@ int LaunchPaStreamReduce(const AtbmiPaShape &shape, const PaArgs &args, const Pa
     }
     if (grid > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "pa_reduce: grid of %lld workgroups is out of range", (long long)grid);
+    }
+    if (plan.maxRangesPerRow > 8 && !args.partHalf && args.Dv % 4 == 0 && args.Dv / 4 * SLICES <= REDUCE_THREADS) {
+        const int slicedRowsPerWg = REDUCE_THREADS / (args.Dv / 4 * SLICES);
+        const int64_t slicedGrid = (rows + slicedRowsPerWg - 1) / slicedRowsPerWg;
+        if (slicedGrid <= 0x7fffffffLL) {
+            if (args.qIsBf16) {
+                PaStreamReduceSlicedKernel<true><<<static_cast<unsigned>(slicedGrid), REDUCE_THREADS, 0, stream>>>(args, plan);
+            } else {
+                PaStreamReduceSlicedKernel<false><<<static_cast<unsigned>(slicedGrid), REDUCE_THREADS, 0, stream>>>(args, plan);
+            }
+            ATBMI_HIP_CHECK(hipGetLastError());
+            return OK;
+        }
     }
     const unsigned blocks = static_cast<unsigned>(grid);
     if (args.partHalf) {
