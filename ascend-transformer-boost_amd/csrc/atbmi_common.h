@@ -149,6 +149,10 @@ struct PaStreamPlan {
     int32_t foldTokens;       // query tokens of one sequence that may share a head tile (1: none do);
                               // a partial slot then holds foldTokens x H rows
     int32_t maxRangesPerRow;  // most wave ranges any one pass spans (the merge kernel sizes itself by it)
+    int32_t rowStartSteps;    // steps at the head of every pass that stand for no tokens: what starting a row costs a
+                              // wave (its query, the block table, a cold first tile, the partial row it leaves), so
+                              // that equal ranges are equal work. Step s of a pass holds the tokens of its step
+                              // s - rowStartSteps; a range that only has such steps of a pass leaves an empty partial row.
     PaSeq inlineSeqs[PA_INLINE_SEQS + 1];
     uint16_t inlineFirst[PA_INLINE_RANGES];
 };

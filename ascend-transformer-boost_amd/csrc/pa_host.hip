@@ -189,6 +189,7 @@ struct AtbmiPaPlan {
     int mfmaWaves = 8;       // MFMA kernel: waves per workgroup
     int numCus = DEFAULT_CUS; // compute units of the device the plan was created on
     int64_t chunkOverride = 0;
+    int64_t rowStartOverride = -1; // ATBMI_PA_ROW_START_STEPS (test and tuning hook): steps charged for the start of a row
     int64_t minStepsOverride = 0;
 
     // MFMA kernel: the stream plan (see PaStreamPlan) and its host-side pieces
@@ -344,6 +345,7 @@ extern "C" int atbmi_pa_plan_create(const AtbmiPaShape *shape, AtbmiPaPlan **pla
     }
     p->numCus = DeviceComputeUnits();
     p->chunkOverride = EnvInt("ATBMI_PA_CHUNK_TOKENS", 0);
+    p->rowStartOverride = EnvInt("ATBMI_PA_ROW_START_STEPS", -1);
     p->minStepsOverride = EnvInt("ATBMI_PA_MIN_STEPS", 0);
     *plan = p;
     return OK;
@@ -381,9 +383,17 @@ int PlanStream(AtbmiPaPlan *plan)
     if (headTiles == 1 && !PaMlaWide(s) && plan->maxQueryLen > 1 && !plan->causalRows) {
         fold = std::min(PA_MFMA_HEAD_TILE / groupSize, plan->maxQueryLen);
     }
+    // What starting a row costs a wave, in steps (PaStreamPlan::rowStartSteps), measured on the 8B- and 70B-shaped
+    // batches: a wave whose range holds the start of a row left 3 us (16-bit caches) / 8 us (int8: descales to fetch
+    // and fold into the query, twice the steps per byte) later than its neighbours with the same number of steps.
+    // The 128-head kernel takes whole ranges of tokens only.
+    const int rowStartSteps = PaMlaWide(s) || plan->chunkOverride > 0 ? 0
+                              : plan->rowStartOverride >= 0 ? static_cast<int>(plan->rowStartOverride)
+                              : s.kvDtype == ATBMI_INT8 ? 3 : 1;
     try {
         plan->seqTable.clear();
         int64_t steps = 0;
+        int64_t tokenSteps = 0; // the steps that hold tokens
         for (size_t r = 0; r < plan->rows.size();) {
             // consecutive rows of one sequence, `fold` at a time
             size_t e = r + 1;
@@ -395,7 +405,8 @@ int PlanStream(AtbmiPaPlan *plan)
             sq.nTok = static_cast<int32_t>(e - r);
             sq.stepBegin = static_cast<int32_t>(steps);
             plan->seqTable.push_back(sq);
-            steps += (sq.ctxLen + PA_MFMA_STEP - 1) / PA_MFMA_STEP;
+            steps += rowStartSteps + (sq.ctxLen + PA_MFMA_STEP - 1) / PA_MFMA_STEP;
+            tokenSteps += (sq.ctxLen + PA_MFMA_STEP - 1) / PA_MFMA_STEP;
             r = e;
             if (steps > 0x3fffffff) {
                 return Fail(ERR_INVALID_PARAM, "pa_plan_update: too many KV tokens for one call");
@@ -424,7 +435,7 @@ int PlanStream(AtbmiPaPlan *plan)
         // A wave range must hold at least one step: an empty range writes no partial row, and the merge
         // kernel reads the slot of every range between a row's first and last. Surplus waves of the last
         // workgroup idle (their range index is past numWaveRanges).
-        const int32_t waveRanges = static_cast<int32_t>(std::max<int64_t>(1, std::min<int64_t>(wgRanges * tokenSlices, steps)));
+        const int32_t waveRanges = static_cast<int32_t>(std::max<int64_t>(1, std::min<int64_t>(wgRanges * tokenSlices, tokenSteps)));
         wgRanges = (waveRanges + tokenSlices - 1) / tokenSlices;
 
         plan->firstSeq.assign(static_cast<size_t>(wgRanges), 0);
@@ -460,6 +471,7 @@ int PlanStream(AtbmiPaPlan *plan)
         sp.headTiles = headTiles;
         sp.foldTokens = fold;
         sp.maxRangesPerRow = maxRanges;
+        sp.rowStartSteps = rowStartSteps;
         // firstSeq is a 16-bit table: batches beyond 65535 sequences go through memory as 16-bit too,
         // so they are refused here rather than silently truncated
         if (numSeqs > 0xffff) {

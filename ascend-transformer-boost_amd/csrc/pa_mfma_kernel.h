@@ -272,9 +272,29 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
         const int seqEnd = PlanSeq(p, seqIdx + 1).stepBegin;
         const int segBegin = max(s0, sq.stepBegin);
         const int segEnd = min(s1, seqEnd);
-        const int tokBegin = (segBegin - sq.stepBegin) * STEP;
-        const int tokEnd = min(sq.ctxLen, (segEnd - sq.stepBegin) * STEP);
+        const int tokBegin = max(0, segBegin - sq.stepBegin - p.rowStartSteps) * STEP;
+        const int tokEnd = min(sq.ctxLen, max(0, segEnd - sq.stepBegin - p.rowStartSteps) * STEP);
         const bool complete = segBegin == sq.stepBegin && segEnd == seqEnd;
+        if (tokBegin >= tokEnd) {
+            // the range ends inside the steps that stand for the start of the row (PaStreamPlan::rowStartSteps): the
+            // merge kernel reads this range's slot like any other, so it must say "no tokens"
+            const bool folded = EXT && p.foldTokens > 1;
+            const int columns = folded ? sq.nTok * a.groupSize : nhTile;
+            if (n < columns) {
+                const int tok = folded ? n / a.groupSize : 0;
+                const int head = h0 + (folded ? n - tok * a.groupSize : n);
+                const int slot = 2 * wr + (segBegin == s0 ? 0 : 1);
+                const int64_t ph = (static_cast<int64_t>(slot) * (EXT ? p.foldTokens : 1) + tok) * a.H + head;
+#pragma unroll
+                for (int i = 0; i < DV / 16; ++i) {
+                    *reinterpret_cast<f32x4 *>(a.partO + ph * DV + i * 16 + kg * 4) = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                }
+                if (kg == 0) {
+                    a.partLse[ph] = -INFINITY;
+                }
+            }
+            continue;
+        }
         // Column n of the tile is head h0 + n of the pass's query token, or, when the plan folds
         // several query tokens of a sequence into one tile (small GQA groups), head h0 + n % group
         // of its query token n / group.
@@ -316,6 +336,10 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                     qreg[j] = LoadGlobal16((MLA && j * 32 >= dn ? qrope : qrow) + j * 32 + kg * 8);
                 }
             }
+        }
+        // The operand form of Q (the q pre-scale rounded in the query's type, the K descales of an int8 cache folded in).
+        // Called behind the loads of the segment's first step, so that the waits in here overlap with those.
+        auto prepareQ = [&]() {
             const bool plain = !KV8 && a.qScale == 0.0f; // raw bits are already the operand
             if (!plain) {
 #pragma unroll
@@ -344,7 +368,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                     }
                 }
             }
-        }
+        };
 
         float m = -INFINITY; // running maximum (base-2 exponent units) of head n
         f32x4 accL = {0.0f, 0.0f, 0.0f, 0.0f}; // running denominator of head n (the same in all four entries)
@@ -484,6 +508,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
         if constexpr (PF && !SHARED) {
             loadStage(tokBegin);
         }
+        prepareQ();
 
         // One 32-token step of attention for this wave's heads, on the tile at kT / vT.
         auto computeStep = [&](int t, const unsigned char *kT, const unsigned char *vT) {
