@@ -525,6 +525,9 @@ int BuildRows(const AtbmiMlaInt8Call *c, std::vector<Row> *rows)
                         c->maskLen);
         }
         if (ctx == 0) {
+            // an empty context still owns its query rows (nothing is written to their outputs): the reference's
+            // tiling moves on by qSeqLen whatever kvSeqLen is (tiling/mla_tiling.cpp:146-149)
+            qRow += nq;
             continue;
         }
         for (int32_t i = 0; i < nq; ++i) {

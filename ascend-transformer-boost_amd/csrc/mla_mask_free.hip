@@ -80,10 +80,8 @@ int BuildRows(const AtbmiMlaMaskFreeCall *c, std::vector<Row> *rows)
             return Fail(ERR_INVALID_PARAM, "mla_mask_free: sequence %d has context %d (mask rows of %d) and %d query tokens",
                         b, k, c->maskLen, q);
         }
-        if (k == 0) {
-            continue; // (takes no query row, as in the decode plan)
-        }
-        if (q > 1) {
+        // (an empty context keeps its query rows, as in the decode plan of MultiLatentAttention: their mask rows are zeros)
+        if (q > 1 && k > 0) {
             // the template must hold every row this sequence reads
             const int n = k - (k - 1) / TILE * TILE;
             const int top = (n < q - 1 && k > TILE ? n + TILE - 1 : n - 1) + q - 1;

@@ -211,6 +211,7 @@ struct AtbmiPaPlan {
     int32_t maxQueryLen = 1; // most query tokens any sequence brings
     std::vector<PaSeq> rows; // the query rows in query/output order (stepBegin unused here)
     bool causalRows = false;            // a sequence's query rows see growing prefixes of its context
+    bool emptyKeepRows = false;         // a sequence without context still owns its query rows (MultiLatentAttention)
     std::vector<int32_t> causalUse;     // empty: every sequence; else one flag per sequence
 
     uint64_t offItems = 0, offSeqs = 0, offPartO = 0, offPartLse = 0, blobBytes = 0, wsBytes = 0;
@@ -532,6 +533,15 @@ extern "C" int atbmi_pa_plan_set_causal_rows(AtbmiPaPlan *plan, int32_t enable, 
     return OK;
 }
 
+extern "C" int atbmi_pa_plan_set_empty_keep_rows(AtbmiPaPlan *plan, int32_t enable)
+{
+    if (!plan) {
+        return Fail(ERR_INVALID_PARAM, "pa_plan_set_empty_keep_rows: null plan");
+    }
+    plan->emptyKeepRows = enable != 0;
+    return OK;
+}
+
 extern "C" int atbmi_pa_plan_update(AtbmiPaPlan *plan, const int32_t *ctx, int32_t batch)
 {
     return atbmi_pa_plan_update_multi(plan, ctx, nullptr, batch);
@@ -547,7 +557,7 @@ extern "C" int atbmi_pa_plan_update_multi(AtbmiPaPlan *plan, const int32_t *ctx,
         return Fail(ERR_INVALID_PARAM, "pa_plan_update: batch %d", batch);
     }
     int64_t total = 0, tableEntries = 0, rowCtx = 0;
-    int64_t nonEmpty = 0;
+    int64_t nonEmpty = 0, rowsSpanned = 0;
     const int64_t maxCtx = static_cast<int64_t>(s.maxBlocksPerSeq) * s.blockSize;
     for (int32_t b = 0; b < batch; ++b) {
         if (ctx[b] < 0 || ctx[b] > maxCtx) {
@@ -568,6 +578,7 @@ extern "C" int atbmi_pa_plan_update_multi(AtbmiPaPlan *plan, const int32_t *ctx,
                         ctx[b], s.maskLen);
         }
         const int32_t n = ctx[b] == 0 ? 0 : (qLens ? qLens[b] : 1);
+        rowsSpanned += ctx[b] == 0 && plan->emptyKeepRows ? (qLens ? qLens[b] : 1) : n;
         if (n > 0) {
             nonEmpty += n;
             total += ctx[b];
@@ -575,14 +586,18 @@ extern "C" int atbmi_pa_plan_update_multi(AtbmiPaPlan *plan, const int32_t *ctx,
             tableEntries += (ctx[b] + s.blockSize - 1) / s.blockSize;
         }
     }
-    if (nonEmpty > s.numQueryRows) {
+    if (rowsSpanned > s.numQueryRows) {
         return Fail(ERR_INVALID_PARAM, "pa_plan_update: %lld query rows planned but the query holds %d",
-                    (long long)nonEmpty, s.numQueryRows);
+                    (long long)rowsSpanned, s.numQueryRows);
     }
     try {
         plan->rows.clear();
+        int32_t nextRow = 0; // of q / out
         for (int32_t b = 0; b < batch; ++b) {
             const int32_t n = ctx[b] == 0 ? 0 : (qLens ? qLens[b] : 1);
+            if (ctx[b] == 0 && plan->emptyKeepRows) {
+                nextRow += qLens ? qLens[b] : 1; // rows that are never read or written
+            }
             for (int32_t i = 0; i < n; ++i) {
                 PaSeq row{};
                 row.tableRow = b;
@@ -591,7 +606,7 @@ extern "C" int atbmi_pa_plan_update_multi(AtbmiPaPlan *plan, const int32_t *ctx,
                     row.ctxLen = ctx[b] - n + i + 1; // (>= 1: n <= ctx[b] was checked above)
                 }
                 row.nTok = 1;
-                const int32_t index = static_cast<int32_t>(plan->rows.size());
+                const int32_t index = nextRow++;
                 row.qRow = index;
                 int32_t bySeq = s.maskSeqDiv > 1 ? b / s.maskSeqDiv : b;
                 bySeq = s.maskSeqMod > 0 ? bySeq % s.maskSeqMod : bySeq;

@@ -472,6 +472,10 @@ protected:
         int rc = atbmi_pa_plan_set_causal_rows(plan_, causalRows ? 1 : 0, causalUse_.empty() ? nullptr : causalUse_.data(),
                                                static_cast<int32_t>(causalUse_.size()));
         if (rc == 0) {
+            // a sequence without context keeps its query rows (reference tiling/mla_tiling.cpp:146-149)
+            rc = atbmi_pa_plan_set_empty_keep_rows(plan_, 1);
+        }
+        if (rc == 0) {
             rc = atbmi_pa_plan_update_multi(plan_, static_cast<const int32_t *>(lens.hostData), queryLens, batch);
         }
         if (rc != 0) {

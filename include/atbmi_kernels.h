@@ -383,6 +383,13 @@ int atbmi_pa_plan_update_multi(AtbmiPaPlan *plan, const int32_t *hostContextLens
  * `count` is refused. enable == 0 returns to whole contexts. Query tokens of a sequence then take a pass each. */
 int atbmi_pa_plan_set_causal_rows(AtbmiPaPlan *plan, int32_t enable, const int32_t *perSequence, int32_t count);
 
+/* Empty sequences for the updates that follow: with enable != 0 a sequence whose context length is 0 still owns its
+ * hostQueryLens[b] (or one) query rows, which are neither read nor written, and the rows of the sequences behind it
+ * stay where they are. This is what the reference's MultiLatentAttention tiling does (it moves on by qSeqLen whatever
+ * kvSeqLen is, src/kernels/mixkernels/multi_latent_attention/tiling/mla_tiling.cpp:146-149), whereas its PagedAttention
+ * tiling gives such a sequence no row (tiling/paged_attention_tiling_dependency.cpp:593,654,706), the default here. */
+int atbmi_pa_plan_set_empty_keep_rows(AtbmiPaPlan *plan, int32_t enable);
+
 /* Device workspace bytes atbmi_pa_decode needs for the current plan. */
 uint64_t atbmi_pa_plan_workspace_size(const AtbmiPaPlan *plan);
 
@@ -478,7 +485,8 @@ int atbmi_mla_prefill(const AtbmiMlaPrefillCall *call, void *workspaceDevice, ui
  *   mask        NULL, or 16-bit [numQueryRows, maskLen] added to the scaled scores of its query row
  *   out         16-bit [numQueryRows, numHeads, 512]     lse        NULL, or fp32 [numQueryRows, numHeads]
  * Sequence b attends to hostContextLens[b] tokens with hostQueryLens[b] consecutive query rows (NULL: one
- * each; a sequence of length 0 takes none). With causalRows != 0 the t-th of a sequence's n query rows
+ * each; a sequence of length 0 keeps its rows, which are neither read nor written, as the reference's tiling
+ * moves on by qSeqLen whatever kvSeqLen is: tiling/mla_tiling.cpp:146-149). With causalRows != 0 the t-th of a sequence's n query rows
  * attends to its first hostContextLens[b] - n + t + 1 tokens only, unless hostCausalUse (NULL, or [batch])
  * holds 0 for the sequence: the reference golden's handling of several query tokens in this mode
  * (test_multi_latent_attention_int8nz.py:356-364). The lengths and flags are host arrays, read during the call.
@@ -587,8 +595,8 @@ int atbmi_pa_int8q_decode(const AtbmiPaInt8QCall *call, void *workspaceDevice, u
  * mask, a template [templateRows, 128] (templateBatch == 0) or [templateBatch = batch, templateRows, 128] of 16-bit
  * values, into one mask row per query token, outMask 16-bit [numQueryRows, maskLen], to be handed to the decode
  * plan as a mask with one row per query row (AtbmiPaShape.maskRowBy = ATBMI_PA_MASK_ROW_QUERY). Sequence b has
- * hostContextLens[b] tokens and hostQueryLens[b] query rows (none when its context is empty), as in
- * atbmi_pa_plan_update_multi; both are host arrays read during the call.
+ * hostContextLens[b] tokens and hostQueryLens[b] query rows (also when its context is empty: rows of zeros), as a
+ * plan with atbmi_pa_plan_set_empty_keep_rows has them; both are host arrays read during the call.
  */
 typedef struct AtbmiMlaMaskFreeCall {
     int32_t batch;

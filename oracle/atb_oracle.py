@@ -521,7 +521,7 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, s
                     k_offset=None, v_descale=None, v_offset=None, mla_v_head_size=0, q_scale=0.0,
                     q_dtype="float32", out_init=0.0, mask=None, logn=None, mask_per_head=None, q_lens=None,
                     mask_rows="sequence", lse_out=None, head_major=False, compress_kv_heads=0, razor_offset=None,
-                    causal_rows=None):
+                    causal_rows=None, empty_keep_rows=False):
     """Decode attention over paged caches.
 
     query [rows, heads, D] float32; key_cache [blocks, block, kv_heads, D];
@@ -570,6 +570,12 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, s
     [batch * n, heads / n, 1, max_len], a 3-dim mask has one row per sequence
     (pair i uses row i // n). razor_offset, float32 [blocks * n, block], is added
     to q k^T of the token in that cache slot before the scale.
+    empty_keep_rows: a sequence without context still owns its q_lens[i] (or one) query rows, which
+    are neither read nor written, and the rows of the sequences behind it stay where they are. This is
+    what the reference's MultiLatentAttention tiling does (it moves on by qSeqLen whatever kvSeqLen
+    is: src/kernels/mixkernels/multi_latent_attention/tiling/mla_tiling.cpp:146-149; its golden for
+    several query tokens does the same, tests/apitest/opstest/python/operations/multi_latent_attention/
+    test_multi_latent_attention_mtp.py:145-151), whereas PagedAttention gives such a sequence no row.
     Returns float32 [rows, heads, Dv]."""
     query = np.asarray(query, dtype=np.float32)
     if compress_kv_heads > 0:
@@ -605,6 +611,8 @@ def paged_attention(query, key_cache, value_cache, block_tables, context_lens, s
     row = 0
     for i, ctx in enumerate(np.asarray(context_lens).tolist()):
         if ctx == 0:
+            if empty_keep_rows:
+                row += 1 if q_lens is None else int(q_lens[i])
             continue
         keys = gather_rows(key_cache, block_tables[i], ctx)
         values = keys[..., :dv] if mla_v_head_size > 0 else gather_rows(value_cache, block_tables[i], ctx)
@@ -727,12 +735,13 @@ def mla_mask_free_rows(template, context_lens, q_lens, mask_len):
     the reference's kernel reads it (src/kernels/mixkernels/multi_latent_attention/op_kernel/mla.cce:3719-3750,
     2581-2592): template [rows, 128] or [batch, rows, 128]; for a sequence of k tokens whose last 128-token tile
     holds n of them, query token i of q adds template row n - 1 + i to the last tile and, when n < q - 1 and there
-    is a tile before it, row n + 127 + i to that one. Sequences of length 0 take no row. Returns float32
-    [query rows, mask_len]; rows the template lacks read as 0."""
+    is a tile before it, row n + 127 + i to that one. A sequence of length 0 keeps its q rows, all zeros (see
+    paged_attention's empty_keep_rows). Returns float32 [query rows, mask_len]; rows the template lacks read as 0."""
     template = np.asarray(template, np.float32)
     rows = []
     for b, (k, q) in enumerate(zip(np.asarray(context_lens).tolist(), np.asarray(q_lens).tolist())):
         if k == 0:
+            rows += [np.zeros(mask_len, np.float32) for _ in range(q)]
             continue
         tmpl = template[b] if template.ndim == 3 else template
         last = (k - 1) // 128
@@ -776,9 +785,11 @@ def mla_int8_decode(q_int8, q_rope, kv_int8, k_rope, block_tables, context_lens,
     row = 0
     for b, ctx in enumerate(np.asarray(context_lens)):
         ctx = int(ctx)
-        if ctx == 0:
-            continue
         n_rows = 1 if q_lens is None else int(q_lens[b])
+        if ctx == 0:
+            # the sequence keeps its query rows, untouched (see paged_attention's empty_keep_rows)
+            row += n_rows
+            continue
         keys = gather_rows(np.asarray(kv_int8), block_tables[b], ctx)[:, 0].astype(np.int32)     # [ctx, 512]
         rope = gather_rows(np.asarray(k_rope, np.float32), block_tables[b], ctx)[:, 0]             # [ctx, 64]
         all_keys, all_rope, whole = keys, rope, ctx

@@ -136,7 +136,7 @@ def mask_strides(mask, per_head):
 def oracle_pa(oracle, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=None, v_scale=None, v_off=None,
               mla_dv=0, q_scale=0.0, out_init=0.0, mask=None, mask_per_head=False, logn=None, q_lens=None,
               mask_rows="sequence", lse_out=None, head_major=False, compress_kv_heads=0, razor_offset=None,
-              causal_rows=None):
+              causal_rows=None, empty_keep_rows=False):
     qd = "bf16" if q.dtype == torch.bfloat16 else "float16"
     return oracle.paged_attention(
         to_oracle(q), to_oracle(kc), to_oracle(vc), tables.cpu().numpy(), np.asarray(ctx_host), scale,
@@ -144,7 +144,7 @@ def oracle_pa(oracle, q, kc, vc, tables, ctx_host, scale, k_scale=None, k_off=No
         q_scale=q_scale, q_dtype=qd, out_init=out_init, mask=to_oracle(mask), logn=to_oracle(logn),
         mask_per_head=mask_per_head if (mask is not None and mask.dim() == 3) else None, q_lens=q_lens,
         mask_rows=mask_rows, lse_out=lse_out, head_major=head_major, compress_kv_heads=compress_kv_heads,
-        razor_offset=to_oracle(razor_offset), causal_rows=causal_rows)
+        razor_offset=to_oracle(razor_offset), causal_rows=causal_rows, empty_keep_rows=empty_keep_rows)
 
 
 def assert_close(got, want, tol, what=""):

@@ -38,7 +38,9 @@ def _case(seed, dev, ctx, heads, dtype, q_lens=None, with_mask=False, causal=Non
     block = 128
     pool = int(((ctx + block - 1) // block).sum()) + 3
     tables = random_tables(rng, ctx, block, pool)
-    rows = int(sum((1 if q_lens is None else q_lens[b]) for b in range(len(ctx)) if ctx[b] > 0))
+    # (a sequence without context keeps its query rows: reference tiling/mla_tiling.cpp:146-149)
+    rows = int(sum((1 if q_lens is None else q_lens[b]) for b in range(len(ctx))))
+    written = np.concatenate([np.full(1 if q_lens is None else q_lens[b], ctx[b] > 0) for b in range(len(ctx))])
     q8 = torch.from_numpy(rng.integers(-5, 6, size=(rows, heads, 512)).astype(np.int8))
     qr = torch.from_numpy(rng.uniform(-5, 5, size=(rows, heads, 64)).astype(np.float32)).to(dtype)
     kv8 = torch.from_numpy(rng.integers(-5, 6, size=(pool, block, 1, 512)).astype(np.int8))
@@ -50,14 +52,14 @@ def _case(seed, dev, ctx, heads, dtype, q_lens=None, with_mask=False, causal=Non
         m = np.zeros((rows, int(ctx.max())), np.float32)
         r = 0
         for b in range(len(ctx)):   # the look-ahead mask of several query tokens: token i of n does not see the last n - 1 - i
-            n = 0 if ctx[b] == 0 else (1 if q_lens is None else q_lens[b])
+            n = 1 if q_lens is None else q_lens[b]
             for i in range(n):
-                if n - 1 - i > 0:
+                if n - 1 - i > 0 and ctx[b] > 0:
                     m[r, ctx[b] - (n - 1 - i):ctx[b]] = -10000.0
                 r += 1
         mask = torch.from_numpy(m).to(dtype)
     return dict(q8=q8, qr=qr, kv8=kv8, kr=kr, tables=torch.from_numpy(tables), ctx=ctx, qd=qd, pd=pd, mask=mask,
-                q_lens=q_lens, rows=rows, heads=heads, dtype=dtype, causal=causal)
+                q_lens=q_lens, rows=rows, heads=heads, dtype=dtype, causal=causal, written=written)
 
 
 def _nz(oracle, t, n0):
@@ -148,10 +150,15 @@ def test_mla_int8_nz_kernel(binding, oracle, dev, stream, case):
     want_lse = np.zeros((c["rows"], heads), np.float32)
     want = _oracle(oracle, c, scale, 128, want_lse)
     got, lse = int8_cabi(binding, oracle, stream, dev, c, scale, want_lse=True)
+    # the rows of a sequence without context are nobody's: the call leaves them as they were (7 / 0 here)
+    idle = torch.from_numpy(~c["written"])
+    assert torch.all(got[idle] == 7.0) and torch.all(lse[idle] == 0.0)
+    want[~c["written"]] = 7.0
     assert_close(got, want, TOL[dtype], "int8 NZ %s" % (case,))
     assert_close(lse, want_lse, 1e-3, "int8 NZ lse")
     # the reference's criterion: errors against the whole-context golden no worse than the tiled golden's
     true_out = _oracle(oracle, c, scale, 1 << 30)
+    true_out[~c["written"]] = 7.0
     rounded = torch.from_numpy(want).to(dtype).float().numpy()
     ok, rates = _double_golden(true_out, rounded, got.float().cpu().numpy(), dtype)
     assert ok, "double-golden rates %s" % (rates,)

@@ -1659,6 +1659,46 @@ def test_multi_latent_attention_operation(binding, oracle, dev, stream, heads, d
     c.close()
 
 
+@pytest.mark.parametrize("heads", [128, 32])
+def test_multi_latent_attention_empty_context_keeps_its_rows(binding, oracle, dev, stream, heads):
+    """A sequence without context in the middle of a batch with several query tokens: its query rows stay its own
+    (nothing is written to their outputs) and the rows of the sequences behind it do not move up, as the reference's
+    tiling lays them out (tiling/mla_tiling.cpp:146-149: beginQ moves on by qSeqLen whatever kvSeqLen is). With the
+    SPEC mask on 32 heads (one mask row per query row, the empty sequence's included) and on the job-per-token path of
+    128 heads, both with the log-sum-exp output."""
+    rng = _rng(470 + heads)
+    d, dv, block, dtype = 576, 512, 128, torch.float16
+    ctx = np.array([700, 0, 300, 0], dtype=np.int32)
+    q_lens = np.array([2, 3, 1, 2], dtype=np.int32)
+    rows = int(q_lens.sum())
+    _, kc, _, tables, _ = _pa_inputs(rng, dev, 4, heads, 1, block, d, d, np.maximum(ctx, 1), dtype, std=0.5)
+    k_nope, k_rope = kc[..., :dv].contiguous(), kc[..., dv:].contiguous()
+    scale = 1.0 / math.sqrt(192.0)
+    lens, qn = torch.from_numpy(ctx), torch.from_numpy(q_lens)
+    q = (torch.rand((rows, heads, d)) * 2 - 1).to(dtype).to(dev)
+    mask = torch.from_numpy(np.where(np.arange(700)[None, :] < 690, rng.standard_normal((rows, 700)), -10000.0)
+                            .astype(np.float32)).to(dtype).to(dev)
+    c = binding.Context(stream)
+    op = binding.OperationRunner("MultiLatentAttentionOperation", binding.MultiLatentAttentionParam(
+        headNum=heads, kvHeadNum=1, qkScale=scale, cacheMode=1, calcType=3, maskType=1), c)
+    out = torch.full((rows, heads, dv), 0.25, dtype=dtype, device=dev)
+    lse = torch.full((rows, heads, 1), 7.0, dtype=dtype, device=dev)
+    with torch.cuda.stream(stream):
+        op.run([q[..., :dv].contiguous(), q[..., dv:].contiguous(), k_nope, k_rope, tables, lens.to(dev), mask, qn.to(dev)],
+               outputs=[out, lse], host_inputs={5: lens, 7: qn})
+    stream.synchronize()
+    per_token = heads == 128
+    want_lse = np.full((rows, heads), 7.0, np.float32)
+    want = oracle_pa(oracle, q, kc, None, tables, ctx, scale, mla_dv=dv, mask=None if per_token else mask, q_lens=q_lens,
+                     mask_rows="query", lse_out=want_lse, causal_rows=True if per_token else None, out_init=0.25,
+                     empty_keep_rows=True)
+    assert_close(out, want, TOL[dtype], "empty context in the middle, %d heads" % heads)
+    assert_close(lse[..., 0], want_lse, TOL[dtype], "its log-sum-exp")
+    assert torch.all(out[2:5] == 0.25) and torch.all(out[6:] == 0.25) and torch.all(lse[2:5] == 7.0)
+    op.close()
+    c.close()
+
+
 @pytest.mark.parametrize("kernel", [1, 2])
 def test_causal_rows_through_the_c_abi(binding, oracle, dev, stream, kernel):
     """atbmi_pa_plan_set_causal_rows: the t-th of n query rows attends to the first ctx - n + t + 1 tokens, per
@@ -1739,7 +1779,7 @@ def test_mask_free_template_expansion_and_operation(binding, oracle, dev, stream
     rng = _rng(495)
     ctx = np.array([700, 33, 1500, 128, 129, 258, 0, 5], dtype=np.int32)
     q_lens = np.array([2, 1, 3, 2, 4, 4, 2, 5], dtype=np.int32)
-    rows = int(sum(n for n, c in zip(q_lens, ctx) if c > 0))
+    rows = int(q_lens.sum())   # (the sequence without context keeps its two rows: zeros)
     mask_len = 1504
     for dtype in (torch.float16, torch.bfloat16):
         standard = np.triu(np.full((125 + 2 * 5, 128), -10000.0, np.float32), 2 - 5)

@@ -594,7 +594,7 @@ def test_multi_latent_attention_counts_shapes_and_setup(binding, ctx):
     assert binding.Operation("MultiLatentAttentionOperation", p).status == e["ERROR_INVALID_PARAM"]
 
     lens = np.array([10, 300, 0, 64], dtype=np.int32)
-    qlens = np.array([1, 3, 2, 2], dtype=np.int32)   # 6 query rows
+    qlens = np.array([1, 3, 2, 2], dtype=np.int32)   # 8 query rows: the sequence without context keeps its two
 
     def pack(rows=4, mask=None, with_qlens=False, lens_host=True, qlens_host=True, dtype="float16", block=128):
         ins = [
@@ -637,11 +637,11 @@ def test_multi_latent_attention_counts_shapes_and_setup(binding, ctx):
 
     spec = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1,
                                                                  calcType=1, maskType=1))
-    assert spec.setup(pack(rows=6, mask=[6, 300], with_qlens=True), outs(rows=6), ctx)[0] == 0
-    assert spec.setup(pack(rows=6, mask=[6, 299], with_qlens=True), outs(rows=6), ctx)[0] == e["ERROR_INVALID_PARAM"]
-    assert spec.setup(pack(rows=6, mask=[5, 300], with_qlens=True), outs(rows=6), ctx)[0] == e["ERROR_INVALID_PARAM"]
-    assert spec.setup(pack(rows=5, mask=[5, 300], with_qlens=True), outs(rows=5), ctx)[0] == e["ERROR_INVALID_PARAM"]
-    assert spec.setup(pack(rows=6, mask=[6, 300], with_qlens=True, qlens_host=False), outs(rows=6), ctx)[0] == \
+    assert spec.setup(pack(rows=8, mask=[8, 300], with_qlens=True), outs(rows=8), ctx)[0] == 0
+    assert spec.setup(pack(rows=8, mask=[8, 299], with_qlens=True), outs(rows=8), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    assert spec.setup(pack(rows=8, mask=[7, 300], with_qlens=True), outs(rows=8), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    assert spec.setup(pack(rows=7, mask=[7, 300], with_qlens=True), outs(rows=7), ctx)[0] == e["ERROR_INVALID_PARAM"]
+    assert spec.setup(pack(rows=8, mask=[8, 300], with_qlens=True, qlens_host=False), outs(rows=8), ctx)[0] == \
         e["ERROR_INVALID_PARAM"]
     spec.close()
 
@@ -654,12 +654,12 @@ def test_multi_latent_attention_causal_rows_and_mask_use_status(binding, ctx):
     e = binding.ERROR_CODE
     mk = binding.MultiLatentAttentionParam
     lens = np.array([10, 300, 0, 64], dtype=np.int32)
-    qlens = np.array([1, 3, 2, 2], dtype=np.int32)   # 6 query rows
+    qlens = np.array([1, 3, 2, 2], dtype=np.int32)   # 8 query rows: the sequence without context keeps its two
     use = np.array([1, 0, 1, 1], dtype=np.int32)
 
     def pack(heads, mask=None, use_shape=None, use_host=True, qlens_host=qlens):
-        ins = [binding.make_tensor("float16", [6, heads, 512], FAKE_DEVICE),
-               binding.make_tensor("float16", [6, heads, 64], FAKE_DEVICE),
+        ins = [binding.make_tensor("float16", [8, heads, 512], FAKE_DEVICE),
+               binding.make_tensor("float16", [8, heads, 64], FAKE_DEVICE),
                binding.make_tensor("float16", [16, 128, 1, 512], FAKE_DEVICE),
                binding.make_tensor("float16", [16, 128, 1, 64], FAKE_DEVICE),
                binding.make_tensor("int32", [4, 3], FAKE_DEVICE),
@@ -672,8 +672,8 @@ def test_multi_latent_attention_causal_rows_and_mask_use_status(binding, ctx):
         return ins
 
     def outs(heads, lse=True):
-        o = [binding.make_tensor("float16", [6, heads, 512], FAKE_DEVICE)]
-        return o + ([binding.make_tensor("float16", [6, heads, 1], FAKE_DEVICE)] if lse else [])
+        o = [binding.make_tensor("float16", [8, heads, 512], FAKE_DEVICE)]
+        return o + ([binding.make_tensor("float16", [8, heads, 1], FAKE_DEVICE)] if lse else [])
 
     # 128 heads: any mask shape passes, because the tensor is not read; the flags come from the host
     op = binding.Operation("MultiLatentAttentionOperation", mk(headNum=128, kvHeadNum=1, qkScale=0.07, cacheMode=1,
@@ -697,7 +697,7 @@ def test_multi_latent_attention_causal_rows_and_mask_use_status(binding, ctx):
                                                                   calcType=1, maskType=3))
     st, ws = op.setup(pack(32, mask=[131, 128]), outs(32, lse=False), ctx)
     st0, ws0 = plain.setup(pack(32), outs(32, lse=False), ctx)
-    assert (st, st0) == (0, 0) and ws >= ws0 + 6 * 16 + 6 * 304 * 2 and ws <= ws0 + 6 * 16 + 6 * 304 * 2 + 1024
+    assert (st, st0) == (0, 0) and ws >= ws0 + 8 * 16 + 8 * 304 * 2 and ws <= ws0 + 8 * 16 + 8 * 304 * 2 + 1024
     assert op.setup(pack(32, mask=[4, 131, 128]), outs(32, lse=False), ctx)[0] == 0           # a template per sequence
     assert op.setup(pack(32, mask=[3, 131, 128]), outs(32, lse=False), ctx)[0] == e["ERROR_INVALID_PARAM"]
     assert op.setup(pack(32, mask=[131, 64]), outs(32, lse=False), ctx)[0] == e["ERROR_INVALID_PARAM"]
@@ -722,7 +722,7 @@ def test_multi_latent_attention_int8_nz_cache_checks(binding, ctx):
     e = binding.ERROR_CODE
     mk = binding.MultiLatentAttentionParam
     lens = np.array([10, 300, 0, 64], dtype=np.int32)
-    qlens = np.array([1, 3, 2, 2], dtype=np.int32)
+    qlens = np.array([1, 3, 2, 2], dtype=np.int32)   # 8 query rows: the sequence without context keeps its two
 
     def pack(rows=4, kv=(16, 16, 128, 32), kr=(16, 4, 128, 16), dtype="float16", with_qlens=False, q_dtype="int8",
              descale=(32,), fmt="fractal_nz", mask=None):
@@ -772,14 +772,14 @@ def test_multi_latent_attention_int8_nz_cache_checks(binding, ctx):
     both = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=2,
                                                                  calcType=3))
     assert both.ok and (both.input_num(), both.output_num()) == (9, 2)
-    assert both.setup(pack(rows=6, with_qlens=True), outs(rows=6, lse="float"), ctx)[0] == 0
+    assert both.setup(pack(rows=8, with_qlens=True), outs(rows=8, lse="float"), ctx)[0] == 0
     both.close()
     spec = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=2,
                                                                  calcType=1, maskType=1))
     assert spec.ok and spec.input_num() == 10
-    assert spec.setup(pack(rows=6, with_qlens=True, mask=(6, 300)), outs(rows=6), ctx)[0] == 0
+    assert spec.setup(pack(rows=8, with_qlens=True, mask=(8, 300)), outs(rows=8), ctx)[0] == 0
     # the int8 kernels of the reference never read the mask (tiling/mla_tiling.cpp:142-144): its shape is not looked at
-    assert spec.setup(pack(rows=6, with_qlens=True, mask=(6, 299)), outs(rows=6), ctx)[0] == 0
+    assert spec.setup(pack(rows=8, with_qlens=True, mask=(8, 299)), outs(rows=8), ctx)[0] == 0
     spec.close()
 
 
@@ -915,7 +915,7 @@ def test_multi_latent_attention_nz_cache_checks(binding, ctx):
     spec = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=3,
                                                                  calcType=1))
     assert spec.ok and spec.input_num() == 7
-    assert spec.setup(pack(rows=6, with_qlens=True), outs(rows=6), ctx)[0] == 0
+    assert spec.setup(pack(rows=8, with_qlens=True), outs(rows=8), ctx)[0] == 0
     spec.close()
 
 

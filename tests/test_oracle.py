@@ -737,6 +737,35 @@ def test_attention_empty_sequences_take_no_query_row(oracle):
     assert np.all(out[3] == np.float32(0.1))
 
 
+def test_attention_empty_sequences_keep_their_rows_on_request(oracle):
+    """empty_keep_rows (MultiLatentAttention; reference tiling/mla_tiling.cpp:146-149): the query rows of a sequence
+    without context are left alone and every other sequence stays at the running sum of ALL query lengths; the mask
+    of a query row is the one at its own index. Each sequence is checked against itself run alone."""
+    rng = _rng(11)
+    _, kc, vc, tables, ctx = _paged_case(rng, batch=4, heads=4, kv_heads=1, max_ctx=40)
+    ctx = np.array([max(int(ctx[0]), 3), 0, max(int(ctx[2]), 2), 0], np.int32)
+    q_lens = np.array([2, 3, 1, 2], np.int32)
+    q = rng.standard_normal((8, 4, kc.shape[3])).astype(np.float32)
+    mask = (rng.standard_normal((8, 40)) * 2).astype(np.float32)
+    lse = np.full((8, 4), 7.0, np.float32)
+    out = oracle.paged_attention(q, kc, vc, tables, ctx, 0.25, q_lens=q_lens, mask=mask, mask_rows="query",
+                                 out_init=0.1, lse_out=lse, empty_keep_rows=True)
+    starts = np.concatenate([[0], np.cumsum(q_lens)])
+    for b in range(4):
+        rows = slice(int(starts[b]), int(starts[b + 1]))
+        if ctx[b] == 0:
+            assert np.all(out[rows] == np.float32(0.1)) and np.all(lse[rows] == 7.0)
+            continue
+        alone_lse = np.zeros((q_lens[b], 4), np.float32)
+        alone = oracle.paged_attention(q[rows], kc, vc, tables[b:b + 1], ctx[b:b + 1], 0.25, q_lens=q_lens[b:b + 1],
+                                       mask=mask[rows], mask_rows="query", lse_out=alone_lse)
+        assert np.array_equal(out[rows], alone) and np.array_equal(lse[rows], alone_lse)
+    # without the option the same call packs the rows (PagedAttention's rule)
+    packed = oracle.paged_attention(q, kc, vc, tables, ctx, 0.25, q_lens=q_lens, out_init=0.1)
+    assert np.array_equal(packed[2], oracle.paged_attention(q[2:3], kc, vc, tables[2:3], ctx[2:3], 0.25)[0])
+    assert np.all(packed[3:] == np.float32(0.1))
+
+
 # ---------------------------------------------------------------- masks and logN
 def _with_empty(ctx, at):
     ctx = ctx.copy()
@@ -961,7 +990,8 @@ def test_mask_free_template_rows_are_the_look_ahead_triangle(oracle):
     per_seq = np.stack([np.triu(np.full((129, 128), -10000.0, np.float32), 0), np.zeros((129, 128), np.float32)])
     got = oracle.mla_mask_free_rows(per_seq, [130, 130], [2, 2], 256)
     assert got[0, 129] == -10000.0 and got[1, 129] == 0.0 and not got[2:].any()
-    assert oracle.mla_mask_free_rows(per_seq, [0, 5], [2, 1], 8).shape == (1, 8)   # an empty sequence takes no row
+    got = oracle.mla_mask_free_rows(per_seq, [0, 5], [2, 1], 8)   # an empty sequence keeps its rows, all zeros
+    assert got.shape == (3, 8) and not got[:2].any() and np.array_equal(got[2], per_seq[1, 4, :8] * (np.arange(8) < 5))
 
 
 # ---------------------------------------------------------------- log-sum-exp output
@@ -1072,7 +1102,7 @@ def _int8_case(rng, ctx, heads=4, block=16, q_lens=None):
     for b in range(len(ctx)):
         tables[b, :nblk[b]] = perm[pos:pos + nblk[b]]
         pos += nblk[b]
-    rows = int(sum((1 if q_lens is None else q_lens[b]) for b in range(len(ctx)) if ctx[b] > 0))
+    rows = int(sum((1 if q_lens is None else q_lens[b]) for b in range(len(ctx))))  # (empty sequences keep theirs)
     q8 = rng.integers(-5, 6, size=(rows, heads, 512)).astype(np.int8)
     qr = rng.uniform(-5, 5, size=(rows, heads, 64)).astype(np.float16).astype(np.float32)
     kv8 = rng.integers(-5, 6, size=(pool, block, 1, 512)).astype(np.int8)
@@ -1105,7 +1135,13 @@ def test_int8_decode_matches_independent_loops(oracle, tile):
                                  lse_out=lse)
     row = 0
     for b, n in enumerate(ctx):
-        for _ in range([2, 1, 1, 1][b] if n > 0 else 0):
+        if n == 0:
+            # the sequence without context keeps its query row (reference tiling/mla_tiling.cpp:146-149): nothing is
+            # written there, and the rows behind it do not move up
+            assert not got[row].any() and not lse[row].any()
+            row += [2, 1, 1, 1][b]
+            continue
+        for _ in range([2, 1, 1, 1][b]):
             for h in range(3):
                 s = []
                 for t in range(n):
