@@ -218,7 +218,7 @@ class AtbmiPaInt8QCall(ctypes.Structure):
                                               "maskLen", "pieceTiles")] + [
         ("qkScale", ctypes.c_float), ("maskSeqStride", ctypes.c_int64), ("maskHeadStride", ctypes.c_int64)] + [
         (n, ctypes.c_void_p) for n in ("hostContextLens", "query", "keyCache", "valueCache", "blockTables", "kDescale",
-                                       "vDescale", "pScale", "mask", "out")]
+                                       "vDescale", "pScale", "mask", "out")] + [("maskRowByQuery", ctypes.c_int32)]
 
 
 class AtbmiMlaMaskFreeCall(ctypes.Structure):

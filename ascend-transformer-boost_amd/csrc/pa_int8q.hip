@@ -529,6 +529,14 @@ int BuildRows(const AtbmiPaInt8QCall *c, std::vector<Row> *rows)
                     "pa_int8q: batch %d, %d blocks of %d tokens, %d blocks a sequence, qkScale %g, mask length %d",
                     c->batch, c->numBlocks, c->blockSize, c->maxBlocksPerSeq, c->qkScale, c->maskLen);
     }
+    if (c->hasMask && (reinterpret_cast<uintptr_t>(c->mask) % 4 != 0 || c->maskSeqStride % 2 != 0 || c->maskHeadStride % 2 != 0 ||
+                       c->maskLen % 2 != 0)) {
+        // the kernel fetches mask values as aligned 32-bit words: a row that starts on an odd element would make it
+        // read two bytes in front of the row, and one that ends on an even element two bytes behind it
+        return Fail(ERR_INVALID_PARAM, "pa_int8q: the mask must start on a 4-byte boundary and have even strides (%lld, %lld) "
+                                       "and an even row length (%d)", (long long)c->maskSeqStride, (long long)c->maskHeadStride,
+                    c->maskLen);
+    }
     int64_t qRow = 0;
     for (int32_t b = 0; b < c->batch; ++b) {
         const int32_t ctx = c->hostContextLens[b];
@@ -550,7 +558,8 @@ int BuildRows(const AtbmiPaInt8QCall *c, std::vector<Row> *rows)
             return Fail(ERR_INVALID_PARAM, "pa_int8q: more than 2^31 query rows");
         }
         if (rows) {
-            rows->push_back(Row{b, 0, ctx, static_cast<int32_t>(qRow), b, -1, 0, 0});
+            rows->push_back(Row{b, 0, ctx, static_cast<int32_t>(qRow), c->maskRowByQuery ? static_cast<int32_t>(qRow) : b,
+                                -1, 0, 0});
         }
         ++qRow;
     }

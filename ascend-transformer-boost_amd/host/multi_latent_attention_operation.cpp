@@ -386,7 +386,8 @@ protected:
             for (int32_t i = 0; i < batch; ++i) {
                 maskLen = std::max<int64_t>(maskLen, ctx[i]);
             }
-            maskLen = std::max<int64_t>(8, (maskLen + 7) / 8 * 8);
+            // (in whole cache blocks: the plan is rebuilt when this changes, which should not be every few decode steps)
+            maskLen = std::max<int64_t>(DECODER_BLOCK_SIZE, (maskLen + DECODER_BLOCK_SIZE - 1) / DECODER_BLOCK_SIZE * DECODER_BLOCK_SIZE);
             maskFreeRows_ = static_cast<int32_t>(m.dims[m.dimNum - 2]);
             maskFreeBatch_ = m.dimNum == 3 ? batch : 0;
             maskLen_ = maskLen;
@@ -489,6 +490,7 @@ protected:
             maskFreeTableBytes_ = maskFreeTableBytes;
             maskFreeMaskOff_ = (maskFreeTableOff_ + maskFreeTableBytes + 255) / 256 * 256;
             workspaceSize = maskFreeMaskOff_ + static_cast<uint64_t>(q.desc.shape.dims[0]) * static_cast<uint64_t>(maskLen) * 2;
+            maskFreeBytes_ = workspaceSize;
         }
         return NO_ERROR;
     }
@@ -512,7 +514,7 @@ protected:
         t.blockTables = static_cast<const int32_t *>(pack.inTensors.at(BLOCK_TABLES).deviceData);
         uint64_t planBytes = workspaceSize;
         if (maskFree_) {
-            if (!workspace || workspaceSize < maskFreeMaskOff_) {
+            if (!workspace || workspaceSize < maskFreeBytes_) {
                 ATB_LOG(ERROR) << "MultiLatentAttention: the workspace is smaller than Setup asked for";
                 return ERROR_INVALID_PARAM;
             }
@@ -714,7 +716,7 @@ private:
     bool causalRows_ = false;
     int64_t maskLen_ = 0;
     int32_t maskFreeRows_ = 0, maskFreeBatch_ = 0;
-    uint64_t planBytes_ = 0, maskFreeTableOff_ = 0, maskFreeTableBytes_ = 0, maskFreeMaskOff_ = 0;
+    uint64_t planBytes_ = 0, maskFreeTableOff_ = 0, maskFreeTableBytes_ = 0, maskFreeMaskOff_ = 0, maskFreeBytes_ = 0;
     uint32_t inputNum_ = 6;
     AtbmiPaPlan *plan_ = nullptr;
     AtbmiPaShape planShape_{};

@@ -22,6 +22,7 @@
 // here; such params are rejected at creation with ERROR_INVALID_PARAM.
 // MASK_TYPE_MASK_FREE can be created and fails InferShape / Setup with
 // ERROR_INVALID_TENSOR_DIM, as the reference does off Atlas 300I Duo.
+#include <vector>
 #include <cmath>
 #include <new>
 #include "atb/infer_op_params.h"
@@ -521,7 +522,7 @@ protected:
             }
         }
         if (qkv_) {
-            return PlanQkv(pack, maskBatchStride, maskHeadStride, maskLen, workspaceSize);
+            return PlanQkv(pack, maskBatchStride, maskHeadStride, maskLen, maskRowBy, workspaceSize);
         }
         const int32_t *queryLens = nullptr;
         if (qLensIdx_ != NONE) {
@@ -637,8 +638,12 @@ private:
     // int8 queries: the kernel-library checks of the reference (src/kernels/mixkernels/pagedattention/
     // paged_attention_operation.cpp:357-403: one descale per query head, fp32) and the call of the kernel layer.
     Status PlanQkv(const VariantPack &pack, int64_t maskSeqStride, int64_t maskHeadStride, int64_t maskLen,
-                   uint64_t &workspaceSize)
+                   int32_t maskRowBy, uint64_t &workspaceSize)
     {
+        if (maskRowBy == ATBMI_PA_MASK_ROW_POSITION) {
+            ATB_LOG(ERROR) << "int8 queries: a mask whose rows go by position belongs to several query tokens";
+            return ERROR_INVALID_PARAM;
+        }
         const int64_t d = pack.inTensors.at(1).desc.shape.dims[3];
         if (d != 64 && d != 128 && d != 256) {
             ATB_LOG(ERROR) << "int8 queries: head size " << d << " (64, 128 and 256 are built)";
@@ -657,6 +662,16 @@ private:
         qkvMaskSeqStride_ = maskSeqStride;
         qkvMaskHeadStride_ = maskHeadStride;
         qkvMaskLen_ = maskLen;
+        qkvMaskRowByQuery_ = maskRowBy == ATBMI_PA_MASK_ROW_QUERY;
+        // the lengths as they are now: Execute works from this copy, like the other paths (the reference reads
+        // hostData during Setup only, src/ops/ops_infer/paged_attention/param.cpp:16-62)
+        const Tensor &lens = pack.inTensors.at(lensIdx_);
+        const int32_t *hostLens = static_cast<const int32_t *>(lens.hostData);
+        try {
+            qkvLens_.assign(hostLens, hostLens + lens.desc.shape.dims[0]);
+        } catch (const std::bad_alloc &) {
+            return ERROR_OUT_OF_HOST_MEMORY;
+        }
         AtbmiPaInt8QCall call = MakeQkvCall(pack);
         int rc = atbmi_pa_int8q_workspace_size(&call, &workspaceSize);
         if (rc != 0) {
@@ -687,7 +702,8 @@ private:
         c.qkScale = param_.qkScale;
         c.maskSeqStride = qkvMaskSeqStride_;
         c.maskHeadStride = qkvMaskHeadStride_;
-        c.hostContextLens = static_cast<const int32_t *>(lens.hostData);
+        c.hostContextLens = qkvLens_.data();
+        c.maskRowByQuery = qkvMaskRowByQuery_ ? 1 : 0;
         c.query = q.deviceData;
         c.keyCache = kc.deviceData;
         c.valueCache = pack.inTensors.at(2).deviceData;
@@ -894,6 +910,8 @@ private:
     int64_t qkvMaskSeqStride_ = 0;
     int64_t qkvMaskHeadStride_ = 0;
     int64_t qkvMaskLen_ = 0;
+    bool qkvMaskRowByQuery_ = false;
+    std::vector<int32_t> qkvLens_; // contextLens as read at Setup
     uint32_t inputNum_ = 5;
     AtbmiPaPlan *plan_ = nullptr;
     AtbmiPaShape planShape_{};

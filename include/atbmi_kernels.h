@@ -416,7 +416,9 @@ int atbmi_pa_decode(AtbmiPaPlan *plan, const AtbmiPaTensors *tensors, void *work
  * plans; more than 160 passes or 512 workgroup ranges): use atbmi_pa_decode then. Kernel timing
  * (atbmi_timing_enable) does not cover it. All calls on one GPU share the array: calls that may overlap on
  * one GPU (different streams, different threads) race; calls on one stream are safe. Results are those of
- * atbmi_pa_decode, bit for bit.
+ * atbmi_pa_decode, bit for bit. The FIRST call on a device, and the first with each kernel variant (head size, cache
+ * type, with or without a mask), looks up the array's address and raises the kernel's LDS limit, two runtime calls
+ * that do not belong inside a stream capture: make one call of each variant before capturing.
  */
 int atbmi_pa_decode_static(AtbmiPaPlan *plan, const AtbmiPaTensors *tensors, void *stream);
 uint64_t atbmi_pa_static_scratch_bytes(void);
@@ -577,6 +579,9 @@ typedef struct AtbmiPaInt8QCall {
     const float *pScale;       /* offline only */
     const void *mask;
     void *out;
+    int32_t maskRowByQuery;    /* 0: the mask row of a sequence is its index in hostContextLens; 1: the index of its query
+                                * row (MASK_TYPE_SPEC: mask [numQueryRows, maskLen], maskSeqStride = maskLen), which differs
+                                * when sequences without context come before it */
 } AtbmiPaInt8QCall;
 
 /* Validates the call (pointers aside) and reports the device workspace it needs: the table of context pieces

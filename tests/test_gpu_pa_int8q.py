@@ -267,25 +267,40 @@ def test_int8q_rejects_what_it_cannot_run(binding, dev, stream):
     assert k.atbmi_pa_int8q_workspace_size(ctypes.byref(call), ctypes.byref(ws)) != 0        # two rows asked for
     call.numQueryRows = 2
     assert k.atbmi_pa_int8q_decode(ctypes.byref(call), None, 0, stream.cuda_stream) != 0     # null tensors
+    # the kernel fetches the mask as aligned 32-bit words: odd strides or row lengths, or a base off a 4-byte
+    # boundary, would make it read outside the rows
+    call.hasMask, call.maskLen, call.maskSeqStride, call.mask = 1, 200, 200, 4096
+    assert k.atbmi_pa_int8q_workspace_size(ctypes.byref(call), ctypes.byref(ws)) == 0
+    for bad in (dict(maskLen=201, maskSeqStride=202), dict(maskSeqStride=201), dict(maskHeadStride=3), dict(mask=4098)):
+        for name, value in {**dict(maskLen=200, maskSeqStride=200, maskHeadStride=0, mask=4096), **bad}.items():
+            setattr(call, name, value)
+        assert k.atbmi_pa_int8q_workspace_size(ctypes.byref(call), ctypes.byref(ws)) != 0, bad
+        assert "4-byte" in binding.last_kernel_error()
 
 
 @pytest.mark.parametrize("offline,mask,dtype", [(False, "norm", torch.bfloat16), (True, None, torch.float16),
-                                                (False, "alibi", torch.float16)])
+                                                (False, "alibi", torch.float16), (False, "spec", torch.float16)])
 def test_paged_attention_operation_with_int8_queries(binding, oracle, dev, stream, offline, mask, dtype):
     """PagedAttentionOperation, quantType TYPE_QUANT_QKV_ONLINE (3) / OFFLINE (2), through Setup / Execute. Inputs:
     query, keyCache, valueCache, blockTables, contextLens, [mask], kDescale, vDescale, [pScale] (reference
     paged_attention_operation.cpp:408-444); the output comes in outDataType."""
     heads, kv_heads, d, block = 32, 2, 128, 128
-    c = _case(750 + int(offline), [3000, 300, 0, 33, 65, 1, 16, 1400, 300], heads, kv_heads, d, block, dtype, mask, offline)
+    # "spec": MASK_TYPE_SPEC, one mask row per QUERY row [rows, maxS]: the rows of the per-sequence mask of the
+    # sequences that have a context, so that the sequence behind the empty one reads row 2, not row 3
+    spec = mask == "spec"
+    c = _case(750 + int(offline), [3000, 300, 0, 33, 65, 1, 16, 1400, 300], heads, kv_heads, d, block, dtype,
+              "norm" if spec else mask, offline)
     scale = 1.0 / math.sqrt(d)
     lens = torch.from_numpy(c["ctx"])
     ctx = binding.Context(stream)
     op = binding.OperationRunner("PagedAttentionOperation", binding.PagedAttentionParam(
         headNum=heads, kvHeadNum=kv_heads, qkScale=scale, quantType=2 if offline else 3,
-        maskType={None: 0, "norm": 1, "alibi": 2}[mask],
+        maskType={None: 0, "norm": 1, "alibi": 2, "spec": 3}[mask],
         outDataType=binding.ACL_BF16 if dtype == torch.bfloat16 else binding.ACL_FLOAT16), ctx)
     ins = [c["q8"].to(dev), c["k8"].to(dev), c["v8"].to(dev), c["tables"].to(dev), lens.to(dev)]
-    if mask is not None:
+    if spec:
+        ins.append(c["mask"][torch.from_numpy(c["ctx"] > 0)][:, 0, :].contiguous().to(dev))
+    elif mask is not None:
         ins.append(c["mask"].to(dev))
     ins += [c["kd"].to(dev), c["vd"].to(dev)]
     if offline:
@@ -293,6 +308,7 @@ def test_paged_attention_operation_with_int8_queries(binding, oracle, dev, strea
     with torch.cuda.stream(stream):
         out = torch.full((c["rows"], heads, d), 7.0, dtype=dtype, device=dev)
         op.run(ins, outputs=[out], host_inputs={4: lens})
+
     stream.synchronize()
     # the operation leaves the cut of long contexts to the library (equal shares of the list of tiles, see
     # library_cuts): online that moves no int8 weight, offline it does (the weights are taken against each piece's own
@@ -301,7 +317,8 @@ def test_paged_attention_operation_with_int8_queries(binding, oracle, dev, strea
     assert cuts
     want = _oracle(oracle, c, scale, "own", piece_cuts=cuts)
     assert_close(out, want, TOL[dtype], "operation")
-    assert torch.equal(out, int8q_cabi(binding, stream, dev, c, scale, piece_tiles=0))
+    if not spec:
+        assert torch.equal(out, int8q_cabi(binding, stream, dev, c, scale, piece_tiles=0))
     ok, rates = _double_golden(_oracle(oracle, c, scale, None), want, out.float().cpu().numpy(), dtype)
     assert ok, rates
     # allocated from InferShape the output has the type outDataType names

@@ -689,15 +689,15 @@ def test_multi_latent_attention_causal_rows_and_mask_use_status(binding, ctx):
     assert op.setup(pack(128, mask=[129, 128], use_shape=[4], qlens_host=np.array([11, 3, 0, 2], np.int32)),
                     outs(128), ctx)[0] == e["ERROR_INVALID_PARAM"]
     op.close()
-    # fewer heads: the template is expanded into the workspace, one row of 304 (300 rounded up to 8) 16-bit values per
-    # query token, after the plan's own bytes and the 16-byte row records
+    # fewer heads: the template is expanded into the workspace, one row of 384 (300 rounded up to whole cache blocks)
+    # 16-bit values per query token, after the plan's own bytes and the 16-byte row records
     op = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1,
                                                                calcType=1, maskType=2))
     plain = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1,
                                                                   calcType=1, maskType=3))
     st, ws = op.setup(pack(32, mask=[131, 128]), outs(32, lse=False), ctx)
     st0, ws0 = plain.setup(pack(32), outs(32, lse=False), ctx)
-    assert (st, st0) == (0, 0) and ws >= ws0 + 8 * 16 + 8 * 304 * 2 and ws <= ws0 + 8 * 16 + 8 * 304 * 2 + 1024
+    assert (st, st0) == (0, 0) and ws >= ws0 + 8 * 16 + 8 * 384 * 2 and ws <= ws0 + 8 * 16 + 8 * 384 * 2 + 1024
     assert op.setup(pack(32, mask=[4, 131, 128]), outs(32, lse=False), ctx)[0] == 0           # a template per sequence
     assert op.setup(pack(32, mask=[3, 131, 128]), outs(32, lse=False), ctx)[0] == e["ERROR_INVALID_PARAM"]
     assert op.setup(pack(32, mask=[131, 64]), outs(32, lse=False), ctx)[0] == e["ERROR_INVALID_PARAM"]

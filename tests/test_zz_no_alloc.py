@@ -100,9 +100,9 @@ def test_static_scratch_decode_refuses_what_does_not_fit(binding):
     t = binding.AtbmiPaTensors()
     dummy = torch.zeros(64, device=dev)
     t.query = t.keyCache = t.blockTables = t.out = dummy.data_ptr()
-    if big > (32 << 20):
-        assert k.atbmi_pa_decode_static(plan, ctypes.byref(t), None) == 1
-        assert "static scratch" in binding.last_kernel_error()
+    assert big > k.atbmi_pa_static_scratch_bytes(), "the case is meant to need more partial rows than the scratch holds"
+    assert k.atbmi_pa_decode_static(plan, ctypes.byref(t), None) == 1
+    assert "static scratch" in binding.last_kernel_error()
     k.atbmi_pa_plan_destroy(plan)
     # a scalar-kernel plan uploads its tables: refused as well
     shape = binding.AtbmiPaShape(qDtype=0, kvDtype=0, numHeads=8, numKvHeads=8, headDimK=128, headDimV=128,
