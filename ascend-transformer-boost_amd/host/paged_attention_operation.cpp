@@ -786,6 +786,14 @@ private:
             batchStride = m.dims[2];
             headStride = 0;
             seqDiv = static_cast<int32_t>(pairs);
+        } else if (!alibi && m.dimNum == 4) {
+            // The reference lets (batch, 1 | heads, 1, maxS) through for every mask type (kernel library
+            // paged_attention_operation.cpp:760) but its tiling derives strides for the 2- and 3-dim NORM
+            // shapes only (tiling/paged_attention_tiling.cpp:62-74): both strides stay 0, and every sequence
+            // and head reads the first row of the tensor. The same here.
+            ok = m.dims[0] == batch && (m.dims[1] == 1 || m.dims[1] == heads) && m.dims[2] == 1 && !compress_;
+            batchStride = 0;
+            headStride = 0;
         } else if (alibi && m.dimNum == 3) {
             ok = m.dims[0] == heads && m.dims[1] == 1;
             batchStride = compress_ ? heads / kvHeads * m.dims[2] : 0;
@@ -798,7 +806,7 @@ private:
             seqDiv = m.dims[1] == 1 ? static_cast<int32_t>(pairs) : 0;
         }
         if (!ok) {
-            ATB_LOG(ERROR) << "mask shape is not one of NORM (1,maxS) / (batch,1,maxS), "
+            ATB_LOG(ERROR) << "mask shape is not one of NORM (1,maxS) / (batch,1,maxS) / (batch,1|heads,1,maxS), "
                               "ALIBI (heads,1,maxS) / (batch,1|heads,1,maxS), or with CALC_TYPE_SPEC "
                               "SPEC (query rows,maxS) / NORM (maxS,maxS)";
             return ERROR_INVALID_PARAM;

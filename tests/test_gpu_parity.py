@@ -1465,6 +1465,34 @@ def test_mask_rows_follow_the_sequence_index_past_empty_sequences(binding, oracl
     assert_close(got, want, 1e-3, "empty+mask")
 
 
+def test_four_dim_norm_mask_reads_its_first_row(binding, oracle, dev, stream):
+    """MASK_TYPE_NORM with a (batch, heads, 1, maxS) mask through the operation: the reference lets the shape through
+    (kernel library paged_attention_operation.cpp:760) while its tiling derives strides for the 2- and 3-dim NORM
+    masks only (tiling/paged_attention_tiling.cpp:62-74), so both strides stay 0 and every sequence and head reads
+    the tensor's first row. The result must equal the oracle with that row as a (1, maxS) mask, and differ from the
+    reading by sequence and head."""
+    rng = _rng(233)
+    heads, kv_heads, d, block, dtype = 8, 2, 128, 16, torch.float16
+    ctx = np.array([300, 17, 0, 129], dtype=np.int32)
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, len(ctx), heads, kv_heads, block, d, d, ctx, dtype)
+    mask = torch.from_numpy((rng.standard_normal((len(ctx), heads, 1, 304)) * 2).astype(np.float32)).to(dtype).to(dev)
+    scale = 1.0 / math.sqrt(d)
+    lens = torch.from_numpy(ctx)
+    c = binding.Context(stream)
+    op = binding.OperationRunner("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=heads, kvHeadNum=kv_heads, qkScale=scale, maskType=1), c)
+    with torch.cuda.stream(stream):
+        out = torch.full((len(ctx), heads, d), 0.1, dtype=dtype, device=dev)
+        op.run([q, kc, vc, tables, lens.to(dev), mask], outputs=[out], host_inputs={4: lens})
+    stream.synchronize()
+    first_row = oracle_pa(oracle, q, kc, vc, tables, ctx, scale, out_init=0.1, mask=mask[0, 0].reshape(1, -1))
+    by_index = oracle_pa(oracle, q, kc, vc, tables, ctx, scale, out_init=0.1, mask=mask)
+    assert np.abs(first_row - by_index).max() > 0.01
+    assert_close(out, first_row, TOL[dtype], "4-dim NORM mask")
+    op.close()
+    c.close()
+
+
 @pytest.mark.parametrize("kernel", [1, 0])
 @pytest.mark.parametrize("chunk", [64, 1024])
 def test_minus_infinity_mask_hides_whole_ranges(binding, oracle, dev, stream, kernel, chunk):
