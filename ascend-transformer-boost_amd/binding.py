@@ -89,6 +89,11 @@ class ReshapeAndCacheWithStrideParam(ReshapeAndCacheParam):
     """Byte image of atb::infer::ReshapeAndCacheWithStrideParam (24 bytes, the same fields)."""
 
 
+class ReshapeAndCacheOmniParam(ctypes.Structure):
+    """Byte image of atb::infer::ReshapeAndCacheOmniParam (8 reserved bytes)."""
+    _fields_ = [("rsv", ctypes.c_uint8 * 8)]
+
+
 class ElewiseParam(ctypes.Structure):
     """Byte image of atb::infer::ElewiseParam (64 bytes: type, QuantParam 32, MulsParam 16, out type, rsv)."""
     _fields_ = [("elewiseType", ctypes.c_int32), ("inputScale", ctypes.c_float), ("asymmetric", ctypes.c_bool),
@@ -253,6 +258,7 @@ def kernels():
         lib.atbmi_reshape_and_cache_strided.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp, i64, vp,
                                                         i64, vp]
         lib.atbmi_reshape_and_cache_compress.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]
+        lib.atbmi_reshape_and_cache_omni.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]
         lib.atbmi_norm_rope_reshape_and_cache.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32,
                                                           ctypes.c_float, vp]
         lib.atbmi_rope.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i32, i32, i32, i32, vp]

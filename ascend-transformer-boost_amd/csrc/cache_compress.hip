@@ -12,6 +12,11 @@
 //     whole sequence (golden test_reshape_and_cache_wins_rope.py:78-131, device
 //     kernel op_kernel/reshape_and_cache_compress_rope.cpp:30-108: fp32 sum in
 //     token order, one fp32 division by the window length, round to nearest even).
+//   drop-window (ReshapeAndCacheOmniOperation): as mean-window, but the window leaves nothing behind: the tokens
+//     before o, then at once the tokens from o + wins[i] on (golden
+//     tests/framework/python/CsvOpsTestTool/data_generation.py:9797-9846 and
+//     tests/apitest/kernelstest/mix/test_reshape_and_cache_omni_compress.py:80-116, device kernel
+//     op_kernel/reshape_and_cache_omni_compress.cpp:87-110 with reshape_and_cache_base.h:276-289).
 //
 // Pure data movement apart from the mean: 16-byte pieces, consecutive lanes on
 // consecutive pieces of a token row. Sequence starts are the prefix sums of
@@ -38,7 +43,7 @@ struct CompressArgs {
     const int32_t *slots;  // [batch * heads] first slot of the pair, < 0: skip
     const int32_t *wins;   // [batch * heads]
     const int32_t *seqLens; // [batch]
-    const int32_t *offsets; // [batch * heads], mean-window only
+    const int32_t *offsets; // [batch * heads], first token of the window (mean-window, drop-window)
     int32_t heads;
     int32_t rowBytes;  // headSize * element size, a multiple of 16
     int64_t numTokens; // rows of key / value
@@ -101,6 +106,44 @@ __global__ __launch_bounds__(CC_THREADS) void CompressKeepLastKernel(const Compr
     const int64_t end = SequenceStart(a.seqLens, b, scratch) + a.seqLens[b];
     const int64_t win = a.wins[pair];
     CopyRows(a, blockIdx.z, h, end - win, slot, win, blockIdx.y, gridDim.y);
+}
+
+// The window [off, off + win) of the sequence is left out, the tokens after it close up.
+__global__ __launch_bounds__(CC_THREADS) void CompressDropWindowKernel(const CompressArgs a)
+{
+    __shared__ int64_t scratch[CC_THREADS / WAVE];
+    const int pair = blockIdx.x;
+    const int32_t slot = a.slots[pair];
+    if (slot < 0) {
+        return;
+    }
+    const int b = pair / a.heads;
+    const int h = pair % a.heads;
+    const int64_t start = SequenceStart(a.seqLens, b, scratch);
+    const int64_t len = a.seqLens[b];
+    const int64_t off = a.offsets[pair];
+    const int64_t win = a.wins[pair];
+    if (off < 0 || win <= 0 || off >= len) { // no window: the whole sequence as it is
+        CopyRows(a, blockIdx.z, h, start, slot, len, blockIdx.y, gridDim.y);
+        return;
+    }
+    // one run of rows for the workers to share: row j comes from token j, or from j + win once past the window
+    const int64_t after = len - off - win > 0 ? len - off - win : 0;
+    const int pieces = a.rowBytes / 16;
+    const int64_t total = (off + after) * pieces;
+    const int which = blockIdx.z;
+    for (int64_t at = static_cast<int64_t>(blockIdx.y) * CC_THREADS + threadIdx.x; at < total;
+         at += static_cast<int64_t>(gridDim.y) * CC_THREADS) {
+        const int64_t j = at / pieces;
+        const int p = static_cast<int>(at % pieces);
+        const int64_t tok = start + (j < off ? j : j + win);
+        const int64_t dst = slot + j;
+        if (tok < 0 || tok >= a.numTokens || dst >= a.numSlots) {
+            continue;
+        }
+        const uint4 v = *reinterpret_cast<const uint4 *>(a.src[which] + (tok * a.heads + h) * a.rowBytes + p * 16);
+        *reinterpret_cast<uint4 *>(a.dst[which] + dst * a.rowBytes + p * 16) = v;
+    }
 }
 
 template <bool BF16>
@@ -211,40 +254,43 @@ __global__ __launch_bounds__(CC_THREADS) void CompressMeanWindowKernel(const Com
 
 using namespace atbmi;
 
-extern "C" int atbmi_reshape_and_cache_compress(const void *key, const void *value, void *keyCache, void *valueCache,
-                                                const int32_t *slotMapping, const int32_t *wins,
-                                                const int32_t *seqLens, const int32_t *offsetIndex, int64_t batch,
-                                                int64_t numHeads, int64_t headSize, int64_t numTokens,
-                                                int64_t numSlots, int32_t dtype, void *stream)
+namespace {
+enum CompressMode { KEEP_LAST, MEAN_WINDOW, DROP_WINDOW };
+
+int CompressImpl(const char *name, CompressMode mode, const void *key, const void *value, void *keyCache,
+                 void *valueCache, const int32_t *slotMapping, const int32_t *wins, const int32_t *seqLens,
+                 const int32_t *offsetIndex, int64_t batch, int64_t numHeads, int64_t headSize, int64_t numTokens,
+                 int64_t numSlots, int32_t dtype, void *stream)
 {
     if (!key || !value || !keyCache || !valueCache || !slotMapping || !wins || !seqLens) {
-        return Fail(ERR_INVALID_PARAM, "reshape_and_cache_compress: key, value, the caches, slotMapping, wins and seqLens "
-                                       "must be non-null");
+        return Fail(ERR_INVALID_PARAM, "%s: key, value, the caches, slotMapping, wins and seqLens must be non-null", name);
+    }
+    if (mode == DROP_WINDOW && !offsetIndex) {
+        return Fail(ERR_INVALID_PARAM, "%s: offsetIndex must be non-null", name);
     }
     if (dtype != ATBMI_F16 && dtype != ATBMI_BF16 && dtype != ATBMI_INT8) {
-        return Fail(ERR_INVALID_PARAM, "reshape_and_cache_compress: dtype %d", dtype);
+        return Fail(ERR_INVALID_PARAM, "%s: dtype %d", name, dtype);
     }
-    if (offsetIndex && dtype == ATBMI_INT8) {
-        return Fail(ERR_INVALID_PARAM, "reshape_and_cache_compress: the mean of a window needs fp16 or bf16 rows");
+    if (mode == MEAN_WINDOW && dtype == ATBMI_INT8) {
+        return Fail(ERR_INVALID_PARAM, "%s: the mean of a window needs fp16 or bf16 rows", name);
     }
     if (batch < 0 || numHeads <= 0 || headSize <= 0 || numTokens < 0 || numSlots <= 0) {
-        return Fail(ERR_INVALID_PARAM, "reshape_and_cache_compress: bad extents");
+        return Fail(ERR_INVALID_PARAM, "%s: bad extents", name);
     }
-    if (offsetIndex && headSize > MEAN_MAX_CHANNELS) {
-        return Fail(ERR_INVALID_PARAM, "reshape_and_cache_compress: the window mean is built for head sizes up to %d, "
-                                       "got %lld", MEAN_MAX_CHANNELS, (long long)headSize);
+    if (mode == MEAN_WINDOW && headSize > MEAN_MAX_CHANNELS) {
+        return Fail(ERR_INVALID_PARAM, "%s: the window mean is built for head sizes up to %d, got %lld", name,
+                    MEAN_MAX_CHANNELS, (long long)headSize);
     }
     if (headSize % 32 != 0) {
-        return Fail(ERR_INVALID_PARAM, "reshape_and_cache_compress: headSize %lld is not a multiple of 32",
-                    (long long)headSize);
+        return Fail(ERR_INVALID_PARAM, "%s: headSize %lld is not a multiple of 32", name, (long long)headSize);
     }
     const int64_t pairs = batch * numHeads;
     if (pairs > 0x7fffffffLL || numHeads > 0x7fffffffLL || headSize > (1 << 20)) {
-        return Fail(ERR_INVALID_PARAM, "reshape_and_cache_compress: extents out of range");
+        return Fail(ERR_INVALID_PARAM, "%s: extents out of range", name);
     }
     for (const void *p : {key, value, static_cast<const void *>(keyCache), static_cast<const void *>(valueCache)}) {
         if (!Aligned(p, 16)) {
-            return Fail(ERR_INVALID_PARAM, "reshape_and_cache_compress: tensors must start on 16-byte boundaries");
+            return Fail(ERR_INVALID_PARAM, "%s: tensors must start on 16-byte boundaries", name);
         }
     }
     if (pairs == 0 || numTokens == 0) {
@@ -267,11 +313,13 @@ extern "C" int atbmi_reshape_and_cache_compress(const void *key, const void *val
     const int64_t rowsPerPair = (numTokens + batch - 1) / batch;
     int64_t workers = (rowsPerPair + 63) / 64;
     workers = workers < 1 ? 1 : (workers > 64 ? 64 : workers);
-    workers += offsetIndex ? 1 : 0; // the one that takes the window's mean
+    workers += mode == MEAN_WINDOW ? 1 : 0; // the one that takes the window's mean
     dim3 grid(static_cast<unsigned>(pairs), static_cast<unsigned>(workers), 2);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (!offsetIndex) {
+    if (mode == KEEP_LAST) {
         CompressKeepLastKernel<<<grid, CC_THREADS, 0, s>>>(a);
+    } else if (mode == DROP_WINDOW) {
+        CompressDropWindowKernel<<<grid, CC_THREADS, 0, s>>>(a);
     } else if (dtype == ATBMI_BF16) {
         CompressMeanWindowKernel<true><<<grid, CC_THREADS, 0, s>>>(a);
     } else {
@@ -279,4 +327,26 @@ extern "C" int atbmi_reshape_and_cache_compress(const void *key, const void *val
     }
     ATBMI_HIP_CHECK(hipGetLastError());
     return OK;
+}
+} // namespace
+
+extern "C" int atbmi_reshape_and_cache_compress(const void *key, const void *value, void *keyCache, void *valueCache,
+                                                const int32_t *slotMapping, const int32_t *wins,
+                                                const int32_t *seqLens, const int32_t *offsetIndex, int64_t batch,
+                                                int64_t numHeads, int64_t headSize, int64_t numTokens,
+                                                int64_t numSlots, int32_t dtype, void *stream)
+{
+    return CompressImpl("reshape_and_cache_compress", offsetIndex ? MEAN_WINDOW : KEEP_LAST, key, value, keyCache,
+                        valueCache, slotMapping, wins, seqLens, offsetIndex, batch, numHeads, headSize, numTokens,
+                        numSlots, dtype, stream);
+}
+
+extern "C" int atbmi_reshape_and_cache_omni(const void *key, const void *value, void *keyCache, void *valueCache,
+                                            const int32_t *slotMapping, const int32_t *wins, const int32_t *seqLens,
+                                            const int32_t *offsetIndex, int64_t batch, int64_t numHeads,
+                                            int64_t headSize, int64_t numTokens, int64_t numSlots, int32_t dtype,
+                                            void *stream)
+{
+    return CompressImpl("reshape_and_cache_omni", DROP_WINDOW, key, value, keyCache, valueCache, slotMapping, wins,
+                        seqLens, offsetIndex, batch, numHeads, headSize, numTokens, numSlots, dtype, stream);
 }

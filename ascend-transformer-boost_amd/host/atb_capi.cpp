@@ -101,6 +101,11 @@ int32_t atb_c_create_operation(const char *opName, const void *param, uint64_t p
         memcpy(static_cast<void *>(&p), param, sizeof(p));
         return atb::CreateOperation(p, out);
     }
+    if (!strcmp(opName, "ReshapeAndCacheOmniOperation") && paramSize == sizeof(atb::infer::ReshapeAndCacheOmniParam)) {
+        atb::infer::ReshapeAndCacheOmniParam p;
+        memcpy(static_cast<void *>(&p), param, sizeof(p));
+        return atb::CreateOperation(p, out);
+    }
     if (!strcmp(opName, "NormRopeReshapeOperation") && paramSize == sizeof(atb::infer::NormRopeReshapeParam)) {
         atb::infer::NormRopeReshapeParam p;
         memcpy(static_cast<void *>(&p), param, sizeof(p));

@@ -15,8 +15,8 @@ Differences from the reference module, all forced by the operators themselves: t
 device ("cuda" in torch); the work runs on torch's current stream of the first device tensor (on a side
 stream ordered after it when that is the null stream, which a Context does not take); operators
 whose outputs are their inputs updated in place (ReshapeAndCache, NormRopeReshape, PagedCacheLoad) return those input
-tensors instead of fresh ones. ReshapeAndCacheWithStrideParam, NormRopeReshapeParam, MultiLatentAttentionParam,
-BlockCopyParam and PagedCacheLoadParam are not bound by the reference's module; they are offered here in the same style
+tensors instead of fresh ones. ReshapeAndCacheWithStrideParam, ReshapeAndCacheOmniParam, NormRopeReshapeParam,
+MultiLatentAttentionParam, BlockCopyParam and PagedCacheLoadParam are not bound by the reference's module; they are offered here in the same style
 (for ReshapeAndCacheWithStride, key / value are [tokens, heads, head_size] tensors that start at the base
 of the storage which the strides and the offset index into).
 """
@@ -122,6 +122,11 @@ class ReshapeAndCacheWithStrideParam(_Param):
         K_CACHE_V_BYPASS = 1
 
 
+class ReshapeAndCacheOmniParam(_Param):
+    _struct = _b.ReshapeAndCacheOmniParam
+    _op_name = "ReshapeAndCacheOmniOperation"
+
+
 class ElewiseParam(_Param):
     _struct = _b.ElewiseParam
     _op_name = "ElewiseOperation"
@@ -184,6 +189,7 @@ class PagedCacheLoadParam(_Param):
 _IN_PLACE = {
     "ReshapeAndCacheOperation": {5: [2, 3], 3: [1], 7: [2, 3], 8: [2, 3]},  # 7 / 8: head compression
     "ReshapeAndCacheWithStrideOperation": {9: [2, 3], 5: [1]},
+    "ReshapeAndCacheOmniOperation": {8: [2, 3]},
     "NormRopeReshapeOperation": {7: [6]},
     "PagedCacheLoadOperation": {7: [4, 5]},
 }

@@ -56,6 +56,14 @@ struct ReshapeAndCacheWithStrideParam {
     uint8_t rsv[16] = {0}; // must stay zero
 };
 
+// ReshapeAndCache for caches compressed by dropping a window of tokens per (sequence, head) pair:
+// inputs key, value [tokens, heads, headSize], keyCache, valueCache [blocks, blockSize, 1, headSize],
+// slotMapping, wins [batch * heads], seqLen [batch], offsetIndex [batch * heads]; outputs the caches
+// (reference include/atb/infer_op_params.h:2883-2894).
+struct ReshapeAndCacheOmniParam {
+    uint8_t rsv[8] = {0}; // must stay zero
+};
+
 // Decode attention: one query token per sequence against that sequence's
 // cached keys/values, found through blockTables and bounded by contextLens.
 struct PagedAttentionParam {
@@ -251,6 +259,7 @@ struct PagedCacheLoadParam {
 
 static_assert(sizeof(ReshapeAndCacheParam) == 24, "ReshapeAndCacheParam ABI size");
 static_assert(sizeof(ReshapeAndCacheWithStrideParam) == 24, "ReshapeAndCacheWithStrideParam ABI size");
+static_assert(sizeof(ReshapeAndCacheOmniParam) == 8, "ReshapeAndCacheOmniParam ABI size");
 static_assert(sizeof(ElewiseParam) == 64 && sizeof(ElewiseParam::QuantParam) == 32 && sizeof(ElewiseParam::MulsParam) == 16,
               "ElewiseParam ABI size");
 static_assert(sizeof(RopeParam) == 16, "RopeParam ABI size");

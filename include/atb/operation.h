@@ -35,7 +35,7 @@ public:
 };
 
 // Specialised for infer::PagedAttentionParam, ReshapeAndCacheParam, ReshapeAndCacheWithStrideParam,
-// RopeParam, ElewiseParam, NormRopeReshapeParam, MultiLatentAttentionParam, BlockCopyParam and PagedCacheLoadParam.
+// ReshapeAndCacheOmniParam, RopeParam, ElewiseParam, NormRopeReshapeParam, MultiLatentAttentionParam, BlockCopyParam and PagedCacheLoadParam.
 template <typename OpParam> Status CreateOperation(const OpParam &opParam, Operation **operation);
 
 Status DestroyOperation(Operation *operation);

@@ -39,12 +39,12 @@ int32_t atb_c_context_set_execute_type(void *context, int32_t type);
 int32_t atb_c_destroy_context(void *context);
 
 /* atb::CreateOperation for infer::PagedAttentionParam, ReshapeAndCacheParam,
- * ReshapeAndCacheWithStrideParam, RopeParam, ElewiseParam, NormRopeReshapeParam, MultiLatentAttentionParam,
- * BlockCopyParam and PagedCacheLoadParam. opName is the operation's name ("PagedAttentionOperation",
- * "ReshapeAndCacheOperation", "ReshapeAndCacheWithStrideOperation", "RopeOperation", "ElewiseOperation",
- * "NormRopeReshapeOperation", "MultiLatentAttentionOperation", "BlockCopyOperation",
- * "PagedCacheLoadOperation"); param points at the bytes of the matching C++ param struct
- * (120 / 24 / 24 / 16 / 64 / 28 / 64 / 16 / 64 bytes). */
+ * ReshapeAndCacheWithStrideParam, ReshapeAndCacheOmniParam, RopeParam, ElewiseParam, NormRopeReshapeParam,
+ * MultiLatentAttentionParam, BlockCopyParam and PagedCacheLoadParam. opName is the operation's name
+ * ("PagedAttentionOperation", "ReshapeAndCacheOperation", "ReshapeAndCacheWithStrideOperation",
+ * "ReshapeAndCacheOmniOperation", "RopeOperation", "ElewiseOperation", "NormRopeReshapeOperation",
+ * "MultiLatentAttentionOperation", "BlockCopyOperation", "PagedCacheLoadOperation"); param points at the bytes of
+ * the matching C++ param struct (120 / 24 / 24 / 8 / 16 / 64 / 28 / 64 / 16 / 64 bytes). */
 int32_t atb_c_create_operation(const char *opName, const void *param, uint64_t paramSize, void **operation);
 /* atb::DestroyOperation. */
 int32_t atb_c_destroy_operation(void *operation);

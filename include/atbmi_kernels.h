@@ -87,6 +87,24 @@ int atbmi_reshape_and_cache_compress(const void *keyDevice, const void *valueDev
                                      void *stream);
 
 /*
+ * KV-cache write of ReshapeAndCacheOmniOperation: the arguments and the layout of atbmi_reshape_and_cache_compress,
+ * offsetIndex required, and a window that leaves nothing behind. With o = offsetIndex[i] and w = wins[i], pair i
+ * writes the tokens [0, o) of its sequence and then at once the tokens [o + w, seqLens[b]) to consecutive slots from
+ * slotMapping[i] on; o == -1, w <= 0 or o >= seqLens[b] copies the whole sequence; a window that runs past the end
+ * of the sequence leaves only the tokens before it. A byte copy (fp16 / bf16 rows in the reference, one-byte rows
+ * work too).
+ * Replaces: reshape_and_cache_omni_compress.cpp:87-110 of the reference (src/kernels/mixkernels/reshape_and_cache/
+ * op_kernel/, parameters read as reshape_and_cache_base.h:276-289 does; goldens
+ * tests/framework/python/CsvOpsTestTool/data_generation.py:9797-9846 and
+ * tests/apitest/kernelstest/mix/test_reshape_and_cache_omni_compress.py:80-116).
+ */
+int atbmi_reshape_and_cache_omni(const void *keyDevice, const void *valueDevice, void *keyCacheDevice,
+                                 void *valueCacheDevice, const int32_t *slotMappingDevice,
+                                 const int32_t *winsDevice, const int32_t *seqLensDevice,
+                                 const int32_t *offsetIndexDevice, int64_t batch, int64_t numHeads, int64_t headSize,
+                                 int64_t numTokens, int64_t numSlots, int32_t dtype, void *stream);
+
+/*
  * KV-cache write into fractal-NZ caches (ReshapeAndCacheParam::K_CACHE_V_CACHE_NZ), the writer of the caches
  * MultiLatentAttention reads with cacheMode NZCACHE / INT8_NZCACHE. keyCache is
  * [numBlocks, keyRowElems / L, blockSize, L] with L = 32 for one-byte and 16 for two-byte keys, valueCache

@@ -22,6 +22,12 @@ the invariants of the mathematics (no function is left "parity unpinned"):
                       tokens of every (sequence, head) pair) and test_reshape_and_cache_wins_rope.py:78-131 (a
                       window replaced by its mean); pinned by element loops over flat addresses, the slot
                       counts, a one-token window = plain copy, and the float64 mean
+  reshape_and_cache_omni
+                      tests/framework/python/CsvOpsTestTool/data_generation.py:9797-9846 and
+                      tests/apitest/kernelstest/mix/test_reshape_and_cache_omni_compress.py:80-116 (a window of
+                      tokens per (sequence, head) pair is left out); pinned by element loops over flat addresses
+                      with an index list built another way, the slot counts, no window = the plain write of one
+                      head, and mean-window's result with its mean slot taken out
   dequant_per_channel tests/apitest/opstest/python/operations/elewise/test_elewise_dequant.py:23-31
   strided_view        tests/unittest/ops/reshape_and_cache_with_stride/test_reshape_and_cache_with_stride.cpp:
                       219-245 (element [i0, i1, i2] of the view is storage[offset + sum(i_k * stride_k)]),
@@ -242,6 +248,38 @@ def reshape_and_cache_compress(key, value, key_cache, value_cache, slot_mapping,
                 slot += 1
             elif j >= off + win:
                 put(slot, key[tok, h], value[tok, h])
+                slot += 1
+    return kc, vc
+
+
+def reshape_and_cache_omni(key, value, key_cache, value_cache, slot_mapping, wins, seq_lens, offset_index):
+    """KV-cache write of ReshapeAndCacheOmniOperation; caches [blocks, block, 1, D] (copied and returned),
+    pairs and sequences as in reshape_and_cache_compress. Token j of the pair's sequence goes to the pair's
+    next free slot when o = offset_index[i] is -1, when j < o, or when j >= o + wins[i]: the window
+    [o, o + wins[i]) leaves nothing behind (reference goldens
+    tests/framework/python/CsvOpsTestTool/data_generation.py:9797-9846 and
+    tests/apitest/kernelstest/mix/test_reshape_and_cache_omni_compress.py:80-116; the device kernel,
+    src/kernels/mixkernels/reshape_and_cache/op_kernel/reshape_and_cache_omni_compress.cpp:87-110 with
+    reshape_and_cache_base.h:276-289, copies [0, o) and then [o + w, seqLen), and takes w == 0 as no window).
+    wins[i] < 0 is outside the reference's domain (its kernel reads the count as unsigned, its golden
+    would skip slots); it is taken as no window here."""
+    kc = np.array(key_cache, copy=True)
+    vc = np.array(value_cache, copy=True)
+    heads = key.shape[1]
+    block = kc.shape[1]
+    ends = np.cumsum(np.asarray(seq_lens, dtype=np.int64))
+    starts = ends - np.asarray(seq_lens, dtype=np.int64)
+    for i, slot in enumerate(np.asarray(slot_mapping).tolist()):
+        if slot < 0:
+            continue
+        b, h = divmod(i, heads)
+        off = int(offset_index[i])
+        win = max(int(wins[i]), 0)
+        for j in range(int(seq_lens[b])):
+            tok = int(starts[b]) + j
+            if off == -1 or j < off or j >= off + win:
+                kc[slot // block, slot % block, 0] = key[tok, h]
+                vc[slot // block, slot % block, 0] = value[tok, h]
                 slot += 1
     return kc, vc
 

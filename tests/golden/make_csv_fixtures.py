@@ -12,6 +12,7 @@ status, tagged C: for CreateOperation, I: for InferShape, S: for Setup):
     tests/apitest/opstest/csv/norm_rope_reshape.csv
     tests/apitest/opstest/csv/rope.csv
     tests/apitest/opstest/csv/elewise.csv (the rows of the two per-channel quantiser types)
+    tests/apitest/opstest/csv/reshape_and_cache_omni.csv
 Those rows are data, not code. This script copies the rows written for the
 Ascend910B feature set (the one this library mirrors) into
     tests/golden/paged_attention_cases.json
@@ -22,6 +23,7 @@ Ascend910B feature set (the one this library mirrors) into
     tests/golden/norm_rope_reshape_cases.json
     tests/golden/rope_cases.json
     tests/golden/elewise_cases.json
+    tests/golden/reshape_and_cache_omni_cases.json
 so the parity tests can run where the reference tree is absent.
 
 Run from the repository root in a container that has /root/reference:
@@ -97,3 +99,4 @@ if __name__ == "__main__":
     convert("norm_rope_reshape", also_untagged=True)
     convert("rope", also_untagged=True)
     convert("elewise", also_untagged=True, keep=lambda p: p.get("elewiseType") in (17, 18))
+    convert("reshape_and_cache_omni")

@@ -365,6 +365,65 @@ def test_reshape_and_cache_head_compression_bit_exact(binding, oracle, dev, stre
         assert torch.equal(_bits(got.cpu()), _bits(want_t)), what
 
 
+OMNI_CASES = [
+    (1, 1, 256, 256, torch.bfloat16, (1024, 4096)),  # reference test_reshape_and_cache_omni_compress.py, one pair
+    (40, 1, 96, 128, torch.float16, (200, 900)),     # its many-sequence shape (head size 96), shorter sequences
+    (3, 8, 128, 128, torch.float16, (1, 700)),
+    (5, 4, 64, 16, torch.bfloat16, (30, 300)),
+]
+
+
+@pytest.mark.parametrize("case", OMNI_CASES, ids=lambda c: "b%d_h%d_d%d_bs%d_%s" % (
+    c[0], c[1], c[2], c[3], str(c[4]).split(".")[-1]))
+def test_reshape_and_cache_omni_bit_exact(binding, oracle, dev, stream, case):
+    """ReshapeAndCacheOmniOperation (a window of tokens per (sequence, head) pair is left out) bit for bit against
+    the oracle: pairs without a window (offset -1, or a window of no tokens), windows at the start, at the end and
+    past the end of their sequence, a skipped pair; slots outside the pairs' stretches keep their contents."""
+    batch, heads, d, block, dtype, (lo, hi) = case
+    rng = _rng(1300 + batch + heads + d)
+    seq = rng.integers(lo, hi, size=batch).astype(np.int32)
+    tokens = int(seq.sum())
+    pairs = batch * heads
+    per_seq = np.repeat(seq, heads)
+    wins = np.minimum(rng.integers(0, hi, size=pairs), per_seq).astype(np.int32)
+    offs = np.array([rng.integers(-1, n - w + 1) for n, w in zip(per_seq, wins)], dtype=np.int32)
+    offs[0] = -1
+    if pairs > 5:
+        wins[1] = 0
+        offs[3], wins[3] = 0, max(1, per_seq[3] // 2)               # the window opens the sequence
+        offs[4] = per_seq[4] - wins[4]                               # ... ends it
+        offs[5], wins[5] = per_seq[5] // 2, per_seq[5]               # ... runs past its end
+    kept = np.where((offs < 0) | (wins == 0), per_seq, np.minimum(offs, per_seq) + np.maximum(per_seq - offs - wins, 0))
+    order = rng.permutation(pairs)
+    nblocks = (kept + block - 1) // block
+    first = np.zeros(pairs, dtype=np.int64)
+    first[order] = np.concatenate([[0], np.cumsum(nblocks[order])[:-1]])
+    slots = (first * block).astype(np.int32)
+    if pairs > 2:
+        slots[2] = -1
+    blocks = int(nblocks.sum()) + 2
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(int(rng.integers(1 << 30)))
+    mk = lambda *shape: ((torch.rand(shape, generator=gen) * 10 - 5)).to(dtype)
+    key, value = mk(tokens, heads, d), mk(tokens, heads, d)
+    kc0, vc0 = mk(blocks, block, 1, d), mk(blocks, block, 1, d)
+    ins = [key.to(dev), value.to(dev), kc0.to(dev), vc0.to(dev)] + \
+          [torch.from_numpy(a).to(dev) for a in (slots, wins, seq, offs)]
+    c = binding.Context(stream)
+    op = binding.OperationRunner("ReshapeAndCacheOmniOperation", binding.ReshapeAndCacheOmniParam(), c)
+    with torch.cuda.stream(stream):
+        op.run(ins, outputs=[ins[2], ins[3]])
+    stream.synchronize()
+    op.close()
+    c.close()
+    want_k, want_v = oracle.reshape_and_cache_omni(to_oracle(key), to_oracle(value), to_oracle(kc0), to_oracle(vc0),
+                                                   slots, wins, seq, offs)
+    assert not np.array_equal(want_k, to_oracle(kc0))
+    for got, want, what in ((ins[2], want_k, "key"), (ins[3], want_v, "value")):
+        want_t = torch.from_numpy(np.ascontiguousarray(want)).to(dtype)
+        assert torch.equal(_bits(got.cpu()), _bits(want_t)), what
+
+
 def test_reshape_and_cache_with_stride_equals_plain_on_contiguous_input(binding, dev, stream):
     """With the strides of a contiguous tensor and offset 0 the operation is ReshapeAndCache."""
     rng = _rng(32)

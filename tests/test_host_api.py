@@ -33,6 +33,7 @@ CACHE_LOAD_CASES = _load("paged_cache_load")
 NORM_ROPE_CASES = _load("norm_rope_reshape")
 ROPE_CASES = _load("rope")
 ELEWISE_CASES = _load("elewise")
+OMNI_CASES = _load("reshape_and_cache_omni")
 
 
 def _pa_unimplemented(p):
@@ -79,6 +80,7 @@ def _make_param(binding, op, p):
            "BlockCopyOperation": binding.BlockCopyParam,
            "PagedCacheLoadOperation": binding.PagedCacheLoadParam,
            "ReshapeAndCacheWithStrideOperation": binding.ReshapeAndCacheWithStrideParam,
+           "ReshapeAndCacheOmniOperation": binding.ReshapeAndCacheOmniParam,
            "NormRopeReshapeOperation": binding.NormRopeReshapeParam,
            "RopeOperation": binding.RopeParam,
            "ElewiseOperation": binding.ElewiseParam,
@@ -256,6 +258,60 @@ def test_reshape_and_cache_table(binding, ctx, case):
     _check(binding, case, ctx, _rac_unimplemented(case["param"]) and not case["expected"].startswith("C:"))
 
 
+@pytest.mark.parametrize("case", OMNI_CASES, ids=lambda c: "%d-%s" % (c["csv_line"], c["name"]))
+def test_reshape_and_cache_omni_table(binding, ctx, case):
+    _check(binding, case, ctx, False)
+
+
+def test_reshape_and_cache_omni_checks(binding, ctx):
+    """What the reference's table (all refusals) leaves open: the name and tensor counts
+    (reshape_and_cache_omni_operation.cpp:45,53-64), a pack that passes (shapes of the golden,
+    tests/apitest/opstest/python/operations/reshape_and_cache_omni/test_reshape_and_cache_omni.py:134-150),
+    the outputs taking the caches' descs (:77-83), each dim rule of :101-152 and the Setup rule of :164-169."""
+    E = binding.ERROR_CODE
+    P = binding.ReshapeAndCacheOmniParam
+    assert ctypes.sizeof(P) == 8   # reference include/atb/infer_op_params.h:2889-2894
+    op = binding.Operation("ReshapeAndCacheOmniOperation", P())
+    assert op.status == 0 and op.get_name() == "ReshapeAndCacheOmniOperation"
+    assert (op.input_num(), op.output_num()) == (8, 2)
+    mk = binding.make_tensor
+
+    def ins(dtype="float16", tokens=600, heads=4, d=128, batch=2, blocks=64, block=128, **over):
+        shapes = {"key": [tokens, heads, d], "value": [tokens, heads, d], "kc": [blocks, block, 1, d],
+                  "vc": [blocks, block, 1, d], "slots": [batch * heads], "wins": [batch * heads], "seq": [batch],
+                  "offs": [batch * heads]}
+        shapes.update(over)
+        types = [dtype] * 4 + ["int32"] * 4
+        return [mk(t, shapes[n], FAKE_DEVICE) for t, n in zip(types, ("key", "value", "kc", "vc", "slots", "wins",
+                                                                     "seq", "offs"))]
+
+    def outs(dtype="float16", kc=(64, 128, 1, 128), vc=(64, 128, 1, 128)):
+        return [mk(dtype, list(kc), FAKE_DEVICE), mk(dtype, list(vc), FAKE_DEVICE)]
+
+    for dtype in ("float16", "bf16"):
+        st, descs = op.infer_shape(ins(dtype))
+        assert st == 0 and [[d.dims[i] for i in range(d.dimNum)] for d in descs] == [[64, 128, 1, 128]] * 2
+        assert op.setup(ins(dtype), outs(dtype), ctx) == (0, 0)
+    assert op.infer_shape(ins("int8"))[0] == E["ERROR_INVALID_TENSOR_INI_MATCH"]
+    assert op.infer_shape(ins(key=[600, 512]))[0] == E["ERROR_INVALID_TENSOR_DIM_NUM"]
+    assert op.infer_shape(ins(seq=[2, 1]))[0] == E["ERROR_INVALID_TENSOR_DIM_NUM"]
+    bad = [dict(d=48, kc=[64, 128, 1, 48], vc=[64, 128, 1, 48], key=[600, 4, 48], value=[600, 4, 48]),  # 32 | headSize
+           dict(value=[599, 4, 128]), dict(value=[600, 2, 128]), dict(slots=[7]), dict(wins=[9]), dict(offs=[4]),
+           dict(value=[600, 4, 64]), dict(kc=[64, 128, 1, 64]), dict(vc=[64, 128, 1, 256]), dict(vc=[32, 128, 1, 128]),
+           dict(vc=[64, 64, 1, 128]), dict(kc=[64, 128, 2, 128]), dict(vc=[64, 128, 4, 128]),
+           dict(batch=125)]  # 125 * 4 = 500 pairs
+    for over in bad:
+        assert op.infer_shape(ins(**over))[0] == E["ERROR_INVALID_TENSOR_DIM"], over
+    assert op.infer_shape(ins(batch=124, tokens=1000))[0] == 0   # 496 pairs
+    assert op.setup(ins(value=[599, 4, 128]), outs(), ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.setup(ins(), outs(kc=(64, 128, 1, 64)), ctx)[0] == E["ERROR_INVALID_TENSOR_DIM"]
+    assert op.setup(ins(), outs("bf16"), ctx)[0] != 0
+    op.close()
+    p = P()
+    p.rsv[7] = 1
+    assert binding.Operation("ReshapeAndCacheOmniOperation", p).status == E["ERROR_INVALID_PARAM"]
+
+
 def test_table_coverage():
     """Most rows of the reference tables must be checked at face value, not as deviations."""
     pa_dev = [c for c in PA_CASES if (_pa_unimplemented(c["param"]) and not c["expected"].startswith("C:")) or
@@ -266,6 +322,7 @@ def test_table_coverage():
     # every MultiLatentAttention row is replayed at face value
     mla_dev = [c for c in MLA_CASES if _mla_unimplemented(c["param"]) and not c["expected"].startswith("C:")]
     assert len(MLA_CASES) == 147 and len(mla_dev) == 0
+    assert len(OMNI_CASES) == 15   # all at face value
 
 
 def test_param_sizes(binding):
@@ -1437,6 +1494,7 @@ def test_cpp_api_symbols_are_exported(pkg):
         "atb::CreateOperation<atb::infer::PagedAttentionParam>",
         "atb::CreateOperation<atb::infer::ReshapeAndCacheParam>",
         "atb::CreateOperation<atb::infer::ReshapeAndCacheWithStrideParam>",
+        "atb::CreateOperation<atb::infer::ReshapeAndCacheOmniParam>",
         "atb::CreateOperation<atb::infer::NormRopeReshapeParam>",
         "atb::CreateOperation<atb::infer::RopeParam>",
         "atb::CreateOperation<atb::infer::ElewiseParam>",
@@ -1558,6 +1616,11 @@ def test_pa_plan_refuses_inconsistent_layout_and_compression_fields(binding):
     assert k.atbmi_reshape_and_cache_compress(16, 16, 16, 16, 16, None, 16, None, 2, 4, 128, 100, 256, 0, None) == 1
     assert k.atbmi_reshape_and_cache_compress(16, 8, 16, 16, 16, 16, 16, None, 2, 4, 128, 100, 256, 0, None) == 1   # alignment
     assert k.atbmi_reshape_and_cache_compress(16, 16, 16, 16, 16, 16, 16, None, 0, 4, 128, 0, 256, 0, None) == 0    # nothing to do
+    assert k.atbmi_reshape_and_cache_omni(16, 16, 16, 16, 16, 16, 16, None, 2, 4, 128, 100, 256, 0, None) == 1      # offsetIndex
+    assert b"offsetIndex" in k.atbmi_last_error()
+    assert k.atbmi_reshape_and_cache_omni(16, 16, 16, 16, 16, 16, 16, 16, 2, 4, 48, 100, 256, 0, None) == 1
+    assert k.atbmi_reshape_and_cache_omni(16, 16, 16, 8, 16, 16, 16, 16, 2, 4, 128, 100, 256, 0, None) == 1
+    assert k.atbmi_reshape_and_cache_omni(16, 16, 16, 16, 16, 16, 16, 16, 0, 4, 128, 0, 256, 0, None) == 0
 
 
 def test_mask_free_is_created_and_refused_at_infer_shape(binding, ctx):

@@ -531,6 +531,72 @@ def test_compress_mean_window_invariants(oracle):
     assert np.array_equal(kc16, kc32.astype(np.float16))
 
 
+def test_omni_drop_window_by_flat_addresses_and_relations(oracle):
+    """ReshapeAndCacheOmni: (1) against element loops over flat addresses whose token list is built another way
+    (np.delete of the window from the sequence's token numbers); (2) a pair fills seqLen - win slots (seqLen
+    without a window) and nothing else; (3) with no window anywhere the result is the plain cache write of each
+    head's rows; (4) it is mean-window's result with the mean's slot taken out."""
+    rng = _rng(43)
+    batch, heads, d, block = 3, 2, 32, 16
+    seq, key, value = _compress_case(rng, batch, heads, d, block)
+    pairs = batch * heads
+    stride = 64
+    slots = (np.arange(pairs) * stride).astype(np.int32)
+    slots[4] = -1
+    blocks = pairs * stride // block
+    marker = np.float16(-555.0)
+    kc0 = np.full((blocks, block, 1, d), marker, dtype=np.float16)
+    wins = np.array([5, 1, 0, 7, 20, 3], dtype=np.int32)
+    offs = np.array([3, 0, 2, -1, 0, int(seq[2]) - 3], dtype=np.int32)  # last: the window ends the sequence
+    kc, vc = oracle.reshape_and_cache_omni(key, value, kc0, kc0, slots, wins, seq, offs)
+    assert np.array_equal(kc0, np.full_like(kc0, marker))  # the inputs are not written
+    starts = np.cumsum(seq) - seq
+    want_k, want_v = kc0.ravel().copy(), kc0.ravel().copy()
+    kf, vf = key.ravel(), value.ravel()
+    counts = []
+    for i in range(pairs):
+        b, h = divmod(i, heads)
+        toks = np.arange(starts[b], starts[b] + seq[b])
+        if offs[i] != -1:
+            toks = np.delete(toks, np.arange(offs[i], offs[i] + wins[i]))
+        counts.append(len(toks))
+        if slots[i] < 0:
+            continue
+        for n, tok in enumerate(toks.tolist()):
+            for c in range(d):
+                want_k[(slots[i] + n) * d + c] = kf[(tok * heads + h) * d + c]
+                want_v[(slots[i] + n) * d + c] = vf[(tok * heads + h) * d + c]
+    assert np.array_equal(kc.ravel(), want_k) and np.array_equal(vc.ravel(), want_v)
+    per_seq = np.repeat(seq, heads)
+    assert counts == np.where(offs == -1, per_seq, per_seq - wins).tolist()
+    # (3) no window: every head's rows through the plain write
+    none = np.full(pairs, -1, dtype=np.int32)
+    kc_all, vc_all = oracle.reshape_and_cache_omni(key, value, kc0, kc0, slots, wins, seq, none)
+    for i in range(pairs):
+        if slots[i] < 0:
+            continue
+        b, h = divmod(i, heads)
+        rows = slice(int(starts[b]), int(starts[b] + seq[b]))
+        plain_k, plain_v = oracle.reshape_and_cache(key[rows, h:h + 1], value[rows, h:h + 1], kc0, kc0,
+                                                    np.arange(slots[i], slots[i] + seq[b], dtype=np.int32))
+        mine = slice(int(slots[i]), int(slots[i]) + stride)
+        assert np.array_equal(kc_all.reshape(-1, d)[mine], plain_k.reshape(-1, d)[mine])
+        assert np.array_equal(vc_all.reshape(-1, d)[mine], plain_v.reshape(-1, d)[mine])
+    zero_win, _ = oracle.reshape_and_cache_omni(key, value, kc0, kc0, slots, np.zeros(pairs, np.int32), seq, offs)
+    assert np.array_equal(zero_win, kc_all)
+    # (4) mean-window keeps one slot for the window, this one none
+    mean_k, _ = oracle.reshape_and_cache_compress(key, value, kc0, kc0, slots, wins, seq, offs, out_dtype="float16")
+    for i in range(pairs):
+        if slots[i] < 0:
+            continue
+        mine = kc.reshape(-1, d)[slots[i]:slots[i] + stride]
+        other = mean_k.reshape(-1, d)[slots[i]:slots[i] + stride]
+        if offs[i] == -1 or wins[i] == 0:
+            assert np.array_equal(mine, other), i
+        else:
+            assert np.array_equal(mine[:stride - 1], np.delete(other, offs[i], axis=0)), i
+
+
 # ---------------------------------------------------------------- attention
 def test_attention_matches_independent_loops(oracle):
     rng = _rng(2)
