@@ -2226,6 +2226,26 @@ def test_repeated_execute_and_changing_lengths(binding, oracle, dev, stream):
     c.close()
 
 
+@pytest.mark.parametrize("charged", [3, 12, 40])
+@pytest.mark.parametrize("ctx", [[33, 700, 5, 64, 1500, 90, 2100], [4000, 40, 40, 40, 3000, 1]],
+                         ids=["mixed", "long_and_tiny"])
+def test_ranges_that_hold_only_the_steps_charged_for_a_row_start(binding, oracle, dev, stream, monkeypatch, ctx, charged):
+    """The planner charges the start of every row some steps of its own; with the charge raised
+    (ATBMI_PA_ROW_START_STEPS) above the length of a wave range, whole ranges fall into charged steps and leave
+    empty partial rows (zeros, log-sum-exp -inf), which the merge must weigh as nothing. The result stays the
+    oracle's and within rounding of the default plan's."""
+    rng = _rng(98)
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, len(ctx), 32, 8, 128, 128, 128, ctx, torch.float16)
+    scale = 1.0 / math.sqrt(128)
+    want = oracle_pa(oracle, q, kc, vc, tables, ctx, scale)
+    plain = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, kernel=0)
+    monkeypatch.setenv("ATBMI_PA_ROW_START_STEPS", str(charged))
+    for rep in range(3):  # (reused workspace: the empty rows must be written every time)
+        got = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, kernel=0, poison_workspace=rep == 1)
+        assert_close(got, want, 1e-3, "charged %d, repetition %d" % (charged, rep))
+        assert_close(got, plain.float().cpu().numpy(), 1e-3, "against the default plan")
+
+
 @pytest.mark.parametrize("heads,kv_heads", [(30, 2), (8, 2), (8, 4), (32, 8), (16, 1)])
 def test_rows_spanning_wave_ranges_merge_consistently(binding, oracle, dev, stream, heads, kv_heads):
     """Rows cut across several wave ranges leave partial rows in the workspace, written by CUs of
