@@ -1623,6 +1623,41 @@ def test_pa_plan_refuses_inconsistent_layout_and_compression_fields(binding):
     assert k.atbmi_reshape_and_cache_omni(16, 16, 16, 16, 16, 16, 16, 16, 0, 4, 128, 0, 256, 0, None) == 0
 
 
+def test_int8_query_mask_fetches_stay_inside_the_rows(binding):
+    """The int8-query kernel fetches 16-bit mask values as aligned 32-bit words, from the word that holds a
+    row's first element to the word that holds its last. Host arithmetic over every parity of base, strides and
+    row length: the words stay inside the row exactly when base % 4 == 0 and strides and length are even, and
+    that is the rule the call checks (by name) before anything touches the device."""
+    k = binding.kernels()
+    lens = np.array([6, 5], dtype=np.int32)
+
+    def call(mask, seq_stride, head_stride, mask_len):
+        c = binding.AtbmiPaInt8QCall(outDtype=binding.ATBMI_F16, numHeads=4, numKvHeads=2, headDim=128, blockSize=128,
+                                     numBlocks=4, maxBlocksPerSeq=2, batch=2, numQueryRows=2, hasMask=1,
+                                     maskLen=mask_len, qkScale=1.0, maskSeqStride=seq_stride,
+                                     maskHeadStride=head_stride, hostContextLens=lens.ctypes.data, mask=mask)
+        size = ctypes.c_uint64(0)
+        return k.atbmi_pa_int8q_workspace_size(ctypes.byref(c), ctypes.byref(size))
+
+    for base in (0x10000, 0x10002):
+        for seq_stride in (0, 6, 7, 8):
+            for head_stride in (0, 6, 7):
+                for mask_len in (6, 7, 8):
+                    inside = True
+                    for b in range(2):
+                        for h in range(4):
+                            row = base + 2 * (b * seq_stride + h * head_stride)   # byte address of the row
+                            first = row // 4 * 4
+                            last = (row + 2 * (mask_len - 1)) // 4 * 4
+                            inside &= first >= row and last + 4 <= row + 2 * mask_len
+                    rule = base % 4 == 0 and seq_stride % 2 == 0 and head_stride % 2 == 0 and mask_len % 2 == 0
+                    assert inside == rule, (base, seq_stride, head_stride, mask_len)
+                    rc = call(base, seq_stride, head_stride, mask_len)
+                    assert (rc == 0) == rule, (base, seq_stride, head_stride, mask_len)
+                    if rc != 0:
+                        assert b"4-byte" in k.atbmi_last_error()
+
+
 def test_mask_free_is_created_and_refused_at_infer_shape(binding, ctx):
     """MASK_TYPE_MASK_FREE off Atlas 300I Duo (reference paged_attention_operation.cpp:769-791,805-840): the
     operation is created, InferShape and Setup return ERROR_INVALID_TENSOR_DIM; NORM_COMPRESS is refused at creation."""
