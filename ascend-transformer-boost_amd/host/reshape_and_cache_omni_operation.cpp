@@ -47,7 +47,8 @@ bool SameDesc(const TensorDesc &a, const TensorDesc &b)
 
 class ReshapeAndCacheOmniOperation : public OperationBase {
 public:
-    ReshapeAndCacheOmniOperation() : OperationBase("ReshapeAndCacheOmniOperation")
+    explicit ReshapeAndCacheOmniOperation(const Param &param)
+        : OperationBase("ReshapeAndCacheOmniOperation"), param_(param)
     {
         static const OpIr table = MakeIr();
         ir_ = &table;
@@ -55,6 +56,8 @@ public:
 
     uint32_t GetInputNum() const override { return 8; }
     uint32_t GetOutputNum() const override { return 2; }
+    const Param &GetParam() const { return param_; }
+    void SetParam(const Param &param) { param_ = param; }
 
 protected:
     Status InferShapeImpl(const SVector<TensorDesc> &in, SVector<TensorDesc> &out) const override
@@ -172,6 +175,8 @@ private:
         }
         return NO_ERROR;
     }
+
+    Param param_;
 };
 } // namespace
 
@@ -185,10 +190,35 @@ template <> Status CreateOperation(const infer::ReshapeAndCacheOmniParam &opPara
         ATB_LOG(ERROR) << "ReshapeAndCacheOmniParam rsv has a non-zero byte";
         return ERROR_INVALID_PARAM;
     }
-    *operation = new (std::nothrow) ReshapeAndCacheOmniOperation();
+    *operation = new (std::nothrow) ReshapeAndCacheOmniOperation(opParam);
     if (*operation == nullptr) {
         return ERROR_OUT_OF_HOST_MEMORY;
     }
+    return NO_ERROR;
+}
+
+// Reference src/atb/operation/op_param_funcs.h:36-48.
+template <> Status CloneOperationParam(const Operation *operation, infer::ReshapeAndCacheOmniParam &opParam)
+{
+    const auto *op = dynamic_cast<const ReshapeAndCacheOmniOperation *>(operation);
+    if (op == nullptr) {
+        ATB_LOG(ERROR) << "CloneOperationParam: not a ReshapeAndCacheOmniOperation";
+        return ERROR_INVALID_PARAM;
+    }
+    opParam = op->GetParam();
+    return NO_ERROR;
+}
+
+// Reference src/atb/operation/op_param_funcs.h:50-70 (the param holds reserved bytes only, so every legal
+// param equals the current one: reshape_and_cache_omni_ops_runner.h:29-34).
+template <> Status UpdateOperationParam(Operation *operation, const infer::ReshapeAndCacheOmniParam &opParam)
+{
+    auto *op = dynamic_cast<ReshapeAndCacheOmniOperation *>(operation);
+    if (op == nullptr) {
+        ATB_LOG(ERROR) << "UpdateOperationParam: not a ReshapeAndCacheOmniOperation";
+        return ERROR_INVALID_PARAM;
+    }
+    op->SetParam(opParam);
     return NO_ERROR;
 }
 } // namespace atb

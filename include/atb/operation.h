@@ -39,5 +39,12 @@ public:
 template <typename OpParam> Status CreateOperation(const OpParam &opParam, Operation **operation);
 
 Status DestroyOperation(Operation *operation);
+
+// Copies the param an operation was created with / replaces it (no-op when equal). Specialised for
+// infer::ReshapeAndCacheOmniParam, the one operation of this library whose reference counterpart exports them
+// (reference include/atb/operation.h:130,140; src/atb/operation/op_param_funcs.h:36-70). An operation of another type
+// gives ERROR_INVALID_PARAM.
+template <typename OpParam> Status CloneOperationParam(const Operation *operation, OpParam &opParam);
+template <typename OpParam> Status UpdateOperationParam(Operation *operation, const OpParam &opParam);
 } // namespace atb
 #endif

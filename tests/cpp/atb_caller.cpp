@@ -90,6 +90,19 @@ int main()
     atb::Operation *none = nullptr;
     EXPECT(atb::CreateOperation(bad, &none) == atb::ERROR_INVALID_PARAM && none == nullptr);
 
+    // the operation whose param can be read back and replaced (reference include/atb/operation.h:130,140)
+    atb::infer::ReshapeAndCacheOmniParam omniParam;
+    atb::Operation *omni = nullptr;
+    EXPECT(atb::CreateOperation(omniParam, &omni) == atb::NO_ERROR && omni != nullptr);
+    EXPECT(omni->GetName() == "ReshapeAndCacheOmniOperation" && omni->GetInputNum() == 8 && omni->GetOutputNum() == 2);
+    atb::infer::ReshapeAndCacheOmniParam readBack;
+    readBack.rsv[3] = 9;
+    EXPECT(atb::CloneOperationParam(omni, readBack) == atb::NO_ERROR && readBack.rsv[3] == 0);
+    EXPECT(atb::UpdateOperationParam(omni, omniParam) == atb::NO_ERROR);
+    EXPECT(atb::CloneOperationParam(attention, readBack) == atb::ERROR_INVALID_PARAM);   // another operation's type
+    EXPECT(atb::UpdateOperationParam(static_cast<atb::Operation *>(nullptr), omniParam) == atb::ERROR_INVALID_PARAM);
+    EXPECT(atb::DestroyOperation(omni) == atb::NO_ERROR);
+
     EXPECT(atb::DestroyOperation(attention) == atb::NO_ERROR);
     EXPECT(atb::DestroyOperation(cacheWrite) == atb::NO_ERROR);
     EXPECT(atb::DestroyContext(context) == atb::NO_ERROR);

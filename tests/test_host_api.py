@@ -1495,6 +1495,8 @@ def test_cpp_api_symbols_are_exported(pkg):
         "atb::CreateOperation<atb::infer::ReshapeAndCacheParam>",
         "atb::CreateOperation<atb::infer::ReshapeAndCacheWithStrideParam>",
         "atb::CreateOperation<atb::infer::ReshapeAndCacheOmniParam>",
+        "atb::CloneOperationParam<atb::infer::ReshapeAndCacheOmniParam>",
+        "atb::UpdateOperationParam<atb::infer::ReshapeAndCacheOmniParam>",
         "atb::CreateOperation<atb::infer::NormRopeReshapeParam>",
         "atb::CreateOperation<atb::infer::RopeParam>",
         "atb::CreateOperation<atb::infer::ElewiseParam>",
