@@ -4,8 +4,8 @@ prints one JSON line per operation: BlockCopy (512 blocks of 256 KB copied in ea
 PagedCacheLoad (all 158 839 cached rows of the 64 sequences gathered) and NormRopeReshape (the
 producer of the combined MLA cache, at the 65 536 tokens of the reference's kernel test) and Rope
 (8 192 tokens of a Llama-3-8B-shaped layer) and the per-channel quantiser / dequantiser of
-ElewiseOperation (3 072 x 16 384) and the head-compressed forms of ReshapeAndCache (4 sequences of 4 000
-tokens, windows of 1 501), through
+ElewiseOperation (3 072 x 16 384) and the head-compressed forms of ReshapeAndCache and ReshapeAndCacheOmni
+(4 sequences of 4 000 tokens, windows of 1 501), through
 atb::Operation (Setup + Execute per call; NormRopeReshape, Rope and Elewise: Setup once). All are HBM-bound; `roofline.achieved` is their
 algorithmic bytes (every source byte read once, every destination byte written once) over the
 mean kernel time between HIP events on the launch stream.
@@ -219,15 +219,19 @@ def main():
     value = torch.randn_like(key)
     seq_d = torch.full((batch,), length, dtype=torch.int32, device=dev)
     wins_d = torch.full((pairs,), win, dtype=torch.int32, device=dev)
-    for name, compress, rows_out in (("keep-last windows", 1, win), ("mean windows", 2, length - win + 1)):
+    for name, compress, rows_out in (("keep-last windows", 1, win), ("mean windows", 2, length - win + 1),
+                                     ("dropped windows", 3, length - win)):
         per_pair = (rows_out + block - 1) // block
         cache_k = torch.zeros((pairs * per_pair, block, 1, d), dtype=torch.bfloat16, device=dev)
         cache_v = torch.zeros_like(cache_k)
         slots_d = (torch.arange(pairs, dtype=torch.int32, device=dev) * (per_pair * block)).contiguous()
         tensors = [key, value, cache_k, cache_v, slots_d, wins_d, seq_d]
-        if compress == 2:
+        if compress >= 2:
             tensors.append(torch.from_numpy(rng.integers(0, length - win + 1, size=pairs).astype(np.int32)).to(dev))
-        op = b.OperationRunner("ReshapeAndCacheOperation", b.ReshapeAndCacheParam(compressType=compress), ctx)
+        if compress == 3:  # the operation of its own that leaves the window out altogether
+            op = b.OperationRunner("ReshapeAndCacheOmniOperation", b.ReshapeAndCacheOmniParam(), ctx)
+        else:
+            op = b.OperationRunner("ReshapeAndCacheOperation", b.ReshapeAndCacheParam(compressType=compress), ctx)
         ins = [b.tensor_of(t) for t in tensors]
         outs = [b.tensor_of(cache_k), b.tensor_of(cache_v)]
         st, ws = op.op.setup(ins, outs, ctx)
@@ -236,9 +240,10 @@ def main():
         def execute_compress():
             assert op.op.execute(ins, outs, None, 0, ctx) == 0
         ms = timed(execute_compress, stream, args.steps, args.warmup)
-        rows_in = win if compress == 1 else length
+        rows_in = win if compress == 1 else (length if compress == 2 else rows_out)
         alg = 2 * pairs * (rows_in + rows_out) * d * 2
-        print(json.dumps({"operation": "ReshapeAndCacheOperation (head compression, %s)" % name,
+        print(json.dumps({"operation": ("ReshapeAndCacheOmniOperation (%s)" if compress == 3 else
+                                        "ReshapeAndCacheOperation (head compression, %s)") % name,
                           "workload": "%d sequences of %d tokens, %d heads of %d channels, windows of %d tokens, bf16 "
                           "(Setup once, Execute per call)" % (batch, length, heads, d, win), "ms_per_call": ms,
                           "roofline": {"bound": "hbm", "achieved": alg / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
