@@ -916,7 +916,9 @@ int DecodeImpl(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void *workspace, uint
     a.ropeRowStride = static_cast<int64_t>(s.numKvHeads) * s.ropeDim;
     a.lse = t->lse;
     a.nzShift = s.kvLayout == ATBMI_PA_KV_FRACTAL_NZ ? __builtin_ctz(static_cast<unsigned>(s.blockSize)) : 0;
-    a.partHalf = (plan->useMfma && PaMlaWide(s)) ? 1 : 0;
+    // 16-bit partial rows: the 128-head MLA kernel always; the MFMA kernel when the plan folds several query tokens
+    // of a sequence into one tile over 16-bit caches (a slot then holds that many times the rows)
+    a.partHalf = (plan->useMfma && (PaMlaWide(s) || (plan->stream.foldTokens > 1 && s.kvDtype != ATBMI_INT8))) ? 1 : 0;
 
     TimedLaunch timed;
     if (mayAllocate) {

@@ -287,7 +287,12 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                 const int64_t ph = (static_cast<int64_t>(slot) * (EXT ? p.foldTokens : 1) + tok) * a.H + head;
 #pragma unroll
                 for (int i = 0; i < DV / 16; ++i) {
-                    *reinterpret_cast<f32x4 *>(a.partO + ph * DV + i * 16 + kg * 4) = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                    if (EXT && a.partHalf) {
+                        *reinterpret_cast<u32x2 *>(reinterpret_cast<uint16_t *>(a.partO) + ph * DV + i * 16 + kg * 4) =
+                            u32x2{0u, 0u};
+                    } else {
+                        *reinterpret_cast<f32x4 *>(a.partO + ph * DV + i * 16 + kg * 4) = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                    }
                 }
                 if (kg == 0) {
                     a.partLse[ph] = -INFINITY;
@@ -854,7 +859,21 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                             o[r] = (o[r] + (a.vOff ? static_cast<float>(a.vOff[c + r]) : 0.0f)) * vs[r];
                         }
                     }
-                    *reinterpret_cast<f32x4 *>(a.partO + ph * DV + i * 16 + kg * 4) = o;
+                    if (EXT && a.partHalf) {
+                        // partial rows in the query's 16-bit type (plans that fold several query tokens into a tile:
+                        // their slots hold that many times the rows)
+                        u32x2 packed;
+                        if (qBf16) {
+                            packed[0] = Pack2<true>(o[0], o[1]);
+                            packed[1] = Pack2<true>(o[2], o[3]);
+                        } else {
+                            packed[0] = Pack2<false>(o[0], o[1]);
+                            packed[1] = Pack2<false>(o[2], o[3]);
+                        }
+                        *reinterpret_cast<u32x2 *>(reinterpret_cast<uint16_t *>(a.partO) + ph * DV + i * 16 + kg * 4) = packed;
+                    } else {
+                        *reinterpret_cast<f32x4 *>(a.partO + ph * DV + i * 16 + kg * 4) = o;
+                    }
                 }
                 if (kg == 0) {
                     a.partLse[ph] = m + log2f(l);
