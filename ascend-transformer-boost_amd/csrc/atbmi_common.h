@@ -107,9 +107,8 @@ struct PaArgs {
     int32_t nzShift;     // > 0: fractal-NZ caches of the split latent layout, log2 of the block size; channel c of
                          // the token at offset t of block b sits at ((b * (dn / 16) + c / 16) << nzShift) * 16 + t * 16 +
                          // c % 16 (dn channels per row of that cache)
-    int32_t partHalf;    // 1: partO holds 16-bit values of the query's type (the 128-head MLA kernel, whose partial rows
-                         // are a third of what a segment moves, and plans that fold several query tokens into one
-                         // tile over 16-bit caches: a normalised row loses little the final rounding would keep)
+    int32_t partHalf;    // 1: partO holds 16-bit values of the query's type (every plan of the MFMA kernels but those
+                         // over int8 caches with offsets): a normalised row loses little the final rounding would keep
 };
 
 // ---- Plan of the MFMA kernel ------------------------------------------------

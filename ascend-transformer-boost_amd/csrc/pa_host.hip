@@ -916,9 +916,13 @@ int DecodeImpl(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void *workspace, uint
     a.ropeRowStride = static_cast<int64_t>(s.numKvHeads) * s.ropeDim;
     a.lse = t->lse;
     a.nzShift = s.kvLayout == ATBMI_PA_KV_FRACTAL_NZ ? __builtin_ctz(static_cast<unsigned>(s.blockSize)) : 0;
-    // 16-bit partial rows: the 128-head MLA kernel always; the MFMA kernel when the plan folds several query tokens
-    // of a sequence into one tile over 16-bit caches (a slot then holds that many times the rows)
-    a.partHalf = (plan->useMfma && (PaMlaWide(s) || (plan->stream.foldTokens > 1 && s.kvDtype != ATBMI_INT8))) ? 1 : 0;
+    // Partial rows travel in the query's 16-bit type: they are normalised rows that end in a 16-bit output anyway, and
+    // writing them is what a wave does at every row boundary of its range (halving them took 2 - 6 us off the calls
+    // measured). Kept in fp32 only for int8 caches with offsets: the merge adds the offset to the merged row, and a sum
+    // that cancels would magnify the rounding of a 16-bit row.
+    const bool int8Kv = s.kvDtype == ATBMI_INT8;
+    const bool halfPays = !(int8Kv && s.hasOffset);
+    a.partHalf = (plan->useMfma && (PaMlaWide(s) || halfPays)) ? 1 : 0;
 
     TimedLaunch timed;
     if (mayAllocate) {

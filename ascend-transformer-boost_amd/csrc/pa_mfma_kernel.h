@@ -287,7 +287,7 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                 const int64_t ph = (static_cast<int64_t>(slot) * (EXT ? p.foldTokens : 1) + tok) * a.H + head;
 #pragma unroll
                 for (int i = 0; i < DV / 16; ++i) {
-                    if (EXT && a.partHalf) {
+                    if (a.partHalf) {
                         *reinterpret_cast<u32x2 *>(reinterpret_cast<uint16_t *>(a.partO) + ph * DV + i * 16 + kg * 4) =
                             u32x2{0u, 0u};
                     } else {
@@ -859,9 +859,8 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                             o[r] = (o[r] + (a.vOff ? static_cast<float>(a.vOff[c + r]) : 0.0f)) * vs[r];
                         }
                     }
-                    if (EXT && a.partHalf) {
-                        // partial rows in the query's 16-bit type (plans that fold several query tokens into a tile:
-                        // their slots hold that many times the rows)
+                    if (a.partHalf) {
+                        // partial rows in the query's 16-bit type (PaArgs::partHalf)
                         u32x2 packed;
                         if (qBf16) {
                             packed[0] = Pack2<true>(o[0], o[1]);

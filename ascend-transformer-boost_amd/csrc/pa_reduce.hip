@@ -222,12 +222,12 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaA
 // The same merge for plans whose rows span many ranges (a few long sequences in a batch): SLICES threads share each
 // piece of an output row, thread s taking the ranges s, s + SLICES, ... eight at a time; each ends with a maximum, a
 // sum of weights and a weighted sum of its own, and the first of them joins these through LDS. A row of 40 ranges is
-// then two memory round trips, not five. fp32 partial rows of up to 128 channels.
+// then two memory round trips, not five. Partial rows of up to 128 (fp32) or 256 (HALF: 16-bit) channels.
 constexpr int SLICES = 4;
-template <bool BF16>
+template <bool HALF, bool BF16>
 __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceSlicedKernel(const PaArgs a, const PaStreamPlan p)
 {
-    constexpr int CH = 4;
+    constexpr int CH = PartialPiece<HALF>::CH;
     constexpr int MAX_HELD = 8;
     __shared__ float joined[REDUCE_THREADS * (CH + 2)];
     const int vecs = a.Dv / CH;                  // pieces per row
@@ -257,13 +257,17 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceSlicedKernel(con
     auto rowOf = [&](int k) { return k == 0 ? ph0 : phEven + k * stride; };
     auto pow2 = [](float x) { return __builtin_amdgcn_exp2f(x); };
 
-    float acc[CH] = {0.0f, 0.0f, 0.0f, 0.0f};
+    float acc[CH];
+#pragma unroll
+    for (int e = 0; e < CH; ++e) {
+        acc[e] = 0.0f;
+    }
     float sum = 0.0f;
     float mx = -INFINITY;
 #pragma unroll 1
     for (int k0 = slice; k0 < count; k0 += MAX_HELD * SLICES) {
         float lseHeld[MAX_HELD];
-        PartialPiece<false> piece[MAX_HELD];
+        PartialPiece<HALF> piece[MAX_HELD];
 #pragma unroll
         for (int k = 0; k < MAX_HELD; ++k) {
             lseHeld[k] = -INFINITY;
@@ -294,7 +298,7 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceSlicedKernel(con
             sum += w;
 #pragma unroll
             for (int e = 0; e < CH; ++e) {
-                acc[e] += w * piece[k].Get(e, false);
+                acc[e] += w * piece[k].Get(e, BF16);
             }
         }
     }
@@ -344,9 +348,17 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceSlicedKernel(con
         }
         bits[e] = BF16 ? FloatToBf16(o) : FloatToHalfBits(o);
     }
+    uint32_t packed[CH / 2];
+#pragma unroll
+    for (int e = 0; e < CH / 2; ++e) {
+        packed[e] = static_cast<uint32_t>(bits[2 * e]) | (static_cast<uint32_t>(bits[2 * e + 1]) << 16);
+    }
     uint16_t *dst = reinterpret_cast<uint16_t *>(a.out) + outRow * a.Dv + c * CH;
-    *reinterpret_cast<uint2 *>(dst) = uint2{static_cast<uint32_t>(bits[0]) | (static_cast<uint32_t>(bits[1]) << 16),
-                                            static_cast<uint32_t>(bits[2]) | (static_cast<uint32_t>(bits[3]) << 16)};
+    if constexpr (HALF) {
+        *reinterpret_cast<uint4 *>(dst) = uint4{packed[0], packed[1], packed[2], packed[3]};
+    } else {
+        *reinterpret_cast<uint2 *>(dst) = uint2{packed[0], packed[1]};
+    }
     if (a.lse && c == 0) {
         Store16(a.lse, outRow, (top + log2f(sum)) * LN2, BF16);
     }
@@ -368,14 +380,22 @@ int LaunchPaStreamReduce(const AtbmiPaShape &shape, const PaArgs &args, const Pa
     if (grid > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "pa_reduce: grid of %lld workgroups is out of range", (long long)grid);
     }
-    if (plan.maxRangesPerRow > 8 && !args.partHalf && args.Dv % 4 == 0 && args.Dv / 4 * SLICES <= REDUCE_THREADS) {
-        const int slicedRowsPerWg = REDUCE_THREADS / (args.Dv / 4 * SLICES);
+    const int slicedCh = args.partHalf ? 8 : 4;
+    if (plan.maxRangesPerRow > 8 && args.Dv % slicedCh == 0 && args.Dv / slicedCh * SLICES <= REDUCE_THREADS) {
+        const int slicedRowsPerWg = REDUCE_THREADS / (args.Dv / slicedCh * SLICES);
         const int64_t slicedGrid = (rows + slicedRowsPerWg - 1) / slicedRowsPerWg;
         if (slicedGrid <= 0x7fffffffLL) {
-            if (args.qIsBf16) {
-                PaStreamReduceSlicedKernel<true><<<static_cast<unsigned>(slicedGrid), REDUCE_THREADS, 0, stream>>>(args, plan);
+            const unsigned slicedBlocks = static_cast<unsigned>(slicedGrid);
+            if (args.partHalf) {
+                if (args.qIsBf16) {
+                    PaStreamReduceSlicedKernel<true, true><<<slicedBlocks, REDUCE_THREADS, 0, stream>>>(args, plan);
+                } else {
+                    PaStreamReduceSlicedKernel<true, false><<<slicedBlocks, REDUCE_THREADS, 0, stream>>>(args, plan);
+                }
+            } else if (args.qIsBf16) {
+                PaStreamReduceSlicedKernel<false, true><<<slicedBlocks, REDUCE_THREADS, 0, stream>>>(args, plan);
             } else {
-                PaStreamReduceSlicedKernel<false><<<static_cast<unsigned>(slicedGrid), REDUCE_THREADS, 0, stream>>>(args, plan);
+                PaStreamReduceSlicedKernel<false, false><<<slicedBlocks, REDUCE_THREADS, 0, stream>>>(args, plan);
             }
             ATBMI_HIP_CHECK(hipGetLastError());
             return OK;
