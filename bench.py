@@ -54,11 +54,11 @@ WORKLOAD_SOURCES = {
 # sources at the time it was measured: a changed workload or changed kernels report null, not a stale figure.
 MEASURED_TRAFFIC = {
     # (workload, algorithmic bytes): (HBM bytes, summary under profiles/, source hash of the workload)
-    ("c2", 651658484): (664795161, "pa_mfma_bf16_d128_c2_trace_and_traffic.md", "7dc8d2c16b9c"),
-    ("c2_fp16", 651658484): (664806888, "pa_mfma_fp16_d128_c2_fp16_trace_and_traffic.md", "66dc868ff51e"),
-    ("c3", 1364204576): (1394601719, "pa_mfma_int8_d128_c3_trace_and_traffic.md", "771d22aad2c5"),
-    ("c4", 722875880): (733172752, "pa_mfma_fp16_d128_c4_trace_and_traffic.md", "66dc868ff51e"),
-    ("c5", 253384304): (349294098, "pa_mla_bf16_d576_c5_trace_and_traffic.md", "632da305c15f"),
+    ("c2", 651658484): (659481330, "pa_mfma_bf16_d128_c2_trace_and_traffic.md", "a296c1e2d7ec"),
+    ("c2_fp16", 651658484): (659459938, "pa_mfma_fp16_d128_c2_fp16_trace_and_traffic.md", "129c0af1d726"),
+    ("c3", 1364204576): (1381732860, "pa_mfma_int8_d128_c3_trace_and_traffic.md", "4852b0217877"),
+    ("c4", 722875880): (728782264, "pa_mfma_fp16_d128_c4_trace_and_traffic.md", "129c0af1d726"),
+    ("c5", 253384304): (349292145, "pa_mla_bf16_d576_c5_trace_and_traffic.md", "685780ffcbee"),
 }
 OTHER_WORKLOADS = ["c2_fp16", "c3", "c3_int8q", "c4", "c5"]  # timed in the same run as the headline workload
 MIN_KERNEL_LAUNCHES = 100  # launches behind every kernel figure, whatever --steps says
