@@ -91,7 +91,7 @@ struct Args {
     void *out;
     const Row *rows;
     const MergeRow *mergeRows;
-    float *partO;   // [partial rows][kvHeads x headTiles][16 heads][D], normalised
+    uint16_t *partO; // [partial rows][kvHeads x headTiles][16 heads][D], normalised, in the output's type
     float *partLse; // [partial rows][kvHeads x headTiles][16 heads]
     int64_t maskSeqStride;  // elements between the mask rows of two sequences (0: shared)
     int64_t maskHeadStride; // elements between the mask rows of two heads (0: shared)
@@ -400,10 +400,21 @@ __global__ __launch_bounds__(MaxWaves<D>() * WAVE) void PaInt8QKernel(const Args
                 const float inv = runSum > 0.0f ? 1.0f / runSum : 0.0f;
                 if (cur.partial >= 0) {
                     const int64_t slot = (static_cast<int64_t>(cur.partial) * a.G + g) * headTiles + ht;
-                    float *prow = a.partO + (slot * HT + n) * D + kg * 4;
+                    // (in the output's 16-bit type: a normalised row that ends in that type anyway; half the bytes a wave
+                    // writes between two pieces of its stream)
+                    uint16_t *prow = a.partO + (slot * HT + n) * D + kg * 4;
 #pragma unroll
                     for (int ct = 0; ct < CT; ++ct) {
-                        *reinterpret_cast<f32x4 *>(prow + ct * 16) = acc[ct] * inv;
+                        uint16_t bits[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float o = acc[ct][e] * inv;
+                            bits[e] = a.bf16 ? FloatToBf16(o) : FloatToHalfBits(o);
+                        }
+                        uint2 row2;
+                        row2.x = static_cast<uint32_t>(bits[0]) | (static_cast<uint32_t>(bits[1]) << 16);
+                        row2.y = static_cast<uint32_t>(bits[2]) | (static_cast<uint32_t>(bits[3]) << 16);
+                        *reinterpret_cast<uint2 *>(prow + ct * 16) = row2;
                     }
                     if (kg == 0) {
                         a.partLse[slot * HT + n] = runSum > 0.0f ? __logf(runSum) + runMax : -INFINITY;
@@ -493,7 +504,15 @@ __global__ __launch_bounds__(MERGE_THREADS) void PaInt8QMergeKernel(const Args a
     for (int p = 0; p < m.numPartials; ++p) {
         const float w = weightOf(a.partLse[first + p * perPartial]);
         total += w;
-        acc += *reinterpret_cast<const f32x4 *>(a.partO + (first + p * perPartial) * D + d) * w;
+        const uint2 raw = *reinterpret_cast<const uint2 *>(a.partO + (first + p * perPartial) * D + d);
+        const uint32_t words[2] = {raw.x, raw.y};
+        f32x4 row;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint16_t bits = static_cast<uint16_t>(words[e >> 1] >> ((e & 1) * 16));
+            row[e] = a.bf16 ? Bf16ToFloat(bits) : HalfBitsToFloat(bits);
+        }
+        acc += row * w;
     }
     const float inv = total > 0.0f ? 1.0f / total : 0.0f;
     uint16_t bits[4];
@@ -707,7 +726,7 @@ Layout PlanPieces(const AtbmiPaInt8QCall *c, const std::vector<Row> &seqs)
     lay.mergeOffset = align(lay.pieces.size() * sizeof(Row));
     lay.partOOffset = align(lay.mergeOffset + lay.merges.size() * sizeof(MergeRow));
     const uint64_t headRows = static_cast<uint64_t>(lay.numPartials) * sh.pairs * HT;
-    lay.partLseOffset = align(lay.partOOffset + headRows * c->headDim * sizeof(float));
+    lay.partLseOffset = align(lay.partOOffset + headRows * c->headDim * sizeof(uint16_t));
     lay.bytes = lay.partLseOffset + headRows * sizeof(float);
     return lay;
 }
@@ -825,7 +844,7 @@ extern "C" int atbmi_pa_int8q_decode(const AtbmiPaInt8QCall *call, void *workspa
     a.out = call->out;
     a.rows = reinterpret_cast<const int8q::Row *>(ws);
     a.mergeRows = reinterpret_cast<const int8q::MergeRow *>(ws + lay.mergeOffset);
-    a.partO = reinterpret_cast<float *>(ws + lay.partOOffset);
+    a.partO = reinterpret_cast<uint16_t *>(ws + lay.partOOffset);
     a.partLse = reinterpret_cast<float *>(ws + lay.partLseOffset);
     a.maskSeqStride = call->maskSeqStride;
     a.maskHeadStride = call->maskHeadStride;

@@ -1335,8 +1335,8 @@ def test_int8_query_quantisation_param_and_tensor_rules(binding, ctx):
         outs = [binding.make_tensor("bf16", [4, 32, 128], FAKE_DEVICE)]
         st, ws = op.setup(pack(offline), outs, ctx)
         # 13 tiles of 64 tokens in three shares: the sequence of 700 tokens is cut twice; piece table, merge table,
-        # three partial rows of 2 x 16 heads
-        assert st == 0 and ws == 256 + 256 + 3 * 2 * 16 * 128 * 4 + 3 * 2 * 16 * 4
+        # three partial rows of 2 x 16 heads in the output's 16-bit type, their log-sum-exps in fp32
+        assert st == 0 and ws == 256 + 256 + 3 * 2 * 16 * 128 * 2 + 3 * 2 * 16 * 4
         assert op.setup(pack(offline, heads=2), outs, ctx)[0] == e["ERROR_INVALID_PARAM"]        # descales per query head
         assert op.setup(pack(offline, mask="float16"), outs, ctx)[0] == e["ERROR_INVALID_TENSOR_INI_MATCH"]
         assert op.setup(pack(offline, q="float16"), outs, ctx)[0] == e["ERROR_INVALID_TENSOR_INI_MATCH"]
