@@ -66,7 +66,9 @@ struct PaArgs {
     void *out;
     const PaWorkItem *items;
     const PaSeqInfo *seqs;
-    float *partO;   // [numPartials][H][Dv] normalised partial outputs: fp32, or the query's 16-bit type when partHalf
+    float *partO;   // [numPartials][H][Dv] normalised partial outputs: fp32 for the scalar kernel's chunks; the stream
+                    // plans of the MFMA kernels keep 16-bit values of the query's type there (half the bytes a wave
+                    // writes at a row boundary, for rows that end in a 16-bit output anyway)
     float *partLse; // [numPartials][H] log2-domain log-sum-exp
     int32_t H, G, D, Dv;
     int32_t blockSize, maxBlocksPerSeq;
@@ -81,7 +83,8 @@ struct PaArgs {
     int64_t kRowStride; // key cache
     int64_t vRowStride; // value cache (the key cache's when V aliases K)
     int32_t vHeadStride; // value cache (D - ropeDim when V aliases K)
-    int32_t finishV;     // 1: partial outputs are still in int8 units; the final write applies vScale/vOff
+    int32_t finishV;     // 1: partial outputs are still in int8 units; the final write applies vScale (int8 caches
+                         // without offsets and without head compression; otherwise the attention kernel descales them)
     // Additive score bias (null: none), in the query's type: the score of the sequence in batch row b,
     // head h, token t gets mask[b * maskBatchStride + h * maskHeadStride + t] added after scaling.
     const void *mask;
@@ -107,8 +110,6 @@ struct PaArgs {
     int32_t nzShift;     // > 0: fractal-NZ caches of the split latent layout, log2 of the block size; channel c of
                          // the token at offset t of block b sits at ((b * (dn / 16) + c / 16) << nzShift) * 16 + t * 16 +
                          // c % 16 (dn channels per row of that cache)
-    int32_t partHalf;    // 1: partO holds 16-bit values of the query's type (every plan of the MFMA kernels but those
-                         // over int8 caches with offsets): a normalised row loses little the final rounding would keep
 };
 
 // ---- Plan of the MFMA kernel ------------------------------------------------

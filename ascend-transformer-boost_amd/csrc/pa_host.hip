@@ -127,15 +127,6 @@ int StaticScratch(void **ptr)
     return OK;
 }
 
-// Partial rows of the MFMA kernels travel in the query's 16-bit type: they are normalised rows that end in a 16-bit
-// output anyway, and writing them is what a wave does at every row boundary of its range (halving them took 2 - 6 us
-// off the calls measured). Kept in fp32 only for int8 caches with offsets: the merge adds the offset to the merged
-// row, and a sum that cancels would magnify the rounding of a 16-bit row.
-bool PartialRowsAreHalf(const AtbmiPaShape &s)
-{
-    return PaMlaWide(s) || !(s.kvDtype == ATBMI_INT8 && s.hasOffset);
-}
-
 std::mutex g_timingMutex;
 int g_timingEvery = 0;   // 0: off; n: bracket every n-th decode launch with events
 bool g_timingWhole = false; // no event between the attention kernel and its merge kernel: the call as one interval
@@ -513,7 +504,8 @@ int PlanStream(AtbmiPaPlan *plan)
     const uint64_t slots = plan->streamNeedsReduce ? 2ull * plan->stream.numWaveRanges * fold : 0;
     plan->numPartials = static_cast<int64_t>(slots);
     plan->offPartO = AlignUp(plan->blobBytes, WS_ALIGN);
-    const uint64_t partOBytes = slots * s.numHeads * s.headDimV * (PartialRowsAreHalf(s) ? sizeof(uint16_t) : sizeof(float));
+    // (partial rows of the MFMA kernels are 16-bit values of the query's type)
+    const uint64_t partOBytes = slots * s.numHeads * s.headDimV * sizeof(uint16_t);
     plan->offPartLse = AlignUp(plan->offPartO + partOBytes, WS_ALIGN);
     plan->wsBytes = AlignUp(plan->offPartLse + slots * s.numHeads * sizeof(float), WS_ALIGN);
     if (plan->blobBytes == 0 && slots == 0) {
@@ -905,7 +897,10 @@ int DecodeImpl(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void *workspace, uint
         a.vHeadStride = s.mlaCombined ? s.headDimK - s.ropeDim : s.headDimV;
     }
     // (with per-sequence descale slices the attention kernel descales its partial rows itself)
-    a.finishV = (plan->useMfma && s.kvDtype == ATBMI_INT8 && s.descaleHeads == 0) ? 1 : 0;
+    // With offsets (or under head compression, where the merge kernel cannot tell the descale slice) the attention
+    // kernel descales its partial rows itself: added to a row already rounded to 16 bits, an offset that cancels
+    // would magnify the rounding.
+    a.finishV = (plan->useMfma && s.kvDtype == ATBMI_INT8 && s.descaleHeads == 0 && !s.hasOffset) ? 1 : 0;
     a.descaleHeads = s.kvDtype == ATBMI_INT8 ? s.descaleHeads : 0;
     a.razor = s.hasRazorOffset ? t->razorOffset : nullptr;
     if (s.hasMask) {
@@ -925,7 +920,6 @@ int DecodeImpl(AtbmiPaPlan *plan, const AtbmiPaTensors *t, void *workspace, uint
     a.ropeRowStride = static_cast<int64_t>(s.numKvHeads) * s.ropeDim;
     a.lse = t->lse;
     a.nzShift = s.kvLayout == ATBMI_PA_KV_FRACTAL_NZ ? __builtin_ctz(static_cast<unsigned>(s.blockSize)) : 0;
-    a.partHalf = (plan->useMfma && PartialRowsAreHalf(s)) ? 1 : 0;
 
     TimedLaunch timed;
     if (mayAllocate) {

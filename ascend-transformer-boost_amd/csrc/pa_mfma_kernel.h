@@ -287,12 +287,8 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                 const int64_t ph = (static_cast<int64_t>(slot) * (EXT ? p.foldTokens : 1) + tok) * a.H + head;
 #pragma unroll
                 for (int i = 0; i < DV / 16; ++i) {
-                    if (a.partHalf) {
-                        *reinterpret_cast<u32x2 *>(reinterpret_cast<uint16_t *>(a.partO) + ph * DV + i * 16 + kg * 4) =
-                            u32x2{0u, 0u};
-                    } else {
-                        *reinterpret_cast<f32x4 *>(a.partO + ph * DV + i * 16 + kg * 4) = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-                    }
+                    *reinterpret_cast<u32x2 *>(reinterpret_cast<uint16_t *>(a.partO) + ph * DV + i * 16 + kg * 4) =
+                        u32x2{0u, 0u};
                 }
                 if (kg == 0) {
                     a.partLse[ph] = -INFINITY;
@@ -849,9 +845,10 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
 #pragma unroll
                 for (int i = 0; i < NO; ++i) {
                     f32x4 o = acc[i] * inv - bias;
-                    if (EXT && KV8 && a.descaleHeads > 0) {
-                        // the merge kernel cannot tell the slice: descale here (an affine map of rows whose
-                        // merge weights sum to one commutes with the merge)
+                    if (KV8 && !a.finishV) {
+                        // descale here (an affine map of rows whose merge weights sum to one commutes with the
+                        // merge): under head compression the merge kernel cannot tell the slice, and with offsets
+                        // the sum must be taken before the row is rounded to 16 bits
                         const int c = gs * DV + i * 16 + kg * 4;
                         const f32x4 vs = LoadScale4(a.vScale, c, a.scaleStride);
 #pragma unroll
@@ -859,20 +856,16 @@ __global__ __launch_bounds__(NW *WAVE) void PaMfmaKernel(const PaArgs a, const P
                             o[r] = (o[r] + (a.vOff ? static_cast<float>(a.vOff[c + r]) : 0.0f)) * vs[r];
                         }
                     }
-                    if (a.partHalf) {
-                        // partial rows in the query's 16-bit type (PaArgs::partHalf)
-                        u32x2 packed;
-                        if (qBf16) {
-                            packed[0] = Pack2<true>(o[0], o[1]);
-                            packed[1] = Pack2<true>(o[2], o[3]);
-                        } else {
-                            packed[0] = Pack2<false>(o[0], o[1]);
-                            packed[1] = Pack2<false>(o[2], o[3]);
-                        }
-                        *reinterpret_cast<u32x2 *>(reinterpret_cast<uint16_t *>(a.partO) + ph * DV + i * 16 + kg * 4) = packed;
+                    // partial rows travel in the query's 16-bit type
+                    u32x2 packed;
+                    if (qBf16) {
+                        packed[0] = Pack2<true>(o[0], o[1]);
+                        packed[1] = Pack2<true>(o[2], o[3]);
                     } else {
-                        *reinterpret_cast<f32x4 *>(a.partO + ph * DV + i * 16 + kg * 4) = o;
+                        packed[0] = Pack2<false>(o[0], o[1]);
+                        packed[1] = Pack2<false>(o[2], o[3]);
                     }
+                    *reinterpret_cast<u32x2 *>(reinterpret_cast<uint16_t *>(a.partO) + ph * DV + i * 16 + kg * 4) = packed;
                 }
                 if (kg == 0) {
                     a.partLse[ph] = m + log2f(l);

@@ -66,22 +66,10 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaReduceKernel(const PaArgs a)
 // head): it takes the maximum of the row's log-sum-exps, then adds up the
 // weighted partial rows with 16-byte loads. A workgroup of 128 threads covers as
 // many whole rows as fit (four for 128 channels, one for 512).
-// HALF: the partial rows are 16-bit values of the query's type and a thread owns eight channels.
-typedef float ReduceF4 __attribute__((ext_vector_type(4)));
+// The partial rows are 16-bit values of the query's type; a thread owns eight channels.
 
 // A thread's piece of one partial row, kept as loaded (16 bytes) until it is accumulated.
-template <bool HALF> struct PartialPiece;
-template <> struct PartialPiece<false> {
-    static constexpr int CH = 4;
-    ReduceF4 raw;
-    __device__ __forceinline__ void Clear() { raw = ReduceF4{0.0f, 0.0f, 0.0f, 0.0f}; }
-    __device__ __forceinline__ void Load(const float *partO, int64_t elem)
-    {
-        raw = *reinterpret_cast<const ReduceF4 *>(partO + elem);
-    }
-    __device__ __forceinline__ float Get(int e, bool) const { return raw[e]; }
-};
-template <> struct PartialPiece<true> {
+struct PartialPiece {
     static constexpr int CH = 8;
     uint32_t raw[4];
     __device__ __forceinline__ void Clear() { raw[0] = raw[1] = raw[2] = raw[3] = 0u; }
@@ -100,10 +88,10 @@ template <> struct PartialPiece<true> {
     }
 };
 
-template <bool HALF, bool BF16>
+template <bool BF16>
 __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaArgs a, const PaStreamPlan p)
 {
-    constexpr int CH = PartialPiece<HALF>::CH;                        // channels per thread
+    constexpr int CH = PartialPiece::CH;                              // channels per thread
     const int vecs = a.Dv / CH;                                       // threads per row
     const int rowsPerWg = vecs >= REDUCE_THREADS ? 1 : REDUCE_THREADS / vecs;
     const int rowsPerSlot = a.H * p.foldTokens;
@@ -155,7 +143,7 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaA
 #pragma unroll 1
         for (int k0 = 0; k0 < count; k0 += MAX_HELD) {
             float lseHeld[MAX_HELD];
-            PartialPiece<HALF> piece[MAX_HELD];
+            PartialPiece piece[MAX_HELD];
 #pragma unroll
             for (int k = 0; k < MAX_HELD; ++k) {
                 lseHeld[k] = -INFINITY;
@@ -208,11 +196,7 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaA
             packed[e] = static_cast<uint32_t>(bits[2 * e]) | (static_cast<uint32_t>(bits[2 * e + 1]) << 16);
         }
         uint16_t *dst = reinterpret_cast<uint16_t *>(a.out) + outRow * a.Dv + c * CH;
-        if constexpr (HALF) {
-            *reinterpret_cast<uint4 *>(dst) = uint4{packed[0], packed[1], packed[2], packed[3]};
-        } else {
-            *reinterpret_cast<uint2 *>(dst) = uint2{packed[0], packed[1]};
-        }
+        *reinterpret_cast<uint4 *>(dst) = uint4{packed[0], packed[1], packed[2], packed[3]};
         if (a.lse && c == 0) {
             Store16(a.lse, outRow, (mx + log2f(sum)) * LN2, bf16);
         }
@@ -222,12 +206,12 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceKernel(const PaA
 // The same merge for plans whose rows span many ranges (a few long sequences in a batch): SLICES threads share each
 // piece of an output row, thread s taking the ranges s, s + SLICES, ... eight at a time; each ends with a maximum, a
 // sum of weights and a weighted sum of its own, and the first of them joins these through LDS. A row of 40 ranges is
-// then two memory round trips, not five. Partial rows of up to 128 (fp32) or 256 (HALF: 16-bit) channels.
+// then two memory round trips, not five. Partial rows of up to 256 channels.
 constexpr int SLICES = 4;
-template <bool HALF, bool BF16>
+template <bool BF16>
 __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceSlicedKernel(const PaArgs a, const PaStreamPlan p)
 {
-    constexpr int CH = PartialPiece<HALF>::CH;
+    constexpr int CH = PartialPiece::CH;
     constexpr int MAX_HELD = 8;
     __shared__ float joined[REDUCE_THREADS * (CH + 2)];
     const int vecs = a.Dv / CH;                  // pieces per row
@@ -267,7 +251,7 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceSlicedKernel(con
 #pragma unroll 1
     for (int k0 = slice; k0 < count; k0 += MAX_HELD * SLICES) {
         float lseHeld[MAX_HELD];
-        PartialPiece<HALF> piece[MAX_HELD];
+        PartialPiece piece[MAX_HELD];
 #pragma unroll
         for (int k = 0; k < MAX_HELD; ++k) {
             lseHeld[k] = -INFINITY;
@@ -354,11 +338,7 @@ __global__ __launch_bounds__(REDUCE_THREADS) void PaStreamReduceSlicedKernel(con
         packed[e] = static_cast<uint32_t>(bits[2 * e]) | (static_cast<uint32_t>(bits[2 * e + 1]) << 16);
     }
     uint16_t *dst = reinterpret_cast<uint16_t *>(a.out) + outRow * a.Dv + c * CH;
-    if constexpr (HALF) {
-        *reinterpret_cast<uint4 *>(dst) = uint4{packed[0], packed[1], packed[2], packed[3]};
-    } else {
-        *reinterpret_cast<uint2 *>(dst) = uint2{packed[0], packed[1]};
-    }
+    *reinterpret_cast<uint4 *>(dst) = uint4{packed[0], packed[1], packed[2], packed[3]};
     if (a.lse && c == 0) {
         Store16(a.lse, outRow, (top + log2f(sum)) * LN2, BF16);
     }
@@ -370,7 +350,11 @@ int LaunchPaStreamReduce(const AtbmiPaShape &shape, const PaArgs &args, const Pa
                          hipStream_t stream)
 {
     (void)shape;
-    const int vecs = args.Dv / (args.partHalf ? 8 : 4);
+    constexpr int CH = PartialPiece::CH;
+    if (args.Dv % CH != 0) {
+        return Fail(ERR_INVALID_PARAM, "pa_reduce: %d channels a row, not a multiple of %d", args.Dv, CH);
+    }
+    const int vecs = args.Dv / CH;
     const int rowsPerWg = vecs >= REDUCE_THREADS ? 1 : REDUCE_THREADS / vecs;
     const int64_t rows = static_cast<int64_t>(plan.numSeqs) * plan.foldTokens * args.H;
     const int64_t grid = (rows + rowsPerWg - 1) / rowsPerWg;
@@ -380,38 +364,25 @@ int LaunchPaStreamReduce(const AtbmiPaShape &shape, const PaArgs &args, const Pa
     if (grid > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "pa_reduce: grid of %lld workgroups is out of range", (long long)grid);
     }
-    const int slicedCh = args.partHalf ? 8 : 4;
-    if (plan.maxRangesPerRow > 8 && args.Dv % slicedCh == 0 && args.Dv / slicedCh * SLICES <= REDUCE_THREADS) {
-        const int slicedRowsPerWg = REDUCE_THREADS / (args.Dv / slicedCh * SLICES);
+    if (plan.maxRangesPerRow > 8 && vecs * SLICES <= REDUCE_THREADS) {
+        const int slicedRowsPerWg = REDUCE_THREADS / (vecs * SLICES);
         const int64_t slicedGrid = (rows + slicedRowsPerWg - 1) / slicedRowsPerWg;
         if (slicedGrid <= 0x7fffffffLL) {
             const unsigned slicedBlocks = static_cast<unsigned>(slicedGrid);
-            if (args.partHalf) {
-                if (args.qIsBf16) {
-                    PaStreamReduceSlicedKernel<true, true><<<slicedBlocks, REDUCE_THREADS, 0, stream>>>(args, plan);
-                } else {
-                    PaStreamReduceSlicedKernel<true, false><<<slicedBlocks, REDUCE_THREADS, 0, stream>>>(args, plan);
-                }
-            } else if (args.qIsBf16) {
-                PaStreamReduceSlicedKernel<false, true><<<slicedBlocks, REDUCE_THREADS, 0, stream>>>(args, plan);
+            if (args.qIsBf16) {
+                PaStreamReduceSlicedKernel<true><<<slicedBlocks, REDUCE_THREADS, 0, stream>>>(args, plan);
             } else {
-                PaStreamReduceSlicedKernel<false, false><<<slicedBlocks, REDUCE_THREADS, 0, stream>>>(args, plan);
+                PaStreamReduceSlicedKernel<false><<<slicedBlocks, REDUCE_THREADS, 0, stream>>>(args, plan);
             }
             ATBMI_HIP_CHECK(hipGetLastError());
             return OK;
         }
     }
     const unsigned blocks = static_cast<unsigned>(grid);
-    if (args.partHalf) {
-        if (args.qIsBf16) {
-            PaStreamReduceKernel<true, true><<<blocks, REDUCE_THREADS, 0, stream>>>(args, plan);
-        } else {
-            PaStreamReduceKernel<true, false><<<blocks, REDUCE_THREADS, 0, stream>>>(args, plan);
-        }
-    } else if (args.qIsBf16) {
-        PaStreamReduceKernel<false, true><<<blocks, REDUCE_THREADS, 0, stream>>>(args, plan);
+    if (args.qIsBf16) {
+        PaStreamReduceKernel<true><<<blocks, REDUCE_THREADS, 0, stream>>>(args, plan);
     } else {
-        PaStreamReduceKernel<false, false><<<blocks, REDUCE_THREADS, 0, stream>>>(args, plan);
+        PaStreamReduceKernel<false><<<blocks, REDUCE_THREADS, 0, stream>>>(args, plan);
     }
     ATBMI_HIP_CHECK(hipGetLastError());
     return OK;
