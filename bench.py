@@ -54,11 +54,12 @@ WORKLOAD_SOURCES = {
 # sources at the time it was measured: a changed workload or changed kernels report null, not a stale figure.
 MEASURED_TRAFFIC = {
     # (workload, algorithmic bytes): (HBM bytes, summary under profiles/, source hash of the workload)
-    ("c2", 651658484): (659481330, "pa_mfma_bf16_d128_c2_trace_and_traffic.md", "a296c1e2d7ec"),
-    ("c2_fp16", 651658484): (659459938, "pa_mfma_fp16_d128_c2_fp16_trace_and_traffic.md", "129c0af1d726"),
-    ("c3", 1364204576): (1381732860, "pa_mfma_int8_d128_c3_trace_and_traffic.md", "4852b0217877"),
-    ("c4", 722875880): (728782264, "pa_mfma_fp16_d128_c4_trace_and_traffic.md", "129c0af1d726"),
-    ("c5", 253384304): (349292145, "pa_mla_bf16_d576_c5_trace_and_traffic.md", "685780ffcbee"),
+    ("c2", 651658484): (659472752, "pa_mfma_bf16_d128_c2_trace_and_traffic.md", "0ec4f74cf281"),
+    ("c2_fp16", 651658484): (659458917, "pa_mfma_fp16_d128_c2_fp16_trace_and_traffic.md", "146af6162386"),
+    ("c3", 1364204576): (1381773585, "pa_mfma_int8_d128_c3_trace_and_traffic.md", "fcfddfac51e2"),
+    ("c3_int8q", 1363148320): (1379216115, "pa_int8q_d128_c3_sizes_trace_counters_traffic.md", "92c707eb4b3b"),
+    ("c4", 722875880): (728761947, "pa_mfma_fp16_d128_c4_trace_and_traffic.md", "146af6162386"),
+    ("c5", 253384304): (349281878, "pa_mla_bf16_d576_c5_trace_and_traffic.md", "917a54b85783"),
 }
 OTHER_WORKLOADS = ["c2_fp16", "c3", "c3_int8q", "c4", "c5"]  # timed in the same run as the headline workload
 MIN_KERNEL_LAUNCHES = 100  # launches behind every kernel figure, whatever --steps says
