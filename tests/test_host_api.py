@@ -1720,3 +1720,11 @@ def test_plan_refuses_a_context_longer_than_the_mask_row(binding):
     assert k.atbmi_pa_plan_update(plan, arr.ctypes.data, 2) == 1
     assert b"mask" in k.atbmi_last_error()
     k.atbmi_pa_plan_destroy(plan)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark is a one-GPU program: asked for more it says so and exits, before it touches a device."""
+    import sys
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], stdout=subprocess.PIPE,
+                         stderr=subprocess.PIPE, text=True, timeout=120)
+    assert run.returncode != 0 and "one GPU" in run.stderr and run.stdout.strip() == ""
