@@ -603,7 +603,8 @@ typedef struct AtbmiPaInt8QCall {
 } AtbmiPaInt8QCall;
 
 /* Validates the call (pointers aside) and reports the device workspace it needs: the table of context pieces
- * (32 bytes each) and, for sequences cut into several pieces, their fp32 partial rows. The library's own cut
+ * (32 bytes each) and, for sequences cut into several pieces, their partial rows (in the output's 16-bit type) and
+ * fp32 log-sum-exps. The library's own cut
  * (pieceTiles = 0) follows the number of CUs of the current device, so size and launch belong on the same device;
  * a launch that finds the workspace too small fails with an error and runs nothing. */
 int atbmi_pa_int8q_workspace_size(const AtbmiPaInt8QCall *call, uint64_t *bytes);
