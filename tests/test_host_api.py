@@ -1270,6 +1270,9 @@ def test_torch_atb_surface(pkg):
                                                     calc_type=ta.MultiLatentAttentionParam.CalcType.CALC_TYPE_RING))
     assert (mla.input_num, mla.output_num) == (6, 2)
     mla.close()
+    omni = ta.Operation(ta.ReshapeAndCacheOmniParam())
+    assert (omni.name, omni.input_num, omni.output_num) == ("ReshapeAndCacheOmniOperation", 8, 2)
+    omni.close()
 
 
 def test_dequant_vector_lengths(binding, ctx):
