@@ -318,6 +318,10 @@ def atb():
         tp = ctypes.POINTER(AtbCTensor)
         lib.atb_c_create_context.argtypes = [vp, ctypes.POINTER(vp)]
         lib.atb_c_context_set_stream.argtypes = [vp, vp]
+        lib.atb_c_context_set_streams.argtypes = [vp, ctypes.POINTER(vp), u32]
+        lib.atb_c_op_set_stream_id.argtypes = [vp, u32]
+        lib.atb_c_op_get_stream_id.argtypes = [vp]
+        lib.atb_c_op_get_stream_id.restype = u32
         lib.atb_c_context_set_execute_type.argtypes = [vp, i32]
         lib.atb_c_destroy_context.argtypes = [vp]
         lib.atb_c_create_operation.argtypes = [ctypes.c_char_p, vp, u64, ctypes.POINTER(vp)]
@@ -426,6 +430,13 @@ class Context:
     def set_execute_type(self, t):
         return atb().atb_c_context_set_execute_type(self.ptr, int(t))
 
+    def set_streams(self, streams):
+        """Context::SetExecuteStreams: torch streams or raw handles; an operation picks one by its stream id."""
+        handles = [s.cuda_stream if hasattr(s, "cuda_stream") else s for s in streams]
+        arr = (ctypes.c_void_p * max(1, len(handles)))(*handles)
+        self.streams = list(streams)  # (kept alive)
+        return atb().atb_c_context_set_streams(self.ptr, arr, len(handles))
+
     def close(self):
         if self.ptr:
             atb().atb_c_destroy_context(self.ptr)
@@ -453,6 +464,12 @@ class Operation:
     @property
     def ok(self):
         return self.status == 0 and bool(self.ptr)
+
+    def set_stream_id(self, stream_id):
+        return atb().atb_c_op_set_stream_id(self.ptr, int(stream_id))
+
+    def get_stream_id(self):
+        return atb().atb_c_op_get_stream_id(self.ptr)
 
     def input_num(self):
         return atb().atb_c_op_input_num(self.ptr)

@@ -1,6 +1,8 @@
 // Flat C view of the atb::Operation API (see atb_capi.h).
 #include "atb_capi.h"
 #include <cstring>
+#include <new>
+#include <vector>
 #include <exception>
 #include <string>
 #include "atb/atb_infer.h"
@@ -66,6 +68,18 @@ int32_t atb_c_create_context(void *stream, void **context)
 int32_t atb_c_context_set_stream(void *context, void *stream)
 {
     return context ? static_cast<atb::Context *>(context)->SetExecuteStream(stream) : atb::ERROR_INVALID_PARAM;
+}
+
+int32_t atb_c_context_set_streams(void *context, void *const *streams, uint32_t count)
+{
+    if (!context || (!streams && count > 0)) {
+        return atb::ERROR_INVALID_PARAM;
+    }
+    try {
+        return static_cast<atb::Context *>(context)->SetExecuteStreams(std::vector<aclrtStream>(streams, streams + count));
+    } catch (const std::bad_alloc &) {
+        return atb::ERROR_OUT_OF_HOST_MEMORY;
+    }
 }
 
 int32_t atb_c_context_set_execute_type(void *context, int32_t type)
@@ -138,6 +152,16 @@ int32_t atb_c_create_operation(const char *opName, const void *param, uint64_t p
         return atb::CreateOperation(p, out);
     }
     return atb::ERROR_INVALID_PARAM;
+}
+
+int32_t atb_c_op_set_stream_id(void *operation, uint32_t streamId)
+{
+    return atb::SetExecuteStreamId(static_cast<atb::Operation *>(operation), streamId);
+}
+
+uint32_t atb_c_op_get_stream_id(void *operation)
+{
+    return atb::GetExecuteStreamId(static_cast<atb::Operation *>(operation));
 }
 
 int32_t atb_c_destroy_operation(void *operation)

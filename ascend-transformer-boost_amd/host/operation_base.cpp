@@ -174,6 +174,16 @@ Status OperationBase::Setup(const VariantPack &variantPack, uint64_t &workspaceS
     return NO_ERROR;
 }
 
+aclrtStream OperationBase::ExecuteStream() const
+{
+    const std::vector<aclrtStream> streams = context_->GetExecuteStreams();
+    if (streams.size() < static_cast<size_t>(streamId_) + 1) {
+        ATB_LOG(ERROR) << name_ << ": stream id " << streamId_ << ", the context holds " << streams.size() << " streams";
+        return nullptr;
+    }
+    return streams.at(streamId_);
+}
+
 Status OperationBase::PreLaunch(const VariantPack &variantPack, uint8_t *workspace, uint64_t workspaceSize,
                                 Context *context)
 {
@@ -181,7 +191,7 @@ Status OperationBase::PreLaunch(const VariantPack &variantPack, uint8_t *workspa
         ATB_LOG(ERROR) << name_ << " Execute: no successful Setup before Execute";
         return ERROR_INVALID_PARAM;
     }
-    if (context_->GetExecuteStream() == nullptr) {
+    if (ExecuteStream() == nullptr) {
         ATB_LOG(ERROR) << name_ << " Execute: execute stream is null";
         return ERROR_INVALID_PARAM;
     }
@@ -256,7 +266,7 @@ Status OperationBase::Execute(const VariantPack &variantPack, uint8_t *workspace
                 preLaunched_ = true;
                 return NO_ERROR;
             }
-            return LaunchImpl(variantPack, workspace, workspaceSize, context_->GetExecuteStream());
+            return LaunchImpl(variantPack, workspace, workspaceSize, ExecuteStream());
         }
         // EXECUTE_LAUNCH: second half of a split execute.
         if (!setupOk_ || !preLaunched_ || context != context_) {
@@ -264,7 +274,7 @@ Status OperationBase::Execute(const VariantPack &variantPack, uint8_t *workspace
             return ERROR_INVALID_PARAM;
         }
         preLaunched_ = false;
-        return LaunchImpl(launchPack_, launchWorkspace_, launchWorkspaceSize_, context_->GetExecuteStream());
+        return LaunchImpl(launchPack_, launchWorkspace_, launchWorkspaceSize_, ExecuteStream());
     } catch (const std::exception &e) {
         ATB_LOG(ERROR) << name_ << " Execute threw: " << e.what();
         return ERROR_RT_FAIL;
@@ -275,5 +285,26 @@ Status DestroyOperation(Operation *operation)
 {
     delete operation;
     return NO_ERROR;
+}
+
+// Reference src/atb/operation/operation.cpp:24-55.
+Status SetExecuteStreamId(Operation *operation, uint32_t streamId)
+{
+    OperationBase *base = dynamic_cast<OperationBase *>(operation);
+    if (base == nullptr) {
+        return ERROR_INVALID_PARAM;
+    }
+    base->SetExecuteStreamId(streamId);
+    return NO_ERROR;
+}
+
+uint32_t GetExecuteStreamId(Operation *operation)
+{
+    OperationBase *base = dynamic_cast<OperationBase *>(operation);
+    if (base == nullptr) {
+        ATB_LOG(ERROR) << "GetExecuteStreamId: not an operation of this library";
+        return 0;
+    }
+    return base->GetExecuteStreamId();
 }
 } // namespace atb

@@ -38,6 +38,9 @@ public:
     Status Setup(const VariantPack &variantPack, uint64_t &workspaceSize, Context *context) final;
     Status Execute(const VariantPack &variantPack, uint8_t *workspace, uint64_t workspaceSize,
                    Context *context) final;
+    // Which of the context's execute streams the launches go to (reference operation_base.cpp:1356-1379).
+    void SetExecuteStreamId(uint32_t streamId) { streamId_ = streamId; }
+    uint32_t GetExecuteStreamId() const { return streamId_; }
 
 protected:
     // Operator-specific hooks.
@@ -65,8 +68,11 @@ private:
     Status CheckShapes(const SVector<Tensor> &tensors, const char *what, bool inputs) const;
     bool IrMatch(const SVector<TensorDesc> &inDescs, const SVector<TensorDesc> *outDescs) const;
     Status PreLaunch(const VariantPack &variantPack, uint8_t *workspace, uint64_t workspaceSize, Context *context);
+    // Stream number streamId_ of the Setup context, null when the context holds fewer streams.
+    aclrtStream ExecuteStream() const;
 
     std::string name_;
+    uint32_t streamId_ = 0;
     bool setupOk_ = false;
     ContextImpl *context_ = nullptr;
     uint64_t workspaceSize_ = 0;

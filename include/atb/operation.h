@@ -40,6 +40,12 @@ template <typename OpParam> Status CreateOperation(const OpParam &opParam, Opera
 
 Status DestroyOperation(Operation *operation);
 
+// Chooses which of the context's execute streams (Context::SetExecuteStreams) an operation's launches go to; the
+// default is stream 0. Execute fails with ERROR_INVALID_PARAM when the context holds fewer streams
+// (reference include/atb/operation.h:150,159).
+Status SetExecuteStreamId(Operation *operation, uint32_t streamId);
+uint32_t GetExecuteStreamId(Operation *operation);
+
 // Copies the param an operation was created with / replaces it (no-op when equal). Specialised for
 // infer::ReshapeAndCacheOmniParam, the one operation of this library whose reference counterpart exports them
 // (reference include/atb/operation.h:130,140; src/atb/operation/op_param_funcs.h:36-70). An operation of another type

@@ -33,6 +33,8 @@ typedef struct AtbCTensor {
 int32_t atb_c_create_context(void *stream, void **context);
 /* Context::SetExecuteStream. */
 int32_t atb_c_context_set_stream(void *context, void *stream);
+/* Context::SetExecuteStreams: `count` streams, the first of which is the one atb_c_context_set_stream sets. */
+int32_t atb_c_context_set_streams(void *context, void *const *streams, uint32_t count);
 /* Context::SetExecuteType (0 normal, 1 pre-launch, 2 launch). */
 int32_t atb_c_context_set_execute_type(void *context, int32_t type);
 /* atb::DestroyContext. */
@@ -64,6 +66,10 @@ int32_t atb_c_op_setup(void *operation, const AtbCTensor *inTensors, uint32_t nu
 int32_t atb_c_op_execute(void *operation, const AtbCTensor *inTensors, uint32_t numIn,
                          const AtbCTensor *outTensors, uint32_t numOut, void *workspace, uint64_t workspaceSize,
                          void *context);
+
+/* atb::SetExecuteStreamId / atb::GetExecuteStreamId: which of the context's streams the operation launches on. */
+int32_t atb_c_op_set_stream_id(void *operation, uint32_t streamId);
+uint32_t atb_c_op_get_stream_id(void *operation);
 
 /* atb::Utils::GetTensorSize on the desc fields. */
 uint64_t atb_c_tensor_size(const AtbCTensor *tensor);

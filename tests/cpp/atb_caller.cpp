@@ -101,6 +101,9 @@ int main()
     EXPECT(atb::UpdateOperationParam(omni, omniParam) == atb::NO_ERROR);
     EXPECT(atb::CloneOperationParam(attention, readBack) == atb::ERROR_INVALID_PARAM);   // another operation's type
     EXPECT(atb::UpdateOperationParam(static_cast<atb::Operation *>(nullptr), omniParam) == atb::ERROR_INVALID_PARAM);
+    EXPECT(atb::GetExecuteStreamId(omni) == 0 && atb::SetExecuteStreamId(omni, 2) == atb::NO_ERROR &&
+           atb::GetExecuteStreamId(omni) == 2);
+    EXPECT(atb::SetExecuteStreamId(nullptr, 1) == atb::ERROR_INVALID_PARAM);
     EXPECT(atb::DestroyOperation(omni) == atb::NO_ERROR);
 
     EXPECT(atb::DestroyOperation(attention) == atb::NO_ERROR);

@@ -2203,6 +2203,35 @@ def test_q_scale_premultiply(binding, oracle, dev, stream, dtype):
         assert_close(got, oracle_pa(oracle, q, kc, vc, tables, ctx, 0.2, q_scale=0.7), TOL[dtype], "qScale")
 
 
+def test_operation_runs_on_the_stream_its_id_names(binding, oracle, dev, stream):
+    """A context with two execute streams: the operation with stream id 1 launches on the second one (the first is
+    held busy by a long copy queued before, and the result is complete once the second stream alone has been waited for)."""
+    rng = _rng(96)
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, 4, 32, 8, 128, 128, 128, [700, 1500, 128, 3000], torch.float16)
+    scale = 1.0 / math.sqrt(128)
+    second = torch.cuda.Stream(device=dev)
+    c = binding.Context(stream)
+    assert c.set_streams([stream, second]) == 0
+    pa = binding.OperationRunner("PagedAttentionOperation", binding.PagedAttentionParam(
+        headNum=32, kvHeadNum=8, qkScale=scale), c)
+    assert pa.op.set_stream_id(1) == 0 and pa.op.get_stream_id() == 1
+    lens = torch.from_numpy(ctx)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        big = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        for _ in range(60):  # some ten milliseconds of work on the first stream
+            big.fill_(1)
+    with torch.cuda.stream(second):
+        out, = pa.run([q, kc, vc, tables, lens.to(dev)], host_inputs={4: lens})
+    second.synchronize()
+    busy = not stream.query()
+    assert_close(out, oracle_pa(oracle, q, kc, vc, tables, ctx, scale), 1e-3, "stream 1")
+    stream.synchronize()
+    assert busy, "the first stream was meant to be still busy when the second one had finished"
+    pa.close()
+    c.close()
+
+
 def test_repeated_execute_and_changing_lengths(binding, oracle, dev, stream):
     """One operation, Setup + Execute repeatedly with growing context lengths, no sync in between."""
     rng = _rng(95)

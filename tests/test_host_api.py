@@ -432,6 +432,29 @@ def test_setup_workspace_grows_with_split_count(binding, ctx):
     op.close()
 
 
+def test_operation_stream_id(binding):
+    """SetExecuteStreamId / GetExecuteStreamId (reference include/atb/operation.h:150,159,
+    src/atb/operation/operation.cpp:24-55, operation_base.cpp:1356-1379): the default is stream 0, the id is
+    kept, and Execute refuses an id the context has no stream for."""
+    e = binding.ERROR_CODE
+    op = binding.Operation("PagedAttentionOperation",
+                           binding.PagedAttentionParam(headNum=8, kvHeadNum=8, qkScale=0.088))
+    assert op.get_stream_id() == 0
+    assert op.set_stream_id(1) == 0 and op.get_stream_id() == 1
+    assert binding.atb().atb_c_op_set_stream_id(None, 1) == e["ERROR_INVALID_PARAM"]
+    assert binding.atb().atb_c_op_get_stream_id(None) == 0
+    lens = np.array([469, 339, 432, 71], dtype=np.int32)
+    ins, outs = _c1_pack(binding, lens)
+    one = binding.Context(0x1)
+    st, ws = op.setup(ins, outs, one)
+    assert st == 0
+    # the context holds one stream only: nothing is launched
+    assert op.execute(ins, outs, FAKE_DEVICE, max(ws, 1), one) == e["ERROR_INVALID_PARAM"]
+    assert one.set_streams([]) == e["ERROR_INVALID_PARAM"]
+    one.close()
+    op.close()
+
+
 def test_setup_and_execute_error_paths(binding, ctx):
     e = binding.ERROR_CODE
     op = binding.Operation("PagedAttentionOperation",
