@@ -1310,6 +1310,30 @@ def test_paged_attention_int8_cache(binding, oracle, dev, stream, case):
         assert_close(got, want, INT8_TOL, "kernel=%d" % kernel)
 
 
+def test_int8_offsets_that_cancel_the_values_on_split_rows(binding, oracle, dev, stream):
+    """Values around +100 with an offset of -100: the dequantised values are small differences of large numbers.
+    Rows cut across wave ranges travel as 16-bit partial rows, which the attention kernel descales before it rounds
+    them, so the merged result keeps the accuracy of an unsplit row (a partial row kept in int8 units and rounded
+    to 16 bits first would be off by about 2e-3 here)."""
+    rng = _rng(47)
+    heads, kv_heads, d = 8, 2, 128
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, 2, heads, kv_heads, 128, d, d, [3000, 1500], torch.float16, kv_int8=True)
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(5)
+    vc = torch.randint(96, 105, tuple(vc.shape), generator=gen, dtype=torch.int8).to(dev)
+    ks = torch.full((kv_heads * d,), 0.05, dtype=torch.float32, device=dev)
+    vs = torch.full((kv_heads * d,), 0.05, dtype=torch.float32, device=dev)
+    ko = torch.zeros(kv_heads * d, dtype=torch.int32, device=dev)
+    vo = torch.full((kv_heads * d,), -100, dtype=torch.int32, device=dev)
+    scale = 1.0 / math.sqrt(d)
+    want = oracle_pa(oracle, q, kc, vc, tables, ctx, scale, ks, ko, vs, vo)
+    assert np.abs(want).max() < 0.25  # (the values lie within +-0.2)
+    got, info = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, ks, ko, vs, vo, kernel=0,
+                               return_plan_info=True)
+    assert info["chunks"] > 8  # the rows are cut
+    assert_close(got, want, 3e-4, "cancelling offsets")
+
+
 def test_int8_through_operation_api_with_offsets(binding, oracle, dev, stream):
     rng = _rng(41)
     heads, kv_heads, d = 32, 16, 128
