@@ -16,19 +16,35 @@
 //
 // A workgroup of eight waves owns one query row and 32 heads (16 when the call has no more) and walks the
 // row's context block by block. The int8 rows of a block go from the cache to LDS without passing through
-// registers (global_load_lds_dwordx4), one block ahead of the arithmetic, into one of two 64 KiB buffers; the
-// rotary rows, which only the wave that scores their tokens needs, are prefetched into that wave's registers.
+// registers (global_load_lds_dwordx4) into one of two 64 KiB buffers; the rotary rows, which only the wave that
+// scores their tokens needs, are prefetched into that wave's registers.
 //   scores  wave w for tokens 16 w .. 16 w + 15: S^T[token, head] = K . Q^T, eight int8 MFMAs over the 512
 //           latent channels (K rows from LDS as A, the query resident in registers as B) and two 16-bit MFMAs
-//           over the rotary channels, per tile of 16 heads;
-//   softmax 16 (32) lanes a head, 8 (4) tokens a lane; int8 weights P[head][token] go to LDS;
+//           over the rotary channels, per tile of 16 heads. The scores stay in the lanes the MFMA left them in
+//           (lane (head n, kg): tokens 16 w + 4 kg .. + 3), in units of log 2;
+//   softmax the waves exchange only the largest score each has for a head (8 floats a head through LDS); every
+//           lane then makes the weights of its own four tokens, keeps its own share of the running sum (the
+//           shares are added once, at the end of the row) and writes four int8 weights P[head][token] to LDS;
 //   values  wave w for channels 64 w .. 64 w + 63: O^T[channel, head] += V^T . P^T, V^T read from the token-major
 //           buffer by the transposing ds_read_b64_tr_b8 (lane (channel, kg) gets the bytes of 8 consecutive
-//           tokens), P^T as 16 consecutive bytes of a head's weights.
+//           tokens), P^T as 16 consecutive bytes of a head's weights. The accumulators are kept in units of the
+//           last tile's step: acc = acc x (keep x previous step / step) + int32 sum, two vector instructions a
+//           value, and pvDescale x step is applied with 1 / sum when the row is written.
+// Two barriers a block: [values of block i - 1, scores of block i] | [weights of block i, V^T of block i into
+// registers]. A wave asks for its eight pieces of block i + 1 (the channels only it reads for the values) during
+// the first span, as soon as it holds V^T of block i - 1 in registers, one piece at a time between its matrix
+// instructions, and waits for them before the second barrier: the path from a compute unit to its cache takes
+// one wave's 1 KiB request in about 16 cycles, and a wave that finds the path full stalls with all it has to do.
+// The kernel is bound by the vector instructions of a workgroup (about 230 a wave and block, four cycles each,
+// two waves a SIMD), not by HBM or the matrix pipe, so the code is written to spend few of them: no pass that
+// quiets NaNs around max, rint(fp16(x)) as one packed fp16 addition of 1024 for two weights, tokens past the
+// row's end masked only in its last block, the mask a template parameter.
 // Operand layout of v_mfma_i32_16x16x64_i8 (checked with a probe on the device): lane (n = lane % 16, kg =
 // lane / 16) supplies the 16 contraction values 16 kg .. 16 kg + 15 of row n (A) / column n (B) and receives
 // D[4 kg + e][n], e = 0 .. 3.
-// Three barriers a block, one pass per query row (no split over the context).
+// One pass per query row (no split over the context).
+#include <algorithm>
+#include <type_traits>
 #include <vector>
 #include "pa_internal.h"
 #include "upload_ring.h"
@@ -42,6 +58,7 @@ typedef int i32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int TILE = 128;            // tokens per tile = the block size of the cache
 constexpr int DN = 512;              // int8 channels (keys and values)
@@ -62,15 +79,13 @@ __host__ __device__ constexpr int PlaceOfToken(int t) // among the 32 tokens of 
 {
     return t ^ ((t & 16) >> 1);
 }
-constexpr int S_PITCH = (TILE + 4) * 4; // 16 heads' 16-byte writes touch every bank once
-constexpr int P_PITCH = TILE + 16;      // likewise for 16 heads' 16-byte reads
+constexpr int P_PITCH = TILE + 16;      // 16 heads' 16-byte reads touch every bank once
 template <int NT> struct Lds {
-    static constexpr int K = 0;                          // two blocks
-    static constexpr int S = 2 * K_BYTES;                // [16 NT] fp32 scores
-    static constexpr int P = S + NT * HT * S_PITCH;      // [16 NT] int8 weights
-    static constexpr int STAT = P + NT * HT * P_PITCH;   // [16 NT] {keep, value scale, 1 / sum, lse}
-    static constexpr int BYTES = STAT + NT * HT * 16;
-    static_assert(BYTES <= 160 * 1024 && S % 16 == 0 && P % 16 == 0 && STAT % 16 == 0, "LDS layout");
+    static constexpr int K = 0;                            // two blocks
+    static constexpr int P = 2 * K_BYTES;                  // [16 NT][tokens] int8 weights
+    static constexpr int MAXB = P + NT * HT * P_PITCH;     // [16 NT][waves] fp32: the waves' largest scores of a tile
+    static constexpr int BYTES = MAXB + NT * HT * NWAVES * 4;
+    static_assert(BYTES <= 160 * 1024 && P % 16 == 0 && MAXB % 16 == 0, "LDS layout");
 };
 static_assert(TILE == NWAVES * 16 && DN == NWAVES * 64 && PIECES_PER_WAVE == 8,
               "eight waves share a tile this way");
@@ -83,6 +98,8 @@ struct Row {
     int32_t pad;
 };
 
+constexpr int INLINE_ROWS = 128; // calls with up to this many query rows carry them in the kernel arguments
+
 struct Args {
     const int8_t *q8;
     const void *qRope;
@@ -94,12 +111,13 @@ struct Args {
     const void *mask;
     void *out;
     float *lse;
-    const Row *rows;
+    const Row *rows; // null: inlineRows
     int32_t H;
     int32_t numRows;
     int32_t maxBlocksPerSeq;
     int32_t maskLen;
     float qkScale;
+    Row inlineRows[INLINE_ROWS];
 };
 
 __device__ __forceinline__ float Load16AsFloat(uint32_t bits, bool bf16)
@@ -118,28 +136,28 @@ template <bool BF16> __device__ __forceinline__ f32x4 Mma16(u32x4 a, u32x4 b, f3
     }
 }
 
-// Eight transfers of 16 bytes per lane, cache to LDS without passing through registers: transfer i reads
-// base + laneOffset + 1024 i and writes LDS address ldsBase + 1024 i + 16 x lane (the instruction's offset field
-// moves both ends, so both bases are given 4096 bytes in). base and ldsBase are wave-uniform. The compiler does
-// not count these loads: the kernel waits for them with WaitForLoads.
-__device__ __forceinline__ void TransferPiecesToLds(uint32_t ldsBase, const void *base, uint32_t laneOffset)
+// One transfer of 16 bytes per lane, cache to LDS without passing through registers: lane l's 16 bytes at
+// base + laneOffset + OFFSET go to LDS address ldsBase + OFFSET + 16 l (the instruction's offset field moves both
+// ends). base and ldsBase are wave-uniform. With WAIT the LDS reads this wave has asked for are waited for first:
+// the transfer may land where they read. The compiler does not count these loads: the kernel waits for them with
+// WaitForLoads. A wave asks for one piece at a time, between pieces of arithmetic: the path from the compute unit
+// to its cache takes a wave's request for 1 KiB in about 16 cycles, and a wave whose request finds that path full
+// waits with everything else it has to do.
+template <int OFFSET, bool WAIT>
+__device__ __forceinline__ void TransferPieceToLds(uint32_t ldsBase, const unsigned char *base, uint32_t laneOffset)
 {
-    const uint64_t src = reinterpret_cast<uint64_t>(base) + 4096u;
-    const uint64_t srcUniform =
-        (static_cast<uint64_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(src >> 32))) << 32) |
-        static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(src)));
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
-                 "global_load_lds_dwordx4 %1, %2 offset:-4096\n\t"
-                 "global_load_lds_dwordx4 %1, %2 offset:-3072\n\t"
-                 "global_load_lds_dwordx4 %1, %2 offset:-2048\n\t"
-                 "global_load_lds_dwordx4 %1, %2 offset:-1024\n\t"
-                 "global_load_lds_dwordx4 %1, %2\n\t"
-                 "global_load_lds_dwordx4 %1, %2 offset:1024\n\t"
-                 "global_load_lds_dwordx4 %1, %2 offset:2048\n\t"
-                 "global_load_lds_dwordx4 %1, %2 offset:3072"
-                 :
-                 : "s"(ldsBase + 4096u), "v"(laneOffset), "s"(srcUniform)
-                 : "memory", "m0");
+    static_assert(OFFSET >= -4096 && OFFSET < 4096, "13-bit offset field");
+    if constexpr (WAIT) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_waitcnt lgkmcnt(0)\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
+                     :
+                     : "s"(ldsBase), "v"(laneOffset), "s"(base), "n"(OFFSET)
+                     : "memory", "m0");
+    } else {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
+                     :
+                     : "s"(ldsBase), "v"(laneOffset), "s"(base), "n"(OFFSET)
+                     : "memory", "m0");
+    }
 }
 
 __device__ __forceinline__ void WaitForLoads()
@@ -154,42 +172,46 @@ template <typename T> __device__ __forceinline__ void Pin(T &v)
     asm volatile("" : "+v"(v));
 }
 
-// All-reduce over the 16 lanes of a row (lanes 16 r .. 16 r + 15) by rotations inside the row.
-template <int ROR> __device__ __forceinline__ float RowRotate(float x)
+// max without the pass that quiets signalling NaNs (scores are finite or -inf)
+__device__ __forceinline__ float Max(float a, float b)
 {
-    const int v = __builtin_bit_cast(int, x);
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(v, v, 0x120 + ROR, 0xf, 0xf, true));
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
 }
-template <int LANES> __device__ __forceinline__ float GroupMax(float x)
+__device__ __forceinline__ float Max3(float a, float b, float c)
 {
-    x = fmaxf(x, RowRotate<8>(x));
-    x = fmaxf(x, RowRotate<4>(x));
-    x = fmaxf(x, RowRotate<2>(x));
-    x = fmaxf(x, RowRotate<1>(x));
-    if constexpr (LANES == 32) {
-        x = fmaxf(x, __shfl_xor(x, 16));
-    }
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// Largest / sum of the values lanes n, n + 16, n + 32 and n + 48 hold, in all four of them: the rows of 16 lanes
+// change places pairwise (rows 1 and 2, then the halves of the wave).
+__device__ __forceinline__ float RowsMax(float x)
+{
+    float y = x;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1\n\tv_max_f32 %0, %0, %1\n\tv_mov_b32 %1, %0\n\t"
+                 "s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1\n\tv_max_f32 %0, %0, %1"
+                 : "+v"(x), "+v"(y));
     return x;
 }
-template <int LANES> __device__ __forceinline__ float GroupSum(float x)
+__device__ __forceinline__ float RowsSum(float x)
 {
-    x += RowRotate<8>(x);
-    x += RowRotate<4>(x);
-    x += RowRotate<2>(x);
-    x += RowRotate<1>(x);
-    if constexpr (LANES == 32) {
-        x += __shfl_xor(x, 16);
-    }
+    float y = x;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1\n\tv_add_f32 %0, %0, %1\n\tv_mov_b32 %1, %0\n\t"
+                 "s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1\n\tv_add_f32 %0, %0, %1"
+                 : "+v"(x), "+v"(y));
     return x;
 }
 
-template <bool BF16, int NT>
+template <bool BF16, int NT, bool MASK>
 __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
 {
     using L = Lds<NT>;
-    constexpr int HW = NT * HT;          // heads of the workgroup
-    constexpr int CH = THREADS / HW;     // softmax: lanes a head
-    constexpr int TPL = TILE / CH;       // softmax: tokens a lane
+    constexpr int HW = NT * HT; // heads of the workgroup
+    constexpr float LOG2E = 1.44269504088896f;
+    constexpr float LN2 = 0.693147180559945f;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x;
     const int lane = tid & (WAVE - 1);
@@ -203,7 +225,7 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
     if (work >= a.numRows * headTiles) {
         return;
     }
-    const Row row = a.rows[work / headTiles];
+    const Row row = a.rows ? a.rows[work / headTiles] : a.inlineRows[work / headTiles];
     const int h0 = (work % headTiles) * HW;
     const int nh = min(HW, a.H - h0); // heads past the last one compute on zeros and store nothing
     const int32_t *table = a.tables + static_cast<int64_t>(row.tableRow) * a.maxBlocksPerSeq;
@@ -211,13 +233,18 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
     const uint32_t ldsBase =
         static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char *)smem));
 
-    // ---- requests for a block: this wave's eight pieces of the int8 rows, and its tokens' rotary rows
+    // ---- requests for a block: this wave's eight pieces of the int8 rows (channels 64 wave .. + 63 of all 128
+    // tokens: what this wave, and only this wave, reads for the values) and its tokens' rotary rows and mask values
     const uint32_t pieceLane = PlaceOfToken(lane & 31) * 32 + (lane >> 5) * 16; // place lane % 32, half lane / 32
-    auto requestBlock = [&](int64_t blk, int buf) {
-        const unsigned char *src =
-            reinterpret_cast<const unsigned char *>(a.kv8) + blk * K_BYTES + wave * (PIECES_PER_WAVE * PIECE);
-        const uint32_t dst = ldsBase + L::K + buf * K_BYTES + wave * (PIECES_PER_WAVE * PIECE);
-        TransferPiecesToLds(__builtin_amdgcn_readfirstlane(dst), src, pieceLane);
+    // (source and destination of a block's pieces are given 4096 bytes into this wave's eight, so that the offset
+    // field reaches all of them)
+    auto sourceOf = [&](int32_t blk) {
+        return reinterpret_cast<const unsigned char *>(a.kv8) +
+               static_cast<int64_t>(__builtin_amdgcn_readfirstlane(blk)) * K_BYTES + wave * (PIECES_PER_WAVE * PIECE) + 4096;
+    };
+    auto placeOf = [&](int buf) {
+        return static_cast<uint32_t>(
+            __builtin_amdgcn_readfirstlane(ldsBase + L::K + buf * K_BYTES + wave * (PIECES_PER_WAVE * PIECE) + 4096));
     };
     // lane (token n of the wave's 16, kg): rotary channels 32 m + 8 kg .. + 8, NZ [4][128][16]
     const int ropeLane = (kg >> 1) * (TILE * 32) + (wave * 16 + n) * 32 + (kg & 1) * 16;
@@ -228,17 +255,25 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
             r[m] = *reinterpret_cast<const u32x4 *>(src + m * (2 * TILE * 32));
         }
     };
+    const uint16_t *maskRow = reinterpret_cast<const uint16_t *>(a.mask) + static_cast<int64_t>(row.qRow) * a.maskLen;
+    auto loadMask = [&](int block, uint32_t(&bits)[4]) { // this lane's four tokens of the block
+        if constexpr (MASK) {
+            const int tok = block * TILE + wave * 16 + kg * 4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                bits[e] = maskRow[min(tok + e, row.ctxLen - 1)];
+            }
+        }
+    };
     u32x4 ropeNext[DR / 32] = {};
-    if (numBlocks > 0) {
-        const int64_t blk = table[0];
-        loadRope(blk, ropeNext);
-        requestBlock(blk, 0);
-    }
+    uint32_t maskNext[4] = {0u, 0u, 0u, 0u};
+    int32_t nextId; // id of the block after the one being scored, asked for a block ahead
+    int32_t firstId = table[0]; // (asked for before the query, used after it: the two answers travel together)
 
     // ---- Q^T as B operands: lane (n, kg) holds q8[head n][64 j + 16 kg .. +16) and qRope[head n][32 m + 8 kg .. +8)
     i32x4 q8[NT][DN / 64];
     u32x4 qr[NT][DR / 32];
-    float descale[NT];
+    float descale[NT], pvDescale[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         const bool live = nt * HT + n < nh;
@@ -260,20 +295,39 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
             }
         }
         descale[nt] = a.qkDescale[hn];
+        pvDescale[nt] = a.pvDescale[hn];
     }
-    const uint16_t *maskRow = a.mask ? reinterpret_cast<const uint16_t *>(a.mask) + static_cast<int64_t>(row.qRow) * a.maskLen
-                                     : nullptr;
-    // softmax: lane (head tid / CH, tokens 4 (tid % CH + CH k) .. + 4 for k < TPL / 4); a head's lanes all hold its
-    // running maximum and sum
-    const int smHead = tid / CH;
-    const int smTok = (tid % CH) * 4;
-    const float smPvDescale = a.pvDescale[h0 + min(smHead, nh - 1)];
-    float runMax = -INFINITY;
-    float runSum = 0.0f;
+    {
+        Pin(firstId);
+        const int64_t blk = firstId;
+        loadRope(blk, ropeNext);
+        loadMask(0, maskNext);
+        const unsigned char *src = sourceOf(firstId);
+        const uint32_t dst = placeOf(0);
+        TransferPieceToLds<-4096, false>(dst, src, pieceLane);
+        TransferPieceToLds<-3072, false>(dst, src, pieceLane);
+        TransferPieceToLds<-2048, false>(dst, src, pieceLane);
+        TransferPieceToLds<-1024, false>(dst, src, pieceLane);
+        TransferPieceToLds<0, false>(dst, src, pieceLane);
+        TransferPieceToLds<1024, false>(dst, src, pieceLane);
+        TransferPieceToLds<2048, false>(dst, src, pieceLane);
+        TransferPieceToLds<3072, false>(dst, src, pieceLane);
+        nextId = table[min(1, numBlocks - 1)];
+    }
+
+    const float scale2 = a.qkScale * LOG2E; // scores are kept in units of log 2: the weights are powers of two
+    // Softmax state of head 16 nt + n, the same in all lanes and waves that hold it except sumPart: the running
+    // maximum, this lane's share of the running sum (its four tokens of every tile), and the unit the accumulators
+    // are in: acc x pvDescale x unitStep are the weighted values.
+    float runMax[NT], sumPart[NT], unitStep[NT], ratio[NT];
     // values: channels 64 wave + 16 cs + 4 kg + e of head 16 nt + n
     f32x4 acc[NT][4];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
+        runMax[nt] = -INFINITY;
+        sumPart[nt] = 0.0f;
+        unitStep[nt] = 0.0f;
+        ratio[nt] = 0.0f;
 #pragma unroll
         for (int cs = 0; cs < 4; ++cs) {
             acc[nt][cs] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -285,21 +339,62 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
     // points at token r + n / 2, channels (n % 2) * 8 .. + 8
     const int valueLane = wave * 8192 + (kg >> 1) * PIECE + PlaceOfToken((kg & 1) * 16 + (n >> 1)) * 16 + (n & 1) * 8;
     const int valueHigh = (kg & 1) ? -128 : 128; // to the tokens eight further on
-
-    for (int i = 0; i < numBlocks; ++i) {
-        const int t0 = i * TILE;
-        const int tok = t0 + wave * 16 + kg * 4; // scores: this lane's four tokens
-        uint32_t maskBits[4] = {0u, 0u, 0u, 0u};
-        if (maskRow) {
+    float *maxRow[NT]; // the eight waves' entries of head 16 nt + n
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                maskBits[e] = maskRow[min(tok + e, row.ctxLen - 1)];
+    for (int nt = 0; nt < NT; ++nt) {
+        maxRow[nt] = reinterpret_cast<float *>(smem + L::MAXB) + (nt * HT + n) * NWAVES;
+    }
+
+    // V^T of this wave's 64 channels of the block in vbuf: [channel tile][token half], the two 8-byte halves of every
+    // A operand
+    auto readValues = [&](const unsigned char *vbuf, i32x2(&vlo)[4][TILE / 64], i32x2(&vhi)[4][TILE / 64]) {
+#pragma unroll
+        for (int cs = 0; cs < 4; ++cs) {
+#pragma unroll
+            for (int hh = 0; hh < TILE / 64; ++hh) {
+                const unsigned char *vp = vbuf + valueLane + (cs >> 1) * 4096 + (cs & 1) * 512 + hh * 2048;
+                vlo[cs][hh] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2 *)(vp));
+                vhi[cs][hh] =
+                    __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2 *)(vp + valueHigh));
             }
         }
-        const bool more = i + 1 < numBlocks;
-        const int64_t nextBlk = more ? table[i + 1] : 0;
-        WaitForLoads(); // this wave's pieces of block i are in LDS, its rotary rows and mask values in registers
+    };
+    // O^T[channel, head] += V^T . P^T for channel tile cs, with the weights pw
+    auto values = [&](int cs, const i32x2(&vlo)[4][TILE / 64], const i32x2(&vhi)[4][TILE / 64],
+                      const i32x4(&pw)[NT][TILE / 64]) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            i32x4 iacc = {0, 0, 0, 0};
+#pragma unroll
+            for (int hh = 0; hh < TILE / 64; ++hh) {
+                const i32x4 vt = {vlo[cs][hh][0], vlo[cs][hh][1], vhi[cs][hh][0], vhi[cs][hh][1]};
+                iacc = __builtin_amdgcn_mfma_i32_16x16x64_i8(vt, pw[nt][hh], iacc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                acc[nt][cs][e] = __builtin_fmaf(acc[nt][cs][e], ratio[nt], static_cast<float>(iacc[e]));
+            }
+        }
+    };
+    auto loadWeights = [&](i32x4(&pw)[NT][TILE / 64]) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+            for (int hh = 0; hh < TILE / 64; ++hh) {
+                pw[nt][hh] = *reinterpret_cast<const i32x4 *>(smem + L::P + (nt * HT + n) * P_PITCH + hh * 64 + kg * 16);
+            }
+        }
+    };
+
+    i32x2 vlo[4][TILE / 64], vhi[4][TILE / 64]; // V^T of the block whose weights are being made, read while they are made
+    WaitForLoads();
+    __syncthreads(); // block 0 is complete
+    auto iteration = [&](int i, auto firstTag, auto moreTag) __attribute__((always_inline)) {
+        constexpr bool FIRST = decltype(firstTag)::value;
+        constexpr bool MORE = decltype(moreTag)::value;
+        const unsigned char *kbuf = smem + L::K + (i & 1) * K_BYTES;
         u32x4 rope[DR / 32];
+        uint32_t maskBits[4];
 #pragma unroll
         for (int m = 0; m < DR / 32; ++m) {
             Pin(ropeNext[m]);
@@ -307,162 +402,184 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            Pin(maskBits[e]);
+            Pin(maskNext[e]);
+            maskBits[e] = maskNext[e];
         }
-        __syncthreads(); // block i is complete; everybody has left block i - 1, the scores and the weights
-        if (more) {
-            loadRope(nextBlk, ropeNext);
-            requestBlock(nextBlk, (i + 1) & 1);
-        }
-        const unsigned char *kbuf = smem + L::K + (i & 1) * K_BYTES;
-        // ---- scores of tokens 16 wave .. + 15
-        {
-            i32x4 kk[DN / 64];
-#pragma unroll
-            for (int j = 0; j < DN / 64; ++j) {
-                kk[j] = *reinterpret_cast<const i32x4 *>(kbuf + scoreLane + j * 8192);
+        Pin(nextId);
+        const int64_t nextBlk = nextId;
+        const unsigned char *src = sourceOf(nextId);
+        const uint32_t dst = placeOf((i + 1) & 1);
+        // ---- the values of block i - 1, whose V^T this wave holds in registers: its channels of block i + 1 may take
+        // their place in LDS (nobody else reads them before the next barrier but one)
+        if constexpr (!FIRST) {
+            i32x4 pw[NT][TILE / 64];
+            loadWeights(pw);
+            values(0, vlo, vhi, pw);
+            values(1, vlo, vhi, pw);
+            if constexpr (MORE) {
+                TransferPieceToLds<-4096, true>(dst, src, pieceLane); // (all reads of the block have arrived)
             }
+            values(2, vlo, vhi, pw);
+            if constexpr (MORE) {
+                TransferPieceToLds<-3072, false>(dst, src, pieceLane);
+            }
+            values(3, vlo, vhi, pw);
+            if constexpr (MORE) {
+                TransferPieceToLds<-2048, false>(dst, src, pieceLane);
+            }
+        } else if constexpr (MORE) {
+            TransferPieceToLds<-4096, false>(dst, src, pieceLane);
+            TransferPieceToLds<-3072, false>(dst, src, pieceLane);
+            TransferPieceToLds<-2048, false>(dst, src, pieceLane);
+        }
+        if constexpr (MORE) {
+            loadRope(nextBlk, ropeNext);
+            loadMask(i + 1, maskNext);
+            nextId = table[min(i + 2, numBlocks - 1)];
+        }
+        // ---- scores of tokens 16 wave .. + 15, in units of log 2
+        float x2[NT][4];
+        {
+            const int tok = i * TILE + wave * 16 + kg * 4; // this lane's four tokens
+            // every piece of the rows serves all head tiles as it arrives
+            i32x4 dots[NT];
+            f32x4 rdots[NT];
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                i32x4 dot = {0, 0, 0, 0};
-#pragma unroll
-                for (int j = 0; j < DN / 64; ++j) {
-                    dot = __builtin_amdgcn_mfma_i32_16x16x64_i8(kk[j], q8[nt][j], dot, 0, 0, 0);
-                }
-                f32x4 rdot = {0.0f, 0.0f, 0.0f, 0.0f};
+                dots[nt] = i32x4{0, 0, 0, 0};
+                rdots[nt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int m = 0; m < DR / 32; ++m) {
-                    rdot = Mma16<BF16>(rope[m], qr[nt][m], rdot);
-                }
-                f32x4 sc;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const bool live = tok + e < row.ctxLen;
-                    const float bias = maskRow ? Load16AsFloat(maskBits[e], BF16) : 0.0f;
-                    const float x = (static_cast<float>(dot[e]) * descale[nt] + rdot[e]) * a.qkScale + bias;
-                    sc[e] = live ? x : -INFINITY;
-                }
-                *reinterpret_cast<f32x4 *>(smem + L::S + (nt * HT + n) * S_PITCH + (wave * 16 + kg * 4) * 4) = sc;
-            }
-        }
-        __syncthreads();
-        // ---- weights of the tile
-        {
-            float w[TPL];
-            const float *srow = reinterpret_cast<const float *>(smem + L::S + smHead * S_PITCH) + smTok;
-            float tileMax = -INFINITY;
-#pragma unroll
-            for (int k = 0; k < TPL; k += 4) {
-                const f32x4 v = *reinterpret_cast<const f32x4 *>(srow + k * CH);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    w[k + e] = v[e];
-                    tileMax = fmaxf(tileMax, v[e]);
-                }
-            }
-            tileMax = GroupMax<CH>(tileMax);
-            const float newMax = fmaxf(runMax, tileMax);
-            const bool any = newMax > -INFINITY; // (a mask of -inf can hide everything seen so far)
-            float sum = 0.0f, wmax = 0.0f;
-#pragma unroll
-            for (int k = 0; k < TPL; ++k) {
-                w[k] = any ? __expf(w[k] - newMax) : 0.0f;
-                sum += w[k];
-                wmax = fmaxf(wmax, w[k]);
-            }
-            sum = GroupSum<CH>(sum);
-            wmax = GroupMax<CH>(wmax);
-            const float keep = (any && runMax > -INFINITY) ? __expf(runMax - newMax) : 0.0f;
-            runSum = runSum * keep + sum;
-            runMax = newMax;
-            // rint(fp16(w / step)), 0 .. 127. The quotient by a multiplication with 1 / step and one fused
-            // correction (the division's own sequence without its rescaling); a step too small for that takes
-            // the division.
-            const float step = wmax / 127.0f;
-            uint32_t packed[TPL / 4] = {};
-            if (step >= 1.0e-30f) {
-                const float y = __builtin_amdgcn_rcpf(step);
-#pragma unroll
-                for (int k = 0; k < TPL; ++k) {
-                    const float q0 = w[k] * y;
-                    const float q = __builtin_fmaf(__builtin_fmaf(-q0, step, w[k]), y, q0);
-                    const float p = rintf(static_cast<float>(static_cast<_Float16>(q)));
-                    packed[k / 4] = __builtin_amdgcn_cvt_pk_u8_f32(p, k % 4, packed[k / 4]);
-                }
-            } else if (wmax > 0.0f) {
-#pragma unroll
-                for (int k = 0; k < TPL; ++k) {
-                    const float p = rintf(static_cast<float>(static_cast<_Float16>(__fdiv_rn(w[k], step))));
-                    packed[k / 4] = __builtin_amdgcn_cvt_pk_u8_f32(p, k % 4, packed[k / 4]);
-                }
-            }
-            unsigned char *prow = smem + L::P + smHead * P_PITCH + smTok;
-#pragma unroll
-            for (int k = 0; k < TPL / 4; ++k) {
-                *reinterpret_cast<uint32_t *>(prow + k * CH * 4) = packed[k];
-            }
-            if (tid % CH == 0) {
-                float *stat = reinterpret_cast<float *>(smem + L::STAT) + smHead * 4;
-                stat[0] = keep;
-                stat[1] = smPvDescale * wmax / 127.0f;
-            }
-        }
-        __syncthreads();
-        // ---- values: O^T[channel, head] += V^T . P^T for channels 64 wave .. + 63
-        {
-            float keep[NT], vscale[NT];
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const float *stat = reinterpret_cast<const float *>(smem + L::STAT) + (nt * HT + n) * 4;
-                keep[nt] = stat[0];
-                vscale[nt] = stat[1];
-            }
-            i32x4 pw[NT][TILE / 64];
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-#pragma unroll
-                for (int hh = 0; hh < TILE / 64; ++hh) {
-                    pw[nt][hh] = *reinterpret_cast<const i32x4 *>(smem + L::P + (nt * HT + n) * P_PITCH + hh * 64 + kg * 16);
+                    rdots[nt] = Mma16<BF16>(rope[m], qr[nt][m], rdots[nt]);
                 }
             }
 #pragma unroll
-            for (int cs = 0; cs < 4; ++cs) {
-                i32x4 vt[TILE / 64];
-#pragma unroll
-                for (int hh = 0; hh < TILE / 64; ++hh) {
-                    const unsigned char *vp = kbuf + valueLane + (cs >> 1) * 4096 + (cs & 1) * 512 + hh * 2048;
-                    const i32x2 lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2 *)(vp));
-                    const i32x2 hi =
-                        __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2 *)(vp + valueHigh));
-                    vt[hh] = i32x4{lo[0], lo[1], hi[0], hi[1]};
-                }
+            for (int j = 0; j < DN / 64; ++j) {
+                const i32x4 kk = *reinterpret_cast<const i32x4 *>(kbuf + scoreLane + j * 8192);
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
-                    i32x4 iacc = {0, 0, 0, 0};
+                    dots[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(kk, q8[nt][j], dots[nt], 0, 0, 0);
+                }
+            }
+            if constexpr (MORE) {
+                TransferPieceToLds<-1024, false>(dst, src, pieceLane);
+            }
 #pragma unroll
-                    for (int hh = 0; hh < TILE / 64; ++hh) {
-                        iacc = __builtin_amdgcn_mfma_i32_16x16x64_i8(vt[hh], pw[nt][hh], iacc, 0, 0, 0);
+            for (int nt = 0; nt < NT; ++nt) {
+                const i32x4 dot = dots[nt];
+                const f32x4 rdot = rdots[nt];
+                if constexpr (MORE) {
+                    if (nt == 0) {
+                        TransferPieceToLds<0, false>(dst, src, pieceLane);
+                        if constexpr (NT == 1) {
+                            TransferPieceToLds<2048, false>(dst, src, pieceLane);
+                        }
+                    } else {
+                        TransferPieceToLds<2048, false>(dst, src, pieceLane);
                     }
+                }
+                float tileMax;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        acc[nt][cs][e] = acc[nt][cs][e] * keep[nt] + static_cast<float>(iacc[e]) * vscale[nt];
+                for (int e = 0; e < 4; ++e) {
+                    float x = __builtin_fmaf(static_cast<float>(dot[e]), descale[nt], rdot[e]) * scale2;
+                    if constexpr (MASK) {
+                        x = __builtin_fmaf(Load16AsFloat(maskBits[e], BF16), LOG2E, x);
+                    }
+                    // (only the last block of a row has tokens past its end)
+                    x2[nt][e] = (MORE || tok + e < row.ctxLen) ? x : -INFINITY;
+                }
+                tileMax = RowsMax(Max(Max(x2[nt][0], x2[nt][1]), Max(x2[nt][2], x2[nt][3])));
+                maxRow[nt][wave] = tileMax; // (the four lanes that hold a head all write its value)
+                if constexpr (MORE) {
+                    if (nt == 0) {
+                        TransferPieceToLds<1024, false>(dst, src, pieceLane);
+                        if constexpr (NT == 1) {
+                            TransferPieceToLds<3072, false>(dst, src, pieceLane);
+                        }
+                    } else {
+                        TransferPieceToLds<3072, false>(dst, src, pieceLane);
                     }
                 }
             }
         }
+        __syncthreads(); // every wave's largest scores of block i are there; everybody has left the weights of block i - 1
+        readValues(kbuf, vlo, vhi); // (for the values of this block, after the next barrier)
+        // ---- weights of the tile: this lane's four tokens of head 16 nt + n
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const f32x4 m0 = *reinterpret_cast<const f32x4 *>(maxRow[nt]);
+            const f32x4 m1 = *reinterpret_cast<const f32x4 *>(maxRow[nt] + 4);
+            const float tileMax = Max(Max3(m0[0], m0[1], m0[2]), Max3(Max3(m0[3], m1[0], m1[1]), m1[2], m1[3]));
+            // the reference point of the weights: the largest score so far (a mask of -inf can hide everything seen so
+            // far: the largest finite number below zero then stands in, and every weight is 0)
+            const float ref = Max3(runMax[nt], tileMax, -3.402823466e38f);
+            const float keep = __builtin_amdgcn_exp2f(runMax[nt] - ref);
+            const float wmax = __builtin_amdgcn_exp2f(tileMax - ref); // the largest weight of the tile
+            runMax[nt] = Max(runMax[nt], tileMax);
+            // int8 weights rint(fp16(w / step)), step = wmax / 127. A tile whose largest weight is below 2^-40 of
+            // the largest so far contributes nothing a float accumulator would notice and gets weights of 0.
+            const bool counts = wmax >= 0x1p-40f;
+            const float step = wmax * (1.0f / 127.0f);
+            const float perStep = counts ? __builtin_amdgcn_rcpf(step) : 0.0f;
+            float w[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                w[e] = __builtin_amdgcn_exp2f(x2[nt][e] - ref);
+            }
+            const float sum = (w[0] + w[1]) + (w[2] + w[3]);
+            // fp16(w / step) + 1024 in fp16 is 1024 + rint(fp16(w / step)): the integer is the low byte of the half
+            const f16x2 k1024 = {static_cast<_Float16>(1024.0f), static_cast<_Float16>(1024.0f)};
+            const f16x2 q01 = f16x2{static_cast<_Float16>(w[0] * perStep), static_cast<_Float16>(w[1] * perStep)} + k1024;
+            const f16x2 q23 = f16x2{static_cast<_Float16>(w[2] * perStep), static_cast<_Float16>(w[3] * perStep)} + k1024;
+            const uint32_t packed = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, q23), __builtin_bit_cast(uint32_t, q01),
+                                                          0x06040200u);
+            *reinterpret_cast<uint32_t *>(smem + L::P + (nt * HT + n) * P_PITCH + wave * 16 + kg * 4) = packed;
+            sumPart[nt] = __builtin_fmaf(sumPart[nt], keep, sum);
+            // the accumulators change their unit to this tile's step
+            ratio[nt] = counts ? keep * unitStep[nt] * perStep : keep;
+            unitStep[nt] = counts ? step : unitStep[nt];
+        }
+        if constexpr (MORE) {
+            WaitForLoads(); // this wave's pieces of block i + 1 are in LDS, its rotary rows and mask values in registers
+        }
+        __syncthreads(); // the weights of block i are there; block i + 1 is complete
+    };
+    using Yes = std::true_type;
+    using No = std::false_type;
+    if (numBlocks == 1) {
+        iteration(0, Yes{}, No{});
+    } else {
+        iteration(0, Yes{}, Yes{});
+        for (int i = 1; i < numBlocks - 1; ++i) {
+            iteration(i, No{}, Yes{});
+        }
+        iteration(numBlocks - 1, No{}, No{});
     }
-    // ---- the rows: acc / sum, and log(sum) + max
-    __syncthreads();
-    if (tid % CH == 0) {
-        float *stat = reinterpret_cast<float *>(smem + L::STAT) + smHead * 4;
-        stat[2] = runSum > 0.0f ? 1.0f / runSum : 0.0f;
-        stat[3] = runSum > 0.0f ? logf(runSum) + runMax : -INFINITY;
+    // ---- the values of the last block
+    {
+        i32x4 pw[NT][TILE / 64];
+        loadWeights(pw);
+        values(0, vlo, vhi, pw);
+        values(1, vlo, vhi, pw);
+        values(2, vlo, vhi, pw);
+        values(3, vlo, vhi, pw);
+    }
+    // ---- the rows: acc x unit / sum, and log(sum) + max
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const float s = RowsSum(sumPart[nt]);
+        if (kg == 0) {
+            maxRow[nt][wave] = s; // (the largest scores were last read before the loop's last barrier)
+        }
     }
     __syncthreads();
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
+        const f32x4 s0 = *reinterpret_cast<const f32x4 *>(maxRow[nt]);
+        const f32x4 s1 = *reinterpret_cast<const f32x4 *>(maxRow[nt] + 4);
+        const float total = ((s0[0] + s0[1]) + (s0[2] + s0[3])) + ((s1[0] + s1[1]) + (s1[2] + s1[3]));
         if (nt * HT + n < nh) {
-            const float inv = reinterpret_cast<const float *>(smem + L::STAT)[(nt * HT + n) * 4 + 2];
+            const float inv = total > 0.0f ? pvDescale[nt] * unitStep[nt] / total : 0.0f;
             uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) +
                              (static_cast<int64_t>(row.qRow) * a.H + h0 + nt * HT + n) * DN + wave * 64 + kg * 4;
 #pragma unroll
@@ -478,10 +595,11 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
                 w.y = static_cast<uint32_t>(bits[2]) | (static_cast<uint32_t>(bits[3]) << 16);
                 *reinterpret_cast<uint2 *>(orow + cs * 16) = w;
             }
+            if (a.lse && wave == 0 && kg == 0) {
+                a.lse[static_cast<int64_t>(row.qRow) * a.H + h0 + nt * HT + n] =
+                    total > 0.0f ? logf(total) + runMax[nt] * LN2 : -INFINITY;
+            }
         }
-    }
-    if (a.lse && tid < nh) {
-        a.lse[static_cast<int64_t>(row.qRow) * a.H + h0 + tid] = reinterpret_cast<const float *>(smem + L::STAT)[tid * 4 + 3];
     }
 }
 
@@ -593,9 +711,12 @@ extern "C" int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspa
         return Fail(ERR_INVALID_PARAM, "mla_int8: %lld workgroups", (long long)grid);
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    rc = UploadTable(rows.data(), bytes, workspaceDevice, s);
-    if (rc != OK) {
-        return rc;
+    const bool inlineRows = rows.size() <= static_cast<size_t>(mlaint8::INLINE_ROWS);
+    if (!inlineRows) {
+        rc = UploadTable(rows.data(), bytes, workspaceDevice, s);
+        if (rc != OK) {
+            return rc;
+        }
     }
     mlaint8::Args a{};
     a.q8 = static_cast<const int8_t *>(call->query);
@@ -608,15 +729,23 @@ extern "C" int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspa
     a.mask = call->hasMask ? call->mask : nullptr;
     a.out = call->out;
     a.lse = call->lse;
-    a.rows = static_cast<const mlaint8::Row *>(workspaceDevice);
+    a.rows = inlineRows ? nullptr : static_cast<const mlaint8::Row *>(workspaceDevice);
+    if (inlineRows) {
+        std::copy(rows.begin(), rows.end(), a.inlineRows);
+    }
     a.H = call->numHeads;
     a.numRows = static_cast<int32_t>(rows.size());
     a.maxBlocksPerSeq = call->maxBlocksPerSeq;
     a.maskLen = call->maskLen;
     a.qkScale = call->qkScale;
     const bool bf16 = call->outDtype == ATBMI_BF16;
-    auto kernel = nt == 2 ? (bf16 ? mlaint8::MlaInt8Kernel<true, 2> : mlaint8::MlaInt8Kernel<false, 2>)
-                          : (bf16 ? mlaint8::MlaInt8Kernel<true, 1> : mlaint8::MlaInt8Kernel<false, 1>);
+    using Kernel = void (*)(const mlaint8::Args);
+    static const Kernel kernels[2][2][2] = {
+        {{mlaint8::MlaInt8Kernel<false, 1, false>, mlaint8::MlaInt8Kernel<false, 1, true>},
+         {mlaint8::MlaInt8Kernel<false, 2, false>, mlaint8::MlaInt8Kernel<false, 2, true>}},
+        {{mlaint8::MlaInt8Kernel<true, 1, false>, mlaint8::MlaInt8Kernel<true, 1, true>},
+         {mlaint8::MlaInt8Kernel<true, 2, false>, mlaint8::MlaInt8Kernel<true, 2, true>}}};
+    const Kernel kernel = kernels[bf16 ? 1 : 0][nt - 1][call->hasMask ? 1 : 0];
     const int ldsBytes = nt == 2 ? mlaint8::Lds<2>::BYTES : mlaint8::Lds<1>::BYTES;
     rc = ConfigureKernelLds(reinterpret_cast<const void *>(kernel), ldsBytes);
     if (rc != OK) {

@@ -540,7 +540,8 @@ typedef struct AtbmiMlaInt8Call {
 
 /* Validates the call (pointers aside) and reports the device workspace it needs (16 bytes per query row). */
 int atbmi_mla_int8_workspace_size(const AtbmiMlaInt8Call *call, uint64_t *bytes);
-/* Uploads the row list into the workspace and launches the kernel on `stream`; does not wait. */
+/* Launches the kernel on `stream`; does not wait. The list of query rows travels in the kernel arguments when it
+ * has at most 128 entries and is uploaded into the workspace otherwise (the workspace is asked for either way). */
 int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspaceDevice, uint64_t workspaceBytes, void *stream);
 
 /*

@@ -138,6 +138,8 @@ INT8_MATRIX = [
     ([256, 256], 128, torch.float16, [2, 2], False, True),
     ([515, 129, 2048, 4], 64, torch.bfloat16, [2, 1, 3, 4], False, True),
     ([300, 1000, 0, 130], 16, torch.float16, [2, 2, 1, 4], False, [1, 0, 1, 1]),
+    # more query rows than travel in the kernel arguments: the row list goes through the workspace
+    ([130] * 70, 16, torch.float16, [2] * 70, False, True),
 ]
 
 
@@ -162,6 +164,31 @@ def test_mla_int8_nz_kernel(binding, oracle, dev, stream, case):
     rounded = torch.from_numpy(want).to(dtype).float().numpy()
     ok, rates = _double_golden(true_out, rounded, got.float().cpu().numpy(), dtype)
     assert ok, "double-golden rates %s" % (rates,)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_mla_int8_nz_tiles_far_apart(binding, oracle, dev, stream, dtype):
+    """Tiles whose scores lie far apart (a bias per cache block through the kernel layer's mask input): blocks that
+    weigh 2^-29 and 2^-87 of the heaviest, a heaviest block that comes late, blocks hidden altogether, a row whose
+    first blocks are all hidden. The online rescaling, the unit the accumulators are kept in and the tiles that are
+    too light to count all have to agree with the golden's plain arithmetic."""
+    ctx = [1100, 640, 384]
+    c = _case(777, dev, ctx, 32, dtype, None, True, None)
+    bias = np.zeros((3, max(ctx)), np.float32)
+    for b, per_block in enumerate([[0, -20, -60, 15, -np.inf, -3, 30, -45, -20],
+                                   [-np.inf, -np.inf, -60, 0, 12],
+                                   [-60, -60, -60]]):
+        for k, v in enumerate(per_block):
+            bias[b, k * 128:(k + 1) * 128] = v
+    bias[0, 700] = -np.inf      # single hidden tokens inside a visible block
+    bias[1, 639] = 25.0         # the last token alone outweighs everything before it
+    c["mask"] = torch.from_numpy(bias).to(dtype)
+    scale = 1.0 / math.sqrt(576.0)
+    want_lse = np.zeros((c["rows"], 32), np.float32)
+    want = _oracle(oracle, c, scale, 128, want_lse)
+    got, lse = int8_cabi(binding, oracle, stream, dev, c, scale, want_lse=True)
+    assert_close(got, want, TOL[dtype], "int8 NZ, tiles far apart")
+    assert_close(lse, want_lse, 1e-3, "int8 NZ lse, tiles far apart")
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
