@@ -172,7 +172,9 @@ template <typename T> __device__ __forceinline__ void Pin(T &v)
     asm volatile("" : "+v"(v));
 }
 
-// max without the pass that quiets signalling NaNs (scores are finite or -inf)
+// max without the pass that quiets signalling NaNs (scores are finite or -inf). The compiler does not look into the
+// statement when it spaces instructions for the hardware: an operand must not be the result of a transcendental
+// instruction (v_exp_f32, v_rcp_f32), which a reader has to follow at a distance.
 __device__ __forceinline__ float Max(float a, float b)
 {
     float r;
@@ -514,13 +516,13 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
             // far: the largest finite number below zero then stands in, and every weight is 0)
             const float ref = Max3(runMax[nt], tileMax, -3.402823466e38f);
             const float keep = __builtin_amdgcn_exp2f(runMax[nt] - ref);
-            const float wmax = __builtin_amdgcn_exp2f(tileMax - ref); // the largest weight of the tile
             runMax[nt] = Max(runMax[nt], tileMax);
-            // int8 weights rint(fp16(w / step)), step = wmax / 127. A tile whose largest weight is below 2^-40 of
-            // the largest so far contributes nothing a float accumulator would notice and gets weights of 0.
-            const bool counts = wmax >= 0x1p-40f;
+            // int8 weights rint(fp16(w / step)), step = wmax / 127, but no finer than 2^-40 / 127: a tile whose largest
+            // weight is below 2^-40 of the largest so far (or that is hidden altogether) contributes less than a float
+            // accumulator notices, and is quantised with that step instead of its own
+            const float wmax = __builtin_amdgcn_exp2f(Max(tileMax - ref, -40.0f)); // the largest weight of the tile
             const float step = wmax * (1.0f / 127.0f);
-            const float perStep = counts ? __builtin_amdgcn_rcpf(step) : 0.0f;
+            const float perStep = __builtin_amdgcn_rcpf(step);
             float w[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -536,8 +538,8 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
             *reinterpret_cast<uint32_t *>(smem + L::P + (nt * HT + n) * P_PITCH + wave * 16 + kg * 4) = packed;
             sumPart[nt] = __builtin_fmaf(sumPart[nt], keep, sum);
             // the accumulators change their unit to this tile's step
-            ratio[nt] = counts ? keep * unitStep[nt] * perStep : keep;
-            unitStep[nt] = counts ? step : unitStep[nt];
+            ratio[nt] = keep * unitStep[nt] * perStep;
+            unitStep[nt] = step;
         }
         if constexpr (MORE) {
             WaitForLoads(); // this wave's pieces of block i + 1 are in LDS, its rotary rows and mask values in registers
