@@ -17,10 +17,8 @@ bool PaMfmaSupports(const AtbmiPaShape &s)
     if (d != dv) {
         return false;
     }
-    if (s.kvDtype == ATBMI_INT8) {
-        return d == 64 || d == 128 || d == 256;
-    }
-    return d == 64 || d == 96 || d == 128 || d == 256;
+    // every multiple of 32 up to 256 (int8 rows: from 64)
+    return d % 32 == 0 && d >= (s.kvDtype == ATBMI_INT8 ? 64 : 32) && d <= 256;
 }
 
 bool PaMlaWide(const AtbmiPaShape &s)

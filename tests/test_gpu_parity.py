@@ -991,6 +991,40 @@ def test_paged_attention_matrix(binding, oracle, dev, stream, case):
         assert_close(got, want, TOL[dtype], "kernel=%d" % kernel)
 
 
+# Every head size that is a multiple of 32 has an MFMA build, for 16-bit caches and (from 64) for int8 caches (the
+# reference's tests hold 64, 96, 128 and 256): batch, heads, kv_heads, block, d, ctx, dtype, int8 cache
+HEAD_SIZES = [
+    (3, 8, 2, 16, 32, [100, 700, 33], torch.float16, False),
+    (2, 12, 4, 128, 160, [900, 129], torch.bfloat16, False),
+    (2, 8, 8, 64, 192, [600, 2100], torch.float16, False),
+    (2, 6, 2, 128, 224, [1500, 40], torch.bfloat16, False),
+    (2, 10, 2, 128, 96, [513, 1300], torch.bfloat16, True),
+    (2, 12, 4, 128, 160, [900, 129], torch.float16, True),
+    (2, 8, 8, 64, 192, [600, 2100], torch.bfloat16, True),
+    (2, 6, 2, 128, 224, [1500, 40], torch.float16, True),
+]
+
+
+@pytest.mark.parametrize("case", HEAD_SIZES, ids=lambda c: "d%d_%s%s" % (c[4], str(c[6]).split(".")[-1], "_int8" if c[7] else ""))
+def test_mfma_kernel_on_every_multiple_of_32(binding, oracle, dev, stream, case):
+    batch, heads, kv_heads, block, d, ctx, dtype, int8 = case
+    rng = _rng(900 + d + int(int8))
+    q, kc, vc, tables, ctx = _pa_inputs(rng, dev, batch, heads, kv_heads, block, d, d, ctx, dtype, kv_int8=int8)
+    scale = 1.0 / math.sqrt(d)
+    ks = ko = vs = vo = None
+    if int8:
+        ks = torch.from_numpy(rng.uniform(0.05, 0.5, size=kv_heads * d).astype(np.float32)).to(dev)
+        vs = torch.from_numpy(rng.uniform(0.05, 0.5, size=kv_heads * d).astype(np.float32)).to(dev)
+        ko = torch.from_numpy(rng.integers(-20, 20, size=kv_heads * d).astype(np.int32)).to(dev)
+        vo = torch.from_numpy(rng.integers(-20, 20, size=kv_heads * d).astype(np.int32)).to(dev)
+    want = oracle_pa(oracle, q, kc, vc, tables, ctx, scale, ks, ko, vs, vo)
+    # asked for by name: the plan refuses a shape the MFMA kernel does not cover
+    got = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, ks, ko, vs, vo, kernel=binding.ATBMI_PA_KERNEL_MFMA)
+    assert_close(got, want, INT8_TOL if int8 else TOL[dtype], "MFMA kernel, head size %d" % d)
+    got = pa_decode_cabi(binding, stream, q, kc, vc, tables, ctx, scale, ks, ko, vs, vo, kernel=binding.ATBMI_PA_KERNEL_SCALAR)
+    assert_close(got, want, INT8_TOL if int8 else TOL[dtype], "scalar kernel, head size %d" % d)
+
+
 # Fewer 32-token steps than the waves of a workgroup: batch, heads, kv_heads, d, ctx, dtype
 TINY_PLANS = [
     (1, 8, 1, 128, [96], torch.float16),
