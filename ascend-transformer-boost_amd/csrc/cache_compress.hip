@@ -193,24 +193,38 @@ __global__ __launch_bounds__(CC_THREADS) void CompressMeanWindowKernel(const Com
     for (int i = 0; i < MEAN_MAX_CHANNELS / CC_THREADS; ++i) {
         sum[i] = 0.0f;
     }
+    // The rows of the next run travel while this one is added up: a run's loads are asked for one run ahead and
+    // wait in registers (one workgroup has nothing else to hide their latency behind).
+    constexpr int HELD = MEAN_STAGE_BYTES / 16 / CC_THREADS; // 16-byte pieces per thread and run
+    auto countOf = [&](int64_t k0) {
+        return static_cast<int>(inRange - k0 < chunkTokens ? inRange - k0 : chunkTokens);
+    };
+#define ATBMI_REQUEST_RUN(k0_, count_)                                                                        \
+    _Pragma("unroll") for (int u = 0; u < HELD; ++u)                                                          \
+    { /* lanes past the run's end repeat its last piece */                                                    \
+        const int last = (count_) * pieces - 1;                                                               \
+        const int at = threadIdx.x + u * CC_THREADS < last ? threadIdx.x + u * CC_THREADS : last;             \
+        held[u] = *reinterpret_cast<const Piece *>(src + ((first + (k0_) + at / pieces) * a.heads + h) * a.rowBytes + \
+                                                   (at % pieces) * 16);                                       \
+    }
+    // (a plain vector type: arrays of the runtime's uint4 structure that live across loop iterations stay in memory)
+    typedef unsigned int Piece __attribute__((ext_vector_type(4)));
+    Piece held[HELD];
+    if (inRange > 0) {
+        ATBMI_REQUEST_RUN(0, countOf(0))
+    }
     for (int64_t k0 = 0; k0 < inRange; k0 += chunkTokens) {
-        const int count = static_cast<int>(inRange - k0 < chunkTokens ? inRange - k0 : chunkTokens);
+        const int count = countOf(k0);
         __syncthreads(); // the previous run has been added up
-        constexpr int HELD = MEAN_STAGE_BYTES / 16 / CC_THREADS; // 16-byte pieces per thread and run
-        uint4 held[HELD];
-#pragma unroll
-        for (int u = 0; u < HELD; ++u) { // all loads of the run first (lanes past its end repeat its last piece)
-            const int last = count * pieces - 1;
-            const int at = threadIdx.x + u * CC_THREADS < last ? threadIdx.x + u * CC_THREADS : last;
-            held[u] = *reinterpret_cast<const uint4 *>(
-                src + ((first + k0 + at / pieces) * a.heads + h) * a.rowBytes + (at % pieces) * 16);
-        }
 #pragma unroll
         for (int u = 0; u < HELD; ++u) {
             const int at = threadIdx.x + u * CC_THREADS;
             if (at < count * pieces) {
-                *reinterpret_cast<uint4 *>(stage + static_cast<size_t>(at) * 16) = held[u];
+                *reinterpret_cast<Piece *>(stage + static_cast<size_t>(at) * 16) = held[u];
             }
+        }
+        if (k0 + chunkTokens < inRange) {
+            ATBMI_REQUEST_RUN(k0 + chunkTokens, countOf(k0 + chunkTokens))
         }
         __syncthreads();
 #pragma unroll
@@ -238,6 +252,7 @@ __global__ __launch_bounds__(CC_THREADS) void CompressMeanWindowKernel(const Com
             }
         }
     }
+#undef ATBMI_REQUEST_RUN
     uint16_t *dst = reinterpret_cast<uint16_t *>(a.dst[which]);
 #pragma unroll
     for (int i = 0; i < MEAN_MAX_CHANNELS / CC_THREADS; ++i) {
