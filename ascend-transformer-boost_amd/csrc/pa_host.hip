@@ -377,7 +377,7 @@ int PlanStream(AtbmiPaPlan *plan)
         headsPerWg = PA_MLA_HEADS_PER_WG / PA_MFMA_HEAD_TILE;
         tokenSlices = 1;
     }
-    const int headGroups = virtualHeads / headsPerWg;
+    const int headGroups = (virtualHeads + headsPerWg - 1) / headsPerWg; // (only the 128-head kernel leaves a remainder)
     // Several query tokens of one sequence share a pass over its context when a GQA group
     // leaves columns of the 16-wide head tile free: 16 / group tokens per pass.
     int fold = 1;

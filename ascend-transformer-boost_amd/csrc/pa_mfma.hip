@@ -28,7 +28,7 @@ bool PaMlaWide(const AtbmiPaShape &s)
         return !(v && v[0] == '0');
     }();
     return enabled && s.mlaCombined && s.kvDtype != ATBMI_INT8 && s.headDimK == 576 && s.headDimV == 512 &&
-           s.numKvHeads == 1 && s.numHeads % PA_MLA_HEADS_PER_WG == 0 && s.blockSize >= 16 &&
+           s.numKvHeads == 1 && s.numHeads >= 1 && s.blockSize >= 16 &&
            (s.blockSize & (s.blockSize - 1)) == 0 && // (the kernel finds a token's block by shifting)
            (s.qScale == 0.0f || s.qScale == 1.0f) && !s.hasMask && !s.hasLogN; // those take the 16-head kernel
 }

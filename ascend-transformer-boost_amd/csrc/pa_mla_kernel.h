@@ -83,6 +83,7 @@ struct Segment {
     uint32_t tokBegin;    // multiple of 32
     uint32_t tokEnd;      // > tokBegin
     uint32_t complete;    // 1: the segment is the whole row, write the final output
+    uint32_t heads;       // how many of the wave's 32 heads the call has (0: none; q then points at any valid row)
 };
 
 // One segment from start to finish: stages the first tiles, loads Q, runs the pipelined step loop, writes
@@ -106,6 +107,7 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     const uint32_t ropeRowBytes = uni(sg.ropeRowBytes);
     const uint32_t rowBytes = uni(sg.rowBytes), blockShift = uni(sg.blockShift), tokBegin = uni(sg.tokBegin);
     const uint32_t tokEnd = uni(sg.tokEnd), complete = uni(sg.complete);
+    const uint32_t heads = uni(sg.heads), lastHead = uni(sg.heads > 0 ? sg.heads - 1 : 0);
     ldsBase = uni(ldsBase);
     wave = uni(wave);
     scale2 = __builtin_bit_cast(float, uni(__builtin_bit_cast(uint32_t, scale2)));
@@ -542,13 +544,34 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
       s_cbranch_scc0 5f
       // a whole tile three steps ahead: its transfers ride along
       DMA_PREP
+      s_cmp_eq_u32 %[nh], 0
+      s_cbranch_scc1 20f
       QK_PHASE \SN, \SO
       PV_PHASE 1
+      s_branch 21f
+      20:
+      // a wave without heads only moves its rows of the tile
+      s_add_u32 s53, s58, s41
+      s_add_u32 s54, s53, 8192
+      s_mov_b32 m0, s54
+      s_nop 0
+      DMA_ONE 8
+      DMA_ONE 9
+      s_add_u32 s54, s53, 4096
+      s_mov_b32 m0, s54
+      s_nop 0
+      .irp i,0,1,2,3,4,5,6,7
+        DMA_ONE \i
+      .endr
+      21:
       s_waitcnt vmcnt(NDMA)                // all but the tile just requested have landed
       s_branch 6f
       5:
+      s_cmp_eq_u32 %[nh], 0
+      s_cbranch_scc1 22f
       QK_PHASE \SN, \SO
       PV_PHASE 0
+      22:
       s_cmp_lt_u32 s59, s37
       s_cbranch_scc0 7f
       DMA_PREP                             // the segment's last, partial tile
@@ -657,11 +680,13 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     v_min_u32 v91, s43, v91
     v_lshlrev_b32 v91, 2, v91
     global_load_dword v98, v91, %[table]
-    // ---- Q: lane (n, kh) holds q[h0 + n][16 j + 8 kh .. +8) for the 36 pieces j
+    // ---- Q: lane (n, kh) holds q[h0 + n][16 j + 8 kh .. +8) for the 36 pieces j; a wave with fewer than 32 heads
+    // repeats its last one in the lanes past it (their rows are computed and not stored)
+    v_min_u32 v93, %[qlast], v89
     .if SPLIT
-      v_lshlrev_b32 v88, 10, v89
+      v_lshlrev_b32 v88, 10, v93
       v_lshl_add_u32 v88, v90, 4, v88      // rows of 512 channels
-      v_lshlrev_b32 v91, 7, v89
+      v_lshlrev_b32 v91, 7, v93
       v_lshl_add_u32 v91, v90, 4, v91      // rows of 64 channels
       .irp j,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15,16,17,18,19,20,21,22,23,24,25,26,27,28,29,30,31
         global_load_dwordx4 v[112+4*\j:115+4*\j], v88, %[q] offset:32*\j
@@ -670,7 +695,7 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
         global_load_dwordx4 v[112+4*\j:115+4*\j], v91, %[qrope] offset:32*(\j-32)
       .endr
     .else
-      v_mul_u32_u24 v88, 1152, v89
+      v_mul_u32_u24 v88, 1152, v93
       v_lshl_add_u32 v88, v90, 4, v88
       .irp j,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15,16,17,18,19,20,21,22,23,24,25,26,27,28,29,30,31,32,33,34,35
         global_load_dwordx4 v[112+4*\j:115+4*\j], v88, %[q] offset:32*\j
@@ -717,6 +742,8 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     s_barrier
     // ---- scores of the first tile
     v_add_u32 v94, s38, v96
+    s_cmp_eq_u32 %[nh], 0
+    s_cbranch_scc1 1f
     QK_PHASE 0, -1
     s_nop 15
     s_nop 1
@@ -725,11 +752,15 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     BODY 0, 16, 3f
     s_branch 1b
     2:
+    s_cmp_eq_u32 %[nh], 0
+    s_cbranch_scc1 4f
     v_add_u32 v95, s38, v97
     SM_ALONE 0
     PV_PHASE 0
     s_branch 4f
     3:
+    s_cmp_eq_u32 %[nh], 0
+    s_cbranch_scc1 4f
     v_add_u32 v95, s38, v97
     SM_ALONE 16
     PV_PHASE 0
@@ -792,15 +823,22 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
       .endr
       s_waitcnt lgkmcnt(0)
       .irp k,0,1,2,3
+        s_cmp_gt_u32 %[nh], 8*\b+\k          // (row 8 b + k belongs to a head of the call)
+        s_cselect_b64 exec, -1, 0
+        s_nop 1
         global_store_dwordx4 v92, v[4*\k:4*\k+3], s[50:51] offset:1024*\k
       .endr
       s_add_u32 s50, s50, 4096
       s_addc_u32 s51, s51, 0
       .irp k,4,5,6,7
+        s_cmp_gt_u32 %[nh], 8*\b+\k
+        s_cselect_b64 exec, -1, 0
+        s_nop 1
         global_store_dwordx4 v92, v[4*\k:4*\k+3], s[50:51] offset:1024*(\k-4)
       .endr
       s_add_u32 s50, s50, 4096
       s_addc_u32 s51, s51, 0
+      s_mov_b64 exec, -1
     .endr
     s_barrier                                // the next segment's transfers may take the buffers
     s_mov_b64 s[60:61], exec
@@ -816,7 +854,7 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     .else
       v_cvt_f16_f32 v85, v85
     .endif
-    s_mov_b64 exec, 0xffffffff
+    s_bfm_b64 exec, %[nh], 0                 // lanes 0 .. heads - 1
     s_nop 1
     global_store_short v91, v85, %[lse]
     s_mov_b64 exec, s[60:61]
@@ -824,7 +862,7 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     13:
     // partial row: its base-2 log-sum-exp, fp32
     v_lshlrev_b32 v91, 2, v89
-    s_mov_b64 exec, 0xffffffff
+    s_bfm_b64 exec, %[nh], 0
     s_nop 1
     global_store_dword v91, v85, %[lse]
     s_mov_b64 exec, s[60:61]
@@ -848,7 +886,7 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
                    [rope_hi] "s"(ropeHi), [roperowbytes] "s"(ropeRowBytes), [scale] "s"(scale2), [bshift] "s"(blockShift), [table] "s"(table),
                    [rowbytes] "s"(rowBytes), [cache_lo] "s"(cacheLo), [cache_hi] "s"(cacheHi), [q] "s"(q), [out] "s"(out),
                    [lse] "s"(lse), [tokbegin] "s"(tokBegin), [tokend] "s"(tokEnd), [lds] "s"(ldsBase), [wave] "s"(wave),
-                   [complete] "s"(complete)
+                   [complete] "s"(complete), [nh] "s"(heads), [qlast] "s"(lastHead)
                  : "memory", "vcc", "scc", "m0", ATBMI_REGS_0_99("v"), ATBMI_REGS_112_255("v"), ATBMI_REGS_0_99("a"),
                    ATBMI_REGS_100_111("a"), ATBMI_REGS_112_255("a"), ATBMI_SREGS_36_69("s"));
 }
@@ -878,7 +916,11 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaAsmKernel(const PaArgs a, const
     }
     const uint32_t ldsBase = static_cast<uint32_t>(
         reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char *)smem));
+    // (a head count that is not a multiple of 128 leaves the last workgroup waves with fewer than 32 heads, or with
+    // none: those still stage their rows of every tile, compute on a repeated query row and store nothing)
     const int h0 = hgIdx * PA_MLA_HEADS_PER_WG + static_cast<int>(wave) * HPW;
+    const int liveHeads = min(max(a.H - h0, 0), HPW);
+    const int hq = liveHeads > 0 ? h0 : 0; // where this wave's query rows are read from
     constexpr float LOG2E = 1.4426950408889634f;
     const float scale2 = a.qkScale * LOG2E;
     const uint32_t blockShift = static_cast<uint32_t>(__builtin_ctz(static_cast<unsigned>(a.blockSize)));
@@ -909,8 +951,10 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaAsmKernel(const PaArgs a, const
         sg.tokEnd = static_cast<uint32_t>(min(ctxLen, (segEnd - stepBegin) * STEP));
         sg.complete = (segBegin == stepBegin && segEnd == seqEnd) ? 1u : 0u;
         const int64_t rowHead = static_cast<int64_t>(qRow) * a.H + h0;
-        sg.q = reinterpret_cast<const uint16_t *>(a.q) + rowHead * (SPLIT ? DV : D);
-        sg.qRope = SPLIT ? reinterpret_cast<const uint16_t *>(a.qRope) + rowHead * (D - DV) : nullptr;
+        const int64_t rowQuery = static_cast<int64_t>(qRow) * a.H + hq;
+        sg.heads = static_cast<uint32_t>(liveHeads);
+        sg.q = reinterpret_cast<const uint16_t *>(a.q) + rowQuery * (SPLIT ? DV : D);
+        sg.qRope = SPLIT ? reinterpret_cast<const uint16_t *>(a.qRope) + rowQuery * (D - DV) : nullptr;
         sg.ropeCache = SPLIT ? a.kRope : nullptr;
         sg.ropeRowBytes = SPLIT ? static_cast<uint32_t>(a.ropeRowStride * 2) : 0u;
         if (sg.complete) {
@@ -935,7 +979,7 @@ template <bool BF16, bool SPLIT, bool NZ = false> int LaunchAsm(const PaArgs &ar
         return configured;
     }
     if (plan.tokenSlices != 1 || plan.numWaveRanges != plan.numWgRanges ||
-        plan.headGroups * PA_MLA_HEADS_PER_WG != args.H || args.G != 1 || args.D != D || args.Dv != DV ||
+        plan.headGroups != (args.H + PA_MLA_HEADS_PER_WG - 1) / PA_MLA_HEADS_PER_WG || args.G != 1 || args.D != D || args.Dv != DV ||
         args.ropeDim != (SPLIT ? D - DV : 0) || (args.nzShift > 0) != NZ || args.blockSize < 16 || (args.blockSize & (args.blockSize - 1)) != 0 ||
         args.kRowStride * 2 > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: plan or shape does not fit the 128-head MLA kernel");

@@ -44,10 +44,13 @@ CONFIGS["c2_bnsd"] = dict(CONFIGS["c2"], bnsd=True)
 CONFIGS["c5_split"] = dict(CONFIGS["c5"], split=True)
 CONFIGS["c5_nz"] = dict(CONFIGS["c5"], split=True, nz=True)
 CONFIGS["c5_int8"] = dict(CONFIGS["c5"], split=True, nz=True, int8nz=True)
+# C5 as one of eight / four tensor-parallel ranks sees it: the same cache, 16 / 32 of the 128 query heads
+CONFIGS["c5_h16"] = dict(CONFIGS["c5"], heads=16)
+CONFIGS["c5_h32"] = dict(CONFIGS["c5"], heads=32)
 # C3 with int8 queries as well (PagedAttentionParam quantType QKV online): the same int8 caches, one descale per query head
 CONFIGS["c3_int8q"] = dict(CONFIGS["c3"], int8q=True)
 
-SEEDS = {"c1": 1001, "c2": 1002, "c2_fp16": 1002, "c2_alibi": 1002, "c2_norm": 1002, "c2_mtp4": 1002, "c2_bnsd": 1002, "c3": 1003, "c4": 1004, "c5": 1005, "c5_split": 1005, "c5_nz": 1005, "c5_int8": 1005, "c3_int8q": 1003}
+SEEDS = {"c1": 1001, "c2": 1002, "c2_fp16": 1002, "c2_alibi": 1002, "c2_norm": 1002, "c2_mtp4": 1002, "c2_bnsd": 1002, "c3": 1003, "c4": 1004, "c5": 1005, "c5_split": 1005, "c5_nz": 1005, "c5_int8": 1005, "c5_h16": 1005, "c5_h32": 1005, "c3_int8q": 1003}
 
 
 def config(name, **overrides):

@@ -43,7 +43,7 @@ WORKLOAD_SOURCES = {
     "c2_mtp4": _MFMA + ["pa_mfma_bf16.hip"], "c2_bnsd": _MFMA + ["pa_mfma_bf16.hip"],
     "c1": _MFMA + ["pa_mfma_f16.hip"], "c2_fp16": _MFMA + ["pa_mfma_f16.hip"], "c4": _MFMA + ["pa_mfma_f16.hip"],
     "c3": _MFMA + ["pa_mfma_int8.hip"],
-    "c5": _MLA, "c5_split": _MLA, "c5_nz": _MLA,
+    "c5": _MLA, "c5_split": _MLA, "c5_nz": _MLA, "c5_h16": _MLA, "c5_h32": _MLA,
     "c5_int8": ["atbmi_common.h", "pa_internal.h", "mla_int8.hip"],
     "c3_int8q": ["atbmi_common.h", "pa_internal.h", "pa_int8q.hip"],
 }
@@ -114,6 +114,10 @@ DESCRIPTIONS = {
                "fractal-NZ, bf16 rotary parts; random int8 contents), attention only: batch 64, 128 q heads, block 128, "
                "ctx U[2048,4096]",
     "c5": "C5 MLA bf16 decode: batch 64, 128 q heads, 1 latent kv head, d576/dv512, block 128, ctx U[2048,4096]",
+    "c5_h16": "C5 on one of eight tensor-parallel ranks (16 of the 128 q heads, the whole latent cache): batch 64, "
+              "d576/dv512, block 128, ctx U[2048,4096], bf16",
+    "c5_h32": "C5 on one of four tensor-parallel ranks (32 of the 128 q heads, the whole latent cache): batch 64, "
+              "d576/dv512, block 128, ctx U[2048,4096], bf16",
 }
 
 

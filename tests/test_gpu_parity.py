@@ -1437,11 +1437,18 @@ MLA_WIDE_MATRIX = [
     (2, 128, 16, [18000, 500], torch.bfloat16, None, "block size 16, many short ranges"),
     (5, 128, 32, [96, 4100, 1, 160, 2047], torch.float16, 4096, "block size 32, ranges spanning sequences"),
     (1, 128, 128, [12345], torch.float16, 320, "one long row merged from many ranges"),
+    # head counts that are not a multiple of 128 (tensor-parallel ranks): waves with fewer than 32 heads, or none
+    (3, 16, 128, [700, 45, 1], torch.bfloat16, None, "16 heads: half a wave"),
+    (4, 32, 128, [2100, 333, 32, 64], torch.float16, None, "32 heads: one wave"),
+    (3, 64, 64, [1500, 257, 31], torch.bfloat16, 64, "64 heads, rows cut everywhere"),
+    (2, 40, 128, [900, 129], torch.float16, None, "40 heads: a wave and a quarter of one"),
+    (2, 136, 128, [900, 129], torch.bfloat16, None, "136 heads: a second group of 8"),
+    (2, 8, 16, [3000, 5], torch.float16, None, "8 heads, block size 16"),
 ]
 
 
-@pytest.mark.parametrize("case", MLA_WIDE_MATRIX, ids=lambda c: "b%d_h%d_bs%d_%s" % (
-    c[0], c[1], c[2], str(c[4]).split(".")[-1]))
+@pytest.mark.parametrize("case", MLA_WIDE_MATRIX, ids=lambda c: "b%d_h%d_bs%d_%s_%s" % (
+    c[0], c[1], c[2], str(c[4]).split(".")[-1], c[5]))
 def test_paged_attention_mla_128_head_kernel(binding, oracle, dev, stream, case):
     """Checked against the oracle and, element by element, against the fp32 scalar kernel."""
     batch, heads, block, ctx, dtype, chunk, _ = case

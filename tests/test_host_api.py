@@ -778,10 +778,11 @@ def test_multi_latent_attention_causal_rows_and_mask_use_status(binding, ctx):
     # 16-bit values per query token, after the plan's own bytes and the 16-byte row records
     op = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1,
                                                                calcType=1, maskType=2))
+    # (the same call with the mask rows handed over ready-made plans the same kernel and needs only the plan's bytes)
     plain = binding.Operation("MultiLatentAttentionOperation", mk(headNum=32, kvHeadNum=1, qkScale=0.07, cacheMode=1,
-                                                                  calcType=1, maskType=3))
+                                                                  calcType=1, maskType=1))
     st, ws = op.setup(pack(32, mask=[131, 128]), outs(32, lse=False), ctx)
-    st0, ws0 = plain.setup(pack(32), outs(32, lse=False), ctx)
+    st0, ws0 = plain.setup(pack(32, mask=[8, 384]), outs(32, lse=False), ctx)
     assert (st, st0) == (0, 0) and ws >= ws0 + 8 * 16 + 8 * 384 * 2 and ws <= ws0 + 8 * 16 + 8 * 384 * 2 + 1024
     assert op.setup(pack(32, mask=[4, 131, 128]), outs(32, lse=False), ctx)[0] == 0           # a template per sequence
     assert op.setup(pack(32, mask=[3, 131, 128]), outs(32, lse=False), ctx)[0] == e["ERROR_INVALID_PARAM"]
