@@ -54,12 +54,13 @@ WORKLOAD_SOURCES = {
 # sources at the time it was measured: a changed workload or changed kernels report null, not a stale figure.
 MEASURED_TRAFFIC = {
     # (workload, algorithmic bytes): (HBM bytes, summary under profiles/, source hash of the workload)
-    ("c2", 651658484): (659484594, "pa_mfma_bf16_d128_c2_trace_and_traffic.md", "2c904a8627a2"),
-    ("c2_fp16", 651658484): (659480767, "pa_mfma_fp16_d128_c2_fp16_trace_and_traffic.md", "14304002c36b"),
-    ("c3", 1364204576): (1381770597, "pa_mfma_int8_d128_c3_trace_and_traffic.md", "3f838484daed"),
+    ("c2", 651658484): (659483215, "pa_mfma_bf16_d128_c2_trace_and_traffic.md", "553ef2d3185e"),
+    ("c2_fp16", 651658484): (659483056, "pa_mfma_fp16_d128_c2_fp16_trace_and_traffic.md", "a0b9bba458c5"),
+    ("c3", 1364204576): (1381771991, "pa_mfma_int8_d128_c3_trace_and_traffic.md", "763094e7afeb"),
     ("c3_int8q", 1363148320): (1379216115, "pa_int8q_d128_c3_sizes_trace_counters_traffic.md", "92c707eb4b3b"),
-    ("c4", 722875880): (728782791, "pa_mfma_fp16_d128_c4_trace_and_traffic.md", "14304002c36b"),
-    ("c5", 253384304): (349275948, "pa_mla_bf16_d576_c5_trace_and_traffic.md", "e76fc61fbe37"),
+    ("c4", 722875880): (728783244, "pa_mfma_fp16_d128_c4_trace_and_traffic.md", "a0b9bba458c5"),
+    ("c5_h16", 237786736): (250863269, "pa_mla_bf16_d576_c5_16_heads_trace_and_traffic.md", "d4abb8fe1f36"),
+    ("c5", 253384304): (349335955, "pa_mla_bf16_d576_c5_trace_and_traffic.md", "d4abb8fe1f36"),
 }
 OTHER_WORKLOADS = ["c2_fp16", "c3", "c3_int8q", "c4", "c5"]  # timed in the same run as the headline workload
 MIN_KERNEL_LAUNCHES = 100  # launches behind every kernel figure, whatever --steps says
