@@ -32,8 +32,9 @@ bool PaMfmaSharedTile(const AtbmiPaShape &shape);
 int LaunchPaMfma(const AtbmiPaShape &shape, const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream);
 
 // 128-head kernel for the combined 576/512 cache (one latent KV head, any number of query heads: waves past the
-// last head only stage tiles): four waves of 32 heads each share one staged latent tile. The plan must then use one wave range
-// per workgroup and numHeads / 128 head groups. ATBMI_PA_MLA_WIDE=0 in the environment turns it off.
+// last head only stage tiles): four waves of 32 heads each share one staged latent tile. The plan must then use one
+// wave range per workgroup and one head group per 128 heads or part of them. ATBMI_PA_MLA_WIDE=0 in the environment
+// turns it off.
 constexpr int PA_MLA_WAVES = 4;
 constexpr int PA_MLA_HEADS_PER_WG = 128;
 bool PaMlaWide(const AtbmiPaShape &shape);
