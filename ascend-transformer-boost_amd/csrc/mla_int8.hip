@@ -706,7 +706,11 @@ extern "C" int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspa
         return Fail(ERR_INVALID_PARAM, "mla_int8: workspace of %llu bytes, %llu needed", (unsigned long long)workspaceBytes,
                     (unsigned long long)bytes);
     }
-    const int nt = call->numHeads > mlaint8::HT ? 2 : 1; // head tiles of 16 a workgroup
+    // Head tiles of 16 a workgroup: two share a block's rows in LDS and cost 1.35 times one tile's time a block, so
+    // two are taken when tiles of one would need more workgroups than the chip holds at once (one a CU), and one when
+    // they fit: the call lasts as long as its longest row, and more, lighter workgroups then end sooner.
+    const int64_t tilesOfOne = static_cast<int64_t>(rows.size()) * ((call->numHeads + mlaint8::HT - 1) / mlaint8::HT);
+    const int nt = (call->numHeads > mlaint8::HT && tilesOfOne > DeviceComputeUnits()) ? 2 : 1;
     const int headsPerWg = nt * mlaint8::HT;
     const int64_t grid = (static_cast<int64_t>(rows.size()) * ((call->numHeads + headsPerWg - 1) / headsPerWg) + 7) / 8 * 8;
     if (grid > 0x7fffffffLL) {
