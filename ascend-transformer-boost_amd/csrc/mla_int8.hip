@@ -42,7 +42,8 @@
 // Operand layout of v_mfma_i32_16x16x64_i8 (checked with a probe on the device): lane (n = lane % 16, kg =
 // lane / 16) supplies the 16 contraction values 16 kg .. 16 kg + 15 of row n (A) / column n (B) and receives
 // D[4 kg + e][n], e = 0 .. 3.
-// One pass per query row (no split over the context).
+// One pass per query row when the call has workgroups enough for the chip; a call with few heads cuts every row's
+// blocks into up to four equal pieces, each a workgroup's, and MlaInt8MergeKernel joins them (SplitFor).
 #include <algorithm>
 #include <type_traits>
 #include <vector>
@@ -90,13 +91,15 @@ template <int NT> struct Lds {
 static_assert(TILE == NWAVES * 16 && DN == NWAVES * 64 && PIECES_PER_WAVE == 8,
               "eight waves share a tile this way");
 
-// One query row: its sequence's block-table row and context length, the row of query / out, the mask row.
+// One query row, or one of the equal pieces its context is cut into (Args::pieces > 1, piece `piece` of every row
+// in turn): its sequence's block-table row and context length, the row of query / out / mask.
 struct Row {
     int32_t tableRow;
     int32_t ctxLen;
     int32_t qRow;
-    int32_t pad;
+    int32_t piece;
 };
+constexpr int MAX_PIECES = 4;
 
 constexpr int INLINE_ROWS = 128; // calls with up to this many query rows carry them in the kernel arguments
 
@@ -112,6 +115,9 @@ struct Args {
     void *out;
     float *lse;
     const Row *rows; // null: inlineRows
+    void *partO;     // pieces > 1: [entries][H][512] rows of the pieces, each normalised on its own, in the type of out
+    float *partLse;  // pieces > 1: [entries][H] their base-2 log-sum-exps (-inf: a piece without tokens)
+    int32_t pieces;  // pieces a row's blocks are cut into (1: none; the kernel then writes out and lse itself)
     int32_t H;
     int32_t numRows;
     int32_t maxBlocksPerSeq;
@@ -227,11 +233,21 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
     if (work >= a.numRows * headTiles) {
         return;
     }
-    const Row row = a.rows ? a.rows[work / headTiles] : a.inlineRows[work / headTiles];
+    const int entry = work / headTiles;
+    const Row row = a.rows ? a.rows[entry] : a.inlineRows[entry];
     const int h0 = (work % headTiles) * HW;
     const int nh = min(HW, a.H - h0); // heads past the last one compute on zeros and store nothing
-    const int32_t *table = a.tables + static_cast<int64_t>(row.tableRow) * a.maxBlocksPerSeq;
-    const int numBlocks = (row.ctxLen + TILE - 1) / TILE;
+    // this workgroup's blocks of the row: all of them, or piece `row.piece` of a.pieces equal shares
+    const int allBlocks = (row.ctxLen + TILE - 1) / TILE;
+    const int firstBlock = a.pieces > 1 ? allBlocks * row.piece / a.pieces : 0;
+    const int numBlocks = (a.pieces > 1 ? allBlocks * (row.piece + 1) / a.pieces : allBlocks) - firstBlock;
+    if (numBlocks <= 0) { // (a row with fewer blocks than pieces)
+        if (tid < nh) {
+            a.partLse[static_cast<int64_t>(entry) * a.H + h0 + tid] = -INFINITY;
+        }
+        return;
+    }
+    const int32_t *table = a.tables + static_cast<int64_t>(row.tableRow) * a.maxBlocksPerSeq + firstBlock;
     const uint32_t ldsBase =
         static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char *)smem));
 
@@ -260,7 +276,7 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
     const uint16_t *maskRow = reinterpret_cast<const uint16_t *>(a.mask) + static_cast<int64_t>(row.qRow) * a.maskLen;
     auto loadMask = [&](int block, uint32_t(&bits)[4]) { // this lane's four tokens of the block
         if constexpr (MASK) {
-            const int tok = block * TILE + wave * 16 + kg * 4;
+            const int tok = (firstBlock + block) * TILE + wave * 16 + kg * 4;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 bits[e] = maskRow[min(tok + e, row.ctxLen - 1)];
@@ -442,7 +458,7 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
         // ---- scores of tokens 16 wave .. + 15, in units of log 2
         float x2[NT][4];
         {
-            const int tok = i * TILE + wave * 16 + kg * 4; // this lane's four tokens
+            const int tok = (firstBlock + i) * TILE + wave * 16 + kg * 4; // this lane's four tokens
             // every piece of the rows serves all head tiles as it arrives
             i32x4 dots[NT];
             f32x4 rdots[NT];
@@ -582,8 +598,10 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
         const float total = ((s0[0] + s0[1]) + (s0[2] + s0[3])) + ((s1[0] + s1[1]) + (s1[2] + s1[3]));
         if (nt * HT + n < nh) {
             const float inv = total > 0.0f ? pvDescale[nt] * unitStep[nt] / total : 0.0f;
-            uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) +
-                             (static_cast<int64_t>(row.qRow) * a.H + h0 + nt * HT + n) * DN + wave * 64 + kg * 4;
+            // the row itself, or this piece's share of it for the merge kernel
+            const int64_t rowHead = a.pieces > 1 ? static_cast<int64_t>(entry) * a.H + h0 + nt * HT + n
+                                                 : static_cast<int64_t>(row.qRow) * a.H + h0 + nt * HT + n;
+            uint16_t *orow = reinterpret_cast<uint16_t *>(a.pieces > 1 ? a.partO : a.out) + rowHead * DN + wave * 64 + kg * 4;
 #pragma unroll
             for (int cs = 0; cs < 4; ++cs) {
                 uint16_t bits[4];
@@ -597,12 +615,122 @@ __global__ __launch_bounds__(THREADS) void MlaInt8Kernel(const Args a)
                 w.y = static_cast<uint32_t>(bits[2]) | (static_cast<uint32_t>(bits[3]) << 16);
                 *reinterpret_cast<uint2 *>(orow + cs * 16) = w;
             }
-            if (a.lse && wave == 0 && kg == 0) {
-                a.lse[static_cast<int64_t>(row.qRow) * a.H + h0 + nt * HT + n] =
-                    total > 0.0f ? logf(total) + runMax[nt] * LN2 : -INFINITY;
+            if (wave == 0 && kg == 0) {
+                if (a.pieces > 1) {
+                    a.partLse[rowHead] = total > 0.0f ? __log2f(total) + runMax[nt] : -INFINITY;
+                } else if (a.lse) {
+                    a.lse[rowHead] = total > 0.0f ? logf(total) + runMax[nt] * LN2 : -INFINITY;
+                }
             }
         }
     }
+}
+
+// Joins the pieces of every row: one wave per (row, head), eight channels a lane. A piece weighs 2^(its log-sum-exp
+// less the largest of the row's).
+constexpr int MERGE_THREADS = 256;
+template <bool BF16> __global__ __launch_bounds__(MERGE_THREADS) void MlaInt8MergeKernel(const Args a)
+{
+    constexpr float LN2 = 0.693147180559945f;
+    const int lane = threadIdx.x % WAVE;
+    const int64_t pair = static_cast<int64_t>(blockIdx.x) * (MERGE_THREADS / WAVE) + threadIdx.x / WAVE;
+    const int rowIdx = static_cast<int>(pair / a.H);
+    const int head = static_cast<int>(pair % a.H);
+    if (rowIdx >= a.numRows / a.pieces) {
+        return;
+    }
+    const int entry0 = rowIdx * a.pieces;
+    const Row row = a.rows ? a.rows[entry0] : a.inlineRows[entry0];
+    float lse[MAX_PIECES];
+    float top = -INFINITY;
+    for (int p = 0; p < a.pieces; ++p) {
+        lse[p] = a.partLse[static_cast<int64_t>(entry0 + p) * a.H + head];
+        top = fmaxf(top, lse[p]);
+    }
+    float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    float sum = 0.0f;
+    for (int p = 0; p < a.pieces; ++p) {
+        if (lse[p] == -INFINITY) {
+            continue; // (nothing was written for a piece without tokens)
+        }
+        const float w = exp2f(lse[p] - top);
+        sum += w;
+        const uint4 raw = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(a.partO) +
+                                                           (static_cast<int64_t>(entry0 + p) * a.H + head) * DN + lane * 8);
+        const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            acc[2 * k] += w * Load16AsFloat(words[k] & 0xffffu, BF16);
+            acc[2 * k + 1] += w * Load16AsFloat(words[k] >> 16, BF16);
+        }
+    }
+    const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
+    uint32_t packed[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float lo = acc[2 * k] * inv, hi = acc[2 * k + 1] * inv;
+        packed[k] = static_cast<uint32_t>(BF16 ? FloatToBf16(lo) : FloatToHalfBits(lo)) |
+                    (static_cast<uint32_t>(BF16 ? FloatToBf16(hi) : FloatToHalfBits(hi)) << 16);
+    }
+    const int64_t rowHead = static_cast<int64_t>(row.qRow) * a.H + head;
+    *reinterpret_cast<uint4 *>(reinterpret_cast<uint16_t *>(a.out) + rowHead * DN + lane * 8) =
+        uint4{packed[0], packed[1], packed[2], packed[3]};
+    if (a.lse && lane == 0) {
+        a.lse[rowHead] = sum > 0.0f ? (top + log2f(sum)) * LN2 : -INFINITY;
+    }
+}
+
+// How a call is dealt to the chip: head tiles of 16 a workgroup (one or two) and the equal pieces every row's blocks
+// are cut into (one to four). A call lasts as long as its longest workgroup, and one workgroup runs on a CU at a
+// time. Two head tiles share a block's rows in LDS and take 1.5 times one tile's time a block; pieces fill CUs that
+// would idle, at the price of the merge kernel (3 to 5 us) and of a workgroup's fixed cost. Measured at batch 64,
+// contexts of 2 048 to 4 096 tokens: 128 heads are fastest as two tiles and whole rows (65 us), 64 heads as two
+// tiles and two pieces (44 us against 48 as whole rows of one tile), 32 heads as one tile and two pieces (36 us
+// against 47), 16 heads as one tile and four pieces (32 us against 47). The rule below gives those: one tile when at
+// least two pieces of it fit the chip, as many pieces as fit (of at least four blocks in the longest row).
+struct Split {
+    int headTiles;
+    int pieces;
+};
+Split SplitFor(const AtbmiMlaInt8Call *c, const std::vector<Row> &rows)
+{
+    const int64_t cus = DeviceComputeUnits();
+    const int64_t tilesOfOne = static_cast<int64_t>(rows.size()) * ((c->numHeads + HT - 1) / HT);
+    const int64_t tilesOfTwo = static_cast<int64_t>(rows.size()) * ((c->numHeads + 2 * HT - 1) / (2 * HT));
+    Split split{1, 1};
+    if (tilesOfOne == 0) {
+        return split;
+    }
+    split.headTiles = (c->numHeads > HT && 2 * tilesOfOne > cus) ? 2 : 1;
+    int32_t longest = 0;
+    for (const Row &r : rows) {
+        longest = std::max(longest, (r.ctxLen + TILE - 1) / TILE);
+    }
+    const int64_t workgroups = split.headTiles == 2 ? tilesOfTwo : tilesOfOne;
+    int pieces = static_cast<int>(std::min<int64_t>(MAX_PIECES, cus / workgroups));
+    while (pieces > 1 && longest < 4 * pieces) {
+        --pieces;
+    }
+    split.pieces = std::max(pieces, 1);
+    return split;
+}
+
+// Bytes of the workspace's parts: the table of rows (entries x 16, to a multiple of 256), the pieces' rows and
+// their log-sum-exps (none when the rows are whole).
+struct WorkspaceLayout {
+    size_t table, partO, partLse;
+    size_t Total() const { return table + partO + partLse; }
+};
+WorkspaceLayout LayoutFor(const AtbmiMlaInt8Call *c, size_t rowCount, int pieces)
+{
+    const size_t entries = rowCount * static_cast<size_t>(pieces);
+    WorkspaceLayout l{};
+    l.table = (entries * sizeof(Row) + 255) / 256 * 256;
+    if (pieces > 1) {
+        l.partO = entries * static_cast<size_t>(c->numHeads) * DN * sizeof(uint16_t);
+        l.partLse = (entries * static_cast<size_t>(c->numHeads) * sizeof(float) + 255) / 256 * 256;
+    }
+    return l;
 }
 
 // Checks the call and lists its query rows (sequences of length 0 take none).
@@ -682,7 +810,7 @@ extern "C" int atbmi_mla_int8_workspace_size(const AtbmiMlaInt8Call *call, uint6
     if (rc != OK) {
         return rc;
     }
-    *bytes = rows.size() * sizeof(mlaint8::Row);
+    *bytes = mlaint8::LayoutFor(call, rows.size(), mlaint8::SplitFor(call, rows).pieces).Total();
     return OK;
 }
 
@@ -701,16 +829,25 @@ extern "C" int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspa
         !call->qkDescale || !call->pvDescale || !call->out || (call->hasMask && !call->mask)) {
         return Fail(ERR_INVALID_PARAM, "mla_int8: null tensor pointer");
     }
-    const size_t bytes = rows.size() * sizeof(mlaint8::Row);
+    const mlaint8::Split split = mlaint8::SplitFor(call, rows);
+    const int pieces = split.pieces;
+    const mlaint8::WorkspaceLayout layout = mlaint8::LayoutFor(call, rows.size(), pieces);
+    const size_t bytes = layout.Total();
+    if (pieces > 1) { // every row once per piece, a row's pieces next to each other
+        std::vector<mlaint8::Row> entries;
+        entries.reserve(rows.size() * pieces);
+        for (const mlaint8::Row &r : rows) {
+            for (int p = 0; p < pieces; ++p) {
+                entries.push_back(mlaint8::Row{r.tableRow, r.ctxLen, r.qRow, p});
+            }
+        }
+        rows.swap(entries);
+    }
     if (!workspaceDevice || workspaceBytes < bytes) {
         return Fail(ERR_INVALID_PARAM, "mla_int8: workspace of %llu bytes, %llu needed", (unsigned long long)workspaceBytes,
                     (unsigned long long)bytes);
     }
-    // Head tiles of 16 a workgroup: two share a block's rows in LDS and cost 1.35 times one tile's time a block, so
-    // two are taken when tiles of one would need more workgroups than the chip holds at once (one a CU), and one when
-    // they fit: the call lasts as long as its longest row, and more, lighter workgroups then end sooner.
-    const int64_t tilesOfOne = static_cast<int64_t>(rows.size()) * ((call->numHeads + mlaint8::HT - 1) / mlaint8::HT);
-    const int nt = (call->numHeads > mlaint8::HT && tilesOfOne > DeviceComputeUnits()) ? 2 : 1;
+    const int nt = split.headTiles;
     const int headsPerWg = nt * mlaint8::HT;
     const int64_t grid = (static_cast<int64_t>(rows.size()) * ((call->numHeads + headsPerWg - 1) / headsPerWg) + 7) / 8 * 8;
     if (grid > 0x7fffffffLL) {
@@ -719,7 +856,7 @@ extern "C" int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspa
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool inlineRows = rows.size() <= static_cast<size_t>(mlaint8::INLINE_ROWS);
     if (!inlineRows) {
-        rc = UploadTable(rows.data(), bytes, workspaceDevice, s);
+        rc = UploadTable(rows.data(), rows.size() * sizeof(mlaint8::Row), workspaceDevice, s);
         if (rc != OK) {
             return rc;
         }
@@ -739,6 +876,10 @@ extern "C" int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspa
     if (inlineRows) {
         std::copy(rows.begin(), rows.end(), a.inlineRows);
     }
+    a.partO = pieces > 1 ? static_cast<unsigned char *>(workspaceDevice) + layout.table : nullptr;
+    a.partLse = pieces > 1 ? reinterpret_cast<float *>(static_cast<unsigned char *>(workspaceDevice) + layout.table + layout.partO)
+                           : nullptr;
+    a.pieces = pieces;
     a.H = call->numHeads;
     a.numRows = static_cast<int32_t>(rows.size());
     a.maxBlocksPerSeq = call->maxBlocksPerSeq;
@@ -765,5 +906,19 @@ extern "C" int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspa
     kernel<<<static_cast<unsigned>(grid), mlaint8::THREADS, ldsBytes, s>>>(a);
     ATBMI_HIP_CHECK(hipGetLastError());
     rc = TimedLaunchKernelDone(s, timed);
-    return rc != OK ? rc : TimedLaunchEnd(s, timed, false);
+    if (rc != OK) {
+        return rc;
+    }
+    if (pieces > 1) {
+        const int64_t pairs = static_cast<int64_t>(rows.size() / pieces) * call->numHeads;
+        const int perGroup = mlaint8::MERGE_THREADS / WAVE;
+        const unsigned mergeGrid = static_cast<unsigned>((pairs + perGroup - 1) / perGroup);
+        if (bf16) {
+            mlaint8::MlaInt8MergeKernel<true><<<mergeGrid, mlaint8::MERGE_THREADS, 0, s>>>(a);
+        } else {
+            mlaint8::MlaInt8MergeKernel<false><<<mergeGrid, mlaint8::MERGE_THREADS, 0, s>>>(a);
+        }
+        ATBMI_HIP_CHECK(hipGetLastError());
+    }
+    return TimedLaunchEnd(s, timed, pieces > 1);
 }

@@ -1652,6 +1652,38 @@ def test_pa_plan_refuses_inconsistent_layout_and_compression_fields(binding):
     assert k.atbmi_reshape_and_cache_omni(16, 16, 16, 16, 16, 16, 16, 16, 0, 4, 128, 0, 256, 0, None) == 0
 
 
+def test_mla_int8_rows_are_cut_when_heads_are_few(binding):
+    """The int8 MLA kernel runs one workgroup a CU: a call with few heads cuts every row's blocks into equal pieces
+    (and asks for room for the pieces' rows and log-sum-exps), a call that fills the chip does not."""
+    k = binding.kernels()
+    lens = np.full(64, 4096, dtype=np.int32)
+
+    def size(heads, batch=64):
+        call = binding.AtbmiMlaInt8Call(outDtype=binding.ATBMI_BF16, numHeads=heads, blockSize=128, numBlocks=4096,
+                                        maxBlocksPerSeq=32, batch=batch, numQueryRows=batch, hasMask=0, maskLen=0,
+                                        qkScale=0.1, hostContextLens=lens.ctypes.data)
+        ws = ctypes.c_uint64(0)
+        assert k.atbmi_mla_int8_workspace_size(ctypes.byref(call), ctypes.byref(ws)) == 0, binding.last_kernel_error()
+        return int(ws.value)
+
+    def pieces(heads, batch=64):
+        table_only = lambda p: (batch * p * 16 + 255) // 256 * 256
+        for p in (1, 2, 3, 4):
+            rows = batch * p
+            want = table_only(p) + (0 if p == 1 else rows * heads * 512 * 2 + (rows * heads * 4 + 255) // 256 * 256)
+            if size(heads, batch) == want:
+                return p
+        raise AssertionError("unexpected workspace size %d" % size(heads, batch))
+
+    assert pieces(128) == 1      # 256 workgroups of two head tiles
+    assert pieces(64) == 2       # 128 workgroups of two head tiles, twice
+    assert pieces(32) == 2       # 128 workgroups of one head tile, twice
+    assert pieces(16) == 4       # 64 workgroups, four times
+    assert pieces(128, batch=8) == 4
+    lens[:] = 1000               # eight blocks a row: pieces of at least four blocks in the longest row
+    assert pieces(16) == 2
+
+
 def test_int8_query_mask_fetches_stay_inside_the_rows(binding):
     """The int8-query kernel fetches 16-bit mask values as aligned 32-bit words, from the word that holds a
     row's first element to the word that holds its last. Host arithmetic over every parity of base, strides and
