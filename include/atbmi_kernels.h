@@ -538,10 +538,13 @@ typedef struct AtbmiMlaInt8Call {
     float *lse;
 } AtbmiMlaInt8Call;
 
-/* Validates the call (pointers aside) and reports the device workspace it needs (16 bytes per query row). */
+/* Validates the call (pointers aside) and reports the device workspace it needs: 16 bytes per query row, and, when
+ * the call has too few heads to fill the chip and its rows are cut into pieces (up to four), the pieces' output rows
+ * and log-sum-exps. */
 int atbmi_mla_int8_workspace_size(const AtbmiMlaInt8Call *call, uint64_t *bytes);
-/* Launches the kernel on `stream`; does not wait. The list of query rows travels in the kernel arguments when it
- * has at most 128 entries and is uploaded into the workspace otherwise (the workspace is asked for either way). */
+/* Launches the kernel (and, for rows cut into pieces, the merge kernel) on `stream`; does not wait. The list of
+ * query rows travels in the kernel arguments when it has at most 128 entries and is uploaded into the workspace
+ * otherwise (the workspace is asked for either way). */
 int atbmi_mla_int8_decode(const AtbmiMlaInt8Call *call, void *workspaceDevice, uint64_t workspaceBytes, void *stream);
 
 /*
