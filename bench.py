@@ -57,7 +57,7 @@ MEASURED_TRAFFIC = {
     ("c2", 651658484): (659482436, "pa_mfma_bf16_d128_c2_trace_and_traffic.md", "bfde6c8e2f5d"),
     ("c2_fp16", 651658484): (659481493, "pa_mfma_fp16_d128_c2_fp16_trace_and_traffic.md", "e352b3749fd0"),
     ("c3", 1364204576): (1381770303, "pa_mfma_int8_d128_c3_trace_and_traffic.md", "a5a50be360bb"),
-    ("c3_int8q", 1363148320): (1379216115, "pa_int8q_d128_c3_sizes_trace_counters_traffic.md", "92c707eb4b3b"),
+    ("c3_int8q", 1363148320): (1379036066, "pa_int8q_d128_c3_sizes_trace_counters_traffic.md", "f19d2f9626c2"),
     ("c4", 722875880): (728782961, "pa_mfma_fp16_d128_c4_trace_and_traffic.md", "e352b3749fd0"),
     ("c5_h16", 237786736): (250872196, "pa_mla_bf16_d576_c5_16_heads_trace_and_traffic.md", "4dce44fe9d89"),
     ("c5", 253384304): (349328455, "pa_mla_bf16_d576_c5_trace_and_traffic.md", "4dce44fe9d89"),
