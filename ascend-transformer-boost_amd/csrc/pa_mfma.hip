@@ -30,7 +30,9 @@ bool PaMlaWide(const AtbmiPaShape &s)
     return enabled && s.mlaCombined && s.kvDtype != ATBMI_INT8 && s.headDimK == 576 && s.headDimV == 512 &&
            s.numKvHeads == 1 && s.numHeads >= 1 && s.blockSize >= 16 &&
            (s.blockSize & (s.blockSize - 1)) == 0 && // (the kernel finds a token's block by shifting)
-           (s.qScale == 0.0f || s.qScale == 1.0f) && !s.hasMask && !s.hasLogN; // those take the 16-head kernel
+           (s.qScale == 0.0f || s.qScale == 1.0f) && !s.hasLogN && // (those take the 16-head kernel)
+           // a mask with one row per query row or sequence (no stride between heads), rows on even elements
+           (!s.hasMask || (s.maskHeadStride == 0 && s.maskBatchStride % 2 == 0));
 }
 
 bool PaMfmaSharedTile(const AtbmiPaShape &s)

@@ -29,6 +29,10 @@
 //     it last, and LDS latency exceeds the MFMA's operand fetch;
 //   - counted lgkmcnt waits only ever count LDS instructions (no scalar loads anywhere in the loop);
 //   - M0 (LDS base of the transfers) is only written when no LDS read of the wave is in flight.
+//
+// MASK builds add a bias per (query row, token) to the scaled scores: the 32 values of a tile come through four
+// buffer loads a lane (a descriptor over the mask row: what lies past its end reads as zero), asked for one step
+// ahead, in front of that step's tile transfers, so that the step's own wait for the transfers covers them.
 #ifndef ATBMI_PA_MLA_KERNEL_H
 #define ATBMI_PA_MLA_KERNEL_H
 #include "pa_mfma_kernel.h"
@@ -84,11 +88,13 @@ struct Segment {
     uint32_t tokEnd;      // > tokBegin
     uint32_t complete;    // 1: the segment is the whole row, write the final output
     uint32_t heads;       // how many of the wave's 32 heads the call has (0: none; q then points at any valid row)
+    const void *mask;     // MASK builds: the query row's mask row (16-bit values of the query's type, 4-byte aligned)
+    uint32_t maskBytes;   // ... and its length in bytes, rounded up to 4
 };
 
 // One segment from start to finish: stages the first tiles, loads Q, runs the pipelined step loop, writes
 // the (partial) row. All four waves of a workgroup call it with the same token range and block table.
-template <bool BF16, bool SPLIT, bool NZ>
+template <bool BF16, bool SPLIT, bool NZ, bool MASK>
 __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, uint32_t wave, float scale2)
 {
     // Every input is wave-uniform; saying so value by value keeps each of them in scalar registers, which
@@ -108,6 +114,9 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     const uint32_t rowBytes = uni(sg.rowBytes), blockShift = uni(sg.blockShift), tokBegin = uni(sg.tokBegin);
     const uint32_t tokEnd = uni(sg.tokEnd), complete = uni(sg.complete);
     const uint32_t heads = uni(sg.heads), lastHead = uni(sg.heads > 0 ? sg.heads - 1 : 0);
+    const uint64_t mask = uni64(sg.mask);
+    const uint32_t maskLo = static_cast<uint32_t>(mask), maskHi = static_cast<uint32_t>(mask >> 32) & 0xffffu;
+    const uint32_t maskBytes = uni(sg.maskBytes);
     ldsBase = uni(ldsBase);
     wave = uni(wave);
     scale2 = __builtin_bit_cast(float, uni(__builtin_bit_cast(uint32_t, scale2)));
@@ -129,6 +138,19 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     .set BF16, %[bf16]
     .set SPLIT, %[split]
     .set NZ, %[nz]
+    .set MASK, %[mask_on]
+    // MASK: v[100:107] the mask values of the tile whose softmax comes next (16-bit pairs: register 2 g + h holds
+    // tokens 8 g + 4 kh + 2 h, + 1 of the tile); s[68:71] the buffer descriptor of the mask row.
+    // the four loads of the mask values of the tile at token \tok (a scalar register)
+    .macro MASK_LOAD tok
+      .if MASK
+        s_lshl_b32 s46, \tok, 1
+        v_lshl_add_u32 v88, v87, 1, s46      // byte of token tok + 4 kh
+        .irp g,0,1,2,3
+          buffer_load_dwordx2 v[100+2*\g:101+2*\g], v88, s[68:71], 0 offen offset:16*\g
+        .endr
+      .endif
+    .endm
     // SPLIT: the last 64 channels of every cache row come from a cache of their own (rows of 128 bytes) and
     // those of every query row from a tensor of their own. A transfer then takes its lanes from two sources:
     // lanes whose slot (64 i + lane, 73 slots a row, the last one padding) holds one of the first 64 pieces
@@ -195,6 +217,23 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     // ---- softmax slice k (k = the QK slot it rides on) of the scores at v[SO : SO+15]; P goes to v[64:71]
     .macro SM_SLICE k, SO
       .if \k == 0
+        .if MASK
+          // scores <- scores x scale + mask x log2(e): the softmax below then works on scaled scores
+          .irp p,0,1,2,3,4,5,6,7
+            .if BF16
+              v_lshlrev_b32 v88, 16, v[100+\p]
+              v_and_b32 v89, 0xffff0000, v[100+\p]
+            .else
+              v_lshrrev_b32 v89, 16, v[100+\p]
+              v_cvt_f32_f16 v88, v[100+\p]
+              v_cvt_f32_f16 v89, v89
+            .endif
+            v_mul_f32 v88, 0x3fb8aa3b, v88
+            v_mul_f32 v89, 0x3fb8aa3b, v89
+            v_fma_f32 v[\SO+4*(\p/2)+2*(\p%%2)], v[\SO+4*(\p/2)+2*(\p%%2)], %[scale], v88
+            v_fma_f32 v[\SO+4*(\p/2)+2*(\p%%2)+1], v[\SO+4*(\p/2)+2*(\p%%2)+1], %[scale], v89
+          .endr
+        .endif
         v_max3_f32 v84, v[\SO+0], v[\SO+1], v[\SO+2]
       .elseif \k == 1
         v_max3_f32 v88, v[\SO+3], v[\SO+4], v[\SO+5]
@@ -214,7 +253,9 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
       .elseif \k == 10
         // (the exchange was issued before K piece 10 was requested: the wait for that piece covers it)
         v_max_f32 v84, v84, v88
-        v_mul_f32 v84, %[scale], v84
+        .if !MASK
+          v_mul_f32 v84, %[scale], v84
+        .endif
         v_add_f32 v89, 0x41000000, v82
         v_cmp_gt_f32 vcc, v84, v89
         s_cbranch_vccz 10f
@@ -238,7 +279,11 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
         .endr
         10:
       .elseif (\k >= 11) && (\k <= 26)
-        v_fma_f32 v[88+(\k%%2)], v[\SO+\k-11], %[scale], -v82
+        .if MASK
+          v_sub_f32 v[88+(\k%%2)], v[\SO+\k-11], v82
+        .else
+          v_fma_f32 v[88+(\k%%2)], v[\SO+\k-11], %[scale], -v82
+        .endif
         s_nop 0
         v_exp_f32 v[\SO+\k-11], v[88+(\k%%2)]
       .elseif (\k >= 27) && (\k <= 34)
@@ -511,6 +556,10 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
       .endif
     .endm
     .macro PV_PHASE DMA
+      .if MASK
+        s_add_u32 s47, s36, 32
+        MASK_LOAD s47                      // of the tile whose softmax rides on the next step's QK phase
+      .endif
       .if \DMA
         // both LDS bases are set while none of the wave's LDS reads is in flight
         s_add_u32 s53, s58, s41
@@ -658,6 +707,12 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
       v_and_b32 v92, 7, v92
       v_lshl_or_b32 v99, v92, 3*\i, v99
     .endr
+    .if MASK
+      s_mov_b32 s68, %[mask_lo]
+      s_mov_b32 s69, %[mask_hi]              // (stride 0: a raw buffer)
+      s_mov_b32 s70, %[mask_bytes]
+      s_mov_b32 s71, 0x00020000
+    .endif
     // ---- segment state
     s_mov_b32 s36, %[tokbegin]
     s_mov_b32 s37, %[tokend]
@@ -736,7 +791,12 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
         v_mfma_f32_32x32x16_f16 a[16*\i:16*\i+15], v[64:67], v[64:67], 0
       .endif
     .endr
-    v_mov_b32 v82, 0xff800000
+    .if MASK
+      v_mov_b32 v82, 0xf149f2ca            // -1e30: a tile that the mask hides altogether leaves -inf - m = -inf, not NaN
+      MASK_LOAD s36
+    .else
+      v_mov_b32 v82, 0xff800000
+    .endif
     v_mov_b32 v83, 0
     s_waitcnt vmcnt(0) lgkmcnt(0)
     s_barrier
@@ -780,6 +840,14 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     v_log_f32 v85, v83
     s_nop 1
     v_add_f32 v85, v85, v82                // log2 of the sum of 2^score
+    .if MASK
+      v_cmp_lt_f32 vcc, 0, v83             // a row that the mask hides altogether: zeros, log-sum-exp -inf
+      s_nop 1
+      v_cndmask_b32 v84, 0, v84, vcc
+      v_mov_b32 v88, 0xff800000
+      s_nop 0
+      v_cndmask_b32 v85, v88, v85, vcc
+    .endif
     // ---- the rows in the query's type, out[h0 + n][0 .. 512) (a partial row has the same form). A lane holds
     // four channels at a time (32 i + 8 r + 4 kh ..): stored from there, a row would reach memory in 64 pieces of
     // 16 bytes. The rows go through LDS instead (the tile buffers are idle now: buffer `wave` holds this wave's
@@ -867,6 +935,10 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     global_store_dword v91, v85, %[lse]
     s_mov_b64 exec, s[60:61]
     14:
+    .if MASK
+      s_waitcnt vmcnt(0)                   // (the last step asked for mask values nobody reads: none may land later)
+    .endif
+    .purgem MASK_LOAD
     .purgem LDK
     .purgem LDV
     .purgem SM_SLICE
@@ -882,17 +954,18 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     .purgem BODY
     )ASM"
                  :
-                 : [bf16] "n"(BF16 ? 1 : 0), [split] "n"(SPLIT ? 1 : 0), [nz] "n"(NZ ? 1 : 0), [qrope] "s"(qRope), [rope_lo] "s"(ropeLo),
+                 : [bf16] "n"(BF16 ? 1 : 0), [split] "n"(SPLIT ? 1 : 0), [nz] "n"(NZ ? 1 : 0), [mask_on] "n"(MASK ? 1 : 0),
+                   [mask_lo] "s"(maskLo), [mask_hi] "s"(maskHi), [mask_bytes] "s"(maskBytes), [qrope] "s"(qRope), [rope_lo] "s"(ropeLo),
                    [rope_hi] "s"(ropeHi), [roperowbytes] "s"(ropeRowBytes), [scale] "s"(scale2), [bshift] "s"(blockShift), [table] "s"(table),
                    [rowbytes] "s"(rowBytes), [cache_lo] "s"(cacheLo), [cache_hi] "s"(cacheHi), [q] "s"(q), [out] "s"(out),
                    [lse] "s"(lse), [tokbegin] "s"(tokBegin), [tokend] "s"(tokEnd), [lds] "s"(ldsBase), [wave] "s"(wave),
                    [complete] "s"(complete), [nh] "s"(heads), [qlast] "s"(lastHead)
-                 : "memory", "vcc", "scc", "m0", ATBMI_REGS_0_99("v"), ATBMI_REGS_112_255("v"), ATBMI_REGS_0_99("a"),
-                   ATBMI_REGS_100_111("a"), ATBMI_REGS_112_255("a"), ATBMI_SREGS_36_69("s"));
+                 : "memory", "vcc", "scc", "m0", ATBMI_REGS_0_99("v"), ATBMI_REGS_100_111("v"), ATBMI_REGS_112_255("v"),
+                   ATBMI_REGS_0_99("a"), ATBMI_REGS_100_111("a"), ATBMI_REGS_112_255("a"), ATBMI_SREGS_36_69("s"), "s70", "s71");
 }
 
 // One wave range per workgroup; the grid is a multiple of 8 x head groups.
-template <bool BF16, bool SPLIT, bool NZ>
+template <bool BF16, bool SPLIT, bool NZ, bool MASK>
 __global__ __launch_bounds__(NW *WAVE) void PaMlaAsmKernel(const PaArgs a, const PaStreamPlan p)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -966,14 +1039,22 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaAsmKernel(const PaArgs a, const
             sg.out = reinterpret_cast<uint16_t *>(a.partO) + ph * DV;
             sg.lse = a.partLse + ph;
         }
-        RunSegment<BF16, SPLIT, NZ>(sg, ldsBase, wave, scale2);
+        if (MASK) {
+            // one mask row per query row (no stride between heads): the row of this pass
+            sg.mask = reinterpret_cast<const uint16_t *>(a.mask) + static_cast<int64_t>(uniform(sq.maskRow)) * a.maskBatchStride;
+            sg.maskBytes = (static_cast<uint32_t>(a.maskLen) * 2u + 3u) & ~3u;
+        } else {
+            sg.mask = nullptr;
+            sg.maskBytes = 0;
+        }
+        RunSegment<BF16, SPLIT, NZ, MASK>(sg, ldsBase, wave, scale2);
     }
 }
 
-template <bool BF16, bool SPLIT, bool NZ = false> int LaunchAsm(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
+template <bool BF16, bool SPLIT, bool NZ, bool MASK> int LaunchAsmBuild(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
 {
     static_assert(SPLIT || !NZ, "fractal-NZ caches come with the split layout");
-    auto kernel = PaMlaAsmKernel<BF16, SPLIT, NZ>;
+    auto kernel = PaMlaAsmKernel<BF16, SPLIT, NZ, MASK>;
     const int configured = ConfigureKernelLds(reinterpret_cast<const void *>(kernel), LDS_BYTES);
     if (configured != OK) {
         return configured;
@@ -988,9 +1069,18 @@ template <bool BF16, bool SPLIT, bool NZ = false> int LaunchAsm(const PaArgs &ar
     if (grid <= 0 || grid > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: grid of %lld workgroups is out of range", (long long)grid);
     }
+    if (MASK && (args.maskHeadStride != 0 || args.maskBatchStride % 2 != 0 || reinterpret_cast<uintptr_t>(args.mask) % 4 != 0)) {
+        return Fail(ERR_INVALID_PARAM, "pa_decode: the 128-head MLA kernel takes one mask row per query row, rows 4-byte aligned");
+    }
     kernel<<<static_cast<unsigned>(grid), NW * WAVE, LDS_BYTES, stream>>>(args, plan);
     ATBMI_HIP_CHECK(hipGetLastError());
     return OK;
+}
+
+template <bool BF16, bool SPLIT, bool NZ = false> int LaunchAsm(const PaArgs &args, const PaStreamPlan &plan, hipStream_t stream)
+{
+    return args.mask != nullptr ? LaunchAsmBuild<BF16, SPLIT, NZ, true>(args, plan, stream)
+                                : LaunchAsmBuild<BF16, SPLIT, NZ, false>(args, plan, stream);
 }
 
 } // namespace mla

@@ -251,6 +251,11 @@ def run_workload(pkg, name, steps, warmup, attention_only=False, kernel_events=T
         elif mla:
             pa_in = [step["q"], step["key_cache"], step["block_tables"], lens_dev]
             host_idx = 3
+            if mask_type:
+                pa_in.append(step["mask"])
+            if q_len > 1:
+                host_inputs[len(pa_in)] = step["q_lens"]
+                pa_in.append(step["q_lens"].to(dev))
             rac = b.OperationRunner("ReshapeAndCacheOperation", b.ReshapeAndCacheParam(kvCacheCfg=1), ctx)
             rac_in = [step["k_new"], step["key_cache"], step["slot_mapping"]]
             rac_out = [step["key_cache"]]

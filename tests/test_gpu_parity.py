@@ -1468,6 +1468,44 @@ def test_paged_attention_mla_128_head_kernel(binding, oracle, dev, stream, case)
         assert torch.equal(again, got), "relaunch %d differs" % rep
 
 
+# heads, block, ctx, mask row length, dtype, mask layout, ranges   (the 128-head kernel's masked build)
+MLA_WIDE_MASKED = [
+    (128, 128, [700, 45, 1, 2049], 2050, torch.bfloat16, "norm3", None),
+    (16, 128, [333, 1000, 31], 1000, torch.float16, "norm3", None),        # rows as long as the longest context
+    (40, 64, [515, 129, 2048, 4], 2048, torch.bfloat16, "norm3", 64),      # rows cut everywhere
+    (32, 16, [3000, 5], 3002, torch.float16, "norm2", None),               # one row shared by all sequences
+    (128, 128, [257, 130], 1026, torch.float16, "hidden", None),           # -inf over whole tiles and whole rows
+]
+
+
+@pytest.mark.parametrize("case", MLA_WIDE_MASKED, ids=lambda c: "h%d_bs%d_%s_%s" % (
+    c[0], c[1], str(c[4]).split(".")[-1], c[5]))
+def test_paged_attention_mla_128_head_kernel_with_a_mask(binding, oracle, dev, stream, case):
+    """The combined-cache kernel with a mask row per sequence: against the oracle and against the fp32 scalar kernel."""
+    heads, block, ctx, max_len, dtype, kind, chunk = case
+    rng = _rng(400 + heads + block)
+    q, kc, _, tables, ctx = _pa_inputs(rng, dev, len(ctx), heads, 1, block, 576, 512, ctx, dtype, std=0.5)
+    if kind == "hidden":
+        m = rng.standard_normal((len(ctx), 1, max_len)).astype(np.float32)
+        m[0, 0, :64] = -np.inf        # the first two tiles of the first sequence
+        m[0, 0, 100:131] = -np.inf
+        m[1, 0, :] = -np.inf          # all of the second sequence: its rows come out as zeros
+        mask = torch.from_numpy(m).to(dtype).to(dev).contiguous()
+    else:
+        mask, _ = _mask_tensor(oracle, rng, dev, kind, ctx, heads, max_len, dtype)
+    scale = 1.0 / math.sqrt(576)
+    with np.errstate(invalid="ignore"):
+        want = oracle_pa(oracle, q, kc, None, tables, ctx, scale, mla_dv=512, mask=mask)
+    if kind == "hidden":
+        want[1] = 0.0  # (the oracle's softmax of a row of -inf is not a number; the kernels write zeros)
+    got, info = pa_decode_cabi(binding, stream, q, kc, None, tables, ctx, scale, mla_dv=512, mask=mask,
+                               kernel=binding.ATBMI_PA_KERNEL_MFMA, chunk_tokens=chunk, return_plan_info=True)
+    assert_close(got, want, TOL[dtype], "128-head kernel with a mask, %d ranges" % info["chunks"])
+    ref = pa_decode_cabi(binding, stream, q, kc, None, tables, ctx, scale, mla_dv=512, mask=mask,
+                         kernel=binding.ATBMI_PA_KERNEL_SCALAR)
+    assert_close(got, ref.float().cpu().numpy(), TOL[dtype], "128-head kernel with a mask vs scalar kernel")
+
+
 def test_mla_through_operation_api_and_split_head_sizes(binding, oracle, dev, stream):
     rng = _rng(61)
     c = binding.Context(stream)
