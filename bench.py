@@ -54,13 +54,13 @@ WORKLOAD_SOURCES = {
 # sources at the time it was measured: a changed workload or changed kernels report null, not a stale figure.
 MEASURED_TRAFFIC = {
     # (workload, algorithmic bytes): (HBM bytes, summary under profiles/, source hash of the workload)
-    ("c2", 651658484): (659482436, "pa_mfma_bf16_d128_c2_trace_and_traffic.md", "bfde6c8e2f5d"),
-    ("c2_fp16", 651658484): (659481493, "pa_mfma_fp16_d128_c2_fp16_trace_and_traffic.md", "e352b3749fd0"),
-    ("c3", 1364204576): (1381770303, "pa_mfma_int8_d128_c3_trace_and_traffic.md", "a5a50be360bb"),
+    ("c2", 651658484): (659490296, "pa_mfma_bf16_d128_c2_trace_and_traffic.md", "785f75cad0de"),
+    ("c2_fp16", 651658484): (659488863, "pa_mfma_fp16_d128_c2_fp16_trace_and_traffic.md", "84f8833991ec"),
+    ("c3", 1364204576): (1381765670, "pa_mfma_int8_d128_c3_trace_and_traffic.md", "44e89ae892f2"),
     ("c3_int8q", 1363148320): (1379036066, "pa_int8q_d128_c3_sizes_trace_counters_traffic.md", "f19d2f9626c2"),
-    ("c4", 722875880): (728782961, "pa_mfma_fp16_d128_c4_trace_and_traffic.md", "e352b3749fd0"),
-    ("c5_h16", 237786736): (250872196, "pa_mla_bf16_d576_c5_16_heads_trace_and_traffic.md", "4dce44fe9d89"),
-    ("c5", 253384304): (349328455, "pa_mla_bf16_d576_c5_trace_and_traffic.md", "4dce44fe9d89"),
+    ("c4", 722875880): (728779964, "pa_mfma_fp16_d128_c4_trace_and_traffic.md", "84f8833991ec"),
+    ("c5_h16", 237786736): (251795818, "pa_mla_bf16_d576_c5_16_heads_trace_and_traffic.md", "555591b346cd"),
+    ("c5", 253384304): (350318449, "pa_mla_bf16_d576_c5_trace_and_traffic.md", "555591b346cd"),
 }
 OTHER_WORKLOADS = ["c2_fp16", "c3", "c3_int8q", "c4", "c5"]  # timed in the same run as the headline workload
 MIN_KERNEL_LAUNCHES = 100  # launches behind every kernel figure, whatever --steps says
