@@ -377,13 +377,19 @@ int PlanStream(AtbmiPaPlan *plan)
         headsPerWg = PA_MLA_HEADS_PER_WG / PA_MFMA_HEAD_TILE;
         tokenSlices = 1;
     }
-    const int headGroups = (virtualHeads + headsPerWg - 1) / headsPerWg; // (only the 128-head kernel leaves a remainder)
     // Several query tokens of one sequence share a pass over its context when a GQA group
-    // leaves columns of the 16-wide head tile free: 16 / group tokens per pass.
+    // leaves columns of the 16-wide head tile free: 16 / group tokens per pass. The 128-head kernel takes
+    // them as more heads of the same pass (q and out rows of consecutive tokens follow each other in memory
+    // exactly as more heads would): 128 / heads tokens.
     int fold = 1;
     if (headTiles == 1 && !PaMlaWide(s) && plan->maxQueryLen > 1 && !plan->causalRows) {
         fold = std::min(PA_MFMA_HEAD_TILE / groupSize, plan->maxQueryLen);
     }
+    if (PaMlaWide(s) && plan->maxQueryLen > 1 && !plan->causalRows && s.numHeads < PA_MLA_HEADS_PER_WG) {
+        fold = std::max(1, std::min(std::min(PA_MLA_HEADS_PER_WG / s.numHeads, 8), plan->maxQueryLen)); // (the kernel tells 8 tokens apart)
+    }
+    const int headGroups = PaMlaWide(s) ? (fold * s.numHeads + PA_MLA_HEADS_PER_WG - 1) / PA_MLA_HEADS_PER_WG
+                                        : virtualHeads / headsPerWg;
     // What starting a row costs a wave, in steps (PaStreamPlan::rowStartSteps), measured on the 8B- and 70B-shaped
     // batches: a wave whose range holds the start of a row left 3 us (16-bit caches) / 8 us (int8: descales to fetch
     // and fold into the query, twice the steps per byte) later than its neighbours with the same number of steps.

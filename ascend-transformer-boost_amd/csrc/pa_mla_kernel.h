@@ -88,8 +88,11 @@ struct Segment {
     uint32_t tokEnd;      // > tokBegin
     uint32_t complete;    // 1: the segment is the whole row, write the final output
     uint32_t heads;       // how many of the wave's 32 heads the call has (0: none; q then points at any valid row)
-    const void *mask;     // MASK builds: the query row's mask row (16-bit values of the query's type, 4-byte aligned)
-    uint32_t maskBytes;   // ... and its length in bytes, rounded up to 4
+    const void *mask;     // MASK builds: the mask row of the pass's first query token (16-bit values of the query's
+                          // type, 4-byte aligned)
+    uint32_t maskBytes;   // ... bytes from there to the end of its last token's row, rounded up to 4
+    uint32_t maskTokenBytes; // ... bytes between the rows of consecutive query tokens of the pass
+    uint32_t realHeads;   // heads of the call: lane v of the pass (its 32 wave + n-th row) is token v / realHeads
 };
 
 // One segment from start to finish: stages the first tiles, loads Q, runs the pipelined step loop, writes
@@ -116,7 +119,7 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     const uint32_t heads = uni(sg.heads), lastHead = uni(sg.heads > 0 ? sg.heads - 1 : 0);
     const uint64_t mask = uni64(sg.mask);
     const uint32_t maskLo = static_cast<uint32_t>(mask), maskHi = static_cast<uint32_t>(mask >> 32) & 0xffffu;
-    const uint32_t maskBytes = uni(sg.maskBytes);
+    const uint32_t maskBytes = uni(sg.maskBytes), maskTokenBytes = uni(sg.maskTokenBytes), realHeads = uni(sg.realHeads);
     ldsBase = uni(ldsBase);
     wave = uni(wave);
     scale2 = __builtin_bit_cast(float, uni(__builtin_bit_cast(uint32_t, scale2)));
@@ -140,12 +143,13 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     .set NZ, %[nz]
     .set MASK, %[mask_on]
     // MASK: v[100:107] the mask values of the tile whose softmax comes next (16-bit pairs: register 2 g + h holds
-    // tokens 8 g + 4 kh + 2 h, + 1 of the tile); s[68:71] the buffer descriptor of the mask row.
+    // tokens 8 g + 4 kh + 2 h, + 1 of the tile); v108 the lane's byte offset into the mask rows (its query token's
+    // row, 8 kh); s[68:71] the buffer descriptor of the mask rows of the pass.
     // the four loads of the mask values of the tile at token \tok (a scalar register)
     .macro MASK_LOAD tok
       .if MASK
         s_lshl_b32 s46, \tok, 1
-        v_lshl_add_u32 v88, v87, 1, s46      // byte of token tok + 4 kh
+        v_add_u32 v88, s46, v108             // byte of token tok + 4 kh in the lane's row
         .irp g,0,1,2,3
           buffer_load_dwordx2 v[100+2*\g:101+2*\g], v88, s[68:71], 0 offen offset:16*\g
         .endr
@@ -708,6 +712,18 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
       v_lshl_or_b32 v99, v92, 3*\i, v99
     .endr
     .if MASK
+      // the lane's query token: row v = 32 wave + n of the pass belongs to token v / heads (at most 8 tokens a pass)
+      s_lshl_b32 s46, %[wave], 5
+      v_add_u32 v91, s46, v89
+      v_mov_b32 v92, 0
+      .irp k,1,2,3,4,5,6,7
+        s_mul_i32 s47, %[real_heads], \k
+        v_cmp_le_u32 vcc, s47, v91
+        s_nop 1
+        v_addc_co_u32 v92, vcc, 0, v92, vcc
+      .endr
+      v_mul_lo_u32 v108, v92, %[mask_token_bytes]
+      v_lshl_add_u32 v108, v87, 1, v108
       s_mov_b32 s68, %[mask_lo]
       s_mov_b32 s69, %[mask_hi]              // (stride 0: a raw buffer)
       s_mov_b32 s70, %[mask_bytes]
@@ -955,7 +971,8 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     )ASM"
                  :
                  : [bf16] "n"(BF16 ? 1 : 0), [split] "n"(SPLIT ? 1 : 0), [nz] "n"(NZ ? 1 : 0), [mask_on] "n"(MASK ? 1 : 0),
-                   [mask_lo] "s"(maskLo), [mask_hi] "s"(maskHi), [mask_bytes] "s"(maskBytes), [qrope] "s"(qRope), [rope_lo] "s"(ropeLo),
+                   [mask_lo] "s"(maskLo), [mask_hi] "s"(maskHi), [mask_bytes] "s"(maskBytes), [mask_token_bytes] "s"(maskTokenBytes),
+                   [real_heads] "s"(realHeads), [qrope] "s"(qRope), [rope_lo] "s"(ropeLo),
                    [rope_hi] "s"(ropeHi), [roperowbytes] "s"(ropeRowBytes), [scale] "s"(scale2), [bshift] "s"(blockShift), [table] "s"(table),
                    [rowbytes] "s"(rowBytes), [cache_lo] "s"(cacheLo), [cache_hi] "s"(cacheHi), [q] "s"(q), [out] "s"(out),
                    [lse] "s"(lse), [tokbegin] "s"(tokBegin), [tokend] "s"(tokEnd), [lds] "s"(ldsBase), [wave] "s"(wave),
@@ -992,8 +1009,8 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaAsmKernel(const PaArgs a, const
     // (a head count that is not a multiple of 128 leaves the last workgroup waves with fewer than 32 heads, or with
     // none: those still stage their rows of every tile, compute on a repeated query row and store nothing)
     const int h0 = hgIdx * PA_MLA_HEADS_PER_WG + static_cast<int>(wave) * HPW;
-    const int liveHeads = min(max(a.H - h0, 0), HPW);
-    const int hq = liveHeads > 0 ? h0 : 0; // where this wave's query rows are read from
+    // (a pass may hold several query tokens of its sequence: their rows follow each other in q and out as more heads
+    // would, so the pass has tokens x heads rows)
     constexpr float LOG2E = 1.4426950408889634f;
     const float scale2 = a.qkScale * LOG2E;
     const uint32_t blockShift = static_cast<uint32_t>(__builtin_ctz(static_cast<unsigned>(a.blockSize)));
@@ -1023,6 +1040,9 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaAsmKernel(const PaArgs a, const
         sg.tokBegin = static_cast<uint32_t>((segBegin - stepBegin) * STEP);
         sg.tokEnd = static_cast<uint32_t>(min(ctxLen, (segEnd - stepBegin) * STEP));
         sg.complete = (segBegin == stepBegin && segEnd == seqEnd) ? 1u : 0u;
+        const int passHeads = uniform(sq.nTok) * a.H;
+        const int liveHeads = min(max(passHeads - h0, 0), HPW);
+        const int hq = liveHeads > 0 ? h0 : 0; // where this wave's query rows are read from
         const int64_t rowHead = static_cast<int64_t>(qRow) * a.H + h0;
         const int64_t rowQuery = static_cast<int64_t>(qRow) * a.H + hq;
         sg.heads = static_cast<uint32_t>(liveHeads);
@@ -1035,18 +1055,21 @@ __global__ __launch_bounds__(NW *WAVE) void PaMlaAsmKernel(const PaArgs a, const
             sg.lse = a.lse ? reinterpret_cast<uint16_t *>(a.lse) + rowHead : nullptr;
         } else {
             const int slot = 2 * wr + (segBegin == s0 ? 0 : 1);
-            const int64_t ph = static_cast<int64_t>(slot) * a.H + h0;
+            const int64_t ph = static_cast<int64_t>(slot) * p.foldTokens * a.H + h0;
             sg.out = reinterpret_cast<uint16_t *>(a.partO) + ph * DV;
             sg.lse = a.partLse + ph;
         }
         if (MASK) {
             // one mask row per query row (no stride between heads): the row of this pass
             sg.mask = reinterpret_cast<const uint16_t *>(a.mask) + static_cast<int64_t>(uniform(sq.maskRow)) * a.maskBatchStride;
-            sg.maskBytes = (static_cast<uint32_t>(a.maskLen) * 2u + 3u) & ~3u;
+            sg.maskTokenBytes = static_cast<uint32_t>(a.maskRowStep * a.maskBatchStride * 2);
+            sg.maskBytes = (static_cast<uint32_t>(uniform(sq.nTok) - 1) * sg.maskTokenBytes + static_cast<uint32_t>(a.maskLen) * 2u + 3u) & ~3u;
         } else {
             sg.mask = nullptr;
             sg.maskBytes = 0;
+            sg.maskTokenBytes = 0;
         }
+        sg.realHeads = static_cast<uint32_t>(a.H);
         RunSegment<BF16, SPLIT, NZ, MASK>(sg, ldsBase, wave, scale2);
     }
 }
@@ -1059,8 +1082,8 @@ template <bool BF16, bool SPLIT, bool NZ, bool MASK> int LaunchAsmBuild(const Pa
     if (configured != OK) {
         return configured;
     }
-    if (plan.tokenSlices != 1 || plan.numWaveRanges != plan.numWgRanges ||
-        plan.headGroups != (args.H + PA_MLA_HEADS_PER_WG - 1) / PA_MLA_HEADS_PER_WG || args.G != 1 || args.D != D || args.Dv != DV ||
+    if (plan.tokenSlices != 1 || plan.numWaveRanges != plan.numWgRanges || plan.foldTokens < 1 || plan.foldTokens > 8 ||
+        plan.headGroups != (plan.foldTokens * args.H + PA_MLA_HEADS_PER_WG - 1) / PA_MLA_HEADS_PER_WG || args.G != 1 || args.D != D || args.Dv != DV ||
         args.ropeDim != (SPLIT ? D - DV : 0) || (args.nzShift > 0) != NZ || args.blockSize < 16 || (args.blockSize & (args.blockSize - 1)) != 0 ||
         args.kRowStride * 2 > 0x7fffffffLL) {
         return Fail(ERR_INVALID_PARAM, "pa_decode: plan or shape does not fit the 128-head MLA kernel");

@@ -54,13 +54,13 @@ WORKLOAD_SOURCES = {
 # sources at the time it was measured: a changed workload or changed kernels report null, not a stale figure.
 MEASURED_TRAFFIC = {
     # (workload, algorithmic bytes): (HBM bytes, summary under profiles/, source hash of the workload)
-    ("c2", 651658484): (659490296, "pa_mfma_bf16_d128_c2_trace_and_traffic.md", "785f75cad0de"),
-    ("c2_fp16", 651658484): (659488863, "pa_mfma_fp16_d128_c2_fp16_trace_and_traffic.md", "84f8833991ec"),
-    ("c3", 1364204576): (1381765670, "pa_mfma_int8_d128_c3_trace_and_traffic.md", "44e89ae892f2"),
+    ("c2", 651658484): (659493149, "pa_mfma_bf16_d128_c2_trace_and_traffic.md", "39ccea2a1dcb"),
+    ("c2_fp16", 651658484): (659489879, "pa_mfma_fp16_d128_c2_fp16_trace_and_traffic.md", "81b016f9ec73"),
+    ("c3", 1364204576): (1381768462, "pa_mfma_int8_d128_c3_trace_and_traffic.md", "61638a628ebd"),
     ("c3_int8q", 1363148320): (1379036066, "pa_int8q_d128_c3_sizes_trace_counters_traffic.md", "f19d2f9626c2"),
-    ("c4", 722875880): (728779964, "pa_mfma_fp16_d128_c4_trace_and_traffic.md", "84f8833991ec"),
-    ("c5_h16", 237786736): (251795818, "pa_mla_bf16_d576_c5_16_heads_trace_and_traffic.md", "555591b346cd"),
-    ("c5", 253384304): (350318449, "pa_mla_bf16_d576_c5_trace_and_traffic.md", "555591b346cd"),
+    ("c4", 722875880): (728783707, "pa_mfma_fp16_d128_c4_trace_and_traffic.md", "81b016f9ec73"),
+    ("c5_h16", 237786736): (251192985, "pa_mla_bf16_d576_c5_16_heads_trace_and_traffic.md", "431073af82e3"),
+    ("c5", 253384304): (349637123, "pa_mla_bf16_d576_c5_trace_and_traffic.md", "431073af82e3"),
 }
 OTHER_WORKLOADS = ["c2_fp16", "c3", "c3_int8q", "c4", "c5"]  # timed in the same run as the headline workload
 MIN_KERNEL_LAUNCHES = 100  # launches behind every kernel figure, whatever --steps says

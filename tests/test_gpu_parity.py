@@ -2194,6 +2194,53 @@ def test_paged_attention_several_query_tokens(binding, oracle, dev, stream, case
         assert_close(got, want, TOL[dtype], "kernel=%d" % kernel)
 
 
+# heads, block, ctx, q_lens, mask, dtype, chunk override: the 128-head kernel takes the query tokens of a sequence
+# as more heads of one pass, 128 / heads of them (at most 8) at a time
+MLA_WIDE_TOKENS = [
+    (16, 128, [700, 33, 1500], [2, 1, 3], "query", torch.bfloat16, None),
+    (16, 128, [900, 40, 300], [8, 11, 5], "query", torch.float16, None),       # 8 a pass, then the rest
+    (16, 64, [2100, 64], [4, 2], "query", torch.bfloat16, 128),                # partial rows of every token
+    (8, 128, [515, 1030], [9, 3], "position", torch.float16, None),            # 8 tokens fill half the rows
+    (48, 16, [1200, 77, 300], [2, 2, 1], "query", torch.bfloat16, 256),        # 96 rows: a wave without any
+    (40, 128, [640, 1300], [3, 3], None, torch.float16, None),                 # 120 rows, a pass of one token behind
+    (64, 128, [513, 4000], [2, 2], "sequence", torch.bfloat16, None),          # one mask row for both tokens
+    (32, 128, [3000, 3000, 3000, 3000], [4, 4, 4, 4], None, torch.bfloat16, 512),
+]
+
+
+@pytest.mark.parametrize("case", MLA_WIDE_TOKENS, ids=lambda c: "h%d_bs%d_q%s_%s_%s%s" % (
+    c[0], c[1], "-".join(map(str, c[3])), c[4], str(c[5]).split(".")[-1], "_chunk%d" % c[6] if c[6] else ""))
+def test_paged_attention_mla_128_head_kernel_with_several_query_tokens(binding, oracle, dev, stream, case):
+    """Several query tokens per sequence over the combined cache, with the log-sum-exp output: against the oracle and
+    against the fp32 scalar kernel."""
+    heads, block, ctx, q_lens, kind, dtype, chunk = case
+    rng = _rng(700 + heads + block + len(ctx))
+    _, kc, _, tables, ctx = _pa_inputs(rng, dev, len(ctx), heads, 1, block, 576, 576, ctx, dtype, std=0.5)
+    rows = int(sum(n for n, c in zip(q_lens, ctx) if c > 0))
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(int(rng.integers(1 << 30)))
+    q = (torch.rand((rows + 1, heads, 576), generator=gen) * 2 - 1).to(dtype).to(dev)
+    if kind == "sequence":
+        mask, _ = _mask_tensor(oracle, rng, dev, "norm3", ctx, heads, int(max(ctx)), dtype)
+    else:
+        mask = None if kind is None else _spec_mask(rng, dev, kind, ctx, q_lens, dtype)
+    mode = kind or "sequence"
+    scale = 1.0 / math.sqrt(192.0)
+    want_lse = np.zeros((rows + 1, heads), np.float32)
+    want = oracle_pa(oracle, q, kc, None, tables, ctx, scale, mla_dv=512, out_init=0.25, mask=mask, q_lens=q_lens,
+                     mask_rows=mode, lse_out=want_lse)
+    results = []
+    for kernel in (binding.ATBMI_PA_KERNEL_MFMA, binding.ATBMI_PA_KERNEL_SCALAR):
+        out = torch.full((rows + 1, heads, 512), 0.25, dtype=dtype, device=dev)
+        lse = torch.zeros((rows + 1, heads), dtype=dtype, device=dev)
+        got = pa_decode_cabi(binding, stream, q, kc, None, tables, ctx, scale, mla_dv=512, kernel=kernel, out=out,
+                             mask=mask, q_lens=q_lens, mask_rows=mode, lse=lse, chunk_tokens=chunk)
+        assert_close(got, want, TOL[dtype], "kernel=%d" % kernel)
+        assert_close(lse[:rows], want_lse[:rows], TOL[dtype], "lse kernel=%d" % kernel)
+        results.append(got.float().cpu().numpy())
+    assert_close(results[0], results[1], TOL[dtype], "128-head kernel vs scalar kernel")
+
+
 def test_several_query_tokens_through_operation_api(binding, oracle, dev, stream):
     """calcType = CALC_TYPE_SPEC: inputs q, caches, tables, contextLens, mask, qSeqLens
     (reference paged_attention_operation.cpp:408-426), both lengths with hostData."""
