@@ -2205,6 +2205,7 @@ MLA_WIDE_TOKENS = [
     (40, 128, [640, 1300], [3, 3], None, torch.float16, None),                 # 120 rows, a pass of one token behind
     (64, 128, [513, 4000], [2, 2], "sequence", torch.bfloat16, None),          # one mask row for both tokens
     (32, 128, [3000, 3000, 3000, 3000], [4, 4, 4, 4], None, torch.bfloat16, 512),
+    (16, 128, [700, 0, 300, 64, 2], [3, 2, 0, 5, 2], "query", torch.float16, None),   # no context, no query tokens
 ]
 
 
