@@ -148,18 +148,18 @@ template <bool BF16> __device__ __forceinline__ f32x4 Mma16(u32x4 a, u32x4 b, f3
 // the transfer may land where they read. The compiler does not count these loads: the kernel waits for them with
 // WaitForLoads. A wave asks for one piece at a time, between pieces of arithmetic: the path from the compute unit
 // to its cache takes a wave's request for 1 KiB in about 16 cycles, and a wave whose request finds that path full
-// waits with everything else it has to do.
+// waits with everything else it has to do. The requests carry the non-temporal hint: a cache row is read once a call.
 template <int OFFSET, bool WAIT>
 __device__ __forceinline__ void TransferPieceToLds(uint32_t ldsBase, const unsigned char *base, uint32_t laneOffset)
 {
     static_assert(OFFSET >= -4096 && OFFSET < 4096, "13-bit offset field");
     if constexpr (WAIT) {
-        asm volatile("s_mov_b32 m0, %0\n\ts_waitcnt lgkmcnt(0)\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
+        asm volatile("s_mov_b32 m0, %0\n\ts_waitcnt lgkmcnt(0)\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3 nt"
                      :
                      : "s"(ldsBase), "v"(laneOffset), "s"(base), "n"(OFFSET)
                      : "memory", "m0");
     } else {
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3 nt"
                      :
                      : "s"(ldsBase), "v"(laneOffset), "s"(base), "n"(OFFSET)
                      : "memory", "m0");

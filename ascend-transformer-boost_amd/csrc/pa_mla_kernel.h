@@ -441,11 +441,12 @@ __device__ __forceinline__ void RunSegment(const Segment &sg, uint32_t ldsBase, 
     .endm
     // the instruction of transfer i from the source base in s[base : base+1]; M0 = region + 4096 for i < 8,
     // region + 8192 after
+    // (non-temporal: a cache row is read once a step; the hint is worth a twentieth of the stream from HBM)
     .macro DMA_LOAD i, base
       .if \i < 8
-        global_load_lds_dwordx4 v[72+\i], s[\base:\base+1] offset:(\i-4)*1024
+        global_load_lds_dwordx4 v[72+\i], s[\base:\base+1] offset:(\i-4)*1024 nt
       .else
-        global_load_lds_dwordx4 v[72+\i], s[\base:\base+1] offset:(\i-8)*1024
+        global_load_lds_dwordx4 v[72+\i], s[\base:\base+1] offset:(\i-8)*1024 nt
       .endif
     .endm
     // transfer i of a tile whose rows all lie inside the segment

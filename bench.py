@@ -59,8 +59,8 @@ MEASURED_TRAFFIC = {
     ("c3", 1364204576): (1381768462, "pa_mfma_int8_d128_c3_trace_and_traffic.md", "61638a628ebd"),
     ("c3_int8q", 1363148320): (1379036066, "pa_int8q_d128_c3_sizes_trace_counters_traffic.md", "f19d2f9626c2"),
     ("c4", 722875880): (728783707, "pa_mfma_fp16_d128_c4_trace_and_traffic.md", "81b016f9ec73"),
-    ("c5_h16", 237786736): (251192985, "pa_mla_bf16_d576_c5_16_heads_trace_and_traffic.md", "431073af82e3"),
-    ("c5", 253384304): (349637123, "pa_mla_bf16_d576_c5_trace_and_traffic.md", "431073af82e3"),
+    ("c5_h16", 237786736): (249995659, "pa_mla_bf16_d576_c5_16_heads_trace_and_traffic.md", "af5ed28e4ff4"),
+    ("c5", 253384304): (342817654, "pa_mla_bf16_d576_c5_trace_and_traffic.md", "af5ed28e4ff4"),
 }
 OTHER_WORKLOADS = ["c2_fp16", "c3", "c3_int8q", "c4", "c5"]  # timed in the same run as the headline workload
 MIN_KERNEL_LAUNCHES = 100  # launches behind every kernel figure, whatever --steps says
@@ -285,13 +285,25 @@ def run_workload(pkg, name, steps, warmup, attention_only=False, kernel_events=T
         # the same tensors: such a workload gets copies of its caches, enough for 768 MB, and the steps go
         # round them, so that a step's rows were last touched at least 512 MB of traffic ago.
         pools = [(pa_in, rac_in if rac is not None else None, rac_out if rac is not None else None)]
-        cache_ids = {id(step[n]): n for n in ("key_cache", "value_cache") if step.get(n) is not None}
-        cache_bytes = sum(step[n].numel() * step[n].element_size() for n in cache_ids.values())
-        if not split and not int8 and not cfg.get("bnsd") and 0 < cache_bytes < MALL_BYTES * 2:
+        caches = []        # (an object of the lists above, what makes a copy of it, the bytes the attention reads of it)
+        alive = []         # tensors behind the descriptors of copies
+        size = lambda t: t.numel() * t.element_size()
+        if split:
+            caches += [(t, t.clone, 0 if nz else size(t)) for t in (nope, rope)]
+            if nz:
+                def described_copy(t):
+                    alive.append(t.clone())
+                    return b.make_tensor(b._torch_acl_dtype(alive[-1]), list(alive[-1].shape),
+                                         device_ptr=alive[-1].data_ptr(), fmt="fractal_nz")
+                caches += [(pa_in[2 + i], (lambda t=t: described_copy(t)), size(t)) for i, t in enumerate(nz_caches)]
+        elif not int8 and not cfg.get("bnsd"):
+            caches += [(step[n], step[n].clone, size(step[n])) for n in ("key_cache", "value_cache")
+                       if step.get(n) is not None]
+        cache_bytes = sum(c[2] for c in caches)
+        if 0 < cache_bytes < MALL_BYTES * 2:
             for _ in range(-(-MALL_BYTES * 3 // cache_bytes) - 1):
-                copies = {n: step[n].clone() for n in cache_ids.values()}
-                swap = lambda ts: None if ts is None else [copies[cache_ids[id(t)]] if id(t) in cache_ids else t
-                                                           for t in ts]
+                copies = {id(obj): copy() for obj, copy, _ in caches}
+                swap = lambda ts: None if ts is None else [copies.get(id(t), t) for t in ts]
                 pools.append((swap(pa_in), swap(pools[0][1]), swap(pools[0][2])))
     slots = cfg["block"] * step["layout"]["pool"]
     turn = [0]
