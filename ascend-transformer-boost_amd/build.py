@@ -81,8 +81,17 @@ def build_host():
     return target
 
 
+def build_tools():
+    """The stand-alone HBM streaming benchmark (an executable, not part of the libraries)."""
+    os.makedirs(LIB, exist_ok=True)
+    target = os.path.join(LIB, "bench_hbm_stream")
+    _run([HIPCC, "-O3", "-std=c++17", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+          "-packed-fp32-ops", os.path.join(PKG, "bench_hbm_stream.hip"), "-o", target])
+    return target
+
+
 def build_all(jobs=8):
-    return [build_kernels(jobs), build_host()]
+    return [build_kernels(jobs), build_host(), build_tools()]
 
 
 def sanitizer_runtime():
