@@ -1766,6 +1766,38 @@ def test_no_wave_range_of_a_plan_is_empty(binding):
         k.atbmi_pa_plan_destroy(plan)
 
 
+def test_query_tokens_of_a_sequence_share_a_pass_of_the_128_head_mla_kernel(binding):
+    """With fewer than 128 heads the 128-head MLA kernel takes the query tokens of a sequence as more heads of one pass
+    over its context (128 / heads of them, at most 8): the plan then has the steps, and so the ranges, of one token per
+    sequence. With 128 heads, or a mask whose rows the kernel cannot address (odd stride: the 16-head tiles take it, one
+    pass per token), every token is a pass of its own."""
+    k = binding.kernels()
+
+    def ranges(heads, q_len, mask_stride=0):
+        shape = binding.AtbmiPaShape(qDtype=1, kvDtype=1, numHeads=heads, numKvHeads=1, headDimK=576, headDimV=512,
+                                     blockSize=128, numBlocks=64, maxBlocksPerSeq=32, numQueryRows=2 * q_len,
+                                     mlaCombined=1, qkScale=1.0, kernel=binding.ATBMI_PA_KERNEL_MFMA,
+                                     hasMask=1 if mask_stride else 0, maskLen=mask_stride, maskBatchStride=mask_stride,
+                                     maskRowBy=1 if mask_stride else 0)
+        plan = ctypes.c_void_p()
+        assert k.atbmi_pa_plan_create(ctypes.byref(shape), ctypes.byref(plan)) == 0, k.atbmi_last_error()
+        lens, qn = np.array([4096, 4096], dtype=np.int32), np.array([q_len, q_len], dtype=np.int32)
+        assert k.atbmi_pa_plan_update_multi(plan, lens.ctypes.data, qn.ctypes.data, 2) == 0, k.atbmi_last_error()
+        n, ws = k.atbmi_pa_plan_num_chunks(plan), k.atbmi_pa_plan_workspace_size(plan)
+        k.atbmi_pa_plan_destroy(plan)
+        return n, ws
+
+    one, ws_one = ranges(16, 1)
+    four, ws_four = ranges(16, 4)
+    assert four == one and ws_four > ws_one          # the same ranges; a slot holds the partial rows of four tokens
+    assert ranges(16, 8)[0] == one and ranges(16, 9)[0] > one   # eight tokens a pass at most
+    assert ranges(32, 4)[0] == one and ranges(64, 2)[0] == one
+    assert ranges(64, 3)[0] > one                    # 128 / 64 = 2 tokens a pass
+    assert ranges(128, 2)[0] > ranges(128, 1)[0]     # the rows of 128 heads are full
+    assert ranges(16, 4, mask_stride=4096)[0] == one
+    assert ranges(16, 4, mask_stride=4097)[0] > one
+
+
 def test_plan_refuses_a_context_longer_than_the_mask_row(binding):
     k = binding.kernels()
     shape = binding.AtbmiPaShape(qDtype=0, kvDtype=0, numHeads=8, numKvHeads=8, headDimK=128, headDimV=128,
